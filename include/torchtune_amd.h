@@ -1,0 +1,188 @@
+/*
+ * torchtune_amd C ABI — MI355X (gfx950) kernels for the QLoRA / QAT quantized-linear path.
+ *
+ * The reference (pytorch/torchtune) has no native layer: the arithmetic of this path lives in eager
+ * PyTorch op sequences inside the third-party `torchao` package.  Each entry point below therefore
+ * cites the Python call site(s) in the reference whose work it replaces, not an FFI declaration.
+ *
+ * Conventions (all entry points):
+ *   - plain C, no torch types; every pointer is a caller-owned DEVICE pointer unless stated, 16-byte
+ *     aligned, row-major contiguous;
+ *   - `stream` is a `hipStream_t` passed as `void*` (NULL = the default stream); work is enqueued
+ *     asynchronously on it, nothing synchronises the host;
+ *   - the return value is 0 on success or a negative `TTAMD_E*` code; `ttamd_last_error()` then gives
+ *     a thread-local, human-readable message;
+ *   - nothing here allocates or frees device memory: scratch space is passed in as `workspace`,
+ *     sized by the matching `*_workspace_bytes` query;
+ *   - the calls are re-entrant and keep no stream or device state between calls.
+ *
+ * dtype codes: TTAMD_BF16 = bfloat16, TTAMD_F32 = float32.
+ */
+#ifndef TORCHTUNE_AMD_H
+#define TORCHTUNE_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TTAMD_ABI_VERSION 1
+
+#define TTAMD_BF16 0
+#define TTAMD_F32 1
+
+#define TTAMD_OK 0
+#define TTAMD_EINVAL (-1)     /* bad argument: null pointer, misaligned pointer, shape or divisibility violation */
+#define TTAMD_EUNSUPPORTED (-2) /* valid request this build has no kernel for (e.g. fused GEMM with block_size != 64) */
+#define TTAMD_EWORKSPACE (-3) /* workspace too small */
+#define TTAMD_ELAUNCH (-4)    /* the HIP runtime reported an error at launch */
+
+/* ABI version of the loaded library (== TTAMD_ABI_VERSION it was built with). */
+int ttamd_version(void);
+
+/* Message for the last non-zero return on the calling thread ("" if none). Host pointer, valid until the
+ * next failing call on the same thread. */
+const char* ttamd_last_error(void);
+
+/* ------------------------------------------------------------------------------------------------
+ * NF4 double-quantisation codec
+ * ---------------------------------------------------------------------------------------------- */
+
+/*
+ * to_nf4(tensor, block_size, scaler_block_size): replaces torchao's NF4Tensor.from_tensor as called at
+ *   torchtune/modules/peft/lora.py:86, torchtune/modules/low_precision/nf4_linear.py:49,
+ *   torchtune/modules/low_precision/_register_nf4_dispatch_ops.py:20, torchtune/training/_distributed.py:404.
+ *
+ * w                    [numel] `dtype` (the flattened [N,K] weight)
+ * quantized_data  out  [numel/2] uint8, two 4-bit codes per byte, even element in the high nibble
+ * quantized_scalers out [numel/block_size] int8
+ * quantization_factor out [numel/block_size/scaler_block_size] `dtype`
+ * scaler_mean     out  [1] `dtype`
+ * workspace            ttamd_nf4_quantize_workspace_bytes(numel, block_size) bytes
+ *
+ * Requires numel % block_size == 0, (numel/block_size) % scaler_block_size == 0, block_size % 8 == 0.
+ * All arithmetic is carried out in `dtype` with round-to-nearest-even after every operation, as the eager
+ * reference does.  A block whose absmax is 0 (0/0 = NaN distances) gets code 0 for every element; a NaN
+ * scaled scaler quantises to 0.
+ */
+size_t ttamd_nf4_quantize_workspace_bytes(int64_t numel, int block_size);
+int ttamd_nf4_quantize(const void* w, int dtype, int64_t numel, int block_size, int scaler_block_size,
+                       uint8_t* quantized_data, int8_t* quantized_scalers, void* quantization_factor,
+                       void* scaler_mean, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * NF4Tensor.get_original_weight() / NF4Tensor.to(dtype): replaces the torchao dequantisation chain reached from
+ *   torchtune/modules/common_utils.py:57 (state-dict hook), torchtune/modules/peft/dora.py:137,183,
+ *   torchtune/modules/low_precision/_register_nf4_dispatch_ops.py:20, torchtune/training/_distributed.py:523,
+ *   and implicitly by linear_nf4 (lora.py:138, nf4_linear.py:67) in every forward and backward.
+ *
+ * `dtype` is the dtype of quantization_factor / scaler_mean and of `out` (the tensor's original dtype).
+ * out [numel] `dtype`.
+ */
+int ttamd_nf4_dequantize(const uint8_t* quantized_data, const int8_t* quantized_scalers,
+                         const void* quantization_factor, const void* scaler_mean, int dtype, int64_t numel,
+                         int block_size, int scaler_block_size, void* out, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * Fused NF4 + LoRA linear (bf16 activations, fp32 accumulate, NF4 block_size 64)
+ *
+ * One LoRALinear.forward (torchtune/modules/peft/lora.py:128-147) is two calls: ttamd_lora_hidden_bf16, then
+ * ttamd_nf4_lora_linear_fwd_bf16.  Its backward is ttamd_lora_bwd_bf16 followed by ttamd_nf4_linear_bwd_dx_bf16.
+ * FrozenNF4Linear.forward / linear_nf4 (torchtune/modules/low_precision/nf4_linear.py:56-70) is the rank == 0 case
+ * of the two GEMM entry points alone.
+ * ---------------------------------------------------------------------------------------------- */
+
+/*
+ * Dequantised block scalers of an NF4 tensor, one bf16 per 64-element block:
+ *     block_scalers[b] = bf16( dtype( dtype(quantized_scalers[b] / quantization_factor[b / SB]) + scaler_mean ) )
+ * This is the `dequantize_scalers` step of NF4Tensor.get_original_weight (torchao; reached from lora.py:138 on
+ * every call).  The weight is frozen, so callers compute it once per tensor and keep it; the GEMMs below take it
+ * in place of the three scaler tensors.  `dtype` is the dtype of quantization_factor / scaler_mean.
+ */
+int ttamd_nf4_block_scalers(const int8_t* quantized_scalers, const void* quantization_factor, const void* scaler_mean,
+                            int dtype, int64_t n_blocks, int scaler_block_size, void* block_scalers, void* stream);
+
+/*
+ * h = bf16(x . lora_a^T): the adapter's hidden activation `self.lora_a(self.dropout(x))` (lora.py:144).
+ * x [M,K] bf16, lora_a [rank,K] bf16, h out [M,rank] bf16; rank a multiple of 8 in [8,64], K % 64 == 0.
+ * workspace: ttamd_lora_fwd_workspace_bytes(M, K, rank) bytes.
+ */
+size_t ttamd_lora_fwd_workspace_bytes(int64_t M, int64_t K, int rank);
+int ttamd_lora_hidden_bf16(const void* x, const void* lora_a, void* h, int64_t M, int64_t K, int rank, void* workspace,
+                           size_t workspace_bytes, void* stream);
+
+/*
+ * y = x . D(W)^T (+ bias) + scale . h . lora_b^T          (lora.py:137-147; nf4_linear.py:67-70 when rank == 0)
+ *
+ * x [M,K] bf16; quantized_data = NF4 codes of the [N,K] weight (block_size 64); block_scalers from
+ * ttamd_nf4_block_scalers; h [M,rank] bf16 from ttamd_lora_hidden_bf16 and lora_b [N,rank] bf16 (both NULL iff
+ * rank == 0); bias [N] bf16 or NULL; scale = alpha / rank; y out [M,N] bf16.
+ * Requires K % 64 == 0, N % 64 == 0, rank % 8 == 0, 0 <= rank <= 64.
+ * D(W) is bit-identical to ttamd_nf4_dequantize's output; all products are accumulated in fp32 and the sum is
+ * rounded to bf16 once (the eager reference rounds after each of its five ops).
+ */
+int ttamd_nf4_lora_linear_fwd_bf16(const void* x, const uint8_t* quantized_data, const void* block_scalers, const void* h,
+                                   const void* lora_b, int rank, float scale, const void* bias, void* y, int64_t M,
+                                   int64_t N, int64_t K, void* stream);
+
+/*
+ * gx = gy . D(W) + gh . lora_a: LinearNF4.backward (torchao; reached from lora.py:138, nf4_linear.py:67) plus the
+ * term autograd adds for lora_a's input.  gy [M,N] bf16; gh [M,rank] bf16 from ttamd_lora_bwd_bf16 and
+ * lora_a [rank,K] bf16 (both NULL iff rank == 0); gx out [M,K] bf16.  Same divisibility rules as the forward.
+ */
+int ttamd_nf4_linear_bwd_dx_bf16(const void* gy, const uint8_t* quantized_data, const void* block_scalers, const void* gh,
+                                 const void* lora_a, int rank, void* gx, int64_t M, int64_t N, int64_t K, void* stream);
+
+/*
+ * Adapter gradients (what autograd derives for lora.py:144-146):
+ *     gh = scale . gy . B        [M,rank] bf16
+ *     gA = gh^T . x              [rank,K] bf16
+ *     gB = scale . gy^T . h      [N,rank] bf16
+ * gy [M,N], x [M,K], h [M,rank] (from the forward), lora_b [N,rank]; all bf16, fp32 accumulation in a fixed order.
+ * workspace: ttamd_lora_bwd_workspace_bytes(M,N,K,rank) bytes.
+ */
+size_t ttamd_lora_bwd_workspace_bytes(int64_t M, int64_t N, int64_t K, int rank);
+int ttamd_lora_bwd_bf16(const void* gy, const void* x, const void* h, const void* lora_b, float scale, void* gh, void* ga,
+                        void* gb, int64_t M, int64_t N, int64_t K, int rank, void* workspace, size_t workspace_bytes,
+                        void* stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * QAT fake quantisation (int8 dynamic per-token activations, int4 per-group symmetric weights)
+ * ---------------------------------------------------------------------------------------------- */
+
+/*
+ * FakeQuantizer.forward for FakeQuantizeConfig(torch.int8, "per_token", is_symmetric=False) — torchao; built by
+ * Int8DynActInt4WeightQATQuantizer.prepare (recipes/qat_single_device.py:378-386) and at
+ * torchtune/modules/peft/lora.py:232,258.
+ *
+ * x [rows,K] `dtype`; out [rows,K] `dtype` = dequantise(quantise(x)) with per-row asymmetric int8 qparams computed
+ * in fp32; scale out [rows] fp32 and zero_point out [rows] int32 may be NULL.  K % 8 == 0.
+ * The straight-through backward is the identity and needs no kernel.
+ */
+int ttamd_fq_per_token_int8_asym(const void* x, int dtype, int64_t rows, int64_t K, void* out, float* scale,
+                                 int32_t* zero_point, void* stream);
+
+/*
+ * FakeQuantizer.forward for FakeQuantizeConfig(torch.int4, group_size=g, is_symmetric=True) — torchao; same call
+ * sites (weight side: lora.py:245,259).
+ *
+ * w [rows,K] `dtype`, groups of `group_size` consecutive elements along K (K % group_size == 0, group_size a
+ * power of two in [8, 512]); out [rows,K] `dtype`; scale out [rows, K/group_size] fp32 may be NULL.
+ */
+int ttamd_fq_per_group_int4_sym(const void* w, int dtype, int64_t rows, int64_t K, int group_size, void* out,
+                                float* scale, void* stream);
+
+/*
+ * quantizer.convert(model) (recipes/quantize.py:92): the real int4 weights of an 8da4w linear.
+ * q out [rows,K] int8 holding values in [-8,7]; scale out [rows,K/group_size] fp32; zero_point out
+ * [rows,K/group_size] fp32 (all zero for the symmetric scheme; may be NULL).
+ */
+int ttamd_quantize_per_group_int4(const void* w, int dtype, int64_t rows, int64_t K, int group_size, int8_t* q,
+                                  float* scale, float* zero_point, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TORCHTUNE_AMD_H */

@@ -1,0 +1,119 @@
+"""CPU oracle for the QAT fake-quantisation arithmetic (8da4w: int8 dynamic per-token activations, int4
+per-group symmetric weights).
+
+TEST INFRASTRUCTURE ONLY — never imported by the shipped package.
+
+Eager-PyTorch restatement of what the reference runs through ``torchao.quantization.qat``:
+
+* ``fq_per_token_int8_asym``   <- ``FakeQuantizer`` built from ``FakeQuantizeConfig(torch.int8, "per_token",
+  is_symmetric=False)``; reference: ``torchtune/modules/peft/lora.py:232,258``, created for every linear by
+  ``Int8DynActInt4WeightQATQuantizer.prepare`` (``recipes/qat_single_device.py:378-386``).
+* ``fq_per_group_int4_sym``    <- ``FakeQuantizer`` built from ``FakeQuantizeConfig(torch.int4, group_size=g,
+  is_symmetric=True)``; reference: ``torchtune/modules/peft/lora.py:245,259``.
+* ``quantize_per_group_int4``  <- ``quantizer.convert(model)`` (``recipes/quantize.py:92``).
+* ``fake_quantized_linear``    <- ``FakeQuantizedLinear.forward``: ``F.linear(fq(x), fq(W))`` with the
+  straight-through estimator in backward; the prose description is at
+  ``docs/source/tutorials/qat_finetune.rst:40-50``.
+
+Parity status: PARITY UNPINNED against torchao itself (not importable here; the reference holds no vectors
+for these functions).  Pinned instead by closed forms and invariants in tests/test_oracle_fake_quant.py
+(scale = (max-min)/255 and the zero-point formula on hand-built rows, outputs on the scale*(q-zp) grid,
+idempotence for fixed qparams, exhaustive tiny cases) and by the independent C restatement oracle/nf4_ref.c.
+
+Numerics: qparams are computed in fp32 from the fp32-promoted input; eps = finfo(float32).eps;
+``round`` is round-half-to-even; the dequantised value is ``(q - zp)`` cast to the input dtype, times the fp32
+scale, cast back to the input dtype.  The backward mask ``(q >= qmin) & (q <= qmax)`` is evaluated on the
+clamped ``q`` and is therefore all ones: the gradient passes straight through.
+"""
+from __future__ import annotations
+
+import torch
+import torch.nn.functional as F
+
+_EPS = torch.finfo(torch.float32).eps
+
+
+def choose_qparams_per_token_asym(x: torch.Tensor):
+    """int8 asymmetric qparams for each row of the last dimension -> (scale fp32 [...,1], zero_point int32 [...,1])."""
+    qmin, qmax = -128, 127
+    xf = x.to(torch.float32)
+    mn = torch.amin(xf, dim=-1, keepdim=True)
+    mx = torch.amax(xf, dim=-1, keepdim=True)
+    mn_neg = torch.min(mn, torch.zeros_like(mn))
+    mx_pos = torch.max(mx, torch.zeros_like(mx))
+    scale = (mx_pos - mn_neg) / float(qmax - qmin)
+    scale = scale.clamp(min=_EPS)
+    descaled_min = mn_neg / scale
+    descaled_max = mx_pos / scale
+    zp_from_min_err = qmin + descaled_min
+    zp_from_max_err = qmax + descaled_max
+    zp = torch.where(zp_from_min_err + zp_from_max_err > 0, qmin - descaled_min, qmax - descaled_max)
+    zp = torch.clamp(zp, qmin, qmax).round()
+    return scale, zp.to(torch.int32)
+
+
+def _fake_quantize(x: torch.Tensor, scale: torch.Tensor, zp: torch.Tensor, qmin: int, qmax: int):
+    q = torch.clamp(torch.round(x * (1.0 / scale)) + zp, qmin, qmax)
+    dq = (q.to(torch.int32) - zp.to(torch.int32)).to(x.dtype)
+    dq = (dq * scale).to(x.dtype)
+    return q, dq
+
+
+def fq_per_token_int8_asym(x: torch.Tensor):
+    """returns (fake-quantised x, scale [rows] fp32, zero_point [rows] int32)"""
+    scale, zp = choose_qparams_per_token_asym(x)
+    _, dq = _fake_quantize(x, scale, zp, -128, 127)
+    return dq, scale.reshape(-1), zp.reshape(-1)
+
+
+def choose_qparams_per_group_sym(w: torch.Tensor, group_size: int):
+    """int4 symmetric qparams per group of `group_size` along the last dim -> scale fp32 [rows, K/g]."""
+    qmin, qmax = -8, 7
+    rows, K = w.shape
+    g = w.to(torch.float32).view(rows, K // group_size, group_size)
+    mn = torch.amin(g, dim=-1)
+    mx = torch.amax(g, dim=-1)
+    mn_neg = torch.min(mn, torch.zeros_like(mn))
+    mx_pos = torch.max(mx, torch.zeros_like(mx))
+    amax = torch.max(-mn_neg, mx_pos)
+    scale = amax / (float(qmax - qmin) / 2)
+    return scale.clamp(min=_EPS)
+
+
+def fq_per_group_int4_sym(w: torch.Tensor, group_size: int):
+    """returns (fake-quantised w, scale [rows, K/g] fp32)"""
+    rows, K = w.shape
+    scale = choose_qparams_per_group_sym(w, group_size)
+    wg = w.view(rows, K // group_size, group_size)
+    zp = torch.zeros_like(scale, dtype=torch.int32)
+    _, dq = _fake_quantize(wg, scale[..., None], zp[..., None], -8, 7)
+    return dq.reshape(rows, K), scale
+
+
+def quantize_per_group_int4(w: torch.Tensor, group_size: int):
+    """convert(): returns (int8 tensor of int4 values [rows,K], scale [rows,K/g] fp32, zeros [rows,K/g] fp32)"""
+    rows, K = w.shape
+    scale = choose_qparams_per_group_sym(w, group_size)
+    wg = w.view(rows, K // group_size, group_size)
+    q = torch.clamp(torch.round(wg * (1.0 / scale[..., None])), -8, 7).to(torch.int8)
+    return q.reshape(rows, K), scale, torch.zeros_like(scale)
+
+
+class _STE(torch.autograd.Function):
+    """y = fq(x) in forward, dy/dx = 1 in backward (the all-ones mask of the reference)."""
+
+    @staticmethod
+    def forward(ctx, x, fq):
+        return fq
+
+    @staticmethod
+    def backward(ctx, g):
+        return g, None
+
+
+def fake_quantized_linear(x: torch.Tensor, w: torch.Tensor, group_size: int, bias=None) -> torch.Tensor:
+    """FakeQuantizedLinear.forward with both fake quantisers enabled; differentiable w.r.t. x and w."""
+    x2 = x.reshape(-1, x.shape[-1])
+    x_fq = _STE.apply(x2, fq_per_token_int8_asym(x2.detach())[0]).reshape(x.shape)
+    w_fq = _STE.apply(w, fq_per_group_int4_sym(w.detach(), group_size)[0])
+    return F.linear(x_fq, w_fq, bias)

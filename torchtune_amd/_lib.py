@@ -1,0 +1,107 @@
+"""ctypes binding of ``libtorchtune_amd.so`` (the C ABI declared in ``include/torchtune_amd.h``).
+
+The library is the only compute path of this package: if it cannot be loaded, every op raises.  There is no
+eager-PyTorch or CPU substitute behind it.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import threading
+from pathlib import Path
+
+LIB_PATH = Path(__file__).resolve().parent / "lib" / "libtorchtune_amd.so"
+ABI_VERSION = 1
+
+TTAMD_BF16 = 0
+TTAMD_F32 = 1
+
+_c_void_p = ctypes.c_void_p
+_i64 = ctypes.c_int64
+_int = ctypes.c_int
+_f32 = ctypes.c_float
+_size = ctypes.c_size_t
+
+# name -> (restype, argtypes); one entry per symbol declared in include/torchtune_amd.h
+SIGNATURES = {
+    "ttamd_version": (_int, []),
+    "ttamd_last_error": (ctypes.c_char_p, []),
+    "ttamd_nf4_quantize_workspace_bytes": (_size, [_i64, _int]),
+    "ttamd_nf4_quantize": (
+        _int,
+        [_c_void_p, _int, _i64, _int, _int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _size, _c_void_p],
+    ),
+    "ttamd_nf4_dequantize": (
+        _int,
+        [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _int, _i64, _int, _int, _c_void_p, _c_void_p],
+    ),
+    "ttamd_nf4_block_scalers": (_int, [_c_void_p, _c_void_p, _c_void_p, _int, _i64, _int, _c_void_p, _c_void_p]),
+    "ttamd_lora_fwd_workspace_bytes": (_size, [_i64, _i64, _int]),
+    "ttamd_lora_hidden_bf16": (_int, [_c_void_p, _c_void_p, _c_void_p, _i64, _i64, _int, _c_void_p, _size, _c_void_p]),
+    "ttamd_nf4_lora_linear_fwd_bf16": (
+        _int,
+        [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _int, _f32, _c_void_p, _c_void_p, _i64, _i64, _i64, _c_void_p],
+    ),
+    "ttamd_nf4_linear_bwd_dx_bf16": (
+        _int,
+        [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _int, _c_void_p, _i64, _i64, _i64, _c_void_p],
+    ),
+    "ttamd_lora_bwd_workspace_bytes": (_size, [_i64, _i64, _i64, _int]),
+    "ttamd_lora_bwd_bf16": (
+        _int,
+        [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _f32, _c_void_p, _c_void_p, _c_void_p, _i64, _i64, _i64, _int,
+         _c_void_p, _size, _c_void_p],
+    ),
+    "ttamd_fq_per_token_int8_asym": (_int, [_c_void_p, _int, _i64, _i64, _c_void_p, _c_void_p, _c_void_p, _c_void_p]),
+    "ttamd_fq_per_group_int4_sym": (_int, [_c_void_p, _int, _i64, _i64, _int, _c_void_p, _c_void_p, _c_void_p]),
+    "ttamd_quantize_per_group_int4": (
+        _int,
+        [_c_void_p, _int, _i64, _i64, _int, _c_void_p, _c_void_p, _c_void_p, _c_void_p],
+    ),
+}
+
+_lock = threading.Lock()
+_lib = None
+
+
+class LibraryNotBuiltError(RuntimeError):
+    pass
+
+
+def load() -> ctypes.CDLL:
+    """Load the shared library (once) and attach the prototypes.  Raises if it is missing or stale."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        if not LIB_PATH.exists():
+            raise LibraryNotBuiltError(
+                f"{LIB_PATH} is missing: torchtune_amd has no compute path without its HIP library. "
+                "Build it with `python -m torchtune_amd.build` (needs hipcc)."
+            )
+        lib = ctypes.CDLL(os.fspath(LIB_PATH))
+        for name, (restype, argtypes) in SIGNATURES.items():
+            try:
+                fn = getattr(lib, name)
+            except AttributeError as err:
+                raise LibraryNotBuiltError(f"{LIB_PATH} does not export {name}; rebuild it") from err
+            fn.restype = restype
+            fn.argtypes = argtypes
+        if lib.ttamd_version() != ABI_VERSION:
+            raise LibraryNotBuiltError(
+                f"{LIB_PATH} has ABI version {lib.ttamd_version()}, this package needs {ABI_VERSION}; rebuild it"
+            )
+        _lib = lib
+    return _lib
+
+
+def check(rc: int, what: str) -> None:
+    """Turn a negative C-ABI return code into the matching Python exception."""
+    if rc == 0:
+        return
+    msg = load().ttamd_last_error().decode("utf-8", "replace")
+    if rc == -1:
+        raise ValueError(f"{what}: {msg}")
+    raise RuntimeError(f"{what} failed (code {rc}): {msg}")

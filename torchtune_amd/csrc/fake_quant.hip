@@ -1,0 +1,349 @@
+// QAT fake-quantisation kernels for gfx950 (8da4w scheme): per-token asymmetric int8 for activations,
+// per-group symmetric int4 for weights, and the real int4 conversion.  All three are HBM-bound streaming
+// kernels: one read and one write of the tensor (4 B/element in bf16) plus the small qparam arrays.
+//
+// Reductions are wavefront reductions: a token row (or a weight group) lives in the registers of one
+// wave (or of g/8 neighbouring lanes) and min/max travel over cross-lane shuffles, so the data is read
+// from HBM exactly once.
+#include "common.h"
+#include "nf4_math.h"
+
+namespace ttamd {
+namespace {
+
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+constexpr float kF32Eps = 1.1920928955078125e-07f;  // torch.finfo(torch.float32).eps
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  bf16x2_t v;
+  v.x = (__bf16)lo;
+  v.y = (__bf16)hi;
+  return __builtin_bit_cast(uint32_t, v);
+}
+
+// Eight consecutive elements held in registers in their storage format.
+template <bool BF16>
+struct Chunk8;
+
+template <>
+struct Chunk8<true> {
+  u32x4_t raw;
+  __device__ __forceinline__ void load(const void* base, int64_t chunk) {
+    raw = reinterpret_cast<const u32x4_t*>(base)[chunk];
+  }
+  __device__ __forceinline__ void zero() { raw = u32x4_t{0, 0, 0, 0}; }
+  __device__ __forceinline__ float get(int i) const {
+    uint32_t d = raw[i >> 1];
+    return bits_f32((i & 1) ? (d & 0xffff0000u) : (d << 16));
+  }
+  static __device__ __forceinline__ void store(void* base, int64_t chunk, const float v[8]) {
+    u32x4_t o;
+    o.x = pack_bf16x2(v[0], v[1]);
+    o.y = pack_bf16x2(v[2], v[3]);
+    o.z = pack_bf16x2(v[4], v[5]);
+    o.w = pack_bf16x2(v[6], v[7]);
+    __builtin_nontemporal_store(o, reinterpret_cast<u32x4_t*>(base) + chunk);
+  }
+};
+
+template <>
+struct Chunk8<false> {
+  f32x4_t a, b;
+  __device__ __forceinline__ void load(const void* base, int64_t chunk) {
+    const f32x4_t* p = reinterpret_cast<const f32x4_t*>(base) + 2 * chunk;
+    a = p[0];
+    b = p[1];
+  }
+  __device__ __forceinline__ void zero() {
+    a = f32x4_t{0, 0, 0, 0};
+    b = a;
+  }
+  __device__ __forceinline__ float get(int i) const { return i < 4 ? a[i] : b[i - 4]; }
+  static __device__ __forceinline__ void store(void* base, int64_t chunk, const float v[8]) {
+    f32x4_t* p = reinterpret_cast<f32x4_t*>(base) + 2 * chunk;
+    f32x4_t lo = {v[0], v[1], v[2], v[3]}, hi = {v[4], v[5], v[6], v[7]};
+    __builtin_nontemporal_store(lo, p);
+    __builtin_nontemporal_store(hi, p + 1);
+  }
+};
+
+struct TokenQParams {
+  float scale, inv_scale, zp;
+};
+
+// asymmetric int8 qparams from the row extrema (already widened to include 0)
+__device__ __forceinline__ TokenQParams token_qparams(float mn, float mx) {
+  TokenQParams p;
+  float scale = (mx - mn) / 255.0f;
+  scale = scale > kF32Eps ? scale : kF32Eps;
+  const float dmin = mn / scale, dmax = mx / scale;
+  float zp = ((-128.0f + dmin) + (127.0f + dmax) > 0.0f) ? (-128.0f - dmin) : (127.0f - dmax);
+  zp = zp < -128.0f ? -128.0f : (zp > 127.0f ? 127.0f : zp);
+  p.zp = __builtin_rintf(zp);
+  p.scale = scale;
+  p.inv_scale = 1.0f / scale;
+  return p;
+}
+
+template <bool BF16>
+__device__ __forceinline__ float token_fq(float x, const TokenQParams& p) {
+  float q = __builtin_rintf(x * p.inv_scale) + p.zp;
+  q = q < -128.0f ? -128.0f : (q > 127.0f ? 127.0f : q);
+  return Arith<BF16>::rnd((q - p.zp) * p.scale);
+}
+
+__device__ __forceinline__ void wave_minmax(float& mn, float& mx) {
+#pragma unroll
+  for (int off = 1; off < kWave; off <<= 1) {
+    mn = fminf(mn, __shfl_xor(mn, off, kWave));
+    mx = fmaxf(mx, __shfl_xor(mx, off, kWave));
+  }
+}
+
+// One wave per token row, the whole row resident in registers: NV chunks of 8 elements per lane.
+template <bool BF16, int NV>
+__global__ __launch_bounds__(256) void fq_per_token_regs_kernel(const void* __restrict__ x, int64_t rows, int64_t K,
+                                                                void* __restrict__ out, float* __restrict__ scale_out,
+                                                                int32_t* __restrict__ zp_out) {
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int lane = threadIdx.x & 63;
+  const int chunks_per_row = (int)(K >> 3);
+  const int64_t row_chunk0 = row * chunks_per_row;
+  Chunk8<BF16> c[NV];
+  float mn = 0.f, mx = 0.f;  // the qparams use min(amin, 0) and max(amax, 0): zero is the neutral start
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int ch = i * kWave + lane;
+    if (ch < chunks_per_row)
+      c[i].load(x, row_chunk0 + ch);
+    else
+      c[i].zero();
+  }
+#pragma unroll
+  for (int i = 0; i < NV; ++i)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float v = c[i].get(e);
+      mn = fminf(mn, v);
+      mx = fmaxf(mx, v);
+    }
+  wave_minmax(mn, mx);
+  const TokenQParams p = token_qparams(mn, mx);
+  if (lane == 0) {
+    if (scale_out) scale_out[row] = p.scale;
+    if (zp_out) zp_out[row] = (int32_t)p.zp;
+  }
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int ch = i * kWave + lane;
+    if (ch < chunks_per_row) {
+      float v[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = token_fq<BF16>(c[i].get(e), p);
+      Chunk8<BF16>::store(out, row_chunk0 + ch, v);
+    }
+  }
+}
+
+// Rows too long for the register file: two passes over the row (the second one normally hits in L2).
+template <bool BF16>
+__global__ __launch_bounds__(256) void fq_per_token_stream_kernel(const void* __restrict__ x, int64_t rows, int64_t K,
+                                                                  void* __restrict__ out, float* __restrict__ scale_out,
+                                                                  int32_t* __restrict__ zp_out) {
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int lane = threadIdx.x & 63;
+  const int64_t chunks_per_row = K >> 3;
+  const int64_t row_chunk0 = row * chunks_per_row;
+  float mn = 0.f, mx = 0.f;
+  for (int64_t ch = lane; ch < chunks_per_row; ch += kWave) {
+    Chunk8<BF16> c;
+    c.load(x, row_chunk0 + ch);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float v = c.get(e);
+      mn = fminf(mn, v);
+      mx = fmaxf(mx, v);
+    }
+  }
+  wave_minmax(mn, mx);
+  const TokenQParams p = token_qparams(mn, mx);
+  if (lane == 0) {
+    if (scale_out) scale_out[row] = p.scale;
+    if (zp_out) zp_out[row] = (int32_t)p.zp;
+  }
+  for (int64_t ch = lane; ch < chunks_per_row; ch += kWave) {
+    Chunk8<BF16> c;
+    c.load(x, row_chunk0 + ch);
+    float v[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = token_fq<BF16>(c.get(e), p);
+    Chunk8<BF16>::store(out, row_chunk0 + ch, v);
+  }
+}
+
+// Per-group symmetric int4.  A group of g elements is held by g/8 neighbouring lanes.
+// EMIT_INT = false: write the fake-quantised tensor (training).  true: write int8-held int4 values (convert).
+constexpr int kGroupChunksPerThread = 4;
+
+template <bool BF16, bool EMIT_INT>
+__global__ __launch_bounds__(256) void fq_per_group_kernel(const void* __restrict__ w, int64_t n_chunks, int lanes_per_group,
+                                                           int log2_lpg, void* __restrict__ out_fq,
+                                                           int8_t* __restrict__ out_q, float* __restrict__ scale_out,
+                                                           float* __restrict__ zero_out) {
+  const int64_t base = (int64_t)blockIdx.x * (256 * kGroupChunksPerThread) + threadIdx.x;
+  Chunk8<BF16> c[kGroupChunksPerThread];
+#pragma unroll
+  for (int u = 0; u < kGroupChunksPerThread; ++u) {
+    const int64_t ch = base + u * 256;
+    if (ch < n_chunks)
+      c[u].load(w, ch);
+    else
+      c[u].zero();
+  }
+#pragma unroll
+  for (int u = 0; u < kGroupChunksPerThread; ++u) {
+    const int64_t ch = base + u * 256;
+    float mn = 0.f, mx = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float v = c[u].get(e);
+      mn = fminf(mn, v);
+      mx = fmaxf(mx, v);
+    }
+    for (int off = 1; off < lanes_per_group; off <<= 1) {
+      mn = fminf(mn, __shfl_xor(mn, off, kWave));
+      mx = fmaxf(mx, __shfl_xor(mx, off, kWave));
+    }
+    if (ch >= n_chunks) continue;
+    const float amax = fmaxf(-mn, mx);
+    float scale = amax / 7.5f;
+    scale = scale > kF32Eps ? scale : kF32Eps;
+    const float inv = 1.0f / scale;
+    if ((threadIdx.x & (lanes_per_group - 1)) == 0) {
+      if (scale_out) scale_out[ch >> log2_lpg] = scale;
+      if (zero_out) zero_out[ch >> log2_lpg] = 0.0f;
+    }
+    float q[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      float t = __builtin_rintf(c[u].get(e) * inv);
+      t = t < -8.0f ? -8.0f : (t > 7.0f ? 7.0f : t);
+      q[e] = (float)(int)t;  // through the integer grid: rint(-0.3) = -0.0 must dequantise to +0.0
+    }
+    if constexpr (EMIT_INT) {
+      uint32_t lo = 0, hi = 0;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        lo |= ((uint32_t)(int)q[e] & 0xffu) << (8 * e);
+        hi |= ((uint32_t)(int)q[e + 4] & 0xffu) << (8 * e);
+      }
+      reinterpret_cast<uint2*>(out_q)[ch] = make_uint2(lo, hi);
+    } else {
+      float v[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = Arith<BF16>::rnd(q[e] * scale);
+      Chunk8<BF16>::store(out_fq, ch, v);
+    }
+  }
+}
+
+int log2_exact(int64_t v) {
+  int l = 0;
+  while ((int64_t(1) << l) < v) ++l;
+  return l;
+}
+
+template <bool BF16>
+int launch_per_token(const void* x, int64_t rows, int64_t K, void* out, float* scale, int32_t* zp, hipStream_t s) {
+  const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
+  const int64_t nv = (K / 8 + kWave - 1) / kWave;
+  constexpr int kMaxRegChunks = BF16 ? 32 : 16;
+#define TT_LAUNCH_TOKEN(NV)                                                                          \
+  if (nv <= NV) {                                                                                    \
+    fq_per_token_regs_kernel<BF16, NV><<<grid, block, 0, s>>>(x, rows, K, out, scale, zp);           \
+    return check_launch("fq_per_token_int8_asym");                                                   \
+  }
+  TT_LAUNCH_TOKEN(1)
+  TT_LAUNCH_TOKEN(2)
+  TT_LAUNCH_TOKEN(4)
+  TT_LAUNCH_TOKEN(8)
+  TT_LAUNCH_TOKEN(16)
+  if constexpr (kMaxRegChunks >= 32) {
+    TT_LAUNCH_TOKEN(32)
+  }
+#undef TT_LAUNCH_TOKEN
+  fq_per_token_stream_kernel<BF16><<<grid, block, 0, s>>>(x, rows, K, out, scale, zp);
+  return check_launch("fq_per_token_int8_asym");
+}
+
+int check_group_args(const void* w, int dtype, int64_t rows, int64_t K, int group_size) {
+  TT_REQUIRE(dtype == TTAMD_BF16 || dtype == TTAMD_F32, "fake_quant: unknown dtype code %d", dtype);
+  TT_REQUIRE(w != nullptr && aligned16(w), "fake_quant: input must be a non-null 16-byte aligned pointer");
+  TT_REQUIRE(rows > 0 && K > 0, "fake_quant: rows and K must be positive");
+  TT_REQUIRE(group_size >= 8 && group_size <= 512 && is_pow2(group_size),
+             "fake_quant: group_size must be a power of two in [8, 512] (got %d)", group_size);
+  TT_REQUIRE(K % group_size == 0, "fake_quant: K (%lld) must be divisible by group_size (%d)", (long long)K,
+             group_size);
+  return TTAMD_OK;
+}
+
+}  // namespace
+}  // namespace ttamd
+
+using namespace ttamd;
+
+extern "C" int ttamd_fq_per_token_int8_asym(const void* x, int dtype, int64_t rows, int64_t K, void* out, float* scale,
+                                            int32_t* zero_point, void* stream) {
+  TT_REQUIRE(dtype == TTAMD_BF16 || dtype == TTAMD_F32, "fq_per_token: unknown dtype code %d", dtype);
+  TT_REQUIRE(x && out && aligned16(x) && aligned16(out), "fq_per_token: x/out must be non-null, 16-byte aligned");
+  TT_REQUIRE(rows > 0 && K > 0 && K % 8 == 0, "fq_per_token: K (%lld) must be a positive multiple of 8",
+             (long long)K);
+  TT_REQUIRE((rows + 3) / 4 < (int64_t(1) << 31), "fq_per_token: too many rows for one launch");
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  return dtype == TTAMD_BF16 ? launch_per_token<true>(x, rows, K, out, scale, zero_point, s)
+                             : launch_per_token<false>(x, rows, K, out, scale, zero_point, s);
+}
+
+extern "C" int ttamd_fq_per_group_int4_sym(const void* w, int dtype, int64_t rows, int64_t K, int group_size, void* out,
+                                           float* scale, void* stream) {
+  if (int rc = check_group_args(w, dtype, rows, K, group_size)) return rc;
+  TT_REQUIRE(out && aligned16(out), "fq_per_group: out must be non-null, 16-byte aligned");
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const int64_t n_chunks = rows * K / 8;
+  const int64_t per_wg = 256 * kGroupChunksPerThread;
+  const int64_t grid = (n_chunks + per_wg - 1) / per_wg;
+  TT_REQUIRE(grid < (int64_t(1) << 31), "fq_per_group: tensor too large for one launch");
+  const int lpg = group_size / 8;
+  if (dtype == TTAMD_BF16)
+    fq_per_group_kernel<true, false><<<dim3((unsigned)grid), dim3(256), 0, s>>>(w, n_chunks, lpg, log2_exact(lpg), out,
+                                                                                 nullptr, scale, nullptr);
+  else
+    fq_per_group_kernel<false, false><<<dim3((unsigned)grid), dim3(256), 0, s>>>(w, n_chunks, lpg, log2_exact(lpg), out,
+                                                                                  nullptr, scale, nullptr);
+  return check_launch("fq_per_group_int4_sym");
+}
+
+extern "C" int ttamd_quantize_per_group_int4(const void* w, int dtype, int64_t rows, int64_t K, int group_size, int8_t* q,
+                                             float* scale, float* zero_point, void* stream) {
+  if (int rc = check_group_args(w, dtype, rows, K, group_size)) return rc;
+  TT_REQUIRE(q && scale && (reinterpret_cast<uintptr_t>(q) & 7u) == 0,
+             "quantize_per_group_int4: q (8-byte aligned) and scale must be non-null");
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const int64_t n_chunks = rows * K / 8;
+  const int64_t per_wg = 256 * kGroupChunksPerThread;
+  const int64_t grid = (n_chunks + per_wg - 1) / per_wg;
+  TT_REQUIRE(grid < (int64_t(1) << 31), "quantize_per_group_int4: tensor too large for one launch");
+  const int lpg = group_size / 8;
+  if (dtype == TTAMD_BF16)
+    fq_per_group_kernel<true, true><<<dim3((unsigned)grid), dim3(256), 0, s>>>(w, n_chunks, lpg, log2_exact(lpg), nullptr,
+                                                                                q, scale, zero_point);
+  else
+    fq_per_group_kernel<false, true><<<dim3((unsigned)grid), dim3(256), 0, s>>>(w, n_chunks, lpg, log2_exact(lpg), nullptr,
+                                                                                 q, scale, zero_point);
+  return check_launch("quantize_per_group_int4");
+}

@@ -1,0 +1,11 @@
+from ._utils import AdapterModule, get_adapter_params, set_trainable_params
+from .lora import LoRALinear, QATLoRALinear, TrainableParams
+
+__all__ = [
+    "AdapterModule",
+    "LoRALinear",
+    "QATLoRALinear",
+    "TrainableParams",
+    "get_adapter_params",
+    "set_trainable_params",
+]

@@ -1,0 +1,256 @@
+"""``LoRALinear`` / ``QATLoRALinear`` with the QLoRA case running on fused HIP kernels.
+
+Drop-in for ``torchtune.modules.peft.LoRALinear`` (``torchtune/modules/peft/lora.py:27-147``) and
+``QATLoRALinear`` (``:150-306``): same constructor arguments, attributes (``in_dim, out_dim, rank, alpha,
+use_bias, _quantize_base, disabled, merged, weight, bias, dropout, lora_a, lora_b``), parameter names,
+initialisation and error messages.
+
+With ``quantize_base=True``, bf16 activations on the GPU and a rank that is a multiple of 8, the whole layer
+
+    y = x . D(W)^T (+ bias) + (alpha / rank) . (x . A^T) . B^T
+
+is one autograd node: the adapter's hidden activation comes from a skinny MFMA kernel, everything else from
+one GEMM that dequantises NF4 into LDS and folds the adapter in as extra contraction steps; the backward
+mirrors it (``gx`` from one fused GEMM, ``gA``/``gB`` from two streaming reductions).  Only the packed weight,
+``x`` and the [M, rank] hidden activation are kept for backward.  Other cases (fp32, odd ranks, other NF4
+block sizes, adapter dropout in training) compose the same result from ``linear_nf4`` and ``F.linear``.
+"""
+from __future__ import annotations
+
+import math
+from enum import Enum
+from typing import List, Optional, Union
+
+import torch
+import torch.nn.functional as F
+from torch import nn
+
+from ... import ops
+from ...nf4_tensor import NF4Tensor, _fused_ok, linear_nf4, to_nf4
+from ..low_precision import _register_nf4_dispatch_ops  # noqa: F401  (clone override must be active)
+
+
+class TrainableParams(Enum):
+    FULL = "full"
+    LORA = "lora"
+    FROZEN = "frozen"
+
+
+class _QLoRALinearFn(torch.autograd.Function):
+    """Fused QLoRA linear.  Inputs: x [..., K] bf16, NF4 weight [N, K], lora_a [r, K], lora_b [N, r], bias or None."""
+
+    @staticmethod
+    def forward(ctx, x, weight, lora_a, lora_b, bias, scale: float):
+        N, K = weight.shape
+        x2 = x.reshape(-1, K)
+        h = ops.lora_hidden(x2, lora_a)
+        y = ops.nf4_lora_linear_fwd(x2, weight.quantized_data, weight.block_scalers(), N, h, lora_b, scale, bias)
+        ctx.save_for_backward(x2, h, weight, lora_a, lora_b)
+        ctx.scale = scale
+        ctx.x_shape = x.shape
+        ctx.has_bias = bias is not None
+        return y.view(*x.shape[:-1], N)
+
+    @staticmethod
+    def backward(ctx, gy):
+        x2, h, weight, lora_a, lora_b = ctx.saved_tensors
+        N, K = weight.shape
+        gy2 = gy.reshape(-1, N)
+        need_x, _, need_a, need_b, need_bias, _ = ctx.needs_input_grad
+        gx = ga = gb = gbias = None
+        if need_x or need_a or need_b:
+            gh, ga, gb = ops.lora_bwd(gy2, x2, h, lora_b, ctx.scale)
+            if need_x:
+                gx = ops.nf4_linear_bwd_dx(gy2, weight.quantized_data, weight.block_scalers(), K, gh, lora_a)
+                gx = gx.view(ctx.x_shape)
+            if not need_a:
+                ga = None
+            if not need_b:
+                gb = None
+        if ctx.has_bias and need_bias:
+            gbias = gy2.sum(dim=0)
+        return gx, None, ga, gb, gbias, None
+
+
+class LoRALinear(nn.Module):
+    """Linear layer with a low-rank adapter: ``x -> W0 x + (alpha / r) B A x``.
+
+    Args:
+        in_dim (int): input dimension
+        out_dim (int): output dimension
+        rank (int): rank of the adapter
+        alpha (float): adapter scaling numerator
+        dropout (float): dropout on the adapter's input. Default 0.0
+        use_bias (bool): whether the base linear has a bias. Default False
+        quantize_base (bool): hold the base weight as NF4. Default False
+        **quantization_kwargs: forwarded to ``to_nf4`` (``block_size``, ``scaler_block_size``); only valid
+            with ``quantize_base=True``
+
+    Raises:
+        ValueError: if quantisation arguments are given while ``quantize_base`` is False
+    """
+
+    def __init__(
+        self,
+        in_dim: int,
+        out_dim: int,
+        rank: int,
+        alpha: float,
+        dropout: float = 0.0,
+        use_bias: bool = False,
+        quantize_base: bool = False,
+        **quantization_kwargs,
+    ):
+        super().__init__()
+        self.in_dim = in_dim
+        self.out_dim = out_dim
+        self.rank = rank
+        self.alpha = alpha
+        self.use_bias = use_bias
+        self._quantize_base = quantize_base
+
+        if not quantize_base and any(v for v in quantization_kwargs.values()):
+            raise ValueError(
+                f"``quantize_base`` is False, but received the following quantization arguments: {quantization_kwargs}"
+            )
+
+        base = nn.Linear(in_features=in_dim, out_features=out_dim, bias=use_bias)
+        weight = to_nf4(base.weight, **quantization_kwargs) if quantize_base else base.weight
+        self.disabled = False  # True: act as the frozen base layer only (reference policy in DPO)
+        self.register_parameter("weight", nn.Parameter(weight))
+        self.register_parameter("bias", nn.Parameter(base.bias) if use_bias else None)
+        self.dropout = nn.Dropout(p=dropout) if dropout > 0.0 else nn.Identity()
+        self.lora_a = nn.Linear(in_features=in_dim, out_features=rank, bias=False)
+        self.lora_b = nn.Linear(in_features=rank, out_features=out_dim, bias=False)
+        self.merged = False
+        self.initialize_parameters()
+
+    def to_empty(self, *, device: Optional[Union[str, torch.device, int]], recurse: bool = True):
+        self.lora_a.to_empty(device=device, recurse=recurse)
+        self.lora_b.to_empty(device=device, recurse=recurse)
+
+    def initialize_parameters(self):
+        _lora_a_init_params(self.lora_a)
+        _lora_b_init_params(self.lora_b)
+
+    def adapter_params(self) -> List[str]:
+        """Names of this module's adapter parameters."""
+        return ["lora_a.weight", "lora_b.weight"]
+
+    def _fused(self, x: torch.Tensor) -> bool:
+        dropping = self.training and isinstance(self.dropout, nn.Dropout) and self.dropout.p > 0.0
+        return (
+            self._quantize_base
+            and not dropping
+            and self.rank > 0
+            and isinstance(self.weight, NF4Tensor)
+            and _fused_ok(x, self.weight, self.rank)
+            and self.lora_a.weight.dtype == torch.bfloat16
+            and self.lora_b.weight.dtype == torch.bfloat16
+            and (self.bias is None or self.bias.dtype == torch.bfloat16)
+        )
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        """x ``(..., in_dim)`` -> ``(..., out_dim)``"""
+        if not self.disabled and self._fused(x):
+            return _QLoRALinearFn.apply(
+                x, self.weight, self.lora_a.weight, self.lora_b.weight, self.bias, self.alpha / self.rank
+            )
+        if self._quantize_base:
+            out = linear_nf4(input=x, weight=self.weight)
+            if self.use_bias:
+                out = out + self.bias
+        else:
+            out = F.linear(x, self.weight, self.bias)
+        if self.disabled:
+            return out
+        lora_out = self.lora_a(self.dropout(x))
+        lora_out = (self.alpha / self.rank) * self.lora_b(lora_out)
+        return out + lora_out
+
+
+class QATLoRALinear(LoRALinear):
+    """LoRA linear whose frozen base path sees fake-quantised activations and weights:
+    ``x -> fq(W) fq(x) + (alpha / r) B A x``.
+
+    Args:
+        in_dim, out_dim, rank, alpha, dropout: as for :class:`LoRALinear`
+        activation_qat_config (Optional[FakeQuantizeConfig]): how to fake-quantise the input; None = identity
+        weight_qat_config (Optional[FakeQuantizeConfig]): how to fake-quantise the base weight; None = identity
+
+    Raises:
+        ValueError: if ``in_dim`` is not divisible by the weight ``group_size``
+    """
+
+    def __init__(
+        self,
+        in_dim: int,
+        out_dim: int,
+        rank: int,
+        alpha: float,
+        dropout: float = 0.0,
+        activation_qat_config: Optional["FakeQuantizeConfig"] = None,  # noqa: F821
+        weight_qat_config: Optional["FakeQuantizeConfig"] = None,  # noqa: F821
+    ):
+        super().__init__(in_dim, out_dim, rank, alpha, dropout, use_bias=False, quantize_base=False)
+        from ...qat import FakeQuantizeConfig, FakeQuantizer
+
+        if activation_qat_config is not None:
+            assert isinstance(activation_qat_config, FakeQuantizeConfig)
+            self.activation_fake_quantizer = FakeQuantizer(activation_qat_config)
+        else:
+            self.activation_fake_quantizer = nn.Identity()
+
+        if weight_qat_config is not None:
+            assert isinstance(weight_qat_config, FakeQuantizeConfig)
+            group_size = weight_qat_config.group_size
+            if group_size is not None and in_dim % group_size != 0:
+                raise ValueError("in_dim (%s) must be divisible by group_size (%s)" % (in_dim, group_size))
+            self.weight_fake_quantizer = FakeQuantizer(weight_qat_config)
+        else:
+            self.weight_fake_quantizer = nn.Identity()
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        out = F.linear(self.activation_fake_quantizer(x), self.weight_fake_quantizer(self.weight))
+        if self.disabled:
+            return out
+        lora_out = self.lora_a(self.dropout(x))
+        lora_out = (self.alpha / self.rank) * self.lora_b(lora_out)
+        return out + lora_out
+
+    @classmethod
+    def from_lora_linear(
+        cls,
+        lora_linear: LoRALinear,
+        activation_qat_config: Optional["FakeQuantizeConfig"] = None,  # noqa: F821
+        weight_qat_config: Optional["FakeQuantizeConfig"] = None,  # noqa: F821
+    ) -> "QATLoRALinear":
+        """Build a ``QATLoRALinear`` that shares the weights and adapters of ``lora_linear``."""
+        if lora_linear.bias is not None:
+            raise ValueError("Bias is not supported in QAT + LoRA yet")
+        if lora_linear._quantize_base:
+            raise ValueError("quantize_base is not compatible with QAT + LoRA")
+        p = lora_linear.dropout.p if isinstance(lora_linear.dropout, nn.Dropout) else 0.0
+        new = cls(
+            lora_linear.in_dim, lora_linear.out_dim, lora_linear.rank, lora_linear.alpha, p, activation_qat_config,
+            weight_qat_config,
+        )
+        meta = torch.device("meta")
+        # a meta-device source has no values to share (distributed construction)
+        if lora_linear.weight.device != meta:
+            new.weight = lora_linear.weight
+        if lora_linear.lora_a.weight.device != meta:
+            new.lora_a.weight = lora_linear.lora_a.weight
+        if lora_linear.lora_b.weight.device != meta:
+            new.lora_b.weight = lora_linear.lora_b.weight
+        return new
+
+
+def _lora_a_init_params(x: nn.Linear) -> None:
+    """Kaiming-uniform, a = sqrt(5)."""
+    nn.init.kaiming_uniform_(x.weight, a=math.sqrt(5))
+
+
+def _lora_b_init_params(x: nn.Linear) -> None:
+    """Zeros: the adapter starts as a no-op."""
+    nn.init.zeros_(x.weight)

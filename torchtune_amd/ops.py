@@ -1,0 +1,269 @@
+"""Tensor-level wrappers over the C ABI: validate, allocate outputs, pass raw device pointers and the
+caller's current HIP stream.  PyTorch is used here for device memory and streams only.
+
+Every function requires HIP (``cuda``) tensors.  There is no CPU implementation in this package.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+
+_DTYPE_CODE = {torch.bfloat16: _lib.TTAMD_BF16, torch.float32: _lib.TTAMD_F32}
+
+
+def _code(dtype: torch.dtype, what: str) -> int:
+    try:
+        return _DTYPE_CODE[dtype]
+    except KeyError:
+        raise TypeError(f"{what}: dtype {dtype} is not supported (bfloat16 and float32 are)") from None
+
+
+def _need_gpu(t: torch.Tensor, what: str) -> None:
+    if not t.is_cuda:
+        raise RuntimeError(
+            f"{what}: expected a tensor on an AMD GPU (device 'cuda'), got device '{t.device}'. "
+            "torchtune_amd computes only through its HIP kernels."
+        )
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _workspace(nbytes: int, device: torch.device) -> torch.Tensor:
+    return torch.empty(max(int(nbytes), 16), dtype=torch.uint8, device=device)
+
+
+# ---------------------------------------------------------------------------------------------------
+# NF4 codec
+# ---------------------------------------------------------------------------------------------------
+def nf4_quantize(w: torch.Tensor, block_size: int, scaler_block_size: int):
+    """-> (quantized_data u8 [numel/2], quantized_scalers i8 [n_blocks], quantization_factor dtype [n_sb],
+    scaler_mean dtype 0-dim)"""
+    _need_gpu(w, "nf4_quantize")
+    code = _code(w.dtype, "nf4_quantize")
+    w = w.detach().contiguous()
+    numel = w.numel()
+    if block_size <= 0 or numel % block_size != 0:
+        raise ValueError(f"nf4_quantize: numel ({numel}) must be divisible by block_size ({block_size})")
+    n_blocks = numel // block_size
+    if scaler_block_size <= 0 or n_blocks % scaler_block_size != 0:
+        raise ValueError(
+            f"nf4_quantize: number of blocks ({n_blocks}) must be divisible by scaler_block_size ({scaler_block_size})"
+        )
+    lib = _lib.load()
+    dev = w.device
+    qdata = torch.empty(numel // 2, dtype=torch.uint8, device=dev)
+    qscalers = torch.empty(n_blocks, dtype=torch.int8, device=dev)
+    qfactor = torch.empty(n_blocks // scaler_block_size, dtype=w.dtype, device=dev)
+    mean = torch.empty((), dtype=w.dtype, device=dev)
+    ws_bytes = lib.ttamd_nf4_quantize_workspace_bytes(numel, block_size)
+    ws = _workspace(ws_bytes, dev)
+    with torch.cuda.device(dev):
+        rc = lib.ttamd_nf4_quantize(
+            w.data_ptr(), code, numel, block_size, scaler_block_size, qdata.data_ptr(), qscalers.data_ptr(),
+            qfactor.data_ptr(), mean.data_ptr(), ws.data_ptr(), ws.numel(), _stream(w),
+        )
+    _lib.check(rc, "nf4_quantize")
+    return qdata, qscalers, qfactor, mean
+
+
+def nf4_dequantize(
+    qdata: torch.Tensor, qscalers: torch.Tensor, qfactor: torch.Tensor, mean: torch.Tensor, shape, block_size: int,
+    scaler_block_size: int,
+) -> torch.Tensor:
+    _need_gpu(qdata, "nf4_dequantize")
+    dtype = qfactor.dtype
+    code = _code(dtype, "nf4_dequantize")
+    numel = qdata.numel() * 2
+    out = torch.empty(numel, dtype=dtype, device=qdata.device)
+    lib = _lib.load()
+    with torch.cuda.device(qdata.device):
+        rc = lib.ttamd_nf4_dequantize(
+            qdata.data_ptr(), qscalers.data_ptr(), qfactor.data_ptr(), mean.data_ptr(), code, numel, block_size,
+            scaler_block_size, out.data_ptr(), _stream(qdata),
+        )
+    _lib.check(rc, "nf4_dequantize")
+    return out.view(shape)
+
+
+def nf4_block_scalers(qscalers: torch.Tensor, qfactor: torch.Tensor, mean: torch.Tensor, scaler_block_size: int) -> torch.Tensor:
+    _need_gpu(qscalers, "nf4_block_scalers")
+    code = _code(qfactor.dtype, "nf4_block_scalers")
+    out = torch.empty(qscalers.numel(), dtype=torch.bfloat16, device=qscalers.device)
+    lib = _lib.load()
+    with torch.cuda.device(qscalers.device):
+        rc = lib.ttamd_nf4_block_scalers(
+            qscalers.data_ptr(), qfactor.data_ptr(), mean.data_ptr(), code, qscalers.numel(), scaler_block_size,
+            out.data_ptr(), _stream(qscalers),
+        )
+    _lib.check(rc, "nf4_block_scalers")
+    return out
+
+
+# ---------------------------------------------------------------------------------------------------
+# fused NF4 + LoRA linear
+# ---------------------------------------------------------------------------------------------------
+def fused_shape_ok(N: int, K: int, rank: int) -> bool:
+    """Shapes the fused bf16 GEMM accepts (NF4 block_size must also be 64)."""
+    return K % 64 == 0 and N % 64 == 0 and rank % 8 == 0 and 0 <= rank <= 64
+
+
+def _bf16_2d(t: torch.Tensor, what: str) -> torch.Tensor:
+    _need_gpu(t, what)
+    if t.dtype != torch.bfloat16 or t.dim() != 2:
+        raise TypeError(f"{what}: expected a 2-D bfloat16 tensor, got {tuple(t.shape)} {t.dtype}")
+    return t.contiguous()
+
+
+def lora_hidden(x: torch.Tensor, lora_a: torch.Tensor) -> torch.Tensor:
+    """h = bf16(x @ lora_a.T);  x [M,K], lora_a [r,K] -> [M,r]"""
+    x = _bf16_2d(x, "lora_hidden")
+    lora_a = _bf16_2d(lora_a, "lora_hidden")
+    M, K = x.shape
+    r = lora_a.shape[0]
+    lib = _lib.load()
+    h = torch.empty(M, r, dtype=torch.bfloat16, device=x.device)
+    ws = _workspace(lib.ttamd_lora_fwd_workspace_bytes(M, K, r), x.device)
+    with torch.cuda.device(x.device):
+        rc = lib.ttamd_lora_hidden_bf16(x.data_ptr(), lora_a.data_ptr(), h.data_ptr(), M, K, r, ws.data_ptr(), ws.numel(),
+                                        _stream(x))
+    _lib.check(rc, "lora_hidden")
+    return h
+
+
+def nf4_lora_linear_fwd(
+    x: torch.Tensor, qdata: torch.Tensor, block_scalers: torch.Tensor, N: int, h: Optional[torch.Tensor] = None,
+    lora_b: Optional[torch.Tensor] = None, scale: float = 0.0, bias: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """y = x @ D(W).T (+bias) + scale * h @ lora_b.T ;  x [M,K] -> [M,N]"""
+    x = _bf16_2d(x, "nf4_lora_linear_fwd")
+    M, K = x.shape
+    rank = 0
+    if h is not None:
+        h = _bf16_2d(h, "nf4_lora_linear_fwd")
+        lora_b = _bf16_2d(lora_b, "nf4_lora_linear_fwd")
+        rank = h.shape[1]
+    if bias is not None:
+        bias = bias.contiguous()
+        if bias.dtype != torch.bfloat16:
+            raise TypeError("nf4_lora_linear_fwd: bias must be bfloat16")
+    y = torch.empty(M, N, dtype=torch.bfloat16, device=x.device)
+    lib = _lib.load()
+    with torch.cuda.device(x.device):
+        rc = lib.ttamd_nf4_lora_linear_fwd_bf16(
+            x.data_ptr(), qdata.data_ptr(), block_scalers.data_ptr(), _ptr(h), _ptr(lora_b), rank, float(scale), _ptr(bias),
+            y.data_ptr(), M, N, K, _stream(x),
+        )
+    _lib.check(rc, "nf4_lora_linear_fwd")
+    return y
+
+
+def nf4_linear_bwd_dx(
+    gy: torch.Tensor, qdata: torch.Tensor, block_scalers: torch.Tensor, K: int, gh: Optional[torch.Tensor] = None,
+    lora_a: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """gx = gy @ D(W) + gh @ lora_a ;  gy [M,N] -> [M,K]"""
+    gy = _bf16_2d(gy, "nf4_linear_bwd_dx")
+    M, N = gy.shape
+    rank = 0
+    if gh is not None:
+        gh = _bf16_2d(gh, "nf4_linear_bwd_dx")
+        lora_a = _bf16_2d(lora_a, "nf4_linear_bwd_dx")
+        rank = gh.shape[1]
+    gx = torch.empty(M, K, dtype=torch.bfloat16, device=gy.device)
+    lib = _lib.load()
+    with torch.cuda.device(gy.device):
+        rc = lib.ttamd_nf4_linear_bwd_dx_bf16(
+            gy.data_ptr(), qdata.data_ptr(), block_scalers.data_ptr(), _ptr(gh), _ptr(lora_a), rank, gx.data_ptr(), M, N, K,
+            _stream(gy),
+        )
+    _lib.check(rc, "nf4_linear_bwd_dx")
+    return gx
+
+
+def lora_bwd(
+    gy: torch.Tensor, x: torch.Tensor, h: torch.Tensor, lora_b: torch.Tensor, scale: float
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """-> (gh [M,r], gA [r,K], gB [N,r])"""
+    gy = _bf16_2d(gy, "lora_bwd")
+    x = _bf16_2d(x, "lora_bwd")
+    h = _bf16_2d(h, "lora_bwd")
+    lora_b = _bf16_2d(lora_b, "lora_bwd")
+    M, N = gy.shape
+    K = x.shape[1]
+    r = h.shape[1]
+    dev = gy.device
+    gh = torch.empty(M, r, dtype=torch.bfloat16, device=dev)
+    ga = torch.empty(r, K, dtype=torch.bfloat16, device=dev)
+    gb = torch.empty(N, r, dtype=torch.bfloat16, device=dev)
+    lib = _lib.load()
+    ws = _workspace(lib.ttamd_lora_bwd_workspace_bytes(M, N, K, r), dev)
+    with torch.cuda.device(dev):
+        rc = lib.ttamd_lora_bwd_bf16(
+            gy.data_ptr(), x.data_ptr(), h.data_ptr(), lora_b.data_ptr(), float(scale), gh.data_ptr(), ga.data_ptr(),
+            gb.data_ptr(), M, N, K, r, ws.data_ptr(), ws.numel(), _stream(gy),
+        )
+    _lib.check(rc, "lora_bwd")
+    return gh, ga, gb
+
+
+# ---------------------------------------------------------------------------------------------------
+# QAT fake quantisation
+# ---------------------------------------------------------------------------------------------------
+def fq_per_token_int8_asym(x: torch.Tensor, want_qparams: bool = True):
+    """x [..., K] -> (fake-quantised x, scale fp32 [rows] | None, zero_point int32 [rows] | None)"""
+    _need_gpu(x, "fq_per_token_int8_asym")
+    code = _code(x.dtype, "fq_per_token_int8_asym")
+    xc = x.contiguous()
+    K = xc.shape[-1]
+    rows = xc.numel() // K
+    out = torch.empty_like(xc)
+    scale = torch.empty(rows, dtype=torch.float32, device=x.device) if want_qparams else None
+    zp = torch.empty(rows, dtype=torch.int32, device=x.device) if want_qparams else None
+    lib = _lib.load()
+    with torch.cuda.device(x.device):
+        rc = lib.ttamd_fq_per_token_int8_asym(xc.data_ptr(), code, rows, K, out.data_ptr(), _ptr(scale), _ptr(zp), _stream(x))
+    _lib.check(rc, "fq_per_token_int8_asym")
+    return out, scale, zp
+
+
+def fq_per_group_int4_sym(w: torch.Tensor, group_size: int, want_scale: bool = True):
+    """w [..., K] -> (fake-quantised w, scale fp32 [rows, K/g] | None)"""
+    _need_gpu(w, "fq_per_group_int4_sym")
+    code = _code(w.dtype, "fq_per_group_int4_sym")
+    wc = w.contiguous()
+    K = wc.shape[-1]
+    rows = wc.numel() // K
+    out = torch.empty_like(wc)
+    scale = torch.empty(rows, K // max(group_size, 1), dtype=torch.float32, device=w.device) if want_scale else None
+    lib = _lib.load()
+    with torch.cuda.device(w.device):
+        rc = lib.ttamd_fq_per_group_int4_sym(wc.data_ptr(), code, rows, K, group_size, out.data_ptr(), _ptr(scale), _stream(w))
+    _lib.check(rc, "fq_per_group_int4_sym")
+    return out, scale
+
+
+def quantize_per_group_int4(w: torch.Tensor, group_size: int):
+    """w [rows, K] -> (int8 tensor of int4 values, scale fp32 [rows, K/g], zeros fp32 [rows, K/g])"""
+    _need_gpu(w, "quantize_per_group_int4")
+    code = _code(w.dtype, "quantize_per_group_int4")
+    wc = w.contiguous()
+    K = wc.shape[-1]
+    rows = wc.numel() // K
+    q = torch.empty(wc.shape, dtype=torch.int8, device=w.device)
+    scale = torch.empty(rows, K // max(group_size, 1), dtype=torch.float32, device=w.device)
+    zeros = torch.empty_like(scale)
+    lib = _lib.load()
+    with torch.cuda.device(w.device):
+        rc = lib.ttamd_quantize_per_group_int4(wc.data_ptr(), code, rows, K, group_size, q.data_ptr(), scale.data_ptr(),
+                                               zeros.data_ptr(), _stream(w))
+    _lib.check(rc, "quantize_per_group_int4")
+    return q, scale, zeros

@@ -1,0 +1,341 @@
+"""Quantisation-aware training for the 8da4w scheme (int8 dynamic per-token activations, int4 per-group
+symmetric weights) on the HIP fake-quant kernels.
+
+The reference obtains all of this from ``torchao.quantization.qat``:
+
+* ``Int8DynActInt4WeightQATQuantizer`` — re-exported at ``torchtune/training/quantization.py:26-29`` and
+  instantiated from YAML by ``recipes/qat_single_device.py:375-386`` (``prepare``) and ``recipes/quantize.py:88-95``
+  (``convert``);
+* ``FakeQuantizeConfig`` / ``FakeQuantizer`` — used directly by ``QATLoRALinear``
+  (``torchtune/modules/peft/lora.py:222-250``);
+* ``FakeQuantizedLinear`` — what ``_enable_linear_fake_quant`` toggles
+  (``torchtune/training/quantization.py:56-71``).
+
+The same names and call signatures are provided here.  Only the two schemes named above have kernels;
+any other configuration raises ``NotImplementedError`` instead of silently computing something else.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Optional, Union
+
+import torch
+import torch.nn.functional as F
+from torch import nn
+
+from . import ops
+
+
+@dataclass
+class PerToken:
+    """One set of qparams per row of the last dimension."""
+
+
+@dataclass
+class PerGroup:
+    """One set of qparams per ``group_size`` consecutive elements of the last dimension."""
+
+    group_size: int
+
+
+class FakeQuantizeConfig:
+    """How a tensor is fake-quantised.
+
+    Args:
+        dtype: ``torch.int8`` (activations) or ``torch.int4`` (weights)
+        granularity: ``"per_token"``, ``"per_group"``, a ``PerToken()`` or a ``PerGroup(n)``
+        group_size: keyword shortcut for ``PerGroup(group_size)``
+        is_symmetric: symmetric (zero-point 0) or asymmetric mapping
+        scale_precision, zero_point_precision: dtypes of the qparams kept on the quantizer
+        is_dynamic: qparams are recomputed from each input (the only supported mode)
+    """
+
+    def __init__(
+        self,
+        dtype: torch.dtype,
+        granularity: Union[str, PerToken, PerGroup, None] = None,
+        mapping_type: Optional[str] = None,
+        scale_precision: torch.dtype = torch.float32,
+        zero_point_precision: torch.dtype = torch.int32,
+        is_dynamic: bool = True,
+        *,
+        group_size: Optional[int] = None,
+        is_symmetric: Optional[bool] = None,
+    ):
+        if dtype not in (torch.int8, torch.int4):
+            raise NotImplementedError(f"FakeQuantizeConfig: dtype {dtype} has no kernel (int8 and int4 do)")
+        self.dtype = dtype
+        if granularity is not None and group_size is not None:
+            raise ValueError("Cannot set both `granularity` and `group_size`")
+        if isinstance(granularity, str):
+            if granularity == "per_token":
+                granularity = PerToken()
+            elif granularity == "per_group":
+                if group_size is None:
+                    raise ValueError("Granularity was 'per_group' but no `group_size` was set")
+                granularity = PerGroup(group_size)
+            else:
+                raise ValueError(f"Unexpected granularity: '{granularity}'; expected 'per_token' or 'per_group'")
+        elif granularity is None:
+            if group_size is None:
+                raise ValueError("At least one of `granularity` or `group_size` must be set")
+            granularity = PerGroup(group_size)
+        if not isinstance(granularity, (PerToken, PerGroup)):
+            raise ValueError(f"Granularity '{granularity}' is not supported")
+        self.granularity = granularity
+        if mapping_type is not None and is_symmetric is not None:
+            raise ValueError("Cannot set both `mapping_type` and `is_symmetric`")
+        if mapping_type is not None:
+            if str(mapping_type).lower().endswith("asymmetric"):
+                is_symmetric = False
+            elif str(mapping_type).lower().endswith("symmetric"):
+                is_symmetric = True
+            else:
+                raise ValueError(f"Unexpected mapping_type: {mapping_type}")
+        self.is_symmetric = True if is_symmetric is None else bool(is_symmetric)
+        self.scale_precision = scale_precision
+        self.zero_point_precision = zero_point_precision
+        self.is_dynamic = is_dynamic
+        if not is_dynamic:
+            raise NotImplementedError("FakeQuantizeConfig: only dynamic qparams have a kernel")
+
+    @property
+    def group_size(self) -> Optional[int]:
+        return self.granularity.group_size if isinstance(self.granularity, PerGroup) else None
+
+    @property
+    def mapping_type(self) -> str:
+        return "SYMMETRIC" if self.is_symmetric else "ASYMMETRIC"
+
+    def __repr__(self) -> str:
+        return (
+            f"FakeQuantizeConfig(dtype={self.dtype}, granularity={self.granularity}, mapping_type={self.mapping_type}, "
+            f"scale_precision={self.scale_precision}, zero_point_precision={self.zero_point_precision}, "
+            f"is_dynamic={self.is_dynamic})"
+        )
+
+
+class _StraightThrough(torch.autograd.Function):
+    """y = fake_quantise(x); dy/dx = 1.  The reference masks the gradient with (qmin <= q <= qmax) evaluated on the
+    already clamped q, which is identically true."""
+
+    @staticmethod
+    def forward(ctx, x, fq):
+        return fq
+
+    @staticmethod
+    def backward(ctx, g):
+        return g, None
+
+
+class FakeQuantizer(nn.Module):
+    """Fake-quantise the input according to ``config``.  ``enabled = False`` makes it the identity."""
+
+    def __init__(self, config: FakeQuantizeConfig):
+        super().__init__()
+        self.config = config
+        self.enabled = True
+        self.scale: Optional[torch.Tensor] = None
+        self.zero_point: Optional[torch.Tensor] = None
+        g = config.granularity
+        if isinstance(g, PerToken):
+            if config.dtype != torch.int8 or config.is_symmetric:
+                raise NotImplementedError("per-token fake quantisation has a kernel for asymmetric int8 only")
+        elif isinstance(g, PerGroup):
+            if config.dtype != torch.int4 or not config.is_symmetric:
+                raise NotImplementedError("per-group fake quantisation has a kernel for symmetric int4 only")
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        if not self.enabled:
+            return x
+        with torch.no_grad():
+            if isinstance(self.config.granularity, PerToken):
+                fq, scale, zp = ops.fq_per_token_int8_asym(x.detach())
+                self.scale = scale.to(self.config.scale_precision)
+                self.zero_point = zp.to(self.config.zero_point_precision)
+            else:
+                gs = self.config.group_size
+                if x.shape[-1] % gs != 0:
+                    raise ValueError(f"last dimension ({x.shape[-1]}) must be divisible by group_size ({gs})")
+                fq, scale = ops.fq_per_group_int4_sym(x.detach(), gs)
+                self.scale = scale.to(self.config.scale_precision)
+                self.zero_point = None
+        return _StraightThrough.apply(x, fq.view(x.shape))
+
+    def __repr__(self) -> str:
+        return f"FakeQuantizer({self.config})"
+
+
+class FakeQuantizedLinear(nn.Linear):
+    """``nn.Linear`` that fake-quantises its input and/or weight before the matmul."""
+
+    def __init__(
+        self,
+        in_features: int,
+        out_features: int,
+        bias: bool = False,
+        activation_config: Optional[FakeQuantizeConfig] = None,
+        weight_config: Optional[FakeQuantizeConfig] = None,
+        *args,
+        **kwargs,
+    ) -> None:
+        super().__init__(in_features, out_features, bias, *args, **kwargs)
+        self.activation_fake_quantizer = FakeQuantizer(activation_config) if activation_config is not None else None
+        if weight_config is not None:
+            gs = weight_config.group_size
+            if gs is not None and in_features % gs != 0:
+                raise ValueError("in_features (%s) %% group_size (%s) must be == 0" % (in_features, gs))
+            self.weight_fake_quantizer = FakeQuantizer(weight_config)
+        else:
+            self.weight_fake_quantizer = None
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        if self.activation_fake_quantizer is not None:
+            x = self.activation_fake_quantizer(x)
+        w = self.weight if self.weight_fake_quantizer is None else self.weight_fake_quantizer(self.weight)
+        return F.linear(x, w, self.bias)
+
+    def to_linear(self) -> nn.Linear:
+        new = nn.Linear(self.in_features, self.out_features, self.bias is not None, device=self.weight.device,
+                        dtype=self.weight.dtype)
+        if self.weight.device != torch.device("meta"):
+            new.weight = self.weight
+            new.bias = self.bias
+        return new
+
+    @classmethod
+    def from_linear(cls, mod: nn.Linear, activation_config=None, weight_config=None) -> "FakeQuantizedLinear":
+        new = cls(mod.in_features, mod.out_features, mod.bias is not None, activation_config, weight_config,
+                  device=mod.weight.device, dtype=mod.weight.dtype)
+        if mod.weight.device != torch.device("meta"):
+            new.weight = mod.weight
+            new.bias = mod.bias
+        return new
+
+
+class Int8DynActInt4WeightQATLinear(FakeQuantizedLinear):
+    """The linear ``Int8DynActInt4WeightQATQuantizer.prepare`` swaps in: per-token asymmetric int8 fake
+    quantisation of the input, per-group symmetric int4 fake quantisation of the weight."""
+
+    def __init__(
+        self,
+        in_features: int,
+        out_features: int,
+        bias: bool = False,
+        device: Optional[torch.device] = None,
+        groupsize: int = 256,
+        precision: torch.dtype = torch.float32,
+        scales_precision: torch.dtype = torch.float32,
+    ) -> None:
+        act = FakeQuantizeConfig(torch.int8, "per_token", is_symmetric=False, scale_precision=scales_precision)
+        wgt = FakeQuantizeConfig(torch.int4, group_size=groupsize, is_symmetric=True, scale_precision=scales_precision)
+        super().__init__(in_features, out_features, bias, act, wgt, device=device, dtype=precision)
+        self.groupsize = groupsize
+        self.precision = precision
+        self.scales_precision = scales_precision
+
+    def enable_fake_quant(self, enabled: bool = True):
+        self.activation_fake_quantizer.enabled = enabled
+        self.weight_fake_quantizer.enabled = enabled
+
+    def disable_fake_quant(self):
+        self.enable_fake_quant(False)
+
+
+class Int8DynActInt4WeightLinear(nn.Module):
+    """Result of ``convert``: int4 weight values held in int8 plus per-group scales and zeros; the input is
+    quantised per token on the fly.  Forward reproduces the arithmetic the fake-quantised layer trained with."""
+
+    def __init__(self, in_features: int, out_features: int, bias: bool = False, device=None, groupsize: int = 256,
+                 precision: torch.dtype = torch.float32, scales_precision: torch.dtype = torch.float32) -> None:
+        super().__init__()
+        assert in_features % groupsize == 0, f"require in_features:{in_features} % groupsize:{groupsize} == 0"
+        self.in_features = in_features
+        self.out_features = out_features
+        self.groupsize = groupsize
+        self.precision = precision
+        self.scales_precision = scales_precision
+        self.register_buffer("weight", torch.zeros((out_features, in_features), dtype=torch.int8, device=device))
+        self.register_buffer(
+            "scales", torch.zeros((out_features, in_features // groupsize), dtype=scales_precision, device=device)
+        )
+        self.register_buffer(
+            "zeros", torch.zeros((out_features, in_features // groupsize), dtype=scales_precision, device=device)
+        )
+        self.bias = nn.Parameter(torch.zeros(out_features, dtype=precision, device=device)) if bias else None
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        x = x.to(self.precision)
+        x_q, _, _ = ops.fq_per_token_int8_asym(x, want_qparams=False)
+        N, K = self.weight.shape
+        g = self.groupsize
+        w = (self.weight.view(N, K // g, g).to(self.precision) - self.zeros.view(N, K // g, 1).to(self.precision))
+        w = (w * self.scales.view(N, K // g, 1)).to(self.precision).view(N, K)
+        return F.linear(x_q, w, self.bias)
+
+
+class Int8DynActInt4WeightQATQuantizer:
+    """QAT quantizer for int8 dynamic per-token activations + int4 per-group symmetric weights.
+
+    ``prepare(model)`` swaps every eligible ``nn.Linear`` for :class:`Int8DynActInt4WeightQATLinear`;
+    ``convert(model)`` swaps those for :class:`Int8DynActInt4WeightLinear` holding real int4 values.
+    """
+
+    def __init__(
+        self,
+        groupsize: int = 256,
+        padding_allowed: bool = False,
+        precision: torch.dtype = torch.float32,
+        scales_precision: torch.dtype = torch.float32,
+    ) -> None:
+        self.groupsize = groupsize
+        self.padding_allowed = padding_allowed
+        self.precision = precision
+        self.scales_precision = scales_precision
+        if padding_allowed:
+            raise NotImplementedError("padding_allowed=True is not supported")
+
+    def get_activation_fake_quantize_config(self) -> FakeQuantizeConfig:
+        return FakeQuantizeConfig(torch.int8, "per_token", is_symmetric=False, scale_precision=self.scales_precision)
+
+    def get_weight_fake_quantize_config(self) -> FakeQuantizeConfig:
+        return FakeQuantizeConfig(torch.int4, group_size=self.groupsize, is_symmetric=True,
+                                  scale_precision=self.scales_precision)
+
+    def _eligible(self, lin: nn.Linear) -> bool:
+        return lin.in_features % self.groupsize == 0
+
+    def prepare(self, model: nn.Module, *args, **kwargs) -> nn.Module:
+        for name, child in list(model.named_children()):
+            if type(child) is nn.Linear and self._eligible(child):
+                new = Int8DynActInt4WeightQATLinear(
+                    child.in_features, child.out_features, child.bias is not None, device=child.weight.device,
+                    groupsize=self.groupsize, precision=self.precision, scales_precision=self.scales_precision,
+                )
+                # keep the trained values; cast to the quantizer's precision as the swap in the reference does
+                if child.weight.device != torch.device("meta"):
+                    new.weight = nn.Parameter(child.weight.detach().to(self.precision), requires_grad=child.weight.requires_grad)
+                    if child.bias is not None:
+                        new.bias = nn.Parameter(child.bias.detach().to(self.precision), requires_grad=child.bias.requires_grad)
+                setattr(model, name, new)
+            else:
+                self.prepare(child)
+        return model
+
+    def convert(self, model: nn.Module, *args, **kwargs) -> nn.Module:
+        for name, child in list(model.named_children()):
+            if isinstance(child, Int8DynActInt4WeightQATLinear):
+                new = Int8DynActInt4WeightLinear(
+                    child.in_features, child.out_features, child.bias is not None, device=child.weight.device,
+                    groupsize=child.groupsize, precision=child.weight.dtype, scales_precision=child.scales_precision,
+                )
+                q, scale, zeros = ops.quantize_per_group_int4(child.weight.detach(), child.groupsize)
+                new.weight.copy_(q)
+                new.scales.copy_(scale.to(child.scales_precision))
+                new.zeros.copy_(zeros.to(child.scales_precision))
+                if child.bias is not None:
+                    new.bias = nn.Parameter(child.bias.detach(), requires_grad=False)
+                setattr(model, name, new)
+            else:
+                self.convert(child)
+        return model
