@@ -1,0 +1,136 @@
+"""GPU parity of the fake-quant kernels and the QAT modules against the CPU oracle (bit-exact values and qparams)."""
+import pytest
+import torch
+from torch import nn
+
+from oracle import fake_quant_oracle as fq
+from tests.helpers import bits_equal
+from torchtune_amd import ops
+from torchtune_amd.qat import (
+    FakeQuantizeConfig,
+    FakeQuantizer,
+    Int8DynActInt4WeightLinear,
+    Int8DynActInt4WeightQATLinear,
+    Int8DynActInt4WeightQATQuantizer,
+)
+from torchtune_amd.training import quantization
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("rows,K", [(1, 8), (5, 24), (64, 4096), (7, 14336), (3, 28672), (4, 40000), (130, 512)])
+def test_per_token_bit_exact(dtype, rows, K):
+    g = torch.Generator().manual_seed(rows * 1000 + K)
+    x = (torch.randn(rows, K, generator=g) * 1.7).to(dtype)
+    if rows > 4:
+        x[1] = 0
+        x[2] = x[2].abs()
+        x[3] = -x[3].abs()
+        x[4, ::2] *= 50
+    want, ws, wz = fq.fq_per_token_int8_asym(x)
+    got, gs, gz = ops.fq_per_token_int8_asym(x.to(DEV))
+    assert bits_equal(got.cpu(), want) and torch.equal(gs.cpu(), ws) and torch.equal(gz.cpu(), wz)
+    out_only, s_none, z_none = ops.fq_per_token_int8_asym(x.to(DEV), want_qparams=False)
+    assert s_none is None and z_none is None and bits_equal(out_only.cpu(), want)
+
+
+def test_per_token_keeps_leading_dimensions():
+    x = torch.randn(2, 3, 64, generator=torch.Generator().manual_seed(0)).to(torch.bfloat16)
+    got, s, z = ops.fq_per_token_int8_asym(x.to(DEV))
+    want, ws, wz = fq.fq_per_token_int8_asym(x.view(6, 64))
+    assert got.shape == x.shape and s.shape == (6,) and bits_equal(got.cpu().view(6, 64), want)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("g", [8, 16, 32, 64, 256, 512])
+def test_per_group_and_convert_bit_exact(dtype, g):
+    gen = torch.Generator().manual_seed(g)
+    w = (torch.randn(96, 1024, generator=gen) * 0.02).to(dtype)
+    w[0, :g] = 0
+    w[1, :g] = 7.5 * 0.01
+    want, ws = fq.fq_per_group_int4_sym(w, g)
+    got, gs = ops.fq_per_group_int4_sym(w.to(DEV), g)
+    assert bits_equal(got.cpu(), want) and torch.equal(gs.cpu(), ws)
+    wq, ws2, wz = fq.quantize_per_group_int4(w, g)
+    gq, gs2, gz = ops.quantize_per_group_int4(w.to(DEV), g)
+    assert gq.dtype == torch.int8 and torch.equal(gq.cpu(), wq) and torch.equal(gs2.cpu(), ws2) and torch.equal(gz.cpu(), wz)
+
+
+def test_ragged_tail_of_the_last_workgroup():
+    # 3 x 40 elements with groups of 8: 15 chunks, far less than one workgroup's 1024
+    w = (torch.randn(3, 40, generator=torch.Generator().manual_seed(1)) * 0.1).to(torch.bfloat16)
+    want, ws = fq.fq_per_group_int4_sym(w, 8)
+    got, gs = ops.fq_per_group_int4_sym(w.to(DEV), 8)
+    assert bits_equal(got.cpu(), want) and torch.equal(gs.cpu(), ws)
+
+
+def test_fake_quantizer_modules_and_straight_through_gradient():
+    act = FakeQuantizer(FakeQuantizeConfig(torch.int8, "per_token", is_symmetric=False))
+    wgt = FakeQuantizer(FakeQuantizeConfig(torch.int4, group_size=32))
+    x = torch.randn(4, 8, 128, generator=torch.Generator().manual_seed(2)).to(torch.bfloat16)
+    xd = x.to(DEV).requires_grad_()
+    y = act(xd)
+    want, ws, wz = fq.fq_per_token_int8_asym(x.view(-1, 128))
+    assert bits_equal(y.detach().cpu().view(-1, 128), want)
+    assert torch.equal(act.scale.cpu(), ws) and torch.equal(act.zero_point.cpu(), wz) and act.zero_point.dtype == torch.int32
+    gy = torch.randn_like(y)
+    y.backward(gy)
+    assert torch.equal(xd.grad, gy)  # dy/dx = 1
+    act.enabled = False
+    assert act(xd) is xd
+    w = (torch.randn(64, 128, generator=torch.Generator().manual_seed(3)) * 0.02).to(torch.bfloat16)
+    assert bits_equal(wgt(w.to(DEV)).cpu(), fq.fq_per_group_int4_sym(w, 32)[0])
+    assert torch.equal(wgt.scale.cpu(), fq.fq_per_group_int4_sym(w, 32)[1]) and wgt.zero_point is None
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_qat_linear_forward_backward_vs_oracle(dtype):
+    gen = torch.Generator().manual_seed(4)
+    N, K, M, g = 256, 512, 96, 32
+    w = (torch.randn(N, K, generator=gen) * 0.02).to(dtype)
+    x = torch.randn(M, K, generator=gen).to(dtype)
+    lin = Int8DynActInt4WeightQATLinear(K, N, bias=False, device=DEV, groupsize=g, precision=dtype)
+    with torch.no_grad():
+        lin.weight.copy_(w)
+    xd = x.to(DEV).requires_grad_()
+    y = lin(xd)
+    (y.float() ** 2).sum().backward()
+    xo, wo = x.clone().requires_grad_(), w.clone().requires_grad_()
+    yo = fq.fake_quantized_linear(xo, wo, g)
+    (yo.float() ** 2).sum().backward()
+    tol = dict(rtol=1e-2, atol=1e-2) if dtype == torch.bfloat16 else dict(rtol=1e-4, atol=1e-4)
+    torch.testing.assert_close(y.detach().cpu().float(), yo.detach().float(), **tol)
+    torch.testing.assert_close(xd.grad.cpu().float(), xo.grad.float(), **tol)
+    gw, gwo = lin.weight.grad.cpu().float(), wo.grad.float()
+    torch.testing.assert_close(gw, gwo, rtol=2e-2, atol=2e-2 * float(gwo.abs().max()))
+    # toggles of torchtune/training/quantization.py:56-71
+    lin.apply(quantization._get_disable_fake_quant("8da4w-qat"))
+    torch.testing.assert_close(lin(xd).detach().cpu().float(), (x.float() @ w.float().T), **(tol if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)))
+    lin.apply(quantization._get_enable_fake_quant("8da4w-qat"))
+    assert lin.weight_fake_quantizer.enabled and lin.activation_fake_quantizer.enabled
+
+
+def test_prepare_then_convert_is_bit_exact_and_consistent():
+    gen = torch.Generator().manual_seed(5)
+    model = nn.Sequential(nn.Linear(256, 512, bias=False), nn.Sequential(nn.Linear(512, 128, bias=True))).to(DEV).to(torch.bfloat16)
+    with torch.no_grad():
+        for p in model.parameters():
+            p.copy_((torch.randn(p.shape, generator=gen) * 0.05).to(torch.bfloat16))
+    w0 = model[0].weight.detach().cpu().clone()
+    w1 = model[1][0].weight.detach().cpu().clone()
+    qz = Int8DynActInt4WeightQATQuantizer(groupsize=32, precision=torch.bfloat16)
+    model = qz.prepare(model)
+    x = torch.randn(10, 256, generator=gen).to(torch.bfloat16).to(DEV)
+    y_fake = model(x)
+    model = qz.convert(model)
+    c0, c1 = model[0], model[1][0]
+    assert isinstance(c0, Int8DynActInt4WeightLinear) and isinstance(c1, Int8DynActInt4WeightLinear)
+    for conv, w in ((c0, w0), (c1, w1)):
+        q, s, z = fq.quantize_per_group_int4(w, 32)
+        assert conv.weight.dtype == torch.int8 and torch.equal(conv.weight.cpu(), q)
+        assert int(conv.weight.min()) >= -8 and int(conv.weight.max()) <= 7
+        assert torch.equal(conv.scales.cpu(), s) and torch.equal(conv.zeros.cpu(), z) and conv.scales.shape == (w.shape[0], w.shape[1] // 32)
+    # the converted model computes what the fake-quantised model computed
+    torch.testing.assert_close(model(x).float(), y_fake.float(), rtol=1e-2, atol=1e-2)

@@ -1,0 +1,157 @@
+"""The reference's own module-level tests for this path, restated against this package on the GPU
+(tests/torchtune/modules/peft/test_lora.py, tests/torchtune/modules/low_precision/test_nf4_linear.py,
+tests/torchtune/modules/low_precision/test_nf4_dispatch_registration.py)."""
+import copy
+from functools import partial
+
+import pytest
+import torch
+from torch import nn
+
+from oracle import lora_oracle
+from torchtune_amd.modules.common_utils import reparametrize_as_dtype_state_dict_post_hook
+from torchtune_amd.modules.low_precision import FrozenNF4Linear
+from torchtune_amd.modules.peft import LoRALinear
+from torchtune_amd.nf4_tensor import NF4Tensor, to_nf4
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+class _default_dtype:
+    def __init__(self, dtype):
+        self.dtype = dtype
+
+    def __enter__(self):
+        self.prev = torch.get_default_dtype()
+        torch.set_default_dtype(self.dtype)
+
+    def __exit__(self, *a):
+        torch.set_default_dtype(self.prev)
+
+
+def _fixed_init(model):
+    with torch.no_grad():
+        for _, p in model.named_parameters():
+            p.copy_(lora_oracle.fixed_init_tensor(p.shape, dtype=p.dtype).to(p.device))
+
+
+def _qlora(use_bias, dtype, **kw):
+    with _default_dtype(dtype), torch.device(DEV):
+        m = LoRALinear(512, 512, rank=4, alpha=1.0, use_bias=use_bias, quantize_base=True, **kw)
+    _fixed_init(m)
+    return m
+
+
+def _lora(use_bias, dtype):
+    with _default_dtype(dtype), torch.device(DEV):
+        m = LoRALinear(512, 512, rank=4, alpha=1.0, use_bias=use_bias)
+    _fixed_init(m)
+    return m
+
+
+def test_inplace_copy_attribute_set():
+    z = to_nf4(torch.rand(512, 512, dtype=torch.bfloat16, device=DEV))
+    assert set(z.__dict__.keys()) == {"block_size", "n_blocks", "scaler_block_size", "quantized_scalers", "quantization_factor",
+                                      "scaler_mean", "quantized_data", "nf4"}
+
+
+@pytest.mark.parametrize("use_bias", [True, False])
+def test_lora_weight_nf4_when_quantized(use_bias):
+    m = _qlora(use_bias, torch.bfloat16)
+    assert isinstance(m.weight, NF4Tensor)
+    if use_bias:
+        assert not isinstance(m.bias, NF4Tensor) and m.bias.dtype == torch.bfloat16
+    m2 = _qlora(True, torch.bfloat16, block_size=8, scaler_block_size=4)
+    assert m2.weight.block_size == 8 and m2.weight.scaler_block_size == 4 and not isinstance(m2.bias, NF4Tensor)
+
+
+@pytest.mark.parametrize("use_bias,dtype", [(False, torch.bfloat16), (True, torch.float32), (False, torch.float32)])
+def test_qlora_parity(use_bias, dtype):
+    # tests/torchtune/modules/peft/test_lora.py:157-182: same output as a dense LoRA layer holding the dequantised weight
+    torch.manual_seed(16)
+    q = _qlora(use_bias, dtype)
+    d = _lora(use_bias, dtype)
+    d.weight.data = q.weight.to(dtype)
+    if use_bias:
+        d.bias.data = q.bias.detach().clone()
+    x = torch.randn(2, 32, 512, dtype=dtype, device=DEV)
+    out_d, out_q = d(x), q(x)
+    if dtype == torch.bfloat16:
+        # rank 4 is not a multiple of 8, so this goes through linear_nf4 (fused base GEMM) + library adapter GEMMs
+        torch.testing.assert_close(out_d, out_q, rtol=1.6e-2, atol=1e-5)  # the reference's own (default bf16) tolerances
+    else:
+        torch.testing.assert_close(out_d, out_q, rtol=1e-4, atol=1e-3)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_quantized_state_dict(dtype):
+    # tests/torchtune/modules/peft/test_lora.py:184-237
+    with _default_dtype(dtype), torch.device(DEV):
+        layer = LoRALinear(512, 512, rank=4, alpha=1.0, quantize_base=True)
+    layer._register_state_dict_hook(partial(reparametrize_as_dtype_state_dict_post_hook, dtype=dtype, offload_to_cpu=False))
+    sd = layer.state_dict()
+    for v in sd.values():
+        assert v.dtype == dtype and not isinstance(v, NF4Tensor)
+    with _default_dtype(dtype), torch.device(DEV):
+        reload = LoRALinear(512, 512, rank=4, alpha=1.0, quantize_base=True)
+    reload.weight = nn.Parameter(to_nf4(torch.zeros_like(layer.weight.get_original_weight(), dtype=dtype, device=layer.weight.device)))
+    assert not torch.allclose(layer.weight.quantized_data, reload.weight.quantized_data)
+    reload.load_state_dict(sd)
+    assert torch.allclose(layer.weight.quantized_data, reload.weight.quantized_data)
+    assert torch.equal(layer.weight.quantized_scalers, reload.weight.quantized_scalers)
+    # the offloading variant returns CPU tensors
+    sd_cpu = {"weight": layer.weight.detach()}
+    reparametrize_as_dtype_state_dict_post_hook(layer, sd_cpu, dtype=dtype)
+    assert sd_cpu["weight"].device.type == "cpu" and torch.equal(sd_cpu["weight"], sd["weight"].cpu())
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_frozen_nf4_linear(dtype):
+    # tests/torchtune/modules/low_precision/test_nf4_linear.py:24-70
+    lin = FrozenNF4Linear(512, 512, device=DEV, dtype=dtype)
+    params = list(lin.parameters())
+    assert len(params) == 1 and isinstance(params[0], NF4Tensor) and not params[0].requires_grad
+    sd = lin.state_dict()
+    assert len(sd) == 1 and isinstance(sd["weight"], NF4Tensor)
+    for bias in (True, False):
+        l2 = FrozenNF4Linear(512, 512, device=DEV, dtype=dtype, bias=bias)
+        inp = torch.randn(2, 512, dtype=dtype, device=DEV, requires_grad=True)
+        out = l2(inp)
+        assert out.dtype == dtype
+        out.sum().backward()
+        assert inp.grad is not None and inp.grad.dtype == dtype and l2.weight.grad is None
+    l3 = FrozenNF4Linear(512, 512, device=DEV, dtype=torch.bfloat16, block_size=16, scaler_block_size=256)
+    assert l3.weight.block_size == 16 and l3.weight.scaler_block_size == 256
+
+
+def test_clone_deepcopy_and_block_scaler_cache():
+    t = to_nf4((torch.randn(512, 512, device=DEV) * 0.02).to(torch.bfloat16), 64, 32)
+    c = t.clone()  # re-quantisation of the dequantised weight with the default granularity
+    assert isinstance(c, NF4Tensor) and c.block_size == 64 and c.scaler_block_size == 256
+    assert torch.equal(c.quantized_data, t.quantized_data)
+    lin = FrozenNF4Linear(512, 512, device=DEV, dtype=torch.bfloat16)
+    lin2 = copy.deepcopy(lin)
+    assert isinstance(lin2.weight, NF4Tensor) and torch.equal(lin2.weight.quantized_data, lin.weight.quantized_data)
+    assert lin2.weight.quantized_data.data_ptr() != lin.weight.quantized_data.data_ptr()
+    s1 = lin.weight.block_scalers()
+    assert lin.weight.block_scalers() is s1  # cached
+    with torch.no_grad():
+        lin.weight.copy_((torch.randn(512, 512, device=DEV) * 0.05).to(torch.bfloat16))
+    s2 = lin.weight.block_scalers()
+    assert s2 is not s1 and not torch.equal(s1, s2)  # in-place re-quantisation invalidates the cache
+    x = torch.randn(4, 512, device=DEV, dtype=torch.bfloat16)
+    torch.testing.assert_close(lin(x).float(), x.float() @ lin.weight.get_original_weight().float().T, rtol=1e-2, atol=1e-2)
+
+
+def test_load_dense_state_dict_into_nf4_model_and_back():
+    with _default_dtype(torch.bfloat16), torch.device(DEV):
+        layer = LoRALinear(512, 512, rank=8, alpha=16.0, quantize_base=True)
+    dense = {"weight": (torch.randn(512, 512) * 0.02).to(torch.bfloat16), "lora_a.weight": torch.randn(8, 512).to(torch.bfloat16),
+             "lora_b.weight": torch.randn(512, 8).to(torch.bfloat16)}
+    layer.load_state_dict(dense)
+    want = to_nf4(dense["weight"].to(DEV))
+    assert torch.equal(layer.weight.quantized_data, want.quantized_data)
+    fp32 = {k: v.float() for k, v in dense.items()}
+    layer.load_state_dict(fp32)  # a float32 checkpoint loads too (cast to the parameter dtype, then quantised)
+    assert torch.equal(layer.weight.quantized_data, want.quantized_data)

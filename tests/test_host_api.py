@@ -1,0 +1,295 @@
+"""CPU-only checks of the host side: the C-ABI library loads and exports every declared symbol, argument
+validation works without a GPU, the shared rounding code matches the oracle exhaustively, and the Python surface
+mirrors the reference's (names, attributes, error messages)."""
+import ctypes
+import os
+import re
+import subprocess
+
+import pytest
+import torch
+from torch import nn
+
+import torchtune_amd
+from oracle import lora_oracle, nf4_oracle
+from torchtune_amd import _lib, ops
+from torchtune_amd.modules.low_precision import FrozenNF4Linear
+from torchtune_amd.modules.peft import LoRALinear, QATLoRALinear, get_adapter_params, set_trainable_params
+from torchtune_amd.nf4_tensor import NF4Tensor, to_nf4
+from torchtune_amd.qat import (
+    FakeQuantizeConfig,
+    FakeQuantizedLinear,
+    FakeQuantizer,
+    Int8DynActInt4WeightQATLinear,
+    Int8DynActInt4WeightQATQuantizer,
+)
+from torchtune_amd.training import quantization
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "torchtune_amd.h")
+
+
+def _declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(ttamd_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    declared = _declared_symbols()
+    assert len(declared) >= 15
+    for name in declared:
+        assert hasattr(lib, name), f"{name} is declared in the header but not exported"
+    assert sorted(_lib.SIGNATURES) == declared, "ctypes prototypes and header disagree"
+    assert lib.ttamd_version() == _lib.ABI_VERSION == 1
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", tmp_path / "nope.so")
+    with pytest.raises(_lib.LibraryNotBuiltError, match="no compute path without its HIP library"):
+        _lib.load()
+
+
+def test_argument_validation_needs_no_gpu():
+    lib = _lib.load()
+    buf = (ctypes.c_char * 4096)()
+    p = ctypes.cast(buf, ctypes.c_void_p)
+    aligned = ctypes.c_void_p((p.value + 255) & ~255)
+    # numel not divisible by the block size
+    rc = lib.ttamd_nf4_quantize(aligned, 0, 100, 64, 256, aligned, aligned, aligned, aligned, aligned, 4096, None)
+    assert rc == -1 and b"divisible by block_size" in lib.ttamd_last_error()
+    rc = lib.ttamd_nf4_quantize(aligned, 0, 64 * 10, 64, 256, aligned, aligned, aligned, aligned, aligned, 4096, None)
+    assert rc == -1 and b"scaler_block_size" in lib.ttamd_last_error()
+    rc = lib.ttamd_nf4_quantize(aligned, 7, 64 * 256, 64, 256, aligned, aligned, aligned, aligned, aligned, 4096, None)
+    assert rc == -1 and b"dtype" in lib.ttamd_last_error()
+    rc = lib.ttamd_nf4_quantize(None, 0, 64 * 256, 64, 256, aligned, aligned, aligned, aligned, aligned, 4096, None)
+    assert rc == -1 and b"null" in lib.ttamd_last_error()
+    # workspace too small is its own code
+    rc = lib.ttamd_nf4_quantize(aligned, 0, 64 * 256, 64, 256, aligned, aligned, aligned, aligned, aligned, 16, None)
+    assert rc == -3 and b"workspace" in lib.ttamd_last_error()
+    assert lib.ttamd_nf4_quantize_workspace_bytes(64 * 256, 64) >= 256 * 4
+    # fused GEMM shape rules
+    rc = lib.ttamd_nf4_lora_linear_fwd_bf16(aligned, aligned, aligned, None, None, 0, 0.0, None, aligned, 8, 64, 100, None)
+    assert rc == -1 and b"multiple of the NF4 block size" in lib.ttamd_last_error()
+    rc = lib.ttamd_nf4_lora_linear_fwd_bf16(aligned, aligned, aligned, None, None, 8, 2.0, None, aligned, 8, 64, 64, None)
+    assert rc == -1 and b"adapter pointers" in lib.ttamd_last_error()
+    rc = lib.ttamd_nf4_linear_bwd_dx_bf16(aligned, aligned, aligned, aligned, aligned, 12, aligned, 8, 64, 64, None)
+    assert rc == -1 and b"rank" in lib.ttamd_last_error()
+    rc = lib.ttamd_fq_per_group_int4_sym(aligned, 0, 4, 64, 24, aligned, None, None)
+    assert rc == -1 and b"group_size" in lib.ttamd_last_error()
+    rc = lib.ttamd_fq_per_token_int8_asym(aligned, 0, 4, 12, aligned, None, None, None)
+    assert rc == -1 and b"multiple of 8" in lib.ttamd_last_error()
+    with pytest.raises(ValueError, match="multiple of 8"):
+        _lib.check(rc, "fq_per_token")
+
+
+@pytest.fixture(scope="module")
+def host_math(tmp_path_factory):
+    """torchtune_amd/csrc/nf4_math.h compiled for the host: the same source the kernels use."""
+    d = tmp_path_factory.mktemp("hostmath")
+    src = d / "host_math.cpp"
+    src.write_text(
+        '#include "%s"\n'
+        'extern "C" int code_bf16(float s) { return ttamd::nf4_nearest_code<true>(s); }\n'
+        'extern "C" int code_f32(float s) { return ttamd::nf4_nearest_code<false>(s); }\n'
+        'extern "C" float scaler_bf16(int q, float f, float m) { return ttamd::nf4_block_scaler<true>(q, f, m); }\n'
+        'extern "C" float scaler_f32(int q, float f, float m) { return ttamd::nf4_block_scaler<false>(q, f, m); }\n'
+        'extern "C" void codes_bf16(const float* s, int n, int* out) { for (int i = 0; i < n; ++i) out[i] = code_bf16(s[i]); }\n'
+        'extern "C" void codes_f32(const float* s, int n, int* out) { for (int i = 0; i < n; ++i) out[i] = code_f32(s[i]); }\n'
+        % os.path.join(ROOT, "torchtune_amd", "csrc", "nf4_math.h")
+    )
+    so = d / "host_math.so"
+    subprocess.run(["g++", "-O2", "-std=c++17", "-shared", "-fPIC", "-ffp-contract=off", str(src), "-o", str(so)], check=True)
+    lib = ctypes.CDLL(str(so))
+    lib.scaler_bf16.restype = ctypes.c_float
+    lib.scaler_bf16.argtypes = [ctypes.c_int, ctypes.c_float, ctypes.c_float]
+    lib.scaler_f32.restype = ctypes.c_float
+    lib.scaler_f32.argtypes = [ctypes.c_int, ctypes.c_float, ctypes.c_float]
+    return lib
+
+
+def test_kernel_code_search_matches_oracle_on_every_bf16_pattern(host_math):
+    pats = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+    table = torch.tensor(nf4_oracle.NF4_TABLE, dtype=torch.bfloat16)
+    want = (pats[:, None] - table[None, :]).abs().argmin(dim=-1).to(torch.int32)
+    want[pats.isnan()] = 0
+    s = pats.float().contiguous()
+    got = torch.empty(65536, dtype=torch.int32)
+    host_math.codes_bf16(ctypes.c_void_p(s.data_ptr()), 65536, ctypes.c_void_p(got.data_ptr()))
+    assert torch.equal(got, want)
+
+
+def test_kernel_code_search_matches_oracle_fp32(host_math):
+    g = torch.Generator().manual_seed(0)
+    table = torch.tensor(nf4_oracle.NF4_TABLE)
+    mids = (table[1:] + table[:-1]) / 2
+    near = torch.cat([mids + d for d in (-2e-7, -6e-8, 0.0, 6e-8, 2e-7)])
+    s = torch.cat([torch.rand(200000, generator=g) * 2 - 1, table, near, torch.tensor([float("nan"), 0.0, -0.0])]).contiguous()
+    want = (s[:, None] - table[None, :]).abs().argmin(dim=-1).to(torch.int32)
+    want[s.isnan()] = 0
+    got = torch.empty(s.numel(), dtype=torch.int32)
+    host_math.codes_f32(ctypes.c_void_p(s.data_ptr()), s.numel(), ctypes.c_void_p(got.data_ptr()))
+    assert torch.equal(got, want)
+
+
+def test_kernel_block_scaler_matches_oracle(host_math):
+    for dtype, fn in ((torch.bfloat16, host_math.scaler_bf16), (torch.float32, host_math.scaler_f32)):
+        for factor, mean in ((257.0, 0.0625), (999.0, 0.0211), (3.0, -0.5)):
+            qs = torch.arange(-128, 128, dtype=torch.int8)
+            p = nf4_oracle.NF4Parts(64, 256, 256, qs, torch.tensor([factor], dtype=dtype), torch.tensor(mean, dtype=dtype),
+                                    torch.zeros(64 * 128, dtype=torch.uint8), torch.tensor(nf4_oracle.NF4_TABLE, dtype=dtype),
+                                    torch.Size([256, 64]), dtype)
+            want = nf4_oracle.nf4_dequantize_scalers(p).float()
+            f, m = p.quantization_factor.float().item(), p.scaler_mean.float().item()
+            got = torch.tensor([fn(int(q), f, m) for q in qs])
+            assert torch.equal(got, want)
+
+
+# ---- Python surface ---------------------------------------------------------------------------------------
+def test_lora_linear_surface_and_known_answer():
+    m = LoRALinear(in_dim=64, out_dim=128, rank=4, alpha=1.0, use_bias=True)
+    for attr in ("in_dim", "out_dim", "rank", "alpha", "use_bias", "_quantize_base", "disabled", "merged", "weight", "bias",
+                 "dropout", "lora_a", "lora_b"):
+        assert hasattr(m, attr)
+    assert m.adapter_params() == ["lora_a.weight", "lora_b.weight"]
+    assert isinstance(m.dropout, nn.Identity) and isinstance(LoRALinear(8, 8, 2, 1.0, dropout=0.1).dropout, nn.Dropout)
+    assert torch.all(m.lora_b.weight == 0)  # B starts at zero
+    assert m.lora_a.weight.abs().max() <= 1 / 64 ** 0.5
+    assert [n for n, _ in m.named_parameters()] == ["weight", "bias", "lora_a.weight", "lora_b.weight"]
+    with torch.no_grad():
+        for _, p in m.named_parameters():
+            p.copy_(lora_oracle.fixed_init_tensor(p.shape))
+    torch.manual_seed(16)
+    x = torch.randn(2, 32, 64)
+    torch.testing.assert_close(m(x).mean(), torch.tensor(1.1252), atol=1e-4, rtol=1e-6)
+    m.disabled = True
+    torch.testing.assert_close(m(x), torch.nn.functional.linear(x, m.weight, m.bias))
+    set_trainable_params(m, get_adapter_params(m))
+    assert [n for n, p in m.named_parameters() if p.requires_grad] == ["lora_a.weight", "lora_b.weight"]
+
+
+def test_lora_linear_rejects_quantisation_kwargs_without_quantize_base():
+    with pytest.raises(ValueError, match="``quantize_base`` is False, but received the following quantization arguments"):
+        LoRALinear(512, 512, 4, 1.0, use_bias=True, quantize_base=False, block_size=8, scaler_block_size=4)
+
+
+def test_qat_lora_linear_surface():
+    base = LoRALinear(64, 128, 4, 1.0)
+    with torch.no_grad():
+        for _, p in base.named_parameters():
+            p.copy_(lora_oracle.fixed_init_tensor(p.shape))
+    q = QATLoRALinear.from_lora_linear(base)
+    assert isinstance(q.activation_fake_quantizer, nn.Identity) and isinstance(q.weight_fake_quantizer, nn.Identity)
+    assert q.weight is base.weight and q.lora_a.weight is base.lora_a.weight
+    torch.manual_seed(16)
+    torch.testing.assert_close(q(torch.randn(2, 32, 64)).mean(), torch.tensor(0.6291), atol=1e-4, rtol=1e-6)
+    with pytest.raises(ValueError, match="Bias is not supported in QAT \\+ LoRA yet"):
+        QATLoRALinear.from_lora_linear(LoRALinear(64, 128, 4, 1.0, use_bias=True))
+    with pytest.raises(ValueError, match="in_dim \\(100\\) must be divisible by group_size \\(32\\)"):
+        QATLoRALinear(100, 64, 4, 1.0, weight_qat_config=FakeQuantizeConfig(torch.int4, group_size=32))
+
+
+def test_quantisation_needs_a_gpu_and_says_so():
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    with pytest.raises(RuntimeError, match="needs an AMD GPU"):
+        to_nf4(torch.randn(512, 512))
+    with pytest.raises(RuntimeError, match="needs an AMD GPU"):
+        LoRALinear(512, 512, 8, 16.0, quantize_base=True)
+    with pytest.raises(RuntimeError, match="expected a tensor on an AMD GPU"):
+        ops.fq_per_token_int8_asym(torch.randn(4, 64))
+
+
+def _cpu_nf4(shape=(512, 512), dtype=torch.bfloat16, bs=64, sbs=256) -> NF4Tensor:
+    """An NF4Tensor assembled from oracle parts, so the host-side tensor mechanics can run without a GPU."""
+    p = nf4_oracle.nf4_quantize((torch.randn(shape, generator=torch.Generator().manual_seed(0)) * 0.02).to(dtype), bs, sbs)
+    return NF4Tensor(p.shape, p.dtype, p.block_size, p.n_blocks, p.scaler_block_size, p.quantized_scalers,
+                     p.quantization_factor, p.scaler_mean, p.quantized_data, p.nf4)
+
+
+def test_nf4_tensor_host_mechanics():
+    t = _cpu_nf4()
+    # the attribute set pinned by tests/torchtune/modules/low_precision/test_nf4_dispatch_registration.py:22-31
+    assert set(t.__dict__.keys()) == {"block_size", "n_blocks", "scaler_block_size", "quantized_scalers", "quantization_factor",
+                                      "scaler_mean", "quantized_data", "nf4"}
+    assert t.shape == (512, 512) and t.dtype == torch.bfloat16 and t.device.type == "cpu" and not t.is_meta
+    assert t.quantized_data.dtype == torch.uint8 and t.quantized_data.numel() == 512 * 512 // 2
+    assert t.quantized_scalers.dtype == torch.int8 and t.quantization_factor.dtype == torch.bfloat16 and t.nf4.numel() == 16
+    d = t.detach()
+    assert isinstance(d, NF4Tensor) and d.quantized_data.data_ptr() == t.quantized_data.data_ptr()
+    p = nn.Parameter(t, requires_grad=False)
+    assert isinstance(p, NF4Tensor) and not p.requires_grad
+    lin = nn.Linear(512, 512, bias=False, dtype=torch.bfloat16)
+    torch.utils.swap_tensors(lin.weight, p)
+    assert isinstance(lin.weight, NF4Tensor)
+    sd = lin.state_dict()
+    assert isinstance(sd["weight"], NF4Tensor) and len(sd) == 1
+    # same-layout NF4 -> NF4 copy_ copies the packed representation without arithmetic
+    other = _cpu_nf4()
+    other.quantized_data.zero_()
+    other.copy_(t)
+    assert torch.equal(other.quantized_data, t.quantized_data) and torch.equal(other, t)
+    assert "NF4Tensor(shape=(512, 512)" in repr(t)
+    names, ctx = t.__tensor_flatten__()
+    back = NF4Tensor.__tensor_unflatten__({n: getattr(t, n) for n in names}, ctx)
+    assert torch.equal(back, t)
+
+
+def test_fake_quantize_config_validation():
+    c = FakeQuantizeConfig(torch.int8, "per_token", is_symmetric=False)
+    assert c.group_size is None and not c.is_symmetric and c.scale_precision == torch.float32 and c.zero_point_precision == torch.int32
+    w = FakeQuantizeConfig(torch.int4, group_size=32)
+    assert w.group_size == 32 and w.is_symmetric and w.mapping_type == "SYMMETRIC"
+    assert FakeQuantizeConfig(torch.int4, "per_group", group_size=8).group_size == 8
+    with pytest.raises(ValueError, match="Cannot set both"):
+        FakeQuantizeConfig(torch.int4, "per_group", group_size=8, mapping_type="symmetric", is_symmetric=True)
+    with pytest.raises(ValueError, match="At least one of"):
+        FakeQuantizeConfig(torch.int4)
+    with pytest.raises(ValueError, match="Unexpected granularity"):
+        FakeQuantizeConfig(torch.int8, "per_banana")
+    with pytest.raises(NotImplementedError):
+        FakeQuantizer(FakeQuantizeConfig(torch.int8, "per_token", is_symmetric=True))
+    with pytest.raises(NotImplementedError):
+        FakeQuantizeConfig(torch.float16, "per_token")
+
+
+def test_quantizer_prepare_and_toggles_on_cpu():
+    model = nn.Sequential(nn.Linear(64, 128, bias=False), nn.ReLU(), nn.Sequential(nn.Linear(128, 64), nn.Linear(50, 8)))
+    qz = Int8DynActInt4WeightQATQuantizer(groupsize=32)
+    assert quantization.get_quantizer_mode(qz) == "8da4w-qat" and quantization.get_quantizer_mode(object()) is None
+    w0 = model[0].weight.detach().clone()
+    model = qz.prepare(model)
+    assert isinstance(model[0], Int8DynActInt4WeightQATLinear) and isinstance(model[0], FakeQuantizedLinear)
+    assert isinstance(model[2][0], Int8DynActInt4WeightQATLinear) and model[2][0].bias is not None
+    assert type(model[2][1]) is nn.Linear  # 50 % 32 != 0: left alone
+    assert torch.equal(model[0].weight, w0)
+    assert model[0].activation_fake_quantizer.config.granularity.__class__.__name__ == "PerToken"
+    assert model[0].weight_fake_quantizer.config.group_size == 32
+    assert qz.get_weight_fake_quantize_config().group_size == 32 and not qz.get_activation_fake_quantize_config().is_symmetric
+    disable = quantization._get_disable_fake_quant("8da4w-qat")
+    enable = quantization._get_enable_fake_quant("8da4w-qat")
+    model.apply(disable)
+    assert not model[0].activation_fake_quantizer.enabled and not model[0].weight_fake_quantizer.enabled
+    x = torch.randn(3, 64)
+    torch.testing.assert_close(model[0](x), x @ w0.T)  # disabled fake quant = plain linear, no kernel involved
+    model.apply(enable)
+    assert model[2][0].weight_fake_quantizer.enabled
+    assert quantization._get_enable_fake_quant("4w") is None
+    with pytest.raises(ValueError, match="must be == 0"):
+        FakeQuantizedLinear(50, 8, weight_config=FakeQuantizeConfig(torch.int4, group_size=32))
+
+
+def test_swap_lora_linear_with_qat():
+    model = nn.Sequential(LoRALinear(64, 64, 4, 1.0), nn.Sequential(LoRALinear(64, 32, 4, 1.0)))
+    quantization.swap_lora_linear_with_qat(model, None, FakeQuantizeConfig(torch.int4, group_size=32))
+    assert isinstance(model[0], QATLoRALinear) and isinstance(model[1][0], QATLoRALinear)
+    assert isinstance(model[0].weight_fake_quantizer, FakeQuantizer) and isinstance(model[0].activation_fake_quantizer, nn.Identity)
+
+
+def test_package_exports():
+    for name in ("NF4Tensor", "to_nf4", "linear_nf4", "implements", "FrozenNF4Linear", "LoRALinear", "QATLoRALinear",
+                 "Int8DynActInt4WeightQATQuantizer", "FakeQuantizeConfig", "FakeQuantizer", "FakeQuantizedLinear"):
+        assert hasattr(torchtune_amd, name)
+    assert FrozenNF4Linear.__mro__[1] is nn.Linear

@@ -1,0 +1,137 @@
+"""Pins the fake-quant oracle (oracle/fake_quant_oracle.py, oracle/nf4_ref.c): closed forms, grid and range
+invariants, idempotence, tiny exhaustive cases, agreement of the two restatements, straight-through backward."""
+import pytest
+import torch
+
+from oracle import fake_quant_oracle as fq
+from tests.helpers import bits_equal, c_fq_per_group, c_fq_per_token
+
+DTYPES = [torch.bfloat16, torch.float32]
+EPS = torch.finfo(torch.float32).eps
+
+
+def test_per_token_qparams_closed_form():
+    # row spanning [-1, 3]: scale = 4/255; zp: descaled min = -63.75, max = 191.25;
+    # (-128 - 63.75) + (127 + 191.25) > 0 -> zp = qmin - descaled_min = -128 + 63.75 = -64.25 -> round -> -64
+    x = torch.tensor([[-1.0, 0.5, 3.0, 0.0]])
+    scale, zp = fq.choose_qparams_per_token_asym(x)
+    assert scale.item() == pytest.approx(4.0 / 255.0, rel=1e-7)
+    assert zp.item() == -64 and zp.dtype == torch.int32 and scale.dtype == torch.float32
+    # all-positive row: the range is widened to include 0 -> min 0 maps to qmin exactly
+    x = torch.tensor([[1.0, 2.0, 4.0, 3.0]])
+    scale, zp = fq.choose_qparams_per_token_asym(x)
+    assert scale.item() == pytest.approx(4.0 / 255.0, rel=1e-7) and zp.item() == -128
+    # all-negative row -> max 0 maps to qmax
+    scale, zp = fq.choose_qparams_per_token_asym(-x)
+    assert zp.item() == 127
+    # all-zero row: scale falls back to eps, zero-point stays in range, output is exactly zero
+    out, scale, zp = fq.fq_per_token_int8_asym(torch.zeros(1, 8))
+    assert scale.item() == EPS and -128 <= zp.item() <= 127 and torch.all(out == 0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_per_token_outputs_lie_on_the_grid(dtype):
+    g = torch.Generator().manual_seed(0)
+    x = (torch.randn(16, 256, generator=g) * 3).to(dtype)
+    out, scale, zp = fq.fq_per_token_int8_asym(x)
+    assert out.dtype == dtype and out.shape == x.shape
+    # every output equals dtype(k * scale) for an integer k in [qmin - zp, qmax - zp]
+    k = torch.round(out.float() / scale[:, None])
+    assert torch.all(k >= (-128 - zp)[:, None]) and torch.all(k <= (127 - zp)[:, None])
+    assert bits_equal((k.to(dtype) * scale[:, None]).to(dtype), out)
+    # quantisation error of in-range values is at most half a step (plus the dtype's own rounding)
+    tol = 0.5 * scale[:, None] + out.float().abs() * (2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -23)
+    assert torch.all((out.float() - x.float()).abs() <= tol * 1.0001)
+    # the row extremes are representable: min/max are reproduced within half a step
+    assert torch.all((out.float().amax(1) - x.float().amax(1).clamp(min=0)).abs() <= scale)
+
+
+def test_per_token_fixed_qparams_idempotent():
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(8, 128, generator=g)
+    scale, zp = fq.choose_qparams_per_token_asym(x)
+    _, once = fq._fake_quantize(x, scale, zp, -128, 127)
+    _, twice = fq._fake_quantize(once, scale, zp, -128, 127)
+    assert torch.equal(once, twice)
+
+
+def test_per_token_tiny_exhaustive():
+    # rows of 2 values on a coarse grid: brute-force nearest grid point (ties to even code) must match
+    vals = torch.linspace(-2, 2, 17)
+    for a in vals:
+        for b in vals:
+            x = torch.tensor([[a.item(), b.item()]])
+            out, scale, zp = fq.fq_per_token_int8_asym(x)
+            codes = torch.arange(-128, 128)
+            grid = (codes - zp.item()).float() * scale.item()
+            for j in range(2):
+                pos = x[0, j] * (1.0 / scale.item())
+                q = int(torch.clamp(torch.round(pos) + zp.item(), -128, 127).item())
+                assert out[0, j].item() == grid[q + 128].item()
+                assert abs(out[0, j].item() - x[0, j].item()) <= 0.5 * scale.item() * 1.001
+
+
+def test_per_group_closed_form():
+    # one group [-7.5 .. 7.5]: amax 7.5 -> scale exactly 1; codes = round half to even, clamped to [-8, 7]
+    w = torch.tensor([[-7.5, -6.5, -0.5, 0.5, 1.5, 2.5, 7.4, 7.5]])
+    out, scale = fq.fq_per_group_int4_sym(w, 8)
+    assert scale.item() == 1.0
+    assert out.tolist() == [[-8.0, -6.0, -0.0 + 0.0, 0.0, 2.0, 2.0, 7.0, 7.0]]  # 7.5 -> round 8 -> clamp 7
+    q, s2, zeros = fq.quantize_per_group_int4(w, 8)
+    assert q.dtype == torch.int8 and q.tolist() == [[-8, -6, 0, 0, 2, 2, 7, 7]]
+    assert torch.equal(s2, scale) and torch.all(zeros == 0)
+    # a zero group: eps scale, zero output
+    out, scale = fq.fq_per_group_int4_sym(torch.zeros(1, 8), 8)
+    assert scale.item() == EPS and torch.all(out == 0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("g", [8, 32, 256])
+def test_per_group_invariants(dtype, g):
+    gen = torch.Generator().manual_seed(2)
+    w = (torch.randn(32, 512, generator=gen) * 0.02).to(dtype)
+    out, scale = fq.fq_per_group_int4_sym(w, g)
+    q, s2, _ = fq.quantize_per_group_int4(w, g)
+    assert torch.equal(scale, s2) and scale.shape == (32, 512 // g)
+    assert int(q.min()) >= -8 and int(q.max()) <= 7
+    amax = w.float().view(32, -1, g).abs().amax(-1)
+    assert torch.equal(scale, (amax / 7.5).clamp(min=EPS))
+    # fake-quant output == dequantised convert() output
+    deq = (q.view(32, -1, g).to(dtype) * scale[..., None]).to(dtype).view(32, 512)
+    assert bits_equal(deq, out)
+    # the group's absmax element maps to +-7.5 up to rounding of w * (1/scale) -> code 7, -7 or -8
+    idx = w.float().view(32, -1, g).abs().argmax(-1, keepdim=True)
+    at = q.view(32, -1, g).gather(-1, idx)
+    assert torch.all((at == 7) | (at == -7) | (at == -8) | (amax[..., None] == 0))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_two_restatements_agree(c_oracle, dtype):
+    gen = torch.Generator().manual_seed(3)
+    x = (torch.randn(64, 512, generator=gen) * 2).to(dtype)
+    x[3] = 0
+    x[4] = x[4].abs()
+    ot, st, zt = fq.fq_per_token_int8_asym(x)
+    oc, sc, zc = c_fq_per_token(c_oracle, x)
+    assert bits_equal(ot, oc) and torch.equal(st, sc) and torch.equal(zt, zc)
+    w = (torch.randn(64, 512, generator=gen) * 0.02).to(dtype)
+    w[0, :32] = 0
+    for g in (8, 32, 128):
+        ft, s1 = fq.fq_per_group_int4_sym(w, g)
+        qt, _, _ = fq.quantize_per_group_int4(w, g)
+        fc, qc, s2 = c_fq_per_group(c_oracle, w, g)
+        assert bits_equal(ft, fc) and torch.equal(qt, qc) and torch.equal(s1, s2)
+
+
+def test_straight_through_backward():
+    gen = torch.Generator().manual_seed(4)
+    x = torch.randn(4, 64, generator=gen, requires_grad=True)
+    w = (torch.randn(16, 64, generator=gen) * 0.1).requires_grad_()
+    y = fq.fake_quantized_linear(x, w, 32)
+    gy = torch.randn(4, 16, generator=gen)
+    y.backward(gy)
+    x_fq = fq.fq_per_token_int8_asym(x.detach())[0]
+    w_fq = fq.fq_per_group_int4_sym(w.detach(), 32)[0]
+    torch.testing.assert_close(y, x_fq @ w_fq.T)
+    torch.testing.assert_close(x.grad, gy @ w_fq)  # gradient passes straight through both fake quantisers
+    torch.testing.assert_close(w.grad, gy.T @ x_fq)

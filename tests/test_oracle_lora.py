@@ -1,0 +1,92 @@
+"""Pins the LoRA oracle (oracle/lora_oracle.py) with the reference's own known answers and with closed forms."""
+import json
+import os
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import lora_oracle, nf4_oracle
+
+GOLDEN = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "reference_known_answers.json")))
+
+
+def _fixed_layer(use_bias):
+    fi = lora_oracle.fixed_init_tensor
+    return fi((128, 64)), (fi((128,)) if use_bias else None), fi((4, 64)), fi((128, 4))
+
+
+def _inputs():
+    torch.manual_seed(GOLDEN["lora_forward"]["seed"])
+    return torch.randn(2, 32, 64)
+
+
+def test_reference_known_answer_lora_forward():
+    # tests/torchtune/modules/peft/test_lora.py:111-116 (EXPECTED_VAL = 1.1252)
+    W, b, A, B = _fixed_layer(True)
+    y = lora_oracle.lora_linear_forward(_inputs(), W, A, B, alpha=1.0, rank=4, bias=b)
+    assert y.shape == (2, 32, 128)
+    torch.testing.assert_close(y.mean(), torch.tensor(GOLDEN["lora_forward"]["expected_mean"]), atol=1e-4, rtol=1e-6)
+
+
+def test_reference_known_answer_qat_lora_forward():
+    # tests/torchtune/modules/peft/test_lora.py:239-245 (QAT_EXPECTED_VAL = 0.6291): no bias, identity fake-quant
+    W, _, A, B = _fixed_layer(False)
+    y = lora_oracle.lora_linear_forward(_inputs(), W, A, B, alpha=1.0, rank=4)
+    torch.testing.assert_close(y.mean(), torch.tensor(GOLDEN["qat_lora_forward"]["expected_mean"]), atol=1e-4, rtol=1e-6)
+    # the two known answers differ by mean(bias) of the fixed initialiser
+    assert GOLDEN["lora_forward"]["expected_mean"] - GOLDEN["qat_lora_forward"]["expected_mean"] == pytest.approx(
+        lora_oracle.fixed_init_tensor((128,)).mean().item(), abs=1e-4)
+
+
+def test_matches_the_independent_formula():
+    # tests/torchtune/models/llama2/scripts/compare_lora.py:99-112: F.linear(x, W, b) + (x @ A.T @ B.T) * alpha / r
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(3, 7, 32, generator=g, dtype=torch.float64)
+    W = torch.randn(16, 32, generator=g, dtype=torch.float64)
+    b = torch.randn(16, generator=g, dtype=torch.float64)
+    A = torch.randn(4, 32, generator=g, dtype=torch.float64)
+    B = torch.randn(16, 4, generator=g, dtype=torch.float64)
+    y = lora_oracle.lora_linear_forward(x, W, A, B, alpha=3.0, rank=4, bias=b)
+    torch.testing.assert_close(y, F.linear(x, W, b) + (x @ A.T @ B.T) * (3.0 / 4))
+    torch.testing.assert_close(lora_oracle.lora_linear_forward(x, W, A, B, 3.0, 4, bias=b, disabled=True), F.linear(x, W, b))
+
+
+def test_gradients_closed_form_and_gradcheck():
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(5, 12, generator=g, dtype=torch.float64, requires_grad=True)
+    W = torch.randn(6, 12, generator=g, dtype=torch.float64)
+    A = torch.randn(2, 12, generator=g, dtype=torch.float64, requires_grad=True)
+    B = torch.randn(6, 2, generator=g, dtype=torch.float64, requires_grad=True)
+    s = 16.0 / 2
+    y = lora_oracle.lora_linear_forward(x, W, A, B, alpha=16.0, rank=2)
+    gy = torch.randn(5, 6, generator=g, dtype=torch.float64)
+    y.backward(gy)
+    gh = s * gy @ B.detach()
+    torch.testing.assert_close(x.grad, gy @ W + gh @ A.detach())
+    torch.testing.assert_close(A.grad, gh.T @ x.detach())
+    torch.testing.assert_close(B.grad, s * gy.T @ (x.detach() @ A.detach().T))
+    assert torch.autograd.gradcheck(lambda x_, a_, b_: lora_oracle.lora_linear_forward(x_, W, a_, b_, 16.0, 2), (x, A, B))
+
+
+def test_quantised_base_gives_no_weight_gradient_and_uses_dequantised_weight():
+    g = torch.Generator().manual_seed(2)
+    W = torch.randn(64, 128, generator=g) * 0.02
+    p = nf4_oracle.nf4_quantize(W, 64, 32)
+    x = torch.randn(4, 128, generator=g, requires_grad=True)
+    A = torch.randn(8, 128, generator=g).requires_grad_()
+    B = torch.randn(64, 8, generator=g).requires_grad_()
+    y = lora_oracle.lora_linear_forward(x, p, A, B, alpha=16.0, rank=8)
+    D = nf4_oracle.nf4_dequantize(p)
+    torch.testing.assert_close(y, F.linear(x, D) + 2.0 * (x @ A.T @ B.T))
+    y.sum().backward()
+    torch.testing.assert_close(x.grad, torch.ones(4, 64) @ D + 2.0 * torch.ones(4, 64) @ B.detach() @ A.detach())
+
+
+def test_lora_a_init_bound():
+    a = lora_oracle.lora_a_init_(torch.empty(8, 2048), torch.Generator().manual_seed(0))
+    bound = 1.0 / 2048 ** 0.5  # kaiming-uniform with a = sqrt(5): gain sqrt(1/3), bound = gain * sqrt(3 / fan_in)
+    assert a.abs().max() <= bound and a.abs().max() > 0.99 * bound
+    ref = torch.empty(8, 2048)
+    torch.nn.init.kaiming_uniform_(ref, a=5 ** 0.5)
+    assert ref.abs().max() <= bound

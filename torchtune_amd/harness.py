@@ -1,0 +1,240 @@
+"""A Llama-shaped decoder that drives the quantized linears the way the reference's model does.
+
+The reference composes ``LoRALinear`` / ``FrozenNF4Linear`` inside ``MultiHeadAttention``
+(``torchtune/modules/attention.py:228-303``), ``FeedForward`` (``torchtune/modules/feed_forward.py:50-54``),
+``TransformerSelfAttentionLayer`` (``torchtune/modules/transformer.py:88-141``) and ``TransformerDecoder``
+(``:574-689``), with a chunked output-projection + cross-entropy loss
+(``torchtune/modules/loss/cross_entropy_loss.py:147-188``).  Those classes are not part of the quantized path;
+this file reproduces only their call pattern with stock PyTorch ops so that the benchmark and the smoke test
+exercise the seven projections per layer with the reference's shapes and order:
+
+    RMSNorm -> q, k, v (same input) -> RoPE -> causal GQA attention -> o -> residual
+            -> RMSNorm -> w2(silu(w1 x) * w3 x) -> residual
+
+Shapes come from the reference's builders: ``llama3_2_1b`` (``torchtune/models/llama3_2/_model_builders.py:20-46``),
+``llama3_1_8b`` / ``llama3_1_70b`` (``torchtune/models/llama3_1/_model_builders.py:20-59``); LoRA placement from
+``lora_llama3_attention`` / ``lora_llama3_mlp`` (``torchtune/models/llama3_1/_component_builders.py:338-401,433-456``).
+The output projection is a plain frozen bf16 linear, never NF4 (``_component_builders.py:251-257``).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Optional
+
+import torch
+import torch.nn.functional as F
+from torch import nn
+from torch.utils.checkpoint import checkpoint
+
+from .modules.peft import LoRALinear, get_adapter_params, set_trainable_params
+from .qat import Int8DynActInt4WeightQATQuantizer
+
+
+@dataclass(frozen=True)
+class LlamaShape:
+    name: str
+    n_layers: int
+    dim: int
+    n_heads: int
+    n_kv_heads: int
+    hidden: int
+    vocab: int = 128256
+    rope_base: float = 500000.0
+    norm_eps: float = 1e-5
+
+    @property
+    def head_dim(self) -> int:
+        return self.dim // self.n_heads
+
+
+SHAPES = {
+    "llama3_2_1b": LlamaShape("llama3_2_1b", 16, 2048, 32, 8, 8192),
+    "llama3_1_8b": LlamaShape("llama3_1_8b", 32, 4096, 32, 8, 14336),
+    "llama3_1_70b": LlamaShape("llama3_1_70b", 80, 8192, 64, 8, 28672),
+    # a toy shape for tests: same structure, every dimension still a multiple of 64
+    "tiny": LlamaShape("tiny", 2, 256, 4, 2, 512, vocab=1024),
+}
+
+
+class RMSNorm(nn.Module):
+    """fp32 RMS normalisation (``torchtune/modules/rms_norm.py:28-41``)."""
+
+    def __init__(self, dim: int, eps: float):
+        super().__init__()
+        self.eps = eps
+        self.scale = nn.Parameter(torch.ones(dim))
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        xf = x.float()
+        xf = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + self.eps)
+        return (xf * self.scale.float()).to(x.dtype)
+
+
+def rope_cache(seq_len: int, head_dim: int, base: float, device) -> torch.Tensor:
+    """[seq, head_dim/2, 2] cos/sin table."""
+    theta = 1.0 / (base ** (torch.arange(0, head_dim, 2, device=device, dtype=torch.float32) / head_dim))
+    idx = torch.outer(torch.arange(seq_len, device=device, dtype=torch.float32), theta)
+    return torch.stack([idx.cos(), idx.sin()], dim=-1)
+
+
+def apply_rope(x: torch.Tensor, cache: torch.Tensor) -> torch.Tensor:
+    """x [b, s, n_h, h_d]; rotates interleaved pairs, fp32 math."""
+    xs = x.float().reshape(*x.shape[:-1], -1, 2)
+    c = cache.view(1, xs.size(1), 1, xs.size(3), 2)
+    out = torch.stack(
+        [xs[..., 0] * c[..., 0] - xs[..., 1] * c[..., 1], xs[..., 1] * c[..., 0] + xs[..., 0] * c[..., 1]], dim=-1
+    )
+    return out.flatten(3).to(x.dtype)
+
+
+def _linear(in_dim: int, out_dim: int, rank: int, alpha: float, quantize_base: bool) -> nn.Module:
+    if rank > 0:
+        return LoRALinear(in_dim, out_dim, rank=rank, alpha=alpha, quantize_base=quantize_base)
+    return nn.Linear(in_dim, out_dim, bias=False)
+
+
+class Attention(nn.Module):
+    def __init__(self, s: LlamaShape, rank: int, alpha: float, quantize_base: bool):
+        super().__init__()
+        self.n_heads, self.n_kv, self.head_dim = s.n_heads, s.n_kv_heads, s.head_dim
+        self.q_proj = _linear(s.dim, s.n_heads * s.head_dim, rank, alpha, quantize_base)
+        self.k_proj = _linear(s.dim, s.n_kv_heads * s.head_dim, rank, alpha, quantize_base)
+        self.v_proj = _linear(s.dim, s.n_kv_heads * s.head_dim, rank, alpha, quantize_base)
+        self.output_proj = _linear(s.dim, s.dim, rank, alpha, quantize_base)
+
+    def forward(self, x: torch.Tensor, rope: torch.Tensor) -> torch.Tensor:
+        b, sl, _ = x.shape
+        q = self.q_proj(x).view(b, sl, self.n_heads, self.head_dim)
+        k = self.k_proj(x).view(b, sl, self.n_kv, self.head_dim)
+        v = self.v_proj(x).view(b, sl, self.n_kv, self.head_dim)
+        q = apply_rope(q, rope)
+        k = apply_rope(k, rope)
+        if self.n_kv != self.n_heads:  # expand kv heads to query heads, as the reference does before SDPA
+            rep = self.n_heads // self.n_kv
+            k = k.unsqueeze(3).expand(b, sl, self.n_kv, rep, self.head_dim).flatten(2, 3)
+            v = v.unsqueeze(3).expand(b, sl, self.n_kv, rep, self.head_dim).flatten(2, 3)
+        o = F.scaled_dot_product_attention(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), is_causal=True)
+        return self.output_proj(o.transpose(1, 2).reshape(b, sl, -1))
+
+
+class FeedForward(nn.Module):
+    def __init__(self, s: LlamaShape, rank: int, alpha: float, quantize_base: bool):
+        super().__init__()
+        self.w1 = _linear(s.dim, s.hidden, rank, alpha, quantize_base)  # gate
+        self.w2 = _linear(s.hidden, s.dim, rank, alpha, quantize_base)  # down
+        self.w3 = _linear(s.dim, s.hidden, rank, alpha, quantize_base)  # up
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return self.w2(F.silu(self.w1(x)) * self.w3(x))
+
+
+class DecoderLayer(nn.Module):
+    def __init__(self, s: LlamaShape, rank: int, alpha: float, quantize_base: bool):
+        super().__init__()
+        self.sa_norm = RMSNorm(s.dim, s.norm_eps)
+        self.attn = Attention(s, rank, alpha, quantize_base)
+        self.mlp_norm = RMSNorm(s.dim, s.norm_eps)
+        self.mlp = FeedForward(s, rank, alpha, quantize_base)
+
+    def forward(self, x: torch.Tensor, rope: torch.Tensor) -> torch.Tensor:
+        h = x + self.attn(self.sa_norm(x), rope)
+        return h + self.mlp(self.mlp_norm(h))
+
+
+class Decoder(nn.Module):
+    """Token ids -> final hidden states; ``loss`` adds the chunked output projection + cross entropy."""
+
+    def __init__(self, s: LlamaShape, rank: int, alpha: float, quantize_base: bool, activation_checkpointing: bool = False,
+                 loss_chunks: int = 8):
+        super().__init__()
+        self.shape = s
+        self.ac = activation_checkpointing
+        self.loss_chunks = loss_chunks
+        self.tok_embeddings = nn.Embedding(s.vocab, s.dim)
+        self.layers = nn.ModuleList(DecoderLayer(s, rank, alpha, quantize_base) for _ in range(s.n_layers))
+        self.norm = RMSNorm(s.dim, s.norm_eps)
+        self.output = nn.Linear(s.dim, s.vocab, bias=False)
+
+    def forward(self, tokens: torch.Tensor) -> torch.Tensor:
+        rope = rope_cache(tokens.shape[1], self.shape.head_dim, self.shape.rope_base, tokens.device)
+        h = self.tok_embeddings(tokens)
+        for layer in self.layers:
+            if self.ac and torch.is_grad_enabled():
+                h = checkpoint(layer, h, rope, use_reentrant=False)
+            else:
+                h = layer(h, rope)
+        return self.norm(h)
+
+    def loss(self, tokens: torch.Tensor, labels: torch.Tensor) -> torch.Tensor:
+        """Mean next-token cross entropy; the vocabulary projection is applied chunk by chunk over the sequence."""
+        h = self.forward(tokens)
+        hidden = h.reshape(-1, h.shape[-1])
+        target = labels.reshape(-1)
+        total = hidden.new_zeros((), dtype=torch.float32)
+        for hc, tc in zip(hidden.chunk(self.loss_chunks), target.chunk(self.loss_chunks)):
+            logits = self.output(hc).float()
+            total = total + F.cross_entropy(logits, tc, reduction="sum")
+        return total / target.numel()
+
+
+@torch.no_grad()
+def _init_weights(model: Decoder, seed: int, std: float = 0.02) -> None:
+    """Base weights ~ N(0, std) generated on the device one tensor at a time (an NF4 parameter re-quantises on
+    ``copy_``, so the dense model never exists); lora_b ~ N(0, 0.01) so the adapter path is not a no-op."""
+    dev = model.tok_embeddings.weight.device
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(seed)
+    for name, p in model.named_parameters():
+        if name.endswith("scale"):
+            continue
+        if "lora_a" in name:
+            bound = 1.0 / (p.shape[1] ** 0.5)
+            p.copy_(torch.empty(p.shape, device=dev, dtype=torch.float32).uniform_(-bound, bound, generator=gen))
+        elif "lora_b" in name:
+            p.copy_(torch.randn(p.shape, device=dev, dtype=torch.float32, generator=gen) * 0.01)
+        else:
+            p.copy_((torch.randn(p.shape, device=dev, dtype=torch.float32, generator=gen) * std).to(torch.bfloat16))
+
+
+def build_qlora_decoder(shape: str | LlamaShape, rank: int, alpha: float, device="cuda", seed: int = 0,
+                        activation_checkpointing: bool = False, dtype: torch.dtype = torch.bfloat16) -> Decoder:
+    """QLoRA model: NF4 base + LoRA on all seven projections, everything but the adapters frozen."""
+    s = SHAPES[shape] if isinstance(shape, str) else shape
+    prev = torch.get_default_dtype()
+    torch.set_default_dtype(dtype)
+    try:
+        with torch.device(device):
+            model = Decoder(s, rank, alpha, quantize_base=True, activation_checkpointing=activation_checkpointing)
+    finally:
+        torch.set_default_dtype(prev)
+    _init_weights(model, seed)
+    set_trainable_params(model, get_adapter_params(model))
+    return model
+
+
+def build_qat_decoder(shape: str | LlamaShape, groupsize: int = 32, device="cuda", seed: int = 0,
+                      activation_checkpointing: bool = False, dtype: torch.dtype = torch.bfloat16,
+                      quantize_output: bool = True) -> Decoder:
+    """Full-finetune model prepared for 8da4w QAT: every linear swapped for the fake-quantised one."""
+    s = SHAPES[shape] if isinstance(shape, str) else shape
+    prev = torch.get_default_dtype()
+    torch.set_default_dtype(dtype)
+    try:
+        with torch.device(device):
+            model = Decoder(s, 0, 0.0, quantize_base=False, activation_checkpointing=activation_checkpointing)
+    finally:
+        torch.set_default_dtype(prev)
+    _init_weights(model, seed)
+    quantizer = Int8DynActInt4WeightQATQuantizer(groupsize=groupsize, precision=dtype)
+    if quantize_output:
+        quantizer.prepare(model)
+    else:
+        quantizer.prepare(model.layers)
+    return model
+
+
+def train_step(model: Decoder, tokens: torch.Tensor, labels: torch.Tensor) -> torch.Tensor:
+    """One forward + backward; returns the detached loss."""
+    loss = model.loss(tokens, labels)
+    loss.backward()
+    return loss.detach()

@@ -289,6 +289,9 @@ def _nf4_copy_(func, args, kwargs):
     if not isinstance(dst, NF4Tensor):
         # dense.copy_(nf4): materialise
         return func(dst, src.get_original_weight(), **kwargs)
+    # in-place writes issued from inside __torch_dispatch__ do not advance the version counters the
+    # block-scaler cache is keyed on, so drop the cache explicitly
+    dst.quantized_scalers._ttamd_block_scalers = None
     if isinstance(src, NF4Tensor):
         same_meta = (
             src.block_size == dst.block_size

@@ -111,6 +111,17 @@ def nf4_block_scalers(qscalers: torch.Tensor, qfactor: torch.Tensor, mean: torch
 # ---------------------------------------------------------------------------------------------------
 # fused NF4 + LoRA linear
 # ---------------------------------------------------------------------------------------------------
+_gemm_timer = None
+
+
+def set_gemm_timer(timer) -> None:
+    """Install (or with None remove) a callback ``timer(kind, M, N, K, rank) -> (start_event, end_event)``; the two
+    events are recorded on the launch stream immediately before and after every fused-GEMM launch.  Used by the
+    benchmark to time the dominant kernel in place."""
+    global _gemm_timer
+    _gemm_timer = timer
+
+
 def fused_shape_ok(N: int, K: int, rank: int) -> bool:
     """Shapes the fused bf16 GEMM accepts (NF4 block_size must also be 64)."""
     return K % 64 == 0 and N % 64 == 0 and rank % 8 == 0 and 0 <= rank <= 64
@@ -158,10 +169,15 @@ def nf4_lora_linear_fwd(
     y = torch.empty(M, N, dtype=torch.bfloat16, device=x.device)
     lib = _lib.load()
     with torch.cuda.device(x.device):
+        events = _gemm_timer("fwd", M, N, K, rank) if _gemm_timer is not None else None
+        if events:
+            events[0].record()
         rc = lib.ttamd_nf4_lora_linear_fwd_bf16(
             x.data_ptr(), qdata.data_ptr(), block_scalers.data_ptr(), _ptr(h), _ptr(lora_b), rank, float(scale), _ptr(bias),
             y.data_ptr(), M, N, K, _stream(x),
         )
+        if events:
+            events[1].record()
     _lib.check(rc, "nf4_lora_linear_fwd")
     return y
 
@@ -181,10 +197,15 @@ def nf4_linear_bwd_dx(
     gx = torch.empty(M, K, dtype=torch.bfloat16, device=gy.device)
     lib = _lib.load()
     with torch.cuda.device(gy.device):
+        events = _gemm_timer("bwd", M, N, K, rank) if _gemm_timer is not None else None
+        if events:
+            events[0].record()
         rc = lib.ttamd_nf4_linear_bwd_dx_bf16(
             gy.data_ptr(), qdata.data_ptr(), block_scalers.data_ptr(), _ptr(gh), _ptr(lora_a), rank, gx.data_ptr(), M, N, K,
             _stream(gy),
         )
+        if events:
+            events[1].record()
     _lib.check(rc, "nf4_linear_bwd_dx")
     return gx
 

@@ -65,8 +65,8 @@ class FakeQuantizeConfig:
         if dtype not in (torch.int8, torch.int4):
             raise NotImplementedError(f"FakeQuantizeConfig: dtype {dtype} has no kernel (int8 and int4 do)")
         self.dtype = dtype
-        if granularity is not None and group_size is not None:
-            raise ValueError("Cannot set both `granularity` and `group_size`")
+        if group_size is not None and granularity is not None and granularity != "per_group":
+            raise ValueError("`group_size` conflicts with granularity '%s'" % (granularity,))
         if isinstance(granularity, str):
             if granularity == "per_token":
                 granularity = PerToken()
