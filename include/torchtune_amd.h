@@ -95,8 +95,9 @@ int ttamd_nf4_dequantize(const uint8_t* quantized_data, const int8_t* quantized_
  * ---------------------------------------------------------------------------------------------- */
 
 /*
- * Dequantised block scalers of an NF4 tensor, one bf16 per 64-element block:
- *     block_scalers[b] = bf16( dtype( dtype(quantized_scalers[b] / quantization_factor[b / SB]) + scaler_mean ) )
+ * Dequantised block scalers of an NF4 tensor, one fp32 per 64-element block (the value is the tensor-dtype
+ * result, widened exactly):
+ *     block_scalers[b] = float( dtype( dtype(quantized_scalers[b] / quantization_factor[b / SB]) + scaler_mean ) )
  * This is the `dequantize_scalers` step of NF4Tensor.get_original_weight (torchao; reached from lora.py:138 on
  * every call).  The weight is frozen, so callers compute it once per tensor and keep it; the GEMMs below take it
  * in place of the three scaler tensors.  `dtype` is the dtype of quantization_factor / scaler_mean.

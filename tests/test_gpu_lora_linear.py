@@ -167,7 +167,7 @@ def test_raw_c_abi_sequence_matches_python_layer():
     t = to_nf4(W.to(DEV), 64, sbs)
     xd, gyd, Ad, Bd = x.to(DEV), gy.to(DEV), A.to(DEV), B.to(DEV)
     stream = torch.cuda.current_stream().cuda_stream
-    bscal = torch.empty(t.n_blocks, dtype=BF, device=DEV)
+    bscal = torch.empty(t.n_blocks, dtype=torch.float32, device=DEV)
     assert lib.ttamd_nf4_block_scalers(t.quantized_scalers.data_ptr(), t.quantization_factor.data_ptr(), t.scaler_mean.data_ptr(), 0,
                                        t.n_blocks, sbs, bscal.data_ptr(), stream) == 0
     ws = torch.empty(max(lib.ttamd_lora_fwd_workspace_bytes(M, K, r), lib.ttamd_lora_bwd_workspace_bytes(M, N, K, r)),

@@ -41,7 +41,7 @@ __device__ __forceinline__ float bf16hi(uint32_t d) { return bits_f32(d & 0xffff
 struct GemmArgs {
   const uint16_t* A;      // [M, Kc] bf16: x (forward) or gy (backward)
   const uint8_t* qdata;   // NF4 codes of W [N, K]
-  const uint16_t* bscal;  // dequantised block scalers, bf16 [N*K/64]
+  const float* bscal;     // dequantised block scalers, fp32 [N*K/64]
   const uint16_t* lA;     // adapter operand on the A side: h (forward) or gh (backward), [M, R] bf16, or null
   const uint16_t* lB;     // adapter operand on the W side: lora_b [N, R] (forward) or lora_a [R, K] (backward)
   const uint16_t* bias;   // [N] bf16 or null (forward only)
@@ -138,14 +138,14 @@ __global__ __launch_bounds__(256) void nf4_gemm_kernel(const GemmArgs g) {
         u32x2_t v0 = reinterpret_cast<const u32x2_t*>(src)[0];
         wq[0] = v0.x; wq[1] = v0.y;
       }
-      wscal[0] = bf16_bits_to_f32(g.bscal[(int64_t)f_n * kblocks_per_row + kt]);
+      wscal[0] = g.bscal[(int64_t)f_n * kblocks_per_row + kt];
     } else {
       if (b_active) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
           const int n = k0 + b_ng * 8 + i;  // contraction index: always < N because N % 64 == 0
           wq[i] = *reinterpret_cast<const uint32_t*>(g.qdata + (((int64_t)n * g.K + b_kcol) >> 1));
-          wscal[i] = bf16_bits_to_f32(g.bscal[(int64_t)n * kblocks_per_row + (b_kcol >> 6)]);
+          wscal[i] = g.bscal[(int64_t)n * kblocks_per_row + (b_kcol >> 6)];
         }
       }
     }
@@ -297,11 +297,11 @@ __global__ __launch_bounds__(256) void nf4_gemm_kernel(const GemmArgs g) {
   }
 }
 
-// bf16 block scalers: scaler[b] = dtype(dtype(int8[b] / factor[b / SB]) + mean), then cast to bf16.
+// block scalers: scaler[b] = dtype(dtype(int8[b] / factor[b / SB]) + mean), widened to fp32 (exact).
 template <bool BF16>
 __global__ __launch_bounds__(256) void nf4_block_scalers_kernel(const int8_t* __restrict__ qs, const void* __restrict__ qf,
                                                                 const void* __restrict__ mean, int64_t n_blocks, int SB,
-                                                                uint16_t* __restrict__ out) {
+                                                                float* __restrict__ out) {
   const int64_t b = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (b >= n_blocks) return;
   float f, m;
@@ -312,7 +312,7 @@ __global__ __launch_bounds__(256) void nf4_block_scalers_kernel(const int8_t* __
     f = reinterpret_cast<const float*>(qf)[b / SB];
     m = reinterpret_cast<const float*>(mean)[0];
   }
-  out[b] = f32_to_bf16_bits(nf4_block_scaler<BF16>((int)qs[b], f, m));
+  out[b] = nf4_block_scaler<BF16>((int)qs[b], f, m);
 }
 
 template <int BM, int BN, bool TRANS_W>
@@ -359,6 +359,11 @@ int check_gemm_args(const char* who, const void* a, const uint8_t* qdata, const 
 }
 
 }  // namespace
+
+// nf4_gemm_rs.hip
+int run_gemm_rs(const void* X, const uint8_t* codes, const void* scal, bool per_elem, const void* lX, const void* lW,
+                bool lw_row_major, int R, float lscale, const void* bias, void* C, int64_t M, int64_t Nout, int64_t Kc,
+                hipStream_t s);
 }  // namespace ttamd
 
 using namespace ttamd;
@@ -375,10 +380,10 @@ extern "C" int ttamd_nf4_block_scalers(const int8_t* quantized_scalers, const vo
   const dim3 grid((unsigned)((n_blocks + 255) / 256)), block(256);
   if (dtype == TTAMD_BF16)
     nf4_block_scalers_kernel<true><<<grid, block, 0, s>>>(quantized_scalers, quantization_factor, scaler_mean, n_blocks,
-                                                          scaler_block_size, reinterpret_cast<uint16_t*>(block_scalers));
+                                                          scaler_block_size, reinterpret_cast<float*>(block_scalers));
   else
     nf4_block_scalers_kernel<false><<<grid, block, 0, s>>>(quantized_scalers, quantization_factor, scaler_mean, n_blocks,
-                                                           scaler_block_size, reinterpret_cast<uint16_t*>(block_scalers));
+                                                           scaler_block_size, reinterpret_cast<float*>(block_scalers));
   return check_launch("nf4_block_scalers");
 }
 
@@ -386,17 +391,8 @@ extern "C" int ttamd_nf4_lora_linear_fwd_bf16(const void* x, const uint8_t* quan
                                               const void* h, const void* lora_b, int rank, float scale, const void* bias,
                                               void* y, int64_t M, int64_t N, int64_t K, void* stream) {
   if (int rc = check_gemm_args("nf4_lora_linear_fwd", x, quantized_data, block_scalers, y, M, N, K, rank, h, lora_b)) return rc;
-  GemmArgs g;
-  g.A = reinterpret_cast<const uint16_t*>(x);
-  g.qdata = quantized_data;
-  g.bscal = reinterpret_cast<const uint16_t*>(block_scalers);
-  g.lA = reinterpret_cast<const uint16_t*>(h);
-  g.lB = reinterpret_cast<const uint16_t*>(lora_b);
-  g.bias = reinterpret_cast<const uint16_t*>(bias);
-  g.C = reinterpret_cast<uint16_t*>(y);
-  g.M = (int)M; g.N = (int)N; g.K = (int)K; g.R = rank;
-  g.lscale = scale;
-  return dispatch_gemm<false>(g, reinterpret_cast<hipStream_t>(stream));
+  return run_gemm_rs(x, quantized_data, block_scalers, false, h, lora_b, true, rank, scale, bias, y, M, N, K,
+                     reinterpret_cast<hipStream_t>(stream));
 }
 
 extern "C" int ttamd_nf4_linear_bwd_dx_bf16(const void* gy, const uint8_t* quantized_data, const void* block_scalers,
@@ -406,7 +402,7 @@ extern "C" int ttamd_nf4_linear_bwd_dx_bf16(const void* gy, const uint8_t* quant
   GemmArgs g;
   g.A = reinterpret_cast<const uint16_t*>(gy);
   g.qdata = quantized_data;
-  g.bscal = reinterpret_cast<const uint16_t*>(block_scalers);
+  g.bscal = reinterpret_cast<const float*>(block_scalers);
   g.lA = reinterpret_cast<const uint16_t*>(gh);
   g.lB = reinterpret_cast<const uint16_t*>(lora_a);
   g.bias = nullptr;

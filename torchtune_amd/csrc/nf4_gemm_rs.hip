@@ -1,0 +1,462 @@
+// Fused NF4-dequantise + bf16 MFMA GEMM, second generation: the weight operand never goes through LDS as bf16.
+//
+//     C[M, Nout] = X[M, Kc] . D(Wv)[Nout, Kc]^T  (+ bias)  + (lscale . lX)[M, R] . lW[Nout, R]^T
+//
+// `Wv` is a "weight view" whose rows are output columns and whose packed 4-bit codes run along the
+// contraction dimension:
+//   forward  : Wv = W   [N, K]  (the NF4 tensor as stored),   one scaler per row per 64 contraction elements
+//   backward : Wv = W^T [K, N]  (a transposed copy of the codes), one scaler per contraction element per
+//              64 output columns (NF4 blocks run along K, i.e. along the output columns of this view)
+//
+// Work split.  256 threads = 4 waves; the workgroup owns a BM x 256 tile of C, wave w the 64 output columns
+// [64w, 64w+64) for ALL BM rows.  A lane of the MFMA weight operand needs 8 consecutive contraction elements
+// of one output column: exactly one dword of codes.  Each lane expands its own code dwords in registers
+// (byte -> pair of fp32 code points from a 256-entry LDS table, multiply by the scaler in fp32, round to bf16:
+// bit-identical to the stand-alone dequantise kernel) one k-substep ahead of the MFMA that consumes them.
+//
+// Every global read of the main loop is a direct-to-LDS load (global_load_lds_*): the activation tile with an
+// XOR swizzle applied on the global-address side, the code bytes and the scalers into wave-private slots.
+// That keeps the vector-memory counter free of register-destination loads, so a single explicit
+// `s_waitcnt vmcnt(one batch)` per k-step lets the next batch stay in flight (prefetch distance two k-steps;
+// four activation stages so that one workgroup barrier per k-step suffices).
+//
+// Per 64-wide k-step a wave issues 64 v_mfma_f32_32x32x16_bf16 against ~2.5 VALU ops per weight element,
+// 12 direct-to-LDS loads, BM/32 x 4 operand reads and 32 table reads.
+#include <stdlib.h>
+
+#include "common.h"
+#include "nf4_math.h"
+
+namespace ttamd {
+namespace {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+
+__device__ __constant__ float kNF4Rs[16] = TT_NF4_TABLE;
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  bf16x2_t v;
+  v.x = (__bf16)lo;
+  v.y = (__bf16)hi;
+  return __builtin_bit_cast(uint32_t, v);
+}
+
+#define TT_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
+#ifndef TT_EXP
+#define TT_EXP 0
+#endif
+
+struct RsArgs {
+  const uint16_t* X;     // [M, Kc] bf16 activations
+  const uint8_t* codes;  // [Nout, Kc/2] packed NF4 codes of the weight view
+  const float* scal;     // !PER_ELEM: fp32 [Nout, Kc/64];  PER_ELEM: fp32 [Nout/64, Kc]
+  const uint16_t* lX;    // adapter activations [M, R] bf16 or null
+  const uint16_t* lW;    // adapter weights: [Nout, R] (lw_row_major) or [R, Nout] bf16, or null
+  const uint16_t* bias;  // [Nout] bf16 or null
+  uint16_t* C;           // [M, Nout] bf16
+  int M, Nout, Kc, R;
+  int lw_row_major;
+  float lscale;
+  int tiles_m, tiles_n;
+  long long* dbg;
+};
+
+constexpr int kBN = 256;
+constexpr int kLutBytes = 256 * 8;  // 256 byte values x (fp32 nf4[hi nibble], fp32 nf4[lo nibble])
+
+// LDS: a ring of 4 activation tiles (shared by the waves), a ring of 3 wave-private {code bytes, scalers} slots, the table
+template <int BM>
+struct RsLayout {
+  static constexpr int kStageA = BM * 128;   // activation tile: BM rows x 64 bf16
+  static constexpr int kAStages = 4;
+  static constexpr int kWOff = kAStages * kStageA;
+  static constexpr int kStageW = 8192 + 2048;  // code bytes [wave][tile j][lane] x 16 B, then scalers [wave] x 512 B
+  static constexpr int kWStages = 3;
+  static constexpr int kLutOff = kWOff + kWStages * kStageW;
+  static constexpr int kTotal = kLutOff;  // dynamic part; the table is a static LDS object of kLutBytes
+};
+
+template <int BM, bool PER_ELEM>
+__global__ __launch_bounds__(256) void nf4_gemm_rs_kernel(const RsArgs g) {
+#if defined(__HIP_DEVICE_COMPILE__)  // the body uses LDS address-space casts and gfx950 builtins the host pass cannot parse
+  static_assert(BM == 256 || BM == 128, "BM");
+  using L = RsLayout<BM>;
+  constexpr int MT = BM / 32;       // activation tiles (MFMA columns) per wave
+  constexpr int NT = 2;             // weight tiles (MFMA rows) per wave
+  constexpr int kALoads = BM / 32;  // direct-to-LDS instructions per wave per k-step for the activation tile (8 rows each)
+  constexpr int kBatch = kALoads + NT + (PER_ELEM ? 1 : NT);  // vector-memory operations per wave per k-step
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l31 = lane & 31, h = lane >> 5;
+  long long tstamp[6];
+  tstamp[0] = wall_clock64();
+
+  int tile_m, tile_n;
+  {
+    // workgroup ids are dealt round-robin to the 8 XCDs (one L2 each): give every XCD a band of m-tiles
+    const int id = blockIdx.x;
+    if ((g.tiles_m & 7) == 0) {
+      const int xcd = id & 7, slot = id >> 3;
+      tile_m = xcd * (g.tiles_m >> 3) + slot / g.tiles_n;
+      tile_n = slot % g.tiles_n;
+    } else {
+      tile_m = id / g.tiles_n;
+      tile_n = id % g.tiles_n;
+    }
+  }
+  const int m0 = tile_m * BM, n0 = tile_n * kBN;
+  const int Kc = g.Kc;
+  const int nk = Kc >> 6;
+
+  // ---- table: entry(byte) = (nf4[byte >> 4], nf4[byte & 15]) as two fp32 (each exactly a bf16 value)
+  //      It is a separate LDS object so that the compiler can tell table reads from the direct-to-LDS destinations.
+  __shared__ float2 lut_s[256];
+  lut_s[tid] = make_float2(round_to_bf16(kNF4Rs[tid >> 4]), round_to_bf16(kNF4Rs[tid & 15]));
+  const char* lut = reinterpret_cast<const char*>(lut_s);
+
+  // ---- activation tile.  A row is eight 16-byte chunks; chunk c of row r is stored in slot c ^ ((r >> 1) & 7), which
+  //      makes the 128-bit operand reads below bank-conflict free.  A direct-to-LDS instruction writes lane l to
+  //      linear slot l, so the lane fetches the chunk that belongs there.
+  const int a_r8 = lane >> 3;
+  uint32_t a_off[kALoads];  // byte offset of this lane's chunk from X + k0
+#pragma unroll
+  for (int i = 0; i < kALoads; ++i) {
+    const int trow = wv * (BM / 4) + 8 * i + a_r8;  // row inside the tile
+    const int chunk = (lane & 7) ^ ((trow >> 1) & 7);
+    int row = m0 + trow;
+    row = row < g.M ? row : g.M - 1;
+    a_off[i] = ((uint32_t)row * (uint32_t)Kc + chunk * 8) * 2u;
+  }
+  // ---- weight view rows of this lane: tile j -> output column n0 + 64 wv + 32 j + l31; half h owns code bytes [16h, 16h+16)
+  uint32_t w_off[NT], s_off[NT];  // byte offsets from codes + k0/2 and from scal + tk
+#pragma unroll
+  for (int j = 0; j < NT; ++j) {
+    int col = n0 + wv * 64 + 32 * j + l31;
+    col = col < g.Nout ? col : g.Nout - 1;
+    w_off[j] = (uint32_t)(((int64_t)col * Kc) >> 1) + 16 * h;
+    s_off[j] = (uint32_t)col * (uint32_t)nk * 4u;
+  }
+  if constexpr (PER_ELEM) {
+    // scalers of the wave's 64-column block for the 64 contraction elements of a k-step: lane l fetches element l
+    int ob = (n0 >> 6) + wv;
+    const int nob = g.Nout >> 6;
+    ob = ob < nob ? ob : nob - 1;
+    s_off[0] = ((uint32_t)ob * (uint32_t)Kc + lane) * 4u;
+  }
+
+  // Direct-to-LDS loads are written as inline assembly: `voff` is this lane's 32-bit byte offset from the uniform
+  // `base`, the wave's 64 lanes land in LDS at `lds`, `lds` + size, ...  Issued this way the compiler keeps no
+  // bookkeeping for them (it would otherwise wait for ALL outstanding loads before the next LDS read it cannot prove
+  // disjoint); completion is awaited explicitly with s_waitcnt vmcnt below.
+  auto dma16 = [&](uint32_t voff, const char* base, uint32_t lds) {
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(base), "s"(lds) : "memory");
+  };
+  auto dma4 = [&](uint32_t voff, const char* base, uint32_t lds) {
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dword %0, %1" ::"v"(voff), "s"(base), "s"(lds) : "memory");
+  };
+  const uint32_t lds0 = (uint32_t)(uintptr_t)TT_LDS_PTR(smem);
+  // A batch (k-step t) is kBatch loads: the activation tile -> A stage, this wave's code bytes and scalers -> W stage.
+  // They are issued one at a time between MFMAs (slot d of the batch), never back to back: the address unit takes
+  // tens of cycles per 64-lane load and a wave that finds its queue full cannot issue anything else meanwhile.
+  struct BatchAddr {
+    const char *xb, *cb, *sb;
+    uint32_t abase, wbase;
+  };
+  auto batch_addr = [&](int t, int sa, int sw) -> BatchAddr {
+    const int tk = t < nk ? t : nk - 1;  // past the end: reload the last tile (never consumed)
+    BatchAddr b;
+    b.xb = reinterpret_cast<const char*>(g.X) + ((int64_t)tk << 7);      // + k0 * 2 bytes
+    b.cb = reinterpret_cast<const char*>(g.codes) + ((int64_t)tk << 5);  // + k0 / 2 bytes
+    b.sb = reinterpret_cast<const char*>(g.scal) + (PER_ELEM ? ((int64_t)tk << 8) : ((int64_t)tk << 2));
+    b.abase = lds0 + sa * L::kStageA + wv * (BM / 4) * 128;
+    b.wbase = lds0 + L::kWOff + sw * L::kStageW;
+    return b;
+  };
+  auto issue_one = [&](const BatchAddr& b, int d) {  // d is a compile-time constant after unrolling
+    if (TT_EXP & 1) return;
+    if (d < kALoads) {
+      dma16(a_off[d], b.xb, b.abase + d * 1024);
+    } else if (d < kALoads + NT) {
+      const int j = d - kALoads;
+      dma16(w_off[j], b.cb, b.wbase + (wv * NT + j) * 1024);
+    } else if (d < kBatch) {
+      const int j = d - kALoads - NT;
+      dma4(s_off[j], b.sb, b.wbase + 8192 + wv * 512 + j * 256);
+    }
+  };
+  auto issue = [&](int t, int sa, int sw) {
+    const BatchAddr b = batch_addr(t, sa, sw);
+#pragma unroll
+    for (int d = 0; d < kBatch; ++d) issue_one(b, d);
+  };
+
+  // weights of one k-substep: a code byte -> one fp32 pair from the table (fetch), scaled and rounded to bf16 (finish)
+  uint32_t codes[NT][4];  // this lane's code dwords of the k-step being expanded: [tile][k-substep]
+  float sc[NT], sc_next[NT];
+  float2 pend[NT][4];     // table entries fetched in one phase, finished in the next: [tile][code byte]
+  u32x4_t wfa[NT], wfb[NT];  // weight operands (8 bf16 each) of two consecutive k-substeps
+  bf16x8_t xfa[MT], xfb[MT];
+
+  auto fetch_byte = [&](int j, int ks, int b) {
+    if (TT_EXP & 2) return;
+    pend[j][b] = *reinterpret_cast<const float2*>(lut + (((codes[j][ks] >> (8 * b)) & 0xffu) << 3));
+  };
+  // finish byte b of tile j into wf[j]; s8 = the eight per-element scalers of the substep (PER_ELEM), s = the row's scaler
+  auto finish_byte = [&](u32x4_t (&wf)[NT], int j, int b, const float (&s)[NT], const float (&s8)[8]) {
+    if (TT_EXP & 2) return;
+    if constexpr (PER_ELEM)
+      wf[j][b] = pack_bf16x2(pend[j][b].x * s8[2 * b], pend[j][b].y * s8[2 * b + 1]);
+    else
+      wf[j][b] = pack_bf16x2(pend[j][b].x * s[j], pend[j][b].y * s[j]);
+  };
+  auto load_s8 = [&](float (&s8)[8], int sw, int ks) {
+    if constexpr (PER_ELEM) {
+      const f32x4_t* sp = reinterpret_cast<const f32x4_t*>(smem + L::kWOff + sw * L::kStageW + 8192 + wv * 512 + (32 * h + 8 * ks) * 4);
+      const f32x4_t a = sp[0], b = sp[1];
+      s8[0] = a.x; s8[1] = a.y; s8[2] = a.z; s8[3] = a.w; s8[4] = b.x; s8[5] = b.y; s8[6] = b.z; s8[7] = b.w;
+    }
+  };
+  auto load_codes = [&](int sw, float (&s_out)[NT]) {
+    const char* wbase = smem + L::kWOff + sw * L::kStageW;
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+      const u32x4_t v = *reinterpret_cast<const u32x4_t*>(wbase + (wv * NT + j) * 1024 + lane * 16);
+      codes[j][0] = v.x; codes[j][1] = v.y; codes[j][2] = v.z; codes[j][3] = v.w;
+      if constexpr (!PER_ELEM) s_out[j] = *reinterpret_cast<const float*>(wbase + 8192 + wv * 512 + j * 256 + lane * 4);
+    }
+  };
+
+  f32x16_t acc[NT][MT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j)
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[j][i][v] = 0.f;
+
+  // operand read offsets inside a stage: row 32 i + l31, chunk 4h + ks, slot = chunk ^ ((row >> 1) & 7)
+  int x_off[4];
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) x_off[ks] = l31 * 128 + (((4 * h + ks) ^ ((l31 >> 1) & 7)) << 4);
+
+  // One phase = the 16 (NT x MT) MFMAs of a k-substep, cut into quarters.  Quarter q:
+  //   MFMAs of weight tile q/2 against activation tiles [MT/2 (q%2), +MT/2)
+  //   operand reads of the NEXT phase: activation tiles [MT/4 q, +MT/4)
+  //   finish + fetch of code bytes 2(q%2), 2(q%2)+1 of weight tile q/2 (finish: previous fetch -> wf_next)
+  //   up to two direct-to-LDS loads of batch `b` (slots d0, d0+1)
+  // and the scheduler is asked to alternate MFMA / VALU / LDS inside the quarter.
+  auto phase = [&](const bf16x8_t (&xf_use)[MT], const u32x4_t (&wf_use)[NT], bf16x8_t (&xf_next)[MT], int st_next, int ks_next,
+                   u32x4_t (&wf_next)[NT], const float (&s_fin)[NT], int sw_fin, int ks_fin, int ks_fetch, const BatchAddr& b,
+                   int d_first, int d_per_quarter_even, int d_per_quarter_odd) {
+    float s8[8];
+    load_s8(s8, sw_fin, ks_fin);
+    const char* sA = smem + st_next * L::kStageA;
+    int d = d_first;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int j = q >> 1;
+      const int nd = (q & 1) ? d_per_quarter_odd : d_per_quarter_even;
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+        if (u < nd) issue_one(b, d + u);
+      d += nd;
+#pragma unroll
+      for (int i = (MT / 4) * q; i < (MT / 4) * (q + 1); ++i)
+        xf_next[i] = *reinterpret_cast<const bf16x8_t*>(sA + i * 4096 + x_off[ks_next]);
+#pragma unroll
+      for (int i = (MT / 2) * (q & 1); i < (MT / 2) * ((q & 1) + 1); ++i)
+        acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, wf_use[j]), xf_use[i], acc[j][i], 0, 0, 0);
+#pragma unroll
+      for (int bb = 2 * (q & 1); bb < 2 * (q & 1) + 2; ++bb) {
+        finish_byte(wf_next, j, bb, s_fin, s8);
+        fetch_byte(j, ks_fetch, bb);
+      }
+#pragma unroll
+      for (int r = 0; r < MT / 2; ++r) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
+        __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);  // VALU
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+  // ---- software pipeline.  Activation tile t lives in A stage t % 4, this wave's codes of k-step t in W stage t % 3.
+  // Step t:
+  //   phase 0,1 : MFMAs on substeps 0,1 of tile t; batch t+2 is issued, one load per quarter phase
+  //   wait for this wave's batch t+1 (batch t+2 stays in flight); barrier: tile t+1 is visible to all waves
+  //   phase 2,3 : MFMAs on substeps 2,3; codes of k-step t+1 are read back; phase 3 pre-reads the operands of step t+1
+  // That one barrier per step also orders stage reuse: a wave issuing batch t+2 into the A stage of tile t-2 has
+  // passed barrier t-1, which every wave reaches only after finishing step t-2.  W stages are wave-private.
+  // Weights are expanded just in time: substep ks is fetched two phases and finished one phase before its MFMAs.
+  issue(0, 0, 0);
+  issue(1, 1, 1);
+  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kBatch) : "memory");  // batch 0 landed everywhere, table written
+  load_codes(0, sc);
+  {
+    float s8[8];
+    load_s8(s8, 0, 0);
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        fetch_byte(j, 0, b);
+        finish_byte(wfa, j, b, sc, s8);
+        fetch_byte(j, 1, b);
+      }
+  }
+#pragma unroll
+  for (int i = 0; i < MT; ++i) xfa[i] = *reinterpret_cast<const bf16x8_t*>(smem + i * 4096 + x_off[0]);
+  tstamp[1] = wall_clock64();
+
+  constexpr int kDEven = (kBatch + 7) / 8 > 1 ? 2 : 1;  // loads per even quarter over the 8 quarters of phases 0 and 1
+  constexpr int kDOdd = (kBatch - 4 * kDEven + 3) / 4;  // and per odd quarter
+  static_assert(4 * kDEven + 4 * kDOdd >= kBatch && kDOdd <= 2 && kDOdd >= 0, "batch does not fit the 8 quarter phases");
+  int a0 = 0, w0 = 0;  // A / W stage of k-step kt
+  for (int kt = 0; kt < nk; ++kt) {
+    const int a1 = (a0 + 1) & 3, a2 = (a0 + 2) & 3;
+    const int w1 = w0 == 2 ? 0 : w0 + 1, w2 = w1 == 2 ? 0 : w1 + 1;
+    const BatchAddr b = batch_addr(kt + 2, a2, w2);
+    phase(xfa, wfa, xfb, a0, 1, wfb, sc, w0, 1, 2, b, 0, kDEven, kDOdd);
+    phase(xfb, wfb, xfa, a0, 2, wfa, sc, w0, 2, 3, b, 2 * (kDEven + kDOdd), kDEven, kDOdd);
+    if (TT_EXP & 8) asm volatile("s_barrier" ::: "memory");
+    else if (!(TT_EXP & 4)) asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kBatch) : "memory");
+    load_codes(w1, sc_next);
+    phase(xfa, wfa, xfb, a0, 3, wfb, sc, w0, 3, 0, b, kBatch, 0, 0);
+    phase(xfb, wfb, xfa, a1, 0, wfa, sc_next, w1, 0, 1, b, kBatch, 0, 0);
+#pragma unroll
+    for (int j = 0; j < NT; ++j) sc[j] = sc_next[j];
+    a0 = a1;
+    w0 = w1;
+  }
+
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the clamped batches issued by the last two steps
+  tstamp[2] = wall_clock64();
+  // ---- adapter: R extra contraction steps, operands straight from global memory
+  if (g.R > 0) {
+    for (int rc = 0; rc < g.R; rc += 16) {
+      const int r0 = rc + 8 * h;
+      const bool in = r0 < g.R;  // R % 8 == 0: a lane's 8 indices are all in or all out
+      bf16x8_t wfr[NT], xfr[MT];
+#pragma unroll
+      for (int j = 0; j < NT; ++j) {
+        int col = n0 + wv * 64 + 32 * j + l31;
+        col = col < g.Nout ? col : g.Nout - 1;
+        u32x4_t raw = {0, 0, 0, 0};
+        if (in) {
+          if (g.lw_row_major) {
+            raw = *reinterpret_cast<const u32x4_t*>(g.lW + (int64_t)col * g.R + r0);
+          } else {
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+              const uint32_t lo = g.lW[(int64_t)(r0 + 2 * d) * g.Nout + col];
+              const uint32_t hi = g.lW[(int64_t)(r0 + 2 * d + 1) * g.Nout + col];
+              raw[d] = lo | (hi << 16);
+            }
+          }
+        }
+        wfr[j] = __builtin_bit_cast(bf16x8_t, raw);
+      }
+#pragma unroll
+      for (int i = 0; i < MT; ++i) {
+        int row = m0 + 32 * i + l31;
+        row = row < g.M ? row : g.M - 1;
+        u32x4_t raw = {0, 0, 0, 0};
+        if (in) raw = *reinterpret_cast<const u32x4_t*>(g.lX + (int64_t)row * g.R + r0);
+        if (g.lscale != 1.0f) {
+#pragma unroll
+          for (int d = 0; d < 4; ++d)
+            raw[d] = pack_bf16x2(bits_f32(raw[d] << 16) * g.lscale, bits_f32(raw[d] & 0xffff0000u) * g.lscale);
+        }
+        xfr[i] = __builtin_bit_cast(bf16x8_t, raw);
+      }
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+          acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wfr[j], xfr[i], acc[j][i], 0, 0, 0);
+    }
+  }
+
+  tstamp[3] = wall_clock64();
+  // ---- epilogue.  acc[j][i][v] = C[m][n] with m = m0 + 32 i + l31 and n = n0 + 64 wv + 32 j + 8 (v/4) + 4 h + v%4:
+  //      four consecutive n per lane -> one 8-byte store
+#pragma unroll
+  for (int j = 0; j < NT; ++j)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int n = n0 + wv * 64 + 32 * j + 8 * q + 4 * h;
+      if (n >= g.Nout) continue;
+      float b4[4] = {0.f, 0.f, 0.f, 0.f};
+      if (g.bias) {
+        const u32x2_t bb = *reinterpret_cast<const u32x2_t*>(g.bias + n);
+        b4[0] = bits_f32(bb.x << 16); b4[1] = bits_f32(bb.x & 0xffff0000u);
+        b4[2] = bits_f32(bb.y << 16); b4[3] = bits_f32(bb.y & 0xffff0000u);
+      }
+#pragma unroll
+      for (int i = 0; i < MT; ++i) {
+        const int m = m0 + 32 * i + l31;
+        if (m >= g.M) continue;
+        u32x2_t o;
+        o.x = pack_bf16x2(acc[j][i][4 * q + 0] + b4[0], acc[j][i][4 * q + 1] + b4[1]);
+        o.y = pack_bf16x2(acc[j][i][4 * q + 2] + b4[2], acc[j][i][4 * q + 3] + b4[3]);
+        *reinterpret_cast<u32x2_t*>(g.C + (int64_t)m * g.Nout + n) = o;
+      }
+    }
+  tstamp[4] = wall_clock64();
+  if (g.dbg && tid == 0 && (blockIdx.x == 0 || blockIdx.x == 300)) { for (int i = 0; i < 5; ++i) g.dbg[(blockIdx.x ? 8 : 0) + i] = tstamp[i]; }
+#endif
+}
+
+template <int BM, bool PER_ELEM>
+int launch_rs(RsArgs& g, hipStream_t s) {
+  using L = RsLayout<BM>;
+  g.tiles_m = (g.M + BM - 1) / BM;
+  g.tiles_n = (g.Nout + kBN - 1) / kBN;
+  static bool attr_set = false;  // idempotent; a race only repeats the call
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&nf4_gemm_rs_kernel<BM, PER_ELEM>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, L::kTotal);
+    if (e != hipSuccess)
+      return fail(TTAMD_ELAUNCH, "nf4_gemm_rs: cannot reserve %d bytes of LDS: %s", L::kTotal, hipGetErrorString(e));
+    attr_set = true;
+  }
+  nf4_gemm_rs_kernel<BM, PER_ELEM><<<dim3((unsigned)(g.tiles_m * g.tiles_n)), dim3(256), L::kTotal, s>>>(g);
+  return check_launch("nf4_gemm_rs");
+}
+
+}  // namespace
+
+// Entry used by the C-ABI wrappers in nf4_gemm.hip.
+int run_gemm_rs(const void* X, const uint8_t* codes, const void* scal, bool per_elem, const void* lX, const void* lW,
+                bool lw_row_major, int R, float lscale, const void* bias, void* C, int64_t M, int64_t Nout, int64_t Kc,
+                hipStream_t s) {
+  RsArgs g;
+  g.X = reinterpret_cast<const uint16_t*>(X);
+  g.codes = codes;
+  g.scal = reinterpret_cast<const float*>(scal);
+  g.lX = reinterpret_cast<const uint16_t*>(lX);
+  g.lW = reinterpret_cast<const uint16_t*>(lW);
+  g.bias = reinterpret_cast<const uint16_t*>(bias);
+  g.C = reinterpret_cast<uint16_t*>(C);
+  g.M = (int)M; g.Nout = (int)Nout; g.Kc = (int)Kc; g.R = R;
+  g.lw_row_major = lw_row_major ? 1 : 0;
+  g.lscale = lscale;
+  { static long long* d = nullptr; if (!d && getenv("TTAMD_DBG")) { hipMalloc(&d, 256); } g.dbg = d; }
+  const int64_t tiles256 = ((M + 255) / 256) * ((Nout + kBN - 1) / kBN);
+  const bool big = tiles256 >= 256;
+  if (per_elem) return big ? launch_rs<256, true>(g, s) : launch_rs<128, true>(g, s);
+  int rc = big ? launch_rs<256, false>(g, s) : launch_rs<128, false>(g, s);
+  if (g.dbg) { long long h[16]; hipDeviceSynchronize(); hipMemcpy(h, g.dbg, 128, hipMemcpyDeviceToHost); for (int b = 0; b < 2; ++b) printf("WG%d: prologue %lld main %lld lora %lld epilogue %lld (x10ns)\n", b, h[8*b+1]-h[8*b], h[8*b+2]-h[8*b+1], h[8*b+3]-h[8*b+2], h[8*b+4]-h[8*b+3]); }
+  return rc;
+}
+
+}  // namespace ttamd

@@ -194,7 +194,7 @@ class NF4Tensor(torch.Tensor):
 
     @torch.no_grad()
     def block_scalers(self) -> torch.Tensor:
-        """Dequantised per-block scalers as bf16 [n_blocks] on the GPU, cached while the scaler tensors are
+        """Dequantised per-block scalers as fp32 [n_blocks] on the GPU, cached while the scaler tensors are
         unchanged (the cache rides on the ``quantized_scalers`` tensor object and is keyed by the in-place
         version counters of the three scaler tensors)."""
         qs = self.quantized_scalers

@@ -97,7 +97,7 @@ def nf4_dequantize(
 def nf4_block_scalers(qscalers: torch.Tensor, qfactor: torch.Tensor, mean: torch.Tensor, scaler_block_size: int) -> torch.Tensor:
     _need_gpu(qscalers, "nf4_block_scalers")
     code = _code(qfactor.dtype, "nf4_block_scalers")
-    out = torch.empty(qscalers.numel(), dtype=torch.bfloat16, device=qscalers.device)
+    out = torch.empty(qscalers.numel(), dtype=torch.float32, device=qscalers.device)
     lib = _lib.load()
     with torch.cuda.device(qscalers.device):
         rc = lib.ttamd_nf4_block_scalers(
