@@ -129,11 +129,25 @@ int ttamd_nf4_lora_linear_fwd_bf16(const void* x, const uint8_t* quantized_data,
                                    int64_t N, int64_t K, void* stream);
 
 /*
+ * Optional transposed copy of an NF4 weight for the grad-input GEMM.  NF4 blocks run along K, the grad-input GEMM
+ * contracts over N; with the codes re-packed along N (quantized_data_t [K, N/2], even n in the high nibble) and the
+ * block scalers transposed (block_scalers_t fp32 [K/64, N]) that GEMM streams the weight exactly like the forward
+ * one.  Costs another 0.5625 B per weight element of device memory; derived data, built once per frozen tensor.
+ * The reference has no counterpart (its backward re-materialises the whole bf16 weight: torchao LinearNF4.backward,
+ * reached from torchtune/modules/peft/lora.py:138).
+ */
+int ttamd_nf4_transpose_for_backward(const uint8_t* quantized_data, const void* block_scalers, int64_t N, int64_t K,
+                                     uint8_t* quantized_data_t, void* block_scalers_t, void* stream);
+
+/*
  * gx = gy . D(W) + gh . lora_a: LinearNF4.backward (torchao; reached from lora.py:138, nf4_linear.py:67) plus the
  * term autograd adds for lora_a's input.  gy [M,N] bf16; gh [M,rank] bf16 from ttamd_lora_bwd_bf16 and
  * lora_a [rank,K] bf16 (both NULL iff rank == 0); gx out [M,K] bf16.  Same divisibility rules as the forward.
+ * quantized_data_t / block_scalers_t: the copies made by ttamd_nf4_transpose_for_backward, or both NULL to run
+ * the variant that transposes the weight tile on the fly (slower, no extra memory).
  */
-int ttamd_nf4_linear_bwd_dx_bf16(const void* gy, const uint8_t* quantized_data, const void* block_scalers, const void* gh,
+int ttamd_nf4_linear_bwd_dx_bf16(const void* gy, const uint8_t* quantized_data, const void* block_scalers,
+                                 const uint8_t* quantized_data_t, const void* block_scalers_t, const void* gh,
                                  const void* lora_a, int rank, void* gx, int64_t M, int64_t N, int64_t K, void* stream);
 
 /*

@@ -183,12 +183,25 @@ def test_raw_c_abi_sequence_matches_python_layer():
                                               Bd.data_ptr(), r, 2.0, None, y.data_ptr(), M, N, K, stream) == 0
     assert lib.ttamd_lora_bwd_bf16(gyd.data_ptr(), xd.data_ptr(), h.data_ptr(), Bd.data_ptr(), 2.0, gh.data_ptr(), ga.data_ptr(),
                                    gb.data_ptr(), M, N, K, r, ws.data_ptr(), ws.numel(), stream) == 0
-    assert lib.ttamd_nf4_linear_bwd_dx_bf16(gyd.data_ptr(), t.quantized_data.data_ptr(), bscal.data_ptr(), gh.data_ptr(),
-                                            Ad.data_ptr(), r, gx.data_ptr(), M, N, K, stream) == 0
+    assert lib.ttamd_nf4_linear_bwd_dx_bf16(gyd.data_ptr(), t.quantized_data.data_ptr(), bscal.data_ptr(), None, None,
+                                            gh.data_ptr(), Ad.data_ptr(), r, gx.data_ptr(), M, N, K, stream) == 0
+    # the same with the transposed copy of the weight (the fast grad-input path)
+    qt = torch.empty(K * N // 2, dtype=torch.uint8, device=DEV)
+    st = torch.empty(K // 64, N, dtype=torch.float32, device=DEV)
+    gx2 = torch.empty(M, K, dtype=BF, device=DEV)
+    assert lib.ttamd_nf4_transpose_for_backward(t.quantized_data.data_ptr(), bscal.data_ptr(), N, K, qt.data_ptr(), st.data_ptr(),
+                                                stream) == 0
+    assert lib.ttamd_nf4_linear_bwd_dx_bf16(gyd.data_ptr(), t.quantized_data.data_ptr(), bscal.data_ptr(), qt.data_ptr(),
+                                            st.data_ptr(), gh.data_ptr(), Ad.data_ptr(), r, gx2.data_ptr(), M, N, K, stream) == 0
     torch.cuda.synchronize()
+    # transposed codes: element (k, n) of the copy is element (n, k) of the original
+    codes = torch.stack([t.quantized_data >> 4, t.quantized_data & 0xF], dim=1).flatten().view(N, K)
+    codes_t = torch.stack([qt >> 4, qt & 0xF], dim=1).flatten().view(K, N)
+    assert torch.equal(codes_t, codes.t()) and torch.equal(st, bscal.view(N, K // 64).t())
     p, y_o, gx_o, gA_o, gB_o = _oracle(W, sbs, A, B, None, x, gy, 2.0 * r, r)
     _close(y, y_o, 1e-2, 1e-2)
     _close(gx, gx_o, 1e-2, 1e-2)
+    _close(gx2, gx_o, 1e-2, 1e-2)
     _close(ga, gA_o, 2e-2, 2e-2 * float(gA_o.float().abs().max()))
     _close(gb, gB_o, 2e-2, 2e-2 * float(gB_o.float().abs().max()))
     _close(h, (x.float() @ A.float().T), 4e-3, 4e-3)
@@ -213,9 +226,10 @@ def test_fused_gemm_is_deterministic_and_matches_dequant_plus_library_gemm_at_8b
         ref = (x.float() @ D.float().T)
         torch.testing.assert_close(y1.float(), ref, rtol=1e-2, atol=1e-2)
         torch.testing.assert_close(y1.float(), torch.nn.functional.linear(x, D).float(), rtol=1e-2, atol=1e-2)
-        g1 = ops.nf4_linear_bwd_dx(gy, t.quantized_data, t.block_scalers(), K)
-        assert torch.equal(g1, ops.nf4_linear_bwd_dx(gy, t.quantized_data, t.block_scalers(), K))
-        torch.testing.assert_close(g1.float(), gy.float() @ D.float(), rtol=1e-2, atol=1e-2)
+        for tr in (None, t.backward_copy()):
+            g1 = ops.nf4_linear_bwd_dx(gy, t.quantized_data, t.block_scalers(), K, transposed=tr)
+            assert torch.equal(g1, ops.nf4_linear_bwd_dx(gy, t.quantized_data, t.block_scalers(), K, transposed=tr))
+            torch.testing.assert_close(g1.float(), gy.float() @ D.float(), rtol=1e-2, atol=1e-2)
         # linearity in the activations, a size-independent property of the fused path
         y3 = ops.nf4_lora_linear_fwd((2 * x), t.quantized_data, t.block_scalers(), N)
         assert torch.equal(y3.float(), 2 * y1.float())

@@ -140,8 +140,27 @@ def test_clone_deepcopy_and_block_scaler_cache():
         lin.weight.copy_((torch.randn(512, 512, device=DEV) * 0.05).to(torch.bfloat16))
     s2 = lin.weight.block_scalers()
     assert s2 is not s1 and not torch.equal(s1, s2)  # in-place re-quantisation invalidates the cache
-    x = torch.randn(4, 512, device=DEV, dtype=torch.bfloat16)
+    x = torch.randn(4, 512, device=DEV, dtype=torch.bfloat16, requires_grad=True)
     torch.testing.assert_close(lin(x).float(), x.float() @ lin.weight.get_original_weight().float().T, rtol=1e-2, atol=1e-2)
+    # the transposed copy used by the grad-input GEMM follows the weight too, and can be switched off
+    import torchtune_amd.nf4_tensor as nf4_mod
+    c1 = lin.weight.backward_copy()
+    assert lin.weight.backward_copy() is c1
+    gy = torch.randn(4, 512, device=DEV, dtype=torch.bfloat16)
+    (g_fast,) = torch.autograd.grad(lin(x), x, gy)
+    with torch.no_grad():
+        lin.weight.copy_((torch.randn(512, 512, device=DEV) * 0.05).to(torch.bfloat16))
+    assert lin.weight.backward_copy() is not c1
+    (g_new,) = torch.autograd.grad(lin(x), x, gy)
+    torch.testing.assert_close(g_new.float(), gy.float() @ lin.weight.get_original_weight().float(), rtol=1e-2, atol=1e-2)
+    assert not torch.equal(g_new, g_fast)
+    nf4_mod.BACKWARD_COPY = False
+    try:
+        assert lin.weight.backward_copy() is None
+        (g_slow,) = torch.autograd.grad(lin(x), x, gy)
+    finally:
+        nf4_mod.BACKWARD_COPY = True
+    torch.testing.assert_close(g_slow.float(), g_new.float(), rtol=1e-2, atol=1e-2)
 
 
 def test_load_dense_state_dict_into_nf4_model_and_back():

@@ -75,7 +75,7 @@ def test_argument_validation_needs_no_gpu():
     assert rc == -1 and b"multiple of the NF4 block size" in lib.ttamd_last_error()
     rc = lib.ttamd_nf4_lora_linear_fwd_bf16(aligned, aligned, aligned, None, None, 8, 2.0, None, aligned, 8, 64, 64, None)
     assert rc == -1 and b"adapter pointers" in lib.ttamd_last_error()
-    rc = lib.ttamd_nf4_linear_bwd_dx_bf16(aligned, aligned, aligned, aligned, aligned, 12, aligned, 8, 64, 64, None)
+    rc = lib.ttamd_nf4_linear_bwd_dx_bf16(aligned, aligned, aligned, None, None, aligned, aligned, 12, aligned, 8, 64, 64, None)
     assert rc == -1 and b"rank" in lib.ttamd_last_error()
     rc = lib.ttamd_fq_per_group_int4_sym(aligned, 0, 4, 64, 24, aligned, None, None)
     assert rc == -1 and b"group_size" in lib.ttamd_last_error()

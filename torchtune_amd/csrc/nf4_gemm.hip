@@ -315,6 +315,34 @@ __global__ __launch_bounds__(256) void nf4_block_scalers_kernel(const int8_t* __
   out[b] = nf4_block_scaler<BF16>((int)qs[b], f, m);
 }
 
+// Transposed copy of the codes for the grad-input GEMM: out[k][n] = code of W[n][k], packed along n
+// (byte (k*N + n)/2, even n in the high nibble).  One thread makes one output dword = 8 consecutive n.
+__global__ __launch_bounds__(256) void nf4_transpose_codes_kernel(const uint8_t* __restrict__ q, int N, int K,
+                                                                  uint32_t* __restrict__ qt) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;  // = k * (N/8) + n8
+  const int n8s = N >> 3;
+  if (idx >= (int64_t)K * n8s) return;
+  const int k = (int)(idx / n8s), n8 = (int)(idx % n8s);
+  const int shift = (k & 1) ? 0 : 4;
+  uint32_t packed = 0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const uint32_t byte = q[((int64_t)(n8 * 8 + i) * K + k) >> 1];
+    const uint32_t code = (byte >> shift) & 0xfu;
+    packed |= code << (8 * (i >> 1) + ((i & 1) ? 0 : 4));
+  }
+  qt[idx] = packed;
+}
+
+// Transposed block scalers: out[kb][n] = scalers[n][kb]
+__global__ __launch_bounds__(256) void nf4_transpose_scalers_kernel(const float* __restrict__ sc, int N, int KB,
+                                                                    float* __restrict__ out) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;  // = kb * N + n
+  if (idx >= (int64_t)N * KB) return;
+  const int kb = (int)(idx / N), n = (int)(idx % N);
+  out[idx] = sc[(int64_t)n * KB + kb];
+}
+
 template <int BM, int BN, bool TRANS_W>
 int launch_gemm(GemmArgs& g, hipStream_t s) {
   const int Nout = TRANS_W ? g.K : g.N;
@@ -395,10 +423,34 @@ extern "C" int ttamd_nf4_lora_linear_fwd_bf16(const void* x, const uint8_t* quan
                      reinterpret_cast<hipStream_t>(stream));
 }
 
+extern "C" int ttamd_nf4_transpose_for_backward(const uint8_t* quantized_data, const void* block_scalers, int64_t N, int64_t K,
+                                                uint8_t* quantized_data_t, void* block_scalers_t, void* stream) {
+  TT_REQUIRE(quantized_data && block_scalers && quantized_data_t && block_scalers_t, "nf4_transpose_for_backward: null pointer");
+  TT_REQUIRE(N > 0 && K > 0 && N % 64 == 0 && K % 64 == 0 && N < (1 << 30) && K < (1 << 30),
+             "nf4_transpose_for_backward: N (%lld) and K (%lld) must be positive multiples of 64", (long long)N, (long long)K);
+  TT_REQUIRE((reinterpret_cast<uintptr_t>(quantized_data_t) & 3u) == 0, "nf4_transpose_for_backward: output must be 4-byte aligned");
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const int64_t n1 = K * (N / 8), n2 = N * (K / 64);
+  TT_REQUIRE((n1 + 255) / 256 < (int64_t(1) << 31), "nf4_transpose_for_backward: tensor too large for one launch");
+  nf4_transpose_codes_kernel<<<dim3((unsigned)((n1 + 255) / 256)), dim3(256), 0, s>>>(quantized_data, (int)N, (int)K,
+                                                                                     reinterpret_cast<uint32_t*>(quantized_data_t));
+  nf4_transpose_scalers_kernel<<<dim3((unsigned)((n2 + 255) / 256)), dim3(256), 0, s>>>(
+      reinterpret_cast<const float*>(block_scalers), (int)N, (int)(K / 64), reinterpret_cast<float*>(block_scalers_t));
+  return check_launch("nf4_transpose_for_backward");
+}
+
 extern "C" int ttamd_nf4_linear_bwd_dx_bf16(const void* gy, const uint8_t* quantized_data, const void* block_scalers,
-                                            const void* gh, const void* lora_a, int rank, void* gx, int64_t M, int64_t N,
-                                            int64_t K, void* stream) {
+                                            const uint8_t* quantized_data_t, const void* block_scalers_t, const void* gh,
+                                            const void* lora_a, int rank, void* gx, int64_t M, int64_t N, int64_t K,
+                                            void* stream) {
   if (int rc = check_gemm_args("nf4_linear_bwd_dx", gy, quantized_data, block_scalers, gx, M, N, K, rank, gh, lora_a)) return rc;
+  TT_REQUIRE((quantized_data_t == nullptr) == (block_scalers_t == nullptr),
+             "nf4_linear_bwd_dx: the transposed codes and scalers must be given together");
+  if (quantized_data_t != nullptr) {
+    TT_REQUIRE(aligned16(quantized_data_t) && aligned16(block_scalers_t), "nf4_linear_bwd_dx: transposed copies must be 16-byte aligned");
+    return run_gemm_rs(gy, quantized_data_t, block_scalers_t, true, gh, lora_a, false, rank, 1.0f, nullptr, gx, M, K, N,
+                       reinterpret_cast<hipStream_t>(stream));
+  }
   GemmArgs g;
   g.A = reinterpret_cast<const uint16_t*>(gy);
   g.qdata = quantized_data;

@@ -22,7 +22,6 @@
 //
 // Per 64-wide k-step a wave issues 64 v_mfma_f32_32x32x16_bf16 against ~2.5 VALU ops per weight element,
 // 12 direct-to-LDS loads, BM/32 x 4 operand reads and 32 table reads.
-#include <stdlib.h>
 
 #include "common.h"
 #include "nf4_math.h"
@@ -47,9 +46,6 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
 }
 
 #define TT_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
-#ifndef TT_EXP
-#define TT_EXP 0
-#endif
 
 struct RsArgs {
   const uint16_t* X;     // [M, Kc] bf16 activations
@@ -63,7 +59,6 @@ struct RsArgs {
   int lw_row_major;
   float lscale;
   int tiles_m, tiles_n;
-  long long* dbg;
 };
 
 constexpr int kBN = 256;
@@ -96,8 +91,6 @@ __global__ __launch_bounds__(256) void nf4_gemm_rs_kernel(const RsArgs g) {
   const int lane = tid & 63;
   const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l31 = lane & 31, h = lane >> 5;
-  long long tstamp[6];
-  tstamp[0] = wall_clock64();
 
   int tile_m, tile_n;
   {
@@ -181,7 +174,6 @@ __global__ __launch_bounds__(256) void nf4_gemm_rs_kernel(const RsArgs g) {
     return b;
   };
   auto issue_one = [&](const BatchAddr& b, int d) {  // d is a compile-time constant after unrolling
-    if (TT_EXP & 1) return;
     if (d < kALoads) {
       dma16(a_off[d], b.xb, b.abase + d * 1024);
     } else if (d < kALoads + NT) {
@@ -206,12 +198,10 @@ __global__ __launch_bounds__(256) void nf4_gemm_rs_kernel(const RsArgs g) {
   bf16x8_t xfa[MT], xfb[MT];
 
   auto fetch_byte = [&](int j, int ks, int b) {
-    if (TT_EXP & 2) return;
     pend[j][b] = *reinterpret_cast<const float2*>(lut + (((codes[j][ks] >> (8 * b)) & 0xffu) << 3));
   };
   // finish byte b of tile j into wf[j]; s8 = the eight per-element scalers of the substep (PER_ELEM), s = the row's scaler
   auto finish_byte = [&](u32x4_t (&wf)[NT], int j, int b, const float (&s)[NT], const float (&s8)[8]) {
-    if (TT_EXP & 2) return;
     if constexpr (PER_ELEM)
       wf[j][b] = pack_bf16x2(pend[j][b].x * s8[2 * b], pend[j][b].y * s8[2 * b + 1]);
     else
@@ -315,7 +305,6 @@ __global__ __launch_bounds__(256) void nf4_gemm_rs_kernel(const RsArgs g) {
   }
 #pragma unroll
   for (int i = 0; i < MT; ++i) xfa[i] = *reinterpret_cast<const bf16x8_t*>(smem + i * 4096 + x_off[0]);
-  tstamp[1] = wall_clock64();
 
   constexpr int kDEven = (kBatch + 7) / 8 > 1 ? 2 : 1;  // loads per even quarter over the 8 quarters of phases 0 and 1
   constexpr int kDOdd = (kBatch - 4 * kDEven + 3) / 4;  // and per odd quarter
@@ -327,8 +316,7 @@ __global__ __launch_bounds__(256) void nf4_gemm_rs_kernel(const RsArgs g) {
     const BatchAddr b = batch_addr(kt + 2, a2, w2);
     phase(xfa, wfa, xfb, a0, 1, wfb, sc, w0, 1, 2, b, 0, kDEven, kDOdd);
     phase(xfb, wfb, xfa, a0, 2, wfa, sc, w0, 2, 3, b, 2 * (kDEven + kDOdd), kDEven, kDOdd);
-    if (TT_EXP & 8) asm volatile("s_barrier" ::: "memory");
-    else if (!(TT_EXP & 4)) asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kBatch) : "memory");
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kBatch) : "memory");
     load_codes(w1, sc_next);
     phase(xfa, wfa, xfb, a0, 3, wfb, sc, w0, 3, 0, b, kBatch, 0, 0);
     phase(xfb, wfb, xfa, a1, 0, wfa, sc_next, w1, 0, 1, b, kBatch, 0, 0);
@@ -339,7 +327,6 @@ __global__ __launch_bounds__(256) void nf4_gemm_rs_kernel(const RsArgs g) {
   }
 
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the clamped batches issued by the last two steps
-  tstamp[2] = wall_clock64();
   // ---- adapter: R extra contraction steps, operands straight from global memory
   if (g.R > 0) {
     for (int rc = 0; rc < g.R; rc += 16) {
@@ -386,7 +373,6 @@ __global__ __launch_bounds__(256) void nf4_gemm_rs_kernel(const RsArgs g) {
     }
   }
 
-  tstamp[3] = wall_clock64();
   // ---- epilogue.  acc[j][i][v] = C[m][n] with m = m0 + 32 i + l31 and n = n0 + 64 wv + 32 j + 8 (v/4) + 4 h + v%4:
   //      four consecutive n per lane -> one 8-byte store
 #pragma unroll
@@ -411,8 +397,6 @@ __global__ __launch_bounds__(256) void nf4_gemm_rs_kernel(const RsArgs g) {
         *reinterpret_cast<u32x2_t*>(g.C + (int64_t)m * g.Nout + n) = o;
       }
     }
-  tstamp[4] = wall_clock64();
-  if (g.dbg && tid == 0 && (blockIdx.x == 0 || blockIdx.x == 300)) { for (int i = 0; i < 5; ++i) g.dbg[(blockIdx.x ? 8 : 0) + i] = tstamp[i]; }
 #endif
 }
 
@@ -450,12 +434,10 @@ int run_gemm_rs(const void* X, const uint8_t* codes, const void* scal, bool per_
   g.M = (int)M; g.Nout = (int)Nout; g.Kc = (int)Kc; g.R = R;
   g.lw_row_major = lw_row_major ? 1 : 0;
   g.lscale = lscale;
-  { static long long* d = nullptr; if (!d && getenv("TTAMD_DBG")) { hipMalloc(&d, 256); } g.dbg = d; }
   const int64_t tiles256 = ((M + 255) / 256) * ((Nout + kBN - 1) / kBN);
   const bool big = tiles256 >= 256;
   if (per_elem) return big ? launch_rs<256, true>(g, s) : launch_rs<128, true>(g, s);
   int rc = big ? launch_rs<256, false>(g, s) : launch_rs<128, false>(g, s);
-  if (g.dbg) { long long h[16]; hipDeviceSynchronize(); hipMemcpy(h, g.dbg, 128, hipMemcpyDeviceToHost); for (int b = 0; b < 2; ++b) printf("WG%d: prologue %lld main %lld lora %lld epilogue %lld (x10ns)\n", b, h[8*b+1]-h[8*b], h[8*b+2]-h[8*b+1], h[8*b+3]-h[8*b+2], h[8*b+4]-h[8*b+3]); }
   return rc;
 }
 

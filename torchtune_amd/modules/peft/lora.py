@@ -61,7 +61,8 @@ class _QLoRALinearFn(torch.autograd.Function):
         if need_x or need_a or need_b:
             gh, ga, gb = ops.lora_bwd(gy2, x2, h, lora_b, ctx.scale)
             if need_x:
-                gx = ops.nf4_linear_bwd_dx(gy2, weight.quantized_data, weight.block_scalers(), K, gh, lora_a)
+                gx = ops.nf4_linear_bwd_dx(gy2, weight.quantized_data, weight.block_scalers(), K, gh, lora_a,
+                                           transposed=weight.backward_copy())
                 gx = gx.view(ctx.x_shape)
             if not need_a:
                 ga = None

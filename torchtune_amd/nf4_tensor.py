@@ -27,6 +27,9 @@ aten = torch.ops.aten
 DEFAULT_BLOCK_SIZE = 64
 DEFAULT_SCALER_BLOCK_SIZE = 256
 
+# Keep a transposed copy of the codes for the grad-input GEMM (see NF4Tensor.backward_copy).
+BACKWARD_COPY = True
+
 NF4_TABLE = (
     -1.0,
     -0.6961928009986877,
@@ -206,6 +209,25 @@ class NF4Tensor(torch.Tensor):
         qs._ttamd_block_scalers = (key, val)
         return val
 
+    @torch.no_grad()
+    def backward_copy(self):
+        """(codes re-packed along N, block scalers transposed) for the grad-input GEMM, or None when disabled.
+
+        Derived data for a 2-D bf16 tensor with 64-element blocks, cached like ``block_scalers`` (same key).  It
+        costs another 0.5625 B per element of device memory; set ``torchtune_amd.nf4_tensor.BACKWARD_COPY = False``
+        to trade that memory for a slower grad-input GEMM that transposes the weight tile on the fly."""
+        if not BACKWARD_COPY:
+            return None
+        qs = self.quantized_scalers
+        key = (qs._version, self.quantization_factor._version, self.scaler_mean._version, self.quantized_data._version,
+               qs.data_ptr())
+        cached = getattr(qs, "_ttamd_backward_copy", None)
+        if cached is not None and cached[0] == key:
+            return cached[1]
+        val = ops.nf4_transpose_for_backward(self.quantized_data, self.block_scalers(), self.shape[0], self.shape[1])
+        qs._ttamd_backward_copy = (key, val)
+        return val
+
     # ---- tensor-subclass protocol --------------------------------------------------------------------
     def __tensor_flatten__(self):
         ctx = {
@@ -292,6 +314,7 @@ def _nf4_copy_(func, args, kwargs):
     # in-place writes issued from inside __torch_dispatch__ do not advance the version counters the
     # block-scaler cache is keyed on, so drop the cache explicitly
     dst.quantized_scalers._ttamd_block_scalers = None
+    dst.quantized_scalers._ttamd_backward_copy = None
     if isinstance(src, NF4Tensor):
         same_meta = (
             src.block_size == dst.block_size
@@ -452,7 +475,8 @@ class _LinearNF4(torch.autograd.Function):
             return None, None
         if _fused_ok(grad_output, weight, 0):
             g2 = grad_output.reshape(-1, grad_output.shape[-1])
-            gx = ops.nf4_linear_bwd_dx(g2, weight.quantized_data, weight.block_scalers(), weight.shape[1])
+            gx = ops.nf4_linear_bwd_dx(g2, weight.quantized_data, weight.block_scalers(), weight.shape[1],
+                                       transposed=weight.backward_copy())
             return gx.view(ctx.in_shape), None
         return grad_output @ weight.to(grad_output.dtype), None
 
@@ -464,6 +488,7 @@ def _fused_ok(x: torch.Tensor, weight: NF4Tensor, rank: int) -> bool:
         x.is_cuda
         and weight.quantized_data.is_cuda
         and x.dtype == torch.bfloat16
+        and weight.dtype == torch.bfloat16
         and weight.dim() == 2
         and weight.block_size == 64
         and x.numel() > 0

@@ -182,11 +182,25 @@ def nf4_lora_linear_fwd(
     return y
 
 
+def nf4_transpose_for_backward(qdata: torch.Tensor, block_scalers: torch.Tensor, N: int, K: int):
+    """-> (codes re-packed along N: u8 [K*N/2], block scalers transposed: fp32 [K/64, N])"""
+    _need_gpu(qdata, "nf4_transpose_for_backward")
+    qdata_t = torch.empty(K * N // 2, dtype=torch.uint8, device=qdata.device)
+    scal_t = torch.empty(K // 64, N, dtype=torch.float32, device=qdata.device)
+    lib = _lib.load()
+    with torch.cuda.device(qdata.device):
+        rc = lib.ttamd_nf4_transpose_for_backward(qdata.data_ptr(), block_scalers.data_ptr(), N, K, qdata_t.data_ptr(),
+                                                  scal_t.data_ptr(), _stream(qdata))
+    _lib.check(rc, "nf4_transpose_for_backward")
+    return qdata_t, scal_t
+
+
 def nf4_linear_bwd_dx(
     gy: torch.Tensor, qdata: torch.Tensor, block_scalers: torch.Tensor, K: int, gh: Optional[torch.Tensor] = None,
-    lora_a: Optional[torch.Tensor] = None,
+    lora_a: Optional[torch.Tensor] = None, transposed=None,
 ) -> torch.Tensor:
-    """gx = gy @ D(W) + gh @ lora_a ;  gy [M,N] -> [M,K]"""
+    """gx = gy @ D(W) + gh @ lora_a ;  gy [M,N] -> [M,K].  `transposed` = the pair from nf4_transpose_for_backward
+    (fast path) or None (the weight tile is transposed on the fly)."""
     gy = _bf16_2d(gy, "nf4_linear_bwd_dx")
     M, N = gy.shape
     rank = 0
@@ -201,8 +215,8 @@ def nf4_linear_bwd_dx(
         if events:
             events[0].record()
         rc = lib.ttamd_nf4_linear_bwd_dx_bf16(
-            gy.data_ptr(), qdata.data_ptr(), block_scalers.data_ptr(), _ptr(gh), _ptr(lora_a), rank, gx.data_ptr(), M, N, K,
-            _stream(gy),
+            gy.data_ptr(), qdata.data_ptr(), block_scalers.data_ptr(), _ptr(transposed[0]) if transposed else None,
+            _ptr(transposed[1]) if transposed else None, _ptr(gh), _ptr(lora_a), rank, gx.data_ptr(), M, N, K, _stream(gy),
         )
         if events:
             events[1].record()
