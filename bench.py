@@ -103,6 +103,9 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--workload", default="llama3_1_8b", choices=sorted(WORKLOADS))
     ap.add_argument("--cpu-tokens", type=int, default=128, help="tokens in the CPU-baseline sample (0 = skip)")
+    ap.add_argument("--calibration-copy-mib", type=int, default=0,
+                    help="before the steps, run one elementwise kernel that reads and writes this many MiB: the known-size "
+                         "dispatch that FETCH_SIZE / WRITE_SIZE counter runs are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (--gpus 1); multi-GPU runs are not part of it", file=sys.stderr)
@@ -128,6 +131,12 @@ def main() -> int:
         model.zero_grad(set_to_none=True)
         return loss
 
+    if args.calibration_copy_mib > 0:
+        src = torch.ones(args.calibration_copy_mib << 18, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        torch.add(src, 1.0, out=dst)  # one vectorized_elementwise_kernel dispatch: reads and writes exactly src.nbytes
+        torch.cuda.synchronize()
+        del src, dst
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()

@@ -373,30 +373,46 @@ __global__ __launch_bounds__(256) void nf4_gemm_rs_kernel(const RsArgs g) {
     }
   }
 
-  // ---- epilogue.  acc[j][i][v] = C[m][n] with m = m0 + 32 i + l31 and n = n0 + 64 wv + 32 j + 8 (v/4) + 4 h + v%4:
-  //      four consecutive n per lane -> one 8-byte store
+  // ---- epilogue.  acc[j][i][v] = C[m][n] with m = m0 + 32 i + l31 and n = n0 + 64 wv + 32 j + 8 (v/4) + 4 h + v%4.
+  //      Stored straight from these registers a wave would write 16-byte pieces of 32 different rows per instruction,
+  //      which the memory system turns into partial-line read-modify-writes.  Instead each wave transposes its
+  //      BM x 64 band through LDS (the activation ring is free now: BM x 128 bytes per wave) and writes whole
+  //      128-byte row segments.  16-byte chunk c of row r sits in slot c ^ (r & 7): both sides are conflict-free.
+  __syncthreads();                      // every wave is done reading the activation ring
+  if (n0 + wv * 64 >= g.Nout) return;  // the whole 64-column band of this wave lies outside (no barrier follows)
+  {
+    char* band = smem + wv * (BM * 128);
 #pragma unroll
-  for (int j = 0; j < NT; ++j)
+    for (int j = 0; j < NT; ++j)
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int n = n0 + wv * 64 + 32 * j + 8 * q + 4 * h;
-      if (n >= g.Nout) continue;
-      float b4[4] = {0.f, 0.f, 0.f, 0.f};
-      if (g.bias) {
-        const u32x2_t bb = *reinterpret_cast<const u32x2_t*>(g.bias + n);
-        b4[0] = bits_f32(bb.x << 16); b4[1] = bits_f32(bb.x & 0xffff0000u);
-        b4[2] = bits_f32(bb.y << 16); b4[3] = bits_f32(bb.y & 0xffff0000u);
+      for (int q = 0; q < 4; ++q) {
+        float b4[4] = {0.f, 0.f, 0.f, 0.f};
+        if (g.bias) {
+          const u32x2_t bb = *reinterpret_cast<const u32x2_t*>(g.bias + n0 + wv * 64 + 32 * j + 8 * q + 4 * h);
+          b4[0] = bits_f32(bb.x << 16); b4[1] = bits_f32(bb.x & 0xffff0000u);
+          b4[2] = bits_f32(bb.y << 16); b4[3] = bits_f32(bb.y & 0xffff0000u);
+        }
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+          const int r = 32 * i + l31;
+          u32x2_t o;
+          o.x = pack_bf16x2(acc[j][i][4 * q + 0] + b4[0], acc[j][i][4 * q + 1] + b4[1]);
+          o.y = pack_bf16x2(acc[j][i][4 * q + 2] + b4[2], acc[j][i][4 * q + 3] + b4[3]);
+          *reinterpret_cast<u32x2_t*>(band + r * 128 + (((4 * j + q) ^ (r & 7)) << 4) + 8 * h) = o;
+        }
       }
-#pragma unroll
-      for (int i = 0; i < MT; ++i) {
-        const int m = m0 + 32 * i + l31;
-        if (m >= g.M) continue;
-        u32x2_t o;
-        o.x = pack_bf16x2(acc[j][i][4 * q + 0] + b4[0], acc[j][i][4 * q + 1] + b4[1]);
-        o.y = pack_bf16x2(acc[j][i][4 * q + 2] + b4[2], acc[j][i][4 * q + 3] + b4[3]);
-        *reinterpret_cast<u32x2_t*>(g.C + (int64_t)m * g.Nout + n) = o;
-      }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const int c = lane & 7;
+    uint16_t* crow = g.C + n0 + wv * 64 + 8 * c;
+#pragma unroll 8
+    for (int t = 0; t < BM / 8; ++t) {
+      const int r = 8 * t + (lane >> 3);
+      const u32x4_t v = *reinterpret_cast<const u32x4_t*>(band + r * 128 + ((c ^ (r & 7)) << 4));
+      if (m0 + r < g.M) *reinterpret_cast<u32x4_t*>(crow + (int64_t)(m0 + r) * g.Nout) = v;
     }
+  }
 #endif
 }
 
