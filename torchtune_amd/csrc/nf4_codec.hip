@@ -164,11 +164,16 @@ __global__ __launch_bounds__(256) void nf4_quantize_scalers_kernel(const float* 
 }
 
 // ---------------------------------------------------------------------------------------------------
-// dequantise.  One lane expands one dword of codes (8 elements) into one 128-bit bf16 store (two for
-// fp32), so every load and store instruction of a wave covers one contiguous span.  Code pairs are looked
-// up a byte at a time in a 256-entry LDS table of (nf4[hi], nf4[lo]) in fp32.
+// dequantise.  A workgroup expands 16384 elements.  It first evaluates the block scalers of its span once
+// (one thread per block, into LDS: the division is done once per block, not once per lane), then every
+// lane turns one dword of codes (8 elements) into one 128-bit bf16 store (two for fp32), so each load and
+// store instruction of a wave covers one contiguous span.  Code pairs are looked up a byte at a time in a
+// 256-entry LDS table of (nf4[hi], nf4[lo]) in fp32; for bf16 the product is rounded once, by the packing
+// conversion (round to nearest even, the same rounding the eager reference applies to the product).
 // ---------------------------------------------------------------------------------------------------
 constexpr int kDequantDwordsPerThread = 8;
+constexpr int kDequantElemsPerWg = 256 * kDequantDwordsPerThread * 8;  // 16384
+constexpr int kDequantMaxBlocksPerWg = kDequantElemsPerWg / 8;         // smallest block size is 8
 
 template <bool BF16>
 __global__ __launch_bounds__(256) void nf4_dequantize_kernel(const uint32_t* __restrict__ qdata,
@@ -176,39 +181,41 @@ __global__ __launch_bounds__(256) void nf4_dequantize_kernel(const uint32_t* __r
                                                              const void* __restrict__ qfactor,
                                                              const void* __restrict__ scaler_mean, int64_t n_dwords,
                                                              int log2_dwords_per_block, int SB, int log2_SB,
-                                                             void* __restrict__ out) {
+                                                             int64_t n_blocks, void* __restrict__ out) {
   __shared__ float2 lut[256];
-  {
-    const int t = threadIdx.x;
-    lut[t] = make_float2(Arith<BF16>::rnd(kNF4Dev[t >> 4]), Arith<BF16>::rnd(kNF4Dev[t & 15]));
-  }
-  __syncthreads();
-  const float mean = load1<BF16>(scaler_mean, 0);
-  const int64_t base = (int64_t)blockIdx.x * (256 * kDequantDwordsPerThread) + threadIdx.x;
+  __shared__ float scal[kDequantMaxBlocksPerWg];
+  const int t = threadIdx.x;
+  const int64_t base = (int64_t)blockIdx.x * (256 * kDequantDwordsPerThread) + t;
   uint32_t code[kDequantDwordsPerThread];
-  float scaler[kDequantDwordsPerThread];
 #pragma unroll
   for (int u = 0; u < kDequantDwordsPerThread; ++u) {
     const int64_t idx = base + u * 256;
-    code[u] = 0;
-    scaler[u] = 0.f;
-    if (idx < n_dwords) {
-      code[u] = __builtin_nontemporal_load(qdata + idx);
-      const int64_t blk = idx >> log2_dwords_per_block;
+    code[u] = idx < n_dwords ? __builtin_nontemporal_load(qdata + idx) : 0u;
+  }
+  lut[t] = make_float2(Arith<BF16>::rnd(kNF4Dev[t >> 4]), Arith<BF16>::rnd(kNF4Dev[t & 15]));
+  {
+    const float mean = load1<BF16>(scaler_mean, 0);
+    const int blocks_per_wg = (256 * kDequantDwordsPerThread) >> log2_dwords_per_block;
+    const int64_t blk0 = (int64_t)blockIdx.x * blocks_per_wg;
+    for (int i = t; i < blocks_per_wg; i += 256) {
+      const int64_t blk = blk0 + i;
+      if (blk >= n_blocks) break;
       const int64_t sb = log2_SB >= 0 ? (blk >> log2_SB) : (blk / SB);
-      scaler[u] = nf4_block_scaler<BF16>((int)qscalers[blk], load1<BF16>(qfactor, sb), mean);
+      scal[i] = nf4_block_scaler<BF16>((int)qscalers[blk], load1<BF16>(qfactor, sb), mean);
     }
   }
+  __syncthreads();
 #pragma unroll
   for (int u = 0; u < kDequantDwordsPerThread; ++u) {
     const int64_t idx = base + u * 256;
     if (idx >= n_dwords) continue;
+    const float sc = scal[(u * 256 + t) >> log2_dwords_per_block];
     float v[8];
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
       const float2 pr = lut[(code[u] >> (8 * b)) & 0xffu];
-      v[2 * b] = Arith<BF16>::rnd(pr.x * scaler[u]);
-      v[2 * b + 1] = Arith<BF16>::rnd(pr.y * scaler[u]);
+      v[2 * b] = pr.x * sc;
+      v[2 * b + 1] = pr.y * sc;
     }
     if constexpr (BF16) {
       u32x4_t o;
@@ -329,10 +336,10 @@ extern "C" int ttamd_nf4_dequantize(const uint8_t* quantized_data, const int8_t*
   if (dtype == TTAMD_BF16)
     nf4_dequantize_kernel<true><<<dim3((unsigned)grid), dim3(256), 0, s>>>(
         reinterpret_cast<const uint32_t*>(quantized_data), quantized_scalers, quantization_factor, scaler_mean, n_dwords,
-        l2dpb, scaler_block_size, l2sb, out);
+        l2dpb, scaler_block_size, l2sb, numel / block_size, out);
   else
     nf4_dequantize_kernel<false><<<dim3((unsigned)grid), dim3(256), 0, s>>>(
         reinterpret_cast<const uint32_t*>(quantized_data), quantized_scalers, quantization_factor, scaler_mean, n_dwords,
-        l2dpb, scaler_block_size, l2sb, out);
+        l2dpb, scaler_block_size, l2sb, numel / block_size, out);
   return check_launch("nf4_dequantize");
 }
