@@ -29,6 +29,9 @@ WORKLOADS = {
     "llama3_1_70b": ("llama3_1_70b", 16, 32.0, 1, 4096, True),
 }
 MFMA_BF16_PEAK_TFLOPS = 2500.0
+# HBM-side bytes per fused-GEMM launch (average over the launches of one step), from the FETCH_SIZE / WRITE_SIZE counter
+# runs summarised in profiles/nf4_gemm_rs_kernel_hbm_traffic.txt (counters cannot be read from inside this process).
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"llama3_1_8b": 495.8e6}
 
 
 class GemmTimer:
@@ -62,9 +65,12 @@ class GemmTimer:
         return len(self.records), total_ms, total_flops, per_shape
 
 
-def cpu_baseline(shape_name: str, rank: int, alpha: float, tokens_sample: int, layers: int):
+def cpu_baseline(shape_name: str, rank: int, alpha: float, tokens_sample: int, layers: int, max_tokens: int,
+                 min_seconds: float = 10.0):
     """Time the CPU oracle (eager PyTorch, the op sequence the reference executes) on one decoder layer's seven
-    QLoRA linears at `tokens_sample` tokens, forward + backward, and scale to tokens/s for the full depth."""
+    QLoRA linears, forward + backward, and scale to tokens/s for the full depth.  The token count of the sample
+    starts at `tokens_sample` and is quadrupled up to the workload's tokens per step, then the pass is repeated, until
+    the sample takes at least `min_seconds`."""
     from oracle import lora_oracle, nf4_oracle
     from torchtune_amd.harness import SHAPES
 
@@ -73,26 +79,36 @@ def cpu_baseline(shape_name: str, rank: int, alpha: float, tokens_sample: int, l
     dims = [(s.dim, s.dim), (kv, s.dim), (kv, s.dim), (s.dim, s.dim), (s.hidden, s.dim), (s.hidden, s.dim), (s.dim, s.hidden)]
     gen = torch.Generator().manual_seed(0)
     cores = torch.get_num_threads()
-    prepared = []
+    weights = []
     for N, K in dims:
         W = (torch.randn(N, K, generator=gen) * 0.02).to(torch.bfloat16)
         parts = nf4_oracle.nf4_quantize(W, 64, 256)
         A = lora_oracle.lora_a_init_(torch.empty(rank, K), gen).to(torch.bfloat16).requires_grad_()
         B = (torch.randn(N, rank, generator=gen) * 0.01).to(torch.bfloat16).requires_grad_()
-        x = torch.randn(tokens_sample, K, generator=gen).to(torch.bfloat16).requires_grad_()
-        prepared.append((parts, A, B, x))
-    t0 = time.perf_counter()
-    for parts, A, B, x in prepared:
-        y = lora_oracle.lora_linear_forward(x, parts, A, B, alpha, rank)
-        (y.float() ** 2).sum().backward()
-    dt = time.perf_counter() - t0
+        weights.append((K, parts, A, B))
+    tokens = tokens_sample
+    reps = 1
+    while True:
+        xs = [torch.randn(tokens, K, generator=gen).to(torch.bfloat16).requires_grad_() for K, _, _, _ in weights]
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            for (K, parts, A, B), x in zip(weights, xs):
+                y = lora_oracle.lora_linear_forward(x, parts, A, B, alpha, rank)
+                (y.float() ** 2).sum().backward()
+        dt = time.perf_counter() - t0
+        if dt >= min_seconds:
+            break
+        if tokens < max_tokens:
+            tokens = min(max_tokens, tokens * 4)
+        else:
+            reps = max(reps + 1, int(reps * 1.2 * min_seconds / dt) + 1)
     return {
-        "value": round(tokens_sample / (dt * layers), 3),
+        "value": round(tokens * reps / (dt * layers), 3),
         "unit": "tokens/s",
         "cores": cores,
         "kind": "port",
-        "sample": f"eager-PyTorch oracle, fwd+bwd of one {shape_name} layer's seven NF4+LoRA linears at {tokens_sample} tokens "
-                  f"({dt:.2f} s), extrapolated x{layers} layers; attention, norms and loss not included",
+        "sample": f"eager-PyTorch oracle, fwd+bwd of one {shape_name} layer's seven NF4+LoRA linears at {tokens} tokens x {reps} passes "
+                  f"({dt:.1f} s on {cores} threads), extrapolated x{layers} layers; attention, norms and loss not included",
     }
 
 
@@ -102,7 +118,8 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--workload", default="llama3_1_8b", choices=sorted(WORKLOADS))
-    ap.add_argument("--cpu-tokens", type=int, default=128, help="tokens in the CPU-baseline sample (0 = skip)")
+    ap.add_argument("--cpu-tokens", type=int, default=512,
+                    help="starting token count of the CPU-baseline sample, grown until it takes >= 10 s (0 = skip)")
     ap.add_argument("--calibration-copy-mib", type=int, default=0,
                     help="before the steps, run one elementwise kernel that reads and writes this many MiB: the known-size "
                          "dispatch that FETCH_SIZE / WRITE_SIZE counter runs are scaled by")
@@ -177,19 +194,20 @@ def main() -> int:
         },
         "roofline": {
             "bound": "mfma",
-            "kernel": "nf4_gemm_kernel (fused NF4-dequant + LoRA bf16 MFMA GEMM, forward and grad-input launches)",
+            "kernel": "nf4_gemm_rs_kernel (fused NF4-dequant + LoRA bf16 MFMA GEMM, forward and grad-input launches)",
             "achieved": round(achieved, 1),
             "peak": MFMA_BF16_PEAK_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4),
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(args.workload),
+            "traffic_unit": "bytes per launch (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, rocprofv3 --pmc; algorithmic 210.4e6)",
             "launches_timed": launches,
             "gemm_ms_per_step": round(gemm_ms / args.steps, 2),
             "per_shape": per_shape,
         },
     }
     if args.cpu_tokens > 0:
-        result["cpu_baseline"] = cpu_baseline(shape_name, rank, alpha, args.cpu_tokens, SHAPES[shape_name].n_layers)
+        result["cpu_baseline"] = cpu_baseline(shape_name, rank, alpha, args.cpu_tokens, SHAPES[shape_name].n_layers, batch * seq)
     print(json.dumps(result))
     return 0
 

@@ -94,12 +94,14 @@ __global__ __launch_bounds__(256) void nf4_gemm_rs_kernel(const RsArgs g) {
 
   int tile_m, tile_n;
   {
-    // workgroup ids are dealt round-robin to the 8 XCDs (one L2 each): give every XCD a band of m-tiles
+    // workgroup ids are dealt round-robin to the 8 XCDs (one L2 each): give every XCD a band of m-tiles and walk it
+    // column by column, so the workgroups resident on an XCD share each weight tile through its L2 (the weight is
+    // then fetched once per XCD instead of once per m-tile)
     const int id = blockIdx.x;
     if ((g.tiles_m & 7) == 0) {
-      const int xcd = id & 7, slot = id >> 3;
-      tile_m = xcd * (g.tiles_m >> 3) + slot / g.tiles_n;
-      tile_n = slot % g.tiles_n;
+      const int xcd = id & 7, slot = id >> 3, band = g.tiles_m >> 3;
+      tile_m = xcd * band + slot % band;
+      tile_n = slot / band;
     } else {
       tile_m = id / g.tiles_n;
       tile_n = id % g.tiles_n;
@@ -150,10 +152,10 @@ __global__ __launch_bounds__(256) void nf4_gemm_rs_kernel(const RsArgs g) {
   // bookkeeping for them (it would otherwise wait for ALL outstanding loads before the next LDS read it cannot prove
   // disjoint); completion is awaited explicitly with s_waitcnt vmcnt below.
   auto dma16 = [&](uint32_t voff, const char* base, uint32_t lds) {
-    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(base), "s"(lds) : "memory");
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(base), "s"(lds) : "memory", "m0");
   };
   auto dma4 = [&](uint32_t voff, const char* base, uint32_t lds) {
-    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dword %0, %1" ::"v"(voff), "s"(base), "s"(lds) : "memory");
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" ::"v"(voff), "s"(base), "s"(lds) : "memory", "m0");
   };
   const uint32_t lds0 = (uint32_t)(uintptr_t)TT_LDS_PTR(smem);
   // A batch (k-step t) is kBatch loads: the activation tile -> A stage, this wave's code bytes and scalers -> W stage.
