@@ -112,6 +112,37 @@ def cpu_baseline(shape_name: str, rank: int, alpha: float, tokens_sample: int, l
     }
 
 
+def secondary_kernels(dev) -> dict:
+    """Achieved HBM GB/s of the bandwidth-bound kernels of the path on the largest 8B weight / activation shapes:
+    algorithmic bytes (2.515747 B/element for the NF4 codec, 4 B/element for fake quant) / HIP-event time."""
+    from torchtune_amd import ops, to_nf4
+
+    def timed(fn, iters=20):
+        for _ in range(3):
+            fn()
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(iters):
+            fn()
+        end.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(end) / iters * 1e-3
+
+    out = {}
+    gen = torch.Generator(device=dev).manual_seed(2)
+    W = (torch.randn(14336, 4096, device=dev, generator=gen) * 0.02).to(torch.bfloat16)
+    t = to_nf4(W)
+    n = W.numel()
+    out["nf4_dequantize 14336x4096 bf16"] = round(n * 2.515747 / timed(t.get_original_weight) / 1e9, 1)
+    out["nf4_quantize 14336x4096 bf16"] = round(n * 2.515747 / timed(lambda: ops.nf4_quantize(W, 64, 256)) / 1e9, 1)
+    out["fq_per_group_int4_sym g32 14336x4096 bf16"] = round(
+        (n * 4 + n / 32 * 4) / timed(lambda: ops.fq_per_group_int4_sym(W, 32)) / 1e9, 1)
+    x = torch.randn(8192, 14336, device=dev, generator=gen).to(torch.bfloat16)
+    out["fq_per_token_int8_asym 8192x14336 bf16"] = round(
+        x.numel() * 4 / timed(lambda: ops.fq_per_token_int8_asym(x, want_qparams=False)) / 1e9, 1)
+    return {"unit": "GB/s (algorithmic bytes / HIP-event time, HBM peak 8000)", **out}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -206,6 +237,9 @@ def main() -> int:
             "per_shape": per_shape,
         },
     }
+    del model
+    torch.cuda.empty_cache()
+    result["hbm_bound_kernels"] = secondary_kernels(dev)
     if args.cpu_tokens > 0:
         result["cpu_baseline"] = cpu_baseline(shape_name, rank, alpha, args.cpu_tokens, SHAPES[shape_name].n_layers, batch * seq)
     print(json.dumps(result))

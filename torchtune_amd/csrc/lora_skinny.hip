@@ -6,10 +6,10 @@
 //   gA = gh^T . x        [R,K]   contraction over M  (backward)
 //   gB = s . gy^T . h    [N,R]   contraction over M  (backward)
 //
-// The first two contract along the contiguous dimension of the activation: MFMA with the activation rows
+// The first two contract along the contiguous dimension of the activation: bf16 MFMA with the activation rows
 // as the A operand, fragments loaded straight from global memory (a lane's 8 contraction elements are 16
-// contiguous bytes).  The last two contract over rows; a lane owns 4 consecutive columns and accumulates
-// 4 x 16 outputs with scalar-broadcast adapter values.  Both split the contraction over many workgroups to
+// contiguous bytes).  The last two contract over rows: fp32 MFMA (one contraction index per lane, so both
+// operands are read row-major as they lie in memory).  Both split the contraction over many workgroups to
 // put enough loads in flight and combine the fp32 partial sums in a second, fixed-order pass, so results
 // are deterministic.
 #include "common.h"
@@ -27,61 +27,104 @@ typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 
 // ---------------------------------------------------------------------------------------------------
 // skinny_nt: part[split][m][r] = sum_{k in split} X[m][k] * Bm[r][k]        (X [M,Kc], Bm [R,Kc], R <= 64)
-// One wave = 32 rows of X x one split of Kc; RT = number of 32-column tiles of R.
+// Workgroup = 4 waves on the same 32 rows of X; the split's 64-wide contraction chunks are dealt to the waves in
+// turn and the four partial sums are combined through LDS in a fixed order.  MFMA v_mfma_f32_16x16x32_bf16 with the
+// rows of X as the row operand: lane (g = l / 16, i = l % 16) loads the 32 contiguous bytes X[m + i][k0 + 16 g ..
+// + 16) - the four lane groups cover one whole 128-byte line per row - and uses its first 8 elements for one MFMA and
+// the last 8 for the next (the contraction index may be permuted freely as long as both operands agree).
+// RT = number of 16-wide tiles of R.
 // ---------------------------------------------------------------------------------------------------
 template <int RT>
 __global__ __launch_bounds__(256) void skinny_nt_kernel(const uint16_t* __restrict__ X, const uint16_t* __restrict__ Bm,
-                                                        float* __restrict__ part, int M, int Kc, int R, int m_tiles,
-                                                        int splits, int chunks_per_split) {
-  const int wave_global = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (wave_global >= m_tiles * splits) return;
-  const int mt = wave_global % m_tiles, split = wave_global / m_tiles;
-  const int lane = threadIdx.x & 63, l31 = lane & 31, lhi = lane >> 5;
-  int row = mt * 32 + l31;
-  row = row < M ? row : M - 1;
-  const uint16_t* xrow = X + (int64_t)row * Kc + 8 * lhi;
+                                                        float* __restrict__ part, int M, int Kc, int R,
+                                                        int chunks_per_split) {
+  __shared__ float red[3][2 * RT * 4][64];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int g = lane >> 4, i = lane & 15;
+  const int m0 = blockIdx.x * 32;
+  const int split = blockIdx.y;
+  const uint16_t* xrow[2];
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    int row = m0 + 16 * t + i;
+    row = row < M ? row : M - 1;
+    xrow[t] = X + (int64_t)row * Kc + 16 * g;
+  }
   const uint16_t* brow[RT];
   bool bvalid[RT];
 #pragma unroll
   for (int t = 0; t < RT; ++t) {
-    const int r = t * 32 + l31;
+    const int r = t * 16 + i;
     bvalid[t] = r < R;
-    brow[t] = Bm + (int64_t)(bvalid[t] ? r : 0) * Kc + 8 * lhi;
+    brow[t] = Bm + (int64_t)(bvalid[t] ? r : 0) * Kc + 16 * g;
   }
-  f32x16_t acc[RT];
+  f32x4_t acc[2][RT];
 #pragma unroll
-  for (int t = 0; t < RT; ++t)
+  for (int t = 0; t < 2; ++t)
 #pragma unroll
-    for (int v = 0; v < 16; ++v) acc[t][v] = 0.f;
+    for (int u = 0; u < RT; ++u) acc[t][u] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
   const int total_chunks = Kc >> 6;
   const int c0 = split * chunks_per_split;
   int c1 = c0 + chunks_per_split;
   c1 = c1 < total_chunks ? c1 : total_chunks;
-  for (int c = c0; c < c1; ++c) {
+  // Workgroups that run side by side differ in their row tile only; were they all to start at the same column, every
+  // one of them would be on the same few memory channels (rows are a power-of-two number of bytes apart).  Each row
+  // tile therefore walks its chunks in a rotated order.  The order is a fixed function of the tile: deterministic.
+  const int nc = c1 - c0;
+  const int rot = nc > 0 ? (int)((blockIdx.x * 4u) % (unsigned)nc) : 0;
+#pragma unroll 2
+  for (int j = wave; j < nc; j += 4) {
+    int c = j + rot;
+    c = c0 + (c >= nc ? c - nc : c);
     const int k0 = c * 64;
-    bf16x8_t a[4];
+    u32x4_t xa[2][2], wb[RT][2];
 #pragma unroll
-    for (int s = 0; s < 4; ++s) a[s] = *reinterpret_cast<const bf16x8_t*>(xrow + k0 + 16 * s);
+    for (int t = 0; t < 2; ++t)
 #pragma unroll
-    for (int t = 0; t < RT; ++t) {
+      for (int hh = 0; hh < 2; ++hh)
+        xa[t][hh] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(xrow[t] + k0 + 8 * hh));
 #pragma unroll
-      for (int s = 0; s < 4; ++s) {
-        u32x4_t raw = {0, 0, 0, 0};
-        if (bvalid[t]) raw = *reinterpret_cast<const u32x4_t*>(brow[t] + k0 + 16 * s);
-        acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[s], __builtin_bit_cast(bf16x8_t, raw), acc[t], 0, 0, 0);
+    for (int u = 0; u < RT; ++u)
+#pragma unroll
+      for (int hh = 0; hh < 2; ++hh) {
+        wb[u][hh] = u32x4_t{0, 0, 0, 0};
+        if (bvalid[u]) wb[u][hh] = *reinterpret_cast<const u32x4_t*>(brow[u] + k0 + 8 * hh);
       }
-    }
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int u = 0; u < RT; ++u)
+#pragma unroll
+        for (int hh = 0; hh < 2; ++hh)
+          acc[t][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, xa[t][hh]),
+                                                             __builtin_bit_cast(bf16x8_t, wb[u][hh]), acc[t][u], 0, 0, 0);
   }
+  // acc[t][u][v] = C[m0 + 16 t + 4 g + v][16 u + i]
+  if (wave > 0) {
 #pragma unroll
-  for (int t = 0; t < RT; ++t) {
-    const int col = t * 32 + l31;
-    if (col >= R) continue;
+    for (int t = 0; t < 2; ++t)
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      const int r = mt * 32 + 8 * (v >> 2) + 4 * lhi + (v & 3);
-      if (r < M) part[((int64_t)split * M + r) * R + col] = acc[t][v];
-    }
+      for (int u = 0; u < RT; ++u)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) red[wave - 1][(t * RT + u) * 4 + v][lane] = acc[t][u][v];
+  }
+  __syncthreads();
+  if (wave == 0) {
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int u = 0; u < RT; ++u) {
+        const int col = 16 * u + i;
+        if (col >= R) continue;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          const int r = m0 + 16 * t + 4 * g + v;
+          const int e = (t * RT + u) * 4 + v;
+          if (r < M) part[((int64_t)split * M + r) * R + col] = ((acc[t][u][v] + red[0][e][lane]) + red[1][e][lane]) + red[2][e][lane];
+        }
+      }
   }
 }
 
@@ -91,6 +134,7 @@ __global__ __launch_bounds__(256) void sum_partials_kernel(const float* __restri
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (i >= n) return;
   float s = 0.f;
+#pragma unroll 8
   for (int p = 0; p < splits; ++p) s += part[(int64_t)p * n + i];
   out[i] = f32_to_bf16_bits(s * scale);
 }
@@ -106,57 +150,81 @@ __global__ __launch_bounds__(256) void transpose_small_kernel(const uint16_t* __
 }
 
 // ---------------------------------------------------------------------------------------------------
-// skinny_tn: part[split][r][k] = sum_{m in split} G[m][r0 + r] * X[m][k]      (G [M,R], X [M,Kc])
-// Workgroup = 4 waves on the same 256 columns, each wave a quarter of the split's rows; lane owns 4 columns.
+// skinny_tn: part[split][r0 + r][c] = sum_{m in split} G[m][r0 + r] * X[m][c]   (G [M,R], X [M,Kc], r < 16)
+// The contraction runs over rows, so both operands are read in their natural row-major layout by the fp32 MFMA
+// v_mfma_f32_16x16x4_f32, whose operands hold ONE contraction index per lane: lane (g = l / 16, q = l % 16) supplies
+// G[m + g][r0 + q] as the row operand and X[m + g][c] as the column operand, four rows m..m+3 per instruction.
+// A lane loads 8 consecutive columns (16 bytes) of its row and feeds them to 8 MFMAs, so MFMA e of the wave covers the
+// columns {c0 + 8 q + e}; its 16x16 result D[r][.] is lane q's column c0 + 8 q + e, i.e. a lane ends up with 8
+// consecutive columns for each of its 4 result rows r = 4 g + v.
+// Workgroup = 4 waves on the same 128 columns, taking the split's 4-row steps in turn; partial sums are combined
+// through LDS in a fixed order, then across splits by sum_partials_tn_kernel.
 // ---------------------------------------------------------------------------------------------------
-template <int RC>
+constexpr int kTnCols = 128;   // columns per workgroup
+constexpr int kTnUnroll = 4;   // 4-row steps in flight per wave
+
 __global__ __launch_bounds__(256) void skinny_tn_kernel(const uint16_t* __restrict__ G, const uint16_t* __restrict__ X,
                                                         float* __restrict__ part, int M, int Kc, int R, int r0,
                                                         int rows_per_split) {
-  __shared__ float red[3][RC * 4][64];
+  __shared__ float red[3][32][64];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int col = blockIdx.x * 256 + lane * 4;
-  const bool col_ok = col < Kc;  // Kc % 8 == 0, so a lane's 4 columns are in or out together
+  const int g = lane >> 4, q = lane & 15;
+  const int col = blockIdx.x * kTnCols + q * 8;
+  const bool col_ok = col < Kc;  // Kc % 8 == 0: a lane's 8 columns are in or out together
+  const bool r_ok = r0 + q < R;
   const int split = blockIdx.y;
   const int m_begin = split * rows_per_split;
   int m_end = m_begin + rows_per_split;
   m_end = m_end < M ? m_end : M;
-  float acc[RC][4];
-#pragma unroll
-  for (int r = 0; r < RC; ++r)
-#pragma unroll
-    for (int e = 0; e < 4; ++e) acc[r][e] = 0.f;
 
-  const uint16_t* xcol = X + (col_ok ? col : 0);
-  for (int m = m_begin + wave; m < m_end; m += 4) {
-    u32x2_t xv = {0, 0};
-    if (col_ok) xv = *reinterpret_cast<const u32x2_t*>(xcol + (int64_t)m * Kc);
-    const float x0 = bits_f32(xv.x << 16), x1 = bits_f32(xv.x & 0xffff0000u);
-    const float x2 = bits_f32(xv.y << 16), x3 = bits_f32(xv.y & 0xffff0000u);
-    const uint32_t* grow = reinterpret_cast<const uint32_t*>(G + (int64_t)m * R + r0);  // wave-uniform address
+  f32x4_t acc[8];
 #pragma unroll
-    for (int rp = 0; rp < RC / 2; ++rp) {
-      const uint32_t gp = grow[rp];
-      const float g0 = bits_f32(gp << 16), g1 = bits_f32(gp & 0xffff0000u);
-      acc[2 * rp][0] += g0 * x0; acc[2 * rp][1] += g0 * x1; acc[2 * rp][2] += g0 * x2; acc[2 * rp][3] += g0 * x3;
-      acc[2 * rp + 1][0] += g1 * x0; acc[2 * rp + 1][1] += g1 * x1; acc[2 * rp + 1][2] += g1 * x2; acc[2 * rp + 1][3] += g1 * x3;
+  for (int e = 0; e < 8; ++e) acc[e] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+  const uint16_t* xp = X + (col_ok ? col : 0);
+  const uint16_t* gp = G + (r_ok ? r0 + q : 0);
+  for (int m = m_begin + 4 * wave; m < m_end; m += 16 * kTnUnroll) {
+    u32x4_t xv[kTnUnroll];
+    uint32_t gv[kTnUnroll];
+#pragma unroll
+    for (int u = 0; u < kTnUnroll; ++u) {
+      const int row = m + 16 * u + g;
+      const bool ok = row < m_end;
+      xv[u] = u32x4_t{0, 0, 0, 0};
+      gv[u] = 0;
+      if (ok && col_ok) xv[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(xp + (int64_t)row * Kc));
+      if (ok && r_ok) gv[u] = gp[(int64_t)row * R];
+    }
+#pragma unroll
+    for (int u = 0; u < kTnUnroll; ++u) {
+      const float a = bits_f32(gv[u] << 16);
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {
+        acc[2 * d] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, bits_f32(xv[u][d] << 16), acc[2 * d], 0, 0, 0);
+        acc[2 * d + 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, bits_f32(xv[u][d] & 0xffff0000u), acc[2 * d + 1], 0, 0, 0);
+      }
     }
   }
   if (wave > 0) {
 #pragma unroll
-    for (int r = 0; r < RC; ++r)
+    for (int e = 0; e < 8; ++e)
 #pragma unroll
-      for (int e = 0; e < 4; ++e) red[wave - 1][r * 4 + e][lane] = acc[r][e];
+      for (int v = 0; v < 4; ++v) red[wave - 1][v * 8 + e][lane] = acc[e][v];
   }
   __syncthreads();
   if (wave == 0 && col_ok) {
 #pragma unroll
-    for (int r = 0; r < RC; ++r) {
-      f32x4_t o;
+    for (int v = 0; v < 4; ++v) {
+      const int r = r0 + 4 * g + v;
+      if (r >= R) continue;
+      float o[8];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) o[e] = ((acc[r][e] + red[0][r * 4 + e][lane]) + red[1][r * 4 + e][lane]) + red[2][r * 4 + e][lane];
-      *reinterpret_cast<f32x4_t*>(part + ((int64_t)split * R + r0 + r) * Kc + col) = o;
+      for (int e = 0; e < 8; ++e)
+        o[e] = ((acc[e][v] + red[0][v * 8 + e][lane]) + red[1][v * 8 + e][lane]) + red[2][v * 8 + e][lane];
+      float* dst = part + ((int64_t)split * R + r) * Kc + col;
+      *reinterpret_cast<f32x4_t*>(dst) = f32x4_t{o[0], o[1], o[2], o[3]};
+      *reinterpret_cast<f32x4_t*>(dst + 4) = f32x4_t{o[4], o[5], o[6], o[7]};
     }
   }
 }
@@ -169,6 +237,7 @@ __global__ __launch_bounds__(256) void sum_partials_tn_kernel(const float* __res
   const int64_t n = (int64_t)R * Kc;
   if (i >= n) return;
   float s = 0.f;
+#pragma unroll 8
   for (int p = 0; p < splits; ++p) s += part[(int64_t)p * n + i];
   const int64_t r = i / Kc, k = i % Kc;
   out[r * stride_r + k * stride_k] = f32_to_bf16_bits(s * scale);
@@ -183,9 +252,10 @@ NtPlan plan_nt(int64_t M, int64_t Kc) {
   NtPlan p;
   p.m_tiles = (int)((M + 31) / 32);
   const int total_chunks = (int)(Kc / 64);
-  int s = kTargetWaves / p.m_tiles;
+  int s = kTargetWaves / 4 / p.m_tiles;  // workgroups of 4 waves
   s = s < 1 ? 1 : s;
-  s = s > total_chunks ? total_chunks : s;
+  const int max_s = (total_chunks + 7) / 8;  // at least two chunks per wave
+  s = s > max_s ? max_s : s;
   p.chunks_per_split = (total_chunks + s - 1) / s;
   p.splits = (total_chunks + p.chunks_per_split - 1) / p.chunks_per_split;
   return p;
@@ -197,12 +267,12 @@ struct TnPlan {
 };
 TnPlan plan_tn(int64_t M, int64_t Kc) {
   TnPlan p;
-  p.col_groups = (int)((Kc + 255) / 256);
-  int s = kTargetWaves / 4 / p.col_groups;
+  p.col_groups = (int)((Kc + kTnCols - 1) / kTnCols);
+  int s = kTargetWaves / 4 / p.col_groups;  // workgroups of 4 waves
   s = s < 1 ? 1 : s;
-  const int max_s = (int)((M + 15) / 16);  // at least 4 rows per wave
+  const int max_s = (int)((M + 63) / 64);  // at least 64 rows per split: four 4-row steps per wave
   s = s > max_s ? max_s : s;
-  p.rows_per_split = (int)((M + s - 1) / s);
+  p.rows_per_split = (int)(((M + s - 1) / s + 15) / 16 * 16);  // whole rounds of the four waves
   p.splits = (int)((M + p.rows_per_split - 1) / p.rows_per_split);
   return p;
 }
@@ -213,12 +283,13 @@ size_t align256(size_t v) { return (v + 255) & ~size_t(255); }
 int run_nt(const uint16_t* X, const uint16_t* Bm, int64_t M, int64_t Kc, int R, float scale, uint16_t* out, float* ws,
            hipStream_t s) {
   const NtPlan p = plan_nt(M, Kc);
-  const int waves = p.m_tiles * p.splits;
-  const dim3 grid((unsigned)((waves + 3) / 4)), block(256);
-  if (R <= 32)
-    skinny_nt_kernel<1><<<grid, block, 0, s>>>(X, Bm, ws, (int)M, (int)Kc, R, p.m_tiles, p.splits, p.chunks_per_split);
+  const dim3 grid((unsigned)p.m_tiles, (unsigned)p.splits), block(256);
+  if (R <= 16)
+    skinny_nt_kernel<1><<<grid, block, 0, s>>>(X, Bm, ws, (int)M, (int)Kc, R, p.chunks_per_split);
+  else if (R <= 32)
+    skinny_nt_kernel<2><<<grid, block, 0, s>>>(X, Bm, ws, (int)M, (int)Kc, R, p.chunks_per_split);
   else
-    skinny_nt_kernel<2><<<grid, block, 0, s>>>(X, Bm, ws, (int)M, (int)Kc, R, p.m_tiles, p.splits, p.chunks_per_split);
+    skinny_nt_kernel<4><<<grid, block, 0, s>>>(X, Bm, ws, (int)M, (int)Kc, R, p.chunks_per_split);
   const int64_t n = M * R;
   sum_partials_kernel<<<dim3((unsigned)((n + 255) / 256)), block, 0, s>>>(ws, n, p.splits, scale, out);
   return check_launch("skinny_nt");
@@ -228,10 +299,8 @@ int run_tn(const uint16_t* G, const uint16_t* X, int64_t M, int64_t Kc, int R, f
            int64_t stride_k, uint16_t* out, float* ws, hipStream_t s) {
   const TnPlan p = plan_tn(M, Kc);
   const dim3 grid((unsigned)p.col_groups, (unsigned)p.splits), block(256);
-  int r0 = 0;
-  for (; r0 + 16 <= R; r0 += 16)
-    skinny_tn_kernel<16><<<grid, block, 0, s>>>(G, X, ws, (int)M, (int)Kc, R, r0, p.rows_per_split);
-  if (r0 < R) skinny_tn_kernel<8><<<grid, block, 0, s>>>(G, X, ws, (int)M, (int)Kc, R, r0, p.rows_per_split);
+  for (int r0 = 0; r0 < R; r0 += 16)
+    skinny_tn_kernel<<<grid, block, 0, s>>>(G, X, ws, (int)M, (int)Kc, R, r0, p.rows_per_split);
   const int64_t n = (int64_t)R * Kc;
   sum_partials_tn_kernel<<<dim3((unsigned)((n + 255) / 256)), block, 0, s>>>(ws, R, (int)Kc, p.splits, scale, stride_r,
                                                                              stride_k, out);
