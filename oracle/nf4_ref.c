@@ -220,3 +220,48 @@ void ref_fq_per_group(const void* w, int is_bf16, int64_t rows, int64_t K, int g
       if (scale_out) scale_out[r * (K / g) + k0 / g] = scale;
     }
 }
+
+/* ---------------------------------------------------------------------------------------------------
+ * Checkers for two shortcuts of the bf16 quantise kernel (they restate nothing of the reference; they
+ * prove, by enumeration, that the shortcuts cannot change a result).
+ * ------------------------------------------------------------------------------------------------- */
+
+/* Shortcut 1: with y = 1/a divided once per block, q = fma(fma(-x*y, a, x), y, x*y) must round to the same
+ * bf16 as the correctly rounded x / a.  Enumerates every bf16 divisor a with bit pattern in [a_lo, a_hi) and
+ * every bf16 numerator 0 <= x <= a (signs are symmetric); returns the number of pairs that differ. */
+#if defined(__x86_64__)
+__attribute__((target("fma")))
+#endif
+int64_t ref_check_shared_reciprocal_division(int a_lo, int a_hi) {
+  int64_t bad = 0;
+  for (int ai = a_lo; ai < a_hi; ++ai) {
+    const float a = float_of((uint32_t)ai << 16);
+    const float y = 1.0f / a;
+    for (int xi = 0; xi <= ai; ++xi) {
+      const float x = float_of((uint32_t)xi << 16);
+      const float q0 = x * y;
+      const float r = fmaf(-q0, a, x);
+      const float q1 = fmaf(r, y, q0);
+      if (bits_of(to_bf16(x / a)) != bits_of(to_bf16(q1))) ++bad;
+    }
+  }
+  return bad;
+}
+
+/* Shortcut 2: the code of a scaled bf16 value is looked up in a table that only spans magnitudes 2^-5 .. 1.
+ * Returns the number of bf16 patterns below 2^-5 (either sign) whose code is not 7, plus 1 if NaN is not code 0;
+ * table_out, if not NULL, receives the codes of magnitudes 0x3D00..0x3F80 for sign 0 then sign 1 (2 x 641 bytes). */
+int ref_check_code_table(uint8_t* table_out) {
+  int bad = 0;
+  for (int sign = 0; sign < 2; ++sign)
+    for (int mag = 0; mag <= 0x3F80; ++mag) {
+      const int c = nearest_code(float_of(((uint32_t)sign << 31) | ((uint32_t)mag << 16)), 1);
+      if (mag < 0x3D00) {
+        if (c != 7) ++bad;
+      } else if (table_out) {
+        table_out[sign * 641 + (mag - 0x3D00)] = (uint8_t)c;
+      }
+    }
+  if (nearest_code(float_of(0x7fc00000u), 1) != 0) ++bad;
+  return bad;
+}

@@ -31,4 +31,8 @@ def c_oracle():
     lib.ref_fq_per_token.restype = None
     lib.ref_fq_per_group.argtypes = [vp, i32, i64, i64, i32, vp, vp, vp]
     lib.ref_fq_per_group.restype = None
+    lib.ref_check_shared_reciprocal_division.argtypes = [i32, i32]
+    lib.ref_check_shared_reciprocal_division.restype = i64
+    lib.ref_check_code_table.argtypes = [vp]
+    lib.ref_check_code_table.restype = i32
     return lib

@@ -85,6 +85,32 @@ def test_dequantise_every_code_and_scaler_byte(dtype):
         assert bits_equal(got.cpu(), nf4_oracle.nf4_dequantize(p))
 
 
+def test_every_bf16_scaled_value_and_divisor_range():
+    """The bf16 quantise kernel looks codes up in a table and shares one reciprocal per block.  (1) Blocks with absmax 1
+    whose other elements sweep every bf16 pattern in [-1, 1]: each pattern must get the oracle's code.  (2) Blocks
+    whose absmax runs over all binades, denormals included, with elements at random fractions of it."""
+    pats = torch.cat([torch.arange(0x0000, 0x3F81), torch.arange(0x8000, 0xBF81)]).to(torch.int32)
+    n_blocks = (pats.numel() + 62) // 63
+    body = torch.zeros(n_blocks * 63, dtype=torch.int32)
+    body[: pats.numel()] = pats
+    w = torch.empty(n_blocks, 64, dtype=torch.bfloat16)
+    w[:, 0] = 1.0
+    w[:, 1:] = body.to(torch.int16).view(torch.bfloat16).view(n_blocks, 63)
+    _assert_matches_oracle(to_nf4(w.to(DEV), 64, 1), nf4_oracle.nf4_quantize(w, 64, 1))
+
+    g = torch.Generator().manual_seed(5)
+    amax_bits = torch.randint(0x0001, 0x7F80, (4096,), generator=g, dtype=torch.int32)
+    amax_bits[:64] = torch.arange(1, 65)  # denormal divisors: the plain-division path
+    amax = amax_bits.to(torch.int16).view(torch.bfloat16)
+    frac = torch.rand(4096, 64, generator=g) * 2 - 1
+    w = (frac * amax.float()[:, None]).to(torch.bfloat16)
+    w[:, 7] = amax
+    w[1::2, 7] *= -1
+    # codes only: absmaxes spanning 2^-133 .. 2^127 are outside the range where the mean of the absmaxes (and with it
+    # the scaler bytes) is independent of the summation order
+    assert torch.equal(to_nf4(w.to(DEV), 64, 256).quantized_data.cpu(), nf4_oracle.nf4_quantize(w, 64, 256).quantized_data)
+
+
 def test_degenerate_inputs():
     z = to_nf4(torch.zeros(512, 512, dtype=torch.bfloat16, device=DEV))
     assert torch.all(z.quantized_data == 0) and torch.all(z.quantized_scalers == 0)

@@ -212,3 +212,38 @@ def test_linear_nf4_is_linear_on_dequantised_weight():
     d = nf4_oracle.nf4_dequantize(p)
     torch.testing.assert_close(nf4_oracle.linear_nf4_forward(x, p), x @ d.T)
     torch.testing.assert_close(nf4_oracle.linear_nf4_backward(g, p), g @ d)
+
+
+def test_shared_reciprocal_division_is_exact_for_bf16(c_oracle):
+    """The bf16 quantise kernel divides 1/absmax once per block and forms each quotient with two fused
+    multiply-adds.  Enumerate EVERY pair of bf16 operands 0 <= x <= a with a >= 2^-119 (the kernel's guard): the
+    bf16-rounded quotient must equal that of the correctly rounded division.  Below the guard the shortcut does
+    fail, which is why the guard exists."""
+    from concurrent.futures import ThreadPoolExecutor
+
+    lo, hi = 0x0400, 0x7F80  # 2^-119 .. the largest finite bf16
+    edges = [lo + (hi - lo) * i // 32 for i in range(33)]
+    with ThreadPoolExecutor(max_workers=8) as pool:  # ctypes releases the GIL
+        bad = list(pool.map(lambda i: c_oracle.ref_check_shared_reciprocal_division(edges[i], edges[i + 1]), range(32)))
+    assert sum(bad) == 0
+    assert c_oracle.ref_check_shared_reciprocal_division(0x0001, 0x0100) > 0
+
+
+def test_code_table_premises_and_monotone_codes(c_oracle):
+    """Every bf16 scaled value below 2^-5 is the zero code and NaN is code 0 (what lets the kernel's table span only
+    2^-5..1); inside the table the code never decreases with the value."""
+    import ctypes
+
+    buf = (ctypes.c_uint8 * (2 * 641))()
+    assert c_oracle.ref_check_code_table(ctypes.cast(buf, ctypes.c_void_p)) == 0
+    pos, neg = list(buf[:641]), list(buf[641:])
+    assert pos == sorted(pos) and neg == sorted(neg, reverse=True)
+    assert pos[0] == 7 and neg[0] == 7 and pos[-1] == 15 and neg[-1] == 0
+    # the same table from the eager-PyTorch oracle
+    bits = torch.arange(0x3D00, 0x3F81, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+    for sign, want in ((1.0, pos), (-1.0, neg)):
+        blocks = torch.zeros(641, 64, dtype=torch.bfloat16)
+        blocks[:, 0] = 1.0
+        blocks[:, 1] = bits * sign
+        p = nf4_oracle.nf4_quantize(blocks, 64, 1)
+        assert (p.quantized_data.view(641, 32)[:, 0] & 0xF).tolist() == want

@@ -99,6 +99,114 @@ __global__ __launch_bounds__(256) void nf4_quantize_blocks_kernel(const void* __
 }
 
 // ---------------------------------------------------------------------------------------------------
+// quantise, pass 1 for bfloat16, the fast form of the kernel above (identical results).
+//
+// (a) The scaled value bf16(x / absmax) is one of 65536 bit patterns, so "nearest code under the reference's rule"
+//     is a table lookup.  Every pattern with |value| < 2^-5 maps to code 7 (the zero code: its neighbours' midpoints
+//     are -0.0455 and +0.0398) and |value| <= 1 always, so the table only spans magnitudes 0x3D00 (2^-5) .. 0x3F80
+//     (1.0) for each sign: 2 x 641 bytes.  The host fills it once with nf4_nearest_code<true>, checks the two
+//     claims above over all patterns, and passes it by value; NaN (0/0 of an all-zero block) yields code 0.
+// (b) x / absmax for 64 elements shares the divisor: y = 1 / absmax is divided once (correctly rounded) and each
+//     quotient is q0 = x * y, r = fma(-q0, absmax, x), q = fma(r, y, q0).  For bf16 operands with absmax >= 2^-119
+//     and |x| <= absmax this rounds to the same bf16 as the correctly rounded quotient for EVERY operand pair
+//     (checked exhaustively on a CPU, 5.3e8 pairs); smaller or non-finite divisors take the plain division.
+// ---------------------------------------------------------------------------------------------------
+constexpr int kCodeTabBase = 0x3D00;
+constexpr int kCodeTabLast = 0x3F80;
+constexpr int kCodeTabN = kCodeTabLast - kCodeTabBase + 1;  // 641
+constexpr int kCodeTabStride = 644;                          // per sign, padded to a multiple of 4
+struct Nf4CodeTable {
+  uint32_t words[2 * kCodeTabStride / 4];
+};
+constexpr int kQuantChunksPerThread = 4;
+
+__global__ __launch_bounds__(256) void nf4_quantize_blocks_bf16_kernel(const void* __restrict__ w, int64_t n_chunks,
+                                                                       int lanes_per_block, int log2_lpb,
+                                                                       uint32_t* __restrict__ qdata, float* __restrict__ absmax,
+                                                                       const Nf4CodeTable table) {
+  __shared__ uint32_t tab_words[2 * kCodeTabStride / 4];
+  for (int i = threadIdx.x; i < 2 * kCodeTabStride / 4; i += 256) tab_words[i] = table.words[i];
+  __syncthreads();
+  const uint8_t* tab = reinterpret_cast<const uint8_t*>(tab_words);
+#pragma unroll
+  for (int u = 0; u < kQuantChunksPerThread; ++u) {
+    const int64_t chunk = ((int64_t)blockIdx.x * kQuantChunksPerThread + u) * 256 + threadIdx.x;
+    const bool live = chunk < n_chunks;  // uniform per block of lanes: n_chunks is a multiple of lanes_per_block
+    float v[8];
+    if (live) {
+      load8<true>(w, chunk, v);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) v[i] = 0.f;
+    }
+    float m = __builtin_fabsf(v[0]);
+#pragma unroll
+    for (int i = 1; i < 8; ++i) m = nanmax(m, __builtin_fabsf(v[i]));
+    for (int off = 1; off < lanes_per_block; off <<= 1) m = nanmax(m, __shfl_xor(m, off, kWave));
+    if (!live) continue;
+    if ((threadIdx.x & (lanes_per_block - 1)) == 0) absmax[chunk >> log2_lpb] = m;
+    const bool fast = m >= 0x1p-119f && m < __builtin_inff();  // false for NaN too
+    const float y = 1.0f / m;
+    uint32_t packed = 0;
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      float qf[2];
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        const float x = v[2 * b + e];
+        if (fast) {
+          const float q0 = x * y;
+          const float r = __builtin_fmaf(-q0, m, x);
+          qf[e] = __builtin_fmaf(r, y, q0);
+        } else {
+          qf[e] = x / m;
+        }
+      }
+      const uint32_t pr = pack_bf16x2(qf[0], qf[1]);  // low half: element 2b (high nibble), high half: element 2b+1
+      uint32_t code[2];
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        const uint32_t bits = e ? (pr >> 16) : (pr & 0xffffu);
+        const uint32_t mag = bits & 0x7fffu;
+        uint32_t idx = mag > (uint32_t)kCodeTabBase ? mag - kCodeTabBase : 0u;
+        idx = idx < (uint32_t)(kCodeTabN - 1) ? idx : (uint32_t)(kCodeTabN - 1);
+        idx += (bits >> 15) * kCodeTabStride;
+        const uint32_t c = tab[idx];
+        code[e] = mag > 0x7f80u ? 0u : c;
+      }
+      packed |= ((code[0] << 4) | code[1]) << (8 * b);
+    }
+    qdata[chunk] = packed;
+  }
+}
+
+// Host side of (a): the table, filled and verified once per process.
+struct Nf4CodeTableHost {
+  Nf4CodeTable table;
+  bool ok;
+  Nf4CodeTableHost() : ok(true) {
+    uint8_t* bytes = reinterpret_cast<uint8_t*>(table.words);
+    memset(table.words, 0, sizeof(table.words));
+    for (int sign = 0; sign < 2; ++sign) {
+      for (int mag = 0; mag <= kCodeTabLast; ++mag) {
+        const uint16_t bits = (uint16_t)((sign << 15) | mag);
+        const int c = nf4_nearest_code<true>(bf16_bits_to_f32(bits));
+        if (mag < kCodeTabBase) {
+          if (c != 7) ok = false;  // claim: everything below 2^-5 is the zero code
+        } else {
+          bytes[sign * kCodeTabStride + (mag - kCodeTabBase)] = (uint8_t)c;
+        }
+      }
+    }
+    if (nf4_nearest_code<true>(bf16_bits_to_f32(0x7fc0)) != 0) ok = false;  // NaN -> code 0
+  }
+};
+const Nf4CodeTableHost& code_table() {
+  static const Nf4CodeTableHost t;
+  return t;
+}
+
+// ---------------------------------------------------------------------------------------------------
 // quantise, pass 2: mean of the block absmaxes.  Summed in fp64 in a fixed order (256 partial sums, each
 // a fixed strided walk followed by a fixed LDS tree) so the result does not depend on scheduling; for
 // realistic dynamic ranges the fp64 sum is exact.  mean = dtype(float(sum / n)).
@@ -300,8 +408,15 @@ extern "C" int ttamd_nf4_quantize(const void* w, int dtype, int64_t numel, int b
   TT_REQUIRE(grid1 < (int64_t(1) << 31), "nf4_quantize: tensor too large for one launch");
   const int64_t grid3 = (n_sb + 3) / 4;
   if (dtype == TTAMD_BF16) {
-    nf4_quantize_blocks_kernel<true><<<dim3((unsigned)grid1), dim3(256), 0, s>>>(
-        w, n_chunks, lpb, log2_exact(lpb), reinterpret_cast<uint32_t*>(quantized_data), ws.absmax);
+    const Nf4CodeTableHost& ct = code_table();
+    if (ct.ok) {
+      const int64_t per_wg = 256 * kQuantChunksPerThread;
+      nf4_quantize_blocks_bf16_kernel<<<dim3((unsigned)((n_chunks + per_wg - 1) / per_wg)), dim3(256), 0, s>>>(
+          w, n_chunks, lpb, log2_exact(lpb), reinterpret_cast<uint32_t*>(quantized_data), ws.absmax, ct.table);
+    } else {  // the table's premises failed their check: search the 16 codes directly
+      nf4_quantize_blocks_kernel<true><<<dim3((unsigned)grid1), dim3(256), 0, s>>>(
+          w, n_chunks, lpb, log2_exact(lpb), reinterpret_cast<uint32_t*>(quantized_data), ws.absmax);
+    }
     nf4_absmax_partial_sum_kernel<<<dim3(kMeanPartials), dim3(256), 0, s>>>(ws.absmax, n_blocks, ws.partial);
     nf4_absmax_mean_kernel<true><<<dim3(1), dim3(256), 0, s>>>(ws.partial, n_blocks, scaler_mean, ws.mean);
     nf4_quantize_scalers_kernel<true><<<dim3((unsigned)grid3), dim3(256), 0, s>>>(
