@@ -27,7 +27,10 @@ WORKLOADS = {
     "llama3_2_1b": ("llama3_2_1b", 8, 16.0, 4, 2048, False),
     "llama3_1_8b": ("llama3_1_8b", 16, 32.0, 4, 2048, False),
     "llama3_1_70b": ("llama3_1_70b", 16, 32.0, 1, 4096, True),
+    # 8da4w QAT of the 8B shape (rank/alpha unused): every linear fake-quantised, group size 32, batch 2 x 4096
+    "llama3_1_8b_qat": ("llama3_1_8b", 0, 0.0, 2, 4096, False),
 }
+HBM_PEAK_GBPS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 # HBM-side bytes per fused-GEMM launch (average over the launches of one step), from the FETCH_SIZE / WRITE_SIZE counter
 # runs summarised in profiles/nf4_gemm_rs_kernel_hbm_traffic.txt (counters cannot be read from inside this process).
@@ -63,6 +66,64 @@ class GemmTimer:
         per_shape = {k: {"launches": v[0], "avg_us": round(1e3 * v[1] / v[0], 1), "tflops": round(v[2] / v[1] / 1e9, 1)}
                      for k, v in by.items()}
         return len(self.records), total_ms, total_flops, per_shape
+
+
+class FqTimer:
+    """Collects (bytes, start event, end event) for every fake-quant launch while installed in ``ops``.
+    Algorithmic bytes: one read and one write of the tensor, plus the fp32 qparams the launch writes."""
+
+    def __init__(self):
+        self.records = []
+
+    def __call__(self, kind, rows, K, group_size, elem_bytes):
+        n = rows * K
+        nbytes = 2 * n * elem_bytes + (rows * 8 if kind == "per_token" else n // group_size * 4)
+        start = torch.cuda.Event(enable_timing=True)
+        end = torch.cuda.Event(enable_timing=True)
+        self.records.append((kind, nbytes, start, end))
+        return start, end
+
+    def summary(self):
+        by = {}
+        for kind, nbytes, s, e in self.records:
+            acc = by.setdefault(kind, [0, 0.0, 0.0])
+            acc[0] += 1
+            acc[1] += s.elapsed_time(e)
+            acc[2] += nbytes
+        return {k: {"launches": v[0], "avg_us": round(1e3 * v[1] / v[0], 1), "gbps": round(v[2] / v[1] / 1e6, 1),
+                    "ms": v[1], "bytes": v[2]} for k, v in by.items()}
+
+
+def cpu_baseline_qat(shape_name: str, group: int, layers: int, max_tokens: int, min_seconds: float = 10.0):
+    """CPU oracle of the fake-quantised linear (eager PyTorch: fq(x), fq(W), F.linear, straight-through backward) on
+    one decoder layer's seven linears at the workload's token count, repeated until `min_seconds`; tokens/s for the
+    full depth."""
+    from oracle import fake_quant_oracle as fqo
+    from torchtune_amd.harness import SHAPES
+
+    s = SHAPES[shape_name]
+    kv = s.n_kv_heads * s.head_dim
+    dims = [(s.dim, s.dim), (kv, s.dim), (kv, s.dim), (s.dim, s.dim), (s.hidden, s.dim), (s.hidden, s.dim), (s.dim, s.hidden)]
+    gen = torch.Generator().manual_seed(0)
+    cores = torch.get_num_threads()
+    ws = [(torch.randn(N, K, generator=gen) * 0.02).to(torch.bfloat16).requires_grad_() for N, K in dims]
+    xs = [torch.randn(max_tokens, K, generator=gen).to(torch.bfloat16).requires_grad_() for _, K in dims]
+    reps, dt = 0, 0.0
+    t0 = time.perf_counter()
+    while dt < min_seconds:
+        for w, x in zip(ws, xs):
+            y = fqo.fake_quantized_linear(x, w, group)
+            (y.float() ** 2).sum().backward()
+        reps += 1
+        dt = time.perf_counter() - t0
+    return {
+        "value": round(max_tokens * reps / (dt * layers), 3),
+        "unit": "tokens/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"eager-PyTorch oracle, fwd+bwd of one {shape_name} layer's seven 8da4w fake-quantised linears (group {group}) "
+                  f"at {max_tokens} tokens x {reps} passes ({dt:.1f} s on {cores} threads), extrapolated x{layers} layers",
+    }
 
 
 def cpu_baseline(shape_name: str, rank: int, alpha: float, tokens_sample: int, layers: int, max_tokens: int,
@@ -163,12 +224,17 @@ def main() -> int:
         return 2
 
     from torchtune_amd import ops
-    from torchtune_amd.harness import SHAPES, build_qlora_decoder, train_step
+    from torchtune_amd.harness import SHAPES, build_qat_decoder, build_qlora_decoder, train_step
 
     shape_name, rank, alpha, batch, seq, ac = WORKLOADS[args.workload]
+    qat = args.workload.endswith("_qat")
+    qat_group = 32
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
-    model = build_qlora_decoder(shape_name, rank, alpha, device=dev, seed=0, activation_checkpointing=ac)
+    if qat:
+        model = build_qat_decoder(shape_name, groupsize=qat_group, device=dev, seed=0, activation_checkpointing=ac)
+    else:
+        model = build_qlora_decoder(shape_name, rank, alpha, device=dev, seed=0, activation_checkpointing=ac)
     gen = torch.Generator(device=dev).manual_seed(1)
     vocab = SHAPES[shape_name].vocab
     tokens = torch.randint(0, vocab, (batch, seq), device=dev, generator=gen)
@@ -189,7 +255,9 @@ def main() -> int:
         step()
     torch.cuda.synchronize()
     timer = GemmTimer()
+    fq_timer = FqTimer()
     ops.set_gemm_timer(timer)
+    ops.set_fq_timer(fq_timer)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
@@ -197,10 +265,57 @@ def main() -> int:
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     ops.set_gemm_timer(None)
+    ops.set_fq_timer(None)
+    ms_per_step = 1e3 * dt / args.steps
+
+    if qat:
+        fq = fq_timer.summary()
+        fq_ms = sum(v["ms"] for v in fq.values())
+        fq_bytes = sum(v["bytes"] for v in fq.values())
+        achieved = fq_bytes / fq_ms / 1e6 if fq_ms > 0 else 0.0
+        result = {
+            "metric": "8da4w QAT fwd+bwd tokens/sec (Llama-3.1-8B, 1 GPU)",
+            "value": round(batch * seq * args.steps / dt, 1),
+            "unit": "tokens/s",
+            "n_gpus": 1,
+            "steps": args.steps,
+            "warmup": args.warmup,
+            "ms_per_step": round(ms_per_step, 2),
+            "higher_is_better": True,
+            "scaling": "weak",
+            "vs_baseline": None,
+            "dtype": "bf16",
+            "data": "synthetic (uniform random token ids, random-init N(0,0.02) bf16 weights)",
+            "config": {
+                "workload": f"{shape_name}-shaped decoder, every linear (incl. output) 8da4w fake-quantised: per-token int8 "
+                            f"activations, per-group({qat_group}) int4 weights, batch {batch} x seq {seq}, fwd+bwd with weight "
+                            "gradients, output projection and cross-entropy",
+                "global_batch": batch,
+                "seq_len": seq,
+                "loss": float(loss),
+            },
+            "roofline": {
+                "bound": "hbm",
+                "kernel": "fq_per_token_regs_kernel + fq_per_group_kernel (the fake-quant launches of the step; the matmuls "
+                          "are stock hipBLASLt)",
+                "achieved": round(achieved, 1),
+                "peak": HBM_PEAK_GBPS,
+                "unit": "GB/s",
+                "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                "traffic": None,
+                "fq_ms_per_step": round(fq_ms / args.steps, 2),
+                "per_kernel": {k: {kk: vv for kk, vv in v.items() if kk in ("launches", "avg_us", "gbps")} for k, v in fq.items()},
+            },
+        }
+        del model
+        torch.cuda.empty_cache()
+        if args.cpu_tokens > 0:
+            result["cpu_baseline"] = cpu_baseline_qat(shape_name, qat_group, SHAPES[shape_name].n_layers, batch * seq)
+        print(json.dumps(result))
+        return 0
 
     launches, gemm_ms, gemm_flops, per_shape = timer.summary()
     achieved = gemm_flops / gemm_ms / 1e9 if gemm_ms > 0 else 0.0
-    ms_per_step = 1e3 * dt / args.steps
     result = {
         "metric": "QLoRA fwd+bwd tokens/sec (Llama-3.1-8B, 1 GPU)" if args.workload == "llama3_1_8b"
         else f"QLoRA fwd+bwd tokens/sec ({args.workload}, 1 GPU)",

@@ -253,6 +253,17 @@ def lora_bwd(
 # ---------------------------------------------------------------------------------------------------
 # QAT fake quantisation
 # ---------------------------------------------------------------------------------------------------
+_fq_timer = None
+
+
+def set_fq_timer(timer) -> None:
+    """Install (or with None remove) a callback ``timer(kind, rows, K, group_size, elem_bytes) -> (start_event,
+    end_event)``; the events are recorded on the launch stream around every fake-quant launch (``kind`` is
+    ``"per_token"`` or ``"per_group"``).  Used by the benchmark to time the kernels in place."""
+    global _fq_timer
+    _fq_timer = timer
+
+
 def fq_per_token_int8_asym(x: torch.Tensor, want_qparams: bool = True):
     """x [..., K] -> (fake-quantised x, scale fp32 [rows] | None, zero_point int32 [rows] | None)"""
     _need_gpu(x, "fq_per_token_int8_asym")
@@ -265,7 +276,12 @@ def fq_per_token_int8_asym(x: torch.Tensor, want_qparams: bool = True):
     zp = torch.empty(rows, dtype=torch.int32, device=x.device) if want_qparams else None
     lib = _lib.load()
     with torch.cuda.device(x.device):
+        events = _fq_timer("per_token", rows, K, 0, xc.element_size()) if _fq_timer is not None else None
+        if events:
+            events[0].record()
         rc = lib.ttamd_fq_per_token_int8_asym(xc.data_ptr(), code, rows, K, out.data_ptr(), _ptr(scale), _ptr(zp), _stream(x))
+        if events:
+            events[1].record()
     _lib.check(rc, "fq_per_token_int8_asym")
     return out, scale, zp
 
@@ -281,7 +297,12 @@ def fq_per_group_int4_sym(w: torch.Tensor, group_size: int, want_scale: bool = T
     scale = torch.empty(rows, K // max(group_size, 1), dtype=torch.float32, device=w.device) if want_scale else None
     lib = _lib.load()
     with torch.cuda.device(w.device):
+        events = _fq_timer("per_group", rows, K, group_size, wc.element_size()) if _fq_timer is not None else None
+        if events:
+            events[0].record()
         rc = lib.ttamd_fq_per_group_int4_sym(wc.data_ptr(), code, rows, K, group_size, out.data_ptr(), _ptr(scale), _stream(w))
+        if events:
+            events[1].record()
     _lib.check(rc, "fq_per_group_int4_sym")
     return out, scale
 
