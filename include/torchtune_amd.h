@@ -106,6 +106,21 @@ int ttamd_nf4_block_scalers(const int8_t* quantized_scalers, const void* quantiz
                             int dtype, int64_t n_blocks, int scaler_block_size, void* block_scalers, void* stream);
 
 /*
+ * Merged checkpoint weight of one QLoRA linear in a single pass over the packed weight:
+ *   out = bf16( D(W) + bf16( scale * bf16(lora_b . lora_a) ) )
+ * replaces the state-dict hook's NF4Tensor.to(bf16) (torchtune/modules/common_utils.py:55-59) followed by
+ * get_merged_lora_ckpt's `weight += (alpha / rank) * lora_b @ lora_a` (torchtune/modules/peft/_utils.py:264-266),
+ * with the same three bf16 roundings; the rank-r sum is accumulated in fp32 in ascending r.
+ *
+ * quantized_data = NF4 codes of the [N,K] weight (block_size 64); block_scalers fp32 [N*K/64] from
+ * ttamd_nf4_block_scalers; lora_a [rank,K] bf16; lora_b [N,rank] bf16; scale = alpha / rank; out [N,K] bf16.
+ * Requires K % 64 == 0, rank a multiple of 8 in [8,64].
+ */
+int ttamd_nf4_dequantize_merge_bf16(const uint8_t* quantized_data, const void* block_scalers, const void* lora_a,
+                                    const void* lora_b, int rank, float scale, void* out, int64_t N, int64_t K,
+                                    void* stream);
+
+/*
  * h = bf16(x . lora_a^T): the adapter's hidden activation `self.lora_a(self.dropout(x))` (lora.py:144).
  * x [M,K] bf16, lora_a [rank,K] bf16, h out [M,rank] bf16; rank a multiple of 8 in [8,64], K % 64 == 0.
  * workspace: ttamd_lora_fwd_workspace_bytes(M, K, rank) bytes.

@@ -60,3 +60,12 @@ def fixed_init_tensor(shape, dtype=torch.float32) -> torch.Tensor:
     (``tests/test_utils.py:206-225``)."""
     n = math.prod(shape)
     return torch.arange(0.0, 1.0, 1.0 / n, dtype=dtype).reshape(shape)
+
+
+def merged_weight(parts: "nf4_oracle.NF4Parts", lora_a: torch.Tensor, lora_b: torch.Tensor, alpha: float, rank: int) -> torch.Tensor:
+    """Checkpoint weight of a QLoRA linear: the state-dict hook's ``NF4Tensor.to(dtype)``
+    (``torchtune/modules/common_utils.py:55-59``) followed by ``weight += (alpha / rank) * lora_b @ lora_a``
+    (``torchtune/modules/peft/_utils.py:264-266``), eager ops in the weight dtype."""
+    w = nf4_oracle.nf4_dequantize(parts).clone()
+    w += (alpha / rank) * lora_b @ lora_a
+    return w

@@ -293,3 +293,28 @@ def test_package_exports():
                  "Int8DynActInt4WeightQATQuantizer", "FakeQuantizeConfig", "FakeQuantizer", "FakeQuantizedLinear"):
         assert hasattr(torchtune_amd, name)
     assert FrozenNF4Linear.__mro__[1] is nn.Linear
+
+
+def test_reference_known_answer_merged_lora_ckpt():
+    """The 6x4 merged weight the reference's own test holds (tests/torchtune/modules/peft/test_utils.py:451-480),
+    through get_merged_lora_ckpt on dense CPU tensors; the adapter entries are deleted and the dict is returned."""
+    import json
+    import os
+
+    from torchtune_amd.modules.peft import get_merged_lora_ckpt
+
+    with open(os.path.join(os.path.dirname(__file__), "golden", "reference_known_answers.json")) as f:
+        kat = json.load(f)["merged_lora_ckpt"]
+    sd = {
+        "0.weight": 3 * torch.ones(6, 4),
+        "0.lora_a.weight": torch.tensor(kat["lora_a"], dtype=torch.float32),
+        "0.lora_b.weight": torch.tensor(kat["lora_b"], dtype=torch.float32),
+        "1.weight": torch.zeros(3, 6),
+        "1.bias": torch.zeros(3),
+    }
+    out = get_merged_lora_ckpt(sd, rank=kat["rank"], alpha=kat["alpha"])
+    assert out is sd and out.keys() == {"0.weight", "1.weight", "1.bias"}
+    torch.testing.assert_close(out["0.weight"], torch.tensor(kat["expected_merged_weight"]), atol=kat["atol"], rtol=kat["rtol"])
+    with pytest.raises(NotImplementedError):
+        get_merged_lora_ckpt({"m.weight": torch.ones(2, 2), "m.lora_a.weight": torch.ones(1, 2), "m.lora_b.weight": torch.ones(2, 1),
+                              "m.magnitude": torch.ones(2)}, rank=1, alpha=1.0)

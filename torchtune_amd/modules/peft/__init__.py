@@ -1,4 +1,4 @@
-from ._utils import AdapterModule, get_adapter_params, set_trainable_params
+from ._utils import AdapterModule, get_adapter_params, get_merged_lora_ckpt, set_trainable_params
 from .lora import LoRALinear, QATLoRALinear, TrainableParams
 
 __all__ = [
@@ -7,5 +7,6 @@ __all__ = [
     "QATLoRALinear",
     "TrainableParams",
     "get_adapter_params",
+    "get_merged_lora_ckpt",
     "set_trainable_params",
 ]

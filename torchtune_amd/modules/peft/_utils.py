@@ -1,11 +1,15 @@
-"""The small part of the adapter bookkeeping that callers of ``LoRALinear`` need
-(``torchtune/modules/peft/_utils.py:19-83``): the ``AdapterModule`` protocol and the helpers that pick out and
-freeze parameters by it."""
+"""The part of the adapter bookkeeping that callers of ``LoRALinear`` need
+(``torchtune/modules/peft/_utils.py:19-83,193-271``): the ``AdapterModule`` protocol, the helpers that pick out
+and freeze parameters by it, and the merge of the adapters into the base weights for a checkpoint."""
 from __future__ import annotations
 
-from typing import Dict, List, Protocol
+from typing import Any, Dict, List, Protocol, Set
 
+import torch
 from torch import nn
+
+from ... import ops
+from ...nf4_tensor import NF4Tensor
 
 
 class AdapterModule(Protocol):
@@ -35,3 +39,41 @@ def set_trainable_params(model: nn.Module, adapter_params: Dict[str, nn.Paramete
     """Freeze everything except the given parameters."""
     for name, p in model.named_parameters():
         p.requires_grad_(name in adapter_params)
+
+
+def _get_lora_modules(state_dict: Dict[str, Any]) -> Set[str]:
+    """Module prefixes that own a ``lora_a.weight`` / ``lora_b.weight`` pair in ``state_dict``."""
+    return {k[: -len(".lora_a.weight")] for k in state_dict if k.endswith(".lora_a.weight")}
+
+
+@torch.no_grad()
+def get_merged_lora_ckpt(state_dict: Dict[str, Any], rank: int, alpha: float) -> Dict[str, Any]:
+    """Fold every LoRA pair of ``state_dict`` into its base weight, ``W += (alpha / rank) * B @ A``, and delete the
+    adapter entries; modifies and returns ``state_dict`` (``torchtune/modules/peft/_utils.py:193-271``, vanilla
+    LoRA branch; DoRA magnitudes and MoE experts raise).
+
+    A base weight that is still an ``NF4Tensor`` on the GPU (a state dict taken without the dequantising hook) is
+    dequantised and merged in one pass by the HIP kernel; a dense weight is updated in place as the reference does.
+    """
+    for module in sorted(_get_lora_modules(state_dict)):
+        if f"{module}.magnitude" in state_dict or "experts" in module:
+            raise NotImplementedError(f"{module}: merging DoRA magnitudes / MoE experts is not part of this build")
+        a = state_dict[f"{module}.lora_a.weight"]
+        b = state_dict[f"{module}.lora_b.weight"]
+        w = state_dict[f"{module}.weight"]
+        if (
+            isinstance(w, NF4Tensor) and w.is_cuda and w.block_size == 64 and w.dtype == torch.bfloat16
+            and a.dtype == torch.bfloat16 and b.dtype == torch.bfloat16 and a.shape[0] % 8 == 0 and 0 < a.shape[0] <= 64
+        ):
+            N, K = w.shape
+            state_dict[f"{module}.weight"] = ops.nf4_dequantize_merge(
+                w.quantized_data, w.block_scalers(), N, K, a.to(w.device), b.to(w.device), alpha / rank
+            )
+        else:
+            if isinstance(w, NF4Tensor):
+                w = w.to(a.dtype)
+                state_dict[f"{module}.weight"] = w
+            w += (alpha / rank) * b @ a
+        del state_dict[f"{module}.lora_a.weight"]
+        del state_dict[f"{module}.lora_b.weight"]
+    return state_dict

@@ -94,6 +94,24 @@ def nf4_dequantize(
     return out.view(shape)
 
 
+def nf4_dequantize_merge(qdata: torch.Tensor, block_scalers: torch.Tensor, N: int, K: int, lora_a: torch.Tensor,
+                         lora_b: torch.Tensor, scale: float) -> torch.Tensor:
+    """bf16(D(W) + bf16(scale * bf16(lora_b @ lora_a))) for an NF4 [N, K] weight (block size 64) in one pass."""
+    _need_gpu(qdata, "nf4_dequantize_merge")
+    a = _bf16_2d(lora_a, "nf4_dequantize_merge: lora_a")
+    b = _bf16_2d(lora_b, "nf4_dequantize_merge: lora_b")
+    rank = a.shape[0]
+    if a.shape != (rank, K) or b.shape != (N, rank):
+        raise ValueError(f"nf4_dequantize_merge: lora_a {tuple(a.shape)} / lora_b {tuple(b.shape)} do not fit [{N}, {K}]")
+    out = torch.empty(N, K, dtype=torch.bfloat16, device=qdata.device)
+    lib = _lib.load()
+    with torch.cuda.device(qdata.device):
+        rc = lib.ttamd_nf4_dequantize_merge_bf16(qdata.data_ptr(), block_scalers.data_ptr(), a.data_ptr(), b.data_ptr(), rank,
+                                                 float(scale), out.data_ptr(), N, K, _stream(qdata))
+    _lib.check(rc, "nf4_dequantize_merge")
+    return out
+
+
 def nf4_block_scalers(qscalers: torch.Tensor, qfactor: torch.Tensor, mean: torch.Tensor, scaler_block_size: int) -> torch.Tensor:
     _need_gpu(qscalers, "nf4_block_scalers")
     code = _code(qfactor.dtype, "nf4_block_scalers")
