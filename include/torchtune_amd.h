@@ -212,6 +212,45 @@ int ttamd_fq_per_group_int4_sym(const void* w, int dtype, int64_t rows, int64_t 
 int ttamd_quantize_per_group_int4(const void* w, int dtype, int64_t rows, int64_t K, int group_size, int8_t* q,
                                   float* scale, float* zero_point, void* stream);
 
+/* ------------------------------------------------------------------------------------------------
+ * Neighbours of the quantized linears inside a decoder layer (one pass over HBM each, bf16 tensors, fp32 math).
+ * Floating-point kernels: results agree with the eager sequences to a tolerance (summation order and hardware
+ * exp / rsqrt differ), not bit for bit.
+ * ---------------------------------------------------------------------------------------------- */
+
+/*
+ * RMSNorm.forward (torchtune/modules/rms_norm.py:28-41): y = bf16( bf16(x * rsqrt(mean(x^2) + eps)) * scale ).
+ * x, y [rows, D] bf16; scale [D] bf16; rstd out [rows] fp32 (kept for the backward; may be NULL).
+ * D a multiple of 8, at most 8192.
+ */
+int ttamd_rms_norm_fwd_bf16(const void* x, const void* scale, float eps, void* y, float* rstd, int64_t rows, int64_t D,
+                            void* stream);
+
+/*
+ * Backward of the above: gx [rows, D] bf16, and (if gscale is not NULL) gscale [D] bf16 = sum over rows of
+ * gy * bf16(x * rstd), summed in a fixed order.  workspace (only read when gscale is given):
+ * ttamd_rms_norm_bwd_workspace_bytes(D) bytes.
+ */
+size_t ttamd_rms_norm_bwd_workspace_bytes(int64_t D);
+int ttamd_rms_norm_bwd_bf16(const void* gy, const void* x, const void* scale, const float* rstd, void* gx, void* gscale,
+                            int64_t rows, int64_t D, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Rotary position embedding (torchtune/models/llama3_1/_position_embeddings.py:128-190, positions 0..S-1):
+ * x, y [B, S, n_heads, head_dim] bf16; cache [S, head_dim/2, 2] fp32 (cos, sin); consecutive pairs are rotated in
+ * fp32.  inverse != 0 rotates by the negative angle, which is the backward pass.  head_dim a multiple of 8.
+ */
+int ttamd_rope_bf16(const void* x, const float* cache, void* y, int64_t B, int64_t S, int64_t n_heads, int64_t head_dim,
+                    int inverse, void* stream);
+
+/*
+ * FeedForward gate (torchtune/modules/feed_forward.py:50-53): out = bf16( bf16(silu(gate)) * up ), and its backward
+ * ggate, gup from gout.  All [numel] bf16, numel a multiple of 8.
+ */
+int ttamd_swiglu_fwd_bf16(const void* gate, const void* up, void* out, int64_t numel, void* stream);
+int ttamd_swiglu_bwd_bf16(const void* gout, const void* gate, const void* up, void* ggate, void* gup, int64_t numel,
+                          void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,110 @@
+"""GPU parity of the single-pass RMSNorm / rotary / SwiGLU kernels (forward and backward, through autograd and through the
+C ABI) against the eager CPU oracle.  Floating-point kernels: bf16 results within rtol 1e-2 / atol 1e-2 of the oracle
+(both sides compute in fp32 and round to bf16 at the same points; summation order and exp / rsqrt differ), and for the
+element-wise ones at most one bf16 ulp apart."""
+import pytest
+import torch
+
+from oracle import layer_oracle as lo
+from torchtune_amd import _lib, ops
+from torchtune_amd.modules import layer_ops
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+BF = torch.bfloat16
+
+
+def _close(got, want, rtol=1e-2, atol=1e-2):
+    torch.testing.assert_close(got.float().cpu(), want.float(), rtol=rtol, atol=atol)
+
+
+def _within_ulps(got, want, n):
+    w = want.float()
+    ulp = torch.maximum(w.abs(), torch.tensor(2.0 ** -120)) * 2.0 ** -7
+    assert torch.all((got.float().cpu() - w).abs() <= n * ulp)
+
+
+@pytest.mark.parametrize("rows,D", [(5, 64), (33, 2048), (64, 4096), (9, 8192), (7, 4104)])
+def test_rms_norm_forward_backward(rows, D):
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(rows, D, generator=g).to(BF).requires_grad_()
+    w = (torch.rand(D, generator=g) + 0.5).to(BF).requires_grad_()
+    gy = torch.randn(rows, D, generator=g).to(BF)
+    want = lo.rms_norm(x, w, 1e-5)
+    want.backward(gy)
+    m = layer_ops.RMSNorm(D, 1e-5).to(DEV, BF)
+    with torch.no_grad():
+        m.scale.copy_(w)
+    xd = x.detach().to(DEV).requires_grad_()
+    got = m(xd)
+    got.backward(gy.to(DEV))
+    _within_ulps(got, want, 2)
+    _close(xd.grad, x.grad)
+    _close(m.scale.grad, w.grad, rtol=2e-2, atol=2e-2 * float(w.grad.float().abs().max()))
+    # frozen scale: no scale gradient is computed, the input gradient is unchanged
+    m.scale.requires_grad_(False)
+    xd2 = x.detach().to(DEV).requires_grad_()
+    m(xd2).backward(gy.to(DEV))
+    assert torch.equal(xd2.grad, xd.grad)
+
+
+def test_rms_norm_leading_dimensions_and_validation():
+    x = torch.randn(2, 3, 256, device=DEV).to(BF)
+    w = torch.ones(256, device=DEV, dtype=BF)
+    y, rstd = ops.rms_norm_fwd(x, w, 1e-6)
+    assert y.shape == x.shape and rstd.shape == (6,)
+    _close(y, lo.rms_norm(x.cpu(), w.cpu(), 1e-6))
+    lib = _lib.load()
+    assert lib.ttamd_rms_norm_fwd_bf16(x.data_ptr(), w.data_ptr(), 1e-6, y.data_ptr(), None, 6, 100, None) == -1
+    assert b"multiple of 8" in lib.ttamd_last_error()
+    with pytest.raises(RuntimeError, match="HIP kernels"):
+        ops.rms_norm_fwd(x.cpu(), w.cpu(), 1e-6)
+
+
+@pytest.mark.parametrize("b,s,nh,hd", [(1, 5, 1, 8), (2, 37, 4, 64), (2, 128, 8, 128)])
+def test_rope_forward_backward(b, s, nh, hd):
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(b, s, nh, hd, generator=g).to(BF).requires_grad_()
+    gy = torch.randn(b, s, nh, hd, generator=g).to(BF)
+    cache = lo.rope_cache(s + 3, hd, 500000.0)  # a longer table than the sequence: only the first s rows are used
+    want = lo.rope(x, cache)
+    want.backward(gy)
+    xd = x.detach().to(DEV).requires_grad_()
+    got = layer_ops.apply_rope(xd, cache.to(DEV))
+    got.backward(gy.to(DEV))
+    _within_ulps(got, want, 1)
+    _within_ulps(xd.grad, x.grad, 1)
+    assert torch.equal(got[:, 0].cpu(), x.detach()[:, 0])
+
+
+@pytest.mark.parametrize("shape", [(8,), (3, 40), (4, 128, 1024)])
+def test_swiglu_forward_backward(shape):
+    g = torch.Generator().manual_seed(2)
+    a = (torch.randn(shape, generator=g) * 3).to(BF).requires_grad_()
+    u = torch.randn(shape, generator=g).to(BF).requires_grad_()
+    go = torch.randn(shape, generator=g).to(BF)
+    want = lo.swiglu(a, u)
+    want.backward(go)
+    ad, ud = a.detach().to(DEV).requires_grad_(), u.detach().to(DEV).requires_grad_()
+    got = layer_ops.swiglu(ad, ud)
+    got.backward(go.to(DEV))
+    _within_ulps(got, want, 2)
+    _close(ad.grad, a.grad)
+    _close(ud.grad, u.grad)
+
+
+def test_full_size_properties_8b_activations():
+    """8192 x 4096 / 8192 x 14336: properties that hold at any size."""
+    g = torch.Generator(device=DEV).manual_seed(3)
+    x = torch.randn(8192, 4096, device=DEV, generator=g).to(BF)
+    y, rstd = ops.rms_norm_fwd(x, torch.ones(4096, device=DEV, dtype=BF), 0.0)
+    torch.testing.assert_close(y.float().pow(2).mean(-1), torch.ones(8192, device=DEV), rtol=1e-2, atol=1e-2)
+    torch.testing.assert_close(rstd, torch.rsqrt(x.float().pow(2).mean(-1)), rtol=1e-5, atol=1e-6)
+    q = torch.randn(4, 2048, 32, 128, device=DEV, generator=g).to(BF)
+    cache = lo.rope_cache(2048, 128, 500000.0).to(DEV)
+    r = ops.rope(q, cache)
+    torch.testing.assert_close(r.float().view(-1, 2).norm(dim=-1), q.float().view(-1, 2).norm(dim=-1), rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(ops.rope(r, cache, inverse=True).float(), q.float(), rtol=2e-2, atol=2e-2)
+    a = torch.randn(8192, 14336, device=DEV, generator=g).to(BF)
+    z = ops.swiglu_fwd(a, torch.ones_like(a))
+    torch.testing.assert_close(z.float(), torch.nn.functional.silu(a.float()), rtol=1e-2, atol=1e-2)

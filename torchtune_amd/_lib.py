@@ -61,6 +61,15 @@ SIGNATURES = {
         _int,
         [_c_void_p, _int, _i64, _i64, _int, _c_void_p, _c_void_p, _c_void_p, _c_void_p],
     ),
+    "ttamd_rms_norm_fwd_bf16": (_int, [_c_void_p, _c_void_p, _f32, _c_void_p, _c_void_p, _i64, _i64, _c_void_p]),
+    "ttamd_rms_norm_bwd_workspace_bytes": (_size, [_i64]),
+    "ttamd_rms_norm_bwd_bf16": (
+        _int,
+        [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _i64, _i64, _c_void_p, _size, _c_void_p],
+    ),
+    "ttamd_rope_bf16": (_int, [_c_void_p, _c_void_p, _c_void_p, _i64, _i64, _i64, _i64, _int, _c_void_p]),
+    "ttamd_swiglu_fwd_bf16": (_int, [_c_void_p, _c_void_p, _c_void_p, _i64, _c_void_p]),
+    "ttamd_swiglu_bwd_bf16": (_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _i64, _c_void_p]),
 }
 
 _lock = threading.Lock()

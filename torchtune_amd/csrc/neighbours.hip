@@ -1,0 +1,366 @@
+// The memory-bound neighbours of the quantized linears inside a decoder layer, one pass over HBM each:
+//
+//   RMSNorm in fp32        torchtune/modules/rms_norm.py:28-41
+//   rotary embedding       torchtune/models/llama3_1/_position_embeddings.py:128-190 (interleaved pairs, fp32 math)
+//   SwiGLU gate            torchtune/modules/feed_forward.py:50-53   silu(w1 x) * w3 x
+//
+// and their backward passes.  In the eager reference each is a chain of 5-10 elementwise / reduction kernels that
+// each read and write the whole activation; here a forward or backward is one kernel that touches every tensor once.
+// Rounding points follow the eager sequence (a bf16 rounding wherever eager materialises a bf16 tensor); sums and
+// transcendental functions are fp32 but not bit-identical to eager's (different summation order, hardware exp / rsqrt),
+// so these kernels are checked to a tolerance, not bit for bit.
+#include "common.h"
+#include "nf4_math.h"
+
+namespace ttamd {
+namespace {
+
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+  bf16x2_t v;
+  v.x = (__bf16)lo;
+  v.y = (__bf16)hi;
+  return __builtin_bit_cast(uint32_t, v);
+}
+__device__ __forceinline__ float lo_f(uint32_t d) { return bits_f32(d << 16); }
+__device__ __forceinline__ float hi_f(uint32_t d) { return bits_f32(d & 0xffff0000u); }
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = 1; off < kWave; off <<= 1) v += __shfl_xor(v, off, kWave);
+  return v;
+}
+
+// ---------------------------------------------------------------------------------------------------
+// RMSNorm.  One wave per row, the row held in registers (NV 16-byte chunks per lane, chunk = lane + 64 i).
+//   forward : xn = bf16(x * rsqrt(mean(x^2) + eps));  y = bf16(xn * scale);  rstd saved for backward
+//   backward: g = bf16(gy * scale) (eager's bf16 product), c = mean(g * x) * rstd^2,
+//             gx = bf16(rstd * (g - x * c));  gscale partial[w][d] = sum over the wave's rows of gy * xn
+// ---------------------------------------------------------------------------------------------------
+template <int NV>
+__global__ __launch_bounds__(256) void rms_norm_fwd_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ scale,
+                                                           float eps, uint16_t* __restrict__ y, float* __restrict__ rstd_out,
+                                                           int64_t rows, int D) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int chunks = D >> 3;
+  const u32x4_t* xr = reinterpret_cast<const u32x4_t*>(x + row * D);
+  u32x4_t v[NV];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = lane + 64 * i;
+    v[i] = u32x4_t{0, 0, 0, 0};
+    if (c < chunks) v[i] = __builtin_nontemporal_load(xr + c);
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      const float a = lo_f(v[i][d]), b = hi_f(v[i][d]);
+      ss += a * a;
+      ss += b * b;
+    }
+  }
+  ss = wave_sum(ss);
+  const float rstd = __builtin_amdgcn_rsqf(ss / (float)D + eps);
+  if (lane == 0 && rstd_out) rstd_out[row] = rstd;
+  u32x4_t* yr = reinterpret_cast<u32x4_t*>(y + row * D);
+  const u32x4_t* sr = reinterpret_cast<const u32x4_t*>(scale);
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = lane + 64 * i;
+    if (c >= chunks) continue;
+    const u32x4_t s = sr[c];
+    u32x4_t o;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      const float n0 = round_to_bf16(lo_f(v[i][d]) * rstd), n1 = round_to_bf16(hi_f(v[i][d]) * rstd);
+      o[d] = pack2(n0 * lo_f(s[d]), n1 * hi_f(s[d]));
+    }
+    __builtin_nontemporal_store(o, yr + c);
+  }
+}
+
+template <int NV, bool GSCALE>
+__global__ __launch_bounds__(256) void rms_norm_bwd_kernel(const uint16_t* __restrict__ gy, const uint16_t* __restrict__ x,
+                                                           const uint16_t* __restrict__ scale, const float* __restrict__ rstd_in,
+                                                           uint16_t* __restrict__ gx, float* __restrict__ gscale_part,
+                                                           int64_t rows, int D) {
+  const int lane = threadIdx.x & 63;
+  const int wave_global = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int n_waves = gridDim.x * 4;
+  const int chunks = D >> 3;
+  const u32x4_t* sr = reinterpret_cast<const u32x4_t*>(scale);
+  float gs[GSCALE ? NV : 1][8];
+  if constexpr (GSCALE) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) gs[i][e] = 0.f;
+  }
+  for (int64_t row = wave_global; row < rows; row += n_waves) {
+    const u32x4_t* xr = reinterpret_cast<const u32x4_t*>(x + row * D);
+    const u32x4_t* gr = reinterpret_cast<const u32x4_t*>(gy + row * D);
+    const float rstd = rstd_in[row];
+    u32x4_t xv[NV], gv[NV];
+    float dot = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int c = lane + 64 * i;
+      xv[i] = u32x4_t{0, 0, 0, 0};
+      gv[i] = u32x4_t{0, 0, 0, 0};
+      if (c < chunks) {
+        xv[i] = __builtin_nontemporal_load(xr + c);
+        const u32x4_t go = __builtin_nontemporal_load(gr + c);
+        const u32x4_t s = sr[c];
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+          if constexpr (GSCALE) {
+            gs[i][2 * d] += lo_f(go[d]) * round_to_bf16(lo_f(xv[i][d]) * rstd);
+            gs[i][2 * d + 1] += hi_f(go[d]) * round_to_bf16(hi_f(xv[i][d]) * rstd);
+          }
+          gv[i][d] = pack2(lo_f(go[d]) * lo_f(s[d]), hi_f(go[d]) * hi_f(s[d]));  // g = bf16(gy * scale)
+          dot += lo_f(gv[i][d]) * lo_f(xv[i][d]);
+          dot += hi_f(gv[i][d]) * hi_f(xv[i][d]);
+        }
+      }
+    }
+    dot = wave_sum(dot);
+    const float c2 = dot / (float)D * rstd * rstd;
+    u32x4_t* outr = reinterpret_cast<u32x4_t*>(gx + row * D);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int c = lane + 64 * i;
+      if (c >= chunks) continue;
+      u32x4_t o;
+#pragma unroll
+      for (int d = 0; d < 4; ++d)
+        o[d] = pack2(rstd * (lo_f(gv[i][d]) - lo_f(xv[i][d]) * c2), rstd * (hi_f(gv[i][d]) - hi_f(xv[i][d]) * c2));
+      __builtin_nontemporal_store(o, outr + c);
+    }
+  }
+  if constexpr (GSCALE) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int c = lane + 64 * i;
+      if (c >= chunks) continue;
+      float* p = gscale_part + (int64_t)wave_global * D + 8 * c;
+      *reinterpret_cast<f32x4_t*>(p) = f32x4_t{gs[i][0], gs[i][1], gs[i][2], gs[i][3]};
+      *reinterpret_cast<f32x4_t*>(p + 4) = f32x4_t{gs[i][4], gs[i][5], gs[i][6], gs[i][7]};
+    }
+  }
+}
+
+// gscale[d] = bf16(sum_w part[w][d]), fixed order
+__global__ __launch_bounds__(256) void rms_norm_gscale_kernel(const float* __restrict__ part, int n_waves, int D,
+                                                              uint16_t* __restrict__ gscale) {
+  const int d = blockIdx.x * 256 + threadIdx.x;
+  if (d >= D) return;
+  float s = 0.f;
+#pragma unroll 8
+  for (int w = 0; w < n_waves; ++w) s += part[(int64_t)w * D + d];
+  gscale[d] = f32_to_bf16_bits(s);
+}
+
+constexpr int kRmsBwdWgs = 256;  // persistent workgroups of the backward: 1024 waves, one partial gscale row each
+
+// ---------------------------------------------------------------------------------------------------
+// Rotary embedding on [b, s, n_h, h_d] with a [s, h_d/2, 2] fp32 (cos, sin) table; `inverse` rotates by -theta,
+// which is the backward pass (the map is orthogonal).  One lane = 8 elements = 4 pairs.
+// ---------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void rope_kernel(const uint16_t* __restrict__ x, const float* __restrict__ cache,
+                                                   uint16_t* __restrict__ y, int64_t n_chunks, int S, int row_elems, int h_d,
+                                                   int inverse) {
+  const int64_t chunk = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (chunk >= n_chunks) return;
+  const int64_t e = chunk * 8;
+  const int pos = (int)((e / row_elems) % S);
+  const int d = (int)(e % h_d);  // even; h_d % 8 == 0 keeps the 4 pairs inside one head
+  const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(x) + chunk);
+  const f32x4_t* cp = reinterpret_cast<const f32x4_t*>(cache + ((int64_t)pos * (h_d >> 1) + (d >> 1)) * 2);
+  const f32x4_t c01 = cp[0], c23 = cp[1];
+  const float cs[4] = {c01.x, c01.z, c23.x, c23.z};
+  float sn[4] = {c01.y, c01.w, c23.y, c23.w};
+  u32x4_t o;
+#pragma unroll
+  for (int p = 0; p < 4; ++p) {
+    const float a = lo_f(v[p]), b = hi_f(v[p]);
+    const float s = inverse ? -sn[p] : sn[p];
+    o[p] = pack2(a * cs[p] - b * s, b * cs[p] + a * s);
+  }
+  __builtin_nontemporal_store(o, reinterpret_cast<u32x4_t*>(y) + chunk);
+}
+
+// ---------------------------------------------------------------------------------------------------
+// SwiGLU gate.  forward: a = bf16(silu(g)); out = bf16(a * u).
+// backward: gu = bf16(go * a); ga = bf16(go * u); gg = bf16(ga * silu'(g)), silu'(g) = s (1 + g (1 - s)), s = sigmoid(g).
+// ---------------------------------------------------------------------------------------------------
+__device__ __forceinline__ float sigmoid_f(float g) {
+  return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * g));
+}
+
+__global__ __launch_bounds__(256) void swiglu_fwd_kernel(const uint16_t* __restrict__ g, const uint16_t* __restrict__ u,
+                                                         uint16_t* __restrict__ out, int64_t n_chunks) {
+  const int64_t chunk = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (chunk >= n_chunks) return;
+  const u32x4_t gv = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(g) + chunk);
+  const u32x4_t uv = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(u) + chunk);
+  u32x4_t o;
+#pragma unroll
+  for (int d = 0; d < 4; ++d) {
+    const float g0 = lo_f(gv[d]), g1 = hi_f(gv[d]);
+    const float a0 = round_to_bf16(g0 * sigmoid_f(g0)), a1 = round_to_bf16(g1 * sigmoid_f(g1));
+    o[d] = pack2(a0 * lo_f(uv[d]), a1 * hi_f(uv[d]));
+  }
+  __builtin_nontemporal_store(o, reinterpret_cast<u32x4_t*>(out) + chunk);
+}
+
+__global__ __launch_bounds__(256) void swiglu_bwd_kernel(const uint16_t* __restrict__ go, const uint16_t* __restrict__ g,
+                                                         const uint16_t* __restrict__ u, uint16_t* __restrict__ gg,
+                                                         uint16_t* __restrict__ gu, int64_t n_chunks) {
+  const int64_t chunk = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (chunk >= n_chunks) return;
+  const u32x4_t ov = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(go) + chunk);
+  const u32x4_t gv = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(g) + chunk);
+  const u32x4_t uv = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(u) + chunk);
+  u32x4_t og, ou;
+#pragma unroll
+  for (int d = 0; d < 4; ++d) {
+    float rg[2], ru[2];
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+      const float gval = e ? hi_f(gv[d]) : lo_f(gv[d]);
+      const float uval = e ? hi_f(uv[d]) : lo_f(uv[d]);
+      const float oval = e ? hi_f(ov[d]) : lo_f(ov[d]);
+      const float s = sigmoid_f(gval);
+      const float a = round_to_bf16(gval * s);
+      ru[e] = oval * a;
+      const float ga = round_to_bf16(oval * uval);
+      rg[e] = ga * (s * (1.0f + gval * (1.0f - s)));
+    }
+    og[d] = pack2(rg[0], rg[1]);
+    ou[d] = pack2(ru[0], ru[1]);
+  }
+  __builtin_nontemporal_store(og, reinterpret_cast<u32x4_t*>(gg) + chunk);
+  __builtin_nontemporal_store(ou, reinterpret_cast<u32x4_t*>(gu) + chunk);
+}
+
+int nv_for(int64_t D) {
+  const int64_t chunks = D / 8;
+  int nv = 1;
+  while ((int64_t)nv * 64 < chunks) nv <<= 1;
+  return nv;
+}
+
+}  // namespace
+}  // namespace ttamd
+
+using namespace ttamd;
+
+extern "C" int ttamd_rms_norm_fwd_bf16(const void* x, const void* scale, float eps, void* y, float* rstd, int64_t rows,
+                                       int64_t D, void* stream) {
+  TT_REQUIRE(x && scale && y, "rms_norm_fwd: null pointer argument");
+  TT_REQUIRE(aligned16(x) && aligned16(scale) && aligned16(y), "rms_norm_fwd: pointers must be 16-byte aligned");
+  TT_REQUIRE(rows > 0 && D > 0 && D % 8 == 0 && D <= 8192 && rows < (int64_t(1) << 32),
+             "rms_norm_fwd: bad shape rows=%lld D=%lld (D must be a multiple of 8, at most 8192)", (long long)rows, (long long)D);
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
+  const uint16_t* X = reinterpret_cast<const uint16_t*>(x);
+  const uint16_t* S = reinterpret_cast<const uint16_t*>(scale);
+  uint16_t* Y = reinterpret_cast<uint16_t*>(y);
+  switch (nv_for(D)) {
+    case 1: rms_norm_fwd_kernel<1><<<grid, block, 0, s>>>(X, S, eps, Y, rstd, rows, (int)D); break;
+    case 2: rms_norm_fwd_kernel<2><<<grid, block, 0, s>>>(X, S, eps, Y, rstd, rows, (int)D); break;
+    case 4: rms_norm_fwd_kernel<4><<<grid, block, 0, s>>>(X, S, eps, Y, rstd, rows, (int)D); break;
+    case 8: rms_norm_fwd_kernel<8><<<grid, block, 0, s>>>(X, S, eps, Y, rstd, rows, (int)D); break;
+    default: rms_norm_fwd_kernel<16><<<grid, block, 0, s>>>(X, S, eps, Y, rstd, rows, (int)D); break;
+  }
+  return check_launch("rms_norm_fwd");
+}
+
+extern "C" size_t ttamd_rms_norm_bwd_workspace_bytes(int64_t D) {
+  return D > 0 ? (size_t)kRmsBwdWgs * 4 * (size_t)D * sizeof(float) : 0;
+}
+
+extern "C" int ttamd_rms_norm_bwd_bf16(const void* gy, const void* x, const void* scale, const float* rstd, void* gx,
+                                       void* gscale, int64_t rows, int64_t D, void* workspace, size_t workspace_bytes,
+                                       void* stream) {
+  TT_REQUIRE(gy && x && scale && rstd && gx, "rms_norm_bwd: null pointer argument");
+  TT_REQUIRE(aligned16(gy) && aligned16(x) && aligned16(scale) && aligned16(gx), "rms_norm_bwd: pointers must be 16-byte aligned");
+  TT_REQUIRE(rows > 0 && D > 0 && D % 8 == 0 && D <= 8192 && rows < (int64_t(1) << 32),
+             "rms_norm_bwd: bad shape rows=%lld D=%lld (D must be a multiple of 8, at most 8192)", (long long)rows, (long long)D);
+  if (gscale) {
+    TT_REQUIRE(workspace && aligned16(workspace), "rms_norm_bwd: the scale gradient needs a 16-byte aligned workspace");
+    if (workspace_bytes < ttamd_rms_norm_bwd_workspace_bytes(D))
+      return fail(TTAMD_EWORKSPACE, "rms_norm_bwd: workspace has %zu bytes, needs %zu", workspace_bytes,
+                  ttamd_rms_norm_bwd_workspace_bytes(D));
+  }
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  // without a scale gradient: one wave per row; with it: a fixed number of persistent waves, each of which writes one
+  // row of partial sums (zeros if it had no row)
+  const int64_t wgs = gscale ? kRmsBwdWgs : (rows + 3) / 4;
+  const dim3 grid((unsigned)wgs), block(256);
+  const uint16_t* G = reinterpret_cast<const uint16_t*>(gy);
+  const uint16_t* X = reinterpret_cast<const uint16_t*>(x);
+  const uint16_t* S = reinterpret_cast<const uint16_t*>(scale);
+  uint16_t* GX = reinterpret_cast<uint16_t*>(gx);
+  float* part = reinterpret_cast<float*>(workspace);
+#define TT_RMS_BWD(NVV)                                                                                          \
+  if (gscale)                                                                                                    \
+    rms_norm_bwd_kernel<NVV, true><<<grid, block, 0, s>>>(G, X, S, rstd, GX, part, rows, (int)D);                \
+  else                                                                                                           \
+    rms_norm_bwd_kernel<NVV, false><<<grid, block, 0, s>>>(G, X, S, rstd, GX, nullptr, rows, (int)D);
+  switch (nv_for(D)) {
+    case 1: TT_RMS_BWD(1) break;
+    case 2: TT_RMS_BWD(2) break;
+    case 4: TT_RMS_BWD(4) break;
+    case 8: TT_RMS_BWD(8) break;
+    default: TT_RMS_BWD(16) break;
+  }
+#undef TT_RMS_BWD
+  if (gscale)
+    rms_norm_gscale_kernel<<<dim3((unsigned)((D + 255) / 256)), block, 0, s>>>(part, kRmsBwdWgs * 4, (int)D,
+                                                                               reinterpret_cast<uint16_t*>(gscale));
+  return check_launch("rms_norm_bwd");
+}
+
+extern "C" int ttamd_rope_bf16(const void* x, const float* cache, void* y, int64_t B, int64_t S, int64_t n_heads,
+                               int64_t head_dim, int inverse, void* stream) {
+  TT_REQUIRE(x && cache && y, "rope: null pointer argument");
+  TT_REQUIRE(aligned16(x) && aligned16(cache) && aligned16(y), "rope: pointers must be 16-byte aligned");
+  TT_REQUIRE(B > 0 && S > 0 && n_heads > 0 && head_dim > 0 && head_dim % 8 == 0 && S < (1 << 30) && n_heads * head_dim < (1 << 30),
+             "rope: bad shape b=%lld s=%lld n_h=%lld h_d=%lld (h_d must be a multiple of 8)", (long long)B, (long long)S,
+             (long long)n_heads, (long long)head_dim);
+  const int64_t n_chunks = B * S * n_heads * head_dim / 8;
+  TT_REQUIRE((n_chunks + 255) / 256 < (int64_t(1) << 31), "rope: tensor too large for one launch");
+  rope_kernel<<<dim3((unsigned)((n_chunks + 255) / 256)), dim3(256), 0, reinterpret_cast<hipStream_t>(stream)>>>(
+      reinterpret_cast<const uint16_t*>(x), cache, reinterpret_cast<uint16_t*>(y), n_chunks, (int)S, (int)(n_heads * head_dim),
+      (int)head_dim, inverse);
+  return check_launch("rope");
+}
+
+extern "C" int ttamd_swiglu_fwd_bf16(const void* gate, const void* up, void* out, int64_t numel, void* stream) {
+  TT_REQUIRE(gate && up && out, "swiglu_fwd: null pointer argument");
+  TT_REQUIRE(aligned16(gate) && aligned16(up) && aligned16(out), "swiglu_fwd: pointers must be 16-byte aligned");
+  TT_REQUIRE(numel > 0 && numel % 8 == 0 && (numel / 8 + 255) / 256 < (int64_t(1) << 31), "swiglu_fwd: numel (%lld) must be a positive multiple of 8",
+             (long long)numel);
+  const int64_t n_chunks = numel / 8;
+  swiglu_fwd_kernel<<<dim3((unsigned)((n_chunks + 255) / 256)), dim3(256), 0, reinterpret_cast<hipStream_t>(stream)>>>(
+      reinterpret_cast<const uint16_t*>(gate), reinterpret_cast<const uint16_t*>(up), reinterpret_cast<uint16_t*>(out), n_chunks);
+  return check_launch("swiglu_fwd");
+}
+
+extern "C" int ttamd_swiglu_bwd_bf16(const void* gout, const void* gate, const void* up, void* ggate, void* gup, int64_t numel,
+                                     void* stream) {
+  TT_REQUIRE(gout && gate && up && ggate && gup, "swiglu_bwd: null pointer argument");
+  TT_REQUIRE(aligned16(gout) && aligned16(gate) && aligned16(up) && aligned16(ggate) && aligned16(gup),
+             "swiglu_bwd: pointers must be 16-byte aligned");
+  TT_REQUIRE(numel > 0 && numel % 8 == 0 && (numel / 8 + 255) / 256 < (int64_t(1) << 31), "swiglu_bwd: numel (%lld) must be a positive multiple of 8",
+             (long long)numel);
+  const int64_t n_chunks = numel / 8;
+  swiglu_bwd_kernel<<<dim3((unsigned)((n_chunks + 255) / 256)), dim3(256), 0, reinterpret_cast<hipStream_t>(stream)>>>(
+      reinterpret_cast<const uint16_t*>(gout), reinterpret_cast<const uint16_t*>(gate), reinterpret_cast<const uint16_t*>(up),
+      reinterpret_cast<uint16_t*>(ggate), reinterpret_cast<uint16_t*>(gup), n_chunks);
+  return check_launch("swiglu_bwd");
+}

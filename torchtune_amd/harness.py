@@ -26,6 +26,7 @@ import torch.nn.functional as F
 from torch import nn
 from torch.utils.checkpoint import checkpoint
 
+from .modules import layer_ops
 from .modules.peft import LoRALinear, get_adapter_params, set_trainable_params
 from .qat import Int8DynActInt4WeightQATQuantizer
 
@@ -56,6 +57,15 @@ SHAPES = {
 }
 
 
+# True: RMSNorm, RoPE and the SwiGLU gate run as single-pass HIP kernels (bf16 on the GPU); False: the eager op chains
+# of the reference.  The quantized linears are unaffected.
+FUSED_LAYER_OPS = True
+
+
+def _fused(x: torch.Tensor) -> bool:
+    return FUSED_LAYER_OPS and x.is_cuda and x.dtype == torch.bfloat16
+
+
 class RMSNorm(nn.Module):
     """fp32 RMS normalisation (``torchtune/modules/rms_norm.py:28-41``)."""
 
@@ -65,9 +75,11 @@ class RMSNorm(nn.Module):
         self.scale = nn.Parameter(torch.ones(dim))
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
+        if _fused(x) and self.scale.dtype == torch.bfloat16 and x.shape[-1] % 8 == 0 and x.shape[-1] <= 8192:
+            return layer_ops._RMSNormFn.apply(x, self.scale, self.eps)
         xf = x.float()
-        xf = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + self.eps)
-        return (xf * self.scale.float()).to(x.dtype)
+        x_normed = (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + self.eps)).type_as(x)
+        return x_normed * self.scale
 
 
 def rope_cache(seq_len: int, head_dim: int, base: float, device) -> torch.Tensor:
@@ -79,6 +91,8 @@ def rope_cache(seq_len: int, head_dim: int, base: float, device) -> torch.Tensor
 
 def apply_rope(x: torch.Tensor, cache: torch.Tensor) -> torch.Tensor:
     """x [b, s, n_h, h_d]; rotates interleaved pairs, fp32 math."""
+    if _fused(x) and x.shape[-1] % 8 == 0:
+        return layer_ops.apply_rope(x, cache)
     xs = x.float().reshape(*x.shape[:-1], -1, 2)
     c = cache.view(1, xs.size(1), 1, xs.size(3), 2)
     out = torch.stack(
@@ -125,7 +139,8 @@ class FeedForward(nn.Module):
         self.w3 = _linear(s.dim, s.hidden, rank, alpha, quantize_base)  # up
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        return self.w2(F.silu(self.w1(x)) * self.w3(x))
+        g, u = self.w1(x), self.w3(x)
+        return self.w2(layer_ops.swiglu(g, u) if _fused(g) else F.silu(g) * u)
 
 
 class DecoderLayer(nn.Module):

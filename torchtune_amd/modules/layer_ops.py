@@ -1,0 +1,81 @@
+"""RMSNorm, rotary embedding and the SwiGLU gate as single-pass HIP kernels with autograd.
+
+These are the memory-bound neighbours of the quantized linears inside a decoder layer.  The reference runs each as
+a chain of eager kernels: ``RMSNorm`` (``torchtune/modules/rms_norm.py:11-41``), ``Llama3ScaledRoPE.forward``
+(``torchtune/models/llama3_1/_position_embeddings.py:128-190``), ``FeedForward.forward``
+(``torchtune/modules/feed_forward.py:50-53``).  Same arguments and results (to floating-point tolerance); bf16
+tensors on the GPU only, anything else raises.
+"""
+from __future__ import annotations
+
+import torch
+from torch import nn
+
+from .. import ops
+
+
+class _RMSNormFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, scale, eps: float):
+        y, rstd = ops.rms_norm_fwd(x, scale, eps)
+        ctx.save_for_backward(x, scale, rstd)
+        return y.view(x.shape)
+
+    @staticmethod
+    def backward(ctx, gy):
+        x, scale, rstd = ctx.saved_tensors
+        gx, gscale = ops.rms_norm_bwd(gy, x, scale, rstd, want_gscale=ctx.needs_input_grad[1])
+        return (gx.view(x.shape) if ctx.needs_input_grad[0] else None), gscale, None
+
+
+class RMSNorm(nn.Module):
+    """Root-mean-square normalisation computed in fp32: ``bf16(x * rsqrt(mean(x^2) + eps)) * scale``.
+
+    Args:
+        dim (int): embedding size
+        eps (float): added to the mean square. Default: 1e-6
+    """
+
+    def __init__(self, dim: int, eps: float = 1e-6) -> None:
+        super().__init__()
+        self.normalized_shape = (dim,)
+        self.eps = eps
+        self.scale = nn.Parameter(torch.ones(dim))
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return _RMSNormFn.apply(x, self.scale, self.eps)
+
+
+class _RopeFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, cache):
+        ctx.save_for_backward(cache)
+        return ops.rope(x, cache, inverse=False)
+
+    @staticmethod
+    def backward(ctx, gy):
+        (cache,) = ctx.saved_tensors
+        return ops.rope(gy, cache, inverse=True), None
+
+
+def apply_rope(x: torch.Tensor, cache: torch.Tensor) -> torch.Tensor:
+    """Rotate consecutive pairs of ``x [b, s, n_h, h_d]`` by the angles in ``cache [s, h_d/2, 2]`` (cos, sin), fp32 math."""
+    return _RopeFn.apply(x, cache)
+
+
+class _SwiGLUFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, gate, up):
+        ctx.save_for_backward(gate, up)
+        return ops.swiglu_fwd(gate, up)
+
+    @staticmethod
+    def backward(ctx, gout):
+        gate, up = ctx.saved_tensors
+        gg, gu = ops.swiglu_bwd(gout, gate, up)
+        return gg, gu
+
+
+def swiglu(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    """``silu(gate) * up`` with the eager sequence's two bf16 roundings."""
+    return _SwiGLUFn.apply(gate, up)

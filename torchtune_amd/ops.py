@@ -341,3 +341,91 @@ def quantize_per_group_int4(w: torch.Tensor, group_size: int):
                                                zeros.data_ptr(), _stream(w))
     _lib.check(rc, "quantize_per_group_int4")
     return q, scale, zeros
+
+
+# ---------------------------------------------------------------------------------------------------
+# neighbours of the quantized linears in a decoder layer: RMSNorm, rotary embedding, SwiGLU gate
+# ---------------------------------------------------------------------------------------------------
+def _bf16_any(t: torch.Tensor, what: str) -> torch.Tensor:
+    _need_gpu(t, what)
+    if t.dtype != torch.bfloat16:
+        raise TypeError(f"{what}: expected a bfloat16 tensor, got {t.dtype}")
+    return t.contiguous()
+
+
+def rms_norm_fwd(x: torch.Tensor, scale: torch.Tensor, eps: float):
+    """x [..., D] bf16, scale [D] bf16 -> (y like x, rstd fp32 [rows])"""
+    xc = _bf16_any(x, "rms_norm_fwd: x")
+    sc = _bf16_any(scale, "rms_norm_fwd: scale")
+    D = xc.shape[-1]
+    rows = xc.numel() // D
+    y = torch.empty_like(xc)
+    rstd = torch.empty(rows, dtype=torch.float32, device=x.device)
+    lib = _lib.load()
+    with torch.cuda.device(x.device):
+        rc = lib.ttamd_rms_norm_fwd_bf16(xc.data_ptr(), sc.data_ptr(), float(eps), y.data_ptr(), rstd.data_ptr(), rows, D, _stream(x))
+    _lib.check(rc, "rms_norm_fwd")
+    return y, rstd
+
+
+def rms_norm_bwd(gy: torch.Tensor, x: torch.Tensor, scale: torch.Tensor, rstd: torch.Tensor, want_gscale: bool):
+    """-> (gx like x, gscale [D] bf16 | None)"""
+    gc = _bf16_any(gy, "rms_norm_bwd: gy")
+    xc = _bf16_any(x, "rms_norm_bwd: x")
+    sc = _bf16_any(scale, "rms_norm_bwd: scale")
+    D = xc.shape[-1]
+    rows = xc.numel() // D
+    gx = torch.empty_like(xc)
+    lib = _lib.load()
+    gscale = torch.empty(D, dtype=torch.bfloat16, device=x.device) if want_gscale else None
+    nbytes = lib.ttamd_rms_norm_bwd_workspace_bytes(D) if want_gscale else 0
+    ws = _workspace(nbytes, x.device) if want_gscale else None
+    with torch.cuda.device(x.device):
+        rc = lib.ttamd_rms_norm_bwd_bf16(gc.data_ptr(), xc.data_ptr(), sc.data_ptr(), rstd.data_ptr(), gx.data_ptr(), _ptr(gscale),
+                                         rows, D, _ptr(ws), nbytes, _stream(x))
+    _lib.check(rc, "rms_norm_bwd")
+    return gx, gscale
+
+
+def rope(x: torch.Tensor, cache: torch.Tensor, inverse: bool = False) -> torch.Tensor:
+    """x [b, s, n_h, h_d] bf16, cache [s, h_d/2, 2] fp32 -> rotated x (inverse: by the negative angle)"""
+    xc = _bf16_any(x, "rope: x")
+    if xc.dim() != 4:
+        raise ValueError(f"rope: expected [b, s, n_h, h_d], got {tuple(x.shape)}")
+    b, s, nh, hd = xc.shape
+    _need_gpu(cache, "rope: cache")
+    if cache.dtype != torch.float32 or cache.numel() < s * hd or cache.shape[-1] != 2 or cache.shape[-2] != hd // 2:
+        raise ValueError(f"rope: cache must be fp32 [>= {s}, {hd // 2}, 2], got {tuple(cache.shape)} {cache.dtype}")
+    cc = cache.contiguous()
+    y = torch.empty_like(xc)
+    lib = _lib.load()
+    with torch.cuda.device(x.device):
+        rc = lib.ttamd_rope_bf16(xc.data_ptr(), cc.data_ptr(), y.data_ptr(), b, s, nh, hd, int(bool(inverse)), _stream(x))
+    _lib.check(rc, "rope")
+    return y
+
+
+def swiglu_fwd(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    g = _bf16_any(gate, "swiglu_fwd: gate")
+    u = _bf16_any(up, "swiglu_fwd: up")
+    if g.shape != u.shape:
+        raise ValueError(f"swiglu_fwd: shapes differ: {tuple(g.shape)} vs {tuple(u.shape)}")
+    out = torch.empty_like(g)
+    lib = _lib.load()
+    with torch.cuda.device(g.device):
+        rc = lib.ttamd_swiglu_fwd_bf16(g.data_ptr(), u.data_ptr(), out.data_ptr(), g.numel(), _stream(g))
+    _lib.check(rc, "swiglu_fwd")
+    return out
+
+
+def swiglu_bwd(gout: torch.Tensor, gate: torch.Tensor, up: torch.Tensor):
+    go = _bf16_any(gout, "swiglu_bwd: gout")
+    g = _bf16_any(gate, "swiglu_bwd: gate")
+    u = _bf16_any(up, "swiglu_bwd: up")
+    gg = torch.empty_like(g)
+    gu = torch.empty_like(u)
+    lib = _lib.load()
+    with torch.cuda.device(g.device):
+        rc = lib.ttamd_swiglu_bwd_bf16(go.data_ptr(), g.data_ptr(), u.data_ptr(), gg.data_ptr(), gu.data_ptr(), g.numel(), _stream(g))
+    _lib.check(rc, "swiglu_bwd")
+    return gg, gu
