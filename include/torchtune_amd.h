@@ -133,15 +133,17 @@ int ttamd_lora_hidden_bf16(const void* x, const void* lora_a, void* h, int64_t M
  * y = x . D(W)^T (+ bias) + scale . h . lora_b^T          (lora.py:137-147; nf4_linear.py:67-70 when rank == 0)
  *
  * x [M,K] bf16; quantized_data = NF4 codes of the [N,K] weight (block_size 64); block_scalers from
- * ttamd_nf4_block_scalers; h [M,rank] bf16 from ttamd_lora_hidden_bf16 and lora_b [N,rank] bf16 (both NULL iff
+ * ttamd_nf4_block_scalers; block_scalers_t = NULL or the same scalers transposed, fp32 [K/64, N], as
+ * ttamd_nf4_transpose_for_backward writes them (then a wave fetches the 64 scalers of a k-step with one coalesced
+ * load instead of two gathers; results are identical); h [M,rank] bf16 from ttamd_lora_hidden_bf16 and lora_b [N,rank] bf16 (both NULL iff
  * rank == 0); bias [N] bf16 or NULL; scale = alpha / rank; y out [M,N] bf16.
  * Requires K % 64 == 0, N % 64 == 0, rank % 8 == 0, 0 <= rank <= 64.
  * D(W) is bit-identical to ttamd_nf4_dequantize's output; all products are accumulated in fp32 and the sum is
  * rounded to bf16 once (the eager reference rounds after each of its five ops).
  */
-int ttamd_nf4_lora_linear_fwd_bf16(const void* x, const uint8_t* quantized_data, const void* block_scalers, const void* h,
-                                   const void* lora_b, int rank, float scale, const void* bias, void* y, int64_t M,
-                                   int64_t N, int64_t K, void* stream);
+int ttamd_nf4_lora_linear_fwd_bf16(const void* x, const uint8_t* quantized_data, const void* block_scalers,
+                                   const void* block_scalers_t, const void* h, const void* lora_b, int rank, float scale,
+                                   const void* bias, void* y, int64_t M, int64_t N, int64_t K, void* stream);
 
 /*
  * Optional transposed copy of an NF4 weight for the grad-input GEMM.  NF4 blocks run along K, the grad-input GEMM

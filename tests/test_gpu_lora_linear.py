@@ -179,7 +179,7 @@ def test_raw_c_abi_sequence_matches_python_layer():
     gb = torch.empty(N, r, dtype=BF, device=DEV)
     gx = torch.empty(M, K, dtype=BF, device=DEV)
     assert lib.ttamd_lora_hidden_bf16(xd.data_ptr(), Ad.data_ptr(), h.data_ptr(), M, K, r, ws.data_ptr(), ws.numel(), stream) == 0
-    assert lib.ttamd_nf4_lora_linear_fwd_bf16(xd.data_ptr(), t.quantized_data.data_ptr(), bscal.data_ptr(), h.data_ptr(),
+    assert lib.ttamd_nf4_lora_linear_fwd_bf16(xd.data_ptr(), t.quantized_data.data_ptr(), bscal.data_ptr(), None, h.data_ptr(),
                                               Bd.data_ptr(), r, 2.0, None, y.data_ptr(), M, N, K, stream) == 0
     assert lib.ttamd_lora_bwd_bf16(gyd.data_ptr(), xd.data_ptr(), h.data_ptr(), Bd.data_ptr(), 2.0, gh.data_ptr(), ga.data_ptr(),
                                    gb.data_ptr(), M, N, K, r, ws.data_ptr(), ws.numel(), stream) == 0
@@ -193,7 +193,12 @@ def test_raw_c_abi_sequence_matches_python_layer():
                                                 stream) == 0
     assert lib.ttamd_nf4_linear_bwd_dx_bf16(gyd.data_ptr(), t.quantized_data.data_ptr(), bscal.data_ptr(), qt.data_ptr(),
                                             st.data_ptr(), gh.data_ptr(), Ad.data_ptr(), r, gx2.data_ptr(), M, N, K, stream) == 0
+    # forward again with the transposed scalers: the same arithmetic, so the same bits
+    y_t = torch.empty_like(y)
+    assert lib.ttamd_nf4_lora_linear_fwd_bf16(xd.data_ptr(), t.quantized_data.data_ptr(), bscal.data_ptr(), st.data_ptr(),
+                                              h.data_ptr(), Bd.data_ptr(), r, 2.0, None, y_t.data_ptr(), M, N, K, stream) == 0
     torch.cuda.synchronize()
+    assert torch.equal(y_t, y)
     # transposed codes: element (k, n) of the copy is element (n, k) of the original
     codes = torch.stack([t.quantized_data >> 4, t.quantized_data & 0xF], dim=1).flatten().view(N, K)
     codes_t = torch.stack([qt >> 4, qt & 0xF], dim=1).flatten().view(K, N)

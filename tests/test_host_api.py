@@ -71,9 +71,9 @@ def test_argument_validation_needs_no_gpu():
     assert rc == -3 and b"workspace" in lib.ttamd_last_error()
     assert lib.ttamd_nf4_quantize_workspace_bytes(64 * 256, 64) >= 256 * 4
     # fused GEMM shape rules
-    rc = lib.ttamd_nf4_lora_linear_fwd_bf16(aligned, aligned, aligned, None, None, 0, 0.0, None, aligned, 8, 64, 100, None)
+    rc = lib.ttamd_nf4_lora_linear_fwd_bf16(aligned, aligned, aligned, None, None, None, 0, 0.0, None, aligned, 8, 64, 100, None)
     assert rc == -1 and b"multiple of the NF4 block size" in lib.ttamd_last_error()
-    rc = lib.ttamd_nf4_lora_linear_fwd_bf16(aligned, aligned, aligned, None, None, 8, 2.0, None, aligned, 8, 64, 64, None)
+    rc = lib.ttamd_nf4_lora_linear_fwd_bf16(aligned, aligned, aligned, None, None, None, 8, 2.0, None, aligned, 8, 64, 64, None)
     assert rc == -1 and b"adapter pointers" in lib.ttamd_last_error()
     rc = lib.ttamd_nf4_linear_bwd_dx_bf16(aligned, aligned, aligned, None, None, aligned, aligned, 12, aligned, 8, 64, 64, None)
     assert rc == -1 and b"rank" in lib.ttamd_last_error()

@@ -41,7 +41,8 @@ SIGNATURES = {
     "ttamd_lora_hidden_bf16": (_int, [_c_void_p, _c_void_p, _c_void_p, _i64, _i64, _int, _c_void_p, _size, _c_void_p]),
     "ttamd_nf4_lora_linear_fwd_bf16": (
         _int,
-        [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _int, _f32, _c_void_p, _c_void_p, _i64, _i64, _i64, _c_void_p],
+        [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _int, _f32, _c_void_p, _c_void_p, _i64, _i64, _i64,
+         _c_void_p],
     ),
     "ttamd_nf4_transpose_for_backward": (_int, [_c_void_p, _c_void_p, _i64, _i64, _c_void_p, _c_void_p, _c_void_p]),
     "ttamd_nf4_linear_bwd_dx_bf16": (

@@ -50,7 +50,7 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
 struct RsArgs {
   const uint16_t* X;     // [M, Kc] bf16 activations
   const uint8_t* codes;  // [Nout, Kc/2] packed NF4 codes of the weight view
-  const float* scal;     // !PER_ELEM: fp32 [Nout, Kc/64];  PER_ELEM: fp32 [Nout/64, Kc]
+  const float* scal;     // block scalers, fp32: MODE 0 [Nout, Kc/64]; MODE 2 [Kc/64, Nout]; MODE 1 per element [Nout/64, Kc]
   const uint16_t* lX;    // adapter activations [M, R] bf16 or null
   const uint16_t* lW;    // adapter weights: [Nout, R] (lw_row_major) or [R, Nout] bf16, or null
   const uint16_t* bias;  // [Nout] bf16 or null
@@ -76,15 +76,20 @@ struct RsLayout {
   static constexpr int kTotal = kLutOff;  // dynamic part; the table is a static LDS object of kLutBytes
 };
 
-template <int BM, bool PER_ELEM>
+// MODE 0: one scaler per (output column, 64-wide k-step), scaler tensor laid out like the weight's blocks
+// MODE 2: the same scalers, tensor transposed so that the 64 columns of a wave are contiguous (one coalesced load)
+// MODE 1: one scaler per contraction element, shared by the wave's 64 columns (the transposed weight of the backward)
+template <int BM, int MODE>
 __global__ __launch_bounds__(256) void nf4_gemm_rs_kernel(const RsArgs g) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the body uses LDS address-space casts and gfx950 builtins the host pass cannot parse
   static_assert(BM == 256 || BM == 128, "BM");
+  constexpr bool PER_ELEM = MODE == 1;
+  constexpr bool SCAL_T = MODE == 2;
   using L = RsLayout<BM>;
   constexpr int MT = BM / 32;       // activation tiles (MFMA columns) per wave
   constexpr int NT = 2;             // weight tiles (MFMA rows) per wave
   constexpr int kALoads = BM / 32;  // direct-to-LDS instructions per wave per k-step for the activation tile (8 rows each)
-  constexpr int kBatch = kALoads + NT + (PER_ELEM ? 1 : NT);  // vector-memory operations per wave per k-step
+  constexpr int kBatch = kALoads + NT + (MODE == 0 ? NT : 1);  // vector-memory operations per wave per k-step
   extern __shared__ __attribute__((aligned(16))) char smem[];
 
   const int tid = threadIdx.x;
@@ -139,6 +144,11 @@ __global__ __launch_bounds__(256) void nf4_gemm_rs_kernel(const RsArgs g) {
     w_off[j] = (uint32_t)(((int64_t)col * Kc) >> 1) + 16 * h;
     s_off[j] = (uint32_t)col * (uint32_t)nk * 4u;
   }
+  if constexpr (SCAL_T) {
+    int col = n0 + wv * 64 + lane;  // lane l fetches the scaler of the wave's column l
+    col = col < g.Nout ? col : g.Nout - 1;
+    s_off[0] = (uint32_t)col * 4u;
+  }
   if constexpr (PER_ELEM) {
     // scalers of the wave's 64-column block for the 64 contraction elements of a k-step: lane l fetches element l
     int ob = (n0 >> 6) + wv;
@@ -170,7 +180,8 @@ __global__ __launch_bounds__(256) void nf4_gemm_rs_kernel(const RsArgs g) {
     BatchAddr b;
     b.xb = reinterpret_cast<const char*>(g.X) + ((int64_t)tk << 7);      // + k0 * 2 bytes
     b.cb = reinterpret_cast<const char*>(g.codes) + ((int64_t)tk << 5);  // + k0 / 2 bytes
-    b.sb = reinterpret_cast<const char*>(g.scal) + (PER_ELEM ? ((int64_t)tk << 8) : ((int64_t)tk << 2));
+    b.sb = reinterpret_cast<const char*>(g.scal) +
+           (PER_ELEM ? ((int64_t)tk << 8) : SCAL_T ? (int64_t)tk * g.Nout * 4 : ((int64_t)tk << 2));
     b.abase = lds0 + sa * L::kStageA + wv * (BM / 4) * 128;
     b.wbase = lds0 + L::kWOff + sw * L::kStageW;
     return b;
@@ -222,7 +233,8 @@ __global__ __launch_bounds__(256) void nf4_gemm_rs_kernel(const RsArgs g) {
     for (int j = 0; j < NT; ++j) {
       const u32x4_t v = *reinterpret_cast<const u32x4_t*>(wbase + (wv * NT + j) * 1024 + lane * 16);
       codes[j][0] = v.x; codes[j][1] = v.y; codes[j][2] = v.z; codes[j][3] = v.w;
-      if constexpr (!PER_ELEM) s_out[j] = *reinterpret_cast<const float*>(wbase + 8192 + wv * 512 + j * 256 + lane * 4);
+      if constexpr (MODE == 0) s_out[j] = *reinterpret_cast<const float*>(wbase + 8192 + wv * 512 + j * 256 + lane * 4);
+      if constexpr (SCAL_T) s_out[j] = *reinterpret_cast<const float*>(wbase + 8192 + wv * 512 + (32 * j + l31) * 4);
     }
   };
 
@@ -418,27 +430,27 @@ __global__ __launch_bounds__(256) void nf4_gemm_rs_kernel(const RsArgs g) {
 #endif
 }
 
-template <int BM, bool PER_ELEM>
+template <int BM, int MODE>
 int launch_rs(RsArgs& g, hipStream_t s) {
   using L = RsLayout<BM>;
   g.tiles_m = (g.M + BM - 1) / BM;
   g.tiles_n = (g.Nout + kBN - 1) / kBN;
   static bool attr_set = false;  // idempotent; a race only repeats the call
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&nf4_gemm_rs_kernel<BM, PER_ELEM>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&nf4_gemm_rs_kernel<BM, MODE>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, L::kTotal);
     if (e != hipSuccess)
       return fail(TTAMD_ELAUNCH, "nf4_gemm_rs: cannot reserve %d bytes of LDS: %s", L::kTotal, hipGetErrorString(e));
     attr_set = true;
   }
-  nf4_gemm_rs_kernel<BM, PER_ELEM><<<dim3((unsigned)(g.tiles_m * g.tiles_n)), dim3(256), L::kTotal, s>>>(g);
+  nf4_gemm_rs_kernel<BM, MODE><<<dim3((unsigned)(g.tiles_m * g.tiles_n)), dim3(256), L::kTotal, s>>>(g);
   return check_launch("nf4_gemm_rs");
 }
 
 }  // namespace
 
 // Entry used by the C-ABI wrappers in nf4_gemm.hip.
-int run_gemm_rs(const void* X, const uint8_t* codes, const void* scal, bool per_elem, const void* lX, const void* lW,
+int run_gemm_rs(const void* X, const uint8_t* codes, const void* scal, int mode, const void* lX, const void* lW,
                 bool lw_row_major, int R, float lscale, const void* bias, void* C, int64_t M, int64_t Nout, int64_t Kc,
                 hipStream_t s) {
   RsArgs g;
@@ -454,9 +466,9 @@ int run_gemm_rs(const void* X, const uint8_t* codes, const void* scal, bool per_
   g.lscale = lscale;
   const int64_t tiles256 = ((M + 255) / 256) * ((Nout + kBN - 1) / kBN);
   const bool big = tiles256 >= 256;
-  if (per_elem) return big ? launch_rs<256, true>(g, s) : launch_rs<128, true>(g, s);
-  int rc = big ? launch_rs<256, false>(g, s) : launch_rs<128, false>(g, s);
-  return rc;
+  if (mode == 1) return big ? launch_rs<256, 1>(g, s) : launch_rs<128, 1>(g, s);
+  if (mode == 2) return big ? launch_rs<256, 2>(g, s) : launch_rs<128, 2>(g, s);
+  return big ? launch_rs<256, 0>(g, s) : launch_rs<128, 0>(g, s);
 }
 
 }  // namespace ttamd

@@ -44,7 +44,9 @@ class _QLoRALinearFn(torch.autograd.Function):
         N, K = weight.shape
         x2 = x.reshape(-1, K)
         h = ops.lora_hidden(x2, lora_a)
-        y = ops.nf4_lora_linear_fwd(x2, weight.quantized_data, weight.block_scalers(), N, h, lora_b, scale, bias)
+        tr = weight.backward_copy()
+        y = ops.nf4_lora_linear_fwd(x2, weight.quantized_data, weight.block_scalers(), N, h, lora_b, scale, bias,
+                                    block_scalers_t=tr[1] if tr else None)
         ctx.save_for_backward(x2, h, weight, lora_a, lora_b)
         ctx.scale = scale
         ctx.x_shape = x.shape

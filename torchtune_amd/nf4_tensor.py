@@ -464,7 +464,9 @@ class _LinearNF4(torch.autograd.Function):
         ctx.in_shape = input.shape
         if _fused_ok(input, weight, 0):
             x2 = input.reshape(-1, input.shape[-1])
-            y = ops.nf4_lora_linear_fwd(x2, weight.quantized_data, weight.block_scalers(), weight.shape[0])
+            tr = weight.backward_copy()
+            y = ops.nf4_lora_linear_fwd(x2, weight.quantized_data, weight.block_scalers(), weight.shape[0],
+                                        block_scalers_t=tr[1] if tr else None)
             return y.view(*input.shape[:-1], weight.shape[0])
         return F.linear(input, weight.to(input.dtype))
 

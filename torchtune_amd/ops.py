@@ -171,8 +171,10 @@ def lora_hidden(x: torch.Tensor, lora_a: torch.Tensor) -> torch.Tensor:
 def nf4_lora_linear_fwd(
     x: torch.Tensor, qdata: torch.Tensor, block_scalers: torch.Tensor, N: int, h: Optional[torch.Tensor] = None,
     lora_b: Optional[torch.Tensor] = None, scale: float = 0.0, bias: Optional[torch.Tensor] = None,
+    block_scalers_t: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
-    """y = x @ D(W).T (+bias) + scale * h @ lora_b.T ;  x [M,K] -> [M,N]"""
+    """y = x @ D(W).T (+bias) + scale * h @ lora_b.T ;  x [M,K] -> [M,N].  ``block_scalers_t``: the scalers transposed
+    ([K/64, N] fp32, second tensor of ``nf4_transpose_for_backward``): same result, cheaper scaler loads."""
     x = _bf16_2d(x, "nf4_lora_linear_fwd")
     M, K = x.shape
     rank = 0
@@ -191,8 +193,8 @@ def nf4_lora_linear_fwd(
         if events:
             events[0].record()
         rc = lib.ttamd_nf4_lora_linear_fwd_bf16(
-            x.data_ptr(), qdata.data_ptr(), block_scalers.data_ptr(), _ptr(h), _ptr(lora_b), rank, float(scale), _ptr(bias),
-            y.data_ptr(), M, N, K, _stream(x),
+            x.data_ptr(), qdata.data_ptr(), block_scalers.data_ptr(), _ptr(block_scalers_t), _ptr(h), _ptr(lora_b), rank,
+            float(scale), _ptr(bias), y.data_ptr(), M, N, K, _stream(x),
         )
         if events:
             events[1].record()
