@@ -161,11 +161,15 @@ __global__ __launch_bounds__(256) void nf4_gemm_rs_kernel(const RsArgs g) {
   // `base`, the wave's 64 lanes land in LDS at `lds`, `lds` + size, ...  Issued this way the compiler keeps no
   // bookkeeping for them (it would otherwise wait for ALL outstanding loads before the next LDS read it cannot prove
   // disjoint); completion is awaited explicitly with s_waitcnt vmcnt below.
-  auto dma16 = [&](uint32_t voff, const char* base, uint32_t lds) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(base), "s"(lds) : "memory", "m0");
+  // M0 (the LDS destination) is formed by the scalar add itself: `lds` is a wave-uniform base, `imm` a compile-time
+  // offset.  One wait state must separate a scalar write of M0 from the load that reads it.
+  auto dma16 = [&](uint32_t voff, const char* base, uint32_t lds, int imm) {
+    asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 ::"v"(voff), "s"(base), "s"(lds), "n"(imm) : "memory", "m0", "scc");
   };
-  auto dma4 = [&](uint32_t voff, const char* base, uint32_t lds) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" ::"v"(voff), "s"(base), "s"(lds) : "memory", "m0");
+  auto dma4 = [&](uint32_t voff, const char* base, uint32_t lds, int imm) {
+    asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1"
+                 ::"v"(voff), "s"(base), "s"(lds), "n"(imm) : "memory", "m0", "scc");
   };
   const uint32_t lds0 = (uint32_t)(uintptr_t)TT_LDS_PTR(smem);
   // A batch (k-step t) is kBatch loads: the activation tile -> A stage, this wave's code bytes and scalers -> W stage.
@@ -173,28 +177,36 @@ __global__ __launch_bounds__(256) void nf4_gemm_rs_kernel(const RsArgs g) {
   // tens of cycles per 64-lane load and a wave that finds its queue full cannot issue anything else meanwhile.
   struct BatchAddr {
     const char *xb, *cb, *sb;
-    uint32_t abase, wbase;
+    uint32_t abase, wcodes, wscal;  // LDS bases of this wave's share of the A stage, of its code bytes and of its scalers
+  };
+  // Global bases of k-step t are base + min(t, nk - 1) * stride (past the end the last tile is reloaded, never
+  // consumed).  The main loop carries the three pointers and bumps them by a constant instead of recomputing them.
+  const int64_t s_stride = PER_ELEM ? 256 : SCAL_T ? (int64_t)g.Nout * 4 : 4;
+  auto batch_addr_at = [&](const char* xb, const char* cb, const char* sb, int sa, int sw) -> BatchAddr {
+    BatchAddr b;
+    b.xb = xb;
+    b.cb = cb;
+    b.sb = sb;
+    b.abase = lds0 + sa * L::kStageA + wv * (BM / 4) * 128;
+    b.wcodes = lds0 + L::kWOff + sw * L::kStageW + wv * NT * 1024;
+    b.wscal = lds0 + L::kWOff + sw * L::kStageW + 8192 + wv * 512;
+    return b;
   };
   auto batch_addr = [&](int t, int sa, int sw) -> BatchAddr {
-    const int tk = t < nk ? t : nk - 1;  // past the end: reload the last tile (never consumed)
-    BatchAddr b;
-    b.xb = reinterpret_cast<const char*>(g.X) + ((int64_t)tk << 7);      // + k0 * 2 bytes
-    b.cb = reinterpret_cast<const char*>(g.codes) + ((int64_t)tk << 5);  // + k0 / 2 bytes
-    b.sb = reinterpret_cast<const char*>(g.scal) +
-           (PER_ELEM ? ((int64_t)tk << 8) : SCAL_T ? (int64_t)tk * g.Nout * 4 : ((int64_t)tk << 2));
-    b.abase = lds0 + sa * L::kStageA + wv * (BM / 4) * 128;
-    b.wbase = lds0 + L::kWOff + sw * L::kStageW;
-    return b;
+    const int tk = t < nk ? t : nk - 1;
+    return batch_addr_at(reinterpret_cast<const char*>(g.X) + ((int64_t)tk << 7),      // + k0 * 2 bytes
+                         reinterpret_cast<const char*>(g.codes) + ((int64_t)tk << 5),  // + k0 / 2 bytes
+                         reinterpret_cast<const char*>(g.scal) + tk * s_stride, sa, sw);
   };
   auto issue_one = [&](const BatchAddr& b, int d) {  // d is a compile-time constant after unrolling
     if (d < kALoads) {
-      dma16(a_off[d], b.xb, b.abase + d * 1024);
+      dma16(a_off[d], b.xb, b.abase, d * 1024);
     } else if (d < kALoads + NT) {
       const int j = d - kALoads;
-      dma16(w_off[j], b.cb, b.wbase + (wv * NT + j) * 1024);
+      dma16(w_off[j], b.cb, b.wcodes, j * 1024);
     } else if (d < kBatch) {
       const int j = d - kALoads - NT;
-      dma4(s_off[j], b.sb, b.wbase + 8192 + wv * 512 + j * 256);
+      dma4(s_off[j], b.sb, b.wscal, j * 256);
     }
   };
   auto issue = [&](int t, int sa, int sw) {
@@ -211,7 +223,16 @@ __global__ __launch_bounds__(256) void nf4_gemm_rs_kernel(const RsArgs g) {
   bf16x8_t xfa[MT], xfb[MT];
 
   auto fetch_byte = [&](int j, int ks, int b) {
-    pend[j][b] = *reinterpret_cast<const float2*>(lut + (((codes[j][ks] >> (8 * b)) & 0xffu) << 3));
+    uint32_t off;
+    if (b == 0) {
+      // byte 0 as one sub-dword-addressed shift, like the compiler's own choice for bytes 1-3 (it would otherwise
+      // emit a mask and a shift here)
+      asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_0"
+          : "=v"(off) : "v"(3u), "v"(codes[j][ks]));
+    } else {
+      off = ((codes[j][ks] >> (8 * b)) & 0xffu) << 3;
+    }
+    pend[j][b] = *reinterpret_cast<const float2*>(lut + off);
   };
   // finish byte b of tile j into wf[j]; s8 = the eight per-element scalers of the substep (PER_ELEM), s = the row's scaler
   auto finish_byte = [&](u32x4_t (&wf)[NT], int j, int b, const float (&s)[NT], const float (&s8)[8]) {
@@ -324,10 +345,21 @@ __global__ __launch_bounds__(256) void nf4_gemm_rs_kernel(const RsArgs g) {
   constexpr int kDOdd = (kBatch - 4 * kDEven + 3) / 4;  // and per odd quarter
   static_assert(4 * kDEven + 4 * kDOdd >= kBatch && kDOdd <= 2 && kDOdd >= 0, "batch does not fit the 8 quarter phases");
   int a0 = 0, w0 = 0;  // A / W stage of k-step kt
+  const char *pxb, *pcb, *psb;  // global bases of k-step kt + 2
+  {
+    const BatchAddr b2 = batch_addr(2, 0, 0);
+    pxb = b2.xb; pcb = b2.cb; psb = b2.sb;
+  }
   for (int kt = 0; kt < nk; ++kt) {
     const int a1 = (a0 + 1) & 3, a2 = (a0 + 2) & 3;
     const int w1 = w0 == 2 ? 0 : w0 + 1, w2 = w1 == 2 ? 0 : w1 + 1;
-    const BatchAddr b = batch_addr(kt + 2, a2, w2);
+    const BatchAddr b = batch_addr_at(pxb, pcb, psb, a2, w2);
+    {
+      const int64_t adv = kt + 3 < nk ? 1 : 0;
+      pxb += adv << 7;
+      pcb += adv << 5;
+      psb += adv * s_stride;
+    }
     phase(xfa, wfa, xfb, a0, 1, wfb, sc, w0, 1, 2, b, 0, kDEven, kDOdd);
     phase(xfb, wfb, xfa, a0, 2, wfa, sc, w0, 2, 3, b, 2 * (kDEven + kDOdd), kDEven, kDOdd);
     asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kBatch) : "memory");
