@@ -346,7 +346,8 @@ def main() -> int:
             "unit": "TFLOP/s",
             "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4),
             "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(args.workload),
-            "traffic_unit": "bytes per launch (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, rocprofv3 --pmc; algorithmic 210.4e6)",
+            "traffic_unit": "bytes per launch, average over a step's launches (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 from rocprofv3 "
+                            "--pmc runs; algorithmic 210.4e6)" if args.workload in MEASURED_TRAFFIC_BYTES_PER_LAUNCH else None,
             "launches_timed": launches,
             "gemm_ms_per_step": round(gemm_ms / args.steps, 2),
             "per_shape": per_shape,

@@ -284,3 +284,35 @@ def test_adapter_dropout_and_disabled_paths_still_correct():
     torch.manual_seed(0)
     y_train = layer(x.to(DEV))
     assert y_train.shape == (M, N) and not torch.equal(y_train.cpu(), layer.eval()(x.to(DEV)).cpu())
+
+
+def test_empty_single_row_and_ragged_token_counts():
+    """Token counts that are empty, one, or not a multiple of any tile: the layer still equals the oracle; an empty
+    batch gives an empty output and zero adapter gradients (the composed path: nothing to launch)."""
+    torch.manual_seed(7)
+    K, N, r = 256, 320, 8
+    prev = torch.get_default_dtype()
+    torch.set_default_dtype(BF)
+    try:
+        with torch.device(DEV):
+            layer = LoRALinear(K, N, rank=r, alpha=16.0, use_bias=True, quantize_base=True)
+    finally:
+        torch.set_default_dtype(prev)
+    W = (torch.randn(N, K) * 0.02).to(BF)
+    B = (torch.randn(N, r) * 0.05).to(BF)
+    with torch.no_grad():
+        layer.weight.copy_(W.to(DEV))
+        layer.lora_b.weight.copy_(B.to(DEV))
+    parts = nf4_oracle.nf4_quantize(W, 64, 256)
+    for shape in [(0, K), (1, K), (3, 0, K), (1, 1, K), (257, K), (2, 131, K)]:
+        x = torch.randn(*shape).to(BF)
+        xd = x.to(DEV).requires_grad_()
+        y = layer(xd)
+        assert y.shape == (*shape[:-1], N)
+        want = lora_oracle.lora_linear_forward(x, parts, layer.lora_a.weight.detach().cpu(), B, 16.0, r, bias=layer.bias.detach().cpu())
+        _close(y.detach().cpu(), want, 1e-2, 1e-2)
+        layer.zero_grad()
+        y.float().sum().backward()
+        assert xd.grad.shape == xd.shape and layer.lora_a.weight.grad.shape == (r, K)
+        if x.numel() == 0:
+            assert float(layer.lora_b.weight.grad.abs().sum()) == 0.0
