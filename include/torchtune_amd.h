@@ -146,6 +146,35 @@ int ttamd_nf4_lora_linear_fwd_bf16(const void* x, const uint8_t* quantized_data,
                                    const void* bias, void* y, int64_t M, int64_t N, int64_t K, void* stream);
 
 /*
+ * DoRALinear (torchtune/modules/peft/dora.py:156-192) over an NF4 base weight.
+ *
+ * ttamd_nf4_dora_weight_norm_bf16: weight_norm[n] = bf16(|| D(W)[n,:] + bf16(scale * bf16(lora_b . lora_a))[n,:] ||_2)
+ *   (dora.py:141-144, called in every forward at :183 and by initialize_dora_magnitude at :139), computed in one pass
+ *   over the packed weight without materialising it; if magnitude [N] bf16 is given, also
+ *   mag_norm_scale[n] = bf16(magnitude[n] / weight_norm[n]) (:185).  workspace:
+ *   ttamd_dora_weight_norm_workspace_bytes(N, K) bytes.
+ * ttamd_nf4_dora_linear_fwd_bf16: y = (x . D(W)^T + bias + scale . h . lora_b^T) * col_scale per output column,
+ *   col_scale = mag_norm_scale [N] bf16 (:187-191 rearranged: (s - 1) base + s lora scale + base = s (base + lora scale));
+ *   otherwise identical to ttamd_nf4_lora_linear_fwd_bf16.
+ * ttamd_dora_bwd_prologue_bf16: from gy [M,N] and the layer's saved output y [M,N]:
+ *   gy0 = bf16(gy * mag_norm_scale), the gradient for ttamd_lora_bwd_bf16 / ttamd_nf4_linear_bwd_dx_bf16, and
+ *   gmagnitude[n] = bf16(sum_m gy[m,n] * y[m,n] / magnitude[n]) (fixed summation order; the norm is a constant in the
+ *   reference's graph, :184).  workspace: ttamd_dora_bwd_workspace_bytes(N) bytes.
+ */
+size_t ttamd_dora_weight_norm_workspace_bytes(int64_t N, int64_t K);
+int ttamd_nf4_dora_weight_norm_bf16(const uint8_t* quantized_data, const void* block_scalers, const void* lora_a,
+                                    const void* lora_b, int rank, float scale, const void* magnitude, void* weight_norm,
+                                    void* mag_norm_scale, int64_t N, int64_t K, void* workspace, size_t workspace_bytes,
+                                    void* stream);
+int ttamd_nf4_dora_linear_fwd_bf16(const void* x, const uint8_t* quantized_data, const void* block_scalers,
+                                   const void* block_scalers_t, const void* h, const void* lora_b, int rank, float scale,
+                                   const void* bias, const void* col_scale, void* y, int64_t M, int64_t N, int64_t K,
+                                   void* stream);
+size_t ttamd_dora_bwd_workspace_bytes(int64_t N);
+int ttamd_dora_bwd_prologue_bf16(const void* gy, const void* out, const void* mag_norm_scale, const void* magnitude, void* gy0,
+                                 void* gmagnitude, int64_t M, int64_t N, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * Optional transposed copy of an NF4 weight for the grad-input GEMM.  NF4 blocks run along K, the grad-input GEMM
  * contracts over N; with the codes re-packed along N (quantized_data_t [K, N/2], even n in the high nibble) and the
  * block scalers transposed (block_scalers_t fp32 [K/64, N]) that GEMM streams the weight exactly like the forward

@@ -69,3 +69,34 @@ def merged_weight(parts: "nf4_oracle.NF4Parts", lora_a: torch.Tensor, lora_b: to
     w = nf4_oracle.nf4_dequantize(parts).clone()
     w += (alpha / rank) * lora_b @ lora_a
     return w
+
+
+def dora_linear_forward(x, weight, lora_a, lora_b, magnitude, alpha: float, rank: int, bias=None, disabled: bool = False):
+    """``DoRALinear.forward`` (``torchtune/modules/peft/dora.py:156-192``) op for op.  ``weight`` is a dense tensor or
+    the NF4 parts of one; the weight norm is a constant of the graph (``.detach()``, ``:183-184``)."""
+    scaling = alpha / rank
+    if isinstance(weight, nf4_oracle.NF4Parts):
+        base_out = _LinearNF4.apply(x, weight)
+        if bias is not None:
+            base_out = base_out + bias
+        dense = nf4_oracle.nf4_dequantize(weight).to(x.dtype)
+    else:
+        base_out = F.linear(x, weight, bias)
+        dense = weight.to(x.dtype)
+    if disabled:
+        return base_out
+    lora_out = F.linear(F.linear(x, lora_a), lora_b)
+    x_eye = torch.eye(lora_a.shape[1], dtype=x.dtype)
+    lora_weight = F.linear(F.linear(x_eye, lora_a), lora_b).T
+    merged = dense + scaling * lora_weight.detach()
+    weight_norm = torch.linalg.norm(merged, dim=1).to(merged.dtype).detach()
+    mag_norm_scale = (magnitude / weight_norm).view(1, -1)
+    dora_out = (mag_norm_scale - 1) * base_out + mag_norm_scale * lora_out * scaling
+    return dora_out + base_out
+
+
+def dora_weight_norm(weight, lora_a, lora_b, alpha: float, rank: int) -> torch.Tensor:
+    """``DoRALinear._get_weight_norm`` as used by ``initialize_dora_magnitude`` (``dora.py:137-144``)."""
+    dense = nf4_oracle.nf4_dequantize(weight).to(lora_a.dtype) if isinstance(weight, nf4_oracle.NF4Parts) else weight
+    merged = dense + (alpha / rank) * (lora_b @ lora_a)
+    return torch.linalg.norm(merged, dim=1).to(merged.dtype)

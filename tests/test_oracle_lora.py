@@ -90,3 +90,50 @@ def test_lora_a_init_bound():
     ref = torch.empty(8, 2048)
     torch.nn.init.kaiming_uniform_(ref, a=5 ** 0.5)
     assert ref.abs().max() <= bound
+
+
+def test_reference_known_answer_dora_forward():
+    # tests/torchtune/modules/peft/test_dora.py:106-111 (EXPECTED_VAL = 0.05201): fixed-init layer incl. the magnitude
+    W, _, A, B = _fixed_layer(False)
+    mag = lora_oracle.fixed_init_tensor((128,))
+    y = lora_oracle.dora_linear_forward(_inputs(), W, A, B, mag, alpha=1.0, rank=4)
+    assert y.shape == (2, 32, 128)
+    torch.testing.assert_close(y.mean(), torch.tensor(GOLDEN["dora_forward"]["expected_mean"]), atol=1e-4, rtol=1e-6)
+
+
+def test_dora_closed_forms():
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(5, 24, generator=g, dtype=torch.float64)
+    W = torch.randn(16, 24, generator=g, dtype=torch.float64)
+    A = torch.randn(4, 24, generator=g, dtype=torch.float64)
+    B = torch.randn(16, 4, generator=g, dtype=torch.float64)
+    merged = W + 0.5 * B @ A
+    norm = merged.norm(dim=1)
+    torch.testing.assert_close(lora_oracle.dora_weight_norm(W, A, B, alpha=2.0, rank=4), norm)
+    # with the magnitude at its initial value (the row norms) DoRA is exactly LoRA
+    y = lora_oracle.dora_linear_forward(x, W, A, B, norm, alpha=2.0, rank=4)
+    torch.testing.assert_close(y, lora_oracle.lora_linear_forward(x, W, A, B, alpha=2.0, rank=4))
+    # in general it is the merged linear with every output row rescaled to norm `magnitude`
+    mag = torch.rand(16, generator=g, dtype=torch.float64) + 0.5
+    y = lora_oracle.dora_linear_forward(x, W, A, B, mag, alpha=2.0, rank=4)
+    torch.testing.assert_close(y, x @ (merged * (mag / norm)[:, None]).T)
+    # the norm is a constant of the graph: d y / d magnitude = y / magnitude
+    mag.requires_grad_()
+    y = lora_oracle.dora_linear_forward(x, W, A, B, mag, alpha=2.0, rank=4)
+    (gm,) = torch.autograd.grad(y.sum(), mag)
+    torch.testing.assert_close(gm, (y.detach() / mag.detach()).sum(0))
+
+
+def test_dora_module_dense_path_reproduces_the_known_answer():
+    """The module's composed path (dense fp32 weights, CPU) against the reference's known answer."""
+    from torchtune_amd.modules.peft import DoRALinear
+
+    layer = DoRALinear(in_dim=64, out_dim=128, rank=4, alpha=1.0, use_bias=False)
+    with torch.no_grad():
+        for p in layer.parameters():
+            p.copy_(lora_oracle.fixed_init_tensor(tuple(p.shape)))
+    y = layer(_inputs())
+    torch.testing.assert_close(y.mean(), torch.tensor(GOLDEN["dora_forward"]["expected_mean"]), atol=1e-4, rtol=1e-6)
+    assert layer.adapter_params() == ["lora_a.weight", "lora_b.weight", "magnitude"]
+    with pytest.raises(ValueError, match="quantize_base"):
+        DoRALinear(8, 8, 2, 1.0, block_size=64)

@@ -6,7 +6,7 @@ All arithmetic runs in ``lib/libtorchtune_amd.so`` (hand-written HIP, plain C AB
 """
 from .nf4_tensor import NF4Tensor, implements, linear_nf4, to_nf4
 from .modules.low_precision import FrozenNF4Linear
-from .modules.peft import LoRALinear, QATLoRALinear
+from .modules.peft import DoRALinear, LoRALinear, QATLoRALinear
 from .qat import (
     FakeQuantizeConfig,
     FakeQuantizedLinear,
@@ -23,6 +23,7 @@ __all__ = [
     "implements",
     "FrozenNF4Linear",
     "LoRALinear",
+    "DoRALinear",
     "QATLoRALinear",
     "FakeQuantizeConfig",
     "FakeQuantizer",

@@ -44,6 +44,22 @@ SIGNATURES = {
         [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _int, _f32, _c_void_p, _c_void_p, _i64, _i64, _i64,
          _c_void_p],
     ),
+    "ttamd_dora_weight_norm_workspace_bytes": (_size, [_i64, _i64]),
+    "ttamd_nf4_dora_weight_norm_bf16": (
+        _int,
+        [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _int, _f32, _c_void_p, _c_void_p, _c_void_p, _i64, _i64, _c_void_p, _size,
+         _c_void_p],
+    ),
+    "ttamd_nf4_dora_linear_fwd_bf16": (
+        _int,
+        [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _int, _f32, _c_void_p, _c_void_p, _c_void_p, _i64, _i64,
+         _i64, _c_void_p],
+    ),
+    "ttamd_dora_bwd_workspace_bytes": (_size, [_i64]),
+    "ttamd_dora_bwd_prologue_bf16": (
+        _int,
+        [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _i64, _i64, _c_void_p, _size, _c_void_p],
+    ),
     "ttamd_nf4_transpose_for_backward": (_int, [_c_void_p, _c_void_p, _i64, _i64, _c_void_p, _c_void_p, _c_void_p]),
     "ttamd_nf4_linear_bwd_dx_bf16": (
         _int,

@@ -390,8 +390,8 @@ int check_gemm_args(const char* who, const void* a, const uint8_t* qdata, const 
 
 // nf4_gemm_rs.hip
 int run_gemm_rs(const void* X, const uint8_t* codes, const void* scal, int mode, const void* lX, const void* lW,
-                bool lw_row_major, int R, float lscale, const void* bias, void* C, int64_t M, int64_t Nout, int64_t Kc,
-                hipStream_t s);
+                bool lw_row_major, int R, float lscale, const void* bias, const void* cscale, void* C, int64_t M, int64_t Nout,
+                int64_t Kc, hipStream_t s);
 }  // namespace ttamd
 
 using namespace ttamd;
@@ -415,18 +415,39 @@ extern "C" int ttamd_nf4_block_scalers(const int8_t* quantized_scalers, const vo
   return check_launch("nf4_block_scalers");
 }
 
+namespace {
+int lora_linear_fwd(const char* who, const void* x, const uint8_t* quantized_data, const void* block_scalers,
+                    const void* block_scalers_t, const void* h, const void* lora_b, int rank, float scale, const void* bias,
+                    const void* col_scale, void* y, int64_t M, int64_t N, int64_t K, void* stream) {
+  if (int rc = check_gemm_args(who, x, quantized_data, block_scalers, y, M, N, K, rank, h, lora_b)) return rc;
+  TT_REQUIRE((bias == nullptr || (reinterpret_cast<uintptr_t>(bias) & 7u) == 0) &&
+                 (col_scale == nullptr || (reinterpret_cast<uintptr_t>(col_scale) & 7u) == 0),
+             "%s: bias / col_scale must be 8-byte aligned", who);
+  if (block_scalers_t) {
+    TT_REQUIRE(aligned16(block_scalers_t), "%s: block_scalers_t must be 16-byte aligned", who);
+    return run_gemm_rs(x, quantized_data, block_scalers_t, 2, h, lora_b, true, rank, scale, bias, col_scale, y, M, N, K,
+                       reinterpret_cast<hipStream_t>(stream));
+  }
+  return run_gemm_rs(x, quantized_data, block_scalers, 0, h, lora_b, true, rank, scale, bias, col_scale, y, M, N, K,
+                     reinterpret_cast<hipStream_t>(stream));
+}
+}  // namespace
+
 extern "C" int ttamd_nf4_lora_linear_fwd_bf16(const void* x, const uint8_t* quantized_data, const void* block_scalers,
                                               const void* block_scalers_t, const void* h, const void* lora_b, int rank,
                                               float scale, const void* bias, void* y, int64_t M, int64_t N, int64_t K,
                                               void* stream) {
-  if (int rc = check_gemm_args("nf4_lora_linear_fwd", x, quantized_data, block_scalers, y, M, N, K, rank, h, lora_b)) return rc;
-  if (block_scalers_t) {
-    TT_REQUIRE(aligned16(block_scalers_t), "nf4_lora_linear_fwd: block_scalers_t must be 16-byte aligned");
-    return run_gemm_rs(x, quantized_data, block_scalers_t, 2, h, lora_b, true, rank, scale, bias, y, M, N, K,
-                       reinterpret_cast<hipStream_t>(stream));
-  }
-  return run_gemm_rs(x, quantized_data, block_scalers, 0, h, lora_b, true, rank, scale, bias, y, M, N, K,
-                     reinterpret_cast<hipStream_t>(stream));
+  return lora_linear_fwd("nf4_lora_linear_fwd", x, quantized_data, block_scalers, block_scalers_t, h, lora_b, rank, scale, bias,
+                         nullptr, y, M, N, K, stream);
+}
+
+extern "C" int ttamd_nf4_dora_linear_fwd_bf16(const void* x, const uint8_t* quantized_data, const void* block_scalers,
+                                              const void* block_scalers_t, const void* h, const void* lora_b, int rank,
+                                              float scale, const void* bias, const void* col_scale, void* y, int64_t M,
+                                              int64_t N, int64_t K, void* stream) {
+  TT_REQUIRE(col_scale, "nf4_dora_linear_fwd: col_scale is null");
+  return lora_linear_fwd("nf4_dora_linear_fwd", x, quantized_data, block_scalers, block_scalers_t, h, lora_b, rank, scale, bias,
+                         col_scale, y, M, N, K, stream);
 }
 
 extern "C" int ttamd_nf4_transpose_for_backward(const uint8_t* quantized_data, const void* block_scalers, int64_t N, int64_t K,
@@ -454,7 +475,7 @@ extern "C" int ttamd_nf4_linear_bwd_dx_bf16(const void* gy, const uint8_t* quant
              "nf4_linear_bwd_dx: the transposed codes and scalers must be given together");
   if (quantized_data_t != nullptr) {
     TT_REQUIRE(aligned16(quantized_data_t) && aligned16(block_scalers_t), "nf4_linear_bwd_dx: transposed copies must be 16-byte aligned");
-    return run_gemm_rs(gy, quantized_data_t, block_scalers_t, 1, gh, lora_a, false, rank, 1.0f, nullptr, gx, M, K, N,
+    return run_gemm_rs(gy, quantized_data_t, block_scalers_t, 1, gh, lora_a, false, rank, 1.0f, nullptr, nullptr, gx, M, K, N,
                        reinterpret_cast<hipStream_t>(stream));
   }
   GemmArgs g;

@@ -54,6 +54,7 @@ struct RsArgs {
   const uint16_t* lX;    // adapter activations [M, R] bf16 or null
   const uint16_t* lW;    // adapter weights: [Nout, R] (lw_row_major) or [R, Nout] bf16, or null
   const uint16_t* bias;  // [Nout] bf16 or null
+  const uint16_t* cscale;  // [Nout] bf16 or null: C = (acc + bias) * cscale per column (DoRA's magnitude / norm)
   uint16_t* C;           // [M, Nout] bf16
   int M, Nout, Kc, R;
   int lw_row_major;
@@ -438,12 +439,18 @@ __global__ __launch_bounds__(256) void nf4_gemm_rs_kernel(const RsArgs g) {
           b4[0] = bits_f32(bb.x << 16); b4[1] = bits_f32(bb.x & 0xffff0000u);
           b4[2] = bits_f32(bb.y << 16); b4[3] = bits_f32(bb.y & 0xffff0000u);
         }
+        float c4[4] = {1.f, 1.f, 1.f, 1.f};
+        if (g.cscale) {
+          const u32x2_t cc = *reinterpret_cast<const u32x2_t*>(g.cscale + n0 + wv * 64 + 32 * j + 8 * q + 4 * h);
+          c4[0] = bits_f32(cc.x << 16); c4[1] = bits_f32(cc.x & 0xffff0000u);
+          c4[2] = bits_f32(cc.y << 16); c4[3] = bits_f32(cc.y & 0xffff0000u);
+        }
 #pragma unroll
         for (int i = 0; i < MT; ++i) {
           const int r = 32 * i + l31;
           u32x2_t o;
-          o.x = pack_bf16x2(acc[j][i][4 * q + 0] + b4[0], acc[j][i][4 * q + 1] + b4[1]);
-          o.y = pack_bf16x2(acc[j][i][4 * q + 2] + b4[2], acc[j][i][4 * q + 3] + b4[3]);
+          o.x = pack_bf16x2((acc[j][i][4 * q + 0] + b4[0]) * c4[0], (acc[j][i][4 * q + 1] + b4[1]) * c4[1]);
+          o.y = pack_bf16x2((acc[j][i][4 * q + 2] + b4[2]) * c4[2], (acc[j][i][4 * q + 3] + b4[3]) * c4[3]);
           *reinterpret_cast<u32x2_t*>(band + r * 128 + (((4 * j + q) ^ (r & 7)) << 4) + 8 * h) = o;
         }
       }
@@ -483,8 +490,8 @@ int launch_rs(RsArgs& g, hipStream_t s) {
 
 // Entry used by the C-ABI wrappers in nf4_gemm.hip.
 int run_gemm_rs(const void* X, const uint8_t* codes, const void* scal, int mode, const void* lX, const void* lW,
-                bool lw_row_major, int R, float lscale, const void* bias, void* C, int64_t M, int64_t Nout, int64_t Kc,
-                hipStream_t s) {
+                bool lw_row_major, int R, float lscale, const void* bias, const void* cscale, void* C, int64_t M, int64_t Nout,
+                int64_t Kc, hipStream_t s) {
   RsArgs g;
   g.X = reinterpret_cast<const uint16_t*>(X);
   g.codes = codes;
@@ -492,6 +499,7 @@ int run_gemm_rs(const void* X, const uint8_t* codes, const void* scal, int mode,
   g.lX = reinterpret_cast<const uint16_t*>(lX);
   g.lW = reinterpret_cast<const uint16_t*>(lW);
   g.bias = reinterpret_cast<const uint16_t*>(bias);
+  g.cscale = reinterpret_cast<const uint16_t*>(cscale);
   g.C = reinterpret_cast<uint16_t*>(C);
   g.M = (int)M; g.Nout = (int)Nout; g.Kc = (int)Kc; g.R = R;
   g.lw_row_major = lw_row_major ? 1 : 0;

@@ -171,7 +171,7 @@ def lora_hidden(x: torch.Tensor, lora_a: torch.Tensor) -> torch.Tensor:
 def nf4_lora_linear_fwd(
     x: torch.Tensor, qdata: torch.Tensor, block_scalers: torch.Tensor, N: int, h: Optional[torch.Tensor] = None,
     lora_b: Optional[torch.Tensor] = None, scale: float = 0.0, bias: Optional[torch.Tensor] = None,
-    block_scalers_t: Optional[torch.Tensor] = None,
+    block_scalers_t: Optional[torch.Tensor] = None, col_scale: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """y = x @ D(W).T (+bias) + scale * h @ lora_b.T ;  x [M,K] -> [M,N].  ``block_scalers_t``: the scalers transposed
     ([K/64, N] fp32, second tensor of ``nf4_transpose_for_backward``): same result, cheaper scaler loads."""
@@ -192,10 +192,17 @@ def nf4_lora_linear_fwd(
         events = _gemm_timer("fwd", M, N, K, rank) if _gemm_timer is not None else None
         if events:
             events[0].record()
-        rc = lib.ttamd_nf4_lora_linear_fwd_bf16(
-            x.data_ptr(), qdata.data_ptr(), block_scalers.data_ptr(), _ptr(block_scalers_t), _ptr(h), _ptr(lora_b), rank,
-            float(scale), _ptr(bias), y.data_ptr(), M, N, K, _stream(x),
-        )
+        if col_scale is None:
+            rc = lib.ttamd_nf4_lora_linear_fwd_bf16(
+                x.data_ptr(), qdata.data_ptr(), block_scalers.data_ptr(), _ptr(block_scalers_t), _ptr(h), _ptr(lora_b), rank,
+                float(scale), _ptr(bias), y.data_ptr(), M, N, K, _stream(x),
+            )
+        else:  # DoRA: every output column times magnitude / weight norm
+            col_scale = _bf16_any(col_scale, "nf4_lora_linear_fwd: col_scale")
+            rc = lib.ttamd_nf4_dora_linear_fwd_bf16(
+                x.data_ptr(), qdata.data_ptr(), block_scalers.data_ptr(), _ptr(block_scalers_t), _ptr(h), _ptr(lora_b), rank,
+                float(scale), _ptr(bias), col_scale.data_ptr(), y.data_ptr(), M, N, K, _stream(x),
+            )
         if events:
             events[1].record()
     _lib.check(rc, "nf4_lora_linear_fwd")
@@ -431,3 +438,48 @@ def swiglu_bwd(gout: torch.Tensor, gate: torch.Tensor, up: torch.Tensor):
         rc = lib.ttamd_swiglu_bwd_bf16(go.data_ptr(), g.data_ptr(), u.data_ptr(), gg.data_ptr(), gu.data_ptr(), g.numel(), _stream(g))
     _lib.check(rc, "swiglu_bwd")
     return gg, gu
+
+
+# ---------------------------------------------------------------------------------------------------
+# DoRA over an NF4 base weight
+# ---------------------------------------------------------------------------------------------------
+def nf4_dora_weight_norm(qdata: torch.Tensor, block_scalers: torch.Tensor, N: int, K: int, lora_a: torch.Tensor,
+                         lora_b: torch.Tensor, scale: float, magnitude: Optional[torch.Tensor] = None):
+    """-> (weight_norm [N] bf16, magnitude / weight_norm [N] bf16 | None): row norms of D(W) + scale * B @ A"""
+    _need_gpu(qdata, "nf4_dora_weight_norm")
+    a = _bf16_2d(lora_a, "nf4_dora_weight_norm: lora_a")
+    b = _bf16_2d(lora_b, "nf4_dora_weight_norm: lora_b")
+    rank = a.shape[0]
+    if a.shape != (rank, K) or b.shape != (N, rank):
+        raise ValueError(f"nf4_dora_weight_norm: lora_a {tuple(a.shape)} / lora_b {tuple(b.shape)} do not fit [{N}, {K}]")
+    mag = _bf16_any(magnitude, "nf4_dora_weight_norm: magnitude") if magnitude is not None else None
+    norm = torch.empty(N, dtype=torch.bfloat16, device=qdata.device)
+    mns = torch.empty(N, dtype=torch.bfloat16, device=qdata.device) if mag is not None else None
+    lib = _lib.load()
+    nbytes = lib.ttamd_dora_weight_norm_workspace_bytes(N, K)
+    ws = _workspace(nbytes, qdata.device)
+    with torch.cuda.device(qdata.device):
+        rc = lib.ttamd_nf4_dora_weight_norm_bf16(qdata.data_ptr(), block_scalers.data_ptr(), a.data_ptr(), b.data_ptr(), rank,
+                                                 float(scale), _ptr(mag), norm.data_ptr(), _ptr(mns), N, K, ws.data_ptr(), nbytes,
+                                                 _stream(qdata))
+    _lib.check(rc, "nf4_dora_weight_norm")
+    return norm, mns
+
+
+def dora_bwd_prologue(gy: torch.Tensor, out: torch.Tensor, mag_norm_scale: torch.Tensor, magnitude: torch.Tensor):
+    """gy, out [M, N] bf16 -> (gy * mag_norm_scale [M, N] bf16, grad of magnitude [N] bf16)"""
+    g = _bf16_2d(gy, "dora_bwd_prologue: gy")
+    o = _bf16_2d(out, "dora_bwd_prologue: out")
+    mns = _bf16_any(mag_norm_scale, "dora_bwd_prologue: mag_norm_scale")
+    mag = _bf16_any(magnitude, "dora_bwd_prologue: magnitude")
+    M, N = g.shape
+    gy0 = torch.empty_like(g)
+    gmag = torch.empty(N, dtype=torch.bfloat16, device=g.device)
+    lib = _lib.load()
+    nbytes = lib.ttamd_dora_bwd_workspace_bytes(N)
+    ws = _workspace(nbytes, g.device)
+    with torch.cuda.device(g.device):
+        rc = lib.ttamd_dora_bwd_prologue_bf16(g.data_ptr(), o.data_ptr(), mns.data_ptr(), mag.data_ptr(), gy0.data_ptr(),
+                                              gmag.data_ptr(), M, N, ws.data_ptr(), nbytes, _stream(g))
+    _lib.check(rc, "dora_bwd_prologue")
+    return gy0, gmag
