@@ -282,6 +282,16 @@ int ttamd_swiglu_fwd_bf16(const void* gate, const void* up, void* out, int64_t n
 int ttamd_swiglu_bwd_bf16(const void* gout, const void* gate, const void* up, void* ggate, void* gup, int64_t numel,
                           void* stream);
 
+/*
+ * The per-chunk body of LinearCrossEntropyLoss (torchtune/modules/loss/cross_entropy_loss.py:86-112):
+ * F.cross_entropy(logits.float(), target, reduction="sum", ignore_index), forward and backward in one pass.
+ * logits [rows, V] bf16; target [rows] int64 (class index in [0, V), or ignore_index); loss out [rows] fp32 =
+ * logsumexp - logit[target] (0 for an ignored row; the caller sums); grad_logits out [rows, V] bf16 =
+ * grad_scale * (softmax - onehot) (0 for an ignored row).  V a multiple of 8, at most 131072.
+ */
+int ttamd_cross_entropy_fwd_bwd_bf16(const void* logits, const int64_t* target, int64_t ignore_index, float grad_scale,
+                                     float* loss, void* grad_logits, int64_t rows, int64_t V, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

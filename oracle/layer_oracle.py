@@ -50,3 +50,9 @@ def rope(x: torch.Tensor, cache: torch.Tensor) -> torch.Tensor:
 
 def swiglu(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     return F.silu(gate) * up
+
+
+def cross_entropy_sum(logits: torch.Tensor, target: torch.Tensor, ignore_index: int = -100) -> torch.Tensor:
+    """The per-chunk loss of ``LinearCrossEntropyLoss.compute_cross_entropy``
+    (``torchtune/modules/loss/cross_entropy_loss.py:86-112``): the library routine itself."""
+    return F.cross_entropy(logits.float(), target, reduction="sum", ignore_index=ignore_index)

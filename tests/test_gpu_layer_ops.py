@@ -108,3 +108,24 @@ def test_full_size_properties_8b_activations():
     a = torch.randn(8192, 14336, device=DEV, generator=g).to(BF)
     z = ops.swiglu_fwd(a, torch.ones_like(a))
     torch.testing.assert_close(z.float(), torch.nn.functional.silu(a.float()), rtol=1e-2, atol=1e-2)
+
+
+@pytest.mark.parametrize("rows,V", [(7, 1024), (33, 128256), (5, 131072), (4, 8)])
+def test_cross_entropy_forward_backward(rows, V):
+    g = torch.Generator().manual_seed(4)
+    logits = (torch.randn(rows, V, generator=g) * 3).to(BF).requires_grad_()
+    target = torch.randint(0, V, (rows,), generator=g)
+    target[rows // 2] = -100  # an ignored row
+    target[0] = V - 1
+    want = lo.cross_entropy_sum(logits, target) * 0.25
+    want.backward()
+    ld = logits.detach().to(DEV).requires_grad_()
+    got = layer_ops.cross_entropy_sum(ld, target.to(DEV), scale=0.25)
+    (got * 2.0).backward()  # the incoming gradient rescales the stored one
+    torch.testing.assert_close(got.cpu(), want.detach(), rtol=1e-4, atol=1e-4)
+    # gradients are probabilities (<= 1) times 0.25 * 2, rounded to bf16
+    torch.testing.assert_close(ld.grad.cpu().float(), 2.0 * logits.grad.float(), rtol=1e-2, atol=1e-5)
+    assert torch.count_nonzero(ld.grad[rows // 2]) == 0
+    per_row, _ = ops.cross_entropy_fwd_bwd(ld.detach(), target.to(DEV))
+    ref_rows = torch.nn.functional.cross_entropy(logits.detach().float(), target, reduction="none")
+    torch.testing.assert_close(per_row.cpu(), ref_rows, rtol=1e-4, atol=1e-4)

@@ -55,3 +55,22 @@ def test_swiglu_against_fp64_and_gradients():
     ga, gu = torch.autograd.grad(lo.swiglu(a, u).sum(), (a, u))
     torch.testing.assert_close(ga, u * s * (1 + a * (1 - s)))
     torch.testing.assert_close(gu, a * s)
+
+
+def test_cross_entropy_sum_closed_forms():
+    # uniform logits: loss = log(V) per row; a dominant correct class: loss -> 0; ignored rows contribute nothing
+    V = 50
+    z = torch.zeros(3, V)
+    t = torch.tensor([1, 7, -100])
+    torch.testing.assert_close(lo.cross_entropy_sum(z, t), torch.tensor(2 * torch.log(torch.tensor(float(V)))))
+    big = torch.full((1, V), -30.0)
+    big[0, 4] = 30.0
+    assert float(lo.cross_entropy_sum(big, torch.tensor([4]))) < 1e-6
+    # gradient = softmax - onehot
+    x = torch.randn(2, V, dtype=torch.float64, requires_grad=True)
+    tt = torch.tensor([3, 9])
+    lo.cross_entropy_sum(x, tt).backward()
+    want = torch.softmax(x.detach().float(), -1)
+    want[0, 3] -= 1
+    want[1, 9] -= 1
+    torch.testing.assert_close(x.grad.float(), want, rtol=1e-5, atol=1e-6)

@@ -394,3 +394,128 @@ extern "C" int ttamd_swiglu_bwd_bf16(const void* gout, const void* gate, const v
       reinterpret_cast<uint16_t*>(ggate), reinterpret_cast<uint16_t*>(gup), n_chunks);
   return check_launch("swiglu_bwd");
 }
+
+// ---------------------------------------------------------------------------------------------------
+// Cross entropy over bf16 logits, forward and backward in one pass (the per-chunk body of the reference's
+// LinearCrossEntropyLoss, torchtune/modules/loss/cross_entropy_loss.py:86-112: F.cross_entropy(logits.float(),
+// target, reduction="sum", ignore_index)).  A workgroup of 1024 threads holds one row of logits in registers
+// (16 chunks of 8 per thread: up to 131072 classes), reduces max and sum of exponentials through LDS, and writes
+//   loss[row]  = logsumexp(row) - row[target]                      (0 for an ignored row)
+//   grad[row]  = bf16(grad_scale * (softmax(row) - onehot(target)))  (0 for an ignored row)
+// so the logits are read once and never widened to fp32 in memory.
+// ---------------------------------------------------------------------------------------------------
+namespace ttamd {
+namespace {
+
+constexpr int kCeThreads = 1024;
+constexpr int kCeChunks = 16;
+
+__global__ __launch_bounds__(kCeThreads) void cross_entropy_kernel(const uint16_t* __restrict__ logits,
+                                                                    const int64_t* __restrict__ target, int64_t ignore_index,
+                                                                    float grad_scale, float* __restrict__ loss,
+                                                                    uint16_t* __restrict__ grad, int V) {
+  __shared__ float red[kCeThreads / 64];
+  __shared__ float bcast;
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int64_t row = blockIdx.x;
+  const int chunks = V >> 3;
+  const u32x4_t* xr = reinterpret_cast<const u32x4_t*>(logits + row * V);
+  u32x4_t* gr = reinterpret_cast<u32x4_t*>(grad + row * V);
+  const int64_t tgt = target[row];
+  if (tgt == ignore_index) {  // uniform over the workgroup
+    for (int i = 0; i < kCeChunks; ++i) {
+      const int c = t + kCeThreads * i;
+      if (c < chunks) __builtin_nontemporal_store(u32x4_t{0, 0, 0, 0}, gr + c);
+    }
+    if (t == 0) loss[row] = 0.f;
+    return;
+  }
+  u32x4_t v[kCeChunks];
+  float mx = -__builtin_inff();
+#pragma unroll
+  for (int i = 0; i < kCeChunks; ++i) {
+    const int c = t + kCeThreads * i;
+    v[i] = u32x4_t{0xff80ff80u, 0xff80ff80u, 0xff80ff80u, 0xff80ff80u};  // -inf pairs: neutral for max and exp
+    if (c < chunks) v[i] = __builtin_nontemporal_load(xr + c);
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      mx = __builtin_fmaxf(mx, lo_f(v[i][d]));
+      mx = __builtin_fmaxf(mx, hi_f(v[i][d]));
+    }
+  }
+#pragma unroll
+  for (int off = 1; off < kWave; off <<= 1) mx = __builtin_fmaxf(mx, __shfl_xor(mx, off, kWave));
+  if (lane == 0) red[wave] = mx;
+  __syncthreads();
+  if (t == 0) {
+    float m = red[0];
+    for (int w = 1; w < kCeThreads / 64; ++w) m = __builtin_fmaxf(m, red[w]);
+    bcast = m;
+  }
+  __syncthreads();
+  mx = bcast;
+  float se = 0.f;
+#pragma unroll
+  for (int i = 0; i < kCeChunks; ++i)
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      se += __builtin_amdgcn_exp2f((lo_f(v[i][d]) - mx) * 1.4426950408889634f);
+      se += __builtin_amdgcn_exp2f((hi_f(v[i][d]) - mx) * 1.4426950408889634f);
+    }
+  se = wave_sum(se);
+  __syncthreads();  // everyone has read bcast
+  if (lane == 0) red[wave] = se;
+  __syncthreads();
+  if (t == 0) {
+    float s = red[0];
+    for (int w = 1; w < kCeThreads / 64; ++w) s += red[w];
+    bcast = s;
+  }
+  __syncthreads();
+  se = bcast;
+  const float inv = grad_scale / se;
+  if (t == 0) {
+    const bool valid = tgt >= 0 && tgt < V;  // an out-of-range class gives NaN, never an out-of-bounds read
+    const float xt = bf16_bits_to_f32(logits[row * V + (valid ? tgt : 0)]);
+    loss[row] = valid ? (mx - xt) + __builtin_logf(se) : __builtin_nanf("");
+  }
+#pragma unroll
+  for (int i = 0; i < kCeChunks; ++i) {
+    const int c = t + kCeThreads * i;
+    if (c >= chunks) continue;
+    float p[8];
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      p[2 * d] = __builtin_amdgcn_exp2f((lo_f(v[i][d]) - mx) * 1.4426950408889634f) * inv;
+      p[2 * d + 1] = __builtin_amdgcn_exp2f((hi_f(v[i][d]) - mx) * 1.4426950408889634f) * inv;
+    }
+    const int64_t e0 = (int64_t)c * 8;
+    if (tgt >= e0 && tgt < e0 + 8) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        if (e0 + e == tgt) p[e] -= grad_scale;
+    }
+    u32x4_t o;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) o[d] = pack2(p[2 * d], p[2 * d + 1]);
+    __builtin_nontemporal_store(o, gr + c);
+  }
+}
+
+}  // namespace
+}  // namespace ttamd
+
+extern "C" int ttamd_cross_entropy_fwd_bwd_bf16(const void* logits, const int64_t* target, int64_t ignore_index, float grad_scale,
+                                                float* loss, void* grad_logits, int64_t rows, int64_t V, void* stream) {
+  TT_REQUIRE(logits && target && loss && grad_logits, "cross_entropy: null pointer argument");
+  TT_REQUIRE(aligned16(logits) && aligned16(grad_logits), "cross_entropy: logits and grad_logits must be 16-byte aligned");
+  TT_REQUIRE(rows > 0 && rows < (int64_t(1) << 31) && V > 0 && V % 8 == 0, "cross_entropy: bad shape rows=%lld V=%lld (V must be a multiple of 8)",
+             (long long)rows, (long long)V);
+  if (V > (int64_t)kCeThreads * kCeChunks * 8)
+    return fail(TTAMD_EUNSUPPORTED, "cross_entropy: V (%lld) exceeds the %d classes one workgroup holds in registers", (long long)V,
+                kCeThreads * kCeChunks * 8);
+  cross_entropy_kernel<<<dim3((unsigned)rows), dim3(kCeThreads), 0, reinterpret_cast<hipStream_t>(stream)>>>(
+      reinterpret_cast<const uint16_t*>(logits), target, ignore_index, grad_scale, loss, reinterpret_cast<uint16_t*>(grad_logits),
+      (int)V);
+  return check_launch("cross_entropy");
+}

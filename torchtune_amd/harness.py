@@ -189,10 +189,14 @@ class Decoder(nn.Module):
         hidden = h.reshape(-1, h.shape[-1])
         target = labels.reshape(-1)
         total = hidden.new_zeros((), dtype=torch.float32)
+        n = target.numel()
         for hc, tc in zip(hidden.chunk(self.loss_chunks), target.chunk(self.loss_chunks)):
-            logits = self.output(hc).float()
-            total = total + F.cross_entropy(logits, tc, reduction="sum")
-        return total / target.numel()
+            logits = self.output(hc)
+            if _fused(logits) and logits.shape[-1] % 8 == 0 and logits.shape[-1] <= 131072:
+                total = total + layer_ops.cross_entropy_sum(logits, tc, scale=1.0 / n)
+            else:
+                total = total + F.cross_entropy(logits.float(), tc, reduction="sum") / n
+        return total
 
 
 @torch.no_grad()

@@ -1,4 +1,4 @@
-"""RMSNorm, rotary embedding and the SwiGLU gate as single-pass HIP kernels with autograd.
+"""RMSNorm, rotary embedding, the SwiGLU gate and the chunk cross entropy as single-pass HIP kernels with autograd.
 
 These are the memory-bound neighbours of the quantized linears inside a decoder layer.  The reference runs each as
 a chain of eager kernels: ``RMSNorm`` (``torchtune/modules/rms_norm.py:11-41``), ``Llama3ScaledRoPE.forward``
@@ -79,3 +79,24 @@ class _SwiGLUFn(torch.autograd.Function):
 def swiglu(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     """``silu(gate) * up`` with the eager sequence's two bf16 roundings."""
     return _SwiGLUFn.apply(gate, up)
+
+
+class _CrossEntropySumFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, logits, target, ignore_index: int, scale: float):
+        loss, grad = ops.cross_entropy_fwd_bwd(logits, target, ignore_index, scale)
+        ctx.save_for_backward(grad)
+        return loss.sum() * scale
+
+    @staticmethod
+    def backward(ctx, g):
+        (grad,) = ctx.saved_tensors
+        return grad.mul_(g.to(grad.dtype)), None, None, None
+
+
+def cross_entropy_sum(logits: torch.Tensor, target: torch.Tensor, ignore_index: int = -100, scale: float = 1.0) -> torch.Tensor:
+    """``scale * F.cross_entropy(logits.float(), target, reduction="sum", ignore_index=ignore_index)`` for bf16 logits
+    ``[rows, V]``: the per-chunk body of the reference's ``LinearCrossEntropyLoss``
+    (``torchtune/modules/loss/cross_entropy_loss.py:86-112``).  The gradient w.r.t. the logits is produced in the same
+    pass (pre-multiplied by ``scale``) and only rescaled by the incoming gradient in backward; call backward once."""
+    return _CrossEntropySumFn.apply(logits, target, ignore_index, scale)

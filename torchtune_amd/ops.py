@@ -483,3 +483,21 @@ def dora_bwd_prologue(gy: torch.Tensor, out: torch.Tensor, mag_norm_scale: torch
                                               gmag.data_ptr(), M, N, ws.data_ptr(), nbytes, _stream(g))
     _lib.check(rc, "dora_bwd_prologue")
     return gy0, gmag
+
+
+def cross_entropy_fwd_bwd(logits: torch.Tensor, target: torch.Tensor, ignore_index: int = -100, grad_scale: float = 1.0):
+    """logits [rows, V] bf16, target [rows] int64 -> (per-row loss fp32 [rows], grad_scale * dloss/dlogits bf16 [rows, V])"""
+    lg = _bf16_2d(logits, "cross_entropy_fwd_bwd: logits")
+    _need_gpu(target, "cross_entropy_fwd_bwd: target")
+    if target.dtype != torch.int64 or target.shape != (lg.shape[0],):
+        raise TypeError(f"cross_entropy_fwd_bwd: target must be int64 [{lg.shape[0]}], got {tuple(target.shape)} {target.dtype}")
+    tg = target.contiguous()
+    rows, V = lg.shape
+    loss = torch.empty(rows, dtype=torch.float32, device=lg.device)
+    grad = torch.empty_like(lg)
+    lib = _lib.load()
+    with torch.cuda.device(lg.device):
+        rc = lib.ttamd_cross_entropy_fwd_bwd_bf16(lg.data_ptr(), tg.data_ptr(), int(ignore_index), float(grad_scale), loss.data_ptr(),
+                                                  grad.data_ptr(), rows, V, _stream(lg))
+    _lib.check(rc, "cross_entropy_fwd_bwd")
+    return loss, grad
