@@ -70,7 +70,7 @@ def _close(got, want, rtol, atol):
 
 CASES = [
     # M, N, K, rank, bias
-    (2048, 2048, 2048, 8, False),  # BASELINE config 1 shape
+    (2048, 2048, 2048, 8, False),  # the single-layer benchmark configuration (2048 x 2048, rank 8)
     (1, 64, 64, 8, False),
     (37, 192, 128, 16, True),
     (300, 320, 448, 24, False),
@@ -124,7 +124,7 @@ def test_layer_forward_backward_vs_oracle(M, N, K, r, bias):
 
 
 def test_config1_single_layer_sum_of_squares():
-    # BASELINE config 1: W bf16 [2048,2048] N(0,0.02) seed 0, rank 8, alpha 16, B ~ N(0,0.01), x [4,512,2048], loss sum(y^2) in fp32
+    # single-layer benchmark configuration: W bf16 [2048,2048] N(0,0.02) seed 0, rank 8, alpha 16, B ~ N(0,0.01), x [4,512,2048], loss sum(y^2) in fp32
     torch.manual_seed(0)
     W = (torch.randn(2048, 2048) * 0.02).to(BF)
     A = lora_oracle.lora_a_init_(torch.empty(8, 2048)).to(BF)

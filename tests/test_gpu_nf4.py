@@ -46,7 +46,7 @@ def test_quantise_and_dequantise_bit_exact(dtype, shape, bs, sbs):
 
 
 def test_config1_weight_through_raw_c_abi():
-    # BASELINE config 1: bf16 [2048, 2048] ~ N(0, 0.02), seed 0, block 64 / scaler block 256
+    # single-layer benchmark configuration: bf16 [2048, 2048] ~ N(0, 0.02), seed 0, block 64 / scaler block 256
     torch.manual_seed(0)
     w = (torch.randn(2048, 2048) * 0.02).to(torch.bfloat16)
     p = nf4_oracle.nf4_quantize(w, 64, 256)
