@@ -474,13 +474,16 @@ int launch_rs(RsArgs& g, hipStream_t s) {
   using L = RsLayout<BM>;
   g.tiles_m = (g.M + BM - 1) / BM;
   g.tiles_n = (g.Nout + kBN - 1) / kBN;
-  static bool attr_set = false;  // idempotent; a race only repeats the call
-  if (!attr_set) {
+  // the limit is a per-device attribute of the function: set it for the current device once (a race only repeats the call)
+  static bool attr_set[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = -1;
+  if (dev < 0 || !attr_set[dev]) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&nf4_gemm_rs_kernel<BM, MODE>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, L::kTotal);
     if (e != hipSuccess)
       return fail(TTAMD_ELAUNCH, "nf4_gemm_rs: cannot reserve %d bytes of LDS: %s", L::kTotal, hipGetErrorString(e));
-    attr_set = true;
+    if (dev >= 0) attr_set[dev] = true;
   }
   nf4_gemm_rs_kernel<BM, MODE><<<dim3((unsigned)(g.tiles_m * g.tiles_n)), dim3(256), L::kTotal, s>>>(g);
   return check_launch("nf4_gemm_rs");
@@ -492,6 +495,11 @@ int launch_rs(RsArgs& g, hipStream_t s) {
 int run_gemm_rs(const void* X, const uint8_t* codes, const void* scal, int mode, const void* lX, const void* lW,
                 bool lw_row_major, int R, float lscale, const void* bias, const void* cscale, void* C, int64_t M, int64_t Nout,
                 int64_t Kc, hipStream_t s) {
+  // per-lane byte offsets inside the kernel are 32-bit
+  TT_REQUIRE(M * Kc * 2 < (int64_t(1) << 32) && Nout * Kc / 2 < (int64_t(1) << 32) && Nout * (Kc / 64) * 4 < (int64_t(1) << 32) &&
+                 M * Nout * 2 < (int64_t(1) << 40),
+             "nf4_gemm: operand too large for 32-bit offsets (M=%lld Nout=%lld Kc=%lld); split the token dimension", (long long)M,
+             (long long)Nout, (long long)Kc);
   RsArgs g;
   g.X = reinterpret_cast<const uint16_t*>(X);
   g.codes = codes;
