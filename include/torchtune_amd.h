@@ -243,6 +243,15 @@ int ttamd_fq_per_group_int4_sym(const void* w, int dtype, int64_t rows, int64_t 
 int ttamd_quantize_per_group_int4(const void* w, int dtype, int64_t rows, int64_t K, int group_size, int8_t* q,
                                   float* scale, float* zero_point, void* stream);
 
+/*
+ * Dense weight of the converted 8da4w linear (what Int8DynActInt4WeightLinear.forward rebuilds before its matmul; the
+ * converted model is what recipes/quantize.py:92-95 saves and evaluates): out = dtype((q - zero_point) * scale).
+ * q [rows,K] int8 holding int4 values; scale, zero_point fp32 [rows, K/group_size] (zero_point may be NULL = 0);
+ * out [rows,K] `dtype`.
+ */
+int ttamd_dequantize_per_group_int4(const int8_t* q, const float* scale, const float* zero_point, int dtype, int64_t rows,
+                                    int64_t K, int group_size, void* out, void* stream);
+
 /* ------------------------------------------------------------------------------------------------
  * Neighbours of the quantized linears inside a decoder layer (one pass over HBM each, bf16 tensors, fp32 math).
  * Floating-point kernels: results agree with the eager sequences to a tolerance (summation order and hardware

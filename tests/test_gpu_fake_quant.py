@@ -134,3 +134,20 @@ def test_prepare_then_convert_is_bit_exact_and_consistent():
         assert torch.equal(conv.scales.cpu(), s) and torch.equal(conv.zeros.cpu(), z) and conv.scales.shape == (w.shape[0], w.shape[1] // 32)
     # the converted model computes what the fake-quantised model computed
     torch.testing.assert_close(model(x).float(), y_fake.float(), rtol=1e-2, atol=1e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("g", [8, 32, 256])
+def test_converted_weight_dequantises_to_the_fake_quantised_weight(dtype, g):
+    """dequantise(convert(W)) must be bit-identical to fake_quantise(W): that is what makes the converted model compute
+    what the fake-quantised model trained with; also with non-zero zero points against the eager formula."""
+    gen = torch.Generator().manual_seed(9)
+    w = (torch.randn(96, 512, generator=gen) * 0.1).to(dtype)
+    fq_w, _ = fq.fq_per_group_int4_sym(w, g)
+    q, s, z = fq.quantize_per_group_int4(w, g)
+    got = ops.dequantize_per_group_int4(q.to(DEV), s.to(DEV), z.to(DEV), g, dtype)
+    assert bits_equal(got.cpu(), fq_w)
+    assert bits_equal(ops.dequantize_per_group_int4(q.to(DEV), s.to(DEV), None, g, dtype).cpu(), fq_w)
+    zz = torch.randint(-3, 4, z.shape, generator=gen).float()
+    want = ((q.view(96, -1, g).float() - zz[:, :, None]) * s[:, :, None]).to(dtype).view(96, 512)
+    assert bits_equal(ops.dequantize_per_group_int4(q.to(DEV), s.to(DEV), zz.to(DEV), g, dtype).cpu(), want)

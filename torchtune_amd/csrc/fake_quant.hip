@@ -281,6 +281,26 @@ int launch_per_token(const void* x, int64_t rows, int64_t K, void* out, float* s
   return check_launch("fq_per_token_int8_asym");
 }
 
+// Dense weight of a converted 8da4w linear: out = dtype((q - zero) * scale), q int8-held int4 values, one fp32 scale
+// and zero per group of the last dimension.  One lane = 8 elements (8 bytes in, 16 or 32 bytes out).
+template <bool BF16>
+__global__ __launch_bounds__(256) void dequant_per_group_kernel(const int8_t* __restrict__ q, const float* __restrict__ scale,
+                                                                const float* __restrict__ zero, int64_t n_chunks, int log2_lpg,
+                                                                void* __restrict__ out) {
+  const int64_t ch = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (ch >= n_chunks) return;
+  const uint2 raw = reinterpret_cast<const uint2*>(q)[ch];
+  const float sc = scale[ch >> log2_lpg];
+  const float z = zero ? zero[ch >> log2_lpg] : 0.0f;
+  float v[8];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    v[e] = Arith<BF16>::rnd(((float)(int8_t)(raw.x >> (8 * e)) - z) * sc);
+    v[e + 4] = Arith<BF16>::rnd(((float)(int8_t)(raw.y >> (8 * e)) - z) * sc);
+  }
+  Chunk8<BF16>::store(out, ch, v);
+}
+
 int check_group_args(const void* w, int dtype, int64_t rows, int64_t K, int group_size) {
   TT_REQUIRE(dtype == TTAMD_BF16 || dtype == TTAMD_F32, "fake_quant: unknown dtype code %d", dtype);
   TT_REQUIRE(w != nullptr && aligned16(w), "fake_quant: input must be a non-null 16-byte aligned pointer");
@@ -346,4 +366,25 @@ extern "C" int ttamd_quantize_per_group_int4(const void* w, int dtype, int64_t r
     fq_per_group_kernel<false, true><<<dim3((unsigned)grid), dim3(256), 0, s>>>(w, n_chunks, lpg, log2_exact(lpg), nullptr,
                                                                                  q, scale, zero_point);
   return check_launch("quantize_per_group_int4");
+}
+
+extern "C" int ttamd_dequantize_per_group_int4(const int8_t* q, const float* scale, const float* zero_point, int dtype,
+                                               int64_t rows, int64_t K, int group_size, void* out, void* stream) {
+  TT_REQUIRE(dtype == TTAMD_BF16 || dtype == TTAMD_F32, "dequantize_per_group_int4: unknown dtype code %d", dtype);
+  TT_REQUIRE(q && scale && out && (reinterpret_cast<uintptr_t>(q) & 7u) == 0 && aligned16(out),
+             "dequantize_per_group_int4: q (8-byte aligned), scale and out (16-byte aligned) must be non-null");
+  TT_REQUIRE(rows > 0 && K > 0, "dequantize_per_group_int4: rows and K must be positive");
+  TT_REQUIRE(group_size >= 8 && group_size <= 512 && is_pow2(group_size) && K % group_size == 0,
+             "dequantize_per_group_int4: group_size (%d) must be a power of two in [8, 512] dividing K (%lld)", group_size,
+             (long long)K);
+  const int64_t n_chunks = rows * K / 8;
+  const int64_t grid = (n_chunks + 255) / 256;
+  TT_REQUIRE(grid < (int64_t(1) << 31), "dequantize_per_group_int4: tensor too large for one launch");
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const int l2 = log2_exact(group_size / 8);
+  if (dtype == TTAMD_BF16)
+    dequant_per_group_kernel<true><<<dim3((unsigned)grid), dim3(256), 0, s>>>(q, scale, zero_point, n_chunks, l2, out);
+  else
+    dequant_per_group_kernel<false><<<dim3((unsigned)grid), dim3(256), 0, s>>>(q, scale, zero_point, n_chunks, l2, out);
+  return check_launch("dequantize_per_group_int4");
 }

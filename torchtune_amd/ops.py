@@ -355,6 +355,28 @@ def quantize_per_group_int4(w: torch.Tensor, group_size: int):
 # ---------------------------------------------------------------------------------------------------
 # neighbours of the quantized linears in a decoder layer: RMSNorm, rotary embedding, SwiGLU gate
 # ---------------------------------------------------------------------------------------------------
+def dequantize_per_group_int4(q: torch.Tensor, scale: torch.Tensor, zeros: Optional[torch.Tensor], group_size: int,
+                              dtype: torch.dtype) -> torch.Tensor:
+    """q [rows, K] int8 (int4 values), scale/zeros fp32 [rows, K/g] -> dtype((q - zeros) * scale) [rows, K]"""
+    _need_gpu(q, "dequantize_per_group_int4")
+    code = _code(dtype, "dequantize_per_group_int4")
+    if q.dtype != torch.int8 or q.dim() != 2:
+        raise TypeError(f"dequantize_per_group_int4: q must be a 2-D int8 tensor, got {tuple(q.shape)} {q.dtype}")
+    qc = q.contiguous()
+    rows, K = qc.shape
+    sc = scale.to(torch.float32).contiguous()
+    zc = zeros.to(torch.float32).contiguous() if zeros is not None else None
+    if sc.numel() != rows * (K // max(group_size, 1)) or (zc is not None and zc.numel() != sc.numel()):
+        raise ValueError("dequantize_per_group_int4: scale / zeros must have rows * K / group_size elements")
+    out = torch.empty(rows, K, dtype=dtype, device=q.device)
+    lib = _lib.load()
+    with torch.cuda.device(q.device):
+        rc = lib.ttamd_dequantize_per_group_int4(qc.data_ptr(), sc.data_ptr(), _ptr(zc), code, rows, K, group_size, out.data_ptr(),
+                                                 _stream(q))
+    _lib.check(rc, "dequantize_per_group_int4")
+    return out
+
+
 def _bf16_any(t: torch.Tensor, what: str) -> torch.Tensor:
     _need_gpu(t, what)
     if t.dtype != torch.bfloat16:

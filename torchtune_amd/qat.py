@@ -267,10 +267,7 @@ class Int8DynActInt4WeightLinear(nn.Module):
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         x = x.to(self.precision)
         x_q, _, _ = ops.fq_per_token_int8_asym(x, want_qparams=False)
-        N, K = self.weight.shape
-        g = self.groupsize
-        w = (self.weight.view(N, K // g, g).to(self.precision) - self.zeros.view(N, K // g, 1).to(self.precision))
-        w = (w * self.scales.view(N, K // g, 1)).to(self.precision).view(N, K)
+        w = ops.dequantize_per_group_int4(self.weight, self.scales, self.zeros, self.groupsize, self.precision)
         return F.linear(x_q, w, self.bias)
 
 
