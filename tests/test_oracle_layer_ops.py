@@ -62,7 +62,9 @@ def test_cross_entropy_sum_closed_forms():
     V = 50
     z = torch.zeros(3, V)
     t = torch.tensor([1, 7, -100])
-    torch.testing.assert_close(lo.cross_entropy_sum(z, t), torch.tensor(2 * torch.log(torch.tensor(float(V)))))
+    import math
+
+    torch.testing.assert_close(lo.cross_entropy_sum(z, t), torch.tensor(2 * math.log(V)))
     big = torch.full((1, V), -30.0)
     big[0, 4] = 30.0
     assert float(lo.cross_entropy_sum(big, torch.tensor([4]))) < 1e-6
