@@ -1,14 +1,18 @@
+"""Adapter layers of the quantized-linear path (LoRA, QAT + LoRA, DoRA over dense or NF4 base weights) and the small
+amount of adapter bookkeeping their callers need."""
+from ._adapter_base import LowRankAdapterLinear
 from ._utils import AdapterModule, get_adapter_params, get_merged_lora_ckpt, set_trainable_params
 from .dora import DoRALinear
 from .lora import LoRALinear, QATLoRALinear, TrainableParams
 
-__all__ = [
-    "AdapterModule",
-    "DoRALinear",
+__all__ = (
     "LoRALinear",
     "QATLoRALinear",
+    "DoRALinear",
+    "LowRankAdapterLinear",
     "TrainableParams",
+    "AdapterModule",
     "get_adapter_params",
-    "get_merged_lora_ckpt",
     "set_trainable_params",
-]
+    "get_merged_lora_ckpt",
+)

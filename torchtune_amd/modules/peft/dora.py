@@ -19,13 +19,10 @@ from __future__ import annotations
 from typing import List, Optional, Union
 
 import torch
-import torch.nn.functional as F
 from torch import nn
 
 from ... import ops
-from ...nf4_tensor import NF4Tensor, _fused_ok, linear_nf4, to_nf4
-from ..low_precision import _register_nf4_dispatch_ops  # noqa: F401
-from .lora import _lora_a_init_params, _lora_b_init_params
+from ._adapter_base import LowRankAdapterLinear
 
 
 class _QDoRALinearFn(torch.autograd.Function):
@@ -63,7 +60,7 @@ class _QDoRALinearFn(torch.autograd.Function):
         return gx, None, (ga if need_a else None), (gb if need_b else None), (gmag if need_m else None), gbias, None
 
 
-class DoRALinear(nn.Module):
+class DoRALinear(LowRankAdapterLinear):
     """DoRA linear layer: ``x -> (m / ||W0 + (alpha / r) B A||) * (W0 x + (alpha / r) B A x)``.
 
     Args:
@@ -80,61 +77,19 @@ class DoRALinear(nn.Module):
         ValueError: If ``quantize_base`` is False, but quantization kwargs are provided.
     """
 
-    def __init__(
-        self,
-        in_dim: int,
-        out_dim: int,
-        rank: int,
-        alpha: float,
-        dropout: float = 0.0,
-        use_bias: bool = False,
-        quantize_base: bool = False,
-        **quantization_kwargs,
-    ):
+    def __init__(self, in_dim: int, out_dim: int, rank: int, alpha: float, dropout: float = 0.0, use_bias: bool = False,
+                 quantize_base: bool = False, **quantization_kwargs):
         super().__init__()
-        self.in_dim = in_dim
-        self.out_dim = out_dim
         self.scaling = alpha / rank
-        self.use_bias = use_bias
-        self._quantize_base = quantize_base
-
-        if not self._quantize_base and any([v for v in quantization_kwargs.values()]):
-            raise ValueError(
-                f"``quantize_base`` is False, but received the following quantization arguments: {quantization_kwargs}"
-            )
-
-        linear = nn.Linear(in_features=in_dim, out_features=out_dim, bias=self.use_bias)
-        weight = linear.weight if not self._quantize_base else to_nf4(linear.weight, **quantization_kwargs)
-        bias = linear.bias if self.use_bias else None
-
-        self.disabled = False  # True: act as the frozen base layer only
-        self.register_parameter("weight", nn.Parameter(weight))
-        self.register_parameter("bias", nn.Parameter(bias) if bias is not None else None)
-        self.dropout = nn.Dropout(p=dropout) if dropout > 0.0 else nn.Identity()
-        self.lora_a = nn.Linear(in_features=in_dim, out_features=rank, bias=False)
-        self.lora_b = nn.Linear(in_features=rank, out_features=out_dim, bias=False)
+        self._build(in_dim, out_dim, rank, dropout, use_bias, quantize_base, quantization_kwargs)
         self.magnitude = nn.Parameter(torch.empty(out_dim))
         self.initialize_parameters()
 
     def to_empty(self, *, device: Optional[Union[str, torch.device, int]], recurse: bool = True):
-        self.lora_a.to_empty(device=device, recurse=recurse)
-        self.lora_b.to_empty(device=device, recurse=recurse)
-        magnitude = nn.Parameter(torch.empty_like(self.magnitude, device=device), requires_grad=self.magnitude.requires_grad)
-        torch.utils.swap_tensors(self.magnitude, magnitude)
+        super().to_empty(device=device, recurse=recurse)
+        fresh = nn.Parameter(torch.empty_like(self.magnitude, device=device), requires_grad=self.magnitude.requires_grad)
+        torch.utils.swap_tensors(self.magnitude, fresh)
         return self
-
-    def initialize_parameters(self):
-        _lora_a_init_params(self.lora_a)
-        _lora_b_init_params(self.lora_b)
-
-    def _nf4_kernels_apply(self, dtype: torch.dtype) -> bool:
-        w = self.weight
-        rank = self.lora_a.weight.shape[0]
-        return (
-            isinstance(w, NF4Tensor) and w.is_cuda and w.dim() == 2 and w.block_size == 64 and w.dtype == torch.bfloat16
-            and dtype == torch.bfloat16 and self.lora_a.weight.dtype == torch.bfloat16
-            and self.lora_b.weight.dtype == torch.bfloat16 and ops.fused_shape_ok(w.shape[0], w.shape[1], rank) and rank > 0
-        )
 
     @torch.no_grad()
     def initialize_dora_magnitude(self):
@@ -144,58 +99,41 @@ class DoRALinear(nn.Module):
         Raises:
             RuntimeError: If base or LoRA parameters are still on meta device.
         """
-        if any([self.weight.is_meta, self.lora_a.weight.is_meta, self.lora_b.weight.is_meta]):
+        if self.weight.is_meta or self.lora_a.weight.is_meta or self.lora_b.weight.is_meta:
             raise RuntimeError("Cannot initialize DoRA magnitude if base or LoRA parameters are still on meta device.")
         if self._nf4_kernels_apply(self.lora_a.weight.dtype):
-            N, K = self.weight.shape
-            norm, _ = ops.nf4_dora_weight_norm(self.weight.quantized_data, self.weight.block_scalers(), N, K,
+            n, k = self.weight.shape
+            norm, _ = ops.nf4_dora_weight_norm(self.weight.quantized_data, self.weight.block_scalers(), n, k,
                                                self.lora_a.weight, self.lora_b.weight, self.scaling)
-            self.magnitude.copy_(norm)
-            return
-        base_weight = self.weight.to(self.lora_a.weight.dtype)
-        lora_weight = self.lora_b.weight @ self.lora_a.weight
-        self.magnitude.copy_(self._get_weight_norm(base_weight, lora_weight))
+        else:
+            norm = self._get_weight_norm(self.weight.to(self.lora_a.weight.dtype), self.lora_b.weight @ self.lora_a.weight)
+        self.magnitude.copy_(norm)
 
     def _get_weight_norm(self, weight, lora_weight):
-        weight = weight + self.scaling * lora_weight
-        return torch.linalg.norm(weight, dim=1).to(weight.dtype)
+        merged = weight + self.scaling * lora_weight
+        return torch.linalg.norm(merged, dim=1).to(merged.dtype)
 
     def adapter_params(self) -> List[str]:
         """Names of this module's adapter parameters: ``lora_a.weight``, ``lora_b.weight`` and ``magnitude``."""
         return ["lora_a.weight", "lora_b.weight", "magnitude"]
 
     def _fused(self, x: torch.Tensor) -> bool:
-        dropping = self.training and isinstance(self.dropout, nn.Dropout) and self.dropout.p > 0.0
-        return (
-            self._quantize_base
-            and not dropping
-            and self._nf4_kernels_apply(x.dtype)
-            and _fused_ok(x, self.weight, self.lora_a.weight.shape[0])
-            and self.magnitude.dtype == torch.bfloat16
-            and self.magnitude.is_cuda
-            and (self.bias is None or self.bias.dtype == torch.bfloat16)
-        )
+        return self._fused_path(x) and self.magnitude.dtype == torch.bfloat16 and self.magnitude.is_cuda
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         """x ``(..., in_dim)`` -> ``(..., out_dim)``"""
         if not self.disabled and self._fused(x):
             return _QDoRALinearFn.apply(x, self.weight, self.lora_a.weight, self.lora_b.weight, self.magnitude, self.bias,
                                         self.scaling)
-        if self._quantize_base:
-            base_out = linear_nf4(input=x, weight=self.weight)
-            if self.use_bias:
-                base_out = base_out + self.bias
-        else:
-            base_out = F.linear(x, self.weight, self.bias)
+        base_out = self._base_out(x)
         if self.disabled:
             return base_out
-
+        # composed path, the reference's op order: the direction B A is read off an identity batch, its row norm is a
+        # constant of the graph
         x = self.dropout(x)
         lora_out = self.lora_b(self.lora_a(x))
-        x_eye = torch.eye(self.lora_a.weight.shape[1], device=self.lora_a.weight.device, dtype=x.dtype)
-        lora_weight = self.lora_b(self.lora_a(x_eye)).T
-        weight = self.weight.to(x.dtype)
-        weight_norm = self._get_weight_norm(weight, lora_weight.detach()).detach()
-        mag_norm_scale = (self.magnitude / weight_norm).view(1, -1)
-        dora_out = (mag_norm_scale - 1) * base_out + mag_norm_scale * lora_out * self.scaling
-        return dora_out + base_out
+        eye = torch.eye(self.in_dim, device=self.lora_a.weight.device, dtype=x.dtype)
+        direction = self.lora_b(self.lora_a(eye)).T.detach()
+        norm = self._get_weight_norm(self.weight.to(x.dtype), direction).detach()
+        c = (self.magnitude / norm).view(1, -1)
+        return (c - 1) * base_out + c * lora_out * self.scaling + base_out

@@ -17,7 +17,6 @@ block sizes, adapter dropout in training) compose the same result from ``linear_
 """
 from __future__ import annotations
 
-import math
 from enum import Enum
 from typing import List, Optional, Union
 
@@ -26,8 +25,7 @@ import torch.nn.functional as F
 from torch import nn
 
 from ... import ops
-from ...nf4_tensor import NF4Tensor, _fused_ok, linear_nf4, to_nf4
-from ..low_precision import _register_nf4_dispatch_ops  # noqa: F401  (clone override must be active)
+from ._adapter_base import LowRankAdapterLinear, _lora_a_init_params, _lora_b_init_params  # noqa: F401
 
 
 class TrainableParams(Enum):
@@ -75,7 +73,7 @@ class _QLoRALinearFn(torch.autograd.Function):
         return gx, None, ga, gb, gbias, None
 
 
-class LoRALinear(nn.Module):
+class LoRALinear(LowRankAdapterLinear):
     """Linear layer with a low-rank adapter: ``x -> W0 x + (alpha / r) B A x``.
 
     Args:
@@ -93,83 +91,31 @@ class LoRALinear(nn.Module):
         ValueError: if quantisation arguments are given while ``quantize_base`` is False
     """
 
-    def __init__(
-        self,
-        in_dim: int,
-        out_dim: int,
-        rank: int,
-        alpha: float,
-        dropout: float = 0.0,
-        use_bias: bool = False,
-        quantize_base: bool = False,
-        **quantization_kwargs,
-    ):
+    def __init__(self, in_dim: int, out_dim: int, rank: int, alpha: float, dropout: float = 0.0, use_bias: bool = False,
+                 quantize_base: bool = False, **quantization_kwargs):
         super().__init__()
-        self.in_dim = in_dim
-        self.out_dim = out_dim
         self.rank = rank
         self.alpha = alpha
-        self.use_bias = use_bias
-        self._quantize_base = quantize_base
-
-        if not quantize_base and any(v for v in quantization_kwargs.values()):
-            raise ValueError(
-                f"``quantize_base`` is False, but received the following quantization arguments: {quantization_kwargs}"
-            )
-
-        base = nn.Linear(in_features=in_dim, out_features=out_dim, bias=use_bias)
-        weight = to_nf4(base.weight, **quantization_kwargs) if quantize_base else base.weight
-        self.disabled = False  # True: act as the frozen base layer only (reference policy in DPO)
-        self.register_parameter("weight", nn.Parameter(weight))
-        self.register_parameter("bias", nn.Parameter(base.bias) if use_bias else None)
-        self.dropout = nn.Dropout(p=dropout) if dropout > 0.0 else nn.Identity()
-        self.lora_a = nn.Linear(in_features=in_dim, out_features=rank, bias=False)
-        self.lora_b = nn.Linear(in_features=rank, out_features=out_dim, bias=False)
+        self._build(in_dim, out_dim, rank, dropout, use_bias, quantize_base, quantization_kwargs)
         self.merged = False
         self.initialize_parameters()
-
-    def to_empty(self, *, device: Optional[Union[str, torch.device, int]], recurse: bool = True):
-        self.lora_a.to_empty(device=device, recurse=recurse)
-        self.lora_b.to_empty(device=device, recurse=recurse)
-
-    def initialize_parameters(self):
-        _lora_a_init_params(self.lora_a)
-        _lora_b_init_params(self.lora_b)
 
     def adapter_params(self) -> List[str]:
         """Names of this module's adapter parameters."""
         return ["lora_a.weight", "lora_b.weight"]
 
     def _fused(self, x: torch.Tensor) -> bool:
-        dropping = self.training and isinstance(self.dropout, nn.Dropout) and self.dropout.p > 0.0
-        return (
-            self._quantize_base
-            and not dropping
-            and self.rank > 0
-            and isinstance(self.weight, NF4Tensor)
-            and _fused_ok(x, self.weight, self.rank)
-            and self.lora_a.weight.dtype == torch.bfloat16
-            and self.lora_b.weight.dtype == torch.bfloat16
-            and (self.bias is None or self.bias.dtype == torch.bfloat16)
-        )
+        return self._fused_path(x)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         """x ``(..., in_dim)`` -> ``(..., out_dim)``"""
+        scale = self.alpha / self.rank
         if not self.disabled and self._fused(x):
-            return _QLoRALinearFn.apply(
-                x, self.weight, self.lora_a.weight, self.lora_b.weight, self.bias, self.alpha / self.rank
-            )
-        if self._quantize_base:
-            out = linear_nf4(input=x, weight=self.weight)
-            if self.use_bias:
-                out = out + self.bias
-        else:
-            out = F.linear(x, self.weight, self.bias)
+            return _QLoRALinearFn.apply(x, self.weight, self.lora_a.weight, self.lora_b.weight, self.bias, scale)
+        out = self._base_out(x)
         if self.disabled:
             return out
-        lora_out = self.lora_a(self.dropout(x))
-        lora_out = (self.alpha / self.rank) * self.lora_b(lora_out)
-        return out + lora_out
+        return out + scale * self.lora_b(self.lora_a(self.dropout(x)))
 
 
 class QATLoRALinear(LoRALinear):
@@ -247,13 +193,3 @@ class QATLoRALinear(LoRALinear):
         if lora_linear.lora_b.weight.device != meta:
             new.lora_b.weight = lora_linear.lora_b.weight
         return new
-
-
-def _lora_a_init_params(x: nn.Linear) -> None:
-    """Kaiming-uniform, a = sqrt(5)."""
-    nn.init.kaiming_uniform_(x.weight, a=math.sqrt(5))
-
-
-def _lora_b_init_params(x: nn.Linear) -> None:
-    """Zeros: the adapter starts as a no-op."""
-    nn.init.zeros_(x.weight)
