@@ -84,7 +84,7 @@ __global__ __launch_bounds__(256) void skinny_nt_kernel(const uint16_t* __restri
     for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int hh = 0; hh < 2; ++hh)
-        xa[t][hh] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(xrow[t] + k0 + 8 * hh));
+        xa[t][hh] = *reinterpret_cast<const u32x4_t*>(xrow[t] + k0 + 8 * hh);
 #pragma unroll
     for (int u = 0; u < RT; ++u)
 #pragma unroll
@@ -193,7 +193,7 @@ __global__ __launch_bounds__(256) void skinny_tn_kernel(const uint16_t* __restri
       const bool ok = row < m_end;
       xv[u] = u32x4_t{0, 0, 0, 0};
       gv[u] = 0;
-      if (ok && col_ok) xv[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(xp + (int64_t)row * Kc));
+      if (ok && col_ok) xv[u] = *reinterpret_cast<const u32x4_t*>(xp + (int64_t)row * Kc);
       if (ok && r_ok) gv[u] = gp[(int64_t)row * R];
     }
 #pragma unroll
@@ -243,7 +243,8 @@ __global__ __launch_bounds__(256) void sum_partials_tn_kernel(const float* __res
   out[r * stride_r + k * stride_k] = f32_to_bf16_bits(s * scale);
 }
 
-constexpr int kTargetWaves = 4096;
+constexpr int kTargetWaves = 4096;    // row contractions (skinny_tn)
+constexpr int kTargetWavesNt = 2048;  // column contractions (skinny_nt): fewer, longer waves measured faster
 
 struct NtPlan {
   int m_tiles, splits, chunks_per_split;
@@ -252,7 +253,7 @@ NtPlan plan_nt(int64_t M, int64_t Kc) {
   NtPlan p;
   p.m_tiles = (int)((M + 31) / 32);
   const int total_chunks = (int)(Kc / 64);
-  int s = kTargetWaves / 4 / p.m_tiles;  // workgroups of 4 waves
+  int s = kTargetWavesNt / 4 / p.m_tiles;  // workgroups of 4 waves
   s = s < 1 ? 1 : s;
   const int max_s = (total_chunks + 7) / 8;  // at least two chunks per wave
   s = s > max_s ? max_s : s;

@@ -54,7 +54,7 @@ __global__ __launch_bounds__(256) void rms_norm_fwd_kernel(const uint16_t* __res
   for (int i = 0; i < NV; ++i) {
     const int c = lane + 64 * i;
     v[i] = u32x4_t{0, 0, 0, 0};
-    if (c < chunks) v[i] = __builtin_nontemporal_load(xr + c);
+    if (c < chunks) v[i] = *(xr + c);
 #pragma unroll
     for (int d = 0; d < 4; ++d) {
       const float a = lo_f(v[i][d]), b = hi_f(v[i][d]);
@@ -111,8 +111,8 @@ __global__ __launch_bounds__(256) void rms_norm_bwd_kernel(const uint16_t* __res
       xv[i] = u32x4_t{0, 0, 0, 0};
       gv[i] = u32x4_t{0, 0, 0, 0};
       if (c < chunks) {
-        xv[i] = __builtin_nontemporal_load(xr + c);
-        const u32x4_t go = __builtin_nontemporal_load(gr + c);
+        xv[i] = *(xr + c);
+        const u32x4_t go = *(gr + c);
         const u32x4_t s = sr[c];
 #pragma unroll
         for (int d = 0; d < 4; ++d) {
@@ -192,7 +192,7 @@ __global__ __launch_bounds__(256) void rope_kernel(const uint16_t* __restrict__ 
   const int64_t e = chunk * 8;
   const int pos = (int)((e / row_elems) % S);
   const int d = (int)(e % h_d);  // even; h_d % 8 == 0 keeps the 4 pairs inside one head
-  const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(x) + chunk);
+  const u32x4_t v = *(reinterpret_cast<const u32x4_t*>(x) + chunk);
   const f32x4_t* cp = reinterpret_cast<const f32x4_t*>(cache + ((int64_t)pos * (h_d >> 1) + (d >> 1)) * 2);
   const f32x4_t c01 = cp[0], c23 = cp[1];
   const float cs[4] = {c01.x, c01.z, c23.x, c23.z};
