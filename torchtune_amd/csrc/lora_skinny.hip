@@ -37,7 +37,9 @@ typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 template <int RT>
 __global__ __launch_bounds__(256) void skinny_nt_kernel(const uint16_t* __restrict__ X, const uint16_t* __restrict__ Bm,
                                                         float* __restrict__ part, int M, int Kc, int R,
-                                                        int chunks_per_split) {
+                                                        int chunks_per_split, uint16_t* __restrict__ direct_out,
+                                                        float scale) {
+  // direct_out != null (only with a single split): write bf16(scale * sum) straight to the [M, R] output
   __shared__ float red[3][2 * RT * 4][64];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -122,7 +124,12 @@ __global__ __launch_bounds__(256) void skinny_nt_kernel(const uint16_t* __restri
         for (int v = 0; v < 4; ++v) {
           const int r = m0 + 16 * t + 4 * g + v;
           const int e = (t * RT + u) * 4 + v;
-          if (r < M) part[((int64_t)split * M + r) * R + col] = ((acc[t][u][v] + red[0][e][lane]) + red[1][e][lane]) + red[2][e][lane];
+          if (r >= M) continue;
+          const float sum = ((acc[t][u][v] + red[0][e][lane]) + red[1][e][lane]) + red[2][e][lane];
+          if (direct_out)
+            direct_out[(int64_t)r * R + col] = f32_to_bf16_bits(sum * scale);
+          else
+            part[((int64_t)split * M + r) * R + col] = sum;
         }
       }
   }
@@ -244,7 +251,7 @@ __global__ __launch_bounds__(256) void sum_partials_tn_kernel(const float* __res
 }
 
 constexpr int kTargetWaves = 4096;    // row contractions (skinny_tn)
-constexpr int kTargetWavesNt = 2048;  // column contractions (skinny_nt): fewer, longer waves measured faster
+constexpr int kTargetWavesNt = 1024;  // column contractions (skinny_nt): few, long waves; one split needs no second pass
 
 struct NtPlan {
   int m_tiles, splits, chunks_per_split;
@@ -285,14 +292,17 @@ int run_nt(const uint16_t* X, const uint16_t* Bm, int64_t M, int64_t Kc, int R, 
            hipStream_t s) {
   const NtPlan p = plan_nt(M, Kc);
   const dim3 grid((unsigned)p.m_tiles, (unsigned)p.splits), block(256);
+  uint16_t* direct = p.splits == 1 ? out : nullptr;
   if (R <= 16)
-    skinny_nt_kernel<1><<<grid, block, 0, s>>>(X, Bm, ws, (int)M, (int)Kc, R, p.chunks_per_split);
+    skinny_nt_kernel<1><<<grid, block, 0, s>>>(X, Bm, ws, (int)M, (int)Kc, R, p.chunks_per_split, direct, scale);
   else if (R <= 32)
-    skinny_nt_kernel<2><<<grid, block, 0, s>>>(X, Bm, ws, (int)M, (int)Kc, R, p.chunks_per_split);
+    skinny_nt_kernel<2><<<grid, block, 0, s>>>(X, Bm, ws, (int)M, (int)Kc, R, p.chunks_per_split, direct, scale);
   else
-    skinny_nt_kernel<4><<<grid, block, 0, s>>>(X, Bm, ws, (int)M, (int)Kc, R, p.chunks_per_split);
-  const int64_t n = M * R;
-  sum_partials_kernel<<<dim3((unsigned)((n + 255) / 256)), block, 0, s>>>(ws, n, p.splits, scale, out);
+    skinny_nt_kernel<4><<<grid, block, 0, s>>>(X, Bm, ws, (int)M, (int)Kc, R, p.chunks_per_split, direct, scale);
+  if (!direct) {
+    const int64_t n = M * R;
+    sum_partials_kernel<<<dim3((unsigned)((n + 255) / 256)), block, 0, s>>>(ws, n, p.splits, scale, out);
+  }
   return check_launch("skinny_nt");
 }
 
