@@ -201,7 +201,47 @@ def secondary_kernels(dev) -> dict:
     x = torch.randn(8192, 14336, device=dev, generator=gen).to(torch.bfloat16)
     out["fq_per_token_int8_asym 8192x14336 bf16"] = round(
         x.numel() * 4 / timed(lambda: ops.fq_per_token_int8_asym(x, want_qparams=False)) / 1e9, 1)
+    host = torch.empty(14336, 4096, dtype=torch.bfloat16, pin_memory=True)
+    out["checkpoint offload: nf4_dequantize 14336x4096 written into pinned host memory (PCIe-bound, host bytes only)"] = round(
+        n * 2 / timed(lambda: t.get_original_weight(out=host), iters=5) / 1e9, 1)
     return {"unit": "GB/s (algorithmic bytes / HIP-event time, HBM peak 8000)", **out}
+
+
+def optimizer_leg(model, tokens, labels, train_step, qat: bool, steps: int, tokens_per_step: int):
+    """fwd + bwd + optimizer step, with the optimizer of the reference's configs: ``torch.optim.AdamW(fused=True)``,
+    lr 3e-4 / weight decay 0.01 for QLoRA (``recipes/configs/llama3_1/8B_qlora_single_device.yaml:60-64``), lr 2e-5
+    for QAT (``recipes/configs/llama3_1/8B_qat_full.yaml:66-69``).  The reference's own ``tokens_per_second_per_gpu``
+    includes the optimizer (``recipes/lora_finetune_single_device.py:666-671``); the headline metric does not."""
+    if steps <= 0:
+        return None
+    params = [p for p in model.parameters() if p.requires_grad]
+    opt = (torch.optim.AdamW(params, lr=2e-5, fused=True) if qat
+           else torch.optim.AdamW(params, lr=3e-4, weight_decay=0.01, fused=True))
+
+    def opt_step():
+        loss = train_step(model, tokens, labels)
+        opt.step()
+        opt.zero_grad(set_to_none=True)
+        return loss
+
+    opt_step()  # allocates the optimizer state
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        loss = opt_step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    out = {
+        "value": round(tokens_per_step * steps / dt, 1),
+        "unit": "tokens/s",
+        "ms_per_step": round(1e3 * dt / steps, 2),
+        "steps": steps,
+        "optimizer": "torch.optim.AdamW(fused=True) over %d tensors / %.1f M trainable parameters" % (
+            len(params), sum(p.numel() for p in params) / 1e6),
+        "loss_after": float(loss),
+    }
+    del opt
+    return out
 
 
 def main() -> int:
@@ -212,6 +252,9 @@ def main() -> int:
     ap.add_argument("--workload", default="llama3_1_8b", choices=sorted(WORKLOADS))
     ap.add_argument("--cpu-tokens", type=int, default=512,
                     help="starting token count of the CPU-baseline sample, grown until it takes >= 10 s (0 = skip)")
+    ap.add_argument("--optimizer-steps", type=int, default=3,
+                    help="after the timed fwd+bwd steps, time this many steps that also run the recipe's fused AdamW "
+                         "(reported beside the metric as `with_adamw`; 0 = skip)")
     ap.add_argument("--calibration-copy-mib", type=int, default=0,
                     help="before the steps, run one elementwise kernel that reads and writes this many MiB: the known-size "
                          "dispatch that FETCH_SIZE / WRITE_SIZE counter runs are scaled by")
@@ -267,6 +310,7 @@ def main() -> int:
     ops.set_gemm_timer(None)
     ops.set_fq_timer(None)
     ms_per_step = 1e3 * dt / args.steps
+    with_adamw = optimizer_leg(model, tokens, labels, train_step, qat, args.optimizer_steps, batch * seq)
 
     if qat:
         fq = fq_timer.summary()
@@ -307,6 +351,7 @@ def main() -> int:
                 "per_kernel": {k: {kk: vv for kk, vv in v.items() if kk in ("launches", "avg_us", "gbps")} for k, v in fq.items()},
             },
         }
+        result["with_adamw"] = with_adamw
         del model
         torch.cuda.empty_cache()
         if args.cpu_tokens > 0:
@@ -353,6 +398,7 @@ def main() -> int:
             "per_shape": per_shape,
         },
     }
+    result["with_adamw"] = with_adamw
     del model
     torch.cuda.empty_cache()
     result["hbm_bound_kernels"] = secondary_kernels(dev)

@@ -106,6 +106,32 @@ def test_quantized_state_dict(dtype):
     assert sd_cpu["weight"].device.type == "cpu" and torch.equal(sd_cpu["weight"], sd["weight"].cpu())
 
 
+@pytest.mark.parametrize("pinned", [True, False])
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+def test_state_dict_offload_writes_host_memory_directly(pinned, out_dtype, monkeypatch):
+    """`offload_to_cpu=True` (the default of torchtune/modules/common_utils.py:24-59): the dense weight must equal
+    the on-device dequantisation bit for bit whether it lands in pinned memory or goes through the staging buffer."""
+    from torchtune_amd.modules import common_utils
+
+    monkeypatch.setattr(common_utils, "PINNED_OFFLOAD", pinned)
+    w = to_nf4((torch.randn(768, 1024, device=DEV) * 0.02).to(torch.bfloat16))
+    other = torch.ones(3, device=DEV)
+    expect = w.get_original_weight().to(out_dtype).cpu()
+    for _ in range(2):  # the second pass reuses the staging buffer
+        sd = {"weight": w, "other": other}
+        reparametrize_as_dtype_state_dict_post_hook(None, sd, dtype=out_dtype, offload_to_cpu=True)
+        got = sd["weight"]
+        assert got.device.type == "cpu" and got.dtype == out_dtype and got.shape == (768, 1024)
+        assert got.is_pinned() == pinned
+        assert torch.equal(got, expect)
+        assert sd["other"] is other
+    # the kernel refuses host memory it cannot reach
+    with pytest.raises(ValueError, match="pinned host memory"):
+        w.get_original_weight(out=torch.empty(768, 1024, dtype=torch.bfloat16))
+    with pytest.raises(ValueError, match="contiguous"):
+        w.get_original_weight(out=torch.empty(768, 512, dtype=torch.bfloat16, device=DEV))
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 def test_frozen_nf4_linear(dtype):
     # tests/torchtune/modules/low_precision/test_nf4_linear.py:24-70

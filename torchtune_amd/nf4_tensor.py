@@ -185,13 +185,18 @@ class NF4Tensor(torch.Tensor):
 
     # ---- dequantisation ----------------------------------------------------------------------------
     @torch.no_grad()
-    def get_original_weight(self) -> torch.Tensor:
-        """The dequantised weight in the original dtype and shape."""
+    def get_original_weight(self, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """The dequantised weight in the original dtype and shape.  With ``out`` (same dtype and element count, on
+        the weight's GPU or in pinned host memory) the kernel stores into it directly; for host memory the caller
+        synchronises the current stream before reading the values."""
         home = self.quantized_data.device
         dev = _compute_device(self.quantized_data)
         parts = [self.quantized_data, self.quantized_scalers, self.quantization_factor, self.scaler_mean]
         if home != dev:
             parts = [t.to(dev) for t in parts]
+        if out is not None:
+            ops.nf4_dequantize(*parts, self.shape, self.block_size, self.scaler_block_size, out=out)
+            return out
         out = ops.nf4_dequantize(*parts, self.shape, self.block_size, self.scaler_block_size)
         return out if home == dev else out.to(home)
 

@@ -77,13 +77,23 @@ def nf4_quantize(w: torch.Tensor, block_size: int, scaler_block_size: int):
 
 def nf4_dequantize(
     qdata: torch.Tensor, qscalers: torch.Tensor, qfactor: torch.Tensor, mean: torch.Tensor, shape, block_size: int,
-    scaler_block_size: int,
+    scaler_block_size: int, out: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
+    """Dense weight of an NF4 tensor.  ``out`` may be a contiguous tensor on the same GPU or in pinned host memory;
+    the kernel then stores straight into it (over PCIe for host memory: the caller synchronises the stream before
+    reading it on the CPU)."""
     _need_gpu(qdata, "nf4_dequantize")
     dtype = qfactor.dtype
     code = _code(dtype, "nf4_dequantize")
     numel = qdata.numel() * 2
-    out = torch.empty(numel, dtype=dtype, device=qdata.device)
+    if out is None:
+        out = torch.empty(numel, dtype=dtype, device=qdata.device)
+    else:
+        on_device = out.is_cuda and out.device == qdata.device
+        if not (on_device or (out.device.type == "cpu" and out.is_pinned())):
+            raise ValueError("nf4_dequantize: `out` must live on the weight's GPU or in pinned host memory")
+        if out.dtype != dtype or out.numel() != numel or not out.is_contiguous():
+            raise ValueError(f"nf4_dequantize: `out` must be a contiguous {dtype} tensor of {numel} elements")
     lib = _lib.load()
     with torch.cuda.device(qdata.device):
         rc = lib.ttamd_nf4_dequantize(
