@@ -102,3 +102,36 @@ def test_raw_c_abi_validation():
     assert lib.ttamd_dora_bwd_prologue_bf16(p, p, p, p, p, p, 8, 12, p, 1 << 20, None) == -1
     assert lib.ttamd_nf4_dora_linear_fwd_bf16(p, p, p, None, None, None, 0, 0.0, None, None, p, 8, 64, 64, None) == -1
     assert b"col_scale" in lib.ttamd_last_error()
+
+
+@pytest.mark.parametrize("with_hook", [False, True])
+def test_merged_dora_checkpoint_reproduces_the_layer(with_hook):
+    """get_merged_lora_ckpt with a magnitude entry (torchtune/modules/peft/_utils.py:245-263): the merged dense
+    weight, used as a plain linear, gives the DoRA layer's output; the NF4 weight goes through the one-pass
+    dequantise + merge kernel (`with_hook=False`) or arrives already dense on the CPU (`with_hook=True`)."""
+    from torchtune_amd.modules.common_utils import reparametrize_as_dtype_state_dict_post_hook
+    from torchtune_amd.modules.peft import get_merged_lora_ckpt
+
+    K, N, r, alpha = 1024, 768, 16, 32.0
+    layer, parts, A, B, _ = _layer(K, N, r, alpha, False, seed=5)
+    layer.initialize_dora_magnitude()
+    with torch.no_grad():
+        layer.magnitude.mul_(torch.linspace(0.5, 1.5, N, device=DEV).to(BF))
+    sd = {"l." + k: v.detach() for k, v in layer.state_dict().items()}
+    if with_hook:
+        reparametrize_as_dtype_state_dict_post_hook(layer, sd, dtype=BF, offload_to_cpu=True)
+        assert sd["l.weight"].device.type == "cpu"
+        sd = {k: v.cpu() for k, v in sd.items()}
+    out = get_merged_lora_ckpt(sd, rank=r, alpha=alpha)
+    assert out.keys() == {"l.weight"}
+    merged = out["l.weight"]
+    assert merged.dtype == BF and merged.shape == (N, K)
+    # closed form in fp32 from the oracle's dequantised weight
+    Wd = nf4_oracle.nf4_dequantize(parts).float()
+    full = Wd + (alpha / r) * (B.float() @ A.float())
+    want = full * (layer.magnitude.detach().float().cpu() / full.norm(dim=1)).view(-1, 1)
+    torch.testing.assert_close(merged.float().cpu(), want, rtol=2e-2, atol=2e-3)
+    x = (torch.randn(64, K, generator=torch.Generator().manual_seed(6))).to(BF).to(DEV)
+    y_layer = layer(x)
+    y_merged = torch.nn.functional.linear(x, merged.to(DEV))
+    torch.testing.assert_close(y_merged.float(), y_layer.float(), rtol=2e-2, atol=3e-2)

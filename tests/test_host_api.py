@@ -315,6 +315,18 @@ def test_reference_known_answer_merged_lora_ckpt():
     out = get_merged_lora_ckpt(sd, rank=kat["rank"], alpha=kat["alpha"])
     assert out is sd and out.keys() == {"0.weight", "1.weight", "1.bias"}
     torch.testing.assert_close(out["0.weight"], torch.tensor(kat["expected_merged_weight"]), atol=kat["atol"], rtol=kat["rtol"])
+    # the DoRA variant of the same test (test_utils.py:435-447,459-468): the magnitude is folded in and deleted
+    sd = {
+        "0.weight": 3 * torch.ones(6, 4),
+        "0.lora_a.weight": torch.tensor(kat["lora_a"], dtype=torch.float32),
+        "0.lora_b.weight": torch.tensor(kat["lora_b"], dtype=torch.float32),
+        "0.magnitude": torch.tensor(kat["magnitude"], dtype=torch.float32),
+        "1.weight": torch.zeros(3, 6),
+        "1.bias": torch.zeros(3),
+    }
+    out = get_merged_lora_ckpt(sd, rank=kat["rank"], alpha=kat["alpha"])
+    assert out is sd and out.keys() == {"0.weight", "1.weight", "1.bias"}
+    torch.testing.assert_close(out["0.weight"], torch.tensor(kat["expected_merged_dora_weight"]), atol=kat["atol"], rtol=kat["rtol"])
     with pytest.raises(NotImplementedError):
-        get_merged_lora_ckpt({"m.weight": torch.ones(2, 2), "m.lora_a.weight": torch.ones(1, 2), "m.lora_b.weight": torch.ones(2, 1),
-                              "m.magnitude": torch.ones(2)}, rank=1, alpha=1.0)
+        get_merged_lora_ckpt({"m.experts.weight": torch.ones(2, 2), "m.experts.lora_a.weight": torch.ones(1, 2),
+                              "m.experts.lora_b.weight": torch.ones(2, 1)}, rank=1, alpha=1.0)

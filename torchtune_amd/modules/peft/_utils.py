@@ -48,32 +48,40 @@ def _get_lora_modules(state_dict: Dict[str, Any]) -> Set[str]:
 
 @torch.no_grad()
 def get_merged_lora_ckpt(state_dict: Dict[str, Any], rank: int, alpha: float) -> Dict[str, Any]:
-    """Fold every LoRA pair of ``state_dict`` into its base weight, ``W += (alpha / rank) * B @ A``, and delete the
-    adapter entries; modifies and returns ``state_dict`` (``torchtune/modules/peft/_utils.py:193-271``, vanilla
-    LoRA branch; DoRA magnitudes and MoE experts raise).
+    """Fold every LoRA pair of ``state_dict`` into its base weight and delete the adapter entries; modifies and
+    returns ``state_dict`` (``torchtune/modules/peft/_utils.py:193-271``; MoE experts raise).
+
+    Plain LoRA: ``W += (alpha / rank) * B @ A``.  With a DoRA ``magnitude`` entry the merged weight is
+    ``(W + (alpha / rank) * B @ A) * (magnitude / ||W + (alpha / rank) * B @ A||_row)`` and the magnitude is deleted too.
 
     A base weight that is still an ``NF4Tensor`` on the GPU (a state dict taken without the dequantising hook) is
-    dequantised and merged in one pass by the HIP kernel; a dense weight is updated in place as the reference does.
+    dequantised and merged in one pass by the HIP kernel; a dense weight is updated as the reference does.
     """
+    scale = alpha / rank
     for module in sorted(_get_lora_modules(state_dict)):
-        if f"{module}.magnitude" in state_dict or "experts" in module:
-            raise NotImplementedError(f"{module}: merging DoRA magnitudes / MoE experts is not part of this build")
+        if "experts" in module:
+            raise NotImplementedError(f"{module}: merging MoE experts is not part of this build")
         a = state_dict[f"{module}.lora_a.weight"]
         b = state_dict[f"{module}.lora_b.weight"]
         w = state_dict[f"{module}.weight"]
-        if (
+        magnitude = state_dict.get(f"{module}.magnitude", None)
+        fused = (
             isinstance(w, NF4Tensor) and w.is_cuda and w.block_size == 64 and w.dtype == torch.bfloat16
             and a.dtype == torch.bfloat16 and b.dtype == torch.bfloat16 and a.shape[0] % 8 == 0 and 0 < a.shape[0] <= 64
-        ):
+        )
+        if fused:
             N, K = w.shape
-            state_dict[f"{module}.weight"] = ops.nf4_dequantize_merge(
-                w.quantized_data, w.block_scalers(), N, K, a.to(w.device), b.to(w.device), alpha / rank
-            )
+            merged = ops.nf4_dequantize_merge(w.quantized_data, w.block_scalers(), N, K, a.to(w.device), b.to(w.device), scale)
+        elif magnitude is not None or isinstance(w, NF4Tensor):
+            merged = w.to(a.dtype) + scale * b @ a
         else:
-            if isinstance(w, NF4Tensor):
-                w = w.to(a.dtype)
-                state_dict[f"{module}.weight"] = w
-            w += (alpha / rank) * b @ a
+            w += scale * b @ a
+            merged = w
+        if magnitude is not None:
+            weight_norm = torch.linalg.norm(merged, dim=1)
+            merged *= (magnitude.to(merged.device) / weight_norm).view(-1, 1)
+            del state_dict[f"{module}.magnitude"]
+        state_dict[f"{module}.weight"] = merged
         del state_dict[f"{module}.lora_a.weight"]
         del state_dict[f"{module}.lora_b.weight"]
     return state_dict
