@@ -198,6 +198,8 @@ def secondary_kernels(dev) -> dict:
     out["nf4_quantize 14336x4096 bf16"] = round(n * 2.515747 / timed(lambda: ops.nf4_quantize(W, 64, 256)) / 1e9, 1)
     out["fq_per_group_int4_sym g32 14336x4096 bf16"] = round(
         (n * 4 + n / 32 * 4) / timed(lambda: ops.fq_per_group_int4_sym(W, 32)) / 1e9, 1)
+    out["fq_per_group_uint4_asym g256 14336x4096 bf16 (4w-qat)"] = round(
+        (n * 4 + n / 256 * 8) / timed(lambda: ops.fq_per_group_uint4_asym(W, 256, want_qparams=True)) / 1e9, 1)
     x = torch.randn(8192, 14336, device=dev, generator=gen).to(torch.bfloat16)
     out["fq_per_token_int8_asym 8192x14336 bf16"] = round(
         x.numel() * 4 / timed(lambda: ops.fq_per_token_int8_asym(x, want_qparams=False)) / 1e9, 1)

@@ -252,6 +252,33 @@ int ttamd_quantize_per_group_int4(const void* w, int dtype, int64_t rows, int64_
 int ttamd_dequantize_per_group_int4(const int8_t* q, const float* scale, const float* zero_point, int dtype, int64_t rows,
                                     int64_t K, int group_size, void* out, void* stream);
 
+/*
+ * The weight-only "4w-qat" mode (Int4WeightOnlyQATQuantizer, re-exported and mapped to "4w-qat" at
+ * torchtune/training/quantization.py:27,125-127): FakeQuantizer.forward for
+ * FakeQuantizeConfig(torch.uint4, group_size=g, is_symmetric=False, zero_point_domain=FLOAT) — torchao.
+ *
+ * Per group: scale = clamp((max - min) / 15, 1e-6), zero_point = min + 8 * scale (a float), both rounded to
+ * `qparam_dtype` (TTAMD_BF16 / TTAMD_F32); q = clamp(round((w - (zero_point - 8 * scale)) / scale), 0, 15);
+ * out = (q - 8) * scale + zero_point.  Every operation is rounded to `dtype` like the eager sequence.
+ * w, out [rows,K] `dtype`; scale / zero_point out [rows, K/group_size] fp32, may be NULL.
+ */
+int ttamd_fq_per_group_uint4_asym(const void* w, int dtype, int64_t rows, int64_t K, int group_size, int qparam_dtype,
+                                  void* out, float* scale, float* zero_point, void* stream);
+
+/*
+ * Int4WeightOnlyQATQuantizer.convert (same quantizer; recipes/quantize.py:92): the codes of the scheme above packed
+ * two per byte, even element in the high nibble: q out [rows, K/2] uint8; scale, zero_point out [rows, K/group_size] fp32.
+ */
+int ttamd_quantize_per_group_uint4(const void* w, int dtype, int64_t rows, int64_t K, int group_size, int qparam_dtype,
+                                   uint8_t* q, float* scale, float* zero_point, void* stream);
+
+/*
+ * Dense weight of the converted weight-only int4 linear: out = dtype((q - 8) * scale + zero_point), each operation
+ * rounded to `dtype`.  q [rows, K/2] uint8 as written by ttamd_quantize_per_group_uint4.
+ */
+int ttamd_dequantize_per_group_uint4(const uint8_t* q, const float* scale, const float* zero_point, int dtype, int64_t rows,
+                                     int64_t K, int group_size, void* out, void* stream);
+
 /* ------------------------------------------------------------------------------------------------
  * Neighbours of the quantized linears inside a decoder layer (one pass over HBM each, bf16 tensors, fp32 math).
  * Floating-point kernels: results agree with the eager sequences to a tolerance (summation order and hardware

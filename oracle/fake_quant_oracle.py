@@ -15,6 +15,10 @@ Eager-PyTorch restatement of what the reference runs through ``torchao.quantizat
   straight-through estimator in backward; the prose description is at
   ``docs/source/tutorials/qat_finetune.rst:40-50``.
 
+* ``fq_per_group_uint4_asym`` / ``quantize_per_group_uint4`` / ``dequantize_per_group_uint4`` <- the weight-only
+  ``Int4WeightOnlyQATQuantizer`` (``torchtune/training/quantization.py:27,125-127``, mode ``"4w-qat"``): group-wise
+  asymmetric uint4 with a floating-point zero point, qparams in bf16.
+
 Parity status: PARITY UNPINNED against torchao itself (not importable here; the reference holds no vectors
 for these functions).  Pinned instead by closed forms and invariants in tests/test_oracle_fake_quant.py
 (scale = (max-min)/255 and the zero-point formula on hand-built rows, outputs on the scale*(q-zp) grid,
@@ -97,6 +101,59 @@ def quantize_per_group_int4(w: torch.Tensor, group_size: int):
     wg = w.view(rows, K // group_size, group_size)
     q = torch.clamp(torch.round(wg * (1.0 / scale[..., None])), -8, 7).to(torch.int8)
     return q.reshape(rows, K), scale, torch.zeros_like(scale)
+
+
+# ---- weight-only int4 ("4w-qat": asymmetric uint4 with a floating-point zero point) --------------------------
+def choose_qparams_per_group_uint4_asym(w: torch.Tensor, group_size: int, qparam_dtype: torch.dtype = torch.bfloat16):
+    """Group-wise affine qparams of the weight-only int4 scheme, computed op by op in the dtype of ``w`` (the
+    eager sequence rounds after every operation) and then cast to ``qparam_dtype``:
+    ``scale = clamp((max - min) / 15, 1e-6)``, ``zero_point = min + scale * 8``.  The group extrema are NOT widened
+    to include 0.  -> (scale, zero_point), each [rows, K/g] in ``qparam_dtype``."""
+    rows, K = w.shape
+    g = w.view(rows, K // group_size, group_size)
+    mn = torch.amin(g, dim=-1)
+    mx = torch.amax(g, dim=-1)
+    scale = (mx - mn) / 15.0
+    scale = torch.clamp(scale, min=1e-6)
+    zero = mn + scale * 8.0
+    return scale.to(qparam_dtype), zero.to(qparam_dtype)
+
+
+def _uint4_codes(w: torch.Tensor, scale: torch.Tensor, zero: torch.Tensor, group_size: int) -> torch.Tensor:
+    rows, K = w.shape
+    g = w.view(rows, K // group_size, group_size)
+    sc = scale.to(w.dtype)[..., None]
+    zp = zero.to(w.dtype)[..., None]
+    lowest = zp - sc * 8.0
+    return torch.clamp(torch.round((g - lowest) / sc), 0, 15)
+
+
+def fq_per_group_uint4_asym(w: torch.Tensor, group_size: int, qparam_dtype: torch.dtype = torch.bfloat16):
+    """returns (fake-quantised w, scale [rows, K/g], zero_point [rows, K/g]) — qparams in ``qparam_dtype``."""
+    rows, K = w.shape
+    scale, zero = choose_qparams_per_group_uint4_asym(w, group_size, qparam_dtype)
+    q = _uint4_codes(w, scale, zero, group_size)
+    dq = (q - 8.0) * scale.to(w.dtype)[..., None]
+    dq = dq + zero.to(w.dtype)[..., None]
+    return dq.reshape(rows, K), scale, zero
+
+
+def quantize_per_group_uint4(w: torch.Tensor, group_size: int, qparam_dtype: torch.dtype = torch.bfloat16):
+    """convert() of the weight-only scheme: (uint8 [rows, K/2], even element in the high nibble; scale; zero_point)."""
+    rows, K = w.shape
+    scale, zero = choose_qparams_per_group_uint4_asym(w, group_size, qparam_dtype)
+    q = _uint4_codes(w, scale, zero, group_size).reshape(rows, K).to(torch.uint8)
+    return (q[:, ::2] << 4) | q[:, 1::2], scale, zero
+
+
+def dequantize_per_group_uint4(packed: torch.Tensor, scale: torch.Tensor, zero: torch.Tensor, group_size: int,
+                               dtype: torch.dtype) -> torch.Tensor:
+    rows, half = packed.shape
+    q = torch.stack([packed >> 4, packed & 15], dim=-1).reshape(rows, half * 2).to(dtype)
+    g = q.view(rows, -1, group_size)
+    dq = (g - 8.0) * scale.to(dtype)[..., None]
+    dq = dq + zero.to(dtype)[..., None]
+    return dq.reshape(rows, half * 2)
 
 
 class _STE(torch.autograd.Function):

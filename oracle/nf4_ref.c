@@ -13,6 +13,8 @@
  *   ref_fq_per_token     FakeQuantizer, int8 per-token asymmetric  (torchao; torchtune/modules/peft/lora.py:232,258)
  *   ref_fq_per_group     FakeQuantizer, int4 per-group symmetric   (torchao; torchtune/modules/peft/lora.py:245,259)
  *   ref_quantize_per_group  convert() to real int4 values       (torchao; recipes/quantize.py:92)
+ *   ref_fq_per_group_uint4_asym  FakeQuantizer / convert of the weight-only "4w-qat" scheme
+ *                        (torchao Int4WeightOnlyQATQuantizer; torchtune/training/quantization.py:27,125-127)
  *
  * Parity status: bit-level agreement with torchao is PARITY UNPINNED (torchao is not available and the
  * reference's tests hold no vectors for these functions); the restatement is pinned by the checks listed in
@@ -219,6 +221,47 @@ void ref_fq_per_group(const void* w, int is_bf16, int64_t rows, int64_t K, int g
       }
       if (scale_out) scale_out[r * (K / g) + k0 / g] = scale;
     }
+}
+
+/* per-group asymmetric uint4 with a floating-point zero point (the weight-only "4w-qat" scheme), every operation
+ * rounded to the tensor dtype, qparams additionally to bf16 when qp_bf16; fq_out, q_out (one code per byte),
+ * scale_out, zero_out may each be NULL */
+void ref_fq_per_group_uint4_asym(const void* w, int is_bf16, int qp_bf16, int64_t rows, int64_t K, int g, void* fq_out,
+                                 uint8_t* q_out, float* scale_out, float* zero_out) {
+#define RND(v) (is_bf16 ? to_bf16(v) : (v))
+  for (int64_t r = 0; r < rows; ++r)
+    for (int64_t k0 = 0; k0 < K; k0 += g) {
+      float mn = load_elem(w, r * K + k0, is_bf16), mx = mn;
+      for (int i = 1; i < g; ++i) {
+        const float v = load_elem(w, r * K + k0 + i, is_bf16);
+        if (v < mn) mn = v;
+        if (v > mx) mx = v;
+      }
+      float range = RND(mx - mn);
+      float scale = RND(range / 15.0f);
+      if (scale < 1e-6f) scale = RND(1e-6f);
+      float eight = RND(scale * 8.0f);
+      float zero = RND(mn + eight);
+      if (qp_bf16) {
+        scale = to_bf16(scale);
+        zero = to_bf16(zero);
+      }
+      eight = RND(scale * 8.0f);
+      const float lowest = RND(zero - eight);
+      for (int i = 0; i < g; ++i) {
+        const float d = RND(load_elem(w, r * K + k0 + i, is_bf16) - lowest);
+        float q = rintf(RND(d / scale));
+        q = q < 0.0f ? 0.0f : (q > 15.0f ? 15.0f : q);
+        if (q_out) q_out[r * K + k0 + i] = (uint8_t)q;
+        if (fq_out) {
+          const float t = RND((q - 8.0f) * scale);
+          store_elem(fq_out, r * K + k0 + i, t + zero, is_bf16);
+        }
+      }
+      if (scale_out) scale_out[r * (K / g) + k0 / g] = scale;
+      if (zero_out) zero_out[r * (K / g) + k0 / g] = zero;
+    }
+#undef RND
 }
 
 /* ---------------------------------------------------------------------------------------------------

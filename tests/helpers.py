@@ -53,6 +53,18 @@ def c_fq_per_group(lib, w: torch.Tensor, g: int):
     return fq, q, scale
 
 
+def c_fq_per_group_uint4_asym(lib, w: torch.Tensor, g: int, qp_bf16: bool = True):
+    w = w.contiguous()
+    rows, K = w.shape
+    fq = torch.empty_like(w)
+    q = torch.empty(w.shape, dtype=torch.uint8)
+    scale = torch.empty(rows, K // g, dtype=torch.float32)
+    zero = torch.empty(rows, K // g, dtype=torch.float32)
+    lib.ref_fq_per_group_uint4_asym(ptr(w), int(w.dtype == torch.bfloat16), int(qp_bf16), rows, K, g, ptr(fq), ptr(q),
+                                    ptr(scale), ptr(zero))
+    return fq, q, scale, zero
+
+
 def bits_equal(a: torch.Tensor, b: torch.Tensor) -> bool:
     """Bit-for-bit equality (distinguishes -0.0 from 0.0, treats equal NaN payloads as equal)."""
     if a.shape != b.shape or a.dtype != b.dtype:

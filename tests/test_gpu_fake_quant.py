@@ -151,3 +151,81 @@ def test_converted_weight_dequantises_to_the_fake_quantised_weight(dtype, g):
     zz = torch.randint(-3, 4, z.shape, generator=gen).float()
     want = ((q.view(96, -1, g).float() - zz[:, :, None]) * s[:, :, None]).to(dtype).view(96, 512)
     assert bits_equal(ops.dequantize_per_group_int4(q.to(DEV), s.to(DEV), zz.to(DEV), g, dtype).cpu(), want)
+
+
+# ---- weight-only int4 ("4w-qat") -------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype,qp", [(torch.bfloat16, torch.bfloat16), (torch.float32, torch.bfloat16), (torch.float32, torch.float32)])
+@pytest.mark.parametrize("g", [8, 32, 64, 128, 256, 512])
+def test_uint4_asym_fake_quant_convert_and_dequant_bit_exact(dtype, qp, g):
+    gen = torch.Generator().manual_seed(100 + g)
+    w = (torch.randn(96, 1024, generator=gen) * 0.02 + 0.003).to(dtype)
+    w[0, :g] = 0.25          # constant group: the 1e-6 floor of the scale
+    w[1, :g] = w[1, :g].abs() + 1.0  # all-positive group far from zero
+    w[2, :g] *= 1e-5         # tiny dynamic range
+    want, ws, wz = fq.fq_per_group_uint4_asym(w, g, qp)
+    got, gs, gz = ops.fq_per_group_uint4_asym(w.to(DEV), g, qp)
+    assert bits_equal(got.cpu(), want)
+    assert bits_equal(gs.cpu(), ws.float()) and bits_equal(gz.cpu(), wz.float())
+    only, s_none, z_none = ops.fq_per_group_uint4_asym(w.to(DEV), g, qp, want_qparams=False)
+    assert s_none is None and z_none is None and bits_equal(only.cpu(), want)
+    wq, ws2, wz2 = fq.quantize_per_group_uint4(w, g, qp)
+    gq, gs2, gz2 = ops.quantize_per_group_uint4(w.to(DEV), g, qp)
+    assert gq.dtype == torch.uint8 and gq.shape == (96, 512) and torch.equal(gq.cpu(), wq)
+    assert bits_equal(gs2.cpu(), ws2.float()) and bits_equal(gz2.cpu(), wz2.float())
+    dense = ops.dequantize_per_group_uint4(gq, gs2, gz2, g, dtype)
+    assert bits_equal(dense.cpu(), want)  # the converted weight is exactly what training saw
+
+
+def test_uint4_asym_ragged_tail_and_validation():
+    # a chunk count that does not fill the last workgroup, and leading dimensions
+    w = torch.randn(3, 5, 64, generator=torch.Generator().manual_seed(9)).to(torch.bfloat16)
+    got, s, z = ops.fq_per_group_uint4_asym(w.to(DEV), 32)
+    want, ws, wz = fq.fq_per_group_uint4_asym(w.view(15, 64), 32)
+    assert got.shape == w.shape and s.shape == (15, 2) and bits_equal(got.cpu().view(15, 64), want)
+    with pytest.raises(ValueError, match="divisible by group_size"):
+        ops.fq_per_group_uint4_asym(torch.zeros(4, 48, device=DEV), 32)
+    with pytest.raises(ValueError, match="power of two"):
+        ops.quantize_per_group_uint4(torch.zeros(4, 48, device=DEV), 24)
+    with pytest.raises(TypeError):
+        ops.dequantize_per_group_uint4(torch.zeros(4, 24, dtype=torch.int8, device=DEV), torch.ones(4, 1), torch.ones(4, 1), 48, torch.bfloat16)
+
+
+def test_weight_only_int4_qat_prepare_train_convert():
+    """Int4WeightOnlyQATQuantizer end to end: the prepared layer computes F.linear(x, fq(W)) with straight-through
+    gradients; the converted layer reproduces the same output from packed codes and bf16 scales_and_zeros."""
+    from torchtune_amd.qat import Int4WeightOnlyQATLinear, Int4WeightOnlyQATQuantizer, WeightOnlyInt4Linear
+
+    gen = torch.Generator().manual_seed(21)
+    K, N, g = 512, 192, 64
+    W = (torch.randn(N, K, generator=gen) * 0.05).to(torch.bfloat16)
+    x = torch.randn(4, 33, K, generator=gen).to(torch.bfloat16)
+    model = nn.Sequential(nn.Linear(K, N, bias=False)).to(torch.bfloat16)
+    with torch.no_grad():
+        model[0].weight.copy_(W)
+    model = model.to(DEV)
+    qz = Int4WeightOnlyQATQuantizer(groupsize=g)
+    model = qz.prepare(model)
+    layer = model[0]
+    assert isinstance(layer, Int4WeightOnlyQATLinear)
+    xd = x.to(DEV).requires_grad_(True)
+    y = layer(xd)
+    w_fq, ws, wz = fq.fq_per_group_uint4_asym(W, g)
+    torch.testing.assert_close(y.float().cpu(), (x.float() @ w_fq.float().T), rtol=1e-2, atol=1e-2)
+    assert bits_equal(layer.weight_fake_quantizer.scale.cpu(), ws) and bits_equal(layer.weight_fake_quantizer.zero_point.cpu(), wz)
+    gy = torch.randn(y.shape, generator=gen).to(torch.bfloat16)
+    y.backward(gy.to(DEV))
+    # straight-through: the weight gradient is gy^T x, the input gradient goes through the fake-quantised weight
+    torch.testing.assert_close(layer.weight.grad.float().cpu(), gy.float().view(-1, N).T @ x.float().view(-1, K), rtol=1e-2, atol=2e-2)
+    torch.testing.assert_close(xd.grad.float().cpu(), gy.float() @ w_fq.float(), rtol=1e-2, atol=1e-2)
+    y_ref = y.detach()
+    model = qz.convert(model)
+    conv = model[0]
+    assert isinstance(conv, WeightOnlyInt4Linear) and conv.weight.dtype == torch.uint8 and conv.weight.shape == (N, K // 2)
+    wq, _, _ = fq.quantize_per_group_uint4(W, g)
+    assert torch.equal(conv.weight.cpu(), wq)
+    assert bits_equal(conv.scales_and_zeros[..., 0].t().contiguous().cpu(), ws)
+    assert bits_equal(conv.scales_and_zeros[..., 1].t().contiguous().cpu(), wz)
+    assert bits_equal(conv.dense_weight().cpu(), w_fq)
+    assert bits_equal(conv(x.to(DEV)), y_ref)
+    sd = conv.state_dict()
+    assert set(sd) == {"weight", "scales_and_zeros"}

@@ -281,6 +281,39 @@ def test_quantizer_prepare_and_toggles_on_cpu():
         FakeQuantizedLinear(50, 8, weight_config=FakeQuantizeConfig(torch.int4, group_size=32))
 
 
+def test_weight_only_int4_quantizer_prepare_and_toggles_on_cpu():
+    """The "4w-qat" mode (torchtune/training/quantization.py:27,125-127): module swap, shape rule, config, toggles."""
+    from torchtune_amd.qat import Int4WeightOnlyQATLinear, Int4WeightOnlyQATQuantizer, WeightOnlyInt4Linear, ZeroPointDomain
+
+    model = nn.Sequential(nn.Linear(256, 64, bias=False), nn.Linear(256, 8, bias=True), nn.Linear(160, 8, bias=False)).to(torch.bfloat16)
+    qz = Int4WeightOnlyQATQuantizer(groupsize=32)
+    assert quantization.get_quantizer_mode(qz) == "4w-qat"
+    w0 = model[0].weight.detach().clone()
+    model = qz.prepare(model)
+    assert isinstance(model[0], Int4WeightOnlyQATLinear) and isinstance(model[0], FakeQuantizedLinear)
+    assert type(model[1]) is nn.Linear  # has a bias: left alone
+    assert type(model[2]) is nn.Linear  # 160 % (16 * inner_k_tiles) != 0: left alone
+    assert model[0].activation_fake_quantizer is None and torch.equal(model[0].weight, w0)
+    cfg = model[0].weight_fake_quantizer.config
+    assert (cfg.dtype, cfg.group_size, cfg.is_symmetric, cfg.zero_point_domain) == (torch.uint4, 32, False, ZeroPointDomain.FLOAT)
+    assert cfg.scale_precision == torch.bfloat16 and cfg.zero_point_precision == torch.bfloat16
+    model.apply(quantization._get_disable_fake_quant("4w-qat"))
+    assert not model[0].weight_fake_quantizer.enabled
+    x = torch.randn(3, 256).to(torch.bfloat16)
+    torch.testing.assert_close(model[0](x), x @ w0.T)  # disabled fake quant = plain linear, no kernel involved
+    model.apply(quantization._get_enable_fake_quant("4w-qat"))
+    assert model[0].weight_fake_quantizer.enabled
+    with pytest.raises(ValueError, match="Padding for QAT 4w is not supported yet"):
+        Int4WeightOnlyQATLinear(160, 8, groupsize=32)
+    with pytest.raises(AssertionError):
+        Int4WeightOnlyQATQuantizer(groupsize=48)
+    with pytest.raises(NotImplementedError):  # integer zero points for uint4 have no kernel
+        FakeQuantizer(FakeQuantizeConfig(torch.uint4, group_size=32, is_symmetric=False))
+    conv = WeightOnlyInt4Linear(256, 64, groupsize=32)
+    assert conv.weight.shape == (64, 128) and conv.weight.dtype == torch.uint8
+    assert conv.scales_and_zeros.shape == (8, 64, 2) and conv.scales_and_zeros.dtype == torch.bfloat16
+
+
 def test_swap_lora_linear_with_qat():
     model = nn.Sequential(LoRALinear(64, 64, 4, 1.0), nn.Sequential(LoRALinear(64, 32, 4, 1.0)))
     quantization.swap_lora_linear_with_qat(model, None, FakeQuantizeConfig(torch.int4, group_size=32))

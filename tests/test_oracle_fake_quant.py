@@ -135,3 +135,73 @@ def test_straight_through_backward():
     torch.testing.assert_close(y, x_fq @ w_fq.T)
     torch.testing.assert_close(x.grad, gy @ w_fq)  # gradient passes straight through both fake quantisers
     torch.testing.assert_close(w.grad, gy.T @ x_fq)
+
+
+# ---- weight-only int4 ("4w-qat"): asymmetric uint4 with a floating-point zero point --------------------------
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_uint4_asym_closed_form(dtype):
+    # a group that is exactly the 16-point grid min + k * step: scale = step, zero = min + 8 * step, codes = k,
+    # fake quantisation is the identity (all values exact in bf16)
+    k = torch.arange(16, dtype=torch.float32)
+    for lo, step in ((-1.0, 0.125), (1.0, 0.125), (-4.0, 0.25)):
+        w = (lo + step * k).to(dtype)[None, :]
+        out, scale, zero = fq.fq_per_group_uint4_asym(w, 16)
+        assert scale.dtype == torch.bfloat16 and zero.dtype == torch.bfloat16
+        assert scale.item() == step and zero.item() == lo + 8 * step
+        assert bits_equal(out, w)
+        packed, _, _ = fq.quantize_per_group_uint4(w, 16)
+        # even element in the high nibble
+        assert packed.tolist() == [[(2 * i) << 4 | (2 * i + 1) for i in range(8)]]
+    # the range is NOT widened to include zero: an all-positive group keeps its own minimum as code 0
+    w = torch.tensor([[1.0, 2.875] + [2.0] * 14]).to(dtype)
+    packed, scale, zero = fq.quantize_per_group_uint4(w, 16)
+    assert scale.item() == 0.125 and zero.item() == 2.0 and packed[0, 0].item() == (0 << 4) | 15
+    # a constant group: scale falls back to 1e-6 (rounded to the qparam dtype) and the value survives within a step
+    w = torch.full((1, 16), 0.5).to(dtype)
+    out, scale, zero = fq.fq_per_group_uint4_asym(w, 16)
+    assert scale.item() == torch.tensor(1e-6).to(torch.bfloat16).item()
+    assert torch.all((out.float() - 0.5).abs() <= 2.0 ** -8)
+
+
+@pytest.mark.parametrize("g", [32, 128, 256])
+def test_uint4_asym_invariants(g):
+    gen = torch.Generator().manual_seed(3)
+    w = torch.randn(24, 512, generator=gen) * 0.05 + 0.01
+    out, scale, zero = fq.fq_per_group_uint4_asym(w, g, qparam_dtype=torch.float32)
+    packed, s2, z2 = fq.quantize_per_group_uint4(w, g, qparam_dtype=torch.float32)
+    assert torch.equal(scale, s2) and torch.equal(zero, z2)
+    codes = torch.stack([packed >> 4, packed & 15], dim=-1).reshape(24, 512).float()
+    assert codes.min() == 0 and codes.max() == 15
+    wg, cg = w.view(24, 512 // g, g), codes.view(24, 512 // g, g)
+    # the group minimum takes code 0 and the maximum code 15
+    assert torch.all(cg.gather(-1, wg.argmin(-1, keepdim=True)) == 0)
+    assert torch.all(cg.gather(-1, wg.argmax(-1, keepdim=True)) == 15)
+    # codes are monotone in the value, the error is at most half a step (fp32 arithmetic slack aside)
+    order = wg.argsort(-1)
+    assert torch.all(cg.gather(-1, order).diff(dim=-1) >= 0)
+    assert torch.all((out - w).view(24, 512 // g, g).abs() <= 0.5 * scale[..., None] * 1.001)
+    # brute force: the chosen code is the nearest of the 16 grid points zero + (q - 8) * scale
+    grid = zero[..., None, None] + (torch.arange(16.0) - 8.0) * scale[..., None, None]  # [rows, G, 1, 16]
+    dist = (wg[..., None] - grid).abs()
+    best = dist.min(-1).values
+    chosen = dist.gather(-1, cg.long()[..., None])[..., 0]
+    assert torch.all(chosen <= best + 1e-6 * scale[..., None])
+    # dequantising the packed codes reproduces the fake-quantised tensor bit for bit
+    assert bits_equal(fq.dequantize_per_group_uint4(packed, scale, zero, g, torch.float32), out)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("qp", [torch.bfloat16, torch.float32])
+def test_uint4_asym_two_restatements_agree(c_oracle, dtype, qp):
+    from tests.helpers import c_fq_per_group_uint4_asym
+
+    gen = torch.Generator().manual_seed(4)
+    for g, std, shift in ((32, 0.02, 0.0), (64, 1.0, 0.3), (256, 5.0, -2.0), (8, 1e-7, 0.0)):
+        w = (torch.randn(16, 512, generator=gen) * std + shift).to(dtype)
+        out, scale, zero = fq.fq_per_group_uint4_asym(w, g, qparam_dtype=qp)
+        packed, _, _ = fq.quantize_per_group_uint4(w, g, qparam_dtype=qp)
+        fc, qc, sc, zc = c_fq_per_group_uint4_asym(c_oracle, w, g, qp == torch.bfloat16)
+        assert bits_equal(scale.float(), sc) and bits_equal(zero.float(), zc)
+        assert torch.equal(torch.stack([packed >> 4, packed & 15], dim=-1).reshape(16, 512), qc)
+        assert bits_equal(out, fc)
+        assert bits_equal(fq.dequantize_per_group_uint4(packed, scale, zero, g, dtype), out)

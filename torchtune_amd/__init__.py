@@ -11,9 +11,13 @@ from .qat import (
     FakeQuantizeConfig,
     FakeQuantizedLinear,
     FakeQuantizer,
+    Int4WeightOnlyQATLinear,
+    Int4WeightOnlyQATQuantizer,
     Int8DynActInt4WeightLinear,
     Int8DynActInt4WeightQATLinear,
     Int8DynActInt4WeightQATQuantizer,
+    WeightOnlyInt4Linear,
+    ZeroPointDomain,
 )
 
 __all__ = [
@@ -31,4 +35,8 @@ __all__ = [
     "Int8DynActInt4WeightQATQuantizer",
     "Int8DynActInt4WeightQATLinear",
     "Int8DynActInt4WeightLinear",
+    "Int4WeightOnlyQATQuantizer",
+    "Int4WeightOnlyQATLinear",
+    "WeightOnlyInt4Linear",
+    "ZeroPointDomain",
 ]

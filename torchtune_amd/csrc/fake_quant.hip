@@ -301,6 +301,118 @@ __global__ __launch_bounds__(256) void dequant_per_group_kernel(const int8_t* __
   Chunk8<BF16>::store(out, ch, v);
 }
 
+// Per-group asymmetric uint4 with a floating-point zero point (the weight-only "4w" scheme).  Same lane layout
+// as the symmetric kernel.  Every operation is rounded to the tensor dtype, the qparams additionally to their
+// own precision, so the result equals the op-by-op eager sequence:
+//   scale = clamp((max - min) / 15, 1e-6);  zero = min + scale * 8
+//   q     = clamp(round((w - (zero - scale * 8)) / scale), 0, 15);  fq = (q - 8) * scale + zero
+// EMIT_INT = true writes the codes packed two per byte (even element in the high nibble) instead of fq.
+template <bool BF16, bool QP_BF16, bool EMIT_INT>
+__global__ __launch_bounds__(256) void fq_per_group_asym_kernel(const void* __restrict__ w, int64_t n_chunks,
+                                                                int lanes_per_group, int log2_lpg,
+                                                                void* __restrict__ out_fq, uint32_t* __restrict__ out_q,
+                                                                float* __restrict__ scale_out, float* __restrict__ zero_out) {
+  using A = Arith<BF16>;
+  using Q = Arith<QP_BF16>;
+  const int64_t base = (int64_t)blockIdx.x * (256 * kGroupChunksPerThread) + threadIdx.x;
+  Chunk8<BF16> c[kGroupChunksPerThread];
+#pragma unroll
+  for (int u = 0; u < kGroupChunksPerThread; ++u) {
+    const int64_t ch = base + u * 256;
+    if (ch < n_chunks)
+      c[u].load(w, ch);
+    else
+      c[u].zero();
+  }
+#pragma unroll
+  for (int u = 0; u < kGroupChunksPerThread; ++u) {
+    const int64_t ch = base + u * 256;
+    float mn = c[u].get(0), mx = mn;
+#pragma unroll
+    for (int e = 1; e < 8; ++e) {
+      const float v = c[u].get(e);
+      mn = fminf(mn, v);
+      mx = fmaxf(mx, v);
+    }
+    for (int off = 1; off < lanes_per_group; off <<= 1) {
+      mn = fminf(mn, __shfl_xor(mn, off, kWave));
+      mx = fmaxf(mx, __shfl_xor(mx, off, kWave));
+    }
+    if (ch >= n_chunks) continue;
+    float scale = A::rnd(A::rnd(mx - mn) / 15.0f);
+    scale = A::rnd(fmaxf(scale, 1e-6f));
+    float zero = A::rnd(mn + A::rnd(scale * 8.0f));
+    scale = Q::rnd(scale);
+    zero = Q::rnd(zero);
+    if ((threadIdx.x & (lanes_per_group - 1)) == 0) {
+      if (scale_out) scale_out[ch >> log2_lpg] = scale;
+      if (zero_out) zero_out[ch >> log2_lpg] = zero;
+    }
+    const float lowest = A::rnd(zero - A::rnd(scale * 8.0f));
+    float q[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      float t = A::rnd(A::rnd(c[u].get(e) - lowest) / scale);
+      t = __builtin_rintf(t);
+      q[e] = t < 0.0f ? 0.0f : (t > 15.0f ? 15.0f : t);
+    }
+    if constexpr (EMIT_INT) {
+      uint32_t packed = 0;
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        packed |= (((uint32_t)(int)q[2 * e] << 4) | (uint32_t)(int)q[2 * e + 1]) << (8 * e);
+      out_q[ch] = packed;
+    } else {
+      float v[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = A::rnd(A::rnd((q[e] - 8.0f) * scale) + zero);
+      Chunk8<BF16>::store(out_fq, ch, v);
+    }
+  }
+}
+
+template <bool BF16>
+__global__ __launch_bounds__(256) void dequant_per_group_uint4_kernel(const uint32_t* __restrict__ q,
+                                                                      const float* __restrict__ scale,
+                                                                      const float* __restrict__ zero, int64_t n_chunks,
+                                                                      int log2_lpg, void* __restrict__ out) {
+  using A = Arith<BF16>;
+  const int64_t ch = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (ch >= n_chunks) return;
+  const uint32_t raw = q[ch];
+  const float sc = scale[ch >> log2_lpg];
+  const float z = zero[ch >> log2_lpg];
+  float v[8];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const uint32_t b = (raw >> (8 * e)) & 0xffu;
+    v[2 * e] = A::rnd(A::rnd(((float)(b >> 4) - 8.0f) * sc) + z);
+    v[2 * e + 1] = A::rnd(A::rnd(((float)(b & 15u) - 8.0f) * sc) + z);
+  }
+  Chunk8<BF16>::store(out, ch, v);
+}
+
+template <bool EMIT_INT>
+int launch_group_asym(const void* w, int dtype, int qparam_dtype, int64_t rows, int64_t K, int group_size, void* out_fq,
+                      uint32_t* out_q, float* scale, float* zero, hipStream_t s, const char* what) {
+  const int64_t n_chunks = rows * K / 8;
+  const int64_t per_wg = 256 * kGroupChunksPerThread;
+  const int64_t grid = (n_chunks + per_wg - 1) / per_wg;
+  TT_REQUIRE(grid < (int64_t(1) << 31), "%s: tensor too large for one launch", what);
+  const int lpg = group_size / 8, l2 = log2_exact(lpg);
+  const dim3 g((unsigned)grid), b(256);
+  const bool bf = dtype == TTAMD_BF16, qbf = qparam_dtype == TTAMD_BF16;
+  if (bf && qbf)
+    fq_per_group_asym_kernel<true, true, EMIT_INT><<<g, b, 0, s>>>(w, n_chunks, lpg, l2, out_fq, out_q, scale, zero);
+  else if (bf)
+    fq_per_group_asym_kernel<true, false, EMIT_INT><<<g, b, 0, s>>>(w, n_chunks, lpg, l2, out_fq, out_q, scale, zero);
+  else if (qbf)
+    fq_per_group_asym_kernel<false, true, EMIT_INT><<<g, b, 0, s>>>(w, n_chunks, lpg, l2, out_fq, out_q, scale, zero);
+  else
+    fq_per_group_asym_kernel<false, false, EMIT_INT><<<g, b, 0, s>>>(w, n_chunks, lpg, l2, out_fq, out_q, scale, zero);
+  return check_launch(what);
+}
+
 int check_group_args(const void* w, int dtype, int64_t rows, int64_t K, int group_size) {
   TT_REQUIRE(dtype == TTAMD_BF16 || dtype == TTAMD_F32, "fake_quant: unknown dtype code %d", dtype);
   TT_REQUIRE(w != nullptr && aligned16(w), "fake_quant: input must be a non-null 16-byte aligned pointer");
@@ -387,4 +499,47 @@ extern "C" int ttamd_dequantize_per_group_int4(const int8_t* q, const float* sca
   else
     dequant_per_group_kernel<false><<<dim3((unsigned)grid), dim3(256), 0, s>>>(q, scale, zero_point, n_chunks, l2, out);
   return check_launch("dequantize_per_group_int4");
+}
+
+extern "C" int ttamd_fq_per_group_uint4_asym(const void* w, int dtype, int64_t rows, int64_t K, int group_size,
+                                             int qparam_dtype, void* out, float* scale, float* zero_point, void* stream) {
+  if (int rc = check_group_args(w, dtype, rows, K, group_size)) return rc;
+  TT_REQUIRE(qparam_dtype == TTAMD_BF16 || qparam_dtype == TTAMD_F32, "fq_per_group_uint4_asym: unknown qparam dtype code %d",
+             qparam_dtype);
+  TT_REQUIRE(out && aligned16(out), "fq_per_group_uint4_asym: out must be non-null, 16-byte aligned");
+  return launch_group_asym<false>(w, dtype, qparam_dtype, rows, K, group_size, out, nullptr, scale, zero_point,
+                                  reinterpret_cast<hipStream_t>(stream), "fq_per_group_uint4_asym");
+}
+
+extern "C" int ttamd_quantize_per_group_uint4(const void* w, int dtype, int64_t rows, int64_t K, int group_size,
+                                              int qparam_dtype, uint8_t* q, float* scale, float* zero_point, void* stream) {
+  if (int rc = check_group_args(w, dtype, rows, K, group_size)) return rc;
+  TT_REQUIRE(qparam_dtype == TTAMD_BF16 || qparam_dtype == TTAMD_F32, "quantize_per_group_uint4: unknown qparam dtype code %d",
+             qparam_dtype);
+  TT_REQUIRE(q && scale && zero_point && (reinterpret_cast<uintptr_t>(q) & 3u) == 0,
+             "quantize_per_group_uint4: q (4-byte aligned), scale and zero_point must be non-null");
+  return launch_group_asym<true>(w, dtype, qparam_dtype, rows, K, group_size, nullptr, reinterpret_cast<uint32_t*>(q), scale,
+                                 zero_point, reinterpret_cast<hipStream_t>(stream), "quantize_per_group_uint4");
+}
+
+extern "C" int ttamd_dequantize_per_group_uint4(const uint8_t* q, const float* scale, const float* zero_point, int dtype,
+                                                int64_t rows, int64_t K, int group_size, void* out, void* stream) {
+  TT_REQUIRE(dtype == TTAMD_BF16 || dtype == TTAMD_F32, "dequantize_per_group_uint4: unknown dtype code %d", dtype);
+  TT_REQUIRE(q && scale && zero_point && out && (reinterpret_cast<uintptr_t>(q) & 3u) == 0 && aligned16(out),
+             "dequantize_per_group_uint4: q (4-byte aligned), scale, zero_point and out (16-byte aligned) must be non-null");
+  TT_REQUIRE(rows > 0 && K > 0, "dequantize_per_group_uint4: rows and K must be positive");
+  TT_REQUIRE(group_size >= 8 && group_size <= 512 && is_pow2(group_size) && K % group_size == 0,
+             "dequantize_per_group_uint4: group_size (%d) must be a power of two in [8, 512] dividing K (%lld)", group_size,
+             (long long)K);
+  const int64_t n_chunks = rows * K / 8;
+  const int64_t grid = (n_chunks + 255) / 256;
+  TT_REQUIRE(grid < (int64_t(1) << 31), "dequantize_per_group_uint4: tensor too large for one launch");
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const int l2 = log2_exact(group_size / 8);
+  const uint32_t* q32 = reinterpret_cast<const uint32_t*>(q);
+  if (dtype == TTAMD_BF16)
+    dequant_per_group_uint4_kernel<true><<<dim3((unsigned)grid), dim3(256), 0, s>>>(q32, scale, zero_point, n_chunks, l2, out);
+  else
+    dequant_per_group_uint4_kernel<false><<<dim3((unsigned)grid), dim3(256), 0, s>>>(q32, scale, zero_point, n_chunks, l2, out);
+  return check_launch("dequantize_per_group_uint4");
 }

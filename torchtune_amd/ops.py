@@ -362,9 +362,76 @@ def quantize_per_group_int4(w: torch.Tensor, group_size: int):
     return q, scale, zeros
 
 
-# ---------------------------------------------------------------------------------------------------
-# neighbours of the quantized linears in a decoder layer: RMSNorm, rotary embedding, SwiGLU gate
-# ---------------------------------------------------------------------------------------------------
+def fq_per_group_uint4_asym(w: torch.Tensor, group_size: int, qparam_dtype: torch.dtype = torch.bfloat16,
+                            want_qparams: bool = True):
+    """Weight-only int4 scheme (asymmetric uint4, floating-point zero point):
+    w [..., K] -> (fake-quantised w, scale fp32 [rows, K/g] | None, zero_point fp32 [rows, K/g] | None);
+    the qparams hold values already rounded to ``qparam_dtype``."""
+    _need_gpu(w, "fq_per_group_uint4_asym")
+    code = _code(w.dtype, "fq_per_group_uint4_asym")
+    qcode = _code(qparam_dtype, "fq_per_group_uint4_asym (qparams)")
+    wc = w.contiguous()
+    K = wc.shape[-1]
+    rows = wc.numel() // K
+    out = torch.empty_like(wc)
+    scale = torch.empty(rows, K // max(group_size, 1), dtype=torch.float32, device=w.device) if want_qparams else None
+    zero = torch.empty_like(scale) if want_qparams else None
+    lib = _lib.load()
+    with torch.cuda.device(w.device):
+        events = _fq_timer("per_group", rows, K, group_size, wc.element_size()) if _fq_timer is not None else None
+        if events:
+            events[0].record()
+        rc = lib.ttamd_fq_per_group_uint4_asym(wc.data_ptr(), code, rows, K, group_size, qcode, out.data_ptr(), _ptr(scale),
+                                               _ptr(zero), _stream(w))
+        if events:
+            events[1].record()
+    _lib.check(rc, "fq_per_group_uint4_asym")
+    return out, scale, zero
+
+
+def quantize_per_group_uint4(w: torch.Tensor, group_size: int, qparam_dtype: torch.dtype = torch.bfloat16):
+    """w [rows, K] -> (uint8 [rows, K/2], two codes per byte with the even element in the high nibble,
+    scale fp32 [rows, K/g], zero_point fp32 [rows, K/g])"""
+    _need_gpu(w, "quantize_per_group_uint4")
+    code = _code(w.dtype, "quantize_per_group_uint4")
+    qcode = _code(qparam_dtype, "quantize_per_group_uint4 (qparams)")
+    if w.dim() != 2:
+        raise ValueError(f"quantize_per_group_uint4: expected a 2-D weight, got {tuple(w.shape)}")
+    wc = w.contiguous()
+    rows, K = wc.shape
+    q = torch.empty(rows, K // 2, dtype=torch.uint8, device=w.device)
+    scale = torch.empty(rows, K // max(group_size, 1), dtype=torch.float32, device=w.device)
+    zero = torch.empty_like(scale)
+    lib = _lib.load()
+    with torch.cuda.device(w.device):
+        rc = lib.ttamd_quantize_per_group_uint4(wc.data_ptr(), code, rows, K, group_size, qcode, q.data_ptr(), scale.data_ptr(),
+                                                zero.data_ptr(), _stream(w))
+    _lib.check(rc, "quantize_per_group_uint4")
+    return q, scale, zero
+
+
+def dequantize_per_group_uint4(q: torch.Tensor, scale: torch.Tensor, zero: torch.Tensor, group_size: int,
+                               dtype: torch.dtype) -> torch.Tensor:
+    """q [rows, K/2] uint8 (packed codes), scale / zero fp32 [rows, K/g] -> dtype((q - 8) * scale + zero) [rows, K]"""
+    _need_gpu(q, "dequantize_per_group_uint4")
+    code = _code(dtype, "dequantize_per_group_uint4")
+    if q.dtype != torch.uint8 or q.dim() != 2:
+        raise TypeError(f"dequantize_per_group_uint4: q must be a 2-D uint8 tensor, got {tuple(q.shape)} {q.dtype}")
+    qc = q.contiguous()
+    rows, K = qc.shape[0], qc.shape[1] * 2
+    sc = scale.to(torch.float32).contiguous()
+    zc = zero.to(torch.float32).contiguous()
+    if sc.numel() != rows * (K // max(group_size, 1)) or zc.numel() != sc.numel():
+        raise ValueError("dequantize_per_group_uint4: scale / zero must have rows * K / group_size elements")
+    out = torch.empty(rows, K, dtype=dtype, device=q.device)
+    lib = _lib.load()
+    with torch.cuda.device(q.device):
+        rc = lib.ttamd_dequantize_per_group_uint4(qc.data_ptr(), sc.data_ptr(), zc.data_ptr(), code, rows, K, group_size,
+                                                  out.data_ptr(), _stream(q))
+    _lib.check(rc, "dequantize_per_group_uint4")
+    return out
+
+
 def dequantize_per_group_int4(q: torch.Tensor, scale: torch.Tensor, zeros: Optional[torch.Tensor], group_size: int,
                               dtype: torch.dtype) -> torch.Tensor:
     """q [rows, K] int8 (int4 values), scale/zeros fp32 [rows, K/g] -> dtype((q - zeros) * scale) [rows, K]"""
@@ -387,6 +454,9 @@ def dequantize_per_group_int4(q: torch.Tensor, scale: torch.Tensor, zeros: Optio
     return out
 
 
+# ---------------------------------------------------------------------------------------------------
+# neighbours of the quantized linears in a decoder layer: RMSNorm, rotary embedding, SwiGLU gate
+# ---------------------------------------------------------------------------------------------------
 def _bf16_any(t: torch.Tensor, what: str) -> torch.Tensor:
     _need_gpu(t, what)
     if t.dtype != torch.bfloat16:

@@ -1,22 +1,26 @@
 """Quantisation-aware training for the 8da4w scheme (int8 dynamic per-token activations, int4 per-group
-symmetric weights) on the HIP fake-quant kernels.
+symmetric weights) and the weight-only 4w scheme (uint4 per-group asymmetric weights with a floating-point zero
+point) on the HIP fake-quant kernels.
 
 The reference obtains all of this from ``torchao.quantization.qat``:
 
 * ``Int8DynActInt4WeightQATQuantizer`` — re-exported at ``torchtune/training/quantization.py:26-29`` and
   instantiated from YAML by ``recipes/qat_single_device.py:375-386`` (``prepare``) and ``recipes/quantize.py:88-95``
   (``convert``);
+* ``Int4WeightOnlyQATQuantizer`` — re-exported at ``torchtune/training/quantization.py:27`` and mapped to the
+  ``"4w-qat"`` mode at ``:125-127``;
 * ``FakeQuantizeConfig`` / ``FakeQuantizer`` — used directly by ``QATLoRALinear``
   (``torchtune/modules/peft/lora.py:222-250``);
 * ``FakeQuantizedLinear`` — what ``_enable_linear_fake_quant`` toggles
   (``torchtune/training/quantization.py:56-71``).
 
-The same names and call signatures are provided here.  Only the two schemes named above have kernels;
+The same names and call signatures are provided here.  Only the schemes named above have kernels;
 any other configuration raises ``NotImplementedError`` instead of silently computing something else.
 """
 from __future__ import annotations
 
 from dataclasses import dataclass
+from enum import Enum, auto
 from typing import Optional, Union
 
 import torch
@@ -38,16 +42,25 @@ class PerGroup:
     group_size: int
 
 
+class ZeroPointDomain(Enum):
+    """Whether the zero point lives on the integer grid or in the floating-point domain."""
+
+    INT = auto()
+    FLOAT = auto()
+    NONE = auto()
+
+
 class FakeQuantizeConfig:
     """How a tensor is fake-quantised.
 
     Args:
-        dtype: ``torch.int8`` (activations) or ``torch.int4`` (weights)
+        dtype: ``torch.int8`` (activations), ``torch.int4`` (weights) or ``torch.uint4`` (weight-only scheme)
         granularity: ``"per_token"``, ``"per_group"``, a ``PerToken()`` or a ``PerGroup(n)``
         group_size: keyword shortcut for ``PerGroup(group_size)``
         is_symmetric: symmetric (zero-point 0) or asymmetric mapping
         scale_precision, zero_point_precision: dtypes of the qparams kept on the quantizer
         is_dynamic: qparams are recomputed from each input (the only supported mode)
+        zero_point_domain: ``ZeroPointDomain.INT`` (default) or ``ZeroPointDomain.FLOAT`` (the weight-only scheme)
     """
 
     def __init__(
@@ -61,10 +74,14 @@ class FakeQuantizeConfig:
         *,
         group_size: Optional[int] = None,
         is_symmetric: Optional[bool] = None,
+        zero_point_domain: ZeroPointDomain = ZeroPointDomain.INT,
     ):
-        if dtype not in (torch.int8, torch.int4):
-            raise NotImplementedError(f"FakeQuantizeConfig: dtype {dtype} has no kernel (int8 and int4 do)")
+        if dtype not in (torch.int8, torch.int4, torch.uint4):
+            raise NotImplementedError(f"FakeQuantizeConfig: dtype {dtype} has no kernel (int8, int4 and uint4 do)")
         self.dtype = dtype
+        if zero_point_domain not in (ZeroPointDomain.INT, ZeroPointDomain.FLOAT):
+            raise ValueError("Please use ZeroPointDomain.INT or ZeroPointDomain.FLOAT")
+        self.zero_point_domain = zero_point_domain
         if group_size is not None and granularity is not None and granularity != "per_group":
             raise ValueError("`group_size` conflicts with granularity '%s'" % (granularity,))
         if isinstance(granularity, str):
@@ -142,8 +159,17 @@ class FakeQuantizer(nn.Module):
             if config.dtype != torch.int8 or config.is_symmetric:
                 raise NotImplementedError("per-token fake quantisation has a kernel for asymmetric int8 only")
         elif isinstance(g, PerGroup):
-            if config.dtype != torch.int4 or not config.is_symmetric:
-                raise NotImplementedError("per-group fake quantisation has a kernel for symmetric int4 only")
+            sym_int4 = config.dtype == torch.int4 and config.is_symmetric and config.zero_point_domain == ZeroPointDomain.INT
+            if not (sym_int4 or self._weight_only_int4(config)):
+                raise NotImplementedError(
+                    "per-group fake quantisation has kernels for symmetric int4 and for asymmetric uint4 with a "
+                    "floating-point zero point only")
+
+    @staticmethod
+    def _weight_only_int4(config: FakeQuantizeConfig) -> bool:
+        return (config.dtype == torch.uint4 and not config.is_symmetric and config.zero_point_domain == ZeroPointDomain.FLOAT
+                and config.scale_precision in (torch.bfloat16, torch.float32)
+                and config.zero_point_precision == config.scale_precision)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         if not self.enabled:
@@ -157,9 +183,14 @@ class FakeQuantizer(nn.Module):
                 gs = self.config.group_size
                 if x.shape[-1] % gs != 0:
                     raise ValueError(f"last dimension ({x.shape[-1]}) must be divisible by group_size ({gs})")
-                fq, scale = ops.fq_per_group_int4_sym(x.detach(), gs)
-                self.scale = scale.to(self.config.scale_precision)
-                self.zero_point = None
+                if self._weight_only_int4(self.config):
+                    fq, scale, zp = ops.fq_per_group_uint4_asym(x.detach(), gs, self.config.scale_precision)
+                    self.scale = scale.to(self.config.scale_precision)
+                    self.zero_point = zp.to(self.config.zero_point_precision)
+                else:
+                    fq, scale = ops.fq_per_group_int4_sym(x.detach(), gs)
+                    self.scale = scale.to(self.config.scale_precision)
+                    self.zero_point = None
         return _StraightThrough.apply(x, fq.view(x.shape))
 
     def __repr__(self) -> str:
@@ -332,6 +363,148 @@ class Int8DynActInt4WeightQATQuantizer:
                 new.zeros.copy_(zeros.to(child.scales_precision))
                 if child.bias is not None:
                     new.bias = nn.Parameter(child.bias.detach(), requires_grad=False)
+                setattr(model, name, new)
+            else:
+                self.convert(child)
+        return model
+
+
+# ---------------------------------------------------------------------------------------------------
+# weight-only int4 ("4w-qat")
+# ---------------------------------------------------------------------------------------------------
+def _check_linear_int4_k(k: int, groupsize: int = 1, inner_k_tiles: Optional[int] = None) -> bool:
+    """The shape rule of the weight-only int4 linear: K divisible by the group size and by 16 * inner_k_tiles."""
+    ok = k % groupsize == 0
+    if inner_k_tiles is not None:
+        ok = ok and k % (inner_k_tiles * 16) == 0
+    return ok
+
+
+def _get_4w_weight_config(group_size: int, qparams_precision: torch.dtype) -> FakeQuantizeConfig:
+    return FakeQuantizeConfig(
+        dtype=torch.uint4, group_size=group_size, is_symmetric=False, is_dynamic=True, scale_precision=qparams_precision,
+        zero_point_precision=qparams_precision, zero_point_domain=ZeroPointDomain.FLOAT,
+    )
+
+
+class Int4WeightOnlyQATLinear(FakeQuantizedLinear):
+    """The linear ``Int4WeightOnlyQATQuantizer.prepare`` swaps in: the input passes unchanged, the weight is
+    fake-quantised to uint4 per group (asymmetric, floating-point zero point, bf16 qparams)."""
+
+    def __init__(
+        self,
+        in_features: int,
+        out_features: int,
+        bias: bool = False,
+        device: Optional[torch.device] = None,
+        groupsize: int = 256,
+        inner_k_tiles: int = 8,
+        precision: torch.dtype = torch.bfloat16,
+        scales_precision: torch.dtype = torch.bfloat16,
+    ) -> None:
+        assert scales_precision == torch.bfloat16, "only bf16 is supported for scales"
+        if not _check_linear_int4_k(in_features, groupsize, inner_k_tiles):
+            raise ValueError("Padding for QAT 4w is not supported yet")
+        self.groupsize = groupsize
+        self.inner_k_tiles = inner_k_tiles
+        self.precision = precision
+        self.scales_precision = scales_precision
+        super().__init__(in_features, out_features, bias, None, _get_4w_weight_config(groupsize, scales_precision),
+                         device=device, dtype=precision)
+
+    def enable_fake_quant(self, enabled: bool = True):
+        self.weight_fake_quantizer.enabled = enabled
+
+    def disable_fake_quant(self):
+        self.enable_fake_quant(False)
+
+
+class WeightOnlyInt4Linear(nn.Module):
+    """Result of ``Int4WeightOnlyQATQuantizer.convert``: uint4 codes packed two per byte (``weight`` [N, K/2], even
+    element in the high nibble) and ``scales_and_zeros`` [K/groupsize, N, 2] in bf16.  Forward rebuilds the dense
+    weight the fake-quantised layer trained with and multiplies.
+
+    The reference's converted module re-tiles the codes for one specific int4 matmul kernel
+    (``aten._convert_weight_to_int4pack``); that opaque tiling is not reproduced, the plain packing is kept."""
+
+    def __init__(self, in_features: int, out_features: int, bias: bool = False, device=None, groupsize: int = 128,
+                 inner_k_tiles: int = 8, precision: torch.dtype = torch.bfloat16,
+                 scales_precision: torch.dtype = torch.bfloat16) -> None:
+        super().__init__()
+        assert not bias, "require bias=False"
+        if not _check_linear_int4_k(in_features, groupsize, inner_k_tiles):
+            raise ValueError("in_features must be divisible by groupsize and by 16 * inner_k_tiles")
+        self.in_features = in_features
+        self.out_features = out_features
+        self.groupsize = groupsize
+        self.inner_k_tiles = inner_k_tiles
+        self.precision = precision
+        self.scales_precision = scales_precision
+        self.register_buffer("weight", torch.zeros((out_features, in_features // 2), dtype=torch.uint8, device=device))
+        self.register_buffer(
+            "scales_and_zeros",
+            torch.zeros((in_features // groupsize, out_features, 2), dtype=scales_precision, device=device),
+        )
+
+    def dense_weight(self) -> torch.Tensor:
+        sz = self.scales_and_zeros
+        scale = sz[..., 0].t()
+        zero = sz[..., 1].t()
+        return ops.dequantize_per_group_uint4(self.weight, scale, zero, self.groupsize, self.precision)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return F.linear(x.to(self.precision), self.dense_weight())
+
+
+class Int4WeightOnlyQATQuantizer:
+    """QAT quantizer for the weight-only int4 scheme (mode ``"4w-qat"``).
+
+    ``prepare(model)`` swaps every bias-free ``nn.Linear`` whose ``in_features`` fits the shape rule for
+    :class:`Int4WeightOnlyQATLinear`; ``convert(model)`` swaps those for :class:`WeightOnlyInt4Linear`.
+    """
+
+    def __init__(
+        self,
+        groupsize: int = 256,
+        inner_k_tiles: Optional[int] = 8,
+        precision: torch.dtype = torch.bfloat16,
+        scales_precision: torch.dtype = torch.bfloat16,
+    ) -> None:
+        assert inner_k_tiles in [2, 4, 8]
+        assert groupsize in [32, 64, 128, 256]
+        self.groupsize = groupsize
+        self.inner_k_tiles = inner_k_tiles
+        self.precision = precision
+        self.scales_precision = scales_precision
+
+    def get_weight_fake_quantize_config(self) -> FakeQuantizeConfig:
+        return _get_4w_weight_config(self.groupsize, self.scales_precision)
+
+    def prepare(self, model: nn.Module, *args, **kwargs) -> nn.Module:
+        for name, child in list(model.named_children()):
+            if (type(child) is nn.Linear and child.bias is None
+                    and _check_linear_int4_k(child.in_features, self.groupsize, self.inner_k_tiles)):
+                new = Int4WeightOnlyQATLinear(
+                    child.in_features, child.out_features, False, device=child.weight.device, groupsize=self.groupsize,
+                    inner_k_tiles=self.inner_k_tiles, precision=self.precision, scales_precision=self.scales_precision,
+                )
+                if child.weight.device != torch.device("meta"):
+                    new.weight = nn.Parameter(child.weight.detach().to(self.precision), requires_grad=child.weight.requires_grad)
+                setattr(model, name, new)
+            else:
+                self.prepare(child)
+        return model
+
+    def convert(self, model: nn.Module, *args, **kwargs) -> nn.Module:
+        for name, child in list(model.named_children()):
+            if isinstance(child, Int4WeightOnlyQATLinear):
+                new = WeightOnlyInt4Linear(
+                    child.in_features, child.out_features, False, device=child.weight.device, groupsize=child.groupsize,
+                    inner_k_tiles=child.inner_k_tiles, precision=child.weight.dtype, scales_precision=child.scales_precision,
+                )
+                q, scale, zero = ops.quantize_per_group_uint4(child.weight.detach(), child.groupsize, child.scales_precision)
+                new.weight.copy_(q)
+                new.scales_and_zeros.copy_(torch.stack([scale.t(), zero.t()], dim=-1).to(child.scales_precision))
                 setattr(model, name, new)
             else:
                 self.convert(child)

@@ -1,5 +1,5 @@
 """Quantizer names and fake-quant toggles under the dotpaths the reference's recipes and YAML configs use
-(``torchtune/training/quantization.py:26-29,56-71,94-97,167-244``), bound to the HIP-backed implementations."""
+(``torchtune/training/quantization.py:26-29,56-71,94-97,125-127,167-244``), bound to the HIP-backed implementations."""
 from __future__ import annotations
 
 from typing import Callable, Optional
@@ -7,15 +7,21 @@ from typing import Callable, Optional
 from torch import nn
 
 from ..modules.peft.lora import LoRALinear, QATLoRALinear
-from ..qat import FakeQuantizeConfig, FakeQuantizedLinear, Int8DynActInt4WeightQATQuantizer
+from ..qat import (
+    FakeQuantizeConfig,
+    FakeQuantizedLinear,
+    Int4WeightOnlyQATQuantizer,
+    Int8DynActInt4WeightQATQuantizer,
+)
 
 __all__ = [
     "get_quantizer_mode",
+    "Int4WeightOnlyQATQuantizer",
     "Int8DynActInt4WeightQATQuantizer",
     "swap_lora_linear_with_qat",
 ]
 
-_quantizer_to_mode = {Int8DynActInt4WeightQATQuantizer: "8da4w-qat"}
+_quantizer_to_mode = {Int8DynActInt4WeightQATQuantizer: "8da4w-qat", Int4WeightOnlyQATQuantizer: "4w-qat"}
 
 
 def _enable_linear_fake_quant(mod: nn.Module, enabled: bool = True) -> None:
@@ -30,12 +36,13 @@ def _disable_linear_fake_quant(mod: nn.Module) -> None:
     _enable_linear_fake_quant(mod, enabled=False)
 
 
-_quantizer_mode_to_disable_fake_quant = {"8da4w-qat": _disable_linear_fake_quant}
-_quantizer_mode_to_enable_fake_quant = {"8da4w-qat": _enable_linear_fake_quant}
+_quantizer_mode_to_disable_fake_quant = {"8da4w-qat": _disable_linear_fake_quant, "4w-qat": _disable_linear_fake_quant}
+_quantizer_mode_to_enable_fake_quant = {"8da4w-qat": _enable_linear_fake_quant, "4w-qat": _enable_linear_fake_quant}
 
 
 def get_quantizer_mode(quantizer: Optional[Callable]) -> Optional[str]:
-    """"8da4w-qat" for :class:`Int8DynActInt4WeightQATQuantizer`, None for anything unknown."""
+    """"8da4w-qat" for :class:`Int8DynActInt4WeightQATQuantizer`, "4w-qat" for :class:`Int4WeightOnlyQATQuantizer`,
+    None for anything unknown."""
     return _quantizer_to_mode.get(type(quantizer), None)
 
 
