@@ -229,3 +229,42 @@ def test_weight_only_int4_qat_prepare_train_convert():
     assert bits_equal(conv(x.to(DEV)), y_ref)
     sd = conv.state_dict()
     assert set(sd) == {"weight", "scales_and_zeros"}
+
+
+def test_post_training_quantizers_use_the_convert_arithmetic():
+    """Int8DynActInt4WeightQuantizer / Int4WeightOnlyQuantizer `.quantize(model)` (torchtune/training/quantization.py:79-121,
+    what recipes/quantize.py:94 calls for the non-QAT modes) give the layers that QAT `convert` gives for the same weights."""
+    from torchtune_amd.qat import Int4WeightOnlyQATQuantizer, WeightOnlyInt4Linear
+
+    gen = torch.Generator().manual_seed(33)
+    K, N = 512, 128
+    W = (torch.randn(N, K, generator=gen) * 0.03).to(torch.bfloat16)
+    b = (torch.randn(N, generator=gen) * 0.1).to(torch.bfloat16)
+    x = torch.randn(5, K, generator=gen).to(torch.bfloat16).to(DEV)
+
+    def fresh(bias):
+        m = nn.Sequential(nn.Linear(K, N, bias=bias), nn.ReLU(), nn.Sequential(nn.Linear(N, 128, bias=False))).to(torch.bfloat16)
+        with torch.no_grad():
+            m[0].weight.copy_(W)
+            if bias:
+                m[0].bias.copy_(b)
+        return m.to(DEV)
+
+    ptq = quantization.Int8DynActInt4WeightQuantizer(groupsize=32).quantize(fresh(True))
+    assert isinstance(ptq[0], Int8DynActInt4WeightLinear) and isinstance(ptq[2][0], Int8DynActInt4WeightLinear)
+    qz = Int8DynActInt4WeightQATQuantizer(groupsize=32, precision=torch.bfloat16)
+    qat = qz.convert(qz.prepare(fresh(True)))
+    assert torch.equal(ptq[0].weight, qat[0].weight) and torch.equal(ptq[0].scales, qat[0].scales)
+    assert bits_equal(ptq[0](x), qat[0](x))  # (the second layer is randomly initialised per model)
+    wq, ws, _ = fq.quantize_per_group_int4(W, 32)
+    assert torch.equal(ptq[0].weight.cpu(), wq) and torch.equal(ptq[0].scales.cpu(), ws)
+
+    ptq4 = quantization.Int4WeightOnlyQuantizer(groupsize=64).quantize(fresh(True))
+    assert isinstance(ptq4[0], WeightOnlyInt4Linear) and ptq4[0].bias is not None
+    q4 = Int4WeightOnlyQATQuantizer(groupsize=64)
+    qat4 = q4.convert(q4.prepare(fresh(False)))
+    assert torch.equal(ptq4[0].weight, qat4[0].weight) and bits_equal(ptq4[0].scales_and_zeros, qat4[0].scales_and_zeros)
+    w_fq, _, _ = fq.fq_per_group_uint4_asym(W, 64)
+    torch.testing.assert_close(ptq4[0](x).float().cpu(), x.float().cpu() @ w_fq.float().T + b.float(), rtol=1e-2, atol=1e-2)
+    with pytest.raises(ValueError, match="divisible by groupsize"):
+        quantization.Int8DynActInt4WeightQuantizer(groupsize=256).quantize(nn.Sequential(nn.Linear(96, 8)).to(DEV))

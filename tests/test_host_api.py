@@ -314,6 +314,27 @@ def test_weight_only_int4_quantizer_prepare_and_toggles_on_cpu():
     assert conv.scales_and_zeros.shape == (8, 64, 2) and conv.scales_and_zeros.dtype == torch.bfloat16
 
 
+def test_quantizer_modes_cover_the_reference_table():
+    """Every entry of the reference's mode tables (torchtune/training/quantization.py:94-97,124-127,141-163)."""
+    expect = {
+        quantization.Int8DynActInt4WeightQuantizer: "8da4w",
+        quantization.Int8DynActInt4WeightQATQuantizer: "8da4w-qat",
+        quantization.Int4WeightOnlyQuantizer: "4w",
+        quantization.Int4WeightOnlyQATQuantizer: "4w-qat",
+        quantization.Int4WeightOnlyQATQuantizerModuleSwap: "4w-qat-module-swap",
+        quantization.Int8DynActInt4WeightQATQuantizerModuleSwap: "8da4w-qat-module-swap",
+    }
+    for cls, mode in expect.items():
+        assert quantization.get_quantizer_mode(cls()) == mode
+        has_toggle = "qat" in mode
+        assert (quantization._get_enable_fake_quant(mode) is not None) == has_toggle
+        assert (quantization._get_disable_fake_quant(mode) is not None) == has_toggle
+    assert quantization.Int8DynActInt4WeightQuantizer().groupsize == 256
+    assert (quantization.Int4WeightOnlyQuantizer().groupsize, quantization.Int4WeightOnlyQuantizer().inner_k_tiles) == (128, 8)
+    assert quantization.disable_8da4w_fake_quant_module_swap is quantization._disable_linear_fake_quant
+    assert quantization.enable_4w_fake_quant_module_swap is quantization._enable_linear_fake_quant
+
+
 def test_swap_lora_linear_with_qat():
     model = nn.Sequential(LoRALinear(64, 64, 4, 1.0), nn.Sequential(LoRALinear(64, 32, 4, 1.0)))
     quantization.swap_lora_linear_with_qat(model, None, FakeQuantizeConfig(torch.int4, group_size=32))

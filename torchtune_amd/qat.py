@@ -431,7 +431,6 @@ class WeightOnlyInt4Linear(nn.Module):
                  inner_k_tiles: int = 8, precision: torch.dtype = torch.bfloat16,
                  scales_precision: torch.dtype = torch.bfloat16) -> None:
         super().__init__()
-        assert not bias, "require bias=False"
         if not _check_linear_int4_k(in_features, groupsize, inner_k_tiles):
             raise ValueError("in_features must be divisible by groupsize and by 16 * inner_k_tiles")
         self.in_features = in_features
@@ -445,6 +444,7 @@ class WeightOnlyInt4Linear(nn.Module):
             "scales_and_zeros",
             torch.zeros((in_features // groupsize, out_features, 2), dtype=scales_precision, device=device),
         )
+        self.bias = nn.Parameter(torch.zeros(out_features, dtype=precision, device=device), requires_grad=False) if bias else None
 
     def dense_weight(self) -> torch.Tensor:
         sz = self.scales_and_zeros
@@ -453,7 +453,7 @@ class WeightOnlyInt4Linear(nn.Module):
         return ops.dequantize_per_group_uint4(self.weight, scale, zero, self.groupsize, self.precision)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        return F.linear(x.to(self.precision), self.dense_weight())
+        return F.linear(x.to(self.precision), self.dense_weight(), self.bias)
 
 
 class Int4WeightOnlyQATQuantizer:
@@ -509,3 +509,50 @@ class Int4WeightOnlyQATQuantizer:
             else:
                 self.convert(child)
         return model
+
+
+# ---------------------------------------------------------------------------------------------------
+# post-training quantisation with the same arithmetic (what recipes/quantize.py runs for the non-QAT modes)
+# ---------------------------------------------------------------------------------------------------
+def quantize_linears_8da4w(model: nn.Module, groupsize: int) -> nn.Module:
+    """Swap every ``nn.Linear`` for :class:`Int8DynActInt4WeightLinear` holding the int4 codes of its weight."""
+    for name, child in list(model.named_children()):
+        if type(child) is nn.Linear:
+            if child.in_features % groupsize != 0:
+                raise ValueError(f"{name}: in_features ({child.in_features}) must be divisible by groupsize ({groupsize})")
+            new = Int8DynActInt4WeightLinear(
+                child.in_features, child.out_features, child.bias is not None, device=child.weight.device,
+                groupsize=groupsize, precision=child.weight.dtype, scales_precision=torch.float32,
+            )
+            q, scale, zeros = ops.quantize_per_group_int4(child.weight.detach(), groupsize)
+            new.weight.copy_(q)
+            new.scales.copy_(scale)
+            new.zeros.copy_(zeros)
+            if child.bias is not None:
+                new.bias = nn.Parameter(child.bias.detach(), requires_grad=False)
+            setattr(model, name, new)
+        else:
+            quantize_linears_8da4w(child, groupsize)
+    return model
+
+
+def quantize_linears_4w(model: nn.Module, groupsize: int, inner_k_tiles: int) -> nn.Module:
+    """Swap every ``nn.Linear`` for :class:`WeightOnlyInt4Linear` holding the uint4 codes of its weight."""
+    for name, child in list(model.named_children()):
+        if type(child) is nn.Linear:
+            if not _check_linear_int4_k(child.in_features, groupsize, inner_k_tiles):
+                raise ValueError(f"{name}: in_features ({child.in_features}) must be divisible by groupsize ({groupsize}) "
+                                 f"and by 16 * inner_k_tiles ({16 * inner_k_tiles})")
+            new = WeightOnlyInt4Linear(
+                child.in_features, child.out_features, child.bias is not None, device=child.weight.device, groupsize=groupsize,
+                inner_k_tiles=inner_k_tiles, precision=child.weight.dtype, scales_precision=torch.bfloat16,
+            )
+            q, scale, zero = ops.quantize_per_group_uint4(child.weight.detach(), groupsize, torch.bfloat16)
+            new.weight.copy_(q)
+            new.scales_and_zeros.copy_(torch.stack([scale.t(), zero.t()], dim=-1).to(torch.bfloat16))
+            if child.bias is not None:
+                new.bias = nn.Parameter(child.bias.detach(), requires_grad=False)
+            setattr(model, name, new)
+        else:
+            quantize_linears_4w(child, groupsize, inner_k_tiles)
+    return model
