@@ -316,3 +316,36 @@ def test_empty_single_row_and_ragged_token_counts():
         assert xd.grad.shape == xd.shape and layer.lora_a.weight.grad.shape == (r, K)
         if x.numel() == 0:
             assert float(layer.lora_b.weight.grad.abs().sum()) == 0.0
+
+
+def test_token_dimension_beyond_32_bit_offsets_is_split_into_row_ranges():
+    """M * K * 2 bytes >= 2^32: the fused GEMM addresses activations with 32-bit offsets per launch, so the library
+    cuts the token dimension into row ranges.  Compared on the first rows, the rows around the cut and the last rows
+    against the same call on those rows alone (bit-equal: a row's result does not depend on its neighbours)."""
+    K, N, r = 28672, 256, 16
+    M = (1 << 32) // (2 * K) + 700  # 75 598 rows, 4.34 GB of activations
+    g = torch.Generator(device=DEV).manual_seed(11)
+    t = to_nf4((torch.randn(N, K, device=DEV, generator=g) * 0.02).to(BF))
+    x = torch.empty(M, K, device=DEV, dtype=BF)
+    for r0 in range(0, M, 8192):  # filled in slices: no fp32 copy of the whole tensor
+        x[r0:r0 + 8192] = torch.randn(min(8192, M - r0), K, device=DEV, generator=g).to(BF)
+    h = torch.randn(M, r, device=DEV, generator=g).to(BF)
+    B = (torch.randn(N, r, device=DEV, generator=g) * 0.05).to(BF)
+    bs, bst = t.block_scalers(), t.backward_copy()[1]
+    y = ops.nf4_lora_linear_fwd(x, t.quantized_data, bs, N, h, B, 2.0, None, block_scalers_t=bst)
+    assert y.shape == (M, N)
+    cut = ((1 << 32) - 1) // (2 * K) // 256 * 256
+    assert 0 < cut < M
+    for lo, hi in ((0, 512), (cut - 256, cut + 256), (M - 300, M)):
+        part = ops.nf4_lora_linear_fwd(x[lo:hi].contiguous(), t.quantized_data, bs, N, h[lo:hi].contiguous(), B, 2.0, None,
+                                       block_scalers_t=bst)
+        assert torch.equal(y[lo:hi], part)
+    D = t.get_original_weight().float()
+    ref = x[M - 300:].float() @ D.T + 2.0 * (h[M - 300:].float() @ B.float().T)
+    torch.testing.assert_close(y[M - 300:].float(), ref, rtol=1e-2, atol=1e-2)
+    # grad-input with a long token dimension: contraction over N = 256, output M x K (also > 2^32 bytes)
+    gy = torch.randn(M, N, device=DEV, generator=g).to(BF)
+    gx = ops.nf4_linear_bwd_dx(gy, t.quantized_data, bs, K, transposed=t.backward_copy())
+    assert gx.shape == (M, K)
+    torch.testing.assert_close(gx[M - 300:].float(), gy[M - 300:].float() @ D, rtol=1e-2, atol=1e-2)
+    torch.testing.assert_close(gx[:300].float(), gy[:300].float() @ D, rtol=1e-2, atol=1e-2)

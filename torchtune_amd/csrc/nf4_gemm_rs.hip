@@ -495,11 +495,21 @@ int launch_rs(RsArgs& g, hipStream_t s) {
 int run_gemm_rs(const void* X, const uint8_t* codes, const void* scal, int mode, const void* lX, const void* lW,
                 bool lw_row_major, int R, float lscale, const void* bias, const void* cscale, void* C, int64_t M, int64_t Nout,
                 int64_t Kc, hipStream_t s) {
-  // per-lane byte offsets inside the kernel are 32-bit
-  TT_REQUIRE(M * Kc * 2 < (int64_t(1) << 32) && Nout * Kc / 2 < (int64_t(1) << 32) && Nout * (Kc / 64) * 4 < (int64_t(1) << 32) &&
-                 M * Nout * 2 < (int64_t(1) << 40),
-             "nf4_gemm: operand too large for 32-bit offsets (M=%lld Nout=%lld Kc=%lld); split the token dimension", (long long)M,
-             (long long)Nout, (long long)Kc);
+  // per-lane byte offsets inside the kernel are 32-bit: the weight must fit them, and a token dimension too long for
+  // them is cut into row ranges (multiples of the 256-row tile) that are launched one after the other
+  TT_REQUIRE(Nout * Kc / 2 < (int64_t(1) << 32) && Nout * (Kc / 64) * 4 < (int64_t(1) << 32) && Kc * 2 * 256 < (int64_t(1) << 32),
+             "nf4_gemm: weight too large for 32-bit offsets (Nout=%lld Kc=%lld)", (long long)Nout, (long long)Kc);
+  const int64_t max_rows = (((int64_t(1) << 32) - 1) / (Kc * 2)) / 256 * 256;
+  if (M > max_rows) {
+    for (int64_t r0 = 0; r0 < M; r0 += max_rows) {
+      const int64_t rows = M - r0 < max_rows ? M - r0 : max_rows;
+      const int rc = run_gemm_rs(reinterpret_cast<const uint16_t*>(X) + r0 * Kc, codes, scal, mode,
+                                 lX ? reinterpret_cast<const uint16_t*>(lX) + r0 * R : nullptr, lW, lw_row_major, R, lscale, bias,
+                                 cscale, reinterpret_cast<uint16_t*>(C) + r0 * Nout, rows, Nout, Kc, s);
+      if (rc != TTAMD_OK) return rc;
+    }
+    return TTAMD_OK;
+  }
   RsArgs g;
   g.X = reinterpret_cast<const uint16_t*>(X);
   g.codes = codes;
