@@ -271,17 +271,21 @@ void ref_fq_per_group_uint4_asym(const void* w, int is_bf16, int qp_bf16, int64_
 
 /* Shortcut 1: with y = 1/a divided once per block, q = fma(fma(-x*y, a, x), y, x*y) must round to the same
  * bf16 as the correctly rounded x / a.  Enumerates every bf16 divisor a with bit pattern in [a_lo, a_hi) and
- * every bf16 numerator 0 <= x <= a (signs are symmetric); returns the number of pairs that differ. */
+ * every bf16 numerator 0 <= x <= a (signs are symmetric); returns the number of pairs that differ.  The `_upto`
+ * form takes numerators up to max_quotient * a (the weight-only uint4 kernel divides a group's offsets, up to 15 steps
+ * and a rounding's worth more, by its scale). */
 #if defined(__x86_64__)
 __attribute__((target("fma")))
 #endif
-int64_t ref_check_shared_reciprocal_division(int a_lo, int a_hi) {
+int64_t ref_check_shared_reciprocal_division_upto(int a_lo, int a_hi, float max_quotient) {
   int64_t bad = 0;
   for (int ai = a_lo; ai < a_hi; ++ai) {
     const float a = float_of((uint32_t)ai << 16);
     const float y = 1.0f / a;
-    for (int xi = 0; xi <= ai; ++xi) {
+    const float top = a * max_quotient;
+    for (int xi = 0; xi < 0x7F80; ++xi) {
       const float x = float_of((uint32_t)xi << 16);
+      if (x > top) break;
       const float q0 = x * y;
       const float r = fmaf(-q0, a, x);
       const float q1 = fmaf(r, y, q0);
@@ -289,6 +293,13 @@ int64_t ref_check_shared_reciprocal_division(int a_lo, int a_hi) {
     }
   }
   return bad;
+}
+
+#if defined(__x86_64__)
+__attribute__((target("fma")))
+#endif
+int64_t ref_check_shared_reciprocal_division(int a_lo, int a_hi) {
+  return ref_check_shared_reciprocal_division_upto(a_lo, a_hi, 1.0f);
 }
 
 /* Shortcut 2: the code of a scaled bf16 value is looked up in a table that only spans magnitudes 2^-5 .. 1.

@@ -162,6 +162,9 @@ def test_uint4_asym_fake_quant_convert_and_dequant_bit_exact(dtype, qp, g):
     w[0, :g] = 0.25          # constant group: the 1e-6 floor of the scale
     w[1, :g] = w[1, :g].abs() + 1.0  # all-positive group far from zero
     w[2, :g] *= 1e-5         # tiny dynamic range
+    w[3, :g] = 1.0           # a range of one bf16 ulp next to 1.0: the rounded zero point pushes offsets far
+    w[3, 1] = 1.0078125      # beyond 15 steps (they clamp)
+    w[4, :g] = w[4, :g] * 3e3 - 7e4  # large magnitudes, range much smaller than the offset
     want, ws, wz = fq.fq_per_group_uint4_asym(w, g, qp)
     got, gs, gz = ops.fq_per_group_uint4_asym(w.to(DEV), g, qp)
     assert bits_equal(got.cpu(), want)

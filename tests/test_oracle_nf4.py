@@ -229,6 +229,23 @@ def test_shared_reciprocal_division_is_exact_for_bf16(c_oracle):
     assert c_oracle.ref_check_shared_reciprocal_division(0x0001, 0x0100) > 0
 
 
+def test_shared_reciprocal_division_is_exact_for_uint4_group_offsets(c_oracle):
+    """The weight-only uint4 fake-quant kernel uses the same shortcut for (w - lowest) / scale: divisors are bf16
+    scales >= 1e-6, quotients of interest reach 15.5 (larger ones clamp to 15).  Enumerate every bf16 divisor from
+    2^-20 up and every bf16 numerator up to 17 times the divisor."""
+    import ctypes
+    from concurrent.futures import ThreadPoolExecutor
+
+    fn = c_oracle.ref_check_shared_reciprocal_division_upto
+    fn.restype = ctypes.c_int64
+    fn.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_float]
+    lo, hi = 0x3580, 0x7F80  # 2^-20 (below bf16(1e-6) = 0x3586) .. the largest finite bf16
+    edges = [lo + (hi - lo) * i // 32 for i in range(33)]
+    with ThreadPoolExecutor(max_workers=8) as pool:
+        bad = list(pool.map(lambda i: fn(edges[i], edges[i + 1], 17.0), range(32)))
+    assert sum(bad) == 0
+
+
 def test_code_table_premises_and_monotone_codes(c_oracle):
     """Every bf16 scaled value below 2^-5 is the zero code and NaN is code 0 (what lets the kernel's table span only
     2^-5..1); inside the table the code never decreases with the value."""
