@@ -22,7 +22,10 @@ Eager-PyTorch restatement of what the reference runs through ``torchao.quantizat
 Parity status: PARITY UNPINNED against torchao itself (not importable here; the reference holds no vectors
 for these functions).  Pinned instead by closed forms and invariants in tests/test_oracle_fake_quant.py
 (scale = (max-min)/255 and the zero-point formula on hand-built rows, outputs on the scale*(q-zp) grid,
-idempotence for fixed qparams, exhaustive tiny cases) and by the independent C restatement oracle/nf4_ref.c.
+idempotence for fixed qparams, exhaustive tiny cases), by the independent C restatement oracle/nf4_ref.c, and by
+agreement (qparams, codes and values, bit for bit on fp32 inputs) with the implementation of the same per-token /
+per-group scheme that ships inside PyTorch itself, ``torch.ops.quantized_decomposed``
+(``torch/ao/quantization/fx/_decomposed.py``).
 
 Numerics: qparams are computed in fp32 from the fp32-promoted input; eps = finfo(float32).eps;
 ``round`` is round-half-to-even; the dequantised value is ``(q - zp)`` cast to the input dtype, times the fp32

@@ -205,3 +205,49 @@ def test_uint4_asym_two_restatements_agree(c_oracle, dtype, qp):
         assert torch.equal(torch.stack([packed >> 4, packed & 15], dim=-1).reshape(16, 512), qc)
         assert bits_equal(out, fc)
         assert bits_equal(fq.dequantize_per_group_uint4(packed, scale, zero, g, dtype), out)
+
+
+# ---- an independent implementation: the quantized_decomposed ops that ship inside PyTorch itself -------------
+def _decomposed_ops():
+    from torch.ao.quantization.fx import _decomposed  # noqa: F401  (registers torch.ops.quantized_decomposed)
+
+    return torch.ops.quantized_decomposed
+
+
+def test_per_token_agrees_with_pytorchs_own_decomposed_ops():
+    """torch/ao/quantization/fx/_decomposed.py holds PyTorch's implementation of the same 8-bit dynamic per-token
+    asymmetric scheme (qparams after XNNPACK, quantise = mul(1/scale).add(zp).round().clamp, dequantise = (q - zp) * scale).
+    The oracle must give the same qparams, codes and fake-quantised values on fp32 rows."""
+    ops = _decomposed_ops()
+    gen = torch.Generator().manual_seed(7)
+    x = torch.randn(64, 384, generator=gen) * 2.5
+    x[0] = 0
+    x[1] = x[1].abs() + 0.5
+    x[2] = -x[2].abs() - 0.5
+    x[3, ::3] *= 40
+    scale, zp = ops.choose_qparams_per_token_asymmetric(x, torch.int8)
+    got, s, z = fq.fq_per_token_int8_asym(x)
+    assert torch.equal(scale.to(torch.float32).reshape(-1), s) and torch.equal(zp.to(torch.int32).reshape(-1), z)
+    q = ops.quantize_per_token(x, scale.to(torch.float32), zp.to(torch.int32), -128, 127, torch.int8)
+    dq = ops.dequantize_per_token(q, scale.to(torch.float32), zp.to(torch.int32), -128, 127, torch.int8, torch.float32)
+    assert bits_equal(dq, got)
+    q_oracle, _ = fq._fake_quantize(x, s[:, None], z[:, None], -128, 127)
+    assert torch.equal(q.to(torch.float32), q_oracle)
+
+
+@pytest.mark.parametrize("g", [32, 256])
+def test_per_group_agrees_with_pytorchs_own_decomposed_ops(g):
+    """Same for the group-wise int4 weights: with the oracle's scales, PyTorch's quantize_per_channel_group /
+    dequantize_per_channel_group give the oracle's int4 codes and fake-quantised weight."""
+    ops = _decomposed_ops()
+    gen = torch.Generator().manual_seed(8)
+    w = torch.randn(48, 512, generator=gen) * 0.03
+    w[0, :g] = 0
+    want, scale = fq.fq_per_group_int4_sym(w, g)
+    codes, s2, zeros = fq.quantize_per_group_int4(w, g)
+    assert torch.equal(scale, s2) and torch.all(zeros == 0)
+    zp = torch.zeros_like(scale, dtype=torch.int32)
+    q = ops.quantize_per_channel_group(w, scale, zp, -8, 7, torch.int8, g)
+    assert torch.equal(q, codes)
+    dq = ops.dequantize_per_channel_group(q, scale, zp, -8, 7, torch.int8, g, torch.float32)
+    assert bits_equal(dq, want)
