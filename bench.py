@@ -257,6 +257,9 @@ def main() -> int:
     ap.add_argument("--optimizer-steps", type=int, default=3,
                     help="after the timed fwd+bwd steps, time this many steps that also run the recipe's fused AdamW "
                          "(reported beside the metric as `with_adamw`; 0 = skip)")
+    ap.add_argument("--qat-scales", default="float32", choices=["float32", "bfloat16"],
+                    help="scales_precision of the QAT workload: float32 is the reference quantizer's default, bfloat16 rounds "
+                         "every scale before it quantises and dequantises")
     ap.add_argument("--calibration-copy-mib", type=int, default=0,
                     help="before the steps, run one elementwise kernel that reads and writes this many MiB: the known-size "
                          "dispatch that FETCH_SIZE / WRITE_SIZE counter runs are scaled by")
@@ -277,7 +280,8 @@ def main() -> int:
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
     if qat:
-        model = build_qat_decoder(shape_name, groupsize=qat_group, device=dev, seed=0, activation_checkpointing=ac)
+        model = build_qat_decoder(shape_name, groupsize=qat_group, device=dev, seed=0, activation_checkpointing=ac,
+                                  scales_precision=getattr(torch, args.qat_scales))
     else:
         model = build_qlora_decoder(shape_name, rank, alpha, device=dev, seed=0, activation_checkpointing=ac)
     gen = torch.Generator(device=dev).manual_seed(1)
@@ -333,9 +337,10 @@ def main() -> int:
             "dtype": "bf16",
             "data": "synthetic (uniform random token ids, random-init N(0,0.02) bf16 weights)",
             "config": {
-                "workload": f"{shape_name}-shaped decoder, every linear (incl. output) 8da4w fake-quantised: per-token int8 "
-                            f"activations, per-group({qat_group}) int4 weights, batch {batch} x seq {seq}, fwd+bwd with weight "
-                            "gradients, output projection and cross-entropy",
+                "workload": f"{shape_name}-shaped decoder, every linear (incl. output) 8da4w fake-quantised as the reference's "
+                            "quantizer does it: per-token asymmetric int8 activations (min/max with zero point), "
+                            f"per-group({qat_group}) symmetric int4 weights, {args.qat_scales} scales, batch {batch} x seq {seq}, "
+                            "fwd+bwd with weight gradients, output projection and cross-entropy",
                 "global_batch": batch,
                 "seq_len": seq,
                 "loss": float(loss),

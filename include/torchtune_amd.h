@@ -220,9 +220,12 @@ int ttamd_lora_bwd_bf16(const void* gy, const void* x, const void* h, const void
  *
  * x [rows,K] `dtype`; out [rows,K] `dtype` = dequantise(quantise(x)) with per-row asymmetric int8 qparams computed
  * in fp32; scale out [rows] fp32 and zero_point out [rows] int32 may be NULL.  K % 8 == 0.
+ * qparam_dtype = the config's scale_precision (TTAMD_F32, the reference's default, or TTAMD_BF16): with bf16 the scale
+ * is rounded to bf16 after the zero point has been chosen, and the rounded scale quantises and dequantises (it is also
+ * what `scale` receives, widened).  The same argument of the two group-wise entry points below means the same.
  * The straight-through backward is the identity and needs no kernel.
  */
-int ttamd_fq_per_token_int8_asym(const void* x, int dtype, int64_t rows, int64_t K, void* out, float* scale,
+int ttamd_fq_per_token_int8_asym(const void* x, int dtype, int64_t rows, int64_t K, int qparam_dtype, void* out, float* scale,
                                  int32_t* zero_point, void* stream);
 
 /*
@@ -232,7 +235,7 @@ int ttamd_fq_per_token_int8_asym(const void* x, int dtype, int64_t rows, int64_t
  * w [rows,K] `dtype`, groups of `group_size` consecutive elements along K (K % group_size == 0, group_size a
  * power of two in [8, 512]); out [rows,K] `dtype`; scale out [rows, K/group_size] fp32 may be NULL.
  */
-int ttamd_fq_per_group_int4_sym(const void* w, int dtype, int64_t rows, int64_t K, int group_size, void* out,
+int ttamd_fq_per_group_int4_sym(const void* w, int dtype, int64_t rows, int64_t K, int group_size, int qparam_dtype, void* out,
                                 float* scale, void* stream);
 
 /*
@@ -240,8 +243,8 @@ int ttamd_fq_per_group_int4_sym(const void* w, int dtype, int64_t rows, int64_t 
  * q out [rows,K] int8 holding values in [-8,7]; scale out [rows,K/group_size] fp32; zero_point out
  * [rows,K/group_size] fp32 (all zero for the symmetric scheme; may be NULL).
  */
-int ttamd_quantize_per_group_int4(const void* w, int dtype, int64_t rows, int64_t K, int group_size, int8_t* q,
-                                  float* scale, float* zero_point, void* stream);
+int ttamd_quantize_per_group_int4(const void* w, int dtype, int64_t rows, int64_t K, int group_size, int qparam_dtype,
+                                  int8_t* q, float* scale, float* zero_point, void* stream);
 
 /*
  * Dense weight of the converted 8da4w linear (what Int8DynActInt4WeightLinear.forward rebuilds before its matmul; the

@@ -27,7 +27,8 @@ agreement (qparams, codes and values, bit for bit on fp32 inputs) with the imple
 per-group scheme that ships inside PyTorch itself, ``torch.ops.quantized_decomposed``
 (``torch/ao/quantization/fx/_decomposed.py``).
 
-Numerics: qparams are computed in fp32 from the fp32-promoted input; eps = finfo(float32).eps;
+Numerics: qparams are computed in fp32 from the fp32-promoted input (and cast to the config's ``scale_precision``
+— float32 by default, the reference's documented setting — before they are used); eps = finfo(float32).eps;
 ``round`` is round-half-to-even; the dequantised value is ``(q - zp)`` cast to the input dtype, times the fp32
 scale, cast back to the input dtype.  The backward mask ``(q >= qmin) & (q <= qmax)`` is evaluated on the
 clamped ``q`` and is therefore all ones: the gradient passes straight through.
@@ -66,9 +67,16 @@ def _fake_quantize(x: torch.Tensor, scale: torch.Tensor, zp: torch.Tensor, qmin:
     return q, dq
 
 
-def fq_per_token_int8_asym(x: torch.Tensor):
-    """returns (fake-quantised x, scale [rows] fp32, zero_point [rows] int32)"""
+def _to_scale_precision(scale: torch.Tensor, scale_dtype: torch.dtype) -> torch.Tensor:
+    """The qparams are cast to the config's ``scale_precision`` before use; the value is widened back for the arithmetic."""
+    return scale.to(scale_dtype).to(torch.float32)
+
+
+def fq_per_token_int8_asym(x: torch.Tensor, scale_dtype: torch.dtype = torch.float32):
+    """returns (fake-quantised x, scale [rows] fp32, zero_point [rows] int32); with ``scale_dtype=bfloat16`` the scale is
+    rounded to bf16 after the zero point has been chosen, and the rounded scale quantises and dequantises"""
     scale, zp = choose_qparams_per_token_asym(x)
+    scale = _to_scale_precision(scale, scale_dtype)
     _, dq = _fake_quantize(x, scale, zp, -128, 127)
     return dq, scale.reshape(-1), zp.reshape(-1)
 
@@ -87,20 +95,20 @@ def choose_qparams_per_group_sym(w: torch.Tensor, group_size: int):
     return scale.clamp(min=_EPS)
 
 
-def fq_per_group_int4_sym(w: torch.Tensor, group_size: int):
+def fq_per_group_int4_sym(w: torch.Tensor, group_size: int, scale_dtype: torch.dtype = torch.float32):
     """returns (fake-quantised w, scale [rows, K/g] fp32)"""
     rows, K = w.shape
-    scale = choose_qparams_per_group_sym(w, group_size)
+    scale = _to_scale_precision(choose_qparams_per_group_sym(w, group_size), scale_dtype)
     wg = w.view(rows, K // group_size, group_size)
     zp = torch.zeros_like(scale, dtype=torch.int32)
     _, dq = _fake_quantize(wg, scale[..., None], zp[..., None], -8, 7)
     return dq.reshape(rows, K), scale
 
 
-def quantize_per_group_int4(w: torch.Tensor, group_size: int):
+def quantize_per_group_int4(w: torch.Tensor, group_size: int, scale_dtype: torch.dtype = torch.float32):
     """convert(): returns (int8 tensor of int4 values [rows,K], scale [rows,K/g] fp32, zeros [rows,K/g] fp32)"""
     rows, K = w.shape
-    scale = choose_qparams_per_group_sym(w, group_size)
+    scale = _to_scale_precision(choose_qparams_per_group_sym(w, group_size), scale_dtype)
     wg = w.view(rows, K // group_size, group_size)
     q = torch.clamp(torch.round(wg * (1.0 / scale[..., None])), -8, 7).to(torch.int8)
     return q.reshape(rows, K), scale, torch.zeros_like(scale)

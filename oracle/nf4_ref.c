@@ -161,8 +161,8 @@ void ref_nf4_dequantize(const uint8_t* qdata, const int8_t* qscalers, const void
 static const float F32_EPS = 1.1920928955078125e-07f;
 
 /* per-token (per-row) asymmetric int8; qparams in fp32.  scale_out / zp_out may be NULL */
-void ref_fq_per_token(const void* x, int is_bf16, int64_t rows, int64_t K, void* out, float* scale_out,
-                      int32_t* zp_out) {
+void ref_fq_per_token_qp(const void* x, int is_bf16, int qp_bf16, int64_t rows, int64_t K, void* out, float* scale_out,
+                         int32_t* zp_out) {
   for (int64_t r = 0; r < rows; ++r) {
     float mn = load_elem(x, r * K, is_bf16), mx = mn;
     for (int64_t k = 1; k < K; ++k) {
@@ -178,6 +178,7 @@ void ref_fq_per_token(const void* x, int is_bf16, int64_t rows, int64_t K, void*
     float zp = ((-128.0f + dmin) + (127.0f + dmax) > 0.0f) ? (-128.0f - dmin) : (127.0f - dmax);
     zp = zp < -128.0f ? -128.0f : (zp > 127.0f ? 127.0f : zp);
     zp = rintf(zp);
+    if (qp_bf16) scale = to_bf16(scale); /* scale_precision = bf16: the rounded scale quantises and dequantises */
     const float inv = 1.0f / scale;
     for (int64_t k = 0; k < K; ++k) {
       float q = rintf(load_elem(x, r * K + k, is_bf16) * inv) + zp;
@@ -188,6 +189,11 @@ void ref_fq_per_token(const void* x, int is_bf16, int64_t rows, int64_t K, void*
     if (scale_out) scale_out[r] = scale;
     if (zp_out) zp_out[r] = (int32_t)zp;
   }
+}
+
+void ref_fq_per_token(const void* x, int is_bf16, int64_t rows, int64_t K, void* out, float* scale_out,
+                      int32_t* zp_out) {
+  ref_fq_per_token_qp(x, is_bf16, 0, rows, K, out, scale_out, zp_out);
 }
 
 static float group_scale(const void* w, int64_t base, int g, int is_bf16) {
@@ -206,11 +212,12 @@ static float group_scale(const void* w, int64_t base, int g, int is_bf16) {
 }
 
 /* per-group symmetric int4 along K; fq_out and/or q_out may be NULL */
-void ref_fq_per_group(const void* w, int is_bf16, int64_t rows, int64_t K, int g, void* fq_out, int8_t* q_out,
-                      float* scale_out) {
+void ref_fq_per_group_qp(const void* w, int is_bf16, int qp_bf16, int64_t rows, int64_t K, int g, void* fq_out,
+                         int8_t* q_out, float* scale_out) {
   for (int64_t r = 0; r < rows; ++r)
     for (int64_t k0 = 0; k0 < K; k0 += g) {
-      const float scale = group_scale(w, r * K + k0, g, is_bf16);
+      float scale = group_scale(w, r * K + k0, g, is_bf16);
+      if (qp_bf16) scale = to_bf16(scale);
       const float inv = 1.0f / scale;
       for (int i = 0; i < g; ++i) {
         float q = rintf(load_elem(w, r * K + k0 + i, is_bf16) * inv);
@@ -221,6 +228,11 @@ void ref_fq_per_group(const void* w, int is_bf16, int64_t rows, int64_t K, int g
       }
       if (scale_out) scale_out[r * (K / g) + k0 / g] = scale;
     }
+}
+
+void ref_fq_per_group(const void* w, int is_bf16, int64_t rows, int64_t K, int g, void* fq_out, int8_t* q_out,
+                      float* scale_out) {
+  ref_fq_per_group_qp(w, is_bf16, 0, rows, K, g, fq_out, q_out, scale_out);
 }
 
 /* per-group asymmetric uint4 with a floating-point zero point (the weight-only "4w-qat" scheme), every operation

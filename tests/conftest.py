@@ -31,6 +31,12 @@ def c_oracle():
     lib.ref_fq_per_token.restype = None
     lib.ref_fq_per_group.argtypes = [vp, i32, i64, i64, i32, vp, vp, vp]
     lib.ref_fq_per_group.restype = None
+    lib.ref_fq_per_token_qp.argtypes = [vp, i32, i32, i64, i64, vp, vp, vp]
+    lib.ref_fq_per_token_qp.restype = None
+    lib.ref_fq_per_group_qp.argtypes = [vp, i32, i32, i64, i64, i32, vp, vp, vp]
+    lib.ref_fq_per_group_qp.restype = None
+    lib.ref_fq_per_group_uint4_asym.argtypes = [vp, i32, i32, i64, i64, i32, vp, vp, vp, vp]
+    lib.ref_fq_per_group_uint4_asym.restype = None
     lib.ref_check_shared_reciprocal_division.argtypes = [i32, i32]
     lib.ref_check_shared_reciprocal_division.restype = i64
     lib.ref_check_code_table.argtypes = [vp]

@@ -33,23 +33,25 @@ def c_nf4_dequantize(lib, p: nf4_oracle.NF4Parts) -> torch.Tensor:
     return out.view(p.shape)
 
 
-def c_fq_per_token(lib, x: torch.Tensor):
+def c_fq_per_token(lib, x: torch.Tensor, qp_bf16: bool = False):
     x = x.contiguous()
     rows, K = x.shape
     out = torch.empty_like(x)
     scale = torch.empty(rows, dtype=torch.float32)
     zp = torch.empty(rows, dtype=torch.int32)
-    lib.ref_fq_per_token(ptr(x), int(x.dtype == torch.bfloat16), rows, K, ptr(out), ptr(scale), ptr(zp))
+    lib.ref_fq_per_token_qp(ptr(x), int(x.dtype == torch.bfloat16), int(qp_bf16), rows, K,
+                            ptr(out), ptr(scale), ptr(zp))
     return out, scale, zp
 
 
-def c_fq_per_group(lib, w: torch.Tensor, g: int):
+def c_fq_per_group(lib, w: torch.Tensor, g: int, qp_bf16: bool = False):
     w = w.contiguous()
     rows, K = w.shape
     fq = torch.empty_like(w)
     q = torch.empty(w.shape, dtype=torch.int8)
     scale = torch.empty(rows, K // g, dtype=torch.float32)
-    lib.ref_fq_per_group(ptr(w), int(w.dtype == torch.bfloat16), rows, K, g, ptr(fq), ptr(q), ptr(scale))
+    lib.ref_fq_per_group_qp(ptr(w), int(w.dtype == torch.bfloat16), int(qp_bf16), rows, K, g,
+                            ptr(fq), ptr(q), ptr(scale))
     return fq, q, scale
 
 
@@ -60,8 +62,7 @@ def c_fq_per_group_uint4_asym(lib, w: torch.Tensor, g: int, qp_bf16: bool = True
     q = torch.empty(w.shape, dtype=torch.uint8)
     scale = torch.empty(rows, K // g, dtype=torch.float32)
     zero = torch.empty(rows, K // g, dtype=torch.float32)
-    lib.ref_fq_per_group_uint4_asym(ptr(w), int(w.dtype == torch.bfloat16), int(qp_bf16), rows, K, g, ptr(fq), ptr(q),
-                                    ptr(scale), ptr(zero))
+    lib.ref_fq_per_group_uint4_asym(ptr(w), int(w.dtype == torch.bfloat16), int(qp_bf16), rows, K, g, ptr(fq), ptr(q), ptr(scale), ptr(zero))
     return fq, q, scale, zero
 
 

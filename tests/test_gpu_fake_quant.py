@@ -271,3 +271,45 @@ def test_post_training_quantizers_use_the_convert_arithmetic():
     torch.testing.assert_close(ptq4[0](x).float().cpu(), x.float().cpu() @ w_fq.float().T + b.float(), rtol=1e-2, atol=1e-2)
     with pytest.raises(ValueError, match="divisible by groupsize"):
         quantization.Int8DynActInt4WeightQuantizer(groupsize=256).quantize(nn.Sequential(nn.Linear(96, 8)).to(DEV))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_bf16_scale_precision_bit_exact(dtype):
+    """scale_precision = bfloat16 (BASELINE config 4 asks for bf16 scales; the reference's default is float32): the scale
+    is rounded to bf16 once chosen and the rounded scale quantises and dequantises, in the per-token, the per-group and
+    the convert kernels, and the converted layer reproduces the fake-quantised one."""
+    gen = torch.Generator().manual_seed(41)
+    x = (torch.randn(37, 1024, generator=gen) * 1.9).to(dtype)
+    x[1] = 0
+    want, ws, wz = fq.fq_per_token_int8_asym(x, torch.bfloat16)
+    got, gs, gz = ops.fq_per_token_int8_asym(x.to(DEV), qparam_dtype=torch.bfloat16)
+    assert bits_equal(got.cpu(), want) and torch.equal(gs.cpu(), ws) and torch.equal(gz.cpu(), wz)
+    long_row = (torch.randn(3, 40000, generator=gen) * 1.1).to(dtype)  # the streaming variant of the kernel
+    want, ws, _ = fq.fq_per_token_int8_asym(long_row, torch.bfloat16)
+    got, gs, _ = ops.fq_per_token_int8_asym(long_row.to(DEV), qparam_dtype=torch.bfloat16)
+    assert bits_equal(got.cpu(), want) and torch.equal(gs.cpu(), ws)
+    w = (torch.randn(64, 1024, generator=gen) * 0.02).to(dtype)
+    for g in (32, 256):
+        want, ws = fq.fq_per_group_int4_sym(w, g, torch.bfloat16)
+        got, gs = ops.fq_per_group_int4_sym(w.to(DEV), g, qparam_dtype=torch.bfloat16)
+        assert bits_equal(got.cpu(), want) and torch.equal(gs.cpu(), ws)
+        wq, ws2, _ = fq.quantize_per_group_int4(w, g, torch.bfloat16)
+        gq, gs2, _ = ops.quantize_per_group_int4(w.to(DEV), g, torch.bfloat16)
+        assert torch.equal(gq.cpu(), wq) and torch.equal(gs2.cpu(), ws2)
+    # module level: prepare -> forward -> convert with bf16 scales
+    lin = nn.Sequential(nn.Linear(1024, 64, bias=False)).to(dtype)
+    with torch.no_grad():
+        lin[0].weight.copy_(w)
+    lin = lin.to(DEV)
+    qz = Int8DynActInt4WeightQATQuantizer(groupsize=32, precision=dtype, scales_precision=torch.bfloat16)
+    lin = qz.prepare(lin)
+    xd = x.to(DEV)
+    y_fq = lin(xd)
+    x_fq, _, _ = fq.fq_per_token_int8_asym(x, torch.bfloat16)
+    w_fq, w_s = fq.fq_per_group_int4_sym(w, 32, torch.bfloat16)
+    torch.testing.assert_close(y_fq.float().cpu(), x_fq.float() @ w_fq.float().T, rtol=1e-2, atol=1e-2)
+    assert lin[0].weight_fake_quantizer.scale.dtype == torch.bfloat16
+    assert torch.equal(lin[0].weight_fake_quantizer.scale.float().cpu(), w_s)
+    conv = qz.convert(lin)
+    assert conv[0].scales.dtype == torch.bfloat16 and torch.equal(conv[0].scales.float().cpu(), w_s)
+    assert bits_equal(conv(xd), y_fq)  # the converted layer computes what training saw

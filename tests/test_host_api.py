@@ -77,9 +77,9 @@ def test_argument_validation_needs_no_gpu():
     assert rc == -1 and b"adapter pointers" in lib.ttamd_last_error()
     rc = lib.ttamd_nf4_linear_bwd_dx_bf16(aligned, aligned, aligned, None, None, aligned, aligned, 12, aligned, 8, 64, 64, None)
     assert rc == -1 and b"rank" in lib.ttamd_last_error()
-    rc = lib.ttamd_fq_per_group_int4_sym(aligned, 0, 4, 64, 24, aligned, None, None)
+    rc = lib.ttamd_fq_per_group_int4_sym(aligned, 0, 4, 64, 24, 1, aligned, None, None)
     assert rc == -1 and b"group_size" in lib.ttamd_last_error()
-    rc = lib.ttamd_fq_per_token_int8_asym(aligned, 0, 4, 12, aligned, None, None, None)
+    rc = lib.ttamd_fq_per_token_int8_asym(aligned, 0, 4, 12, 1, aligned, None, None, None)
     assert rc == -1 and b"multiple of 8" in lib.ttamd_last_error()
     with pytest.raises(ValueError, match="multiple of 8"):
         _lib.check(rc, "fq_per_token")

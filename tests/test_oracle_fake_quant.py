@@ -106,21 +106,43 @@ def test_per_group_invariants(dtype, g):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_two_restatements_agree(c_oracle, dtype):
+@pytest.mark.parametrize("scale_dtype", [torch.float32, torch.bfloat16])
+def test_two_restatements_agree(c_oracle, dtype, scale_dtype):
+    qp_bf16 = scale_dtype == torch.bfloat16
     gen = torch.Generator().manual_seed(3)
     x = (torch.randn(64, 512, generator=gen) * 2).to(dtype)
     x[3] = 0
     x[4] = x[4].abs()
-    ot, st, zt = fq.fq_per_token_int8_asym(x)
-    oc, sc, zc = c_fq_per_token(c_oracle, x)
+    ot, st, zt = fq.fq_per_token_int8_asym(x, scale_dtype)
+    oc, sc, zc = c_fq_per_token(c_oracle, x, qp_bf16)
     assert bits_equal(ot, oc) and torch.equal(st, sc) and torch.equal(zt, zc)
     w = (torch.randn(64, 512, generator=gen) * 0.02).to(dtype)
     w[0, :32] = 0
     for g in (8, 32, 128):
-        ft, s1 = fq.fq_per_group_int4_sym(w, g)
-        qt, _, _ = fq.quantize_per_group_int4(w, g)
-        fc, qc, s2 = c_fq_per_group(c_oracle, w, g)
+        ft, s1 = fq.fq_per_group_int4_sym(w, g, scale_dtype)
+        qt, _, _ = fq.quantize_per_group_int4(w, g, scale_dtype)
+        fc, qc, s2 = c_fq_per_group(c_oracle, w, g, qp_bf16)
         assert bits_equal(ft, fc) and torch.equal(qt, qc) and torch.equal(s1, s2)
+
+
+def test_bf16_scale_precision_rounds_the_scale_before_use():
+    """scale_precision = bf16: the scale the kernel reports is a bf16 value, the zero point is the one chosen with the
+    fp32 scale, and outputs lie on the grid of the ROUNDED scale."""
+    gen = torch.Generator().manual_seed(12)
+    x = torch.randn(16, 256, generator=gen) * 1.3
+    o32, s32, z32 = fq.fq_per_token_int8_asym(x)
+    o16, s16, z16 = fq.fq_per_token_int8_asym(x, torch.bfloat16)
+    assert torch.equal(z32, z16) and torch.equal(s16, s32.to(torch.bfloat16).float()) and not torch.equal(s16, s32)
+    k = torch.round(o16 / s16[:, None])
+    assert bits_equal(k * s16[:, None], o16) and not bits_equal(o16, o32)
+    w = torch.randn(8, 256, generator=gen) * 0.02
+    f16, sw16 = fq.fq_per_group_int4_sym(w, 32, torch.bfloat16)
+    _, sw32 = fq.fq_per_group_int4_sym(w, 32)
+    assert torch.equal(sw16, sw32.to(torch.bfloat16).float())
+    kk = torch.round(f16.view(8, 8, 32) / sw16[..., None])
+    assert bits_equal((kk * sw16[..., None]).view(8, 256), f16) and kk.abs().max() <= 8
+    q16, _, _ = fq.quantize_per_group_int4(w, 32, torch.bfloat16)
+    assert torch.equal(q16.float().view(8, 8, 32), kk)
 
 
 def test_straight_through_backward():

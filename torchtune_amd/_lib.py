@@ -72,11 +72,11 @@ SIGNATURES = {
         [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _f32, _c_void_p, _c_void_p, _c_void_p, _i64, _i64, _i64, _int,
          _c_void_p, _size, _c_void_p],
     ),
-    "ttamd_fq_per_token_int8_asym": (_int, [_c_void_p, _int, _i64, _i64, _c_void_p, _c_void_p, _c_void_p, _c_void_p]),
-    "ttamd_fq_per_group_int4_sym": (_int, [_c_void_p, _int, _i64, _i64, _int, _c_void_p, _c_void_p, _c_void_p]),
+    "ttamd_fq_per_token_int8_asym": (_int, [_c_void_p, _int, _i64, _i64, _int, _c_void_p, _c_void_p, _c_void_p, _c_void_p]),
+    "ttamd_fq_per_group_int4_sym": (_int, [_c_void_p, _int, _i64, _i64, _int, _int, _c_void_p, _c_void_p, _c_void_p]),
     "ttamd_quantize_per_group_int4": (
         _int,
-        [_c_void_p, _int, _i64, _i64, _int, _c_void_p, _c_void_p, _c_void_p, _c_void_p],
+        [_c_void_p, _int, _i64, _i64, _int, _int, _c_void_p, _c_void_p, _c_void_p, _c_void_p],
     ),
     "ttamd_dequantize_per_group_int4": (_int, [_c_void_p, _c_void_p, _c_void_p, _int, _i64, _i64, _int, _c_void_p, _c_void_p]),
     "ttamd_fq_per_group_uint4_asym": (

@@ -75,7 +75,9 @@ struct TokenQParams {
 };
 
 // asymmetric int8 qparams from the row extrema (already widened to include 0)
-__device__ __forceinline__ TokenQParams token_qparams(float mn, float mx) {
+// (the zero point is chosen with the fp32 scale; a bf16 qparam precision rounds the scale afterwards, and the rounded
+// scale is what quantises and dequantises)
+__device__ __forceinline__ TokenQParams token_qparams(float mn, float mx, bool qp_bf16) {
   TokenQParams p;
   float scale = (mx - mn) / 255.0f;
   scale = scale > kF32Eps ? scale : kF32Eps;
@@ -83,6 +85,7 @@ __device__ __forceinline__ TokenQParams token_qparams(float mn, float mx) {
   float zp = ((-128.0f + dmin) + (127.0f + dmax) > 0.0f) ? (-128.0f - dmin) : (127.0f - dmax);
   zp = zp < -128.0f ? -128.0f : (zp > 127.0f ? 127.0f : zp);
   p.zp = __builtin_rintf(zp);
+  if (qp_bf16) scale = round_to_bf16(scale);
   p.scale = scale;
   p.inv_scale = 1.0f / scale;
   return p;
@@ -107,7 +110,7 @@ __device__ __forceinline__ void wave_minmax(float& mn, float& mx) {
 template <bool BF16, int NV>
 __global__ __launch_bounds__(256) void fq_per_token_regs_kernel(const void* __restrict__ x, int64_t rows, int64_t K,
                                                                 void* __restrict__ out, float* __restrict__ scale_out,
-                                                                int32_t* __restrict__ zp_out) {
+                                                                int32_t* __restrict__ zp_out, bool qp_bf16) {
   const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= rows) return;
   const int lane = threadIdx.x & 63;
@@ -132,7 +135,7 @@ __global__ __launch_bounds__(256) void fq_per_token_regs_kernel(const void* __re
       mx = fmaxf(mx, v);
     }
   wave_minmax(mn, mx);
-  const TokenQParams p = token_qparams(mn, mx);
+  const TokenQParams p = token_qparams(mn, mx, qp_bf16);
   if (lane == 0) {
     if (scale_out) scale_out[row] = p.scale;
     if (zp_out) zp_out[row] = (int32_t)p.zp;
@@ -153,7 +156,7 @@ __global__ __launch_bounds__(256) void fq_per_token_regs_kernel(const void* __re
 template <bool BF16>
 __global__ __launch_bounds__(256) void fq_per_token_stream_kernel(const void* __restrict__ x, int64_t rows, int64_t K,
                                                                   void* __restrict__ out, float* __restrict__ scale_out,
-                                                                  int32_t* __restrict__ zp_out) {
+                                                                  int32_t* __restrict__ zp_out, bool qp_bf16) {
   const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= rows) return;
   const int lane = threadIdx.x & 63;
@@ -171,7 +174,7 @@ __global__ __launch_bounds__(256) void fq_per_token_stream_kernel(const void* __
     }
   }
   wave_minmax(mn, mx);
-  const TokenQParams p = token_qparams(mn, mx);
+  const TokenQParams p = token_qparams(mn, mx, qp_bf16);
   if (lane == 0) {
     if (scale_out) scale_out[row] = p.scale;
     if (zp_out) zp_out[row] = (int32_t)p.zp;
@@ -194,7 +197,7 @@ template <bool BF16, bool EMIT_INT>
 __global__ __launch_bounds__(256) void fq_per_group_kernel(const void* __restrict__ w, int64_t n_chunks, int lanes_per_group,
                                                            int log2_lpg, void* __restrict__ out_fq,
                                                            int8_t* __restrict__ out_q, float* __restrict__ scale_out,
-                                                           float* __restrict__ zero_out) {
+                                                           float* __restrict__ zero_out, bool qp_bf16) {
   const int64_t base = (int64_t)blockIdx.x * (256 * kGroupChunksPerThread) + threadIdx.x;
   Chunk8<BF16> c[kGroupChunksPerThread];
 #pragma unroll
@@ -223,6 +226,7 @@ __global__ __launch_bounds__(256) void fq_per_group_kernel(const void* __restric
     const float amax = fmaxf(-mn, mx);
     float scale = amax / 7.5f;
     scale = scale > kF32Eps ? scale : kF32Eps;
+    if (qp_bf16) scale = round_to_bf16(scale);  // the rounded scale quantises and dequantises
     const float inv = 1.0f / scale;
     if ((threadIdx.x & (lanes_per_group - 1)) == 0) {
       if (scale_out) scale_out[ch >> log2_lpg] = scale;
@@ -259,13 +263,14 @@ int log2_exact(int64_t v) {
 }
 
 template <bool BF16>
-int launch_per_token(const void* x, int64_t rows, int64_t K, void* out, float* scale, int32_t* zp, hipStream_t s) {
+int launch_per_token(const void* x, int64_t rows, int64_t K, void* out, float* scale, int32_t* zp, bool qp_bf16,
+                     hipStream_t s) {
   const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
   const int64_t nv = (K / 8 + kWave - 1) / kWave;
   constexpr int kMaxRegChunks = BF16 ? 32 : 16;
 #define TT_LAUNCH_TOKEN(NV)                                                                          \
   if (nv <= NV) {                                                                                    \
-    fq_per_token_regs_kernel<BF16, NV><<<grid, block, 0, s>>>(x, rows, K, out, scale, zp);           \
+    fq_per_token_regs_kernel<BF16, NV><<<grid, block, 0, s>>>(x, rows, K, out, scale, zp, qp_bf16);  \
     return check_launch("fq_per_token_int8_asym");                                                   \
   }
   TT_LAUNCH_TOKEN(1)
@@ -277,7 +282,7 @@ int launch_per_token(const void* x, int64_t rows, int64_t K, void* out, float* s
     TT_LAUNCH_TOKEN(32)
   }
 #undef TT_LAUNCH_TOKEN
-  fq_per_token_stream_kernel<BF16><<<grid, block, 0, s>>>(x, rows, K, out, scale, zp);
+  fq_per_token_stream_kernel<BF16><<<grid, block, 0, s>>>(x, rows, K, out, scale, zp, qp_bf16);
   return check_launch("fq_per_token_int8_asym");
 }
 
@@ -443,21 +448,25 @@ int check_group_args(const void* w, int dtype, int64_t rows, int64_t K, int grou
 
 using namespace ttamd;
 
-extern "C" int ttamd_fq_per_token_int8_asym(const void* x, int dtype, int64_t rows, int64_t K, void* out, float* scale,
-                                            int32_t* zero_point, void* stream) {
+extern "C" int ttamd_fq_per_token_int8_asym(const void* x, int dtype, int64_t rows, int64_t K, int qparam_dtype, void* out,
+                                            float* scale, int32_t* zero_point, void* stream) {
+  TT_REQUIRE(qparam_dtype == TTAMD_BF16 || qparam_dtype == TTAMD_F32, "fq_per_token: unknown qparam dtype code %d", qparam_dtype);
+  const bool qbf = qparam_dtype == TTAMD_BF16;
   TT_REQUIRE(dtype == TTAMD_BF16 || dtype == TTAMD_F32, "fq_per_token: unknown dtype code %d", dtype);
   TT_REQUIRE(x && out && aligned16(x) && aligned16(out), "fq_per_token: x/out must be non-null, 16-byte aligned");
   TT_REQUIRE(rows > 0 && K > 0 && K % 8 == 0, "fq_per_token: K (%lld) must be a positive multiple of 8",
              (long long)K);
   TT_REQUIRE((rows + 3) / 4 < (int64_t(1) << 31), "fq_per_token: too many rows for one launch");
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  return dtype == TTAMD_BF16 ? launch_per_token<true>(x, rows, K, out, scale, zero_point, s)
-                             : launch_per_token<false>(x, rows, K, out, scale, zero_point, s);
+  return dtype == TTAMD_BF16 ? launch_per_token<true>(x, rows, K, out, scale, zero_point, qbf, s)
+                             : launch_per_token<false>(x, rows, K, out, scale, zero_point, qbf, s);
 }
 
-extern "C" int ttamd_fq_per_group_int4_sym(const void* w, int dtype, int64_t rows, int64_t K, int group_size, void* out,
-                                           float* scale, void* stream) {
+extern "C" int ttamd_fq_per_group_int4_sym(const void* w, int dtype, int64_t rows, int64_t K, int group_size, int qparam_dtype,
+                                           void* out, float* scale, void* stream) {
   if (int rc = check_group_args(w, dtype, rows, K, group_size)) return rc;
+  TT_REQUIRE(qparam_dtype == TTAMD_BF16 || qparam_dtype == TTAMD_F32, "fq_per_group: unknown qparam dtype code %d", qparam_dtype);
+  const bool qbf = qparam_dtype == TTAMD_BF16;
   TT_REQUIRE(out && aligned16(out), "fq_per_group: out must be non-null, 16-byte aligned");
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   const int64_t n_chunks = rows * K / 8;
@@ -467,16 +476,19 @@ extern "C" int ttamd_fq_per_group_int4_sym(const void* w, int dtype, int64_t row
   const int lpg = group_size / 8;
   if (dtype == TTAMD_BF16)
     fq_per_group_kernel<true, false><<<dim3((unsigned)grid), dim3(256), 0, s>>>(w, n_chunks, lpg, log2_exact(lpg), out,
-                                                                                 nullptr, scale, nullptr);
+                                                                                 nullptr, scale, nullptr, qbf);
   else
     fq_per_group_kernel<false, false><<<dim3((unsigned)grid), dim3(256), 0, s>>>(w, n_chunks, lpg, log2_exact(lpg), out,
-                                                                                  nullptr, scale, nullptr);
+                                                                                  nullptr, scale, nullptr, qbf);
   return check_launch("fq_per_group_int4_sym");
 }
 
-extern "C" int ttamd_quantize_per_group_int4(const void* w, int dtype, int64_t rows, int64_t K, int group_size, int8_t* q,
-                                             float* scale, float* zero_point, void* stream) {
+extern "C" int ttamd_quantize_per_group_int4(const void* w, int dtype, int64_t rows, int64_t K, int group_size,
+                                             int qparam_dtype, int8_t* q, float* scale, float* zero_point, void* stream) {
   if (int rc = check_group_args(w, dtype, rows, K, group_size)) return rc;
+  TT_REQUIRE(qparam_dtype == TTAMD_BF16 || qparam_dtype == TTAMD_F32, "quantize_per_group_int4: unknown qparam dtype code %d",
+             qparam_dtype);
+  const bool qbf = qparam_dtype == TTAMD_BF16;
   TT_REQUIRE(q && scale && (reinterpret_cast<uintptr_t>(q) & 7u) == 0,
              "quantize_per_group_int4: q (8-byte aligned) and scale must be non-null");
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
@@ -487,10 +499,10 @@ extern "C" int ttamd_quantize_per_group_int4(const void* w, int dtype, int64_t r
   const int lpg = group_size / 8;
   if (dtype == TTAMD_BF16)
     fq_per_group_kernel<true, true><<<dim3((unsigned)grid), dim3(256), 0, s>>>(w, n_chunks, lpg, log2_exact(lpg), nullptr,
-                                                                                q, scale, zero_point);
+                                                                                q, scale, zero_point, qbf);
   else
     fq_per_group_kernel<false, true><<<dim3((unsigned)grid), dim3(256), 0, s>>>(w, n_chunks, lpg, log2_exact(lpg), nullptr,
-                                                                                 q, scale, zero_point);
+                                                                                 q, scale, zero_point, qbf);
   return check_launch("quantize_per_group_int4");
 }
 

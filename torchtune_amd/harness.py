@@ -236,8 +236,9 @@ def build_qlora_decoder(shape: str | LlamaShape, rank: int, alpha: float, device
 
 def build_qat_decoder(shape: str | LlamaShape, groupsize: int = 32, device="cuda", seed: int = 0,
                       activation_checkpointing: bool = False, dtype: torch.dtype = torch.bfloat16,
-                      quantize_output: bool = True) -> Decoder:
-    """Full-finetune model prepared for 8da4w QAT: every linear swapped for the fake-quantised one."""
+                      quantize_output: bool = True, scales_precision: torch.dtype = torch.float32) -> Decoder:
+    """Full-finetune model prepared for 8da4w QAT: every linear swapped for the fake-quantised one.
+    ``scales_precision`` float32 is the reference quantizer's default; bfloat16 rounds every scale before use."""
     s = SHAPES[shape] if isinstance(shape, str) else shape
     prev = torch.get_default_dtype()
     torch.set_default_dtype(dtype)
@@ -247,7 +248,7 @@ def build_qat_decoder(shape: str | LlamaShape, groupsize: int = 32, device="cuda
     finally:
         torch.set_default_dtype(prev)
     _init_weights(model, seed)
-    quantizer = Int8DynActInt4WeightQATQuantizer(groupsize=groupsize, precision=dtype)
+    quantizer = Int8DynActInt4WeightQATQuantizer(groupsize=groupsize, precision=dtype, scales_precision=scales_precision)
     if quantize_output:
         quantizer.prepare(model)
     else:

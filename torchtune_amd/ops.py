@@ -301,10 +301,12 @@ def set_fq_timer(timer) -> None:
     _fq_timer = timer
 
 
-def fq_per_token_int8_asym(x: torch.Tensor, want_qparams: bool = True):
-    """x [..., K] -> (fake-quantised x, scale fp32 [rows] | None, zero_point int32 [rows] | None)"""
+def fq_per_token_int8_asym(x: torch.Tensor, want_qparams: bool = True, qparam_dtype: torch.dtype = torch.float32):
+    """x [..., K] -> (fake-quantised x, scale fp32 [rows] | None, zero_point int32 [rows] | None).
+    ``qparam_dtype=torch.bfloat16`` rounds the scale to bf16 before it quantises and dequantises."""
     _need_gpu(x, "fq_per_token_int8_asym")
     code = _code(x.dtype, "fq_per_token_int8_asym")
+    qcode = _code(qparam_dtype, "fq_per_token_int8_asym (qparams)")
     xc = x.contiguous()
     K = xc.shape[-1]
     rows = xc.numel() // K
@@ -316,17 +318,21 @@ def fq_per_token_int8_asym(x: torch.Tensor, want_qparams: bool = True):
         events = _fq_timer("per_token", rows, K, 0, xc.element_size()) if _fq_timer is not None else None
         if events:
             events[0].record()
-        rc = lib.ttamd_fq_per_token_int8_asym(xc.data_ptr(), code, rows, K, out.data_ptr(), _ptr(scale), _ptr(zp), _stream(x))
+        rc = lib.ttamd_fq_per_token_int8_asym(xc.data_ptr(), code, rows, K, qcode, out.data_ptr(), _ptr(scale), _ptr(zp),
+                                              _stream(x))
         if events:
             events[1].record()
     _lib.check(rc, "fq_per_token_int8_asym")
     return out, scale, zp
 
 
-def fq_per_group_int4_sym(w: torch.Tensor, group_size: int, want_scale: bool = True):
-    """w [..., K] -> (fake-quantised w, scale fp32 [rows, K/g] | None)"""
+def fq_per_group_int4_sym(w: torch.Tensor, group_size: int, want_scale: bool = True,
+                          qparam_dtype: torch.dtype = torch.float32):
+    """w [..., K] -> (fake-quantised w, scale fp32 [rows, K/g] | None).
+    ``qparam_dtype=torch.bfloat16`` rounds the scales to bf16 before they quantise and dequantise."""
     _need_gpu(w, "fq_per_group_int4_sym")
     code = _code(w.dtype, "fq_per_group_int4_sym")
+    qcode = _code(qparam_dtype, "fq_per_group_int4_sym (qparams)")
     wc = w.contiguous()
     K = wc.shape[-1]
     rows = wc.numel() // K
@@ -337,17 +343,19 @@ def fq_per_group_int4_sym(w: torch.Tensor, group_size: int, want_scale: bool = T
         events = _fq_timer("per_group", rows, K, group_size, wc.element_size()) if _fq_timer is not None else None
         if events:
             events[0].record()
-        rc = lib.ttamd_fq_per_group_int4_sym(wc.data_ptr(), code, rows, K, group_size, out.data_ptr(), _ptr(scale), _stream(w))
+        rc = lib.ttamd_fq_per_group_int4_sym(wc.data_ptr(), code, rows, K, group_size, qcode, out.data_ptr(), _ptr(scale),
+                                             _stream(w))
         if events:
             events[1].record()
     _lib.check(rc, "fq_per_group_int4_sym")
     return out, scale
 
 
-def quantize_per_group_int4(w: torch.Tensor, group_size: int):
+def quantize_per_group_int4(w: torch.Tensor, group_size: int, qparam_dtype: torch.dtype = torch.float32):
     """w [rows, K] -> (int8 tensor of int4 values, scale fp32 [rows, K/g], zeros fp32 [rows, K/g])"""
     _need_gpu(w, "quantize_per_group_int4")
     code = _code(w.dtype, "quantize_per_group_int4")
+    qcode = _code(qparam_dtype, "quantize_per_group_int4 (qparams)")
     wc = w.contiguous()
     K = wc.shape[-1]
     rows = wc.numel() // K
@@ -356,7 +364,7 @@ def quantize_per_group_int4(w: torch.Tensor, group_size: int):
     zeros = torch.empty_like(scale)
     lib = _lib.load()
     with torch.cuda.device(w.device):
-        rc = lib.ttamd_quantize_per_group_int4(wc.data_ptr(), code, rows, K, group_size, q.data_ptr(), scale.data_ptr(),
+        rc = lib.ttamd_quantize_per_group_int4(wc.data_ptr(), code, rows, K, group_size, qcode, q.data_ptr(), scale.data_ptr(),
                                                zeros.data_ptr(), _stream(w))
     _lib.check(rc, "quantize_per_group_int4")
     return q, scale, zeros

@@ -155,6 +155,8 @@ class FakeQuantizer(nn.Module):
         self.scale: Optional[torch.Tensor] = None
         self.zero_point: Optional[torch.Tensor] = None
         g = config.granularity
+        if config.scale_precision not in (torch.float32, torch.bfloat16):
+            raise NotImplementedError("fake quantisation has kernels for float32 and bfloat16 scale_precision only")
         if isinstance(g, PerToken):
             if config.dtype != torch.int8 or config.is_symmetric:
                 raise NotImplementedError("per-token fake quantisation has a kernel for asymmetric int8 only")
@@ -176,7 +178,7 @@ class FakeQuantizer(nn.Module):
             return x
         with torch.no_grad():
             if isinstance(self.config.granularity, PerToken):
-                fq, scale, zp = ops.fq_per_token_int8_asym(x.detach())
+                fq, scale, zp = ops.fq_per_token_int8_asym(x.detach(), qparam_dtype=self.config.scale_precision)
                 self.scale = scale.to(self.config.scale_precision)
                 self.zero_point = zp.to(self.config.zero_point_precision)
             else:
@@ -188,7 +190,7 @@ class FakeQuantizer(nn.Module):
                     self.scale = scale.to(self.config.scale_precision)
                     self.zero_point = zp.to(self.config.zero_point_precision)
                 else:
-                    fq, scale = ops.fq_per_group_int4_sym(x.detach(), gs)
+                    fq, scale = ops.fq_per_group_int4_sym(x.detach(), gs, qparam_dtype=self.config.scale_precision)
                     self.scale = scale.to(self.config.scale_precision)
                     self.zero_point = None
         return _StraightThrough.apply(x, fq.view(x.shape))
@@ -297,7 +299,7 @@ class Int8DynActInt4WeightLinear(nn.Module):
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         x = x.to(self.precision)
-        x_q, _, _ = ops.fq_per_token_int8_asym(x, want_qparams=False)
+        x_q, _, _ = ops.fq_per_token_int8_asym(x, want_qparams=False, qparam_dtype=self.scales_precision)
         w = ops.dequantize_per_group_int4(self.weight, self.scales, self.zeros, self.groupsize, self.precision)
         return F.linear(x_q, w, self.bias)
 
@@ -357,7 +359,7 @@ class Int8DynActInt4WeightQATQuantizer:
                     child.in_features, child.out_features, child.bias is not None, device=child.weight.device,
                     groupsize=child.groupsize, precision=child.weight.dtype, scales_precision=child.scales_precision,
                 )
-                q, scale, zeros = ops.quantize_per_group_int4(child.weight.detach(), child.groupsize)
+                q, scale, zeros = ops.quantize_per_group_int4(child.weight.detach(), child.groupsize, child.scales_precision)
                 new.weight.copy_(q)
                 new.scales.copy_(scale.to(child.scales_precision))
                 new.zeros.copy_(zeros.to(child.scales_precision))
