@@ -38,58 +38,84 @@ MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"llama3_1_8b": 496.3e6}
 
 
 class GemmTimer:
-    """Collects (flops, start event, end event) for every fused-GEMM launch while installed in ``ops``."""
+    """HIP-event timing of the fused-GEMM launches while installed in ``ops``.
 
-    def __init__(self):
+    An event pair costs the stream about 6 us per timed launch (the GPU idles around the markers), 1.6 % of a step if
+    every one of its 445 launches is timed.  So every ``stride``-th launch of each (kind, shape) is timed and the
+    others only counted: the averages still come from the timed region itself, the step pays a quarter of the cost."""
+
+    def __init__(self, stride: int = 4):
+        self.stride = max(1, stride)
         self.records = []
+        self.counts = {}
 
     def __call__(self, kind, M, N, K, rank):
         flops = 2.0 * M * N * K + 2.0 * M * rank * (N if kind == "fwd" else K)
+        key = (kind, M, N, K)
+        seen = self.counts.get(key, [0, flops])
+        self.counts[key] = [seen[0] + 1, flops]
+        if seen[0] % self.stride:
+            return None
         start = torch.cuda.Event(enable_timing=True)
         end = torch.cuda.Event(enable_timing=True)
-        self.records.append((kind, (M, N, K), flops, start, end))
+        self.records.append((key, start, end))
         return start, end
 
     def summary(self):
-        total_ms = 0.0
-        total_flops = 0.0
-        by = {}
-        for kind, shape, flops, s, e in self.records:
-            ms = s.elapsed_time(e)
-            total_ms += ms
-            total_flops += flops
-            key = f"{kind} M{shape[0]} N{shape[1]} K{shape[2]}"
-            acc = by.setdefault(key, [0, 0.0, 0.0])
+        """-> (launches, launches timed, estimated ms of all launches, flops of all launches, per-shape table)"""
+        timed = {}
+        for key, s, e in self.records:
+            acc = timed.setdefault(key, [0, 0.0])
             acc[0] += 1
-            acc[1] += ms
-            acc[2] += flops
-        per_shape = {k: {"launches": v[0], "avg_us": round(1e3 * v[1] / v[0], 1), "tflops": round(v[2] / v[1] / 1e9, 1)}
-                     for k, v in by.items()}
-        return len(self.records), total_ms, total_flops, per_shape
+            acc[1] += s.elapsed_time(e)
+        total_ms = total_flops = 0.0
+        per_shape = {}
+        for key, (n, flops) in self.counts.items():
+            n_timed, ms = timed[key]
+            avg_ms = ms / n_timed
+            total_ms += avg_ms * n
+            total_flops += flops * n
+            per_shape[f"{key[0]} M{key[1]} N{key[2]} K{key[3]}"] = {
+                "launches": n, "timed": n_timed, "avg_us": round(1e3 * avg_ms, 1), "tflops": round(flops / avg_ms / 1e9, 1)}
+        return sum(v[0] for v in self.counts.values()), len(self.records), total_ms, total_flops, per_shape
 
 
 class FqTimer:
-    """Collects (bytes, start event, end event) for every fake-quant launch while installed in ``ops``.
-    Algorithmic bytes: one read and one write of the tensor, plus the fp32 qparams the launch writes."""
+    """HIP-event timing of the fake-quant launches while installed in ``ops``; every ``stride``-th launch of each
+    (kind, shape) is timed, like the GEMM launches.  Algorithmic bytes: one read and one write of the tensor, plus
+    the fp32 qparams the launch writes."""
 
-    def __init__(self):
+    def __init__(self, stride: int = 4):
+        self.stride = max(1, stride)
         self.records = []
+        self.counts = {}
 
     def __call__(self, kind, rows, K, group_size, elem_bytes):
         n = rows * K
         nbytes = 2 * n * elem_bytes + (rows * 8 if kind == "per_token" else n // group_size * 4)
+        key = (kind, rows, K, group_size, elem_bytes)
+        seen = self.counts.get(key, [0, nbytes])
+        self.counts[key] = [seen[0] + 1, nbytes]
+        if seen[0] % self.stride:
+            return None
         start = torch.cuda.Event(enable_timing=True)
         end = torch.cuda.Event(enable_timing=True)
-        self.records.append((kind, nbytes, start, end))
+        self.records.append((key, start, end))
         return start, end
 
     def summary(self):
-        by = {}
-        for kind, nbytes, s, e in self.records:
-            acc = by.setdefault(kind, [0, 0.0, 0.0])
+        timed = {}
+        for key, s, e in self.records:
+            acc = timed.setdefault(key, [0, 0.0])
             acc[0] += 1
             acc[1] += s.elapsed_time(e)
-            acc[2] += nbytes
+        by = {}
+        for key, (n, nbytes) in self.counts.items():
+            n_timed, ms = timed[key]
+            acc = by.setdefault(key[0], [0, 0.0, 0.0])
+            acc[0] += n
+            acc[1] += ms / n_timed * n
+            acc[2] += float(nbytes) * n
         return {k: {"launches": v[0], "avg_us": round(1e3 * v[1] / v[0], 1), "gbps": round(v[2] / v[1] / 1e6, 1),
                     "ms": v[1], "bytes": v[2]} for k, v in by.items()}
 
@@ -260,6 +286,8 @@ def main() -> int:
     ap.add_argument("--qat-scales", default="float32", choices=["float32", "bfloat16"],
                     help="scales_precision of the QAT workload: float32 is the reference quantizer's default, bfloat16 rounds "
                          "every scale before it quantises and dequantises")
+    ap.add_argument("--gemm-timing-stride", type=int, default=4,
+                    help="time every n-th fused-GEMM / fake-quant launch of each shape with HIP events (1 = every launch)")
     ap.add_argument("--calibration-copy-mib", type=int, default=0,
                     help="before the steps, run one elementwise kernel that reads and writes this many MiB: the known-size "
                          "dispatch that FETCH_SIZE / WRITE_SIZE counter runs are scaled by")
@@ -303,8 +331,8 @@ def main() -> int:
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
-    timer = GemmTimer()
-    fq_timer = FqTimer()
+    timer = GemmTimer(args.gemm_timing_stride)
+    fq_timer = FqTimer(args.gemm_timing_stride)
     ops.set_gemm_timer(timer)
     ops.set_fq_timer(fq_timer)
     torch.cuda.synchronize()
@@ -355,6 +383,8 @@ def main() -> int:
                 "frac": round(achieved / HBM_PEAK_GBPS, 4),
                 "traffic": None,
                 "fq_ms_per_step": round(fq_ms / args.steps, 2),
+                "timing": f"HIP events on the launch stream around every {fq_timer.stride}th launch of each shape inside the "
+                          "timed steps; achieved = sum(bytes) / sum(average duration x launches)",
                 "per_kernel": {k: {kk: vv for kk, vv in v.items() if kk in ("launches", "avg_us", "gbps")} for k, v in fq.items()},
             },
         }
@@ -366,7 +396,7 @@ def main() -> int:
         print(json.dumps(result))
         return 0
 
-    launches, gemm_ms, gemm_flops, per_shape = timer.summary()
+    launches, launches_timed, gemm_ms, gemm_flops, per_shape = timer.summary()
     achieved = gemm_flops / gemm_ms / 1e9 if gemm_ms > 0 else 0.0
     result = {
         "metric": "QLoRA fwd+bwd tokens/sec (Llama-3.1-8B, 1 GPU)" if args.workload == "llama3_1_8b"
@@ -400,7 +430,10 @@ def main() -> int:
             "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(args.workload),
             "traffic_unit": "bytes per launch, average over a step's launches (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 from rocprofv3 "
                             "--pmc runs; algorithmic 210.4e6)" if args.workload in MEASURED_TRAFFIC_BYTES_PER_LAUNCH else None,
-            "launches_timed": launches,
+            "launches": launches,
+            "launches_timed": launches_timed,
+            "timing": f"HIP events on the launch stream around every {timer.stride}th launch of each shape inside the timed steps "
+                      "(an event pair idles the GPU for about 6 us); achieved = sum(flops) / sum(average duration x launches)",
             "gemm_ms_per_step": round(gemm_ms / args.steps, 2),
             "per_shape": per_shape,
         },
