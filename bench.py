@@ -32,9 +32,11 @@ WORKLOADS = {
 }
 HBM_PEAK_GBPS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
-# HBM-side bytes per fused-GEMM launch (average over the launches of one step), from the FETCH_SIZE / WRITE_SIZE counter
-# runs summarised in profiles/nf4_gemm_rs_kernel_hbm_traffic.txt (counters cannot be read from inside this process).
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"llama3_1_8b": 496.3e6}
+# HBM-side bytes per launch of the workload's dominant kernel (fused GEMM; fake quant for the QAT workload), average over
+# the launches of one step, from the FETCH_SIZE / WRITE_SIZE counter runs summarised in
+# profiles/nf4_gemm_rs_kernel_hbm_traffic.txt and profiles/fake_quant_and_layer_kernels_hbm_traffic.txt (counters cannot
+# be read from inside this process).
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"llama3_1_8b": 496.3e6, "llama3_1_8b_qat": 164.1e6}
 
 
 class GemmTimer:
@@ -381,7 +383,9 @@ def main() -> int:
                 "peak": HBM_PEAK_GBPS,
                 "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                "traffic": None,
+                "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(args.workload),
+                "traffic_unit": "bytes per launch, average over a step's fake-quant launches (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 "
+                                f"from rocprofv3 --pmc runs); algorithmic {fq_bytes / max(1, sum(v['launches'] for v in fq.values())) / 1e6:.1f}e6",
                 "fq_ms_per_step": round(fq_ms / args.steps, 2),
                 "timing": f"HIP events on the launch stream around every {fq_timer.stride}th launch of each shape inside the "
                           "timed steps; achieved = sum(bytes) / sum(average duration x launches)",

@@ -454,6 +454,11 @@ __global__ __launch_bounds__(kCeThreads) void cross_entropy_kernel(const uint16_
   }
   __syncthreads();
   mx = bcast;
+  // Each pass unpacks the row from its packed registers again: the barriers stop the compiler from keeping the 128
+  // unpacked (or exponentiated) values of one pass alive for the next, which would not fit the 128 registers a
+  // 1024-thread workgroup leaves each lane and would spill to scratch memory (three times the kernel's HBM traffic).
+#pragma unroll
+  for (int i = 0; i < kCeChunks; ++i) asm volatile("" : "+v"(v[i]));
   float se = 0.f;
 #pragma unroll
   for (int i = 0; i < kCeChunks; ++i)
@@ -474,6 +479,8 @@ __global__ __launch_bounds__(kCeThreads) void cross_entropy_kernel(const uint16_
   __syncthreads();
   se = bcast;
   const float inv = grad_scale / se;
+#pragma unroll
+  for (int i = 0; i < kCeChunks; ++i) asm volatile("" : "+v"(v[i]));
   if (t == 0) {
     const bool valid = tgt >= 0 && tgt < V;  // an out-of-range class gives NaN, never an out-of-bounds read
     const float xt = bf16_bits_to_f32(logits[row * V + (valid ? tgt : 0)]);
