@@ -316,22 +316,43 @@ __global__ __launch_bounds__(256) void nf4_block_scalers_kernel(const int8_t* __
 }
 
 // Transposed copy of the codes for the grad-input GEMM: out[k][n] = code of W[n][k], packed along n
-// (byte (k*N + n)/2, even n in the high nibble).  One thread makes one output dword = 8 consecutive n.
+// (byte (k*N + n)/2, even n in the high nibble).  A workgroup moves a tile of 64 rows n x 128 columns k through LDS:
+// it reads 64-byte row pieces and writes 32-byte row pieces of the transposed tensor, so both sides use whole sectors
+// (reading single bytes down a column fetched eight times the tensor).
+constexpr int kTrTileK = 128;  // columns k per tile = 64 bytes of a row
+constexpr int kTrPitch = 68;   // LDS row pitch in bytes (64 + 4: rows of a column land in different banks)
+
 __global__ __launch_bounds__(256) void nf4_transpose_codes_kernel(const uint8_t* __restrict__ q, int N, int K,
                                                                   uint32_t* __restrict__ qt) {
-  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;  // = k * (N/8) + n8
-  const int n8s = N >> 3;
-  if (idx >= (int64_t)K * n8s) return;
-  const int k = (int)(idx / n8s), n8 = (int)(idx % n8s);
-  const int shift = (k & 1) ? 0 : 4;
-  uint32_t packed = 0;
+  __shared__ __attribute__((aligned(16))) uint8_t tile[64 * kTrPitch];
+  const int t = threadIdx.x;
+  const int n0 = blockIdx.x * 64, k0 = blockIdx.y * kTrTileK;
+  {
+    const int r = t >> 2, piece = t & 3;  // row of the tile, 16-byte piece (32 codes) of its 64 bytes
+    uint32_t v[4] = {0, 0, 0, 0};
+    if (k0 + 32 * piece < K) {            // K % 64 == 0: a piece is in or out as a whole
+      const uint4 ld = *reinterpret_cast<const uint4*>(q + (((int64_t)(n0 + r) * K + k0) >> 1) + 16 * piece);
+      v[0] = ld.x; v[1] = ld.y; v[2] = ld.z; v[3] = ld.w;
+    }
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const uint32_t byte = q[((int64_t)(n8 * 8 + i) * K + k) >> 1];
-    const uint32_t code = (byte >> shift) & 0xfu;
-    packed |= code << (8 * (i >> 1) + ((i & 1) ? 0 : 4));
+    for (int d = 0; d < 4; ++d) *reinterpret_cast<uint32_t*>(tile + r * kTrPitch + 16 * piece + 4 * d) = v[d];
   }
-  qt[idx] = packed;
+  __syncthreads();
+  const int n8s = N >> 3;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int o = t + 256 * j;       // output dword of the tile: row k, eight consecutive n
+    const int k = o >> 3, n8 = o & 7;
+    if (k0 + k >= K) continue;
+    const int shift = (k & 1) ? 0 : 4;
+    uint32_t packed = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const uint32_t code = ((uint32_t)tile[(n8 * 8 + i) * kTrPitch + (k >> 1)] >> shift) & 0xfu;
+      packed |= code << (8 * (i >> 1) + ((i & 1) ? 0 : 4));
+    }
+    qt[(int64_t)(k0 + k) * n8s + (n0 >> 3) + n8] = packed;
+  }
 }
 
 // Transposed block scalers: out[kb][n] = scalers[n][kb]
@@ -457,10 +478,11 @@ extern "C" int ttamd_nf4_transpose_for_backward(const uint8_t* quantized_data, c
              "nf4_transpose_for_backward: N (%lld) and K (%lld) must be positive multiples of 64", (long long)N, (long long)K);
   TT_REQUIRE((reinterpret_cast<uintptr_t>(quantized_data_t) & 3u) == 0, "nf4_transpose_for_backward: output must be 4-byte aligned");
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  const int64_t n1 = K * (N / 8), n2 = N * (K / 64);
-  TT_REQUIRE((n1 + 255) / 256 < (int64_t(1) << 31), "nf4_transpose_for_backward: tensor too large for one launch");
-  nf4_transpose_codes_kernel<<<dim3((unsigned)((n1 + 255) / 256)), dim3(256), 0, s>>>(quantized_data, (int)N, (int)K,
-                                                                                     reinterpret_cast<uint32_t*>(quantized_data_t));
+  const int64_t n2 = N * (K / 64);
+  TT_REQUIRE((K + kTrTileK - 1) / kTrTileK < 65536, "nf4_transpose_for_backward: K too large for one launch");
+  TT_REQUIRE(aligned16(quantized_data), "nf4_transpose_for_backward: quantized_data must be 16-byte aligned");
+  nf4_transpose_codes_kernel<<<dim3((unsigned)(N / 64), (unsigned)((K + kTrTileK - 1) / kTrTileK)), dim3(256), 0, s>>>(
+      quantized_data, (int)N, (int)K, reinterpret_cast<uint32_t*>(quantized_data_t));
   nf4_transpose_scalers_kernel<<<dim3((unsigned)((n2 + 255) / 256)), dim3(256), 0, s>>>(
       reinterpret_cast<const float*>(block_scalers), (int)N, (int)(K / 64), reinterpret_cast<float*>(block_scalers_t));
   return check_launch("nf4_transpose_for_backward");
