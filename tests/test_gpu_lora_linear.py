@@ -349,3 +349,62 @@ def test_token_dimension_beyond_32_bit_offsets_is_split_into_row_ranges():
     assert gx.shape == (M, K)
     torch.testing.assert_close(gx[M - 300:].float(), gy[M - 300:].float() @ D, rtol=1e-2, atol=1e-2)
     torch.testing.assert_close(gx[:300].float(), gy[:300].float() @ D, rtol=1e-2, atol=1e-2)
+
+
+def test_seeded_sweep_of_shapes_ranks_and_options_against_fp32_reference():
+    """Forty seeded combinations of (M, N, K, rank, bias, column scale, scaler layout, backward copy) through the raw ops,
+    against fp32 matmuls of the bit-exact dequantised weight on the same device.  M is arbitrary, N and K any multiples
+    of 64 (so tiles are ragged in every direction), ranks over the whole supported set."""
+    import random
+
+    rng = random.Random(20240607)
+    g = torch.Generator(device=DEV).manual_seed(99)
+    for case in range(40):
+        M = rng.choice([1, 2, 31, 64, 127, 128, 129, 255, 256, 257, 300, 511, 513, 777, 1025])
+        while True:  # to_nf4 needs whole scaler blocks of 256 blocks: (N / 64) * K must be a multiple of 256
+            N = 64 * rng.randint(1, 17)
+            K = 64 * rng.randint(1, 33)
+            if (N // 64) * K % 256 == 0:
+                break
+        r = rng.choice([0, 8, 16, 24, 40, 64])
+        use_bias, use_cs, use_t, use_copy = (rng.random() < 0.5 for _ in range(4))
+        t = to_nf4((torch.randn(N, K, device=DEV, generator=g) * 0.02).to(BF))
+        D = t.get_original_weight().float()
+        x = torch.randn(M, K, device=DEV, generator=g).to(BF)
+        gy = torch.randn(M, N, device=DEV, generator=g).to(BF)
+        A = (torch.randn(max(r, 1), K, device=DEV, generator=g) * 0.05).to(BF)[:r]
+        B = (torch.randn(N, max(r, 1), device=DEV, generator=g) * 0.05).to(BF)[:, :r]
+        bias = (torch.randn(N, device=DEV, generator=g) * 0.1).to(BF) if use_bias else None
+        cs = (torch.rand(N, device=DEV, generator=g) + 0.5).to(BF) if use_cs else None
+        tag = f"case {case}: M{M} N{N} K{K} r{r} bias{int(use_bias)} cs{int(use_cs)} t{int(use_t)} copy{int(use_copy)}"
+        print(tag, flush=True)
+        bs = t.block_scalers()
+        copy = t.backward_copy()
+        h = ops.lora_hidden(x, A.contiguous()) if r else None
+        y = ops.nf4_lora_linear_fwd(x, t.quantized_data, bs, N, h, B.contiguous() if r else None, 2.0, bias,
+                                    block_scalers_t=copy[1] if use_t else None, col_scale=cs)
+        ref = x.float() @ D.T
+        if use_bias:
+            ref = ref + bias.float()
+        if r:
+            torch.testing.assert_close(h.float(), x.float() @ A.float().T, rtol=1e-2, atol=1e-2, msg=tag)
+            ref = ref + 2.0 * (h.float() @ B.float().T)
+        if use_cs:
+            ref = ref * cs.float()
+        torch.testing.assert_close(y.float(), ref, rtol=1e-2, atol=1e-2, msg=tag)
+        if r:
+            gh, ga, gb = ops.lora_bwd(gy, x, h, B.contiguous(), 2.0)
+            gh_ref = 2.0 * (gy.float() @ B.float())
+            torch.testing.assert_close(gh.float(), gh_ref, rtol=1e-2, atol=1e-2 * float(gh_ref.abs().max()), msg=tag)
+            ga_ref = gh.float().T @ x.float()
+            gb_ref = 2.0 * (gy.float().T @ h.float())
+            torch.testing.assert_close(ga.float(), ga_ref, rtol=1e-2, atol=1e-2 * float(ga_ref.abs().max()) + 1e-6, msg=tag)
+            torch.testing.assert_close(gb.float(), gb_ref, rtol=1e-2, atol=1e-2 * float(gb_ref.abs().max()) + 1e-6, msg=tag)
+        else:
+            gh = None
+        gx = ops.nf4_linear_bwd_dx(gy, t.quantized_data, bs, K, gh, A.contiguous() if r else None,
+                                   transposed=copy if use_copy else None)
+        gx_ref = gy.float() @ D
+        if r:
+            gx_ref = gx_ref + gh.float() @ A.float()
+        torch.testing.assert_close(gx.float(), gx_ref, rtol=1e-2, atol=1e-2 * max(1.0, float(gx_ref.abs().max()) / 8), msg=tag)
