@@ -288,6 +288,9 @@ def main() -> int:
     ap.add_argument("--qat-scales", default="float32", choices=["float32", "bfloat16"],
                     help="scales_precision of the QAT workload: float32 is the reference quantizer's default, bfloat16 rounds "
                          "every scale before it quantises and dequantises")
+    ap.add_argument("--sdpa", default="efficient", choices=["efficient", "flash", "default"],
+                    help="which of PyTorch's scaled_dot_product_attention backends the stack asks for (attention is stock "
+                         "PyTorch; 'flash' is what the dispatcher picks by itself)")
     ap.add_argument("--gemm-timing-stride", type=int, default=4,
                     help="time every n-th fused-GEMM / fake-quant launch of each shape with HIP events (1 = every launch)")
     ap.add_argument("--calibration-copy-mib", type=int, default=0,
@@ -302,7 +305,10 @@ def main() -> int:
         return 2
 
     from torchtune_amd import ops
+    from torchtune_amd import harness
     from torchtune_amd.harness import SHAPES, build_qat_decoder, build_qlora_decoder, train_step
+
+    harness.SDPA_BACKEND = args.sdpa
 
     shape_name, rank, alpha, batch, seq, ac = WORKLOADS[args.workload]
     qat = args.workload.endswith("_qat")
@@ -370,7 +376,8 @@ def main() -> int:
                 "workload": f"{shape_name}-shaped decoder, every linear (incl. output) 8da4w fake-quantised as the reference's "
                             "quantizer does it: per-token asymmetric int8 activations (min/max with zero point), "
                             f"per-group({qat_group}) symmetric int4 weights, {args.qat_scales} scales, batch {batch} x seq {seq}, "
-                            "fwd+bwd with weight gradients, output projection and cross-entropy",
+                            "fwd+bwd with weight gradients, output projection and cross-entropy; "
+                            f"attention = torch SDPA, backend '{args.sdpa}'",
                 "global_batch": batch,
                 "seq_len": seq,
                 "loss": float(loss),
@@ -419,7 +426,8 @@ def main() -> int:
         "config": {
             "workload": f"{args.workload}-shaped QLoRA decoder, all 7 projections NF4(64/256)+LoRA r={rank} alpha={alpha:g}, "
                         f"batch {batch} x seq {seq}, fwd+bwd incl. output projection and cross-entropy"
-                        + (", activation checkpointing" if ac else ""),
+                        + (", activation checkpointing" if ac else "")
+                        + f"; attention = torch SDPA, backend '{args.sdpa}'",
             "global_batch": batch,
             "seq_len": seq,
             "loss": float(loss),

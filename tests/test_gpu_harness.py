@@ -50,3 +50,40 @@ def test_tiny_qat_decoder_step():
     loss = harness.train_step(model, tokens, tokens)
     assert torch.isfinite(loss)
     assert all(p.grad is not None for n, p in model.named_parameters() if "weight" in n and "tok_embeddings" not in n)
+
+
+def test_attention_backends_agree_and_match_an_fp32_reference(monkeypatch):
+    """The stack asks PyTorch for its "efficient" attention backend (its backward is much faster here than "flash").
+    Output and q/k/v gradients of both backends must agree with an fp32 softmax(QK^T)V computed with plain matmuls,
+    at the 8B head shape, and one decoder step must give the same loss and gradients with either backend."""
+    g = torch.Generator(device=DEV).manual_seed(5)
+    b, h, s, d = 2, 8, 512, 128
+    q, k, v = (torch.randn(b, s, h, d, device=DEV, generator=g).to(torch.bfloat16).requires_grad_() for _ in range(3))
+    go = torch.randn(b, h, s, d, device=DEV, generator=g).to(torch.bfloat16)
+    qf, kf, vf = (t.detach().float().transpose(1, 2).requires_grad_() for t in (q, k, v))
+    att = (qf @ kf.transpose(-1, -2)) / d ** 0.5
+    att = att.masked_fill(torch.ones(s, s, device=DEV, dtype=torch.bool).triu(1), float("-inf")).softmax(-1)
+    ref = att @ vf
+    ref.backward(go.float())
+    for backend in ("efficient", "flash"):
+        monkeypatch.setattr(harness, "SDPA_BACKEND", backend)
+        for t in (q, k, v):
+            t.grad = None
+        out = harness._sdpa(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2))
+        out.backward(go)
+        torch.testing.assert_close(out.float(), ref.detach(), rtol=2e-2, atol=2e-2, msg=backend)
+        for got, want in ((q.grad, qf.grad), (k.grad, kf.grad), (v.grad, vf.grad)):
+            want = want.transpose(1, 2)
+            torch.testing.assert_close(got.float(), want, rtol=2e-2, atol=2e-2 * float(want.abs().max()), msg=backend)
+    model = harness.build_qlora_decoder("tiny", rank=8, alpha=16.0, device=DEV, seed=0)
+    tokens = torch.randint(0, 1024, (2, 192), device=DEV, generator=g)
+    results = {}
+    for backend in ("efficient", "flash"):
+        monkeypatch.setattr(harness, "SDPA_BACKEND", backend)
+        model.zero_grad(set_to_none=True)
+        loss = harness.train_step(model, tokens, tokens)
+        results[backend] = (loss, {n: p.grad.clone() for n, p in model.named_parameters() if p.grad is not None})
+    torch.testing.assert_close(results["efficient"][0], results["flash"][0], rtol=2e-3, atol=2e-3)
+    for n, ge in results["efficient"][1].items():
+        gf = results["flash"][1][n].float()
+        torch.testing.assert_close(ge.float(), gf, rtol=5e-2, atol=5e-2 * float(gf.abs().max()) + 1e-6, msg=n)

@@ -24,6 +24,7 @@ from typing import Optional
 import torch
 import torch.nn.functional as F
 from torch import nn
+from torch.nn.attention import SDPBackend, sdpa_kernel
 from torch.utils.checkpoint import checkpoint
 
 from .modules import layer_ops
@@ -60,6 +61,24 @@ SHAPES = {
 # True: RMSNorm, RoPE and the SwiGLU gate run as single-pass HIP kernels (bf16 on the GPU); False: the eager op chains
 # of the reference.  The quantized linears are unaffected.
 FUSED_LAYER_OPS = True
+
+
+# Which of PyTorch's own scaled_dot_product_attention backends the stack asks for (attention is stock PyTorch here, as
+# in the reference, which calls F.scaled_dot_product_attention and takes the dispatcher's first choice, "flash").  On
+# this GPU the backward of the "efficient" backend takes 0.77 ms per 8B layer against 2.2 ms for "flash" (forward equal),
+# so "efficient" is the default; "flash" restores the dispatcher's own choice, "default" leaves the dispatcher alone.
+SDPA_BACKEND = "efficient"
+_SDPA_CHOICES = {
+    "efficient": [SDPBackend.EFFICIENT_ATTENTION, SDPBackend.MATH],
+    "flash": [SDPBackend.FLASH_ATTENTION, SDPBackend.MATH],
+}
+
+
+def _sdpa(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> torch.Tensor:
+    if SDPA_BACKEND == "default" or not q.is_cuda:
+        return F.scaled_dot_product_attention(q, k, v, is_causal=True)
+    with sdpa_kernel(_SDPA_CHOICES[SDPA_BACKEND]):
+        return F.scaled_dot_product_attention(q, k, v, is_causal=True)
 
 
 def _fused(x: torch.Tensor) -> bool:
@@ -127,7 +146,7 @@ class Attention(nn.Module):
             rep = self.n_heads // self.n_kv
             k = k.unsqueeze(3).expand(b, sl, self.n_kv, rep, self.head_dim).flatten(2, 3)
             v = v.unsqueeze(3).expand(b, sl, self.n_kv, rep, self.head_dim).flatten(2, 3)
-        o = F.scaled_dot_product_attention(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), is_causal=True)
+        o = _sdpa(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2))
         return self.output_proj(o.transpose(1, 2).reshape(b, sl, -1))
 
 
