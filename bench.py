@@ -206,8 +206,8 @@ def secondary_kernels(dev) -> dict:
     algorithmic bytes (2.515747 B/element for the NF4 codec, 4 B/element for fake quant) / HIP-event time."""
     from torchtune_amd import ops, to_nf4
 
-    def timed(fn, iters=20):
-        for _ in range(3):
+    def timed(fn, iters=30):
+        for _ in range(10):
             fn()
         start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         start.record()
@@ -222,7 +222,9 @@ def secondary_kernels(dev) -> dict:
     W = (torch.randn(14336, 4096, device=dev, generator=gen) * 0.02).to(torch.bfloat16)
     t = to_nf4(W)
     n = W.numel()
-    out["nf4_dequantize 14336x4096 bf16"] = round(n * 2.515747 / timed(t.get_original_weight) / 1e9, 1)
+    dense = torch.empty_like(W)  # preallocated: with the allocator in the loop the host barely keeps ahead of a 25 us kernel
+    out["nf4_dequantize 14336x4096 bf16"] = round(n * 2.515747 / timed(lambda: t.get_original_weight(out=dense)) / 1e9, 1)
+    del dense
     out["nf4_quantize 14336x4096 bf16"] = round(n * 2.515747 / timed(lambda: ops.nf4_quantize(W, 64, 256)) / 1e9, 1)
     out["fq_per_group_int4_sym g32 14336x4096 bf16"] = round(
         (n * 4 + n / 32 * 4) / timed(lambda: ops.fq_per_group_int4_sym(W, 32)) / 1e9, 1)
