@@ -313,3 +313,66 @@ def test_bf16_scale_precision_bit_exact(dtype):
     conv = qz.convert(lin)
     assert conv[0].scales.dtype == torch.bfloat16 and torch.equal(conv[0].scales.float().cpu(), w_s)
     assert bits_equal(conv(xd), y_fq)  # the converted layer computes what training saw
+
+
+def test_qat_lora_linear_forward_backward_and_frozen_weight_cache():
+    """QATLoRALinear (torchtune/modules/peft/lora.py:150-306) with both fake quantisers on the GPU:
+    y = F.linear(fq(x), fq(W)) + (alpha / r) B A x against the oracle's fake quantisation; gradients reach x and the
+    adapters only.  The fake-quantised frozen weight is built once and rebuilt after the weight is written."""
+    from torchtune_amd.modules.peft import LoRALinear, QATLoRALinear
+
+    gen = torch.Generator().manual_seed(77)
+    K, N, r, alpha, g = 256, 192, 8, 16.0, 32
+    W = (torch.randn(N, K, generator=gen) * 0.05).to(torch.bfloat16)
+    A = (torch.randn(r, K, generator=gen) * 0.05).to(torch.bfloat16)
+    B = (torch.randn(N, r, generator=gen) * 0.05).to(torch.bfloat16)
+    x = torch.randn(3, 17, K, generator=gen).to(torch.bfloat16)
+    prev = torch.get_default_dtype()
+    torch.set_default_dtype(torch.bfloat16)
+    try:
+        with torch.device(DEV):
+            base = LoRALinear(K, N, rank=r, alpha=alpha)
+    finally:
+        torch.set_default_dtype(prev)
+    with torch.no_grad():
+        base.weight.copy_(W.to(DEV))
+        base.lora_a.weight.copy_(A.to(DEV))
+        base.lora_b.weight.copy_(B.to(DEV))
+    layer = QATLoRALinear.from_lora_linear(
+        base, FakeQuantizeConfig(torch.int8, "per_token", is_symmetric=False), FakeQuantizeConfig(torch.int4, group_size=g))
+    layer.weight.requires_grad_(False)
+    xd = x.to(DEV).requires_grad_()
+
+    def expected(Wc):
+        x_fq, _, _ = fq.fq_per_token_int8_asym(x.view(-1, K))
+        w_fq, _ = fq.fq_per_group_int4_sym(Wc, g)
+        out = x_fq.float() @ w_fq.float().T + (alpha / r) * ((x.view(-1, K).float() @ A.float().T) @ B.float().T)
+        return out.view(3, 17, N), w_fq
+
+    want, w_fq = expected(W)
+    launches = []
+    ops.set_fq_timer(lambda kind, *a: launches.append(kind))  # counts launches; returning None records no events
+    try:
+        y = layer(xd)
+        y2 = layer(xd)
+        assert launches.count("per_group") == 1 and launches.count("per_token") == 2  # the weight side ran once
+        torch.testing.assert_close(y.float().cpu(), want, rtol=2e-2, atol=2e-2)
+        assert bits_equal(y, y2)
+        y.float().sum().backward()
+        assert xd.grad is not None and layer.lora_a.weight.grad is not None and layer.lora_b.weight.grad is not None
+        assert layer.weight.grad is None
+        torch.testing.assert_close(xd.grad.float().cpu().view(-1, K)[0],
+                                   (w_fq.float().sum(0) + (alpha / r) * (B.float().sum(0) @ A.float())), rtol=2e-2, atol=2e-2)
+        # writing the weight invalidates the cached fake-quantised copy
+        W2 = (W.float() * 1.5).to(torch.bfloat16)
+        with torch.no_grad():
+            layer.weight.copy_(W2.to(DEV))
+        y3 = layer(xd)
+        assert launches.count("per_group") == 2
+        torch.testing.assert_close(y3.float().cpu(), expected(W2)[0], rtol=2e-2, atol=2e-2)
+        # a trainable base weight is never cached (its gradient must flow through the straight-through estimator)
+        layer.weight.requires_grad_(True)
+        layer(xd).float().sum().backward()
+        assert layer.weight.grad is not None and launches.count("per_group") == 3
+    finally:
+        ops.set_fq_timer(None)

@@ -159,8 +159,29 @@ class QATLoRALinear(LoRALinear):
         else:
             self.weight_fake_quantizer = nn.Identity()
 
+    # The base weight of a QAT + LoRA layer is frozen, so its fake-quantised form only changes when the weight is
+    # written (load_state_dict, copy_).  With 288 GB of HBM it is kept instead of being rebuilt in every forward; set
+    # to False to recompute it each time, as the reference does.
+    cache_frozen_weight_fake_quant = True
+
+    def _fake_quantized_weight(self) -> torch.Tensor:
+        w, fq = self.weight, self.weight_fake_quantizer
+        cacheable = (
+            self.cache_frozen_weight_fake_quant and not w.requires_grad and w.is_cuda and getattr(fq, "enabled", False)
+        )
+        if not cacheable:
+            self._fq_weight_cache = None
+            return fq(w)
+        key = (w.data_ptr(), w._version, w.dtype, tuple(w.shape))
+        cached = getattr(self, "_fq_weight_cache", None)
+        if cached is None or cached[0] != key:
+            with torch.no_grad():
+                cached = (key, fq(w).detach())
+            self._fq_weight_cache = cached
+        return cached[1]
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        out = F.linear(self.activation_fake_quantizer(x), self.weight_fake_quantizer(self.weight))
+        out = F.linear(self.activation_fake_quantizer(x), self._fake_quantized_weight())
         if self.disabled:
             return out
         lora_out = self.lora_a(self.dropout(x))
