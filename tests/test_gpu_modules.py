@@ -229,3 +229,7 @@ def test_merged_checkpoint_weight_vs_oracle(N, K, r):
     assert (got.view(torch.int16) == want.view(torch.int16)).float().mean() > 0.98
     sd0 = {"l.weight": t, "l.lora_a.weight": A.to(DEV), "l.lora_b.weight": torch.zeros_like(B).to(DEV)}
     assert torch.equal(get_merged_lora_ckpt(sd0, rank=r, alpha=alpha)["l.weight"], t.get_original_weight())
+    # offloading variant: the kernel stores the merged weight straight into pinned host memory, same bits
+    sd_h = {"l.weight": t, "l.lora_a.weight": A.to(DEV), "l.lora_b.weight": B.to(DEV)}
+    host = get_merged_lora_ckpt(sd_h, rank=r, alpha=alpha, offload_to_cpu=True)["l.weight"]
+    assert host.device.type == "cpu" and host.is_pinned() and torch.equal(host, got)

@@ -47,7 +47,7 @@ def _get_lora_modules(state_dict: Dict[str, Any]) -> Set[str]:
 
 
 @torch.no_grad()
-def get_merged_lora_ckpt(state_dict: Dict[str, Any], rank: int, alpha: float) -> Dict[str, Any]:
+def get_merged_lora_ckpt(state_dict: Dict[str, Any], rank: int, alpha: float, offload_to_cpu: bool = False) -> Dict[str, Any]:
     """Fold every LoRA pair of ``state_dict`` into its base weight and delete the adapter entries; modifies and
     returns ``state_dict`` (``torchtune/modules/peft/_utils.py:193-271``; MoE experts raise).
 
@@ -56,7 +56,10 @@ def get_merged_lora_ckpt(state_dict: Dict[str, Any], rank: int, alpha: float) ->
 
     A base weight that is still an ``NF4Tensor`` on the GPU (a state dict taken without the dequantising hook) is
     dequantised and merged in one pass by the HIP kernel; a dense weight is updated as the reference does.
+    ``offload_to_cpu`` (not in the reference's signature) makes that kernel store the merged weight of a plain LoRA
+    module straight into pinned host memory, so the dense merged weight never exists on the GPU.
     """
+    wrote_to_host = None
     scale = alpha / rank
     for module in sorted(_get_lora_modules(state_dict)):
         if "experts" in module:
@@ -71,7 +74,12 @@ def get_merged_lora_ckpt(state_dict: Dict[str, Any], rank: int, alpha: float) ->
         )
         if fused:
             N, K = w.shape
-            merged = ops.nf4_dequantize_merge(w.quantized_data, w.block_scalers(), N, K, a.to(w.device), b.to(w.device), scale)
+            host = None
+            if offload_to_cpu and magnitude is None:
+                host = torch.empty(N, K, dtype=torch.bfloat16, pin_memory=True)
+                wrote_to_host = w.device
+            merged = ops.nf4_dequantize_merge(w.quantized_data, w.block_scalers(), N, K, a.to(w.device), b.to(w.device), scale,
+                                              out=host)
         elif magnitude is not None or isinstance(w, NF4Tensor):
             merged = w.to(a.dtype) + scale * b @ a
         else:
@@ -81,7 +89,11 @@ def get_merged_lora_ckpt(state_dict: Dict[str, Any], rank: int, alpha: float) ->
             weight_norm = torch.linalg.norm(merged, dim=1)
             merged *= (magnitude.to(merged.device) / weight_norm).view(-1, 1)
             del state_dict[f"{module}.magnitude"]
+        if offload_to_cpu and merged.is_cuda:
+            merged = merged.cpu()
         state_dict[f"{module}.weight"] = merged
         del state_dict[f"{module}.lora_a.weight"]
         del state_dict[f"{module}.lora_b.weight"]
+    if wrote_to_host is not None:
+        torch.cuda.current_stream(wrote_to_host).synchronize()
     return state_dict

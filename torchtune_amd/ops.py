@@ -105,15 +105,24 @@ def nf4_dequantize(
 
 
 def nf4_dequantize_merge(qdata: torch.Tensor, block_scalers: torch.Tensor, N: int, K: int, lora_a: torch.Tensor,
-                         lora_b: torch.Tensor, scale: float) -> torch.Tensor:
-    """bf16(D(W) + bf16(scale * bf16(lora_b @ lora_a))) for an NF4 [N, K] weight (block size 64) in one pass."""
+                         lora_b: torch.Tensor, scale: float, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """bf16(D(W) + bf16(scale * bf16(lora_b @ lora_a))) for an NF4 [N, K] weight (block size 64) in one pass.
+    ``out`` may be a contiguous bf16 [N, K] tensor on the same GPU or in pinned host memory (the kernel then stores over
+    PCIe; the caller synchronises the stream before reading it on the CPU)."""
     _need_gpu(qdata, "nf4_dequantize_merge")
     a = _bf16_2d(lora_a, "nf4_dequantize_merge: lora_a")
     b = _bf16_2d(lora_b, "nf4_dequantize_merge: lora_b")
     rank = a.shape[0]
     if a.shape != (rank, K) or b.shape != (N, rank):
         raise ValueError(f"nf4_dequantize_merge: lora_a {tuple(a.shape)} / lora_b {tuple(b.shape)} do not fit [{N}, {K}]")
-    out = torch.empty(N, K, dtype=torch.bfloat16, device=qdata.device)
+    if out is None:
+        out = torch.empty(N, K, dtype=torch.bfloat16, device=qdata.device)
+    else:
+        on_device = out.is_cuda and out.device == qdata.device
+        if not (on_device or (out.device.type == "cpu" and out.is_pinned())):
+            raise ValueError("nf4_dequantize_merge: `out` must live on the weight's GPU or in pinned host memory")
+        if out.dtype != torch.bfloat16 or tuple(out.shape) != (N, K) or not out.is_contiguous():
+            raise ValueError(f"nf4_dequantize_merge: `out` must be a contiguous bfloat16 [{N}, {K}] tensor")
     lib = _lib.load()
     with torch.cuda.device(qdata.device):
         rc = lib.ttamd_nf4_dequantize_merge_bf16(qdata.data_ptr(), block_scalers.data_ptr(), a.data_ptr(), b.data_ptr(), rank,
