@@ -408,3 +408,41 @@ def test_seeded_sweep_of_shapes_ranks_and_options_against_fp32_reference():
         if r:
             gx_ref = gx_ref + gh.float() @ A.float()
         torch.testing.assert_close(gx.float(), gx_ref, rtol=1e-2, atol=1e-2 * max(1.0, float(gx_ref.abs().max()) / 8), msg=tag)
+
+
+@pytest.mark.parametrize("N,K", [(64, 64), (192, 320 * 4), (1024, 4096), (4096, 1024 + 64), (8192, 256 + 64), (256, 8192 + 64)])
+def test_few_tokens_take_the_weight_streaming_kernel(N, K):
+    """M <= 64 (decode / evaluation): the library streams the packed weight once instead of tiling.  Every token count
+    from 1 to 64 that touches a tile edge, K with and without a half chunk at the end, adapter ranks, bias and column
+    scale, against fp32 matmuls of the bit-exact dequantised weight; and the M = 64 / M = 65 results (two different
+    kernels) agree row for row within the same tolerance.  The last two shapes take the wide-layer (two row tiles per
+    workgroup) and the long-contraction (sixteen waves) configurations."""
+    if (N // 64) * K % 256:
+        pytest.skip("to_nf4 needs whole scaler blocks")
+    g = torch.Generator(device=DEV).manual_seed(N + K)
+    t = to_nf4((torch.randn(N, K, device=DEV, generator=g) * 0.02).to(BF))
+    D = t.get_original_weight().float()
+    bs = t.block_scalers()
+    for M, r, use_bias, use_cs in [(1, 0, False, False), (2, 8, True, False), (7, 16, False, True), (15, 64, True, True),
+                                   (16, 24, False, False), (17, 8, True, True), (32, 0, True, False), (33, 16, False, False),
+                                   (48, 40, True, True), (63, 8, False, True), (64, 16, True, False)]:
+        x = torch.randn(M, K, device=DEV, generator=g).to(BF)
+        h = (torch.randn(M, max(r, 1), device=DEV, generator=g)).to(BF)[:, :r].contiguous() if r else None
+        B = (torch.randn(N, max(r, 1), device=DEV, generator=g) * 0.05).to(BF)[:, :r].contiguous() if r else None
+        bias = (torch.randn(N, device=DEV, generator=g) * 0.1).to(BF) if use_bias else None
+        cs = (torch.rand(N, device=DEV, generator=g) + 0.5).to(BF) if use_cs else None
+        y = ops.nf4_lora_linear_fwd(x, t.quantized_data, bs, N, h, B, 0.5, bias, col_scale=cs)
+        ref = x.float() @ D.T
+        if r:
+            ref = ref + (h.float() * 0.5).to(BF).float() @ B.float().T
+        if use_bias:
+            ref = ref + bias.float()
+        if use_cs:
+            ref = ref * cs.float()
+        torch.testing.assert_close(y.float(), ref, rtol=1e-2, atol=1e-2, msg=f"M{M} r{r}")
+        assert torch.equal(y, ops.nf4_lora_linear_fwd(x, t.quantized_data, bs, N, h, B, 0.5, bias, col_scale=cs))
+    x65 = torch.randn(65, K, device=DEV, generator=g).to(BF)
+    y65 = ops.nf4_lora_linear_fwd(x65, t.quantized_data, bs, N)
+    y64 = ops.nf4_lora_linear_fwd(x65[:64].contiguous(), t.quantized_data, bs, N)
+    torch.testing.assert_close(y64.float(), y65[:64].float(), rtol=1e-2, atol=1e-2)
+    torch.testing.assert_close(y65.float(), x65.float() @ D.T, rtol=1e-2, atol=1e-2)

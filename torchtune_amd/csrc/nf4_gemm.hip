@@ -413,6 +413,10 @@ int check_gemm_args(const char* who, const void* a, const uint8_t* qdata, const 
 int run_gemm_rs(const void* X, const uint8_t* codes, const void* scal, int mode, const void* lX, const void* lW,
                 bool lw_row_major, int R, float lscale, const void* bias, const void* cscale, void* C, int64_t M, int64_t Nout,
                 int64_t Kc, hipStream_t s);
+// nf4_small_m.hip
+int small_m_limit();
+int run_small_m(const void* x, const uint8_t* codes, const void* bscal, const void* h, const void* lora_b, int R, float lscale,
+                const void* bias, const void* cscale, void* y, int64_t M, int64_t N, int64_t K, hipStream_t s);
 }  // namespace ttamd
 
 using namespace ttamd;
@@ -444,6 +448,9 @@ int lora_linear_fwd(const char* who, const void* x, const uint8_t* quantized_dat
   TT_REQUIRE((bias == nullptr || (reinterpret_cast<uintptr_t>(bias) & 7u) == 0) &&
                  (col_scale == nullptr || (reinterpret_cast<uintptr_t>(col_scale) & 7u) == 0),
              "%s: bias / col_scale must be 8-byte aligned", who);
+  if (M <= small_m_limit())  // a handful of tokens: stream the packed weight once (nf4_small_m.hip)
+    return run_small_m(x, quantized_data, block_scalers, h, lora_b, rank, scale, bias, col_scale, y, M, N, K,
+                       reinterpret_cast<hipStream_t>(stream));
   if (block_scalers_t) {
     TT_REQUIRE(aligned16(block_scalers_t), "%s: block_scalers_t must be 16-byte aligned", who);
     return run_gemm_rs(x, quantized_data, block_scalers_t, 2, h, lora_b, true, rank, scale, bias, col_scale, y, M, N, K,
