@@ -140,6 +140,8 @@ int ttamd_lora_hidden_bf16(const void* x, const void* lora_a, void* h, int64_t M
  * Requires K % 64 == 0, N % 64 == 0, rank % 8 == 0, 0 <= rank <= 64.
  * D(W) is bit-identical to ttamd_nf4_dequantize's output; all products are accumulated in fp32 and the sum is
  * rounded to bf16 once (the eager reference rounds after each of its five ops).
+ * M <= 64 (decode, evaluation) runs a kernel that streams the packed weight once instead of the tiled one; same
+ * operands, same expansion of the weight, fp32 sums in a different but fixed order.
  */
 int ttamd_nf4_lora_linear_fwd_bf16(const void* x, const uint8_t* quantized_data, const void* block_scalers,
                                    const void* block_scalers_t, const void* h, const void* lora_b, int rank, float scale,
