@@ -199,6 +199,29 @@ int ttamd_nf4_linear_bwd_dx_bf16(const void* gy, const uint8_t* quantized_data, 
                                  const void* lora_a, int rank, void* gx, int64_t M, int64_t N, int64_t K, void* stream);
 
 /*
+ * The same two GEMMs for token counts between the few-token kernel and a full grid (64 < M, at most 128 output tiles
+ * of 128 x 256): with a workspace the contraction is cut into up to 16 slices, one workgroup per tile per slice, fp32
+ * partial tiles in the workspace, and a second kernel adds the slices in a fixed order, then bias, column scale and
+ * the rounding to bf16.  The plain entry points above are these with workspace = NULL (no slicing: a launch of few
+ * tiles then leaves most of the chip idle).  The reference has no counterpart: it dequantises the weight and calls a
+ * dense GEMM (nf4_linear.py:67-70, lora.py:138).
+ *   ttamd_nf4_gemm_workspace_bytes(M, n_out, k_contract): bytes to pass (0: the launch is not sliced); n_out /
+ *     k_contract = N / K for the forward, K / N for the grad-input.
+ *   ttamd_nf4_lora_linear_fwd_ws_bf16: col_scale NULL = ttamd_nf4_lora_linear_fwd_bf16, else = ttamd_nf4_dora_linear_fwd_bf16.
+ *   ttamd_nf4_linear_bwd_dx_ws_bf16: slices only the variant with the transposed copies.
+ * A workspace smaller than ttamd_nf4_gemm_workspace_bytes says, or NULL, runs the unsliced kernel.
+ */
+size_t ttamd_nf4_gemm_workspace_bytes(int64_t M, int64_t n_out, int64_t k_contract);
+int ttamd_nf4_lora_linear_fwd_ws_bf16(const void* x, const uint8_t* quantized_data, const void* block_scalers,
+                                      const void* block_scalers_t, const void* h, const void* lora_b, int rank, float scale,
+                                      const void* bias, const void* col_scale, void* y, int64_t M, int64_t N, int64_t K,
+                                      void* workspace, size_t workspace_bytes, void* stream);
+int ttamd_nf4_linear_bwd_dx_ws_bf16(const void* gy, const uint8_t* quantized_data, const void* block_scalers,
+                                    const uint8_t* quantized_data_t, const void* block_scalers_t, const void* gh,
+                                    const void* lora_a, int rank, void* gx, int64_t M, int64_t N, int64_t K, void* workspace,
+                                    size_t workspace_bytes, void* stream);
+
+/*
  * Adapter gradients (what autograd derives for lora.py:144-146):
  *     gh = scale . gy . B        [M,rank] bf16
  *     gA = gh^T . x              [rank,K] bf16

@@ -336,9 +336,17 @@ def test_token_dimension_beyond_32_bit_offsets_is_split_into_row_ranges():
     assert y.shape == (M, N)
     cut = ((1 << 32) - 1) // (2 * K) // 256 * 256
     assert 0 < cut < M
+    from torchtune_amd import _lib
+
+    lib = _lib.load()
     for lo, hi in ((0, 512), (cut - 256, cut + 256), (M - 300, M)):
-        part = ops.nf4_lora_linear_fwd(x[lo:hi].contiguous(), t.quantized_data, bs, N, h[lo:hi].contiguous(), B, 2.0, None,
-                                       block_scalers_t=bst)
+        # the same kernel on those rows alone: no workspace, so the contraction of this small launch is not sliced
+        xp, hp = x[lo:hi].contiguous(), h[lo:hi].contiguous()
+        part = torch.empty(hi - lo, N, device=DEV, dtype=BF)
+        assert lib.ttamd_nf4_lora_linear_fwd_bf16(xp.data_ptr(), t.quantized_data.data_ptr(), bs.data_ptr(), bst.data_ptr(),
+                                                  hp.data_ptr(), B.data_ptr(), r, 2.0, None, part.data_ptr(), hi - lo, N, K,
+                                                  None) == 0
+        torch.cuda.synchronize()
         assert torch.equal(y[lo:hi], part)
     D = t.get_original_weight().float()
     ref = x[M - 300:].float() @ D.T + 2.0 * (h[M - 300:].float() @ B.float().T)
@@ -446,3 +454,59 @@ def test_few_tokens_take_the_weight_streaming_kernel(N, K):
     y64 = ops.nf4_lora_linear_fwd(x65[:64].contiguous(), t.quantized_data, bs, N)
     torch.testing.assert_close(y64.float(), y65[:64].float(), rtol=1e-2, atol=1e-2)
     torch.testing.assert_close(y65.float(), x65.float() @ D.T, rtol=1e-2, atol=1e-2)
+
+
+@pytest.mark.parametrize("M,N,K", [(65, 256, 512), (128, 1024, 4096), (200, 4096, 1024 + 192), (512, 1024, 4096), (1000, 512, 2048)])
+def test_few_output_tiles_slice_the_contraction(M, N, K):
+    """64 < M with at most 128 output tiles: given a workspace the library cuts the contraction into slices (one
+    workgroup per tile per slice, fp32 partial tiles, a fixed-order reduction that also adds bias and column scale).
+    Forward (both scaler layouts, adapter, bias, column scale) and grad-input against fp32 matmuls of the dequantised
+    weight, against the unsliced kernel (workspace NULL), and twice for determinism; K = 1216 leaves the last slice
+    shorter than the others."""
+    from torchtune_amd import _lib
+
+    lib = _lib.load()
+    g = torch.Generator(device=DEV).manual_seed(M + N + K)
+    t = to_nf4((torch.randn(N, K, device=DEV, generator=g) * 0.02).to(BF))
+    D = t.get_original_weight().float()
+    bs = t.block_scalers()
+    qt, bst = t.backward_copy()
+    r = 16
+    x = torch.randn(M, K, device=DEV, generator=g).to(BF)
+    A = (torch.randn(r, K, device=DEV, generator=g) * 0.05).to(BF)
+    B = (torch.randn(N, r, device=DEV, generator=g) * 0.05).to(BF)
+    bias = (torch.randn(N, device=DEV, generator=g) * 0.1).to(BF)
+    cs = (torch.rand(N, device=DEV, generator=g) + 0.5).to(BF)
+    h = ops.lora_hidden(x, A)
+    nbytes = lib.ttamd_nf4_gemm_workspace_bytes(M, N, K)
+    assert nbytes > 0 and nbytes % (M * N * 4) == 0 and 2 <= nbytes // (M * N * 4) <= 16
+    assert lib.ttamd_nf4_gemm_workspace_bytes(64, N, K) == 0  # the few-token kernel needs none
+    assert lib.ttamd_nf4_gemm_workspace_bytes(16384, 4096, 4096) == 0  # nor does a full grid
+    ref = ((x.float() @ D.T + bias.float() + 0.5 * (h.float() @ B.float().T)) * cs.float())
+    for scal_t in (None, bst):
+        y = ops.nf4_lora_linear_fwd(x, t.quantized_data, bs, N, h, B, 0.5, bias, block_scalers_t=scal_t, col_scale=cs)
+        torch.testing.assert_close(y.float(), ref, rtol=1e-2, atol=1e-2)
+        assert torch.equal(y, ops.nf4_lora_linear_fwd(x, t.quantized_data, bs, N, h, B, 0.5, bias, block_scalers_t=scal_t,
+                                                      col_scale=cs))
+        y0 = torch.empty_like(y)
+        assert lib.ttamd_nf4_lora_linear_fwd_ws_bf16(
+            x.data_ptr(), t.quantized_data.data_ptr(), bs.data_ptr(), scal_t.data_ptr() if scal_t is not None else None,
+            h.data_ptr(), B.data_ptr(), r, 0.5, bias.data_ptr(), cs.data_ptr(), y0.data_ptr(), M, N, K, None, 0, None) == 0
+        torch.cuda.synchronize()
+        # same operands, fp32 sums in a different order: the two kernels agree to a bf16 rounding step of the result
+        torch.testing.assert_close(y.float(), y0.float(), rtol=1e-2, atol=1e-2)
+    # a workspace that is too small is ignored (the unsliced kernel runs), never written beyond its size
+    small = torch.zeros(1024, dtype=torch.float32, device=DEV)
+    y1 = torch.empty(M, N, dtype=BF, device=DEV)
+    assert lib.ttamd_nf4_lora_linear_fwd_ws_bf16(x.data_ptr(), t.quantized_data.data_ptr(), bs.data_ptr(), None, h.data_ptr(),
+                                                 B.data_ptr(), r, 0.5, bias.data_ptr(), cs.data_ptr(), y1.data_ptr(), M, N, K,
+                                                 small.data_ptr(), 4096, None) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(y1, y0) and float(small.abs().max()) == 0.0
+    # grad-input: contraction over N
+    gy = torch.randn(M, N, device=DEV, generator=g).to(BF)
+    gh = (torch.randn(M, r, device=DEV, generator=g) * 0.1).to(BF)
+    gx = ops.nf4_linear_bwd_dx(gy, t.quantized_data, bs, K, gh, A, transposed=(qt, bst))
+    gx_ref = gy.float() @ D + gh.float() @ A.float()
+    torch.testing.assert_close(gx.float(), gx_ref, rtol=1e-2, atol=1e-2 * max(1.0, float(gx_ref.abs().max()) / 8))
+    assert torch.equal(gx, ops.nf4_linear_bwd_dx(gy, t.quantized_data, bs, K, gh, A, transposed=(qt, bst)))

@@ -412,7 +412,8 @@ int check_gemm_args(const char* who, const void* a, const uint8_t* qdata, const 
 // nf4_gemm_rs.hip
 int run_gemm_rs(const void* X, const uint8_t* codes, const void* scal, int mode, const void* lX, const void* lW,
                 bool lw_row_major, int R, float lscale, const void* bias, const void* cscale, void* C, int64_t M, int64_t Nout,
-                int64_t Kc, hipStream_t s);
+                int64_t Kc, void* workspace, size_t workspace_bytes, hipStream_t s);
+size_t gemm_rs_workspace_bytes(int64_t M, int64_t Nout, int64_t Kc);
 // nf4_small_m.hip
 int small_m_limit();
 int run_small_m(const void* x, const uint8_t* codes, const void* bscal, const void* h, const void* lora_b, int R, float lscale,
@@ -443,7 +444,8 @@ extern "C" int ttamd_nf4_block_scalers(const int8_t* quantized_scalers, const vo
 namespace {
 int lora_linear_fwd(const char* who, const void* x, const uint8_t* quantized_data, const void* block_scalers,
                     const void* block_scalers_t, const void* h, const void* lora_b, int rank, float scale, const void* bias,
-                    const void* col_scale, void* y, int64_t M, int64_t N, int64_t K, void* stream) {
+                    const void* col_scale, void* y, int64_t M, int64_t N, int64_t K, void* workspace, size_t workspace_bytes,
+                    void* stream) {
   if (int rc = check_gemm_args(who, x, quantized_data, block_scalers, y, M, N, K, rank, h, lora_b)) return rc;
   TT_REQUIRE((bias == nullptr || (reinterpret_cast<uintptr_t>(bias) & 7u) == 0) &&
                  (col_scale == nullptr || (reinterpret_cast<uintptr_t>(col_scale) & 7u) == 0),
@@ -454,10 +456,10 @@ int lora_linear_fwd(const char* who, const void* x, const uint8_t* quantized_dat
   if (block_scalers_t) {
     TT_REQUIRE(aligned16(block_scalers_t), "%s: block_scalers_t must be 16-byte aligned", who);
     return run_gemm_rs(x, quantized_data, block_scalers_t, 2, h, lora_b, true, rank, scale, bias, col_scale, y, M, N, K,
-                       reinterpret_cast<hipStream_t>(stream));
+                       workspace, workspace_bytes, reinterpret_cast<hipStream_t>(stream));
   }
   return run_gemm_rs(x, quantized_data, block_scalers, 0, h, lora_b, true, rank, scale, bias, col_scale, y, M, N, K,
-                     reinterpret_cast<hipStream_t>(stream));
+                     workspace, workspace_bytes, reinterpret_cast<hipStream_t>(stream));
 }
 }  // namespace
 
@@ -466,7 +468,20 @@ extern "C" int ttamd_nf4_lora_linear_fwd_bf16(const void* x, const uint8_t* quan
                                               float scale, const void* bias, void* y, int64_t M, int64_t N, int64_t K,
                                               void* stream) {
   return lora_linear_fwd("nf4_lora_linear_fwd", x, quantized_data, block_scalers, block_scalers_t, h, lora_b, rank, scale, bias,
-                         nullptr, y, M, N, K, stream);
+                         nullptr, y, M, N, K, nullptr, 0, stream);
+}
+
+extern "C" size_t ttamd_nf4_gemm_workspace_bytes(int64_t M, int64_t n_out, int64_t k_contract) {
+  if (M <= small_m_limit() || M <= 0 || n_out <= 0 || k_contract <= 0) return 0;
+  return gemm_rs_workspace_bytes(M, n_out, k_contract);
+}
+
+extern "C" int ttamd_nf4_lora_linear_fwd_ws_bf16(const void* x, const uint8_t* quantized_data, const void* block_scalers,
+                                                 const void* block_scalers_t, const void* h, const void* lora_b, int rank,
+                                                 float scale, const void* bias, const void* col_scale, void* y, int64_t M,
+                                                 int64_t N, int64_t K, void* workspace, size_t workspace_bytes, void* stream) {
+  return lora_linear_fwd("nf4_lora_linear_fwd_ws", x, quantized_data, block_scalers, block_scalers_t, h, lora_b, rank, scale,
+                         bias, col_scale, y, M, N, K, workspace, workspace_bytes, stream);
 }
 
 extern "C" int ttamd_nf4_dora_linear_fwd_bf16(const void* x, const uint8_t* quantized_data, const void* block_scalers,
@@ -475,7 +490,7 @@ extern "C" int ttamd_nf4_dora_linear_fwd_bf16(const void* x, const uint8_t* quan
                                               int64_t N, int64_t K, void* stream) {
   TT_REQUIRE(col_scale, "nf4_dora_linear_fwd: col_scale is null");
   return lora_linear_fwd("nf4_dora_linear_fwd", x, quantized_data, block_scalers, block_scalers_t, h, lora_b, rank, scale, bias,
-                         col_scale, y, M, N, K, stream);
+                         col_scale, y, M, N, K, nullptr, 0, stream);
 }
 
 extern "C" int ttamd_nf4_transpose_for_backward(const uint8_t* quantized_data, const void* block_scalers, int64_t N, int64_t K,
@@ -495,17 +510,17 @@ extern "C" int ttamd_nf4_transpose_for_backward(const uint8_t* quantized_data, c
   return check_launch("nf4_transpose_for_backward");
 }
 
-extern "C" int ttamd_nf4_linear_bwd_dx_bf16(const void* gy, const uint8_t* quantized_data, const void* block_scalers,
-                                            const uint8_t* quantized_data_t, const void* block_scalers_t, const void* gh,
-                                            const void* lora_a, int rank, void* gx, int64_t M, int64_t N, int64_t K,
-                                            void* stream) {
+extern "C" int ttamd_nf4_linear_bwd_dx_ws_bf16(const void* gy, const uint8_t* quantized_data, const void* block_scalers,
+                                               const uint8_t* quantized_data_t, const void* block_scalers_t, const void* gh,
+                                               const void* lora_a, int rank, void* gx, int64_t M, int64_t N, int64_t K,
+                                               void* workspace, size_t workspace_bytes, void* stream) {
   if (int rc = check_gemm_args("nf4_linear_bwd_dx", gy, quantized_data, block_scalers, gx, M, N, K, rank, gh, lora_a)) return rc;
   TT_REQUIRE((quantized_data_t == nullptr) == (block_scalers_t == nullptr),
              "nf4_linear_bwd_dx: the transposed codes and scalers must be given together");
   if (quantized_data_t != nullptr) {
     TT_REQUIRE(aligned16(quantized_data_t) && aligned16(block_scalers_t), "nf4_linear_bwd_dx: transposed copies must be 16-byte aligned");
     return run_gemm_rs(gy, quantized_data_t, block_scalers_t, 1, gh, lora_a, false, rank, 1.0f, nullptr, nullptr, gx, M, K, N,
-                       reinterpret_cast<hipStream_t>(stream));
+                       workspace, workspace_bytes, reinterpret_cast<hipStream_t>(stream));
   }
   GemmArgs g;
   g.A = reinterpret_cast<const uint16_t*>(gy);
@@ -518,4 +533,12 @@ extern "C" int ttamd_nf4_linear_bwd_dx_bf16(const void* gy, const uint8_t* quant
   g.M = (int)M; g.N = (int)N; g.K = (int)K; g.R = rank;
   g.lscale = 1.0f;
   return dispatch_gemm<true>(g, reinterpret_cast<hipStream_t>(stream));
+}
+
+extern "C" int ttamd_nf4_linear_bwd_dx_bf16(const void* gy, const uint8_t* quantized_data, const void* block_scalers,
+                                            const uint8_t* quantized_data_t, const void* block_scalers_t, const void* gh,
+                                            const void* lora_a, int rank, void* gx, int64_t M, int64_t N, int64_t K,
+                                            void* stream) {
+  return ttamd_nf4_linear_bwd_dx_ws_bf16(gy, quantized_data, block_scalers, quantized_data_t, block_scalers_t, gh, lora_a, rank,
+                                         gx, M, N, K, nullptr, 0, stream);
 }

@@ -56,7 +56,9 @@ struct RsArgs {
   const uint16_t* bias;  // [Nout] bf16 or null
   const uint16_t* cscale;  // [Nout] bf16 or null: C = (acc + bias) * cscale per column (DoRA's magnitude / norm)
   uint16_t* C;           // [M, Nout] bf16
+  float* part;           // SPLIT: fp32 partial products [splits, M, Nout], summed by nf4_gemm_rs_reduce_kernel
   int M, Nout, Kc, R;
+  int ksteps;            // SPLIT: 64-wide k-steps per slice of the contraction (blockIdx.y = slice)
   int lw_row_major;
   float lscale;
   int tiles_m, tiles_n;
@@ -80,7 +82,10 @@ struct RsLayout {
 // MODE 0: one scaler per (output column, 64-wide k-step), scaler tensor laid out like the weight's blocks
 // MODE 2: the same scalers, tensor transposed so that the 64 columns of a wave are contiguous (one coalesced load)
 // MODE 1: one scaler per contraction element, shared by the wave's 64 columns (the transposed weight of the backward)
-template <int BM, int MODE>
+// SPLIT: the contraction is cut into gridDim.y slices so that a launch with few output tiles still fills the chip; a
+// workgroup then leaves its tile as fp32 in g.part (slice 0 includes the adapter) and bias, column scale and the
+// rounding to bf16 happen in nf4_gemm_rs_reduce_kernel, which adds the slices in a fixed order.
+template <int BM, int MODE, bool SPLIT>
 __global__ __launch_bounds__(256) void nf4_gemm_rs_kernel(const RsArgs g) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the body uses LDS address-space casts and gfx950 builtins the host pass cannot parse
   static_assert(BM == 256 || BM == 128, "BM");
@@ -115,7 +120,12 @@ __global__ __launch_bounds__(256) void nf4_gemm_rs_kernel(const RsArgs g) {
   }
   const int m0 = tile_m * BM, n0 = tile_n * kBN;
   const int Kc = g.Kc;
-  const int nk = Kc >> 6;
+  const int nkf = Kc >> 6;  // k-steps of the whole contraction: the row stride of the MODE 0 scalers
+  int kb = 0, nk = nkf;     // this workgroup's k-steps are [kb, kb + nk)
+  if constexpr (SPLIT) {
+    kb = blockIdx.y * g.ksteps;
+    nk = nkf - kb < g.ksteps ? nkf - kb : g.ksteps;
+  }
 
   // ---- table: entry(byte) = (nf4[byte >> 4], nf4[byte & 15]) as two fp32 (each exactly a bf16 value)
   //      It is a separate LDS object so that the compiler can tell table reads from the direct-to-LDS destinations.
@@ -143,7 +153,7 @@ __global__ __launch_bounds__(256) void nf4_gemm_rs_kernel(const RsArgs g) {
     int col = n0 + wv * 64 + 32 * j + l31;
     col = col < g.Nout ? col : g.Nout - 1;
     w_off[j] = (uint32_t)(((int64_t)col * Kc) >> 1) + 16 * h;
-    s_off[j] = (uint32_t)col * (uint32_t)nk * 4u;
+    s_off[j] = (uint32_t)col * (uint32_t)nkf * 4u;
   }
   if constexpr (SCAL_T) {
     int col = n0 + wv * 64 + lane;  // lane l fetches the scaler of the wave's column l
@@ -194,7 +204,7 @@ __global__ __launch_bounds__(256) void nf4_gemm_rs_kernel(const RsArgs g) {
     return b;
   };
   auto batch_addr = [&](int t, int sa, int sw) -> BatchAddr {
-    const int tk = t < nk ? t : nk - 1;
+    const int tk = kb + (t < nk ? t : nk - 1);
     return batch_addr_at(reinterpret_cast<const char*>(g.X) + ((int64_t)tk << 7),      // + k0 * 2 bytes
                          reinterpret_cast<const char*>(g.codes) + ((int64_t)tk << 5),  // + k0 / 2 bytes
                          reinterpret_cast<const char*>(g.scal) + tk * s_stride, sa, sw);
@@ -375,7 +385,7 @@ __global__ __launch_bounds__(256) void nf4_gemm_rs_kernel(const RsArgs g) {
 
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the clamped batches issued by the last two steps
   // ---- adapter: R extra contraction steps, operands straight from global memory
-  if (g.R > 0) {
+  if (g.R > 0 && (!SPLIT || blockIdx.y == 0)) {
     for (int rc = 0; rc < g.R; rc += 16) {
       const int r0 = rc + 8 * h;
       const bool in = r0 < g.R;  // R % 8 == 0: a lane's 8 indices are all in or all out
@@ -425,6 +435,24 @@ __global__ __launch_bounds__(256) void nf4_gemm_rs_kernel(const RsArgs g) {
   //      which the memory system turns into partial-line read-modify-writes.  Instead each wave transposes its
   //      BM x 64 band through LDS (the activation ring is free now: BM x 128 bytes per wave) and writes whole
   //      128-byte row segments.  16-byte chunk c of row r sits in slot c ^ (r & 7): both sides are conflict-free.
+  if constexpr (SPLIT) {
+    // fp32 partial tile, straight from the registers: a lane holds four consecutive columns of a row (16 bytes), the
+    // two halves of a wave make 32 bytes and the four q of a weight tile complete the row's 128-byte line
+    if (n0 + wv * 64 >= g.Nout) return;
+    float* P = g.part + (int64_t)blockIdx.y * g.M * g.Nout + n0 + wv * 64 + 4 * h;
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+      const int row = m0 + 32 * i + l31;
+      if (row >= g.M) continue;
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          *reinterpret_cast<f32x4_t*>(P + (int64_t)row * g.Nout + 32 * j + 8 * q) =
+              f32x4_t{acc[j][i][4 * q], acc[j][i][4 * q + 1], acc[j][i][4 * q + 2], acc[j][i][4 * q + 3]};
+    }
+    return;
+  }
   __syncthreads();                      // every wave is done reading the activation ring
   if (n0 + wv * 64 >= g.Nout) return;  // the whole 64-column band of this wave lies outside (no barrier follows)
   {
@@ -469,8 +497,47 @@ __global__ __launch_bounds__(256) void nf4_gemm_rs_kernel(const RsArgs g) {
 #endif
 }
 
-template <int BM, int MODE>
-int launch_rs(RsArgs& g, hipStream_t s) {
+// C[m][n] = bf16((sum over slices of part[s][m][n] + bias[n]) * cscale[n]); a thread takes 8 consecutive columns.
+__global__ __launch_bounds__(256) void nf4_gemm_rs_reduce_kernel(const float* __restrict__ part, int splits, int64_t mn,
+                                                                 int Nout, const uint16_t* __restrict__ bias,
+                                                                 const uint16_t* __restrict__ cscale, uint16_t* __restrict__ C) {
+  const int64_t e = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 8;
+  if (e >= mn) return;
+  float v[8];
+  {
+    const f32x4_t a = *reinterpret_cast<const f32x4_t*>(part + e), b = *reinterpret_cast<const f32x4_t*>(part + e + 4);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+  }
+  for (int sidx = 1; sidx < splits; ++sidx) {
+    const float* p = part + (int64_t)sidx * mn + e;
+    const f32x4_t a = *reinterpret_cast<const f32x4_t*>(p), b = *reinterpret_cast<const f32x4_t*>(p + 4);
+    v[0] += a.x; v[1] += a.y; v[2] += a.z; v[3] += a.w; v[4] += b.x; v[5] += b.y; v[6] += b.z; v[7] += b.w;
+  }
+  const int n = (int)(e % Nout);  // Nout % 8 == 0: the 8 columns share a row
+  if (bias) {
+    const u32x4_t bb = *reinterpret_cast<const u32x4_t*>(bias + n);
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      v[2 * d] += bits_f32(bb[d] << 16);
+      v[2 * d + 1] += bits_f32(bb[d] & 0xffff0000u);
+    }
+  }
+  if (cscale) {
+    const u32x4_t cc = *reinterpret_cast<const u32x4_t*>(cscale + n);
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      v[2 * d] *= bits_f32(cc[d] << 16);
+      v[2 * d + 1] *= bits_f32(cc[d] & 0xffff0000u);
+    }
+  }
+  u32x4_t o;
+#pragma unroll
+  for (int d = 0; d < 4; ++d) o[d] = pack_bf16x2(v[2 * d], v[2 * d + 1]);
+  *reinterpret_cast<u32x4_t*>(C + e) = o;
+}
+
+template <int BM, int MODE, bool SPLIT>
+int launch_rs(RsArgs& g, int splits, hipStream_t s) {
   using L = RsLayout<BM>;
   g.tiles_m = (g.M + BM - 1) / BM;
   g.tiles_n = (g.Nout + kBN - 1) / kBN;
@@ -479,22 +546,40 @@ int launch_rs(RsArgs& g, hipStream_t s) {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = -1;
   if (dev < 0 || !attr_set[dev]) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&nf4_gemm_rs_kernel<BM, MODE>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&nf4_gemm_rs_kernel<BM, MODE, SPLIT>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, L::kTotal);
     if (e != hipSuccess)
       return fail(TTAMD_ELAUNCH, "nf4_gemm_rs: cannot reserve %d bytes of LDS: %s", L::kTotal, hipGetErrorString(e));
     if (dev >= 0) attr_set[dev] = true;
   }
-  nf4_gemm_rs_kernel<BM, MODE><<<dim3((unsigned)(g.tiles_m * g.tiles_n)), dim3(256), L::kTotal, s>>>(g);
+  nf4_gemm_rs_kernel<BM, MODE, SPLIT><<<dim3((unsigned)(g.tiles_m * g.tiles_n), (unsigned)splits), dim3(256), L::kTotal, s>>>(g);
   return check_launch("nf4_gemm_rs");
+}
+
+// Slices of the contraction for a launch that would leave half of the chip or more idle: enough to reach about one
+// workgroup per CU, at least four k-steps (256 elements) each, at most 16.  1 = do not split.
+int choose_splits(int64_t M, int64_t Nout, int64_t Kc) {
+  const int64_t tiles = ((M + 127) / 128) * ((Nout + kBN - 1) / kBN);  // small launches use 128-row tiles
+  if (tiles > 128) return 1;
+  int64_t sp = 256 / tiles;
+  const int64_t by_k = (Kc / 64) / 4;
+  sp = sp < by_k ? sp : by_k;
+  sp = sp < 16 ? sp : 16;
+  return sp < 2 ? 1 : (int)sp;
 }
 
 }  // namespace
 
-// Entry used by the C-ABI wrappers in nf4_gemm.hip.
+// Bytes of workspace with which run_gemm_rs cuts the contraction of a small launch into slices (0: it would not).
+size_t gemm_rs_workspace_bytes(int64_t M, int64_t Nout, int64_t Kc) {
+  const int sp = choose_splits(M, Nout, Kc);
+  return sp > 1 ? (size_t)sp * (size_t)M * (size_t)Nout * sizeof(float) : 0;
+}
+
+// Entry used by the C-ABI wrappers in nf4_gemm.hip.  `workspace` may be null: then small launches are not sliced.
 int run_gemm_rs(const void* X, const uint8_t* codes, const void* scal, int mode, const void* lX, const void* lW,
                 bool lw_row_major, int R, float lscale, const void* bias, const void* cscale, void* C, int64_t M, int64_t Nout,
-                int64_t Kc, hipStream_t s) {
+                int64_t Kc, void* workspace, size_t workspace_bytes, hipStream_t s) {
   // per-lane byte offsets inside the kernel are 32-bit: the weight must fit them, and a token dimension too long for
   // them is cut into row ranges (multiples of the 256-row tile) that are launched one after the other
   TT_REQUIRE(Nout * Kc / 2 < (int64_t(1) << 32) && Nout * (Kc / 64) * 4 < (int64_t(1) << 32) && Kc * 2 * 256 < (int64_t(1) << 32),
@@ -505,7 +590,7 @@ int run_gemm_rs(const void* X, const uint8_t* codes, const void* scal, int mode,
       const int64_t rows = M - r0 < max_rows ? M - r0 : max_rows;
       const int rc = run_gemm_rs(reinterpret_cast<const uint16_t*>(X) + r0 * Kc, codes, scal, mode,
                                  lX ? reinterpret_cast<const uint16_t*>(lX) + r0 * R : nullptr, lW, lw_row_major, R, lscale, bias,
-                                 cscale, reinterpret_cast<uint16_t*>(C) + r0 * Nout, rows, Nout, Kc, s);
+                                 cscale, reinterpret_cast<uint16_t*>(C) + r0 * Nout, rows, Nout, Kc, nullptr, 0, s);
       if (rc != TTAMD_OK) return rc;
     }
     return TTAMD_OK;
@@ -522,11 +607,28 @@ int run_gemm_rs(const void* X, const uint8_t* codes, const void* scal, int mode,
   g.M = (int)M; g.Nout = (int)Nout; g.Kc = (int)Kc; g.R = R;
   g.lw_row_major = lw_row_major ? 1 : 0;
   g.lscale = lscale;
+  g.part = nullptr;
+  g.ksteps = 0;
+  const int splits = choose_splits(M, Nout, Kc);
+  if (splits > 1 && workspace != nullptr && workspace_bytes >= gemm_rs_workspace_bytes(M, Nout, Kc)) {
+    TT_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 15u) == 0, "nf4_gemm: workspace must be 16-byte aligned");
+    g.part = reinterpret_cast<float*>(workspace);
+    g.ksteps = (int)(((Kc >> 6) + splits - 1) / splits);
+    const int used = (int)(((Kc >> 6) + g.ksteps - 1) / g.ksteps);  // slices that hold at least one k-step
+    int rc = mode == 1 ? launch_rs<128, 1, true>(g, used, s)
+             : mode == 2 ? launch_rs<128, 2, true>(g, used, s)
+                         : launch_rs<128, 0, true>(g, used, s);
+    if (rc != TTAMD_OK) return rc;
+    const int64_t mn = M * Nout;
+    nf4_gemm_rs_reduce_kernel<<<dim3((unsigned)((mn / 8 + 255) / 256)), dim3(256), 0, s>>>(g.part, used, mn, (int)Nout, g.bias,
+                                                                                          g.cscale, g.C);
+    return check_launch("nf4_gemm_rs_reduce");
+  }
   const int64_t tiles256 = ((M + 255) / 256) * ((Nout + kBN - 1) / kBN);
   const bool big = tiles256 >= 256;
-  if (mode == 1) return big ? launch_rs<256, 1>(g, s) : launch_rs<128, 1>(g, s);
-  if (mode == 2) return big ? launch_rs<256, 2>(g, s) : launch_rs<128, 2>(g, s);
-  return big ? launch_rs<256, 0>(g, s) : launch_rs<128, 0>(g, s);
+  if (mode == 1) return big ? launch_rs<256, 1, false>(g, 1, s) : launch_rs<128, 1, false>(g, 1, s);
+  if (mode == 2) return big ? launch_rs<256, 2, false>(g, 1, s) : launch_rs<128, 2, false>(g, 1, s);
+  return big ? launch_rs<256, 0, false>(g, 1, s) : launch_rs<128, 0, false>(g, 1, s);
 }
 
 }  // namespace ttamd

@@ -187,6 +187,14 @@ def lora_hidden(x: torch.Tensor, lora_a: torch.Tensor) -> torch.Tensor:
     return h
 
 
+def _gemm_workspace(lib, M: int, n_out: int, k_contract: int, device):
+    """fp32 workspace with which the library slices the contraction of a launch of few output tiles (None: not needed)."""
+    nbytes = int(lib.ttamd_nf4_gemm_workspace_bytes(M, n_out, k_contract))
+    if nbytes == 0:
+        return None, 0
+    return torch.empty(nbytes // 4, dtype=torch.float32, device=device), nbytes
+
+
 def nf4_lora_linear_fwd(
     x: torch.Tensor, qdata: torch.Tensor, block_scalers: torch.Tensor, N: int, h: Optional[torch.Tensor] = None,
     lora_b: Optional[torch.Tensor] = None, scale: float = 0.0, bias: Optional[torch.Tensor] = None,
@@ -207,21 +215,17 @@ def nf4_lora_linear_fwd(
             raise TypeError("nf4_lora_linear_fwd: bias must be bfloat16")
     y = torch.empty(M, N, dtype=torch.bfloat16, device=x.device)
     lib = _lib.load()
+    ws, ws_bytes = _gemm_workspace(lib, M, N, K, x.device)
     with torch.cuda.device(x.device):
         events = _gemm_timer("fwd", M, N, K, rank) if _gemm_timer is not None else None
         if events:
             events[0].record()
-        if col_scale is None:
-            rc = lib.ttamd_nf4_lora_linear_fwd_bf16(
-                x.data_ptr(), qdata.data_ptr(), block_scalers.data_ptr(), _ptr(block_scalers_t), _ptr(h), _ptr(lora_b), rank,
-                float(scale), _ptr(bias), y.data_ptr(), M, N, K, _stream(x),
-            )
-        else:  # DoRA: every output column times magnitude / weight norm
+        if col_scale is not None:  # DoRA: every output column times magnitude / weight norm
             col_scale = _bf16_any(col_scale, "nf4_lora_linear_fwd: col_scale")
-            rc = lib.ttamd_nf4_dora_linear_fwd_bf16(
-                x.data_ptr(), qdata.data_ptr(), block_scalers.data_ptr(), _ptr(block_scalers_t), _ptr(h), _ptr(lora_b), rank,
-                float(scale), _ptr(bias), col_scale.data_ptr(), y.data_ptr(), M, N, K, _stream(x),
-            )
+        rc = lib.ttamd_nf4_lora_linear_fwd_ws_bf16(
+            x.data_ptr(), qdata.data_ptr(), block_scalers.data_ptr(), _ptr(block_scalers_t), _ptr(h), _ptr(lora_b), rank,
+            float(scale), _ptr(bias), _ptr(col_scale), y.data_ptr(), M, N, K, _ptr(ws), ws_bytes, _stream(x),
+        )
         if events:
             events[1].record()
     _lib.check(rc, "nf4_lora_linear_fwd")
@@ -256,13 +260,15 @@ def nf4_linear_bwd_dx(
         rank = gh.shape[1]
     gx = torch.empty(M, K, dtype=torch.bfloat16, device=gy.device)
     lib = _lib.load()
+    ws, ws_bytes = _gemm_workspace(lib, M, K, N, gy.device) if transposed else (None, 0)
     with torch.cuda.device(gy.device):
         events = _gemm_timer("bwd", M, N, K, rank) if _gemm_timer is not None else None
         if events:
             events[0].record()
-        rc = lib.ttamd_nf4_linear_bwd_dx_bf16(
+        rc = lib.ttamd_nf4_linear_bwd_dx_ws_bf16(
             gy.data_ptr(), qdata.data_ptr(), block_scalers.data_ptr(), _ptr(transposed[0]) if transposed else None,
-            _ptr(transposed[1]) if transposed else None, _ptr(gh), _ptr(lora_a), rank, gx.data_ptr(), M, N, K, _stream(gy),
+            _ptr(transposed[1]) if transposed else None, _ptr(gh), _ptr(lora_a), rank, gx.data_ptr(), M, N, K, _ptr(ws), ws_bytes,
+            _stream(gy),
         )
         if events:
             events[1].record()
