@@ -192,6 +192,16 @@ int main() {
     }
   check(close_enough(to_host(d_y, M * N), y_ref, 1e-2, 1e-2, "y"), "nf4_lora_linear_fwd: y = x.D(W)^T + bias + s.h.B^T within 1e-2");
 
+  // the same forward with the workspace that lets the library slice the contraction of this six-tile launch
+  const size_t g_ws_bytes = ttamd_nf4_gemm_workspace_bytes(M, N, K);
+  check(g_ws_bytes >= 2 * (size_t)M * N * sizeof(float), "nf4_gemm_workspace_bytes: a launch of few tiles asks for at least two slices");
+  char* d_gws = device_alloc<char>(g_ws_bytes);
+  uint16_t* d_y2 = device_alloc<uint16_t>(M * N);
+  TT_OK(ttamd_nf4_lora_linear_fwd_ws_bf16(d_x, d_codes, d_bs, nullptr, d_h, d_b, rank, scale, d_bias, nullptr, d_y2, M, N, K, d_gws,
+                                          g_ws_bytes, stream));
+  HIP_OK(hipStreamSynchronize(stream));
+  check(close_enough(to_host(d_y2, M * N), y_ref, 1e-2, 1e-2, "y (sliced)"), "nf4_lora_linear_fwd_ws: the sliced contraction gives the same y within 1e-2");
+
   // ---- 4. backward -------------------------------------------------------------------------------------------
   uint16_t* d_gy = to_device(gy);
   uint16_t *d_gh = device_alloc<uint16_t>(M * rank), *d_ga = device_alloc<uint16_t>(rank * K), *d_gb = device_alloc<uint16_t>(N * rank);
