@@ -236,6 +236,23 @@ def secondary_kernels(dev) -> dict:
     host = torch.empty(14336, 4096, dtype=torch.bfloat16, pin_memory=True)
     out["checkpoint offload: nf4_dequantize 14336x4096 written into pinned host memory (PCIe-bound, host bytes only)"] = round(
         n * 2 / timed(lambda: t.get_original_weight(out=host), iters=5) / 1e9, 1)
+    # forward for a handful of tokens (decode): the packed weight is streamed once, 0.5625 B per element.  The kernels
+    # take 7-15 us, less than a launch from Python costs, so 20 launches are captured in a HIP graph and the replay timed.
+    bs, bst = t.block_scalers(), t.backward_copy()[1]
+    for m_tok in (1, 16):
+        xs = torch.randn(m_tok, 4096, device=dev, generator=gen).to(torch.bfloat16)
+        ys = ops.nf4_lora_linear_fwd(xs, t.quantized_data, bs, 14336, block_scalers_t=bst)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for _ in range(20):
+                yg = ops.nf4_lora_linear_fwd(xs, t.quantized_data, bs, 14336, block_scalers_t=bst)
+        sec = timed(graph.replay, iters=10) / 20
+        torch.cuda.synchronize()
+        if not torch.equal(yg, ys):
+            raise RuntimeError("bench: the graph replay of the few-token forward differs from the eager result")
+        out[f"nf4_lora_linear_fwd M={m_tok} 14336x4096 (few-token kernel, packed-weight bytes)"] = round(n * 0.5625 / sec / 1e9, 1)
+        del graph
     return {"unit": "GB/s (algorithmic bytes / HIP-event time, HBM peak 8000)", **out}
 
 
