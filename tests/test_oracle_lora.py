@@ -137,3 +137,24 @@ def test_dora_module_dense_path_reproduces_the_known_answer():
     assert layer.adapter_params() == ["lora_a.weight", "lora_b.weight", "magnitude"]
     with pytest.raises(ValueError, match="quantize_base"):
         DoRALinear(8, 8, 2, 1.0, block_size=64)
+
+
+def test_dora_single_device_init_and_meta_device_error():
+    """tests/torchtune/modules/peft/test_dora.py:239-274 on the CPU: the magnitude becomes the row norms of the merged
+    weight, and a layer still on the meta device refuses to initialise it."""
+    from torch import nn
+
+    from torchtune_amd.modules.peft import DoRALinear
+
+    torch.manual_seed(3)
+    layer = DoRALinear(in_dim=64, out_dim=128, rank=4, alpha=1.0, use_bias=False)
+    layer.lora_a.weight = nn.Parameter(torch.randn_like(layer.lora_a.weight))
+    layer.lora_b.weight = nn.Parameter(torch.randn_like(layer.lora_b.weight))
+    expected = torch.linalg.norm(layer.weight + layer.scaling * layer.lora_b.weight @ layer.lora_a.weight, dim=1)
+    assert not torch.allclose(layer.magnitude, expected)
+    layer.initialize_dora_magnitude()
+    assert torch.allclose(layer.magnitude, expected)
+    with torch.device("meta"):
+        meta = DoRALinear(in_dim=512, out_dim=512, rank=4, alpha=1.0, use_bias=False, quantize_base=False)
+    with pytest.raises(RuntimeError, match="Cannot initialize DoRA magnitude"):
+        meta.initialize_dora_magnitude()
