@@ -384,3 +384,33 @@ def test_reference_known_answer_merged_lora_ckpt():
     with pytest.raises(NotImplementedError):
         get_merged_lora_ckpt({"m.experts.weight": torch.ones(2, 2), "m.experts.lora_a.weight": torch.ones(1, 2),
                               "m.experts.lora_b.weight": torch.ones(2, 1)}, rank=1, alpha=1.0)
+
+
+def test_disable_adapter_and_adapter_state_dict():
+    """tests/torchtune/modules/peft/test_utils.py:214-238,512-522: inside ``disable_adapter`` a LoRA model answers like
+    its base model and the flag is restored afterwards (also after an exception); ``get_adapter_state_dict`` keeps the
+    ``lora`` / ``magnitude`` entries only."""
+    from torch import nn
+
+    from torchtune_amd.modules.peft import DoRALinear, LoRALinear, disable_adapter, get_adapter_state_dict
+
+    torch.manual_seed(0)
+    base = nn.Sequential(nn.Linear(2, 6, bias=False), nn.Linear(6, 3))
+    lora = nn.Sequential(LoRALinear(2, 6, rank=4, alpha=1.0), nn.Linear(6, 3))
+    for p in list(base.parameters()) + list(lora.parameters()):
+        nn.init.constant_(p, 1.0)
+    x = torch.randn(2, 2)
+    assert not torch.allclose(base(x), lora(x))
+    with disable_adapter(lora):
+        assert lora[0].disabled is True
+        out = lora(x)
+    assert lora[0].disabled is False
+    torch.testing.assert_close(base(x), out)
+    with pytest.raises(RuntimeError, match="boom"):
+        with disable_adapter(lora):
+            raise RuntimeError("boom")
+    assert lora[0].disabled is False
+    model = nn.Sequential(LoRALinear(8, 8, rank=2, alpha=1.0), DoRALinear(8, 8, rank=2, alpha=1.0), nn.Linear(8, 8))
+    sd = get_adapter_state_dict(model.state_dict())
+    assert sorted(sd) == ["0.lora_a.weight", "0.lora_b.weight", "1.lora_a.weight", "1.lora_b.weight", "1.magnitude"]
+    assert all(v.device.type == "cpu" for v in sd.values())

@@ -1,7 +1,8 @@
 """Adapter layers of the quantized-linear path (LoRA, QAT + LoRA, DoRA over dense or NF4 base weights) and the small
 amount of adapter bookkeeping their callers need."""
 from ._adapter_base import LowRankAdapterLinear
-from ._utils import AdapterModule, get_adapter_params, get_merged_lora_ckpt, set_trainable_params
+from ._utils import (AdapterModule, disable_adapter, get_adapter_params, get_adapter_state_dict, get_merged_lora_ckpt,
+                     set_trainable_params)
 from .dora import DoRALinear
 from .lora import LoRALinear, QATLoRALinear, TrainableParams
 
@@ -15,4 +16,6 @@ __all__ = (
     "get_adapter_params",
     "set_trainable_params",
     "get_merged_lora_ckpt",
+    "get_adapter_state_dict",
+    "disable_adapter",
 )

@@ -1,9 +1,11 @@
 """The part of the adapter bookkeeping that callers of ``LoRALinear`` need
-(``torchtune/modules/peft/_utils.py:19-83,193-271``): the ``AdapterModule`` protocol, the helpers that pick out
-and freeze parameters by it, and the merge of the adapters into the base weights for a checkpoint."""
+(``torchtune/modules/peft/_utils.py:19-83,115-133,193-321``): the ``AdapterModule`` protocol, the helpers that pick
+out and freeze parameters by it, the adapter part of a state dict, the switch that runs a model without its adapters,
+and the merge of the adapters into the base weights for a checkpoint."""
 from __future__ import annotations
 
-from typing import Any, Dict, List, Protocol, Set
+import contextlib
+from typing import Any, Dict, Generator, List, Optional, Protocol, Set
 
 import torch
 from torch import nn
@@ -39,6 +41,32 @@ def set_trainable_params(model: nn.Module, adapter_params: Dict[str, nn.Paramete
     """Freeze everything except the given parameters."""
     for name, p in model.named_parameters():
         p.requires_grad_(name in adapter_params)
+
+
+def get_adapter_state_dict(state_dict: Dict[str, Any], device: Optional[str] = "cpu") -> Dict[str, Any]:
+    """The adapter entries of an unsharded model state dict (keys that contain ``lora`` or ``magnitude``), moved to
+    ``device`` (``torchtune/modules/peft/_utils.py:115-133``)."""
+    return {k: v.to(device) for k, v in state_dict.items() if "lora" in k or "magnitude" in k}
+
+
+def _adapter_switches(model: nn.Module):
+    for _, mod in model.named_modules():
+        if callable(getattr(mod, "adapter_params", None)) and hasattr(mod, "disabled"):
+            yield mod
+
+
+@contextlib.contextmanager
+def disable_adapter(model: nn.Module) -> Generator[None, None, None]:
+    """Run ``model`` as its base model: every module that declares adapter parameters and has a ``disabled`` flag
+    skips its adapter inside the ``with`` block and gets it back afterwards, also when the block raises
+    (``torchtune/modules/peft/_utils.py:274-321``; DPO uses it to get the reference model out of the policy)."""
+    for mod in _adapter_switches(model):
+        mod.disabled = True
+    try:
+        yield
+    finally:
+        for mod in _adapter_switches(model):
+            mod.disabled = False
 
 
 def _get_lora_modules(state_dict: Dict[str, Any]) -> Set[str]:
