@@ -561,6 +561,7 @@ int launch_rs(RsArgs& g, int splits, hipStream_t s) {
 int choose_splits(int64_t M, int64_t Nout, int64_t Kc) {
   const int64_t tiles = ((M + 127) / 128) * ((Nout + kBN - 1) / kBN);  // small launches use 128-row tiles
   if (tiles > 128) return 1;
+  if (tiles > 64 && Kc < 4096) return 1;  // two slices of a short contraction: the reduction costs what the slicing gains
   int64_t sp = 256 / tiles;
   const int64_t by_k = (Kc / 64) / 4;
   sp = sp < by_k ? sp : by_k;
