@@ -8,8 +8,8 @@
 //
 // The first two contract along the contiguous dimension of the activation: bf16 MFMA with the activation rows
 // as the A operand, fragments loaded straight from global memory (a lane's 8 contraction elements are 16
-// contiguous bytes).  The last two contract over rows: fp32 MFMA (one contraction index per lane, so both
-// operands are read row-major as they lie in memory).  Both split the contraction over many workgroups to
+// contiguous bytes).  The last two contract over rows: bf16 MFMA as well, with both operands transposed on the way
+// through LDS (ds_read_b64_tr_b16).  Both split the contraction over many workgroups to
 // put enough loads in flight and combine the fp32 partial sums in a second, fixed-order pass, so results
 // are deterministic.
 #include "common.h"
@@ -158,61 +158,107 @@ __global__ __launch_bounds__(256) void transpose_small_kernel(const uint16_t* __
 
 // ---------------------------------------------------------------------------------------------------
 // skinny_tn: part[split][r0 + r][c] = sum_{m in split} G[m][r0 + r] * X[m][c]   (G [M,R], X [M,Kc], r < 16)
-// The contraction runs over rows, so both operands are read in their natural row-major layout by the fp32 MFMA
-// v_mfma_f32_16x16x4_f32, whose operands hold ONE contraction index per lane: lane (g = l / 16, q = l % 16) supplies
-// G[m + g][r0 + q] as the row operand and X[m + g][c] as the column operand, four rows m..m+3 per instruction.
-// A lane loads 8 consecutive columns (16 bytes) of its row and feeds them to 8 MFMAs, so MFMA e of the wave covers the
-// columns {c0 + 8 q + e}; its 16x16 result D[r][.] is lane q's column c0 + 8 q + e, i.e. a lane ends up with 8
-// consecutive columns for each of its 4 result rows r = 4 g + v.
-// Workgroup = 4 waves on the same 128 columns, taking the split's 4-row steps in turn; partial sums are combined
-// through LDS in a fixed order, then across splits by sum_partials_tn_kernel.
+// The contraction runs over rows.  The fp32 MFMA v_mfma_f32_16x16x4_f32 takes one contraction index per lane and
+// could read both operands as they lie in memory, but it consumes only 64 elements of X per 32-cycle instruction,
+// which caps a kernel built on it near the HBM rate (measured: 3.7 - 4.8 TB/s).  v_mfma_f32_16x16x32_bf16
+// takes 512, but wants 8 consecutive contraction indices (rows m) of one column in a lane, while memory has 8
+// consecutive columns of one row.  The transposition is done by the LDS: a wave copies its 32 rows x 128 columns of X
+// (and the matching 32 x 16 piece of G) row-major into a private LDS region and reads them back with
+// ds_read_b64_tr_b16.  In a 16-lane group that instruction returns to lane i, as element t, the 16-bit element
+// (i % 4) of the 8 bytes that lane 4 t + i / 4 points at; with lane j pointing at row j / 4, columns 4 (j % 4) .. + 3
+// of a 4 x 16 piece, lane i receives column i of rows 0 .. 3: exactly an MFMA operand.
+// Workgroup = 4 waves on the same 128 columns; wave w takes the 32-row steps w, w + 4, ... of the split.  The partial
+// sums are combined through LDS in a fixed order, then across splits by sum_partials_tn_kernel.
 // ---------------------------------------------------------------------------------------------------
-constexpr int kTnCols = 128;   // columns per workgroup
-constexpr int kTnUnroll = 4;   // 4-row steps in flight per wave
+constexpr int kTnCols = 128;    // columns per workgroup
+constexpr int kTrPitchX = 288;  // bytes per LDS row of the X piece: 256 + 32, so that 4 consecutive rows fall on disjoint banks
+constexpr int kTrWaveLds = 32 * kTrPitchX + 32 * 32;  // X piece + G piece (32 rows x 16 bf16)
+
+__device__ __forceinline__ u32x2_t lds_read_tr16(uint32_t addr, int imm) {
+  u32x2_t v;
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(imm) : "memory");
+  return v;
+}
 
 __global__ __launch_bounds__(256) void skinny_tn_kernel(const uint16_t* __restrict__ G, const uint16_t* __restrict__ X,
-                                                        float* __restrict__ part, int M, int Kc, int R, int r0,
-                                                        int rows_per_split) {
-  __shared__ float red[3][32][64];
+                                                           float* __restrict__ part, int M, int Kc, int R, int r0,
+                                                           int rows_per_split) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  __shared__ __attribute__((aligned(16))) char stage[4 * kTrWaveLds];
+  static_assert(sizeof(stage) >= 3 * 32 * 64 * sizeof(float), "the reduction reuses the staging memory");
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int g = lane >> 4, q = lane & 15;
-  const int col = blockIdx.x * kTnCols + q * 8;
-  const bool col_ok = col < Kc;  // Kc % 8 == 0: a lane's 8 columns are in or out together
-  const bool r_ok = r0 + q < R;
+  const int g = lane >> 4, i = lane & 15;
+  const int c0 = blockIdx.x * kTnCols;
   const int split = blockIdx.y;
   const int m_begin = split * rows_per_split;
   int m_end = m_begin + rows_per_split;
   m_end = m_end < M ? m_end : M;
 
+  char* my = stage + wave * kTrWaveLds;
+  // copy-in roles: X piece, instruction u (0..7): row 4 u + lane / 16, 16-byte chunk lane % 16 (a row is 16 chunks)
+  const int xcol = c0 + 8 * i;
+  const bool xcol_ok = xcol < Kc;  // Kc % 8 == 0
+  const uint16_t* xsrc = X + (xcol_ok ? xcol : 0);
+  char* xdst = my + g * kTrPitchX + 16 * i;
+  // G piece: row lane / 2, half lane % 2 (8 of the 16 adapter columns r0 .. r0 + 15)
+  const int gcol = r0 + 8 * (lane & 1);
+  const bool gcol_ok = gcol < R;  // R % 8 == 0
+  const uint16_t* gsrc = G + (gcol_ok ? gcol : 0);
+  char* gdst = my + 32 * kTrPitchX + (lane >> 1) * 32 + 16 * (lane & 1);
+  // read-back roles: lane j = lane % 16 of group g points at row 8 g + j / 4 (+ 4 for the second half of the operand),
+  // columns 4 (j % 4) .. + 3 of a 16-column group
+  const uint32_t my_lds = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)my);
+  const uint32_t xrd = my_lds + (8 * g + (i >> 2)) * kTrPitchX + 8 * (i & 3);
+  const uint32_t grd = my_lds + 32 * kTrPitchX + (8 * g + (i >> 2)) * 32 + 8 * (i & 3);
+
   f32x4_t acc[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) acc[e] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-  const uint16_t* xp = X + (col_ok ? col : 0);
-  const uint16_t* gp = G + (r_ok ? r0 + q : 0);
-  for (int m = m_begin + 4 * wave; m < m_end; m += 16 * kTnUnroll) {
-    u32x4_t xv[kTnUnroll];
-    uint32_t gv[kTnUnroll];
+  u32x4_t xv[8], gv;
+  auto fetch = [&](int m) {  // rows m .. m + 31 into registers
 #pragma unroll
-    for (int u = 0; u < kTnUnroll; ++u) {
-      const int row = m + 16 * u + g;
-      const bool ok = row < m_end;
+    for (int u = 0; u < 8; ++u) {
+      const int row = m + 4 * u + g;
       xv[u] = u32x4_t{0, 0, 0, 0};
-      gv[u] = 0;
-      if (ok && col_ok) xv[u] = *reinterpret_cast<const u32x4_t*>(xp + (int64_t)row * Kc);
-      if (ok && r_ok) gv[u] = gp[(int64_t)row * R];
+      if (row < m_end && xcol_ok) xv[u] = *reinterpret_cast<const u32x4_t*>(xsrc + (int64_t)row * Kc);
     }
+    const int grow = m + (lane >> 1);
+    gv = u32x4_t{0, 0, 0, 0};
+    if (grow < m_end && gcol_ok) gv = *reinterpret_cast<const u32x4_t*>(gsrc + (int64_t)grow * R);
+  };
+  int m = m_begin + 32 * wave;
+  if (m < m_end) fetch(m);
+  for (; m < m_end; m += 128) {
+    // the previous step's reads of this region are complete: they were waited for before its MFMAs
 #pragma unroll
-    for (int u = 0; u < kTnUnroll; ++u) {
-      const float a = bits_f32(gv[u] << 16);
+    for (int u = 0; u < 8; ++u) *reinterpret_cast<u32x4_t*>(xdst + 4 * u * kTrPitchX) = xv[u];
+    *reinterpret_cast<u32x4_t*>(gdst) = gv;
+    if (m + 128 < m_end) fetch(m + 128);  // in flight while this step is multiplied
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the copy-in has landed (LDS operations of a wave complete in order)
+    u32x2_t ga = lds_read_tr16(grd, 0), gb = lds_read_tr16(grd, 4 * 32);
+    u32x2_t xa[8], xb[8];
 #pragma unroll
-      for (int d = 0; d < 4; ++d) {
-        acc[2 * d] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, bits_f32(xv[u][d] << 16), acc[2 * d], 0, 0, 0);
-        acc[2 * d + 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, bits_f32(xv[u][d] & 0xffff0000u), acc[2 * d + 1], 0, 0, 0);
-      }
+    for (int e = 0; e < 8; ++e) {
+      xa[e] = lds_read_tr16(xrd, 32 * e);
+      xb[e] = lds_read_tr16(xrd, 32 * e + 4 * kTrPitchX);
+    }
+    // The 18 reads return in order.  Each wait names the registers it releases, so that no use can be scheduled
+    // ahead of it: column group e may go once at most 14 - 2 e younger reads are outstanding.
+    asm volatile("s_waitcnt lgkmcnt(14)" : "+v"(ga), "+v"(gb), "+v"(xa[0]), "+v"(xb[0]));
+    const u32x4_t gop = {ga.x, ga.y, gb.x, gb.y};
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      if (e > 0) asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(xa[e]), "+v"(xb[e]) : "n"(14 - 2 * e));
+      const u32x4_t xop = {xa[e].x, xa[e].y, xb[e].x, xb[e].y};
+      acc[e] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, gop), __builtin_bit_cast(bf16x8_t, xop),
+                                                      acc[e], 0, 0, 0);
     }
   }
+  __syncthreads();  // the staging regions are free: the partial sums meet in them
+  float (*red)[32][64] = reinterpret_cast<float (*)[32][64]>(stage);
+  // acc[e][v] = sum over this wave's rows of G[.][r0 + 4 g + v] * X[.][c0 + 16 e + i]
   if (wave > 0) {
 #pragma unroll
     for (int e = 0; e < 8; ++e)
@@ -220,20 +266,21 @@ __global__ __launch_bounds__(256) void skinny_tn_kernel(const uint16_t* __restri
       for (int v = 0; v < 4; ++v) red[wave - 1][v * 8 + e][lane] = acc[e][v];
   }
   __syncthreads();
-  if (wave == 0 && col_ok) {
+  if (wave == 0) {
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
       const int r = r0 + 4 * g + v;
       if (r >= R) continue;
-      float o[8];
 #pragma unroll
-      for (int e = 0; e < 8; ++e)
-        o[e] = ((acc[e][v] + red[0][v * 8 + e][lane]) + red[1][v * 8 + e][lane]) + red[2][v * 8 + e][lane];
-      float* dst = part + ((int64_t)split * R + r) * Kc + col;
-      *reinterpret_cast<f32x4_t*>(dst) = f32x4_t{o[0], o[1], o[2], o[3]};
-      *reinterpret_cast<f32x4_t*>(dst + 4) = f32x4_t{o[4], o[5], o[6], o[7]};
+      for (int e = 0; e < 8; ++e) {
+        const int col = c0 + 16 * e + i;
+        if (col >= Kc) continue;
+        part[((int64_t)split * R + r) * Kc + col] =
+            ((acc[e][v] + red[0][v * 8 + e][lane]) + red[1][v * 8 + e][lane]) + red[2][v * 8 + e][lane];
+      }
     }
   }
+#endif
 }
 
 // out[r*stride_r + k*stride_k] = bf16(scale * sum_s part[s][r][k])
@@ -250,7 +297,7 @@ __global__ __launch_bounds__(256) void sum_partials_tn_kernel(const float* __res
   out[r * stride_r + k * stride_k] = f32_to_bf16_bits(s * scale);
 }
 
-constexpr int kTargetWaves = 4096;    // row contractions (skinny_tn)
+constexpr int kTargetWaves = 2048;    // row contractions (skinny_tn)
 constexpr int kTargetWavesNt = 1024;  // column contractions (skinny_nt): few, long waves; one split needs no second pass
 
 struct NtPlan {
@@ -278,9 +325,9 @@ TnPlan plan_tn(int64_t M, int64_t Kc) {
   p.col_groups = (int)((Kc + kTnCols - 1) / kTnCols);
   int s = kTargetWaves / 4 / p.col_groups;  // workgroups of 4 waves
   s = s < 1 ? 1 : s;
-  const int max_s = (int)((M + 63) / 64);  // at least 64 rows per split: four 4-row steps per wave
+  const int max_s = (int)((M + 127) / 128);  // at least 128 rows per split: one 32-row step per wave
   s = s > max_s ? max_s : s;
-  p.rows_per_split = (int)(((M + s - 1) / s + 15) / 16 * 16);  // whole rounds of the four waves
+  p.rows_per_split = (int)(((M + s - 1) / s + 127) / 128 * 128);  // whole rounds of the four waves
   p.splits = (int)((M + p.rows_per_split - 1) / p.rows_per_split);
   return p;
 }
