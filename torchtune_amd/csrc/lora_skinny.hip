@@ -168,7 +168,7 @@ __global__ __launch_bounds__(256) void transpose_small_kernel(const uint16_t* __
 // (i % 4) of the 8 bytes that lane 4 t + i / 4 points at; with lane j pointing at row j / 4, columns 4 (j % 4) .. + 3
 // of a 4 x 16 piece, lane i receives column i of rows 0 .. 3: exactly an MFMA operand.
 // Workgroup = 4 waves on the same 128 columns; wave w takes the 32-row steps w, w + 4, ... of the split.  The partial
-// sums are combined through LDS in a fixed order, then across splits by sum_partials_tn_kernel.
+// sums are combined through LDS in a fixed order, then across splits by sum_partials_tn_pair_kernel.
 // ---------------------------------------------------------------------------------------------------
 constexpr int kTnCols = 128;    // columns per workgroup
 constexpr int kTrPitchX = 288;  // bytes per LDS row of the X piece: 256 + 32, so that 4 consecutive rows fall on disjoint banks
@@ -180,16 +180,34 @@ __device__ __forceinline__ u32x2_t lds_read_tr16(uint32_t addr, int imm) {
   return v;
 }
 
-__global__ __launch_bounds__(256) void skinny_tn_kernel(const uint16_t* __restrict__ G, const uint16_t* __restrict__ X,
-                                                           float* __restrict__ part, int M, int Kc, int R, int r0,
-                                                           int rows_per_split) {
+// One launch serves the two row contractions of a LoRA backward (gA over x, gB over gy): they share M, R and the row
+// splits, and differ in the operands and the width.  Workgroups [0, col_groups0) belong to problem 0, the rest to 1.
+struct TnProblem {
+  const uint16_t* G;  // [M, R]
+  const uint16_t* X;  // [M, Kc]
+  float* part;        // [splits, R, Kc]
+  int Kc;
+};
+struct TnPair {
+  TnProblem p[2];
+  int col_groups0;
+  int M, R, r0, rows_per_split;
+};
+
+__global__ __launch_bounds__(256) void skinny_tn_kernel(const TnPair a) {
 #if defined(__HIP_DEVICE_COMPILE__)
+  const int which = (int)blockIdx.x >= a.col_groups0 ? 1 : 0;  // uniform over the workgroup
+  const uint16_t* __restrict__ G = a.p[which].G;
+  const uint16_t* __restrict__ X = a.p[which].X;
+  float* __restrict__ part = a.p[which].part;
+  const int Kc = a.p[which].Kc, M = a.M, R = a.R, r0 = a.r0, rows_per_split = a.rows_per_split;
+  const int col_group = (int)blockIdx.x - (which ? a.col_groups0 : 0);
   __shared__ __attribute__((aligned(16))) char stage[4 * kTrWaveLds];
   static_assert(sizeof(stage) >= 3 * 32 * 64 * sizeof(float), "the reduction reuses the staging memory");
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int g = lane >> 4, i = lane & 15;
-  const int c0 = blockIdx.x * kTnCols;
+  const int c0 = col_group * kTnCols;
   const int split = blockIdx.y;
   const int m_begin = split * rows_per_split;
   int m_end = m_begin + rows_per_split;
@@ -284,17 +302,31 @@ __global__ __launch_bounds__(256) void skinny_tn_kernel(const uint16_t* __restri
 }
 
 // out[r*stride_r + k*stride_k] = bf16(scale * sum_s part[s][r][k])
-__global__ __launch_bounds__(256) void sum_partials_tn_kernel(const float* __restrict__ part, int R, int Kc, int splits,
-                                                              float scale, int64_t stride_r, int64_t stride_k,
-                                                              uint16_t* __restrict__ out) {
-  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  const int64_t n = (int64_t)R * Kc;
+struct TnSum {
+  const float* part;
+  uint16_t* out;
+  int Kc;
+  float scale;
+  int64_t stride_r, stride_k;
+};
+struct TnSumPair {
+  TnSum p[2];
+  int64_t n0;  // elements of problem 0: R * Kc
+  int R, splits;
+};
+// The reductions of the two row contractions in one launch: thread i < n0 finishes problem 0, the rest problem 1.
+__global__ __launch_bounds__(256) void sum_partials_tn_pair_kernel(const TnSumPair a) {
+  int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int which = i >= a.n0 ? 1 : 0;
+  if (which) i -= a.n0;
+  const TnSum& P = a.p[which];
+  const int64_t n = (int64_t)a.R * P.Kc;
   if (i >= n) return;
   float s = 0.f;
 #pragma unroll 8
-  for (int p = 0; p < splits; ++p) s += part[(int64_t)p * n + i];
-  const int64_t r = i / Kc, k = i % Kc;
-  out[r * stride_r + k * stride_k] = f32_to_bf16_bits(s * scale);
+  for (int q = 0; q < a.splits; ++q) s += P.part[(int64_t)q * n + i];
+  const int64_t r = i / P.Kc, k = i % P.Kc;
+  P.out[r * P.stride_r + k * P.stride_k] = f32_to_bf16_bits(s * P.scale);
 }
 
 constexpr int kTargetWaves = 2048;    // row contractions (skinny_tn)
@@ -318,12 +350,14 @@ NtPlan plan_nt(int64_t M, int64_t Kc) {
 size_t nt_ws_bytes(int64_t M, int64_t Kc, int R) { return (size_t)plan_nt(M, Kc).splits * M * R * sizeof(float); }
 
 struct TnPlan {
-  int col_groups, splits, rows_per_split;
+  int col_groups0, col_groups1, splits, rows_per_split;
 };
-TnPlan plan_tn(int64_t M, int64_t Kc) {
+// Both products of a backward in one grid: widths K (gA) and N (gB), the same row splits.
+TnPlan plan_tn_pair(int64_t M, int64_t K, int64_t N) {
   TnPlan p;
-  p.col_groups = (int)((Kc + kTnCols - 1) / kTnCols);
-  int s = kTargetWaves / 4 / p.col_groups;  // workgroups of 4 waves
+  p.col_groups0 = (int)((K + kTnCols - 1) / kTnCols);
+  p.col_groups1 = (int)((N + kTnCols - 1) / kTnCols);
+  int s = kTargetWaves / 4 / (p.col_groups0 + p.col_groups1);  // workgroups of 4 waves
   s = s < 1 ? 1 : s;
   const int max_s = (int)((M + 127) / 128);  // at least 128 rows per split: one 32-row step per wave
   s = s > max_s ? max_s : s;
@@ -331,7 +365,9 @@ TnPlan plan_tn(int64_t M, int64_t Kc) {
   p.splits = (int)((M + p.rows_per_split - 1) / p.rows_per_split);
   return p;
 }
-size_t tn_ws_bytes(int64_t M, int64_t Kc, int R) { return (size_t)plan_tn(M, Kc).splits * R * Kc * sizeof(float); }
+size_t tn_pair_ws_bytes(int64_t M, int64_t K, int64_t N, int R) {
+  return (size_t)plan_tn_pair(M, K, N).splits * R * (size_t)(K + N) * sizeof(float);
+}
 
 size_t align256(size_t v) { return (v + 255) & ~size_t(255); }
 
@@ -353,15 +389,30 @@ int run_nt(const uint16_t* X, const uint16_t* Bm, int64_t M, int64_t Kc, int R, 
   return check_launch("skinny_nt");
 }
 
-int run_tn(const uint16_t* G, const uint16_t* X, int64_t M, int64_t Kc, int R, float scale, int64_t stride_r,
-           int64_t stride_k, uint16_t* out, float* ws, hipStream_t s) {
-  const TnPlan p = plan_tn(M, Kc);
-  const dim3 grid((unsigned)p.col_groups, (unsigned)p.splits), block(256);
-  for (int r0 = 0; r0 < R; r0 += 16)
-    skinny_tn_kernel<<<grid, block, 0, s>>>(G, X, ws, (int)M, (int)Kc, R, r0, p.rows_per_split);
-  const int64_t n = (int64_t)R * Kc;
-  sum_partials_tn_kernel<<<dim3((unsigned)((n + 255) / 256)), block, 0, s>>>(ws, R, (int)Kc, p.splits, scale, stride_r,
-                                                                             stride_k, out);
+// gA[r][k] = sum_m gh[m][r] x[m][k]  and  gB[n][r] = scale * sum_m h[m][r] gy[m][n]
+int run_tn_pair(const uint16_t* gh, const uint16_t* x, const uint16_t* h, const uint16_t* gy, int64_t M, int64_t K, int64_t N,
+                int R, float scale, uint16_t* ga, uint16_t* gb, float* ws, hipStream_t s) {
+  const TnPlan p = plan_tn_pair(M, K, N);
+  TnPair a;
+  a.p[0] = TnProblem{gh, x, ws, (int)K};
+  a.p[1] = TnProblem{h, gy, ws + (size_t)p.splits * R * K, (int)N};
+  a.col_groups0 = p.col_groups0;
+  a.M = (int)M;
+  a.R = R;
+  a.rows_per_split = p.rows_per_split;
+  const dim3 grid((unsigned)(p.col_groups0 + p.col_groups1), (unsigned)p.splits), block(256);
+  for (int r0 = 0; r0 < R; r0 += 16) {
+    a.r0 = r0;
+    skinny_tn_kernel<<<grid, block, 0, s>>>(a);
+  }
+  TnSumPair f;
+  f.p[0] = TnSum{a.p[0].part, ga, (int)K, 1.0f, K, 1};
+  f.p[1] = TnSum{a.p[1].part, gb, (int)N, scale, 1, R};
+  f.n0 = (int64_t)R * K;
+  f.R = R;
+  f.splits = p.splits;
+  const int64_t n = (int64_t)R * (K + N);
+  sum_partials_tn_pair_kernel<<<dim3((unsigned)((n + 255) / 256)), block, 0, s>>>(f);
   return check_launch("skinny_tn");
 }
 
@@ -397,9 +448,8 @@ extern "C" int ttamd_lora_hidden_bf16(const void* x, const void* lora_a, void* h
 
 extern "C" size_t ttamd_lora_bwd_workspace_bytes(int64_t M, int64_t N, int64_t K, int rank) {
   if (M <= 0 || N <= 0 || K <= 0 || rank <= 0 || K % 64 || N % 64) return 0;
-  size_t a = nt_ws_bytes(M, N, rank), b = tn_ws_bytes(M, K, rank), c = tn_ws_bytes(M, N, rank);
-  size_t big = a > b ? a : b;
-  big = big > c ? big : c;
+  const size_t a = nt_ws_bytes(M, N, rank), b = tn_pair_ws_bytes(M, K, N, rank);
+  const size_t big = a > b ? a : b;
   return align256((size_t)N * rank * sizeof(uint16_t)) + align256(big);
 }
 
@@ -422,10 +472,7 @@ extern "C" int ttamd_lora_bwd_bf16(const void* gy, const void* x, const void* h,
                                                                                   rank, bt);
   // gh = scale * gy . B
   if (int rc = run_nt(GY, bt, M, N, rank, scale, reinterpret_cast<uint16_t*>(gh), part, s)) return rc;
-  // gA[r][k] = sum_m gh[m][r] x[m][k]
-  if (int rc = run_tn(reinterpret_cast<const uint16_t*>(gh), reinterpret_cast<const uint16_t*>(x), M, K, rank, 1.0f, K, 1,
-                      reinterpret_cast<uint16_t*>(ga), part, s))
-    return rc;
-  // gB[n][r] = scale * sum_m h[m][r] gy[m][n]
-  return run_tn(reinterpret_cast<const uint16_t*>(h), GY, M, N, rank, scale, 1, rank, reinterpret_cast<uint16_t*>(gb), part, s);
+  return run_tn_pair(reinterpret_cast<const uint16_t*>(gh), reinterpret_cast<const uint16_t*>(x),
+                     reinterpret_cast<const uint16_t*>(h), GY, M, K, N, rank, scale, reinterpret_cast<uint16_t*>(ga),
+                     reinterpret_cast<uint16_t*>(gb), part, s);
 }
