@@ -33,19 +33,33 @@ typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 // + 16) - the four lane groups cover one whole 128-byte line per row - and uses its first 8 elements for one MFMA and
 // the last 8 for the next (the contraction index may be permuted freely as long as both operands agree).
 // RT = number of 16-wide tiles of R.
+// BT: Bm is given as it lies in memory for the other contraction, [Kc, R] row-major (lora_b [N, R] for gh = gy . B).
+// The operand then needs 8 consecutive rows of one column in a lane; each wave copies the 64 x R piece of its chunk
+// (contiguous in memory) into a private LDS region and reads it back transposed with ds_read_b64_tr_b16 (lane j of a
+// 16-lane group points at row j / 4, columns 4 (j % 4) .. + 3 of a 4 x 16 piece; lane i receives column i of its 4 rows).
 // ---------------------------------------------------------------------------------------------------
-template <int RT>
+__device__ __forceinline__ u32x2_t lds_read_tr16(uint32_t addr, int imm) {
+  u32x2_t v;
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(imm) : "memory");
+  return v;
+}
+
+template <int RT, bool BT>
 __global__ __launch_bounds__(256) void skinny_nt_kernel(const uint16_t* __restrict__ X, const uint16_t* __restrict__ Bm,
                                                         float* __restrict__ part, int M, int Kc, int R,
                                                         int chunks_per_split, uint16_t* __restrict__ direct_out,
                                                         float scale) {
   // direct_out != null (only with a single split): write bf16(scale * sum) straight to the [M, R] output
   __shared__ float red[3][2 * RT * 4][64];
+  constexpr int kPitchB = 32 * RT;  // bytes per LDS row of the transposed-operand piece: 16 RT columns
+  __shared__ __attribute__((aligned(16))) char bstage[BT ? 4 * 64 * kPitchB : 16];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int g = lane >> 4, i = lane & 15;
   const int m0 = blockIdx.x * 32;
   const int split = blockIdx.y;
+  char* myb = bstage + (BT ? wave * 64 * kPitchB : 0);
+  const uint32_t brd = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)myb) + (16 * g + (i >> 2)) * kPitchB + 8 * (i & 3);
   const uint16_t* xrow[2];
 #pragma unroll
   for (int t = 0; t < 2; ++t) {
@@ -76,24 +90,12 @@ __global__ __launch_bounds__(256) void skinny_nt_kernel(const uint16_t* __restri
   // tile therefore walks its chunks in a rotated order.  The order is a fixed function of the tile: deterministic.
   const int nc = c1 - c0;
   const int rot = nc > 0 ? (int)((blockIdx.x * 4u) % (unsigned)nc) : 0;
-#pragma unroll 2
-  for (int j = wave; j < nc; j += 4) {
+  auto chunk_start = [&](int j) {
     int c = j + rot;
     c = c0 + (c >= nc ? c - nc : c);
-    const int k0 = c * 64;
-    u32x4_t xa[2][2], wb[RT][2];
-#pragma unroll
-    for (int t = 0; t < 2; ++t)
-#pragma unroll
-      for (int hh = 0; hh < 2; ++hh)
-        xa[t][hh] = *reinterpret_cast<const u32x4_t*>(xrow[t] + k0 + 8 * hh);
-#pragma unroll
-    for (int u = 0; u < RT; ++u)
-#pragma unroll
-      for (int hh = 0; hh < 2; ++hh) {
-        wb[u][hh] = u32x4_t{0, 0, 0, 0};
-        if (bvalid[u]) wb[u][hh] = *reinterpret_cast<const u32x4_t*>(brow[u] + k0 + 8 * hh);
-      }
+    return c * 64;
+  };
+  auto multiply = [&](const u32x4_t (&xa)[2][2], const u32x4_t (&wb)[RT][2]) {
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
@@ -102,6 +104,84 @@ __global__ __launch_bounds__(256) void skinny_nt_kernel(const uint16_t* __restri
         for (int hh = 0; hh < 2; ++hh)
           acc[t][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, xa[t][hh]),
                                                              __builtin_bit_cast(bf16x8_t, wb[u][hh]), acc[t][u], 0, 0, 0);
+  };
+  if constexpr (BT) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    // rows k0 .. k0 + 63 of Bm are 64 R contiguous elements: 8 R pieces of 16 bytes, R / 8 pieces to a row.  The piece
+    // of a chunk is requested one chunk ahead, so that waiting for it never waits for the younger loads of X.
+    const int ppr = R >> 3;
+    u32x4_t piece[2 * RT];
+    auto load_piece = [&](int k0) {
+#pragma unroll
+      for (int q = 0; q < 2 * RT; ++q) {
+        const int pc = lane + 64 * q;
+        if (pc < 8 * R) piece[q] = *reinterpret_cast<const u32x4_t*>(Bm + (int64_t)k0 * R + 8 * pc);
+      }
+    };
+    u32x4_t xa[2][2], xn[2][2];
+    auto load_x = [&](u32x4_t (&dst)[2][2], int k0) {
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int hh = 0; hh < 2; ++hh) dst[t][hh] = *reinterpret_cast<const u32x4_t*>(xrow[t] + k0 + 8 * hh);
+    };
+    if (wave < nc) {
+      load_piece(chunk_start(wave));
+      load_x(xa, chunk_start(wave));
+    }
+    for (int j = wave; j < nc; j += 4) {
+#pragma unroll
+      for (int q = 0; q < 2 * RT; ++q) {
+        const int pc = lane + 64 * q;
+        if (pc < 8 * R) *reinterpret_cast<u32x4_t*>(myb + (pc / ppr) * kPitchB + 16 * (pc % ppr)) = piece[q];
+      }
+      if (j + 4 < nc) {  // the next chunk's loads are in flight while this one is multiplied
+        load_piece(chunk_start(j + 4));
+        load_x(xn, chunk_start(j + 4));
+      }
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the piece has landed (LDS operations of a wave complete in order)
+      u32x4_t wb[RT][2];
+      u32x2_t lo[RT][2], hi[RT][2];
+#pragma unroll
+      for (int u = 0; u < RT; ++u)
+#pragma unroll
+        for (int hh = 0; hh < 2; ++hh) {
+          lo[u][hh] = lds_read_tr16(brd, 32 * u + (8 * hh) * kPitchB);
+          hi[u][hh] = lds_read_tr16(brd, 32 * u + (8 * hh + 4) * kPitchB);
+        }
+#pragma unroll
+      for (int u = 0; u < RT; ++u)
+#pragma unroll
+        for (int hh = 0; hh < 2; ++hh) {
+          // waits that name the registers they release: no use can be scheduled ahead of them
+          asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(lo[u][hh]), "+v"(hi[u][hh]));
+          wb[u][hh] = u32x4_t{lo[u][hh].x, lo[u][hh].y, hi[u][hh].x, hi[u][hh].y};
+        }
+      multiply(xa, wb);
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int hh = 0; hh < 2; ++hh) xa[t][hh] = xn[t][hh];
+    }
+#endif
+  } else {
+#pragma unroll 2
+    for (int j = wave; j < nc; j += 4) {
+      const int k0 = chunk_start(j);
+      u32x4_t xa[2][2], wb[RT][2];
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int hh = 0; hh < 2; ++hh) xa[t][hh] = *reinterpret_cast<const u32x4_t*>(xrow[t] + k0 + 8 * hh);
+#pragma unroll
+      for (int u = 0; u < RT; ++u)
+#pragma unroll
+        for (int hh = 0; hh < 2; ++hh) {
+          wb[u][hh] = u32x4_t{0, 0, 0, 0};
+          if (bvalid[u]) wb[u][hh] = *reinterpret_cast<const u32x4_t*>(brow[u] + k0 + 8 * hh);
+        }
+      multiply(xa, wb);
+    }
   }
   // acc[t][u][v] = C[m0 + 16 t + 4 g + v][16 u + i]
   if (wave > 0) {
@@ -146,16 +226,6 @@ __global__ __launch_bounds__(256) void sum_partials_kernel(const float* __restri
   out[i] = f32_to_bf16_bits(s * scale);
 }
 
-// out[r][n] = in[n][r]
-__global__ __launch_bounds__(256) void transpose_small_kernel(const uint16_t* __restrict__ in, int64_t rows, int cols,
-                                                              uint16_t* __restrict__ out) {
-  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (i >= rows * cols) return;
-  const int64_t r = i / cols;
-  const int c = (int)(i % cols);
-  out[(int64_t)c * rows + r] = in[i];
-}
-
 // ---------------------------------------------------------------------------------------------------
 // skinny_tn: part[split][r0 + r][c] = sum_{m in split} G[m][r0 + r] * X[m][c]   (G [M,R], X [M,Kc], r < 16)
 // The contraction runs over rows.  The fp32 MFMA v_mfma_f32_16x16x4_f32 takes one contraction index per lane and
@@ -173,12 +243,6 @@ __global__ __launch_bounds__(256) void transpose_small_kernel(const uint16_t* __
 constexpr int kTnCols = 128;    // columns per workgroup
 constexpr int kTrPitchX = 288;  // bytes per LDS row of the X piece: 256 + 32, so that 4 consecutive rows fall on disjoint banks
 constexpr int kTrWaveLds = 32 * kTrPitchX + 32 * 32;  // X piece + G piece (32 rows x 16 bf16)
-
-__device__ __forceinline__ u32x2_t lds_read_tr16(uint32_t addr, int imm) {
-  u32x2_t v;
-  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(imm) : "memory");
-  return v;
-}
 
 // One launch serves the two row contractions of a LoRA backward (gA over x, gB over gy): they share M, R and the row
 // splits, and differ in the operands and the width.  Workgroups [0, col_groups0) belong to problem 0, the rest to 1.
@@ -371,17 +435,28 @@ size_t tn_pair_ws_bytes(int64_t M, int64_t K, int64_t N, int R) {
 
 size_t align256(size_t v) { return (v + 255) & ~size_t(255); }
 
-int run_nt(const uint16_t* X, const uint16_t* Bm, int64_t M, int64_t Kc, int R, float scale, uint16_t* out, float* ws,
-           hipStream_t s) {
+// b_is_kr: Bm is [Kc, R] row-major (transposed inside the kernel) instead of [R, Kc]
+template <bool BT>
+void launch_nt(const dim3& grid, const uint16_t* X, const uint16_t* Bm, float* ws, int M, int Kc, int R, int chunks_per_split,
+               uint16_t* direct, float scale, hipStream_t s) {
+  const dim3 block(256);
+  if (R <= 16)
+    skinny_nt_kernel<1, BT><<<grid, block, 0, s>>>(X, Bm, ws, M, Kc, R, chunks_per_split, direct, scale);
+  else if (R <= 32)
+    skinny_nt_kernel<2, BT><<<grid, block, 0, s>>>(X, Bm, ws, M, Kc, R, chunks_per_split, direct, scale);
+  else
+    skinny_nt_kernel<4, BT><<<grid, block, 0, s>>>(X, Bm, ws, M, Kc, R, chunks_per_split, direct, scale);
+}
+
+int run_nt(const uint16_t* X, const uint16_t* Bm, bool b_is_kr, int64_t M, int64_t Kc, int R, float scale, uint16_t* out,
+           float* ws, hipStream_t s) {
   const NtPlan p = plan_nt(M, Kc);
   const dim3 grid((unsigned)p.m_tiles, (unsigned)p.splits), block(256);
   uint16_t* direct = p.splits == 1 ? out : nullptr;
-  if (R <= 16)
-    skinny_nt_kernel<1><<<grid, block, 0, s>>>(X, Bm, ws, (int)M, (int)Kc, R, p.chunks_per_split, direct, scale);
-  else if (R <= 32)
-    skinny_nt_kernel<2><<<grid, block, 0, s>>>(X, Bm, ws, (int)M, (int)Kc, R, p.chunks_per_split, direct, scale);
+  if (b_is_kr)
+    launch_nt<true>(grid, X, Bm, ws, (int)M, (int)Kc, R, p.chunks_per_split, direct, scale, s);
   else
-    skinny_nt_kernel<4><<<grid, block, 0, s>>>(X, Bm, ws, (int)M, (int)Kc, R, p.chunks_per_split, direct, scale);
+    launch_nt<false>(grid, X, Bm, ws, (int)M, (int)Kc, R, p.chunks_per_split, direct, scale, s);
   if (!direct) {
     const int64_t n = M * R;
     sum_partials_kernel<<<dim3((unsigned)((n + 255) / 256)), block, 0, s>>>(ws, n, p.splits, scale, out);
@@ -442,15 +517,14 @@ extern "C" int ttamd_lora_hidden_bf16(const void* x, const void* lora_a, void* h
   if (workspace_bytes < ttamd_lora_fwd_workspace_bytes(M, K, rank))
     return fail(TTAMD_EWORKSPACE, "lora_hidden: workspace has %zu bytes, needs %zu", workspace_bytes,
                 ttamd_lora_fwd_workspace_bytes(M, K, rank));
-  return run_nt(reinterpret_cast<const uint16_t*>(x), reinterpret_cast<const uint16_t*>(lora_a), M, K, rank, 1.0f,
+  return run_nt(reinterpret_cast<const uint16_t*>(x), reinterpret_cast<const uint16_t*>(lora_a), false, M, K, rank, 1.0f,
                 reinterpret_cast<uint16_t*>(h), reinterpret_cast<float*>(workspace), reinterpret_cast<hipStream_t>(stream));
 }
 
 extern "C" size_t ttamd_lora_bwd_workspace_bytes(int64_t M, int64_t N, int64_t K, int rank) {
   if (M <= 0 || N <= 0 || K <= 0 || rank <= 0 || K % 64 || N % 64) return 0;
   const size_t a = nt_ws_bytes(M, N, rank), b = tn_pair_ws_bytes(M, K, N, rank);
-  const size_t big = a > b ? a : b;
-  return align256((size_t)N * rank * sizeof(uint16_t)) + align256(big);
+  return align256(a > b ? a : b);
 }
 
 extern "C" int ttamd_lora_bwd_bf16(const void* gy, const void* x, const void* h, const void* lora_b, float scale, void* gh,
@@ -464,14 +538,12 @@ extern "C" int ttamd_lora_bwd_bf16(const void* gy, const void* x, const void* h,
     return fail(TTAMD_EWORKSPACE, "lora_bwd: workspace has %zu bytes, needs %zu", workspace_bytes,
                 ttamd_lora_bwd_workspace_bytes(M, N, K, rank));
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  uint16_t* bt = reinterpret_cast<uint16_t*>(workspace);  // lora_b^T [R, N]
-  float* part = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + align256((size_t)N * rank * sizeof(uint16_t)));
+  float* part = reinterpret_cast<float*>(workspace);
   const uint16_t* GY = reinterpret_cast<const uint16_t*>(gy);
-  const int64_t nb = N * rank;
-  transpose_small_kernel<<<dim3((unsigned)((nb + 255) / 256)), dim3(256), 0, s>>>(reinterpret_cast<const uint16_t*>(lora_b), N,
-                                                                                  rank, bt);
-  // gh = scale * gy . B
-  if (int rc = run_nt(GY, bt, M, N, rank, scale, reinterpret_cast<uint16_t*>(gh), part, s)) return rc;
+  // gh = scale * gy . B, lora_b [N, R] as it lies (the kernel transposes its pieces)
+  if (int rc = run_nt(GY, reinterpret_cast<const uint16_t*>(lora_b), true, M, N, rank, scale, reinterpret_cast<uint16_t*>(gh),
+                      part, s))
+    return rc;
   return run_tn_pair(reinterpret_cast<const uint16_t*>(gh), reinterpret_cast<const uint16_t*>(x),
                      reinterpret_cast<const uint16_t*>(h), GY, M, K, N, rank, scale, reinterpret_cast<uint16_t*>(ga),
                      reinterpret_cast<uint16_t*>(gb), part, s);
