@@ -414,3 +414,20 @@ def test_disable_adapter_and_adapter_state_dict():
     sd = get_adapter_state_dict(model.state_dict())
     assert sorted(sd) == ["0.lora_a.weight", "0.lora_b.weight", "1.lora_a.weight", "1.lora_b.weight", "1.magnitude"]
     assert all(v.device.type == "cpu" for v in sd.values())
+
+
+def test_gemm_workspace_query_is_a_host_function():
+    """``ttamd_nf4_gemm_workspace_bytes`` needs no GPU: it is 0 where the contraction is not sliced (the few-token kernel,
+    M <= 64; launches with more than 128 tiles of 128 x 256; two-slice launches of a short contraction) and otherwise
+    slices * M * n_out * 4 bytes with 2 <= slices <= 16 and at least four 64-wide k-steps per slice."""
+    from torchtune_amd import _lib
+
+    lib = _lib.load()
+    q = lib.ttamd_nf4_gemm_workspace_bytes
+    assert q(1, 4096, 4096) == 0 and q(64, 4096, 4096) == 0
+    assert q(8192, 4096, 4096) == 0 and q(16384, 1024, 4096) == 0
+    assert q(2048, 2048, 2048) == 0  # 128 tiles, two slices of 16 k-steps: not worth the reduction
+    assert q(0, 4096, 4096) == 0 and q(128, 0, 4096) == 0
+    for M, N, K, slices in [(128, 4096, 4096, 16), (512, 4096, 4096, 4), (1024, 4096, 4096, 2), (65, 256, 512, 2),
+                            (300, 512, 1024, 4), (4096, 1024, 8192, 2)]:
+        assert q(M, N, K) == slices * M * N * 4, (M, N, K)
