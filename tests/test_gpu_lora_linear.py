@@ -553,3 +553,29 @@ def test_forward_and_backward_replay_from_a_hip_graph():
             for name, a, b in zip(("y", "gx", "gA", "gB"), outs, want):
                 assert torch.equal(a, b), f"M={M} replay {rep}: {name} differs from the eager result"
         del graph
+
+
+def test_few_token_and_sliced_kernels_at_8b_shapes():
+    """The Llama-3.1-8B projections at decode and evaluation token counts (few-token kernel: M = 1, 16, 64; sliced
+    contraction: M = 256): against the dense fp32 product with the bit-exact dequantised weight, deterministic, exactly
+    linear in the activations (scaling x by 2 scales every bf16 output by 2), and row m of a larger batch equals the
+    same row computed alone wherever the same kernel runs (M = 1 against row 0 of M = 16)."""
+    g = torch.Generator(device=DEV).manual_seed(8)
+    for (N, K) in ((4096, 4096), (1024, 4096), (14336, 4096), (4096, 14336)):
+        t = to_nf4((torch.randn(N, K, device=DEV, generator=g) * 0.02).to(BF))
+        D = t.get_original_weight().float()
+        bs, bst = t.block_scalers(), t.backward_copy()[1]
+        B = (torch.randn(N, 16, device=DEV, generator=g) * 0.05).to(BF)
+        for M in (1, 16, 64, 256):
+            x = torch.randn(M, K, device=DEV, generator=g).to(BF)
+            h = torch.randn(M, 16, device=DEV, generator=g).to(BF)
+            y = ops.nf4_lora_linear_fwd(x, t.quantized_data, bs, N, h, B, 2.0, block_scalers_t=bst)
+            ref = x.float() @ D.T + (2.0 * h.float()).to(BF).float() @ B.float().T
+            torch.testing.assert_close(y.float(), ref, rtol=1e-2, atol=1e-2, msg=f"N{N} K{K} M{M}")
+            assert torch.equal(y, ops.nf4_lora_linear_fwd(x, t.quantized_data, bs, N, h, B, 2.0, block_scalers_t=bst))
+            y2 = ops.nf4_lora_linear_fwd(2 * x, t.quantized_data, bs, N, 2 * h, B, 2.0, block_scalers_t=bst)
+            assert torch.equal(y2.float(), 2 * y.float()), f"N{N} K{K} M{M}: not linear"
+            if M == 16:
+                y_row = ops.nf4_lora_linear_fwd(x[:1].contiguous(), t.quantized_data, bs, N, h[:1].contiguous(), B, 2.0,
+                                                block_scalers_t=bst)
+                assert torch.equal(y_row[0], y[0])
