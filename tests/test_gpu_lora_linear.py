@@ -579,3 +579,54 @@ def test_few_token_and_sliced_kernels_at_8b_shapes():
                 y_row = ops.nf4_lora_linear_fwd(x[:1].contiguous(), t.quantized_data, bs, N, h[:1].contiguous(), B, 2.0,
                                                 block_scalers_t=bst)
                 assert torch.equal(y_row[0], y[0])
+
+
+def test_entry_points_are_reentrant_across_threads_and_streams():
+    """Backward runs on autograd's device thread and callers may use several streams: four Python threads, each on a
+    stream of its own, run forward + backward of differently shaped LoRA linears concurrently; every result must equal
+    the one the same call gives when it runs alone (the library keeps no state between calls and takes the stream from
+    the caller each time)."""
+    import threading
+
+    shapes = [(96, 256, 512, 8), (700, 512, 1024, 16), (33, 1024, 256, 24), (2048, 256, 2048, 64)]
+    g = torch.Generator(device=DEV).manual_seed(21)
+    cases = []
+    for M, N, K, r in shapes:
+        t = to_nf4((torch.randn(N, K, device=DEV, generator=g) * 0.02).to(BF))
+        cases.append(dict(
+            t=t, bs=t.block_scalers(), copy=t.backward_copy(), N=N, K=K,
+            x=torch.randn(M, K, device=DEV, generator=g).to(BF), gy=torch.randn(M, N, device=DEV, generator=g).to(BF),
+            A=(torch.randn(r, K, device=DEV, generator=g) * 0.05).to(BF), B=(torch.randn(N, r, device=DEV, generator=g) * 0.05).to(BF)))
+
+    def run(c):
+        h = ops.lora_hidden(c["x"], c["A"])
+        y = ops.nf4_lora_linear_fwd(c["x"], c["t"].quantized_data, c["bs"], c["N"], h, c["B"], 2.0, block_scalers_t=c["copy"][1])
+        gh, ga, gb = ops.lora_bwd(c["gy"], c["x"], h, c["B"], 2.0)
+        gx = ops.nf4_linear_bwd_dx(c["gy"], c["t"].quantized_data, c["bs"], c["K"], gh, c["A"], transposed=c["copy"])
+        return y, gx, ga, gb
+
+    want = [run(c) for c in cases]
+    torch.cuda.synchronize()
+    got, errors = [None] * len(cases), []
+
+    def worker(i):
+        try:
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream):
+                for _ in range(10):
+                    out = run(cases[i])
+                stream.synchronize()
+            got[i] = out
+        except Exception as e:  # surfaced in the main thread below
+            errors.append((i, repr(e)))
+
+    torch.cuda.synchronize()
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(len(cases))]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert not errors, errors
+    for i, (w, o) in enumerate(zip(want, got)):
+        for name, a, b in zip(("y", "gx", "gA", "gB"), w, o):
+            assert torch.equal(a, b), f"case {i}: {name} differs between the concurrent and the serial run"
