@@ -431,3 +431,15 @@ def test_gemm_workspace_query_is_a_host_function():
     for M, N, K, slices in [(128, 4096, 4096, 16), (512, 4096, 4096, 4), (1024, 4096, 4096, 2), (65, 256, 512, 2),
                             (300, 512, 1024, 4), (4096, 1024, 8192, 2)]:
         assert q(M, N, K) == slices * M * N * 4, (M, N, K)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """``bench.py --gpus N`` with N > 1 exits with a message before touching any device."""
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    root = Path(__file__).resolve().parents[1]
+    proc = subprocess.run([sys.executable, str(root / "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert proc.returncode != 0
+    assert "one GPU" in (proc.stdout + proc.stderr)
