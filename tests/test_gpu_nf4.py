@@ -157,3 +157,15 @@ def test_cpu_resident_tensor_is_staged_through_the_gpu():
     assert bits_equal(t.get_original_weight(), nf4_oracle.nf4_dequantize(nf4_oracle.nf4_quantize(w, 64, 256)))
     g = t.to(DEV)
     assert isinstance(g, NF4Tensor) and g.quantized_data.is_cuda and torch.equal(g.cpu().quantized_data, t.quantized_data)
+
+
+def test_one_dimensional_tensor_round_trip():
+    """``to_nf4`` takes tensors of one or two dimensions (the reference asserts ``dim() <= 2``): a flat tensor gives the
+    same codes and scalers as the same data viewed as a matrix, and dequantises back to its own shape."""
+    g = torch.Generator(device="cuda").manual_seed(3)
+    flat = (torch.randn(256 * 64 * 2, device="cuda", generator=g) * 0.02).to(torch.bfloat16)
+    a = to_nf4(flat)
+    b = to_nf4(flat.view(128, 256))
+    assert a.shape == flat.shape and a.get_original_weight().shape == flat.shape
+    assert torch.equal(a.quantized_data, b.quantized_data) and torch.equal(a.quantized_scalers, b.quantized_scalers)
+    assert torch.equal(a.get_original_weight(), b.get_original_weight().view(-1))

@@ -443,3 +443,18 @@ def test_bench_refuses_more_than_one_gpu():
     proc = subprocess.run([sys.executable, str(root / "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
     assert proc.returncode != 0
     assert "one GPU" in (proc.stdout + proc.stderr)
+
+
+def test_to_nf4_preconditions_are_the_reference_asserts():
+    """The four asserts of ``NF4Tensor.from_tensor`` fire before anything touches a device: at most two dimensions,
+    numel divisible by the block size, contiguous, number of blocks divisible by the scaler block size."""
+    from torchtune_amd import to_nf4
+
+    with pytest.raises(AssertionError, match="dim <= 2"):
+        to_nf4(torch.zeros(2, 64, 256, dtype=torch.bfloat16))
+    with pytest.raises(AssertionError, match="divisible by block size"):
+        to_nf4(torch.zeros(100, 3, dtype=torch.bfloat16))
+    with pytest.raises(AssertionError, match="contiguous"):
+        to_nf4(torch.zeros(512, 512, dtype=torch.bfloat16).t())
+    with pytest.raises(AssertionError, match="divisible by scaler_block_size"):
+        to_nf4(torch.zeros(64, 64, dtype=torch.bfloat16))  # 64 blocks, scaler blocks of 256
