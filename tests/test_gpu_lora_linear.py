@@ -360,21 +360,21 @@ def test_token_dimension_beyond_32_bit_offsets_is_split_into_row_ranges():
 
 
 def test_seeded_sweep_of_shapes_ranks_and_options_against_fp32_reference():
-    """Forty seeded combinations of (M, N, K, rank, bias, column scale, scaler layout, backward copy) through the raw ops,
+    """Sixty seeded combinations of (M, N, K, rank, bias, column scale, scaler layout, backward copy) through the raw ops,
     against fp32 matmuls of the bit-exact dequantised weight on the same device.  M is arbitrary, N and K any multiples
     of 64 (so tiles are ragged in every direction), ranks over the whole supported set."""
     import random
 
     rng = random.Random(20240607)
     g = torch.Generator(device=DEV).manual_seed(99)
-    for case in range(40):
-        M = rng.choice([1, 2, 31, 64, 127, 128, 129, 255, 256, 257, 300, 511, 513, 777, 1025])
+    for case in range(60):
+        M = rng.choice([1, 2, 17, 31, 64, 65, 127, 128, 129, 255, 256, 257, 300, 511, 513, 777, 1025, 2049])
         while True:  # to_nf4 needs whole scaler blocks of 256 blocks: (N / 64) * K must be a multiple of 256
             N = 64 * rng.randint(1, 17)
             K = 64 * rng.randint(1, 33)
             if (N // 64) * K % 256 == 0:
                 break
-        r = rng.choice([0, 8, 16, 24, 40, 64])
+        r = rng.choice([0, 8, 16, 24, 32, 40, 48, 56, 64])
         use_bias, use_cs, use_t, use_copy = (rng.random() < 0.5 for _ in range(4))
         t = to_nf4((torch.randn(N, K, device=DEV, generator=g) * 0.02).to(BF))
         D = t.get_original_weight().float()
