@@ -129,3 +129,36 @@ def test_cross_entropy_forward_backward(rows, V):
     per_row, _ = ops.cross_entropy_fwd_bwd(ld.detach(), target.to(DEV))
     ref_rows = torch.nn.functional.cross_entropy(logits.detach().float(), target, reduction="none")
     torch.testing.assert_close(per_row.cpu(), ref_rows, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("rows,D,V,train_weight", [(37, 256, 1024, False), (64, 128, 4096, True)])
+def test_linear_cross_entropy_node_matches_projection_then_loss(rows, D, V, train_weight):
+    """Vocabulary projection + loss as one autograd node: the same loss as ``cross_entropy_sum(linear(h, W))`` and the
+    same gradients for the hidden states (and the weight when it trains), with an incoming gradient other than 1."""
+    g = torch.Generator(device=DEV).manual_seed(rows + V)
+    h = torch.randn(rows, D, device=DEV, generator=g).to(BF)
+    W = (torch.randn(V, D, device=DEV, generator=g) * 0.1).to(BF)
+    target = torch.randint(0, V, (rows,), device=DEV, generator=g)
+    target[1] = -100
+    outs = []
+    for fused in (False, True):
+        hh = h.clone().requires_grad_()
+        ww = W.clone().requires_grad_(train_weight)
+        if fused:
+            loss = layer_ops.linear_cross_entropy_sum(hh, ww, target, scale=1.0 / rows)
+        else:
+            loss = layer_ops.cross_entropy_sum(torch.nn.functional.linear(hh, ww), target, scale=1.0 / rows)
+        (loss * 3.0).backward()
+        outs.append((loss.detach(), hh.grad, ww.grad))
+    torch.testing.assert_close(outs[0][0], outs[1][0], rtol=0, atol=0)
+    torch.testing.assert_close(outs[0][1].float(), outs[1][1].float(), rtol=2e-2, atol=1e-2 * float(outs[0][1].abs().max()))
+    if train_weight:
+        torch.testing.assert_close(outs[0][2].float(), outs[1][2].float(), rtol=2e-2, atol=1e-2 * float(outs[0][2].abs().max()))
+    else:
+        assert outs[1][2] is None
+    # against fp32 autograd on the same operands
+    hf, wf = h.float().requires_grad_(), W.float().requires_grad_()
+    ref = torch.nn.functional.cross_entropy(hf @ wf.T, target, reduction="sum") / rows
+    (ref * 3.0).backward()
+    torch.testing.assert_close(outs[1][0], ref.detach(), rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(outs[1][1].float(), hf.grad, rtol=5e-2, atol=2e-2 * float(hf.grad.abs().max()))

@@ -209,7 +209,12 @@ class Decoder(nn.Module):
         target = labels.reshape(-1)
         total = hidden.new_zeros((), dtype=torch.float32)
         n = target.numel()
+        out = self.output
+        plain = type(out) is nn.Linear and out.bias is None and out.weight.shape[0] % 8 == 0 and out.weight.shape[0] <= 131072
         for hc, tc in zip(hidden.chunk(self.loss_chunks), target.chunk(self.loss_chunks)):
+            if plain and _fused(hc) and out.weight.dtype == hc.dtype:
+                total = total + layer_ops.linear_cross_entropy_sum(hc, out.weight, tc, scale=1.0 / n)
+                continue
             logits = self.output(hc)
             if _fused(logits) and logits.shape[-1] % 8 == 0 and logits.shape[-1] <= 131072:
                 total = total + layer_ops.cross_entropy_sum(logits, tc, scale=1.0 / n)

@@ -94,6 +94,35 @@ class _CrossEntropySumFn(torch.autograd.Function):
         return grad.mul_(g.to(grad.dtype)), None, None, None
 
 
+class _LinearCrossEntropySumFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, hidden, weight, target, ignore_index: int, scale: float):
+        logits = torch.nn.functional.linear(hidden, weight)
+        loss, grad = ops.cross_entropy_fwd_bwd(logits, target, ignore_index, scale)
+        ctx.save_for_backward(grad, hidden, weight)
+        return loss.sum() * scale
+
+    @staticmethod
+    def backward(ctx, g):
+        grad, hidden, weight = ctx.saved_tensors
+        gh = gw = None
+        # the incoming scalar multiplies the small products, not the [rows, vocabulary] gradient of the logits
+        if ctx.needs_input_grad[0]:
+            gh = (grad @ weight).mul_(g.to(grad.dtype))
+        if ctx.needs_input_grad[1]:
+            gw = (grad.t() @ hidden).mul_(g.to(grad.dtype))
+        return gh, gw, None, None, None
+
+
+def linear_cross_entropy_sum(hidden: torch.Tensor, weight: torch.Tensor, target: torch.Tensor, ignore_index: int = -100,
+                             scale: float = 1.0) -> torch.Tensor:
+    """``scale * F.cross_entropy((hidden @ weight.T).float(), target, reduction="sum")`` for one chunk of rows: the
+    vocabulary projection and the loss of the reference's ``LinearCrossEntropyLoss.compute_cross_entropy``
+    (``torchtune/modules/loss/cross_entropy_loss.py:86-112``) as one autograd node, so that backward scales the
+    ``[rows, dim]`` (and ``[vocabulary, dim]``) products by the incoming gradient instead of the logits' gradient."""
+    return _LinearCrossEntropySumFn.apply(hidden, weight, target, ignore_index, scale)
+
+
 def cross_entropy_sum(logits: torch.Tensor, target: torch.Tensor, ignore_index: int = -100, scale: float = 1.0) -> torch.Tensor:
     """``scale * F.cross_entropy(logits.float(), target, reduction="sum", ignore_index=ignore_index)`` for bf16 logits
     ``[rows, V]``: the per-chunk body of the reference's ``LinearCrossEntropyLoss``
