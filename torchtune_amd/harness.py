@@ -191,9 +191,15 @@ class Decoder(nn.Module):
         self.layers = nn.ModuleList(DecoderLayer(s, rank, alpha, quantize_base) for _ in range(s.n_layers))
         self.norm = RMSNorm(s.dim, s.norm_eps)
         self.output = nn.Linear(s.dim, s.vocab, bias=False)
+        self._rope = None  # (seq_len, device, table): built once per sequence length, as the reference keeps it in a buffer
+
+    def _rope_cache(self, seq_len: int, device) -> torch.Tensor:
+        if self._rope is None or self._rope[0] != seq_len or self._rope[1] != device:
+            self._rope = (seq_len, device, rope_cache(seq_len, self.shape.head_dim, self.shape.rope_base, device))
+        return self._rope[2]
 
     def forward(self, tokens: torch.Tensor) -> torch.Tensor:
-        rope = rope_cache(tokens.shape[1], self.shape.head_dim, self.shape.rope_base, tokens.device)
+        rope = self._rope_cache(tokens.shape[1], tokens.device)
         h = self.tok_embeddings(tokens)
         for layer in self.layers:
             if self.ac and torch.is_grad_enabled():
