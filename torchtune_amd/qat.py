@@ -21,6 +21,7 @@ from __future__ import annotations
 
 from dataclasses import dataclass
 from enum import Enum, auto
+import threading
 from typing import Optional, Union
 
 import torch
@@ -173,12 +174,28 @@ class FakeQuantizer(nn.Module):
                 and config.scale_precision in (torch.bfloat16, torch.float32)
                 and config.zero_point_precision == config.scale_precision)
 
+    # Sibling linears (q/k/v, gate/up) fake-quantise the very same activation tensor one after the other; the dynamic
+    # per-token result depends on the tensor and the scale precision only, so the last one is kept (per thread, together
+    # with the tensor itself, so that its memory cannot be handed to another tensor meanwhile) and reused while the
+    # same, unmodified tensor object comes in again.  ``share_identical_inputs = False`` recomputes every time.
+    share_identical_inputs = True
+    _last = threading.local()
+
+    def _per_token(self, x: torch.Tensor):
+        key = (x._version, self.config.scale_precision)
+        hit = getattr(FakeQuantizer._last, "entry", None)
+        if FakeQuantizer.share_identical_inputs and hit is not None and hit[0] is x and hit[1] == key:
+            return hit[2]
+        out = ops.fq_per_token_int8_asym(x.detach(), qparam_dtype=self.config.scale_precision)
+        FakeQuantizer._last.entry = (x, key, out) if FakeQuantizer.share_identical_inputs else None
+        return out
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         if not self.enabled:
             return x
         with torch.no_grad():
             if isinstance(self.config.granularity, PerToken):
-                fq, scale, zp = ops.fq_per_token_int8_asym(x.detach(), qparam_dtype=self.config.scale_precision)
+                fq, scale, zp = self._per_token(x)
                 self.scale = scale.to(self.config.scale_precision)
                 self.zero_point = zp.to(self.config.zero_point_precision)
             else:
