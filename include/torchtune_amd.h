@@ -339,6 +339,16 @@ int ttamd_rope_bf16(const void* x, const float* cache, void* y, int64_t B, int64
                     int inverse, void* stream);
 
 /*
+ * Grouped-query expansion of the key / value heads before attention
+ * (torchtune/modules/attention.py:284-290: k.unsqueeze(2).expand(...).flatten(1, 2), here on the [b, s, n_kv, h_d] layout):
+ * y [tokens, n_kv * rep, head_dim] with y[t][kv * rep + r] = x[t][kv], and its backward
+ * gx[t][kv] = bf16(sum_r gy[t][kv * rep + r]) (fp32 sums, r ascending).  All bf16, head_dim a multiple of 8.
+ */
+int ttamd_repeat_kv_bf16(const void* x, void* y, int64_t tokens, int64_t n_kv, int64_t rep, int64_t head_dim, void* stream);
+int ttamd_repeat_kv_bwd_bf16(const void* gy, void* gx, int64_t tokens, int64_t n_kv, int64_t rep, int64_t head_dim,
+                             void* stream);
+
+/*
  * FeedForward gate (torchtune/modules/feed_forward.py:50-53): out = bf16( bf16(silu(gate)) * up ), and its backward
  * ggate, gup from gout.  All [numel] bf16, numel a multiple of 8.
  */

@@ -162,3 +162,24 @@ def test_linear_cross_entropy_node_matches_projection_then_loss(rows, D, V, trai
     (ref * 3.0).backward()
     torch.testing.assert_close(outs[1][0], ref.detach(), rtol=2e-2, atol=2e-2)
     torch.testing.assert_close(outs[1][1].float(), hf.grad, rtol=5e-2, atol=2e-2 * float(hf.grad.abs().max()))
+
+
+@pytest.mark.parametrize("b,s,nkv,rep,hd", [(2, 33, 8, 4, 128), (1, 7, 2, 3, 64), (3, 5, 1, 8, 8), (1, 4, 4, 1, 16)])
+def test_repeat_kv_forward_backward(b, s, nkv, rep, hd):
+    """Grouped-query expansion: the forward is exactly ``unsqueeze(3).expand(...).flatten(2, 3)``; the backward is the
+    sum over a head's copies, accumulated in fp32 and rounded once (bit-equal to the fp32 sum rounded to bf16)."""
+    g = torch.Generator(device=DEV).manual_seed(b * 100 + s)
+    x = torch.randn(b, s, nkv, hd, device=DEV, generator=g).to(BF).requires_grad_()
+    y = layer_ops.repeat_kv(x, rep)
+    want = x.detach().unsqueeze(3).expand(b, s, nkv, rep, hd).flatten(2, 3)
+    assert y.shape == (b, s, nkv * rep, hd) and torch.equal(y, want)
+    gy = torch.randn(b, s, nkv * rep, hd, device=DEV, generator=g).to(BF)
+    y.backward(gy)
+    gsum = torch.zeros(b, s, nkv, hd, device=DEV, dtype=torch.float32)
+    for r in range(rep):  # the kernel's order
+        gsum = gsum + gy.view(b, s, nkv, rep, hd)[:, :, :, r].float()
+    assert torch.equal(x.grad, gsum.to(BF))
+    with pytest.raises(ValueError):
+        ops.repeat_kv(x.detach()[0], rep)
+    with pytest.raises(ValueError):
+        ops.repeat_kv_bwd(gy, rep + 1 if (nkv * rep) % (rep + 1) else rep * nkv * 2 + 1)

@@ -102,6 +102,8 @@ SIGNATURES = {
         [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _i64, _i64, _c_void_p, _size, _c_void_p],
     ),
     "ttamd_rope_bf16": (_int, [_c_void_p, _c_void_p, _c_void_p, _i64, _i64, _i64, _i64, _int, _c_void_p]),
+    "ttamd_repeat_kv_bf16": (_int, [_c_void_p, _c_void_p, _i64, _i64, _i64, _i64, _c_void_p]),
+    "ttamd_repeat_kv_bwd_bf16": (_int, [_c_void_p, _c_void_p, _i64, _i64, _i64, _i64, _c_void_p]),
     "ttamd_swiglu_fwd_bf16": (_int, [_c_void_p, _c_void_p, _c_void_p, _i64, _c_void_p]),
     "ttamd_cross_entropy_fwd_bwd_bf16": (_int, [_c_void_p, _c_void_p, _i64, _f32, _c_void_p, _c_void_p, _i64, _i64, _c_void_p]),
     "ttamd_swiglu_bwd_bf16": (_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _i64, _c_void_p]),

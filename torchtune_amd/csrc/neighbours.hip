@@ -369,6 +369,76 @@ extern "C" int ttamd_rope_bf16(const void* x, const float* cache, void* y, int64
   return check_launch("rope");
 }
 
+namespace ttamd {
+namespace {
+
+// Grouped-query expansion: y[t][kv * rep + r][:] = x[t][kv][:] for r < rep (t = token).  One thread per 16-byte chunk of
+// the OUTPUT, so the writes (rep times the reads) are whole lines; the repeated reads hit in cache.
+__global__ __launch_bounds__(256) void repeat_kv_kernel(const u32x4_t* __restrict__ x, u32x4_t* __restrict__ y, int64_t n_out,
+                                                        int chunks_per_head, int n_kv, int rep) {
+  const int64_t oc = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (oc >= n_out) return;
+  const int64_t out_head = oc / chunks_per_head;  // token * (n_kv * rep) + kv * rep + r
+  const int c = (int)(oc - out_head * chunks_per_head);
+  const int64_t tok = out_head / (n_kv * rep);
+  const int kv = (int)(out_head - tok * (n_kv * rep)) / rep;
+  y[oc] = x[(tok * n_kv + kv) * chunks_per_head + c];
+}
+
+// Its backward: gx[t][kv][:] = bf16(sum_r gy[t][kv * rep + r][:]), fp32 sums in the order r = 0 .. rep - 1.
+__global__ __launch_bounds__(256) void repeat_kv_bwd_kernel(const u32x4_t* __restrict__ gy, u32x4_t* __restrict__ gx, int64_t n_in,
+                                                            int chunks_per_head, int rep) {
+  const int64_t ic = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (ic >= n_in) return;
+  const int64_t in_head = ic / chunks_per_head;
+  const int c = (int)(ic - in_head * chunks_per_head);
+  float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  for (int r = 0; r < rep; ++r) {
+    const u32x4_t v = gy[(in_head * rep + r) * chunks_per_head + c];
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      acc[2 * d] += bits_f32(v[d] << 16);
+      acc[2 * d + 1] += bits_f32(v[d] & 0xffff0000u);
+    }
+  }
+  u32x4_t o;
+#pragma unroll
+  for (int d = 0; d < 4; ++d) o[d] = (uint32_t)f32_to_bf16_bits(acc[2 * d]) | ((uint32_t)f32_to_bf16_bits(acc[2 * d + 1]) << 16);
+  gx[ic] = o;
+}
+
+int check_repeat_kv(const char* who, const void* a, const void* b, int64_t tokens, int64_t n_kv, int64_t rep, int64_t head_dim) {
+  TT_REQUIRE(a && b, "%s: null pointer argument", who);
+  TT_REQUIRE(aligned16(a) && aligned16(b), "%s: pointers must be 16-byte aligned", who);
+  TT_REQUIRE(tokens > 0 && n_kv > 0 && rep > 0 && head_dim > 0 && head_dim % 8 == 0 && n_kv * rep < (1 << 20) &&
+                 head_dim < (1 << 20),
+             "%s: bad shape tokens=%lld n_kv=%lld rep=%lld h_d=%lld (h_d must be a multiple of 8)", who, (long long)tokens,
+             (long long)n_kv, (long long)rep, (long long)head_dim);
+  TT_REQUIRE((tokens * n_kv * rep * (head_dim / 8) + 255) / 256 < (int64_t(1) << 31), "%s: tensor too large for one launch", who);
+  return TTAMD_OK;
+}
+
+}  // namespace
+}  // namespace ttamd
+
+extern "C" int ttamd_repeat_kv_bf16(const void* x, void* y, int64_t tokens, int64_t n_kv, int64_t rep, int64_t head_dim,
+                                    void* stream) {
+  if (int rc = check_repeat_kv("repeat_kv", x, y, tokens, n_kv, rep, head_dim)) return rc;
+  const int64_t n_out = tokens * n_kv * rep * (head_dim / 8);
+  repeat_kv_kernel<<<dim3((unsigned)((n_out + 255) / 256)), dim3(256), 0, reinterpret_cast<hipStream_t>(stream)>>>(
+      reinterpret_cast<const u32x4_t*>(x), reinterpret_cast<u32x4_t*>(y), n_out, (int)(head_dim / 8), (int)n_kv, (int)rep);
+  return check_launch("repeat_kv");
+}
+
+extern "C" int ttamd_repeat_kv_bwd_bf16(const void* gy, void* gx, int64_t tokens, int64_t n_kv, int64_t rep, int64_t head_dim,
+                                        void* stream) {
+  if (int rc = check_repeat_kv("repeat_kv_bwd", gy, gx, tokens, n_kv, rep, head_dim)) return rc;
+  const int64_t n_in = tokens * n_kv * (head_dim / 8);
+  repeat_kv_bwd_kernel<<<dim3((unsigned)((n_in + 255) / 256)), dim3(256), 0, reinterpret_cast<hipStream_t>(stream)>>>(
+      reinterpret_cast<const u32x4_t*>(gy), reinterpret_cast<u32x4_t*>(gx), n_in, (int)(head_dim / 8), (int)rep);
+  return check_launch("repeat_kv_bwd");
+}
+
 extern "C" int ttamd_swiglu_fwd_bf16(const void* gate, const void* up, void* out, int64_t numel, void* stream) {
   TT_REQUIRE(gate && up && out, "swiglu_fwd: null pointer argument");
   TT_REQUIRE(aligned16(gate) && aligned16(up) && aligned16(out), "swiglu_fwd: pointers must be 16-byte aligned");

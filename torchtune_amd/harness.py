@@ -144,8 +144,11 @@ class Attention(nn.Module):
         k = apply_rope(k, rope)
         if self.n_kv != self.n_heads:  # expand kv heads to query heads, as the reference does before SDPA
             rep = self.n_heads // self.n_kv
-            k = k.unsqueeze(3).expand(b, sl, self.n_kv, rep, self.head_dim).flatten(2, 3)
-            v = v.unsqueeze(3).expand(b, sl, self.n_kv, rep, self.head_dim).flatten(2, 3)
+            if _fused(k) and self.head_dim % 8 == 0:
+                k, v = layer_ops.repeat_kv(k, rep), layer_ops.repeat_kv(v, rep)
+            else:
+                k = k.unsqueeze(3).expand(b, sl, self.n_kv, rep, self.head_dim).flatten(2, 3)
+                v = v.unsqueeze(3).expand(b, sl, self.n_kv, rep, self.head_dim).flatten(2, 3)
         o = _sdpa(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2))
         return self.output_proj(o.transpose(1, 2).reshape(b, sl, -1))
 

@@ -63,6 +63,24 @@ def apply_rope(x: torch.Tensor, cache: torch.Tensor) -> torch.Tensor:
     return _RopeFn.apply(x, cache)
 
 
+class _RepeatKVFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, rep: int):
+        ctx.rep = rep
+        return ops.repeat_kv(x, rep)
+
+    @staticmethod
+    def backward(ctx, gy):
+        return ops.repeat_kv_bwd(gy, ctx.rep), None
+
+
+def repeat_kv(x: torch.Tensor, rep: int) -> torch.Tensor:
+    """``x.unsqueeze(3).expand(b, s, n_kv, rep, h_d).flatten(2, 3)`` for ``x`` ``[b, s, n_kv, h_d]``: the grouped-query
+    expansion of key / value heads (``torchtune/modules/attention.py:284-290``) as one copy kernel, with the sum over the
+    copies as its backward."""
+    return _RepeatKVFn.apply(x, rep)
+
+
 class _SwiGLUFn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, gate, up):

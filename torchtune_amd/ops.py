@@ -539,6 +539,34 @@ def rope(x: torch.Tensor, cache: torch.Tensor, inverse: bool = False) -> torch.T
     return y
 
 
+def repeat_kv(x: torch.Tensor, rep: int) -> torch.Tensor:
+    """x [b, s, n_kv, h_d] bf16 -> [b, s, n_kv * rep, h_d]: every key / value head ``rep`` times in a row."""
+    xc = _bf16_any(x, "repeat_kv: x")
+    if xc.dim() != 4 or rep < 1:
+        raise ValueError(f"repeat_kv: expected [b, s, n_kv, h_d] and rep >= 1, got {tuple(x.shape)}, rep={rep}")
+    b, s, nkv, hd = xc.shape
+    y = torch.empty(b, s, nkv * rep, hd, dtype=torch.bfloat16, device=xc.device)
+    lib = _lib.load()
+    with torch.cuda.device(x.device):
+        rc = lib.ttamd_repeat_kv_bf16(xc.data_ptr(), y.data_ptr(), b * s, nkv, rep, hd, _stream(x))
+    _lib.check(rc, "repeat_kv")
+    return y
+
+
+def repeat_kv_bwd(gy: torch.Tensor, rep: int) -> torch.Tensor:
+    """gy [b, s, n_kv * rep, h_d] bf16 -> [b, s, n_kv, h_d]: the sum over each head's ``rep`` copies."""
+    g = _bf16_any(gy, "repeat_kv_bwd: gy")
+    if g.dim() != 4 or rep < 1 or g.shape[2] % rep:
+        raise ValueError(f"repeat_kv_bwd: expected [b, s, n_kv * rep, h_d], got {tuple(gy.shape)}, rep={rep}")
+    b, s, nh, hd = g.shape
+    gx = torch.empty(b, s, nh // rep, hd, dtype=torch.bfloat16, device=g.device)
+    lib = _lib.load()
+    with torch.cuda.device(gy.device):
+        rc = lib.ttamd_repeat_kv_bwd_bf16(g.data_ptr(), gx.data_ptr(), b * s, nh // rep, rep, hd, _stream(gy))
+    _lib.check(rc, "repeat_kv_bwd")
+    return gx
+
+
 def swiglu_fwd(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     g = _bf16_any(gate, "swiglu_fwd: gate")
     u = _bf16_any(up, "swiglu_fwd: up")
