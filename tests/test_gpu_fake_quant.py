@@ -418,3 +418,30 @@ def test_per_token_result_is_shared_between_sibling_quantizers(monkeypatch):
     z = y.clone()  # equal values, another tensor: recomputed
     c = qs[2](z)
     assert len(calls) == n + 2 and torch.equal(b, c)
+
+
+def test_prepare_with_default_quantizer_arguments_runs_a_bf16_model():
+    """The north-star QAT config builds the quantizer with a group size only (recipes/configs/llama3/8B_qat_full.yaml:62-64,
+    precision left at its float32 default) on a bf16 model: the prepared model must keep bf16 weights, train, and match
+    the oracle."""
+    gen = torch.Generator().manual_seed(11)
+    model = nn.Sequential(nn.Linear(256, 128, bias=False)).to(DEV).to(torch.bfloat16)
+    w = (torch.randn(128, 256, generator=gen) * 0.05).to(torch.bfloat16)
+    with torch.no_grad():
+        model[0].weight.copy_(w)
+    param = model[0].weight
+    model = Int8DynActInt4WeightQATQuantizer(groupsize=32).prepare(model)
+    assert model[0].weight is param and model[0].weight.dtype == torch.bfloat16
+    x = torch.randn(6, 256, generator=gen).to(torch.bfloat16)
+    xd = x.to(DEV).requires_grad_()
+    y = model(xd)
+    assert y.dtype == torch.bfloat16
+    (y.float() ** 2).sum().backward()
+    xo, wo = x.clone().requires_grad_(), w.clone().requires_grad_()
+    yo = fq.fake_quantized_linear(xo, wo, 32)
+    (yo.float() ** 2).sum().backward()
+    torch.testing.assert_close(y.detach().cpu().float(), yo.detach().float(), rtol=1e-2, atol=1e-2)
+    torch.testing.assert_close(xd.grad.cpu().float(), xo.grad.float(), rtol=1e-2, atol=1e-2)
+    with torch.inference_mode():  # evaluation / generation loops run under inference_mode
+        yi = model(x.to(DEV))
+    torch.testing.assert_close(yi.cpu().float(), yo.detach().float(), rtol=1e-2, atol=1e-2)

@@ -418,7 +418,7 @@ def test_seeded_sweep_of_shapes_ranks_and_options_against_fp32_reference():
         torch.testing.assert_close(gx.float(), gx_ref, rtol=1e-2, atol=1e-2 * max(1.0, float(gx_ref.abs().max()) / 8), msg=tag)
 
 
-@pytest.mark.parametrize("N,K", [(64, 64), (192, 320 * 4), (1024, 4096), (4096, 1024 + 64), (8192, 256 + 64), (256, 8192 + 64)])
+@pytest.mark.parametrize("N,K", [(256, 64), (192, 320 * 4), (1024, 4096), (4096, 1024 + 64), (8192, 256 + 64), (256, 8192 + 64)])
 def test_few_tokens_take_the_weight_streaming_kernel(N, K):
     """M <= 64 (decode / evaluation): the library streams the packed weight once instead of tiling.  Every token count
     from 1 to 64 that touches a tile edge, K with and without a half chunk at the end, adapter ranks, bias and column

@@ -233,3 +233,30 @@ def test_merged_checkpoint_weight_vs_oracle(N, K, r):
     sd_h = {"l.weight": t, "l.lora_a.weight": A.to(DEV), "l.lora_b.weight": B.to(DEV)}
     host = get_merged_lora_ckpt(sd_h, rank=r, alpha=alpha, offload_to_cpu=True)["l.weight"]
     assert host.device.type == "cpu" and host.is_pinned() and torch.equal(host, got)
+
+
+def test_write_through_an_alias_invalidates_the_derived_caches():
+    """``param.data.copy_(w)`` / ``param.detach().copy_(w)`` write through an alias that has inner tensor objects of its
+    own; the fused forward and backward of the original parameter must then use the scalers and the transposed codes of
+    the new weight (checked against the oracle of the new weight)."""
+    torch.manual_seed(3)
+    with _default_dtype(torch.bfloat16), torch.device(DEV):
+        layer = LoRALinear(512, 512, rank=8, alpha=8.0, quantize_base=True)  # rank 8: the fused kernels
+    _fixed_init(layer)
+    x = torch.randn(70, 512, dtype=torch.bfloat16)
+    layer(x.to(DEV)).sum().backward()  # fills the block-scaler and transposed-copy caches of the old weight
+    for write in (lambda w: layer.weight.data.copy_(w), lambda w: layer.weight.detach().copy_(w)):
+        w_new = (torch.randn(512, 512) * 0.3).to(torch.bfloat16)
+        with torch.no_grad():
+            write(w_new.to(DEV))
+        parts = nf4_oracle.nf4_quantize(w_new, 64, 256)
+        assert torch.equal(layer.weight.get_original_weight().cpu(), nf4_oracle.nf4_dequantize(parts))
+        xd = x.to(DEV).requires_grad_()
+        y = layer(xd)
+        (y.float() ** 2).sum().backward()
+        xo = x.clone().requires_grad_()
+        yo = lora_oracle.lora_linear_forward(xo, parts, layer.lora_a.weight.detach().cpu(), layer.lora_b.weight.detach().cpu(), 8.0, 8)
+        (yo.float() ** 2).sum().backward()
+        torch.testing.assert_close(y.detach().cpu().float(), yo.detach().float(), rtol=1e-2, atol=1e-2)
+        gx = xo.grad.float()
+        torch.testing.assert_close(xd.grad.cpu().float(), gx, rtol=1e-2, atol=1e-2 * max(1.0, float(gx.abs().max()) / 8))

@@ -109,7 +109,7 @@ class _CrossEntropySumFn(torch.autograd.Function):
     @staticmethod
     def backward(ctx, g):
         (grad,) = ctx.saved_tensors
-        return grad.mul_(g.to(grad.dtype)), None, None, None
+        return grad.mul_(g.float().reshape(1)), None, None, None  # a 1-D fp32 factor: product in fp32, rounded to bf16 once
 
 
 class _LinearCrossEntropySumFn(torch.autograd.Function):
@@ -126,9 +126,9 @@ class _LinearCrossEntropySumFn(torch.autograd.Function):
         gh = gw = None
         # the incoming scalar multiplies the small products, not the [rows, vocabulary] gradient of the logits
         if ctx.needs_input_grad[0]:
-            gh = (grad @ weight).mul_(g.to(grad.dtype))
+            gh = (grad @ weight).mul_(g.float().reshape(1))
         if ctx.needs_input_grad[1]:
-            gw = (grad.t() @ hidden).mul_(g.to(grad.dtype))
+            gw = (grad.t() @ hidden).mul_(g.float().reshape(1))
         return gh, gw, None, None, None
 
 

@@ -75,7 +75,8 @@ def _get_lora_modules(state_dict: Dict[str, Any]) -> Set[str]:
 
 
 @torch.no_grad()
-def get_merged_lora_ckpt(state_dict: Dict[str, Any], rank: int, alpha: float, offload_to_cpu: bool = False) -> Dict[str, Any]:
+def get_merged_lora_ckpt(state_dict: Dict[str, Any], rank: int, alpha: float, use_distributed_barriers: bool = False, *,
+                         offload_to_cpu: bool = False) -> Dict[str, Any]:
     """Fold every LoRA pair of ``state_dict`` into its base weight and delete the adapter entries; modifies and
     returns ``state_dict`` (``torchtune/modules/peft/_utils.py:193-271``; MoE experts raise).
 
@@ -84,8 +85,11 @@ def get_merged_lora_ckpt(state_dict: Dict[str, Any], rank: int, alpha: float, of
 
     A base weight that is still an ``NF4Tensor`` on the GPU (a state dict taken without the dequantising hook) is
     dequantised and merged in one pass by the HIP kernel; a dense weight is updated as the reference does.
-    ``offload_to_cpu`` (not in the reference's signature) makes that kernel store the merged weight of a plain LoRA
-    module straight into pinned host memory, so the dense merged weight never exists on the GPU.
+    ``use_distributed_barriers`` is the reference's fourth parameter (its checkpoint client passes it by keyword,
+    ``torchtune/training/checkpointing/_checkpoint_client.py:177-182``); there is one process per GPU and no barrier to
+    take here, so it is accepted and ignored.  ``offload_to_cpu`` (keyword only, not in the reference's signature) makes
+    that kernel store the merged weight of a plain LoRA module straight into pinned host memory, so the dense merged
+    weight never exists on the GPU.
     """
     wrote_to_host = None
     scale = alpha / rank

@@ -22,6 +22,7 @@ import torch
 from torch import nn
 
 from ... import ops
+from ...nf4_tensor import _check_in_features
 from ._adapter_base import LowRankAdapterLinear
 
 
@@ -31,6 +32,7 @@ class _QDoRALinearFn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, weight, lora_a, lora_b, magnitude, bias, scale: float):
         N, K = weight.shape
+        _check_in_features(x, weight)
         x2 = x.reshape(-1, K)
         tr = weight.backward_copy()
         _, mns = ops.nf4_dora_weight_norm(weight.quantized_data, weight.block_scalers(), N, K, lora_a, lora_b, scale, magnitude)

@@ -25,6 +25,7 @@ import torch.nn.functional as F
 from torch import nn
 
 from ... import ops
+from ...nf4_tensor import _check_in_features
 from ._adapter_base import LowRankAdapterLinear, _lora_a_init_params, _lora_b_init_params  # noqa: F401
 
 
@@ -40,6 +41,7 @@ class _QLoRALinearFn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, weight, lora_a, lora_b, bias, scale: float):
         N, K = weight.shape
+        _check_in_features(x, weight)
         x2 = x.reshape(-1, K)
         h = ops.lora_hidden(x2, lora_a)
         tr = weight.backward_copy()

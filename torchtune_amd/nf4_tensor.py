@@ -55,6 +55,23 @@ NF4_TORCH_FUNCTIONS: Dict[Any, Callable] = {}
 _INNER_TENSORS = ("quantized_scalers", "quantization_factor", "scaler_mean", "quantized_data", "nf4")
 
 
+# Writes into an NF4 tensor happen inside __torch_dispatch__, where the in-place version counters of the inner tensors do
+# not advance, and an alias (``param.data``, ``param.detach()``) has inner tensor objects of its own over the same
+# storage.  The derived-data caches (block scalers, transposed copy) are therefore keyed on a generation number kept
+# per storage address of the scaler bytes: ``copy_`` bumps it, so every alias sees its cache go stale.
+_WRITE_GENERATION: Dict[int, int] = {}
+
+
+def _generation(qs: torch.Tensor) -> int:
+    return _WRITE_GENERATION.get(qs.untyped_storage().data_ptr(), 0) if qs.device.type != "meta" else 0
+
+
+def _bump_generation(qs: torch.Tensor) -> None:
+    if qs.device.type != "meta":
+        ptr = qs.untyped_storage().data_ptr()
+        _WRITE_GENERATION[ptr] = _WRITE_GENERATION.get(ptr, 0) + 1
+
+
 def implements(aten_ops: Iterable[Any]):
     """Register a ``__torch_dispatch__`` handler for NF4Tensor.  The handler is called as
     ``handler(func, args, kwargs)`` with the positional arguments still packed in one tuple, which is the
@@ -204,9 +221,9 @@ class NF4Tensor(torch.Tensor):
     def block_scalers(self) -> torch.Tensor:
         """Dequantised per-block scalers as fp32 [n_blocks] on the GPU, cached while the scaler tensors are
         unchanged (the cache rides on the ``quantized_scalers`` tensor object and is keyed by the in-place
-        version counters of the three scaler tensors)."""
+        version counters of the three scaler tensors and the write generation of their storage)."""
         qs = self.quantized_scalers
-        key = (qs._version, self.quantization_factor._version, self.scaler_mean._version, qs.data_ptr())
+        key = (qs._version, self.quantization_factor._version, self.scaler_mean._version, qs.data_ptr(), _generation(qs))
         cached = getattr(qs, "_ttamd_block_scalers", None)
         if cached is not None and cached[0] == key:
             return cached[1]
@@ -225,7 +242,7 @@ class NF4Tensor(torch.Tensor):
             return None
         qs = self.quantized_scalers
         key = (qs._version, self.quantization_factor._version, self.scaler_mean._version, self.quantized_data._version,
-               qs.data_ptr())
+               qs.data_ptr(), _generation(qs))
         cached = getattr(qs, "_ttamd_backward_copy", None)
         if cached is not None and cached[0] == key:
             return cached[1]
@@ -290,7 +307,7 @@ def _carry_cache(src: NF4Tensor, dst: NF4Tensor) -> None:
     cached = getattr(src.quantized_scalers, "_ttamd_block_scalers", None)
     if cached is not None and dst.quantized_scalers.data_ptr() == src.quantized_scalers.data_ptr():
         key = (dst.quantized_scalers._version, dst.quantization_factor._version, dst.scaler_mean._version,
-               dst.quantized_scalers.data_ptr())
+               dst.quantized_scalers.data_ptr(), _generation(dst.quantized_scalers))
         if key == cached[0]:
             dst.quantized_scalers._ttamd_block_scalers = cached
 
@@ -316,10 +333,11 @@ def _nf4_copy_(func, args, kwargs):
     if not isinstance(dst, NF4Tensor):
         # dense.copy_(nf4): materialise
         return func(dst, src.get_original_weight(), **kwargs)
-    # in-place writes issued from inside __torch_dispatch__ do not advance the version counters the
-    # block-scaler cache is keyed on, so drop the cache explicitly
+    # in-place writes issued from inside __torch_dispatch__ do not advance the version counters, so the caches of
+    # this tensor object are dropped and the storage's write generation is bumped for those of its aliases
     dst.quantized_scalers._ttamd_block_scalers = None
     dst.quantized_scalers._ttamd_backward_copy = None
+    _bump_generation(dst.quantized_scalers)
     if isinstance(src, NF4Tensor):
         same_meta = (
             src.block_size == dst.block_size
@@ -465,6 +483,7 @@ class _LinearNF4(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, input: torch.Tensor, weight: NF4Tensor):
+        _check_in_features(input, weight)
         ctx.save_for_backward(weight)
         ctx.in_shape = input.shape
         if _fused_ok(input, weight, 0):
@@ -486,6 +505,16 @@ class _LinearNF4(torch.autograd.Function):
                                        transposed=weight.backward_copy())
             return gx.view(ctx.in_shape), None
         return grad_output @ weight.to(grad_output.dtype), None
+
+
+def _check_in_features(x: torch.Tensor, weight: torch.Tensor) -> None:
+    """The shape error ``F.linear`` raises for a dense weight; the fused kernels take K from the activation, so a wrong
+    inner dimension must be stopped on the host."""
+    if weight.dim() == 2 and (x.dim() == 0 or x.shape[-1] != weight.shape[1]):
+        raise RuntimeError(
+            f"mat1 and mat2 shapes cannot be multiplied ({x.numel() // max(x.shape[-1] if x.dim() else 1, 1)}x"
+            f"{x.shape[-1] if x.dim() else 1} and {weight.shape[1]}x{weight.shape[0]})"
+        )
 
 
 def _fused_ok(x: torch.Tensor, weight: NF4Tensor, rank: int) -> bool:

@@ -171,12 +171,36 @@ def _bf16_2d(t: torch.Tensor, what: str) -> torch.Tensor:
     return t.contiguous()
 
 
+def _check_nf4_operands(what: str, N: int, K: int, qdata: torch.Tensor, block_scalers: torch.Tensor,
+                        block_scalers_t: Optional[torch.Tensor] = None) -> None:
+    """The kernels take sizes from the activation and the caller's N; the packed tensors must really hold an [N, K]
+    weight (the C side sees only pointers)."""
+    _need_gpu(qdata, what)
+    if qdata.dtype != torch.uint8 or qdata.numel() * 2 != N * K:
+        raise ValueError(f"{what}: quantized_data holds {qdata.numel() * 2} codes ({qdata.dtype}), the weight is [{N}, {K}]")
+    if block_scalers.dtype != torch.float32 or block_scalers.numel() * 64 != N * K:
+        raise ValueError(f"{what}: block_scalers must be float32 with {N * K // 64} elements, got {block_scalers.numel()} "
+                         f"{block_scalers.dtype}")
+    if block_scalers_t is not None and (block_scalers_t.dtype != torch.float32 or block_scalers_t.numel() * 64 != N * K):
+        raise ValueError(f"{what}: block_scalers_t must be float32 with {N * K // 64} elements")
+
+
+def _check_adapter(what: str, M: int, n_out: int, act: torch.Tensor, weight: torch.Tensor, weight_shape) -> None:
+    rank = act.shape[1]
+    if act.shape[0] != M:
+        raise ValueError(f"{what}: the adapter activation has {act.shape[0]} rows, the input {M}")
+    if tuple(weight.shape) != tuple(weight_shape(rank)):
+        raise ValueError(f"{what}: the adapter weight is {tuple(weight.shape)}, expected {tuple(weight_shape(rank))}")
+
+
 def lora_hidden(x: torch.Tensor, lora_a: torch.Tensor) -> torch.Tensor:
     """h = bf16(x @ lora_a.T);  x [M,K], lora_a [r,K] -> [M,r]"""
     x = _bf16_2d(x, "lora_hidden")
     lora_a = _bf16_2d(lora_a, "lora_hidden")
     M, K = x.shape
     r = lora_a.shape[0]
+    if lora_a.shape[1] != K:
+        raise ValueError(f"lora_hidden: x has {K} columns, lora_a {lora_a.shape[1]}")
     lib = _lib.load()
     h = torch.empty(M, r, dtype=torch.bfloat16, device=x.device)
     ws = _workspace(lib.ttamd_lora_fwd_workspace_bytes(M, K, r), x.device)
@@ -204,15 +228,21 @@ def nf4_lora_linear_fwd(
     ([K/64, N] fp32, second tensor of ``nf4_transpose_for_backward``): same result, cheaper scaler loads."""
     x = _bf16_2d(x, "nf4_lora_linear_fwd")
     M, K = x.shape
+    _check_nf4_operands("nf4_lora_linear_fwd", N, K, qdata, block_scalers, block_scalers_t)
     rank = 0
     if h is not None:
         h = _bf16_2d(h, "nf4_lora_linear_fwd")
         lora_b = _bf16_2d(lora_b, "nf4_lora_linear_fwd")
         rank = h.shape[1]
+        _check_adapter("nf4_lora_linear_fwd", M, N, h, lora_b, lambda r: (N, r))
     if bias is not None:
         bias = bias.contiguous()
         if bias.dtype != torch.bfloat16:
             raise TypeError("nf4_lora_linear_fwd: bias must be bfloat16")
+        if bias.numel() != N:
+            raise ValueError(f"nf4_lora_linear_fwd: bias has {bias.numel()} elements, the layer {N} outputs")
+    if col_scale is not None and col_scale.numel() != N:
+        raise ValueError(f"nf4_lora_linear_fwd: col_scale has {col_scale.numel()} elements, the layer {N} outputs")
     y = torch.empty(M, N, dtype=torch.bfloat16, device=x.device)
     lib = _lib.load()
     ws, ws_bytes = _gemm_workspace(lib, M, N, K, x.device)
@@ -234,7 +264,7 @@ def nf4_lora_linear_fwd(
 
 def nf4_transpose_for_backward(qdata: torch.Tensor, block_scalers: torch.Tensor, N: int, K: int):
     """-> (codes re-packed along N: u8 [K*N/2], block scalers transposed: fp32 [K/64, N])"""
-    _need_gpu(qdata, "nf4_transpose_for_backward")
+    _check_nf4_operands("nf4_transpose_for_backward", N, K, qdata, block_scalers)
     qdata_t = torch.empty(K * N // 2, dtype=torch.uint8, device=qdata.device)
     scal_t = torch.empty(K // 64, N, dtype=torch.float32, device=qdata.device)
     lib = _lib.load()
@@ -253,11 +283,15 @@ def nf4_linear_bwd_dx(
     (fast path) or None (the weight tile is transposed on the fly)."""
     gy = _bf16_2d(gy, "nf4_linear_bwd_dx")
     M, N = gy.shape
+    _check_nf4_operands("nf4_linear_bwd_dx", N, K, qdata, block_scalers, transposed[1] if transposed else None)
+    if transposed and (transposed[0].dtype != torch.uint8 or transposed[0].numel() * 2 != N * K):
+        raise ValueError(f"nf4_linear_bwd_dx: the transposed codes do not hold a [{N}, {K}] weight")
     rank = 0
     if gh is not None:
         gh = _bf16_2d(gh, "nf4_linear_bwd_dx")
         lora_a = _bf16_2d(lora_a, "nf4_linear_bwd_dx")
         rank = gh.shape[1]
+        _check_adapter("nf4_linear_bwd_dx", M, K, gh, lora_a, lambda r: (r, K))
     gx = torch.empty(M, K, dtype=torch.bfloat16, device=gy.device)
     lib = _lib.load()
     ws, ws_bytes = _gemm_workspace(lib, M, K, N, gy.device) if transposed else (None, 0)
@@ -287,6 +321,9 @@ def lora_bwd(
     M, N = gy.shape
     K = x.shape[1]
     r = h.shape[1]
+    if x.shape[0] != M or h.shape[0] != M or tuple(lora_b.shape) != (N, r):
+        raise ValueError(f"lora_bwd: gy {tuple(gy.shape)}, x {tuple(x.shape)}, h {tuple(h.shape)} and lora_b "
+                         f"{tuple(lora_b.shape)} do not belong to one layer")
     dev = gy.device
     gh = torch.empty(M, r, dtype=torch.bfloat16, device=dev)
     ga = torch.empty(r, K, dtype=torch.bfloat16, device=dev)

@@ -22,6 +22,7 @@ from __future__ import annotations
 from dataclasses import dataclass
 from enum import Enum, auto
 import threading
+import weakref
 from typing import Optional, Union
 
 import torch
@@ -175,20 +176,37 @@ class FakeQuantizer(nn.Module):
                 and config.zero_point_precision == config.scale_precision)
 
     # Sibling linears (q/k/v, gate/up) fake-quantise the very same activation tensor one after the other; the dynamic
-    # per-token result depends on the tensor and the scale precision only, so the last one is kept (per thread, together
-    # with the tensor itself, so that its memory cannot be handed to another tensor meanwhile) and reused while the
-    # same, unmodified tensor object comes in again.  ``share_identical_inputs = False`` recomputes every time.
+    # per-token result depends on the tensor and the scale precision only, so the last one is kept (per thread, with a
+    # weak reference to the tensor: the entry is dropped when the tensor dies, so its address cannot come back as another
+    # tensor's) and reused while the same, unmodified tensor object comes in again.
+    # ``share_identical_inputs = False`` recomputes every time.
     share_identical_inputs = True
     _last = threading.local()
 
     def _per_token(self, x: torch.Tensor):
+        # Inference tensors keep no version counter (reading it raises), so nothing is shared under inference_mode.
+        share = FakeQuantizer.share_identical_inputs and not (torch.is_inference_mode_enabled() or x.is_inference())
+        if not share:
+            FakeQuantizer._last.entry = None
+            return ops.fq_per_token_int8_asym(x.detach(), qparam_dtype=self.config.scale_precision)
         key = (x._version, self.config.scale_precision)
         hit = getattr(FakeQuantizer._last, "entry", None)
-        if FakeQuantizer.share_identical_inputs and hit is not None and hit[0] is x and hit[1] == key:
+        if hit is not None and hit[0]() is x and hit[1] == key:
             return hit[2]
         out = ops.fq_per_token_int8_asym(x.detach(), qparam_dtype=self.config.scale_precision)
-        FakeQuantizer._last.entry = (x, key, out) if FakeQuantizer.share_identical_inputs else None
+        # the input is held by weak reference: the entry dies with the activation instead of keeping it (and its
+        # fake-quantised copy) alive after the step; a new tensor replaces the entry
+        try:
+            FakeQuantizer._last.entry = (weakref.ref(x, FakeQuantizer._drop_entry), key, out)
+        except TypeError:
+            FakeQuantizer._last.entry = None
         return out
+
+    @staticmethod
+    def _drop_entry(_ref) -> None:
+        hit = getattr(FakeQuantizer._last, "entry", None)
+        if hit is not None and hit[0] is _ref:
+            FakeQuantizer._last.entry = None
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         if not self.enabled:
@@ -355,15 +373,14 @@ class Int8DynActInt4WeightQATQuantizer:
     def prepare(self, model: nn.Module, *args, **kwargs) -> nn.Module:
         for name, child in list(model.named_children()):
             if type(child) is nn.Linear and self._eligible(child):
+                # built on the meta device (no second copy of the weight is ever allocated), then handed the original
+                # Parameter objects: values, dtype, requires_grad and identity (optimizer state, tied weights) survive
                 new = Int8DynActInt4WeightQATLinear(
-                    child.in_features, child.out_features, child.bias is not None, device=child.weight.device,
+                    child.in_features, child.out_features, child.bias is not None, device=torch.device("meta"),
                     groupsize=self.groupsize, precision=self.precision, scales_precision=self.scales_precision,
                 )
-                # keep the trained values; cast to the quantizer's precision as the swap in the reference does
-                if child.weight.device != torch.device("meta"):
-                    new.weight = nn.Parameter(child.weight.detach().to(self.precision), requires_grad=child.weight.requires_grad)
-                    if child.bias is not None:
-                        new.bias = nn.Parameter(child.bias.detach().to(self.precision), requires_grad=child.bias.requires_grad)
+                new.weight = child.weight
+                new.bias = child.bias
                 setattr(model, name, new)
             else:
                 self.prepare(child)
@@ -504,11 +521,10 @@ class Int4WeightOnlyQATQuantizer:
             if (type(child) is nn.Linear and child.bias is None
                     and _check_linear_int4_k(child.in_features, self.groupsize, self.inner_k_tiles)):
                 new = Int4WeightOnlyQATLinear(
-                    child.in_features, child.out_features, False, device=child.weight.device, groupsize=self.groupsize,
+                    child.in_features, child.out_features, False, device=torch.device("meta"), groupsize=self.groupsize,
                     inner_k_tiles=self.inner_k_tiles, precision=self.precision, scales_precision=self.scales_precision,
                 )
-                if child.weight.device != torch.device("meta"):
-                    new.weight = nn.Parameter(child.weight.detach().to(self.precision), requires_grad=child.weight.requires_grad)
+                new.weight = child.weight  # the original Parameter: same dtype, same object
                 setattr(model, name, new)
             else:
                 self.prepare(child)
