@@ -130,6 +130,19 @@ int ttamd_lora_hidden_bf16(const void* x, const void* lora_a, void* h, int64_t M
                            size_t workspace_bytes, void* stream);
 
 /*
+ * ttamd_lora_hidden_bf16 for callers that cannot allocate device memory or pass a workspace: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Same
+ * arguments and bit-identical result; the partial sums of a launch that is cut along K go to a device array built
+ * into the library (ttamd_lora_hidden_static_max_bytes() = 2 MiB per GPU, held until the process ends) instead of a
+ * workspace.  Neither call allocates, frees or synchronises.  Returns TTAMD_EWORKSPACE if the shape would need more
+ * than the built-in array (the plan of this build never does for rank <= 64).  All calls on one GPU share that
+ * array: calls that overlap on the same GPU (different streams or threads) race on it and must be serialised by the
+ * caller; calls on different GPUs are independent.  Nothing in the array has to start at zero.
+ */
+size_t ttamd_lora_hidden_static_max_bytes(void);
+int ttamd_lora_hidden_static_bf16(const void* x, const void* lora_a, void* h, int64_t M, int64_t K, int rank, void* stream);
+
+/*
  * y = x . D(W)^T (+ bias) + scale . h . lora_b^T          (lora.py:137-147; nf4_linear.py:67-70 when rank == 0)
  *
  * x [M,K] bf16; quantized_data = NF4 codes of the [N,K] weight (block_size 64); block_scalers from

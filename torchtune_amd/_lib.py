@@ -39,6 +39,8 @@ SIGNATURES = {
     "ttamd_nf4_dequantize_merge_bf16": (_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _int, _f32, _c_void_p, _i64, _i64, _c_void_p]),
     "ttamd_lora_fwd_workspace_bytes": (_size, [_i64, _i64, _int]),
     "ttamd_lora_hidden_bf16": (_int, [_c_void_p, _c_void_p, _c_void_p, _i64, _i64, _int, _c_void_p, _size, _c_void_p]),
+    "ttamd_lora_hidden_static_max_bytes": (_size, []),
+    "ttamd_lora_hidden_static_bf16": (_int, [_c_void_p, _c_void_p, _c_void_p, _i64, _i64, _int, _c_void_p]),
     "ttamd_nf4_lora_linear_fwd_bf16": (
         _int,
         [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _int, _f32, _c_void_p, _c_void_p, _i64, _i64, _i64,

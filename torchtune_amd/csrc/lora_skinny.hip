@@ -521,6 +521,53 @@ extern "C" int ttamd_lora_hidden_bf16(const void* x, const void* lora_a, void* h
                 reinterpret_cast<uint16_t*>(h), reinterpret_cast<float*>(workspace), reinterpret_cast<hipStream_t>(stream));
 }
 
+// ---- the same product for callers that cannot allocate ---------------------------------------------------------------
+// Partial sums of a launch that is cut along K live in this file-scope device array instead of a caller's workspace.
+// Every GPU the library runs on holds its own copy until the process ends.  The plan never needs more: with fewer than
+// 256 row tiles it uses at most 256 / row_tiles slices of 32 * row_tiles rows, i.e. at most 8192 partial rows of at most
+// 64 fp32 values, and with 256 row tiles or more it writes the result directly.
+constexpr size_t kStaticScratchBytes = size_t(2) << 20;
+static __device__ __align__(256) unsigned char g_hidden_scratch[kStaticScratchBytes];
+
+namespace {
+// Device address of g_hidden_scratch on the current device.  In host code the array's name is only a handle for the
+// runtime, not a device address: the address is asked for once per device (with that device current) and kept.
+int static_scratch(float** out) {
+  static void* ptr[64] = {};
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(TTAMD_ELAUNCH, "lora_hidden_static: hipGetDevice: %s", hipGetErrorString(e));
+  void* p = (dev >= 0 && dev < 64) ? ptr[dev] : nullptr;
+  if (p == nullptr) {
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(g_hidden_scratch));
+    if (e != hipSuccess || p == nullptr)
+      return fail(TTAMD_ELAUNCH, "lora_hidden_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+    if (dev >= 0 && dev < 64) ptr[dev] = p;  // a race between threads stores the same value twice
+  }
+  *out = reinterpret_cast<float*>(p);
+  return TTAMD_OK;
+}
+}  // namespace
+
+extern "C" size_t ttamd_lora_hidden_static_max_bytes(void) { return kStaticScratchBytes; }
+
+extern "C" int ttamd_lora_hidden_static_bf16(const void* x, const void* lora_a, void* h, int64_t M, int64_t K, int rank,
+                                             void* stream) {
+  if (int rc = check_skinny("lora_hidden_static", M, 64, K, rank)) return rc;
+  TT_REQUIRE(x && lora_a && h, "lora_hidden_static: null pointer argument");
+  TT_REQUIRE(aligned16(x) && aligned16(lora_a), "lora_hidden_static: pointers must be 16-byte aligned");
+  const size_t need = plan_nt(M, K).splits > 1 ? nt_ws_bytes(M, K, rank) : 0;  // one slice writes the result directly
+  if (need > kStaticScratchBytes)
+    return fail(TTAMD_EWORKSPACE, "lora_hidden_static: M=%lld K=%lld rank=%d needs %zu bytes of partial sums, the built-in "
+                "scratch holds %zu; use ttamd_lora_hidden_bf16 with a workspace", (long long)M, (long long)K, rank, need,
+                kStaticScratchBytes);
+  float* scratch = nullptr;
+  if (int rc = static_scratch(&scratch)) return rc;
+  // every partial sum the reduction reads is written by this call's first kernel: nothing has to start at zero
+  return run_nt(reinterpret_cast<const uint16_t*>(x), reinterpret_cast<const uint16_t*>(lora_a), false, M, K, rank, 1.0f,
+                reinterpret_cast<uint16_t*>(h), scratch, reinterpret_cast<hipStream_t>(stream));
+}
+
 extern "C" size_t ttamd_lora_bwd_workspace_bytes(int64_t M, int64_t N, int64_t K, int rank) {
   if (M <= 0 || N <= 0 || K <= 0 || rank <= 0 || K % 64 || N % 64) return 0;
   const size_t a = nt_ws_bytes(M, N, rank), b = tn_pair_ws_bytes(M, K, N, rank);
