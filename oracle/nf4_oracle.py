@@ -87,7 +87,12 @@ def order_independent_mean(absmax: torch.Tensor) -> torch.Tensor:
     return (s / absmax.numel()).to(torch.float32).to(absmax.dtype)
 
 
-def nf4_quantize(tensor: torch.Tensor, block_size: int = 64, scaler_block_size: int = 256) -> NF4Parts:
+def nf4_quantize(tensor: torch.Tensor, block_size: int = 64, scaler_block_size: int = 256,
+                 mean: torch.Tensor | None = None) -> NF4Parts:
+    """``mean``: the scaler mean to use instead of this tensor's own.  The mean is the only quantity of the algorithm
+    that couples distant parts of a tensor, so a slice of whole scaler blocks of a large tensor quantises, given the
+    large tensor's mean, to exactly the corresponding slice of the large tensor's parts (how the tests check tensors too
+    large for an eager CPU pass)."""
     assert tensor.dim() <= 2, "NF4 supports at most 2-D tensors"
     assert tensor.is_contiguous()
     assert tensor.dtype in (torch.bfloat16, torch.float32)
@@ -104,7 +109,7 @@ def nf4_quantize(tensor: torch.Tensor, block_size: int = 64, scaler_block_size: 
     absmax = blocks.abs().max(dim=1).values  # [n_blocks], dtype
 
     # double quantisation of the block scalers
-    mean = order_independent_mean(absmax)
+    mean = order_independent_mean(absmax) if mean is None else mean.detach().cpu().to(dtype).reshape(())
     centred = absmax - mean
     n_sb = n_blocks // scaler_block_size
     centred_sb = centred.view(n_sb, scaler_block_size)
