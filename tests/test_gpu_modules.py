@@ -261,3 +261,31 @@ def test_write_through_an_alias_invalidates_the_derived_caches():
         torch.testing.assert_close(y.detach().cpu().float(), yo.detach().float(), rtol=1e-2, atol=2e-2)
         gx = xo.grad.float()
         torch.testing.assert_close(xd.grad.cpu().float(), gx, rtol=1e-2, atol=2e-2 * max(1.0, float(gx.abs().max()) / 8))  # the oracle's own backward rounds to bf16 after every op
+
+
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+def test_low_ram_state_dict_hook_matches_the_ordinary_hook(out_dtype, monkeypatch):
+    """torchtune/modules/common_utils.py:136-237: with the low-host-RAM switch on, the checkpoint of a QLoRA layer holds
+    the same dense values (bit for bit) as the ordinary hook's, in one file-backed mapping on the CPU, and loads back into
+    an NF4 layer."""
+    from torchtune_amd.modules import common_utils
+
+    layer = _qlora(True, torch.bfloat16)
+    want = {"weight": layer.weight.detach(), "bias": layer.bias.detach(), "lora_a.weight": layer.lora_a.weight.detach(),
+            "lora_b.weight": layer.lora_b.weight.detach()}
+    reparametrize_as_dtype_state_dict_post_hook(layer, want, dtype=out_dtype, offload_to_cpu=True)
+    monkeypatch.setattr(common_utils, "_use_low_cpu_ram", True)
+    common_utils._register_reparametrize_state_dict_hooks(layer, dtype=out_dtype, offload_to_cpu=True)
+    sd = layer.state_dict()
+    assert set(sd) == set(want)
+    storages = {v.untyped_storage().data_ptr() for v in sd.values()}
+    assert len(storages) == 1
+    for k, v in sd.items():
+        assert v.device.type == "cpu" and not isinstance(v, NF4Tensor) and v.dtype == want[k].dtype
+        assert torch.equal(v, want[k].cpu()), k
+    assert sd["weight"].dtype == out_dtype
+    reload = _qlora(True, torch.bfloat16)
+    with torch.no_grad():
+        reload.weight.copy_(torch.zeros(512, 512, dtype=torch.bfloat16, device=DEV))
+    reload.load_state_dict(sd)
+    assert torch.equal(reload.weight.quantized_data, layer.weight.quantized_data)

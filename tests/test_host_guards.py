@@ -171,3 +171,34 @@ def test_get_merged_lora_ckpt_binds_like_the_reference_call():
     assert not sd["m.weight"].is_cuda
     with pytest.raises(TypeError):
         get_merged_lora_ckpt(sd, 2, 4.0, False, True)  # offload_to_cpu is keyword-only
+
+
+def test_low_ram_state_dict_hook_puts_every_entry_in_one_shared_mapping(monkeypatch):
+    """The switch and the contract of torchtune/modules/common_utils.py:136-237 on a model without NF4 entries (those
+    need the GPU): values and dtypes unchanged, every tensor a CPU tensor over the same file-backed storage, no file
+    left behind, and the ordinary hook when the switch is off."""
+    import glob
+    import tempfile
+
+    from torchtune_amd.modules import common_utils
+
+    model = nn.Sequential(nn.Linear(8, 4), nn.Linear(4, 2, bias=False).to(torch.bfloat16))
+    want = {k: v.detach().clone() for k, v in model.state_dict().items()}
+    monkeypatch.setattr(common_utils, "_use_low_cpu_ram", True)
+    common_utils._register_reparametrize_state_dict_hooks(model, dtype=torch.bfloat16, offload_to_cpu=True)
+    sd = model.state_dict()
+    assert list(sd) == list(want)
+    storages = set()
+    for k, v in sd.items():
+        assert v.device.type == "cpu" and v.dtype == want[k].dtype and torch.equal(v, want[k])
+        storages.add(v.untyped_storage().data_ptr())
+    assert len(storages) == 1  # one mapping
+    assert not glob.glob(tempfile.gettempdir() + "/torchtune_amd_state_dict_*")
+    # the entries are copies: writing to the model does not change the checkpoint
+    with torch.no_grad():
+        model[0].weight.add_(1.0)
+    assert torch.equal(sd["0.weight"], want["0.weight"])
+    monkeypatch.setattr(common_utils, "_use_low_cpu_ram", False)
+    plain = nn.Linear(8, 4)
+    common_utils._register_reparametrize_state_dict_hooks(plain)
+    assert plain.state_dict()["weight"].data_ptr() == plain.weight.data_ptr()  # the ordinary hook leaves dense entries alone
