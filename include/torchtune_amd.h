@@ -320,6 +320,40 @@ int ttamd_quantize_per_group_uint4(const void* w, int dtype, int64_t rows, int64
 int ttamd_dequantize_per_group_uint4(const uint8_t* q, const float* scale, const float* zero_point, int dtype, int64_t rows,
                                      int64_t K, int group_size, void* out, void* stream);
 
+/*
+ * Conventions of the fake-quant schemes that differ between versions of the third-party package the reference takes
+ * them from (torchao; the reference pins no version).  The plain entry points above use the defaults below; the `_conv`
+ * variants take the same arguments plus a pointer to this struct (NULL = defaults), so a deployment that pins another
+ * convention needs no other kernel:
+ *   eps_per_token            lower bound of the per-token int8 scale.  Default finfo(float32).eps = 2^-23.
+ *   eps_per_group_sym        lower bound of the per-group symmetric int4 scale.  Default 2^-23; a version that takes
+ *                            eps from the weight dtype uses finfo(bfloat16).eps = 2^-7 for bf16 weights.
+ *   min_scale_uint4          lower bound in the weight-only uint4 scheme.  Default 1e-6.
+ *   uint4_clamp_range_first  0 (default): scale = max((max - min) / 15, min_scale_uint4);
+ *                            1: scale = max(max - min, min_scale_uint4) / 15.
+ * All bounds must be positive.
+ */
+typedef struct ttamd_fq_conventions {
+  float eps_per_token;
+  float eps_per_group_sym;
+  float min_scale_uint4;
+  int uint4_clamp_range_first;
+} ttamd_fq_conventions;
+
+int ttamd_fq_per_token_int8_asym_conv(const void* x, int dtype, int64_t rows, int64_t K, int qparam_dtype, void* out, float* scale,
+                                      int32_t* zero_point, const ttamd_fq_conventions* conventions, void* stream);
+int ttamd_fq_per_group_int4_sym_conv(const void* w, int dtype, int64_t rows, int64_t K, int group_size, int qparam_dtype,
+                                     void* out, float* scale, const ttamd_fq_conventions* conventions, void* stream);
+int ttamd_quantize_per_group_int4_conv(const void* w, int dtype, int64_t rows, int64_t K, int group_size, int qparam_dtype,
+                                       int8_t* q, float* scale, float* zero_point, const ttamd_fq_conventions* conventions,
+                                       void* stream);
+int ttamd_fq_per_group_uint4_asym_conv(const void* w, int dtype, int64_t rows, int64_t K, int group_size, int qparam_dtype,
+                                       void* out, float* scale, float* zero_point, const ttamd_fq_conventions* conventions,
+                                       void* stream);
+int ttamd_quantize_per_group_uint4_conv(const void* w, int dtype, int64_t rows, int64_t K, int group_size, int qparam_dtype,
+                                        uint8_t* q, float* scale, float* zero_point, const ttamd_fq_conventions* conventions,
+                                        void* stream);
+
 /* ------------------------------------------------------------------------------------------------
  * Neighbours of the quantized linears inside a decoder layer (one pass over HBM each, bf16 tensors, fp32 math).
  * Floating-point kernels: results agree with the eager sequences to a tolerance (summation order and hardware

@@ -41,7 +41,7 @@ import torch.nn.functional as F
 _EPS = torch.finfo(torch.float32).eps
 
 
-def choose_qparams_per_token_asym(x: torch.Tensor):
+def choose_qparams_per_token_asym(x: torch.Tensor, eps: float = None):
     """int8 asymmetric qparams for each row of the last dimension -> (scale fp32 [...,1], zero_point int32 [...,1])."""
     qmin, qmax = -128, 127
     xf = x.to(torch.float32)
@@ -50,7 +50,7 @@ def choose_qparams_per_token_asym(x: torch.Tensor):
     mn_neg = torch.min(mn, torch.zeros_like(mn))
     mx_pos = torch.max(mx, torch.zeros_like(mx))
     scale = (mx_pos - mn_neg) / float(qmax - qmin)
-    scale = scale.clamp(min=_EPS)
+    scale = scale.clamp(min=_EPS if eps is None else eps)
     descaled_min = mn_neg / scale
     descaled_max = mx_pos / scale
     zp_from_min_err = qmin + descaled_min
@@ -72,16 +72,16 @@ def _to_scale_precision(scale: torch.Tensor, scale_dtype: torch.dtype) -> torch.
     return scale.to(scale_dtype).to(torch.float32)
 
 
-def fq_per_token_int8_asym(x: torch.Tensor, scale_dtype: torch.dtype = torch.float32):
+def fq_per_token_int8_asym(x: torch.Tensor, scale_dtype: torch.dtype = torch.float32, eps: float = None):
     """returns (fake-quantised x, scale [rows] fp32, zero_point [rows] int32); with ``scale_dtype=bfloat16`` the scale is
     rounded to bf16 after the zero point has been chosen, and the rounded scale quantises and dequantises"""
-    scale, zp = choose_qparams_per_token_asym(x)
+    scale, zp = choose_qparams_per_token_asym(x, eps)
     scale = _to_scale_precision(scale, scale_dtype)
     _, dq = _fake_quantize(x, scale, zp, -128, 127)
     return dq, scale.reshape(-1), zp.reshape(-1)
 
 
-def choose_qparams_per_group_sym(w: torch.Tensor, group_size: int):
+def choose_qparams_per_group_sym(w: torch.Tensor, group_size: int, eps: float = None):
     """int4 symmetric qparams per group of `group_size` along the last dim -> scale fp32 [rows, K/g]."""
     qmin, qmax = -8, 7
     rows, K = w.shape
@@ -92,40 +92,45 @@ def choose_qparams_per_group_sym(w: torch.Tensor, group_size: int):
     mx_pos = torch.max(mx, torch.zeros_like(mx))
     amax = torch.max(-mn_neg, mx_pos)
     scale = amax / (float(qmax - qmin) / 2)
-    return scale.clamp(min=_EPS)
+    return scale.clamp(min=_EPS if eps is None else eps)
 
 
-def fq_per_group_int4_sym(w: torch.Tensor, group_size: int, scale_dtype: torch.dtype = torch.float32):
+def fq_per_group_int4_sym(w: torch.Tensor, group_size: int, scale_dtype: torch.dtype = torch.float32, eps: float = None):
     """returns (fake-quantised w, scale [rows, K/g] fp32)"""
     rows, K = w.shape
-    scale = _to_scale_precision(choose_qparams_per_group_sym(w, group_size), scale_dtype)
+    scale = _to_scale_precision(choose_qparams_per_group_sym(w, group_size, eps), scale_dtype)
     wg = w.view(rows, K // group_size, group_size)
     zp = torch.zeros_like(scale, dtype=torch.int32)
     _, dq = _fake_quantize(wg, scale[..., None], zp[..., None], -8, 7)
     return dq.reshape(rows, K), scale
 
 
-def quantize_per_group_int4(w: torch.Tensor, group_size: int, scale_dtype: torch.dtype = torch.float32):
+def quantize_per_group_int4(w: torch.Tensor, group_size: int, scale_dtype: torch.dtype = torch.float32, eps: float = None):
     """convert(): returns (int8 tensor of int4 values [rows,K], scale [rows,K/g] fp32, zeros [rows,K/g] fp32)"""
     rows, K = w.shape
-    scale = _to_scale_precision(choose_qparams_per_group_sym(w, group_size), scale_dtype)
+    scale = _to_scale_precision(choose_qparams_per_group_sym(w, group_size, eps), scale_dtype)
     wg = w.view(rows, K // group_size, group_size)
     q = torch.clamp(torch.round(wg * (1.0 / scale[..., None])), -8, 7).to(torch.int8)
     return q.reshape(rows, K), scale, torch.zeros_like(scale)
 
 
 # ---- weight-only int4 ("4w-qat": asymmetric uint4 with a floating-point zero point) --------------------------
-def choose_qparams_per_group_uint4_asym(w: torch.Tensor, group_size: int, qparam_dtype: torch.dtype = torch.bfloat16):
+def choose_qparams_per_group_uint4_asym(w: torch.Tensor, group_size: int, qparam_dtype: torch.dtype = torch.bfloat16,
+                                        min_scale: float = 1e-6, clamp_range_first: bool = False):
     """Group-wise affine qparams of the weight-only int4 scheme, computed op by op in the dtype of ``w`` (the
     eager sequence rounds after every operation) and then cast to ``qparam_dtype``:
     ``scale = clamp((max - min) / 15, 1e-6)``, ``zero_point = min + scale * 8``.  The group extrema are NOT widened
-    to include 0.  -> (scale, zero_point), each [rows, K/g] in ``qparam_dtype``."""
+    to include 0.  -> (scale, zero_point), each [rows, K/g] in ``qparam_dtype``.
+    ``clamp_range_first``: the other order found among versions of the scheme, ``scale = clamp(max - min, min_scale) / 15``."""
     rows, K = w.shape
     g = w.view(rows, K // group_size, group_size)
     mn = torch.amin(g, dim=-1)
     mx = torch.amax(g, dim=-1)
-    scale = (mx - mn) / 15.0
-    scale = torch.clamp(scale, min=1e-6)
+    if clamp_range_first:
+        scale = torch.clamp(mx - mn, min=min_scale) / 15.0
+    else:
+        scale = (mx - mn) / 15.0
+        scale = torch.clamp(scale, min=min_scale)
     zero = mn + scale * 8.0
     return scale.to(qparam_dtype), zero.to(qparam_dtype)
 
@@ -139,20 +144,22 @@ def _uint4_codes(w: torch.Tensor, scale: torch.Tensor, zero: torch.Tensor, group
     return torch.clamp(torch.round((g - lowest) / sc), 0, 15)
 
 
-def fq_per_group_uint4_asym(w: torch.Tensor, group_size: int, qparam_dtype: torch.dtype = torch.bfloat16):
+def fq_per_group_uint4_asym(w: torch.Tensor, group_size: int, qparam_dtype: torch.dtype = torch.bfloat16,
+                            min_scale: float = 1e-6, clamp_range_first: bool = False):
     """returns (fake-quantised w, scale [rows, K/g], zero_point [rows, K/g]) — qparams in ``qparam_dtype``."""
     rows, K = w.shape
-    scale, zero = choose_qparams_per_group_uint4_asym(w, group_size, qparam_dtype)
+    scale, zero = choose_qparams_per_group_uint4_asym(w, group_size, qparam_dtype, min_scale, clamp_range_first)
     q = _uint4_codes(w, scale, zero, group_size)
     dq = (q - 8.0) * scale.to(w.dtype)[..., None]
     dq = dq + zero.to(w.dtype)[..., None]
     return dq.reshape(rows, K), scale, zero
 
 
-def quantize_per_group_uint4(w: torch.Tensor, group_size: int, qparam_dtype: torch.dtype = torch.bfloat16):
+def quantize_per_group_uint4(w: torch.Tensor, group_size: int, qparam_dtype: torch.dtype = torch.bfloat16,
+                             min_scale: float = 1e-6, clamp_range_first: bool = False):
     """convert() of the weight-only scheme: (uint8 [rows, K/2], even element in the high nibble; scale; zero_point)."""
     rows, K = w.shape
-    scale, zero = choose_qparams_per_group_uint4_asym(w, group_size, qparam_dtype)
+    scale, zero = choose_qparams_per_group_uint4_asym(w, group_size, qparam_dtype, min_scale, clamp_range_first)
     q = _uint4_codes(w, scale, zero, group_size).reshape(rows, K).to(torch.uint8)
     return (q[:, ::2] << 4) | q[:, 1::2], scale, zero
 

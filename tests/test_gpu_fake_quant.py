@@ -445,3 +445,47 @@ def test_prepare_with_default_quantizer_arguments_runs_a_bf16_model():
     with torch.inference_mode():  # evaluation / generation loops run under inference_mode
         yi = model(x.to(DEV))
     torch.testing.assert_close(yi.cpu().float(), yo.detach().float(), rtol=1e-2, atol=1e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_version_dependent_conventions_are_parameters(dtype):
+    """The constants on which versions of the reference's quantisation package differ (the lower bound of each scale, and
+    whether the weight-only uint4 scheme bounds the range or the quotient) are arguments of the `_conv` entry points and
+    of the oracle; with any setting the kernels stay bit-exact against the oracle, and the defaults are unchanged."""
+    g = torch.Generator().manual_seed(17)
+    w = (torch.randn(96, 1024, generator=g) * 0.02).to(dtype)
+    w[3] *= 1e-4   # groups whose scale falls under the larger bounds
+    w[5] = 0
+    bf16_eps = float(torch.finfo(torch.bfloat16).eps)  # the bound a version that takes eps from a bf16 weight would use
+    for eps in (None, bf16_eps, 1e-5):
+        fqd, sd = ops.fq_per_group_int4_sym(w.to(DEV), 32, eps=eps)
+        fo, so = fq.fq_per_group_int4_sym(w, 32, eps=eps)
+        assert bits_equal(fqd.cpu(), fo) and bits_equal(sd.cpu(), so), eps
+        q, s, z = ops.quantize_per_group_int4(w.to(DEV), 32, eps=eps)
+        qo, so2, zo = fq.quantize_per_group_int4(w, 32, eps=eps)
+        assert torch.equal(q.cpu(), qo) and bits_equal(s.cpu(), so2), eps
+    # with the bf16 bound most groups of an N(0, 0.02) weight sit on the bound: the setting matters
+    assert float((ops.fq_per_group_int4_sym(w.to(DEV), 32, eps=bf16_eps)[1] == bf16_eps).float().mean()) > 0.5
+    x = (torch.randn(40, 512, generator=g) * 1.5).to(dtype)
+    x[1] *= 1e-5
+    x[2] = 0
+    for eps in (None, 1e-3, bf16_eps):
+        od, sd, zd = ops.fq_per_token_int8_asym(x.to(DEV), eps=eps)
+        oo, so, zo = fq.fq_per_token_int8_asym(x, eps=eps)
+        assert bits_equal(od.cpu(), oo) and bits_equal(sd.cpu(), so) and torch.equal(zd.cpu(), zo), eps
+    u = (torch.randn(64, 512, generator=g) * 0.02).to(dtype)
+    u[7] = u[7, 0]            # constant groups: range 0, the bound decides the scale
+    u[9] = u[9] * 1e-5
+    for min_scale, first in ((1e-6, False), (1e-6, True), (1e-3, False), (1e-3, True), (3e-7, True)):
+        od, sd, zd = ops.fq_per_group_uint4_asym(u.to(DEV), 64, torch.bfloat16, min_scale=min_scale, clamp_range_first=first)
+        oo, so, zo = fq.fq_per_group_uint4_asym(u, 64, torch.bfloat16, min_scale=min_scale, clamp_range_first=first)
+        assert bits_equal(od.cpu(), oo), (min_scale, first)
+        assert bits_equal(sd.cpu(), so.float()) and bits_equal(zd.cpu(), zo.float()), (min_scale, first)
+        qd, _, _ = ops.quantize_per_group_uint4(u.to(DEV), 64, torch.bfloat16, min_scale=min_scale, clamp_range_first=first)
+        qo, _, _ = fq.quantize_per_group_uint4(u, 64, torch.bfloat16, min_scale=min_scale, clamp_range_first=first)
+        assert torch.equal(qd.cpu(), qo), (min_scale, first)
+    # the config carries eps to the kernels
+    cfg = FakeQuantizeConfig(torch.int4, group_size=32, is_symmetric=True, eps=bf16_eps)
+    fqz = FakeQuantizer(cfg)
+    out = fqz(w.to(DEV))
+    assert bits_equal(out.cpu(), fq.fq_per_group_int4_sym(w, 32, eps=bf16_eps)[0])

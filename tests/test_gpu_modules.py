@@ -270,7 +270,8 @@ def test_low_ram_state_dict_hook_matches_the_ordinary_hook(out_dtype, monkeypatc
     an NF4 layer."""
     from torchtune_amd.modules import common_utils
 
-    layer = _qlora(True, torch.bfloat16)
+    with _default_dtype(torch.bfloat16), torch.device(DEV):  # random init: no all-zero blocks, so requantisation is exact
+        layer = LoRALinear(512, 512, rank=4, alpha=1.0, use_bias=True, quantize_base=True)
     want = {"weight": layer.weight.detach(), "bias": layer.bias.detach(), "lora_a.weight": layer.lora_a.weight.detach(),
             "lora_b.weight": layer.lora_b.weight.detach()}
     reparametrize_as_dtype_state_dict_post_hook(layer, want, dtype=out_dtype, offload_to_cpu=True)
@@ -284,8 +285,8 @@ def test_low_ram_state_dict_hook_matches_the_ordinary_hook(out_dtype, monkeypatc
         assert v.device.type == "cpu" and not isinstance(v, NF4Tensor) and v.dtype == want[k].dtype
         assert torch.equal(v, want[k].cpu()), k
     assert sd["weight"].dtype == out_dtype
-    reload = _qlora(True, torch.bfloat16)
-    with torch.no_grad():
-        reload.weight.copy_(torch.zeros(512, 512, dtype=torch.bfloat16, device=DEV))
+    with _default_dtype(torch.bfloat16), torch.device(DEV):
+        reload = LoRALinear(512, 512, rank=4, alpha=1.0, use_bias=True, quantize_base=True)
+    assert not torch.equal(reload.weight.quantized_data, layer.weight.quantized_data)
     reload.load_state_dict(sd)
     assert torch.equal(reload.weight.quantized_data, layer.weight.quantized_data)

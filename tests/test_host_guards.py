@@ -112,7 +112,7 @@ def test_fake_quantizer_under_inference_mode_and_cache_lifetime(monkeypatch):
     must not keep an activation alive once the caller has dropped it."""
     calls = []
 
-    def fake_kernel(x, want_qparams=True, qparam_dtype=torch.float32):
+    def fake_kernel(x, want_qparams=True, qparam_dtype=torch.float32, eps=None):
         calls.append(x.shape)
         return x.clone(), torch.ones(x.shape[0]), torch.zeros(x.shape[0], dtype=torch.int32)
 

@@ -97,6 +97,16 @@ SIGNATURES = {
     "ttamd_quantize_per_group_uint4": (
         _int, [_c_void_p, _int, _i64, _i64, _int, _int, _c_void_p, _c_void_p, _c_void_p, _c_void_p]),
     "ttamd_dequantize_per_group_uint4": (_int, [_c_void_p, _c_void_p, _c_void_p, _int, _i64, _i64, _int, _c_void_p, _c_void_p]),
+    "ttamd_fq_per_token_int8_asym_conv": (
+        _int, [_c_void_p, _int, _i64, _i64, _int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p]),
+    "ttamd_fq_per_group_int4_sym_conv": (
+        _int, [_c_void_p, _int, _i64, _i64, _int, _int, _c_void_p, _c_void_p, _c_void_p, _c_void_p]),
+    "ttamd_quantize_per_group_int4_conv": (
+        _int, [_c_void_p, _int, _i64, _i64, _int, _int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p]),
+    "ttamd_fq_per_group_uint4_asym_conv": (
+        _int, [_c_void_p, _int, _i64, _i64, _int, _int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p]),
+    "ttamd_quantize_per_group_uint4_conv": (
+        _int, [_c_void_p, _int, _i64, _i64, _int, _int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p]),
     "ttamd_rms_norm_fwd_bf16": (_int, [_c_void_p, _c_void_p, _f32, _c_void_p, _c_void_p, _i64, _i64, _c_void_p]),
     "ttamd_rms_norm_bwd_workspace_bytes": (_size, [_i64]),
     "ttamd_rms_norm_bwd_bf16": (
@@ -110,6 +120,13 @@ SIGNATURES = {
     "ttamd_cross_entropy_fwd_bwd_bf16": (_int, [_c_void_p, _c_void_p, _i64, _f32, _c_void_p, _c_void_p, _i64, _i64, _c_void_p]),
     "ttamd_swiglu_bwd_bf16": (_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _i64, _c_void_p]),
 }
+
+class FqConventions(ctypes.Structure):
+    """``ttamd_fq_conventions`` of the header: the version-dependent constants of the fake-quant schemes."""
+
+    _fields_ = [("eps_per_token", ctypes.c_float), ("eps_per_group_sym", ctypes.c_float), ("min_scale_uint4", ctypes.c_float),
+                ("uint4_clamp_range_first", ctypes.c_int)]
+
 
 _lock = threading.Lock()
 _lib = None

@@ -77,10 +77,10 @@ struct TokenQParams {
 // asymmetric int8 qparams from the row extrema (already widened to include 0)
 // (the zero point is chosen with the fp32 scale; a bf16 qparam precision rounds the scale afterwards, and the rounded
 // scale is what quantises and dequantises)
-__device__ __forceinline__ TokenQParams token_qparams(float mn, float mx, bool qp_bf16) {
+__device__ __forceinline__ TokenQParams token_qparams(float mn, float mx, bool qp_bf16, float eps) {
   TokenQParams p;
   float scale = (mx - mn) / 255.0f;
-  scale = scale > kF32Eps ? scale : kF32Eps;
+  scale = scale > eps ? scale : eps;
   const float dmin = mn / scale, dmax = mx / scale;
   float zp = ((-128.0f + dmin) + (127.0f + dmax) > 0.0f) ? (-128.0f - dmin) : (127.0f - dmax);
   zp = zp < -128.0f ? -128.0f : (zp > 127.0f ? 127.0f : zp);
@@ -110,7 +110,7 @@ __device__ __forceinline__ void wave_minmax(float& mn, float& mx) {
 template <bool BF16, int NV>
 __global__ __launch_bounds__(256) void fq_per_token_regs_kernel(const void* __restrict__ x, int64_t rows, int64_t K,
                                                                 void* __restrict__ out, float* __restrict__ scale_out,
-                                                                int32_t* __restrict__ zp_out, bool qp_bf16) {
+                                                                int32_t* __restrict__ zp_out, bool qp_bf16, float eps) {
   const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= rows) return;
   const int lane = threadIdx.x & 63;
@@ -135,7 +135,7 @@ __global__ __launch_bounds__(256) void fq_per_token_regs_kernel(const void* __re
       mx = fmaxf(mx, v);
     }
   wave_minmax(mn, mx);
-  const TokenQParams p = token_qparams(mn, mx, qp_bf16);
+  const TokenQParams p = token_qparams(mn, mx, qp_bf16, eps);
   if (lane == 0) {
     if (scale_out) scale_out[row] = p.scale;
     if (zp_out) zp_out[row] = (int32_t)p.zp;
@@ -156,7 +156,7 @@ __global__ __launch_bounds__(256) void fq_per_token_regs_kernel(const void* __re
 template <bool BF16>
 __global__ __launch_bounds__(256) void fq_per_token_stream_kernel(const void* __restrict__ x, int64_t rows, int64_t K,
                                                                   void* __restrict__ out, float* __restrict__ scale_out,
-                                                                  int32_t* __restrict__ zp_out, bool qp_bf16) {
+                                                                  int32_t* __restrict__ zp_out, bool qp_bf16, float eps) {
   const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= rows) return;
   const int lane = threadIdx.x & 63;
@@ -174,7 +174,7 @@ __global__ __launch_bounds__(256) void fq_per_token_stream_kernel(const void* __
     }
   }
   wave_minmax(mn, mx);
-  const TokenQParams p = token_qparams(mn, mx, qp_bf16);
+  const TokenQParams p = token_qparams(mn, mx, qp_bf16, eps);
   if (lane == 0) {
     if (scale_out) scale_out[row] = p.scale;
     if (zp_out) zp_out[row] = (int32_t)p.zp;
@@ -197,7 +197,7 @@ template <bool BF16, bool EMIT_INT>
 __global__ __launch_bounds__(256) void fq_per_group_kernel(const void* __restrict__ w, int64_t n_chunks, int lanes_per_group,
                                                            int log2_lpg, void* __restrict__ out_fq,
                                                            int8_t* __restrict__ out_q, float* __restrict__ scale_out,
-                                                           float* __restrict__ zero_out, bool qp_bf16) {
+                                                           float* __restrict__ zero_out, bool qp_bf16, float eps) {
   const int64_t base = (int64_t)blockIdx.x * (256 * kGroupChunksPerThread) + threadIdx.x;
   Chunk8<BF16> c[kGroupChunksPerThread];
 #pragma unroll
@@ -225,7 +225,7 @@ __global__ __launch_bounds__(256) void fq_per_group_kernel(const void* __restric
     if (ch >= n_chunks) continue;
     const float amax = fmaxf(-mn, mx);
     float scale = amax / 7.5f;
-    scale = scale > kF32Eps ? scale : kF32Eps;
+    scale = scale > eps ? scale : eps;
     if (qp_bf16) scale = round_to_bf16(scale);  // the rounded scale quantises and dequantises
     const float inv = 1.0f / scale;
     if ((threadIdx.x & (lanes_per_group - 1)) == 0) {
@@ -263,14 +263,14 @@ int log2_exact(int64_t v) {
 }
 
 template <bool BF16>
-int launch_per_token(const void* x, int64_t rows, int64_t K, void* out, float* scale, int32_t* zp, bool qp_bf16,
+int launch_per_token(const void* x, int64_t rows, int64_t K, void* out, float* scale, int32_t* zp, bool qp_bf16, float eps,
                      hipStream_t s) {
   const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
   const int64_t nv = (K / 8 + kWave - 1) / kWave;
   constexpr int kMaxRegChunks = BF16 ? 32 : 16;
 #define TT_LAUNCH_TOKEN(NV)                                                                          \
   if (nv <= NV) {                                                                                    \
-    fq_per_token_regs_kernel<BF16, NV><<<grid, block, 0, s>>>(x, rows, K, out, scale, zp, qp_bf16);  \
+    fq_per_token_regs_kernel<BF16, NV><<<grid, block, 0, s>>>(x, rows, K, out, scale, zp, qp_bf16, eps);  \
     return check_launch("fq_per_token_int8_asym");                                                   \
   }
   TT_LAUNCH_TOKEN(1)
@@ -282,7 +282,7 @@ int launch_per_token(const void* x, int64_t rows, int64_t K, void* out, float* s
     TT_LAUNCH_TOKEN(32)
   }
 #undef TT_LAUNCH_TOKEN
-  fq_per_token_stream_kernel<BF16><<<grid, block, 0, s>>>(x, rows, K, out, scale, zp, qp_bf16);
+  fq_per_token_stream_kernel<BF16><<<grid, block, 0, s>>>(x, rows, K, out, scale, zp, qp_bf16, eps);
   return check_launch("fq_per_token_int8_asym");
 }
 
@@ -316,7 +316,8 @@ template <bool BF16, bool QP_BF16, bool EMIT_INT>
 __global__ __launch_bounds__(256) void fq_per_group_asym_kernel(const void* __restrict__ w, int64_t n_chunks,
                                                                 int lanes_per_group, int log2_lpg,
                                                                 void* __restrict__ out_fq, uint32_t* __restrict__ out_q,
-                                                                float* __restrict__ scale_out, float* __restrict__ zero_out) {
+                                                                float* __restrict__ scale_out, float* __restrict__ zero_out,
+                                                                float min_scale, bool clamp_range_first) {
   using A = Arith<BF16>;
   using Q = Arith<QP_BF16>;
   const int64_t base = (int64_t)blockIdx.x * (256 * kGroupChunksPerThread) + threadIdx.x;
@@ -344,8 +345,9 @@ __global__ __launch_bounds__(256) void fq_per_group_asym_kernel(const void* __re
       mx = fmaxf(mx, __shfl_xor(mx, off, kWave));
     }
     if (ch >= n_chunks) continue;
-    float scale = A::rnd(A::rnd(mx - mn) / 15.0f);
-    scale = A::rnd(fmaxf(scale, 1e-6f));
+    // default: divide, then clamp the scale; the other order clamps the range (max - min) first
+    float scale = clamp_range_first ? A::rnd(A::rnd(fmaxf(A::rnd(mx - mn), min_scale)) / 15.0f)
+                                    : A::rnd(fmaxf(A::rnd(A::rnd(mx - mn) / 15.0f), min_scale));
     float zero = A::rnd(mn + A::rnd(scale * 8.0f));
     scale = Q::rnd(scale);
     zero = Q::rnd(zero);
@@ -358,7 +360,7 @@ __global__ __launch_bounds__(256) void fq_per_group_asym_kernel(const void* __re
     // For bf16 operands with the divisor >= 2^-20 (the scale is at least 1e-6) and a quotient up to 17 the bf16-rounded
     // result equals that of the correctly rounded division (enumerated over all operand pairs by the test suite);
     // larger quotients clamp to 15 either way.  fp32 tensors keep the exact division.
-    const bool fast = BF16 && scale < __builtin_inff();
+    const bool fast = BF16 && scale < __builtin_inff() && scale >= 9.5367431640625e-07f;  // 2^-20: the proven range
     const float y = 1.0f / scale;
     float q[8];
 #pragma unroll
@@ -413,7 +415,8 @@ __global__ __launch_bounds__(256) void dequant_per_group_uint4_kernel(const uint
 
 template <bool EMIT_INT>
 int launch_group_asym(const void* w, int dtype, int qparam_dtype, int64_t rows, int64_t K, int group_size, void* out_fq,
-                      uint32_t* out_q, float* scale, float* zero, hipStream_t s, const char* what) {
+                      uint32_t* out_q, float* scale, float* zero, const ttamd_fq_conventions& conv, hipStream_t s,
+                      const char* what) {
   const int64_t n_chunks = rows * K / 8;
   const int64_t per_wg = 256 * kGroupChunksPerThread;
   const int64_t grid = (n_chunks + per_wg - 1) / per_wg;
@@ -422,13 +425,17 @@ int launch_group_asym(const void* w, int dtype, int qparam_dtype, int64_t rows, 
   const dim3 g((unsigned)grid), b(256);
   const bool bf = dtype == TTAMD_BF16, qbf = qparam_dtype == TTAMD_BF16;
   if (bf && qbf)
-    fq_per_group_asym_kernel<true, true, EMIT_INT><<<g, b, 0, s>>>(w, n_chunks, lpg, l2, out_fq, out_q, scale, zero);
+    fq_per_group_asym_kernel<true, true, EMIT_INT><<<g, b, 0, s>>>(w, n_chunks, lpg, l2, out_fq, out_q, scale, zero, conv.min_scale_uint4,
+                                                                     conv.uint4_clamp_range_first != 0);
   else if (bf)
-    fq_per_group_asym_kernel<true, false, EMIT_INT><<<g, b, 0, s>>>(w, n_chunks, lpg, l2, out_fq, out_q, scale, zero);
+    fq_per_group_asym_kernel<true, false, EMIT_INT><<<g, b, 0, s>>>(w, n_chunks, lpg, l2, out_fq, out_q, scale, zero, conv.min_scale_uint4,
+                                                                     conv.uint4_clamp_range_first != 0);
   else if (qbf)
-    fq_per_group_asym_kernel<false, true, EMIT_INT><<<g, b, 0, s>>>(w, n_chunks, lpg, l2, out_fq, out_q, scale, zero);
+    fq_per_group_asym_kernel<false, true, EMIT_INT><<<g, b, 0, s>>>(w, n_chunks, lpg, l2, out_fq, out_q, scale, zero, conv.min_scale_uint4,
+                                                                     conv.uint4_clamp_range_first != 0);
   else
-    fq_per_group_asym_kernel<false, false, EMIT_INT><<<g, b, 0, s>>>(w, n_chunks, lpg, l2, out_fq, out_q, scale, zero);
+    fq_per_group_asym_kernel<false, false, EMIT_INT><<<g, b, 0, s>>>(w, n_chunks, lpg, l2, out_fq, out_q, scale, zero, conv.min_scale_uint4,
+                                                                     conv.uint4_clamp_range_first != 0);
   return check_launch(what);
 }
 
@@ -448,8 +455,34 @@ int check_group_args(const void* w, int dtype, int64_t rows, int64_t K, int grou
 
 using namespace ttamd;
 
+namespace {
+// The caller's conventions, or the defaults (what the plain entry points use); validated.
+int resolve_conventions(const ttamd_fq_conventions* in, ttamd_fq_conventions* out, const char* who) {
+  out->eps_per_token = kF32Eps;
+  out->eps_per_group_sym = kF32Eps;
+  out->min_scale_uint4 = 1e-6f;
+  out->uint4_clamp_range_first = 0;
+  if (in != nullptr) {
+    *out = *in;
+    TT_REQUIRE(out->eps_per_token > 0.0f && out->eps_per_group_sym > 0.0f && out->min_scale_uint4 > 0.0f,
+               "%s: the lower bounds of the scales must be positive", who);
+    TT_REQUIRE(out->uint4_clamp_range_first == 0 || out->uint4_clamp_range_first == 1,
+               "%s: uint4_clamp_range_first must be 0 or 1", who);
+  }
+  return TTAMD_OK;
+}
+}  // namespace
+
 extern "C" int ttamd_fq_per_token_int8_asym(const void* x, int dtype, int64_t rows, int64_t K, int qparam_dtype, void* out,
                                             float* scale, int32_t* zero_point, void* stream) {
+  return ttamd_fq_per_token_int8_asym_conv(x, dtype, rows, K, qparam_dtype, out, scale, zero_point, nullptr, stream);
+}
+
+extern "C" int ttamd_fq_per_token_int8_asym_conv(const void* x, int dtype, int64_t rows, int64_t K, int qparam_dtype, void* out,
+                                                 float* scale, int32_t* zero_point, const ttamd_fq_conventions* conventions,
+                                                 void* stream) {
+  ttamd_fq_conventions conv;
+  if (int rc = resolve_conventions(conventions, &conv, "fq_per_token")) return rc;
   TT_REQUIRE(qparam_dtype == TTAMD_BF16 || qparam_dtype == TTAMD_F32, "fq_per_token: unknown qparam dtype code %d", qparam_dtype);
   const bool qbf = qparam_dtype == TTAMD_BF16;
   TT_REQUIRE(dtype == TTAMD_BF16 || dtype == TTAMD_F32, "fq_per_token: unknown dtype code %d", dtype);
@@ -458,12 +491,19 @@ extern "C" int ttamd_fq_per_token_int8_asym(const void* x, int dtype, int64_t ro
              (long long)K);
   TT_REQUIRE((rows + 3) / 4 < (int64_t(1) << 31), "fq_per_token: too many rows for one launch");
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  return dtype == TTAMD_BF16 ? launch_per_token<true>(x, rows, K, out, scale, zero_point, qbf, s)
-                             : launch_per_token<false>(x, rows, K, out, scale, zero_point, qbf, s);
+  return dtype == TTAMD_BF16 ? launch_per_token<true>(x, rows, K, out, scale, zero_point, qbf, conv.eps_per_token, s)
+                             : launch_per_token<false>(x, rows, K, out, scale, zero_point, qbf, conv.eps_per_token, s);
 }
 
 extern "C" int ttamd_fq_per_group_int4_sym(const void* w, int dtype, int64_t rows, int64_t K, int group_size, int qparam_dtype,
                                            void* out, float* scale, void* stream) {
+  return ttamd_fq_per_group_int4_sym_conv(w, dtype, rows, K, group_size, qparam_dtype, out, scale, nullptr, stream);
+}
+
+extern "C" int ttamd_fq_per_group_int4_sym_conv(const void* w, int dtype, int64_t rows, int64_t K, int group_size, int qparam_dtype,
+                                                void* out, float* scale, const ttamd_fq_conventions* conventions, void* stream) {
+  ttamd_fq_conventions conv;
+  if (int rc = resolve_conventions(conventions, &conv, "fq_per_group")) return rc;
   if (int rc = check_group_args(w, dtype, rows, K, group_size)) return rc;
   TT_REQUIRE(qparam_dtype == TTAMD_BF16 || qparam_dtype == TTAMD_F32, "fq_per_group: unknown qparam dtype code %d", qparam_dtype);
   const bool qbf = qparam_dtype == TTAMD_BF16;
@@ -476,15 +516,23 @@ extern "C" int ttamd_fq_per_group_int4_sym(const void* w, int dtype, int64_t row
   const int lpg = group_size / 8;
   if (dtype == TTAMD_BF16)
     fq_per_group_kernel<true, false><<<dim3((unsigned)grid), dim3(256), 0, s>>>(w, n_chunks, lpg, log2_exact(lpg), out,
-                                                                                 nullptr, scale, nullptr, qbf);
+                                                                                 nullptr, scale, nullptr, qbf, conv.eps_per_group_sym);
   else
     fq_per_group_kernel<false, false><<<dim3((unsigned)grid), dim3(256), 0, s>>>(w, n_chunks, lpg, log2_exact(lpg), out,
-                                                                                  nullptr, scale, nullptr, qbf);
+                                                                                  nullptr, scale, nullptr, qbf, conv.eps_per_group_sym);
   return check_launch("fq_per_group_int4_sym");
 }
 
 extern "C" int ttamd_quantize_per_group_int4(const void* w, int dtype, int64_t rows, int64_t K, int group_size,
                                              int qparam_dtype, int8_t* q, float* scale, float* zero_point, void* stream) {
+  return ttamd_quantize_per_group_int4_conv(w, dtype, rows, K, group_size, qparam_dtype, q, scale, zero_point, nullptr, stream);
+}
+
+extern "C" int ttamd_quantize_per_group_int4_conv(const void* w, int dtype, int64_t rows, int64_t K, int group_size,
+                                                  int qparam_dtype, int8_t* q, float* scale, float* zero_point,
+                                                  const ttamd_fq_conventions* conventions, void* stream) {
+  ttamd_fq_conventions conv;
+  if (int rc = resolve_conventions(conventions, &conv, "quantize_per_group_int4")) return rc;
   if (int rc = check_group_args(w, dtype, rows, K, group_size)) return rc;
   TT_REQUIRE(qparam_dtype == TTAMD_BF16 || qparam_dtype == TTAMD_F32, "quantize_per_group_int4: unknown qparam dtype code %d",
              qparam_dtype);
@@ -499,10 +547,10 @@ extern "C" int ttamd_quantize_per_group_int4(const void* w, int dtype, int64_t r
   const int lpg = group_size / 8;
   if (dtype == TTAMD_BF16)
     fq_per_group_kernel<true, true><<<dim3((unsigned)grid), dim3(256), 0, s>>>(w, n_chunks, lpg, log2_exact(lpg), nullptr,
-                                                                                q, scale, zero_point, qbf);
+                                                                                q, scale, zero_point, qbf, conv.eps_per_group_sym);
   else
     fq_per_group_kernel<false, true><<<dim3((unsigned)grid), dim3(256), 0, s>>>(w, n_chunks, lpg, log2_exact(lpg), nullptr,
-                                                                                 q, scale, zero_point, qbf);
+                                                                                 q, scale, zero_point, qbf, conv.eps_per_group_sym);
   return check_launch("quantize_per_group_int4");
 }
 
@@ -529,23 +577,39 @@ extern "C" int ttamd_dequantize_per_group_int4(const int8_t* q, const float* sca
 
 extern "C" int ttamd_fq_per_group_uint4_asym(const void* w, int dtype, int64_t rows, int64_t K, int group_size,
                                              int qparam_dtype, void* out, float* scale, float* zero_point, void* stream) {
+  return ttamd_fq_per_group_uint4_asym_conv(w, dtype, rows, K, group_size, qparam_dtype, out, scale, zero_point, nullptr, stream);
+}
+
+extern "C" int ttamd_fq_per_group_uint4_asym_conv(const void* w, int dtype, int64_t rows, int64_t K, int group_size,
+                                                  int qparam_dtype, void* out, float* scale, float* zero_point,
+                                                  const ttamd_fq_conventions* conventions, void* stream) {
+  ttamd_fq_conventions conv;
+  if (int rc = resolve_conventions(conventions, &conv, "fq_per_group_uint4_asym")) return rc;
   if (int rc = check_group_args(w, dtype, rows, K, group_size)) return rc;
   TT_REQUIRE(qparam_dtype == TTAMD_BF16 || qparam_dtype == TTAMD_F32, "fq_per_group_uint4_asym: unknown qparam dtype code %d",
              qparam_dtype);
   TT_REQUIRE(out && aligned16(out), "fq_per_group_uint4_asym: out must be non-null, 16-byte aligned");
-  return launch_group_asym<false>(w, dtype, qparam_dtype, rows, K, group_size, out, nullptr, scale, zero_point,
+  return launch_group_asym<false>(w, dtype, qparam_dtype, rows, K, group_size, out, nullptr, scale, zero_point, conv,
                                   reinterpret_cast<hipStream_t>(stream), "fq_per_group_uint4_asym");
 }
 
 extern "C" int ttamd_quantize_per_group_uint4(const void* w, int dtype, int64_t rows, int64_t K, int group_size,
                                               int qparam_dtype, uint8_t* q, float* scale, float* zero_point, void* stream) {
+  return ttamd_quantize_per_group_uint4_conv(w, dtype, rows, K, group_size, qparam_dtype, q, scale, zero_point, nullptr, stream);
+}
+
+extern "C" int ttamd_quantize_per_group_uint4_conv(const void* w, int dtype, int64_t rows, int64_t K, int group_size,
+                                                   int qparam_dtype, uint8_t* q, float* scale, float* zero_point,
+                                                   const ttamd_fq_conventions* conventions, void* stream) {
+  ttamd_fq_conventions conv;
+  if (int rc = resolve_conventions(conventions, &conv, "quantize_per_group_uint4")) return rc;
   if (int rc = check_group_args(w, dtype, rows, K, group_size)) return rc;
   TT_REQUIRE(qparam_dtype == TTAMD_BF16 || qparam_dtype == TTAMD_F32, "quantize_per_group_uint4: unknown qparam dtype code %d",
              qparam_dtype);
   TT_REQUIRE(q && scale && zero_point && (reinterpret_cast<uintptr_t>(q) & 3u) == 0,
              "quantize_per_group_uint4: q (4-byte aligned), scale and zero_point must be non-null");
   return launch_group_asym<true>(w, dtype, qparam_dtype, rows, K, group_size, nullptr, reinterpret_cast<uint32_t*>(q), scale,
-                                 zero_point, reinterpret_cast<hipStream_t>(stream), "quantize_per_group_uint4");
+                                 zero_point, conv, reinterpret_cast<hipStream_t>(stream), "quantize_per_group_uint4");
 }
 
 extern "C" int ttamd_dequantize_per_group_uint4(const uint8_t* q, const float* scale, const float* zero_point, int dtype,

@@ -353,9 +353,28 @@ def set_fq_timer(timer) -> None:
     _fq_timer = timer
 
 
-def fq_per_token_int8_asym(x: torch.Tensor, want_qparams: bool = True, qparam_dtype: torch.dtype = torch.float32):
+def _conventions(eps_per_token=None, eps_per_group_sym=None, min_scale_uint4=None, clamp_range_first=False):
+    """The ``ttamd_fq_conventions`` struct for non-default constants, or None (the library's defaults: 2^-23 for both
+    eps, 1e-6 for the uint4 scale, scale clamped after the division by 15)."""
+    if eps_per_token is None and eps_per_group_sym is None and min_scale_uint4 is None and not clamp_range_first:
+        return None
+    import ctypes
+
+    f32eps = float(torch.finfo(torch.float32).eps)
+    c = _lib.FqConventions(
+        f32eps if eps_per_token is None else float(eps_per_token),
+        f32eps if eps_per_group_sym is None else float(eps_per_group_sym),
+        1e-6 if min_scale_uint4 is None else float(min_scale_uint4),
+        int(bool(clamp_range_first)),
+    )
+    return ctypes.byref(c)
+
+
+def fq_per_token_int8_asym(x: torch.Tensor, want_qparams: bool = True, qparam_dtype: torch.dtype = torch.float32,
+                           eps: Optional[float] = None):
     """x [..., K] -> (fake-quantised x, scale fp32 [rows] | None, zero_point int32 [rows] | None).
-    ``qparam_dtype=torch.bfloat16`` rounds the scale to bf16 before it quantises and dequantises."""
+    ``qparam_dtype=torch.bfloat16`` rounds the scale to bf16 before it quantises and dequantises.
+    ``eps``: lower bound of the scale (None = ``finfo(float32).eps``, the convention the oracle documents)."""
     _need_gpu(x, "fq_per_token_int8_asym")
     code = _code(x.dtype, "fq_per_token_int8_asym")
     qcode = _code(qparam_dtype, "fq_per_token_int8_asym (qparams)")
@@ -370,8 +389,8 @@ def fq_per_token_int8_asym(x: torch.Tensor, want_qparams: bool = True, qparam_dt
         events = _fq_timer("per_token", rows, K, 0, xc.element_size()) if _fq_timer is not None else None
         if events:
             events[0].record()
-        rc = lib.ttamd_fq_per_token_int8_asym(xc.data_ptr(), code, rows, K, qcode, out.data_ptr(), _ptr(scale), _ptr(zp),
-                                              _stream(x))
+        rc = lib.ttamd_fq_per_token_int8_asym_conv(xc.data_ptr(), code, rows, K, qcode, out.data_ptr(), _ptr(scale), _ptr(zp),
+                                                   _conventions(eps_per_token=eps), _stream(x))
         if events:
             events[1].record()
     _lib.check(rc, "fq_per_token_int8_asym")
@@ -379,9 +398,10 @@ def fq_per_token_int8_asym(x: torch.Tensor, want_qparams: bool = True, qparam_dt
 
 
 def fq_per_group_int4_sym(w: torch.Tensor, group_size: int, want_scale: bool = True,
-                          qparam_dtype: torch.dtype = torch.float32):
+                          qparam_dtype: torch.dtype = torch.float32, eps: Optional[float] = None):
     """w [..., K] -> (fake-quantised w, scale fp32 [rows, K/g] | None).
-    ``qparam_dtype=torch.bfloat16`` rounds the scales to bf16 before they quantise and dequantise."""
+    ``qparam_dtype=torch.bfloat16`` rounds the scales to bf16 before they quantise and dequantise.
+    ``eps``: lower bound of the scale (None = ``finfo(float32).eps``)."""
     _need_gpu(w, "fq_per_group_int4_sym")
     code = _code(w.dtype, "fq_per_group_int4_sym")
     qcode = _code(qparam_dtype, "fq_per_group_int4_sym (qparams)")
@@ -395,15 +415,16 @@ def fq_per_group_int4_sym(w: torch.Tensor, group_size: int, want_scale: bool = T
         events = _fq_timer("per_group", rows, K, group_size, wc.element_size()) if _fq_timer is not None else None
         if events:
             events[0].record()
-        rc = lib.ttamd_fq_per_group_int4_sym(wc.data_ptr(), code, rows, K, group_size, qcode, out.data_ptr(), _ptr(scale),
-                                             _stream(w))
+        rc = lib.ttamd_fq_per_group_int4_sym_conv(wc.data_ptr(), code, rows, K, group_size, qcode, out.data_ptr(), _ptr(scale),
+                                                  _conventions(eps_per_group_sym=eps), _stream(w))
         if events:
             events[1].record()
     _lib.check(rc, "fq_per_group_int4_sym")
     return out, scale
 
 
-def quantize_per_group_int4(w: torch.Tensor, group_size: int, qparam_dtype: torch.dtype = torch.float32):
+def quantize_per_group_int4(w: torch.Tensor, group_size: int, qparam_dtype: torch.dtype = torch.float32,
+                            eps: Optional[float] = None):
     """w [rows, K] -> (int8 tensor of int4 values, scale fp32 [rows, K/g], zeros fp32 [rows, K/g])"""
     _need_gpu(w, "quantize_per_group_int4")
     code = _code(w.dtype, "quantize_per_group_int4")
@@ -416,17 +437,18 @@ def quantize_per_group_int4(w: torch.Tensor, group_size: int, qparam_dtype: torc
     zeros = torch.empty_like(scale)
     lib = _lib.load()
     with torch.cuda.device(w.device):
-        rc = lib.ttamd_quantize_per_group_int4(wc.data_ptr(), code, rows, K, group_size, qcode, q.data_ptr(), scale.data_ptr(),
-                                               zeros.data_ptr(), _stream(w))
+        rc = lib.ttamd_quantize_per_group_int4_conv(wc.data_ptr(), code, rows, K, group_size, qcode, q.data_ptr(), scale.data_ptr(),
+                                                    zeros.data_ptr(), _conventions(eps_per_group_sym=eps), _stream(w))
     _lib.check(rc, "quantize_per_group_int4")
     return q, scale, zeros
 
 
 def fq_per_group_uint4_asym(w: torch.Tensor, group_size: int, qparam_dtype: torch.dtype = torch.bfloat16,
-                            want_qparams: bool = True):
+                            want_qparams: bool = True, min_scale: Optional[float] = None, clamp_range_first: bool = False):
     """Weight-only int4 scheme (asymmetric uint4, floating-point zero point):
     w [..., K] -> (fake-quantised w, scale fp32 [rows, K/g] | None, zero_point fp32 [rows, K/g] | None);
-    the qparams hold values already rounded to ``qparam_dtype``."""
+    the qparams hold values already rounded to ``qparam_dtype``.  ``min_scale`` (None = 1e-6) bounds the scale from below;
+    ``clamp_range_first`` applies that bound to ``max - min`` before the division by 15 instead of to the quotient."""
     _need_gpu(w, "fq_per_group_uint4_asym")
     code = _code(w.dtype, "fq_per_group_uint4_asym")
     qcode = _code(qparam_dtype, "fq_per_group_uint4_asym (qparams)")
@@ -441,15 +463,17 @@ def fq_per_group_uint4_asym(w: torch.Tensor, group_size: int, qparam_dtype: torc
         events = _fq_timer("per_group", rows, K, group_size, wc.element_size()) if _fq_timer is not None else None
         if events:
             events[0].record()
-        rc = lib.ttamd_fq_per_group_uint4_asym(wc.data_ptr(), code, rows, K, group_size, qcode, out.data_ptr(), _ptr(scale),
-                                               _ptr(zero), _stream(w))
+        rc = lib.ttamd_fq_per_group_uint4_asym_conv(
+            wc.data_ptr(), code, rows, K, group_size, qcode, out.data_ptr(), _ptr(scale), _ptr(zero),
+            _conventions(min_scale_uint4=min_scale, clamp_range_first=clamp_range_first), _stream(w))
         if events:
             events[1].record()
     _lib.check(rc, "fq_per_group_uint4_asym")
     return out, scale, zero
 
 
-def quantize_per_group_uint4(w: torch.Tensor, group_size: int, qparam_dtype: torch.dtype = torch.bfloat16):
+def quantize_per_group_uint4(w: torch.Tensor, group_size: int, qparam_dtype: torch.dtype = torch.bfloat16,
+                             min_scale: Optional[float] = None, clamp_range_first: bool = False):
     """w [rows, K] -> (uint8 [rows, K/2], two codes per byte with the even element in the high nibble,
     scale fp32 [rows, K/g], zero_point fp32 [rows, K/g])"""
     _need_gpu(w, "quantize_per_group_uint4")
@@ -464,8 +488,9 @@ def quantize_per_group_uint4(w: torch.Tensor, group_size: int, qparam_dtype: tor
     zero = torch.empty_like(scale)
     lib = _lib.load()
     with torch.cuda.device(w.device):
-        rc = lib.ttamd_quantize_per_group_uint4(wc.data_ptr(), code, rows, K, group_size, qcode, q.data_ptr(), scale.data_ptr(),
-                                                zero.data_ptr(), _stream(w))
+        rc = lib.ttamd_quantize_per_group_uint4_conv(
+            wc.data_ptr(), code, rows, K, group_size, qcode, q.data_ptr(), scale.data_ptr(), zero.data_ptr(),
+            _conventions(min_scale_uint4=min_scale, clamp_range_first=clamp_range_first), _stream(w))
     _lib.check(rc, "quantize_per_group_uint4")
     return q, scale, zero
 

@@ -63,6 +63,7 @@ class FakeQuantizeConfig:
         scale_precision, zero_point_precision: dtypes of the qparams kept on the quantizer
         is_dynamic: qparams are recomputed from each input (the only supported mode)
         zero_point_domain: ``ZeroPointDomain.INT`` (default) or ``ZeroPointDomain.FLOAT`` (the weight-only scheme)
+        eps: lower bound of the scale; None keeps the scheme's default
     """
 
     def __init__(
@@ -77,6 +78,7 @@ class FakeQuantizeConfig:
         group_size: Optional[int] = None,
         is_symmetric: Optional[bool] = None,
         zero_point_domain: ZeroPointDomain = ZeroPointDomain.INT,
+        eps: Optional[float] = None,
     ):
         if dtype not in (torch.int8, torch.int4, torch.uint4):
             raise NotImplementedError(f"FakeQuantizeConfig: dtype {dtype} has no kernel (int8, int4 and uint4 do)")
@@ -115,6 +117,9 @@ class FakeQuantizeConfig:
         self.scale_precision = scale_precision
         self.zero_point_precision = zero_point_precision
         self.is_dynamic = is_dynamic
+        # lower bound of the scale; None = the scheme's default (finfo(float32).eps for the integer schemes, 1e-6 for
+        # the weight-only uint4 scheme).  Versions of the reference's quantisation package differ here.
+        self.eps = eps
         if not is_dynamic:
             raise NotImplementedError("FakeQuantizeConfig: only dynamic qparams have a kernel")
 
@@ -188,12 +193,12 @@ class FakeQuantizer(nn.Module):
         share = FakeQuantizer.share_identical_inputs and not (torch.is_inference_mode_enabled() or x.is_inference())
         if not share:
             FakeQuantizer._last.entry = None
-            return ops.fq_per_token_int8_asym(x.detach(), qparam_dtype=self.config.scale_precision)
-        key = (x._version, self.config.scale_precision)
+            return ops.fq_per_token_int8_asym(x.detach(), qparam_dtype=self.config.scale_precision, eps=self.config.eps)
+        key = (x._version, self.config.scale_precision, self.config.eps)
         hit = getattr(FakeQuantizer._last, "entry", None)
         if hit is not None and hit[0]() is x and hit[1] == key:
             return hit[2]
-        out = ops.fq_per_token_int8_asym(x.detach(), qparam_dtype=self.config.scale_precision)
+        out = ops.fq_per_token_int8_asym(x.detach(), qparam_dtype=self.config.scale_precision, eps=self.config.eps)
         # the input is held by weak reference: the entry dies with the activation instead of keeping it (and its
         # fake-quantised copy) alive after the step; a new tensor replaces the entry
         try:
@@ -221,11 +226,11 @@ class FakeQuantizer(nn.Module):
                 if x.shape[-1] % gs != 0:
                     raise ValueError(f"last dimension ({x.shape[-1]}) must be divisible by group_size ({gs})")
                 if self._weight_only_int4(self.config):
-                    fq, scale, zp = ops.fq_per_group_uint4_asym(x.detach(), gs, self.config.scale_precision)
+                    fq, scale, zp = ops.fq_per_group_uint4_asym(x.detach(), gs, self.config.scale_precision, min_scale=self.config.eps)
                     self.scale = scale.to(self.config.scale_precision)
                     self.zero_point = zp.to(self.config.zero_point_precision)
                 else:
-                    fq, scale = ops.fq_per_group_int4_sym(x.detach(), gs, qparam_dtype=self.config.scale_precision)
+                    fq, scale = ops.fq_per_group_int4_sym(x.detach(), gs, qparam_dtype=self.config.scale_precision, eps=self.config.eps)
                     self.scale = scale.to(self.config.scale_precision)
                     self.zero_point = None
         return _StraightThrough.apply(x, fq.view(x.shape))
