@@ -33,10 +33,30 @@ WORKLOADS = {
 HBM_PEAK_GBPS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 # HBM-side bytes per launch of the workload's dominant kernel (fused GEMM; fake quant for the QAT workload), average over
-# the launches of one step, from the FETCH_SIZE / WRITE_SIZE counter runs summarised in
-# profiles/nf4_gemm_rs_kernel_hbm_traffic.txt and profiles/fake_quant_and_layer_kernels_hbm_traffic.txt (counters cannot
-# be read from inside this process).
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"llama3_1_8b": 496.3e6, "llama3_1_8b_qat": 164.1e6}
+# the launches of one step.  Counters cannot be read from inside this process: the figure comes from the FETCH_SIZE /
+# WRITE_SIZE counter runs summarised under profiles/, each of which ends with a line
+#     bench.traffic_bytes_per_launch[<workload>] = <bytes>
+# that is read back here, so the bench line always quotes the committed measurement (null when there is none).
+TRAFFIC_SUMMARIES = {
+    "llama3_1_8b": "profiles/nf4_gemm_rs_kernel_hbm_traffic.txt",
+    "llama3_1_8b_qat": "profiles/fake_quant_and_layer_kernels_hbm_traffic.txt",
+}
+
+
+def measured_traffic(workload: str):
+    """-> (bytes per launch or None, the summary file it was read from or None)"""
+    rel = TRAFFIC_SUMMARIES.get(workload)
+    if rel is None:
+        return None, None
+    try:
+        with open(os.path.join(ROOT, rel)) as f:
+            for line in f:
+                line = line.strip()
+                if line.startswith(f"bench.traffic_bytes_per_launch[{workload}]"):
+                    return float(line.split("=", 1)[1]), rel
+    except (OSError, ValueError):
+        pass
+    return None, rel
 
 
 class GemmTimer:
@@ -53,9 +73,12 @@ class GemmTimer:
 
     def __call__(self, kind, M, N, K, rank):
         flops = 2.0 * M * N * K + 2.0 * M * rank * (N if kind == "fwd" else K)
+        # algorithmic bytes of a launch: both activation tensors once, the packed weight with its fp32 block scalers
+        # (0.5 + 4/64 B per element), the adapter operands
+        nbytes = 2.0 * M * K + 2.0 * M * N + 0.5625 * N * K + 2.0 * rank * (M + (N if kind == "fwd" else K))
         key = (kind, M, N, K)
-        seen = self.counts.get(key, [0, flops])
-        self.counts[key] = [seen[0] + 1, flops]
+        seen = self.counts.get(key, [0, flops, nbytes])
+        self.counts[key] = [seen[0] + 1, flops, nbytes]
         if seen[0] % self.stride:
             return None
         start = torch.cuda.Event(enable_timing=True)
@@ -64,15 +87,18 @@ class GemmTimer:
         return start, end
 
     def summary(self):
-        """-> (launches, launches timed, estimated ms of all launches, flops of all launches, per-shape table)"""
+        """-> (launches, launches timed, estimated ms of all launches, flops of all launches, per-shape table); the
+        algorithmic bytes of all launches are left in ``self.total_bytes``"""
         timed = {}
         for key, s, e in self.records:
             acc = timed.setdefault(key, [0, 0.0])
             acc[0] += 1
             acc[1] += s.elapsed_time(e)
         total_ms = total_flops = 0.0
+        self.total_bytes = 0.0
         per_shape = {}
-        for key, (n, flops) in self.counts.items():
+        for key, (n, flops, nbytes) in self.counts.items():
+            self.total_bytes += nbytes * n
             n_timed, ms = timed[key]
             avg_ms = ms / n_timed
             total_ms += avg_ms * n
@@ -225,6 +251,14 @@ def secondary_kernels(dev) -> dict:
     dense = torch.empty_like(W)  # preallocated: with the allocator in the loop the host barely keeps ahead of a 25 us kernel
     out["nf4_dequantize 14336x4096 bf16"] = round(n * 2.515747 / timed(lambda: t.get_original_weight(out=dense)) / 1e9, 1)
     del dense
+    # the 70B gate / up weight: 118 MB of codes in, 470 MB out — more than the 256 MB last-level cache holds, so this is
+    # the rate against HBM itself (the 8B weight above can live in that cache between launches)
+    Wb = (torch.randn(28672, 8192, device=dev, generator=gen) * 0.02).to(torch.bfloat16)
+    tb = to_nf4(Wb)
+    nb = Wb.numel()
+    out["nf4_dequantize 28672x8192 bf16 (235 M elements, beyond the last-level cache)"] = round(
+        nb * 2.515747 / timed(lambda: tb.get_original_weight(out=Wb), iters=20) / 1e9, 1)
+    del Wb, tb
     out["nf4_quantize 14336x4096 bf16"] = round(n * 2.515747 / timed(lambda: ops.nf4_quantize(W, 64, 256)) / 1e9, 1)
     out["fq_per_group_int4_sym g32 14336x4096 bf16"] = round(
         (n * 4 + n / 32 * 4) / timed(lambda: ops.fq_per_group_int4_sym(W, 32)) / 1e9, 1)
@@ -254,6 +288,105 @@ def secondary_kernels(dev) -> dict:
         out[f"nf4_lora_linear_fwd M={m_tok} 14336x4096 (few-token kernel, packed-weight bytes)"] = round(n * 0.5625 / sec / 1e9, 1)
         del graph
     return {"unit": "GB/s (algorithmic bytes / HIP-event time, HBM peak 8000)", **out}
+
+
+def config1_leg(dev, runs: int = 15, warmups: int = 3) -> dict:
+    """The single-layer configuration (one QLoRA ``LoRALinear``: bf16 [2048, 2048] N(0, 0.02) base weight quantised with
+    ``to_nf4`` (64 / 256), rank 8, alpha 16, A Kaiming-uniform, B ~ N(0, 0.01), x bf16 [4, 512, 2048] ~ N(0, 1), seed 0,
+    forward + backward of sum(y^2)), timed in full on the GPU and on the host: median of ``runs`` after ``warmups``
+    warm-ups each.  The CPU figure is the eager-PyTorch oracle (the reference's op sequence) on this box's host cores."""
+    import statistics
+
+    from oracle import lora_oracle, nf4_oracle
+    from torchtune_amd.modules.peft import LoRALinear
+
+    torch.manual_seed(0)
+    W = (torch.randn(2048, 2048) * 0.02).to(torch.bfloat16)
+    A = lora_oracle.lora_a_init_(torch.empty(8, 2048)).to(torch.bfloat16)
+    B = (torch.randn(2048, 8) * 0.01).to(torch.bfloat16)
+    x = torch.randn(4, 512, 2048).to(torch.bfloat16)
+    prev = torch.get_default_dtype()
+    torch.set_default_dtype(torch.bfloat16)
+    try:
+        with torch.device(dev):
+            layer = LoRALinear(2048, 2048, rank=8, alpha=16.0, quantize_base=True)
+    finally:
+        torch.set_default_dtype(prev)
+    with torch.no_grad():
+        layer.weight.copy_(W.to(dev))
+        layer.lora_a.weight.copy_(A.to(dev))
+        layer.lora_b.weight.copy_(B.to(dev))
+    xd = x.to(dev).requires_grad_()
+
+    def gpu_run():
+        y = layer(xd)
+        (y.float() ** 2).sum().backward()
+        layer.zero_grad(set_to_none=True)
+        xd.grad = None
+
+    gpu_ms = []
+    for i in range(warmups + runs):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        gpu_run()
+        torch.cuda.synchronize()
+        if i >= warmups:
+            gpu_ms.append(1e3 * (time.perf_counter() - t0))
+    # kernel time alone (the layer is a handful of launches, so wall time above is mostly launch latency)
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(runs):
+        gpu_run()
+    end.record()
+    torch.cuda.synchronize()
+    stream_ms = start.elapsed_time(end) / runs
+
+    parts = nf4_oracle.nf4_quantize(W, 64, 256)
+    xo = x.clone().requires_grad_()
+    Ao, Bo = A.clone().requires_grad_(), B.clone().requires_grad_()
+    cpu_ms = []
+    for i in range(warmups + runs):
+        t0 = time.perf_counter()
+        yo = lora_oracle.lora_linear_forward(xo, parts, Ao, Bo, 16.0, 8)
+        (yo.float() ** 2).sum().backward()
+        if i >= warmups:
+            cpu_ms.append(1e3 * (time.perf_counter() - t0))
+        xo.grad = Ao.grad = Bo.grad = None
+    tokens = 4 * 512
+    g, c = statistics.median(gpu_ms), statistics.median(cpu_ms)
+    return {
+        "workload": "one QLoRA LoRALinear 2048x2048 r=8 alpha=16, x [4, 512, 2048], fwd+bwd of sum(y^2), seed 0",
+        "runs": runs, "warmups": warmups,
+        "gpu_ms_median": round(g, 3), "gpu_ms_back_to_back": round(stream_ms, 3), "gpu_tokens_per_s": round(tokens / g * 1e3, 1),
+        "cpu_ms_median": round(c, 2), "cpu_tokens_per_s": round(tokens / c * 1e3, 1), "cpu_cores": torch.get_num_threads(),
+        "cpu_kind": "port (eager-PyTorch oracle, timed in full)",
+    }
+
+
+def memory_leg(build, step, dev) -> dict:
+    """Peak device memory of one forward + backward (``torch.cuda.max_memory_allocated``) with the transposed copy of the
+    codes that the grad-input GEMM streams (0.5625 B per weight element, the default) and without it."""
+    from torchtune_amd import nf4_tensor
+
+    out = {}
+    for keep in (True, False):
+        nf4_tensor.BACKWARD_COPY = keep
+        try:
+            model = build()
+            step(model)  # builds the derived copies, warms the allocator
+            torch.cuda.synchronize()
+            resident = torch.cuda.memory_allocated(dev)
+            torch.cuda.reset_peak_memory_stats(dev)
+            step(model)
+            torch.cuda.synchronize()
+            out["with_backward_copy" if keep else "without_backward_copy"] = {
+                "resident_gib": round(resident / 2**30, 3), "peak_gib": round(torch.cuda.max_memory_allocated(dev) / 2**30, 3)}
+            del model
+            torch.cuda.empty_cache()
+        finally:
+            nf4_tensor.BACKWARD_COPY = True
+    out["unit"] = "GiB (torch.cuda.memory_allocated after a step = weights + derived copies; max_memory_allocated over one fwd+bwd)"
+    return out
 
 
 def optimizer_leg(model, tokens, labels, train_step, qat: bool, steps: int, tokens_per_step: int):
@@ -312,6 +445,9 @@ def main() -> int:
                          "PyTorch; 'flash' is what the dispatcher picks by itself)")
     ap.add_argument("--gemm-timing-stride", type=int, default=4,
                     help="time every n-th fused-GEMM / fake-quant launch of each shape with HIP events (1 = every launch)")
+    ap.add_argument("--no-memory-leg", action="store_true",
+                    help="skip the peak-memory measurement (two extra model builds with one step each)")
+    ap.add_argument("--no-config1", action="store_true", help="skip the single-layer configuration timed on GPU and CPU")
     ap.add_argument("--calibration-copy-mib", type=int, default=0,
                     help="before the steps, run one elementwise kernel that reads and writes this many MiB: the known-size "
                          "dispatch that FETCH_SIZE / WRITE_SIZE counter runs are scaled by")
@@ -363,11 +499,13 @@ def main() -> int:
     ops.set_gemm_timer(timer)
     ops.set_fq_timer(fq_timer)
     torch.cuda.synchronize()
+    torch.cuda.reset_peak_memory_stats(dev)
     t0 = time.perf_counter()
     for _ in range(args.steps):
         loss = step()
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
+    peak_timed = torch.cuda.max_memory_allocated(dev)
     ops.set_gemm_timer(None)
     ops.set_fq_timer(None)
     ms_per_step = 1e3 * dt / args.steps
@@ -409,9 +547,10 @@ def main() -> int:
                 "peak": HBM_PEAK_GBPS,
                 "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(args.workload),
+                "traffic": measured_traffic(args.workload)[0],
                 "traffic_unit": "bytes per launch, average over a step's fake-quant launches (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 "
-                                f"from rocprofv3 --pmc runs); algorithmic {fq_bytes / max(1, sum(v['launches'] for v in fq.values())) / 1e6:.1f}e6",
+                                f"from the rocprofv3 --pmc runs summarised in {measured_traffic(args.workload)[1]}); "
+                                f"algorithmic {fq_bytes / max(1, sum(v['launches'] for v in fq.values())) / 1e6:.1f}e6",
                 "fq_ms_per_step": round(fq_ms / args.steps, 2),
                 "timing": f"HIP events on the launch stream around every {fq_timer.stride}th launch of each shape inside the "
                           "timed steps; achieved = sum(bytes) / sum(average duration x launches)",
@@ -419,6 +558,7 @@ def main() -> int:
             },
         }
         result["with_adamw"] = with_adamw
+        result["peak_memory_gib_timed_steps"] = round(peak_timed / 2**30, 3)
         del model
         torch.cuda.empty_cache()
         if args.cpu_tokens > 0:
@@ -427,6 +567,7 @@ def main() -> int:
         return 0
 
     launches, launches_timed, gemm_ms, gemm_flops, per_shape = timer.summary()
+    gemm_bytes = timer.total_bytes
     achieved = gemm_flops / gemm_ms / 1e9 if gemm_ms > 0 else 0.0
     result = {
         "metric": "QLoRA fwd+bwd tokens/sec (Llama-3.1-8B, 1 GPU)" if args.workload == "llama3_1_8b"
@@ -458,9 +599,10 @@ def main() -> int:
             "peak": MFMA_BF16_PEAK_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(args.workload),
-            "traffic_unit": "bytes per launch, average over a step's launches (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 from rocprofv3 "
-                            "--pmc runs; algorithmic 210.4e6)" if args.workload in MEASURED_TRAFFIC_BYTES_PER_LAUNCH else None,
+            "traffic": measured_traffic(args.workload)[0],
+            "traffic_unit": ("bytes per launch, average over a step's launches (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 from the "
+                             f"rocprofv3 --pmc runs summarised in {measured_traffic(args.workload)[1]}); algorithmic "
+                             f"{gemm_bytes / max(1, launches) / 1e6:.1f}e6") if measured_traffic(args.workload)[1] else None,
             "launches": launches,
             "launches_timed": launches_timed,
             "timing": f"HIP events on the launch stream around every {timer.stride}th launch of each shape inside the timed steps "
@@ -470,8 +612,18 @@ def main() -> int:
         },
     }
     result["with_adamw"] = with_adamw
+    result["peak_memory_gib_timed_steps"] = round(peak_timed / 2**30, 3)
     del model
     torch.cuda.empty_cache()
+    if not args.no_memory_leg:
+        def one_step(m):
+            train_step(m, tokens, labels)
+            m.zero_grad(set_to_none=True)
+
+        result["memory"] = memory_leg(
+            lambda: build_qlora_decoder(shape_name, rank, alpha, device=dev, seed=0, activation_checkpointing=ac), one_step, dev)
+    if not args.no_config1:
+        result["config1_single_layer"] = config1_leg(dev)
     result["hbm_bound_kernels"] = secondary_kernels(dev)
     if args.cpu_tokens > 0:
         result["cpu_baseline"] = cpu_baseline(shape_name, rank, alpha, args.cpu_tokens, SHAPES[shape_name].n_layers, batch * seq)

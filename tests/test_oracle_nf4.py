@@ -264,3 +264,37 @@ def test_code_table_premises_and_monotone_codes(c_oracle):
         blocks[:, 1] = bits * sign
         p = nf4_oracle.nf4_quantize(blocks, 64, 1)
         assert (p.quantized_data.view(641, 32)[:, 0] & 0xF).tolist() == want
+
+
+def test_exact_scaler_mean_against_eager_mean_on_every_benchmark_weight_shape(record_property):
+    """The oracle (and the kernels) define ``scaler_mean`` as the exact mean of the block absmaxes, rounded once; the
+    reference computes ``absmax.mean()``, whose fp32 summation order belongs to the library version.  On every projection
+    shape of the 1B / 8B / 70B configurations with the benchmark's N(0, 0.02) weights (seed 0) the two are compared in
+    bf16 and the number of mismatches is reported; a mismatch would be one bf16 ulp of the mean and would move every scaler
+    byte of that tensor."""
+    shapes = [(2048, 2048), (512, 2048), (8192, 2048), (2048, 8192), (4096, 4096), (1024, 4096), (14336, 4096), (4096, 14336),
+              (8192, 8192), (1024, 8192), (28672, 8192), (8192, 28672)]
+    mismatches = []
+    for N, K in shapes:
+        g = torch.Generator().manual_seed(0)
+        w = (torch.randn(N, K, generator=g) * 0.02).to(torch.bfloat16)
+        absmax = w.view(-1, 64).abs().max(dim=1).values
+        del w
+        exact, eager = nf4_oracle.order_independent_mean(absmax), absmax.mean()
+        if exact.view(torch.int16).item() != eager.view(torch.int16).item():
+            mismatches.append((N, K, float(exact), float(eager)))
+    # the same question where it is hardest: weight scales swept so that the mean crosses bf16 rounding boundaries
+    near = []
+    for i in range(48):
+        g = torch.Generator().manual_seed(100 + i)
+        w = (torch.randn(1024, 4096, generator=g) * (0.015 + 0.0005 * i)).to(torch.bfloat16)
+        absmax = w.view(-1, 64).abs().max(dim=1).values
+        exact, eager = nf4_oracle.order_independent_mean(absmax), absmax.mean()
+        if exact.view(torch.int16).item() != eager.view(torch.int16).item():
+            near.append((i, float(exact), float(eager)))
+            assert abs(int(exact.view(torch.int16)) - int(eager.view(torch.int16))) == 1  # never more than one ulp
+    record_property("scaler_mean_mismatches_benchmark_shapes", len(mismatches))
+    record_property("scaler_mean_mismatches_scale_sweep", len(near))
+    print(f"scaler_mean: {len(mismatches)} of {len(shapes)} benchmark shapes differ from eager mean(); "
+          f"{len(near)} of 48 tensors of the scale sweep differ (by one bf16 ulp)")
+    assert mismatches == [], mismatches
