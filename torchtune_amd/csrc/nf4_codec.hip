@@ -272,18 +272,21 @@ __global__ __launch_bounds__(256) void nf4_quantize_scalers_kernel(const float* 
 }
 
 // ---------------------------------------------------------------------------------------------------
-// dequantise.  A workgroup expands 16384 elements.  It first evaluates the block scalers of its span once
-// (one thread per block, into LDS: the division is done once per block, not once per lane), then every
-// lane turns one dword of codes (8 elements) into one 128-bit bf16 store (two for fp32), so each load and
+// dequantise.  A workgroup expands 256 * DW * 8 elements (DW = dwords of codes per lane).  It first evaluates the
+// block scalers of its span once (one thread per block, into LDS: the division is done once per block, not once per
+// lane), then every lane turns one dword of codes (8 elements) into one 128-bit bf16 store (two for fp32), so each load and
 // store instruction of a wave covers one contiguous span.  Code pairs are looked up a byte at a time in a
 // 256-entry LDS table of (nf4[hi], nf4[lo]) in fp32; for bf16 the product is rounded once, by the packing
 // conversion (round to nearest even, the same rounding the eager reference applies to the product).
+//
+// DW is chosen by the launch: 8 (16384 elements per workgroup) while codes and output together fit the 256 MB
+// last-level cache, where fewer, longer workgroups win (measured 5.9 against 5.6 TB/s on 14336 x 4096), and 4 beyond
+// it, where twice the number of workgroups keeps more HBM requests in flight (6.1 against 5.4 TB/s on 28672 x 8192
+// with the cache defeated by rotating over four weights).
 // ---------------------------------------------------------------------------------------------------
-constexpr int kDequantDwordsPerThread = 8;
-constexpr int kDequantElemsPerWg = 256 * kDequantDwordsPerThread * 8;  // 16384
-constexpr int kDequantMaxBlocksPerWg = kDequantElemsPerWg / 8;         // smallest block size is 8
+constexpr int64_t kDequantCacheResidentBytes = int64_t(192) << 20;
 
-template <bool BF16>
+template <bool BF16, int DW>
 __global__ __launch_bounds__(256) void nf4_dequantize_kernel(const uint32_t* __restrict__ qdata,
                                                              const int8_t* __restrict__ qscalers,
                                                              const void* __restrict__ qfactor,
@@ -291,19 +294,19 @@ __global__ __launch_bounds__(256) void nf4_dequantize_kernel(const uint32_t* __r
                                                              int log2_dwords_per_block, int SB, int log2_SB,
                                                              int64_t n_blocks, void* __restrict__ out) {
   __shared__ float2 lut[256];
-  __shared__ float scal[kDequantMaxBlocksPerWg];
+  __shared__ float scal[256 * DW];  // smallest block size is 8 elements = one dword
   const int t = threadIdx.x;
-  const int64_t base = (int64_t)blockIdx.x * (256 * kDequantDwordsPerThread) + t;
-  uint32_t code[kDequantDwordsPerThread];
+  const int64_t base = (int64_t)blockIdx.x * (256 * DW) + t;
+  uint32_t code[DW];
 #pragma unroll
-  for (int u = 0; u < kDequantDwordsPerThread; ++u) {
+  for (int u = 0; u < DW; ++u) {
     const int64_t idx = base + u * 256;
     code[u] = idx < n_dwords ? __builtin_nontemporal_load(qdata + idx) : 0u;
   }
   lut[t] = make_float2(Arith<BF16>::rnd(kNF4Dev[t >> 4]), Arith<BF16>::rnd(kNF4Dev[t & 15]));
   {
     const float mean = load1<BF16>(scaler_mean, 0);
-    const int blocks_per_wg = (256 * kDequantDwordsPerThread) >> log2_dwords_per_block;
+    const int blocks_per_wg = (256 * DW) >> log2_dwords_per_block;
     const int64_t blk0 = (int64_t)blockIdx.x * blocks_per_wg;
     for (int i = t; i < blocks_per_wg; i += 256) {
       const int64_t blk = blk0 + i;
@@ -314,7 +317,7 @@ __global__ __launch_bounds__(256) void nf4_dequantize_kernel(const uint32_t* __r
   }
   __syncthreads();
 #pragma unroll
-  for (int u = 0; u < kDequantDwordsPerThread; ++u) {
+  for (int u = 0; u < DW; ++u) {
     const int64_t idx = base + u * 256;
     if (idx >= n_dwords) continue;
     const float sc = scal[(u * 256 + t) >> log2_dwords_per_block];
@@ -443,18 +446,22 @@ extern "C" int ttamd_nf4_dequantize(const uint8_t* quantized_data, const int8_t*
              "nf4_dequantize: quantized_data must be 4-byte aligned and out 16-byte aligned");
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   const int64_t n_dwords = numel / 8;
-  const int64_t per_wg = 256 * kDequantDwordsPerThread;
-  const int64_t grid = (n_dwords + per_wg - 1) / per_wg;
-  TT_REQUIRE(grid < (int64_t(1) << 31), "nf4_dequantize: tensor too large for one launch");
   const int l2dpb = log2_exact(block_size / 8);
   const int l2sb = is_pow2(scaler_block_size) ? log2_exact(scaler_block_size) : -1;
-  if (dtype == TTAMD_BF16)
-    nf4_dequantize_kernel<true><<<dim3((unsigned)grid), dim3(256), 0, s>>>(
-        reinterpret_cast<const uint32_t*>(quantized_data), quantized_scalers, quantization_factor, scaler_mean, n_dwords,
-        l2dpb, scaler_block_size, l2sb, numel / block_size, out);
-  else
-    nf4_dequantize_kernel<false><<<dim3((unsigned)grid), dim3(256), 0, s>>>(
-        reinterpret_cast<const uint32_t*>(quantized_data), quantized_scalers, quantization_factor, scaler_mean, n_dwords,
-        l2dpb, scaler_block_size, l2sb, numel / block_size, out);
+  const int64_t bytes_moved = numel / 2 + numel * (dtype == TTAMD_BF16 ? 2 : 4);
+  const int dw = bytes_moved <= kDequantCacheResidentBytes ? 8 : 4;
+  const int64_t per_wg = 256 * dw;
+  const int64_t grid = (n_dwords + per_wg - 1) / per_wg;
+  TT_REQUIRE(grid < (int64_t(1) << 31), "nf4_dequantize: tensor too large for one launch");
+  auto launch = [&](auto kernel) {
+    kernel<<<dim3((unsigned)grid), dim3(256), 0, s>>>(reinterpret_cast<const uint32_t*>(quantized_data), quantized_scalers,
+                                                      quantization_factor, scaler_mean, n_dwords, l2dpb, scaler_block_size,
+                                                      l2sb, numel / block_size, out);
+  };
+  if (dtype == TTAMD_BF16) {
+    if (dw == 8) launch(nf4_dequantize_kernel<true, 8>); else launch(nf4_dequantize_kernel<true, 4>);
+  } else {
+    if (dw == 8) launch(nf4_dequantize_kernel<false, 8>); else launch(nf4_dequantize_kernel<false, 4>);
+  }
   return check_launch("nf4_dequantize");
 }
