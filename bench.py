@@ -72,13 +72,24 @@ class GemmTimer:
         self.counts = {}
 
     def __call__(self, kind, M, N, K, rank):
-        flops = 2.0 * M * N * K + 2.0 * M * rank * (N if kind == "fwd" else K)
+        # "fwd" / "bwd": one layer, one launch.  "fwd_group" / "bwd_group": the layers of a group with a common input (N and
+        # rank are lists): one forward launch per member between the events, or the single grad-input launch whose
+        # contraction runs through all members' output columns.
+        Ns = tuple(N) if isinstance(N, (list, tuple)) else (N,)
+        ranks = tuple(rank) if isinstance(rank, (list, tuple)) else (rank,) * len(Ns)
+        fwd = kind.startswith("fwd")
+        flops = sum(2.0 * M * n * K + 2.0 * M * r * (n if fwd else K) for n, r in zip(Ns, ranks))
         # algorithmic bytes of a launch: both activation tensors once, the packed weight with its fp32 block scalers
         # (0.5 + 4/64 B per element), the adapter operands
-        nbytes = 2.0 * M * K + 2.0 * M * N + 0.5625 * N * K + 2.0 * rank * (M + (N if kind == "fwd" else K))
-        key = (kind, M, N, K)
-        seen = self.counts.get(key, [0, flops, nbytes])
-        self.counts[key] = [seen[0] + 1, flops, nbytes]
+        if fwd:
+            launches = len(Ns)
+            nbytes = sum(2.0 * M * K + 2.0 * M * n + 0.5625 * n * K + 2.0 * r * (M + n) for n, r in zip(Ns, ranks))
+        else:
+            launches = 1
+            nbytes = 2.0 * M * K + sum(2.0 * M * n + 0.5625 * n * K + 2.0 * r * (M + K) for n, r in zip(Ns, ranks))
+        key = (kind, M, Ns if len(Ns) > 1 else Ns[0], K)
+        seen = self.counts.get(key, [0, flops, nbytes, launches])
+        self.counts[key] = [seen[0] + 1, flops, nbytes, launches]
         if seen[0] % self.stride:
             return None
         start = torch.cuda.Event(enable_timing=True)
@@ -97,15 +108,19 @@ class GemmTimer:
         total_ms = total_flops = 0.0
         self.total_bytes = 0.0
         per_shape = {}
-        for key, (n, flops, nbytes) in self.counts.items():
+        n_launches = 0
+        for key, (n, flops, nbytes, launches) in self.counts.items():
             self.total_bytes += nbytes * n
+            n_launches += launches * n
             n_timed, ms = timed[key]
             avg_ms = ms / n_timed
             total_ms += avg_ms * n
             total_flops += flops * n
-            per_shape[f"{key[0]} M{key[1]} N{key[2]} K{key[3]}"] = {
-                "launches": n, "timed": n_timed, "avg_us": round(1e3 * avg_ms, 1), "tflops": round(flops / avg_ms / 1e9, 1)}
-        return sum(v[0] for v in self.counts.values()), len(self.records), total_ms, total_flops, per_shape
+            shape_n = "+".join(map(str, key[2])) if isinstance(key[2], tuple) else key[2]
+            per_shape[f"{key[0]} M{key[1]} N{shape_n} K{key[3]}"] = {
+                "calls": n, "launches": launches * n, "timed": n_timed, "avg_us": round(1e3 * avg_ms, 1),
+                "tflops": round(flops / avg_ms / 1e9, 1)}
+        return n_launches, len(self.records), total_ms, total_flops, per_shape
 
 
 class FqTimer:
@@ -448,6 +463,9 @@ def main() -> int:
     ap.add_argument("--no-memory-leg", action="store_true",
                     help="skip the peak-memory measurement (two extra model builds with one step each)")
     ap.add_argument("--no-config1", action="store_true", help="skip the single-layer configuration timed on GPU and CPU")
+    ap.add_argument("--no-group", action="store_true",
+                    help="one call per projection, as the reference's modules make them, instead of the group kernels for the "
+                         "projections that share an input (q/k/v, gate/up): for A/B timing")
     ap.add_argument("--calibration-copy-mib", type=int, default=0,
                     help="before the steps, run one elementwise kernel that reads and writes this many MiB: the known-size "
                          "dispatch that FETCH_SIZE / WRITE_SIZE counter runs are scaled by")
@@ -464,6 +482,7 @@ def main() -> int:
     from torchtune_amd.harness import SHAPES, build_qat_decoder, build_qlora_decoder, train_step
 
     harness.SDPA_BACKEND = args.sdpa
+    harness.GROUP_SHARED_INPUT = not args.no_group
 
     shape_name, rank, alpha, batch, seq, ac = WORKLOADS[args.workload]
     qat = args.workload.endswith("_qat")

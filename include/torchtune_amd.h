@@ -33,6 +33,8 @@ extern "C" {
 #define TTAMD_BF16 0
 #define TTAMD_F32 1
 
+#define TTAMD_GROUP_MAX 4 /* most members of a group of linears with a common input (ttamd_lora_group_*) */
+
 #define TTAMD_OK 0
 #define TTAMD_EINVAL (-1)     /* bad argument: null pointer, misaligned pointer, shape or divisibility violation */
 #define TTAMD_EUNSUPPORTED (-2) /* valid request this build has no kernel for (e.g. fused GEMM with block_size != 64) */
@@ -246,6 +248,63 @@ size_t ttamd_lora_bwd_workspace_bytes(int64_t M, int64_t N, int64_t K, int rank)
 int ttamd_lora_bwd_bf16(const void* gy, const void* x, const void* h, const void* lora_b, float scale, void* gh, void* ga,
                         void* gb, int64_t M, int64_t N, int64_t K, int rank, void* workspace, size_t workspace_bytes,
                         void* stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * Groups of LoRA linears with a common input
+ *
+ * An addition above the per-linear interface; the reference has no such call.  Its modules call the members one after
+ * the other on the same tensor: q_proj, k_proj, v_proj in torchtune/modules/attention.py:234,262-263 and w1 (gate), w3
+ * (up) in torchtune/modules/feed_forward.py:50-53, each a LoRALinear.forward (torchtune/modules/peft/lora.py:128-147).
+ * A group call computes exactly what the member-by-member calls compute, with fewer passes over the shared operands:
+ *
+ *   forward   h_cat[:, member i] = x . lora_a_i^T for all members in one pass over x (h_cat [M, sum of ranks] bf16,
+ *             member i in columns [sum of the ranks before it, + rank_i); the caller keeps it for the backward);
+ *             y_i = x . D(W_i)^T (+ bias_i) + scale_i . h_i . lora_b_i^T: for M <= 64 one launch for all members that
+ *             get the same launch shape, otherwise one launch per member.  h_cat and every y_i are bit-identical to
+ *             ttamd_lora_hidden_bf16 + ttamd_nf4_lora_linear_fwd_bf16 on the member alone.
+ *   backward  gh_cat[:, member i] = scale_i . gy_i . lora_b_i (one launch, bit-identical to ttamd_lora_bwd_bf16's gh);
+ *             grad_lora_a_i = gh_i^T . x for all members in one pass over x and grad_lora_b_i = scale_i . gy_i^T . h_i in
+ *             the same launch (fp32 partial sums over row ranges chosen for the whole batch: the same values as the
+ *             per-member call up to the order of fp32 additions);
+ *             gx = sum_i gy_i . D(W_i) + gh_i . lora_a_i as ONE GEMM whose contraction runs through the members' output
+ *             columns one member after the other, summed in fp32 and rounded to bf16 once (the member-by-member
+ *             path rounds each member's product to bf16 and adds the rounded tensors).  Every member needs
+ *             quantized_data_t and block_scalers_t for it.
+ *
+ * Requires K % 64 == 0, N_i % 64 == 0, rank_i a positive multiple of 8, sum of ranks <= 64, 1 <= n_members <=
+ * TTAMD_GROUP_MAX, all pointers 16-byte aligned (bias: 8).
+ * ---------------------------------------------------------------------------------------------- */
+typedef struct ttamd_lora_group_member {
+  const uint8_t* quantized_data;   /* NF4 codes of the [N, K] weight */
+  const void* block_scalers;       /* fp32 [N, K/64] (ttamd_nf4_block_scalers) */
+  const void* block_scalers_t;     /* fp32 [K/64, N] or NULL   (ttamd_nf4_transpose_for_backward, second output) */
+  const uint8_t* quantized_data_t; /* codes of the transposed weight, [K, N/2], or NULL (same call, first output) */
+  const void* lora_a;              /* bf16 [rank, K] */
+  const void* lora_b;              /* bf16 [N, rank] */
+  const void* bias;                /* bf16 [N] or NULL (forward only) */
+  void* y;                         /* forward: out, bf16 [M, N].  backward: in, the gradient of that output */
+  void* grad_lora_a;               /* backward: out, bf16 [rank, K] */
+  void* grad_lora_b;               /* backward: out, bf16 [N, rank] */
+  int64_t N;
+  int rank;
+  float scale;                     /* alpha / rank */
+} ttamd_lora_group_member;
+
+/* h_cat out, bf16 [M, sum of ranks] */
+size_t ttamd_lora_group_hidden_workspace_bytes(const ttamd_lora_group_member* members, int n_members, int64_t M, int64_t K);
+int ttamd_lora_group_hidden_bf16(const void* x, const ttamd_lora_group_member* members, int n_members, void* h_cat, int64_t M,
+                                 int64_t K, void* workspace, size_t workspace_bytes, void* stream);
+/* every member's y from x and h_cat; workspace may be NULL (then launches with few output tiles are not sliced) */
+size_t ttamd_lora_group_fwd_workspace_bytes(const ttamd_lora_group_member* members, int n_members, int64_t M, int64_t K);
+int ttamd_nf4_lora_group_fwd_bf16(const void* x, const ttamd_lora_group_member* members, int n_members, const void* h_cat,
+                                  int64_t M, int64_t K, void* workspace, size_t workspace_bytes, void* stream);
+/* gh_cat out, bf16 [M, sum of ranks]; every member's grad_lora_a and grad_lora_b; members[i].y = gy_i */
+size_t ttamd_lora_group_bwd_workspace_bytes(const ttamd_lora_group_member* members, int n_members, int64_t M, int64_t K);
+int ttamd_lora_group_bwd_bf16(const void* x, const void* h_cat, const ttamd_lora_group_member* members, int n_members,
+                              void* gh_cat, int64_t M, int64_t K, void* workspace, size_t workspace_bytes, void* stream);
+/* gx out, bf16 [M, K], from gh_cat and members[i].y = gy_i, quantized_data_t, block_scalers_t, lora_a */
+int ttamd_nf4_group_bwd_dx_bf16(const ttamd_lora_group_member* members, int n_members, const void* gh_cat, void* gx, int64_t M,
+                                int64_t K, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
  * QAT fake quantisation (int8 dynamic per-token activations, int4 per-group symmetric weights)

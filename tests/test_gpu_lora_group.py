@@ -1,0 +1,230 @@
+"""Groups of LoRA linears with a common input (q/k/v, gate/up) on the GPU.
+
+What is compared with what:
+
+* ``h_cat``, every ``y_i`` and ``gh_cat`` against the member-by-member entry points: bit for bit (the group kernels sum
+  in the same order);
+* ``grad A_i`` / ``grad B_i`` against the member-by-member call: the fp32 partial sums are taken over row ranges chosen
+  for the whole batch, so the values agree up to the order of fp32 additions (rtol 1e-2, atol 1e-2 of the largest
+  entry; both sides are bf16 roundings of fp32 sums of the same products);
+* the grouped grad-input against an fp32 evaluation on the bit-exact dequantised weights (rtol 1e-2 / atol scaled like
+  the per-linear tests) and against the sum of the member-by-member results (which rounds each member to bf16 first:
+  the grouped value must be at least as close to the fp32 evaluation);
+* the module-level function against the CPU oracle's unfused graph of the same layers (rtol 1e-2 / atol 1e-2, the bar of
+  the per-linear tests), and against calling the layers one by one.
+"""
+import pytest
+import torch
+
+from oracle import lora_oracle, nf4_oracle
+from torchtune_amd import ops
+from torchtune_amd.modules.peft import LoRALinear, group_applies, lora_linear_group
+from torchtune_amd.nf4_tensor import to_nf4
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+BF = torch.bfloat16
+
+
+def _members(K, Ns, ranks, seed, bias=False):
+    g = torch.Generator().manual_seed(seed)
+    out = []
+    for N, r in zip(Ns, ranks):
+        W = (torch.randn(N, K, generator=g) * 0.02).to(BF)
+        A = lora_oracle.lora_a_init_(torch.empty(r, K), g).to(BF)
+        B = (torch.randn(N, r, generator=g) * 0.01).to(BF)
+        b = (torch.randn(N, generator=g) * 0.1).to(BF) if bias else None
+        t = to_nf4(W.to(DEV))
+        m = ops.GroupMember(t.quantized_data, t.block_scalers(), t.backward_copy(), A.to(DEV), B.to(DEV),
+                            b.to(DEV) if bias else None, 32.0 / r, N)
+        out.append((m, t, W, A, B, b))
+    return out
+
+
+SHAPES = [
+    # M, K, Ns, ranks
+    (1, 512, (256, 64, 64), (8, 8, 8)),
+    (16, 1024, (512, 128, 128), (16, 16, 16)),
+    (33, 2048, (8192, 8192), (16, 16)),            # wide members: two row tiles per workgroup
+    (64, 8192, (512, 64, 64), (8, 16, 8)),          # deep contraction: sixteen waves
+    (40, 1024, (8192, 256), (16, 16)),              # members with different launch shapes: two launches
+    (200, 512, (256, 128, 128), (16, 16, 16)),      # tiled kernels, sliced contraction
+    (1000, 1024, (512, 256, 256, 64), (32, 16, 8, 8)),
+    (4096, 1024, (1024, 256, 256), (16, 16, 16)),   # 256-row tiles, unsliced rank-r products
+    (2048, 256, (4096, 4096), (32, 32)),
+]
+
+
+@pytest.mark.parametrize("M,K,Ns,ranks", SHAPES, ids=[f"M{s[0]}_K{s[1]}_{'x'.join(map(str, s[2]))}_r{'x'.join(map(str, s[3]))}" for s in SHAPES])
+@pytest.mark.parametrize("bias", [False, True], ids=["nobias", "bias"])
+def test_group_forward_matches_member_calls_bitwise(M, K, Ns, ranks, bias):
+    mem = _members(K, Ns, ranks, seed=M + K, bias=bias)
+    x = torch.randn(M, K, generator=torch.Generator().manual_seed(7)).to(BF).to(DEV)
+    h_cat, ys = ops.lora_group_fwd(x, [m[0] for m in mem])
+    off = 0
+    for (m, t, *_), y in zip(mem, ys):
+        r = m.lora_a.shape[0]
+        h = ops.lora_hidden(x, m.lora_a)
+        assert torch.equal(h_cat[:, off:off + r], h), "hidden activation"
+        y1 = ops.nf4_lora_linear_fwd(x, m.qdata, m.block_scalers, m.N, h, m.lora_b, m.scale, m.bias,
+                                     block_scalers_t=m.transposed[1])
+        assert torch.equal(y, y1), "member output"
+        off += r
+    assert off == h_cat.shape[1]
+
+
+@pytest.mark.parametrize("M,K,Ns,ranks", SHAPES, ids=[f"M{s[0]}_K{s[1]}_{'x'.join(map(str, s[2]))}_r{'x'.join(map(str, s[3]))}" for s in SHAPES])
+def test_group_backward_against_member_calls_and_fp32(M, K, Ns, ranks):
+    mem = _members(K, Ns, ranks, seed=3 * M + K)
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(M, K, generator=g).to(BF).to(DEV)
+    gys = [torch.randn(M, N, generator=g).to(BF).to(DEV) for N in Ns]
+    members = [m[0] for m in mem]
+    h_cat, _ = ops.lora_group_fwd(x, members)
+    gx, grads, gh_cat = ops.lora_group_bwd(x, h_cat, members, gys)
+
+    ref_gx = torch.zeros(M, K, dtype=torch.float32, device=DEV)
+    sum_members = None
+    off = 0
+    for (m, t, *_), gy, (ga, gb) in zip(mem, gys, grads):
+        r = m.lora_a.shape[0]
+        h = h_cat[:, off:off + r].contiguous()
+        gh1, ga1, gb1 = ops.lora_bwd(gy, x, h, m.lora_b, m.scale)
+        assert torch.equal(gh_cat[:, off:off + r], gh1), "hidden gradient"
+        for got, want in ((ga, ga1), (gb, gb1)):
+            torch.testing.assert_close(got.float(), want.float(), rtol=1e-2, atol=1e-2 * float(want.float().abs().max()) + 1e-30)
+        # the adapter gradients against fp32 matmuls as well
+        want_a = gh1.float().T @ x.float()
+        want_b = m.scale * (gy.float().T @ h.float())
+        torch.testing.assert_close(ga.float(), want_a, rtol=2e-2, atol=2e-2 * float(want_a.abs().max()) + 1e-30)
+        torch.testing.assert_close(gb.float(), want_b, rtol=2e-2, atol=2e-2 * float(want_b.abs().max()) + 1e-30)
+        gx1 = ops.nf4_linear_bwd_dx(gy, m.qdata, m.block_scalers, K, gh1, m.lora_a, transposed=m.transposed)
+        sum_members = gx1 if sum_members is None else sum_members + gx1
+        ref_gx += gy.float() @ t.get_original_weight().float() + gh1.float() @ m.lora_a.float()
+        off += r
+    scale = max(1.0, float(ref_gx.abs().max()) / 8)
+    torch.testing.assert_close(gx.float(), ref_gx, rtol=1e-2, atol=1e-2 * scale)
+    torch.testing.assert_close(gx.float(), sum_members.float(), rtol=2e-2, atol=2e-2 * scale)
+    # one rounding instead of one per member and per addition: no further from the fp32 evaluation
+    err_group = float((gx.float() - ref_gx).abs().mean())
+    err_members = float((sum_members.float() - ref_gx).abs().mean())
+    assert err_group <= err_members * 1.001 + 1e-12
+    # deterministic
+    gx2, grads2, _ = ops.lora_group_bwd(x, h_cat, members, gys)
+    assert torch.equal(gx, gx2) and all(torch.equal(a, c) and torch.equal(b, d) for (a, b), (c, d) in zip(grads, grads2))
+
+
+def _layers(K, Ns, ranks, alpha, bias, seed):
+    layers = []
+    g = torch.Generator().manual_seed(seed)
+    prev = torch.get_default_dtype()
+    torch.set_default_dtype(BF)
+    try:
+        with torch.device(DEV):
+            for N, r in zip(Ns, ranks):
+                layers.append(LoRALinear(K, N, rank=r, alpha=alpha, use_bias=bias, quantize_base=True))
+    finally:
+        torch.set_default_dtype(prev)
+    params = []
+    with torch.no_grad():
+        for layer, N, r in zip(layers, Ns, ranks):
+            W = (torch.randn(N, K, generator=g) * 0.02).to(BF)
+            A = lora_oracle.lora_a_init_(torch.empty(r, K), g).to(BF)
+            B = (torch.randn(N, r, generator=g) * 0.01).to(BF)
+            b = (torch.randn(N, generator=g) * 0.1).to(BF) if bias else None
+            layer.weight.copy_(W.to(DEV))
+            layer.lora_a.weight.copy_(A.to(DEV))
+            layer.lora_b.weight.copy_(B.to(DEV))
+            if bias:
+                layer.bias.copy_(b.to(DEV))
+            params.append((W, A, B, b))
+    return layers, params
+
+
+@pytest.mark.parametrize("M,K,Ns,ranks,bias", [
+    (8, 512, (256, 64, 64), (8, 8, 8), False),
+    (300, 512, (256, 128, 128), (16, 16, 16), True),
+    (520, 1024, (512, 512), (16, 16), False),
+], ids=["decode_qkv", "qkv_bias", "gate_up"])
+def test_module_group_against_oracle_and_layerwise(M, K, Ns, ranks, bias):
+    alpha = 32.0
+    layers, params = _layers(K, Ns, ranks, alpha, bias, seed=M)
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(M, K, generator=g).to(BF)
+    gys = [torch.randn(M, N, generator=g).to(BF) for N in Ns]
+    xg = x.to(DEV).requires_grad_()
+    assert group_applies(xg, layers)
+    ys = lora_linear_group(xg, layers)
+    torch.autograd.backward(ys, [gy.to(DEV) for gy in gys])
+    got = {"gx": xg.grad.clone(), "ga": [l.lora_a.weight.grad.clone() for l in layers],
+           "gb": [l.lora_b.weight.grad.clone() for l in layers],
+           "gbias": [l.bias.grad.clone() if bias else None for l in layers]}
+
+    # ---- layer by layer through the per-linear path
+    for l in layers:
+        l.zero_grad()
+    xl = x.to(DEV).requires_grad_()
+    yl = [l(xl) for l in layers]
+    torch.autograd.backward(yl, [gy.to(DEV) for gy in gys])
+    for a, b in zip(ys, yl):
+        assert torch.equal(a, b)
+    scale = max(1.0, float(xl.grad.float().abs().max()) / 8)
+    torch.testing.assert_close(got["gx"].float(), xl.grad.float(), rtol=2e-2, atol=2e-2 * scale)
+    for i, l in enumerate(layers):
+        for mine, theirs in ((got["ga"][i], l.lora_a.weight.grad), (got["gb"][i], l.lora_b.weight.grad)):
+            torch.testing.assert_close(mine.float(), theirs.float(), rtol=1e-2, atol=1e-2 * float(theirs.float().abs().max()) + 1e-30)
+        if bias:
+            assert torch.equal(got["gbias"][i], l.bias.grad)
+
+    # ---- the CPU oracle: the reference's unfused bf16 graph of the same layers on the same input
+    xo = x.clone().requires_grad_()
+    outs, leaves = [], []
+    for (W, A, B, b), r in zip(params, ranks):
+        n_blocks = W.numel() // 64
+        p = nf4_oracle.nf4_quantize(W, 64, 256 if n_blocks % 256 == 0 else n_blocks)
+        Ao, Bo = A.clone().requires_grad_(), B.clone().requires_grad_()
+        outs.append(lora_oracle.lora_linear_forward(xo, p, Ao, Bo, alpha, r, bias=b))
+        leaves.append((Ao, Bo))
+    torch.autograd.backward(outs, gys)
+    for y, yo in zip(ys, outs):
+        torch.testing.assert_close(y.detach().cpu().float(), yo.detach().float(), rtol=1e-2, atol=1e-2)
+    sc = max(1.0, float(xo.grad.float().abs().max()) / 8)
+    torch.testing.assert_close(got["gx"].cpu().float(), xo.grad.float(), rtol=1e-2, atol=2e-2 * sc)
+    for i, (Ao, Bo) in enumerate(leaves):
+        for mine, theirs in ((got["ga"][i], Ao.grad), (got["gb"][i], Bo.grad)):
+            torch.testing.assert_close(mine.cpu().float(), theirs.float(), rtol=2e-2, atol=2e-2 * float(theirs.float().abs().max()) + 1e-30)
+
+
+def test_group_falls_back_when_it_does_not_apply():
+    layers, _ = _layers(512, (256, 128), (16, 16), 32.0, False, seed=1)
+    x = torch.randn(4, 512, device=DEV, dtype=BF)
+    layers[1].disabled = True
+    assert not group_applies(x, layers)
+    ys = lora_linear_group(x, layers)
+    assert torch.equal(ys[0], layers[0](x)) and torch.equal(ys[1], layers[1](x))
+    layers[1].disabled = False
+    assert group_applies(x, layers)
+    assert not group_applies(x.float(), layers)
+    five, _ = _layers(512, (64,) * 5, (8,) * 5, 16.0, False, seed=2)
+    assert not group_applies(x, five)
+    big_ranks, _ = _layers(512, (64, 64), (64, 8), 16.0, False, seed=3)
+    assert not group_applies(x, big_ranks)  # ranks sum to more than 64
+    assert len(lora_linear_group(x, big_ranks)) == 2
+
+
+def test_group_rejects_mismatched_operands():
+    mem = _members(512, (128, 64), (8, 8), seed=9)
+    members = [m[0] for m in mem]
+    x = torch.randn(8, 512, device=DEV, dtype=BF)
+    with pytest.raises(ValueError):
+        ops.lora_group_fwd(torch.randn(8, 256, device=DEV, dtype=BF), members)
+    bad = ops.GroupMember(members[0].qdata, members[0].block_scalers, members[0].transposed, members[0].lora_a,
+                          members[1].lora_b, None, 1.0, members[0].N)
+    with pytest.raises(ValueError):
+        ops.lora_group_fwd(x, [bad])
+    h_cat, _ = ops.lora_group_fwd(x, members)
+    with pytest.raises(ValueError):
+        ops.lora_group_bwd(x, h_cat[:, :8].contiguous(), members, [torch.zeros(8, 128, device=DEV, dtype=BF),
+                                                                    torch.zeros(8, 64, device=DEV, dtype=BF)])
+    with pytest.raises(ValueError):
+        ops.lora_group_fwd(x, members * 3)  # six members

@@ -85,6 +85,13 @@ SIGNATURES = {
         [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _f32, _c_void_p, _c_void_p, _c_void_p, _i64, _i64, _i64, _int,
          _c_void_p, _size, _c_void_p],
     ),
+    "ttamd_lora_group_hidden_workspace_bytes": (_size, [_c_void_p, _int, _i64, _i64]),
+    "ttamd_lora_group_hidden_bf16": (_int, [_c_void_p, _c_void_p, _int, _c_void_p, _i64, _i64, _c_void_p, _size, _c_void_p]),
+    "ttamd_lora_group_fwd_workspace_bytes": (_size, [_c_void_p, _int, _i64, _i64]),
+    "ttamd_nf4_lora_group_fwd_bf16": (_int, [_c_void_p, _c_void_p, _int, _c_void_p, _i64, _i64, _c_void_p, _size, _c_void_p]),
+    "ttamd_lora_group_bwd_workspace_bytes": (_size, [_c_void_p, _int, _i64, _i64]),
+    "ttamd_lora_group_bwd_bf16": (_int, [_c_void_p, _c_void_p, _c_void_p, _int, _c_void_p, _i64, _i64, _c_void_p, _size, _c_void_p]),
+    "ttamd_nf4_group_bwd_dx_bf16": (_int, [_c_void_p, _int, _c_void_p, _c_void_p, _i64, _i64, _c_void_p]),
     "ttamd_fq_per_token_int8_asym": (_int, [_c_void_p, _int, _i64, _i64, _int, _c_void_p, _c_void_p, _c_void_p, _c_void_p]),
     "ttamd_fq_per_group_int4_sym": (_int, [_c_void_p, _int, _i64, _i64, _int, _int, _c_void_p, _c_void_p, _c_void_p]),
     "ttamd_quantize_per_group_int4": (
@@ -126,6 +133,18 @@ class FqConventions(ctypes.Structure):
 
     _fields_ = [("eps_per_token", ctypes.c_float), ("eps_per_group_sym", ctypes.c_float), ("min_scale_uint4", ctypes.c_float),
                 ("uint4_clamp_range_first", ctypes.c_int)]
+
+
+GROUP_MAX = 4
+
+
+class LoraGroupMember(ctypes.Structure):
+    """``ttamd_lora_group_member`` of the header: one linear of a group that shares its input."""
+
+    _fields_ = [("quantized_data", _c_void_p), ("block_scalers", _c_void_p), ("block_scalers_t", _c_void_p),
+                ("quantized_data_t", _c_void_p), ("lora_a", _c_void_p), ("lora_b", _c_void_p), ("bias", _c_void_p),
+                ("y", _c_void_p), ("grad_lora_a", _c_void_p), ("grad_lora_b", _c_void_p), ("N", _i64), ("rank", _int),
+                ("scale", _f32)]
 
 
 _lock = threading.Lock()

@@ -1,0 +1,158 @@
+// C entry points for a group of QLoRA linears that share their input: q/k/v of an attention layer
+// (torchtune/modules/attention.py:234,262-263 calls q_proj, k_proj and v_proj on the same tensor) and gate/up of a
+// feed-forward (torchtune/modules/feed_forward.py:50-53: w1 and w3).  The reference has no such call: each LoRALinear
+// (torchtune/modules/peft/lora.py:128-147) is on its own there.  What a group saves over member-by-member calls:
+//   forward   one pass over x for every member's h = x . A^T; a handful of tokens: one launch for the members' outputs
+//   backward  one launch for the members' gh, one pass over x for every member's gA, one launch for all gA / gB sums,
+//             one grad-input GEMM over the members' concatenated output columns instead of one GEMM per member plus
+//             the additions of their results
+#include "common.h"
+#include "group.h"
+
+namespace ttamd {
+namespace {
+
+struct Decoded {
+  GroupSkinny sk;
+  GroupGemm gm;
+  GroupDx dx;
+};
+
+size_t align256(size_t v) { return (v + 255) & ~size_t(255); }
+
+int decode(const char* who, const ttamd_lora_group_member* m, int n, int64_t M, int64_t K, bool backward, Decoded& d) {
+  TT_REQUIRE(m != nullptr && n >= 1 && n <= kGroupMax, "%s: a group has 1 to %d members (got %d)", who, kGroupMax, n);
+  TT_REQUIRE(M > 0 && K > 0 && M < (1 << 30) && K < (1 << 30) && K % 64 == 0, "%s: bad shape M=%lld K=%lld (K must be a multiple of 64)",
+             who, (long long)M, (long long)K);
+  d = Decoded{};
+  d.sk.n = d.gm.n = d.dx.n = n;
+  d.sk.M = d.gm.M = d.dx.M = M;
+  d.sk.K = d.gm.K = d.dx.K = K;
+  int off = 0;
+  for (int i = 0; i < n; ++i) {
+    const ttamd_lora_group_member& e = m[i];
+    TT_REQUIRE(e.N > 0 && e.N < (1 << 30) && e.N % 64 == 0, "%s: member %d: N (%lld) must be a positive multiple of 64", who, i, (long long)e.N);
+    TT_REQUIRE(e.rank > 0 && e.rank % 8 == 0, "%s: member %d: rank (%d) must be a positive multiple of 8", who, i, e.rank);
+    TT_REQUIRE(e.quantized_data && e.block_scalers && e.lora_a && e.lora_b && e.y, "%s: member %d: null pointer", who, i);
+    TT_REQUIRE(aligned16(e.quantized_data) && aligned16(e.block_scalers) && aligned16(e.block_scalers_t) && aligned16(e.lora_a) &&
+                   aligned16(e.lora_b) && aligned16(e.y) && (reinterpret_cast<uintptr_t>(e.bias) & 7u) == 0,
+               "%s: member %d: pointers must be 16-byte aligned (bias: 8)", who, i);
+    if (backward) TT_REQUIRE(e.grad_lora_a && e.grad_lora_b, "%s: member %d: null gradient output", who, i);
+    d.sk.N[i] = d.gm.N[i] = d.dx.N[i] = e.N;
+    d.sk.rank[i] = d.gm.rank[i] = d.dx.rank[i] = e.rank;
+    d.sk.r_off[i] = d.gm.r_off[i] = d.dx.r_off[i] = off;
+    off += e.rank;
+    d.sk.scale[i] = d.gm.scale[i] = e.scale;
+    d.sk.lora_a[i] = d.dx.lora_a[i] = reinterpret_cast<const uint16_t*>(e.lora_a);
+    d.sk.lora_b[i] = d.gm.lora_b[i] = reinterpret_cast<const uint16_t*>(e.lora_b);
+    d.sk.gy[i] = d.dx.gy[i] = reinterpret_cast<const uint16_t*>(e.y);
+    d.sk.ga[i] = reinterpret_cast<uint16_t*>(e.grad_lora_a);
+    d.sk.gb[i] = reinterpret_cast<uint16_t*>(e.grad_lora_b);
+    d.gm.codes[i] = e.quantized_data;
+    d.gm.bscal[i] = reinterpret_cast<const float*>(e.block_scalers);
+    d.gm.bscal_t[i] = reinterpret_cast<const float*>(e.block_scalers_t);
+    d.gm.bias[i] = reinterpret_cast<const uint16_t*>(e.bias);
+    d.gm.y[i] = reinterpret_cast<uint16_t*>(e.y);
+    d.dx.codes_t[i] = e.quantized_data_t;
+    d.dx.scal_t[i] = reinterpret_cast<const float*>(e.block_scalers_t);
+  }
+  TT_REQUIRE(off <= 64, "%s: the ranks of a group sum to at most 64 (got %d)", who, off);
+  d.sk.r_off[n] = d.gm.r_off[n] = d.dx.r_off[n] = off;
+  return TTAMD_OK;
+}
+
+// slices of the largest sliced member GEMM
+size_t fwd_gemm_ws(const Decoded& d) {
+  size_t w = 0;
+  if (d.gm.M > small_m_limit())
+    for (int i = 0; i < d.gm.n; ++i) {
+      const size_t b = gemm_rs_workspace_bytes(d.gm.M, d.gm.N[i], d.gm.K);
+      w = b > w ? b : w;
+    }
+  return w;
+}
+
+}  // namespace
+}  // namespace ttamd
+
+using namespace ttamd;
+
+extern "C" size_t ttamd_lora_group_hidden_workspace_bytes(const ttamd_lora_group_member* members, int n_members, int64_t M,
+                                                          int64_t K) {
+  Decoded d;
+  if (decode("lora_group_hidden_workspace_bytes", members, n_members, M, K, false, d) != TTAMD_OK) return 0;
+  return align256(group_hidden_ws_bytes(M, K, d.sk.r_off[d.sk.n]));
+}
+
+extern "C" int ttamd_lora_group_hidden_bf16(const void* x, const ttamd_lora_group_member* members, int n_members, void* h_cat,
+                                            int64_t M, int64_t K, void* workspace, size_t workspace_bytes, void* stream) {
+  Decoded d;
+  if (int rc = decode("lora_group_hidden", members, n_members, M, K, false, d)) return rc;
+  TT_REQUIRE(x && h_cat && aligned16(x) && aligned16(h_cat), "lora_group_hidden: x and h_cat must be non-null and 16-byte aligned");
+  const size_t need = align256(group_hidden_ws_bytes(M, K, d.sk.r_off[d.sk.n]));
+  if (need > 0) {
+    TT_REQUIRE(workspace && aligned16(workspace), "lora_group_hidden: workspace must be non-null and 16-byte aligned");
+    if (workspace_bytes < need)
+      return fail(TTAMD_EWORKSPACE, "lora_group_hidden: workspace has %zu bytes, needs %zu", workspace_bytes, need);
+  }
+  return run_group_hidden(reinterpret_cast<const uint16_t*>(x), d.sk, reinterpret_cast<uint16_t*>(h_cat),
+                          reinterpret_cast<float*>(workspace), reinterpret_cast<hipStream_t>(stream));
+}
+
+extern "C" size_t ttamd_lora_group_fwd_workspace_bytes(const ttamd_lora_group_member* members, int n_members, int64_t M, int64_t K) {
+  Decoded d;
+  if (decode("lora_group_fwd_workspace_bytes", members, n_members, M, K, false, d) != TTAMD_OK) return 0;
+  return align256(fwd_gemm_ws(d));
+}
+
+extern "C" int ttamd_nf4_lora_group_fwd_bf16(const void* x, const ttamd_lora_group_member* members, int n_members,
+                                             const void* h_cat, int64_t M, int64_t K, void* workspace, size_t workspace_bytes,
+                                             void* stream) {
+  Decoded d;
+  if (int rc = decode("nf4_lora_group_fwd", members, n_members, M, K, false, d)) return rc;
+  TT_REQUIRE(x && h_cat && aligned16(x) && aligned16(h_cat), "nf4_lora_group_fwd: x and h_cat must be non-null and 16-byte aligned");
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (M <= small_m_limit()) return run_small_m_group(x, d.gm, h_cat, s);
+  // slices of the contraction for a member with few output tiles, when the caller brought the memory for them
+  const size_t gem = align256(fwd_gemm_ws(d));
+  const bool sliced = gem > 0 && workspace != nullptr && workspace_bytes >= gem;
+  TT_REQUIRE(!sliced || aligned16(workspace), "nf4_lora_group_fwd: workspace must be 16-byte aligned");
+  const int ldh = d.gm.r_off[d.gm.n];
+  for (int i = 0; i < d.gm.n; ++i) {
+    const void* sc = d.gm.bscal_t[i] ? d.gm.bscal_t[i] : d.gm.bscal[i];
+    if (int rc = run_gemm_rs(x, d.gm.codes[i], sc, d.gm.bscal_t[i] ? 2 : 0, reinterpret_cast<const uint16_t*>(h_cat) + d.gm.r_off[i], ldh,
+                             d.gm.lora_b[i], true, d.gm.rank[i], d.gm.scale[i], d.gm.bias[i], nullptr, d.gm.y[i], M, d.gm.N[i], K,
+                             sliced ? workspace : nullptr, sliced ? workspace_bytes : 0, s))
+      return rc;
+  }
+  return TTAMD_OK;
+}
+
+extern "C" size_t ttamd_lora_group_bwd_workspace_bytes(const ttamd_lora_group_member* members, int n_members, int64_t M, int64_t K) {
+  Decoded d;
+  if (decode("lora_group_bwd_workspace_bytes", members, n_members, M, K, false, d) != TTAMD_OK) return 0;
+  return group_lora_bwd_ws_bytes(d.sk);
+}
+
+extern "C" int ttamd_lora_group_bwd_bf16(const void* x, const void* h_cat, const ttamd_lora_group_member* members, int n_members,
+                                         void* gh_cat, int64_t M, int64_t K, void* workspace, size_t workspace_bytes, void* stream) {
+  Decoded d;
+  if (int rc = decode("lora_group_bwd", members, n_members, M, K, true, d)) return rc;
+  TT_REQUIRE(x && h_cat && gh_cat && workspace, "lora_group_bwd: null pointer argument");
+  TT_REQUIRE(aligned16(x) && aligned16(h_cat) && aligned16(gh_cat) && aligned16(workspace), "lora_group_bwd: pointers must be 16-byte aligned");
+  const size_t need = group_lora_bwd_ws_bytes(d.sk);
+  if (workspace_bytes < need) return fail(TTAMD_EWORKSPACE, "lora_group_bwd: workspace has %zu bytes, needs %zu", workspace_bytes, need);
+  return run_group_lora_bwd(reinterpret_cast<const uint16_t*>(x), reinterpret_cast<const uint16_t*>(h_cat), d.sk,
+                            reinterpret_cast<uint16_t*>(gh_cat), reinterpret_cast<float*>(workspace), reinterpret_cast<hipStream_t>(stream));
+}
+
+extern "C" int ttamd_nf4_group_bwd_dx_bf16(const ttamd_lora_group_member* members, int n_members, const void* gh_cat, void* gx,
+                                           int64_t M, int64_t K, void* stream) {
+  Decoded d;
+  if (int rc = decode("nf4_group_bwd_dx", members, n_members, M, K, false, d)) return rc;
+  TT_REQUIRE(gh_cat && gx && aligned16(gh_cat) && aligned16(gx), "nf4_group_bwd_dx: gh_cat and gx must be non-null and 16-byte aligned");
+  for (int i = 0; i < n_members; ++i)
+    TT_REQUIRE(d.dx.codes_t[i] && d.dx.scal_t[i] && aligned16(d.dx.codes_t[i]),
+               "nf4_group_bwd_dx: member %d: needs the transposed copies (ttamd_nf4_transpose_for_backward), 16-byte aligned", i);
+  return run_gemm_rs_group_dx(d.dx, gh_cat, gx, reinterpret_cast<hipStream_t>(stream));
+}

@@ -13,6 +13,7 @@
 // put enough loads in flight and combine the fp32 partial sums in a second, fixed-order pass, so results
 // are deterministic.
 #include "common.h"
+#include "group.h"
 #include "nf4_math.h"
 
 namespace ttamd {
@@ -44,12 +45,39 @@ __device__ __forceinline__ u32x2_t lds_read_tr16(uint32_t addr, int imm) {
   return v;
 }
 
+constexpr int kMaxGroup = kGroupMax;
+
+// One column contraction.  The R rows of the second operand may be stacked from several matrices (the adapters of a
+// group's members): rows [r_off[b], r_off[b + 1]) are the rows of bm[b].  A launch takes a batch of problems over the
+// same M (blockIdx.z), each with its own operands, width, slicing and output columns.
+struct NtProblem {
+  const uint16_t* X;              // [M, Kc]
+  const uint16_t* bm[kMaxGroup];  // BT: bm[0] is [Kc, R]; otherwise bm[b] is [r_off[b + 1] - r_off[b], Kc]
+  int r_off[kMaxGroup + 1];
+  int nb;                         // matrices in bm
+  float* part;                    // [splits, M, R] fp32, used when splits > 1
+  uint16_t* out;                  // bf16 rows `ldo` elements apart; the problem's R columns start here
+  int Kc, R, ldo, splits, chunks_per_split;
+  float scale;
+};
+struct NtBatch {
+  NtProblem p[kMaxGroup];
+  int M;
+};
+
 template <int RT, bool BT>
-__global__ __launch_bounds__(256) void skinny_nt_kernel(const uint16_t* __restrict__ X, const uint16_t* __restrict__ Bm,
-                                                        float* __restrict__ part, int M, int Kc, int R,
-                                                        int chunks_per_split, uint16_t* __restrict__ direct_out,
-                                                        float scale) {
-  // direct_out != null (only with a single split): write bf16(scale * sum) straight to the [M, R] output
+__global__ __launch_bounds__(256) void skinny_nt_kernel(const NtBatch a) {
+  const NtProblem& P = a.p[blockIdx.z];
+  const int split = blockIdx.y;
+  if (split >= P.splits) return;  // the batch's grid is as deep as its most sliced problem
+  const uint16_t* __restrict__ X = P.X;
+  const uint16_t* __restrict__ Bm = P.bm[0];
+  float* __restrict__ part = P.part;
+  const int M = a.M, Kc = P.Kc, R = P.R, chunks_per_split = P.chunks_per_split;
+  // a single slice writes bf16(scale * sum) straight to the output
+  uint16_t* __restrict__ direct_out = P.splits == 1 ? P.out : nullptr;
+  const int ldo = P.ldo;
+  const float scale = P.scale;
   __shared__ float red[3][2 * RT * 4][64];
   constexpr int kPitchB = 32 * RT;  // bytes per LDS row of the transposed-operand piece: 16 RT columns
   __shared__ __attribute__((aligned(16))) char bstage[BT ? 4 * 64 * kPitchB : 16];
@@ -57,7 +85,6 @@ __global__ __launch_bounds__(256) void skinny_nt_kernel(const uint16_t* __restri
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int g = lane >> 4, i = lane & 15;
   const int m0 = blockIdx.x * 32;
-  const int split = blockIdx.y;
   char* myb = bstage + (BT ? wave * 64 * kPitchB : 0);
   const uint32_t brd = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)myb) + (16 * g + (i >> 2)) * kPitchB + 8 * (i & 3);
   const uint16_t* xrow[2];
@@ -73,7 +100,12 @@ __global__ __launch_bounds__(256) void skinny_nt_kernel(const uint16_t* __restri
   for (int t = 0; t < RT; ++t) {
     const int r = t * 16 + i;
     bvalid[t] = r < R;
-    brow[t] = Bm + (int64_t)(bvalid[t] ? r : 0) * Kc + 16 * g;
+    brow[t] = Bm + 16 * g;
+    if (!BT && bvalid[t]) {
+#pragma unroll
+      for (int b = 0; b < kMaxGroup; ++b)
+        if (b < P.nb && r >= P.r_off[b] && r < P.r_off[b + 1]) brow[t] = P.bm[b] + (int64_t)(r - P.r_off[b]) * Kc + 16 * g;
+    }
   }
   f32x4_t acc[2][RT];
 #pragma unroll
@@ -207,7 +239,7 @@ __global__ __launch_bounds__(256) void skinny_nt_kernel(const uint16_t* __restri
           if (r >= M) continue;
           const float sum = ((acc[t][u][v] + red[0][e][lane]) + red[1][e][lane]) + red[2][e][lane];
           if (direct_out)
-            direct_out[(int64_t)r * R + col] = f32_to_bf16_bits(sum * scale);
+            direct_out[(int64_t)r * ldo + col] = f32_to_bf16_bits(sum * scale);
           else
             part[((int64_t)split * M + r) * R + col] = sum;
         }
@@ -215,57 +247,71 @@ __global__ __launch_bounds__(256) void skinny_nt_kernel(const uint16_t* __restri
   }
 }
 
-// out[i] = bf16(scale * sum_s part[s][i]) for i < n (out and part share the [M,R] layout)
-__global__ __launch_bounds__(256) void sum_partials_kernel(const float* __restrict__ part, int64_t n, int splits, float scale,
-                                                           uint16_t* __restrict__ out) {
+// The second pass of the sliced problems of a batch (blockIdx.y = problem): out[m][c] = bf16(scale * sum_s part[s][m][c])
+__global__ __launch_bounds__(256) void sum_partials_kernel(const NtBatch a) {
+  const NtProblem& P = a.p[blockIdx.y];
+  if (P.splits == 1) return;  // written directly by the first pass
+  const int64_t n = (int64_t)a.M * P.R;
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (i >= n) return;
   float s = 0.f;
 #pragma unroll 8
-  for (int p = 0; p < splits; ++p) s += part[(int64_t)p * n + i];
-  out[i] = f32_to_bf16_bits(s * scale);
+  for (int p = 0; p < P.splits; ++p) s += P.part[(int64_t)p * n + i];
+  P.out[(i / P.R) * P.ldo + i % P.R] = f32_to_bf16_bits(s * P.scale);
 }
 
 // ---------------------------------------------------------------------------------------------------
-// skinny_tn: part[split][r0 + r][c] = sum_{m in split} G[m][r0 + r] * X[m][c]   (G [M,R], X [M,Kc], r < 16)
+// skinny_tn: part[split][r][c] = sum_{m in split} G[m][r] * X[m][c]   (G [M,R], X [M,Kc], R <= 64)
 // The contraction runs over rows.  The fp32 MFMA v_mfma_f32_16x16x4_f32 takes one contraction index per lane and
 // could read both operands as they lie in memory, but it consumes only 64 elements of X per 32-cycle instruction,
 // which caps a kernel built on it near the HBM rate (measured: 3.7 - 4.8 TB/s).  v_mfma_f32_16x16x32_bf16
 // takes 512, but wants 8 consecutive contraction indices (rows m) of one column in a lane, while memory has 8
 // consecutive columns of one row.  The transposition is done by the LDS: a wave copies its 32 rows x 128 columns of X
-// (and the matching 32 x 16 piece of G) row-major into a private LDS region and reads them back with
-// ds_read_b64_tr_b16.  In a 16-lane group that instruction returns to lane i, as element t, the 16-bit element
-// (i % 4) of the 8 bytes that lane 4 t + i / 4 points at; with lane j pointing at row j / 4, columns 4 (j % 4) .. + 3
-// of a 4 x 16 piece, lane i receives column i of rows 0 .. 3: exactly an MFMA operand.
+// (and the matching 32 x R piece of G, in groups of 16 columns) row-major into a private LDS region and reads them
+// back with ds_read_b64_tr_b16.  In a 16-lane group that instruction returns to lane i, as element t, the 16-bit
+// element (i % 4) of the 8 bytes that lane 4 t + i / 4 points at; with lane j pointing at row j / 4, columns
+// 4 (j % 4) .. + 3 of a 4 x 16 piece, lane i receives column i of rows 0 .. 3: exactly an MFMA operand.
+// All R columns of G (up to four groups of 16) are multiplied in the one pass over X.
 // Workgroup = 4 waves on the same 128 columns; wave w takes the 32-row steps w, w + 4, ... of the split.  The partial
-// sums are combined through LDS in a fixed order, then across splits by sum_partials_tn_pair_kernel.
+// sums are combined through LDS in a fixed order, then across splits by sum_partials_tn_kernel.
 // ---------------------------------------------------------------------------------------------------
 constexpr int kTnCols = 128;    // columns per workgroup
+constexpr int kTnMaxRG = 4;     // groups of 16 columns of G
 constexpr int kTrPitchX = 288;  // bytes per LDS row of the X piece: 256 + 32, so that 4 consecutive rows fall on disjoint banks
-constexpr int kTrWaveLds = 32 * kTrPitchX + 32 * 32;  // X piece + G piece (32 rows x 16 bf16)
+constexpr int tn_wave_lds(int rgm) { return 32 * kTrPitchX + rgm * 32 * 32; }  // X piece + G pieces (32 rows x 16 bf16 each)
 
-// One launch serves the two row contractions of a LoRA backward (gA over x, gB over gy): they share M, R and the row
-// splits, and differ in the operands and the width.  Workgroups [0, col_groups0) belong to problem 0, the rest to 1.
+// One launch serves every row contraction of a backward that shares M and the row splits: gA over x (for a group of
+// layers with a common input: the members' gh side by side as one G) and one gB over gy per layer.  They differ in
+// the operands and the width; a workgroup finds its problem from its x index.
 struct TnProblem {
-  const uint16_t* G;  // [M, R]
+  const uint16_t* G;  // rows `ldg` elements apart; the problem's R columns start here
   const uint16_t* X;  // [M, Kc]
   float* part;        // [splits, R, Kc]
-  int Kc;
+  int Kc, R, ldg;
 };
-struct TnPair {
-  TnProblem p[2];
-  int col_groups0;
-  int M, R, r0, rows_per_split;
+constexpr int kTnMaxProblems = 1 + kMaxGroup;
+struct TnBatch {
+  TnProblem p[kTnMaxProblems];
+  int cg_end[kTnMaxProblems];  // workgroups [cg_end[i - 1], cg_end[i]) along x work on problem i
+  int n, M, rows_per_split;
 };
 
-__global__ __launch_bounds__(256) void skinny_tn_kernel(const TnPair a) {
+// RGM: most column groups of G any problem of the batch has (registers and LDS are sized for it)
+template <int RGM>
+__global__ __launch_bounds__(256) void skinny_tn_kernel(const TnBatch a) {
+  constexpr int kTrWaveLds = tn_wave_lds(RGM);
 #if defined(__HIP_DEVICE_COMPILE__)
-  const int which = (int)blockIdx.x >= a.col_groups0 ? 1 : 0;  // uniform over the workgroup
-  const uint16_t* __restrict__ G = a.p[which].G;
-  const uint16_t* __restrict__ X = a.p[which].X;
-  float* __restrict__ part = a.p[which].part;
-  const int Kc = a.p[which].Kc, M = a.M, R = a.R, r0 = a.r0, rows_per_split = a.rows_per_split;
-  const int col_group = (int)blockIdx.x - (which ? a.col_groups0 : 0);
+  int which = 0;  // uniform over the workgroup
+#pragma unroll
+  for (int q = 0; q < kTnMaxProblems - 1; ++q)
+    if (q < a.n - 1 && (int)blockIdx.x >= a.cg_end[q]) which = q + 1;
+  const TnProblem& P = a.p[which];
+  const uint16_t* __restrict__ G = P.G;
+  const uint16_t* __restrict__ X = P.X;
+  float* __restrict__ part = P.part;
+  const int Kc = P.Kc, M = a.M, R = P.R, ldg = P.ldg, rows_per_split = a.rows_per_split;
+  const int rg = (R + 15) >> 4;  // groups of 16 columns of G in use
+  const int col_group = (int)blockIdx.x - (which ? a.cg_end[which - 1] : 0);
   __shared__ __attribute__((aligned(16))) char stage[4 * kTrWaveLds];
   static_assert(sizeof(stage) >= 3 * 32 * 64 * sizeof(float), "the reduction reuses the staging memory");
   const int lane = threadIdx.x & 63;
@@ -283,22 +329,22 @@ __global__ __launch_bounds__(256) void skinny_tn_kernel(const TnPair a) {
   const bool xcol_ok = xcol < Kc;  // Kc % 8 == 0
   const uint16_t* xsrc = X + (xcol_ok ? xcol : 0);
   char* xdst = my + g * kTrPitchX + 16 * i;
-  // G piece: row lane / 2, half lane % 2 (8 of the 16 adapter columns r0 .. r0 + 15)
-  const int gcol = r0 + 8 * (lane & 1);
-  const bool gcol_ok = gcol < R;  // R % 8 == 0
-  const uint16_t* gsrc = G + (gcol_ok ? gcol : 0);
-  char* gdst = my + 32 * kTrPitchX + (lane >> 1) * 32 + 16 * (lane & 1);
+  // G piece of column group q: row lane / 2, half lane % 2 (8 of the group's 16 columns)
+  const int gcol = 8 * (lane & 1);  // + 16 q;  R % 8 == 0: a lane's 8 columns are all in or all out
+  char* gdst = my + 32 * kTrPitchX + (lane >> 1) * 32 + 16 * (lane & 1);  // + 1024 q
   // read-back roles: lane j = lane % 16 of group g points at row 8 g + j / 4 (+ 4 for the second half of the operand),
   // columns 4 (j % 4) .. + 3 of a 16-column group
   const uint32_t my_lds = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)my);
   const uint32_t xrd = my_lds + (8 * g + (i >> 2)) * kTrPitchX + 8 * (i & 3);
   const uint32_t grd = my_lds + 32 * kTrPitchX + (8 * g + (i >> 2)) * 32 + 8 * (i & 3);
 
-  f32x4_t acc[8];
+  f32x4_t acc[RGM][8];
 #pragma unroll
-  for (int e = 0; e < 8; ++e) acc[e] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  for (int q = 0; q < RGM; ++q)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[q][e] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-  u32x4_t xv[8], gv;
+  u32x4_t xv[8], gv[RGM];
   auto fetch = [&](int m) {  // rows m .. m + 31 into registers
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
@@ -307,8 +353,11 @@ __global__ __launch_bounds__(256) void skinny_tn_kernel(const TnPair a) {
       if (row < m_end && xcol_ok) xv[u] = *reinterpret_cast<const u32x4_t*>(xsrc + (int64_t)row * Kc);
     }
     const int grow = m + (lane >> 1);
-    gv = u32x4_t{0, 0, 0, 0};
-    if (grow < m_end && gcol_ok) gv = *reinterpret_cast<const u32x4_t*>(gsrc + (int64_t)grow * R);
+#pragma unroll
+    for (int q = 0; q < RGM; ++q) {
+      gv[q] = u32x4_t{0, 0, 0, 0};
+      if (grow < m_end && gcol + 16 * q < R) gv[q] = *reinterpret_cast<const u32x4_t*>(G + (int64_t)grow * ldg + gcol + 16 * q);
+    }
   };
   int m = m_begin + 32 * wave;
   if (m < m_end) fetch(m);
@@ -316,79 +365,105 @@ __global__ __launch_bounds__(256) void skinny_tn_kernel(const TnPair a) {
     // the previous step's reads of this region are complete: they were waited for before its MFMAs
 #pragma unroll
     for (int u = 0; u < 8; ++u) *reinterpret_cast<u32x4_t*>(xdst + 4 * u * kTrPitchX) = xv[u];
-    *reinterpret_cast<u32x4_t*>(gdst) = gv;
+#pragma unroll
+    for (int q = 0; q < RGM; ++q) *reinterpret_cast<u32x4_t*>(gdst + 1024 * q) = gv[q];  // zeros beyond R
     if (m + 128 < m_end) fetch(m + 128);  // in flight while this step is multiplied
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the copy-in has landed (LDS operations of a wave complete in order)
-    u32x2_t ga = lds_read_tr16(grd, 0), gb = lds_read_tr16(grd, 4 * 32);
+    u32x2_t ga[RGM], gb[RGM];
+#pragma unroll
+    for (int q = 0; q < RGM; ++q) {
+      ga[q] = lds_read_tr16(grd, 1024 * q);
+      gb[q] = lds_read_tr16(grd, 1024 * q + 4 * 32);
+    }
+    // a wait that names the registers it releases, so that no use can be scheduled ahead of it
+#pragma unroll
+    for (int q = 0; q < RGM; ++q) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(ga[q]), "+v"(gb[q]));
     u32x2_t xa[8], xb[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       xa[e] = lds_read_tr16(xrd, 32 * e);
       xb[e] = lds_read_tr16(xrd, 32 * e + 4 * kTrPitchX);
     }
-    // The 18 reads return in order.  Each wait names the registers it releases, so that no use can be scheduled
-    // ahead of it: column group e may go once at most 14 - 2 e younger reads are outstanding.
-    asm volatile("s_waitcnt lgkmcnt(14)" : "+v"(ga), "+v"(gb), "+v"(xa[0]), "+v"(xb[0]));
-    const u32x4_t gop = {ga.x, ga.y, gb.x, gb.y};
+    // The 16 reads return in order: column group e may go once at most 14 - 2 e younger reads are outstanding.
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      if (e > 0) asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(xa[e]), "+v"(xb[e]) : "n"(14 - 2 * e));
+      asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(xa[e]), "+v"(xb[e]) : "n"(14 - 2 * e));
       const u32x4_t xop = {xa[e].x, xa[e].y, xb[e].x, xb[e].y};
-      acc[e] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, gop), __builtin_bit_cast(bf16x8_t, xop),
-                                                      acc[e], 0, 0, 0);
+#pragma unroll
+      for (int q = 0; q < RGM; ++q) {
+        if (q < rg) {
+          const u32x4_t gop = {ga[q].x, ga[q].y, gb[q].x, gb[q].y};
+          acc[q][e] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, gop),
+                                                             __builtin_bit_cast(bf16x8_t, xop), acc[q][e], 0, 0, 0);
+        }
+      }
     }
   }
-  __syncthreads();  // the staging regions are free: the partial sums meet in them
   float (*red)[32][64] = reinterpret_cast<float (*)[32][64]>(stage);
-  // acc[e][v] = sum over this wave's rows of G[.][r0 + 4 g + v] * X[.][c0 + 16 e + i]
-  if (wave > 0) {
+  // acc[q][e][v] = sum over this wave's rows of G[.][16 q + 4 g + v] * X[.][c0 + 16 e + i]; one column group of G at a
+  // time meets in the staging memory
+  for (int q = 0; q < rg; ++q) {
+    __syncthreads();  // the staging regions (or the previous group's sums) are free
+    if (wave > 0) {
 #pragma unroll
-    for (int e = 0; e < 8; ++e)
+      for (int e = 0; e < 8; ++e)
 #pragma unroll
-      for (int v = 0; v < 4; ++v) red[wave - 1][v * 8 + e][lane] = acc[e][v];
-  }
-  __syncthreads();
-  if (wave == 0) {
+        for (int v = 0; v < 4; ++v) {
+          float val = acc[0][e][v];
 #pragma unroll
-    for (int v = 0; v < 4; ++v) {
-      const int r = r0 + 4 * g + v;
-      if (r >= R) continue;
+          for (int qq = 1; qq < RGM; ++qq) val = q == qq ? acc[qq][e][v] : val;
+          red[wave - 1][v * 8 + e][lane] = val;
+        }
+    }
+    __syncthreads();
+    if (wave == 0) {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const int col = c0 + 16 * e + i;
-        if (col >= Kc) continue;
-        part[((int64_t)split * R + r) * Kc + col] =
-            ((acc[e][v] + red[0][v * 8 + e][lane]) + red[1][v * 8 + e][lane]) + red[2][v * 8 + e][lane];
+      for (int v = 0; v < 4; ++v) {
+        const int r = 16 * q + 4 * g + v;
+        if (r >= R) continue;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const int col = c0 + 16 * e + i;
+          if (col >= Kc) continue;
+          float mine = acc[0][e][v];
+#pragma unroll
+          for (int qq = 1; qq < RGM; ++qq) mine = q == qq ? acc[qq][e][v] : mine;
+          part[((int64_t)split * R + r) * Kc + col] =
+              ((mine + red[0][v * 8 + e][lane]) + red[1][v * 8 + e][lane]) + red[2][v * 8 + e][lane];
+        }
       }
     }
   }
 #endif
 }
 
-// out[r*stride_r + k*stride_k] = bf16(scale * sum_s part[s][r][k])
+// out[r * stride_r + k * stride_k] = bf16(scale * sum_s part[s * split_stride + r * Kc + k]) for r < R, k < Kc
 struct TnSum {
   const float* part;
   uint16_t* out;
-  int Kc;
+  int Kc, R;
   float scale;
-  int64_t stride_r, stride_k;
+  int64_t split_stride, stride_r, stride_k;
 };
-struct TnSumPair {
-  TnSum p[2];
-  int64_t n0;  // elements of problem 0: R * Kc
-  int R, splits;
+constexpr int kTnMaxSums = 2 * kMaxGroup;
+struct TnSumBatch {
+  TnSum p[kTnMaxSums];
+  int64_t end[kTnMaxSums];  // threads [end[i - 1], end[i]) finish problem i
+  int n, splits;
 };
-// The reductions of the two row contractions in one launch: thread i < n0 finishes problem 0, the rest problem 1.
-__global__ __launch_bounds__(256) void sum_partials_tn_pair_kernel(const TnSumPair a) {
+// The reductions of every row contraction of a backward in one launch.
+__global__ __launch_bounds__(256) void sum_partials_tn_kernel(const TnSumBatch a) {
   int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  const int which = i >= a.n0 ? 1 : 0;
-  if (which) i -= a.n0;
+  int which = 0;
+#pragma unroll
+  for (int q = 0; q < kTnMaxSums - 1; ++q)
+    if (q < a.n - 1 && i >= a.end[q]) which = q + 1;
+  if (i >= a.end[a.n - 1]) return;
+  if (which) i -= a.end[which - 1];
   const TnSum& P = a.p[which];
-  const int64_t n = (int64_t)a.R * P.Kc;
-  if (i >= n) return;
   float s = 0.f;
 #pragma unroll 8
-  for (int q = 0; q < a.splits; ++q) s += P.part[(int64_t)q * n + i];
+  for (int q = 0; q < a.splits; ++q) s += P.part[(int64_t)q * P.split_stride + i];
   const int64_t r = i / P.Kc, k = i % P.Kc;
   P.out[r * P.stride_r + k * P.stride_k] = f32_to_bf16_bits(s * P.scale);
 }
@@ -411,17 +486,53 @@ NtPlan plan_nt(int64_t M, int64_t Kc) {
   p.splits = (total_chunks + p.chunks_per_split - 1) / p.chunks_per_split;
   return p;
 }
-size_t nt_ws_bytes(int64_t M, int64_t Kc, int R) { return (size_t)plan_nt(M, Kc).splits * M * R * sizeof(float); }
+size_t align256(size_t v) { return (v + 255) & ~size_t(255); }
+// fp32 partial sums of one column contraction; 0 when a single slice writes the result directly
+size_t nt_part_bytes(int64_t M, int64_t Kc, int R) {
+  const int sp = plan_nt(M, Kc).splits;
+  return sp > 1 ? align256((size_t)sp * M * R * sizeof(float)) : 0;
+}
+
+// Fills in the slicing of the batch's problems (operands, Kc, R, ldo, out, scale are the caller's), hands each sliced
+// problem its piece of `ws` and launches: first pass, then the fixed-order sums of the sliced problems.
+// bt: the second operand is [Kc, R] row-major (transposed inside the kernel) instead of [R, Kc].
+int run_nt_batch(NtBatch& b, int n, bool bt, float* ws, hipStream_t s) {
+  int max_splits = 1, max_r = 0;
+  int64_t max_mr = 0;
+  const int m_tiles = plan_nt(b.M, 64).m_tiles;
+  char* w = reinterpret_cast<char*>(ws);
+  for (int i = 0; i < n; ++i) {
+    NtProblem& P = b.p[i];
+    const NtPlan pl = plan_nt(b.M, P.Kc);
+    P.splits = pl.splits;
+    P.chunks_per_split = pl.chunks_per_split;
+    P.part = reinterpret_cast<float*>(w);
+    w += nt_part_bytes(b.M, P.Kc, P.R);
+    max_splits = pl.splits > max_splits ? pl.splits : max_splits;
+    max_r = P.R > max_r ? P.R : max_r;
+    if (pl.splits > 1 && (int64_t)b.M * P.R > max_mr) max_mr = (int64_t)b.M * P.R;
+  }
+  const dim3 grid((unsigned)m_tiles, (unsigned)max_splits, (unsigned)n), block(256);
+  if (bt) {
+    if (max_r <= 16) skinny_nt_kernel<1, true><<<grid, block, 0, s>>>(b);
+    else if (max_r <= 32) skinny_nt_kernel<2, true><<<grid, block, 0, s>>>(b);
+    else skinny_nt_kernel<4, true><<<grid, block, 0, s>>>(b);
+  } else {
+    if (max_r <= 16) skinny_nt_kernel<1, false><<<grid, block, 0, s>>>(b);
+    else if (max_r <= 32) skinny_nt_kernel<2, false><<<grid, block, 0, s>>>(b);
+    else skinny_nt_kernel<4, false><<<grid, block, 0, s>>>(b);
+  }
+  if (max_mr > 0) sum_partials_kernel<<<dim3((unsigned)((max_mr + 255) / 256), (unsigned)n), block, 0, s>>>(b);
+  return check_launch("skinny_nt");
+}
 
 struct TnPlan {
-  int col_groups0, col_groups1, splits, rows_per_split;
+  int splits, rows_per_split;
 };
-// Both products of a backward in one grid: widths K (gA) and N (gB), the same row splits.
-TnPlan plan_tn_pair(int64_t M, int64_t K, int64_t N) {
+// Every row contraction of a backward in one grid: `col_groups` workgroups along x, the same row splits for all.
+TnPlan plan_tn(int64_t M, int64_t col_groups) {
   TnPlan p;
-  p.col_groups0 = (int)((K + kTnCols - 1) / kTnCols);
-  p.col_groups1 = (int)((N + kTnCols - 1) / kTnCols);
-  int s = kTargetWaves / 4 / (p.col_groups0 + p.col_groups1);  // workgroups of 4 waves
+  int s = (int)(kTargetWaves / 4 / col_groups);  // workgroups of 4 waves
   s = s < 1 ? 1 : s;
   const int max_s = (int)((M + 127) / 128);  // at least 128 rows per split: one 32-row step per wave
   s = s > max_s ? max_s : s;
@@ -429,66 +540,69 @@ TnPlan plan_tn_pair(int64_t M, int64_t K, int64_t N) {
   p.splits = (int)((M + p.rows_per_split - 1) / p.rows_per_split);
   return p;
 }
-size_t tn_pair_ws_bytes(int64_t M, int64_t K, int64_t N, int R) {
-  return (size_t)plan_tn_pair(M, K, N).splits * R * (size_t)(K + N) * sizeof(float);
-}
+int64_t tn_col_groups(int64_t Kc) { return (Kc + kTnCols - 1) / kTnCols; }
 
-size_t align256(size_t v) { return (v + 255) & ~size_t(255); }
-
-// b_is_kr: Bm is [Kc, R] row-major (transposed inside the kernel) instead of [R, Kc]
-template <bool BT>
-void launch_nt(const dim3& grid, const uint16_t* X, const uint16_t* Bm, float* ws, int M, int Kc, int R, int chunks_per_split,
-               uint16_t* direct, float scale, hipStream_t s) {
-  const dim3 block(256);
-  if (R <= 16)
-    skinny_nt_kernel<1, BT><<<grid, block, 0, s>>>(X, Bm, ws, M, Kc, R, chunks_per_split, direct, scale);
-  else if (R <= 32)
-    skinny_nt_kernel<2, BT><<<grid, block, 0, s>>>(X, Bm, ws, M, Kc, R, chunks_per_split, direct, scale);
-  else
-    skinny_nt_kernel<4, BT><<<grid, block, 0, s>>>(X, Bm, ws, M, Kc, R, chunks_per_split, direct, scale);
-}
-
-int run_nt(const uint16_t* X, const uint16_t* Bm, bool b_is_kr, int64_t M, int64_t Kc, int R, float scale, uint16_t* out,
-           float* ws, hipStream_t s) {
-  const NtPlan p = plan_nt(M, Kc);
-  const dim3 grid((unsigned)p.m_tiles, (unsigned)p.splits), block(256);
-  uint16_t* direct = p.splits == 1 ? out : nullptr;
-  if (b_is_kr)
-    launch_nt<true>(grid, X, Bm, ws, (int)M, (int)Kc, R, p.chunks_per_split, direct, scale, s);
-  else
-    launch_nt<false>(grid, X, Bm, ws, (int)M, (int)Kc, R, p.chunks_per_split, direct, scale, s);
-  if (!direct) {
-    const int64_t n = M * R;
-    sum_partials_kernel<<<dim3((unsigned)((n + 255) / 256)), block, 0, s>>>(ws, n, p.splits, scale, out);
+// The caller fills G, X, Kc, R, ldg of the n problems of `b` and the outputs of the ns sums of `f` (part, split_stride
+// and end are set here: sum i reads rows [sum_row0[i], + f.p[i].R) of problem sum_problem[i]).
+int run_tn_batch(TnBatch& b, int n, TnSumBatch& f, int ns, const int* sum_problem, const int* sum_row0, float* ws, hipStream_t s) {
+  int64_t groups = 0;
+  for (int i = 0; i < n; ++i) {
+    groups += tn_col_groups(b.p[i].Kc);
+    b.cg_end[i] = (int)groups;
   }
-  return check_launch("skinny_nt");
-}
-
-// gA[r][k] = sum_m gh[m][r] x[m][k]  and  gB[n][r] = scale * sum_m h[m][r] gy[m][n]
-int run_tn_pair(const uint16_t* gh, const uint16_t* x, const uint16_t* h, const uint16_t* gy, int64_t M, int64_t K, int64_t N,
-                int R, float scale, uint16_t* ga, uint16_t* gb, float* ws, hipStream_t s) {
-  const TnPlan p = plan_tn_pair(M, K, N);
-  TnPair a;
-  a.p[0] = TnProblem{gh, x, ws, (int)K};
-  a.p[1] = TnProblem{h, gy, ws + (size_t)p.splits * R * K, (int)N};
-  a.col_groups0 = p.col_groups0;
-  a.M = (int)M;
-  a.R = R;
-  a.rows_per_split = p.rows_per_split;
-  const dim3 grid((unsigned)(p.col_groups0 + p.col_groups1), (unsigned)p.splits), block(256);
-  for (int r0 = 0; r0 < R; r0 += 16) {
-    a.r0 = r0;
-    skinny_tn_kernel<<<grid, block, 0, s>>>(a);
+  const TnPlan pl = plan_tn(b.M, groups);
+  b.n = n;
+  b.rows_per_split = pl.rows_per_split;
+  float* w = ws;
+  for (int i = 0; i < n; ++i) {
+    b.p[i].part = w;
+    w += (size_t)pl.splits * b.p[i].R * b.p[i].Kc;
   }
-  TnSumPair f;
-  f.p[0] = TnSum{a.p[0].part, ga, (int)K, 1.0f, K, 1};
-  f.p[1] = TnSum{a.p[1].part, gb, (int)N, scale, 1, R};
-  f.n0 = (int64_t)R * K;
-  f.R = R;
-  f.splits = p.splits;
-  const int64_t n = (int64_t)R * (K + N);
-  sum_partials_tn_pair_kernel<<<dim3((unsigned)((n + 255) / 256)), block, 0, s>>>(f);
+  int rgm = 1;
+  for (int i = 0; i < n; ++i) rgm = (b.p[i].R + 15) / 16 > rgm ? (b.p[i].R + 15) / 16 : rgm;
+  const dim3 grid((unsigned)groups, (unsigned)pl.splits), block(256);
+  if (rgm == 1) skinny_tn_kernel<1><<<grid, block, 0, s>>>(b);
+  else if (rgm == 2) skinny_tn_kernel<2><<<grid, block, 0, s>>>(b);
+  else if (rgm == 3) skinny_tn_kernel<3><<<grid, block, 0, s>>>(b);
+  else skinny_tn_kernel<4><<<grid, block, 0, s>>>(b);
+  int64_t end = 0;
+  for (int i = 0; i < ns; ++i) {
+    const TnProblem& P = b.p[sum_problem[i]];
+    f.p[i].part = P.part + (int64_t)sum_row0[i] * P.Kc;
+    f.p[i].Kc = P.Kc;
+    f.p[i].split_stride = (int64_t)P.R * P.Kc;
+    end += (int64_t)f.p[i].R * P.Kc;
+    f.end[i] = end;
+  }
+  f.n = ns;
+  f.splits = pl.splits;
+  sum_partials_tn_kernel<<<dim3((unsigned)((end + 255) / 256)), dim3(256), 0, s>>>(f);
   return check_launch("skinny_tn");
+}
+// fp32 partial sums of a batch of row contractions: sum over problems of splits * R * Kc
+size_t tn_part_bytes(int64_t M, int n, const int64_t* Kc, const int* R) {
+  int64_t groups = 0, elems = 0;
+  for (int i = 0; i < n; ++i) {
+    groups += tn_col_groups(Kc[i]);
+    elems += (int64_t)R[i] * Kc[i];
+  }
+  return (size_t)plan_tn(M, groups).splits * elems * sizeof(float);
+}
+
+// h = x . A^T for one layer
+int run_hidden(const uint16_t* x, const uint16_t* lora_a, int64_t M, int64_t K, int R, uint16_t* h, float* ws, hipStream_t s) {
+  NtBatch b = {};
+  b.M = (int)M;
+  NtProblem& P = b.p[0];
+  P.X = x;
+  P.bm[0] = lora_a;
+  P.r_off[0] = 0;
+  P.r_off[1] = R;
+  P.nb = 1;
+  P.out = h;
+  P.Kc = (int)K; P.R = R; P.ldo = R;
+  P.scale = 1.0f;
+  return run_nt_batch(b, 1, false, ws, s);
 }
 
 int check_skinny(const char* who, int64_t M, int64_t N, int64_t K, int rank) {
@@ -500,25 +614,95 @@ int check_skinny(const char* who, int64_t M, int64_t N, int64_t K, int rank) {
 }
 
 }  // namespace
+
+size_t group_hidden_ws_bytes(int64_t M, int64_t K, int r_total) { return nt_part_bytes(M, K, r_total); }
+
+int run_group_hidden(const uint16_t* x, const GroupSkinny& g, uint16_t* h_cat, float* ws, hipStream_t s) {
+  NtBatch b = {};
+  b.M = (int)g.M;
+  NtProblem& P = b.p[0];
+  P.X = x;
+  for (int i = 0; i < g.n; ++i) {
+    P.bm[i] = g.lora_a[i];
+    P.r_off[i] = g.r_off[i];
+  }
+  P.r_off[g.n] = g.r_off[g.n];
+  P.nb = g.n;
+  P.out = h_cat;
+  P.Kc = (int)g.K; P.R = g.r_off[g.n]; P.ldo = g.r_off[g.n];
+  P.scale = 1.0f;
+  return run_nt_batch(b, 1, false, ws, s);
+}
+
+size_t group_lora_bwd_ws_bytes(const GroupSkinny& g) {
+  size_t nt = 0;
+  int64_t widths[kTnMaxProblems];
+  int ranks[kTnMaxProblems];
+  widths[0] = g.K;
+  ranks[0] = g.r_off[g.n];
+  for (int i = 0; i < g.n; ++i) {
+    nt += nt_part_bytes(g.M, g.N[i], g.rank[i]);
+    widths[1 + i] = g.N[i];
+    ranks[1 + i] = g.rank[i];
+  }
+  const size_t tn = tn_part_bytes(g.M, 1 + g.n, widths, ranks);
+  return align256(nt > tn ? nt : tn);
+}
+
+int run_group_lora_bwd(const uint16_t* x, const uint16_t* h_cat, const GroupSkinny& g, uint16_t* gh_cat, float* ws, hipStream_t s) {
+  const int rt = g.r_off[g.n];
+  {
+    NtBatch b = {};
+    b.M = (int)g.M;
+    for (int i = 0; i < g.n; ++i) {
+      NtProblem& P = b.p[i];
+      P.X = g.gy[i];
+      P.bm[0] = g.lora_b[i];
+      P.r_off[1] = g.rank[i];
+      P.nb = 1;
+      P.out = gh_cat + g.r_off[i];
+      P.Kc = (int)g.N[i]; P.R = g.rank[i]; P.ldo = rt;
+      P.scale = g.scale[i];
+    }
+    if (int rc = run_nt_batch(b, g.n, true, ws, s)) return rc;
+  }
+  TnBatch t = {};
+  t.M = (int)g.M;
+  t.p[0] = TnProblem{gh_cat, x, nullptr, (int)g.K, rt, rt};
+  TnSumBatch f = {};
+  int sum_problem[kTnMaxSums], sum_row0[kTnMaxSums];
+  for (int i = 0; i < g.n; ++i) {
+    t.p[1 + i] = TnProblem{h_cat + g.r_off[i], g.gy[i], nullptr, (int)g.N[i], g.rank[i], rt};
+    f.p[i] = TnSum{nullptr, g.ga[i], 0, g.rank[i], 1.0f, 0, g.K, 1};
+    sum_problem[i] = 0;
+    sum_row0[i] = g.r_off[i];
+    f.p[g.n + i] = TnSum{nullptr, g.gb[i], 0, g.rank[i], g.scale[i], 0, 1, g.rank[i]};
+    sum_problem[g.n + i] = 1 + i;
+    sum_row0[g.n + i] = 0;
+  }
+  return run_tn_batch(t, 1 + g.n, f, 2 * g.n, sum_problem, sum_row0, ws, s);
+}
+
 }  // namespace ttamd
 
 using namespace ttamd;
 
 extern "C" size_t ttamd_lora_fwd_workspace_bytes(int64_t M, int64_t K, int rank) {
   if (M <= 0 || K <= 0 || rank <= 0 || K % 64) return 0;
-  return align256(nt_ws_bytes(M, K, rank));
+  return nt_part_bytes(M, K, rank);
 }
 
 extern "C" int ttamd_lora_hidden_bf16(const void* x, const void* lora_a, void* h, int64_t M, int64_t K, int rank,
                                       void* workspace, size_t workspace_bytes, void* stream) {
   if (int rc = check_skinny("lora_hidden", M, 64, K, rank)) return rc;
-  TT_REQUIRE(x && lora_a && h && workspace, "lora_hidden: null pointer argument");
+  TT_REQUIRE(x && lora_a && h, "lora_hidden: null pointer argument");
+  const size_t need = ttamd_lora_fwd_workspace_bytes(M, K, rank);
+  TT_REQUIRE(need == 0 || workspace, "lora_hidden: null workspace");
   TT_REQUIRE(aligned16(x) && aligned16(lora_a) && aligned16(workspace), "lora_hidden: pointers must be 16-byte aligned");
-  if (workspace_bytes < ttamd_lora_fwd_workspace_bytes(M, K, rank))
-    return fail(TTAMD_EWORKSPACE, "lora_hidden: workspace has %zu bytes, needs %zu", workspace_bytes,
-                ttamd_lora_fwd_workspace_bytes(M, K, rank));
-  return run_nt(reinterpret_cast<const uint16_t*>(x), reinterpret_cast<const uint16_t*>(lora_a), false, M, K, rank, 1.0f,
-                reinterpret_cast<uint16_t*>(h), reinterpret_cast<float*>(workspace), reinterpret_cast<hipStream_t>(stream));
+  if (workspace_bytes < need)
+    return fail(TTAMD_EWORKSPACE, "lora_hidden: workspace has %zu bytes, needs %zu", workspace_bytes, need);
+  return run_hidden(reinterpret_cast<const uint16_t*>(x), reinterpret_cast<const uint16_t*>(lora_a), M, K, rank,
+                    reinterpret_cast<uint16_t*>(h), reinterpret_cast<float*>(workspace), reinterpret_cast<hipStream_t>(stream));
 }
 
 // ---- the same product for callers that cannot allocate ---------------------------------------------------------------
@@ -556,7 +740,7 @@ extern "C" int ttamd_lora_hidden_static_bf16(const void* x, const void* lora_a, 
   if (int rc = check_skinny("lora_hidden_static", M, 64, K, rank)) return rc;
   TT_REQUIRE(x && lora_a && h, "lora_hidden_static: null pointer argument");
   TT_REQUIRE(aligned16(x) && aligned16(lora_a), "lora_hidden_static: pointers must be 16-byte aligned");
-  const size_t need = plan_nt(M, K).splits > 1 ? nt_ws_bytes(M, K, rank) : 0;  // one slice writes the result directly
+  const size_t need = nt_part_bytes(M, K, rank);  // 0: one slice writes the result directly
   if (need > kStaticScratchBytes)
     return fail(TTAMD_EWORKSPACE, "lora_hidden_static: M=%lld K=%lld rank=%d needs %zu bytes of partial sums, the built-in "
                 "scratch holds %zu; use ttamd_lora_hidden_bf16 with a workspace", (long long)M, (long long)K, rank, need,
@@ -564,13 +748,15 @@ extern "C" int ttamd_lora_hidden_static_bf16(const void* x, const void* lora_a, 
   float* scratch = nullptr;
   if (int rc = static_scratch(&scratch)) return rc;
   // every partial sum the reduction reads is written by this call's first kernel: nothing has to start at zero
-  return run_nt(reinterpret_cast<const uint16_t*>(x), reinterpret_cast<const uint16_t*>(lora_a), false, M, K, rank, 1.0f,
-                reinterpret_cast<uint16_t*>(h), scratch, reinterpret_cast<hipStream_t>(stream));
+  return run_hidden(reinterpret_cast<const uint16_t*>(x), reinterpret_cast<const uint16_t*>(lora_a), M, K, rank,
+                    reinterpret_cast<uint16_t*>(h), scratch, reinterpret_cast<hipStream_t>(stream));
 }
 
 extern "C" size_t ttamd_lora_bwd_workspace_bytes(int64_t M, int64_t N, int64_t K, int rank) {
   if (M <= 0 || N <= 0 || K <= 0 || rank <= 0 || K % 64 || N % 64) return 0;
-  const size_t a = nt_ws_bytes(M, N, rank), b = tn_pair_ws_bytes(M, K, N, rank);
+  const int64_t widths[2] = {K, N};
+  const int ranks[2] = {rank, rank};
+  const size_t a = nt_part_bytes(M, N, rank), b = tn_part_bytes(M, 2, widths, ranks);
   return align256(a > b ? a : b);
 }
 
@@ -579,19 +765,36 @@ extern "C" int ttamd_lora_bwd_bf16(const void* gy, const void* x, const void* h,
                                    size_t workspace_bytes, void* stream) {
   if (int rc = check_skinny("lora_bwd", M, N, K, rank)) return rc;
   TT_REQUIRE(gy && x && h && lora_b && gh && ga && gb && workspace, "lora_bwd: null pointer argument");
-  TT_REQUIRE(aligned16(gy) && aligned16(x) && aligned16(h) && aligned16(lora_b) && aligned16(workspace),
+  TT_REQUIRE(aligned16(gy) && aligned16(x) && aligned16(h) && aligned16(lora_b) && aligned16(workspace) && aligned16(gh),
              "lora_bwd: pointers must be 16-byte aligned");
   if (workspace_bytes < ttamd_lora_bwd_workspace_bytes(M, N, K, rank))
     return fail(TTAMD_EWORKSPACE, "lora_bwd: workspace has %zu bytes, needs %zu", workspace_bytes,
                 ttamd_lora_bwd_workspace_bytes(M, N, K, rank));
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  float* part = reinterpret_cast<float*>(workspace);
+  float* ws = reinterpret_cast<float*>(workspace);
   const uint16_t* GY = reinterpret_cast<const uint16_t*>(gy);
-  // gh = scale * gy . B, lora_b [N, R] as it lies (the kernel transposes its pieces)
-  if (int rc = run_nt(GY, reinterpret_cast<const uint16_t*>(lora_b), true, M, N, rank, scale, reinterpret_cast<uint16_t*>(gh),
-                      part, s))
-    return rc;
-  return run_tn_pair(reinterpret_cast<const uint16_t*>(gh), reinterpret_cast<const uint16_t*>(x),
-                     reinterpret_cast<const uint16_t*>(h), GY, M, K, N, rank, scale, reinterpret_cast<uint16_t*>(ga),
-                     reinterpret_cast<uint16_t*>(gb), part, s);
+  {
+    // gh = scale * gy . B, lora_b [N, R] as it lies (the kernel transposes its pieces)
+    NtBatch b = {};
+    b.M = (int)M;
+    NtProblem& P = b.p[0];
+    P.X = GY;
+    P.bm[0] = reinterpret_cast<const uint16_t*>(lora_b);
+    P.r_off[1] = rank;
+    P.nb = 1;
+    P.out = reinterpret_cast<uint16_t*>(gh);
+    P.Kc = (int)N; P.R = rank; P.ldo = rank;
+    P.scale = scale;
+    if (int rc = run_nt_batch(b, 1, true, ws, s)) return rc;
+  }
+  // gA[r][k] = sum_m gh[m][r] x[m][k]  and  gB[n][r] = scale * sum_m h[m][r] gy[m][n]
+  TnBatch t = {};
+  t.M = (int)M;
+  t.p[0] = TnProblem{reinterpret_cast<const uint16_t*>(gh), reinterpret_cast<const uint16_t*>(x), nullptr, (int)K, rank, rank};
+  t.p[1] = TnProblem{reinterpret_cast<const uint16_t*>(h), GY, nullptr, (int)N, rank, rank};
+  TnSumBatch f = {};
+  f.p[0] = TnSum{nullptr, reinterpret_cast<uint16_t*>(ga), 0, rank, 1.0f, 0, K, 1};
+  f.p[1] = TnSum{nullptr, reinterpret_cast<uint16_t*>(gb), 0, rank, scale, 0, 1, rank};
+  const int sum_problem[2] = {0, 1}, sum_row0[2] = {0, 0};
+  return run_tn_batch(t, 2, f, 2, sum_problem, sum_row0, ws, s);
 }

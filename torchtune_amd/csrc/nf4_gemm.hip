@@ -16,6 +16,7 @@
 // registers: a thread expands an 8(n) x 8(k) patch (one dword of codes from each of 8 rows) and writes it
 // as eight 16-byte chunks of 8 consecutive n.
 #include "common.h"
+#include "group.h"
 #include "nf4_math.h"
 
 namespace ttamd {
@@ -370,12 +371,15 @@ int launch_gemm(GemmArgs& g, hipStream_t s) {
   g.tiles_m = (g.M + BM - 1) / BM;
   g.tiles_n = (Nout + BN - 1) / BN;
   const size_t smem = 2 * (BM + BN) * kRowBytes + 256 * sizeof(float2);
-  static bool attr_set = false;  // idempotent; a race only repeats the call
-  if (!attr_set) {
+  // the limit is a per-device attribute of the function: set it for the current device once (a race only repeats the call)
+  static bool attr_set_dev[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = -1;
+  if (dev < 0 || !attr_set_dev[dev]) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&nf4_gemm_kernel<BM, BN, TRANS_W>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return fail(TTAMD_ELAUNCH, "nf4_gemm: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
-    attr_set = true;
+    if (dev >= 0) attr_set_dev[dev] = true;
   }
   nf4_gemm_kernel<BM, BN, TRANS_W><<<dim3((unsigned)(g.tiles_m * g.tiles_n)), dim3(256), smem, s>>>(g);
   return check_launch("nf4_gemm");
@@ -409,15 +413,9 @@ int check_gemm_args(const char* who, const void* a, const uint8_t* qdata, const 
 
 }  // namespace
 
-// nf4_gemm_rs.hip
-int run_gemm_rs(const void* X, const uint8_t* codes, const void* scal, int mode, const void* lX, const void* lW,
-                bool lw_row_major, int R, float lscale, const void* bias, const void* cscale, void* C, int64_t M, int64_t Nout,
-                int64_t Kc, void* workspace, size_t workspace_bytes, hipStream_t s);
-size_t gemm_rs_workspace_bytes(int64_t M, int64_t Nout, int64_t Kc);
-// nf4_small_m.hip
-int small_m_limit();
-int run_small_m(const void* x, const uint8_t* codes, const void* bscal, const void* h, const void* lora_b, int R, float lscale,
-                const void* bias, const void* cscale, void* y, int64_t M, int64_t N, int64_t K, hipStream_t s);
+// nf4_small_m.hip (run_gemm_rs, gemm_rs_workspace_bytes and small_m_limit: group.h)
+int run_small_m(const void* x, const uint8_t* codes, const void* bscal, const void* h, int ldh, const void* lora_b, int R,
+                float lscale, const void* bias, const void* cscale, void* y, int64_t M, int64_t N, int64_t K, hipStream_t s);
 }  // namespace ttamd
 
 using namespace ttamd;
@@ -451,14 +449,14 @@ int lora_linear_fwd(const char* who, const void* x, const uint8_t* quantized_dat
                  (col_scale == nullptr || (reinterpret_cast<uintptr_t>(col_scale) & 7u) == 0),
              "%s: bias / col_scale must be 8-byte aligned", who);
   if (M <= small_m_limit())  // a handful of tokens: stream the packed weight once (nf4_small_m.hip)
-    return run_small_m(x, quantized_data, block_scalers, h, lora_b, rank, scale, bias, col_scale, y, M, N, K,
+    return run_small_m(x, quantized_data, block_scalers, h, rank, lora_b, rank, scale, bias, col_scale, y, M, N, K,
                        reinterpret_cast<hipStream_t>(stream));
   if (block_scalers_t) {
     TT_REQUIRE(aligned16(block_scalers_t), "%s: block_scalers_t must be 16-byte aligned", who);
-    return run_gemm_rs(x, quantized_data, block_scalers_t, 2, h, lora_b, true, rank, scale, bias, col_scale, y, M, N, K,
+    return run_gemm_rs(x, quantized_data, block_scalers_t, 2, h, rank, lora_b, true, rank, scale, bias, col_scale, y, M, N, K,
                        workspace, workspace_bytes, reinterpret_cast<hipStream_t>(stream));
   }
-  return run_gemm_rs(x, quantized_data, block_scalers, 0, h, lora_b, true, rank, scale, bias, col_scale, y, M, N, K,
+  return run_gemm_rs(x, quantized_data, block_scalers, 0, h, rank, lora_b, true, rank, scale, bias, col_scale, y, M, N, K,
                      workspace, workspace_bytes, reinterpret_cast<hipStream_t>(stream));
 }
 }  // namespace
@@ -519,7 +517,7 @@ extern "C" int ttamd_nf4_linear_bwd_dx_ws_bf16(const void* gy, const uint8_t* qu
              "nf4_linear_bwd_dx: the transposed codes and scalers must be given together");
   if (quantized_data_t != nullptr) {
     TT_REQUIRE(aligned16(quantized_data_t) && aligned16(block_scalers_t), "nf4_linear_bwd_dx: transposed copies must be 16-byte aligned");
-    return run_gemm_rs(gy, quantized_data_t, block_scalers_t, 1, gh, lora_a, false, rank, 1.0f, nullptr, nullptr, gx, M, K, N,
+    return run_gemm_rs(gy, quantized_data_t, block_scalers_t, 1, gh, rank, lora_a, false, rank, 1.0f, nullptr, nullptr, gx, M, K, N,
                        workspace, workspace_bytes, reinterpret_cast<hipStream_t>(stream));
   }
   GemmArgs g;

@@ -24,6 +24,7 @@
 // 12 direct-to-LDS loads, BM/32 x 4 operand reads and 32 table reads.
 
 #include "common.h"
+#include "group.h"
 #include "nf4_math.h"
 
 namespace ttamd {
@@ -51,7 +52,7 @@ struct RsArgs {
   const uint16_t* X;     // [M, Kc] bf16 activations
   const uint8_t* codes;  // [Nout, Kc/2] packed NF4 codes of the weight view
   const float* scal;     // block scalers, fp32: MODE 0 [Nout, Kc/64]; MODE 2 [Kc/64, Nout]; MODE 1 per element [Nout/64, Kc]
-  const uint16_t* lX;    // adapter activations [M, R] bf16 or null
+  const uint16_t* lX;    // adapter activations [M, R] bf16 (rows ldlx elements apart) or null
   const uint16_t* lW;    // adapter weights: [Nout, R] (lw_row_major) or [R, Nout] bf16, or null
   const uint16_t* bias;  // [Nout] bf16 or null
   const uint16_t* cscale;  // [Nout] bf16 or null: C = (acc + bias) * cscale per column (DoRA's magnitude / norm)
@@ -60,8 +61,23 @@ struct RsArgs {
   int M, Nout, Kc, R;
   int ksteps;            // SPLIT: 64-wide k-steps per slice of the contraction (blockIdx.y = slice)
   int lw_row_major;
+  int ldlx;
   float lscale;
   int tiles_m, tiles_n;
+};
+
+// SEG kernels: the contraction is the concatenation of up to kGroupMax segments, each with its own activation, weight
+// view and adapter (the grad-input of a group of layers with a common input: gx = sum_i gy_i . D(W_i) + gh_i . A_i is
+// one GEMM whose contraction runs over the members' output columns one member after the other).  g.X / codes / scal /
+// Kc / lX / lW / R are then unused; M, Nout, C and ldlx are shared.
+struct RsSegs {
+  const uint16_t* X[kGroupMax];     // [M, Kc[i]]
+  const uint8_t* codes[kGroupMax];  // [Nout, Kc[i] / 2]
+  const float* scal[kGroupMax];     // MODE 1: [Nout / 64, Kc[i]]
+  const uint16_t* lX[kGroupMax];    // adapter activations, rows g.ldlx apart, or null
+  const uint16_t* lW[kGroupMax];    // adapter weights [R[i], Nout]
+  int Kc[kGroupMax], R[kGroupMax];
+  int n;
 };
 
 constexpr int kBN = 256;
@@ -85,10 +101,12 @@ struct RsLayout {
 // SPLIT: the contraction is cut into gridDim.y slices so that a launch with few output tiles still fills the chip; a
 // workgroup then leaves its tile as fp32 in g.part (slice 0 includes the adapter) and bias, column scale and the
 // rounding to bf16 happen in nf4_gemm_rs_reduce_kernel, which adds the slices in a fixed order.
-template <int BM, int MODE, bool SPLIT>
-__global__ __launch_bounds__(256) void nf4_gemm_rs_kernel(const RsArgs g) {
+// SEG: segmented contraction (see RsSegs); only with MODE 1 and without SPLIT.
+template <int BM, int MODE, bool SPLIT, bool SEG = false>
+__global__ __launch_bounds__(256) void nf4_gemm_rs_kernel(const RsArgs g, const RsSegs sg) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the body uses LDS address-space casts and gfx950 builtins the host pass cannot parse
   static_assert(BM == 256 || BM == 128, "BM");
+  static_assert(!SEG || (MODE == 1 && !SPLIT), "segments: grad-input kernels only");
   constexpr bool PER_ELEM = MODE == 1;
   constexpr bool SCAL_T = MODE == 2;
   using L = RsLayout<BM>;
@@ -119,9 +137,12 @@ __global__ __launch_bounds__(256) void nf4_gemm_rs_kernel(const RsArgs g) {
     }
   }
   const int m0 = tile_m * BM, n0 = tile_n * kBN;
-  const int Kc = g.Kc;
+  const int Kc = SEG ? sg.Kc[0] : g.Kc;
   const int nkf = Kc >> 6;  // k-steps of the whole contraction: the row stride of the MODE 0 scalers
   int kb = 0, nk = nkf;     // this workgroup's k-steps are [kb, kb + nk)
+  if constexpr (SEG) {
+    for (int q = 1; q < sg.n; ++q) nk += sg.Kc[q] >> 6;
+  }
   if constexpr (SPLIT) {
     kb = blockIdx.y * g.ksteps;
     nk = nkf - kb < g.ksteps ? nkf - kb : g.ksteps;
@@ -138,35 +159,39 @@ __global__ __launch_bounds__(256) void nf4_gemm_rs_kernel(const RsArgs g) {
   //      linear slot l, so the lane fetches the chunk that belongs there.
   const int a_r8 = lane >> 3;
   uint32_t a_off[kALoads];  // byte offset of this lane's chunk from X + k0
-#pragma unroll
-  for (int i = 0; i < kALoads; ++i) {
-    const int trow = wv * (BM / 4) + 8 * i + a_r8;  // row inside the tile
-    const int chunk = (lane & 7) ^ ((trow >> 1) & 7);
-    int row = m0 + trow;
-    row = row < g.M ? row : g.M - 1;
-    a_off[i] = ((uint32_t)row * (uint32_t)Kc + chunk * 8) * 2u;
-  }
   // ---- weight view rows of this lane: tile j -> output column n0 + 64 wv + 32 j + l31; half h owns code bytes [16h, 16h+16)
   uint32_t w_off[NT], s_off[NT];  // byte offsets from codes + k0/2 and from scal + tk
+  // (the offsets depend on the row length kc of the operands: a SEG kernel recomputes them at every segment boundary)
+  auto set_offsets = [&](int kc) {
 #pragma unroll
-  for (int j = 0; j < NT; ++j) {
-    int col = n0 + wv * 64 + 32 * j + l31;
-    col = col < g.Nout ? col : g.Nout - 1;
-    w_off[j] = (uint32_t)(((int64_t)col * Kc) >> 1) + 16 * h;
-    s_off[j] = (uint32_t)col * (uint32_t)nkf * 4u;
-  }
-  if constexpr (SCAL_T) {
-    int col = n0 + wv * 64 + lane;  // lane l fetches the scaler of the wave's column l
-    col = col < g.Nout ? col : g.Nout - 1;
-    s_off[0] = (uint32_t)col * 4u;
-  }
-  if constexpr (PER_ELEM) {
-    // scalers of the wave's 64-column block for the 64 contraction elements of a k-step: lane l fetches element l
-    int ob = (n0 >> 6) + wv;
-    const int nob = g.Nout >> 6;
-    ob = ob < nob ? ob : nob - 1;
-    s_off[0] = ((uint32_t)ob * (uint32_t)Kc + lane) * 4u;
-  }
+    for (int i = 0; i < kALoads; ++i) {
+      const int trow = wv * (BM / 4) + 8 * i + a_r8;  // row inside the tile
+      const int chunk = (lane & 7) ^ ((trow >> 1) & 7);
+      int row = m0 + trow;
+      row = row < g.M ? row : g.M - 1;
+      a_off[i] = ((uint32_t)row * (uint32_t)kc + chunk * 8) * 2u;
+    }
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+      int col = n0 + wv * 64 + 32 * j + l31;
+      col = col < g.Nout ? col : g.Nout - 1;
+      w_off[j] = (uint32_t)(((int64_t)col * kc) >> 1) + 16 * h;
+      s_off[j] = (uint32_t)col * (uint32_t)(kc >> 6) * 4u;
+    }
+    if constexpr (SCAL_T) {
+      int col = n0 + wv * 64 + lane;  // lane l fetches the scaler of the wave's column l
+      col = col < g.Nout ? col : g.Nout - 1;
+      s_off[0] = (uint32_t)col * 4u;
+    }
+    if constexpr (PER_ELEM) {
+      // scalers of the wave's 64-column block for the 64 contraction elements of a k-step: lane l fetches element l
+      int ob = (n0 >> 6) + wv;
+      const int nob = g.Nout >> 6;
+      ob = ob < nob ? ob : nob - 1;
+      s_off[0] = ((uint32_t)ob * (uint32_t)kc + lane) * 4u;
+    }
+  };
+  set_offsets(Kc);
 
   // Direct-to-LDS loads are written as inline assembly: `voff` is this lane's 32-bit byte offset from the uniform
   // `base`, the wave's 64 lanes land in LDS at `lds`, `lds` + size, ...  Issued this way the compiler keeps no
@@ -333,8 +358,25 @@ __global__ __launch_bounds__(256) void nf4_gemm_rs_kernel(const RsArgs g) {
   // That one barrier per step also orders stage reuse: a wave issuing batch t+2 into the A stage of tile t-2 has
   // passed barrier t-1, which every wave reaches only after finishing step t-2.  W stages are wave-private.
   // Weights are expanded just in time: substep ks is fetched two phases and finished one phase before its MFMAs.
-  issue(0, 0, 0);
-  issue(1, 1, 1);
+  // Global bases of the next batch to issue, carried through the main loop and bumped by a constant per k-step.
+  const char *pxb, *pcb, *psb;
+  auto seg_base = [&](int q, int step) {
+    pxb = reinterpret_cast<const char*>(sg.X[q]) + ((int64_t)step << 7);
+    pcb = reinterpret_cast<const char*>(sg.codes[q]) + ((int64_t)step << 5);
+    psb = reinterpret_cast<const char*>(sg.scal[q]) + (int64_t)step * 256;
+  };
+  if constexpr (SEG) {  // segment 0 has at least two k-steps (the host puts the widest first): batches 0 and 1 are its
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      seg_base(0, t);
+      const BatchAddr bt = batch_addr_at(pxb, pcb, psb, t, t);
+#pragma unroll
+      for (int d = 0; d < kBatch; ++d) issue_one(bt, d);
+    }
+  } else {
+    issue(0, 0, 0);
+    issue(1, 1, 1);
+  }
   asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kBatch) : "memory");  // batch 0 landed everywhere, table written
   load_codes(0, sc);
   {
@@ -355,22 +397,16 @@ __global__ __launch_bounds__(256) void nf4_gemm_rs_kernel(const RsArgs g) {
   constexpr int kDEven = (kBatch + 7) / 8 > 1 ? 2 : 1;  // loads per even quarter over the 8 quarters of phases 0 and 1
   constexpr int kDOdd = (kBatch - 4 * kDEven + 3) / 4;  // and per odd quarter
   static_assert(4 * kDEven + 4 * kDOdd >= kBatch && kDOdd <= 2 && kDOdd >= 0, "batch does not fit the 8 quarter phases");
-  int a0 = 0, w0 = 0;  // A / W stage of k-step kt
-  const char *pxb, *pcb, *psb;  // global bases of k-step kt + 2
-  {
-    const BatchAddr b2 = batch_addr(2, 0, 0);
-    pxb = b2.xb; pcb = b2.cb; psb = b2.sb;
-  }
-  for (int kt = 0; kt < nk; ++kt) {
+  int a0 = 0, w0 = 0;  // A / W stage of the k-step being multiplied
+  // One k-step: multiplies tile kt, issues batch kt + 2 from the carried bases, then moves them on by `adv` k-steps
+  // (0 past the end of the contraction: the last tile is reloaded, never consumed).
+  auto k_step = [&](int64_t adv) {
     const int a1 = (a0 + 1) & 3, a2 = (a0 + 2) & 3;
     const int w1 = w0 == 2 ? 0 : w0 + 1, w2 = w1 == 2 ? 0 : w1 + 1;
     const BatchAddr b = batch_addr_at(pxb, pcb, psb, a2, w2);
-    {
-      const int64_t adv = kt + 3 < nk ? 1 : 0;
-      pxb += adv << 7;
-      pcb += adv << 5;
-      psb += adv * s_stride;
-    }
+    pxb += adv << 7;
+    pcb += adv << 5;
+    psb += adv * s_stride;
     phase(xfa, wfa, xfb, a0, 1, wfb, sc, w0, 1, 2, b, 0, kDEven, kDOdd);
     phase(xfb, wfb, xfa, a0, 2, wfa, sc, w0, 2, 3, b, 2 * (kDEven + kDOdd), kDEven, kDOdd);
     asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kBatch) : "memory");
@@ -381,14 +417,45 @@ __global__ __launch_bounds__(256) void nf4_gemm_rs_kernel(const RsArgs g) {
     for (int j = 0; j < NT; ++j) sc[j] = sc_next[j];
     a0 = a1;
     w0 = w1;
+  };
+  if constexpr (!SEG) {
+    const BatchAddr b2 = batch_addr(2, 0, 0);  // global bases of k-step 2
+    pxb = b2.xb; pcb = b2.cb; psb = b2.sb;
+    for (int kt = 0; kt < nk; ++kt) k_step(kt + 3 < nk ? 1 : 0);
+  } else {
+    // The batches are issued segment by segment; inside a segment the lane offsets are loop constants.  The k-steps
+    // multiplied meanwhile lag two batches behind and do not care which segment their tile came from.  The last
+    // segment runs the two extra steps that drain the pipeline.
+    int issued = 2;  // index of the next batch to issue
+    for (int q = 0; q < sg.n; ++q) {
+      int steps = sg.Kc[q] >> 6;
+      if (q == 0) {
+        steps -= 2;
+        seg_base(0, nk > 2 ? 2 : 1);
+      } else {
+        set_offsets(sg.Kc[q]);
+        seg_base(q, 0);
+      }
+      if (q == sg.n - 1) steps += 2;
+      for (int it = 0; it < steps; ++it) {
+        k_step(issued + 1 < nk ? 1 : 0);
+        ++issued;
+      }
+    }
   }
 
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the clamped batches issued by the last two steps
   // ---- adapter: R extra contraction steps, operands straight from global memory
-  if (g.R > 0 && (!SPLIT || blockIdx.y == 0)) {
-    for (int rc = 0; rc < g.R; rc += 16) {
+  //      (a SEG kernel has one adapter per segment)
+  const int n_adapters = SEG ? sg.n : 1;
+  for (int ad = 0; ad < n_adapters; ++ad) {
+    const uint16_t* __restrict__ lX = SEG ? sg.lX[ad] : g.lX;
+    const uint16_t* __restrict__ lW = SEG ? sg.lW[ad] : g.lW;
+    const int R = SEG ? sg.R[ad] : g.R;
+    if (!(R > 0 && lX != nullptr && (!SPLIT || blockIdx.y == 0))) continue;
+    for (int rc = 0; rc < R; rc += 16) {
       const int r0 = rc + 8 * h;
-      const bool in = r0 < g.R;  // R % 8 == 0: a lane's 8 indices are all in or all out
+      const bool in = r0 < R;  // R % 8 == 0: a lane's 8 indices are all in or all out
       bf16x8_t wfr[NT], xfr[MT];
 #pragma unroll
       for (int j = 0; j < NT; ++j) {
@@ -397,12 +464,12 @@ __global__ __launch_bounds__(256) void nf4_gemm_rs_kernel(const RsArgs g) {
         u32x4_t raw = {0, 0, 0, 0};
         if (in) {
           if (g.lw_row_major) {
-            raw = *reinterpret_cast<const u32x4_t*>(g.lW + (int64_t)col * g.R + r0);
+            raw = *reinterpret_cast<const u32x4_t*>(lW + (int64_t)col * R + r0);
           } else {
 #pragma unroll
             for (int d = 0; d < 4; ++d) {
-              const uint32_t lo = g.lW[(int64_t)(r0 + 2 * d) * g.Nout + col];
-              const uint32_t hi = g.lW[(int64_t)(r0 + 2 * d + 1) * g.Nout + col];
+              const uint32_t lo = lW[(int64_t)(r0 + 2 * d) * g.Nout + col];
+              const uint32_t hi = lW[(int64_t)(r0 + 2 * d + 1) * g.Nout + col];
               raw[d] = lo | (hi << 16);
             }
           }
@@ -414,7 +481,7 @@ __global__ __launch_bounds__(256) void nf4_gemm_rs_kernel(const RsArgs g) {
         int row = m0 + 32 * i + l31;
         row = row < g.M ? row : g.M - 1;
         u32x4_t raw = {0, 0, 0, 0};
-        if (in) raw = *reinterpret_cast<const u32x4_t*>(g.lX + (int64_t)row * g.R + r0);
+        if (in) raw = *reinterpret_cast<const u32x4_t*>(lX + (int64_t)row * g.ldlx + r0);
         if (g.lscale != 1.0f) {
 #pragma unroll
           for (int d = 0; d < 4; ++d)
@@ -536,8 +603,8 @@ __global__ __launch_bounds__(256) void nf4_gemm_rs_reduce_kernel(const float* __
   *reinterpret_cast<u32x4_t*>(C + e) = o;
 }
 
-template <int BM, int MODE, bool SPLIT>
-int launch_rs(RsArgs& g, int splits, hipStream_t s) {
+template <int BM, int MODE, bool SPLIT, bool SEG = false>
+int launch_rs(RsArgs& g, int splits, hipStream_t s, const RsSegs* segs = nullptr) {
   using L = RsLayout<BM>;
   g.tiles_m = (g.M + BM - 1) / BM;
   g.tiles_n = (g.Nout + kBN - 1) / kBN;
@@ -546,13 +613,15 @@ int launch_rs(RsArgs& g, int splits, hipStream_t s) {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = -1;
   if (dev < 0 || !attr_set[dev]) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&nf4_gemm_rs_kernel<BM, MODE, SPLIT>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&nf4_gemm_rs_kernel<BM, MODE, SPLIT, SEG>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, L::kTotal);
     if (e != hipSuccess)
       return fail(TTAMD_ELAUNCH, "nf4_gemm_rs: cannot reserve %d bytes of LDS: %s", L::kTotal, hipGetErrorString(e));
     if (dev >= 0) attr_set[dev] = true;
   }
-  nf4_gemm_rs_kernel<BM, MODE, SPLIT><<<dim3((unsigned)(g.tiles_m * g.tiles_n), (unsigned)splits), dim3(256), L::kTotal, s>>>(g);
+  static const RsSegs no_segs = {};
+  nf4_gemm_rs_kernel<BM, MODE, SPLIT, SEG><<<dim3((unsigned)(g.tiles_m * g.tiles_n), (unsigned)splits), dim3(256), L::kTotal, s>>>(
+      g, segs ? *segs : no_segs);
   return check_launch("nf4_gemm_rs");
 }
 
@@ -577,8 +646,9 @@ size_t gemm_rs_workspace_bytes(int64_t M, int64_t Nout, int64_t Kc) {
   return sp > 1 ? (size_t)sp * (size_t)M * (size_t)Nout * sizeof(float) : 0;
 }
 
-// Entry used by the C-ABI wrappers in nf4_gemm.hip.  `workspace` may be null: then small launches are not sliced.
-int run_gemm_rs(const void* X, const uint8_t* codes, const void* scal, int mode, const void* lX, const void* lW,
+// Entry used by the C-ABI wrappers.  `workspace` may be null: then small launches are not sliced.  The rows of the
+// adapter activation lX are ldlx elements apart (a group keeps its members' activations side by side).
+int run_gemm_rs(const void* X, const uint8_t* codes, const void* scal, int mode, const void* lX, int ldlx, const void* lW,
                 bool lw_row_major, int R, float lscale, const void* bias, const void* cscale, void* C, int64_t M, int64_t Nout,
                 int64_t Kc, void* workspace, size_t workspace_bytes, hipStream_t s) {
   // per-lane byte offsets inside the kernel are 32-bit: the weight must fit them, and a token dimension too long for
@@ -590,7 +660,7 @@ int run_gemm_rs(const void* X, const uint8_t* codes, const void* scal, int mode,
     for (int64_t r0 = 0; r0 < M; r0 += max_rows) {
       const int64_t rows = M - r0 < max_rows ? M - r0 : max_rows;
       const int rc = run_gemm_rs(reinterpret_cast<const uint16_t*>(X) + r0 * Kc, codes, scal, mode,
-                                 lX ? reinterpret_cast<const uint16_t*>(lX) + r0 * R : nullptr, lW, lw_row_major, R, lscale, bias,
+                                 lX ? reinterpret_cast<const uint16_t*>(lX) + r0 * ldlx : nullptr, ldlx, lW, lw_row_major, R, lscale, bias,
                                  cscale, reinterpret_cast<uint16_t*>(C) + r0 * Nout, rows, Nout, Kc, nullptr, 0, s);
       if (rc != TTAMD_OK) return rc;
     }
@@ -607,6 +677,7 @@ int run_gemm_rs(const void* X, const uint8_t* codes, const void* scal, int mode,
   g.C = reinterpret_cast<uint16_t*>(C);
   g.M = (int)M; g.Nout = (int)Nout; g.Kc = (int)Kc; g.R = R;
   g.lw_row_major = lw_row_major ? 1 : 0;
+  g.ldlx = ldlx;
   g.lscale = lscale;
   g.part = nullptr;
   g.ksteps = 0;
@@ -630,6 +701,50 @@ int run_gemm_rs(const void* X, const uint8_t* codes, const void* scal, int mode,
   if (mode == 1) return big ? launch_rs<256, 1, false>(g, 1, s) : launch_rs<128, 1, false>(g, 1, s);
   if (mode == 2) return big ? launch_rs<256, 2, false>(g, 1, s) : launch_rs<128, 2, false>(g, 1, s);
   return big ? launch_rs<256, 0, false>(g, 1, s) : launch_rs<128, 0, false>(g, 1, s);
+}
+
+
+// Grad-input of a group of layers with a common input, as one GEMM over the concatenated contraction:
+//   gx[M, K] = sum_i gy_i[M, N_i] . D(W_i)[N_i, K] + gh_i[M, R_i] . A_i[R_i, K]
+// with the members' transposed copies (codes [K, N_i / 2], per-element scalers [K / 64, N_i]); gh_i = columns
+// [r_off[i], r_off[i + 1]) of gh_cat.  The sum over members is taken in fp32, before the one rounding to bf16.
+int run_gemm_rs_group_dx(const GroupDx& d, const void* gh_cat, void* gx, hipStream_t s) {
+  TT_REQUIRE(d.n >= 1 && d.n <= kGroupMax, "nf4_group_dx: %d members", d.n);
+  RsSegs sg = {};
+  sg.n = d.n;
+  int64_t max_n = 0;
+  int first = 0;  // the widest member goes first: the kernel takes its first two batches from segment 0
+  for (int i = 0; i < d.n; ++i) {
+    TT_REQUIRE(d.N[i] > 0 && d.N[i] % 64 == 0, "nf4_group_dx: N (%lld) must be a positive multiple of 64", (long long)d.N[i]);
+    TT_REQUIRE(aligned16(d.gy[i]) && aligned16(d.codes_t[i]) && aligned16(d.scal_t[i]), "nf4_group_dx: pointers must be 16-byte aligned");
+    if (d.N[i] > max_n) {
+      max_n = d.N[i];
+      first = i;
+    }
+  }
+  if (max_n < 128) return fail(TTAMD_EUNSUPPORTED, "nf4_group_dx: the widest member must have at least 128 outputs (has %lld)", (long long)max_n);
+  for (int k = 0; k < d.n; ++k) {
+    const int i = k == 0 ? first : (k <= first ? k - 1 : k);  // first, then the others in their order
+    sg.X[k] = d.gy[i];
+    sg.codes[k] = d.codes_t[i];
+    sg.scal[k] = d.scal_t[i];
+    sg.lX[k] = d.rank[i] > 0 ? reinterpret_cast<const uint16_t*>(gh_cat) + d.r_off[i] : nullptr;
+    sg.lW[k] = d.lora_a[i];
+    sg.Kc[k] = (int)d.N[i];
+    sg.R[k] = d.rank[i];
+  }
+  // per-lane byte offsets inside the kernel are 32-bit
+  if (!(d.K * max_n / 2 < (int64_t(1) << 32) && d.K / 64 * max_n * 4 < (int64_t(1) << 32) && d.M * max_n * 2 < (int64_t(1) << 32)))
+    return fail(TTAMD_EUNSUPPORTED, "nf4_group_dx: operands too large for 32-bit offsets (M=%lld K=%lld N=%lld)", (long long)d.M,
+                (long long)d.K, (long long)max_n);
+  RsArgs g = {};
+  g.C = reinterpret_cast<uint16_t*>(gx);
+  g.M = (int)d.M; g.Nout = (int)d.K;
+  g.lw_row_major = 0;
+  g.ldlx = d.r_off[d.n];
+  g.lscale = 1.0f;
+  const int64_t tiles256 = ((d.M + 255) / 256) * ((d.K + kBN - 1) / kBN);
+  return tiles256 >= 256 ? launch_rs<256, 1, false, true>(g, 1, s, &sg) : launch_rs<128, 1, false, true>(g, 1, s, &sg);
 }
 
 }  // namespace ttamd

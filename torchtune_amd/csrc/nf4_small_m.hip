@@ -14,6 +14,7 @@
 // bound: a launch lives for a few trips to memory, and the expansion (about three vector instructions per element) is
 // not hidden behind them.
 #include "common.h"
+#include "group.h"
 #include "nf4_math.h"
 
 namespace ttamd {
@@ -38,13 +39,20 @@ struct SmallMArgs {
   const uint16_t* x;       // [M, K] bf16
   const uint8_t* codes;    // [N, K/2]
   const float* bscal;      // [N, K/64]
-  const uint16_t* h;       // [M, R] bf16 or null
+  const uint16_t* h;       // [M, R] bf16 (rows ldh elements apart) or null
   const uint16_t* lora_b;  // [N, R] bf16 or null
   const uint16_t* bias;    // [N] bf16 or null
   const uint16_t* cscale;  // [N] bf16 or null
   uint16_t* y;             // [M, N] bf16
-  int M, N, K, R;
+  int M, N, K, R, ldh;
   float lscale;
+};
+// The layers of one launch: they share x, M and K (projections of a common input); workgroups [wg_end[i - 1], wg_end[i])
+// work on layer i.
+struct SmallMGroup {
+  SmallMArgs m[kGroupMax];
+  int wg_end[kGroupMax];
+  int n;
 };
 
 constexpr int kSmMaxWaves = 16;
@@ -119,7 +127,13 @@ __device__ __forceinline__ float nf4_code_value(int k) {
 
 // MT 16-token tiles of x, RT 16-row tiles of W per workgroup, U chunks of K in flight per wave.
 template <int MT, int RT, int U>
-__global__ __launch_bounds__(64 * kSmMaxWaves) void nf4_small_m_kernel(const SmallMArgs a) {
+__global__ __launch_bounds__(64 * kSmMaxWaves) void nf4_small_m_kernel(const SmallMGroup grp) {
+  int which = 0;  // uniform over the workgroup
+#pragma unroll
+  for (int q = 0; q < kGroupMax - 1; ++q)
+    if (q < grp.n - 1 && (int)blockIdx.x >= grp.wg_end[q]) which = q + 1;
+  const SmallMArgs& a = grp.m[which];
+  const int wg = (int)blockIdx.x - (which ? grp.wg_end[which - 1] : 0);
   constexpr int NACC = MT * RT == 1 ? 4 : (MT * RT == 2 ? 2 : 1);  // independent MFMA chains per lane: at least four
   __shared__ float2 lut[256];
   extern __shared__ float red[];  // [waves - 1][MT * RT * 4][64]
@@ -129,7 +143,7 @@ __global__ __launch_bounds__(64 * kSmMaxWaves) void nf4_small_m_kernel(const Sma
   const int i = lane & 15, g = lane >> 4;
 
   const int K = a.K;
-  const int n0 = blockIdx.x * (16 * RT);  // N % (16 RT) == 0: every row of the workgroup exists
+  const int n0 = wg * (16 * RT);  // N % (16 RT) == 0: every row of the workgroup exists
   const uint8_t* crow = a.codes + (((int64_t)(n0 + i) * K) >> 1) + 16 * g;
   const float* srow = a.bscal + (int64_t)(n0 + i) * (K >> 6) + (g >> 1);
   const int64_t ctile = (int64_t)8 * K, stile = (int64_t)16 * (K >> 6);  // one 16-row tile further on
@@ -213,7 +227,7 @@ __global__ __launch_bounds__(64 * kSmMaxWaves) void nf4_small_m_kernel(const Sma
         // adapter: sum_r bf16(h[m][r] * lscale) * lora_b[n][r], the operands the large-M kernel feeds its MFMA
         float l4[4] = {0.f, 0.f, 0.f, 0.f};
         for (int r0 = 0; r0 < a.R; r0 += 8) {
-          const u32x4_t hv = *reinterpret_cast<const u32x4_t*>(a.h + (int64_t)m * a.R + r0);
+          const u32x4_t hv = *reinterpret_cast<const u32x4_t*>(a.h + (int64_t)m * a.ldh + r0);
           float hs[8];
 #pragma unroll
           for (int d = 0; d < 4; ++d) {
@@ -238,18 +252,47 @@ __global__ __launch_bounds__(64 * kSmMaxWaves) void nf4_small_m_kernel(const Sma
   }
 }
 
+// Shape of a launch: token tiles, row tiles per workgroup, chunks in flight per wave, most waves.  It fixes the order
+// in which a row's products are summed, so a layer gets the same bits alone and inside a group.
+struct SmallMConfig {
+  int mt, rt, u, max_waves;
+  bool operator==(const SmallMConfig& o) const { return mt == o.mt && rt == o.rt && u == o.u && max_waves == o.max_waves; }
+};
+// Measured on MI355X over the projections of an 8B model (kernel time, M = 1 / 8 / 32 / 64): 4096 x 4096
+// 7 / 7 / 13 / 20 us, 14336 x 4096 15 / 17 / 26 / 43 us, 4096 x 14336 14 / 18 / 37 / 64 us.  Wide layers share an x
+// fragment between two row tiles once x is more than one token tile (x comes from L2 once per workgroup); long
+// contractions get sixteen waves, short ones four.
+SmallMConfig small_m_config(int64_t M, int64_t N, int64_t K) {
+  const bool wide = N >= 8192, deep = K >= 8192;
+  if (M <= 16) return {1, 1, 4, 16};
+  if (M <= 32) return wide ? SmallMConfig{2, 2, 4, 4} : SmallMConfig{2, 1, 4, 4};
+  return wide ? SmallMConfig{4, 2, 2, 4} : SmallMConfig{4, 1, 4, deep ? 16 : 4};
+}
+
 template <int MT, int RT, int U>
-int launch_small_m(const SmallMArgs& a, int max_waves, hipStream_t s) {
-  int nw = ((a.K >> 7) + U - 1) / U;  // one group of U chunks per wave when K is short enough
+int launch_small_m(SmallMGroup& g, int max_waves, hipStream_t s) {
+  const int K = g.m[0].K;
+  int nw = ((K >> 7) + U - 1) / U;  // one group of U chunks per wave when K is short enough
   nw = nw > 1 ? nw : 1;
   nw = nw < max_waves ? nw : max_waves;
   // the partial sums of waves 1 .. nw - 1 must fit the 64 KB of LDS a workgroup gets without asking for more
   const int per_wave = MT * RT * 4 * 64 * (int)sizeof(float);
   const int fit = 1 + (63 * 1024) / per_wave;
   nw = nw < fit ? nw : fit;
-  const dim3 grid((unsigned)(a.N / (16 * RT))), block(64 * nw);
-  nf4_small_m_kernel<MT, RT, U><<<grid, block, (size_t)(nw - 1) * per_wave, s>>>(a);
+  int wgs = 0;
+  for (int i = 0; i < g.n; ++i) {
+    wgs += g.m[i].N / (16 * RT);
+    g.wg_end[i] = wgs;
+  }
+  const dim3 grid((unsigned)wgs), block(64 * nw);
+  nf4_small_m_kernel<MT, RT, U><<<grid, block, (size_t)(nw - 1) * per_wave, s>>>(g);
   return check_launch("nf4_small_m");
+}
+
+int dispatch_small_m(SmallMGroup& g, const SmallMConfig& c, hipStream_t s) {
+  if (c.mt == 1) return launch_small_m<1, 1, 4>(g, c.max_waves, s);
+  if (c.mt == 2) return c.rt == 2 ? launch_small_m<2, 2, 4>(g, c.max_waves, s) : launch_small_m<2, 1, 4>(g, c.max_waves, s);
+  return c.rt == 2 ? launch_small_m<4, 2, 2>(g, c.max_waves, s) : launch_small_m<4, 1, 4>(g, c.max_waves, s);
 }
 
 }  // namespace
@@ -257,13 +300,15 @@ int launch_small_m(const SmallMArgs& a, int max_waves, hipStream_t s) {
 // Largest token count the small-M kernel takes; above it the tiled kernel runs.
 int small_m_limit() { return 64; }
 
-// Entry used by the C-ABI wrappers in nf4_gemm.hip (arguments already validated there: N % 64 == 0, K % 64 == 0,
-// R % 8 == 0, pointers aligned).  `bscal` is the natural [N, K/64] scaler layout.
-int run_small_m(const void* x, const uint8_t* codes, const void* bscal, const void* h, const void* lora_b, int R, float lscale,
-                const void* bias, const void* cscale, void* y, int64_t M, int64_t N, int64_t K, hipStream_t s) {
+// Entries used by the C-ABI wrappers (arguments already validated there: N % 64 == 0, K % 64 == 0, R % 8 == 0, pointers
+// aligned).  `bscal` is the natural [N, K/64] scaler layout; the rows of `h` are ldh elements apart.
+int run_small_m(const void* x, const uint8_t* codes, const void* bscal, const void* h, int ldh, const void* lora_b, int R,
+                float lscale, const void* bias, const void* cscale, void* y, int64_t M, int64_t N, int64_t K, hipStream_t s) {
   TT_REQUIRE(M > 0 && M <= small_m_limit(), "nf4_small_m: M (%lld) out of range", (long long)M);
   TT_REQUIRE(N / 16 < (int64_t(1) << 31) && N * K < (int64_t(1) << 40), "nf4_small_m: weight too large");
-  SmallMArgs a;
+  SmallMGroup g = {};
+  g.n = 1;
+  SmallMArgs& a = g.m[0];
   a.x = reinterpret_cast<const uint16_t*>(x);
   a.codes = codes;
   a.bscal = reinterpret_cast<const float*>(bscal);
@@ -272,16 +317,39 @@ int run_small_m(const void* x, const uint8_t* codes, const void* bscal, const vo
   a.bias = reinterpret_cast<const uint16_t*>(bias);
   a.cscale = reinterpret_cast<const uint16_t*>(cscale);
   a.y = reinterpret_cast<uint16_t*>(y);
-  a.M = (int)M; a.N = (int)N; a.K = (int)K; a.R = R;
+  a.M = (int)M; a.N = (int)N; a.K = (int)K; a.R = R; a.ldh = ldh;
   a.lscale = lscale;
-  // Measured on MI355X over the projections of an 8B model (kernel time, M = 1 / 8 / 32 / 64): 4096 x 4096
-  // 7 / 7 / 13 / 20 us, 14336 x 4096 15 / 17 / 26 / 43 us, 4096 x 14336 14 / 18 / 37 / 64 us.  Wide layers share an x
-  // fragment between two row tiles once x is more than one token tile (x comes from L2 once per workgroup); long
-  // contractions get sixteen waves, short ones four.
-  const bool wide = N >= 8192, deep = K >= 8192;
-  if (M <= 16) return launch_small_m<1, 1, 4>(a, 16, s);
-  if (M <= 32) return wide ? launch_small_m<2, 2, 4>(a, 4, s) : launch_small_m<2, 1, 4>(a, 4, s);
-  return wide ? launch_small_m<4, 2, 2>(a, 4, s) : launch_small_m<4, 1, 4>(a, deep ? 16 : 4, s);
+  return dispatch_small_m(g, small_m_config(M, N, K), s);
+}
+
+// The members of a group (same x, M, K) in as few launches as their launch shapes allow: consecutive members with
+// the same shape share one.
+int run_small_m_group(const void* x, const GroupGemm& gg, const void* h_cat, hipStream_t s) {
+  TT_REQUIRE(gg.M > 0 && gg.M <= small_m_limit(), "nf4_small_m: M (%lld) out of range", (long long)gg.M);
+  int i = 0;
+  while (i < gg.n) {
+    const SmallMConfig c = small_m_config(gg.M, gg.N[i], gg.K);
+    SmallMGroup g = {};
+    int j = i;
+    for (; j < gg.n && small_m_config(gg.M, gg.N[j], gg.K) == c; ++j) {
+      TT_REQUIRE(gg.N[j] / 16 < (int64_t(1) << 27) && gg.N[j] * gg.K < (int64_t(1) << 40), "nf4_small_m: weight too large");
+      SmallMArgs& a = g.m[j - i];
+      a.x = reinterpret_cast<const uint16_t*>(x);
+      a.codes = gg.codes[j];
+      a.bscal = gg.bscal[j];
+      a.h = reinterpret_cast<const uint16_t*>(h_cat) + gg.r_off[j];
+      a.lora_b = gg.lora_b[j];
+      a.bias = gg.bias[j];
+      a.cscale = nullptr;
+      a.y = gg.y[j];
+      a.M = (int)gg.M; a.N = (int)gg.N[j]; a.K = (int)gg.K; a.R = gg.rank[j]; a.ldh = gg.r_off[gg.n];
+      a.lscale = gg.scale[j];
+    }
+    g.n = j - i;
+    if (int rc = dispatch_small_m(g, c, s)) return rc;
+    i = j;
+  }
+  return TTAMD_OK;
 }
 
 }  // namespace ttamd

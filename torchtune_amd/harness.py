@@ -28,8 +28,13 @@ from torch.nn.attention import SDPBackend, sdpa_kernel
 from torch.utils.checkpoint import checkpoint
 
 from .modules import layer_ops
-from .modules.peft import LoRALinear, get_adapter_params, set_trainable_params
+from .modules.peft import LoRALinear, get_adapter_params, lora_linear_group, set_trainable_params
 from .qat import Int8DynActInt4WeightQATQuantizer
+
+
+# True: projections that read the same tensor (q/k/v, gate/up) go through the group kernels; False: one call per
+# projection, as the reference's modules make them (kept for A/B timing and for the tests that compare the two)
+GROUP_SHARED_INPUT = True
 
 
 @dataclass(frozen=True)
@@ -137,9 +142,12 @@ class Attention(nn.Module):
 
     def forward(self, x: torch.Tensor, rope: torch.Tensor) -> torch.Tensor:
         b, sl, _ = x.shape
-        q = self.q_proj(x).view(b, sl, self.n_heads, self.head_dim)
-        k = self.k_proj(x).view(b, sl, self.n_kv, self.head_dim)
-        v = self.v_proj(x).view(b, sl, self.n_kv, self.head_dim)
+        # the three projections read the same tensor (torchtune/modules/attention.py:234,262-263): one group
+        q, k, v = lora_linear_group(x, (self.q_proj, self.k_proj, self.v_proj)) if GROUP_SHARED_INPUT else (
+            self.q_proj(x), self.k_proj(x), self.v_proj(x))
+        q = q.view(b, sl, self.n_heads, self.head_dim)
+        k = k.view(b, sl, self.n_kv, self.head_dim)
+        v = v.view(b, sl, self.n_kv, self.head_dim)
         q = apply_rope(q, rope)
         k = apply_rope(k, rope)
         if self.n_kv != self.n_heads:  # expand kv heads to query heads, as the reference does before SDPA
@@ -161,7 +169,8 @@ class FeedForward(nn.Module):
         self.w3 = _linear(s.dim, s.hidden, rank, alpha, quantize_base)  # up
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        g, u = self.w1(x), self.w3(x)
+        # gate and up read the same tensor (torchtune/modules/feed_forward.py:50-53): one group
+        g, u = lora_linear_group(x, (self.w1, self.w3)) if GROUP_SHARED_INPUT else (self.w1(x), self.w3(x))
         return self.w2(layer_ops.swiglu(g, u) if _fused(g) else F.silu(g) * u)
 
 

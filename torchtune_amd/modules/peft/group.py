@@ -1,0 +1,94 @@
+"""LoRA linears that read the same input, computed as one group.
+
+The reference calls such layers one after the other on one tensor: ``q_proj``, ``k_proj`` and ``v_proj`` in
+``torchtune/modules/attention.py:234,262-263`` and ``w1`` / ``w3`` in ``torchtune/modules/feed_forward.py:50-53``, each a
+``LoRALinear.forward`` (``torchtune/modules/peft/lora.py:128-147``).  ``lora_linear_group(x, layers)`` returns what those
+calls return.  When every layer takes the fused QLoRA path it runs the group kernels instead: one pass over ``x`` for all
+hidden activations ``x @ A_i.T``, one launch for the members' outputs at decode sizes, and in backward one pass over
+``x`` for all ``grad A_i`` and a single grad-input GEMM over the members' concatenated output columns (fp32 sum over
+the members, one rounding) in place of one GEMM per member plus the additions autograd would make.  Otherwise it
+falls back to calling the layers in turn.
+"""
+from __future__ import annotations
+
+from typing import List, Sequence, Tuple
+
+import torch
+
+from ... import ops
+from ...nf4_tensor import _check_in_features
+from .lora import LoRALinear
+
+
+def _member(layer: LoRALinear) -> ops.GroupMember:
+    w = layer.weight
+    return ops.GroupMember(w.quantized_data, w.block_scalers(), w.backward_copy(), layer.lora_a.weight, layer.lora_b.weight,
+                           layer.bias, layer.alpha / layer.rank, w.shape[0])
+
+
+class _QLoRAGroupFn(torch.autograd.Function):
+    """Inputs: x [..., K], then per member (weight, lora_a, lora_b, bias or None); outputs: one y per member."""
+
+    @staticmethod
+    def forward(ctx, x, scales: Tuple[float, ...], *flat):
+        n = len(scales)
+        weights, las, lbs, biases = flat[0::4], flat[1::4], flat[2::4], flat[3::4]
+        K = weights[0].shape[1]
+        for w in weights:
+            _check_in_features(x, w)
+        x2 = x.reshape(-1, K)
+        members = [ops.GroupMember(w.quantized_data, w.block_scalers(), w.backward_copy(), a, b, bias, s, w.shape[0])
+                   for w, a, b, bias, s in zip(weights, las, lbs, biases, scales)]
+        h_cat, ys = ops.lora_group_fwd(x2, members)
+        ctx.save_for_backward(x2, h_cat, *weights, *las, *lbs)
+        ctx.scales = scales
+        ctx.x_shape = x.shape
+        ctx.has_bias = tuple(b is not None for b in biases)
+        outs = tuple(y.view(*x.shape[:-1], y.shape[-1]) for y in ys)
+        return outs if n > 1 else outs[0]
+
+    @staticmethod
+    def backward(ctx, *gys):
+        n = len(ctx.scales)
+        saved = ctx.saved_tensors  # read once: activation checkpointing unpacks on every access
+        x2, h_cat = saved[:2]
+        rest = saved[2:]
+        weights, las, lbs = rest[:n], rest[n:2 * n], rest[2 * n:3 * n]
+        gy2 = []
+        for g, w in zip(gys, weights):
+            # an output nobody used arrives as None
+            gy2.append(torch.zeros(x2.shape[0], w.shape[0], dtype=x2.dtype, device=x2.device) if g is None
+                       else g.reshape(-1, w.shape[0]))
+        members = [ops.GroupMember(w.quantized_data, w.block_scalers(), w.backward_copy(), a, b, None, s, w.shape[0])
+                   for w, a, b, s in zip(weights, las, lbs, ctx.scales)]
+        need_x = ctx.needs_input_grad[0]
+        gx, grads, _ = ops.lora_group_bwd(x2, h_cat, members, gy2, want_gx=need_x)
+        out: List = [gx.view(ctx.x_shape) if need_x else None, None]
+        for i in range(n):
+            _, need_a, need_b, need_bias = ctx.needs_input_grad[2 + 4 * i:6 + 4 * i]
+            out += [None, grads[i][0] if need_a else None, grads[i][1] if need_b else None,
+                    gy2[i].sum(dim=0) if (ctx.has_bias[i] and need_bias) else None]
+        return tuple(out)
+
+
+def group_applies(x: torch.Tensor, layers: Sequence[torch.nn.Module]) -> bool:
+    """True when ``lora_linear_group`` runs the group kernels for these layers on this input."""
+    if not 1 <= len(layers) <= ops._lib.GROUP_MAX:
+        return False
+    for layer in layers:
+        if type(layer) is not LoRALinear or layer.disabled or not layer._fused(x):
+            return False
+        if layer.in_dim != layers[0].in_dim or layer.weight.backward_copy() is None:
+            return False
+    return ops.group_shape_ok([l.out_dim for l in layers], layers[0].in_dim, [l.rank for l in layers])
+
+
+def lora_linear_group(x: torch.Tensor, layers: Sequence[torch.nn.Module]) -> Tuple[torch.Tensor, ...]:
+    """``tuple(layer(x) for layer in layers)`` for layers that share the input ``x``."""
+    if not group_applies(x, layers):
+        return tuple(layer(x) for layer in layers)
+    flat = []
+    for layer in layers:
+        flat += [layer.weight, layer.lora_a.weight, layer.lora_b.weight, layer.bias]
+    out = _QLoRAGroupFn.apply(x, tuple(layer.alpha / layer.rank for layer in layers), *flat)
+    return out if isinstance(out, tuple) else (out,)

@@ -5,7 +5,7 @@ Every function requires HIP (``cuda``) tensors.  There is no CPU implementation 
 """
 from __future__ import annotations
 
-from typing import Optional, Tuple
+from typing import Optional, Sequence, Tuple
 
 import torch
 
@@ -153,7 +153,8 @@ _gemm_timer = None
 
 def set_gemm_timer(timer) -> None:
     """Install (or with None remove) a callback ``timer(kind, M, N, K, rank) -> (start_event, end_event)``; the two
-    events are recorded on the launch stream immediately before and after every fused-GEMM launch.  Used by the
+    events are recorded on the launch stream immediately before and after every fused-GEMM launch (``kind`` "fwd" /
+    "bwd"; for the group calls "fwd_group" / "bwd_group" with ``N`` and ``rank`` lists over the members).  Used by the
     benchmark to time the dominant kernel in place."""
     global _gemm_timer
     _gemm_timer = timer
@@ -337,6 +338,126 @@ def lora_bwd(
         )
     _lib.check(rc, "lora_bwd")
     return gh, ga, gb
+
+
+# ---------------------------------------------------------------------------------------------------
+# Groups of LoRA linears with a common input (q/k/v, gate/up)
+# ---------------------------------------------------------------------------------------------------
+class GroupMember:
+    """Operands of one member: the NF4 parts of its [N, K] weight, its adapter, its bias (or None) and alpha / rank.
+    ``transposed`` is the pair from ``nf4_transpose_for_backward`` or None."""
+
+    __slots__ = ("qdata", "block_scalers", "transposed", "lora_a", "lora_b", "bias", "scale", "N")
+
+    def __init__(self, qdata, block_scalers, transposed, lora_a, lora_b, bias, scale: float, N: int):
+        self.qdata, self.block_scalers, self.transposed = qdata, block_scalers, transposed
+        self.lora_a, self.lora_b, self.bias, self.scale, self.N = lora_a, lora_b, bias, float(scale), int(N)
+
+
+def group_shape_ok(Ns: Sequence[int], K: int, ranks: Sequence[int]) -> bool:
+    """Shapes the group entry points accept."""
+    return (1 <= len(Ns) <= _lib.GROUP_MAX and K % 64 == 0 and all(n % 64 == 0 for n in Ns)
+            and all(r > 0 and r % 8 == 0 for r in ranks) and sum(ranks) <= 64 and max(Ns) >= 128)
+
+
+def _group_array(what: str, members: Sequence[GroupMember], K: int, ys: Sequence[torch.Tensor], M: int,
+                 grads: Optional[Sequence[Tuple[torch.Tensor, torch.Tensor]]] = None):
+    """The C array of member descriptors (and the tensors it points into, which the caller keeps alive)."""
+    if not 1 <= len(members) <= _lib.GROUP_MAX:
+        raise ValueError(f"{what}: a group has 1 to {_lib.GROUP_MAX} members, got {len(members)}")
+    arr = (_lib.LoraGroupMember * len(members))()
+    keep = []
+    for i, m in enumerate(members):
+        _check_nf4_operands(what, m.N, K, m.qdata, m.block_scalers, m.transposed[1] if m.transposed else None)
+        if m.transposed and (m.transposed[0].dtype != torch.uint8 or m.transposed[0].numel() * 2 != m.N * K):
+            raise ValueError(f"{what}: the transposed codes of member {i} do not hold a [{m.N}, {K}] weight")
+        a, b = _bf16_2d(m.lora_a, what), _bf16_2d(m.lora_b, what)
+        r = a.shape[0]
+        if tuple(a.shape) != (r, K) or tuple(b.shape) != (m.N, r):
+            raise ValueError(f"{what}: member {i}: lora_a {tuple(a.shape)} / lora_b {tuple(b.shape)} do not fit a [{m.N}, {K}] layer")
+        y = ys[i]
+        if y.dtype != torch.bfloat16 or tuple(y.shape) != (M, m.N) or not y.is_contiguous():
+            raise ValueError(f"{what}: member {i}: expected a contiguous bfloat16 [{M}, {m.N}] tensor, got {tuple(y.shape)} {y.dtype}")
+        bias = None
+        if m.bias is not None:
+            bias = m.bias.contiguous()
+            if bias.dtype != torch.bfloat16 or bias.numel() != m.N:
+                raise ValueError(f"{what}: member {i}: bias must be bfloat16 with {m.N} elements")
+        e = arr[i]
+        e.quantized_data, e.block_scalers = m.qdata.data_ptr(), m.block_scalers.data_ptr()
+        e.block_scalers_t = m.transposed[1].data_ptr() if m.transposed else None
+        e.quantized_data_t = m.transposed[0].data_ptr() if m.transposed else None
+        e.lora_a, e.lora_b, e.bias, e.y = a.data_ptr(), b.data_ptr(), _ptr(bias), y.data_ptr()
+        if grads is not None:
+            e.grad_lora_a, e.grad_lora_b = grads[i][0].data_ptr(), grads[i][1].data_ptr()
+        e.N, e.rank, e.scale = m.N, r, m.scale
+        keep.append((a, b, bias, y))
+    return arr, keep
+
+
+def lora_group_fwd(x: torch.Tensor, members: Sequence[GroupMember]):
+    """-> (h_cat [M, sum of ranks], [y_i [M, N_i]]): every member's ``y_i = x @ D(W_i).T (+ bias_i) + scale_i * h_i @ B_i.T``
+    with ``h_i = x @ A_i.T`` (columns of ``h_cat``), in one pass over ``x`` for the hidden products."""
+    x = _bf16_2d(x, "lora_group_fwd")
+    M, K = x.shape
+    dev = x.device
+    ys = [torch.empty(M, m.N, dtype=torch.bfloat16, device=dev) for m in members]
+    arr, keep = _group_array("lora_group_fwd", members, K, ys, M)
+    n = len(members)
+    r_total = sum(int(e.rank) for e in arr)
+    h_cat = torch.empty(M, r_total, dtype=torch.bfloat16, device=dev)
+    lib = _lib.load()
+    ws = _workspace(max(lib.ttamd_lora_group_hidden_workspace_bytes(arr, n, M, K), lib.ttamd_lora_group_fwd_workspace_bytes(arr, n, M, K)),
+                    dev)
+    with torch.cuda.device(dev):
+        rc = lib.ttamd_lora_group_hidden_bf16(x.data_ptr(), arr, n, h_cat.data_ptr(), M, K, ws.data_ptr(), ws.numel(), _stream(x))
+        _lib.check(rc, "lora_group_hidden")
+        events = _gemm_timer("fwd_group", M, [m.N for m in members], K, [int(e.rank) for e in arr]) if _gemm_timer is not None else None
+        if events:
+            events[0].record()
+        rc = lib.ttamd_nf4_lora_group_fwd_bf16(x.data_ptr(), arr, n, h_cat.data_ptr(), M, K, ws.data_ptr(), ws.numel(), _stream(x))
+        if events:
+            events[1].record()
+    _lib.check(rc, "lora_group_fwd")
+    del keep
+    return h_cat, ys
+
+
+def lora_group_bwd(x: torch.Tensor, h_cat: torch.Tensor, members: Sequence[GroupMember], gys: Sequence[torch.Tensor],
+                   want_gx: bool = True):
+    """-> (gx [M, K] or None, [(gA_i, gB_i)], gh_cat): the backward of ``lora_group_fwd`` given the output gradients."""
+    x = _bf16_2d(x, "lora_group_bwd")
+    h_cat = _bf16_2d(h_cat, "lora_group_bwd")
+    M, K = x.shape
+    dev = x.device
+    gys = [_bf16_2d(g, "lora_group_bwd") for g in gys]
+    grads = [(torch.empty(m.lora_a.shape, dtype=torch.bfloat16, device=dev), torch.empty(m.lora_b.shape, dtype=torch.bfloat16, device=dev))
+             for m in members]
+    arr, keep = _group_array("lora_group_bwd", members, K, gys, M, grads)
+    n = len(members)
+    r_total = sum(int(e.rank) for e in arr)
+    if tuple(h_cat.shape) != (M, r_total):
+        raise ValueError(f"lora_group_bwd: h_cat is {tuple(h_cat.shape)}, expected {(M, r_total)}")
+    if want_gx and any(m.transposed is None for m in members):
+        raise ValueError("lora_group_bwd: the grouped grad-input needs every member's transposed copy")
+    gh_cat = torch.empty(M, r_total, dtype=torch.bfloat16, device=dev)
+    gx = torch.empty(M, K, dtype=torch.bfloat16, device=dev) if want_gx else None
+    lib = _lib.load()
+    ws = _workspace(lib.ttamd_lora_group_bwd_workspace_bytes(arr, n, M, K), dev)
+    with torch.cuda.device(dev):
+        rc = lib.ttamd_lora_group_bwd_bf16(x.data_ptr(), h_cat.data_ptr(), arr, n, gh_cat.data_ptr(), M, K, ws.data_ptr(), ws.numel(),
+                                           _stream(x))
+        _lib.check(rc, "lora_group_bwd")
+        if want_gx:
+            events = _gemm_timer("bwd_group", M, [m.N for m in members], K, [int(e.rank) for e in arr]) if _gemm_timer is not None else None
+            if events:
+                events[0].record()
+            rc = lib.ttamd_nf4_group_bwd_dx_bf16(arr, n, gh_cat.data_ptr(), gx.data_ptr(), M, K, _stream(x))
+            if events:
+                events[1].record()
+            _lib.check(rc, "nf4_group_bwd_dx")
+    del keep
+    return gx, grads, gh_cat
 
 
 # ---------------------------------------------------------------------------------------------------
