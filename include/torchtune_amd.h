@@ -225,8 +225,18 @@ int ttamd_nf4_linear_bwd_dx_bf16(const void* gy, const uint8_t* quantized_data, 
  *   ttamd_nf4_lora_linear_fwd_ws_bf16: col_scale NULL = ttamd_nf4_lora_linear_fwd_bf16, else = ttamd_nf4_dora_linear_fwd_bf16.
  *   ttamd_nf4_linear_bwd_dx_ws_bf16: slices only the variant with the transposed copies.
  * A workspace smaller than ttamd_nf4_gemm_workspace_bytes says, or NULL, runs the unsliced kernel.
+ *
+ * Many tokens (M >= 2048 and at least 256 output tiles of 256 x 256): the same workspace argument then holds the
+ * weight expanded ONCE per call to bf16 (2 * n_out * k_contract bytes, in the order the matrix cores read it), and a
+ * plain bf16 GEMM with the adapter, bias and column scale in its epilogue runs on it: the reference's own order of
+ * work, F.linear(x, weight.to(dtype)) (torchao linear_nf4, reached from torchtune/modules/peft/lora.py:138), for the
+ * token counts at which the fused kernel's per-tile expansion costs more than one pass of the expansion kernel.
+ * ttamd_nf4_gemm_workspace_bytes reports those bytes; passing less (or NULL) keeps the fused kernel.  The expanded
+ * values are the bits ttamd_nf4_dequantize writes.
  */
 size_t ttamd_nf4_gemm_workspace_bytes(int64_t M, int64_t n_out, int64_t k_contract);
+/* 1 when those bytes are the expanded weight of the many-token path, 0 when they are slices (or none) */
+int ttamd_nf4_gemm_expands_weight(int64_t M, int64_t n_out, int64_t k_contract);
 int ttamd_nf4_lora_linear_fwd_ws_bf16(const void* x, const uint8_t* quantized_data, const void* block_scalers,
                                       const void* block_scalers_t, const void* h, const void* lora_b, int rank, float scale,
                                       const void* bias, const void* col_scale, void* y, int64_t M, int64_t N, int64_t K,
@@ -305,6 +315,11 @@ int ttamd_lora_group_bwd_bf16(const void* x, const void* h_cat, const ttamd_lora
 /* gx out, bf16 [M, K], from gh_cat and members[i].y = gy_i, quantized_data_t, block_scalers_t, lora_a */
 int ttamd_nf4_group_bwd_dx_bf16(const ttamd_lora_group_member* members, int n_members, const void* gh_cat, void* gx, int64_t M,
                                 int64_t K, void* stream);
+/* the same with room for the members' weights expanded once (many tokens, see ttamd_nf4_gemm_workspace_bytes): bytes to
+ * pass (0: the shape is served by the fused kernel), and the call; less workspace than that, or NULL, = the call above */
+size_t ttamd_nf4_group_bwd_dx_workspace_bytes(const ttamd_lora_group_member* members, int n_members, int64_t M, int64_t K);
+int ttamd_nf4_group_bwd_dx_ws_bf16(const ttamd_lora_group_member* members, int n_members, const void* gh_cat, void* gx, int64_t M,
+                                   int64_t K, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
  * QAT fake quantisation (int8 dynamic per-token activations, int4 per-group symmetric weights)

@@ -1,0 +1,196 @@
+"""GPU parity of the many-token path of the NF4 + LoRA linear: the weight expanded once per call into scratch memory,
+then the plain bf16 GEMM (``nf4_gemm_dense.hip``), forward and grad-input, single layers and groups.
+
+Three kinds of checks:
+* bit-exact: with one-hot activations every output is a single product 1 * Wd[n][k], so the GEMM's output IS the expanded
+  weight; it must equal ``ops.nf4_dequantize`` (itself bit-exact against the oracle in tests/test_gpu_nf4.py) bit for
+  bit, for the three layouts the expansion kernel reads (natural scalers, transposed scalers, transposed copy);
+* against the CPU oracle (the reference's unfused bf16 graph), rtol 1e-2 / atol 1e-2 as for the fused kernel;
+* against the fused kernel on the same inputs (both accumulate in fp32 and round once, in a different order of
+  summation): rtol 1e-2 / atol 2e-3 at unit-variance activations.
+"""
+import pytest
+import torch
+
+from oracle import lora_oracle, nf4_oracle
+from torchtune_amd import _lib, ops
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+BF = torch.bfloat16
+
+
+def _quantized(N, K, seed):
+    g = torch.Generator().manual_seed(seed)
+    W = (torch.randn(N, K, generator=g) * 0.02).to(BF)
+    n_blocks = N * K // 64
+    sbs = 256 if n_blocks % 256 == 0 else n_blocks
+    qdata, qscal, qfac, mean = ops.nf4_quantize(W.to(DEV), 64, sbs)[:4]
+    bscal = ops.nf4_block_scalers(qscal, qfac, mean, sbs)
+    dense = ops.nf4_dequantize(qdata, qscal, qfac, mean, (N, K), 64, sbs)
+    return W, sbs, qdata, bscal, dense
+
+
+def _expands(M, n_out, k):
+    return bool(_lib.load().ttamd_nf4_gemm_expands_weight(M, n_out, k))
+
+
+def _one_hot(M, K):
+    x = torch.zeros(M, K, dtype=BF, device=DEV)
+    x[torch.arange(M, device=DEV), torch.arange(M, device=DEV) % K] = 1.0
+    return x
+
+
+@pytest.mark.parametrize("N,K,with_transposed_scalers", [(8192, 256, False), (8192, 256, True), (8256, 192, True)])
+def test_forward_output_is_the_expanded_weight_bit_for_bit(N, K, with_transposed_scalers):
+    M = 2048
+    assert _expands(M, N, K)
+    _, _, qdata, bscal, dense = _quantized(N, K, seed=N + K)
+    scal_t = ops.nf4_transpose_for_backward(qdata, bscal, N, K)[1] if with_transposed_scalers else None
+    y = ops.nf4_lora_linear_fwd(_one_hot(M, K), qdata, bscal, N, block_scalers_t=scal_t)
+    want = dense.t().repeat((M + K - 1) // K, 1)[:M]  # row m = column m % K of the weight
+    assert torch.equal(y.view(torch.int16), want.contiguous().view(torch.int16))
+
+
+def test_grad_input_output_is_the_expanded_weight_bit_for_bit():
+    M, N, K = 2048, 256, 8192
+    assert _expands(M, K, N)
+    _, _, qdata, bscal, dense = _quantized(N, K, seed=7)
+    tr = ops.nf4_transpose_for_backward(qdata, bscal, N, K)
+    gx = ops.nf4_linear_bwd_dx(_one_hot(M, N), qdata, bscal, K, transposed=tr)
+    want = dense.repeat((M + N - 1) // N, 1)[:M]  # row m = row m % N of the weight
+    assert torch.equal(gx.view(torch.int16), want.contiguous().view(torch.int16))
+
+
+CASES = [
+    # M, N, K, rank, bias: at least 256 tiles of 256 x 256 and 2048 tokens, so the library expands the weight
+    (2048, 8192, 256, 16, False),
+    (2048 + 37, 8192, 192, 8, True),      # ragged token count (a ninth, partial m-tile)
+    (4096, 4096 + 64, 320, 24, True),     # output width not a multiple of the tile, rank not a multiple of 16
+    (4096, 4096, 512, 64, False),         # two 32-wide steps of the adapter contraction
+    (2048, 8192, 128, 0, True),           # no adapter (FrozenNF4Linear / linear_nf4)
+]
+
+
+def _case(M, N, K, r, bias, seed):
+    g = torch.Generator().manual_seed(seed)
+    W, sbs, qdata, bscal, dense = _quantized(N, K, seed)
+    A = lora_oracle.lora_a_init_(torch.empty(max(r, 1), K), g).to(BF)[:r] if r else None
+    B = (torch.randn(N, r, generator=g) * 0.01).to(BF) if r else None
+    b = (torch.randn(N, generator=g) * 0.1).to(BF) if bias else None
+    x = torch.randn(M, K, generator=g).to(BF)
+    gy = torch.randn(M, N, generator=g).to(BF)
+    return W, sbs, qdata, bscal, dense, A, B, b, x, gy
+
+
+def _run(M, N, K, r, scale, qdata, bscal, A, B, b, x, gy, tr):
+    xd, gyd = x.to(DEV), gy.to(DEV)
+    h = ops.lora_hidden(xd, A.to(DEV)) if r else None
+    y = ops.nf4_lora_linear_fwd(xd, qdata, bscal, N, h, B.to(DEV) if r else None, scale, b.to(DEV) if b is not None else None,
+                                block_scalers_t=tr[1])
+    gh = ops.lora_bwd(gyd, xd, h, B.to(DEV), scale)[0] if r else None
+    gx = ops.nf4_linear_bwd_dx(gyd, qdata, bscal, K, gh, A.to(DEV) if r else None, transposed=tr)
+    return y, gx
+
+
+@pytest.mark.parametrize("M,N,K,r,bias", CASES)
+def test_expanded_path_vs_oracle_and_vs_fused_kernel(M, N, K, r, bias, monkeypatch):
+    assert _expands(M, N, K)
+    alpha = 2.0 * max(r, 1)
+    scale = alpha / max(r, 1)
+    W, sbs, qdata, bscal, dense, A, B, b, x, gy = _case(M, N, K, r, bias, seed=M + N + K + r)
+    tr = ops.nf4_transpose_for_backward(qdata, bscal, N, K)
+    y, gx = _run(M, N, K, r, scale, qdata, bscal, A, B, b, x, gy, tr)
+    monkeypatch.setattr(ops, "EXPANDED_WEIGHT_PATH", False)
+    y_f, gx_f = _run(M, N, K, r, scale, qdata, bscal, A, B, b, x, gy, tr)
+    torch.testing.assert_close(y.float(), y_f.float(), rtol=1e-2, atol=2e-3)
+    if _expands(M, K, N):
+        torch.testing.assert_close(gx.float(), gx_f.float(), rtol=1e-2, atol=2e-3)
+    # the oracle: the reference's unfused bf16 graph on the CPU
+    p = nf4_oracle.nf4_quantize(W, 64, sbs)
+    xo = x.clone().requires_grad_()
+    if r:
+        yo = lora_oracle.lora_linear_forward(xo, p, A, B, alpha, r, bias=b)
+    else:
+        yo = lora_oracle.lora_linear_forward(xo, p, None, None, 0.0, 1, bias=b, disabled=True)
+    yo.backward(gy)
+    torch.testing.assert_close(y.cpu().float(), yo.detach().float(), rtol=1e-2, atol=1e-2)
+    torch.testing.assert_close(gx.cpu().float(), xo.grad.float(), rtol=1e-2, atol=1e-2)
+
+
+def test_grad_input_expanded_at_a_wide_layer_vs_fp32_matmul():
+    """Grad-input with the contraction over a long output dimension (the shape class of gate / up projections)."""
+    M, N, K = 2048, 1024, 8192
+    assert _expands(M, K, N)
+    _, _, qdata, bscal, dense = _quantized(N, K, seed=3)
+    g = torch.Generator().manual_seed(5)
+    gy = torch.randn(M, N, generator=g).to(BF).to(DEV)
+    A = (torch.randn(16, K, generator=g) * 0.02).to(BF).to(DEV)
+    gh = torch.randn(M, 16, generator=g).to(BF).to(DEV)
+    tr = ops.nf4_transpose_for_backward(qdata, bscal, N, K)
+    gx = ops.nf4_linear_bwd_dx(gy, qdata, bscal, K, gh, A, transposed=tr)
+    want = gy.float() @ dense.float() + gh.float() @ A.float()
+    torch.testing.assert_close(gx.float(), want, rtol=1e-2, atol=1e-2)
+
+
+def test_column_scale_in_the_epilogue():
+    """DoRA's per-column factor is applied after the bias, as in the fused kernel: y = (x W^T + s h B^T + bias) * c."""
+    M, N, K, r = 2048, 8192, 128, 16
+    W, sbs, qdata, bscal, dense, A, B, b, x, gy = _case(M, N, K, r, True, seed=11)
+    g = torch.Generator().manual_seed(13)
+    c = (1.0 + 0.1 * torch.randn(N, generator=g)).to(BF)
+    xd = x.to(DEV)
+    h = ops.lora_hidden(xd, A.to(DEV))
+    y = ops.nf4_lora_linear_fwd(xd, qdata, bscal, N, h, B.to(DEV), 2.0, b.to(DEV), col_scale=c.to(DEV))
+    want = (xd.float() @ dense.float().T + 2.0 * h.float() @ B.to(DEV).float().T + b.to(DEV).float()) * c.to(DEV).float()
+    torch.testing.assert_close(y.float(), want, rtol=1e-2, atol=1e-2)
+
+
+def test_group_grad_input_over_concatenated_members(monkeypatch):
+    """gx of q / k / v-like members with a common input: one expanded GEMM over the members' concatenated output
+    columns against the fused kernel's grouped launch and against fp32 matmuls of the dequantised weights."""
+    M, K = 2048, 8192
+    Ns, ranks = (512, 128, 192), (16, 8, 16)
+    g = torch.Generator().manual_seed(17)
+    x = torch.randn(M, K, generator=g).to(BF).to(DEV)
+    members, gys, denses = [], [], []
+    for i, (N, r) in enumerate(zip(Ns, ranks)):
+        _, _, qdata, bscal, dense = _quantized(N, K, seed=20 + i)
+        A = (torch.randn(r, K, generator=g) * 0.02).to(BF).to(DEV)
+        B = (torch.randn(N, r, generator=g) * 0.01).to(BF).to(DEV)
+        tr = ops.nf4_transpose_for_backward(qdata, bscal, N, K)
+        members.append(ops.GroupMember(qdata=qdata, block_scalers=bscal, N=N, lora_a=A, lora_b=B, scale=2.0, bias=None, transposed=tr))
+        gys.append(torch.randn(M, N, generator=g).to(BF).to(DEV))
+        denses.append(dense)
+    assert _lib.load().ttamd_nf4_group_bwd_dx_workspace_bytes(ops._group_array("t", members, K, gys, M)[0], len(members), M, K) == 2 * K * sum(Ns)
+    h_cat, _ = ops.lora_group_fwd(x, members)
+    gx, _, gh_cat = ops.lora_group_bwd(x, h_cat, members, gys)
+    monkeypatch.setattr(ops, "EXPANDED_WEIGHT_PATH", False)
+    gx_f, _, _ = ops.lora_group_bwd(x, h_cat, members, gys)
+    torch.testing.assert_close(gx.float(), gx_f.float(), rtol=1e-2, atol=2e-3)
+    want = torch.zeros(M, K, dtype=torch.float32, device=DEV)
+    off = 0
+    for m, gy, dense, r in zip(members, gys, denses, ranks):
+        want += gy.float() @ dense.float() + gh_cat[:, off:off + r].float() @ m.lora_a.float()
+        off += r
+    torch.testing.assert_close(gx.float(), want, rtol=1e-2, atol=1e-2)
+
+
+def test_smaller_workspace_keeps_the_fused_kernel():
+    """The ABI rule: less workspace than ``ttamd_nf4_gemm_workspace_bytes`` says (or none) is not an error."""
+    M, N, K = 2048, 8192, 128
+    _, _, qdata, bscal, dense = _quantized(N, K, seed=23)
+    x = torch.randn(M, K, generator=torch.Generator().manual_seed(1)).to(BF).to(DEV)
+    lib = _lib.load()
+    need = lib.ttamd_nf4_gemm_workspace_bytes(M, N, K)
+    assert need == 2 * N * K
+    y = [torch.empty(M, N, dtype=BF, device=DEV) for _ in range(3)]
+    ws = torch.empty(need, dtype=torch.uint8, device=DEV)
+    s = torch.cuda.current_stream().cuda_stream
+    for out, (p, nbytes) in zip(y, [(ws.data_ptr(), need), (ws.data_ptr(), need - 1), (None, 0)]):
+        rc = lib.ttamd_nf4_lora_linear_fwd_ws_bf16(x.data_ptr(), qdata.data_ptr(), bscal.data_ptr(), None, None, None, 0, 0.0, None, None,
+                                                   out.data_ptr(), M, N, K, p, nbytes, s)
+        _lib.check(rc, "fwd_ws")
+    assert torch.equal(y[1], y[2])  # both ran the fused kernel
+    torch.testing.assert_close(y[0].float(), y[1].float(), rtol=1e-2, atol=2e-3)
+    torch.testing.assert_close(y[0].float(), x.float() @ dense.float().T, rtol=1e-2, atol=1e-2)

@@ -89,21 +89,23 @@ def test_layer_forward_backward_vs_oracle(M, N, K, r, bias):
 # down compare with fp32 matmuls of the HIP-dequantised weight, which is a parity statement only because that
 # dequantisation is bit-exact against the oracle in tests/test_gpu_nf4.py).
 KERNEL_VARIANTS = [
-    # name, M, N, K, rank, keep the transposed copy for the grad-input GEMM
-    ("few-token forward (weight streaming), tiled grad-input", 8, 1024, 1024, 16, True),
-    ("sliced contraction, forward (8 tiles x 16 slices)", 256, 1024, 4096, 16, True),
-    ("sliced contraction, grad-input (8 tiles x 16 slices)", 256, 4096, 1024, 16, True),
-    ("128-row tiles, forward and grad-input", 4096, 1024, 1024, 8, True),
-    ("256-row tiles, forward and grad-input", 4096, 4096, 512, 8, True),
-    ("grad-input without the transposed copy (tile transposed on the fly)", 1024, 512, 1024, 16, False),
+    # name, M, N, K, rank, keep the transposed copy for the grad-input GEMM, let the library expand the weight once
+    ("few-token forward (weight streaming), tiled grad-input", 8, 1024, 1024, 16, True, True),
+    ("sliced contraction, forward (8 tiles x 16 slices)", 256, 1024, 4096, 16, True, True),
+    ("sliced contraction, grad-input (8 tiles x 16 slices)", 256, 4096, 1024, 16, True, True),
+    ("128-row tiles, forward and grad-input", 4096, 1024, 1024, 8, True, True),
+    ("256-row tiles, forward and grad-input", 4096, 4096, 512, 8, True, False),
+    ("weight expanded once, forward and grad-input", 4096, 4096, 512, 8, True, True),
+    ("grad-input without the transposed copy (tile transposed on the fly)", 1024, 512, 1024, 16, False, True),
 ]
 
 
-@pytest.mark.parametrize("name,M,N,K,r,backward_copy", KERNEL_VARIANTS, ids=[v[0].split(",")[0].split(" (")[0].replace(" ", "_") + f"_{i}" for i, v in enumerate(KERNEL_VARIANTS)])
-def test_each_kernel_variant_vs_oracle(name, M, N, K, r, backward_copy, monkeypatch):
+@pytest.mark.parametrize("name,M,N,K,r,backward_copy,expanded", KERNEL_VARIANTS, ids=[v[0].split(",")[0].split(" (")[0].replace(" ", "_") + f"_{i}" for i, v in enumerate(KERNEL_VARIANTS)])
+def test_each_kernel_variant_vs_oracle(name, M, N, K, r, backward_copy, expanded, monkeypatch):
     from torchtune_amd import nf4_tensor
 
     monkeypatch.setattr(nf4_tensor, "BACKWARD_COPY", backward_copy)
+    monkeypatch.setattr(ops, "EXPANDED_WEIGHT_PATH", expanded)
     _check_layer_vs_oracle(M, N, K, r, False)
 
 
@@ -509,7 +511,7 @@ def test_few_output_tiles_slice_the_contraction(M, N, K):
     nbytes = lib.ttamd_nf4_gemm_workspace_bytes(M, N, K)
     assert nbytes > 0 and nbytes % (M * N * 4) == 0 and 2 <= nbytes // (M * N * 4) <= 16
     assert lib.ttamd_nf4_gemm_workspace_bytes(64, N, K) == 0  # the few-token kernel needs none
-    assert lib.ttamd_nf4_gemm_workspace_bytes(16384, 4096, 4096) == 0  # nor does a full grid
+    assert lib.ttamd_nf4_gemm_workspace_bytes(16384, 4096, 4096) == 2 * 4096 * 4096  # a full grid of many tokens: the expanded weight, no slices
     ref = ((x.float() @ D.T + bias.float() + 0.5 * (h.float() @ B.float().T)) * cs.float())
     for scal_t in (None, bst):
         y = ops.nf4_lora_linear_fwd(x, t.quantized_data, bs, N, h, B, 0.5, bias, block_scalers_t=scal_t, col_scale=cs)

@@ -417,16 +417,24 @@ def test_disable_adapter_and_adapter_state_dict():
 
 
 def test_gemm_workspace_query_is_a_host_function():
-    """``ttamd_nf4_gemm_workspace_bytes`` needs no GPU: it is 0 where the contraction is not sliced (the few-token kernel,
-    M <= 64; launches with more than 128 tiles of 128 x 256; two-slice launches of a short contraction) and otherwise
-    slices * M * n_out * 4 bytes with 2 <= slices <= 16 and at least four 64-wide k-steps per slice."""
+    """``ttamd_nf4_gemm_workspace_bytes`` needs no GPU: it is 0 where the launch uses no scratch memory (the few-token
+    kernel, M <= 64; launches with more than 128 tiles of 128 x 256 but fewer than 256 of 256 x 256 or fewer than 2048
+    tokens; two-slice launches of a short contraction), slices * M * n_out * 4 bytes with 2 <= slices <= 16 and at least
+    four 64-wide k-steps per slice where the contraction is sliced, and 2 * n_out * k bytes (the weight expanded once)
+    from 2048 tokens and 256 tiles of 256 x 256 up, which ``ttamd_nf4_gemm_expands_weight`` tells apart."""
     from torchtune_amd import _lib
 
     lib = _lib.load()
     q = lib.ttamd_nf4_gemm_workspace_bytes
+    e = lib.ttamd_nf4_gemm_expands_weight
     assert q(1, 4096, 4096) == 0 and q(64, 4096, 4096) == 0
-    assert q(8192, 4096, 4096) == 0 and q(16384, 1024, 4096) == 0
+    assert q(8192, 4096, 4096) == 2 * 4096 * 4096 and e(8192, 4096, 4096) == 1
+    assert q(16384, 1024, 4096) == 2 * 1024 * 4096 and e(16384, 1024, 4096) == 1
+    assert q(8192, 14336, 4096) == q(8192, 4096, 14336) == 2 * 4096 * 14336
+    assert q(8192, 1024, 4096) == 0 and e(8192, 1024, 4096) == 0  # 128 tiles of 256 x 256: the fused kernel's 128-row tiles
+    assert q(1536, 16384, 4096) == 0 and e(1536, 16384, 4096) == 0  # fewer than 2048 tokens
     assert q(2048, 2048, 2048) == 0  # 128 tiles, two slices of 16 k-steps: not worth the reduction
+    assert e(1, 4096, 4096) == 0 and e(128, 4096, 4096) == 0 and e(4096, 1024, 8192) == 0
     assert q(0, 4096, 4096) == 0 and q(128, 0, 4096) == 0
     for M, N, K, slices in [(128, 4096, 4096, 16), (512, 4096, 4096, 4), (1024, 4096, 4096, 2), (65, 256, 512, 2),
                             (300, 512, 1024, 4), (4096, 1024, 8192, 2)]:

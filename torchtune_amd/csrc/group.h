@@ -56,6 +56,15 @@ int run_gemm_rs(const void* X, const uint8_t* codes, const void* scal, int mode,
 size_t gemm_rs_workspace_bytes(int64_t M, int64_t Nout, int64_t Kc);
 int run_gemm_rs_group_dx(const GroupDx& d, const void* gh_cat, void* gx, hipStream_t s);
 
+// nf4_gemm_dense.hip: expand the weight once into scratch memory, then a plain bf16 GEMM (many tokens)
+bool dense_path_applies(int64_t M, int64_t Nout, int64_t Kc);
+size_t dense_workspace_bytes(int64_t M, int64_t Nout, int64_t Kc);
+int run_gemm_dense(const void* X, const uint8_t* codes, const void* scal, int mode, const void* lX, int ldlx, const void* lW,
+                   bool lw_row_major, int R, float lscale, const void* bias, const void* cscale, void* C, int64_t M, int64_t Nout,
+                   int64_t Kc, void* workspace, hipStream_t s);
+size_t dense_group_dx_workspace_bytes(const GroupDx& d);
+int run_gemm_dense_group_dx(const GroupDx& d, const void* gh_cat, void* gx, void* workspace, hipStream_t s);
+
 // nf4_small_m.hip: y[i] = x . D(W_i)^T (+ bias) + scale . h_i . lora_b[i]^T for a handful of tokens
 int small_m_limit();
 int run_small_m_group(const void* x, const GroupGemm& g, const void* h_cat, hipStream_t s);

@@ -156,3 +156,23 @@ extern "C" int ttamd_nf4_group_bwd_dx_bf16(const ttamd_lora_group_member* member
                "nf4_group_bwd_dx: member %d: needs the transposed copies (ttamd_nf4_transpose_for_backward), 16-byte aligned", i);
   return run_gemm_rs_group_dx(d.dx, gh_cat, gx, reinterpret_cast<hipStream_t>(stream));
 }
+
+extern "C" size_t ttamd_nf4_group_bwd_dx_workspace_bytes(const ttamd_lora_group_member* members, int n_members, int64_t M, int64_t K) {
+  Decoded d;
+  if (decode("nf4_group_bwd_dx_workspace_bytes", members, n_members, M, K, false, d) != TTAMD_OK) return 0;
+  return dense_group_dx_workspace_bytes(d.dx);
+}
+
+extern "C" int ttamd_nf4_group_bwd_dx_ws_bf16(const ttamd_lora_group_member* members, int n_members, const void* gh_cat, void* gx,
+                                              int64_t M, int64_t K, void* workspace, size_t workspace_bytes, void* stream) {
+  Decoded d;
+  if (int rc = decode("nf4_group_bwd_dx", members, n_members, M, K, false, d)) return rc;
+  const size_t need = dense_group_dx_workspace_bytes(d.dx);
+  if (need == 0 || workspace == nullptr || workspace_bytes < need)
+    return ttamd_nf4_group_bwd_dx_bf16(members, n_members, gh_cat, gx, M, K, stream);
+  TT_REQUIRE(gh_cat && gx && aligned16(gh_cat) && aligned16(gx), "nf4_group_bwd_dx: gh_cat and gx must be non-null and 16-byte aligned");
+  for (int i = 0; i < n_members; ++i)
+    TT_REQUIRE(d.dx.codes_t[i] && d.dx.scal_t[i] && aligned16(d.dx.codes_t[i]),
+               "nf4_group_bwd_dx: member %d: needs the transposed copies (ttamd_nf4_transpose_for_backward), 16-byte aligned", i);
+  return run_gemm_dense_group_dx(d.dx, gh_cat, gx, workspace, reinterpret_cast<hipStream_t>(stream));
+}

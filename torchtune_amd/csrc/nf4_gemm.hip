@@ -474,6 +474,10 @@ extern "C" size_t ttamd_nf4_gemm_workspace_bytes(int64_t M, int64_t n_out, int64
   return gemm_rs_workspace_bytes(M, n_out, k_contract);
 }
 
+extern "C" int ttamd_nf4_gemm_expands_weight(int64_t M, int64_t n_out, int64_t k_contract) {
+  return M > small_m_limit() && n_out > 0 && k_contract > 0 && dense_path_applies(M, n_out, k_contract) ? 1 : 0;
+}
+
 extern "C" int ttamd_nf4_lora_linear_fwd_ws_bf16(const void* x, const uint8_t* quantized_data, const void* block_scalers,
                                                  const void* block_scalers_t, const void* h, const void* lora_b, int rank,
                                                  float scale, const void* bias, const void* col_scale, void* y, int64_t M,

@@ -1,0 +1,509 @@
+// Many-token path of linear_nf4 / LoRALinear.forward (torchtune/modules/peft/lora.py:128-147; torchao's linear_nf4 =
+// F.linear(x, W.to(dtype))) and of its grad-input: the reference's own order of work.  The NF4 weight is expanded ONCE
+// per call into caller-provided scratch memory, then a plain bf16 GEMM runs on the matrix cores with the adapter, bias
+// and column scale in its epilogue.  The fused kernel (nf4_gemm_rs.hip) repeats the expansion once per 256-row tile of
+// the activations; from a few thousand tokens up that repetition costs more than one pass of the dequantise kernel.
+//
+//     C[M, Nout] = X[M, Kc] . Wd[Nout, Kc]^T  (+ bias, * cscale)  + sum_s (lscale . lX_s)[M, R_s] . lW_s[Nout, R_s]^T
+//
+// The contraction may be the concatenation of up to kGroupMax segments (grad-input of layers with a common input:
+// X_s = gy_s, Wd_s = W_s^T), each with its own activation tensor and adapter.
+//
+// The scratch copy `Wd` is written in the order the matrix cores consume it (v_mfma_f32_16x16x32_bf16): for every block
+// of 16 output columns T and every 32-wide k-step t one 1 KiB piece in which lane l of a wave finds, at byte 16 l, the
+// eight bf16 values Wd[16 T + l % 16][32 t + 8 (l / 16) .. + 7]:
+//
+//     tiled[T][t][lane][8]        T < Nout / 16, t < Kc / 32, lane < 64
+//
+// GEMM kernel: workgroup = 8 waves (two per SIMD), tile 256 x 256, k-step 32.  Both operands reach LDS by direct-to-LDS
+// loads (activations as whole 128-byte lines into a ring of three 64-wide entries, weights into a ring of four stages).
+// Wave (wm, wn) owns rows [128 wm, +128) x columns [64 wn, +64): 8 x 4 MFMA tiles, 128 accumulators per lane.  The two
+// waves of a SIMD run half a step apart: while one issues the 32 MFMAs of a step, the other requests loads and reads its
+// operands of the next step, and they swap at a workgroup barrier.  Measured on MI355X, the matrix pipe of a SIMD is
+// handed back and forth without the vector-memory instructions of a wave ever delaying its own MFMAs, which is what
+// limited the one-wave-per-SIMD form of this loop.  The 16 x 16 x 32 MFMA is used because this part is power-limited
+// under matrix load and that shape sustains 13 % more FLOP/s than 32 x 32 x 16 at the same power (2.04 against
+// 1.80 PFLOP/s for MFMA-only loops on random operands).
+#include <type_traits>
+
+#include "common.h"
+#include "group.h"
+#include "nf4_math.h"
+
+namespace ttamd {
+namespace {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  bf16x2_t v;
+  v.x = (__bf16)lo;
+  v.y = (__bf16)hi;
+  return __builtin_bit_cast(uint32_t, v);
+}
+
+#define TT_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
+
+__constant__ float kNF4Dense[16] = TT_NF4_TABLE;
+
+// ---------------------------------------------------------------------------------------------------------------------
+// Expansion into the tiled scratch copy.  A thread takes 32 consecutive contraction indices of one output column
+// (16 bytes of codes) and writes the four 16-byte operands that lanes (col % 16) + 16 g, g = 0..3, of that piece read.
+// Values are the bits ttamd_nf4_dequantize produces: nf4[code] * block scaler in fp32, rounded once to bf16.
+//   MODE 0: codes [Nout, Kc / 2], block scalers [Nout, Kc / 64]            (forward, natural layout)
+//   MODE 2: codes [Nout, Kc / 2], block scalers transposed [Kc / 64, Nout] (forward, when the backward copy exists)
+//   MODE 1: codes of W^T [Nout, Kc / 2] with per-element scalers [Nout / 64, Kc] (grad-input: Nout = K, Kc = N)
+// A workgroup of 256 threads covers 16 columns (one T) x 16 k-steps per iteration of its loop over the contraction.
+// ---------------------------------------------------------------------------------------------------------------------
+template <int MODE>
+__global__ __launch_bounds__(256) void nf4_expand_tiled_kernel(const uint8_t* __restrict__ codes, const float* __restrict__ scal,
+                                                               int Nout, int Kc, int nk_total, int t_off,
+                                                               char* __restrict__ tiled) {
+  __shared__ float2 lut[256];
+  const int tid = threadIdx.x;
+  lut[tid] = make_float2(round_to_bf16(kNF4Dense[tid >> 4]), round_to_bf16(kNF4Dense[tid & 15]));
+  __syncthreads();
+  const int T = blockIdx.x;
+  const int r = tid & 15;        // column inside the block
+  const int col = 16 * T + r;
+  const int nk = Kc >> 5;
+  const int chunks = (nk + 15) >> 4;
+  const int per = (chunks + gridDim.y - 1) / gridDim.y;
+  const int c0 = blockIdx.y * per, c1 = c0 + per < chunks ? c0 + per : chunks;
+  for (int c = c0; c < c1; ++c) {
+    const int t = 16 * c + (tid >> 4);
+    if (t >= nk) break;
+    const u32x4_t cd = *reinterpret_cast<const u32x4_t*>(codes + (int64_t)col * (Kc >> 1) + 16 * t);
+    float sc[32];
+    if (MODE == 1) {
+      const float* sp = scal + (int64_t)(col >> 6) * Kc + 32 * t;
+#pragma unroll
+      for (int q = 0; q < 8; ++q) {
+        const f32x4_t v = *reinterpret_cast<const f32x4_t*>(sp + 4 * q);
+        sc[4 * q] = v.x; sc[4 * q + 1] = v.y; sc[4 * q + 2] = v.z; sc[4 * q + 3] = v.w;
+      }
+    } else {
+      const float s1 = MODE == 0 ? scal[(int64_t)col * (Kc >> 6) + (t >> 1)] : scal[(int64_t)(t >> 1) * Nout + col];
+#pragma unroll
+      for (int q = 0; q < 32; ++q) sc[q] = s1;
+    }
+    char* piece = tiled + ((int64_t)T * nk_total + t_off + t) * 1024;
+#pragma unroll
+    for (int g4 = 0; g4 < 4; ++g4) {
+      const uint32_t w = cd[g4];
+      u32x4_t o;
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        const float2 pr = lut[(w >> (8 * b)) & 0xffu];
+        o[b] = pack_bf16x2(pr.x * sc[8 * g4 + 2 * b], pr.y * sc[8 * g4 + 2 * b + 1]);
+      }
+      *reinterpret_cast<u32x4_t*>(piece + (16 * g4 + r) * 16) = o;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
+struct DenseSeg {
+  const uint16_t* X;   // [M, Kc_s] bf16 activations of the segment
+  const uint16_t* lX;  // adapter activations (rows ldlx apart) or null
+  const uint16_t* lW;  // adapter weights: [Nout, R] (lw_row_major) or [R, Nout]
+  int Kc, R;
+};
+struct DenseArgs {
+  DenseSeg seg[kGroupMax];
+  int nseg;
+  const char* Wt;          // tiled weight, all segments side by side along the contraction
+  const uint16_t* bias;    // [Nout] bf16 or null
+  const uint16_t* cscale;  // [Nout] bf16 or null: C = (acc + bias) * cscale per column
+  uint16_t* C;             // [M, Nout] bf16
+  int M, Nout, Kc;         // Kc: total contraction
+  int lw_row_major, ldlx;
+  float lscale;
+  int tiles_m, tiles_n;
+};
+
+constexpr int kAEntry = 32768;  // activation ring: 3 entries of 256 rows x 64 k
+constexpr int kWBase = 3 * kAEntry;
+constexpr int kWStage = 16384;  // weight ring: 4 stages of 256 columns x 32 k
+constexpr int kLdsDense = kWBase + 4 * kWStage;
+
+__global__ __launch_bounds__(512) void nf4_gemm_dense_kernel(const DenseArgs g) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  constexpr int MT = 8, NT = 4;  // 16 x 16 MFMA tiles per wave
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wv >> 2, wn = wv & 3;
+  const int l15 = lane & 15, g4 = lane >> 4;
+
+  int tile_m, tile_n;
+  {
+    // workgroup ids are dealt round-robin to the 8 XCDs (one L2 each): every XCD gets a band of m-tiles and walks it
+    // column by column, so the workgroups resident on an XCD share each weight tile through its L2
+    const int id = blockIdx.x;
+    if ((g.tiles_m & 7) == 0) {
+      const int xcd = id & 7, slot = id >> 3, band = g.tiles_m >> 3;
+      tile_m = xcd * band + slot % band;
+      tile_n = slot / band;
+    } else {
+      tile_m = id / g.tiles_n;
+      tile_n = id % g.tiles_n;
+    }
+  }
+  const int m0 = tile_m * 256, n0 = tile_n * 256;
+  const int nk = g.Kc >> 5;        // k-steps of 32
+  const int nk2 = g.Kc >> 6;       // activation entries (pairs of k-steps)
+
+  // ---- loads.  Activations: every two k-steps, four instructions per wave (rows [32 wv, +32) of the tile, 8 rows of 128
+  //      bytes each: whole cache lines); chunk c of row r is stored in slot c ^ ((r >> 1) & 7).  Weights: every k-step the
+  //      1 KiB pieces of column blocks 2 wv and 2 wv + 1.
+  int a_row[4], a_chunk[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int trow = wv * 32 + 8 * i + (lane >> 3);
+    a_chunk[i] = ((lane & 7) ^ ((trow >> 1) & 7)) * 16;
+    const int row = m0 + trow;
+    a_row[i] = row < g.M ? row : g.M - 1;
+  }
+  uint32_t a_off[4];
+  int seg = 0, seg_begin = 0, seg_end = g.seg[0].Kc >> 6;  // entries [seg_begin, seg_end) belong to segment seg
+  const char* a_base = reinterpret_cast<const char*>(g.seg[0].X);
+  auto set_segment = [&]() {
+    const uint32_t pitch = (uint32_t)g.seg[seg].Kc * 2u;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) a_off[i] = (uint32_t)a_row[i] * pitch + (uint32_t)a_chunk[i];
+  };
+  set_segment();
+  const int nblocks = g.Nout >> 4;
+  int T0 = (n0 >> 4) + 2 * wv, T1 = T0 + 1;
+  T0 = T0 < nblocks ? T0 : nblocks - 1;
+  T1 = T1 < nblocks ? T1 : nblocks - 1;
+  const char* wsrc0 = g.Wt + (int64_t)T0 * ((int64_t)nk * 1024);
+  const char* wsrc1 = g.Wt + (int64_t)T1 * ((int64_t)nk * 1024);
+  const uint32_t lane16 = (uint32_t)lane * 16u;
+
+  auto dma16 = [&](uint32_t voff, const char* base, uint32_t lds, int imm) {
+    asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 ::"v"(voff), "s"(base), "s"(lds), "n"(imm) : "memory", "m0", "scc");
+  };
+  const uint32_t lds0 = (uint32_t)(uintptr_t)TT_LDS_PTR(smem);
+  auto issue_w = [&](int t, int stage) {
+    const int tk = t < nk ? t : nk - 1;
+    const uint32_t sw = lds0 + kWBase + stage * kWStage + wv * 2048;
+    dma16(lane16, wsrc0 + (int64_t)tk * 1024, sw, 0);
+    dma16(lane16, wsrc1 + (int64_t)tk * 1024, sw, 1024);
+  };
+  // entries are requested in increasing order (past the end: the last one again), so the segment only moves forward
+  auto issue_a = [&](int T2, int entry) {
+    const int tk = T2 < nk2 ? T2 : nk2 - 1;
+    while (tk >= seg_end) {
+      ++seg;
+      seg_begin = seg_end;
+      seg_end += g.seg[seg].Kc >> 6;
+      a_base = reinterpret_cast<const char*>(g.seg[seg].X);
+      set_segment();
+    }
+    const char* xb = a_base + ((int64_t)(tk - seg_begin) << 7);  // + 64 elements * 2 bytes per entry
+    const uint32_t sa = lds0 + entry * kAEntry + wv * 4096;
+    dma16(a_off[0], xb, sa, 0);
+    dma16(a_off[1], xb, sa, 1024);
+    dma16(a_off[2], xb, sa, 2048);
+    dma16(a_off[3], xb, sa, 3072);
+  };
+
+  // operand read offsets: activation tile 0 of this wave, half hf of the entry: row 128 wm + l15, chunk 4 hf + g4
+  int xo[2];
+#pragma unroll
+  for (int hf = 0; hf < 2; ++hf) xo[hf] = (128 * wm + l15) * 128 + (((4 * hf + g4) ^ ((l15 >> 1) & 7)) << 4);
+  const int wo = kWBase + (4 * wn) * 1024 + lane * 16;  // weight block 4 wn + j at + j * 1024
+
+  f32x4_t acc[NT][MT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j)
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) acc[j][i][v] = 0.f;
+
+  bf16x8_t xf[MT], wf[NT];
+  auto read_step = [&](int entry, int hf, int wstage) {
+    const char* sw = smem + wstage * kWStage;
+    const char* sa = smem + entry * kAEntry + xo[hf];
+#pragma unroll
+    for (int j = 0; j < NT; ++j) wf[j] = *reinterpret_cast<const bf16x8_t*>(sw + wo + j * 1024);
+#pragma unroll
+    for (int i = 0; i < MT; ++i) xf[i] = *reinterpret_cast<const bf16x8_t*>(sa + i * 2048);
+  };
+  auto compute = [&]() {
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int i = 0; i < MT; ++i) acc[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[j], xf[i], acc[j][i], 0, 0, 0);
+    __builtin_amdgcn_s_setprio(0);
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_barrier" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  // ---- pipeline.  Every wave alternates memory part M(t) / barrier / compute part C(t) / barrier; the waves with
+  //      wm = 1 pass one extra barrier first, so that between two barriers one wave of each SIMD computes while the other
+  //      is in its memory part.  Numbering the barriers from the one that ends the prologue, the waves with wm = 0 read
+  //      step t between barriers 2t and 2t+1, the others between 2t+1 and 2t+2.  Hence:
+  //        * what M(t) requests may overwrite the stage of step t-1 (last read before barrier 2t): W(t+3) into a ring of
+  //          four stages, and for even t activation entry t/2 + 2 into a ring of three;
+  //        * at the end of M(t) a wave's own loads of step t+1 must have landed (the other waves read them after the
+  //          next barrier).  Loads of a wave complete in order.  Its program order: prologue A(0) x4, W(0) x2, W(1) x2,
+  //          A(1) x4, W(2) x2; M(t): W(t+3) x2, then for even t A(t/2 + 2) x4.  W(t+1) came from M(t-2) and the
+  //          activation entry of step t+1 is older; newer than W(t+1) are 4 + 2 + 6 = 12 loads (t even), 0 + 6 + 2 = 8 (t odd).
+  //      The operand reads of M(t) are awaited by the compiler's own counts before the first MFMA that needs them, after
+  //      the barrier: the other wave's MFMAs are still draining then.
+  issue_a(0, 0);
+  issue_w(0, 0);
+  issue_w(1, 1);
+  issue_a(1, 1);
+  issue_w(2, 2);
+  asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");  // A(0), W(0) landed everywhere
+  if (wm == 1) asm volatile("s_barrier" ::: "memory");
+  int e0 = 0, ws = 0;  // activation entry of the current pair of steps, weight stage of the current step
+  for (int t = 0; t < nk; t += 2) {
+    const int e1 = e0 == 2 ? 0 : e0 + 1, e2 = e1 == 2 ? 0 : e1 + 1;
+    // ---- even step t
+    issue_w(t + 3, (ws + 3) & 3);
+    issue_a((t >> 1) + 2, e2);
+    read_step(e0, 0, ws);
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_waitcnt vmcnt(12)\n\ts_barrier" ::: "memory");
+    compute();
+    // ---- odd step t + 1
+    issue_w(t + 4, ws);
+    read_step(e0, 1, (ws + 1) & 3);
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");
+    compute();
+    e0 = e1;
+    ws = (ws + 2) & 3;
+  }
+  if (wm == 0) asm volatile("s_barrier" ::: "memory");
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the clamped requests of the last steps
+
+  // ---- adapters: one MFMA step per 32 ranks and segment, operands straight from global memory.  Lane (l15, g4) holds
+  //      ranks rc + 8 g4 .. + 7 of weight column / activation row l15 of its tile; ranks beyond R are zero.
+  for (int sidx = 0; sidx < g.nseg; ++sidx) {
+    const int R = g.seg[sidx].R;
+    if (R <= 0) continue;
+    const uint16_t* lX = g.seg[sidx].lX;
+    const uint16_t* lW = g.seg[sidx].lW;
+    for (int rc = 0; rc < R; rc += 32) {
+      const int r0 = rc + 8 * g4;
+      const bool in = r0 < R;  // R % 8 == 0: a lane's 8 ranks are all in or all out
+      bf16x8_t wfr[NT], xfr[MT];
+#pragma unroll
+      for (int j = 0; j < NT; ++j) {
+        int col = n0 + wn * 64 + 16 * j + l15;
+        col = col < g.Nout ? col : g.Nout - 1;
+        u32x4_t raw = {0, 0, 0, 0};
+        if (in) {
+          if (g.lw_row_major) {
+            raw = *reinterpret_cast<const u32x4_t*>(lW + (int64_t)col * R + r0);
+          } else {
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+              const uint32_t lo = lW[(int64_t)(r0 + 2 * d) * g.Nout + col];
+              const uint32_t hi = lW[(int64_t)(r0 + 2 * d + 1) * g.Nout + col];
+              raw[d] = lo | (hi << 16);
+            }
+          }
+        }
+        wfr[j] = __builtin_bit_cast(bf16x8_t, raw);
+      }
+#pragma unroll
+      for (int i = 0; i < MT; ++i) {
+        int row = m0 + 128 * wm + 16 * i + l15;
+        row = row < g.M ? row : g.M - 1;
+        u32x4_t raw = {0, 0, 0, 0};
+        if (in) raw = *reinterpret_cast<const u32x4_t*>(lX + (int64_t)row * g.ldlx + r0);
+        if (g.lscale != 1.0f) {
+#pragma unroll
+          for (int d = 0; d < 4; ++d)
+            raw[d] = pack_bf16x2(bits_f32(raw[d] << 16) * g.lscale, bits_f32(raw[d] & 0xffff0000u) * g.lscale);
+        }
+        xfr[i] = __builtin_bit_cast(bf16x8_t, raw);
+      }
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int i = 0; i < MT; ++i) acc[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wfr[j], xfr[i], acc[j][i], 0, 0, 0);
+    }
+  }
+
+  // ---- epilogue: acc[j][i][v] = C[m][n], m = m0 + 128 wm + 16 i + l15, n = n0 + 64 wn + 16 j + 4 g4 + v.  Each wave
+  //      transposes its 128 x 64 band through LDS (the rings are free now) and writes whole 128-byte row segments;
+  //      16-byte chunk c of row r sits in slot c ^ (r & 7).
+  __syncthreads();
+  if (n0 + wn * 64 >= g.Nout) return;  // the whole band of this wave lies outside (no barrier follows)
+  {
+    char* band = smem + wv * 16384;  // 128 rows x 128 bytes
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+      float b4[4] = {0.f, 0.f, 0.f, 0.f};
+      if (g.bias) {
+        const u32x2_t bb = *reinterpret_cast<const u32x2_t*>(g.bias + n0 + wn * 64 + 16 * j + 4 * g4);
+        b4[0] = bits_f32(bb.x << 16); b4[1] = bits_f32(bb.x & 0xffff0000u);
+        b4[2] = bits_f32(bb.y << 16); b4[3] = bits_f32(bb.y & 0xffff0000u);
+      }
+      float c4[4] = {1.f, 1.f, 1.f, 1.f};
+      if (g.cscale) {
+        const u32x2_t cc = *reinterpret_cast<const u32x2_t*>(g.cscale + n0 + wn * 64 + 16 * j + 4 * g4);
+        c4[0] = bits_f32(cc.x << 16); c4[1] = bits_f32(cc.x & 0xffff0000u);
+        c4[2] = bits_f32(cc.y << 16); c4[3] = bits_f32(cc.y & 0xffff0000u);
+      }
+#pragma unroll
+      for (int i = 0; i < MT; ++i) {
+        const int r = 16 * i + l15;
+        u32x2_t o;
+        o.x = pack_bf16x2((acc[j][i][0] + b4[0]) * c4[0], (acc[j][i][1] + b4[1]) * c4[1]);
+        o.y = pack_bf16x2((acc[j][i][2] + b4[2]) * c4[2], (acc[j][i][3] + b4[3]) * c4[3]);
+        *reinterpret_cast<u32x2_t*>(band + r * 128 + (((2 * j + (g4 >> 1)) ^ (r & 7)) << 4) + 8 * (g4 & 1)) = o;
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const int c = lane & 7;
+    uint16_t* crow = g.C + n0 + wn * 64 + 8 * c;
+    const int mrow0 = m0 + 128 * wm;
+#pragma unroll 8
+    for (int t = 0; t < 16; ++t) {
+      const int r = 8 * t + (lane >> 3);
+      const u32x4_t v = *reinterpret_cast<const u32x4_t*>(band + r * 128 + ((c ^ (r & 7)) << 4));
+      if (mrow0 + r < g.M) *reinterpret_cast<u32x4_t*>(crow + (int64_t)(mrow0 + r) * g.Nout) = v;
+    }
+  }
+#endif
+}
+
+int launch_expand(int mode, const uint8_t* codes, const float* scal, int64_t Nout, int64_t Kc, int64_t nk_total, int64_t t_off,
+                  char* tiled, hipStream_t s) {
+  // one block of 16 columns per blockIdx.x; the contraction is cut along blockIdx.y so that about 2048 workgroups exist
+  const int64_t chunks = ((Kc >> 5) + 15) / 16;
+  int64_t ysplit = (2048 + (Nout >> 4) - 1) / (Nout >> 4);
+  ysplit = ysplit < 1 ? 1 : (ysplit > chunks ? chunks : ysplit);
+  const dim3 grid((unsigned)(Nout >> 4), (unsigned)ysplit), block(256);
+  if (mode == 1)
+    nf4_expand_tiled_kernel<1><<<grid, block, 0, s>>>(codes, scal, (int)Nout, (int)Kc, (int)nk_total, (int)t_off, tiled);
+  else if (mode == 2)
+    nf4_expand_tiled_kernel<2><<<grid, block, 0, s>>>(codes, scal, (int)Nout, (int)Kc, (int)nk_total, (int)t_off, tiled);
+  else
+    nf4_expand_tiled_kernel<0><<<grid, block, 0, s>>>(codes, scal, (int)Nout, (int)Kc, (int)nk_total, (int)t_off, tiled);
+  return check_launch("nf4_expand_tiled");
+}
+
+int launch_dense(DenseArgs& g, hipStream_t s) {
+  g.tiles_m = (g.M + 255) / 256;
+  g.tiles_n = (g.Nout + 255) / 256;
+  // the LDS limit is a per-device attribute of the function: set it for the current device once (a race only repeats
+  // the call)
+  static bool attr_set[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = -1;
+  if (dev < 0 || !attr_set[dev]) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&nf4_gemm_dense_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLdsDense);
+    if (e != hipSuccess) return fail(TTAMD_ELAUNCH, "nf4_gemm_dense: cannot reserve %d bytes of LDS: %s", kLdsDense, hipGetErrorString(e));
+    if (dev >= 0) attr_set[dev] = true;
+  }
+  nf4_gemm_dense_kernel<<<dim3((unsigned)(g.tiles_m * g.tiles_n)), dim3(512), kLdsDense, s>>>(g);
+  return check_launch("nf4_gemm_dense");
+}
+
+}  // namespace
+
+// Fewest tokens from which the expand-once path is taken (below, the fused kernel's repeated expansion is cheaper than
+// one pass of the expansion kernel plus the traffic of the scratch copy).
+constexpr int64_t kDenseMinRows = 2048;
+
+bool dense_path_applies(int64_t M, int64_t Nout, int64_t Kc) {
+  if (M < kDenseMinRows || Nout % 64 != 0 || Kc % 64 != 0) return false;
+  if (((M + 255) / 256) * ((Nout + 255) / 256) < 256) return false;  // fewer tiles than CUs: the fused kernel has 128-row tiles
+  // per-lane byte offsets inside the kernel are 32-bit
+  return M * Kc * 2 < (int64_t(1) << 32) && Kc * 2 * 256 < (int64_t(1) << 32);
+}
+
+size_t dense_workspace_bytes(int64_t M, int64_t Nout, int64_t Kc) {
+  return dense_path_applies(M, Nout, Kc) ? (size_t)Nout * (size_t)Kc * 2 : 0;
+}
+
+// One segment: the ordinary forward (mode 0 / 2) or grad-input (mode 1) of a layer.  Arguments as run_gemm_rs.
+int run_gemm_dense(const void* X, const uint8_t* codes, const void* scal, int mode, const void* lX, int ldlx, const void* lW,
+                   bool lw_row_major, int R, float lscale, const void* bias, const void* cscale, void* C, int64_t M, int64_t Nout,
+                   int64_t Kc, void* workspace, hipStream_t s) {
+  TT_REQUIRE(dense_path_applies(M, Nout, Kc), "nf4_gemm_dense: shape not served (M=%lld Nout=%lld Kc=%lld)", (long long)M,
+             (long long)Nout, (long long)Kc);
+  TT_REQUIRE(aligned16(workspace) && aligned16(X) && aligned16(codes) && aligned16(scal), "nf4_gemm_dense: pointers must be 16-byte aligned");
+  if (int rc = launch_expand(mode, codes, reinterpret_cast<const float*>(scal), Nout, Kc, Kc >> 5, 0, reinterpret_cast<char*>(workspace), s))
+    return rc;
+  DenseArgs g = {};
+  g.nseg = 1;
+  g.seg[0].X = reinterpret_cast<const uint16_t*>(X);
+  g.seg[0].lX = reinterpret_cast<const uint16_t*>(lX);
+  g.seg[0].lW = reinterpret_cast<const uint16_t*>(lW);
+  g.seg[0].Kc = (int)Kc;
+  g.seg[0].R = R;
+  g.Wt = reinterpret_cast<const char*>(workspace);
+  g.bias = reinterpret_cast<const uint16_t*>(bias);
+  g.cscale = reinterpret_cast<const uint16_t*>(cscale);
+  g.C = reinterpret_cast<uint16_t*>(C);
+  g.M = (int)M; g.Nout = (int)Nout; g.Kc = (int)Kc;
+  g.lw_row_major = lw_row_major ? 1 : 0;
+  g.ldlx = ldlx;
+  g.lscale = lscale;
+  return launch_dense(g, s);
+}
+
+// Grad-input of a group of layers with a common input over the concatenated contraction (see run_gemm_rs_group_dx).
+size_t dense_group_dx_workspace_bytes(const GroupDx& d) {
+  int64_t n_total = 0;
+  for (int i = 0; i < d.n; ++i) {
+    if (d.N[i] % 64 != 0) return 0;
+    n_total += d.N[i];
+    if (d.M * d.N[i] * 2 >= (int64_t(1) << 32)) return 0;
+  }
+  if (d.M < kDenseMinRows || d.K % 64 != 0 || ((d.M + 255) / 256) * ((d.K + 255) / 256) < 256) return 0;
+  return (size_t)d.K * (size_t)n_total * 2;
+}
+
+int run_gemm_dense_group_dx(const GroupDx& d, const void* gh_cat, void* gx, void* workspace, hipStream_t s) {
+  TT_REQUIRE(d.n >= 1 && d.n <= kGroupMax && dense_group_dx_workspace_bytes(d) > 0, "nf4_group_dx (dense): shape not served");
+  TT_REQUIRE(aligned16(workspace), "nf4_group_dx (dense): workspace must be 16-byte aligned");
+  int64_t n_total = 0;
+  for (int i = 0; i < d.n; ++i) n_total += d.N[i];
+  DenseArgs g = {};
+  g.nseg = d.n;
+  int64_t t_off = 0;
+  for (int i = 0; i < d.n; ++i) {
+    TT_REQUIRE(aligned16(d.gy[i]) && aligned16(d.codes_t[i]) && aligned16(d.scal_t[i]), "nf4_group_dx (dense): pointers must be 16-byte aligned");
+    if (int rc = launch_expand(1, d.codes_t[i], d.scal_t[i], d.K, d.N[i], n_total >> 5, t_off, reinterpret_cast<char*>(workspace), s)) return rc;
+    t_off += d.N[i] >> 5;
+    g.seg[i].X = d.gy[i];
+    g.seg[i].lX = d.rank[i] > 0 ? reinterpret_cast<const uint16_t*>(gh_cat) + d.r_off[i] : nullptr;
+    g.seg[i].lW = d.lora_a[i];
+    g.seg[i].Kc = (int)d.N[i];
+    g.seg[i].R = d.rank[i];
+  }
+  g.Wt = reinterpret_cast<const char*>(workspace);
+  g.C = reinterpret_cast<uint16_t*>(gx);
+  g.M = (int)d.M; g.Nout = (int)d.K; g.Kc = (int)n_total;
+  g.lw_row_major = 0;
+  g.ldlx = d.r_off[d.n];
+  g.lscale = 1.0f;
+  return launch_dense(g, s);
+}
+
+}  // namespace ttamd

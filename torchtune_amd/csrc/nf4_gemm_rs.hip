@@ -640,10 +640,12 @@ int choose_splits(int64_t M, int64_t Nout, int64_t Kc) {
 
 }  // namespace
 
-// Bytes of workspace with which run_gemm_rs cuts the contraction of a small launch into slices (0: it would not).
+// Bytes of workspace run_gemm_rs can use: slices of the contraction for a small launch, or the expanded copy of the
+// weight for a launch of many tokens (nf4_gemm_dense.hip); the two cases exclude each other.  0: it would use none.
 size_t gemm_rs_workspace_bytes(int64_t M, int64_t Nout, int64_t Kc) {
   const int sp = choose_splits(M, Nout, Kc);
-  return sp > 1 ? (size_t)sp * (size_t)M * (size_t)Nout * sizeof(float) : 0;
+  if (sp > 1) return (size_t)sp * (size_t)M * (size_t)Nout * sizeof(float);
+  return dense_workspace_bytes(M, Nout, Kc);
 }
 
 // Entry used by the C-ABI wrappers.  `workspace` may be null: then small launches are not sliced.  The rows of the
@@ -666,6 +668,9 @@ int run_gemm_rs(const void* X, const uint8_t* codes, const void* scal, int mode,
     }
     return TTAMD_OK;
   }
+  // many tokens and room for the expanded weight: expand once, then the plain bf16 GEMM
+  if (workspace != nullptr && dense_path_applies(M, Nout, Kc) && workspace_bytes >= dense_workspace_bytes(M, Nout, Kc))
+    return run_gemm_dense(X, codes, scal, mode, lX, ldlx, lW, lw_row_major, R, lscale, bias, cscale, C, M, Nout, Kc, workspace, s);
   RsArgs g;
   g.X = reinterpret_cast<const uint16_t*>(X);
   g.codes = codes;

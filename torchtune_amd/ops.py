@@ -212,10 +212,16 @@ def lora_hidden(x: torch.Tensor, lora_a: torch.Tensor) -> torch.Tensor:
     return h
 
 
+# Many tokens: let the library expand the NF4 weight once per call into scratch memory (2 bytes per weight element,
+# freed after the call) and run its plain bf16 GEMM on it.  False keeps the fused kernel, which needs no scratch.
+EXPANDED_WEIGHT_PATH = True
+
+
 def _gemm_workspace(lib, M: int, n_out: int, k_contract: int, device):
-    """fp32 workspace with which the library slices the contraction of a launch of few output tiles (None: not needed)."""
+    """Scratch memory for one NF4 GEMM: fp32 slices of the contraction for a launch of few output tiles, or room for the
+    expanded weight of a many-token launch (None: not needed, or the expanded path is switched off)."""
     nbytes = int(lib.ttamd_nf4_gemm_workspace_bytes(M, n_out, k_contract))
-    if nbytes == 0:
+    if nbytes == 0 or (not EXPANDED_WEIGHT_PATH and lib.ttamd_nf4_gemm_expands_weight(M, n_out, k_contract)):
         return None, 0
     return torch.empty(nbytes // 4, dtype=torch.float32, device=device), nbytes
 
@@ -407,8 +413,10 @@ def lora_group_fwd(x: torch.Tensor, members: Sequence[GroupMember]):
     r_total = sum(int(e.rank) for e in arr)
     h_cat = torch.empty(M, r_total, dtype=torch.bfloat16, device=dev)
     lib = _lib.load()
-    ws = _workspace(max(lib.ttamd_lora_group_hidden_workspace_bytes(arr, n, M, K), lib.ttamd_lora_group_fwd_workspace_bytes(arr, n, M, K)),
-                    dev)
+    fwd_bytes = lib.ttamd_lora_group_fwd_workspace_bytes(arr, n, M, K)
+    if not EXPANDED_WEIGHT_PATH and any(lib.ttamd_nf4_gemm_expands_weight(M, m.N, K) for m in members):
+        fwd_bytes = 0  # less than the library asks for: it keeps the fused kernel
+    ws = _workspace(max(lib.ttamd_lora_group_hidden_workspace_bytes(arr, n, M, K), fwd_bytes), dev)
     with torch.cuda.device(dev):
         rc = lib.ttamd_lora_group_hidden_bf16(x.data_ptr(), arr, n, h_cat.data_ptr(), M, K, ws.data_ptr(), ws.numel(), _stream(x))
         _lib.check(rc, "lora_group_hidden")
@@ -450,9 +458,12 @@ def lora_group_bwd(x: torch.Tensor, h_cat: torch.Tensor, members: Sequence[Group
         _lib.check(rc, "lora_group_bwd")
         if want_gx:
             events = _gemm_timer("bwd_group", M, [m.N for m in members], K, [int(e.rank) for e in arr]) if _gemm_timer is not None else None
+            dx_bytes = int(lib.ttamd_nf4_group_bwd_dx_workspace_bytes(arr, n, M, K)) if EXPANDED_WEIGHT_PATH else 0
+            dx_ws = torch.empty(dx_bytes // 4, dtype=torch.float32, device=dev) if dx_bytes else None
             if events:
                 events[0].record()
-            rc = lib.ttamd_nf4_group_bwd_dx_bf16(arr, n, gh_cat.data_ptr(), gx.data_ptr(), M, K, _stream(x))
+            rc = lib.ttamd_nf4_group_bwd_dx_ws_bf16(arr, n, gh_cat.data_ptr(), gx.data_ptr(), M, K,
+                                                    dx_ws.data_ptr() if dx_ws is not None else None, dx_bytes, _stream(x))
             if events:
                 events[1].record()
             _lib.check(rc, "nf4_group_bwd_dx")
