@@ -466,6 +466,9 @@ def main() -> int:
     ap.add_argument("--no-group", action="store_true",
                     help="one call per projection, as the reference's modules make them, instead of the group kernels for the "
                          "projections that share an input (q/k/v, gate/up): for A/B timing")
+    ap.add_argument("--no-expanded-weight", action="store_true",
+                    help="keep the fused NF4 GEMM (expansion repeated per tile, no scratch memory) also for many tokens, "
+                         "instead of expanding the weight once per call and running the plain bf16 GEMM")
     ap.add_argument("--calibration-copy-mib", type=int, default=0,
                     help="before the steps, run one elementwise kernel that reads and writes this many MiB: the known-size "
                          "dispatch that FETCH_SIZE / WRITE_SIZE counter runs are scaled by")
@@ -483,6 +486,7 @@ def main() -> int:
 
     harness.SDPA_BACKEND = args.sdpa
     harness.GROUP_SHARED_INPUT = not args.no_group
+    ops.EXPANDED_WEIGHT_PATH = not args.no_expanded_weight
 
     shape_name, rank, alpha, batch, seq, ac = WORKLOADS[args.workload]
     qat = args.workload.endswith("_qat")

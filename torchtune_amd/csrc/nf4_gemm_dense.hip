@@ -131,6 +131,7 @@ constexpr int kWBase = 3 * kAEntry;
 constexpr int kWStage = 16384;  // weight ring: 4 stages of 256 columns x 32 k
 constexpr int kLdsDense = kWBase + 4 * kWStage;
 
+template <bool LW_ROW_MAJOR>
 __global__ __launch_bounds__(512) void nf4_gemm_dense_kernel(const DenseArgs g) {
 #if defined(__HIP_DEVICE_COMPILE__)
   constexpr int MT = 8, NT = 4;  // 16 x 16 MFMA tiles per wave
@@ -300,29 +301,42 @@ __global__ __launch_bounds__(512) void nf4_gemm_dense_kernel(const DenseArgs g) 
     if (R <= 0) continue;
     const uint16_t* lX = g.seg[sidx].lX;
     const uint16_t* lW = g.seg[sidx].lW;
+    int pitch = 0;  // bytes per column of the staged adapter weights
+    if constexpr (!LW_ROW_MAJOR) {
+      // lW is [R, Nout]: a lane needs 8 ranks of one column, 8 elements Nout apart.  The workgroup copies the 256
+      // columns of its tile into LDS column by column (the rings are free after the loop), 16 bytes of a rank row per
+      // thread, and every lane then reads its operand as one 16-byte piece.
+      pitch = (R + 8) * 2;
+      __syncthreads();
+      for (int idx = tid; idx < R * 32; idx += 512) {
+        const int r = idx >> 5, c8 = (idx & 31) * 8;
+        u32x4_t raw = {0, 0, 0, 0};
+        if (n0 + c8 < g.Nout) raw = *reinterpret_cast<const u32x4_t*>(lW + (int64_t)r * g.Nout + n0 + c8);
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          *reinterpret_cast<uint16_t*>(smem + (c8 + e) * pitch + 2 * r) = (uint16_t)(raw[e >> 1] >> (16 * (e & 1)));
+      }
+      __syncthreads();
+    }
     for (int rc = 0; rc < R; rc += 32) {
       const int r0 = rc + 8 * g4;
       const bool in = r0 < R;  // R % 8 == 0: a lane's 8 ranks are all in or all out
       bf16x8_t wfr[NT], xfr[MT];
 #pragma unroll
       for (int j = 0; j < NT; ++j) {
-        int col = n0 + wn * 64 + 16 * j + l15;
-        col = col < g.Nout ? col : g.Nout - 1;
         u32x4_t raw = {0, 0, 0, 0};
         if (in) {
-          if (g.lw_row_major) {
+          if constexpr (LW_ROW_MAJOR) {
+            int col = n0 + wn * 64 + 16 * j + l15;
+            col = col < g.Nout ? col : g.Nout - 1;
             raw = *reinterpret_cast<const u32x4_t*>(lW + (int64_t)col * R + r0);
           } else {
-#pragma unroll
-            for (int d = 0; d < 4; ++d) {
-              const uint32_t lo = lW[(int64_t)(r0 + 2 * d) * g.Nout + col];
-              const uint32_t hi = lW[(int64_t)(r0 + 2 * d + 1) * g.Nout + col];
-              raw[d] = lo | (hi << 16);
-            }
+            raw = *reinterpret_cast<const u32x4_t*>(smem + (wn * 64 + 16 * j + l15) * pitch + 2 * r0);
           }
         }
         wfr[j] = __builtin_bit_cast(bf16x8_t, raw);
       }
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int i = 0; i < MT; ++i) {
         int row = m0 + 128 * wm + 16 * i + l15;
@@ -414,12 +428,17 @@ int launch_dense(DenseArgs& g, hipStream_t s) {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = -1;
   if (dev < 0 || !attr_set[dev]) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&nf4_gemm_dense_kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLdsDense);
-    if (e != hipSuccess) return fail(TTAMD_ELAUNCH, "nf4_gemm_dense: cannot reserve %d bytes of LDS: %s", kLdsDense, hipGetErrorString(e));
+    for (const void* fn : {reinterpret_cast<const void*>(&nf4_gemm_dense_kernel<true>), reinterpret_cast<const void*>(&nf4_gemm_dense_kernel<false>)}) {
+      hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsDense);
+      if (e != hipSuccess) return fail(TTAMD_ELAUNCH, "nf4_gemm_dense: cannot reserve %d bytes of LDS: %s", kLdsDense, hipGetErrorString(e));
+    }
     if (dev >= 0) attr_set[dev] = true;
   }
-  nf4_gemm_dense_kernel<<<dim3((unsigned)(g.tiles_m * g.tiles_n)), dim3(512), kLdsDense, s>>>(g);
+  const dim3 grid((unsigned)(g.tiles_m * g.tiles_n)), block(512);
+  if (g.lw_row_major)
+    nf4_gemm_dense_kernel<true><<<grid, block, kLdsDense, s>>>(g);
+  else
+    nf4_gemm_dense_kernel<false><<<grid, block, kLdsDense, s>>>(g);
   return check_launch("nf4_gemm_dense");
 }
 
