@@ -194,3 +194,36 @@ def test_smaller_workspace_keeps_the_fused_kernel():
     assert torch.equal(y[1], y[2])  # both ran the fused kernel
     torch.testing.assert_close(y[0].float(), y[1].float(), rtol=1e-2, atol=2e-3)
     torch.testing.assert_close(y[0].float(), x.float() @ dense.float().T, rtol=1e-2, atol=1e-2)
+
+
+def test_group_forward_over_concatenated_outputs(monkeypatch):
+    """Forward of members with a common input (widths multiples of 256, one of them with a bias): one expanded GEMM over
+    the concatenated output columns against the member-by-member fused kernel and against fp32 matmuls."""
+    M, K = 2048, 192
+    Ns, ranks = (4096, 2048, 2048 + 256), (16, 8, 24)
+    g = torch.Generator().manual_seed(29)
+    x = torch.randn(M, K, generator=g).to(BF).to(DEV)
+    members, denses = [], []
+    for i, (N, r) in enumerate(zip(Ns, ranks)):
+        _, _, qdata, bscal, dense = _quantized(N, K, seed=40 + i)
+        A = (torch.randn(r, K, generator=g) * 0.05).to(BF).to(DEV)
+        B = (torch.randn(N, r, generator=g) * 0.05).to(BF).to(DEV)
+        bias = (torch.randn(N, generator=g) * 0.1).to(BF).to(DEV) if i == 1 else None
+        tr = ops.nf4_transpose_for_backward(qdata, bscal, N, K) if i != 2 else None  # member 2: natural scaler layout
+        members.append(ops.GroupMember(qdata=qdata, block_scalers=bscal, N=N, lora_a=A, lora_b=B, scale=0.5 * (i + 1), bias=bias, transposed=tr))
+        denses.append(dense)
+    ys0 = [torch.empty(M, N, dtype=BF, device=DEV) for N in Ns]
+    arr = ops._group_array("t", members, K, ys0, M)[0]
+    assert _lib.load().ttamd_lora_group_fwd_workspace_bytes(arr, len(members), M, K) == 2 * K * sum(Ns)
+    h_cat, ys = ops.lora_group_fwd(x, members)
+    monkeypatch.setattr(ops, "EXPANDED_WEIGHT_PATH", False)
+    h_cat_f, ys_f = ops.lora_group_fwd(x, members)
+    assert torch.equal(h_cat, h_cat_f)
+    off = 0
+    for m, y, y_f, dense, r in zip(members, ys, ys_f, denses, ranks):
+        torch.testing.assert_close(y.float(), y_f.float(), rtol=1e-2, atol=2e-3)
+        want = x.float() @ dense.float().T + m.scale * h_cat[:, off:off + r].float() @ m.lora_b.float().T
+        if m.bias is not None:
+            want = want + m.bias.float()
+        torch.testing.assert_close(y.float(), want, rtol=1e-2, atol=1e-2)
+        off += r

@@ -58,9 +58,16 @@ SHAPES = [
 @pytest.mark.parametrize("M,K,Ns,ranks", SHAPES, ids=[f"M{s[0]}_K{s[1]}_{'x'.join(map(str, s[2]))}_r{'x'.join(map(str, s[3]))}" for s in SHAPES])
 @pytest.mark.parametrize("bias", [False, True], ids=["nobias", "bias"])
 def test_group_forward_matches_member_calls_bitwise(M, K, Ns, ranks, bias):
+    """Bit-equal wherever the group and the member call run the same kernel.  A group of many tokens can reach the 256
+    output tiles of the expanded-weight GEMM where a member alone does not (then the member runs the fused kernel, with
+    another order of summation inside the matrix instructions): those members are compared at rtol 1e-2 / atol 2e-3."""
+    from torchtune_amd import _lib
+
+    lib = _lib.load()
     mem = _members(K, Ns, ranks, seed=M + K, bias=bias)
     x = torch.randn(M, K, generator=torch.Generator().manual_seed(7)).to(BF).to(DEV)
     h_cat, ys = ops.lora_group_fwd(x, [m[0] for m in mem])
+    group_expands = all(N % 256 == 0 for N in Ns) and bool(lib.ttamd_nf4_gemm_expands_weight(M, sum(Ns), K))
     off = 0
     for (m, t, *_), y in zip(mem, ys):
         r = m.lora_a.shape[0]
@@ -68,7 +75,10 @@ def test_group_forward_matches_member_calls_bitwise(M, K, Ns, ranks, bias):
         assert torch.equal(h_cat[:, off:off + r], h), "hidden activation"
         y1 = ops.nf4_lora_linear_fwd(x, m.qdata, m.block_scalers, m.N, h, m.lora_b, m.scale, m.bias,
                                      block_scalers_t=m.transposed[1])
-        assert torch.equal(y, y1), "member output"
+        if group_expands and not lib.ttamd_nf4_gemm_expands_weight(M, m.N, K):
+            torch.testing.assert_close(y.float(), y1.float(), rtol=1e-2, atol=2e-3)
+        else:
+            assert torch.equal(y, y1), "member output"
         off += r
     assert off == h_cat.shape[1]
 

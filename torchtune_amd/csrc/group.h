@@ -62,6 +62,8 @@ size_t dense_workspace_bytes(int64_t M, int64_t Nout, int64_t Kc);
 int run_gemm_dense(const void* X, const uint8_t* codes, const void* scal, int mode, const void* lX, int ldlx, const void* lW,
                    bool lw_row_major, int R, float lscale, const void* bias, const void* cscale, void* C, int64_t M, int64_t Nout,
                    int64_t Kc, void* workspace, hipStream_t s);
+size_t dense_group_fwd_workspace_bytes(const GroupGemm& d);
+int run_gemm_dense_group_fwd(const void* x, const GroupGemm& d, const void* h_cat, void* workspace, hipStream_t s);
 size_t dense_group_dx_workspace_bytes(const GroupDx& d);
 int run_gemm_dense_group_dx(const GroupDx& d, const void* gh_cat, void* gx, void* workspace, hipStream_t s);
 

@@ -61,9 +61,9 @@ int decode(const char* who, const ttamd_lora_group_member* m, int n, int64_t M, 
   return TTAMD_OK;
 }
 
-// slices of the largest sliced member GEMM
+// slices of the largest sliced member GEMM, or the expanded weight(s) of the many-token path
 size_t fwd_gemm_ws(const Decoded& d) {
-  size_t w = 0;
+  size_t w = d.gm.M > small_m_limit() ? dense_group_fwd_workspace_bytes(d.gm) : 0;
   if (d.gm.M > small_m_limit())
     for (int i = 0; i < d.gm.n; ++i) {
       const size_t b = gemm_rs_workspace_bytes(d.gm.M, d.gm.N[i], d.gm.K);
@@ -117,6 +117,8 @@ extern "C" int ttamd_nf4_lora_group_fwd_bf16(const void* x, const ttamd_lora_gro
   const size_t gem = align256(fwd_gemm_ws(d));
   const bool sliced = gem > 0 && workspace != nullptr && workspace_bytes >= gem;
   TT_REQUIRE(!sliced || aligned16(workspace), "nf4_lora_group_fwd: workspace must be 16-byte aligned");
+  // many tokens: one launch over the members' concatenated output columns, every weight expanded once
+  if (sliced && dense_group_fwd_workspace_bytes(d.gm) > 0) return run_gemm_dense_group_fwd(x, d.gm, h_cat, workspace, s);
   const int ldh = d.gm.r_off[d.gm.n];
   for (int i = 0; i < d.gm.n; ++i) {
     const void* sc = d.gm.bscal_t[i] ? d.gm.bscal_t[i] : d.gm.bscal[i];

@@ -4,10 +4,12 @@
 // and column scale in its epilogue.  The fused kernel (nf4_gemm_rs.hip) repeats the expansion once per 256-row tile of
 // the activations; from a few thousand tokens up that repetition costs more than one pass of the dequantise kernel.
 //
-//     C[M, Nout] = X[M, Kc] . Wd[Nout, Kc]^T  (+ bias, * cscale)  + sum_s (lscale . lX_s)[M, R_s] . lW_s[Nout, R_s]^T
+//     C[M, Nout] = X[M, Kc] . Wd[Nout, Kc]^T  (+ bias, * cscale)  + sum_a (lscale_a . lX_a)[M, R_a] . lW_a[Nout, R_a]^T
 //
-// The contraction may be the concatenation of up to kGroupMax segments (grad-input of layers with a common input:
-// X_s = gy_s, Wd_s = W_s^T), each with its own activation tensor and adapter.
+// Layers with a common input run as one launch either way round.  Grad-input: the contraction is the concatenation of
+// up to kGroupMax segments (X_s = gy_s, Wd_s = W_s^T), each with its own activation tensor, and every member's adapter
+// adds to all output columns.  Forward: the output columns are the concatenation of the members' columns (widths
+// multiples of the 256-wide tile), each member with its own output tensor, bias and adapter.
 //
 // The scratch copy `Wd` is written in the order the matrix cores consume it (v_mfma_f32_16x16x32_bf16): for every block
 // of 16 output columns T and every 32-wide k-step t one 1 KiB piece in which lane l of a wave finds, at byte 16 l, the
@@ -108,21 +110,29 @@ __global__ __launch_bounds__(256) void nf4_expand_tiled_kernel(const uint8_t* __
 
 // ---------------------------------------------------------------------------------------------------------------------
 struct DenseSeg {
-  const uint16_t* X;   // [M, Kc_s] bf16 activations of the segment
-  const uint16_t* lX;  // adapter activations (rows ldlx apart) or null
-  const uint16_t* lW;  // adapter weights: [Nout, R] (lw_row_major) or [R, Nout]
-  int Kc, R;
+  const uint16_t* X;  // [M, Kc] bf16 activations of one segment of the contraction
+  int Kc;
+};
+struct DenseAdapter {   // adds (lscale . lX) . lW^T to the output columns [n_begin, n_end)
+  const uint16_t* lX;   // [M, R] bf16, rows ldlx apart
+  const uint16_t* lW;   // [n_end - n_begin, R] (lw_row_major) or [R, n_end - n_begin] bf16
+  int R, n_begin, n_end;
+  float lscale;
+};
+struct DenseOut {          // output columns [n_begin, n_begin + width) go to their own tensor
+  uint16_t* C;             // [M, width] bf16
+  const uint16_t* bias;    // [width] bf16 or null
+  const uint16_t* cscale;  // [width] bf16 or null: C = (acc + bias) * cscale per column
+  int n_begin, width;
 };
 struct DenseArgs {
   DenseSeg seg[kGroupMax];
-  int nseg;
-  const char* Wt;          // tiled weight, all segments side by side along the contraction
-  const uint16_t* bias;    // [Nout] bf16 or null
-  const uint16_t* cscale;  // [Nout] bf16 or null: C = (acc + bias) * cscale per column
-  uint16_t* C;             // [M, Nout] bf16
-  int M, Nout, Kc;         // Kc: total contraction
+  DenseAdapter ad[kGroupMax];
+  DenseOut out[kGroupMax];
+  int nseg, nad, nout;
+  const char* Wt;   // tiled weight: all output columns, all segments side by side along the contraction
+  int M, Nout, Kc;  // Nout, Kc: totals
   int lw_row_major, ldlx;
-  float lscale;
   int tiles_m, tiles_n;
 };
 
@@ -296,11 +306,14 @@ __global__ __launch_bounds__(512) void nf4_gemm_dense_kernel(const DenseArgs g) 
 
   // ---- adapters: one MFMA step per 32 ranks and segment, operands straight from global memory.  Lane (l15, g4) holds
   //      ranks rc + 8 g4 .. + 7 of weight column / activation row l15 of its tile; ranks beyond R are zero.
-  for (int sidx = 0; sidx < g.nseg; ++sidx) {
-    const int R = g.seg[sidx].R;
-    if (R <= 0) continue;
-    const uint16_t* lX = g.seg[sidx].lX;
-    const uint16_t* lW = g.seg[sidx].lW;
+  for (int aidx = 0; aidx < g.nad; ++aidx) {
+    const int R = g.ad[aidx].R;
+    const int nb = g.ad[aidx].n_begin, ncols = g.ad[aidx].n_end - nb;
+    if (R <= 0 || n0 < nb || n0 >= nb + ncols) continue;  // the same for every wave of the workgroup
+    const uint16_t* lX = g.ad[aidx].lX;
+    const uint16_t* lW = g.ad[aidx].lW;
+    const float lscale = g.ad[aidx].lscale;
+    const int nl0 = n0 - nb;  // first column of the tile among the adapter's columns
     int pitch = 0;  // bytes per column of the staged adapter weights
     if constexpr (!LW_ROW_MAJOR) {
       // lW is [R, Nout]: a lane needs 8 ranks of one column, 8 elements Nout apart.  The workgroup copies the 256
@@ -311,7 +324,7 @@ __global__ __launch_bounds__(512) void nf4_gemm_dense_kernel(const DenseArgs g) 
       for (int idx = tid; idx < R * 32; idx += 512) {
         const int r = idx >> 5, c8 = (idx & 31) * 8;
         u32x4_t raw = {0, 0, 0, 0};
-        if (n0 + c8 < g.Nout) raw = *reinterpret_cast<const u32x4_t*>(lW + (int64_t)r * g.Nout + n0 + c8);
+        if (nl0 + c8 < ncols) raw = *reinterpret_cast<const u32x4_t*>(lW + (int64_t)r * ncols + nl0 + c8);
 #pragma unroll
         for (int e = 0; e < 8; ++e)
           *reinterpret_cast<uint16_t*>(smem + (c8 + e) * pitch + 2 * r) = (uint16_t)(raw[e >> 1] >> (16 * (e & 1)));
@@ -327,8 +340,8 @@ __global__ __launch_bounds__(512) void nf4_gemm_dense_kernel(const DenseArgs g) 
         u32x4_t raw = {0, 0, 0, 0};
         if (in) {
           if constexpr (LW_ROW_MAJOR) {
-            int col = n0 + wn * 64 + 16 * j + l15;
-            col = col < g.Nout ? col : g.Nout - 1;
+            int col = nl0 + wn * 64 + 16 * j + l15;
+            col = col < ncols ? col : ncols - 1;
             raw = *reinterpret_cast<const u32x4_t*>(lW + (int64_t)col * R + r0);
           } else {
             raw = *reinterpret_cast<const u32x4_t*>(smem + (wn * 64 + 16 * j + l15) * pitch + 2 * r0);
@@ -343,10 +356,10 @@ __global__ __launch_bounds__(512) void nf4_gemm_dense_kernel(const DenseArgs g) 
         row = row < g.M ? row : g.M - 1;
         u32x4_t raw = {0, 0, 0, 0};
         if (in) raw = *reinterpret_cast<const u32x4_t*>(lX + (int64_t)row * g.ldlx + r0);
-        if (g.lscale != 1.0f) {
+        if (lscale != 1.0f) {
 #pragma unroll
           for (int d = 0; d < 4; ++d)
-            raw[d] = pack_bf16x2(bits_f32(raw[d] << 16) * g.lscale, bits_f32(raw[d] & 0xffff0000u) * g.lscale);
+            raw[d] = pack_bf16x2(bits_f32(raw[d] << 16) * lscale, bits_f32(raw[d] & 0xffff0000u) * lscale);
         }
         xfr[i] = __builtin_bit_cast(bf16x8_t, raw);
       }
@@ -361,20 +374,26 @@ __global__ __launch_bounds__(512) void nf4_gemm_dense_kernel(const DenseArgs g) 
   //      transposes its 128 x 64 band through LDS (the rings are free now) and writes whole 128-byte row segments;
   //      16-byte chunk c of row r sits in slot c ^ (r & 7).
   __syncthreads();
-  if (n0 + wn * 64 >= g.Nout) return;  // the whole band of this wave lies outside (no barrier follows)
+  int oi = 0;
+  while (oi + 1 < g.nout && n0 >= g.out[oi + 1].n_begin) ++oi;
+  const int nlo = n0 - g.out[oi].n_begin + wn * 64;  // first column of this wave's band in its output tensor
+  const int width = g.out[oi].width;
+  if (nlo >= width) return;  // the whole band of this wave lies outside (no barrier follows)
   {
+    const uint16_t* bias = g.out[oi].bias;
+    const uint16_t* cscale = g.out[oi].cscale;
     char* band = smem + wv * 16384;  // 128 rows x 128 bytes
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
       float b4[4] = {0.f, 0.f, 0.f, 0.f};
-      if (g.bias) {
-        const u32x2_t bb = *reinterpret_cast<const u32x2_t*>(g.bias + n0 + wn * 64 + 16 * j + 4 * g4);
+      if (bias) {
+        const u32x2_t bb = *reinterpret_cast<const u32x2_t*>(bias + nlo + 16 * j + 4 * g4);
         b4[0] = bits_f32(bb.x << 16); b4[1] = bits_f32(bb.x & 0xffff0000u);
         b4[2] = bits_f32(bb.y << 16); b4[3] = bits_f32(bb.y & 0xffff0000u);
       }
       float c4[4] = {1.f, 1.f, 1.f, 1.f};
-      if (g.cscale) {
-        const u32x2_t cc = *reinterpret_cast<const u32x2_t*>(g.cscale + n0 + wn * 64 + 16 * j + 4 * g4);
+      if (cscale) {
+        const u32x2_t cc = *reinterpret_cast<const u32x2_t*>(cscale + nlo + 16 * j + 4 * g4);
         c4[0] = bits_f32(cc.x << 16); c4[1] = bits_f32(cc.x & 0xffff0000u);
         c4[2] = bits_f32(cc.y << 16); c4[3] = bits_f32(cc.y & 0xffff0000u);
       }
@@ -391,13 +410,13 @@ __global__ __launch_bounds__(512) void nf4_gemm_dense_kernel(const DenseArgs g) 
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     const int c = lane & 7;
-    uint16_t* crow = g.C + n0 + wn * 64 + 8 * c;
+    uint16_t* crow = g.out[oi].C + nlo + 8 * c;
     const int mrow0 = m0 + 128 * wm;
 #pragma unroll 8
     for (int t = 0; t < 16; ++t) {
       const int r = 8 * t + (lane >> 3);
       const u32x4_t v = *reinterpret_cast<const u32x4_t*>(band + r * 128 + ((c ^ (r & 7)) << 4));
-      if (mrow0 + r < g.M) *reinterpret_cast<u32x4_t*>(crow + (int64_t)(mrow0 + r) * g.Nout) = v;
+      if (mrow0 + r < g.M) *reinterpret_cast<u32x4_t*>(crow + (int64_t)(mrow0 + r) * width) = v;
     }
   }
 #endif
@@ -459,7 +478,7 @@ size_t dense_workspace_bytes(int64_t M, int64_t Nout, int64_t Kc) {
   return dense_path_applies(M, Nout, Kc) ? (size_t)Nout * (size_t)Kc * 2 : 0;
 }
 
-// One segment: the ordinary forward (mode 0 / 2) or grad-input (mode 1) of a layer.  Arguments as run_gemm_rs.
+// One layer: the ordinary forward (mode 0 / 2) or grad-input (mode 1).  Arguments as run_gemm_rs.
 int run_gemm_dense(const void* X, const uint8_t* codes, const void* scal, int mode, const void* lX, int ldlx, const void* lW,
                    bool lw_row_major, int R, float lscale, const void* bias, const void* cscale, void* C, int64_t M, int64_t Nout,
                    int64_t Kc, void* workspace, hipStream_t s) {
@@ -469,20 +488,69 @@ int run_gemm_dense(const void* X, const uint8_t* codes, const void* scal, int mo
   if (int rc = launch_expand(mode, codes, reinterpret_cast<const float*>(scal), Nout, Kc, Kc >> 5, 0, reinterpret_cast<char*>(workspace), s))
     return rc;
   DenseArgs g = {};
-  g.nseg = 1;
+  g.nseg = g.nout = 1;
   g.seg[0].X = reinterpret_cast<const uint16_t*>(X);
-  g.seg[0].lX = reinterpret_cast<const uint16_t*>(lX);
-  g.seg[0].lW = reinterpret_cast<const uint16_t*>(lW);
   g.seg[0].Kc = (int)Kc;
-  g.seg[0].R = R;
+  g.nad = R > 0 ? 1 : 0;
+  g.ad[0].lX = reinterpret_cast<const uint16_t*>(lX);
+  g.ad[0].lW = reinterpret_cast<const uint16_t*>(lW);
+  g.ad[0].R = R;
+  g.ad[0].n_begin = 0;
+  g.ad[0].n_end = (int)Nout;
+  g.ad[0].lscale = lscale;
+  g.out[0].C = reinterpret_cast<uint16_t*>(C);
+  g.out[0].bias = reinterpret_cast<const uint16_t*>(bias);
+  g.out[0].cscale = reinterpret_cast<const uint16_t*>(cscale);
+  g.out[0].n_begin = 0;
+  g.out[0].width = (int)Nout;
   g.Wt = reinterpret_cast<const char*>(workspace);
-  g.bias = reinterpret_cast<const uint16_t*>(bias);
-  g.cscale = reinterpret_cast<const uint16_t*>(cscale);
-  g.C = reinterpret_cast<uint16_t*>(C);
   g.M = (int)M; g.Nout = (int)Nout; g.Kc = (int)Kc;
   g.lw_row_major = lw_row_major ? 1 : 0;
   g.ldlx = ldlx;
-  g.lscale = lscale;
+  return launch_dense(g, s);
+}
+
+// Forward of a group of layers with a common input as one launch over the members' concatenated output columns.
+size_t dense_group_fwd_workspace_bytes(const GroupGemm& d) {
+  int64_t n_total = 0;
+  for (int i = 0; i < d.n; ++i) {
+    if (d.N[i] % 256 != 0) return 0;  // a tile belongs to one member
+    n_total += d.N[i];
+  }
+  return d.n >= 2 && dense_path_applies(d.M, n_total, d.K) ? (size_t)n_total * (size_t)d.K * 2 : 0;
+}
+
+int run_gemm_dense_group_fwd(const void* x, const GroupGemm& d, const void* h_cat, void* workspace, hipStream_t s) {
+  TT_REQUIRE(d.n >= 2 && d.n <= kGroupMax && dense_group_fwd_workspace_bytes(d) > 0, "nf4_lora_group_fwd (expanded): shape not served");
+  TT_REQUIRE(aligned16(workspace) && aligned16(x), "nf4_lora_group_fwd (expanded): pointers must be 16-byte aligned");
+  DenseArgs g = {};
+  g.nseg = 1;
+  g.seg[0].X = reinterpret_cast<const uint16_t*>(x);
+  g.seg[0].Kc = (int)d.K;
+  g.nout = g.nad = d.n;
+  int64_t n_off = 0;
+  for (int i = 0; i < d.n; ++i) {
+    const bool tr = d.bscal_t[i] != nullptr;
+    if (int rc = launch_expand(tr ? 2 : 0, d.codes[i], tr ? d.bscal_t[i] : d.bscal[i], d.N[i], d.K, d.K >> 5, 0,
+                               reinterpret_cast<char*>(workspace) + n_off * d.K * 2, s))
+      return rc;
+    g.ad[i].lX = reinterpret_cast<const uint16_t*>(h_cat) + d.r_off[i];
+    g.ad[i].lW = d.lora_b[i];
+    g.ad[i].R = d.rank[i];
+    g.ad[i].n_begin = (int)n_off;
+    g.ad[i].n_end = (int)(n_off + d.N[i]);
+    g.ad[i].lscale = d.scale[i];
+    g.out[i].C = d.y[i];
+    g.out[i].bias = d.bias[i];
+    g.out[i].cscale = nullptr;
+    g.out[i].n_begin = (int)n_off;
+    g.out[i].width = (int)d.N[i];
+    n_off += d.N[i];
+  }
+  g.Wt = reinterpret_cast<const char*>(workspace);
+  g.M = (int)d.M; g.Nout = (int)n_off; g.Kc = (int)d.K;
+  g.lw_row_major = 1;
+  g.ldlx = d.r_off[d.n];
   return launch_dense(g, s);
 }
 
@@ -499,29 +567,37 @@ size_t dense_group_dx_workspace_bytes(const GroupDx& d) {
 }
 
 int run_gemm_dense_group_dx(const GroupDx& d, const void* gh_cat, void* gx, void* workspace, hipStream_t s) {
-  TT_REQUIRE(d.n >= 1 && d.n <= kGroupMax && dense_group_dx_workspace_bytes(d) > 0, "nf4_group_dx (dense): shape not served");
-  TT_REQUIRE(aligned16(workspace), "nf4_group_dx (dense): workspace must be 16-byte aligned");
+  TT_REQUIRE(d.n >= 1 && d.n <= kGroupMax && dense_group_dx_workspace_bytes(d) > 0, "nf4_group_dx (expanded): shape not served");
+  TT_REQUIRE(aligned16(workspace), "nf4_group_dx (expanded): workspace must be 16-byte aligned");
   int64_t n_total = 0;
   for (int i = 0; i < d.n; ++i) n_total += d.N[i];
   DenseArgs g = {};
   g.nseg = d.n;
+  g.nout = 1;
   int64_t t_off = 0;
   for (int i = 0; i < d.n; ++i) {
-    TT_REQUIRE(aligned16(d.gy[i]) && aligned16(d.codes_t[i]) && aligned16(d.scal_t[i]), "nf4_group_dx (dense): pointers must be 16-byte aligned");
+    TT_REQUIRE(aligned16(d.gy[i]) && aligned16(d.codes_t[i]) && aligned16(d.scal_t[i]), "nf4_group_dx (expanded): pointers must be 16-byte aligned");
     if (int rc = launch_expand(1, d.codes_t[i], d.scal_t[i], d.K, d.N[i], n_total >> 5, t_off, reinterpret_cast<char*>(workspace), s)) return rc;
     t_off += d.N[i] >> 5;
     g.seg[i].X = d.gy[i];
-    g.seg[i].lX = d.rank[i] > 0 ? reinterpret_cast<const uint16_t*>(gh_cat) + d.r_off[i] : nullptr;
-    g.seg[i].lW = d.lora_a[i];
     g.seg[i].Kc = (int)d.N[i];
-    g.seg[i].R = d.rank[i];
+    if (d.rank[i] > 0) {
+      DenseAdapter& a = g.ad[g.nad++];
+      a.lX = reinterpret_cast<const uint16_t*>(gh_cat) + d.r_off[i];
+      a.lW = d.lora_a[i];
+      a.R = d.rank[i];
+      a.n_begin = 0;
+      a.n_end = (int)d.K;
+      a.lscale = 1.0f;
+    }
   }
+  g.out[0].C = reinterpret_cast<uint16_t*>(gx);
+  g.out[0].n_begin = 0;
+  g.out[0].width = (int)d.K;
   g.Wt = reinterpret_cast<const char*>(workspace);
-  g.C = reinterpret_cast<uint16_t*>(gx);
   g.M = (int)d.M; g.Nout = (int)d.K; g.Kc = (int)n_total;
   g.lw_row_major = 0;
   g.ldlx = d.r_off[d.n];
-  g.lscale = 1.0f;
   return launch_dense(g, s);
 }
 
