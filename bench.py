@@ -38,7 +38,8 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 #     bench.traffic_bytes_per_launch[<workload>] = <bytes>
 # that is read back here, so the bench line always quotes the committed measurement (null when there is none).
 TRAFFIC_SUMMARIES = {
-    "llama3_1_8b": "profiles/nf4_gemm_rs_kernel_hbm_traffic.txt",
+    "llama3_1_8b": "profiles/nf4_gemm_dense_kernel_hbm_traffic.txt",             # weight expanded once per call (default)
+    "llama3_1_8b/fused": "profiles/nf4_gemm_rs_kernel_hbm_traffic.txt",           # --no-expanded-weight
     "llama3_1_8b_qat": "profiles/fake_quant_and_layer_kernels_hbm_traffic.txt",
 }
 
@@ -70,23 +71,33 @@ class GemmTimer:
         self.stride = max(1, stride)
         self.records = []
         self.counts = {}
+        self.expanded_calls = 0
 
     def __call__(self, kind, M, N, K, rank):
-        # "fwd" / "bwd": one layer, one launch.  "fwd_group" / "bwd_group": the layers of a group with a common input (N and
-        # rank are lists): one forward launch per member between the events, or the single grad-input launch whose
-        # contraction runs through all members' output columns.
+        # "fwd" / "bwd": one layer, one call of the library.  "fwd_group" / "bwd_group": the layers of a group with a common
+        # input (N and rank are lists), one call.  Between the events lie all launches of the call: with the weight expanded
+        # once per call (many tokens) one expansion launch per member and one GEMM launch; otherwise one fused launch per
+        # member (forward) or the single fused grad-input launch over all members' output columns.
+        from torchtune_amd import _lib, ops
+
         Ns = tuple(N) if isinstance(N, (list, tuple)) else (N,)
         ranks = tuple(rank) if isinstance(rank, (list, tuple)) else (rank,) * len(Ns)
         fwd = kind.startswith("fwd")
         flops = sum(2.0 * M * n * K + 2.0 * M * r * (n if fwd else K) for n, r in zip(Ns, ranks))
-        # algorithmic bytes of a launch: both activation tensors once, the packed weight with its fp32 block scalers
-        # (0.5 + 4/64 B per element), the adapter operands
+        n_out, k_contract = (sum(Ns), K) if fwd else (K, sum(Ns))
+        expanded = bool(ops.EXPANDED_WEIGHT_PATH and _lib.load().ttamd_nf4_gemm_expands_weight(M, n_out, k_contract)
+                        and (len(Ns) == 1 or not fwd or all(n % 256 == 0 for n in Ns)))
+        # algorithmic bytes of a call: both activation tensors once, the packed weight with its fp32 block scalers
+        # (0.5 + 4/64 B per element), the adapter operands; with the weight expanded once also the bf16 copy written and
+        # read back (4 B per element)
+        per_w = 0.5625 + (4.0 if expanded else 0.0)
         if fwd:
-            launches = len(Ns)
-            nbytes = sum(2.0 * M * K + 2.0 * M * n + 0.5625 * n * K + 2.0 * r * (M + n) for n, r in zip(Ns, ranks))
+            launches = 1 if expanded else len(Ns)
+            nbytes = (2.0 * M * K if expanded else 2.0 * M * K * len(Ns)) + sum(2.0 * M * n + per_w * n * K + 2.0 * r * (M + n) for n, r in zip(Ns, ranks))
         else:
             launches = 1
-            nbytes = 2.0 * M * K + sum(2.0 * M * n + 0.5625 * n * K + 2.0 * r * (M + K) for n, r in zip(Ns, ranks))
+            nbytes = 2.0 * M * K + sum(2.0 * M * n + per_w * n * K + 2.0 * r * (M + K) for n, r in zip(Ns, ranks))
+        self.expanded_calls += 1 if expanded else 0
         key = (kind, M, Ns if len(Ns) > 1 else Ns[0], K)
         seen = self.counts.get(key, [0, flops, nbytes, launches])
         self.counts[key] = [seen[0] + 1, flops, nbytes, launches]
@@ -242,7 +253,7 @@ def cpu_baseline(shape_name: str, rank: int, alpha: float, tokens_sample: int, l
     }
 
 
-def secondary_kernels(dev) -> dict:
+def secondary_kernels(dev, offload_leg: bool = True) -> dict:
     """Achieved HBM GB/s of the bandwidth-bound kernels of the path on the largest 8B weight / activation shapes:
     algorithmic bytes (2.515747 B/element for the NF4 codec, 4 B/element for fake quant) / HIP-event time."""
     from torchtune_amd import ops, to_nf4
@@ -282,9 +293,10 @@ def secondary_kernels(dev) -> dict:
     x = torch.randn(8192, 14336, device=dev, generator=gen).to(torch.bfloat16)
     out["fq_per_token_int8_asym 8192x14336 bf16"] = round(
         x.numel() * 4 / timed(lambda: ops.fq_per_token_int8_asym(x, want_qparams=False)) / 1e9, 1)
-    host = torch.empty(14336, 4096, dtype=torch.bfloat16, pin_memory=True)
-    out["checkpoint offload: nf4_dequantize 14336x4096 written into pinned host memory (PCIe-bound, host bytes only)"] = round(
-        n * 2 / timed(lambda: t.get_original_weight(out=host), iters=5) / 1e9, 1)
+    if offload_leg:
+        host = torch.empty(14336, 4096, dtype=torch.bfloat16, pin_memory=True)
+        out["checkpoint offload: nf4_dequantize 14336x4096 written into pinned host memory (PCIe-bound, host bytes only)"] = round(
+            n * 2 / timed(lambda: t.get_original_weight(out=host), iters=5) / 1e9, 1)
     # forward for a handful of tokens (decode): the packed weight is streamed once, 0.5625 B per element.  The kernels
     # take 7-15 us, less than a launch from Python costs, so 20 launches are captured in a HIP graph and the replay timed.
     bs, bst = t.block_scalers(), t.backward_copy()[1]
@@ -446,7 +458,11 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
-    ap.add_argument("--workload", default="llama3_1_8b", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="llama3_1_8b", choices=sorted(WORKLOADS) + ["hbm_kernels"],
+                    help="a decoder configuration, or 'hbm_kernels': only the bandwidth-bound kernels in isolation (NF4 "
+                         "dequantise / quantise, fake quant, few-token forward), the launches a kernel trace of them should hold")
+    ap.add_argument("--no-offload-leg", action="store_true",
+                    help="hbm_kernels: skip the dequantise-into-pinned-host-memory leg (PCIe-bound launches of the same kernel)")
     ap.add_argument("--cpu-tokens", type=int, default=512,
                     help="starting token count of the CPU-baseline sample, grown until it takes >= 10 s (0 = skip)")
     ap.add_argument("--optimizer-steps", type=int, default=3,
@@ -488,6 +504,20 @@ def main() -> int:
     harness.GROUP_SHARED_INPUT = not args.no_group
     ops.EXPANDED_WEIGHT_PATH = not args.no_expanded_weight
 
+    if args.workload == "hbm_kernels":
+        dev = torch.device("cuda", 0)
+        torch.cuda.set_device(dev)
+        table = secondary_kernels(dev, offload_leg=not args.no_offload_leg)
+        key = "nf4_dequantize 28672x8192 bf16 (235 M elements, beyond the last-level cache)"
+        print(json.dumps({
+            "metric": "NF4 dequantise GB/s beyond the last-level cache (28672x8192, 1 GPU)", "value": table[key], "unit": "GB/s",
+            "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": None, "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "bf16", "data": "synthetic (random-init N(0,0.02) weights)",
+            "config": {"workload": "bandwidth-bound kernels of the path in isolation"},
+            "roofline": {"bound": "hbm", "kernel": "nf4_dequantize_kernel", "achieved": table[key], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                         "frac": round(table[key] / HBM_PEAK_GBPS, 4), "traffic": None},
+            "hbm_bound_kernels": table}))
+        return 0
     shape_name, rank, alpha, batch, seq, ac = WORKLOADS[args.workload]
     qat = args.workload.endswith("_qat")
     qat_group = 32
@@ -591,6 +621,8 @@ def main() -> int:
 
     launches, launches_timed, gemm_ms, gemm_flops, per_shape = timer.summary()
     gemm_bytes = timer.total_bytes
+    calls = sum(v["calls"] for v in per_shape.values())
+    traffic_key = args.workload if timer.expanded_calls * 2 > calls else args.workload + "/fused"
     achieved = gemm_flops / gemm_ms / 1e9 if gemm_ms > 0 else 0.0
     result = {
         "metric": "QLoRA fwd+bwd tokens/sec (Llama-3.1-8B, 1 GPU)" if args.workload == "llama3_1_8b"
@@ -617,19 +649,24 @@ def main() -> int:
         },
         "roofline": {
             "bound": "mfma",
-            "kernel": "nf4_gemm_rs_kernel (fused NF4-dequant + LoRA bf16 MFMA GEMM, forward and grad-input launches)",
+            "kernel": ("nf4_gemm_dense_kernel with the nf4_expand_tiled_kernel launches that precede it in the same call (NF4 weight "
+                       "expanded once per call into scratch memory, then a bf16 MFMA GEMM with the LoRA adapter in its epilogue; forward "
+                       "and grad-input calls)" if timer.expanded_calls * 2 > calls else
+                       "nf4_gemm_rs_kernel (fused NF4-dequant + LoRA bf16 MFMA GEMM, forward and grad-input launches)"),
             "achieved": round(achieved, 1),
             "peak": MFMA_BF16_PEAK_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4),
-            "traffic": measured_traffic(args.workload)[0],
-            "traffic_unit": ("bytes per launch, average over a step's launches (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 from the "
-                             f"rocprofv3 --pmc runs summarised in {measured_traffic(args.workload)[1]}); algorithmic "
-                             f"{gemm_bytes / max(1, launches) / 1e6:.1f}e6") if measured_traffic(args.workload)[1] else None,
+            "traffic": measured_traffic(traffic_key)[0],
+            "traffic_unit": ("bytes per GEMM launch, average over a step's launches, expansion launches included with their GEMM "
+                             "(FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 from the "
+                             f"rocprofv3 --pmc runs summarised in {measured_traffic(traffic_key)[1]}); algorithmic "
+                             f"{gemm_bytes / max(1, launches) / 1e6:.1f}e6") if measured_traffic(traffic_key)[1] else None,
             "launches": launches,
+            "calls_with_expanded_weight": timer.expanded_calls,
             "launches_timed": launches_timed,
-            "timing": f"HIP events on the launch stream around every {timer.stride}th launch of each shape inside the timed steps "
-                      "(an event pair idles the GPU for about 6 us); achieved = sum(flops) / sum(average duration x launches)",
+            "timing": f"HIP events on the launch stream around every {timer.stride}th call of each shape inside the timed steps "
+                      "(an event pair idles the GPU for about 6 us); achieved = sum(flops) / sum(average duration x calls)",
             "gemm_ms_per_step": round(gemm_ms / args.steps, 2),
             "per_shape": per_shape,
         },
