@@ -314,6 +314,29 @@ def secondary_kernels(dev, offload_leg: bool = True) -> dict:
             raise RuntimeError("bench: the graph replay of the few-token forward differs from the eager result")
         out[f"nf4_lora_linear_fwd M={m_tok} 14336x4096 (few-token kernel, packed-weight bytes)"] = round(n * 0.5625 / sec / 1e9, 1)
         del graph
+    # the same for two layers with a common input (gate / up: 2 x 14336 x 4096, rank 16) as one group call: one launch for
+    # both hidden products, one for both outputs
+    t2 = to_nf4((torch.randn(14336, 4096, device=dev, generator=gen) * 0.02).to(torch.bfloat16))
+    members = []
+    for tt in (t, t2):
+        la = (torch.randn(16, 4096, device=dev, generator=gen) * 0.02).to(torch.bfloat16)
+        lb = (torch.randn(14336, 16, device=dev, generator=gen) * 0.02).to(torch.bfloat16)
+        members.append(ops.GroupMember(tt.quantized_data, tt.block_scalers(), tt.backward_copy(), la, lb, None, 2.0, 14336))
+    for m_tok in (1, 16):
+        xs = torch.randn(m_tok, 4096, device=dev, generator=gen).to(torch.bfloat16)
+        _, ys = ops.lora_group_fwd(xs, members)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for _ in range(20):
+                _, yg = ops.lora_group_fwd(xs, members)
+        sec = timed(graph.replay, iters=10) / 20
+        torch.cuda.synchronize()
+        if not all(torch.equal(a, b) for a, b in zip(yg, ys)):
+            raise RuntimeError("bench: the graph replay of the grouped few-token forward differs from the eager result")
+        out[f"lora_group_fwd M={m_tok} 2 x 14336x4096 r=16 (gate / up as one group, packed-weight bytes, both launches)"] = round(
+            2 * n * 0.5625 / sec / 1e9, 1)
+        del graph
     return {"unit": "GB/s (algorithmic bytes / HIP-event time, HBM peak 8000)", **out}
 
 
