@@ -299,7 +299,8 @@ def secondary_kernels(dev, offload_leg: bool = True) -> dict:
             n * 2 / timed(lambda: t.get_original_weight(out=host), iters=5) / 1e9, 1)
     # forward for a handful of tokens (decode): the packed weight is streamed once, 0.5625 B per element.  The kernels
     # take 7-15 us, less than a launch from Python costs, so 20 launches are captured in a HIP graph and the replay timed.
-    bs, bst = t.block_scalers(), t.backward_copy()[1]
+    bs = t.block_scalers()
+    bst = t.backward_copy()[1] if t.backward_copy() is not None else None
     for m_tok in (1, 16):
         xs = torch.randn(m_tok, 4096, device=dev, generator=gen).to(torch.bfloat16)
         ys = ops.nf4_lora_linear_fwd(xs, t.quantized_data, bs, 14336, block_scalers_t=bst)
@@ -414,13 +415,17 @@ def config1_leg(dev, runs: int = 15, warmups: int = 3) -> dict:
 
 
 def memory_leg(build, step, dev) -> dict:
-    """Peak device memory of one forward + backward (``torch.cuda.max_memory_allocated``) with the transposed copy of the
-    codes that the grad-input GEMM streams (0.5625 B per weight element, the default) and without it."""
-    from torchtune_amd import nf4_tensor
+    """Peak device memory of one forward + backward (``torch.cuda.max_memory_allocated``) for the three ways the NF4 GEMMs
+    can run: the weight expanded once per call (the default at training sizes: scratch memory of one weight or group at a
+    time, no transposed copy ever built), the fused kernel with the transposed copy of the codes its grad-input streams
+    (0.5625 B per weight element), and the fused kernel without it (first-generation grad-input kernel)."""
+    from torchtune_amd import nf4_tensor, ops
 
     out = {}
-    for keep in (True, False):
-        nf4_tensor.BACKWARD_COPY = keep
+    keep_expanded, keep_copy = ops.EXPANDED_WEIGHT_PATH, nf4_tensor.BACKWARD_COPY
+    for name, expanded, copy in (("expanded_weight_per_call", True, True), ("fused_with_backward_copy", False, True),
+                                 ("fused_without_backward_copy", False, False)):
+        ops.EXPANDED_WEIGHT_PATH, nf4_tensor.BACKWARD_COPY = expanded, copy
         try:
             model = build()
             step(model)  # builds the derived copies, warms the allocator
@@ -429,12 +434,11 @@ def memory_leg(build, step, dev) -> dict:
             torch.cuda.reset_peak_memory_stats(dev)
             step(model)
             torch.cuda.synchronize()
-            out["with_backward_copy" if keep else "without_backward_copy"] = {
-                "resident_gib": round(resident / 2**30, 3), "peak_gib": round(torch.cuda.max_memory_allocated(dev) / 2**30, 3)}
+            out[name] = {"resident_gib": round(resident / 2**30, 3), "peak_gib": round(torch.cuda.max_memory_allocated(dev) / 2**30, 3)}
             del model
             torch.cuda.empty_cache()
         finally:
-            nf4_tensor.BACKWARD_COPY = True
+            ops.EXPANDED_WEIGHT_PATH, nf4_tensor.BACKWARD_COPY = keep_expanded, keep_copy
     out["unit"] = "GiB (torch.cuda.memory_allocated after a step = weights + derived copies; max_memory_allocated over one fwd+bwd)"
     return out
 
@@ -508,6 +512,9 @@ def main() -> int:
     ap.add_argument("--no-expanded-weight", action="store_true",
                     help="keep the fused NF4 GEMM (expansion repeated per tile, no scratch memory) also for many tokens, "
                          "instead of expanding the weight once per call and running the plain bf16 GEMM")
+    ap.add_argument("--no-backward-copy", action="store_true",
+                    help="keep no transposed copy of the NF4 codes (0.5625 B per weight element less): the expanded-weight path then "
+                         "builds W^T from the weight's own codes, the fused path falls back to its first-generation grad-input kernel")
     ap.add_argument("--calibration-copy-mib", type=int, default=0,
                     help="before the steps, run one elementwise kernel that reads and writes this many MiB: the known-size "
                          "dispatch that FETCH_SIZE / WRITE_SIZE counter runs are scaled by")
@@ -526,6 +533,9 @@ def main() -> int:
     harness.SDPA_BACKEND = args.sdpa
     harness.GROUP_SHARED_INPUT = not args.no_group
     ops.EXPANDED_WEIGHT_PATH = not args.no_expanded_weight
+    if args.no_backward_copy:
+        from torchtune_amd import nf4_tensor
+        nf4_tensor.BACKWARD_COPY = False
 
     if args.workload == "hbm_kernels":
         dev = torch.device("cuda", 0)

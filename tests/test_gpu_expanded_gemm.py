@@ -227,3 +227,39 @@ def test_group_forward_over_concatenated_outputs(monkeypatch):
             want = want + m.bias.float()
         torch.testing.assert_close(y.float(), want, rtol=1e-2, atol=1e-2)
         off += r
+
+
+@pytest.mark.parametrize("N,K", [(256, 8192), (320, 8192 + 64)])
+def test_grad_input_without_transposed_copy_is_the_expanded_weight_bit_for_bit(N, K):
+    """No transposed copy: W^T is expanded from the weight's own codes (a block turned through LDS)."""
+    M = 2048
+    assert _expands(M, K, N)
+    _, _, qdata, bscal, dense = _quantized(N, K, seed=N + 3)
+    gx = ops.nf4_linear_bwd_dx(_one_hot(M, N), qdata, bscal, K, transposed=None)
+    want = dense.repeat((M + N - 1) // N, 1)[:M]
+    assert torch.equal(gx.view(torch.int16), want.contiguous().view(torch.int16))
+
+
+def test_group_without_transposed_copies_equals_group_with_them():
+    """A group whose members keep no transposed copy: forward from natural scalers, grad-input expanded from the weights'
+    own codes; both bit-equal to the same group with the copies (the GEMM sees the same expanded values)."""
+    M, K = 2048, 8192
+    Ns, ranks = (512, 256), (16, 8)
+    g = torch.Generator().manual_seed(31)
+    x = torch.randn(M, K, generator=g).to(BF).to(DEV)
+    with_tr, without = [], []
+    gys = []
+    for i, (N, r) in enumerate(zip(Ns, ranks)):
+        _, _, qdata, bscal, _ = _quantized(N, K, seed=50 + i)
+        A = (torch.randn(r, K, generator=g) * 0.02).to(BF).to(DEV)
+        B = (torch.randn(N, r, generator=g) * 0.01).to(BF).to(DEV)
+        tr = ops.nf4_transpose_for_backward(qdata, bscal, N, K)
+        with_tr.append(ops.GroupMember(qdata, bscal, tr, A, B, None, 2.0, N))
+        without.append(ops.GroupMember(qdata, bscal, None, A, B, None, 2.0, N))
+        gys.append(torch.randn(M, N, generator=g).to(BF).to(DEV))
+    assert ops.group_dx_expands(M, K, Ns)
+    h1, _ = ops.lora_group_fwd(x, with_tr)
+    gx1, _, _ = ops.lora_group_bwd(x, h1, with_tr, gys)
+    h2, _ = ops.lora_group_fwd(x, without)
+    gx2, _, _ = ops.lora_group_bwd(x, h2, without, gys)
+    assert torch.equal(h1, h2) and torch.equal(gx1, gx2)

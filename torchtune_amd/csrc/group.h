@@ -44,8 +44,10 @@ struct GroupDx {
   int64_t N[kGroupMax];
   int rank[kGroupMax], r_off[kGroupMax + 1];
   const uint16_t* gy[kGroupMax];       // [M, N]
-  const uint8_t* codes_t[kGroupMax];   // [K, N/2]
-  const float* scal_t[kGroupMax];      // [K/64, N]
+  const uint8_t* codes_t[kGroupMax];   // [K, N/2] or null (then codes / bscal serve the expanded-weight path)
+  const float* scal_t[kGroupMax];      // [K/64, N] or null
+  const uint8_t* codes[kGroupMax];     // [N, K/2]
+  const float* bscal[kGroupMax];       // [N, K/64]
   const uint16_t* lora_a[kGroupMax];   // [rank, K]
 };
 

@@ -54,7 +54,9 @@ int decode(const char* who, const ttamd_lora_group_member* m, int n, int64_t M, 
     d.gm.bias[i] = reinterpret_cast<const uint16_t*>(e.bias);
     d.gm.y[i] = reinterpret_cast<uint16_t*>(e.y);
     d.dx.codes_t[i] = e.quantized_data_t;
-    d.dx.scal_t[i] = reinterpret_cast<const float*>(e.block_scalers_t);
+    d.dx.scal_t[i] = e.quantized_data_t ? reinterpret_cast<const float*>(e.block_scalers_t) : nullptr;
+    d.dx.codes[i] = e.quantized_data;
+    d.dx.bscal[i] = reinterpret_cast<const float*>(e.block_scalers);
   }
   TT_REQUIRE(off <= 64, "%s: the ranks of a group sum to at most 64 (got %d)", who, off);
   d.sk.r_off[n] = d.gm.r_off[n] = d.dx.r_off[n] = off;
@@ -173,8 +175,6 @@ extern "C" int ttamd_nf4_group_bwd_dx_ws_bf16(const ttamd_lora_group_member* mem
   if (need == 0 || workspace == nullptr || workspace_bytes < need)
     return ttamd_nf4_group_bwd_dx_bf16(members, n_members, gh_cat, gx, M, K, stream);
   TT_REQUIRE(gh_cat && gx && aligned16(gh_cat) && aligned16(gx), "nf4_group_bwd_dx: gh_cat and gx must be non-null and 16-byte aligned");
-  for (int i = 0; i < n_members; ++i)
-    TT_REQUIRE(d.dx.codes_t[i] && d.dx.scal_t[i] && aligned16(d.dx.codes_t[i]),
-               "nf4_group_bwd_dx: member %d: needs the transposed copies (ttamd_nf4_transpose_for_backward), 16-byte aligned", i);
+  // members without transposed copies are expanded from the weight's own codes
   return run_gemm_dense_group_dx(d.dx, gh_cat, gx, workspace, reinterpret_cast<hipStream_t>(stream));
 }

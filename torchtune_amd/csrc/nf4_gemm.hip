@@ -524,6 +524,10 @@ extern "C" int ttamd_nf4_linear_bwd_dx_ws_bf16(const void* gy, const uint8_t* qu
     return run_gemm_rs(gy, quantized_data_t, block_scalers_t, 1, gh, rank, lora_a, false, rank, 1.0f, nullptr, nullptr, gx, M, K, N,
                        workspace, workspace_bytes, reinterpret_cast<hipStream_t>(stream));
   }
+  // no transposed copy, many tokens and room for the expanded weight: W^T is expanded from the weight's own codes
+  if (workspace != nullptr && dense_path_applies(M, K, N) && workspace_bytes >= dense_workspace_bytes(M, K, N))
+    return run_gemm_dense(gy, quantized_data, block_scalers, 3, gh, rank, lora_a, false, rank, 1.0f, nullptr, nullptr, gx, M, K, N,
+                          workspace, reinterpret_cast<hipStream_t>(stream));
   GemmArgs g;
   g.A = reinterpret_cast<const uint16_t*>(gy);
   g.qdata = quantized_data;

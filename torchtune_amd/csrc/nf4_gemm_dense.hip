@@ -59,6 +59,7 @@ __constant__ float kNF4Dense[16] = TT_NF4_TABLE;
 //   MODE 0: codes [Nout, Kc / 2], block scalers [Nout, Kc / 64]            (forward, natural layout)
 //   MODE 2: codes [Nout, Kc / 2], block scalers transposed [Kc / 64, Nout] (forward, when the backward copy exists)
 //   MODE 1: codes of W^T [Nout, Kc / 2] with per-element scalers [Nout / 64, Kc] (grad-input: Nout = K, Kc = N)
+//   (mode 3 of the launcher: grad-input from the weight's own codes, nf4_expand_tiled_transposed_kernel below)
 // A workgroup of 256 threads covers 16 columns (one T) x 16 k-steps per iteration of its loop over the contraction.
 // ---------------------------------------------------------------------------------------------------------------------
 template <int MODE>
@@ -105,6 +106,49 @@ __global__ __launch_bounds__(256) void nf4_expand_tiled_kernel(const uint8_t* __
       }
       *reinterpret_cast<u32x4_t*>(piece + (16 * g4 + r) * 16) = o;
     }
+  }
+}
+
+// The same for the grad-input when the weight has no transposed copy: codes [N, K / 2] and block scalers [N, K / 64] as
+// they lie, output = tiles of W^T (rows: k, contraction: n).  A workgroup expands 32 rows n (one 32-wide step of the
+// contraction) x 256 columns k, turns the block through LDS (row pitch 80 bytes: both the 2-byte writes down a column
+// and the 16-byte reads along a row spread over the banks) and writes sixteen 1 KiB pieces.
+__global__ __launch_bounds__(256) void nf4_expand_tiled_transposed_kernel(const uint8_t* __restrict__ codes, const float* __restrict__ scal,
+                                                                          int N, int K, int nk_total, int t_off, char* __restrict__ tiled) {
+  constexpr int kPitch = 80;
+  __shared__ float2 lut[256];
+  __shared__ __attribute__((aligned(16))) char sm[256 * kPitch];
+  const int tid = threadIdx.x;
+  lut[tid] = make_float2(round_to_bf16(kNF4Dense[tid >> 4]), round_to_bf16(kNF4Dense[tid & 15]));
+  __syncthreads();
+  const int r = tid & 31, c = tid >> 5;
+  const int n = 32 * blockIdx.x + r;
+  const int kk0 = 256 * blockIdx.y + 32 * c;
+  if (kk0 < K) {
+    const u32x4_t cd = *reinterpret_cast<const u32x4_t*>(codes + (int64_t)n * (K >> 1) + (kk0 >> 1));
+    const float sc = scal[(int64_t)n * (K >> 6) + (kk0 >> 6)];
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      const uint32_t w = cd[d];
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        const float2 pr = lut[(w >> (8 * b)) & 0xffu];
+        const uint32_t two = pack_bf16x2(pr.x * sc, pr.y * sc);
+        const int j = 32 * c + 8 * d + 2 * b;
+        *reinterpret_cast<uint16_t*>(sm + j * kPitch + 2 * r) = (uint16_t)two;
+        *reinterpret_cast<uint16_t*>(sm + (j + 1) * kPitch + 2 * r) = (uint16_t)(two >> 16);
+      }
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int idx = tid + 256 * i;
+    const int Tl = idx >> 6, l = idx & 63;
+    const int T = 16 * blockIdx.y + Tl;
+    if (16 * T >= K) break;
+    const u32x4_t v = *reinterpret_cast<const u32x4_t*>(sm + (16 * Tl + (l & 15)) * kPitch + 16 * (l >> 4));
+    *reinterpret_cast<u32x4_t*>(tiled + ((int64_t)T * nk_total + t_off + blockIdx.x) * 1024 + l * 16) = v;
   }
 }
 
@@ -429,6 +473,12 @@ int launch_expand(int mode, const uint8_t* codes, const float* scal, int64_t Nou
   int64_t ysplit = (2048 + (Nout >> 4) - 1) / (Nout >> 4);
   ysplit = ysplit < 1 ? 1 : (ysplit > chunks ? chunks : ysplit);
   const dim3 grid((unsigned)(Nout >> 4), (unsigned)ysplit), block(256);
+  if (mode == 3) {  // Nout = K, Kc = N of the weight: codes and scalers in the weight's own layout
+    TT_REQUIRE((Nout + 255) / 256 < 65536, "nf4_expand_tiled: K too large for one launch");
+    nf4_expand_tiled_transposed_kernel<<<dim3((unsigned)(Kc >> 5), (unsigned)((Nout + 255) / 256)), block, 0, s>>>(
+        codes, scal, (int)Kc, (int)Nout, (int)nk_total, (int)t_off, tiled);
+    return check_launch("nf4_expand_tiled_transposed");
+  }
   if (mode == 1)
     nf4_expand_tiled_kernel<1><<<grid, block, 0, s>>>(codes, scal, (int)Nout, (int)Kc, (int)nk_total, (int)t_off, tiled);
   else if (mode == 2)
@@ -576,8 +626,12 @@ int run_gemm_dense_group_dx(const GroupDx& d, const void* gh_cat, void* gx, void
   g.nout = 1;
   int64_t t_off = 0;
   for (int i = 0; i < d.n; ++i) {
-    TT_REQUIRE(aligned16(d.gy[i]) && aligned16(d.codes_t[i]) && aligned16(d.scal_t[i]), "nf4_group_dx (expanded): pointers must be 16-byte aligned");
-    if (int rc = launch_expand(1, d.codes_t[i], d.scal_t[i], d.K, d.N[i], n_total >> 5, t_off, reinterpret_cast<char*>(workspace), s)) return rc;
+    const bool tr = d.codes_t[i] != nullptr;
+    TT_REQUIRE(aligned16(d.gy[i]) && (tr ? aligned16(d.codes_t[i]) && aligned16(d.scal_t[i]) : aligned16(d.codes[i]) && d.bscal[i] != nullptr),
+               "nf4_group_dx (expanded): pointers must be 16-byte aligned");
+    if (int rc = launch_expand(tr ? 1 : 3, tr ? d.codes_t[i] : d.codes[i], tr ? d.scal_t[i] : d.bscal[i], d.K, d.N[i], n_total >> 5, t_off,
+                               reinterpret_cast<char*>(workspace), s))
+      return rc;
     t_off += d.N[i] >> 5;
     g.seg[i].X = d.gy[i];
     g.seg[i].Kc = (int)d.N[i];

@@ -34,7 +34,7 @@ class _QDoRALinearFn(torch.autograd.Function):
         N, K = weight.shape
         _check_in_features(x, weight)
         x2 = x.reshape(-1, K)
-        tr = weight.backward_copy()
+        tr = weight.backward_copy_for(x2.shape[0], True)
         _, mns = ops.nf4_dora_weight_norm(weight.quantized_data, weight.block_scalers(), N, K, lora_a, lora_b, scale, magnitude)
         h = ops.lora_hidden(x2, lora_a)
         y = ops.nf4_lora_linear_fwd(x2, weight.quantized_data, weight.block_scalers(), N, h, lora_b, scale, bias,
@@ -56,7 +56,7 @@ class _QDoRALinearFn(torch.autograd.Function):
             gh, ga, gb = ops.lora_bwd(gy0, x2, h, lora_b, ctx.scale)
             if need_x:
                 gx = ops.nf4_linear_bwd_dx(gy0, weight.quantized_data, weight.block_scalers(), K, gh, lora_a,
-                                           transposed=weight.backward_copy()).view(ctx.x_shape)
+                                           transposed=weight.backward_copy_for(gy0.shape[0], False)).view(ctx.x_shape)
         if ctx.has_bias and need_bias:
             gbias = gy0.sum(dim=0)
         return gx, None, (ga if need_a else None), (gb if need_b else None), (gmag if need_m else None), gbias, None

@@ -15,15 +15,17 @@ from typing import List, Sequence, Tuple
 
 import torch
 
-from ... import ops
+from ... import nf4_tensor, ops
 from ...nf4_tensor import _check_in_features
 from .lora import LoRALinear
 
 
-def _member(layer: LoRALinear) -> ops.GroupMember:
-    w = layer.weight
-    return ops.GroupMember(w.quantized_data, w.block_scalers(), w.backward_copy(), layer.lora_a.weight, layer.lora_b.weight,
-                           layer.bias, layer.alpha / layer.rank, w.shape[0])
+def _copies(weights, tokens: int):
+    """The members' transposed copies for a call over ``tokens`` rows: none when the grouped grad-input runs on the
+    expanded-weight path (it reads the weights' own codes), else every member's ``backward_copy()``."""
+    if ops.group_dx_expands(tokens, weights[0].shape[1], [w.shape[0] for w in weights]):
+        return [None] * len(weights)
+    return [w.backward_copy() for w in weights]
 
 
 class _QLoRAGroupFn(torch.autograd.Function):
@@ -37,8 +39,8 @@ class _QLoRAGroupFn(torch.autograd.Function):
         for w in weights:
             _check_in_features(x, w)
         x2 = x.reshape(-1, K)
-        members = [ops.GroupMember(w.quantized_data, w.block_scalers(), w.backward_copy(), a, b, bias, s, w.shape[0])
-                   for w, a, b, bias, s in zip(weights, las, lbs, biases, scales)]
+        members = [ops.GroupMember(w.quantized_data, w.block_scalers(), tr, a, b, bias, s, w.shape[0])
+                   for w, tr, a, b, bias, s in zip(weights, _copies(weights, x2.shape[0]), las, lbs, biases, scales)]
         h_cat, ys = ops.lora_group_fwd(x2, members)
         ctx.save_for_backward(x2, h_cat, *weights, *las, *lbs)
         ctx.scales = scales
@@ -59,8 +61,8 @@ class _QLoRAGroupFn(torch.autograd.Function):
             # an output nobody used arrives as None
             gy2.append(torch.zeros(x2.shape[0], w.shape[0], dtype=x2.dtype, device=x2.device) if g is None
                        else g.reshape(-1, w.shape[0]))
-        members = [ops.GroupMember(w.quantized_data, w.block_scalers(), w.backward_copy(), a, b, None, s, w.shape[0])
-                   for w, a, b, s in zip(weights, las, lbs, ctx.scales)]
+        members = [ops.GroupMember(w.quantized_data, w.block_scalers(), tr, a, b, None, s, w.shape[0])
+                   for w, tr, a, b, s in zip(weights, _copies(weights, x2.shape[0]), las, lbs, ctx.scales)]
         need_x = ctx.needs_input_grad[0]
         gx, grads, _ = ops.lora_group_bwd(x2, h_cat, members, gy2, want_gx=need_x)
         out: List = [gx.view(ctx.x_shape) if need_x else None, None]
@@ -78,7 +80,12 @@ def group_applies(x: torch.Tensor, layers: Sequence[torch.nn.Module]) -> bool:
     for layer in layers:
         if type(layer) is not LoRALinear or layer.disabled or not layer._fused(x):
             return False
-        if layer.in_dim != layers[0].in_dim or layer.weight.backward_copy() is None:
+        if layer.in_dim != layers[0].in_dim:
+            return False
+    if not nf4_tensor.BACKWARD_COPY:
+        # without the transposed copies the grouped grad-input exists only on the expanded-weight path (many tokens)
+        M = x.numel() // layers[0].in_dim
+        if not ops.group_dx_expands(M, layers[0].in_dim, [l.out_dim for l in layers]):
             return False
     return ops.group_shape_ok([l.out_dim for l in layers], layers[0].in_dim, [l.rank for l in layers])
 

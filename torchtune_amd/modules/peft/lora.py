@@ -44,7 +44,7 @@ class _QLoRALinearFn(torch.autograd.Function):
         _check_in_features(x, weight)
         x2 = x.reshape(-1, K)
         h = ops.lora_hidden(x2, lora_a)
-        tr = weight.backward_copy()
+        tr = weight.backward_copy_for(x2.shape[0], True)
         y = ops.nf4_lora_linear_fwd(x2, weight.quantized_data, weight.block_scalers(), N, h, lora_b, scale, bias,
                                     block_scalers_t=tr[1] if tr else None)
         ctx.save_for_backward(x2, h, weight, lora_a, lora_b)
@@ -64,7 +64,7 @@ class _QLoRALinearFn(torch.autograd.Function):
             gh, ga, gb = ops.lora_bwd(gy2, x2, h, lora_b, ctx.scale)
             if need_x:
                 gx = ops.nf4_linear_bwd_dx(gy2, weight.quantized_data, weight.block_scalers(), K, gh, lora_a,
-                                           transposed=weight.backward_copy())
+                                           transposed=weight.backward_copy_for(gy2.shape[0], False))
                 gx = gx.view(ctx.x_shape)
             if not need_a:
                 ga = None

@@ -250,6 +250,16 @@ class NF4Tensor(torch.Tensor):
         qs._ttamd_backward_copy = (key, val)
         return val
 
+    def backward_copy_for(self, tokens: int, forward: bool):
+        """The transposed copy a GEMM call over ``tokens`` rows would use: None when the library serves that call from the
+        weight expanded once per call (many tokens; it then reads the weight's own codes, so a purely many-token
+        training run never builds the copy), otherwise ``backward_copy()``."""
+        N, K = self.shape
+        n_out, k_contract = (N, K) if forward else (K, N)
+        if ops.gemm_expands_weight(tokens, n_out, k_contract):
+            return None
+        return self.backward_copy()
+
     # ---- tensor-subclass protocol --------------------------------------------------------------------
     def __tensor_flatten__(self):
         ctx = {
@@ -488,7 +498,7 @@ class _LinearNF4(torch.autograd.Function):
         ctx.in_shape = input.shape
         if _fused_ok(input, weight, 0):
             x2 = input.reshape(-1, input.shape[-1])
-            tr = weight.backward_copy()
+            tr = weight.backward_copy_for(x2.shape[0], True)
             y = ops.nf4_lora_linear_fwd(x2, weight.quantized_data, weight.block_scalers(), weight.shape[0],
                                         block_scalers_t=tr[1] if tr else None)
             return y.view(*input.shape[:-1], weight.shape[0])
@@ -502,7 +512,7 @@ class _LinearNF4(torch.autograd.Function):
         if _fused_ok(grad_output, weight, 0):
             g2 = grad_output.reshape(-1, grad_output.shape[-1])
             gx = ops.nf4_linear_bwd_dx(g2, weight.quantized_data, weight.block_scalers(), weight.shape[1],
-                                       transposed=weight.backward_copy())
+                                       transposed=weight.backward_copy_for(g2.shape[0], False))
             return gx.view(ctx.in_shape), None
         return grad_output @ weight.to(grad_output.dtype), None
 

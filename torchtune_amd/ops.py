@@ -217,6 +217,11 @@ def lora_hidden(x: torch.Tensor, lora_a: torch.Tensor) -> torch.Tensor:
 EXPANDED_WEIGHT_PATH = True
 
 
+def gemm_expands_weight(M: int, n_out: int, k_contract: int) -> bool:
+    """True when an NF4 GEMM call of this shape runs on the weight expanded once per call (needs no transposed copy)."""
+    return bool(EXPANDED_WEIGHT_PATH and _lib.load().ttamd_nf4_gemm_expands_weight(M, n_out, k_contract))
+
+
 def _gemm_workspace(lib, M: int, n_out: int, k_contract: int, device):
     """Scratch memory for one NF4 GEMM: fp32 slices of the contraction for a launch of few output tiles, or room for the
     expanded weight of a many-token launch (None: not needed, or the expanded path is switched off)."""
@@ -301,7 +306,8 @@ def nf4_linear_bwd_dx(
         _check_adapter("nf4_linear_bwd_dx", M, K, gh, lora_a, lambda r: (r, K))
     gx = torch.empty(M, K, dtype=torch.bfloat16, device=gy.device)
     lib = _lib.load()
-    ws, ws_bytes = _gemm_workspace(lib, M, K, N, gy.device) if transposed else (None, 0)
+    # without the transposed copy only the expanded-weight path takes a workspace (the first-generation kernel slices nothing)
+    ws, ws_bytes = _gemm_workspace(lib, M, K, N, gy.device) if transposed or lib.ttamd_nf4_gemm_expands_weight(M, K, N) else (None, 0)
     with torch.cuda.device(gy.device):
         events = _gemm_timer("bwd", M, N, K, rank) if _gemm_timer is not None else None
         if events:
@@ -364,6 +370,11 @@ def group_shape_ok(Ns: Sequence[int], K: int, ranks: Sequence[int]) -> bool:
     """Shapes the group entry points accept."""
     return (1 <= len(Ns) <= _lib.GROUP_MAX and K % 64 == 0 and all(n % 64 == 0 for n in Ns)
             and all(r > 0 and r % 8 == 0 for r in ranks) and sum(ranks) <= 64 and max(Ns) >= 128)
+
+
+def group_dx_expands(M: int, K: int, Ns: Sequence[int]) -> bool:
+    """True when the grouped grad-input of these members runs on the expanded-weight path, which needs no transposed copies."""
+    return bool(EXPANDED_WEIGHT_PATH and all(n % 64 == 0 for n in Ns) and _lib.load().ttamd_nf4_gemm_expands_weight(M, K, sum(Ns)))
 
 
 def _group_array(what: str, members: Sequence[GroupMember], K: int, ys: Sequence[torch.Tensor], M: int,
@@ -446,8 +457,10 @@ def lora_group_bwd(x: torch.Tensor, h_cat: torch.Tensor, members: Sequence[Group
     r_total = sum(int(e.rank) for e in arr)
     if tuple(h_cat.shape) != (M, r_total):
         raise ValueError(f"lora_group_bwd: h_cat is {tuple(h_cat.shape)}, expected {(M, r_total)}")
-    if want_gx and any(m.transposed is None for m in members):
-        raise ValueError("lora_group_bwd: the grouped grad-input needs every member's transposed copy")
+    if want_gx and any(m.transposed is None for m in members) and not (
+            EXPANDED_WEIGHT_PATH and _lib.load().ttamd_nf4_group_bwd_dx_workspace_bytes(arr, len(members), M, K)):
+        raise ValueError("lora_group_bwd: the grouped grad-input needs every member's transposed copy (or a shape the "
+                         "expanded-weight path serves)")
     gh_cat = torch.empty(M, r_total, dtype=torch.bfloat16, device=dev)
     gx = torch.empty(M, K, dtype=torch.bfloat16, device=dev) if want_gx else None
     lib = _lib.load()
