@@ -83,6 +83,15 @@ class GemmTimer:
         Ns = tuple(N) if isinstance(N, (list, tuple)) else (N,)
         ranks = tuple(rank) if isinstance(rank, (list, tuple)) else (rank,) * len(Ns)
         fwd = kind.startswith("fwd")
+        if kind == "tiled":  # the plain GEMM on a bf16 weight already in tile order (QAT): y [M, N] = x [M, K] . Wd^T
+            key = (kind, M, Ns[0], K)
+            seen = self.counts.get(key, [0, 2.0 * M * Ns[0] * K, 2.0 * (M * K + M * Ns[0] + Ns[0] * K), 1])
+            self.counts[key] = [seen[0] + 1] + seen[1:]
+            if seen[0] % self.stride:
+                return None
+            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            self.records.append((key, start, end))
+            return start, end
         flops = sum(2.0 * M * n * K + 2.0 * M * r * (n if fwd else K) for n, r in zip(Ns, ranks))
         n_out, k_contract = (sum(Ns), K) if fwd else (K, sum(Ns))
         expanded = bool(ops.EXPANDED_WEIGHT_PATH and _lib.load().ttamd_nf4_gemm_expands_weight(M, n_out, k_contract)
@@ -146,7 +155,9 @@ class FqTimer:
 
     def __call__(self, kind, rows, K, group_size, elem_bytes):
         n = rows * K
-        nbytes = 2 * n * elem_bytes + (rows * 8 if kind == "per_token" else n // group_size * 4)
+        # "per_group_tiled1" / "per_group_tiled2": the weight fake-quantised into one / both tile orders of the library's GEMM
+        outputs = 2 if kind == "per_group_tiled2" else 1
+        nbytes = (1 + outputs) * n * elem_bytes + (rows * 8 if kind == "per_token" else n // group_size * 4)
         key = (kind, rows, K, group_size, elem_bytes)
         seen = self.counts.get(key, [0, nbytes])
         self.counts[key] = [seen[0] + 1, nbytes]
@@ -512,6 +523,9 @@ def main() -> int:
     ap.add_argument("--no-expanded-weight", action="store_true",
                     help="keep the fused NF4 GEMM (expansion repeated per tile, no scratch memory) also for many tokens, "
                          "instead of expanding the weight once per call and running the plain bf16 GEMM")
+    ap.add_argument("--no-qat-tiled-gemm", action="store_true",
+                    help="QAT workload: row-major fq(W) and the vendor library's GEMM for every matmul, instead of fake-quantising "
+                         "the weights straight into the tile order of the library's own GEMM for forward and grad-input")
     ap.add_argument("--no-backward-copy", action="store_true",
                     help="keep no transposed copy of the NF4 codes (0.5625 B per weight element less): the expanded-weight path then "
                          "builds W^T from the weight's own codes, the fused path falls back to its first-generation grad-input kernel")
@@ -533,6 +547,9 @@ def main() -> int:
     harness.SDPA_BACKEND = args.sdpa
     harness.GROUP_SHARED_INPUT = not args.no_group
     ops.EXPANDED_WEIGHT_PATH = not args.no_expanded_weight
+    if args.no_qat_tiled_gemm:
+        from torchtune_amd import qat as qat_module
+        qat_module.TILED_GEMM = False
     if args.no_backward_copy:
         from torchtune_amd import nf4_tensor
         nf4_tensor.BACKWARD_COPY = False
@@ -599,6 +616,14 @@ def main() -> int:
 
     if qat:
         fq = fq_timer.summary()
+        own_gemm = None
+        if timer.counts:
+            g_launches, g_timed, g_ms, g_flops, g_shapes = timer.summary()
+            own_gemm = {"kernel": "nf4_gemm_dense_kernel on weights fake-quantised straight into its tile order (forward and "
+                                  "grad-input of every linear; the weight gradients run on the vendor library)",
+                        "launches": g_launches, "tflops": round(g_flops / g_ms / 1e9, 1), "frac_of_bf16_mfma_peak":
+                        round(g_flops / g_ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4), "gemm_ms_per_step": round(g_ms / args.steps, 2),
+                        "per_shape": g_shapes}
         fq_ms = sum(v["ms"] for v in fq.values())
         fq_bytes = sum(v["bytes"] for v in fq.values())
         achieved = fq_bytes / fq_ms / 1e6 if fq_ms > 0 else 0.0
@@ -627,8 +652,8 @@ def main() -> int:
             },
             "roofline": {
                 "bound": "hbm",
-                "kernel": "fq_per_token_regs_kernel + fq_per_group_kernel (the fake-quant launches of the step; the matmuls "
-                          "are stock hipBLASLt)",
+                "kernel": "fq_per_token_regs_kernel + fq_int4_sym_tiled_kernel / fq_per_group_kernel (the fake-quant launches of "
+                          "the step; forward and grad-input matmuls: see own_gemm, weight gradients: vendor library)",
                 "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBPS,
                 "unit": "GB/s",
@@ -643,6 +668,7 @@ def main() -> int:
                 "per_kernel": {k: {kk: vv for kk, vv in v.items() if kk in ("launches", "avg_us", "gbps")} for k, v in fq.items()},
             },
         }
+        result["own_gemm"] = own_gemm
         result["with_adamw"] = with_adamw
         result["peak_memory_gib_timed_steps"] = round(peak_timed / 2**30, 3)
         del model

@@ -428,6 +428,27 @@ int ttamd_quantize_per_group_uint4_conv(const void* w, int dtype, int64_t rows, 
                                         uint8_t* q, float* scale, float* zero_point, const ttamd_fq_conventions* conventions,
                                         void* stream);
 
+/*
+ * The weight side of FakeQuantizedLinear.forward = F.linear(fq(x), fq(W)) (torchao; reached from
+ * recipes/qat_single_device.py:378-386 through Int8DynActInt4WeightQATQuantizer.prepare) on this library's own GEMM:
+ *   ttamd_fq_per_group_int4_sym_tiled_bf16: ttamd_fq_per_group_int4_sym of a bf16 weight [N, K] (same values bit for bit,
+ *     same scales), written straight into the layout ttamd_tiled_linear_bf16 reads instead of row-major: tiled_fwd
+ *     (fq(W), for y = x . fq(W)^T) and / or tiled_bwd (fq(W)^T, for gx = gy . fq(W)); either may be NULL, each holds
+ *     ttamd_tiled_weight_bytes(N, K) = 2 N K bytes.  group_size 32, 64, 128 or 256 (else TTAMD_EUNSUPPORTED); eps: lower
+ *     bound of the scale (2^-23 is what the plain entry point uses); scale out fp32 [N, K / group_size] or NULL.
+ *   ttamd_tiled_linear_bf16: y[M, n_out] = x[M, k_contract] . Wd^T (+ bias) with Wd in the tiled layout
+ *     (forward: n_out = N, k_contract = K, tiled_fwd; grad-input: n_out = K, k_contract = N, tiled_bwd, bias NULL).
+ *     n_out and k_contract multiples of 64.  The kernel of the many-token NF4 path; meant for M of a few thousand rows.
+ * Layout: for every block of 16 output columns T and every 32-wide step t of the contraction one 1 KiB piece,
+ * piece (T, t) at byte ((T * k_contract / 32) + t) * 1024; in it lane l (0..63) finds, at byte 16 l, the eight bf16
+ * values Wd[16 T + l % 16][32 t + 8 (l / 16) .. + 7] (the operand order of v_mfma_f32_16x16x32_bf16).
+ */
+size_t ttamd_tiled_weight_bytes(int64_t N, int64_t K);
+int ttamd_fq_per_group_int4_sym_tiled_bf16(const void* w, int64_t N, int64_t K, int group_size, int qparam_dtype, float eps,
+                                           void* tiled_fwd, void* tiled_bwd, float* scale, void* stream);
+int ttamd_tiled_linear_bf16(const void* x, const void* tiled_weight, const void* bias, void* y, int64_t M, int64_t n_out,
+                            int64_t k_contract, void* stream);
+
 /* ------------------------------------------------------------------------------------------------
  * Neighbours of the quantized linears inside a decoder layer (one pass over HBM each, bf16 tensors, fp32 math).
  * Floating-point kernels: results agree with the eager sequences to a tolerance (summation order and hardware

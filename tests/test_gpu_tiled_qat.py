@@ -1,0 +1,98 @@
+"""GPU parity of the 8da4w fake-quantised linear on the library's own GEMM: the weight's per-group int4 fake quantisation
+written straight into the GEMM's tile order (``ttamd_fq_per_group_int4_sym_tiled_bf16``) and the plain tiled GEMM
+(``ttamd_tiled_linear_bf16``) for forward and grad-input.
+
+The staged values are checked bit for bit: with one-hot rows as activations every output of the GEMM is a single product
+1 * fq(W)[n][k], so the GEMM's output IS the staged weight and must equal ``ops.fq_per_group_int4_sym`` (itself bit-exact
+against the CPU oracle in tests/test_gpu_fake_quant.py) — for the forward tiles and for the transposed tiles."""
+import pytest
+import torch
+
+from oracle import fake_quant_oracle as fq
+from torchtune_amd import ops, qat
+from torchtune_amd.qat import Int8DynActInt4WeightQATLinear
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+BF = torch.bfloat16
+
+
+def _weight(N, K, seed):
+    g = torch.Generator().manual_seed(seed)
+    w = (torch.randn(N, K, generator=g) * 0.02).to(BF)
+    w[0, :64] = 0                 # an all-zero group: the scale falls back to eps
+    w[1, :32] = 7.5 * 0.01        # exact grid points
+    w[2] = -w[2].abs()            # one-signed rows
+    return w
+
+
+def _one_hot(M, K):
+    x = torch.zeros(M, K, dtype=BF, device=DEV)
+    x[torch.arange(M, device=DEV), torch.arange(M, device=DEV) % K] = 1.0
+    return x
+
+
+@pytest.mark.parametrize("N,K,g", [(256, 512, 32), (192, 448, 64), (320, 1024, 128), (128, 768, 256)])
+@pytest.mark.parametrize("scales", [torch.float32, torch.bfloat16])
+def test_staged_fake_quantised_weight_is_bit_exact_in_both_layouts(N, K, g, scales):
+    w = _weight(N, K, seed=N + K + g)
+    want, want_scale = ops.fq_per_group_int4_sym(w.to(DEV), g, qparam_dtype=scales)
+    ref, ref_scale = fq.fq_per_group_int4_sym(w, g) if scales == torch.float32 else (None, None)
+    if ref is not None:  # the row-major kernel against the oracle, for completeness of the chain
+        assert torch.equal(want.cpu().view(torch.int16), ref.view(torch.int16)) and torch.equal(want_scale.cpu(), ref_scale)
+    tf, tb, scale = ops.fq_per_group_int4_sym_tiled(w.to(DEV), g, qparam_dtype=scales)
+    assert torch.equal(scale, want_scale)
+    M = max(K, N)
+    y = ops.tiled_linear(_one_hot(M, K), tf, N)            # row m = column m % K of fq(W)
+    assert torch.equal(y[:K].view(torch.int16), want.t().contiguous().view(torch.int16))
+    gx = ops.tiled_linear(_one_hot(M, N), tb, K)           # row m = row m % N of fq(W)
+    assert torch.equal(gx[:N].view(torch.int16), want.view(torch.int16))
+    only_f = ops.fq_per_group_int4_sym_tiled(w.to(DEV), g, backward=False, want_scale=False, qparam_dtype=scales)
+    assert only_f[1] is None and only_f[2] is None and torch.equal(only_f[0], tf)
+
+
+def test_unsupported_group_size_is_refused():
+    w = _weight(128, 512, 1).to(DEV)
+    with pytest.raises(ValueError):
+        ops.fq_per_group_int4_sym_tiled(w, 16)
+
+
+@pytest.mark.parametrize("bias", [False, True])
+def test_qat_linear_on_the_tiled_gemm_vs_oracle_and_vs_default_path(bias, monkeypatch):
+    gen = torch.Generator().manual_seed(5)
+    N, K, M, g = 320, 512, 2048 + 19, 32
+    w = (torch.randn(N, K, generator=gen) * 0.02).to(BF)
+    b = (torch.randn(N, generator=gen) * 0.1).to(BF) if bias else None
+    x = torch.randn(M, K, generator=gen).to(BF)
+
+    def run(tiled):
+        monkeypatch.setattr(qat, "TILED_GEMM", tiled)
+        lin = Int8DynActInt4WeightQATLinear(K, N, bias=bias, device=DEV, groupsize=g, precision=BF)
+        with torch.no_grad():
+            lin.weight.copy_(w)
+            if bias:
+                lin.bias.copy_(b)
+        xd = x.to(DEV).requires_grad_()
+        y = lin(xd)
+        (y.float() ** 2).sum().backward()
+        return y.detach(), xd.grad, lin.weight.grad, (lin.bias.grad if bias else None), lin.weight_fake_quantizer.scale
+
+    y1, gx1, gw1, gb1, s1 = run(True)
+    y0, gx0, gw0, gb0, s0 = run(False)
+    assert torch.equal(s1, s0)
+    torch.testing.assert_close(y1.float(), y0.float(), rtol=1e-2, atol=2e-3)
+    torch.testing.assert_close(gx1.float(), gx0.float(), rtol=1e-2, atol=1e-2)
+    torch.testing.assert_close(gw1.float(), gw0.float(), rtol=2e-2, atol=2e-2 * float(gw0.float().abs().max()))
+    if bias:
+        torch.testing.assert_close(gb1.float(), gb0.float(), rtol=1e-2, atol=1e-2 * float(gb0.float().abs().max()))
+    # the CPU oracle (the reference's op sequence)
+    xo, wo = x.clone().requires_grad_(), w.clone().requires_grad_()
+    yo = fq.fake_quantized_linear(xo, wo, g)
+    if bias:
+        yo = yo + b
+    (yo.float() ** 2).sum().backward()
+    torch.testing.assert_close(y1.cpu().float(), yo.detach().float(), rtol=1e-2, atol=1e-2)
+    gxo = xo.grad.float()
+    torch.testing.assert_close(gx1.cpu().float(), gxo, rtol=1e-2, atol=1e-2 * max(1.0, float(gxo.abs().max()) / 8))
+    gwo = wo.grad.float()
+    torch.testing.assert_close(gw1.cpu().float(), gwo, rtol=2e-2, atol=2e-2 * float(gwo.abs().max()))

@@ -153,6 +153,109 @@ __global__ __launch_bounds__(256) void nf4_expand_tiled_transposed_kernel(const 
 }
 
 // ---------------------------------------------------------------------------------------------------------------------
+// Per-group symmetric int4 fake quantisation of a bf16 weight [N, K] (FakeQuantizer.forward of the weight in
+// FakeQuantizedLinear, torchao; same arithmetic, bit for bit, as fq_per_group_kernel in fake_quant.hip) written straight
+// into the tiled layout the GEMM reads, for the forward (tiles of fq(W)) and / or the grad-input (tiles of fq(W)^T), so that
+// the row-major fq(W) never exists.  A workgroup takes 32 rows x 256 columns; a thread 32 consecutive columns of one row
+// (t = tid % 8, row = tid / 8), so the lanes of a group of up to 256 elements are neighbours.  Both outputs are staged in
+// LDS in tile order and leave as 1 KiB pieces.
+// ---------------------------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void fq_int4_sym_tiled_kernel(const uint16_t* __restrict__ w, int N, int K, int threads_per_group,
+                                                                char* __restrict__ tiled_fwd, char* __restrict__ tiled_bwd,
+                                                                float* __restrict__ scale_out, int groups_per_row, bool qp_bf16, float eps) {
+  constexpr int kPieceF = 1040;  // forward staging: piece pitch, 16 bytes of padding spread the 16-byte writes over the banks
+  constexpr int kPitchB = 80;    // backward staging: bytes per column k (32 rows x 2 bytes + padding)
+  __shared__ __attribute__((aligned(16))) char smf[16 * kPieceF];
+  __shared__ __attribute__((aligned(16))) char smb[256 * kPitchB];
+  const int tid = threadIdx.x;
+  const int t8 = tid & 7, r = tid >> 3;
+  const int n = 32 * blockIdx.x + r;
+  const int t = 8 * blockIdx.y + t8;  // 32-wide step along K
+  const int nk = K >> 5;
+  const bool live = t < nk;
+  float v[32];
+  if (live) {
+    const u32x4_t* src = reinterpret_cast<const u32x4_t*>(w + (int64_t)n * K + 32 * t);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const u32x4_t raw = src[q];
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {
+        v[8 * q + 2 * d] = bits_f32(raw[d] << 16);
+        v[8 * q + 2 * d + 1] = bits_f32(raw[d] & 0xffff0000u);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < 32; ++e) v[e] = 0.f;
+  }
+  // a thread holds 32 elements; a group is 32, 64, 128 or 256 elements = 1, 2, 4 or 8 neighbouring threads of a row
+  uint32_t o[16];
+  {
+    float mn = 0.f, mx = 0.f;
+#pragma unroll
+    for (int e = 0; e < 32; ++e) {
+      mn = fminf(mn, v[e]);
+      mx = fmaxf(mx, v[e]);
+    }
+    for (int off = 1; off < threads_per_group; off <<= 1) {
+      mn = fminf(mn, __shfl_xor(mn, off, kWave));
+      mx = fmaxf(mx, __shfl_xor(mx, off, kWave));
+    }
+    const float amax = fmaxf(-mn, mx);
+    float scale = amax / 7.5f;
+    scale = scale > eps ? scale : eps;
+    if (qp_bf16) scale = round_to_bf16(scale);  // the rounded scale quantises and dequantises
+    const float inv = 1.0f / scale;
+    if (live && scale_out && (t8 & (threads_per_group - 1)) == 0) scale_out[(int64_t)n * groups_per_row + t / threads_per_group] = scale;
+#pragma unroll
+    for (int e = 0; e < 32; e += 2) {
+      float q2[2];
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        float tq = __builtin_rintf(v[e + h] * inv);
+        tq = tq < -8.0f ? -8.0f : (tq > 7.0f ? 7.0f : tq);
+        q2[h] = (float)(int)tq;  // through the integer grid: rint(-0.3) = -0.0 must dequantise to +0.0
+      }
+      o[e >> 1] = pack_bf16x2(q2[0] * scale, q2[1] * scale);
+    }
+  }
+  // ---- stage: forward piece t8 of row block r / 16, lane (r % 16) + 16 g4; backward column 32 t8 + j, row r
+  if (tiled_fwd) {
+#pragma unroll
+    for (int g4 = 0; g4 < 4; ++g4)
+      *reinterpret_cast<u32x4_t*>(smf + ((r >> 4) * 8 + t8) * kPieceF + (16 * g4 + (r & 15)) * 16) =
+          u32x4_t{o[4 * g4], o[4 * g4 + 1], o[4 * g4 + 2], o[4 * g4 + 3]};
+  }
+  if (tiled_bwd) {
+#pragma unroll
+    for (int j = 0; j < 32; ++j)
+      *reinterpret_cast<uint16_t*>(smb + (32 * t8 + j) * kPitchB + 2 * r) = (uint16_t)(o[j >> 1] >> (16 * (j & 1)));
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int idx = tid + 256 * i;
+    const int p = idx >> 6, l = idx & 63;  // 16 pieces of 64 lanes each
+    if (tiled_fwd) {
+      const int tp = 8 * blockIdx.y + (p & 7);
+      if (tp < nk) {
+        const u32x4_t val = *reinterpret_cast<const u32x4_t*>(smf + p * kPieceF + l * 16);
+        const int T = 2 * blockIdx.x + (p >> 3);
+        *reinterpret_cast<u32x4_t*>(tiled_fwd + ((int64_t)T * nk + tp) * 1024 + l * 16) = val;
+      }
+    }
+    if (tiled_bwd) {
+      const int Tk = 16 * blockIdx.y + p;  // block of 16 columns k
+      if (16 * Tk < K) {
+        const u32x4_t val = *reinterpret_cast<const u32x4_t*>(smb + (16 * p + (l & 15)) * kPitchB + 16 * (l >> 4));
+        *reinterpret_cast<u32x4_t*>(tiled_bwd + ((int64_t)Tk * (N >> 5) + blockIdx.x) * 1024 + l * 16) = val;
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
 struct DenseSeg {
   const uint16_t* X;  // [M, Kc] bf16 activations of one segment of the contraction
   int Kc;
@@ -656,3 +759,49 @@ int run_gemm_dense_group_dx(const GroupDx& d, const void* gh_cat, void* gx, void
 }
 
 }  // namespace ttamd
+
+using namespace ttamd;
+
+extern "C" size_t ttamd_tiled_weight_bytes(int64_t N, int64_t K) { return N > 0 && K > 0 ? (size_t)N * (size_t)K * 2 : 0; }
+
+extern "C" int ttamd_fq_per_group_int4_sym_tiled_bf16(const void* w, int64_t N, int64_t K, int group_size, int qparam_dtype, float eps,
+                                                      void* tiled_fwd, void* tiled_bwd, float* scale, void* stream) {
+  TT_REQUIRE(w && aligned16(w) && (tiled_fwd || tiled_bwd), "fq_per_group_int4_sym_tiled: w must be non-null and 16-byte aligned, one output given");
+  TT_REQUIRE((!tiled_fwd || aligned16(tiled_fwd)) && (!tiled_bwd || aligned16(tiled_bwd)), "fq_per_group_int4_sym_tiled: outputs must be 16-byte aligned");
+  TT_REQUIRE(N > 0 && K > 0 && N % 64 == 0 && K % 64 == 0 && N < (1 << 30) && K < (1 << 30),
+             "fq_per_group_int4_sym_tiled: N (%lld) and K (%lld) must be positive multiples of 64", (long long)N, (long long)K);
+  TT_REQUIRE(qparam_dtype == TTAMD_BF16 || qparam_dtype == TTAMD_F32, "fq_per_group_int4_sym_tiled: unknown qparam dtype code %d", qparam_dtype);
+  TT_REQUIRE(eps > 0.0f, "fq_per_group_int4_sym_tiled: eps must be positive");
+  if (!(group_size == 32 || group_size == 64 || group_size == 128 || group_size == 256) || K % group_size != 0)
+    return fail(TTAMD_EUNSUPPORTED, "fq_per_group_int4_sym_tiled: group size %d (serves 32, 64, 128, 256 dividing K)", group_size);
+  const int64_t gy = (K + 255) / 256;
+  TT_REQUIRE(gy < 65536, "fq_per_group_int4_sym_tiled: K too large for one launch");
+  fq_int4_sym_tiled_kernel<<<dim3((unsigned)(N / 32), (unsigned)gy), dim3(256), 0, reinterpret_cast<hipStream_t>(stream)>>>(
+      reinterpret_cast<const uint16_t*>(w), (int)N, (int)K, group_size / 32, reinterpret_cast<char*>(tiled_fwd),
+      reinterpret_cast<char*>(tiled_bwd), scale, (int)(K / group_size), qparam_dtype == TTAMD_BF16, eps);
+  return check_launch("fq_per_group_int4_sym_tiled");
+}
+
+extern "C" int ttamd_tiled_linear_bf16(const void* x, const void* tiled_weight, const void* bias, void* y, int64_t M, int64_t n_out,
+                                       int64_t k_contract, void* stream) {
+  TT_REQUIRE(x && tiled_weight && y && aligned16(x) && aligned16(tiled_weight) && aligned16(y), "tiled_linear: pointers must be non-null and 16-byte aligned");
+  TT_REQUIRE(bias == nullptr || (reinterpret_cast<uintptr_t>(bias) & 7u) == 0, "tiled_linear: bias must be 8-byte aligned");
+  TT_REQUIRE(M > 0 && n_out > 0 && k_contract > 0 && n_out % 64 == 0 && k_contract % 64 == 0,
+             "tiled_linear: n_out (%lld) and k_contract (%lld) must be positive multiples of 64", (long long)n_out, (long long)k_contract);
+  if (!(M * k_contract * 2 < (int64_t(1) << 32) && k_contract * 2 * 256 < (int64_t(1) << 32) && M < (1 << 30) && n_out < (1 << 30)))
+    return fail(TTAMD_EUNSUPPORTED, "tiled_linear: operands too large for 32-bit offsets (M=%lld k=%lld)", (long long)M, (long long)k_contract);
+  DenseArgs g = {};
+  g.nseg = g.nout = 1;
+  g.nad = 0;
+  g.seg[0].X = reinterpret_cast<const uint16_t*>(x);
+  g.seg[0].Kc = (int)k_contract;
+  g.out[0].C = reinterpret_cast<uint16_t*>(y);
+  g.out[0].bias = reinterpret_cast<const uint16_t*>(bias);
+  g.out[0].n_begin = 0;
+  g.out[0].width = (int)n_out;
+  g.Wt = reinterpret_cast<const char*>(tiled_weight);
+  g.M = (int)M; g.Nout = (int)n_out; g.Kc = (int)k_contract;
+  g.lw_row_major = 1;
+  g.ldlx = 0;
+  return launch_dense(g, reinterpret_cast<hipStream_t>(stream));
+}

@@ -568,6 +568,63 @@ def fq_per_group_int4_sym(w: torch.Tensor, group_size: int, want_scale: bool = T
     return out, scale
 
 
+def tiled_weight_shape_ok(N: int, K: int, group_size: int) -> bool:
+    """Shapes ``fq_per_group_int4_sym_tiled`` / ``tiled_linear`` serve."""
+    return N % 64 == 0 and K % 64 == 0 and group_size in (32, 64, 128, 256) and K % group_size == 0
+
+
+def fq_per_group_int4_sym_tiled(w: torch.Tensor, group_size: int, forward: bool = True, backward: bool = True,
+                                want_scale: bool = True, qparam_dtype: torch.dtype = torch.float32, eps: Optional[float] = None):
+    """bf16 w [N, K] -> (fq(w) in the tiled layout ``tiled_linear`` reads for ``x @ fq(w).T`` | None, fq(w).T in that layout
+    for ``gy @ fq(w)`` | None, scale fp32 [N, K/g] | None): the values of ``fq_per_group_int4_sym``, never written row-major."""
+    _need_gpu(w, "fq_per_group_int4_sym_tiled")
+    if w.dtype != torch.bfloat16 or w.dim() != 2:
+        raise TypeError("fq_per_group_int4_sym_tiled: w must be a 2-D bfloat16 tensor")
+    qcode = _code(qparam_dtype, "fq_per_group_int4_sym_tiled (qparams)")
+    wc = w.contiguous()
+    N, K = wc.shape
+    if not tiled_weight_shape_ok(N, K, group_size):
+        raise ValueError(f"fq_per_group_int4_sym_tiled: N ({N}) and K ({K}) must be multiples of 64, group_size ({group_size}) one of 32/64/128/256 dividing K")
+    tf = torch.empty(N * K, dtype=torch.bfloat16, device=w.device) if forward else None
+    tb = torch.empty(N * K, dtype=torch.bfloat16, device=w.device) if backward else None
+    scale = torch.empty(N, K // group_size, dtype=torch.float32, device=w.device) if want_scale else None
+    lib = _lib.load()
+    with torch.cuda.device(w.device):
+        events = _fq_timer(f"per_group_tiled{int(forward) + int(backward)}", N, K, group_size, 2) if _fq_timer is not None else None
+        if events:
+            events[0].record()
+        rc = lib.ttamd_fq_per_group_int4_sym_tiled_bf16(wc.data_ptr(), N, K, group_size, qcode,
+                                                        float(torch.finfo(torch.float32).eps) if eps is None else float(eps),
+                                                        _ptr(tf), _ptr(tb), _ptr(scale), _stream(w))
+        if events:
+            events[1].record()
+    _lib.check(rc, "fq_per_group_int4_sym_tiled")
+    return tf, tb, scale
+
+
+def tiled_linear(x: torch.Tensor, tiled: torch.Tensor, n_out: int, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """y [M, n_out] = x [M, k] @ Wd.T (+ bias) for a bf16 weight ``Wd`` [n_out, k] held in the tiled layout."""
+    x = _bf16_2d(x, "tiled_linear")
+    M, K = x.shape
+    if tiled.dtype != torch.bfloat16 or tiled.numel() != n_out * K or not tiled.is_contiguous():
+        raise ValueError(f"tiled_linear: the tiled weight must be a contiguous bfloat16 tensor of {n_out} x {K} elements")
+    if bias is not None:
+        bias = bias.contiguous()
+        if bias.dtype != torch.bfloat16 or bias.numel() != n_out:
+            raise ValueError(f"tiled_linear: bias must be bfloat16 with {n_out} elements")
+    y = torch.empty(M, n_out, dtype=torch.bfloat16, device=x.device)
+    lib = _lib.load()
+    with torch.cuda.device(x.device):
+        events = _gemm_timer("tiled", M, n_out, K, 0) if _gemm_timer is not None else None
+        if events:
+            events[0].record()
+        rc = lib.ttamd_tiled_linear_bf16(x.data_ptr(), tiled.data_ptr(), _ptr(bias), y.data_ptr(), M, n_out, K, _stream(x))
+        if events:
+            events[1].record()
+    _lib.check(rc, "tiled_linear")
+    return y
+
+
 def quantize_per_group_int4(w: torch.Tensor, group_size: int, qparam_dtype: torch.dtype = torch.float32,
                             eps: Optional[float] = None):
     """w [rows, K] -> (int8 tensor of int4 values, scale fp32 [rows, K/g], zeros fp32 [rows, K/g])"""
