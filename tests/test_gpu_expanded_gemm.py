@@ -263,3 +263,33 @@ def test_group_without_transposed_copies_equals_group_with_them():
     h2, _ = ops.lora_group_fwd(x, without)
     gx2, _, _ = ops.lora_group_bwd(x, h2, without, gys)
     assert torch.equal(h1, h2) and torch.equal(gx1, gx2)
+
+
+SWEEP = [
+    # M, N, K, rank: shortest contractions (one and two 64-wide entries), ragged rows, widths off the 256 grid
+    (2048, 8192, 64, 8), (2048, 8192, 128, 16), (2049, 8192 + 192, 192, 8), (2304, 7424, 320, 32), (3000, 5568, 448, 16),
+    (8192, 2048, 256, 8), (4096, 4096, 1024, 16), (2048, 16384, 64, 0),
+]
+
+
+@pytest.mark.parametrize("M,N,K,r", SWEEP)
+def test_expanded_path_sweep_vs_fp32_matmul_of_the_dequantised_weight(M, N, K, r):
+    """Forward and (where the transposed shape is served too) grad-input over a sweep of shapes, against fp32 matmuls of
+    the dequantised weight — a parity statement because that dequantisation is bit-exact against the oracle
+    (tests/test_gpu_nf4.py) and the expanded copy is bit-exact against it (first tests of this file)."""
+    assert _expands(M, N, K)
+    W, sbs, qdata, bscal, dense, A, B, b, x, gy = _case(M, N, K, r, True, seed=M + 7 * N + K + r)
+    xd, gyd = x.to(DEV), gy.to(DEV)
+    h = ops.lora_hidden(xd, A.to(DEV)) if r else None
+    y = ops.nf4_lora_linear_fwd(xd, qdata, bscal, N, h, B.to(DEV) if r else None, 1.5, b.to(DEV))
+    want = xd.float() @ dense.float().T + b.to(DEV).float()
+    if r:
+        want = want + 1.5 * h.float() @ B.to(DEV).float().T
+    torch.testing.assert_close(y.float(), want, rtol=1e-2, atol=1e-2)
+    if _expands(M, K, N):
+        gh = ops.lora_bwd(gyd, xd, h, B.to(DEV), 1.5)[0] if r else None
+        gx = ops.nf4_linear_bwd_dx(gyd, qdata, bscal, K, gh, A.to(DEV) if r else None, transposed=None)
+        want = gyd.float() @ dense.float()
+        if r:
+            want = want + gh.float() @ A.to(DEV).float()
+        torch.testing.assert_close(gx.float(), want, rtol=1e-2, atol=1e-2 * max(1.0, float(want.abs().max()) / 8))
