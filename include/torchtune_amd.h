@@ -232,7 +232,9 @@ int ttamd_nf4_linear_bwd_dx_bf16(const void* gy, const uint8_t* quantized_data, 
  * work, F.linear(x, weight.to(dtype)) (torchao linear_nf4, reached from torchtune/modules/peft/lora.py:138), for the
  * token counts at which the fused kernel's per-tile expansion costs more than one pass of the expansion kernel.
  * ttamd_nf4_gemm_workspace_bytes reports those bytes; passing less (or NULL) keeps the fused kernel.  The expanded
- * values are the bits ttamd_nf4_dequantize writes.
+ * values are the bits ttamd_nf4_dequantize writes.  The grad-input takes this path with or without the transposed
+ * copies (without them W^T is expanded from quantized_data / block_scalers themselves, at the same speed), so a
+ * caller that only ever runs many-token calls need not build them.
  */
 size_t ttamd_nf4_gemm_workspace_bytes(int64_t M, int64_t n_out, int64_t k_contract);
 /* 1 when those bytes are the expanded weight of the many-token path, 0 when they are slices (or none) */

@@ -466,3 +466,36 @@ def test_to_nf4_preconditions_are_the_reference_asserts():
         to_nf4(torch.zeros(512, 512, dtype=torch.bfloat16).t())
     with pytest.raises(AssertionError, match="divisible by scaler_block_size"):
         to_nf4(torch.zeros(64, 64, dtype=torch.bfloat16))  # 64 blocks, scaler blocks of 256
+
+
+def test_tiled_entry_points_validate_their_arguments_on_the_host():
+    """``ttamd_tiled_linear_bf16`` / ``ttamd_fq_per_group_int4_sym_tiled_bf16`` refuse bad arguments before any launch
+    (no GPU needed): null or misaligned pointers, dimensions that are not multiples of 64, group sizes the kernel does
+    not serve (``TTAMD_EUNSUPPORTED``), a non-positive eps."""
+    import ctypes
+
+    from torchtune_amd import _lib
+
+    lib = _lib.load()
+    buf = (ctypes.c_char * 4096)()
+    p = ctypes.addressof(buf)
+    p = (p + 15) & ~15
+    assert lib.ttamd_tiled_weight_bytes(128, 256) == 2 * 128 * 256 and lib.ttamd_tiled_weight_bytes(0, 256) == 0
+    EINVAL, EUNSUPPORTED = -1, -2
+    codes = {lib.ttamd_tiled_linear_bf16(None, p, None, p, 64, 64, 64, None),
+             lib.ttamd_tiled_linear_bf16(p, p, None, p + 2, 64, 64, 64, None),
+             lib.ttamd_tiled_linear_bf16(p, p, None, p, 64, 96, 64, None),
+             lib.ttamd_tiled_linear_bf16(p, p, None, p, 64, 64, 32, None),
+             lib.ttamd_tiled_linear_bf16(p, p, None, p, 0, 64, 64, None)}
+    assert codes == {EINVAL}, codes
+    assert b"tiled_linear" in lib.ttamd_last_error()
+    F32 = 1  # TTAMD_F32
+    q = lib.ttamd_fq_per_group_int4_sym_tiled_bf16
+    assert q(None, 64, 64, 32, F32, 1e-7, p, None, None, None) == EINVAL
+    assert q(p, 64, 64, 32, F32, 1e-7, None, None, None, None) == EINVAL          # no output at all
+    assert q(p, 64, 96, 32, F32, 1e-7, p, None, None, None) == EINVAL             # K not a multiple of 64
+    assert q(p, 64, 64, 32, F32, 0.0, p, None, None, None) == EINVAL              # eps
+    assert q(p, 64, 64, 32, 7, 1e-7, p, None, None, None) == EINVAL               # qparam dtype code
+    assert q(p, 64, 64, 16, F32, 1e-7, p, None, None, None) == EUNSUPPORTED       # group size
+    assert q(p, 64, 192, 128, F32, 1e-7, p, None, None, None) == EUNSUPPORTED     # group does not divide K
+    assert b"group size" in lib.ttamd_last_error()
