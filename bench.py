@@ -83,7 +83,8 @@ class GemmTimer:
         Ns = tuple(N) if isinstance(N, (list, tuple)) else (N,)
         ranks = tuple(rank) if isinstance(rank, (list, tuple)) else (rank,) * len(Ns)
         fwd = kind.startswith("fwd")
-        if kind == "tiled":  # the plain GEMM on a bf16 weight already in tile order (QAT): y [M, N] = x [M, K] . Wd^T
+        if kind in ("tiled", "tn"):  # QAT: the plain GEMM on a bf16 weight already in tile order, y [M, N] = x [M, K] . Wd^T,
+            # and the weight gradient c [N, K] = a [M, N]^T . b [M, K]
             key = (kind, M, Ns[0], K)
             seen = self.counts.get(key, [0, 2.0 * M * Ns[0] * K, 2.0 * (M * K + M * Ns[0] + Ns[0] * K), 1])
             self.counts[key] = [seen[0] + 1] + seen[1:]
@@ -620,7 +621,8 @@ def main() -> int:
         if timer.counts:
             g_launches, g_timed, g_ms, g_flops, g_shapes = timer.summary()
             own_gemm = {"kernel": "nf4_gemm_dense_kernel on weights fake-quantised straight into its tile order (forward and "
-                                  "grad-input of every linear; the weight gradients run on the vendor library)",
+                                  "grad-input of every linear) and gemm_tn_kernel (weight gradients; those of the 1024-wide k / v "
+                                  "projections run on the vendor library)",
                         "launches": g_launches, "tflops": round(g_flops / g_ms / 1e9, 1), "frac_of_bf16_mfma_peak":
                         round(g_flops / g_ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4), "gemm_ms_per_step": round(g_ms / args.steps, 2),
                         "per_shape": g_shapes}
@@ -653,7 +655,7 @@ def main() -> int:
             "roofline": {
                 "bound": "hbm",
                 "kernel": "fq_per_token_regs_kernel + fq_int4_sym_tiled_kernel / fq_per_group_kernel (the fake-quant launches of "
-                          "the step; forward and grad-input matmuls: see own_gemm, weight gradients: vendor library)",
+                          "the step; the matmuls: see own_gemm)",
                 "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBPS,
                 "unit": "GB/s",

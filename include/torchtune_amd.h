@@ -446,6 +446,14 @@ int ttamd_quantize_per_group_uint4_conv(const void* w, int dtype, int64_t rows, 
  * values Wd[16 T + l % 16][32 t + 8 (l / 16) .. + 7] (the operand order of v_mfma_f32_16x16x32_bf16).
  */
 size_t ttamd_tiled_weight_bytes(int64_t N, int64_t K);
+/*
+ * The third matmul of that layer's training step, the weight gradient c[N, K] = a[M, N]^T . b[M, K] (a = gy, b = fq(x),
+ * both bf16 row-major as autograd hands them over; c bf16): both operands are transposed on their way through LDS.
+ * M a multiple of 32, N and K multiples of 256 (ttamd_gemm_tn_applies: 1 / 0; otherwise TTAMD_EUNSUPPORTED).  Meant for
+ * shapes with a few hundred output tiles of 256 x 256 or more.
+ */
+int ttamd_gemm_tn_applies(int64_t M, int64_t N, int64_t K);
+int ttamd_gemm_tn_bf16(const void* a, const void* b, void* c, int64_t M, int64_t N, int64_t K, void* stream);
 int ttamd_fq_per_group_int4_sym_tiled_bf16(const void* w, int64_t N, int64_t K, int group_size, int qparam_dtype, float eps,
                                            void* tiled_fwd, void* tiled_bwd, float* scale, void* stream);
 int ttamd_tiled_linear_bf16(const void* x, const void* tiled_weight, const void* bias, void* y, int64_t M, int64_t n_out,

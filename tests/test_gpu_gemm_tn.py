@@ -1,0 +1,78 @@
+"""GPU parity of the weight-gradient GEMM ``c = a.T @ b`` (both operands transposed on their way through LDS) and a
+determinism check of the two-waves-per-SIMD GEMM kernels.
+
+Oracle: the product in fp32 / fp64 on the same bf16 inputs (the reference computes this matmul in bf16 with fp32
+accumulation as well); tolerance rtol 1e-2 / atol 1e-2 scaled with the magnitude of the result, as for the other GEMMs.
+With one-hot rows in ``a`` the result is a row of ``b`` exactly (one product 1 * b[m][k], zeros elsewhere), which pins the
+operand transposition and the swizzled LDS layout bit for bit."""
+import pytest
+import torch
+
+from torchtune_amd import _lib, ops
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+BF = torch.bfloat16
+
+
+def test_one_hot_rows_select_rows_of_b_bit_for_bit():
+    M, N, K = 512, 256, 512
+    g = torch.Generator().manual_seed(0)
+    b = torch.randn(M, K, generator=g).to(BF).to(DEV)
+    a = torch.zeros(M, N, dtype=BF, device=DEV)
+    perm = torch.randperm(M, generator=g)[:N].to(DEV)          # column n of a is one-hot at row perm[n]
+    a[perm, torch.arange(N, device=DEV)] = 1.0
+    c = ops.gemm_tn(a, b)
+    assert torch.equal(c.view(torch.int16), b[perm].contiguous().view(torch.int16))
+    # and the other way round: one-hot columns of b select columns of a
+    a2 = torch.randn(M, N, generator=g).to(BF).to(DEV)
+    b2 = torch.zeros(M, K, dtype=BF, device=DEV)
+    perm2 = torch.randperm(M, generator=g)[:K].to(DEV)
+    b2[perm2, torch.arange(K, device=DEV)] = 1.0
+    c2 = ops.gemm_tn(a2, b2)
+    assert torch.equal(c2.view(torch.int16), a2[perm2].t().contiguous().view(torch.int16))
+
+
+@pytest.mark.parametrize("M,N,K", [(32, 256, 256), (96, 256, 512), (1024, 512, 256), (4096, 1024, 768), (8192, 4096, 4096), (2080, 1792, 1280)])
+def test_against_fp32_matmul(M, N, K):
+    assert ops.gemm_tn_applies(M, N, K)
+    g = torch.Generator().manual_seed(M + N + K)
+    a = torch.randn(M, N, generator=g).to(BF).to(DEV)
+    b = torch.randn(M, K, generator=g).to(BF).to(DEV)
+    c = ops.gemm_tn(a, b)
+    want = a.float().t() @ b.float()
+    scale = max(1.0, float(want.abs().max()) / 8)
+    torch.testing.assert_close(c.float(), want, rtol=1e-2, atol=1e-2 * scale)
+
+
+def test_unsupported_shapes_are_refused():
+    lib = _lib.load()
+    assert not ops.gemm_tn_applies(100, 256, 256) and not ops.gemm_tn_applies(64, 320, 256) and not ops.gemm_tn_applies(64, 256, 64)
+    a = torch.zeros(64, 320, dtype=BF, device=DEV)
+    b = torch.zeros(64, 256, dtype=BF, device=DEV)
+    with pytest.raises(Exception):
+        ops.gemm_tn(a, b)
+    assert b"gemm_tn" in lib.ttamd_last_error()
+
+
+def test_two_waves_per_simd_kernels_are_deterministic():
+    """The same launch twenty times over: identical bits every time, for the expanded-weight GEMM (forward of an NF4
+    layer), the tiled GEMM and the transposing GEMM.  The waves of these kernels hand LDS stages to each other across
+    workgroup barriers while loads are in flight; a read that raced with a later load would show up here."""
+    M, N, K = 4096, 4096, 2048
+    g = torch.Generator().manual_seed(3)
+    W = (torch.randn(N, K, generator=g) * 0.02).to(BF).to(DEV)
+    qdata, qscal, qfac, mean = ops.nf4_quantize(W, 64, 256)
+    bscal = ops.nf4_block_scalers(qscal, qfac, mean, 256)
+    x = torch.randn(M, K, generator=g).to(BF).to(DEV)
+    gy = torch.randn(M, N, generator=g).to(BF).to(DEV)
+    tf, tb, _ = ops.fq_per_group_int4_sym_tiled(W, 32)
+    first = None
+    for _ in range(20):
+        out = (ops.nf4_lora_linear_fwd(x, qdata, bscal, N), ops.nf4_linear_bwd_dx(gy, qdata, bscal, K, transposed=None),
+               ops.tiled_linear(x, tf, N), ops.tiled_linear(gy, tb, K), ops.gemm_tn(gy, x))
+        if first is None:
+            first = out
+        else:
+            for a, b in zip(first, out):
+                assert torch.equal(a, b)

@@ -96,6 +96,8 @@ SIGNATURES = {
     "ttamd_nf4_group_bwd_dx_workspace_bytes": (_size, [_c_void_p, _int, _i64, _i64]),
     "ttamd_nf4_group_bwd_dx_ws_bf16": (_int, [_c_void_p, _int, _c_void_p, _c_void_p, _i64, _i64, _c_void_p, _size, _c_void_p]),
     "ttamd_tiled_weight_bytes": (_size, [_i64, _i64]),
+    "ttamd_gemm_tn_applies": (_int, [_i64, _i64, _i64]),
+    "ttamd_gemm_tn_bf16": (_int, [_c_void_p, _c_void_p, _c_void_p, _i64, _i64, _i64, _c_void_p]),
     "ttamd_fq_per_group_int4_sym_tiled_bf16": (_int, [_c_void_p, _i64, _i64, _int, _int, _f32, _c_void_p, _c_void_p, _c_void_p, _c_void_p]),
     "ttamd_tiled_linear_bf16": (_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _i64, _i64, _i64, _c_void_p]),
     "ttamd_fq_per_token_int8_asym": (_int, [_c_void_p, _int, _i64, _i64, _int, _c_void_p, _c_void_p, _c_void_p, _c_void_p]),

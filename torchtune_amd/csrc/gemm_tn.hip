@@ -1,0 +1,249 @@
+// Weight gradient of a linear layer over many tokens: C[N, K] = A[M, N]^T . B[M, K] for bf16 A = gy and B = x as they lie in
+// memory (rows = tokens), the third matmul of FakeQuantizedLinear's training step (autograd of F.linear(fq(x), fq(W)),
+// torchao; reached from recipes/qat_single_device.py:378-386).  The contraction runs over the rows of both operands, so
+// neither has the 8 consecutive contraction elements per lane that v_mfma_f32_16x16x32_bf16 wants: the LDS transposes them
+// (ds_read_b64_tr_b16 returns to lane i of a 16-lane group column i of the four rows the group points at).
+//
+// Skeleton of nf4_gemm_dense.hip: workgroup = 8 waves (two per SIMD), tile 256 x 256 of C, step = 32 rows of A and B, both
+// tiles (32 rows x 512 bytes each) into a ring of four LDS stages by direct-to-LDS loads; wave (wm, wn) owns rows
+// [128 wm, +128) x columns [64 wn, +64) of the tile (128 accumulators per lane); the two waves of a SIMD run half a step
+// apart, one in its MFMA part while the other requests loads and reads operands, swapping at workgroup barriers.
+// LDS layout of a stage: row r of the 32 at r * 512, its 16-byte chunk c in slot c ^ (2 (r % 4)) - applied on the
+// global-address side of the loads - so that the four rows a 16-lane group reads together fall on disjoint banks.
+#include "common.h"
+#include "nf4_math.h"
+
+namespace ttamd {
+namespace {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  bf16x2_t v;
+  v.x = (__bf16)lo;
+  v.y = (__bf16)hi;
+  return __builtin_bit_cast(uint32_t, v);
+}
+
+#define TT_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
+
+struct TnArgs {
+  const uint16_t* A;  // [M, N] bf16
+  const uint16_t* B;  // [M, K] bf16
+  uint16_t* C;        // [N, K] bf16
+  int M, N, K;
+  int tiles_n, tiles_k;
+};
+
+constexpr int kTnStage = 32768;  // 32 rows x 512 bytes of A, then the same of B
+constexpr int kTnLds = 4 * kTnStage;
+constexpr int kLgkmMax = 15;  // the counter field of s_waitcnt holds 4 bits: waiting for fewer outstanding reads is always safe
+
+__global__ __launch_bounds__(512) void gemm_tn_kernel(const TnArgs g) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  constexpr int MT = 8, NT = 4;  // 16 x 16 MFMA tiles per wave: MT along the rows of C (columns of A), NT along its columns
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wv >> 2, wn = wv & 3;
+  const int l15 = lane & 15, g4 = lane >> 4;
+
+  int tile_n, tile_k;
+  {
+    // workgroup ids are dealt round-robin to the 8 XCDs: every XCD gets a band of row tiles and walks it column by column
+    const int id = blockIdx.x;
+    if ((g.tiles_n & 7) == 0) {
+      const int xcd = id & 7, slot = id >> 3, band = g.tiles_n >> 3;
+      tile_n = xcd * band + slot % band;
+      tile_k = slot / band;
+    } else {
+      tile_n = id / g.tiles_k;
+      tile_k = id % g.tiles_k;
+    }
+  }
+  const int n0 = tile_n * 256, k0 = tile_k * 256;
+  const int nk = g.M >> 5;  // steps of 32 rows
+
+  // ---- loads: per step and wave two instructions for A (rows 4 wv .. + 3 of the 32, two rows of 512 bytes each) and two
+  //      for B; lane l of an instruction fetches chunk (l % 32) ^ (2 (row % 4)) of row l / 32 of its pair
+  uint32_t a_off[2], b_off[2];
+#pragma unroll
+  for (int d = 0; d < 2; ++d) {
+    const int rl = 4 * wv + 2 * d + (lane >> 5);
+    const int chunk = (lane & 31) ^ ((rl & 3) << 1);
+    a_off[d] = (uint32_t)rl * (uint32_t)g.N * 2u + (uint32_t)n0 * 2u + (uint32_t)chunk * 16u;
+    b_off[d] = (uint32_t)rl * (uint32_t)g.K * 2u + (uint32_t)k0 * 2u + (uint32_t)chunk * 16u;
+  }
+  auto dma16 = [&](uint32_t voff, const char* base, uint32_t lds, int imm) {
+    asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 ::"v"(voff), "s"(base), "s"(lds), "n"(imm) : "memory", "m0", "scc");
+  };
+  const uint32_t lds0 = (uint32_t)(uintptr_t)TT_LDS_PTR(smem);
+  auto issue = [&](int t) {
+    const int tk = t < nk ? t : nk - 1;
+    const char* ab = reinterpret_cast<const char*>(g.A) + (int64_t)tk * 32 * g.N * 2;
+    const char* bb = reinterpret_cast<const char*>(g.B) + (int64_t)tk * 32 * g.K * 2;
+    const uint32_t st = lds0 + (t & 3) * kTnStage + wv * 2048;
+    dma16(a_off[0], ab, st, 0);
+    dma16(a_off[1], ab, st, 1024);
+    dma16(b_off[0], bb, st, 16384);
+    dma16(b_off[1], bb, st, 16384 + 1024);
+  };
+
+  // ---- operand reads.  Lane (l15, g4) of ds_read_b64_tr_b16 points at row 8 g4 + l15 / 4 (+ 4 for the second half of the
+  //      operand), columns 4 (l15 % 4) .. + 3 of a 16-column group e, and receives column l15 of that group for rows
+  //      8 g4 .. + 3 (+ 4): with both halves the 8 contraction elements of an MFMA operand.  Group e of a row with
+  //      row % 4 = q sits at byte 32 (e ^ q) of the row.  A groups of this wave: 8 wm + i; B groups: 4 wn + j.
+  uint32_t ra[4], rb[4];
+  {
+    const int q = (l15 >> 2) & 3;
+    const uint32_t rowbase = (uint32_t)(8 * g4 + (l15 >> 2)) * 512u + 8u * (l15 & 3);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      ra[e] = lds0 + rowbase + 32u * (8 * wm) + 32u * (e ^ q);
+      rb[e] = lds0 + 16384u + rowbase + 32u * (4 * wn) + 32u * (e ^ q);
+    }
+  }
+  auto tr16 = [&](uint32_t addr) {
+    u32x2_t v;
+    asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(v) : "v"(addr) : "memory");
+    return v;
+  };
+
+  f32x4_t acc[NT][MT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j)
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) acc[j][i][v] = 0.f;
+
+  u32x2_t alo[MT], ahi[MT], blo[NT], bhi[NT];
+  auto read_step = [&](int t) {
+    const uint32_t st = (uint32_t)(t & 3) * kTnStage;
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+      blo[j] = tr16(rb[j] + st);
+      bhi[j] = tr16(rb[j] + st + 2048u);
+    }
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+      alo[i] = tr16(ra[i & 3] + st + 128u * (i >> 2));
+      ahi[i] = tr16(ra[i & 3] + st + 128u * (i >> 2) + 2048u);
+    }
+  };
+
+  // ---- pipeline, as in nf4_gemm_dense.hip: memory part M(t) / barrier / compute part C(t) / barrier, the waves with wm = 1
+  //      one barrier behind.  M(t) requests step t + 3 (four loads) and reads the operands of step t.  At the end of M(t) a
+  //      wave's own loads of step t + 1 must have landed (the other waves read them after the next barrier): they came
+  //      from M(t - 2), newer are the 4 + 4 loads of M(t - 1) and M(t).  The transposing reads are written in assembly, so
+  //      the wait for them is explicit too and names the registers it releases.
+  issue(0);
+  issue(1);
+  issue(2);
+  asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");  // step 0 landed everywhere
+  if (wm == 1) asm volatile("s_barrier" ::: "memory");
+  for (int t = 0; t < nk; ++t) {
+    issue(t + 3);
+    read_step(t);
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+      asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(blo[j]), "+v"(bhi[j]) : "n"(kLgkmMax < 2 * MT + 2 * (NT - 1 - j) ? kLgkmMax : 2 * MT + 2 * (NT - 1 - j)));
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+      asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(alo[i]), "+v"(ahi[i]) : "n"(kLgkmMax < 2 * (MT - 1 - i) ? kLgkmMax : 2 * (MT - 1 - i)));
+      const u32x4_t aop = {alo[i].x, alo[i].y, ahi[i].x, ahi[i].y};
+#pragma unroll
+      for (int j = 0; j < NT; ++j) {
+        const u32x4_t bop = {blo[j].x, blo[j].y, bhi[j].x, bhi[j].y};
+        acc[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, bop), __builtin_bit_cast(bf16x8_t, aop),
+                                                           acc[j][i], 0, 0, 0);
+      }
+    }
+    __builtin_amdgcn_s_setprio(0);
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_barrier" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  if (wm == 0) asm volatile("s_barrier" ::: "memory");
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the clamped requests of the last steps
+
+  // ---- epilogue: acc[j][i][v] = C[n][k], n = n0 + 128 wm + 16 i + l15, k = k0 + 64 wn + 16 j + 4 g4 + v.  Each wave
+  //      transposes its 128 x 64 band through LDS and writes whole 128-byte row segments.
+  __syncthreads();
+  {
+    char* band = smem + wv * 16384;  // 128 rows x 128 bytes
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int i = 0; i < MT; ++i) {
+        const int r = 16 * i + l15;
+        u32x2_t o;
+        o.x = pack_bf16x2(acc[j][i][0], acc[j][i][1]);
+        o.y = pack_bf16x2(acc[j][i][2], acc[j][i][3]);
+        *reinterpret_cast<u32x2_t*>(band + r * 128 + (((2 * j + (g4 >> 1)) ^ (r & 7)) << 4) + 8 * (g4 & 1)) = o;
+      }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const int c = lane & 7;
+    uint16_t* crow = g.C + k0 + wn * 64 + 8 * c;
+    const int nrow0 = n0 + 128 * wm;
+#pragma unroll 8
+    for (int t = 0; t < 16; ++t) {
+      const int r = 8 * t + (lane >> 3);
+      const u32x4_t v = *reinterpret_cast<const u32x4_t*>(band + r * 128 + ((c ^ (r & 7)) << 4));
+      *reinterpret_cast<u32x4_t*>(crow + (int64_t)(nrow0 + r) * g.K) = v;
+    }
+  }
+#endif
+}
+
+}  // namespace
+
+bool gemm_tn_applies(int64_t M, int64_t N, int64_t K) {
+  if (M < 32 || M % 32 != 0 || N <= 0 || K <= 0 || N % 256 != 0 || K % 256 != 0) return false;
+  // per-lane byte offsets inside the kernel are 32-bit: a step of 32 rows of either operand
+  return N * 2 * 32 < (int64_t(1) << 31) && K * 2 * 32 < (int64_t(1) << 31) && (N / 256) * (K / 256) < (int64_t(1) << 31);
+}
+
+}  // namespace ttamd
+
+using namespace ttamd;
+
+extern "C" int ttamd_gemm_tn_applies(int64_t M, int64_t N, int64_t K) { return gemm_tn_applies(M, N, K) ? 1 : 0; }
+
+extern "C" int ttamd_gemm_tn_bf16(const void* a, const void* b, void* c, int64_t M, int64_t N, int64_t K, void* stream) {
+  TT_REQUIRE(a && b && c && aligned16(a) && aligned16(b) && aligned16(c), "gemm_tn: pointers must be non-null and 16-byte aligned");
+  TT_REQUIRE(M > 0 && N > 0 && K > 0, "gemm_tn: bad shape M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
+  if (!gemm_tn_applies(M, N, K))
+    return fail(TTAMD_EUNSUPPORTED, "gemm_tn: M (%lld) must be a multiple of 32, N (%lld) and K (%lld) multiples of 256", (long long)M,
+                (long long)N, (long long)K);
+  TnArgs g;
+  g.A = reinterpret_cast<const uint16_t*>(a);
+  g.B = reinterpret_cast<const uint16_t*>(b);
+  g.C = reinterpret_cast<uint16_t*>(c);
+  g.M = (int)M; g.N = (int)N; g.K = (int)K;
+  g.tiles_n = (int)(N / 256);
+  g.tiles_k = (int)(K / 256);
+  // the LDS limit is a per-device attribute of the function: set it for the current device once (a race only repeats the call)
+  static bool attr_set[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = -1;
+  if (dev < 0 || !attr_set[dev]) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tn_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kTnLds);
+    if (e != hipSuccess) return fail(TTAMD_ELAUNCH, "gemm_tn: cannot reserve %d bytes of LDS: %s", kTnLds, hipGetErrorString(e));
+    if (dev >= 0) attr_set[dev] = true;
+  }
+  gemm_tn_kernel<<<dim3((unsigned)(g.tiles_n * g.tiles_k)), dim3(512), kTnLds, reinterpret_cast<hipStream_t>(stream)>>>(g);
+  return check_launch("gemm_tn");
+}

@@ -625,6 +625,32 @@ def tiled_linear(x: torch.Tensor, tiled: torch.Tensor, n_out: int, bias: Optiona
     return y
 
 
+def gemm_tn_applies(M: int, N: int, K: int) -> bool:
+    """Shapes ``gemm_tn`` serves: M a multiple of 32, N and K multiples of 256."""
+    return bool(_lib.load().ttamd_gemm_tn_applies(M, N, K))
+
+
+def gemm_tn(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """a [M, N], b [M, K] bf16 -> a.T @ b [N, K] bf16 (fp32 accumulation): the weight gradient of a linear layer."""
+    a = _bf16_2d(a, "gemm_tn")
+    b = _bf16_2d(b, "gemm_tn")
+    M, N = a.shape
+    if b.shape[0] != M:
+        raise ValueError(f"gemm_tn: a has {M} rows, b {b.shape[0]}")
+    K = b.shape[1]
+    c = torch.empty(N, K, dtype=torch.bfloat16, device=a.device)
+    lib = _lib.load()
+    with torch.cuda.device(a.device):
+        events = _gemm_timer("tn", M, N, K, 0) if _gemm_timer is not None else None
+        if events:
+            events[0].record()
+        rc = lib.ttamd_gemm_tn_bf16(a.data_ptr(), b.data_ptr(), c.data_ptr(), M, N, K, _stream(a))
+        if events:
+            events[1].record()
+    _lib.check(rc, "gemm_tn")
+    return c
+
+
 def quantize_per_group_int4(w: torch.Tensor, group_size: int, qparam_dtype: torch.dtype = torch.float32,
                             eps: Optional[float] = None):
     """w [rows, K] -> (int8 tensor of int4 values, scale fp32 [rows, K/g], zeros fp32 [rows, K/g])"""

@@ -241,10 +241,11 @@ class FakeQuantizer(nn.Module):
 
 # FakeQuantizedLinear on the library's own GEMM: the weight's fake quantisation is written in the GEMM's tile order (once
 # for the forward, once transposed for the grad-input) and never row-major; forward and grad-input run on
-# ``ttamd_tiled_linear_bf16``, the weight gradient on the vendor library.  Step time equals the all-vendor path at the 8B
-# shapes (396 against 397 ms).  False: row-major fq(W) and ``F.linear`` for everything.
+# ``ttamd_tiled_linear_bf16``, the weight gradient on ``ttamd_gemm_tn_bf16`` (layers of fewer than 192 output tiles of
+# 256 x 256: the vendor library).  False: row-major fq(W) and ``F.linear`` for everything.
 TILED_GEMM = True
 TILED_GEMM_MIN_ROWS = 2048
+TN_GEMM_MIN_TILES = 192
 
 
 class _TiledFakeQuantLinearFn(torch.autograd.Function):
@@ -275,7 +276,12 @@ class _TiledFakeQuantLinearFn(torch.autograd.Function):
         gy2 = gy.reshape(-1, N)
         need_x, need_w, need_b, _ = ctx.needs_input_grad
         gx = ops.tiled_linear(gy2, tb, K).view(ctx.x_shape) if need_x else None
-        gw = gy2.t().matmul(x2) if need_w else None
+        gw = None
+        if need_w:
+            # a few hundred output tiles fill the chip: the transposing GEMM of this library (1.2 - 1.3 PFLOP/s at the 8B
+            # shapes against 0.95 - 1.1 for the vendor library's); narrower layers (k / v) stay on the vendor library
+            own = ops.gemm_tn_applies(gy2.shape[0], N, K) and (N // 256) * (K // 256) >= TN_GEMM_MIN_TILES
+            gw = ops.gemm_tn(gy2, x2) if own else gy2.t().matmul(x2)
         gb = gy2.sum(dim=0) if (ctx.has_bias and need_b) else None
         return gx, gw, gb, None
 
