@@ -152,7 +152,12 @@ __global__ __launch_bounds__(512) void gemm_tn_kernel(const TnArgs g) {
     issue(t + 3);
     read_step(t);
     __builtin_amdgcn_sched_barrier(0);
-    asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");
+    // what the waves with wm = 1 read here is overwritten by requests the waves with wm = 0 issue right after the next
+    // barrier: they let their reads complete before they pass it (the others' reads have a whole interval more)
+    if (wm == 1)
+      asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    else
+      asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_s_setprio(1);
 #pragma unroll

@@ -421,7 +421,9 @@ __global__ __launch_bounds__(512) void nf4_gemm_dense_kernel(const DenseArgs g) 
   //          A(1) x4, W(2) x2; M(t): W(t+3) x2, then for even t A(t/2 + 2) x4.  W(t+1) came from M(t-2) and the
   //          activation entry of step t+1 is older; newer than W(t+1) are 4 + 2 + 6 = 12 loads (t even), 0 + 6 + 2 = 8 (t odd).
   //      The operand reads of M(t) are awaited by the compiler's own counts before the first MFMA that needs them, after
-  //      the barrier: the other wave's MFMAs are still draining then.
+  //      the barrier: the other wave's MFMAs are still draining then.  The waves with wm = 1 are the exception: what they
+  //      read in one interval is overwritten by requests the waves with wm = 0 issue right after the next barrier, so
+  //      they let their reads complete before they pass it (the others' reads have a whole interval more).
   issue_a(0, 0);
   issue_w(0, 0);
   issue_w(1, 1);
@@ -437,13 +439,19 @@ __global__ __launch_bounds__(512) void nf4_gemm_dense_kernel(const DenseArgs g) 
     issue_a((t >> 1) + 2, e2);
     read_step(e0, 0, ws);
     __builtin_amdgcn_sched_barrier(0);
-    asm volatile("s_waitcnt vmcnt(12)\n\ts_barrier" ::: "memory");
+    if (wm == 1)
+      asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    else
+      asm volatile("s_waitcnt vmcnt(12)\n\ts_barrier" ::: "memory");
     compute();
     // ---- odd step t + 1
     issue_w(t + 4, ws);
     read_step(e0, 1, (ws + 1) & 3);
     __builtin_amdgcn_sched_barrier(0);
-    asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");
+    if (wm == 1)
+      asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    else
+      asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");
     compute();
     e0 = e1;
     ws = (ws + 2) & 3;
