@@ -45,6 +45,34 @@ def test_against_fp32_matmul(M, N, K):
     torch.testing.assert_close(c.float(), want, rtol=1e-2, atol=1e-2 * scale)
 
 
+@pytest.mark.parametrize("M,N,K", [(8192, 14336, 4096), (8192, 4096, 14336), (4096, 128256, 4096)])
+def test_full_size_weight_gradients_of_the_8b_qat_configuration(M, N, K):
+    """gate / up, down and one 4096-token chunk of the output projection at their real sizes (batch 2 x 4096,
+    ``recipes/configs/llama3_1/8B_qat_full.yaml``; shapes from ``torchtune/models/llama3_1/_model_builders.py:20-59``):
+    one-hot rows pin the large-grid indexing bit for bit, random operands are compared with the fp32 product in row
+    blocks (the fp32 result of the widest case would not be worth its 2 GB)."""
+    assert ops.gemm_tn_applies(M, N, K)
+    g = torch.Generator().manual_seed(N + K)
+    b = torch.randn(M, K, generator=g).to(BF).to(DEV)
+    a = torch.zeros(M, N, dtype=BF, device=DEV)
+    R = min(M, N)
+    cols = torch.randperm(N, generator=g)[:R].to(DEV)           # row m < R of a is one-hot at column cols[m]
+    a[torch.arange(R, device=DEV), cols] = 1.0
+    c = ops.gemm_tn(a, b)
+    assert torch.equal(c[cols].view(torch.int16), b[:R].view(torch.int16))
+    untouched = torch.ones(N, dtype=torch.bool, device=DEV)
+    untouched[cols] = False
+    assert int(c[untouched].view(torch.int16).count_nonzero()) == 0
+    del a, c
+    a = torch.randn(M, N, generator=g).to(BF).to(DEV)
+    c = ops.gemm_tn(a, b)
+    bf = b.float()
+    for n0 in range(0, N, 16384):
+        want = a[:, n0:n0 + 16384].float().t() @ bf
+        scale = max(1.0, float(want.abs().max()) / 8)
+        torch.testing.assert_close(c[n0:n0 + 16384].float(), want, rtol=1e-2, atol=1e-2 * scale)
+
+
 def test_unsupported_shapes_are_refused():
     lib = _lib.load()
     assert not ops.gemm_tn_applies(100, 256, 256) and not ops.gemm_tn_applies(64, 320, 256) and not ops.gemm_tn_applies(64, 256, 64)

@@ -51,6 +51,31 @@ def test_staged_fake_quantised_weight_is_bit_exact_in_both_layouts(N, K, g, scal
     assert only_f[1] is None and only_f[2] is None and torch.equal(only_f[0], tf)
 
 
+@pytest.mark.parametrize("N,K", [(14336, 4096), (4096, 14336), (128256, 4096)])
+def test_staged_weight_at_the_full_sizes_of_the_8b_qat_configuration(N, K):
+    """gate / up, down and the output projection at their real sizes (``torchtune/models/llama3_1/_model_builders.py:20-59``),
+    group 32 as in ``recipes/configs/llama3_1/8B_qat_full.yaml``: every staged value of both layouts, read back through
+    the GEMM with one-hot activations, equals the row-major fake quantisation bit for bit."""
+    g = 32
+    w = _weight(N, K, seed=N + K).to(DEV)
+    want, want_scale = ops.fq_per_group_int4_sym(w, g)
+    tf, tb, scale = ops.fq_per_group_int4_sym_tiled(w, g)
+    assert torch.equal(scale, want_scale)
+    rows = 4096
+    assert K >= rows and N >= rows
+    for k0 in sorted(set(range(0, K - rows + 1, rows)) | {K - rows}):   # forward tiles: row m = column k0 + m of fq(W)
+        x = torch.zeros(rows, K, dtype=BF, device=DEV)
+        x[torch.arange(rows, device=DEV), k0 + torch.arange(rows, device=DEV)] = 1.0
+        y = ops.tiled_linear(x, tf, N)
+        assert torch.equal(y.view(torch.int16), want[:, k0:k0 + rows].t().contiguous().view(torch.int16)), k0
+    bases = {0, (N // 2 // 256) * 256, N - rows} if N > 4 * rows else set(range(0, N - rows + 1, rows)) | {N - rows}
+    for n0 in sorted(bases):                                     # transposed tiles: row m = row n0 + m of fq(W)
+        gy = torch.zeros(rows, N, dtype=BF, device=DEV)
+        gy[torch.arange(rows, device=DEV), n0 + torch.arange(rows, device=DEV)] = 1.0
+        gx = ops.tiled_linear(gy, tb, K)
+        assert torch.equal(gx.view(torch.int16), want[n0:n0 + rows].view(torch.int16)), n0
+
+
 def test_unsupported_group_size_is_refused():
     w = _weight(128, 512, 1).to(DEV)
     with pytest.raises(ValueError):
