@@ -518,6 +518,8 @@ def main() -> int:
     ap.add_argument("--no-memory-leg", action="store_true",
                     help="skip the peak-memory measurement (two extra model builds with one step each)")
     ap.add_argument("--no-config1", action="store_true", help="skip the single-layer configuration timed on GPU and CPU")
+    ap.add_argument("--no-gated-epilogue", action="store_true",
+                    help="A/B: silu(gate) * up as a pass of its own instead of the epilogue of the gate / up GEMM launch")
     ap.add_argument("--no-group", action="store_true",
                     help="one call per projection, as the reference's modules make them, instead of the group kernels for the "
                          "projections that share an input (q/k/v, gate/up): for A/B timing")
@@ -547,6 +549,7 @@ def main() -> int:
 
     harness.SDPA_BACKEND = args.sdpa
     harness.GROUP_SHARED_INPUT = not args.no_group
+    harness.GATED_EPILOGUE = not args.no_gated_epilogue
     ops.EXPANDED_WEIGHT_PATH = not args.no_expanded_weight
     if args.no_qat_tiled_gemm:
         from torchtune_amd import qat as qat_module
@@ -711,8 +714,10 @@ def main() -> int:
         "roofline": {
             "bound": "mfma",
             "kernel": ("nf4_gemm_dense_kernel with the nf4_expand_tiled_kernel launches that precede it in the same call (NF4 weight "
-                       "expanded once per call into scratch memory, then a bf16 MFMA GEMM with the LoRA adapter in its epilogue; forward "
-                       "and grad-input calls)" if timer.expanded_calls * 2 > calls else
+                       "expanded once per call into scratch memory, then a bf16 MFMA GEMM with the LoRA adapter in its epilogue"
+                       + ("; the gate / up launch also forms silu(gate) * up there, counted as zero FLOPs" if harness.GATED_EPILOGUE
+                          and harness.GROUP_SHARED_INPUT else "") + "; forward and grad-input calls)"
+                       if timer.expanded_calls * 2 > calls else
                        "nf4_gemm_rs_kernel (fused NF4-dequant + LoRA bf16 MFMA GEMM, forward and grad-input launches)"),
             "achieved": round(achieved, 1),
             "peak": MFMA_BF16_PEAK_TFLOPS,

@@ -310,6 +310,13 @@ int ttamd_lora_group_hidden_bf16(const void* x, const ttamd_lora_group_member* m
 size_t ttamd_lora_group_fwd_workspace_bytes(const ttamd_lora_group_member* members, int n_members, int64_t M, int64_t K);
 int ttamd_nf4_lora_group_fwd_bf16(const void* x, const ttamd_lora_group_member* members, int n_members, const void* h_cat,
                                   int64_t M, int64_t K, void* workspace, size_t workspace_bytes, void* stream);
+/* The gate / up pair of a SwiGLU feed-forward (torchtune/modules/feed_forward.py:50-53: w2(silu(w1(x)) * w3(x)), w1 and
+ * w3 LoRALinear over NF4): members[0] = w1 (gate), members[1] = w3 (up), equal N.  Writes both members' y as the call above
+ * does and act, bf16 [M, N] = bf16(bf16(silu(y_0)) * y_1) - the bits ttamd_swiglu_fwd_bf16 gives on the two outputs.
+ * With the workspace of ttamd_lora_group_fwd_workspace_bytes and a shape the many-token path serves, the product is
+ * formed in the epilogue of the one GEMM launch (the two outputs are not read back); otherwise in a pass of its own. */
+int ttamd_nf4_lora_group_swiglu_fwd_bf16(const void* x, const ttamd_lora_group_member* members, int n_members, const void* h_cat,
+                                         void* act, int64_t M, int64_t K, void* workspace, size_t workspace_bytes, void* stream);
 /* gh_cat out, bf16 [M, sum of ranks]; every member's grad_lora_a and grad_lora_b; members[i].y = gy_i */
 size_t ttamd_lora_group_bwd_workspace_bytes(const ttamd_lora_group_member* members, int n_members, int64_t M, int64_t K);
 int ttamd_lora_group_bwd_bf16(const void* x, const void* h_cat, const ttamd_lora_group_member* members, int n_members,

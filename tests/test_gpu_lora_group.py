@@ -18,7 +18,8 @@ import torch
 
 from oracle import lora_oracle, nf4_oracle
 from torchtune_amd import ops
-from torchtune_amd.modules.peft import LoRALinear, group_applies, lora_linear_group
+from torchtune_amd.modules import layer_ops
+from torchtune_amd.modules.peft import LoRALinear, group_applies, lora_linear_group, lora_swiglu_group
 from torchtune_amd.nf4_tensor import to_nf4
 
 pytestmark = pytest.mark.gpu
@@ -203,6 +204,74 @@ def test_module_group_against_oracle_and_layerwise(M, K, Ns, ranks, bias):
     for i, (Ao, Bo) in enumerate(leaves):
         for mine, theirs in ((got["ga"][i], Ao.grad), (got["gb"][i], Bo.grad)):
             torch.testing.assert_close(mine.cpu().float(), theirs.float(), rtol=2e-2, atol=2e-2 * float(theirs.float().abs().max()) + 1e-30)
+
+
+GATED_SHAPES = [
+    # M, K, width, ranks, bias        (256 tiles of 256 x 256 and 2048 rows: the product is written by the GEMM launch)
+    (2048, 256, 4096, (16, 16), False),
+    (2048 + 192, 512, 4096, (16, 8), True),     # a last row tile with 192 rows
+    (4096, 1024, 2048, (32, 0 + 16), False),
+    (8192, 256, 1024, (16, 16), True),
+    (16, 512, 1024, (8, 8), False),             # few tokens: group launch + a pass of its own
+    (300, 512, 512, (16, 16), True),            # tiled kernels + a pass of its own
+    (2048, 256, 1152, (16, 16), False),         # many tokens, too few tiles for the expanded path
+]
+
+
+@pytest.mark.parametrize("M,K,width,ranks,bias", GATED_SHAPES, ids=[f"M{s[0]}_K{s[1]}_W{s[2]}" for s in GATED_SHAPES])
+def test_gated_pair_equals_group_forward_plus_swiglu_bitwise(M, K, width, ranks, bias):
+    """``ttamd_nf4_lora_group_swiglu_fwd_bf16``: both projections equal the plain group call's bit for bit (the same GEMM
+    on the same operands, whatever the order of the weight's columns in the scratch copy) and the gated product equals
+    ``ttamd_swiglu_fwd_bf16`` of them bit for bit; that kernel is itself compared with the reference's
+    ``F.silu(g) * u`` in bf16 in tests/test_gpu_layer_ops.py."""
+    mem = _members(K, (width, width), ranks, seed=M + K + width, bias=bias)
+    members = [m[0] for m in mem]
+    x = torch.randn(M, K, generator=torch.Generator().manual_seed(11)).to(BF).to(DEV)
+    h0, (g0, u0) = ops.lora_group_fwd(x, members)
+    h1, (g1, u1, act) = ops.lora_group_fwd(x, members, swiglu=True)
+    assert torch.equal(h0, h1)
+    assert torch.equal(g0.view(torch.int16), g1.view(torch.int16)) and torch.equal(u0.view(torch.int16), u1.view(torch.int16))
+    assert torch.equal(act.view(torch.int16), ops.swiglu_fwd(g0, u0).view(torch.int16))
+    # and the definition, evaluated by torch on the same bf16 projections
+    want = torch.nn.functional.silu(g0) * u0
+    torch.testing.assert_close(act.float(), want.float(), rtol=2e-2, atol=1e-3)
+
+
+def test_gated_pair_rejects_unequal_widths():
+    mem = _members(512, (256, 128), (8, 8), seed=3)
+    x = torch.randn(8, 512, device=DEV, dtype=BF)
+    with pytest.raises(ValueError):
+        ops.lora_group_fwd(x, [m[0] for m in mem], swiglu=True)
+    with pytest.raises(ValueError):
+        ops.lora_group_fwd(x, [mem[0][0]], swiglu=True)
+
+
+@pytest.mark.parametrize("M,K,width", [(2048, 256, 4096), (64, 512, 512)], ids=["epilogue", "own_pass"])
+def test_gated_module_function_matches_group_then_swiglu(M, K, width):
+    """``lora_swiglu_group`` against ``lora_linear_group`` followed by the stand-alone SwiGLU op: output and every
+    gradient bit for bit (same kernels on the same values in backward)."""
+    layers, _ = _layers(K, (width, width), (16, 16), 32.0, False, seed=M + width)
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(M, K, generator=g).to(BF).to(DEV)
+    gact = torch.randn(M, width, generator=g).to(BF).to(DEV)
+
+    def run(gated):
+        for l in layers:
+            l.zero_grad()
+        xg = x.clone().requires_grad_()
+        if gated:
+            act = lora_swiglu_group(xg, layers[0], layers[1])
+            assert act is not None
+        else:
+            gg, uu = lora_linear_group(xg, layers)
+            act = layer_ops.swiglu(gg, uu)
+        act.backward(gact)
+        return [act.detach(), xg.grad] + [p.grad.clone() for l in layers for p in (l.lora_a.weight, l.lora_b.weight)]
+
+    for a, b in zip(run(True), run(False)):
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+    layers[1].disabled = True
+    assert lora_swiglu_group(x, layers[0], layers[1]) is None   # the caller falls back to its own multiply
 
 
 def test_group_falls_back_when_it_does_not_apply():

@@ -499,3 +499,24 @@ def test_tiled_entry_points_validate_their_arguments_on_the_host():
     assert q(p, 64, 64, 16, F32, 1e-7, p, None, None, None) == EUNSUPPORTED       # group size
     assert q(p, 64, 192, 128, F32, 1e-7, p, None, None, None) == EUNSUPPORTED     # group does not divide K
     assert b"group size" in lib.ttamd_last_error()
+
+
+def test_gated_group_entry_point_validates_its_arguments_on_the_host():
+    """``ttamd_nf4_lora_group_swiglu_fwd_bf16`` takes exactly the gate and the up projection, of equal width, and a
+    non-null aligned output for the gated product; refused before any launch."""
+    import ctypes
+
+    from torchtune_amd import _lib
+
+    lib = _lib.load()
+    buf = (ctypes.c_char * 4096)()
+    p = (ctypes.addressof(buf) + 15) & ~15
+    arr = (_lib.LoraGroupMember * 2)()
+    for e, n in zip(arr, (128, 64)):
+        e.N, e.rank, e.scale = n, 8, 1.0
+    f = lib.ttamd_nf4_lora_group_swiglu_fwd_bf16
+    assert f(p, arr, 2, p, p, 8, 64, None, 0, None) == -1 and b"equal width" in lib.ttamd_last_error()
+    assert f(p, arr, 1, p, p, 8, 64, None, 0, None) == -1
+    arr[1].N = 128
+    assert f(p, arr, 2, p, None, 8, 64, None, 0, None) == -1 and b"act" in lib.ttamd_last_error()
+

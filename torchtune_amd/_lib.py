@@ -90,6 +90,8 @@ SIGNATURES = {
     "ttamd_lora_group_hidden_bf16": (_int, [_c_void_p, _c_void_p, _int, _c_void_p, _i64, _i64, _c_void_p, _size, _c_void_p]),
     "ttamd_lora_group_fwd_workspace_bytes": (_size, [_c_void_p, _int, _i64, _i64]),
     "ttamd_nf4_lora_group_fwd_bf16": (_int, [_c_void_p, _c_void_p, _int, _c_void_p, _i64, _i64, _c_void_p, _size, _c_void_p]),
+    "ttamd_nf4_lora_group_swiglu_fwd_bf16": (_int, [_c_void_p, _c_void_p, _int, _c_void_p, _c_void_p, _i64, _i64, _c_void_p, _size,
+                                                    _c_void_p]),
     "ttamd_lora_group_bwd_workspace_bytes": (_size, [_c_void_p, _int, _i64, _i64]),
     "ttamd_lora_group_bwd_bf16": (_int, [_c_void_p, _c_void_p, _c_void_p, _int, _c_void_p, _i64, _i64, _c_void_p, _size, _c_void_p]),
     "ttamd_nf4_group_bwd_dx_bf16": (_int, [_c_void_p, _int, _c_void_p, _c_void_p, _i64, _i64, _c_void_p]),

@@ -65,7 +65,9 @@ int run_gemm_dense(const void* X, const uint8_t* codes, const void* scal, int mo
                    bool lw_row_major, int R, float lscale, const void* bias, const void* cscale, void* C, int64_t M, int64_t Nout,
                    int64_t Kc, void* workspace, hipStream_t s);
 size_t dense_group_fwd_workspace_bytes(const GroupGemm& d);
-int run_gemm_dense_group_fwd(const void* x, const GroupGemm& d, const void* h_cat, void* workspace, hipStream_t s);
+// act != nullptr: two members of equal width (gate, up); the launch also writes act = silu(y[0]) * y[1]
+bool dense_group_gated_applies(const GroupGemm& d);
+int run_gemm_dense_group_fwd(const void* x, const GroupGemm& d, const void* h_cat, void* workspace, hipStream_t s, void* act = nullptr);
 size_t dense_group_dx_workspace_bytes(const GroupDx& d);
 int run_gemm_dense_group_dx(const GroupDx& d, const void* gh_cat, void* gx, void* workspace, hipStream_t s);
 

@@ -107,20 +107,25 @@ extern "C" size_t ttamd_lora_group_fwd_workspace_bytes(const ttamd_lora_group_me
   return align256(fwd_gemm_ws(d));
 }
 
-extern "C" int ttamd_nf4_lora_group_fwd_bf16(const void* x, const ttamd_lora_group_member* members, int n_members,
-                                             const void* h_cat, int64_t M, int64_t K, void* workspace, size_t workspace_bytes,
-                                             void* stream) {
+namespace {
+// The members' outputs; *act_done says whether a launch that was asked for the gated product (act != nullptr) wrote it.
+int group_fwd(const char* who, const void* x, const ttamd_lora_group_member* members, int n_members, const void* h_cat, void* act,
+              bool* act_done, int64_t M, int64_t K, void* workspace, size_t workspace_bytes, void* stream) {
   Decoded d;
-  if (int rc = decode("nf4_lora_group_fwd", members, n_members, M, K, false, d)) return rc;
-  TT_REQUIRE(x && h_cat && aligned16(x) && aligned16(h_cat), "nf4_lora_group_fwd: x and h_cat must be non-null and 16-byte aligned");
+  if (int rc = decode(who, members, n_members, M, K, false, d)) return rc;
+  TT_REQUIRE(x && h_cat && aligned16(x) && aligned16(h_cat), "%s: x and h_cat must be non-null and 16-byte aligned", who);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   if (M <= small_m_limit()) return run_small_m_group(x, d.gm, h_cat, s);
   // slices of the contraction for a member with few output tiles, when the caller brought the memory for them
   const size_t gem = align256(fwd_gemm_ws(d));
   const bool sliced = gem > 0 && workspace != nullptr && workspace_bytes >= gem;
-  TT_REQUIRE(!sliced || aligned16(workspace), "nf4_lora_group_fwd: workspace must be 16-byte aligned");
+  TT_REQUIRE(!sliced || aligned16(workspace), "%s: workspace must be 16-byte aligned", who);
   // many tokens: one launch over the members' concatenated output columns, every weight expanded once
-  if (sliced && dense_group_fwd_workspace_bytes(d.gm) > 0) return run_gemm_dense_group_fwd(x, d.gm, h_cat, workspace, s);
+  if (sliced && dense_group_fwd_workspace_bytes(d.gm) > 0) {
+    const bool gated = act != nullptr && dense_group_gated_applies(d.gm);
+    if (act_done) *act_done = gated;
+    return run_gemm_dense_group_fwd(x, d.gm, h_cat, workspace, s, gated ? act : nullptr);
+  }
   const int ldh = d.gm.r_off[d.gm.n];
   for (int i = 0; i < d.gm.n; ++i) {
     const void* sc = d.gm.bscal_t[i] ? d.gm.bscal_t[i] : d.gm.bscal[i];
@@ -130,6 +135,27 @@ extern "C" int ttamd_nf4_lora_group_fwd_bf16(const void* x, const ttamd_lora_gro
       return rc;
   }
   return TTAMD_OK;
+}
+}  // namespace
+
+extern "C" int ttamd_nf4_lora_group_fwd_bf16(const void* x, const ttamd_lora_group_member* members, int n_members,
+                                             const void* h_cat, int64_t M, int64_t K, void* workspace, size_t workspace_bytes,
+                                             void* stream) {
+  return group_fwd("nf4_lora_group_fwd", x, members, n_members, h_cat, nullptr, nullptr, M, K, workspace, workspace_bytes, stream);
+}
+
+extern "C" int ttamd_nf4_lora_group_swiglu_fwd_bf16(const void* x, const ttamd_lora_group_member* members, int n_members,
+                                                    const void* h_cat, void* act, int64_t M, int64_t K, void* workspace,
+                                                    size_t workspace_bytes, void* stream) {
+  TT_REQUIRE(n_members == 2 && members && members[0].N == members[1].N,
+             "nf4_lora_group_swiglu_fwd: takes the gate and the up projection, two members of equal width");
+  TT_REQUIRE(act && aligned16(act), "nf4_lora_group_swiglu_fwd: act must be non-null and 16-byte aligned");
+  bool done = false;
+  if (int rc = group_fwd("nf4_lora_group_swiglu_fwd", x, members, n_members, h_cat, act, &done, M, K, workspace, workspace_bytes, stream))
+    return rc;
+  if (done) return TTAMD_OK;
+  // shapes the many-token launch does not serve: the same arithmetic as its own pass over the two outputs
+  return ttamd_swiglu_fwd_bf16(members[0].y, members[1].y, act, M * members[0].N, stream);
 }
 
 extern "C" size_t ttamd_lora_group_bwd_workspace_bytes(const ttamd_lora_group_member* members, int n_members, int64_t M, int64_t K) {

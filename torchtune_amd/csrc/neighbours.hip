@@ -11,6 +11,7 @@
 // so these kernels are checked to a tolerance, not bit for bit.
 #include "common.h"
 #include "nf4_math.h"
+#include "swiglu_math.h"
 
 namespace ttamd {
 namespace {
@@ -211,10 +212,6 @@ __global__ __launch_bounds__(256) void rope_kernel(const uint16_t* __restrict__ 
 // SwiGLU gate.  forward: a = bf16(silu(g)); out = bf16(a * u).
 // backward: gu = bf16(go * a); ga = bf16(go * u); gg = bf16(ga * silu'(g)), silu'(g) = s (1 + g (1 - s)), s = sigmoid(g).
 // ---------------------------------------------------------------------------------------------------
-__device__ __forceinline__ float sigmoid_f(float g) {
-  return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * g));
-}
-
 __global__ __launch_bounds__(256) void swiglu_fwd_kernel(const uint16_t* __restrict__ g, const uint16_t* __restrict__ u,
                                                          uint16_t* __restrict__ out, int64_t n_chunks) {
   const int64_t chunk = (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -223,11 +220,7 @@ __global__ __launch_bounds__(256) void swiglu_fwd_kernel(const uint16_t* __restr
   const u32x4_t uv = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(u) + chunk);
   u32x4_t o;
 #pragma unroll
-  for (int d = 0; d < 4; ++d) {
-    const float g0 = lo_f(gv[d]), g1 = hi_f(gv[d]);
-    const float a0 = round_to_bf16(g0 * sigmoid_f(g0)), a1 = round_to_bf16(g1 * sigmoid_f(g1));
-    o[d] = pack2(a0 * lo_f(uv[d]), a1 * hi_f(uv[d]));
-  }
+  for (int d = 0; d < 4; ++d) o[d] = swiglu_gate_pair(gv[d], uv[d]);
   __builtin_nontemporal_store(o, reinterpret_cast<u32x4_t*>(out) + chunk);
 }
 

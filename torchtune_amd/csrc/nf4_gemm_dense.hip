@@ -31,6 +31,7 @@
 #include "common.h"
 #include "group.h"
 #include "nf4_math.h"
+#include "swiglu_math.h"
 
 namespace ttamd {
 namespace {
@@ -65,12 +66,15 @@ __constant__ float kNF4Dense[16] = TT_NF4_TABLE;
 template <int MODE>
 __global__ __launch_bounds__(256) void nf4_expand_tiled_kernel(const uint8_t* __restrict__ codes, const float* __restrict__ scal,
                                                                int Nout, int Kc, int nk_total, int t_off,
-                                                               char* __restrict__ tiled) {
+                                                               char* __restrict__ tiled, int paired) {
   __shared__ float2 lut[256];
   const int tid = threadIdx.x;
   lut[tid] = make_float2(round_to_bf16(kNF4Dense[tid >> 4]), round_to_bf16(kNF4Dense[tid & 15]));
   __syncthreads();
   const int T = blockIdx.x;
+  // paired: two weights of equal shape share one tiled copy, 128 columns (8 blocks) of the one followed by the same
+  // 128 columns of the other (whose `tiled` starts 8 blocks further), so that a 256-wide tile of the GEMM holds both
+  const int To = paired ? ((T >> 3) << 4) + (T & 7) : T;
   const int r = tid & 15;        // column inside the block
   const int col = 16 * T + r;
   const int nk = Kc >> 5;
@@ -94,7 +98,7 @@ __global__ __launch_bounds__(256) void nf4_expand_tiled_kernel(const uint8_t* __
 #pragma unroll
       for (int q = 0; q < 32; ++q) sc[q] = s1;
     }
-    char* piece = tiled + ((int64_t)T * nk_total + t_off + t) * 1024;
+    char* piece = tiled + ((int64_t)To * nk_total + t_off + t) * 1024;
 #pragma unroll
     for (int g4 = 0; g4 < 4; ++g4) {
       const uint32_t w = cd[g4];
@@ -281,6 +285,7 @@ struct DenseArgs {
   int M, Nout, Kc;  // Nout, Kc: totals
   int lw_row_major, ldlx;
   int tiles_m, tiles_n;
+  uint16_t* act;    // GATED launches only: [M, out[0].width] bf16 = silu(out 0) * out 1
 };
 
 constexpr int kAEntry = 32768;  // activation ring: 3 entries of 256 rows x 64 k
@@ -288,7 +293,12 @@ constexpr int kWBase = 3 * kAEntry;
 constexpr int kWStage = 16384;  // weight ring: 4 stages of 256 columns x 32 k
 constexpr int kLdsDense = kWBase + 4 * kWStage;
 
-template <bool LW_ROW_MAJOR>
+// GATED (forward of a gate / up pair, torchtune/modules/feed_forward.py:50-53): the two members' columns alternate in
+// the tiled weight 128 by 128 (the paired layout of the expansion), so a tile holds columns [128 tile_n, + 128) of both:
+// the waves with wn < 2 own the gate's, the others the up projection's.  Each wave writes its member's output as usual;
+// the bf16 bands then meet in LDS and the workgroup also writes act = bf16(bf16(silu(gate)) * up), the arithmetic of
+// ttamd_swiglu_fwd_bf16 on the rounded outputs, bit for bit.
+template <bool LW_ROW_MAJOR, bool GATED = false>
 __global__ __launch_bounds__(512) void nf4_gemm_dense_kernel(const DenseArgs g) {
 #if defined(__HIP_DEVICE_COMPILE__)
   constexpr int MT = 8, NT = 4;  // 16 x 16 MFMA tiles per wave
@@ -464,11 +474,16 @@ __global__ __launch_bounds__(512) void nf4_gemm_dense_kernel(const DenseArgs g) 
   for (int aidx = 0; aidx < g.nad; ++aidx) {
     const int R = g.ad[aidx].R;
     const int nb = g.ad[aidx].n_begin, ncols = g.ad[aidx].n_end - nb;
-    if (R <= 0 || n0 < nb || n0 >= nb + ncols) continue;  // the same for every wave of the workgroup
+    if constexpr (GATED) {
+      if (R <= 0 || aidx != (wn >> 1)) continue;  // adapter i belongs to member i; uniform over the wave, no barrier below
+    } else {
+      if (R <= 0 || n0 < nb || n0 >= nb + ncols) continue;  // the same for every wave of the workgroup
+    }
     const uint16_t* lX = g.ad[aidx].lX;
     const uint16_t* lW = g.ad[aidx].lW;
     const float lscale = g.ad[aidx].lscale;
-    const int nl0 = n0 - nb;  // first column of the tile among the adapter's columns
+    // first column of the tile among the adapter's columns (GATED: such that + 64 wn lands on the wave's own columns)
+    const int nl0 = GATED ? 128 * tile_n - 128 * (wn >> 1) : n0 - nb;
     int pitch = 0;  // bytes per column of the staged adapter weights
     if constexpr (!LW_ROW_MAJOR) {
       // lW is [R, Nout]: a lane needs 8 ranks of one column, 8 elements Nout apart.  The workgroup copies the 256
@@ -530,10 +545,17 @@ __global__ __launch_bounds__(512) void nf4_gemm_dense_kernel(const DenseArgs g) 
   //      16-byte chunk c of row r sits in slot c ^ (r & 7).
   __syncthreads();
   int oi = 0;
-  while (oi + 1 < g.nout && n0 >= g.out[oi + 1].n_begin) ++oi;
-  const int nlo = n0 - g.out[oi].n_begin + wn * 64;  // first column of this wave's band in its output tensor
+  if constexpr (GATED) {
+    oi = wn >> 1;
+  } else {
+    while (oi + 1 < g.nout && n0 >= g.out[oi + 1].n_begin) ++oi;
+  }
+  // first column of this wave's band in its output tensor
+  const int nlo = GATED ? 128 * tile_n + 64 * (wn & 1) : n0 - g.out[oi].n_begin + wn * 64;
   const int width = g.out[oi].width;
-  if (nlo >= width) return;  // the whole band of this wave lies outside (no barrier follows)
+  if constexpr (!GATED) {
+    if (nlo >= width) return;  // the whole band of this wave lies outside (no barrier follows)
+  }
   {
     const uint16_t* bias = g.out[oi].bias;
     const uint16_t* cscale = g.out[oi].cscale;
@@ -561,9 +583,13 @@ __global__ __launch_bounds__(512) void nf4_gemm_dense_kernel(const DenseArgs g) 
         *reinterpret_cast<u32x2_t*>(band + r * 128 + (((2 * j + (g4 >> 1)) ^ (r & 7)) << 4) + 8 * (g4 & 1)) = o;
       }
     }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    if constexpr (GATED) {
+      __syncthreads();  // the gate's and the up projection's bands are read across waves below (widths are multiples of 128: every wave is here)
+    } else {
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
     const int c = lane & 7;
     uint16_t* crow = g.out[oi].C + nlo + 8 * c;
     const int mrow0 = m0 + 128 * wm;
@@ -573,29 +599,48 @@ __global__ __launch_bounds__(512) void nf4_gemm_dense_kernel(const DenseArgs g) 
       const u32x4_t v = *reinterpret_cast<const u32x4_t*>(band + r * 128 + ((c ^ (r & 7)) << 4));
       if (mrow0 + r < g.M) *reinterpret_cast<u32x4_t*>(crow + (int64_t)(mrow0 + r) * width) = v;
     }
+    if constexpr (GATED) {
+      // act: the 128 x 64 piece (wm, wn & 1) is shared by the two waves that hold its gate and up bands, 64 rows each
+      const char* gband = smem + (4 * wm + (wn & 1)) * 16384;
+      const char* uband = gband + 2 * 16384;
+      uint16_t* arow = g.act + nlo + 8 * c;
+#pragma unroll 8
+      for (int t = 0; t < 8; ++t) {
+        const int r = 64 * (wn >> 1) + 8 * t + (lane >> 3);
+        const int slot = r * 128 + ((c ^ (r & 7)) << 4);
+        const u32x4_t gv = *reinterpret_cast<const u32x4_t*>(gband + slot);
+        const u32x4_t uv = *reinterpret_cast<const u32x4_t*>(uband + slot);
+        u32x4_t o;
+#pragma unroll
+        for (int d = 0; d < 4; ++d) o[d] = swiglu_gate_pair(gv[d], uv[d]);
+        if (mrow0 + r < g.M) *reinterpret_cast<u32x4_t*>(arow + (int64_t)(mrow0 + r) * width) = o;
+      }
+    }
   }
 #endif
 }
 
 int launch_expand(int mode, const uint8_t* codes, const float* scal, int64_t Nout, int64_t Kc, int64_t nk_total, int64_t t_off,
-                  char* tiled, hipStream_t s) {
+                  char* tiled, hipStream_t s, bool paired = false) {
   // one block of 16 columns per blockIdx.x; the contraction is cut along blockIdx.y so that about 2048 workgroups exist
   const int64_t chunks = ((Kc >> 5) + 15) / 16;
   int64_t ysplit = (2048 + (Nout >> 4) - 1) / (Nout >> 4);
   ysplit = ysplit < 1 ? 1 : (ysplit > chunks ? chunks : ysplit);
   const dim3 grid((unsigned)(Nout >> 4), (unsigned)ysplit), block(256);
   if (mode == 3) {  // Nout = K, Kc = N of the weight: codes and scalers in the weight's own layout
+    TT_REQUIRE(!paired, "nf4_expand_tiled: the paired layout exists for the forward modes only");
     TT_REQUIRE((Nout + 255) / 256 < 65536, "nf4_expand_tiled: K too large for one launch");
     nf4_expand_tiled_transposed_kernel<<<dim3((unsigned)(Kc >> 5), (unsigned)((Nout + 255) / 256)), block, 0, s>>>(
         codes, scal, (int)Kc, (int)Nout, (int)nk_total, (int)t_off, tiled);
     return check_launch("nf4_expand_tiled_transposed");
   }
+  const int pr = paired ? 1 : 0;
   if (mode == 1)
-    nf4_expand_tiled_kernel<1><<<grid, block, 0, s>>>(codes, scal, (int)Nout, (int)Kc, (int)nk_total, (int)t_off, tiled);
+    nf4_expand_tiled_kernel<1><<<grid, block, 0, s>>>(codes, scal, (int)Nout, (int)Kc, (int)nk_total, (int)t_off, tiled, pr);
   else if (mode == 2)
-    nf4_expand_tiled_kernel<2><<<grid, block, 0, s>>>(codes, scal, (int)Nout, (int)Kc, (int)nk_total, (int)t_off, tiled);
+    nf4_expand_tiled_kernel<2><<<grid, block, 0, s>>>(codes, scal, (int)Nout, (int)Kc, (int)nk_total, (int)t_off, tiled, pr);
   else
-    nf4_expand_tiled_kernel<0><<<grid, block, 0, s>>>(codes, scal, (int)Nout, (int)Kc, (int)nk_total, (int)t_off, tiled);
+    nf4_expand_tiled_kernel<0><<<grid, block, 0, s>>>(codes, scal, (int)Nout, (int)Kc, (int)nk_total, (int)t_off, tiled, pr);
   return check_launch("nf4_expand_tiled");
 }
 
@@ -608,14 +653,20 @@ int launch_dense(DenseArgs& g, hipStream_t s) {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = -1;
   if (dev < 0 || !attr_set[dev]) {
-    for (const void* fn : {reinterpret_cast<const void*>(&nf4_gemm_dense_kernel<true>), reinterpret_cast<const void*>(&nf4_gemm_dense_kernel<false>)}) {
+    for (const void* fn : {reinterpret_cast<const void*>(&nf4_gemm_dense_kernel<true>), reinterpret_cast<const void*>(&nf4_gemm_dense_kernel<false>),
+                           reinterpret_cast<const void*>(&nf4_gemm_dense_kernel<true, true>)}) {
       hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsDense);
       if (e != hipSuccess) return fail(TTAMD_ELAUNCH, "nf4_gemm_dense: cannot reserve %d bytes of LDS: %s", kLdsDense, hipGetErrorString(e));
     }
     if (dev >= 0) attr_set[dev] = true;
   }
   const dim3 grid((unsigned)(g.tiles_m * g.tiles_n)), block(512);
-  if (g.lw_row_major)
+  if (g.act) {
+    TT_REQUIRE(g.lw_row_major && g.nout == 2 && g.nad == 2 && g.nseg == 1 && g.out[0].width == g.out[1].width && g.out[0].width % 128 == 0 &&
+                   g.Nout == 2 * g.out[0].width,
+               "nf4_gemm_dense: the gated launch takes two members of equal width, a multiple of 128");
+    nf4_gemm_dense_kernel<true, true><<<grid, block, kLdsDense, s>>>(g);
+  } else if (g.lw_row_major)
     nf4_gemm_dense_kernel<true><<<grid, block, kLdsDense, s>>>(g);
   else
     nf4_gemm_dense_kernel<false><<<grid, block, kLdsDense, s>>>(g);
@@ -681,10 +732,18 @@ size_t dense_group_fwd_workspace_bytes(const GroupGemm& d) {
   return d.n >= 2 && dense_path_applies(d.M, n_total, d.K) ? (size_t)n_total * (size_t)d.K * 2 : 0;
 }
 
-int run_gemm_dense_group_fwd(const void* x, const GroupGemm& d, const void* h_cat, void* workspace, hipStream_t s) {
+bool dense_group_gated_applies(const GroupGemm& d) {
+  return d.n == 2 && d.N[0] == d.N[1] && d.N[0] % 128 == 0 && dense_group_fwd_workspace_bytes(d) > 0;
+}
+
+// act != nullptr: the pair (gate, up) with act = silu(y_0) * y_1 written by the same launch (dense_group_gated_applies)
+int run_gemm_dense_group_fwd(const void* x, const GroupGemm& d, const void* h_cat, void* workspace, hipStream_t s, void* act) {
   TT_REQUIRE(d.n >= 2 && d.n <= kGroupMax && dense_group_fwd_workspace_bytes(d) > 0, "nf4_lora_group_fwd (expanded): shape not served");
   TT_REQUIRE(aligned16(workspace) && aligned16(x), "nf4_lora_group_fwd (expanded): pointers must be 16-byte aligned");
+  const bool gated = act != nullptr;
+  TT_REQUIRE(!gated || (dense_group_gated_applies(d) && aligned16(act)), "nf4_lora_group_swiglu_fwd (expanded): shape not served");
   DenseArgs g = {};
+  g.act = reinterpret_cast<uint16_t*>(act);
   g.nseg = 1;
   g.seg[0].X = reinterpret_cast<const uint16_t*>(x);
   g.seg[0].Kc = (int)d.K;
@@ -692,8 +751,9 @@ int run_gemm_dense_group_fwd(const void* x, const GroupGemm& d, const void* h_ca
   int64_t n_off = 0;
   for (int i = 0; i < d.n; ++i) {
     const bool tr = d.bscal_t[i] != nullptr;
-    if (int rc = launch_expand(tr ? 2 : 0, d.codes[i], tr ? d.bscal_t[i] : d.bscal[i], d.N[i], d.K, d.K >> 5, 0,
-                               reinterpret_cast<char*>(workspace) + n_off * d.K * 2, s))
+    // gated: the members' column blocks alternate 8 by 8, the second member starting 8 blocks (128 columns) in
+    char* dst = reinterpret_cast<char*>(workspace) + (gated ? (int64_t)i * 128 : n_off) * d.K * 2;
+    if (int rc = launch_expand(tr ? 2 : 0, d.codes[i], tr ? d.bscal_t[i] : d.bscal[i], d.N[i], d.K, d.K >> 5, 0, dst, s, gated))
       return rc;
     g.ad[i].lX = reinterpret_cast<const uint16_t*>(h_cat) + d.r_off[i];
     g.ad[i].lW = d.lora_b[i];

@@ -28,13 +28,15 @@ from torch.nn.attention import SDPBackend, sdpa_kernel
 from torch.utils.checkpoint import checkpoint
 
 from .modules import layer_ops
-from .modules.peft import LoRALinear, get_adapter_params, lora_linear_group, set_trainable_params
+from .modules.peft import LoRALinear, get_adapter_params, lora_linear_group, lora_swiglu_group, set_trainable_params
 from .qat import Int8DynActInt4WeightQATQuantizer
 
 
 # True: projections that read the same tensor (q/k/v, gate/up) go through the group kernels; False: one call per
 # projection, as the reference's modules make them (kept for A/B timing and for the tests that compare the two)
 GROUP_SHARED_INPUT = True
+# silu(w1 x) * w3 x formed in the epilogue of the gate / up GEMM launch instead of a pass of its own
+GATED_EPILOGUE = True
 
 
 @dataclass(frozen=True)
@@ -170,6 +172,10 @@ class FeedForward(nn.Module):
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         # gate and up read the same tensor (torchtune/modules/feed_forward.py:50-53): one group
+        if GROUP_SHARED_INPUT and GATED_EPILOGUE:
+            act = lora_swiglu_group(x, self.w1, self.w3)  # the product written by the pair's GEMM launch
+            if act is not None:
+                return self.w2(act)
         g, u = lora_linear_group(x, (self.w1, self.w3)) if GROUP_SHARED_INPUT else (self.w1(x), self.w3(x))
         return self.w2(layer_ops.swiglu(g, u) if _fused(g) else F.silu(g) * u)
 

@@ -61,16 +61,53 @@ class _QLoRAGroupFn(torch.autograd.Function):
             # an output nobody used arrives as None
             gy2.append(torch.zeros(x2.shape[0], w.shape[0], dtype=x2.dtype, device=x2.device) if g is None
                        else g.reshape(-1, w.shape[0]))
-        members = [ops.GroupMember(w.quantized_data, w.block_scalers(), tr, a, b, None, s, w.shape[0])
-                   for w, tr, a, b, s in zip(weights, _copies(weights, x2.shape[0]), las, lbs, ctx.scales)]
-        need_x = ctx.needs_input_grad[0]
-        gx, grads, _ = ops.lora_group_bwd(x2, h_cat, members, gy2, want_gx=need_x)
-        out: List = [gx.view(ctx.x_shape) if need_x else None, None]
-        for i in range(n):
-            _, need_a, need_b, need_bias = ctx.needs_input_grad[2 + 4 * i:6 + 4 * i]
-            out += [None, grads[i][0] if need_a else None, grads[i][1] if need_b else None,
-                    gy2[i].sum(dim=0) if (ctx.has_bias[i] and need_bias) else None]
-        return tuple(out)
+        return _group_backward(ctx, x2, h_cat, weights, las, lbs, gy2)
+
+
+def _group_backward(ctx, x2, h_cat, weights, las, lbs, gy2):
+    """Gradients of a group call in the order of its inputs (x, scales, then weight, lora_a, lora_b, bias per member)."""
+    n = len(ctx.scales)
+    members = [ops.GroupMember(w.quantized_data, w.block_scalers(), tr, a, b, None, s, w.shape[0])
+               for w, tr, a, b, s in zip(weights, _copies(weights, x2.shape[0]), las, lbs, ctx.scales)]
+    need_x = ctx.needs_input_grad[0]
+    gx, grads, _ = ops.lora_group_bwd(x2, h_cat, members, gy2, want_gx=need_x)
+    out: List = [gx.view(ctx.x_shape) if need_x else None, None]
+    for i in range(n):
+        _, need_a, need_b, need_bias = ctx.needs_input_grad[2 + 4 * i:6 + 4 * i]
+        out += [None, grads[i][0] if need_a else None, grads[i][1] if need_b else None,
+                gy2[i].sum(dim=0) if (ctx.has_bias[i] and need_bias) else None]
+    return tuple(out)
+
+
+class _QLoRAGatedFn(torch.autograd.Function):
+    """``silu(w1(x)) * w3(x)`` for two LoRA linears over NF4 (``torchtune/modules/feed_forward.py:50-53``).  Inputs as
+    for ``_QLoRAGroupFn`` with the members (w1, w3); the one output is the gated product.  The two projections are
+    kept for backward, as autograd keeps them for the reference's separate multiply."""
+
+    @staticmethod
+    def forward(ctx, x, scales: Tuple[float, ...], *flat):
+        weights, las, lbs, biases = flat[0::4], flat[1::4], flat[2::4], flat[3::4]
+        K = weights[0].shape[1]
+        for w in weights:
+            _check_in_features(x, w)
+        x2 = x.reshape(-1, K)
+        members = [ops.GroupMember(w.quantized_data, w.block_scalers(), tr, a, b, bias, s, w.shape[0])
+                   for w, tr, a, b, bias, s in zip(weights, _copies(weights, x2.shape[0]), las, lbs, biases, scales)]
+        h_cat, (gate, up, act) = ops.lora_group_fwd(x2, members, swiglu=True)
+        ctx.save_for_backward(x2, h_cat, gate, up, *weights, *las, *lbs)
+        ctx.scales = scales
+        ctx.x_shape = x.shape
+        ctx.has_bias = tuple(b is not None for b in biases)
+        return act.view(*x.shape[:-1], act.shape[-1])
+
+    @staticmethod
+    def backward(ctx, gact):
+        saved = ctx.saved_tensors
+        x2, h_cat, gate, up = saved[:4]
+        rest = saved[4:]
+        weights, las, lbs = rest[:2], rest[2:4], rest[4:6]
+        ggate, gup = ops.swiglu_bwd(gact.reshape(gate.shape), gate, up)
+        return _group_backward(ctx, x2, h_cat, weights, las, lbs, [ggate, gup])
 
 
 def group_applies(x: torch.Tensor, layers: Sequence[torch.nn.Module]) -> bool:
@@ -88,6 +125,17 @@ def group_applies(x: torch.Tensor, layers: Sequence[torch.nn.Module]) -> bool:
         if not ops.group_dx_expands(M, layers[0].in_dim, [l.out_dim for l in layers]):
             return False
     return ops.group_shape_ok([l.out_dim for l in layers], layers[0].in_dim, [l.rank for l in layers])
+
+
+def lora_swiglu_group(x: torch.Tensor, gate: torch.nn.Module, up: torch.nn.Module):
+    """``silu(gate(x)) * up(x)`` (``torchtune/modules/feed_forward.py:50-53``) with the product formed in the epilogue of
+    the pair's one GEMM launch where the group kernels apply; ``None`` when they do not (the caller multiplies itself)."""
+    if not group_applies(x, (gate, up)) or gate.out_dim != up.out_dim:
+        return None
+    flat = []
+    for layer in (gate, up):
+        flat += [layer.weight, layer.lora_a.weight, layer.lora_b.weight, layer.bias]
+    return _QLoRAGatedFn.apply(x, tuple(layer.alpha / layer.rank for layer in (gate, up)), *flat)
 
 
 def lora_linear_group(x: torch.Tensor, layers: Sequence[torch.nn.Module]) -> Tuple[torch.Tensor, ...]:

@@ -412,12 +412,17 @@ def _group_array(what: str, members: Sequence[GroupMember], K: int, ys: Sequence
     return arr, keep
 
 
-def lora_group_fwd(x: torch.Tensor, members: Sequence[GroupMember]):
+def lora_group_fwd(x: torch.Tensor, members: Sequence[GroupMember], swiglu: bool = False):
     """-> (h_cat [M, sum of ranks], [y_i [M, N_i]]): every member's ``y_i = x @ D(W_i).T (+ bias_i) + scale_i * h_i @ B_i.T``
-    with ``h_i = x @ A_i.T`` (columns of ``h_cat``), in one pass over ``x`` for the hidden products."""
+    with ``h_i = x @ A_i.T`` (columns of ``h_cat``), in one pass over ``x`` for the hidden products.
+
+    ``swiglu=True`` (two members of equal width: gate, up) appends ``act = silu(y_0) * y_1`` to the list, formed in the
+    epilogue of the GEMM launch where the many-token path serves the shape (``ttamd_nf4_lora_group_swiglu_fwd_bf16``)."""
     x = _bf16_2d(x, "lora_group_fwd")
     M, K = x.shape
     dev = x.device
+    if swiglu and (len(members) != 2 or members[0].N != members[1].N):
+        raise ValueError("lora_group_fwd: swiglu takes the gate and the up projection, two members of equal width")
     ys = [torch.empty(M, m.N, dtype=torch.bfloat16, device=dev) for m in members]
     arr, keep = _group_array("lora_group_fwd", members, K, ys, M)
     n = len(members)
@@ -434,12 +439,17 @@ def lora_group_fwd(x: torch.Tensor, members: Sequence[GroupMember]):
         events = _gemm_timer("fwd_group", M, [m.N for m in members], K, [int(e.rank) for e in arr]) if _gemm_timer is not None else None
         if events:
             events[0].record()
-        rc = lib.ttamd_nf4_lora_group_fwd_bf16(x.data_ptr(), arr, n, h_cat.data_ptr(), M, K, ws.data_ptr(), ws.numel(), _stream(x))
+        if swiglu:
+            act = torch.empty(M, members[0].N, dtype=torch.bfloat16, device=dev)
+            rc = lib.ttamd_nf4_lora_group_swiglu_fwd_bf16(x.data_ptr(), arr, n, h_cat.data_ptr(), act.data_ptr(), M, K, ws.data_ptr(),
+                                                          ws.numel(), _stream(x))
+        else:
+            rc = lib.ttamd_nf4_lora_group_fwd_bf16(x.data_ptr(), arr, n, h_cat.data_ptr(), M, K, ws.data_ptr(), ws.numel(), _stream(x))
         if events:
             events[1].record()
     _lib.check(rc, "lora_group_fwd")
     del keep
-    return h_cat, ys
+    return h_cat, (ys + [act] if swiglu else ys)
 
 
 def lora_group_bwd(x: torch.Tensor, h_cat: torch.Tensor, members: Sequence[GroupMember], gys: Sequence[torch.Tensor],
