@@ -75,7 +75,7 @@ class GemmTimer:
 
     def __call__(self, kind, M, N, K, rank):
         # "fwd" / "bwd": one layer, one call of the library.  "fwd_group" / "bwd_group": the layers of a group with a common
-        # input (N and rank are lists), one call.  Between the events lie all launches of the call: with the weight expanded
+        # input (N and rank are lists), one call; "fwd_gated": the gate / up pair with its gated product in the same call.  Between the events lie all launches of the call: with the weight expanded
         # once per call (many tokens) one expansion launch per member and one GEMM launch; otherwise one fused launch per
         # member (forward) or the single fused grad-input launch over all members' output columns.
         from torchtune_amd import _lib, ops
@@ -104,6 +104,8 @@ class GemmTimer:
         if fwd:
             launches = 1 if expanded else len(Ns)
             nbytes = (2.0 * M * K if expanded else 2.0 * M * K * len(Ns)) + sum(2.0 * M * n + per_w * n * K + 2.0 * r * (M + n) for n, r in zip(Ns, ranks))
+            if kind == "fwd_gated":  # the gate / up pair: silu(gate) * up written as well (by a pass of its own when not expanded)
+                nbytes += 2.0 * M * Ns[0] * (1 if expanded else 3)
         else:
             launches = 1
             nbytes = 2.0 * M * K + sum(2.0 * M * n + per_w * n * K + 2.0 * r * (M + K) for n, r in zip(Ns, ranks))

@@ -436,7 +436,8 @@ def lora_group_fwd(x: torch.Tensor, members: Sequence[GroupMember], swiglu: bool
     with torch.cuda.device(dev):
         rc = lib.ttamd_lora_group_hidden_bf16(x.data_ptr(), arr, n, h_cat.data_ptr(), M, K, ws.data_ptr(), ws.numel(), _stream(x))
         _lib.check(rc, "lora_group_hidden")
-        events = _gemm_timer("fwd_group", M, [m.N for m in members], K, [int(e.rank) for e in arr]) if _gemm_timer is not None else None
+        events = (_gemm_timer("fwd_gated" if swiglu else "fwd_group", M, [m.N for m in members], K, [int(e.rank) for e in arr])
+                  if _gemm_timer is not None else None)
         if events:
             events[0].record()
         if swiglu:
