@@ -212,6 +212,8 @@ GATED_SHAPES = [
     (2048 + 192, 512, 4096, (16, 8), True),     # a last row tile with 192 rows
     (4096, 1024, 2048, (32, 0 + 16), False),
     (8192, 256, 1024, (16, 16), True),
+    (8192, 4096, 14336, (16, 16), False),       # the 8B feed-forward at its real size (batch 4 x 2048)
+    (4096, 8192, 28672, (16, 16), False),       # the 70B feed-forward (batch 1 x 4096)
     (16, 512, 1024, (8, 8), False),             # few tokens: group launch + a pass of its own
     (300, 512, 512, (16, 16), True),            # tiled kernels + a pass of its own
     (2048, 256, 1152, (16, 16), False),         # many tokens, too few tiles for the expanded path
