@@ -226,7 +226,8 @@ int ttamd_nf4_linear_bwd_dx_bf16(const void* gy, const uint8_t* quantized_data, 
  *   ttamd_nf4_linear_bwd_dx_ws_bf16: slices only the variant with the transposed copies.
  * A workspace smaller than ttamd_nf4_gemm_workspace_bytes says, or NULL, runs the unsliced kernel.
  *
- * Many tokens (M >= 2048 and at least 256 output tiles of 256 x 256): the same workspace argument then holds the
+ * Many tokens (M >= 2048 and at least 256 output tiles of 256 x 256, or M >= 1280 and more than 128 such tiles, where
+ * the fused kernel would need a second round of its 128-row tiles): the same workspace argument then holds the
  * weight expanded ONCE per call to bf16 (2 * n_out * k_contract bytes, in the order the matrix cores read it), and a
  * plain bf16 GEMM with the adapter, bias and column scale in its epilogue runs on it: the reference's own order of
  * work, F.linear(x, weight.to(dtype)) (torchao linear_nf4, reached from torchtune/modules/peft/lora.py:138), for the

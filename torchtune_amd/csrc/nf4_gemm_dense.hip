@@ -675,13 +675,22 @@ int launch_dense(DenseArgs& g, hipStream_t s) {
 
 }  // namespace
 
-// Fewest tokens from which the expand-once path is taken (below, the fused kernel's repeated expansion is cheaper than
-// one pass of the expansion kernel plus the traffic of the scratch copy).
-constexpr int64_t kDenseMinRows = 2048;
+// When the expand-once path is taken, from its 256 x 256 output tiles against the 256 CUs (measured against the fused
+// kernel, whose tiles have 128 rows, on 8B / 70B shapes):
+//   * at least a full round of tiles and 2048 tokens: always (below 2048 tokens the expansion, which costs as much as
+//     the GEMM of ~360 tokens, and the second round eat the gain);
+//   * between half a round and a full one, from 1280 tokens: the fused kernel needs a second round of its tiles there
+//     (+ 60 %), one partly filled round of this kernel is 15 - 30 % faster;
+//   * up to half a round the fused kernel fills the chip in one round of its own and wins.
+constexpr int64_t kDenseMinRows = 2048, kDenseMinRowsPartRound = 1280;
+
+bool dense_tiles_apply(int64_t M, int64_t tiles) {
+  return (M >= kDenseMinRows && tiles >= 256) || (M >= kDenseMinRowsPartRound && tiles > 128 && tiles < 256);
+}
 
 bool dense_path_applies(int64_t M, int64_t Nout, int64_t Kc) {
-  if (M < kDenseMinRows || Nout % 64 != 0 || Kc % 64 != 0) return false;
-  if (((M + 255) / 256) * ((Nout + 255) / 256) < 256) return false;  // fewer tiles than CUs: the fused kernel has 128-row tiles
+  if (Nout % 64 != 0 || Kc % 64 != 0) return false;
+  if (!dense_tiles_apply(M, ((M + 255) / 256) * ((Nout + 255) / 256))) return false;
   // per-lane byte offsets inside the kernel are 32-bit
   return M * Kc * 2 < (int64_t(1) << 32) && Kc * 2 * 256 < (int64_t(1) << 32);
 }
@@ -783,7 +792,7 @@ size_t dense_group_dx_workspace_bytes(const GroupDx& d) {
     n_total += d.N[i];
     if (d.M * d.N[i] * 2 >= (int64_t(1) << 32)) return 0;
   }
-  if (d.M < kDenseMinRows || d.K % 64 != 0 || ((d.M + 255) / 256) * ((d.K + 255) / 256) < 256) return 0;
+  if (d.K % 64 != 0 || !dense_tiles_apply(d.M, ((d.M + 255) / 256) * ((d.K + 255) / 256))) return 0;
   return (size_t)d.K * (size_t)n_total * 2;
 }
 
