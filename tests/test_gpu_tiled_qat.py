@@ -92,12 +92,14 @@ def test_qat_linear_on_the_tiled_gemm_vs_oracle_and_vs_default_path(bias, monkey
 
     def run(tiled):
         monkeypatch.setattr(qat, "TILED_GEMM", tiled)
+        monkeypatch.setattr(qat, "TILED_GEMM_MIN_TILES", 0)   # a small layer: the path is chosen from a full round of tiles up
         lin = Int8DynActInt4WeightQATLinear(K, N, bias=bias, device=DEV, groupsize=g, precision=BF)
         with torch.no_grad():
             lin.weight.copy_(w)
             if bias:
                 lin.bias.copy_(b)
         xd = x.to(DEV).requires_grad_()
+        assert lin._tiled_ok(xd) == tiled
         y = lin(xd)
         (y.float() ** 2).sum().backward()
         return y.detach(), xd.grad, lin.weight.grad, (lin.bias.grad if bias else None), lin.weight_fake_quantizer.scale

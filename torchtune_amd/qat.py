@@ -242,9 +242,12 @@ class FakeQuantizer(nn.Module):
 # FakeQuantizedLinear on the library's own GEMM: the weight's fake quantisation is written in the GEMM's tile order (once
 # for the forward, once transposed for the grad-input) and never row-major; forward and grad-input run on
 # ``ttamd_tiled_linear_bf16``, the weight gradient on ``ttamd_gemm_tn_bf16`` (layers of fewer than 192 output tiles of
-# 256 x 256: the vendor library).  False: row-major fq(W) and ``F.linear`` for everything.
+# 256 x 256: the vendor library).  Taken from ``TILED_GEMM_MIN_ROWS`` tokens and a full round of 256 x 256 tiles on the
+# 256 CUs in both directions (``TILED_GEMM_MIN_TILES``); with fewer, the vendor library's smaller tiles fill the chip
+# better (M = 2048, 4096 x 4096: 62 against 80 us).  ``TILED_GEMM = False``: row-major fq(W) and ``F.linear`` for everything.
 TILED_GEMM = True
 TILED_GEMM_MIN_ROWS = 2048
+TILED_GEMM_MIN_TILES = 256
 TN_GEMM_MIN_TILES = 192
 
 
@@ -320,7 +323,11 @@ class FakeQuantizedLinear(nn.Linear):
         if not (isinstance(c.granularity, PerGroup) and c.dtype == torch.int4 and c.is_symmetric):
             return False
         rows = x.numel() // max(1, x.shape[-1])
-        return (x.shape[-1] == self.in_features and rows >= TILED_GEMM_MIN_ROWS
+        # a full round of 256 x 256 output tiles on the 256 CUs in both directions (forward: rows x out_features,
+        # grad-input: rows x in_features); with fewer the vendor library's smaller tiles fill the chip better
+        row_tiles = (rows + 255) // 256
+        full_round = row_tiles * min(self.out_features // 256, self.in_features // 256) >= TILED_GEMM_MIN_TILES
+        return (x.shape[-1] == self.in_features and rows >= TILED_GEMM_MIN_ROWS and full_round
                 and ops.tiled_weight_shape_ok(self.out_features, self.in_features, c.group_size))
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
