@@ -14,7 +14,11 @@
  *     a thread-local, human-readable message;
  *   - nothing here allocates or frees device memory: scratch space is passed in as `workspace`,
  *     sized by the matching `*_workspace_bytes` query;
- *   - the calls are re-entrant and keep no stream or device state between calls.
+ *   - the calls are re-entrant and keep no stream or device state between calls.  The one piece of process-wide
+ *     state: the GEMM kernels that use more than 64 KB of LDS record per device, in a flag, that the runtime has
+ *     been told so (`hipFuncSetAttribute`, once per device and kernel); two threads racing on a device's first call
+ *     both make that call, which is harmless.  ttamd_lora_hidden_static_bf16 alone owns device memory (a fixed
+ *     2 MiB array per GPU, see there).
  *
  * dtype codes: TTAMD_BF16 = bfloat16, TTAMD_F32 = float32.
  */
