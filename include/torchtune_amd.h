@@ -470,6 +470,17 @@ int ttamd_fq_per_group_int4_sym_tiled_bf16(const void* w, int64_t N, int64_t K, 
                                            void* tiled_fwd, void* tiled_bwd, float* scale, void* stream);
 int ttamd_tiled_linear_bf16(const void* x, const void* tiled_weight, const void* bias, void* y, int64_t M, int64_t n_out,
                             int64_t k_contract, void* stream);
+/*
+ * The same GEMM with a low-rank adapter in its epilogue, for QATLoRALinear.forward (torchtune/modules/peft/lora.py:248-264:
+ * F.linear(fq(x), fq(W)) + (alpha / r) * lora_b(lora_a(x)), base weight frozen) and its grad-input:
+ *   y[M, n_out] = x . Wd^T (+ bias) + lscale * lx[M, rank] . lw^T
+ * forward:    x = fq(x), Wd = tiled_fwd, lx = x . lora_a^T (ttamd_lora_hidden_bf16 on the unquantised x), lw = lora_b [N, rank]
+ *             (lw_row_major = 1), lscale = alpha / rank;
+ * grad-input: x = gy, Wd = tiled_bwd, lx = gh (ttamd_lora_bwd_bf16), lw = lora_a [rank, K] (lw_row_major = 0), lscale = 1.
+ * rank a multiple of 8, at most 64 (0: no adapter, = ttamd_tiled_linear_bf16).
+ */
+int ttamd_tiled_lora_linear_bf16(const void* x, const void* tiled_weight, const void* lx, const void* lw, int lw_row_major, int rank,
+                                 float lscale, const void* bias, void* y, int64_t M, int64_t n_out, int64_t k_contract, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
  * Neighbours of the quantized linears inside a decoder layer (one pass over HBM each, bf16 tensors, fp32 math).

@@ -379,6 +379,72 @@ def test_qat_lora_linear_forward_backward_and_frozen_weight_cache():
         ops.set_fq_timer(None)
 
 
+def test_qat_lora_linear_on_the_tiled_gemm_many_tokens():
+    """QATLoRALinear.forward (torchtune/modules/peft/lora.py:248-264) at a training size: the frozen weight's fake
+    quantisation held in the GEMM's tile order, base product and adapter from one launch per direction
+    (``ttamd_tiled_lora_linear_bf16``).  Compared with the layer's eager composition (``TILED_GEMM = False``: F.linear on
+    the row-major fake-quantised weight plus the adapter's two matmuls) and with the oracle's fake quantisation in fp32:
+    output, grad-input and adapter gradients (rtol 1e-2 / atol scaled with the magnitude of the result, the bar of the
+    other GEMM tests); the tiles are rebuilt when the weight is written."""
+    from torchtune_amd.modules.peft import LoRALinear, QATLoRALinear
+
+    gen = torch.Generator().manual_seed(3)
+    K, N, r, alpha, g, M = 2048, 2048, 16, 32.0, 32, 8192 + 64   # 33 x 8 = 264 tiles of 256 x 256 in both directions
+    W = (torch.randn(N, K, generator=gen) * 0.02).to(torch.bfloat16)
+    A = (torch.randn(r, K, generator=gen) * 0.02).to(torch.bfloat16)
+    B = (torch.randn(N, r, generator=gen) * 0.02).to(torch.bfloat16)
+    x = torch.randn(M, K, generator=gen).to(torch.bfloat16)
+    gy = (torch.randn(M, N, generator=gen) * 0.1).to(torch.bfloat16)
+    prev = torch.get_default_dtype()
+    torch.set_default_dtype(torch.bfloat16)
+    try:
+        with torch.device(DEV):
+            base = LoRALinear(K, N, rank=r, alpha=alpha)
+    finally:
+        torch.set_default_dtype(prev)
+    with torch.no_grad():
+        base.weight.copy_(W.to(DEV))
+        base.lora_a.weight.copy_(A.to(DEV))
+        base.lora_b.weight.copy_(B.to(DEV))
+    layer = QATLoRALinear.from_lora_linear(
+        base, FakeQuantizeConfig(torch.int8, "per_token", is_symmetric=False), FakeQuantizeConfig(torch.int4, group_size=g))
+    layer.weight.requires_grad_(False)
+
+    def run(tiled):
+        layer.TILED_GEMM = tiled
+        layer.zero_grad()
+        xd = x.to(DEV).requires_grad_()
+        assert layer._tiled_ok(xd) == tiled
+        y = layer(xd)
+        y.backward(gy.to(DEV))
+        return y.detach(), xd.grad, layer.lora_a.weight.grad.clone(), layer.lora_b.weight.grad.clone()
+
+    try:
+        y1, gx1, ga1, gb1 = run(True)
+        y0, gx0, ga0, gb0 = run(False)
+    finally:
+        layer.TILED_GEMM = True
+    assert layer.weight.grad is None
+    for a, b in ((y1, y0), (gx1, gx0), (ga1, ga0), (gb1, gb0)):
+        torch.testing.assert_close(a.float(), b.float(), rtol=1e-2, atol=1e-2 * max(1.0, float(b.float().abs().max()) / 8))
+    # the oracle's fake quantisation, products in fp32 (row blocks keep the CPU work small)
+    rows = slice(0, 512)
+    x_fq, _, _ = fq.fq_per_token_int8_asym(x[rows])
+    w_fq, w_scale = fq.fq_per_group_int4_sym(W, g)
+    want = x_fq.float() @ w_fq.float().T + (alpha / r) * ((x[rows].float() @ A.float().T) @ B.float().T)
+    torch.testing.assert_close(y1[rows].float().cpu(), want, rtol=1e-2, atol=1e-2)
+    want_gx = gy[rows].float() @ w_fq.float() + (alpha / r) * ((gy[rows].float() @ B.float()) @ A.float())
+    torch.testing.assert_close(gx1[rows].float().cpu(), want_gx, rtol=1e-2, atol=1e-2 * max(1.0, float(want_gx.abs().max()) / 8))
+    assert torch.equal(layer.weight_fake_quantizer.scale.float().cpu(), w_scale)
+    # writing the weight rebuilds the tiles
+    with torch.no_grad():
+        layer.weight.copy_((W.float() * 1.5).to(torch.bfloat16).to(DEV))
+    y2 = layer(x.to(DEV))
+    w2_fq, _ = fq.fq_per_group_int4_sym((W.float() * 1.5).to(torch.bfloat16), g)
+    want2 = x_fq.float() @ w2_fq.float().T + (alpha / r) * ((x[rows].float() @ A.float().T) @ B.float().T)
+    torch.testing.assert_close(y2[rows].float().cpu(), want2, rtol=1e-2, atol=1e-2)
+
+
 def test_per_token_result_is_shared_between_sibling_quantizers(monkeypatch):
     """q/k/v (and gate/up) fake-quantise the same activation tensor: the second and third quantizer reuse the first
     one's result while the very same, unmodified tensor object comes in; a modified or different tensor is recomputed;

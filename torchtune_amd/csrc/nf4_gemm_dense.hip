@@ -859,26 +859,49 @@ extern "C" int ttamd_fq_per_group_int4_sym_tiled_bf16(const void* w, int64_t N, 
   return check_launch("fq_per_group_int4_sym_tiled");
 }
 
-extern "C" int ttamd_tiled_linear_bf16(const void* x, const void* tiled_weight, const void* bias, void* y, int64_t M, int64_t n_out,
-                                       int64_t k_contract, void* stream) {
+namespace {
+int tiled_linear(const void* x, const void* tiled_weight, const void* lx, const void* lw, bool lw_row_major, int rank, float lscale,
+                 const void* bias, void* y, int64_t M, int64_t n_out, int64_t k_contract, void* stream) {
   TT_REQUIRE(x && tiled_weight && y && aligned16(x) && aligned16(tiled_weight) && aligned16(y), "tiled_linear: pointers must be non-null and 16-byte aligned");
   TT_REQUIRE(bias == nullptr || (reinterpret_cast<uintptr_t>(bias) & 7u) == 0, "tiled_linear: bias must be 8-byte aligned");
   TT_REQUIRE(M > 0 && n_out > 0 && k_contract > 0 && n_out % 64 == 0 && k_contract % 64 == 0,
              "tiled_linear: n_out (%lld) and k_contract (%lld) must be positive multiples of 64", (long long)n_out, (long long)k_contract);
   if (!(M * k_contract * 2 < (int64_t(1) << 32) && k_contract * 2 * 256 < (int64_t(1) << 32) && M < (1 << 30) && n_out < (1 << 30)))
     return fail(TTAMD_EUNSUPPORTED, "tiled_linear: operands too large for 32-bit offsets (M=%lld k=%lld)", (long long)M, (long long)k_contract);
+  TT_REQUIRE(rank >= 0 && rank % 8 == 0 && rank <= 64, "tiled_linear: the adapter rank (%d) must be a multiple of 8, at most 64", rank);
+  TT_REQUIRE(rank == 0 || (lx && lw && aligned16(lx) && aligned16(lw)), "tiled_linear: adapter operands must be non-null and 16-byte aligned");
   DenseArgs g = {};
   g.nseg = g.nout = 1;
-  g.nad = 0;
+  g.nad = rank > 0 ? 1 : 0;
   g.seg[0].X = reinterpret_cast<const uint16_t*>(x);
   g.seg[0].Kc = (int)k_contract;
   g.out[0].C = reinterpret_cast<uint16_t*>(y);
   g.out[0].bias = reinterpret_cast<const uint16_t*>(bias);
   g.out[0].n_begin = 0;
   g.out[0].width = (int)n_out;
+  if (rank > 0) {
+    g.ad[0].lX = reinterpret_cast<const uint16_t*>(lx);
+    g.ad[0].lW = reinterpret_cast<const uint16_t*>(lw);
+    g.ad[0].R = rank;
+    g.ad[0].n_begin = 0;
+    g.ad[0].n_end = (int)n_out;
+    g.ad[0].lscale = lscale;
+  }
   g.Wt = reinterpret_cast<const char*>(tiled_weight);
   g.M = (int)M; g.Nout = (int)n_out; g.Kc = (int)k_contract;
-  g.lw_row_major = 1;
-  g.ldlx = 0;
+  g.lw_row_major = lw_row_major ? 1 : 0;
+  g.ldlx = rank;
   return launch_dense(g, reinterpret_cast<hipStream_t>(stream));
+}
+}  // namespace
+
+extern "C" int ttamd_tiled_linear_bf16(const void* x, const void* tiled_weight, const void* bias, void* y, int64_t M, int64_t n_out,
+                                       int64_t k_contract, void* stream) {
+  return tiled_linear(x, tiled_weight, nullptr, nullptr, true, 0, 1.0f, bias, y, M, n_out, k_contract, stream);
+}
+
+extern "C" int ttamd_tiled_lora_linear_bf16(const void* x, const void* tiled_weight, const void* lx, const void* lw, int lw_row_major,
+                                            int rank, float lscale, const void* bias, void* y, int64_t M, int64_t n_out,
+                                            int64_t k_contract, void* stream) {
+  return tiled_linear(x, tiled_weight, lx, lw, lw_row_major != 0, rank, lscale, bias, y, M, n_out, k_contract, stream);
 }

@@ -120,6 +120,38 @@ class LoRALinear(LowRankAdapterLinear):
         return out + scale * self.lora_b(self.lora_a(self.dropout(x)))
 
 
+class _QATLoRATiledFn(torch.autograd.Function):
+    """QAT + LoRA linear on the library's own GEMM.  Inputs: x [..., K] bf16 (the adapter's input), x_fq (the base path's
+    input: x fake-quantised, or x itself), the frozen base weight's fake quantisation in the GEMM's tile order (forward
+    and transposed), lora_a [r, K], lora_b [N, r].  The adapter product rides in the epilogue of the base GEMM in both
+    directions; the activation's fake quantisation is straight-through, so the grad-input of both paths is one tensor."""
+
+    @staticmethod
+    def forward(ctx, x, x_fq, tiled_fwd, tiled_bwd, lora_a, lora_b, scale: float):
+        N, K = lora_b.shape[0], lora_a.shape[1]
+        x2 = x.reshape(-1, K)
+        h = ops.lora_hidden(x2, lora_a)
+        y = ops.tiled_lora_linear(x_fq.reshape(-1, K), tiled_fwd, N, h, lora_b, scale, lw_row_major=True)
+        ctx.save_for_backward(x2, h, tiled_bwd, lora_a, lora_b)
+        ctx.scale = scale
+        ctx.x_shape = x.shape
+        return y.view(*x.shape[:-1], N)
+
+    @staticmethod
+    def backward(ctx, gy):
+        x2, h, tiled_bwd, lora_a, lora_b = ctx.saved_tensors
+        N, K = lora_b.shape[0], lora_a.shape[1]
+        gy2 = gy.reshape(-1, N)
+        need_x, need_xfq, _, _, need_a, need_b, _ = ctx.needs_input_grad
+        gh, ga, gb = ops.lora_bwd(gy2, x2, h, lora_b, ctx.scale)
+        gx = None
+        if need_x or need_xfq:
+            gx = ops.tiled_lora_linear(gy2, tiled_bwd, K, gh, lora_a, 1.0, lw_row_major=False).view(ctx.x_shape)
+        # x and x_fq are the same tensor up to the straight-through fake quantisation: the whole gradient goes to x
+        return (gx if need_x else None), (gx if need_xfq and not need_x else None), None, None, ga if need_a else None, \
+            gb if need_b else None, None
+
+
 class QATLoRALinear(LoRALinear):
     """LoRA linear whose frozen base path sees fake-quantised activations and weights:
     ``x -> fq(W) fq(x) + (alpha / r) B A x``.
@@ -182,7 +214,49 @@ class QATLoRALinear(LoRALinear):
             self._fq_weight_cache = cached
         return cached[1]
 
+    # From this many tokens (and a full round of 256 x 256 output tiles in both directions) the layer runs on the library's
+    # own GEMM: the frozen weight's fake quantisation is kept in the GEMM's tile order, forward and transposed (4 B per
+    # element instead of the 2 B of the row-major copy), and the adapter product is part of the GEMM's epilogue.
+    TILED_GEMM = True
+    TILED_GEMM_MIN_ROWS = 2048
+
+    def _tiled_weights(self):
+        """(tiled_fwd, tiled_bwd) of the frozen weight's fake quantisation, rebuilt when the weight is written."""
+        w, c = self.weight, self.weight_fake_quantizer.config
+        key = (w.data_ptr(), w._version, tuple(w.shape), c.group_size, c.scale_precision, c.eps)
+        cached = getattr(self, "_tiled_weight_cache", None)
+        if cached is None or cached[0] != key:
+            with torch.no_grad():
+                tf, tb, scale = ops.fq_per_group_int4_sym_tiled(w.detach(), c.group_size, qparam_dtype=c.scale_precision, eps=c.eps)
+            # what a call of the quantizer leaves behind
+            self.weight_fake_quantizer.scale = scale.to(c.scale_precision)
+            self.weight_fake_quantizer.zero_point = None
+            cached = (key, tf, tb)
+            self._tiled_weight_cache = cached
+        return cached[1], cached[2]
+
+    def _tiled_ok(self, x: torch.Tensor) -> bool:
+        from ...qat import FakeQuantizer, PerGroup
+
+        q = self.weight_fake_quantizer
+        if (not self.TILED_GEMM or self.disabled or not isinstance(q, FakeQuantizer) or not q.enabled or not x.is_cuda
+                or x.dtype != torch.bfloat16 or self.weight.dtype != torch.bfloat16 or self.weight.requires_grad
+                or self.lora_a.weight.dtype != torch.bfloat16 or self.rank % 8 != 0 or not 0 < self.rank <= 64
+                or x.shape[-1] != self.in_dim or (self.training and getattr(self.dropout, "p", 0.0) > 0.0)):
+            return False
+        c = q.config
+        if not (isinstance(c.granularity, PerGroup) and c.dtype == torch.int4 and c.is_symmetric):
+            return False
+        rows = x.numel() // self.in_dim
+        full_round = ((rows + 255) // 256) * min(self.out_dim // 256, self.in_dim // 256) >= 256
+        return rows >= self.TILED_GEMM_MIN_ROWS and full_round and ops.tiled_weight_shape_ok(self.out_dim, self.in_dim, c.group_size)
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
+        if self._tiled_ok(x):
+            tf, tb = self._tiled_weights()
+            # the activation's fake quantisation is straight-through: its input takes the whole gradient inside the node
+            return _QATLoRATiledFn.apply(x, self.activation_fake_quantizer(x).detach(), tf, tb, self.lora_a.weight,
+                                         self.lora_b.weight, self.alpha / self.rank)
         out = F.linear(self.activation_fake_quantizer(x), self._fake_quantized_weight())
         if self.disabled:
             return out

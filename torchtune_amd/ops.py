@@ -636,6 +636,39 @@ def tiled_linear(x: torch.Tensor, tiled: torch.Tensor, n_out: int, bias: Optiona
     return y
 
 
+def tiled_lora_linear(x: torch.Tensor, tiled: torch.Tensor, n_out: int, lx: torch.Tensor, lw: torch.Tensor, lscale: float,
+                      lw_row_major: bool, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``tiled_linear`` with a low-rank adapter in the GEMM's epilogue: ``y = x @ Wd.T (+ bias) + lscale * lx @ lw.T``
+    with ``lw`` [n_out, r] (``lw_row_major``, the forward: ``lora_b``) or ``lw.T`` given as [r, n_out] (the grad-input:
+    ``lora_a``)."""
+    x = _bf16_2d(x, "tiled_lora_linear")
+    lx = _bf16_2d(lx, "tiled_lora_linear")
+    lw = _bf16_2d(lw, "tiled_lora_linear")
+    M, K = x.shape
+    r = lx.shape[1]
+    if tiled.dtype != torch.bfloat16 or tiled.numel() != n_out * K or not tiled.is_contiguous():
+        raise ValueError(f"tiled_lora_linear: the tiled weight must be a contiguous bfloat16 tensor of {n_out} x {K} elements")
+    if lx.shape[0] != M or tuple(lw.shape) != ((n_out, r) if lw_row_major else (r, n_out)) or r % 8 != 0 or not 0 < r <= 64:
+        raise ValueError(f"tiled_lora_linear: adapter operands {tuple(lx.shape)} / {tuple(lw.shape)} do not fit M={M}, n_out={n_out} "
+                         "(rank: a multiple of 8, at most 64)")
+    if bias is not None:
+        bias = bias.contiguous()
+        if bias.dtype != torch.bfloat16 or bias.numel() != n_out:
+            raise ValueError(f"tiled_lora_linear: bias must be bfloat16 with {n_out} elements")
+    y = torch.empty(M, n_out, dtype=torch.bfloat16, device=x.device)
+    lib = _lib.load()
+    with torch.cuda.device(x.device):
+        events = _gemm_timer("tiled", M, n_out, K, 0) if _gemm_timer is not None else None
+        if events:
+            events[0].record()
+        rc = lib.ttamd_tiled_lora_linear_bf16(x.data_ptr(), tiled.data_ptr(), lx.data_ptr(), lw.data_ptr(), 1 if lw_row_major else 0, r,
+                                              float(lscale), _ptr(bias), y.data_ptr(), M, n_out, K, _stream(x))
+        if events:
+            events[1].record()
+    _lib.check(rc, "tiled_lora_linear")
+    return y
+
+
 def gemm_tn_applies(M: int, N: int, K: int) -> bool:
     """Shapes ``gemm_tn`` serves: M a multiple of 32, N and K multiples of 256."""
     return bool(_lib.load().ttamd_gemm_tn_applies(M, N, K))
