@@ -10,6 +10,8 @@
 // apart, one in its MFMA part while the other requests loads and reads operands, swapping at workgroup barriers.
 // LDS layout of a stage: row r of the 32 at r * 512, its 16-byte chunk c in slot c ^ (2 (r % 4)) - applied on the
 // global-address side of the loads - so that the four rows a 16-lane group reads together fall on disjoint banks.
+#include <type_traits>
+
 #include "common.h"
 #include "nf4_math.h"
 
@@ -148,37 +150,45 @@ __global__ __launch_bounds__(512) void gemm_tn_kernel(const TnArgs g) {
   issue(2);
   asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");  // step 0 landed everywhere
   if (wm == 1) asm volatile("s_barrier" ::: "memory");
-  for (int t = 0; t < nk; ++t) {
-    issue(t + 3);
-    read_step(t);
-    __builtin_amdgcn_sched_barrier(0);
-    // what the waves with wm = 1 read here is overwritten by requests the waves with wm = 0 issue right after the next
-    // barrier: they let their reads complete before they pass it (the others' reads have a whole interval more)
-    if (wm == 1)
-      asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-    else
-      asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");
-    __builtin_amdgcn_sched_barrier(0);
-    __builtin_amdgcn_s_setprio(1);
+  // one copy of the loop per wave group: the two differ in one wait, and a branch per step costs 2 - 4 %
+  auto main_loop = [&](auto lgkm) {
+    constexpr bool kLgkm = decltype(lgkm)::value;
+    for (int t = 0; t < nk; ++t) {
+      issue(t + 3);
+      read_step(t);
+      __builtin_amdgcn_sched_barrier(0);
+      // what the waves with wm = 1 read here is overwritten by requests the waves with wm = 0 issue right after the next
+      // barrier: they let their reads complete before they pass it (the others' reads have a whole interval more)
+      if constexpr (kLgkm)
+        asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      else
+        asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");
+      __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_setprio(1);
 #pragma unroll
-    for (int j = 0; j < NT; ++j)
-      asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(blo[j]), "+v"(bhi[j]) : "n"(kLgkmMax < 2 * MT + 2 * (NT - 1 - j) ? kLgkmMax : 2 * MT + 2 * (NT - 1 - j)));
+      for (int j = 0; j < NT; ++j)
+        asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(blo[j]), "+v"(bhi[j]) : "n"(kLgkmMax < 2 * MT + 2 * (NT - 1 - j) ? kLgkmMax : 2 * MT + 2 * (NT - 1 - j)));
 #pragma unroll
-    for (int i = 0; i < MT; ++i) {
-      asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(alo[i]), "+v"(ahi[i]) : "n"(kLgkmMax < 2 * (MT - 1 - i) ? kLgkmMax : 2 * (MT - 1 - i)));
-      const u32x4_t aop = {alo[i].x, alo[i].y, ahi[i].x, ahi[i].y};
+      for (int i = 0; i < MT; ++i) {
+        asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(alo[i]), "+v"(ahi[i]) : "n"(kLgkmMax < 2 * (MT - 1 - i) ? kLgkmMax : 2 * (MT - 1 - i)));
+        const u32x4_t aop = {alo[i].x, alo[i].y, ahi[i].x, ahi[i].y};
 #pragma unroll
-      for (int j = 0; j < NT; ++j) {
-        const u32x4_t bop = {blo[j].x, blo[j].y, bhi[j].x, bhi[j].y};
-        acc[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, bop), __builtin_bit_cast(bf16x8_t, aop),
-                                                           acc[j][i], 0, 0, 0);
+        for (int j = 0; j < NT; ++j) {
+          const u32x4_t bop = {blo[j].x, blo[j].y, bhi[j].x, bhi[j].y};
+          acc[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, bop), __builtin_bit_cast(bf16x8_t, aop),
+                                                             acc[j][i], 0, 0, 0);
+        }
       }
+      __builtin_amdgcn_s_setprio(0);
+      __builtin_amdgcn_sched_barrier(0);
+      asm volatile("s_barrier" ::: "memory");
+      __builtin_amdgcn_sched_barrier(0);
     }
-    __builtin_amdgcn_s_setprio(0);
-    __builtin_amdgcn_sched_barrier(0);
-    asm volatile("s_barrier" ::: "memory");
-    __builtin_amdgcn_sched_barrier(0);
-  }
+  };
+  if (wm == 1)
+    main_loop(std::true_type{});
+  else
+    main_loop(std::false_type{});
   if (wm == 0) asm volatile("s_barrier" ::: "memory");
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the clamped requests of the last steps
 

@@ -441,31 +441,39 @@ __global__ __launch_bounds__(512) void nf4_gemm_dense_kernel(const DenseArgs g) 
   issue_w(2, 2);
   asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");  // A(0), W(0) landed everywhere
   if (wm == 1) asm volatile("s_barrier" ::: "memory");
-  int e0 = 0, ws = 0;  // activation entry of the current pair of steps, weight stage of the current step
-  for (int t = 0; t < nk; t += 2) {
-    const int e1 = e0 == 2 ? 0 : e0 + 1, e2 = e1 == 2 ? 0 : e1 + 1;
-    // ---- even step t
-    issue_w(t + 3, (ws + 3) & 3);
-    issue_a((t >> 1) + 2, e2);
-    read_step(e0, 0, ws);
-    __builtin_amdgcn_sched_barrier(0);
-    if (wm == 1)
-      asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-    else
-      asm volatile("s_waitcnt vmcnt(12)\n\ts_barrier" ::: "memory");
-    compute();
-    // ---- odd step t + 1
-    issue_w(t + 4, ws);
-    read_step(e0, 1, (ws + 1) & 3);
-    __builtin_amdgcn_sched_barrier(0);
-    if (wm == 1)
-      asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-    else
-      asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");
-    compute();
-    e0 = e1;
-    ws = (ws + 2) & 3;
-  }
+  // one copy of the loop per wave group: the two differ in one wait, and a branch per step costs 2 - 4 %
+  auto main_loop = [&](auto lgkm) {
+    constexpr bool kLgkm = decltype(lgkm)::value;
+    int e0 = 0, ws = 0;  // activation entry of the current pair of steps, weight stage of the current step
+    for (int t = 0; t < nk; t += 2) {
+      const int e1 = e0 == 2 ? 0 : e0 + 1, e2 = e1 == 2 ? 0 : e1 + 1;
+      // ---- even step t
+      issue_w(t + 3, (ws + 3) & 3);
+      issue_a((t >> 1) + 2, e2);
+      read_step(e0, 0, ws);
+      __builtin_amdgcn_sched_barrier(0);
+      if constexpr (kLgkm)
+        asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      else
+        asm volatile("s_waitcnt vmcnt(12)\n\ts_barrier" ::: "memory");
+      compute();
+      // ---- odd step t + 1
+      issue_w(t + 4, ws);
+      read_step(e0, 1, (ws + 1) & 3);
+      __builtin_amdgcn_sched_barrier(0);
+      if constexpr (kLgkm)
+        asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      else
+        asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");
+      compute();
+      e0 = e1;
+      ws = (ws + 2) & 3;
+    }
+  };
+  if (wm == 1)
+    main_loop(std::true_type{});
+  else
+    main_loop(std::false_type{});
   if (wm == 0) asm volatile("s_barrier" ::: "memory");
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the clamped requests of the last steps
 
