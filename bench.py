@@ -627,7 +627,9 @@ def main() -> int:
             g_launches, g_timed, g_ms, g_flops, g_shapes = timer.summary()
             own_gemm = {"kernel": "nf4_gemm_dense_kernel on weights fake-quantised straight into its tile order (forward and "
                                   "grad-input) and gemm_tn_kernel (weight gradients) for every linear that gives a full round of "
-                                  "256 x 256 tiles; the 1024-wide k / v projections run on the vendor library",
+                                  "256 x 256 tiles; q / k / v and gate / up run as groups (one forward and one grad-input launch "
+                                  "each) unless --no-group; the weight gradients of the 1024-wide k / v projections run on the "
+                                  "vendor library",
                         "launches": g_launches, "tflops": round(g_flops / g_ms / 1e9, 1), "frac_of_bf16_mfma_peak":
                         round(g_flops / g_ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4), "gemm_ms_per_step": round(g_ms / args.steps, 2),
                         "per_shape": g_shapes}

@@ -481,6 +481,25 @@ int ttamd_tiled_linear_bf16(const void* x, const void* tiled_weight, const void*
  */
 int ttamd_tiled_lora_linear_bf16(const void* x, const void* tiled_weight, const void* lx, const void* lw, int lw_row_major, int rank,
                                  float lscale, const void* bias, void* y, int64_t M, int64_t n_out, int64_t k_contract, void* stream);
+/*
+ * Fake-quantised layers that read the same input (q_proj / k_proj / v_proj, torchtune/modules/attention.py:234,262-263; w1 / w3,
+ * torchtune/modules/feed_forward.py:50-53), as additions above the per-layer calls:
+ *   ttamd_fq_per_group_int4_sym_tiled_at_bf16: ttamd_fq_per_group_int4_sym_tiled_bf16 with a place for the transposed tiles:
+ *     tiled_bwd is the tile buffer of the members' weights stacked along N (bwd_n_total rows in all, 2 * bwd_n_total * K
+ *     bytes) and this weight's rows start at bwd_n_offset (a multiple of 32).  The forward tiles of stacked weights need no
+ *     such argument: member i's start at byte 2 * K * (rows before it) of the common buffer.
+ *   ttamd_tiled_linear_group_fwd_bf16: y_i[M, n_out_i] = x . Wd_i^T (+ bias_i) for the stacked forward tiles, one launch
+ *     (n_out_i multiples of 256; bias NULL or an array with NULL entries allowed).
+ *   ttamd_tiled_linear_group_dx_bf16: gx[M, K] = sum_i gy_i[M, n_out_i] . Wd_i, one launch over the stacked transposed
+ *     tiles (the sum is taken in fp32 inside the GEMM: no separate additions of the members' grad-inputs).
+ */
+int ttamd_fq_per_group_int4_sym_tiled_at_bf16(const void* w, int64_t N, int64_t K, int group_size, int qparam_dtype, float eps,
+                                              void* tiled_fwd, void* tiled_bwd, int64_t bwd_n_total, int64_t bwd_n_offset, float* scale,
+                                              void* stream);
+int ttamd_tiled_linear_group_fwd_bf16(const void* x, const void* tiled_weights, int n_members, const int64_t* n_out,
+                                      const void* const* bias, void* const* y, int64_t M, int64_t k_contract, void* stream);
+int ttamd_tiled_linear_group_dx_bf16(const void* const* gy, const int64_t* n_out, int n_members, const void* tiled_weights_t, void* gx,
+                                     int64_t M, int64_t K, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
  * Neighbours of the quantized linears inside a decoder layer (one pass over HBM each, bf16 tensors, fp32 math).

@@ -123,3 +123,67 @@ def test_qat_linear_on_the_tiled_gemm_vs_oracle_and_vs_default_path(bias, monkey
     torch.testing.assert_close(gx1.cpu().float(), gxo, rtol=1e-2, atol=1e-2 * max(1.0, float(gxo.abs().max()) / 8))
     gwo = wo.grad.float()
     torch.testing.assert_close(gw1.cpu().float(), gwo, rtol=2e-2, atol=2e-2 * float(gwo.abs().max()))
+
+
+@pytest.mark.parametrize("Ns,K,bias", [((512, 256, 256), 512, False), ((1024, 1024), 256, True)], ids=["qkv", "gate_up_bias"])
+def test_fake_quantized_group_matches_layer_by_layer(Ns, K, bias, monkeypatch):
+    """``fake_quantized_linear_group`` (q / k / v, gate / up of a fake-quantised model as one node) against calling the
+    layers in turn on the same tiled GEMM: outputs bit for bit (the same kernel on the same tiles, whatever launch the
+    member's columns ride in), weight and bias gradients bit for bit (the same products), the grad-input within rtol 1e-2
+    (the group sums the members in fp32 inside the GEMM, the layer-by-layer path rounds each member to bf16 and adds)
+    and at least as close to the fp32 evaluation; the stacked tiles hold each member's ``fq_per_group_int4_sym`` values
+    bit for bit (one-hot read-back); every quantizer records the scales of its own weight."""
+    monkeypatch.setattr(qat, "TILED_GEMM_MIN_TILES", 0)
+    gen = torch.Generator().manual_seed(len(Ns) + K)
+    M, g = 2048 + 64, 32
+    layers = []
+    for N in Ns:
+        lin = Int8DynActInt4WeightQATLinear(K, N, bias=bias, device=DEV, groupsize=g, precision=BF)
+        with torch.no_grad():
+            lin.weight.copy_((torch.randn(N, K, generator=gen) * 0.02).to(BF))
+            if bias:
+                lin.bias.copy_((torch.randn(N, generator=gen) * 0.1).to(BF))
+        layers.append(lin)
+    x = torch.randn(M, K, generator=gen).to(BF).to(DEV)
+    gys = [torch.randn(M, N, generator=gen).to(BF).to(DEV) for N in Ns]
+
+    def run(group):
+        for l in layers:
+            l.zero_grad()
+        xd = x.clone().requires_grad_()
+        assert qat._group_tiled_ok(xd, layers)
+        ys = qat.fake_quantized_linear_group(xd, layers) if group else tuple(l(xd) for l in layers)
+        torch.autograd.backward(ys, gys)
+        return ([y.detach() for y in ys], xd.grad, [l.weight.grad.clone() for l in layers],
+                [l.bias.grad.clone() if bias else None for l in layers], [l.weight_fake_quantizer.scale.clone() for l in layers])
+
+    ys1, gx1, gw1, gb1, sc1 = run(True)
+    ys0, gx0, gw0, gb0, sc0 = run(False)
+    for a, b in zip(ys1, ys0):
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+    for a, b in zip(gw1, gw0):
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+    for a, b in zip(sc1, sc0):
+        assert torch.equal(a, b)
+    if bias:
+        for a, b in zip(gb1, gb0):
+            assert torch.equal(a, b)
+    want = sum(gy.float() @ ops.fq_per_group_int4_sym(l.weight.detach(), g)[0].float() for gy, l in zip(gys, layers))
+    scale = max(1.0, float(want.abs().max()) / 8)
+    torch.testing.assert_close(gx1.float(), want, rtol=1e-2, atol=1e-2 * scale)
+    assert float((gx1.float() - want).abs().max()) <= float((gx0.float() - want).abs().max()) + 1e-3 * scale
+    # the stacks, read back through the group GEMMs with one-hot activations
+    tf, tb, _ = ops.fq_int4_sym_tiled_group([l.weight.detach() for l in layers], g)
+    eye = torch.zeros(max(K, 2048), K, dtype=BF, device=DEV)
+    eye[torch.arange(K, device=DEV), torch.arange(K, device=DEV)] = 1.0
+    for y, l in zip(ops.tiled_linear_group_fwd(eye, tf, list(Ns)), layers):
+        want_w = ops.fq_per_group_int4_sym(l.weight.detach(), g)[0]
+        assert torch.equal(y[:K].view(torch.int16), want_w.t().contiguous().view(torch.int16))
+    for i, l in enumerate(layers):   # row m of gy_i one-hot at column m: gx row m = row m of fq(W_i); the other members are zero
+        want_w = ops.fq_per_group_int4_sym(l.weight.detach(), g)[0]
+        rows = max(Ns[i], 2048)
+        hot = [torch.zeros(rows, N, dtype=BF, device=DEV) for N in Ns]
+        hot[i][torch.arange(Ns[i], device=DEV), torch.arange(Ns[i], device=DEV)] = 1.0
+        gx = ops.tiled_linear_group_dx(hot, tb, K)
+        assert torch.equal(gx[:Ns[i]].view(torch.int16), want_w.view(torch.int16))
+

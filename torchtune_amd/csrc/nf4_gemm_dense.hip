@@ -166,7 +166,8 @@ __global__ __launch_bounds__(256) void nf4_expand_tiled_transposed_kernel(const 
 // ---------------------------------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void fq_int4_sym_tiled_kernel(const uint16_t* __restrict__ w, int N, int K, int threads_per_group,
                                                                 char* __restrict__ tiled_fwd, char* __restrict__ tiled_bwd,
-                                                                float* __restrict__ scale_out, int groups_per_row, bool qp_bf16, float eps) {
+                                                                float* __restrict__ scale_out, int groups_per_row, bool qp_bf16, float eps,
+                                                                int bwd_nk_total, int bwd_t_off) {
   constexpr int kPieceF = 1040;  // forward staging: piece pitch, 16 bytes of padding spread the 16-byte writes over the banks
   constexpr int kPitchB = 80;    // backward staging: bytes per column k (32 rows x 2 bytes + padding)
   __shared__ __attribute__((aligned(16))) char smf[16 * kPieceF];
@@ -253,7 +254,8 @@ __global__ __launch_bounds__(256) void fq_int4_sym_tiled_kernel(const uint16_t* 
       const int Tk = 16 * blockIdx.y + p;  // block of 16 columns k
       if (16 * Tk < K) {
         const u32x4_t val = *reinterpret_cast<const u32x4_t*>(smb + (16 * p + (l & 15)) * kPitchB + 16 * (l >> 4));
-        *reinterpret_cast<u32x4_t*>(tiled_bwd + ((int64_t)Tk * (N >> 5) + blockIdx.x) * 1024 + l * 16) = val;
+        // this weight's 32-row step blockIdx.x sits at step bwd_t_off + blockIdx.x of a contraction of bwd_nk_total steps
+        *reinterpret_cast<u32x4_t*>(tiled_bwd + ((int64_t)Tk * bwd_nk_total + bwd_t_off + blockIdx.x) * 1024 + l * 16) = val;
       }
     }
   }
@@ -849,8 +851,12 @@ using namespace ttamd;
 
 extern "C" size_t ttamd_tiled_weight_bytes(int64_t N, int64_t K) { return N > 0 && K > 0 ? (size_t)N * (size_t)K * 2 : 0; }
 
-extern "C" int ttamd_fq_per_group_int4_sym_tiled_bf16(const void* w, int64_t N, int64_t K, int group_size, int qparam_dtype, float eps,
-                                                      void* tiled_fwd, void* tiled_bwd, float* scale, void* stream) {
+extern "C" int ttamd_fq_per_group_int4_sym_tiled_at_bf16(const void* w, int64_t N, int64_t K, int group_size, int qparam_dtype, float eps,
+                                                         void* tiled_fwd, void* tiled_bwd, int64_t bwd_n_total, int64_t bwd_n_offset,
+                                                         float* scale, void* stream) {
+  TT_REQUIRE(bwd_n_total % 64 == 0 && bwd_n_offset % 32 == 0 && bwd_n_offset >= 0 && bwd_n_offset + N <= bwd_n_total && bwd_n_total < (1 << 30),
+             "fq_per_group_int4_sym_tiled: rows [%lld, + %lld) do not fit a contraction of %lld (multiples of 32 / 64)",
+             (long long)bwd_n_offset, (long long)N, (long long)bwd_n_total);
   TT_REQUIRE(w && aligned16(w) && (tiled_fwd || tiled_bwd), "fq_per_group_int4_sym_tiled: w must be non-null and 16-byte aligned, one output given");
   TT_REQUIRE((!tiled_fwd || aligned16(tiled_fwd)) && (!tiled_bwd || aligned16(tiled_bwd)), "fq_per_group_int4_sym_tiled: outputs must be 16-byte aligned");
   TT_REQUIRE(N > 0 && K > 0 && N % 64 == 0 && K % 64 == 0 && N < (1 << 30) && K < (1 << 30),
@@ -863,8 +869,14 @@ extern "C" int ttamd_fq_per_group_int4_sym_tiled_bf16(const void* w, int64_t N, 
   TT_REQUIRE(gy < 65536, "fq_per_group_int4_sym_tiled: K too large for one launch");
   fq_int4_sym_tiled_kernel<<<dim3((unsigned)(N / 32), (unsigned)gy), dim3(256), 0, reinterpret_cast<hipStream_t>(stream)>>>(
       reinterpret_cast<const uint16_t*>(w), (int)N, (int)K, group_size / 32, reinterpret_cast<char*>(tiled_fwd),
-      reinterpret_cast<char*>(tiled_bwd), scale, (int)(K / group_size), qparam_dtype == TTAMD_BF16, eps);
+      reinterpret_cast<char*>(tiled_bwd), scale, (int)(K / group_size), qparam_dtype == TTAMD_BF16, eps, (int)(bwd_n_total >> 5),
+      (int)(bwd_n_offset >> 5));
   return check_launch("fq_per_group_int4_sym_tiled");
+}
+
+extern "C" int ttamd_fq_per_group_int4_sym_tiled_bf16(const void* w, int64_t N, int64_t K, int group_size, int qparam_dtype, float eps,
+                                                      void* tiled_fwd, void* tiled_bwd, float* scale, void* stream) {
+  return ttamd_fq_per_group_int4_sym_tiled_at_bf16(w, N, K, group_size, qparam_dtype, eps, tiled_fwd, tiled_bwd, N, 0, scale, stream);
 }
 
 namespace {
@@ -912,4 +924,61 @@ extern "C" int ttamd_tiled_lora_linear_bf16(const void* x, const void* tiled_wei
                                             int rank, float lscale, const void* bias, void* y, int64_t M, int64_t n_out,
                                             int64_t k_contract, void* stream) {
   return tiled_linear(x, tiled_weight, lx, lw, lw_row_major != 0, rank, lscale, bias, y, M, n_out, k_contract, stream);
+}
+
+// Layers with a common input on weights in the tiled layout (q / k / v, gate / up of a fake-quantised model): the forward
+// over the members' concatenated output columns, the grad-input over the concatenated contraction.
+extern "C" int ttamd_tiled_linear_group_fwd_bf16(const void* x, const void* tiled_weights, int n_members, const int64_t* n_out,
+                                                 const void* const* bias, void* const* y, int64_t M, int64_t k_contract, void* stream) {
+  TT_REQUIRE(x && tiled_weights && n_out && y && aligned16(x) && aligned16(tiled_weights), "tiled_linear_group_fwd: pointers must be non-null and 16-byte aligned");
+  TT_REQUIRE(n_members >= 1 && n_members <= kGroupMax, "tiled_linear_group_fwd: 1 to %d members (got %d)", kGroupMax, n_members);
+  TT_REQUIRE(M > 0 && k_contract > 0 && k_contract % 64 == 0, "tiled_linear_group_fwd: k_contract (%lld) must be a positive multiple of 64", (long long)k_contract);
+  DenseArgs g = {};
+  g.nseg = 1;
+  g.seg[0].X = reinterpret_cast<const uint16_t*>(x);
+  g.seg[0].Kc = (int)k_contract;
+  g.nout = n_members;
+  int64_t n_off = 0;
+  for (int i = 0; i < n_members; ++i) {
+    TT_REQUIRE(n_out[i] > 0 && n_out[i] % 256 == 0, "tiled_linear_group_fwd: member %d: n_out (%lld) must be a positive multiple of 256 (a tile belongs to one member)", i, (long long)n_out[i]);
+    TT_REQUIRE(y[i] && aligned16(y[i]) && (!bias || !bias[i] || (reinterpret_cast<uintptr_t>(bias[i]) & 7u) == 0), "tiled_linear_group_fwd: member %d: output must be non-null and 16-byte aligned, bias 8-byte aligned", i);
+    g.out[i].C = reinterpret_cast<uint16_t*>(y[i]);
+    g.out[i].bias = bias ? reinterpret_cast<const uint16_t*>(bias[i]) : nullptr;
+    g.out[i].n_begin = (int)n_off;
+    g.out[i].width = (int)n_out[i];
+    n_off += n_out[i];
+  }
+  if (!(M * k_contract * 2 < (int64_t(1) << 32) && k_contract * 2 * 256 < (int64_t(1) << 32) && M < (1 << 30) && n_off < (1 << 30)))
+    return fail(TTAMD_EUNSUPPORTED, "tiled_linear_group_fwd: operands too large for 32-bit offsets (M=%lld k=%lld)", (long long)M, (long long)k_contract);
+  g.Wt = reinterpret_cast<const char*>(tiled_weights);
+  g.M = (int)M; g.Nout = (int)n_off; g.Kc = (int)k_contract;
+  g.lw_row_major = 1;
+  return launch_dense(g, reinterpret_cast<hipStream_t>(stream));
+}
+
+extern "C" int ttamd_tiled_linear_group_dx_bf16(const void* const* gy, const int64_t* n_out, int n_members, const void* tiled_weights_t,
+                                                void* gx, int64_t M, int64_t K, void* stream) {
+  TT_REQUIRE(gy && n_out && tiled_weights_t && gx && aligned16(tiled_weights_t) && aligned16(gx), "tiled_linear_group_dx: pointers must be non-null and 16-byte aligned");
+  TT_REQUIRE(n_members >= 1 && n_members <= kGroupMax, "tiled_linear_group_dx: 1 to %d members (got %d)", kGroupMax, n_members);
+  TT_REQUIRE(M > 0 && K > 0 && K % 64 == 0, "tiled_linear_group_dx: K (%lld) must be a positive multiple of 64", (long long)K);
+  DenseArgs g = {};
+  g.nseg = n_members;
+  g.nout = 1;
+  int64_t n_total = 0;
+  for (int i = 0; i < n_members; ++i) {
+    TT_REQUIRE(gy[i] && aligned16(gy[i]) && n_out[i] > 0 && n_out[i] % 64 == 0, "tiled_linear_group_dx: member %d: gradient non-null and 16-byte aligned, n_out (%lld) a multiple of 64", i, (long long)n_out[i]);
+    if (M * n_out[i] * 2 >= (int64_t(1) << 32)) return fail(TTAMD_EUNSUPPORTED, "tiled_linear_group_dx: member %d too large for 32-bit offsets", i);
+    g.seg[i].X = reinterpret_cast<const uint16_t*>(gy[i]);
+    g.seg[i].Kc = (int)n_out[i];
+    n_total += n_out[i];
+  }
+  if (!(n_total * 2 * 256 < (int64_t(1) << 32) && M < (1 << 30) && K < (1 << 30)))
+    return fail(TTAMD_EUNSUPPORTED, "tiled_linear_group_dx: operands too large for 32-bit offsets");
+  g.out[0].C = reinterpret_cast<uint16_t*>(gx);
+  g.out[0].n_begin = 0;
+  g.out[0].width = (int)K;
+  g.Wt = reinterpret_cast<const char*>(tiled_weights_t);
+  g.M = (int)M; g.Nout = (int)K; g.Kc = (int)n_total;
+  g.lw_row_major = 0;
+  return launch_dense(g, reinterpret_cast<hipStream_t>(stream));
 }

@@ -29,7 +29,7 @@ from torch.utils.checkpoint import checkpoint
 
 from .modules import layer_ops
 from .modules.peft import LoRALinear, get_adapter_params, lora_linear_group, lora_swiglu_group, set_trainable_params
-from .qat import Int8DynActInt4WeightQATQuantizer
+from .qat import FakeQuantizedLinear, Int8DynActInt4WeightQATQuantizer, fake_quantized_linear_group
 
 
 # True: projections that read the same tensor (q/k/v, gate/up) go through the group kernels; False: one call per
@@ -37,6 +37,13 @@ from .qat import Int8DynActInt4WeightQATQuantizer
 GROUP_SHARED_INPUT = True
 # silu(w1 x) * w3 x formed in the epilogue of the gate / up GEMM launch instead of a pass of its own
 GATED_EPILOGUE = True
+
+
+def _shared_input(x, layers):
+    """Projections that read the same tensor: the LoRA group kernels, the fake-quantised group, or the layers in turn."""
+    if all(isinstance(layer, FakeQuantizedLinear) for layer in layers):
+        return fake_quantized_linear_group(x, layers)
+    return lora_linear_group(x, layers)
 
 
 @dataclass(frozen=True)
@@ -145,7 +152,7 @@ class Attention(nn.Module):
     def forward(self, x: torch.Tensor, rope: torch.Tensor) -> torch.Tensor:
         b, sl, _ = x.shape
         # the three projections read the same tensor (torchtune/modules/attention.py:234,262-263): one group
-        q, k, v = lora_linear_group(x, (self.q_proj, self.k_proj, self.v_proj)) if GROUP_SHARED_INPUT else (
+        q, k, v = _shared_input(x, (self.q_proj, self.k_proj, self.v_proj)) if GROUP_SHARED_INPUT else (
             self.q_proj(x), self.k_proj(x), self.v_proj(x))
         q = q.view(b, sl, self.n_heads, self.head_dim)
         k = k.view(b, sl, self.n_kv, self.head_dim)
@@ -176,7 +183,7 @@ class FeedForward(nn.Module):
             act = lora_swiglu_group(x, self.w1, self.w3)  # the product written by the pair's GEMM launch
             if act is not None:
                 return self.w2(act)
-        g, u = lora_linear_group(x, (self.w1, self.w3)) if GROUP_SHARED_INPUT else (self.w1(x), self.w3(x))
+        g, u = _shared_input(x, (self.w1, self.w3)) if GROUP_SHARED_INPUT else (self.w1(x), self.w3(x))
         return self.w2(layer_ops.swiglu(g, u) if _fused(g) else F.silu(g) * u)
 
 

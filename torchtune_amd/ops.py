@@ -5,6 +5,7 @@ Every function requires HIP (``cuda``) tensors.  There is no CPU implementation 
 """
 from __future__ import annotations
 
+import ctypes
 from typing import Optional, Sequence, Tuple
 
 import torch
@@ -611,6 +612,100 @@ def fq_per_group_int4_sym_tiled(w: torch.Tensor, group_size: int, forward: bool 
             events[1].record()
     _lib.check(rc, "fq_per_group_int4_sym_tiled")
     return tf, tb, scale
+
+
+def fq_int4_sym_tiled_group(ws: Sequence[torch.Tensor], group_size: int, forward: bool = True, backward: bool = True,
+                            qparam_dtype: torch.dtype = torch.float32, eps: Optional[float] = None):
+    """Weights [N_i, K] of layers with a common input -> (forward tiles of the weights stacked along N | None, transposed
+    tiles of the same stack | None, [scale_i fp32 [N_i, K/g]]): what ``tiled_linear_group_fwd`` / ``tiled_linear_group_dx``
+    read.  Each member's values are those of ``fq_per_group_int4_sym`` on it alone."""
+    K = ws[0].shape[1]
+    for w in ws:
+        _need_gpu(w, "fq_int4_sym_tiled_group")
+        if w.dtype != torch.bfloat16 or w.dim() != 2 or w.shape[1] != K or not tiled_weight_shape_ok(w.shape[0], K, group_size):
+            raise ValueError("fq_int4_sym_tiled_group: members must be 2-D bfloat16 weights over one K, N and K multiples of 64, "
+                             f"group_size ({group_size}) one of 32/64/128/256 dividing K")
+    qcode = _code(qparam_dtype, "fq_int4_sym_tiled_group (qparams)")
+    dev = ws[0].device
+    n_total = sum(w.shape[0] for w in ws)
+    tf = torch.empty(n_total * K, dtype=torch.bfloat16, device=dev) if forward else None
+    tb = torch.empty(n_total * K, dtype=torch.bfloat16, device=dev) if backward else None
+    scales = []
+    lib = _lib.load()
+    e = float(torch.finfo(torch.float32).eps) if eps is None else float(eps)
+    n_off = 0
+    with torch.cuda.device(dev):
+        for w in ws:
+            wc = w.contiguous()
+            N = wc.shape[0]
+            scale = torch.empty(N, K // group_size, dtype=torch.float32, device=dev)
+            events = _fq_timer(f"per_group_tiled{int(forward) + int(backward)}", N, K, group_size, 2) if _fq_timer is not None else None
+            if events:
+                events[0].record()
+            rc = lib.ttamd_fq_per_group_int4_sym_tiled_at_bf16(wc.data_ptr(), N, K, group_size, qcode, e,
+                                                               tf.data_ptr() + 2 * K * n_off if forward else None, _ptr(tb), n_total, n_off,
+                                                               scale.data_ptr(), _stream(w))
+            if events:
+                events[1].record()
+            _lib.check(rc, "fq_int4_sym_tiled_group")
+            scales.append(scale)
+            n_off += N
+    return tf, tb, scales
+
+
+def tiled_linear_group_fwd(x: torch.Tensor, tiled: torch.Tensor, n_outs: Sequence[int],
+                           biases: Optional[Sequence[Optional[torch.Tensor]]] = None):
+    """-> [y_i [M, n_out_i]] = x @ Wd_i.T (+ bias_i) for weights stacked in the tiled layout, one launch."""
+    x = _bf16_2d(x, "tiled_linear_group_fwd")
+    M, K = x.shape
+    n = len(n_outs)
+    if not 1 <= n <= _lib.GROUP_MAX or any(o <= 0 or o % 256 for o in n_outs):
+        raise ValueError(f"tiled_linear_group_fwd: 1 to {_lib.GROUP_MAX} members with widths that are multiples of 256 (got {list(n_outs)})")
+    if tiled.dtype != torch.bfloat16 or tiled.numel() != sum(n_outs) * K or not tiled.is_contiguous():
+        raise ValueError(f"tiled_linear_group_fwd: the tiled weights must be a contiguous bfloat16 tensor of {sum(n_outs)} x {K} elements")
+    ys = [torch.empty(M, o, dtype=torch.bfloat16, device=x.device) for o in n_outs]
+    bs = [None] * n if biases is None else [None if b is None else b.contiguous() for b in biases]
+    for b, o in zip(bs, n_outs):
+        if b is not None and (b.dtype != torch.bfloat16 or b.numel() != o):
+            raise ValueError(f"tiled_linear_group_fwd: a bias must be bfloat16 with {o} elements")
+    c_n = (ctypes.c_int64 * n)(*n_outs)
+    c_b = (ctypes.c_void_p * n)(*[_ptr(b) for b in bs])
+    c_y = (ctypes.c_void_p * n)(*[y.data_ptr() for y in ys])
+    lib = _lib.load()
+    with torch.cuda.device(x.device):
+        events = _gemm_timer("tiled", M, sum(n_outs), K, 0) if _gemm_timer is not None else None
+        if events:
+            events[0].record()
+        rc = lib.ttamd_tiled_linear_group_fwd_bf16(x.data_ptr(), tiled.data_ptr(), n, c_n, c_b, c_y, M, K, _stream(x))
+        if events:
+            events[1].record()
+    _lib.check(rc, "tiled_linear_group_fwd")
+    return ys
+
+
+def tiled_linear_group_dx(gys: Sequence[torch.Tensor], tiled_t: torch.Tensor, K: int) -> torch.Tensor:
+    """-> gx [M, K] = sum_i gy_i @ Wd_i for the transposed tiles of the stacked weights, one launch."""
+    gys = [_bf16_2d(g, "tiled_linear_group_dx") for g in gys]
+    M = gys[0].shape[0]
+    n = len(gys)
+    n_outs = [g.shape[1] for g in gys]
+    if not 1 <= n <= _lib.GROUP_MAX or any(g.shape[0] != M for g in gys) or any(o % 64 for o in n_outs) or K % 64:
+        raise ValueError(f"tiled_linear_group_dx: 1 to {_lib.GROUP_MAX} gradients over the same rows, widths and K multiples of 64")
+    if tiled_t.dtype != torch.bfloat16 or tiled_t.numel() != sum(n_outs) * K or not tiled_t.is_contiguous():
+        raise ValueError(f"tiled_linear_group_dx: the tiled weights must be a contiguous bfloat16 tensor of {sum(n_outs)} x {K} elements")
+    gx = torch.empty(M, K, dtype=torch.bfloat16, device=gys[0].device)
+    c_n = (ctypes.c_int64 * n)(*n_outs)
+    c_g = (ctypes.c_void_p * n)(*[g.data_ptr() for g in gys])
+    lib = _lib.load()
+    with torch.cuda.device(gx.device):
+        events = _gemm_timer("tiled", M, K, sum(n_outs), 0) if _gemm_timer is not None else None
+        if events:
+            events[0].record()
+        rc = lib.ttamd_tiled_linear_group_dx_bf16(c_g, c_n, n, tiled_t.data_ptr(), gx.data_ptr(), M, K, _stream(gx))
+        if events:
+            events[1].record()
+    _lib.check(rc, "tiled_linear_group_dx")
+    return gx
 
 
 def tiled_linear(x: torch.Tensor, tiled: torch.Tensor, n_out: int, bias: Optional[torch.Tensor] = None) -> torch.Tensor:

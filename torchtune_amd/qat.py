@@ -23,7 +23,7 @@ from dataclasses import dataclass
 from enum import Enum, auto
 import threading
 import weakref
-from typing import Optional, Union
+from typing import Optional, Tuple, Union
 
 import torch
 import torch.nn.functional as F
@@ -287,6 +287,93 @@ class _TiledFakeQuantLinearFn(torch.autograd.Function):
             gw = ops.gemm_tn(gy2, x2) if own else gy2.t().matmul(x2)
         gb = gy2.sum(dim=0) if (ctx.has_bias and need_b) else None
         return gx, gw, gb, None
+
+
+class _TiledFakeQuantGroupFn(torch.autograd.Function):
+    """Fake-quantised linears that read the same (already fake-quantised) input, as one node: every weight's fake
+    quantisation goes into one stack of tiles per direction, the forward is one GEMM launch over the members' output
+    columns, the grad-input one launch over their concatenated contraction (fp32 sum over the members, one rounding, no
+    additions of partial grad-inputs afterwards).  Inputs: x, then per member (weight, bias or None); ``quantizers`` are
+    the members' weight quantizers (same config)."""
+
+    @staticmethod
+    def forward(ctx, x, quantizers, *flat):
+        weights, biases = flat[0::2], flat[1::2]
+        c = quantizers[0].config
+        K = weights[0].shape[1]
+        x2 = x.reshape(-1, K)
+        need_gx = ctx.needs_input_grad[0]
+        tf, tb, scales = ops.fq_int4_sym_tiled_group([w.detach() for w in weights], c.group_size, forward=True, backward=need_gx,
+                                                     qparam_dtype=c.scale_precision, eps=c.eps)
+        for q, s in zip(quantizers, scales):
+            q.scale = s.to(c.scale_precision)
+            q.zero_point = None
+        ys = ops.tiled_linear_group_fwd(x2, tf, [w.shape[0] for w in weights], biases)
+        ctx.save_for_backward(x2, tb)
+        ctx.x_shape = x.shape
+        ctx.shapes = tuple(tuple(w.shape) for w in weights)
+        ctx.has_bias = tuple(b is not None for b in biases)
+        return tuple(y.view(*x.shape[:-1], y.shape[-1]) for y in ys)
+
+    @staticmethod
+    def backward(ctx, *gys):
+        x2, tb = ctx.saved_tensors
+        K = ctx.shapes[0][1]
+        gy2 = [torch.zeros(x2.shape[0], N, dtype=x2.dtype, device=x2.device) if g is None else g.reshape(-1, N)
+               for g, (N, _) in zip(gys, ctx.shapes)]
+        out = [ops.tiled_linear_group_dx(gy2, tb, K).view(ctx.x_shape) if ctx.needs_input_grad[0] else None, None]
+        for i, (N, _) in enumerate(ctx.shapes):
+            need_w, need_b = ctx.needs_input_grad[2 + 2 * i:4 + 2 * i]
+            gw = None
+            if need_w:
+                own = ops.gemm_tn_applies(gy2[i].shape[0], N, K) and (N // 256) * (K // 256) >= TN_GEMM_MIN_TILES
+                gw = ops.gemm_tn(gy2[i], x2) if own else gy2[i].t().matmul(x2)
+            out += [gw, gy2[i].sum(dim=0) if (ctx.has_bias[i] and need_b) else None]
+        return tuple(out)
+
+
+def fake_quantized_linear_group(x: torch.Tensor, layers) -> Tuple[torch.Tensor, ...]:
+    """``tuple(layer(x) for layer in layers)`` for ``FakeQuantizedLinear`` layers that read the same input (``q_proj`` /
+    ``k_proj`` / ``v_proj``, ``torchtune/modules/attention.py:234,262-263``; ``w1`` / ``w3``,
+    ``torchtune/modules/feed_forward.py:50-53``).  When every member is the 8da4w kind with one configuration and the
+    shapes give the library's GEMM full rounds of tiles, the group runs as one node (``_TiledFakeQuantGroupFn``): narrow
+    members (the 1024-wide k / v projections) ride in the wide launch instead of falling back to the vendor library, and
+    the members' grad-inputs are summed inside the GEMM.  Otherwise the layers are called in turn."""
+    if not _group_tiled_ok(x, layers):
+        return tuple(layer(x) for layer in layers)
+    first = layers[0]
+    xq = x if first.activation_fake_quantizer is None else first.activation_fake_quantizer(x)
+    for layer in layers[1:]:  # every member's quantizer records its qparams, as a call of its own would (the result is shared)
+        if layer.activation_fake_quantizer is not None:
+            layer.activation_fake_quantizer(x)
+    flat = []
+    for layer in layers:
+        flat += [layer.weight, layer.bias]
+    return _TiledFakeQuantGroupFn.apply(xq, tuple(layer.weight_fake_quantizer for layer in layers), *flat)
+
+
+def _group_tiled_ok(x: torch.Tensor, layers) -> bool:
+    if not TILED_GEMM or not 2 <= len(layers) <= ops._lib.GROUP_MAX or not x.is_cuda or x.dtype != torch.bfloat16:
+        return False
+    first = layers[0]
+    for layer in layers:
+        q = getattr(layer, "weight_fake_quantizer", None)
+        if (not isinstance(layer, FakeQuantizedLinear) or q is None or not q.enabled or layer.weight.dtype != torch.bfloat16
+                or layer.in_features != first.in_features or layer.out_features % 256 != 0):
+            return False
+        c, c0 = q.config, first.weight_fake_quantizer.config
+        if not (isinstance(c.granularity, PerGroup) and c.dtype == torch.int4 and c.is_symmetric and c.group_size == c0.group_size
+                and c.scale_precision == c0.scale_precision and c.eps == c0.eps):
+            return False
+        a, a0 = layer.activation_fake_quantizer, first.activation_fake_quantizer
+        if (a is None) != (a0 is None) or (a is not None and (a.enabled != a0.enabled or repr(a.config) != repr(a0.config))):
+            return False
+    K = first.in_features
+    rows = x.numel() // max(1, x.shape[-1])
+    n_total = sum(layer.out_features for layer in layers)
+    row_tiles = (rows + 255) // 256
+    return (x.shape[-1] == K and rows >= TILED_GEMM_MIN_ROWS and row_tiles * min(n_total // 256, K // 256) >= TILED_GEMM_MIN_TILES
+            and ops.tiled_weight_shape_ok(n_total, K, first.weight_fake_quantizer.config.group_size))
 
 
 class FakeQuantizedLinear(nn.Linear):
