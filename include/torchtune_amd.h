@@ -490,14 +490,19 @@ int ttamd_tiled_lora_linear_bf16(const void* x, const void* tiled_weight, const 
  *     such argument: member i's start at byte 2 * K * (rows before it) of the common buffer.
  *   ttamd_tiled_linear_group_fwd_bf16: y_i[M, n_out_i] = x . Wd_i^T (+ bias_i) for the stacked forward tiles, one launch
  *     (n_out_i multiples of 256; bias NULL or an array with NULL entries allowed).
+ *     act != NULL (two members of equal width, the gate and the up projection of a SwiGLU feed-forward): the launch also
+ *     writes act[M, n_out] = bf16(bf16(silu(y_0)) * y_1) from its epilogue, as ttamd_nf4_lora_group_swiglu_fwd_bf16 does;
+ *     the forward tiles must then be in the paired layout: both members written with fwd_paired = 1, the second one's
+ *     tiled_fwd starting 256 * K bytes (128 columns) after the first one's, so that the two weights' blocks of 128
+ *     columns alternate.
  *   ttamd_tiled_linear_group_dx_bf16: gx[M, K] = sum_i gy_i[M, n_out_i] . Wd_i, one launch over the stacked transposed
  *     tiles (the sum is taken in fp32 inside the GEMM: no separate additions of the members' grad-inputs).
  */
 int ttamd_fq_per_group_int4_sym_tiled_at_bf16(const void* w, int64_t N, int64_t K, int group_size, int qparam_dtype, float eps,
-                                              void* tiled_fwd, void* tiled_bwd, int64_t bwd_n_total, int64_t bwd_n_offset, float* scale,
-                                              void* stream);
+                                              void* tiled_fwd, int fwd_paired, void* tiled_bwd, int64_t bwd_n_total, int64_t bwd_n_offset,
+                                              float* scale, void* stream);
 int ttamd_tiled_linear_group_fwd_bf16(const void* x, const void* tiled_weights, int n_members, const int64_t* n_out,
-                                      const void* const* bias, void* const* y, int64_t M, int64_t k_contract, void* stream);
+                                      const void* const* bias, void* const* y, void* act, int64_t M, int64_t k_contract, void* stream);
 int ttamd_tiled_linear_group_dx_bf16(const void* const* gy, const int64_t* n_out, int n_members, const void* tiled_weights_t, void* gx,
                                      int64_t M, int64_t K, void* stream);
 

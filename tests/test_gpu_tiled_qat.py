@@ -187,3 +187,41 @@ def test_fake_quantized_group_matches_layer_by_layer(Ns, K, bias, monkeypatch):
         gx = ops.tiled_linear_group_dx(hot, tb, K)
         assert torch.equal(gx[:Ns[i]].view(torch.int16), want_w.view(torch.int16))
 
+
+@pytest.mark.parametrize("N,K,M", [(1024, 256, 2048 + 64), (4096, 512, 2048)], ids=["small", "full_round"])
+def test_fake_quantized_gated_pair_matches_group_then_swiglu(N, K, M, monkeypatch):
+    """``fake_quantized_swiglu_group`` (gate / up of a fake-quantised feed-forward with ``silu(gate) * up`` written by the
+    pair's GEMM launch, forward tiles in the paired layout) against the plain group followed by the stand-alone SwiGLU op:
+    the product and every gradient bit for bit."""
+    from torchtune_amd.modules import layer_ops
+
+    monkeypatch.setattr(qat, "TILED_GEMM_MIN_TILES", 0)
+    gen = torch.Generator().manual_seed(N + K)
+    g = 32
+    layers = []
+    for _ in range(2):
+        lin = Int8DynActInt4WeightQATLinear(K, N, bias=False, device=DEV, groupsize=g, precision=BF)
+        with torch.no_grad():
+            lin.weight.copy_((torch.randn(N, K, generator=gen) * 0.05).to(BF))
+        layers.append(lin)
+    x = torch.randn(M, K, generator=gen).to(BF).to(DEV)
+    gact = torch.randn(M, N, generator=gen).to(BF).to(DEV)
+
+    def run(gated):
+        for l in layers:
+            l.zero_grad()
+        xd = x.clone().requires_grad_()
+        if gated:
+            act = qat.fake_quantized_swiglu_group(xd, layers[0], layers[1])
+            assert act is not None
+        else:
+            gg, uu = qat.fake_quantized_linear_group(xd, layers)
+            act = layer_ops.swiglu(gg, uu)
+        act.backward(gact)
+        return [act.detach(), xd.grad] + [l.weight.grad.clone() for l in layers]
+
+    for a, b in zip(run(True), run(False)):
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+    layers[1].weight_fake_quantizer.enabled = False
+    assert qat.fake_quantized_swiglu_group(x, layers[0], layers[1]) is None
+

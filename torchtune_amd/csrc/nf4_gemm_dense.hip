@@ -167,7 +167,7 @@ __global__ __launch_bounds__(256) void nf4_expand_tiled_transposed_kernel(const 
 __global__ __launch_bounds__(256) void fq_int4_sym_tiled_kernel(const uint16_t* __restrict__ w, int N, int K, int threads_per_group,
                                                                 char* __restrict__ tiled_fwd, char* __restrict__ tiled_bwd,
                                                                 float* __restrict__ scale_out, int groups_per_row, bool qp_bf16, float eps,
-                                                                int bwd_nk_total, int bwd_t_off) {
+                                                                int bwd_nk_total, int bwd_t_off, int fwd_paired) {
   constexpr int kPieceF = 1040;  // forward staging: piece pitch, 16 bytes of padding spread the 16-byte writes over the banks
   constexpr int kPitchB = 80;    // backward staging: bytes per column k (32 rows x 2 bytes + padding)
   __shared__ __attribute__((aligned(16))) char smf[16 * kPieceF];
@@ -247,7 +247,9 @@ __global__ __launch_bounds__(256) void fq_int4_sym_tiled_kernel(const uint16_t* 
       if (tp < nk) {
         const u32x4_t val = *reinterpret_cast<const u32x4_t*>(smf + p * kPieceF + l * 16);
         const int T = 2 * blockIdx.x + (p >> 3);
-        *reinterpret_cast<u32x4_t*>(tiled_fwd + ((int64_t)T * nk + tp) * 1024 + l * 16) = val;
+        // paired: the forward tiles of two weights of equal shape alternate 8 blocks (128 columns) by 8 (see nf4_expand_tiled_kernel)
+        const int To = fwd_paired ? ((T >> 3) << 4) + (T & 7) : T;
+        *reinterpret_cast<u32x4_t*>(tiled_fwd + ((int64_t)To * nk + tp) * 1024 + l * 16) = val;
       }
     }
     if (tiled_bwd) {
@@ -672,8 +674,8 @@ int launch_dense(DenseArgs& g, hipStream_t s) {
   }
   const dim3 grid((unsigned)(g.tiles_m * g.tiles_n)), block(512);
   if (g.act) {
-    TT_REQUIRE(g.lw_row_major && g.nout == 2 && g.nad == 2 && g.nseg == 1 && g.out[0].width == g.out[1].width && g.out[0].width % 128 == 0 &&
-                   g.Nout == 2 * g.out[0].width,
+    TT_REQUIRE(g.lw_row_major && g.nout == 2 && (g.nad == 2 || g.nad == 0) && g.nseg == 1 && g.out[0].width == g.out[1].width &&
+                   g.out[0].width % 128 == 0 && g.Nout == 2 * g.out[0].width,
                "nf4_gemm_dense: the gated launch takes two members of equal width, a multiple of 128");
     nf4_gemm_dense_kernel<true, true><<<grid, block, kLdsDense, s>>>(g);
   } else if (g.lw_row_major)
@@ -852,8 +854,9 @@ using namespace ttamd;
 extern "C" size_t ttamd_tiled_weight_bytes(int64_t N, int64_t K) { return N > 0 && K > 0 ? (size_t)N * (size_t)K * 2 : 0; }
 
 extern "C" int ttamd_fq_per_group_int4_sym_tiled_at_bf16(const void* w, int64_t N, int64_t K, int group_size, int qparam_dtype, float eps,
-                                                         void* tiled_fwd, void* tiled_bwd, int64_t bwd_n_total, int64_t bwd_n_offset,
-                                                         float* scale, void* stream) {
+                                                         void* tiled_fwd, int fwd_paired, void* tiled_bwd, int64_t bwd_n_total,
+                                                         int64_t bwd_n_offset, float* scale, void* stream) {
+  TT_REQUIRE(!fwd_paired || N % 128 == 0, "fq_per_group_int4_sym_tiled: the paired forward layout needs N (%lld) to be a multiple of 128", (long long)N);
   TT_REQUIRE(bwd_n_total % 64 == 0 && bwd_n_offset % 32 == 0 && bwd_n_offset >= 0 && bwd_n_offset + N <= bwd_n_total && bwd_n_total < (1 << 30),
              "fq_per_group_int4_sym_tiled: rows [%lld, + %lld) do not fit a contraction of %lld (multiples of 32 / 64)",
              (long long)bwd_n_offset, (long long)N, (long long)bwd_n_total);
@@ -870,13 +873,13 @@ extern "C" int ttamd_fq_per_group_int4_sym_tiled_at_bf16(const void* w, int64_t 
   fq_int4_sym_tiled_kernel<<<dim3((unsigned)(N / 32), (unsigned)gy), dim3(256), 0, reinterpret_cast<hipStream_t>(stream)>>>(
       reinterpret_cast<const uint16_t*>(w), (int)N, (int)K, group_size / 32, reinterpret_cast<char*>(tiled_fwd),
       reinterpret_cast<char*>(tiled_bwd), scale, (int)(K / group_size), qparam_dtype == TTAMD_BF16, eps, (int)(bwd_n_total >> 5),
-      (int)(bwd_n_offset >> 5));
+      (int)(bwd_n_offset >> 5), fwd_paired ? 1 : 0);
   return check_launch("fq_per_group_int4_sym_tiled");
 }
 
 extern "C" int ttamd_fq_per_group_int4_sym_tiled_bf16(const void* w, int64_t N, int64_t K, int group_size, int qparam_dtype, float eps,
                                                       void* tiled_fwd, void* tiled_bwd, float* scale, void* stream) {
-  return ttamd_fq_per_group_int4_sym_tiled_at_bf16(w, N, K, group_size, qparam_dtype, eps, tiled_fwd, tiled_bwd, N, 0, scale, stream);
+  return ttamd_fq_per_group_int4_sym_tiled_at_bf16(w, N, K, group_size, qparam_dtype, eps, tiled_fwd, 0, tiled_bwd, N, 0, scale, stream);
 }
 
 namespace {
@@ -929,7 +932,10 @@ extern "C" int ttamd_tiled_lora_linear_bf16(const void* x, const void* tiled_wei
 // Layers with a common input on weights in the tiled layout (q / k / v, gate / up of a fake-quantised model): the forward
 // over the members' concatenated output columns, the grad-input over the concatenated contraction.
 extern "C" int ttamd_tiled_linear_group_fwd_bf16(const void* x, const void* tiled_weights, int n_members, const int64_t* n_out,
-                                                 const void* const* bias, void* const* y, int64_t M, int64_t k_contract, void* stream) {
+                                                 const void* const* bias, void* const* y, void* act, int64_t M, int64_t k_contract,
+                                                 void* stream) {
+  TT_REQUIRE(act == nullptr || (n_members == 2 && n_out && n_out[0] == n_out[1] && aligned16(act)),
+             "tiled_linear_group_fwd: the gated product takes two members of equal width (paired forward tiles) and a 16-byte aligned output");
   TT_REQUIRE(x && tiled_weights && n_out && y && aligned16(x) && aligned16(tiled_weights), "tiled_linear_group_fwd: pointers must be non-null and 16-byte aligned");
   TT_REQUIRE(n_members >= 1 && n_members <= kGroupMax, "tiled_linear_group_fwd: 1 to %d members (got %d)", kGroupMax, n_members);
   TT_REQUIRE(M > 0 && k_contract > 0 && k_contract % 64 == 0, "tiled_linear_group_fwd: k_contract (%lld) must be a positive multiple of 64", (long long)k_contract);
@@ -953,6 +959,7 @@ extern "C" int ttamd_tiled_linear_group_fwd_bf16(const void* x, const void* tile
   g.Wt = reinterpret_cast<const char*>(tiled_weights);
   g.M = (int)M; g.Nout = (int)n_off; g.Kc = (int)k_contract;
   g.lw_row_major = 1;
+  g.act = reinterpret_cast<uint16_t*>(act);
   return launch_dense(g, reinterpret_cast<hipStream_t>(stream));
 }
 

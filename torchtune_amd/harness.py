@@ -29,7 +29,7 @@ from torch.utils.checkpoint import checkpoint
 
 from .modules import layer_ops
 from .modules.peft import LoRALinear, get_adapter_params, lora_linear_group, lora_swiglu_group, set_trainable_params
-from .qat import FakeQuantizedLinear, Int8DynActInt4WeightQATQuantizer, fake_quantized_linear_group
+from .qat import FakeQuantizedLinear, Int8DynActInt4WeightQATQuantizer, fake_quantized_linear_group, fake_quantized_swiglu_group
 
 
 # True: projections that read the same tensor (q/k/v, gate/up) go through the group kernels; False: one call per
@@ -180,7 +180,9 @@ class FeedForward(nn.Module):
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         # gate and up read the same tensor (torchtune/modules/feed_forward.py:50-53): one group
         if GROUP_SHARED_INPUT and GATED_EPILOGUE:
-            act = lora_swiglu_group(x, self.w1, self.w3)  # the product written by the pair's GEMM launch
+            # the product written by the pair's GEMM launch
+            act = (fake_quantized_swiglu_group(x, self.w1, self.w3) if isinstance(self.w1, FakeQuantizedLinear)
+                   else lora_swiglu_group(x, self.w1, self.w3))
             if act is not None:
                 return self.w2(act)
         g, u = _shared_input(x, (self.w1, self.w3)) if GROUP_SHARED_INPUT else (self.w1(x), self.w3(x))

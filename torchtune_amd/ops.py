@@ -615,11 +615,14 @@ def fq_per_group_int4_sym_tiled(w: torch.Tensor, group_size: int, forward: bool 
 
 
 def fq_int4_sym_tiled_group(ws: Sequence[torch.Tensor], group_size: int, forward: bool = True, backward: bool = True,
-                            qparam_dtype: torch.dtype = torch.float32, eps: Optional[float] = None):
+                            qparam_dtype: torch.dtype = torch.float32, eps: Optional[float] = None, paired: bool = False):
     """Weights [N_i, K] of layers with a common input -> (forward tiles of the weights stacked along N | None, transposed
     tiles of the same stack | None, [scale_i fp32 [N_i, K/g]]): what ``tiled_linear_group_fwd`` / ``tiled_linear_group_dx``
-    read.  Each member's values are those of ``fq_per_group_int4_sym`` on it alone."""
+    read.  Each member's values are those of ``fq_per_group_int4_sym`` on it alone.  ``paired`` (two members of equal
+    shape): the forward tiles alternate 128 columns of the one with 128 of the other, what the gated group forward reads."""
     K = ws[0].shape[1]
+    if paired and (len(ws) != 2 or ws[0].shape != ws[1].shape or ws[0].shape[0] % 128):
+        raise ValueError("fq_int4_sym_tiled_group: the paired layout takes two weights of equal shape, N a multiple of 128")
     for w in ws:
         _need_gpu(w, "fq_int4_sym_tiled_group")
         if w.dtype != torch.bfloat16 or w.dim() != 2 or w.shape[1] != K or not tiled_weight_shape_ok(w.shape[0], K, group_size):
@@ -642,9 +645,10 @@ def fq_int4_sym_tiled_group(ws: Sequence[torch.Tensor], group_size: int, forward
             events = _fq_timer(f"per_group_tiled{int(forward) + int(backward)}", N, K, group_size, 2) if _fq_timer is not None else None
             if events:
                 events[0].record()
+            f_off = (128 if n_off else 0) if paired else n_off  # paired: the second member starts 128 columns in
             rc = lib.ttamd_fq_per_group_int4_sym_tiled_at_bf16(wc.data_ptr(), N, K, group_size, qcode, e,
-                                                               tf.data_ptr() + 2 * K * n_off if forward else None, _ptr(tb), n_total, n_off,
-                                                               scale.data_ptr(), _stream(w))
+                                                               tf.data_ptr() + 2 * K * f_off if forward else None, 1 if paired else 0,
+                                                               _ptr(tb), n_total, n_off, scale.data_ptr(), _stream(w))
             if events:
                 events[1].record()
             _lib.check(rc, "fq_int4_sym_tiled_group")
@@ -654,8 +658,10 @@ def fq_int4_sym_tiled_group(ws: Sequence[torch.Tensor], group_size: int, forward
 
 
 def tiled_linear_group_fwd(x: torch.Tensor, tiled: torch.Tensor, n_outs: Sequence[int],
-                           biases: Optional[Sequence[Optional[torch.Tensor]]] = None):
-    """-> [y_i [M, n_out_i]] = x @ Wd_i.T (+ bias_i) for weights stacked in the tiled layout, one launch."""
+                           biases: Optional[Sequence[Optional[torch.Tensor]]] = None, swiglu: bool = False):
+    """-> [y_i [M, n_out_i]] = x @ Wd_i.T (+ bias_i) for weights stacked in the tiled layout, one launch.  ``swiglu`` (two
+    members of equal width whose forward tiles are in the paired layout): ``silu(y_0) * y_1`` is appended, written by the
+    same launch."""
     x = _bf16_2d(x, "tiled_linear_group_fwd")
     M, K = x.shape
     n = len(n_outs)
@@ -663,7 +669,10 @@ def tiled_linear_group_fwd(x: torch.Tensor, tiled: torch.Tensor, n_outs: Sequenc
         raise ValueError(f"tiled_linear_group_fwd: 1 to {_lib.GROUP_MAX} members with widths that are multiples of 256 (got {list(n_outs)})")
     if tiled.dtype != torch.bfloat16 or tiled.numel() != sum(n_outs) * K or not tiled.is_contiguous():
         raise ValueError(f"tiled_linear_group_fwd: the tiled weights must be a contiguous bfloat16 tensor of {sum(n_outs)} x {K} elements")
+    if swiglu and (n != 2 or n_outs[0] != n_outs[1]):
+        raise ValueError("tiled_linear_group_fwd: swiglu takes the gate and the up projection, two members of equal width")
     ys = [torch.empty(M, o, dtype=torch.bfloat16, device=x.device) for o in n_outs]
+    act = torch.empty(M, n_outs[0], dtype=torch.bfloat16, device=x.device) if swiglu else None
     bs = [None] * n if biases is None else [None if b is None else b.contiguous() for b in biases]
     for b, o in zip(bs, n_outs):
         if b is not None and (b.dtype != torch.bfloat16 or b.numel() != o):
@@ -676,11 +685,11 @@ def tiled_linear_group_fwd(x: torch.Tensor, tiled: torch.Tensor, n_outs: Sequenc
         events = _gemm_timer("tiled", M, sum(n_outs), K, 0) if _gemm_timer is not None else None
         if events:
             events[0].record()
-        rc = lib.ttamd_tiled_linear_group_fwd_bf16(x.data_ptr(), tiled.data_ptr(), n, c_n, c_b, c_y, M, K, _stream(x))
+        rc = lib.ttamd_tiled_linear_group_fwd_bf16(x.data_ptr(), tiled.data_ptr(), n, c_n, c_b, c_y, _ptr(act), M, K, _stream(x))
         if events:
             events[1].record()
     _lib.check(rc, "tiled_linear_group_fwd")
-    return ys
+    return ys + [act] if swiglu else ys
 
 
 def tiled_linear_group_dx(gys: Sequence[torch.Tensor], tiled_t: torch.Tensor, K: int) -> torch.Tensor:

@@ -297,33 +297,41 @@ class _TiledFakeQuantGroupFn(torch.autograd.Function):
     the members' weight quantizers (same config)."""
 
     @staticmethod
-    def forward(ctx, x, quantizers, *flat):
+    def forward(ctx, x, quantizers, swiglu: bool, *flat):
         weights, biases = flat[0::2], flat[1::2]
         c = quantizers[0].config
         K = weights[0].shape[1]
         x2 = x.reshape(-1, K)
         need_gx = ctx.needs_input_grad[0]
         tf, tb, scales = ops.fq_int4_sym_tiled_group([w.detach() for w in weights], c.group_size, forward=True, backward=need_gx,
-                                                     qparam_dtype=c.scale_precision, eps=c.eps)
+                                                     qparam_dtype=c.scale_precision, eps=c.eps, paired=swiglu)
         for q, s in zip(quantizers, scales):
             q.scale = s.to(c.scale_precision)
             q.zero_point = None
-        ys = ops.tiled_linear_group_fwd(x2, tf, [w.shape[0] for w in weights], biases)
-        ctx.save_for_backward(x2, tb)
+        ys = ops.tiled_linear_group_fwd(x2, tf, [w.shape[0] for w in weights], biases, swiglu=swiglu)
         ctx.x_shape = x.shape
         ctx.shapes = tuple(tuple(w.shape) for w in weights)
         ctx.has_bias = tuple(b is not None for b in biases)
+        ctx.swiglu = swiglu
+        if swiglu:  # ``silu(w1 x) * w3 x`` (torchtune/modules/feed_forward.py:50-53) from the launch's epilogue: the one output
+            ctx.save_for_backward(x2, tb, ys[0], ys[1])
+            return ys[2].view(*x.shape[:-1], ys[2].shape[-1])
+        ctx.save_for_backward(x2, tb)
         return tuple(y.view(*x.shape[:-1], y.shape[-1]) for y in ys)
 
     @staticmethod
     def backward(ctx, *gys):
-        x2, tb = ctx.saved_tensors
+        if ctx.swiglu:
+            x2, tb, gate, up = ctx.saved_tensors
+            gys = ops.swiglu_bwd(gys[0].reshape(gate.shape), gate, up)
+        else:
+            x2, tb = ctx.saved_tensors
         K = ctx.shapes[0][1]
         gy2 = [torch.zeros(x2.shape[0], N, dtype=x2.dtype, device=x2.device) if g is None else g.reshape(-1, N)
                for g, (N, _) in zip(gys, ctx.shapes)]
-        out = [ops.tiled_linear_group_dx(gy2, tb, K).view(ctx.x_shape) if ctx.needs_input_grad[0] else None, None]
+        out = [ops.tiled_linear_group_dx(gy2, tb, K).view(ctx.x_shape) if ctx.needs_input_grad[0] else None, None, None]
         for i, (N, _) in enumerate(ctx.shapes):
-            need_w, need_b = ctx.needs_input_grad[2 + 2 * i:4 + 2 * i]
+            need_w, need_b = ctx.needs_input_grad[3 + 2 * i:5 + 2 * i]
             gw = None
             if need_w:
                 own = ops.gemm_tn_applies(gy2[i].shape[0], N, K) and (N // 256) * (K // 256) >= TN_GEMM_MIN_TILES
@@ -332,7 +340,15 @@ class _TiledFakeQuantGroupFn(torch.autograd.Function):
         return tuple(out)
 
 
-def fake_quantized_linear_group(x: torch.Tensor, layers) -> Tuple[torch.Tensor, ...]:
+def fake_quantized_swiglu_group(x: torch.Tensor, gate, up) -> Optional[torch.Tensor]:
+    """``silu(gate(x)) * up(x)`` (``torchtune/modules/feed_forward.py:50-53``) for two ``FakeQuantizedLinear`` layers, with the
+    product written by the pair's one GEMM launch; ``None`` where the group kernels do not apply (the caller multiplies)."""
+    if not _group_tiled_ok(x, (gate, up)) or gate.out_features != up.out_features:
+        return None
+    return fake_quantized_linear_group(x, (gate, up), swiglu=True)
+
+
+def fake_quantized_linear_group(x: torch.Tensor, layers, swiglu: bool = False) -> Tuple[torch.Tensor, ...]:
     """``tuple(layer(x) for layer in layers)`` for ``FakeQuantizedLinear`` layers that read the same input (``q_proj`` /
     ``k_proj`` / ``v_proj``, ``torchtune/modules/attention.py:234,262-263``; ``w1`` / ``w3``,
     ``torchtune/modules/feed_forward.py:50-53``).  When every member is the 8da4w kind with one configuration and the
@@ -340,6 +356,8 @@ def fake_quantized_linear_group(x: torch.Tensor, layers) -> Tuple[torch.Tensor, 
     members (the 1024-wide k / v projections) ride in the wide launch instead of falling back to the vendor library, and
     the members' grad-inputs are summed inside the GEMM.  Otherwise the layers are called in turn."""
     if not _group_tiled_ok(x, layers):
+        if swiglu:
+            raise ValueError("fake_quantized_linear_group: the gated product needs a pair the group kernels serve")
         return tuple(layer(x) for layer in layers)
     first = layers[0]
     xq = x if first.activation_fake_quantizer is None else first.activation_fake_quantizer(x)
@@ -349,7 +367,8 @@ def fake_quantized_linear_group(x: torch.Tensor, layers) -> Tuple[torch.Tensor, 
     flat = []
     for layer in layers:
         flat += [layer.weight, layer.bias]
-    return _TiledFakeQuantGroupFn.apply(xq, tuple(layer.weight_fake_quantizer for layer in layers), *flat)
+    out = _TiledFakeQuantGroupFn.apply(xq, tuple(layer.weight_fake_quantizer for layer in layers), swiglu, *flat)
+    return out
 
 
 def _group_tiled_ok(x: torch.Tensor, layers) -> bool:
