@@ -75,7 +75,8 @@ class GemmTimer:
 
     def __call__(self, kind, M, N, K, rank):
         # "fwd" / "bwd": one layer, one call of the library.  "fwd_group" / "bwd_group": the layers of a group with a common
-        # input (N and rank are lists), one call; "fwd_gated": the gate / up pair with its gated product in the same call.  Between the events lie all launches of the call: with the weight expanded
+        # input (N and rank are lists), one call; "fwd_gated": the gate / up pair with its gated product in the same call;
+        # "bwd_swiglu": the grad-input of the layer after the gated product, carried on to the gradients of gate and up.  Between the events lie all launches of the call: with the weight expanded
         # once per call (many tokens) one expansion launch per member and one GEMM launch; otherwise one fused launch per
         # member (forward) or the single fused grad-input launch over all members' output columns.
         from torchtune_amd import _lib, ops
@@ -109,6 +110,9 @@ class GemmTimer:
         else:
             launches = 1
             nbytes = 2.0 * M * K + sum(2.0 * M * n + per_w * n * K + 2.0 * r * (M + K) for n, r in zip(Ns, ranks))
+            if kind == "bwd_swiglu":  # gate and up read, their two gradients written in place of the one grad-input (expanded);
+                # otherwise the grad-input written, then read again with gate and up by the pass that writes the two gradients
+                nbytes += 2.0 * M * K * (3 if expanded else 5)
         self.expanded_calls += 1 if expanded else 0
         key = (kind, M, Ns if len(Ns) > 1 else Ns[0], K)
         seen = self.counts.get(key, [0, flops, nbytes, launches])
@@ -522,6 +526,9 @@ def main() -> int:
     ap.add_argument("--no-config1", action="store_true", help="skip the single-layer configuration timed on GPU and CPU")
     ap.add_argument("--no-gated-epilogue", action="store_true",
                     help="A/B: silu(gate) * up as a pass of its own instead of the epilogue of the gate / up GEMM launch")
+    ap.add_argument("--swiglu-bwd-epilogue", action="store_true",
+                    help="A/B: the backward of silu(gate) * up from the epilogue of the down projection's grad-input GEMM launch "
+                         "instead of a pass of its own (QLoRA workloads)")
     ap.add_argument("--no-group", action="store_true",
                     help="one call per projection, as the reference's modules make them, instead of the group kernels for the "
                          "projections that share an input (q/k/v, gate/up): for A/B timing")
@@ -552,6 +559,7 @@ def main() -> int:
     harness.SDPA_BACKEND = args.sdpa
     harness.GROUP_SHARED_INPUT = not args.no_group
     harness.GATED_EPILOGUE = not args.no_gated_epilogue
+    harness.SWIGLU_BWD_EPILOGUE = args.swiglu_bwd_epilogue
     ops.EXPANDED_WEIGHT_PATH = not args.no_expanded_weight
     if args.no_qat_tiled_gemm:
         from torchtune_amd import qat as qat_module
@@ -720,7 +728,10 @@ def main() -> int:
             "kernel": ("nf4_gemm_dense_kernel with the nf4_expand_tiled_kernel launches that precede it in the same call (NF4 weight "
                        "expanded once per call into scratch memory, then a bf16 MFMA GEMM with the LoRA adapter in its epilogue"
                        + ("; the gate / up launch also forms silu(gate) * up there, counted as zero FLOPs" if harness.GATED_EPILOGUE
-                          and harness.GROUP_SHARED_INPUT else "") + "; forward and grad-input calls)"
+                          and harness.GROUP_SHARED_INPUT else "")
+                       + (", and the down projection's grad-input launch the backward of that product" if harness.GATED_EPILOGUE
+                          and harness.GROUP_SHARED_INPUT and harness.SWIGLU_BWD_EPILOGUE and not qat else "")
+                       + "; forward and grad-input calls)"
                        if timer.expanded_calls * 2 > calls else
                        "nf4_gemm_rs_kernel (fused NF4-dequant + LoRA bf16 MFMA GEMM, forward and grad-input launches)"),
             "achieved": round(achieved, 1),

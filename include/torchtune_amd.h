@@ -254,6 +254,23 @@ int ttamd_nf4_linear_bwd_dx_ws_bf16(const void* gy, const uint8_t* quantized_dat
                                     size_t workspace_bytes, void* stream);
 
 /*
+ * The grad-input of the layer that consumes a gated product, act = silu(gate) * up (the w2 of
+ * torchtune/modules/feed_forward.py:53 applied to the product of :50-53), carried on to the gradients of gate and up:
+ *     gact  = bf16(gy . D(W) + gh . lora_a)                    (what ttamd_nf4_linear_bwd_dx_ws_bf16 writes as gx)
+ *     ggate, gup = ttamd_swiglu_bwd_bf16(gact, gate, up)       bit for bit
+ * gate, up, ggate, gup [M,K] bf16; the other arguments as for ttamd_nf4_linear_bwd_dx_ws_bf16.  On the many-token path
+ * (the workspace holds the expanded weight) the GEMM's epilogue reads gate and up and writes the two gradients itself:
+ * gact never reaches memory (one write and one read of [M,K] less, and no launch of the stand-alone kernel).  At other
+ * sizes the call runs the two existing steps, with gact parked in ggate.  The reference has no counterpart: autograd
+ * runs the backward of the linear, of the multiply and of silu one after the other.
+ */
+int ttamd_nf4_linear_bwd_dx_swiglu_ws_bf16(const void* gy, const uint8_t* quantized_data, const void* block_scalers,
+                                           const uint8_t* quantized_data_t, const void* block_scalers_t, const void* gh,
+                                           const void* lora_a, int rank, const void* gate, const void* up, void* ggate,
+                                           void* gup, int64_t M, int64_t N, int64_t K, void* workspace, size_t workspace_bytes,
+                                           void* stream);
+
+/*
  * Adapter gradients (what autograd derives for lora.py:144-146):
  *     gh = scale . gy . B        [M,rank] bf16
  *     gA = gh^T . x              [rank,K] bf16

@@ -19,7 +19,7 @@ import torch
 from oracle import lora_oracle, nf4_oracle
 from torchtune_amd import ops
 from torchtune_amd.modules import layer_ops
-from torchtune_amd.modules.peft import LoRALinear, group_applies, lora_linear_group, lora_swiglu_group
+from torchtune_amd.modules.peft import LoRALinear, group_applies, lora_feed_forward, lora_linear_group, lora_swiglu_group
 from torchtune_amd.nf4_tensor import to_nf4
 
 pytestmark = pytest.mark.gpu
@@ -274,6 +274,82 @@ def test_gated_module_function_matches_group_then_swiglu(M, K, width):
         assert torch.equal(a.view(torch.int16), b.view(torch.int16))
     layers[1].disabled = True
     assert lora_swiglu_group(x, layers[0], layers[1]) is None   # the caller falls back to its own multiply
+
+
+DX_SWIGLU_SHAPES = [
+    # M, N (rows of the weight), K (its columns = width of gate and up), rank, transposed copies
+    (4096, 256, 4096, 16, False),            # 256 tiles of 256 x 256: the two gradients leave the GEMM's epilogue
+    (4096, 256, 4096, 16, True),
+    (2048 + 192, 512, 8192, 8, False),       # a last row tile with 192 rows
+    (2048, 320, 4352, 0, False),             # no adapter; 136 tiles (a partly filled round)
+    (8192, 4096, 14336, 16, False),          # the 8B down projection at its real size (batch 4 x 2048)
+    (4096, 8192, 28672, 16, False),          # the 70B one (batch 1 x 4096)
+    (16, 512, 1024, 8, True),                # few tokens: the grad-input as usual, then the stand-alone kernel in place
+    (300, 512, 512, 16, False),
+    (2048, 256, 1152, 16, True),             # many tokens, too few tiles for the expanded path
+]
+
+
+@pytest.mark.parametrize("M,N,K,rank,copies", DX_SWIGLU_SHAPES, ids=[f"M{s[0]}_N{s[1]}_K{s[2]}_r{s[3]}{'_t' if s[4] else ''}" for s in DX_SWIGLU_SHAPES])
+def test_grad_input_carried_through_swiglu_equals_the_two_steps_bitwise(M, N, K, rank, copies):
+    """``ttamd_nf4_linear_bwd_dx_swiglu_ws_bf16`` against ``ttamd_nf4_linear_bwd_dx_ws_bf16`` followed by
+    ``ttamd_swiglu_bwd_bf16``: both gradients bit for bit (the same GEMM, the same arithmetic on its rounded result).
+    Those two are themselves compared with fp32 matmuls of the dequantised weight (tests/test_gpu_lora_linear.py) and
+    with autograd's backward of ``F.silu(g) * u`` in bf16 (tests/test_gpu_layer_ops.py)."""
+    g = torch.Generator().manual_seed(M + N + K)
+    W = (torch.randn(N, K, generator=g) * 0.02).to(BF)
+    t = to_nf4(W.to(DEV))
+    gy = torch.randn(M, N, generator=g).to(BF).to(DEV)
+    gate = torch.randn(M, K, generator=g).to(BF).to(DEV)
+    up = torch.randn(M, K, generator=g).to(BF).to(DEV)
+    gh = A = None
+    if rank:
+        gh = (torch.randn(M, rank, generator=g) * 0.1).to(BF).to(DEV)
+        A = lora_oracle.lora_a_init_(torch.empty(rank, K), g).to(BF).to(DEV)
+    tr = t.backward_copy() if copies else None
+    gx = ops.nf4_linear_bwd_dx(gy, t.quantized_data, t.block_scalers(), K, gh, A, transposed=tr)
+    gg0, gu0 = ops.swiglu_bwd(gx, gate, up)
+    gg1, gu1 = ops.nf4_linear_bwd_dx(gy, t.quantized_data, t.block_scalers(), K, gh, A, transposed=tr, swiglu=(gate, up))
+    assert torch.equal(gg0.view(torch.int16), gg1.view(torch.int16))
+    assert torch.equal(gu0.view(torch.int16), gu1.view(torch.int16))
+
+
+def test_grad_input_carried_through_swiglu_rejects_mismatched_gate():
+    t = to_nf4((torch.randn(128, 256) * 0.02).to(BF).to(DEV))
+    gy = torch.randn(8, 128, device=DEV, dtype=BF)
+    good = torch.randn(8, 256, device=DEV, dtype=BF)
+    with pytest.raises(ValueError):
+        ops.nf4_linear_bwd_dx(gy, t.quantized_data, t.block_scalers(), 256, swiglu=(good, good[:, :128]))
+    with pytest.raises(ValueError):
+        ops.nf4_linear_bwd_dx(gy, t.quantized_data, t.block_scalers(), 256, swiglu=(good[:4], good[:4]))
+
+
+@pytest.mark.parametrize("M,K,width", [(4096, 512, 4096), (64, 512, 512)], ids=["epilogue", "own_pass"])
+def test_feed_forward_node_matches_gated_pair_then_down(M, K, width):
+    """``lora_feed_forward`` against ``down(lora_swiglu_group(x, gate, up))``: output and every gradient bit for bit."""
+    pair, _ = _layers(K, (width, width), (16, 16), 32.0, False, seed=M + width)
+    (down,), _ = _layers(width, (K,), (16,), 32.0, False, seed=M + width + 1)
+    layers = list(pair) + [down]
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(M, K, generator=g).to(BF).to(DEV)
+    gy = torch.randn(M, K, generator=g).to(BF).to(DEV)
+
+    def run(node):
+        for l in layers:
+            l.zero_grad()
+        xg = x.clone().requires_grad_()
+        y = lora_feed_forward(xg, *layers) if node else down(lora_swiglu_group(xg, pair[0], pair[1]))
+        assert y is not None
+        y.backward(gy)
+        return [y.detach(), xg.grad] + [p.grad.clone() for l in layers for p in (l.lora_a.weight, l.lora_b.weight)]
+
+    for a, b in zip(run(True), run(False)):
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+    down.disabled = True
+    assert lora_feed_forward(x, *layers) is None   # the caller composes the layers itself
+    down.disabled = False
+    (narrow,), _ = _layers(width // 2, (K,), (16,), 32.0, False, seed=5)
+    assert lora_feed_forward(x, pair[0], pair[1], narrow) is None
 
 
 def test_group_falls_back_when_it_does_not_apply():

@@ -520,3 +520,22 @@ def test_gated_group_entry_point_validates_its_arguments_on_the_host():
     arr[1].N = 128
     assert f(p, arr, 2, p, None, 8, 64, None, 0, None) == -1 and b"act" in lib.ttamd_last_error()
 
+
+
+def test_grad_input_swiglu_entry_point_validates_its_arguments_on_the_host():
+    """``ttamd_nf4_linear_bwd_dx_swiglu_ws_bf16`` wants gate, up and both gradients (non-null, 16-byte aligned) on top of
+    what the plain grad-input entry point checks; refused before any launch."""
+    import ctypes
+
+    from torchtune_amd import _lib
+
+    lib = _lib.load()
+    buf = (ctypes.c_char * 4096)()
+    p = (ctypes.addressof(buf) + 15) & ~15
+    f = lib.ttamd_nf4_linear_bwd_dx_swiglu_ws_bf16
+    #        gy codes scal codes_t scal_t gh   lora_a rank gate up ggate gup  M  N   K   ws  bytes stream
+    assert f(p, p, p, None, None, None, None, 0, None, p, p, p, 8, 64, 64, None, 0, None) == -1 and b"null" in lib.ttamd_last_error()
+    assert f(p, p, p, None, None, None, None, 0, p, p, p, None, 8, 64, 64, None, 0, None) == -1
+    assert f(p, p, p, None, None, None, None, 0, p, p + 2, p, p, 8, 64, 64, None, 0, None) == -1 and b"aligned" in lib.ttamd_last_error()
+    assert f(p, p, p, None, None, None, None, 0, p, p, p, p, 8, 64, 96, None, 0, None) == -1      # K not a multiple of 64
+    assert f(p, p, p, p, None, None, None, 0, p, p, p, p, 8, 64, 64, None, 0, None) == -1 and b"together" in lib.ttamd_last_error()

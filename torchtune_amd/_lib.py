@@ -80,6 +80,11 @@ SIGNATURES = {
         [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _int, _c_void_p, _i64, _i64, _i64,
          _c_void_p, _size, _c_void_p],
     ),
+    "ttamd_nf4_linear_bwd_dx_swiglu_ws_bf16": (
+        _int,
+        [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _int, _c_void_p, _c_void_p, _c_void_p,
+         _c_void_p, _i64, _i64, _i64, _c_void_p, _size, _c_void_p],
+    ),
     "ttamd_lora_bwd_workspace_bytes": (_size, [_i64, _i64, _i64, _int]),
     "ttamd_lora_bwd_bf16": (
         _int,

@@ -61,9 +61,16 @@ int run_gemm_rs_group_dx(const GroupDx& d, const void* gh_cat, void* gx, hipStre
 // nf4_gemm_dense.hip: expand the weight once into scratch memory, then a plain bf16 GEMM (many tokens)
 bool dense_path_applies(int64_t M, int64_t Nout, int64_t Kc);
 size_t dense_workspace_bytes(int64_t M, int64_t Nout, int64_t Kc);
+// The result taken as the gradient of silu(gate) * up (gate, up [M, Nout] bf16): C receives the gradient of gate, gup
+// that of up, and the result itself is not stored.
+struct DenseSwigluBwd {
+  const void* gate;
+  const void* up;
+  void* gup;
+};
 int run_gemm_dense(const void* X, const uint8_t* codes, const void* scal, int mode, const void* lX, int ldlx, const void* lW,
                    bool lw_row_major, int R, float lscale, const void* bias, const void* cscale, void* C, int64_t M, int64_t Nout,
-                   int64_t Kc, void* workspace, hipStream_t s);
+                   int64_t Kc, void* workspace, hipStream_t s, const DenseSwigluBwd* swiglu_bwd = nullptr);
 size_t dense_group_fwd_workspace_bytes(const GroupGemm& d);
 // act != nullptr: two members of equal width (gate, up); the launch also writes act = silu(y[0]) * y[1]
 bool dense_group_gated_applies(const GroupGemm& d);

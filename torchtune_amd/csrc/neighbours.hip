@@ -226,8 +226,9 @@ __global__ __launch_bounds__(256) void swiglu_fwd_kernel(const uint16_t* __restr
 
 constexpr int kSwigluBwdChunks = 1;  // 16-byte chunks per lane (two measured 9 % slower)
 
-__global__ __launch_bounds__(256) void swiglu_bwd_kernel(const uint16_t* __restrict__ go, const uint16_t* __restrict__ g,
-                                                         const uint16_t* __restrict__ u, uint16_t* __restrict__ gg,
+// go and gg may be the same buffer (a lane reads its chunk of go before it writes that chunk of gg; no other lane touches it)
+__global__ __launch_bounds__(256) void swiglu_bwd_kernel(const uint16_t* go, const uint16_t* __restrict__ g,
+                                                         const uint16_t* __restrict__ u, uint16_t* gg,
                                                          uint16_t* __restrict__ gu, int64_t n_chunks) {
   const int64_t base = (int64_t)blockIdx.x * (256 * kSwigluBwdChunks) + threadIdx.x;
   u32x4_t ov[kSwigluBwdChunks], gv[kSwigluBwdChunks], uv[kSwigluBwdChunks];
@@ -248,20 +249,10 @@ __global__ __launch_bounds__(256) void swiglu_bwd_kernel(const uint16_t* __restr
     u32x4_t og, ou;
 #pragma unroll
     for (int d = 0; d < 4; ++d) {
-      float rg[2], ru[2];
-#pragma unroll
-      for (int e = 0; e < 2; ++e) {
-        const float gval = e ? hi_f(gv[c][d]) : lo_f(gv[c][d]);
-        const float uval = e ? hi_f(uv[c][d]) : lo_f(uv[c][d]);
-        const float oval = e ? hi_f(ov[c][d]) : lo_f(ov[c][d]);
-        const float s = sigmoid_f(gval);
-        const float a = round_to_bf16(gval * s);
-        ru[e] = oval * a;
-        const float ga = round_to_bf16(oval * uval);
-        rg[e] = ga * (s * (1.0f + gval * (1.0f - s)));
-      }
-      og[d] = pack2(rg[0], rg[1]);
-      ou[d] = pack2(ru[0], ru[1]);
+      uint32_t dg, du;
+      swiglu_bwd_pair(ov[c][d], gv[c][d], uv[c][d], dg, du);
+      og[d] = dg;
+      ou[d] = du;
     }
     __builtin_nontemporal_store(og, reinterpret_cast<u32x4_t*>(gg) + chunk);
     __builtin_nontemporal_store(ou, reinterpret_cast<u32x4_t*>(gu) + chunk);

@@ -541,6 +541,30 @@ extern "C" int ttamd_nf4_linear_bwd_dx_ws_bf16(const void* gy, const uint8_t* qu
   return dispatch_gemm<true>(g, reinterpret_cast<hipStream_t>(stream));
 }
 
+extern "C" int ttamd_nf4_linear_bwd_dx_swiglu_ws_bf16(const void* gy, const uint8_t* quantized_data, const void* block_scalers,
+                                                      const uint8_t* quantized_data_t, const void* block_scalers_t, const void* gh,
+                                                      const void* lora_a, int rank, const void* gate, const void* up, void* ggate,
+                                                      void* gup, int64_t M, int64_t N, int64_t K, void* workspace,
+                                                      size_t workspace_bytes, void* stream) {
+  if (int rc = check_gemm_args("nf4_linear_bwd_dx_swiglu", gy, quantized_data, block_scalers, ggate, M, N, K, rank, gh, lora_a)) return rc;
+  TT_REQUIRE(gate && up && gup, "nf4_linear_bwd_dx_swiglu: null pointer argument");
+  TT_REQUIRE(aligned16(gate) && aligned16(up) && aligned16(ggate) && aligned16(gup), "nf4_linear_bwd_dx_swiglu: pointers must be 16-byte aligned");
+  TT_REQUIRE((quantized_data_t == nullptr) == (block_scalers_t == nullptr),
+             "nf4_linear_bwd_dx_swiglu: the transposed codes and scalers must be given together");
+  if (workspace != nullptr && dense_path_applies(M, K, N) && workspace_bytes >= dense_workspace_bytes(M, K, N)) {
+    const DenseSwigluBwd sw = {gate, up, gup};
+    const bool tr = quantized_data_t != nullptr;
+    TT_REQUIRE(!tr || (aligned16(quantized_data_t) && aligned16(block_scalers_t)), "nf4_linear_bwd_dx_swiglu: transposed copies must be 16-byte aligned");
+    return run_gemm_dense(gy, tr ? quantized_data_t : quantized_data, tr ? block_scalers_t : block_scalers, tr ? 1 : 3, gh, rank, lora_a,
+                          false, rank, 1.0f, nullptr, nullptr, ggate, M, K, N, workspace, reinterpret_cast<hipStream_t>(stream), &sw);
+  }
+  // other sizes: the grad-input as usual, parked in ggate, then the stand-alone kernel in place
+  if (int rc = ttamd_nf4_linear_bwd_dx_ws_bf16(gy, quantized_data, block_scalers, quantized_data_t, block_scalers_t, gh, lora_a, rank, ggate,
+                                               M, N, K, workspace, workspace_bytes, stream))
+    return rc;
+  return ttamd_swiglu_bwd_bf16(ggate, gate, up, ggate, gup, M * K, stream);
+}
+
 extern "C" int ttamd_nf4_linear_bwd_dx_bf16(const void* gy, const uint8_t* quantized_data, const void* block_scalers,
                                             const uint8_t* quantized_data_t, const void* block_scalers_t, const void* gh,
                                             const void* lora_a, int rank, void* gx, int64_t M, int64_t N, int64_t K,

@@ -289,8 +289,15 @@ struct DenseArgs {
   int M, Nout, Kc;  // Nout, Kc: totals
   int lw_row_major, ldlx;
   int tiles_m, tiles_n;
-  uint16_t* act;    // GATED launches only: [M, out[0].width] bf16 = silu(out 0) * out 1
+  uint16_t* act;    // gated launches only: [M, out[0].width] bf16 = silu(out 0) * out 1
+  // SwiGLU-backward launches only (one output): the result is the gradient of silu(gate) * up; out[0].C receives the
+  // gradient of gate and sw_gup that of up, both [M, out[0].width] like gate and up themselves
+  const uint16_t* sw_gate;
+  const uint16_t* sw_up;
+  uint16_t* sw_gup;
 };
+
+constexpr int kEpiPlain = 0, kEpiGated = 1, kEpiSwigluBwd = 2;
 
 constexpr int kAEntry = 32768;  // activation ring: 3 entries of 256 rows x 64 k
 constexpr int kWBase = 3 * kAEntry;
@@ -302,9 +309,14 @@ constexpr int kLdsDense = kWBase + 4 * kWStage;
 // the waves with wn < 2 own the gate's, the others the up projection's.  Each wave writes its member's output as usual;
 // the bf16 bands then meet in LDS and the workgroup also writes act = bf16(bf16(silu(gate)) * up), the arithmetic of
 // ttamd_swiglu_fwd_bf16 on the rounded outputs, bit for bit.
-template <bool LW_ROW_MAJOR, bool GATED = false>
+// kEpiSwigluBwd (grad-input of the layer that follows the gated product, feed_forward.py:53): the result o = bf16(...)
+// is the gradient of silu(gate) * up and is not stored; each 16-byte piece of it meets the same piece of gate and up
+// on its way out and the launch writes the gradients of gate and up instead, the arithmetic of ttamd_swiglu_bwd_bf16 on
+// the rounded result, bit for bit.
+template <bool LW_ROW_MAJOR, int EPI = kEpiPlain>
 __global__ __launch_bounds__(512) void nf4_gemm_dense_kernel(const DenseArgs g) {
 #if defined(__HIP_DEVICE_COMPILE__)
+  constexpr bool GATED = EPI == kEpiGated;
   constexpr int MT = 8, NT = 4;  // 16 x 16 MFMA tiles per wave
   extern __shared__ __attribute__((aligned(16))) char smem[];
   const int tid = threadIdx.x;
@@ -572,6 +584,20 @@ __global__ __launch_bounds__(512) void nf4_gemm_dense_kernel(const DenseArgs g) 
     const uint16_t* bias = g.out[oi].bias;
     const uint16_t* cscale = g.out[oi].cscale;
     char* band = smem + wv * 16384;  // 128 rows x 128 bytes
+    // SwiGLU backward: the pieces of gate and up that meet rows [64 half, + 64) of the band; those of the first half are
+    // asked for before the band is staged, the others right after.  Rows beyond M read row M - 1 and are not stored.
+    u32x4_t sw_g[EPI == kEpiSwigluBwd ? 16 : 1], sw_u[EPI == kEpiSwigluBwd ? 16 : 1];
+    const int64_t sw_col = nlo + 8 * (lane & 7);
+    auto sw_fetch = [&](int half) {
+#pragma unroll
+      for (int t = 0; t < (EPI == kEpiSwigluBwd ? 8 : 0); ++t) {
+        const int row = m0 + 128 * wm + 64 * half + 8 * t + (lane >> 3);
+        const int64_t at = (int64_t)(row < g.M ? row : g.M - 1) * width + sw_col;
+        sw_g[8 * half + t] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(g.sw_gate + at));
+        sw_u[8 * half + t] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(g.sw_up + at));
+      }
+    };
+    if constexpr (EPI == kEpiSwigluBwd) sw_fetch(0);
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
       float b4[4] = {0.f, 0.f, 0.f, 0.f};
@@ -605,6 +631,28 @@ __global__ __launch_bounds__(512) void nf4_gemm_dense_kernel(const DenseArgs g) 
     const int c = lane & 7;
     uint16_t* crow = g.out[oi].C + nlo + 8 * c;
     const int mrow0 = m0 + 128 * wm;
+    if constexpr (EPI == kEpiSwigluBwd) {
+      sw_fetch(1);
+#pragma unroll
+      for (int t = 0; t < 16; ++t) {
+        const int r = 8 * t + (lane >> 3);
+        const u32x4_t v = *reinterpret_cast<const u32x4_t*>(band + r * 128 + ((c ^ (r & 7)) << 4));
+        u32x4_t og, ou;
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+          uint32_t dg, du;
+          swiglu_bwd_pair(v[d], sw_g[t][d], sw_u[t][d], dg, du);
+          og[d] = dg;
+          ou[d] = du;
+        }
+        if (mrow0 + r < g.M) {
+          const int64_t at = (int64_t)(mrow0 + r) * width + sw_col;
+          *reinterpret_cast<u32x4_t*>(g.out[oi].C + at) = og;
+          *reinterpret_cast<u32x4_t*>(g.sw_gup + at) = ou;
+        }
+      }
+      return;
+    }
 #pragma unroll 8
     for (int t = 0; t < 16; ++t) {
       const int r = 8 * t + (lane >> 3);
@@ -666,7 +714,9 @@ int launch_dense(DenseArgs& g, hipStream_t s) {
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = -1;
   if (dev < 0 || !attr_set[dev]) {
     for (const void* fn : {reinterpret_cast<const void*>(&nf4_gemm_dense_kernel<true>), reinterpret_cast<const void*>(&nf4_gemm_dense_kernel<false>),
-                           reinterpret_cast<const void*>(&nf4_gemm_dense_kernel<true, true>)}) {
+                           reinterpret_cast<const void*>(&nf4_gemm_dense_kernel<true, kEpiGated>),
+                           reinterpret_cast<const void*>(&nf4_gemm_dense_kernel<true, kEpiSwigluBwd>),
+                           reinterpret_cast<const void*>(&nf4_gemm_dense_kernel<false, kEpiSwigluBwd>)}) {
       hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsDense);
       if (e != hipSuccess) return fail(TTAMD_ELAUNCH, "nf4_gemm_dense: cannot reserve %d bytes of LDS: %s", kLdsDense, hipGetErrorString(e));
     }
@@ -677,7 +727,15 @@ int launch_dense(DenseArgs& g, hipStream_t s) {
     TT_REQUIRE(g.lw_row_major && g.nout == 2 && (g.nad == 2 || g.nad == 0) && g.nseg == 1 && g.out[0].width == g.out[1].width &&
                    g.out[0].width % 128 == 0 && g.Nout == 2 * g.out[0].width,
                "nf4_gemm_dense: the gated launch takes two members of equal width, a multiple of 128");
-    nf4_gemm_dense_kernel<true, true><<<grid, block, kLdsDense, s>>>(g);
+    nf4_gemm_dense_kernel<true, kEpiGated><<<grid, block, kLdsDense, s>>>(g);
+  } else if (g.sw_gup) {
+    TT_REQUIRE(g.nout == 1 && g.out[0].n_begin == 0 && g.out[0].width == g.Nout && !g.out[0].bias && !g.out[0].cscale &&
+                   g.sw_gate && g.sw_up && g.out[0].C,
+               "nf4_gemm_dense: the SwiGLU-backward launch takes one output without bias or column scale");
+    if (g.lw_row_major)
+      nf4_gemm_dense_kernel<true, kEpiSwigluBwd><<<grid, block, kLdsDense, s>>>(g);
+    else
+      nf4_gemm_dense_kernel<false, kEpiSwigluBwd><<<grid, block, kLdsDense, s>>>(g);
   } else if (g.lw_row_major)
     nf4_gemm_dense_kernel<true><<<grid, block, kLdsDense, s>>>(g);
   else
@@ -714,7 +772,7 @@ size_t dense_workspace_bytes(int64_t M, int64_t Nout, int64_t Kc) {
 // One layer: the ordinary forward (mode 0 / 2) or grad-input (mode 1).  Arguments as run_gemm_rs.
 int run_gemm_dense(const void* X, const uint8_t* codes, const void* scal, int mode, const void* lX, int ldlx, const void* lW,
                    bool lw_row_major, int R, float lscale, const void* bias, const void* cscale, void* C, int64_t M, int64_t Nout,
-                   int64_t Kc, void* workspace, hipStream_t s) {
+                   int64_t Kc, void* workspace, hipStream_t s, const DenseSwigluBwd* swiglu_bwd) {
   TT_REQUIRE(dense_path_applies(M, Nout, Kc), "nf4_gemm_dense: shape not served (M=%lld Nout=%lld Kc=%lld)", (long long)M,
              (long long)Nout, (long long)Kc);
   TT_REQUIRE(aligned16(workspace) && aligned16(X) && aligned16(codes) && aligned16(scal), "nf4_gemm_dense: pointers must be 16-byte aligned");
@@ -740,6 +798,14 @@ int run_gemm_dense(const void* X, const uint8_t* codes, const void* scal, int mo
   g.M = (int)M; g.Nout = (int)Nout; g.Kc = (int)Kc;
   g.lw_row_major = lw_row_major ? 1 : 0;
   g.ldlx = ldlx;
+  if (swiglu_bwd) {
+    TT_REQUIRE(swiglu_bwd->gate && swiglu_bwd->up && swiglu_bwd->gup && aligned16(swiglu_bwd->gate) && aligned16(swiglu_bwd->up) &&
+                   aligned16(swiglu_bwd->gup) && aligned16(C),
+               "nf4_gemm_dense: gate, up and their gradients must be non-null and 16-byte aligned");
+    g.sw_gate = reinterpret_cast<const uint16_t*>(swiglu_bwd->gate);
+    g.sw_up = reinterpret_cast<const uint16_t*>(swiglu_bwd->up);
+    g.sw_gup = reinterpret_cast<uint16_t*>(swiglu_bwd->gup);
+  }
   return launch_dense(g, s);
 }
 

@@ -66,7 +66,7 @@ class _QLoRAGroupFn(torch.autograd.Function):
 
 def _group_backward(ctx, x2, h_cat, weights, las, lbs, gy2):
     """Gradients of a group call in the order of its inputs (x, scales, then weight, lora_a, lora_b, bias per member)."""
-    n = len(ctx.scales)
+    n = len(weights)
     members = [ops.GroupMember(w.quantized_data, w.block_scalers(), tr, a, b, None, s, w.shape[0])
                for w, tr, a, b, s in zip(weights, _copies(weights, x2.shape[0]), las, lbs, ctx.scales)]
     need_x = ctx.needs_input_grad[0]
@@ -110,6 +110,52 @@ class _QLoRAGatedFn(torch.autograd.Function):
         return _group_backward(ctx, x2, h_cat, weights, las, lbs, [ggate, gup])
 
 
+class _QLoRAFeedForwardFn(torch.autograd.Function):
+    """``w2(silu(w1(x)) * w3(x))`` for three LoRA linears over NF4 (``torchtune/modules/feed_forward.py:50-53``).
+    Inputs: x, the members' adapter scales, then (weight, lora_a, lora_b, bias or None) of w1, w3 and w2.  Forward as
+    ``_QLoRAGatedFn`` followed by the fused linear; in backward the grad-input GEMM of w2 hands the gradients of the
+    two projections straight to the pair's group backward: its result, the gradient of the gated product, meets gate
+    and up in the GEMM's epilogue and is never written (``ops.nf4_linear_bwd_dx(..., swiglu=...)``)."""
+
+    @staticmethod
+    def forward(ctx, x, scales: Tuple[float, ...], *flat):
+        weights, las, lbs, biases = flat[0::4], flat[1::4], flat[2::4], flat[3::4]
+        K = weights[0].shape[1]
+        for w in weights[:2]:
+            _check_in_features(x, w)
+        x2 = x.reshape(-1, K)
+        members = [ops.GroupMember(w.quantized_data, w.block_scalers(), tr, a, b, bias, s, w.shape[0])
+                   for w, tr, a, b, bias, s in zip(weights[:2], _copies(weights[:2], x2.shape[0]), las, lbs, biases, scales)]
+        h_cat, (gate, up, act) = ops.lora_group_fwd(x2, members, swiglu=True)
+        w2 = weights[2]
+        h2 = ops.lora_hidden(act, las[2])
+        tr = w2.backward_copy_for(act.shape[0], True)
+        y = ops.nf4_lora_linear_fwd(act, w2.quantized_data, w2.block_scalers(), w2.shape[0], h2, lbs[2], scales[2], biases[2],
+                                    block_scalers_t=tr[1] if tr else None)
+        ctx.save_for_backward(x2, h_cat, gate, up, act, h2, *weights, *las, *lbs)
+        ctx.scales = scales
+        ctx.x_shape = x.shape
+        ctx.has_bias = tuple(b is not None for b in biases)
+        return y.view(*x.shape[:-1], y.shape[-1])
+
+    @staticmethod
+    def backward(ctx, gy):
+        saved = ctx.saved_tensors
+        x2, h_cat, gate, up, act, h2 = saved[:6]
+        rest = saved[6:]
+        weights, las, lbs = rest[:3], rest[3:6], rest[6:9]
+        w2 = weights[2]
+        gy2 = gy.reshape(-1, w2.shape[0])
+        gh2, ga2, gb2 = ops.lora_bwd(gy2, act, h2, lbs[2], ctx.scales[2])
+        ggate, gup = ops.nf4_linear_bwd_dx(gy2, w2.quantized_data, w2.block_scalers(), w2.shape[1], gh2, las[2],
+                                           transposed=w2.backward_copy_for(gy2.shape[0], False), swiglu=(gate, up))
+        out = list(_group_backward(ctx, x2, h_cat, weights[:2], las[:2], lbs[:2], [ggate, gup]))
+        _, need_a, need_b, need_bias = ctx.needs_input_grad[10:14]
+        out += [None, ga2 if need_a else None, gb2 if need_b else None,
+                gy2.sum(dim=0) if (ctx.has_bias[2] and need_bias) else None]
+        return tuple(out)
+
+
 def group_applies(x: torch.Tensor, layers: Sequence[torch.nn.Module]) -> bool:
     """True when ``lora_linear_group`` runs the group kernels for these layers on this input."""
     if not 1 <= len(layers) <= ops._lib.GROUP_MAX:
@@ -136,6 +182,24 @@ def lora_swiglu_group(x: torch.Tensor, gate: torch.nn.Module, up: torch.nn.Modul
     for layer in (gate, up):
         flat += [layer.weight, layer.lora_a.weight, layer.lora_b.weight, layer.bias]
     return _QLoRAGatedFn.apply(x, tuple(layer.alpha / layer.rank for layer in (gate, up)), *flat)
+
+
+def lora_feed_forward(x: torch.Tensor, gate: torch.nn.Module, up: torch.nn.Module, down: torch.nn.Module):
+    """``down(silu(gate(x)) * up(x))`` (``torchtune/modules/feed_forward.py:50-53``) as one autograd node: forward as
+    ``lora_swiglu_group`` followed by ``down``; in backward ``down``'s grad-input GEMM writes the gradients of the two
+    projections from its epilogue instead of the gradient of their product.  ``None`` when the group kernels do not
+    apply to the pair or ``down`` does not take the fused path (the caller composes the layers itself)."""
+    if not group_applies(x, (gate, up)) or gate.out_dim != up.out_dim:
+        return None
+    if type(down) is not LoRALinear or down.disabled or down.in_dim != gate.out_dim:
+        return None
+    probe = x.new_empty(1).expand(*x.shape[:-1], down.in_dim)  # x's device, dtype and token count; no memory
+    if not down._fused(probe):
+        return None
+    flat = []
+    for layer in (gate, up, down):
+        flat += [layer.weight, layer.lora_a.weight, layer.lora_b.weight, layer.bias]
+    return _QLoRAFeedForwardFn.apply(x, tuple(layer.alpha / layer.rank for layer in (gate, up, down)), *flat)
 
 
 def lora_linear_group(x: torch.Tensor, layers: Sequence[torch.nn.Module]) -> Tuple[torch.Tensor, ...]:

@@ -290,10 +290,14 @@ def nf4_transpose_for_backward(qdata: torch.Tensor, block_scalers: torch.Tensor,
 
 def nf4_linear_bwd_dx(
     gy: torch.Tensor, qdata: torch.Tensor, block_scalers: torch.Tensor, K: int, gh: Optional[torch.Tensor] = None,
-    lora_a: Optional[torch.Tensor] = None, transposed=None,
-) -> torch.Tensor:
+    lora_a: Optional[torch.Tensor] = None, transposed=None, swiglu: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
+):
     """gx = gy @ D(W) + gh @ lora_a ;  gy [M,N] -> [M,K].  `transposed` = the pair from nf4_transpose_for_backward
-    (fast path) or None (the weight tile is transposed on the fly)."""
+    (fast path) or None (the weight tile is transposed on the fly).
+
+    ``swiglu=(gate, up)`` ([M,K] each): gx is the gradient of ``silu(gate) * up``; the call returns
+    ``(ggate, gup) = swiglu_bwd(gx, gate, up)`` (the same bits) instead of gx, from the GEMM's own epilogue on the
+    many-token path."""
     gy = _bf16_2d(gy, "nf4_linear_bwd_dx")
     M, N = gy.shape
     _check_nf4_operands("nf4_linear_bwd_dx", N, K, qdata, block_scalers, transposed[1] if transposed else None)
@@ -306,22 +310,30 @@ def nf4_linear_bwd_dx(
         rank = gh.shape[1]
         _check_adapter("nf4_linear_bwd_dx", M, K, gh, lora_a, lambda r: (r, K))
     gx = torch.empty(M, K, dtype=torch.bfloat16, device=gy.device)
+    gup = None
+    if swiglu is not None:
+        gate, up = (_bf16_2d(t, "nf4_linear_bwd_dx") for t in swiglu)
+        if tuple(gate.shape) != (M, K) or tuple(up.shape) != (M, K):
+            raise ValueError(f"nf4_linear_bwd_dx: gate {tuple(gate.shape)} and up {tuple(up.shape)} must both be [{M}, {K}]")
+        gup = torch.empty_like(gx)
     lib = _lib.load()
     # without the transposed copy only the expanded-weight path takes a workspace (the first-generation kernel slices nothing)
     ws, ws_bytes = _gemm_workspace(lib, M, K, N, gy.device) if transposed or lib.ttamd_nf4_gemm_expands_weight(M, K, N) else (None, 0)
     with torch.cuda.device(gy.device):
-        events = _gemm_timer("bwd", M, N, K, rank) if _gemm_timer is not None else None
+        events = _gemm_timer("bwd" if swiglu is None else "bwd_swiglu", M, N, K, rank) if _gemm_timer is not None else None
         if events:
             events[0].record()
-        rc = lib.ttamd_nf4_linear_bwd_dx_ws_bf16(
-            gy.data_ptr(), qdata.data_ptr(), block_scalers.data_ptr(), _ptr(transposed[0]) if transposed else None,
-            _ptr(transposed[1]) if transposed else None, _ptr(gh), _ptr(lora_a), rank, gx.data_ptr(), M, N, K, _ptr(ws), ws_bytes,
-            _stream(gy),
-        )
+        head = (gy.data_ptr(), qdata.data_ptr(), block_scalers.data_ptr(), _ptr(transposed[0]) if transposed else None,
+                _ptr(transposed[1]) if transposed else None, _ptr(gh), _ptr(lora_a), rank)
+        if swiglu is None:
+            rc = lib.ttamd_nf4_linear_bwd_dx_ws_bf16(*head, gx.data_ptr(), M, N, K, _ptr(ws), ws_bytes, _stream(gy))
+        else:
+            rc = lib.ttamd_nf4_linear_bwd_dx_swiglu_ws_bf16(*head, gate.data_ptr(), up.data_ptr(), gx.data_ptr(), gup.data_ptr(),
+                                                            M, N, K, _ptr(ws), ws_bytes, _stream(gy))
         if events:
             events[1].record()
     _lib.check(rc, "nf4_linear_bwd_dx")
-    return gx
+    return gx if swiglu is None else (gx, gup)
 
 
 def lora_bwd(
