@@ -125,6 +125,47 @@ def test_group_backward_against_member_calls_and_fp32(M, K, Ns, ranks):
     assert torch.equal(gx, gx2) and all(torch.equal(a, c) and torch.equal(b, d) for (a, b), (c, d) in zip(grads, grads2))
 
 
+WIDE_SHAPES = [
+    # M, K, Ns, ranks: every member at least 8192 wide, of rank <= 16, 1024 rows or more: gh and gB come from one pass over gy
+    (1024, 256, (8192,), (16,)),
+    (1030, 512, (8192 + 64, 8192), (8, 16)),           # a last column group of 64 columns, a last row step of 6 rows, two ranks
+    (2048 + 40, 256, (16384, 8192, 8192), (16, 8, 8)),
+    (8192, 4096, (14336, 14336), (16, 16)),            # the 8B gate / up pair at its real size (batch 4 x 2048)
+]
+
+
+@pytest.mark.parametrize("M,K,Ns,ranks", WIDE_SHAPES, ids=[f"M{s[0]}_K{s[1]}_{'x'.join(map(str, s[2]))}_r{'x'.join(map(str, s[3]))}" for s in WIDE_SHAPES])
+def test_rank_r_backward_of_wide_members_against_fp32(M, K, Ns, ranks):
+    """The adapter gradients of wide members, where ``gh`` and ``grad B`` are two products of one pass over ``gy``: every
+    output against fp32 matmuls of the same bf16 operands (``gh`` and ``grad B`` are bf16 roundings of fp32 sums: rtol 1e-2,
+    atol 1e-2 of the largest entry), the group's ``gh`` against the member-by-member calls bit for bit (its sums are
+    taken per column group, whatever the row ranges), and two runs against each other bit for bit."""
+    mem = _members(K, Ns, ranks, seed=M + K + len(Ns))
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(M, K, generator=g).to(BF).to(DEV)
+    gys = [torch.randn(M, N, generator=g).to(BF).to(DEV) for N in Ns]
+    h_cat = (torch.randn(M, sum(ranks), generator=g) * 0.5).to(BF).to(DEV)
+    members = [m[0] for m in mem]
+    _, grads, gh_cat = ops.lora_group_bwd(x, h_cat, members, gys, want_gx=False)
+    _, grads2, gh_cat2 = ops.lora_group_bwd(x, h_cat, members, gys, want_gx=False)
+    assert torch.equal(gh_cat, gh_cat2) and all(torch.equal(a, c) and torch.equal(b, d) for (a, b), (c, d) in zip(grads, grads2))
+    off = 0
+    for (m, *_), gy, (ga, gb) in zip(mem, gys, grads):
+        r = m.lora_a.shape[0]
+        h = h_cat[:, off:off + r].contiguous()
+        gh = gh_cat[:, off:off + r]
+        want_h = m.scale * (gy.float() @ m.lora_b.float())
+        want_a = gh.float().T @ x.float()
+        want_b = m.scale * (gy.float().T @ h.float())
+        for got, want in ((gh, want_h), (ga, want_a), (gb, want_b)):
+            torch.testing.assert_close(got.float(), want, rtol=1e-2, atol=1e-2 * float(want.abs().max()) + 1e-30)
+        gh1, ga1, gb1 = ops.lora_bwd(gy, x, h, m.lora_b, m.scale)
+        assert torch.equal(gh, gh1), "hidden gradient"
+        for got, want in ((ga, ga1), (gb, gb1)):
+            torch.testing.assert_close(got.float(), want.float(), rtol=1e-2, atol=1e-2 * float(want.float().abs().max()) + 1e-30)
+        off += r
+
+
 def _layers(K, Ns, ranks, alpha, bias, seed):
     layers = []
     g = torch.Generator().manual_seed(seed)

@@ -11,7 +11,8 @@
 // contiguous bytes).  The last two contract over rows: bf16 MFMA as well, with both operands transposed on the way
 // through LDS (ds_read_b64_tr_b16).  Both split the contraction over many workgroups to
 // put enough loads in flight and combine the fp32 partial sums in a second, fixed-order pass, so results
-// are deterministic.
+// are deterministic.  For wide layers of rank <= 16 the two products that read gy (gh and gB) come from one pass over
+// it (skinny_tn_gh_kernel).
 #include "common.h"
 #include "group.h"
 #include "nf4_math.h"
@@ -437,6 +438,228 @@ __global__ __launch_bounds__(256) void skinny_tn_kernel(const TnBatch a) {
 #endif
 }
 
+// ---------------------------------------------------------------------------------------------------
+// skinny_tn_gh: both products of a backward that read gy, from one pass over it (rank <= 16):
+//   part  [split][r][c] = sum_{m in split} H[m][r] * GY[m][c]                   gB, as skinny_tn
+//   part_h[cg][m][r]    = sum_{c in column group cg} GY[m][c] * Bm[c][r]        gh, before scale and rounding
+// A workgroup owns 256 columns (two pieces of 128) and a range of rows; wave w takes the 32-row steps w, w + 4, ... as
+// in skinny_tn.  A piece that has been copied into the wave's LDS region for the transposed read-back is read back a
+// second time as it lies (16 bytes = 8 consecutive columns of one row: the row operand of an MFMA whose contraction runs
+// over columns) and multiplied with the matching 128 x R piece of Bm, which the wave holds in registers for the whole
+// launch (transposed once through LDS like the operand of skinny_nt<., true>).  The 32 x R sums of a step over the
+// workgroup's 256 columns go to part_h; a second pass (sum_partials_kernel) adds the column groups in a fixed order.
+// Against a pass of its own over gy for gh this costs Kc / 256 partial rows of R fp32 per row of gy, written and read
+// once: an eighth of gy's bytes at R = 16.
+// ---------------------------------------------------------------------------------------------------
+constexpr int kTnGhCols = 256;
+struct TnGhProblem {
+  const uint16_t* G;   // h: rows `ldg` elements apart; the problem's R columns start here
+  const uint16_t* X;   // gy [M, Kc]
+  const uint16_t* Bm;  // lora_b [Kc, R]
+  float* part;         // [splits, R, Kc]
+  float* part_h;       // [column groups, M, R]
+  int Kc, R, ldg;
+};
+struct TnGhBatch {
+  TnGhProblem p[kMaxGroup];
+  int cg_end[kMaxGroup];  // workgroups [cg_end[i - 1], cg_end[i]) along x work on problem i
+  int n, M, rows_per_split;
+};
+
+__global__ __launch_bounds__(256) void skinny_tn_gh_kernel(const TnGhBatch a) {
+  constexpr int kTrWaveLds = tn_wave_lds(1);
+#if defined(__HIP_DEVICE_COMPILE__)
+  int which = 0;  // uniform over the workgroup
+#pragma unroll
+  for (int q = 0; q < kMaxGroup - 1; ++q)
+    if (q < a.n - 1 && (int)blockIdx.x >= a.cg_end[q]) which = q + 1;
+  const TnGhProblem& P = a.p[which];
+  const uint16_t* __restrict__ G = P.G;
+  const uint16_t* __restrict__ X = P.X;
+  const uint16_t* __restrict__ Bm = P.Bm;
+  float* __restrict__ part = P.part;
+  float* __restrict__ part_h = P.part_h;
+  const int Kc = P.Kc, M = a.M, R = P.R, ldg = P.ldg, rows_per_split = a.rows_per_split;
+  const int col_group = (int)blockIdx.x - (which ? a.cg_end[which - 1] : 0);
+  __shared__ __attribute__((aligned(16))) char stage[4 * kTrWaveLds];
+  static_assert(sizeof(stage) >= 3 * 32 * 64 * sizeof(float), "the reduction reuses the staging memory");
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int g = lane >> 4, i = lane & 15;
+  const int c0 = col_group * kTnGhCols;
+  const int split = blockIdx.y;
+  const int m_begin = split * rows_per_split;
+  int m_end = m_begin + rows_per_split;
+  m_end = m_end < M ? m_end : M;
+
+  char* my = stage + wave * kTrWaveLds;
+  // copy-in and transposed read-back roles as in skinny_tn; piece p holds columns c0 + 128 p .. + 127
+  bool xcol_ok[2];
+  const uint16_t* xsrc[2];
+#pragma unroll
+  for (int p = 0; p < 2; ++p) {
+    const int xcol = c0 + 128 * p + 8 * i;
+    xcol_ok[p] = xcol < Kc;  // Kc % 8 == 0
+    xsrc[p] = X + (xcol_ok[p] ? xcol : 0);
+  }
+  char* xdst = my + g * kTrPitchX + 16 * i;
+  const int gcol = 8 * (lane & 1);  // R % 8 == 0: a lane's 8 columns are all in or all out
+  char* gdst = my + 32 * kTrPitchX + (lane >> 1) * 32 + 16 * (lane & 1);
+  const uint32_t my_lds = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)my);
+  const uint32_t xrd = my_lds + (8 * g + (i >> 2)) * kTrPitchX + 8 * (i & 3);
+  const uint32_t grd = my_lds + 32 * kTrPitchX + (8 * g + (i >> 2)) * 32 + 8 * (i & 3);
+  // the piece as it lies, for gh: row 16 t + i, the 8 columns 64 H + 16 g + 8 hh .. + 7 (16 bytes)
+  const char* prd = my + i * kTrPitchX + 32 * g;
+
+  // ---- the operand Bm[c0 + 128 p + 64 H + 16 g + 8 hh + (0 .. 7)][i] of every (p, H, hh): rows of Bm are R contiguous
+  //      elements, so a piece is 16 R chunks of 16 bytes; staged at 32 bytes a row (columns R .. 15 stay unwritten: they
+  //      only reach output columns that are never stored), rows beyond Kc as zeros
+  u32x4_t bfrag[2][2][2];
+  {
+    const int ppr = R >> 3;  // chunks per row
+    const uint32_t brd = my_lds + (16 * g + (i >> 2)) * 32 + 8 * (i & 3);
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int pc = lane + 64 * q;
+        if (pc < 16 * R) {
+          const int n = c0 + 128 * p + pc / ppr;
+          u32x4_t v = u32x4_t{0, 0, 0, 0};
+          if (n < Kc) v = *reinterpret_cast<const u32x4_t*>(Bm + (int64_t)n * R + 8 * (pc % ppr));
+          *reinterpret_cast<u32x4_t*>(my + (pc / ppr) * 32 + 16 * (pc % ppr)) = v;
+        }
+      }
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // LDS operations of a wave complete in order
+      u32x2_t lo[2][2], hi[2][2];
+#pragma unroll
+      for (int H = 0; H < 2; ++H)
+#pragma unroll
+        for (int hh = 0; hh < 2; ++hh) {
+          lo[H][hh] = lds_read_tr16(brd, (64 * H + 8 * hh) * 32);
+          hi[H][hh] = lds_read_tr16(brd, (64 * H + 8 * hh + 4) * 32);
+        }
+#pragma unroll
+      for (int H = 0; H < 2; ++H)
+#pragma unroll
+        for (int hh = 0; hh < 2; ++hh) {
+          asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(lo[H][hh]), "+v"(hi[H][hh]));
+          bfrag[p][H][hh] = u32x4_t{lo[H][hh].x, lo[H][hh].y, hi[H][hh].x, hi[H][hh].y};
+        }
+    }
+  }
+
+  f32x4_t acc[2][8];
+#pragma unroll
+  for (int p = 0; p < 2; ++p)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[p][e] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+  u32x4_t xv[2][8], gv;
+  auto fetch = [&](int m) {  // rows m .. m + 31 into registers
+#pragma unroll
+    for (int p = 0; p < 2; ++p)
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int row = m + 4 * u + g;
+        xv[p][u] = u32x4_t{0, 0, 0, 0};
+        if (row < m_end && xcol_ok[p]) xv[p][u] = *reinterpret_cast<const u32x4_t*>(xsrc[p] + (int64_t)row * Kc);
+      }
+    const int grow = m + (lane >> 1);
+    gv = u32x4_t{0, 0, 0, 0};
+    if (grow < m_end && gcol < R) gv = *reinterpret_cast<const u32x4_t*>(G + (int64_t)grow * ldg + gcol);
+  };
+  int m = m_begin + 32 * wave;
+  if (m < m_end) fetch(m);
+  for (; m < m_end; m += 128) {
+    f32x4_t acc_h[2] = {f32x4_t{0.f, 0.f, 0.f, 0.f}, f32x4_t{0.f, 0.f, 0.f, 0.f}};
+    u32x4_t gop;
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {
+      // every read of this region has been waited for before the MFMA that used it
+#pragma unroll
+      for (int u = 0; u < 8; ++u) *reinterpret_cast<u32x4_t*>(xdst + 4 * u * kTrPitchX) = xv[p][u];
+      if (p == 0) *reinterpret_cast<u32x4_t*>(gdst) = gv;  // zeros beyond R
+      if (p == 1 && m + 128 < m_end) fetch(m + 128);      // in flight while this step is multiplied
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the copy-in has landed
+      if (p == 0) {
+        u32x2_t ga = lds_read_tr16(grd, 0), gb = lds_read_tr16(grd, 4 * 32);
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(ga), "+v"(gb));
+        gop = u32x4_t{ga.x, ga.y, gb.x, gb.y};
+      }
+      u32x2_t xa[8], xb[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        xa[e] = lds_read_tr16(xrd, 32 * e);
+        xb[e] = lds_read_tr16(xrd, 32 * e + 4 * kTrPitchX);
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(xa[e]), "+v"(xb[e]) : "n"(14 - 2 * e));
+        const u32x4_t xop = {xa[e].x, xa[e].y, xb[e].x, xb[e].y};
+        acc[p][e] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, gop), __builtin_bit_cast(bf16x8_t, xop),
+                                                           acc[p][e], 0, 0, 0);
+      }
+      u32x4_t pr[2][2][2];
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int H = 0; H < 2; ++H)
+#pragma unroll
+          for (int hh = 0; hh < 2; ++hh)
+            pr[t][H][hh] = *reinterpret_cast<const u32x4_t*>(prd + 16 * t * kTrPitchX + 128 * H + 16 * hh);
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // before the region is written again
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int H = 0; H < 2; ++H)
+#pragma unroll
+          for (int hh = 0; hh < 2; ++hh)
+            acc_h[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, pr[t][H][hh]),
+                                                              __builtin_bit_cast(bf16x8_t, bfrag[p][H][hh]), acc_h[t], 0, 0, 0);
+    }
+    // acc_h[t][v] = sum over the workgroup's columns of GY[m + 16 t + 4 g + v][.] * Bm[.][i]
+    if (i < R) {
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          const int row = m + 16 * t + 4 * g + v;
+          if (row < m_end) part_h[((int64_t)col_group * M + row) * R + i] = acc_h[t][v];
+        }
+    }
+  }
+  float (*red)[32][64] = reinterpret_cast<float (*)[32][64]>(stage);
+  // acc[p][e][v] = sum over this wave's rows of H[.][4 g + v] * GY[.][c0 + 128 p + 16 e + i]; one piece at a time meets in
+  // the staging memory
+#pragma unroll
+  for (int p = 0; p < 2; ++p) {
+    __syncthreads();  // the staging regions (or the previous piece's sums) are free
+    if (wave > 0) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) red[wave - 1][v * 8 + e][lane] = acc[p][e][v];
+    }
+    __syncthreads();
+    if (wave == 0) {
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const int r = 4 * g + v;
+        if (r >= R) continue;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const int col = c0 + 128 * p + 16 * e + i;
+          if (col >= Kc) continue;
+          part[((int64_t)split * R + r) * Kc + col] =
+              ((acc[p][e][v] + red[0][v * 8 + e][lane]) + red[1][v * 8 + e][lane]) + red[2][v * 8 + e][lane];
+        }
+      }
+    }
+  }
+#endif
+}
+
 // out[r * stride_r + k * stride_k] = bf16(scale * sum_s part[s * split_stride + r * Kc + k]) for r < R, k < Kc
 struct TnSum {
   const float* part;
@@ -444,12 +667,13 @@ struct TnSum {
   int Kc, R;
   float scale;
   int64_t split_stride, stride_r, stride_k;
+  int splits;
 };
 constexpr int kTnMaxSums = 2 * kMaxGroup;
 struct TnSumBatch {
   TnSum p[kTnMaxSums];
   int64_t end[kTnMaxSums];  // threads [end[i - 1], end[i]) finish problem i
-  int n, splits;
+  int n;
 };
 // The reductions of every row contraction of a backward in one launch.
 __global__ __launch_bounds__(256) void sum_partials_tn_kernel(const TnSumBatch a) {
@@ -463,7 +687,7 @@ __global__ __launch_bounds__(256) void sum_partials_tn_kernel(const TnSumBatch a
   const TnSum& P = a.p[which];
   float s = 0.f;
 #pragma unroll 8
-  for (int q = 0; q < a.splits; ++q) s += P.part[(int64_t)q * P.split_stride + i];
+  for (int q = 0; q < P.splits; ++q) s += P.part[(int64_t)q * P.split_stride + i];
   const int64_t r = i / P.Kc, k = i % P.Kc;
   P.out[r * P.stride_r + k * P.stride_k] = f32_to_bf16_bits(s * P.scale);
 }
@@ -542,9 +766,11 @@ TnPlan plan_tn(int64_t M, int64_t col_groups) {
 }
 int64_t tn_col_groups(int64_t Kc) { return (Kc + kTnCols - 1) / kTnCols; }
 
-// The caller fills G, X, Kc, R, ldg of the n problems of `b` and the outputs of the ns sums of `f` (part, split_stride
-// and end are set here: sum i reads rows [sum_row0[i], + f.p[i].R) of problem sum_problem[i]).
-int run_tn_batch(TnBatch& b, int n, TnSumBatch& f, int ns, const int* sum_problem, const int* sum_row0, float* ws, hipStream_t s) {
+// The caller fills G, X, Kc, R, ldg of the n problems of `b` and the outputs of the ns sums of `f` (part, split_stride,
+// splits and end are set here: sum i reads rows [sum_row0[i], + f.p[i].R) of problem sum_problem[i]).  The ns_ready sums
+// that follow them in `f` are complete already (partial sums of an earlier launch) and ride along in the one reduction.
+int run_tn_batch(TnBatch& b, int n, TnSumBatch& f, int ns, const int* sum_problem, const int* sum_row0, float* ws, hipStream_t s,
+                 int ns_ready = 0) {
   int64_t groups = 0;
   for (int i = 0; i < n; ++i) {
     groups += tn_col_groups(b.p[i].Kc);
@@ -571,11 +797,15 @@ int run_tn_batch(TnBatch& b, int n, TnSumBatch& f, int ns, const int* sum_proble
     f.p[i].part = P.part + (int64_t)sum_row0[i] * P.Kc;
     f.p[i].Kc = P.Kc;
     f.p[i].split_stride = (int64_t)P.R * P.Kc;
+    f.p[i].splits = pl.splits;
     end += (int64_t)f.p[i].R * P.Kc;
     f.end[i] = end;
   }
-  f.n = ns;
-  f.splits = pl.splits;
+  for (int i = ns; i < ns + ns_ready; ++i) {
+    end += (int64_t)f.p[i].R * f.p[i].Kc;
+    f.end[i] = end;
+  }
+  f.n = ns + ns_ready;
   sum_partials_tn_kernel<<<dim3((unsigned)((end + 255) / 256)), dim3(256), 0, s>>>(f);
   return check_launch("skinny_tn");
 }
@@ -587,6 +817,31 @@ size_t tn_part_bytes(int64_t M, int n, const int64_t* Kc, const int* R) {
     elems += (int64_t)R[i] * Kc[i];
   }
   return (size_t)plan_tn(M, groups).splits * elems * sizeof(float);
+}
+
+// ---- gh and gB from one pass over gy (skinny_tn_gh_kernel) ------------------------------------------------------------
+// Taken when every member is wide and of rank <= 16: the pass over gy that gh alone would need then costs more than the
+// partial sums the fused kernel writes and the launch of their reduction (measured on [8192, 14336] pairs: 88 us for the
+// pass against ~30 us for the partial sums, the second reduction and the extra launch; at 4096 columns both are ~15 us).
+constexpr int64_t kTnGhMinCols = 8192, kTnGhMinRows = 1024;  // fewer rows: the launches themselves are what a backward costs
+bool tn_gh_applies(const GroupSkinny& g) {
+  for (int i = 0; i < g.n; ++i)
+    if (g.N[i] < kTnGhMinCols || g.rank[i] > 16) return false;
+  return g.n >= 1 && g.n <= kMaxGroup && g.M >= kTnGhMinRows;
+}
+int64_t tn_gh_col_groups(int64_t Kc) { return (Kc + kTnGhCols - 1) / kTnGhCols; }
+TnPlan plan_tn_gh(const GroupSkinny& g) {
+  int64_t groups = 0;
+  for (int i = 0; i < g.n; ++i) groups += tn_gh_col_groups(g.N[i]);
+  return plan_tn(g.M, groups);
+}
+// fp32 partial sums of the fused pass: per member the column groups' [M, R] and the row splits' [R, N]
+size_t tn_gh_part_bytes(const GroupSkinny& g) {
+  const TnPlan pl = plan_tn_gh(g);
+  size_t total = 0;
+  for (int i = 0; i < g.n; ++i)
+    total += align256(((size_t)tn_gh_col_groups(g.N[i]) * g.M + (size_t)pl.splits * g.N[i]) * g.rank[i] * sizeof(float));
+  return total;
 }
 
 // h = x . A^T for one layer
@@ -635,6 +890,11 @@ int run_group_hidden(const uint16_t* x, const GroupSkinny& g, uint16_t* h_cat, f
 }
 
 size_t group_lora_bwd_ws_bytes(const GroupSkinny& g) {
+  if (tn_gh_applies(g)) {
+    const int64_t width = g.K;
+    const int r_total = g.r_off[g.n];
+    return align256(tn_gh_part_bytes(g) + tn_part_bytes(g.M, 1, &width, &r_total));
+  }
   size_t nt = 0;
   int64_t widths[kTnMaxProblems];
   int ranks[kTnMaxProblems];
@@ -651,6 +911,51 @@ size_t group_lora_bwd_ws_bytes(const GroupSkinny& g) {
 
 int run_group_lora_bwd(const uint16_t* x, const uint16_t* h_cat, const GroupSkinny& g, uint16_t* gh_cat, float* ws, hipStream_t s) {
   const int rt = g.r_off[g.n];
+  if (tn_gh_applies(g)) {
+    // one pass over every gy for gB and gh, the column groups of gh summed, then gA over x; the reductions of gA and gB
+    // share the last launch
+    const TnPlan pl = plan_tn_gh(g);
+    TnGhBatch b = {};
+    NtBatch sums = {};
+    TnSumBatch f = {};
+    b.M = sums.M = (int)g.M;
+    b.n = g.n;
+    b.rows_per_split = pl.rows_per_split;
+    char* w = reinterpret_cast<char*>(ws);
+    int64_t groups = 0;
+    for (int i = 0; i < g.n; ++i) {
+      const int64_t cg = tn_gh_col_groups(g.N[i]);
+      TnGhProblem& P = b.p[i];
+      P.G = h_cat + g.r_off[i];
+      P.X = g.gy[i];
+      P.Bm = g.lora_b[i];
+      P.part_h = reinterpret_cast<float*>(w);
+      P.part = P.part_h + (size_t)cg * g.M * g.rank[i];
+      w += align256(((size_t)cg * g.M + (size_t)pl.splits * g.N[i]) * g.rank[i] * sizeof(float));
+      P.Kc = (int)g.N[i]; P.R = g.rank[i]; P.ldg = rt;
+      groups += cg;
+      b.cg_end[i] = (int)groups;
+      NtProblem& S = sums.p[i];  // gh_cat[:, member i] = bf16(scale . sum over column groups)
+      S.part = P.part_h;
+      S.out = gh_cat + g.r_off[i];
+      S.R = g.rank[i]; S.ldo = rt; S.splits = (int)cg;
+      S.scale = g.scale[i];
+      f.p[g.n + i] = TnSum{P.part, g.gb[i], (int)g.N[i], g.rank[i], g.scale[i], (int64_t)g.rank[i] * g.N[i], 1, g.rank[i], pl.splits};
+    }
+    skinny_tn_gh_kernel<<<dim3((unsigned)groups, (unsigned)pl.splits), dim3(256), 0, s>>>(b);
+    sum_partials_kernel<<<dim3((unsigned)((g.M * 16 + 255) / 256), (unsigned)g.n), dim3(256), 0, s>>>(sums);
+    if (int rc = check_launch("skinny_tn_gh")) return rc;
+    TnBatch t = {};
+    t.M = (int)g.M;
+    t.p[0] = TnProblem{gh_cat, x, nullptr, (int)g.K, rt, rt};
+    int sum_problem[kTnMaxSums], sum_row0[kTnMaxSums];
+    for (int i = 0; i < g.n; ++i) {
+      f.p[i] = TnSum{nullptr, g.ga[i], 0, g.rank[i], 1.0f, 0, g.K, 1};
+      sum_problem[i] = 0;
+      sum_row0[i] = g.r_off[i];
+    }
+    return run_tn_batch(t, 1, f, g.n, sum_problem, sum_row0, reinterpret_cast<float*>(w), s, g.n);
+  }
   {
     NtBatch b = {};
     b.M = (int)g.M;
@@ -752,12 +1057,27 @@ extern "C" int ttamd_lora_hidden_static_bf16(const void* x, const void* lora_a, 
                     reinterpret_cast<uint16_t*>(h), scratch, reinterpret_cast<hipStream_t>(stream));
 }
 
+namespace {
+// One layer as a group of one: the same launches, the same bits.
+GroupSkinny single_layer(int64_t M, int64_t N, int64_t K, int rank, float scale, const void* gy, const void* lora_b, void* ga, void* gb) {
+  GroupSkinny g = {};
+  g.n = 1;
+  g.M = M; g.K = K;
+  g.N[0] = N;
+  g.rank[0] = rank;
+  g.r_off[1] = rank;
+  g.scale[0] = scale;
+  g.lora_b[0] = reinterpret_cast<const uint16_t*>(lora_b);
+  g.gy[0] = reinterpret_cast<const uint16_t*>(gy);
+  g.ga[0] = reinterpret_cast<uint16_t*>(ga);
+  g.gb[0] = reinterpret_cast<uint16_t*>(gb);
+  return g;
+}
+}  // namespace
+
 extern "C" size_t ttamd_lora_bwd_workspace_bytes(int64_t M, int64_t N, int64_t K, int rank) {
   if (M <= 0 || N <= 0 || K <= 0 || rank <= 0 || K % 64 || N % 64) return 0;
-  const int64_t widths[2] = {K, N};
-  const int ranks[2] = {rank, rank};
-  const size_t a = nt_part_bytes(M, N, rank), b = tn_part_bytes(M, 2, widths, ranks);
-  return align256(a > b ? a : b);
+  return group_lora_bwd_ws_bytes(single_layer(M, N, K, rank, 1.0f, nullptr, nullptr, nullptr, nullptr));
 }
 
 extern "C" int ttamd_lora_bwd_bf16(const void* gy, const void* x, const void* h, const void* lora_b, float scale, void* gh,
@@ -770,31 +1090,9 @@ extern "C" int ttamd_lora_bwd_bf16(const void* gy, const void* x, const void* h,
   if (workspace_bytes < ttamd_lora_bwd_workspace_bytes(M, N, K, rank))
     return fail(TTAMD_EWORKSPACE, "lora_bwd: workspace has %zu bytes, needs %zu", workspace_bytes,
                 ttamd_lora_bwd_workspace_bytes(M, N, K, rank));
-  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  float* ws = reinterpret_cast<float*>(workspace);
-  const uint16_t* GY = reinterpret_cast<const uint16_t*>(gy);
-  {
-    // gh = scale * gy . B, lora_b [N, R] as it lies (the kernel transposes its pieces)
-    NtBatch b = {};
-    b.M = (int)M;
-    NtProblem& P = b.p[0];
-    P.X = GY;
-    P.bm[0] = reinterpret_cast<const uint16_t*>(lora_b);
-    P.r_off[1] = rank;
-    P.nb = 1;
-    P.out = reinterpret_cast<uint16_t*>(gh);
-    P.Kc = (int)N; P.R = rank; P.ldo = rank;
-    P.scale = scale;
-    if (int rc = run_nt_batch(b, 1, true, ws, s)) return rc;
-  }
-  // gA[r][k] = sum_m gh[m][r] x[m][k]  and  gB[n][r] = scale * sum_m h[m][r] gy[m][n]
-  TnBatch t = {};
-  t.M = (int)M;
-  t.p[0] = TnProblem{reinterpret_cast<const uint16_t*>(gh), reinterpret_cast<const uint16_t*>(x), nullptr, (int)K, rank, rank};
-  t.p[1] = TnProblem{reinterpret_cast<const uint16_t*>(h), GY, nullptr, (int)N, rank, rank};
-  TnSumBatch f = {};
-  f.p[0] = TnSum{nullptr, reinterpret_cast<uint16_t*>(ga), 0, rank, 1.0f, 0, K, 1};
-  f.p[1] = TnSum{nullptr, reinterpret_cast<uint16_t*>(gb), 0, rank, scale, 0, 1, rank};
-  const int sum_problem[2] = {0, 1}, sum_row0[2] = {0, 0};
-  return run_tn_batch(t, 2, f, 2, sum_problem, sum_row0, ws, s);
+  // gh = scale . gy . B (lora_b [N, R] as it lies: the kernels transpose its pieces), gA[r][k] = sum_m gh[m][r] x[m][k],
+  // gB[n][r] = scale . sum_m h[m][r] gy[m][n]
+  return run_group_lora_bwd(reinterpret_cast<const uint16_t*>(x), reinterpret_cast<const uint16_t*>(h),
+                            single_layer(M, N, K, rank, scale, gy, lora_b, ga, gb), reinterpret_cast<uint16_t*>(gh),
+                            reinterpret_cast<float*>(workspace), reinterpret_cast<hipStream_t>(stream));
 }
