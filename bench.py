@@ -529,6 +529,8 @@ def main() -> int:
     ap.add_argument("--swiglu-bwd-epilogue", action="store_true",
                     help="A/B: the backward of silu(gate) * up from the epilogue of the down projection's grad-input GEMM launch "
                          "instead of a pass of its own (QLoRA workloads)")
+    ap.add_argument("--no-qat-tn-group", action="store_true",
+                    help="A/B (QAT workloads): one weight-gradient launch per member of a group instead of one for the group")
     ap.add_argument("--no-group", action="store_true",
                     help="one call per projection, as the reference's modules make them, instead of the group kernels for the "
                          "projections that share an input (q/k/v, gate/up): for A/B timing")
@@ -564,6 +566,9 @@ def main() -> int:
     if args.no_qat_tiled_gemm:
         from torchtune_amd import qat as qat_module
         qat_module.TILED_GEMM = False
+    if args.no_qat_tn_group:
+        from torchtune_amd import qat as qat_module
+        qat_module.TN_GROUP_GEMM = False
     if args.no_backward_copy:
         from torchtune_amd import nf4_tensor
         nf4_tensor.BACKWARD_COPY = False

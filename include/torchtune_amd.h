@@ -483,6 +483,15 @@ size_t ttamd_tiled_weight_bytes(int64_t N, int64_t K);
  */
 int ttamd_gemm_tn_applies(int64_t M, int64_t N, int64_t K);
 int ttamd_gemm_tn_bf16(const void* a, const void* b, void* c, int64_t M, int64_t N, int64_t K, void* stream);
+/*
+ * The weight gradients of layers with a common input (q / k / v of torchtune/modules/attention.py:234,262-263, gate / up
+ * of torchtune/modules/feed_forward.py:50-53) as one launch: c[i][N[i], K] = a[i][M, N[i]]^T . b[M, K] for up to
+ * TTAMD_GROUP_MAX members, each result bit-equal to ttamd_gemm_tn_bf16 of that member (same tiles, same order of sums).
+ * The members' row tiles share the launch's rounds of 256 tiles, so a narrow member (a 1024-wide k / v projection: 64
+ * tiles) no longer needs a launch that leaves three quarters of the chip idle.  Every N[i] and K multiples of 256, M of 32.
+ */
+int ttamd_gemm_tn_group_bf16(const void* const* a, const void* b, void* const* c, int n_members, int64_t M, const int64_t* N,
+                             int64_t K, void* stream);
 int ttamd_fq_per_group_int4_sym_tiled_bf16(const void* w, int64_t N, int64_t K, int group_size, int qparam_dtype, float eps,
                                            void* tiled_fwd, void* tiled_bwd, float* scale, void* stream);
 int ttamd_tiled_linear_bf16(const void* x, const void* tiled_weight, const void* bias, void* y, int64_t M, int64_t n_out,

@@ -73,6 +73,35 @@ def test_full_size_weight_gradients_of_the_8b_qat_configuration(M, N, K):
         torch.testing.assert_close(c[n0:n0 + 16384].float(), want, rtol=1e-2, atol=1e-2 * scale)
 
 
+@pytest.mark.parametrize("M,K,Ns", [
+    (64, 256, (256, 256)),
+    (1024, 512, (512, 256, 256, 768)),
+    (8192, 4096, (4096, 1024, 1024)),        # q / k / v of the 8B shape at batch 2 x 4096: 384 tiles, one launch
+    (8192, 4096, (14336, 14336)),            # gate / up: seven full rounds instead of two launches of three and a half
+], ids=["small", "four_members", "qkv_8b", "gate_up_8b"])
+def test_group_launch_equals_member_launches_bitwise(M, K, Ns):
+    """``ttamd_gemm_tn_group_bf16`` against one ``ttamd_gemm_tn_bf16`` per member: the same tiles and the same order of
+    sums, so the same bits; the member launches are themselves compared with fp32 products above."""
+    g = torch.Generator().manual_seed(M + K + len(Ns))
+    b = torch.randn(M, K, generator=g).to(BF).to(DEV)
+    a_list = [torch.randn(M, N, generator=g).to(BF).to(DEV) for N in Ns]
+    cs = ops.gemm_tn_group(a_list, b)
+    assert [tuple(c.shape) for c in cs] == [(N, K) for N in Ns]
+    for a, c in zip(a_list, cs):
+        assert torch.equal(c.view(torch.int16), ops.gemm_tn(a, b).view(torch.int16))
+
+
+def test_group_launch_refuses_bad_members():
+    b = torch.zeros(64, 256, dtype=BF, device=DEV)
+    ok = torch.zeros(64, 256, dtype=BF, device=DEV)
+    with pytest.raises(Exception):
+        ops.gemm_tn_group([ok, torch.zeros(64, 320, dtype=BF, device=DEV)], b)     # width not a multiple of 256
+    with pytest.raises(ValueError):
+        ops.gemm_tn_group([ok, torch.zeros(32, 256, dtype=BF, device=DEV)], b)     # rows differ
+    with pytest.raises(ValueError):
+        ops.gemm_tn_group([ok] * (_lib.GROUP_MAX + 1), b)
+
+
 def test_unsupported_shapes_are_refused():
     lib = _lib.load()
     assert not ops.gemm_tn_applies(100, 256, 256) and not ops.gemm_tn_applies(64, 320, 256) and not ops.gemm_tn_applies(64, 256, 64)

@@ -13,6 +13,7 @@
 #include <type_traits>
 
 #include "common.h"
+#include "group.h"
 #include "nf4_math.h"
 
 namespace ttamd {
@@ -33,12 +34,16 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
 
 #define TT_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
 
+// One launch serves the weight gradients of up to kGroupMax layers with a common input (q / k / v, gate / up): they share
+// B and differ in A and C; row tiles [tile_end[i - 1], tile_end[i]) of the stacked outputs belong to member i.
 struct TnArgs {
-  const uint16_t* A;  // [M, N] bf16
+  const uint16_t* A[kGroupMax];  // [M, N[i]] bf16
+  uint16_t* C[kGroupMax];        // [N[i], K] bf16
+  int N[kGroupMax], tile_end[kGroupMax];
+  int n;
   const uint16_t* B;  // [M, K] bf16
-  uint16_t* C;        // [N, K] bf16
-  int M, N, K;
-  int tiles_n, tiles_k;
+  int M, K;
+  int tiles_n, tiles_k;  // tiles_n: all members
 };
 
 constexpr int kTnStage = 32768;  // 32 rows x 512 bytes of A, then the same of B
@@ -68,7 +73,14 @@ __global__ __launch_bounds__(512) void gemm_tn_kernel(const TnArgs g) {
       tile_k = id % g.tiles_k;
     }
   }
-  const int n0 = tile_n * 256, k0 = tile_k * 256;
+  int which = 0;  // uniform over the workgroup
+#pragma unroll
+  for (int q = 0; q < kGroupMax - 1; ++q)
+    if (q < g.n - 1 && tile_n >= g.tile_end[q]) which = q + 1;
+  const uint16_t* const A = g.A[which];
+  uint16_t* const C = g.C[which];
+  const int N = g.N[which];
+  const int n0 = (tile_n - (which ? g.tile_end[which - 1] : 0)) * 256, k0 = tile_k * 256;  // n0: within the member
   const int nk = g.M >> 5;  // steps of 32 rows
 
   // ---- loads: per step and wave two instructions for A (rows 4 wv .. + 3 of the 32, two rows of 512 bytes each) and two
@@ -78,7 +90,7 @@ __global__ __launch_bounds__(512) void gemm_tn_kernel(const TnArgs g) {
   for (int d = 0; d < 2; ++d) {
     const int rl = 4 * wv + 2 * d + (lane >> 5);
     const int chunk = (lane & 31) ^ ((rl & 3) << 1);
-    a_off[d] = (uint32_t)rl * (uint32_t)g.N * 2u + (uint32_t)n0 * 2u + (uint32_t)chunk * 16u;
+    a_off[d] = (uint32_t)rl * (uint32_t)N * 2u + (uint32_t)n0 * 2u + (uint32_t)chunk * 16u;
     b_off[d] = (uint32_t)rl * (uint32_t)g.K * 2u + (uint32_t)k0 * 2u + (uint32_t)chunk * 16u;
   }
   auto dma16 = [&](uint32_t voff, const char* base, uint32_t lds, int imm) {
@@ -88,7 +100,7 @@ __global__ __launch_bounds__(512) void gemm_tn_kernel(const TnArgs g) {
   const uint32_t lds0 = (uint32_t)(uintptr_t)TT_LDS_PTR(smem);
   auto issue = [&](int t) {
     const int tk = t < nk ? t : nk - 1;
-    const char* ab = reinterpret_cast<const char*>(g.A) + (int64_t)tk * 32 * g.N * 2;
+    const char* ab = reinterpret_cast<const char*>(A) + (int64_t)tk * 32 * N * 2;
     const char* bb = reinterpret_cast<const char*>(g.B) + (int64_t)tk * 32 * g.K * 2;
     const uint32_t st = lds0 + (t & 3) * kTnStage + wv * 2048;
     dma16(a_off[0], ab, st, 0);
@@ -211,7 +223,7 @@ __global__ __launch_bounds__(512) void gemm_tn_kernel(const TnArgs g) {
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     const int c = lane & 7;
-    uint16_t* crow = g.C + k0 + wn * 64 + 8 * c;
+    uint16_t* crow = C + k0 + wn * 64 + 8 * c;
     const int nrow0 = n0 + 128 * wm;
 #pragma unroll 8
     for (int t = 0; t < 16; ++t) {
@@ -237,19 +249,8 @@ using namespace ttamd;
 
 extern "C" int ttamd_gemm_tn_applies(int64_t M, int64_t N, int64_t K) { return gemm_tn_applies(M, N, K) ? 1 : 0; }
 
-extern "C" int ttamd_gemm_tn_bf16(const void* a, const void* b, void* c, int64_t M, int64_t N, int64_t K, void* stream) {
-  TT_REQUIRE(a && b && c && aligned16(a) && aligned16(b) && aligned16(c), "gemm_tn: pointers must be non-null and 16-byte aligned");
-  TT_REQUIRE(M > 0 && N > 0 && K > 0, "gemm_tn: bad shape M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
-  if (!gemm_tn_applies(M, N, K))
-    return fail(TTAMD_EUNSUPPORTED, "gemm_tn: M (%lld) must be a multiple of 32, N (%lld) and K (%lld) multiples of 256", (long long)M,
-                (long long)N, (long long)K);
-  TnArgs g;
-  g.A = reinterpret_cast<const uint16_t*>(a);
-  g.B = reinterpret_cast<const uint16_t*>(b);
-  g.C = reinterpret_cast<uint16_t*>(c);
-  g.M = (int)M; g.N = (int)N; g.K = (int)K;
-  g.tiles_n = (int)(N / 256);
-  g.tiles_k = (int)(K / 256);
+namespace {
+int launch_gemm_tn(TnArgs& g, hipStream_t s) {
   // the LDS limit is a per-device attribute of the function: set it for the current device once (a race only repeats the call)
   static bool attr_set[64] = {};
   int dev = 0;
@@ -259,6 +260,52 @@ extern "C" int ttamd_gemm_tn_bf16(const void* a, const void* b, void* c, int64_t
     if (e != hipSuccess) return fail(TTAMD_ELAUNCH, "gemm_tn: cannot reserve %d bytes of LDS: %s", kTnLds, hipGetErrorString(e));
     if (dev >= 0) attr_set[dev] = true;
   }
-  gemm_tn_kernel<<<dim3((unsigned)(g.tiles_n * g.tiles_k)), dim3(512), kTnLds, reinterpret_cast<hipStream_t>(stream)>>>(g);
+  gemm_tn_kernel<<<dim3((unsigned)(g.tiles_n * g.tiles_k)), dim3(512), kTnLds, s>>>(g);
   return check_launch("gemm_tn");
+}
+}  // namespace
+
+extern "C" int ttamd_gemm_tn_bf16(const void* a, const void* b, void* c, int64_t M, int64_t N, int64_t K, void* stream) {
+  TT_REQUIRE(a && b && c && aligned16(a) && aligned16(b) && aligned16(c), "gemm_tn: pointers must be non-null and 16-byte aligned");
+  TT_REQUIRE(M > 0 && N > 0 && K > 0, "gemm_tn: bad shape M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
+  if (!gemm_tn_applies(M, N, K))
+    return fail(TTAMD_EUNSUPPORTED, "gemm_tn: M (%lld) must be a multiple of 32, N (%lld) and K (%lld) multiples of 256", (long long)M,
+                (long long)N, (long long)K);
+  TnArgs g = {};
+  g.n = 1;
+  g.A[0] = reinterpret_cast<const uint16_t*>(a);
+  g.C[0] = reinterpret_cast<uint16_t*>(c);
+  g.N[0] = (int)N;
+  g.B = reinterpret_cast<const uint16_t*>(b);
+  g.M = (int)M; g.K = (int)K;
+  g.tiles_n = g.tile_end[0] = (int)(N / 256);
+  g.tiles_k = (int)(K / 256);
+  return launch_gemm_tn(g, reinterpret_cast<hipStream_t>(stream));
+}
+
+extern "C" int ttamd_gemm_tn_group_bf16(const void* const* a, const void* b, void* const* c, int n_members, int64_t M,
+                                        const int64_t* N, int64_t K, void* stream) {
+  TT_REQUIRE(a && b && c && N && aligned16(b), "gemm_tn_group: null or misaligned pointer argument");
+  TT_REQUIRE(n_members >= 1 && n_members <= kGroupMax, "gemm_tn_group: %d members (1 .. %d)", n_members, kGroupMax);
+  TT_REQUIRE(M > 0 && K > 0, "gemm_tn_group: bad shape M=%lld K=%lld", (long long)M, (long long)K);
+  TnArgs g = {};
+  g.n = n_members;
+  int64_t tiles = 0;
+  for (int i = 0; i < n_members; ++i) {
+    TT_REQUIRE(a[i] && c[i] && aligned16(a[i]) && aligned16(c[i]), "gemm_tn_group: member %d: pointers must be non-null and 16-byte aligned", i);
+    if (N[i] <= 0 || !gemm_tn_applies(M, N[i], K))
+      return fail(TTAMD_EUNSUPPORTED, "gemm_tn_group: M (%lld) must be a multiple of 32, N[%d] (%lld) and K (%lld) multiples of 256",
+                  (long long)M, i, (long long)N[i], (long long)K);
+    g.A[i] = reinterpret_cast<const uint16_t*>(a[i]);
+    g.C[i] = reinterpret_cast<uint16_t*>(c[i]);
+    g.N[i] = (int)N[i];
+    tiles += N[i] / 256;
+    g.tile_end[i] = (int)tiles;
+  }
+  if (tiles * (K / 256) >= (int64_t(1) << 31)) return fail(TTAMD_EUNSUPPORTED, "gemm_tn_group: too many tiles for one launch");
+  g.B = reinterpret_cast<const uint16_t*>(b);
+  g.M = (int)M; g.K = (int)K;
+  g.tiles_n = (int)tiles;
+  g.tiles_k = (int)(K / 256);
+  return launch_gemm_tn(g, reinterpret_cast<hipStream_t>(stream));
 }

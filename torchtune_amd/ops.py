@@ -6,7 +6,7 @@ Every function requires HIP (``cuda``) tensors.  There is no CPU implementation 
 from __future__ import annotations
 
 import ctypes
-from typing import Optional, Sequence, Tuple
+from typing import List, Optional, Sequence, Tuple
 
 import torch
 
@@ -809,6 +809,34 @@ def gemm_tn(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
             events[1].record()
     _lib.check(rc, "gemm_tn")
     return c
+
+
+def gemm_tn_group(a_list: Sequence[torch.Tensor], b: torch.Tensor) -> List[torch.Tensor]:
+    """``[a.T @ b for a in a_list]`` (each ``a`` [M, N_i], ``b`` [M, K], bf16) as one launch: the weight gradients of layers
+    with a common input.  Each result carries the bits ``gemm_tn(a, b)`` gives."""
+    b = _bf16_2d(b, "gemm_tn_group")
+    a_list = [_bf16_2d(a, "gemm_tn_group") for a in a_list]
+    M, K = b.shape
+    n = len(a_list)
+    if not 1 <= n <= _lib.GROUP_MAX:
+        raise ValueError(f"gemm_tn_group: {n} members (1 .. {_lib.GROUP_MAX})")
+    for a in a_list:
+        if a.shape[0] != M or a.device != b.device:
+            raise ValueError(f"gemm_tn_group: a {tuple(a.shape)} on {a.device} does not go with b {tuple(b.shape)} on {b.device}")
+    cs = [torch.empty(a.shape[1], K, dtype=torch.bfloat16, device=b.device) for a in a_list]
+    a_ptrs = (ctypes.c_void_p * n)(*[a.data_ptr() for a in a_list])
+    c_ptrs = (ctypes.c_void_p * n)(*[c.data_ptr() for c in cs])
+    widths = (ctypes.c_int64 * n)(*[a.shape[1] for a in a_list])
+    lib = _lib.load()
+    with torch.cuda.device(b.device):
+        events = _gemm_timer("tn", M, sum(a.shape[1] for a in a_list), K, 0) if _gemm_timer is not None else None
+        if events:
+            events[0].record()
+        rc = lib.ttamd_gemm_tn_group_bf16(a_ptrs, b.data_ptr(), c_ptrs, n, M, widths, K, _stream(b))
+        if events:
+            events[1].record()
+    _lib.check(rc, "gemm_tn_group")
+    return cs
 
 
 def quantize_per_group_int4(w: torch.Tensor, group_size: int, qparam_dtype: torch.dtype = torch.float32,

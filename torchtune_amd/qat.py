@@ -249,6 +249,8 @@ TILED_GEMM = True
 TILED_GEMM_MIN_ROWS = 2048
 TILED_GEMM_MIN_TILES = 256
 TN_GEMM_MIN_TILES = 192
+# the weight gradients of a group's members (they share fq(x)) as one launch; False: one launch per member (A/B timing)
+TN_GROUP_GEMM = True
 
 
 class _TiledFakeQuantLinearFn(torch.autograd.Function):
@@ -330,11 +332,21 @@ class _TiledFakeQuantGroupFn(torch.autograd.Function):
         gy2 = [torch.zeros(x2.shape[0], N, dtype=x2.dtype, device=x2.device) if g is None else g.reshape(-1, N)
                for g, (N, _) in zip(gys, ctx.shapes)]
         out = [ops.tiled_linear_group_dx(gy2, tb, K).view(ctx.x_shape) if ctx.needs_input_grad[0] else None, None, None]
+        # the members' weight gradients share fq(x): one launch over their stacked rows when every member wants one (a
+        # narrow member then fills the rounds of the wide ones instead of a launch of its own on the vendor library)
+        M = x2.shape[0]
+        need_ws = [ctx.needs_input_grad[3 + 2 * i] for i in range(len(ctx.shapes))]
+        gws = None
+        if (TN_GROUP_GEMM and len(ctx.shapes) > 1 and all(need_ws) and all(ops.gemm_tn_applies(M, N, K) for N, _ in ctx.shapes)
+                and sum(N // 256 for N, _ in ctx.shapes) * (K // 256) >= TN_GEMM_MIN_TILES):
+            gws = ops.gemm_tn_group(gy2, x2)
         for i, (N, _) in enumerate(ctx.shapes):
             need_w, need_b = ctx.needs_input_grad[3 + 2 * i:5 + 2 * i]
             gw = None
-            if need_w:
-                own = ops.gemm_tn_applies(gy2[i].shape[0], N, K) and (N // 256) * (K // 256) >= TN_GEMM_MIN_TILES
+            if gws is not None:
+                gw = gws[i]
+            elif need_w:
+                own = ops.gemm_tn_applies(M, N, K) and (N // 256) * (K // 256) >= TN_GEMM_MIN_TILES
                 gw = ops.gemm_tn(gy2[i], x2) if own else gy2[i].t().matmul(x2)
             out += [gw, gy2[i].sum(dim=0) if (ctx.has_bias[i] and need_b) else None]
         return tuple(out)
