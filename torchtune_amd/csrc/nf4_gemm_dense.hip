@@ -313,8 +313,8 @@ constexpr int kLdsDense = kWBase + 4 * kWStage;
 // is the gradient of silu(gate) * up and is not stored; each 16-byte piece of it meets the same piece of gate and up
 // on its way out and the launch writes the gradients of gate and up instead, the arithmetic of ttamd_swiglu_bwd_bf16 on
 // the rounded result, bit for bit.
-template <bool LW_ROW_MAJOR, int EPI = kEpiPlain>
-__global__ __launch_bounds__(512) void nf4_gemm_dense_kernel(const DenseArgs g) {
+template <bool LW_ROW_MAJOR, int EPI>
+__device__ __forceinline__ void gemm_dense_tile(const DenseArgs g) {
 #if defined(__HIP_DEVICE_COMPILE__)
   constexpr bool GATED = EPI == kEpiGated;
   constexpr int MT = 8, NT = 4;  // 16 x 16 MFMA tiles per wave
@@ -680,6 +680,13 @@ __global__ __launch_bounds__(512) void nf4_gemm_dense_kernel(const DenseArgs g) 
 #endif
 }
 
+template <bool LW_ROW_MAJOR, bool GATED = false>
+__global__ __launch_bounds__(512) void nf4_gemm_dense_kernel(const DenseArgs g) {
+  gemm_dense_tile<LW_ROW_MAJOR, GATED ? kEpiGated : kEpiPlain>(g);
+}
+// grad-input launch (adapter weights [r, K]) whose result goes on through the backward of silu(gate) * up
+__global__ __launch_bounds__(512) void nf4_gemm_dense_swiglu_bwd_kernel(const DenseArgs g) { gemm_dense_tile<false, kEpiSwigluBwd>(g); }
+
 int launch_expand(int mode, const uint8_t* codes, const float* scal, int64_t Nout, int64_t Kc, int64_t nk_total, int64_t t_off,
                   char* tiled, hipStream_t s, bool paired = false) {
   // one block of 16 columns per blockIdx.x; the contraction is cut along blockIdx.y so that about 2048 workgroups exist
@@ -714,9 +721,8 @@ int launch_dense(DenseArgs& g, hipStream_t s) {
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = -1;
   if (dev < 0 || !attr_set[dev]) {
     for (const void* fn : {reinterpret_cast<const void*>(&nf4_gemm_dense_kernel<true>), reinterpret_cast<const void*>(&nf4_gemm_dense_kernel<false>),
-                           reinterpret_cast<const void*>(&nf4_gemm_dense_kernel<true, kEpiGated>),
-                           reinterpret_cast<const void*>(&nf4_gemm_dense_kernel<true, kEpiSwigluBwd>),
-                           reinterpret_cast<const void*>(&nf4_gemm_dense_kernel<false, kEpiSwigluBwd>)}) {
+                           reinterpret_cast<const void*>(&nf4_gemm_dense_kernel<true, true>),
+                           reinterpret_cast<const void*>(&nf4_gemm_dense_swiglu_bwd_kernel)}) {
       hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsDense);
       if (e != hipSuccess) return fail(TTAMD_ELAUNCH, "nf4_gemm_dense: cannot reserve %d bytes of LDS: %s", kLdsDense, hipGetErrorString(e));
     }
@@ -727,15 +733,12 @@ int launch_dense(DenseArgs& g, hipStream_t s) {
     TT_REQUIRE(g.lw_row_major && g.nout == 2 && (g.nad == 2 || g.nad == 0) && g.nseg == 1 && g.out[0].width == g.out[1].width &&
                    g.out[0].width % 128 == 0 && g.Nout == 2 * g.out[0].width,
                "nf4_gemm_dense: the gated launch takes two members of equal width, a multiple of 128");
-    nf4_gemm_dense_kernel<true, kEpiGated><<<grid, block, kLdsDense, s>>>(g);
+    nf4_gemm_dense_kernel<true, true><<<grid, block, kLdsDense, s>>>(g);
   } else if (g.sw_gup) {
-    TT_REQUIRE(g.nout == 1 && g.out[0].n_begin == 0 && g.out[0].width == g.Nout && !g.out[0].bias && !g.out[0].cscale &&
-                   g.sw_gate && g.sw_up && g.out[0].C,
-               "nf4_gemm_dense: the SwiGLU-backward launch takes one output without bias or column scale");
-    if (g.lw_row_major)
-      nf4_gemm_dense_kernel<true, kEpiSwigluBwd><<<grid, block, kLdsDense, s>>>(g);
-    else
-      nf4_gemm_dense_kernel<false, kEpiSwigluBwd><<<grid, block, kLdsDense, s>>>(g);
+    TT_REQUIRE(!g.lw_row_major && g.nout == 1 && g.out[0].n_begin == 0 && g.out[0].width == g.Nout && !g.out[0].bias &&
+                   !g.out[0].cscale && g.sw_gate && g.sw_up && g.out[0].C,
+               "nf4_gemm_dense: the SwiGLU-backward launch is a grad-input launch with one output, no bias or column scale");
+    nf4_gemm_dense_swiglu_bwd_kernel<<<grid, block, kLdsDense, s>>>(g);
   } else if (g.lw_row_major)
     nf4_gemm_dense_kernel<true><<<grid, block, kLdsDense, s>>>(g);
   else
