@@ -20,7 +20,7 @@ DEV = "cuda"
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
-@pytest.mark.parametrize("rows,K", [(1, 8), (5, 24), (64, 4096), (7, 14336), (3, 28672), (4, 40000), (130, 512)])
+@pytest.mark.parametrize("rows,K", [(1, 8), (5, 24), (64, 4096), (9, 4104), (5, 8192), (7, 14336), (3, 28672), (6, 32768), (4, 40000), (130, 512)])
 def test_per_token_bit_exact(dtype, rows, K):
     g = torch.Generator().manual_seed(rows * 1000 + K)
     x = (torch.randn(rows, K, generator=g) * 1.7).to(dtype)

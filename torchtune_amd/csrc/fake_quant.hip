@@ -152,6 +152,62 @@ __global__ __launch_bounds__(256) void fq_per_token_regs_kernel(const void* __re
   }
 }
 
+// One workgroup (four waves) per token row, NV chunks of 8 elements per lane: rows of more than 4096 elements.  A wave
+// that held such a row alone would need most of the register file (one wave per SIMD: nothing else runs while it
+// computes between its loads and its stores); a quarter of the row per wave leaves room for eight.  The extrema of
+// the four waves meet in LDS (min and max do not depend on the order).
+template <bool BF16, int NV>
+__global__ __launch_bounds__(256) void fq_per_token_wg_kernel(const void* __restrict__ x, int64_t rows, int64_t K,
+                                                              void* __restrict__ out, float* __restrict__ scale_out,
+                                                              int32_t* __restrict__ zp_out, bool qp_bf16, float eps) {
+  __shared__ float ext[2][4];
+  const int64_t row = blockIdx.x;
+  const int tid = threadIdx.x;
+  const int chunks_per_row = (int)(K >> 3);
+  const int64_t row_chunk0 = row * chunks_per_row;
+  Chunk8<BF16> c[NV];
+  float mn = 0.f, mx = 0.f;  // the qparams use min(amin, 0) and max(amax, 0): zero is the neutral start
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int ch = i * 256 + tid;
+    if (ch < chunks_per_row)
+      c[i].load(x, row_chunk0 + ch);
+    else
+      c[i].zero();
+  }
+#pragma unroll
+  for (int i = 0; i < NV; ++i)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float v = c[i].get(e);
+      mn = fminf(mn, v);
+      mx = fmaxf(mx, v);
+    }
+  wave_minmax(mn, mx);
+  if ((tid & 63) == 0) {
+    ext[0][tid >> 6] = mn;
+    ext[1][tid >> 6] = mx;
+  }
+  __syncthreads();
+  mn = fminf(fminf(ext[0][0], ext[0][1]), fminf(ext[0][2], ext[0][3]));
+  mx = fmaxf(fmaxf(ext[1][0], ext[1][1]), fmaxf(ext[1][2], ext[1][3]));
+  const TokenQParams p = token_qparams(mn, mx, qp_bf16, eps);
+  if (tid == 0) {
+    if (scale_out) scale_out[row] = p.scale;
+    if (zp_out) zp_out[row] = (int32_t)p.zp;
+  }
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int ch = i * 256 + tid;
+    if (ch < chunks_per_row) {
+      float v[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = token_fq<BF16>(c[i].get(e), p);
+      Chunk8<BF16>::store(out, row_chunk0 + ch, v);
+    }
+  }
+}
+
 // Rows too long for the register file: two passes over the row (the second one normally hits in L2).
 template <bool BF16>
 __global__ __launch_bounds__(256) void fq_per_token_stream_kernel(const void* __restrict__ x, int64_t rows, int64_t K,
@@ -266,8 +322,8 @@ template <bool BF16>
 int launch_per_token(const void* x, int64_t rows, int64_t K, void* out, float* scale, int32_t* zp, bool qp_bf16, float eps,
                      hipStream_t s) {
   const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
-  const int64_t nv = (K / 8 + kWave - 1) / kWave;
-  constexpr int kMaxRegChunks = BF16 ? 32 : 16;
+  const int64_t nv = (K / 8 + kWave - 1) / kWave;     // chunks per lane with a wave per row
+  const int64_t nvw = (K / 8 + 255) / 256;            // with a workgroup per row
 #define TT_LAUNCH_TOKEN(NV)                                                                          \
   if (nv <= NV) {                                                                                    \
     fq_per_token_regs_kernel<BF16, NV><<<grid, block, 0, s>>>(x, rows, K, out, scale, zp, qp_bf16, eps);  \
@@ -277,11 +333,17 @@ int launch_per_token(const void* x, int64_t rows, int64_t K, void* out, float* s
   TT_LAUNCH_TOKEN(2)
   TT_LAUNCH_TOKEN(4)
   TT_LAUNCH_TOKEN(8)
-  TT_LAUNCH_TOKEN(16)
-  if constexpr (kMaxRegChunks >= 32) {
-    TT_LAUNCH_TOKEN(32)
-  }
 #undef TT_LAUNCH_TOKEN
+  // more than 4096 elements a row (up to 32768): a workgroup per row
+#define TT_LAUNCH_TOKEN_WG(NV)                                                                                         \
+  if (nvw <= NV && rows < (int64_t(1) << 31)) {                                                                        \
+    fq_per_token_wg_kernel<BF16, NV><<<dim3((unsigned)rows), block, 0, s>>>(x, rows, K, out, scale, zp, qp_bf16, eps); \
+    return check_launch("fq_per_token_int8_asym");                                                                     \
+  }
+  TT_LAUNCH_TOKEN_WG(4)
+  TT_LAUNCH_TOKEN_WG(8)
+  TT_LAUNCH_TOKEN_WG(16)
+#undef TT_LAUNCH_TOKEN_WG
   fq_per_token_stream_kernel<BF16><<<grid, block, 0, s>>>(x, rows, K, out, scale, zp, qp_bf16, eps);
   return check_launch("fq_per_token_int8_asym");
 }
