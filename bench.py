@@ -674,7 +674,7 @@ def main() -> int:
             },
             "roofline": {
                 "bound": "hbm",
-                "kernel": "fq_per_token_regs_kernel + fq_int4_sym_tiled_kernel / fq_per_group_kernel (the fake-quant launches of "
+                "kernel": "fq_per_token_regs_kernel / fq_per_token_wg_kernel + fq_int4_sym_tiled_kernel / fq_per_group_kernel (the fake-quant launches of "
                           "the step; the matmuls: see own_gemm)",
                 "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBPS,
