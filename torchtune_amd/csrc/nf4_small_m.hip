@@ -125,9 +125,10 @@ __device__ __forceinline__ float nf4_code_value(int k) {
   return v;
 }
 
-// MT 16-token tiles of x, RT 16-row tiles of W per workgroup, U chunks of K in flight per wave.
-template <int MT, int RT, int U>
-__global__ __launch_bounds__(64 * kSmMaxWaves) void nf4_small_m_kernel(const SmallMGroup grp) {
+// MT 16-token tiles of x, RT 16-row tiles of W per workgroup, U chunks of K in flight per wave, at most MAXW waves (the
+// register budget of a lane follows from it: the four-wave shapes hold more tiles per lane).
+template <int MT, int RT, int U, int MAXW>
+__global__ __launch_bounds__(64 * MAXW) void nf4_small_m_kernel(const SmallMGroup grp) {
   int which = 0;  // uniform over the workgroup
 #pragma unroll
   for (int q = 0; q < kGroupMax - 1; ++q)
@@ -269,12 +270,13 @@ SmallMConfig small_m_config(int64_t M, int64_t N, int64_t K) {
   return wide ? SmallMConfig{4, 2, 2, 4} : SmallMConfig{4, 1, 4, deep ? 16 : 4};
 }
 
-template <int MT, int RT, int U>
-int launch_small_m(SmallMGroup& g, int max_waves, hipStream_t s) {
+template <int MT, int RT, int U, int MAXW>
+int launch_small_m(SmallMGroup& g, hipStream_t s) {
+  static_assert(MAXW <= kSmMaxWaves, "the partial sums are laid out for at most kSmMaxWaves waves");
   const int K = g.m[0].K;
   int nw = ((K >> 7) + U - 1) / U;  // one group of U chunks per wave when K is short enough
   nw = nw > 1 ? nw : 1;
-  nw = nw < max_waves ? nw : max_waves;
+  nw = nw < MAXW ? nw : MAXW;
   // the partial sums of waves 1 .. nw - 1 must fit the 64 KB of LDS a workgroup gets without asking for more
   const int per_wave = MT * RT * 4 * 64 * (int)sizeof(float);
   const int fit = 1 + (63 * 1024) / per_wave;
@@ -285,14 +287,15 @@ int launch_small_m(SmallMGroup& g, int max_waves, hipStream_t s) {
     g.wg_end[i] = wgs;
   }
   const dim3 grid((unsigned)wgs), block(64 * nw);
-  nf4_small_m_kernel<MT, RT, U><<<grid, block, (size_t)(nw - 1) * per_wave, s>>>(g);
+  nf4_small_m_kernel<MT, RT, U, MAXW><<<grid, block, (size_t)(nw - 1) * per_wave, s>>>(g);
   return check_launch("nf4_small_m");
 }
 
 int dispatch_small_m(SmallMGroup& g, const SmallMConfig& c, hipStream_t s) {
-  if (c.mt == 1) return launch_small_m<1, 1, 4>(g, c.max_waves, s);
-  if (c.mt == 2) return c.rt == 2 ? launch_small_m<2, 2, 4>(g, c.max_waves, s) : launch_small_m<2, 1, 4>(g, c.max_waves, s);
-  return c.rt == 2 ? launch_small_m<4, 2, 2>(g, c.max_waves, s) : launch_small_m<4, 1, 4>(g, c.max_waves, s);
+  if (c.mt == 1) return launch_small_m<1, 1, 4, 16>(g, s);
+  if (c.mt == 2) return c.rt == 2 ? launch_small_m<2, 2, 4, 4>(g, s) : launch_small_m<2, 1, 4, 4>(g, s);
+  if (c.rt == 2) return launch_small_m<4, 2, 2, 4>(g, s);
+  return c.max_waves > 4 ? launch_small_m<4, 1, 4, 16>(g, s) : launch_small_m<4, 1, 4, 4>(g, s);
 }
 
 }  // namespace
