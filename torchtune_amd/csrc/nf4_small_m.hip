@@ -135,7 +135,9 @@ __global__ __launch_bounds__(64 * MAXW) void nf4_small_m_kernel(const SmallMGrou
     if (q < grp.n - 1 && (int)blockIdx.x >= grp.wg_end[q]) which = q + 1;
   const SmallMArgs& a = grp.m[which];
   const int wg = (int)blockIdx.x - (which ? grp.wg_end[which - 1] : 0);
-  constexpr int NACC = MT * RT == 1 ? 4 : (MT * RT == 2 ? 2 : 1);  // independent MFMA chains per lane: at least four
+  // independent MFMA chains per lane: at least four; one token tile always sums in four chains, whatever the row tiles,
+  // so that a row of up to 16 tokens gets the same bits alone and in a batch
+  constexpr int NACC = MT == 1 ? 4 : (MT * RT == 2 ? 2 : 1);
   __shared__ float2 lut[256];
   extern __shared__ float red[];  // [waves - 1][MT * RT * 4][64]
   const int t = threadIdx.x, lane = t & 63;
@@ -262,10 +264,13 @@ struct SmallMConfig {
 // Measured on MI355X over the projections of an 8B model (kernel time, M = 1 / 8 / 32 / 64): 4096 x 4096
 // 7 / 7 / 13 / 20 us, 14336 x 4096 15 / 17 / 26 / 43 us, 4096 x 14336 14 / 18 / 37 / 64 us.  Wide layers share an x
 // fragment between two row tiles once x is more than one token tile (x comes from L2 once per workgroup); long
-// contractions get sixteen waves, short ones four.
+// contractions get sixteen waves, short ones four.  From 9 tokens on the wide layers take two row tiles per workgroup as
+// well: every workgroup reads all of x (16 tokens x 4096: 128 KB, 3.5 times the packed weight bytes over the 896
+// workgroups of a 14336-wide layer), and twice the rows per workgroup halve that (M = 16: 1.33 -> 1.65 TB/s of packed weight).
 SmallMConfig small_m_config(int64_t M, int64_t N, int64_t K) {
   const bool wide = N >= 8192, deep = K >= 8192;
-  if (M <= 16) return {1, 1, 4, 16};
+  if (M <= 8) return {1, 1, 4, 16};
+  if (M <= 16) return wide ? SmallMConfig{1, 2, 4, 16} : SmallMConfig{1, 1, 4, 16};
   if (M <= 32) return wide ? SmallMConfig{2, 2, 4, 4} : SmallMConfig{2, 1, 4, 4};
   return wide ? SmallMConfig{4, 2, 2, 4} : SmallMConfig{4, 1, 4, deep ? 16 : 4};
 }
@@ -292,7 +297,7 @@ int launch_small_m(SmallMGroup& g, hipStream_t s) {
 }
 
 int dispatch_small_m(SmallMGroup& g, const SmallMConfig& c, hipStream_t s) {
-  if (c.mt == 1) return launch_small_m<1, 1, 4, 16>(g, s);
+  if (c.mt == 1) return c.rt == 2 ? launch_small_m<1, 2, 4, 16>(g, s) : launch_small_m<1, 1, 4, 16>(g, s);
   if (c.mt == 2) return c.rt == 2 ? launch_small_m<2, 2, 4, 4>(g, s) : launch_small_m<2, 1, 4, 4>(g, s);
   if (c.rt == 2) return launch_small_m<4, 2, 2, 4>(g, s);
   return c.max_waves > 4 ? launch_small_m<4, 1, 4, 16>(g, s) : launch_small_m<4, 1, 4, 4>(g, s);
