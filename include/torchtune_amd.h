@@ -160,7 +160,9 @@ int ttamd_lora_hidden_static_bf16(const void* x, const void* lora_a, void* h, in
  * D(W) is bit-identical to ttamd_nf4_dequantize's output; all products are accumulated in fp32 and the sum is
  * rounded to bf16 once (the eager reference rounds after each of its five ops).
  * M <= 64 (decode, evaluation) runs a kernel that streams the packed weight once instead of the tiled one; same
- * operands, same expansion of the weight, fp32 sums in a different but fixed order.
+ * operands, same expansion of the weight, fp32 sums in a different but fixed order.  (Through the _ws entry point below,
+ * with the workspace its query asks for, that kernel serves M <= 16, and M <= 32 on weights of at most 2^25 elements;
+ * above that every one of its workgroups reads more of x than of the weight and the sliced tiled kernel is faster.)
  */
 int ttamd_nf4_lora_linear_fwd_bf16(const void* x, const uint8_t* quantized_data, const void* block_scalers,
                                    const void* block_scalers_t, const void* h, const void* lora_b, int rank, float scale,
@@ -218,8 +220,8 @@ int ttamd_nf4_linear_bwd_dx_bf16(const void* gy, const uint8_t* quantized_data, 
                                  const void* lora_a, int rank, void* gx, int64_t M, int64_t N, int64_t K, void* stream);
 
 /*
- * The same two GEMMs for token counts between the few-token kernel and a full grid (64 < M, at most 128 output tiles
- * of 128 x 256): with a workspace the contraction is cut into up to 16 slices, one workgroup per tile per slice, fp32
+ * The same two GEMMs for token counts between the few-token kernel and a full grid (17 - 64 tokens where the slices beat
+ * the few-token kernel, see above, and 64 < M; at most 128 output tiles of 128 x 256): with a workspace the contraction is cut into up to 16 slices, one workgroup per tile per slice, fp32
  * partial tiles in the workspace, and a second kernel adds the slices in a fixed order, then bias, column scale and
  * the rounding to bf16.  The plain entry points above are these with workspace = NULL (no slicing: a launch of few
  * tiles then leaves most of the chip idle).  The reference has no counterpart: it dequantises the weight and calls a
@@ -293,7 +295,8 @@ int ttamd_lora_bwd_bf16(const void* gy, const void* x, const void* h, const void
  *
  *   forward   h_cat[:, member i] = x . lora_a_i^T for all members in one pass over x (h_cat [M, sum of ranks] bf16,
  *             member i in columns [sum of the ranks before it, + rank_i); the caller keeps it for the backward);
- *             y_i = x . D(W_i)^T (+ bias_i) + scale_i . h_i . lora_b_i^T: for M <= 64 one launch for all members that
+ *             y_i = x . D(W_i)^T (+ bias_i) + scale_i . h_i . lora_b_i^T: where the few-token kernel serves the member
+ *             with the largest weight (the rule of ttamd_nf4_lora_linear_fwd_ws_bf16) one launch for all members that
  *             get the same launch shape, otherwise one launch per member.  h_cat and every y_i are bit-identical to
  *             ttamd_lora_hidden_bf16 + ttamd_nf4_lora_linear_fwd_bf16 on the member alone.
  *   backward  gh_cat[:, member i] = scale_i . gy_i . lora_b_i (one launch, bit-identical to ttamd_lora_bwd_bf16's gh);

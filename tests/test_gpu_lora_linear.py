@@ -510,7 +510,8 @@ def test_few_output_tiles_slice_the_contraction(M, N, K):
     h = ops.lora_hidden(x, A)
     nbytes = lib.ttamd_nf4_gemm_workspace_bytes(M, N, K)
     assert nbytes > 0 and nbytes % (M * N * 4) == 0 and 2 <= nbytes // (M * N * 4) <= 16
-    assert lib.ttamd_nf4_gemm_workspace_bytes(64, N, K) == 0  # the few-token kernel needs none
+    assert lib.ttamd_nf4_gemm_workspace_bytes(16, N, K) == 0  # the few-token kernel needs none
+    assert lib.ttamd_nf4_gemm_workspace_bytes(64, N, K) > 0   # from 33 tokens on the slices serve better than it
     assert lib.ttamd_nf4_gemm_workspace_bytes(16384, 4096, 4096) == 2 * 4096 * 4096  # a full grid of many tokens: the expanded weight, no slices
     ref = ((x.float() @ D.T + bias.float() + 0.5 * (h.float() @ B.float().T)) * cs.float())
     for scal_t in (None, bst):
@@ -609,6 +610,39 @@ def test_few_token_and_sliced_kernels_at_8b_shapes():
                 y_row = ops.nf4_lora_linear_fwd(x[:1].contiguous(), t.quantized_data, bs, N, h[:1].contiguous(), B, 2.0,
                                                 block_scalers_t=bst)
                 assert torch.equal(y_row[0], y[0])
+
+
+@pytest.mark.parametrize("N,K", [(1024, 4096), (4096, 4096), (14336, 4096), (4096, 14336)])
+def test_seventeen_to_sixty_four_tokens_with_and_without_a_workspace(N, K):
+    """Between 17 and 64 tokens the forward entry point runs the few-token kernel when no workspace comes with the call
+    and, given one, the sliced tiled kernel where that is faster (from 17 tokens on weights of more than 2^25 elements,
+    from 33 tokens on all): both against the fp32 product on the dequantised weight, against each other to a bf16
+    rounding step, and the workspace query says which one a caller with a workspace gets."""
+    from torchtune_amd import _lib
+
+    lib = _lib.load()
+    g = torch.Generator(device=DEV).manual_seed(N + K)
+    t = to_nf4((torch.randn(N, K, device=DEV, generator=g) * 0.02).to(BF))
+    D = t.get_original_weight().float()
+    bs = t.block_scalers()
+    B = (torch.randn(N, 16, device=DEV, generator=g) * 0.05).to(BF)
+    for M in (17, 24, 32, 33, 48, 64):
+        sliced = M > 32 or N * K > (1 << 25)
+        assert (lib.ttamd_nf4_gemm_workspace_bytes(M, N, K) > 0) == sliced
+        x = torch.randn(M, K, device=DEV, generator=g).to(BF)
+        h = torch.randn(M, 16, device=DEV, generator=g).to(BF)
+        ref = x.float() @ D.T + (2.0 * h.float()).to(BF).float() @ B.float().T
+        y = ops.nf4_lora_linear_fwd(x, t.quantized_data, bs, N, h, B, 2.0)          # brings the workspace the query asks for
+        torch.testing.assert_close(y.float(), ref, rtol=1e-2, atol=1e-2, msg=f"M{M}")
+        assert torch.equal(y, ops.nf4_lora_linear_fwd(x, t.quantized_data, bs, N, h, B, 2.0))
+        y0 = torch.empty_like(y)
+        assert lib.ttamd_nf4_lora_linear_fwd_ws_bf16(x.data_ptr(), t.quantized_data.data_ptr(), bs.data_ptr(), None, h.data_ptr(),
+                                                     B.data_ptr(), 16, 2.0, None, None, y0.data_ptr(), M, N, K, None, 0, None) == 0
+        torch.cuda.synchronize()
+        torch.testing.assert_close(y0.float(), ref, rtol=1e-2, atol=1e-2, msg=f"M{M} without a workspace")
+        torch.testing.assert_close(y.float(), y0.float(), rtol=1e-2, atol=1e-2)
+        if not sliced:
+            assert torch.equal(y, y0)   # the few-token kernel either way
 
 
 def test_entry_points_are_reentrant_across_threads_and_streams():

@@ -80,6 +80,8 @@ int run_gemm_dense_group_dx(const GroupDx& d, const void* gh_cat, void* gx, void
 
 // nf4_small_m.hip: y[i] = x . D(W_i)^T (+ bias) + scale . h_i . lora_b[i]^T for a handful of tokens
 int small_m_limit();
+// the forward of M tokens on an [N, K] weight runs the few-token kernel (sliced_ok: a slicing workspace is at hand)
+bool small_m_applies(int64_t M, int64_t N, int64_t K, bool sliced_ok);
 int run_small_m_group(const void* x, const GroupGemm& g, const void* h_cat, hipStream_t s);
 
 // lora_skinny.hip

@@ -64,9 +64,17 @@ int decode(const char* who, const ttamd_lora_group_member* m, int n, int64_t M, 
 }
 
 // slices of the largest sliced member GEMM, or the expanded weight(s) of the many-token path
+// the few-token launch serves the group when it would serve the member with the largest weight
+bool group_small_m(const Decoded& d, bool sliced_ok) {
+  int64_t n_max = 0;
+  for (int i = 0; i < d.gm.n; ++i) n_max = d.gm.N[i] > n_max ? d.gm.N[i] : n_max;
+  return small_m_applies(d.gm.M, n_max, d.gm.K, sliced_ok);
+}
+
 size_t fwd_gemm_ws(const Decoded& d) {
-  size_t w = d.gm.M > small_m_limit() ? dense_group_fwd_workspace_bytes(d.gm) : 0;
-  if (d.gm.M > small_m_limit())
+  const bool tiled = !group_small_m(d, true);
+  size_t w = tiled ? dense_group_fwd_workspace_bytes(d.gm) : 0;
+  if (tiled)
     for (int i = 0; i < d.gm.n; ++i) {
       const size_t b = gemm_rs_workspace_bytes(d.gm.M, d.gm.N[i], d.gm.K);
       w = b > w ? b : w;
@@ -115,10 +123,10 @@ int group_fwd(const char* who, const void* x, const ttamd_lora_group_member* mem
   if (int rc = decode(who, members, n_members, M, K, false, d)) return rc;
   TT_REQUIRE(x && h_cat && aligned16(x) && aligned16(h_cat), "%s: x and h_cat must be non-null and 16-byte aligned", who);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  if (M <= small_m_limit()) return run_small_m_group(x, d.gm, h_cat, s);
   // slices of the contraction for a member with few output tiles, when the caller brought the memory for them
   const size_t gem = align256(fwd_gemm_ws(d));
   const bool sliced = gem > 0 && workspace != nullptr && workspace_bytes >= gem;
+  if (group_small_m(d, sliced)) return run_small_m_group(x, d.gm, h_cat, s);
   TT_REQUIRE(!sliced || aligned16(workspace), "%s: workspace must be 16-byte aligned", who);
   // many tokens: one launch over the members' concatenated output columns, every weight expanded once
   if (sliced && dense_group_fwd_workspace_bytes(d.gm) > 0) {

@@ -448,7 +448,8 @@ int lora_linear_fwd(const char* who, const void* x, const uint8_t* quantized_dat
   TT_REQUIRE((bias == nullptr || (reinterpret_cast<uintptr_t>(bias) & 7u) == 0) &&
                  (col_scale == nullptr || (reinterpret_cast<uintptr_t>(col_scale) & 7u) == 0),
              "%s: bias / col_scale must be 8-byte aligned", who);
-  if (M <= small_m_limit())  // a handful of tokens: stream the packed weight once (nf4_small_m.hip)
+  // a handful of tokens: stream the packed weight once (nf4_small_m.hip)
+  if (small_m_applies(M, N, K, workspace != nullptr && workspace_bytes > 0 && workspace_bytes >= gemm_rs_workspace_bytes(M, N, K)))
     return run_small_m(x, quantized_data, block_scalers, h, rank, lora_b, rank, scale, bias, col_scale, y, M, N, K,
                        reinterpret_cast<hipStream_t>(stream));
   if (block_scalers_t) {
@@ -470,7 +471,7 @@ extern "C" int ttamd_nf4_lora_linear_fwd_bf16(const void* x, const uint8_t* quan
 }
 
 extern "C" size_t ttamd_nf4_gemm_workspace_bytes(int64_t M, int64_t n_out, int64_t k_contract) {
-  if (M <= small_m_limit() || M <= 0 || n_out <= 0 || k_contract <= 0) return 0;
+  if (M <= 0 || n_out <= 0 || k_contract <= 0 || small_m_applies(M, n_out, k_contract, true)) return 0;
   return gemm_rs_workspace_bytes(M, n_out, k_contract);
 }
 

@@ -308,6 +308,18 @@ int dispatch_small_m(SmallMGroup& g, const SmallMConfig& c, hipStream_t s) {
 // Largest token count the small-M kernel takes; above it the tiled kernel runs.
 int small_m_limit() { return 64; }
 
+// Whether a forward of M tokens on an [N, K] weight goes to this kernel.  sliced_ok: the caller brought the workspace
+// that lets the tiled kernel cut its contraction into slices.  Without it the tiled kernel fills 16 - 56 workgroups at
+// these sizes and this kernel wins up to 64 tokens.  With it (measured, us, few-token / sliced at 24, 32, 40, 64 tokens):
+// 4096 x 4096 13 / 17, 14 / 18, 20 / 19, 25 / 22; 14336 x 4096 29 / 23, 31 / 24, 40 / 25, 50 / 27; 4096 x 14336 33 / 24,
+// 37 / 25, 50 / 26, 66 / 28: every workgroup of this kernel reads all of x, which at 64 tokens is seven times the
+// packed weight, so from 17 tokens on the large weights and from 33 on all of them are better off in slices.
+bool small_m_applies(int64_t M, int64_t N, int64_t K, bool sliced_ok) {
+  if (M > small_m_limit()) return false;
+  if (M <= 16 || !sliced_ok) return true;
+  return M <= 32 && N * K <= (int64_t(1) << 25);
+}
+
 // Entries used by the C-ABI wrappers (arguments already validated there: N % 64 == 0, K % 64 == 0, R % 8 == 0, pointers
 // aligned).  `bscal` is the natural [N, K/64] scaler layout; the rows of `h` are ldh elements apart.
 int run_small_m(const void* x, const uint8_t* codes, const void* bscal, const void* h, int ldh, const void* lora_b, int R,
