@@ -418,8 +418,8 @@ def test_disable_adapter_and_adapter_state_dict():
 
 def test_gemm_workspace_query_is_a_host_function():
     """``ttamd_nf4_gemm_workspace_bytes`` needs no GPU: it is 0 where the launch uses no scratch memory (the few-token
-    kernel, M <= 64; launches with more than 128 tiles of 128 x 256 but fewer than 256 of 256 x 256 or fewer than 2048
-    tokens; two-slice launches of a short contraction), slices * M * n_out * 4 bytes with 2 <= slices <= 16 and at least
+    kernel: M <= 16, and M <= 32 on weights of at most 2^25 elements; launches with more than 128 tiles of 128 x 256 but
+    fewer than 256 of 256 x 256 or fewer than 2048 tokens; two-slice launches of a short contraction), slices * M * n_out * 4 bytes with 2 <= slices <= 16 and at least
     four 64-wide k-steps per slice where the contraction is sliced, and 2 * n_out * k bytes (the weight expanded once)
     from 2048 tokens and 256 tiles of 256 x 256 up, which ``ttamd_nf4_gemm_expands_weight`` tells apart."""
     from torchtune_amd import _lib
@@ -427,7 +427,9 @@ def test_gemm_workspace_query_is_a_host_function():
     lib = _lib.load()
     q = lib.ttamd_nf4_gemm_workspace_bytes
     e = lib.ttamd_nf4_gemm_expands_weight
-    assert q(1, 4096, 4096) == 0 and q(64, 4096, 4096) == 0
+    assert q(1, 4096, 4096) == 0 and q(16, 14336, 4096) == 0 and q(32, 4096, 4096) == 0
+    assert q(33, 4096, 4096) == 16 * 33 * 4096 * 4 and q(64, 4096, 4096) == 16 * 64 * 4096 * 4   # slices from 33 tokens
+    assert q(17, 14336, 4096) > 0 and q(17, 4096, 14336) > 0                                     # large weights: from 17
     assert q(8192, 4096, 4096) == 2 * 4096 * 4096 and e(8192, 4096, 4096) == 1
     assert q(16384, 1024, 4096) == 2 * 1024 * 4096 and e(16384, 1024, 4096) == 1
     assert q(8192, 14336, 4096) == q(8192, 4096, 14336) == 2 * 4096 * 14336
