@@ -35,10 +35,11 @@ __device__ __forceinline__ float wave_sum(float v) {
 }
 
 // ---------------------------------------------------------------------------------------------------
-// RMSNorm.  One wave per row, the row held in registers (NV 16-byte chunks per lane, chunk = lane + 64 i).
+// RMSNorm.  One wave per row, the row held in registers (NV 16-byte chunks per lane, chunk = lane + 64 i); the
+// backward with a scale gradient takes a workgroup per row (see rms_norm_bwd_gscale_kernel).
 //   forward : xn = bf16(x * rsqrt(mean(x^2) + eps));  y = bf16(xn * scale);  rstd saved for backward
 //   backward: g = bf16(gy * scale) (eager's bf16 product), c = mean(g * x) * rstd^2,
-//             gx = bf16(rstd * (g - x * c));  gscale partial[w][d] = sum over the wave's rows of gy * xn
+//             gx = bf16(rstd * (g - x * c));  gscale partial[w][d] = sum over workgroup w's rows of gy * xn
 // ---------------------------------------------------------------------------------------------------
 template <int NV>
 __global__ __launch_bounds__(256) void rms_norm_fwd_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ scale,
@@ -83,56 +84,80 @@ __global__ __launch_bounds__(256) void rms_norm_fwd_kernel(const uint16_t* __res
   }
 }
 
+// Backward: a workgroup per row (four waves, NV chunks of 8 columns per lane, chunk = thread + 256 i).  Without a scale
+// gradient the grid has one workgroup per row.  With it (GSCALE) a fixed number of workgroups walk the rows with a
+// stride of the grid, and a lane keeps the partial scale gradient of its own columns over all the rows its workgroup
+// sees (8 NV floats); held by one wave per row, those sums took 64 registers beside the row itself and left two waves
+// per SIMD with nothing in flight while they computed (3.4 TB/s at 4096 columns).  The row's dot product meets in LDS in
+// wave order - the same order in both forms, so the input gradient does not depend on whether the scale is trained; the
+// slot alternates with the row, so one barrier per row is enough.  Workgroup w writes row w of the partial sums (zeros
+// if it saw no row).
 template <int NV, bool GSCALE>
 __global__ __launch_bounds__(256) void rms_norm_bwd_kernel(const uint16_t* __restrict__ gy, const uint16_t* __restrict__ x,
                                                            const uint16_t* __restrict__ scale, const float* __restrict__ rstd_in,
                                                            uint16_t* __restrict__ gx, float* __restrict__ gscale_part,
                                                            int64_t rows, int D) {
-  const int lane = threadIdx.x & 63;
-  const int wave_global = blockIdx.x * 4 + (threadIdx.x >> 6);
-  const int n_waves = gridDim.x * 4;
+  __shared__ float dots[2][4];
+  const int t = threadIdx.x, wave = t >> 6;
   const int chunks = D >> 3;
   const u32x4_t* sr = reinterpret_cast<const u32x4_t*>(scale);
   float gs[GSCALE ? NV : 1][8];
-  if constexpr (GSCALE) {
+  u32x4_t sv[NV];
 #pragma unroll
-    for (int i = 0; i < NV; ++i)
+  for (int i = 0; i < NV; ++i) {
+    if constexpr (GSCALE) {
 #pragma unroll
       for (int e = 0; e < 8; ++e) gs[i][e] = 0.f;
+    }
+    const int c = t + 256 * i;
+    sv[i] = c < chunks ? sr[c] : u32x4_t{0, 0, 0, 0};
   }
-  for (int64_t row = wave_global; row < rows; row += n_waves) {
+  // the next row of the workgroup is asked for before this one is worked on
+  u32x4_t xv[NV], gov[NV], xn[NV], gon[NV];
+  auto fetch = [&](int64_t row, u32x4_t (&xd)[NV], u32x4_t (&gd)[NV]) {
     const u32x4_t* xr = reinterpret_cast<const u32x4_t*>(x + row * D);
     const u32x4_t* gr = reinterpret_cast<const u32x4_t*>(gy + row * D);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int c = t + 256 * i;
+      xd[i] = u32x4_t{0, 0, 0, 0};
+      gd[i] = u32x4_t{0, 0, 0, 0};
+      if (c < chunks) {
+        xd[i] = __builtin_nontemporal_load(xr + c);
+        gd[i] = __builtin_nontemporal_load(gr + c);
+      }
+    }
+  };
+  int par = 0;
+  if ((int64_t)blockIdx.x < rows) fetch(blockIdx.x, xv, gov);
+  for (int64_t row = blockIdx.x; row < rows; row += gridDim.x, par ^= 1) {
     const float rstd = rstd_in[row];
-    u32x4_t xv[NV], gv[NV];
+    if (GSCALE && row + gridDim.x < rows) fetch(row + gridDim.x, xn, gon);
+    u32x4_t gv[NV];
     float dot = 0.f;
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
-      const int c = lane + 64 * i;
-      xv[i] = u32x4_t{0, 0, 0, 0};
-      gv[i] = u32x4_t{0, 0, 0, 0};
-      if (c < chunks) {
-        xv[i] = *(xr + c);
-        const u32x4_t go = *(gr + c);
-        const u32x4_t s = sr[c];
+      // chunks beyond the row are zeros: they add nothing to the dot product and are never stored
 #pragma unroll
-        for (int d = 0; d < 4; ++d) {
-          if constexpr (GSCALE) {
-            gs[i][2 * d] += lo_f(go[d]) * round_to_bf16(lo_f(xv[i][d]) * rstd);
-            gs[i][2 * d + 1] += hi_f(go[d]) * round_to_bf16(hi_f(xv[i][d]) * rstd);
-          }
-          gv[i][d] = pack2(lo_f(go[d]) * lo_f(s[d]), hi_f(go[d]) * hi_f(s[d]));  // g = bf16(gy * scale)
-          dot += lo_f(gv[i][d]) * lo_f(xv[i][d]);
-          dot += hi_f(gv[i][d]) * hi_f(xv[i][d]);
+      for (int d = 0; d < 4; ++d) {
+        if constexpr (GSCALE) {
+          gs[i][2 * d] += lo_f(gov[i][d]) * round_to_bf16(lo_f(xv[i][d]) * rstd);
+          gs[i][2 * d + 1] += hi_f(gov[i][d]) * round_to_bf16(hi_f(xv[i][d]) * rstd);
         }
+        gv[i][d] = pack2(lo_f(gov[i][d]) * lo_f(sv[i][d]), hi_f(gov[i][d]) * hi_f(sv[i][d]));  // g = bf16(gy * scale)
+        dot += lo_f(gv[i][d]) * lo_f(xv[i][d]);
+        dot += hi_f(gv[i][d]) * hi_f(xv[i][d]);
       }
     }
     dot = wave_sum(dot);
+    if ((t & 63) == 0) dots[par][wave] = dot;
+    __syncthreads();
+    dot = ((dots[par][0] + dots[par][1]) + dots[par][2]) + dots[par][3];
     const float c2 = dot / (float)D * rstd * rstd;
     u32x4_t* outr = reinterpret_cast<u32x4_t*>(gx + row * D);
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
-      const int c = lane + 64 * i;
+      const int c = t + 256 * i;
       if (c >= chunks) continue;
       u32x4_t o;
 #pragma unroll
@@ -140,16 +165,22 @@ __global__ __launch_bounds__(256) void rms_norm_bwd_kernel(const uint16_t* __res
         o[d] = pack2(rstd * (lo_f(gv[i][d]) - lo_f(xv[i][d]) * c2), rstd * (hi_f(gv[i][d]) - hi_f(xv[i][d]) * c2));
       __builtin_nontemporal_store(o, outr + c);
     }
-  }
-  if constexpr (GSCALE) {
+    if constexpr (GSCALE) {
 #pragma unroll
-    for (int i = 0; i < NV; ++i) {
-      const int c = lane + 64 * i;
-      if (c >= chunks) continue;
-      float* p = gscale_part + (int64_t)wave_global * D + 8 * c;
-      *reinterpret_cast<f32x4_t*>(p) = f32x4_t{gs[i][0], gs[i][1], gs[i][2], gs[i][3]};
-      *reinterpret_cast<f32x4_t*>(p + 4) = f32x4_t{gs[i][4], gs[i][5], gs[i][6], gs[i][7]};
+      for (int i = 0; i < NV; ++i) {
+        xv[i] = xn[i];
+        gov[i] = gon[i];
+      }
     }
+  }
+  if constexpr (!GSCALE) return;
+#pragma unroll
+  for (int i = 0; i < (GSCALE ? NV : 0); ++i) {
+    const int c = t + 256 * i;
+    if (c >= chunks) continue;
+    float* p = gscale_part + (int64_t)blockIdx.x * D + 8 * c;
+    *reinterpret_cast<f32x4_t*>(p) = f32x4_t{gs[i][0], gs[i][1], gs[i][2], gs[i][3]};
+    *reinterpret_cast<f32x4_t*>(p + 4) = f32x4_t{gs[i][4], gs[i][5], gs[i][6], gs[i][7]};
   }
 }
 
@@ -179,7 +210,11 @@ __global__ __launch_bounds__(1024) void rms_norm_gscale_kernel(const float* __re
   }
 }
 
-constexpr int kRmsBwdWgs = 512;  // persistent workgroups of the backward with a scale gradient: 2048 waves, one partial row each
+constexpr int kRmsBwdWgs = 512;  // the workspace of the backward with a scale gradient holds 4 x this many partial rows
+// workgroups of that backward: four per CU, all resident at once with equal shares of the rows (2048 left a second,
+// mostly empty round: 46 us against 42 at 8192 x 4096; asking for a workgroup's next row ahead of time: 37 us)
+constexpr int kRmsBwdGrid = 1024;
+static_assert(kRmsBwdGrid <= kRmsBwdWgs * 4, "one partial row per workgroup");
 
 // ---------------------------------------------------------------------------------------------------
 // Rotary embedding on [b, s, n_h, h_d] with a [s, h_d/2, 2] fp32 (cos, sin) table; `inverse` rotates by -theta,
@@ -301,7 +336,7 @@ extern "C" int ttamd_rms_norm_bwd_bf16(const void* gy, const void* x, const void
                                        void* stream) {
   TT_REQUIRE(gy && x && scale && rstd && gx, "rms_norm_bwd: null pointer argument");
   TT_REQUIRE(aligned16(gy) && aligned16(x) && aligned16(scale) && aligned16(gx), "rms_norm_bwd: pointers must be 16-byte aligned");
-  TT_REQUIRE(rows > 0 && D > 0 && D % 8 == 0 && D <= 8192 && rows < (int64_t(1) << 32),
+  TT_REQUIRE(rows > 0 && D > 0 && D % 8 == 0 && D <= 8192 && rows < (int64_t(1) << 31),
              "rms_norm_bwd: bad shape rows=%lld D=%lld (D must be a multiple of 8, at most 8192)", (long long)rows, (long long)D);
   if (gscale) {
     TT_REQUIRE(workspace && aligned16(workspace), "rms_norm_bwd: the scale gradient needs a 16-byte aligned workspace");
@@ -310,30 +345,31 @@ extern "C" int ttamd_rms_norm_bwd_bf16(const void* gy, const void* x, const void
                   ttamd_rms_norm_bwd_workspace_bytes(D));
   }
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  // without a scale gradient: one wave per row; with it: a fixed number of persistent waves, each of which writes one
-  // row of partial sums (zeros if it had no row)
-  const int64_t wgs = gscale ? kRmsBwdWgs : (rows + 3) / 4;
-  const dim3 grid((unsigned)wgs), block(256);
+  const dim3 block(256);
   const uint16_t* G = reinterpret_cast<const uint16_t*>(gy);
   const uint16_t* X = reinterpret_cast<const uint16_t*>(x);
   const uint16_t* S = reinterpret_cast<const uint16_t*>(scale);
   uint16_t* GX = reinterpret_cast<uint16_t*>(gx);
+  // with a scale gradient: a fixed number of workgroups that walk the rows, each of which writes one row of partial
+  // sums; without: a workgroup per row
   float* part = reinterpret_cast<float*>(workspace);
+  const dim3 grid(gscale ? (unsigned)kRmsBwdGrid : (unsigned)rows);
+  const int64_t nv = (D / 8 + 255) / 256;  // D <= 8192: at most 4
 #define TT_RMS_BWD(NVV)                                                                                          \
   if (gscale)                                                                                                    \
     rms_norm_bwd_kernel<NVV, true><<<grid, block, 0, s>>>(G, X, S, rstd, GX, part, rows, (int)D);                \
   else                                                                                                           \
     rms_norm_bwd_kernel<NVV, false><<<grid, block, 0, s>>>(G, X, S, rstd, GX, nullptr, rows, (int)D);
-  switch (nv_for(D)) {
-    case 1: TT_RMS_BWD(1) break;
-    case 2: TT_RMS_BWD(2) break;
-    case 4: TT_RMS_BWD(4) break;
-    case 8: TT_RMS_BWD(8) break;
-    default: TT_RMS_BWD(16) break;
+  if (nv <= 1) {
+    TT_RMS_BWD(1)
+  } else if (nv <= 2) {
+    TT_RMS_BWD(2)
+  } else {
+    TT_RMS_BWD(4)
   }
 #undef TT_RMS_BWD
   if (gscale)
-    rms_norm_gscale_kernel<<<dim3((unsigned)((D + 63) / 64)), dim3(1024), 0, s>>>(part, kRmsBwdWgs * 4, (int)D,
+    rms_norm_gscale_kernel<<<dim3((unsigned)((D + 63) / 64)), dim3(1024), 0, s>>>(part, kRmsBwdGrid, (int)D,
                                                                                  reinterpret_cast<uint16_t*>(gscale));
   return check_launch("rms_norm_bwd");
 }
