@@ -75,8 +75,12 @@ __global__ __launch_bounds__(256) void nf4_dequant_merge_kernel(const uint32_t* 
       const float b = bsh[i][r];
 #pragma unroll
       for (int d = 0; d < 4; ++d) {
-        m[2 * d] = __builtin_fmaf(b, bits_f32(a[r][d] << 16), m[2 * d]);
-        m[2 * d + 1] = __builtin_fmaf(b, bits_f32(a[r][d] & 0xffff0000u), m[2 * d + 1]);
+        uint32_t ar = a[r][d];
+        // ranks above 32: keep the pair packed inside the row loop; unpacked ahead of it (which the compiler does when it
+        // can) the adapter columns take twice the registers and the kernel spills
+        if constexpr (R8 > 4 && !NORM) asm volatile("" : "+v"(ar));
+        m[2 * d] = __builtin_fmaf(b, bits_f32(ar << 16), m[2 * d]);
+        m[2 * d + 1] = __builtin_fmaf(b, bits_f32(ar & 0xffff0000u), m[2 * d + 1]);
       }
     }
     u32x4_t o;
