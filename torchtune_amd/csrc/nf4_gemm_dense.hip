@@ -63,15 +63,41 @@ __constant__ float kNF4Dense[16] = TT_NF4_TABLE;
 //   (mode 3 of the launcher: grad-input from the weight's own codes, nf4_expand_tiled_transposed_kernel below)
 // A workgroup of 256 threads covers 16 columns (one T) x 16 k-steps per iteration of its loop over the contraction.
 // ---------------------------------------------------------------------------------------------------------------------
+// One launch expands the weights of up to kGroupMax layers (the members of a group: stacked output columns in the forward,
+// the concatenated contraction in the grad-input); workgroups [blk_end[i - 1], blk_end[i]) along x work on member i.
+struct ExpandMember {
+  const uint8_t* codes;
+  const float* scal;
+  char* tiled;   // the copy this member writes into (its own stretch of the forward copy, or the shared grad-input copy)
+  int nout, kc;  // output columns and contraction length of the member's operand
+  int t_off;     // its first 32-wide step in the copy's contraction
+};
+struct ExpandGroup {
+  ExpandMember m[kGroupMax];
+  int blk_end[kGroupMax];
+  int n;
+};
+__device__ __forceinline__ int expand_member(const ExpandGroup& eg, int& blk) {
+  int which = 0;  // uniform over the workgroup
+#pragma unroll
+  for (int q = 0; q < kGroupMax - 1; ++q)
+    if (q < eg.n - 1 && blk >= eg.blk_end[q]) which = q + 1;
+  if (which) blk -= eg.blk_end[which - 1];
+  return which;
+}
+
 template <int MODE>
-__global__ __launch_bounds__(256) void nf4_expand_tiled_kernel(const uint8_t* __restrict__ codes, const float* __restrict__ scal,
-                                                               int Nout, int Kc, int nk_total, int t_off,
-                                                               char* __restrict__ tiled, int paired) {
+__global__ __launch_bounds__(256) void nf4_expand_tiled_kernel(const ExpandGroup eg, int nk_total, int paired) {
   __shared__ float2 lut[256];
   const int tid = threadIdx.x;
   lut[tid] = make_float2(round_to_bf16(kNF4Dense[tid >> 4]), round_to_bf16(kNF4Dense[tid & 15]));
   __syncthreads();
-  const int T = blockIdx.x;
+  int T = blockIdx.x;
+  const ExpandMember& me = eg.m[expand_member(eg, T)];
+  const uint8_t* __restrict__ codes = me.codes;
+  const float* __restrict__ scal = me.scal;
+  char* __restrict__ tiled = me.tiled;
+  const int Nout = me.nout, Kc = me.kc, t_off = me.t_off;
   // paired: two weights of equal shape share one tiled copy, 128 columns (8 blocks) of the one followed by the same
   // 128 columns of the other (whose `tiled` starts 8 blocks further), so that a 256-wide tile of the GEMM holds both
   const int To = paired ? ((T >> 3) << 4) + (T & 7) : T;
@@ -117,16 +143,21 @@ __global__ __launch_bounds__(256) void nf4_expand_tiled_kernel(const uint8_t* __
 // they lie, output = tiles of W^T (rows: k, contraction: n).  A workgroup expands 32 rows n (one 32-wide step of the
 // contraction) x 256 columns k, turns the block through LDS (row pitch 80 bytes: both the 2-byte writes down a column
 // and the 16-byte reads along a row spread over the banks) and writes sixteen 1 KiB pieces.
-__global__ __launch_bounds__(256) void nf4_expand_tiled_transposed_kernel(const uint8_t* __restrict__ codes, const float* __restrict__ scal,
-                                                                          int N, int K, int nk_total, int t_off, char* __restrict__ tiled) {
+__global__ __launch_bounds__(256) void nf4_expand_tiled_transposed_kernel(const ExpandGroup eg, int K, int nk_total) {
   constexpr int kPitch = 80;
   __shared__ float2 lut[256];
   __shared__ __attribute__((aligned(16))) char sm[256 * kPitch];
   const int tid = threadIdx.x;
   lut[tid] = make_float2(round_to_bf16(kNF4Dense[tid >> 4]), round_to_bf16(kNF4Dense[tid & 15]));
   __syncthreads();
+  int step = blockIdx.x;  // 32-row step of the member's contraction
+  const ExpandMember& me = eg.m[expand_member(eg, step)];
+  const uint8_t* __restrict__ codes = me.codes;
+  const float* __restrict__ scal = me.scal;
+  char* __restrict__ tiled = me.tiled;
+  const int t_off = me.t_off;
   const int r = tid & 31, c = tid >> 5;
-  const int n = 32 * blockIdx.x + r;
+  const int n = 32 * step + r;
   const int kk0 = 256 * blockIdx.y + 32 * c;
   if (kk0 < K) {
     const u32x4_t cd = *reinterpret_cast<const u32x4_t*>(codes + (int64_t)n * (K >> 1) + (kk0 >> 1));
@@ -152,7 +183,7 @@ __global__ __launch_bounds__(256) void nf4_expand_tiled_transposed_kernel(const 
     const int T = 16 * blockIdx.y + Tl;
     if (16 * T >= K) break;
     const u32x4_t v = *reinterpret_cast<const u32x4_t*>(sm + (16 * Tl + (l & 15)) * kPitch + 16 * (l >> 4));
-    *reinterpret_cast<u32x4_t*>(tiled + ((int64_t)T * nk_total + t_off + blockIdx.x) * 1024 + l * 16) = v;
+    *reinterpret_cast<u32x4_t*>(tiled + ((int64_t)T * nk_total + t_off + step) * 1024 + l * 16) = v;
   }
 }
 
@@ -687,28 +718,46 @@ __global__ __launch_bounds__(512) void nf4_gemm_dense_kernel(const DenseArgs g) 
 // grad-input launch (adapter weights [r, K]) whose result goes on through the backward of silu(gate) * up
 __global__ __launch_bounds__(512) void nf4_gemm_dense_swiglu_bwd_kernel(const DenseArgs g) { gemm_dense_tile<false, kEpiSwigluBwd>(g); }
 
-int launch_expand(int mode, const uint8_t* codes, const float* scal, int64_t Nout, int64_t Kc, int64_t nk_total, int64_t t_off,
-                  char* tiled, hipStream_t s, bool paired = false) {
-  // one block of 16 columns per blockIdx.x; the contraction is cut along blockIdx.y so that about 2048 workgroups exist
-  const int64_t chunks = ((Kc >> 5) + 15) / 16;
-  int64_t ysplit = (2048 + (Nout >> 4) - 1) / (Nout >> 4);
-  ysplit = ysplit < 1 ? 1 : (ysplit > chunks ? chunks : ysplit);
-  const dim3 grid((unsigned)(Nout >> 4), (unsigned)ysplit), block(256);
-  if (mode == 3) {  // Nout = K, Kc = N of the weight: codes and scalers in the weight's own layout
+// mode 0 / 2 / 1: nf4_expand_tiled_kernel<mode> over the members' stacked blocks of 16 output columns; mode 3: the
+// transposed kernel over the members' 32-row steps (nout = K, kc = N of each member: codes and scalers in the weight's
+// own layout).  blk_end is filled in here.
+int launch_expand_group(int mode, ExpandGroup& eg, int64_t nk_total, hipStream_t s, bool paired = false) {
+  const dim3 block(256);
+  int64_t blocks = 0, max_chunks = 1;
+  for (int i = 0; i < eg.n; ++i) {
+    blocks += mode == 3 ? eg.m[i].kc >> 5 : eg.m[i].nout >> 4;
+    eg.blk_end[i] = (int)blocks;
+    const int64_t chunks = ((eg.m[i].kc >> 5) + 15) / 16;
+    max_chunks = chunks > max_chunks ? chunks : max_chunks;
+  }
+  TT_REQUIRE(blocks > 0 && blocks < (int64_t(1) << 31), "nf4_expand_tiled: bad launch size");
+  if (mode == 3) {
+    const int64_t K = eg.m[0].nout;
     TT_REQUIRE(!paired, "nf4_expand_tiled: the paired layout exists for the forward modes only");
-    TT_REQUIRE((Nout + 255) / 256 < 65536, "nf4_expand_tiled: K too large for one launch");
-    nf4_expand_tiled_transposed_kernel<<<dim3((unsigned)(Kc >> 5), (unsigned)((Nout + 255) / 256)), block, 0, s>>>(
-        codes, scal, (int)Kc, (int)Nout, (int)nk_total, (int)t_off, tiled);
+    TT_REQUIRE((K + 255) / 256 < 65536, "nf4_expand_tiled: K too large for one launch");
+    nf4_expand_tiled_transposed_kernel<<<dim3((unsigned)blocks, (unsigned)((K + 255) / 256)), block, 0, s>>>(eg, (int)K, (int)nk_total);
     return check_launch("nf4_expand_tiled_transposed");
   }
+  // the contraction is cut along blockIdx.y so that about 2048 workgroups exist
+  int64_t ysplit = (2048 + blocks - 1) / blocks;
+  ysplit = ysplit < 1 ? 1 : (ysplit > max_chunks ? max_chunks : ysplit);
+  const dim3 grid((unsigned)blocks, (unsigned)ysplit);
   const int pr = paired ? 1 : 0;
   if (mode == 1)
-    nf4_expand_tiled_kernel<1><<<grid, block, 0, s>>>(codes, scal, (int)Nout, (int)Kc, (int)nk_total, (int)t_off, tiled, pr);
+    nf4_expand_tiled_kernel<1><<<grid, block, 0, s>>>(eg, (int)nk_total, pr);
   else if (mode == 2)
-    nf4_expand_tiled_kernel<2><<<grid, block, 0, s>>>(codes, scal, (int)Nout, (int)Kc, (int)nk_total, (int)t_off, tiled, pr);
+    nf4_expand_tiled_kernel<2><<<grid, block, 0, s>>>(eg, (int)nk_total, pr);
   else
-    nf4_expand_tiled_kernel<0><<<grid, block, 0, s>>>(codes, scal, (int)Nout, (int)Kc, (int)nk_total, (int)t_off, tiled, pr);
+    nf4_expand_tiled_kernel<0><<<grid, block, 0, s>>>(eg, (int)nk_total, pr);
   return check_launch("nf4_expand_tiled");
+}
+
+int launch_expand(int mode, const uint8_t* codes, const float* scal, int64_t Nout, int64_t Kc, int64_t nk_total, int64_t t_off,
+                  char* tiled, hipStream_t s, bool paired = false) {
+  ExpandGroup eg = {};
+  eg.n = 1;
+  eg.m[0] = ExpandMember{codes, scal, tiled, (int)Nout, (int)Kc, (int)t_off};
+  return launch_expand_group(mode, eg, nk_total, s, paired);
 }
 
 int launch_dense(DenseArgs& g, hipStream_t s) {
@@ -839,12 +888,17 @@ int run_gemm_dense_group_fwd(const void* x, const GroupGemm& d, const void* h_ca
   g.seg[0].Kc = (int)d.K;
   g.nout = g.nad = d.n;
   int64_t n_off = 0;
+  // the members' weights are expanded by one launch when they come in the same form (with or without transposed scalers)
+  ExpandGroup eg = {};
+  bool one_launch = true;
+  for (int i = 0; i < d.n; ++i) one_launch = one_launch && (d.bscal_t[i] != nullptr) == (d.bscal_t[0] != nullptr);
   for (int i = 0; i < d.n; ++i) {
     const bool tr = d.bscal_t[i] != nullptr;
     // gated: the members' column blocks alternate 8 by 8, the second member starting 8 blocks (128 columns) in
     char* dst = reinterpret_cast<char*>(workspace) + (gated ? (int64_t)i * 128 : n_off) * d.K * 2;
-    if (int rc = launch_expand(tr ? 2 : 0, d.codes[i], tr ? d.bscal_t[i] : d.bscal[i], d.N[i], d.K, d.K >> 5, 0, dst, s, gated))
-      return rc;
+    eg.m[i] = ExpandMember{d.codes[i], tr ? d.bscal_t[i] : d.bscal[i], dst, (int)d.N[i], (int)d.K, 0};
+    if (!one_launch)
+      if (int rc = launch_expand(tr ? 2 : 0, eg.m[i].codes, eg.m[i].scal, d.N[i], d.K, d.K >> 5, 0, dst, s, gated)) return rc;
     g.ad[i].lX = reinterpret_cast<const uint16_t*>(h_cat) + d.r_off[i];
     g.ad[i].lW = d.lora_b[i];
     g.ad[i].R = d.rank[i];
@@ -857,6 +911,10 @@ int run_gemm_dense_group_fwd(const void* x, const GroupGemm& d, const void* h_ca
     g.out[i].n_begin = (int)n_off;
     g.out[i].width = (int)d.N[i];
     n_off += d.N[i];
+  }
+  if (one_launch) {
+    eg.n = d.n;
+    if (int rc = launch_expand_group(d.bscal_t[0] ? 2 : 0, eg, d.K >> 5, s, gated)) return rc;
   }
   g.Wt = reinterpret_cast<const char*>(workspace);
   g.M = (int)d.M; g.Nout = (int)n_off; g.Kc = (int)d.K;
@@ -886,13 +944,19 @@ int run_gemm_dense_group_dx(const GroupDx& d, const void* gh_cat, void* gx, void
   g.nseg = d.n;
   g.nout = 1;
   int64_t t_off = 0;
+  // one expansion launch for the members when all of them come with, or all without, the transposed copies
+  ExpandGroup eg = {};
+  bool one_launch = true;
+  for (int i = 0; i < d.n; ++i) one_launch = one_launch && (d.codes_t[i] != nullptr) == (d.codes_t[0] != nullptr);
   for (int i = 0; i < d.n; ++i) {
     const bool tr = d.codes_t[i] != nullptr;
     TT_REQUIRE(aligned16(d.gy[i]) && (tr ? aligned16(d.codes_t[i]) && aligned16(d.scal_t[i]) : aligned16(d.codes[i]) && d.bscal[i] != nullptr),
                "nf4_group_dx (expanded): pointers must be 16-byte aligned");
-    if (int rc = launch_expand(tr ? 1 : 3, tr ? d.codes_t[i] : d.codes[i], tr ? d.scal_t[i] : d.bscal[i], d.K, d.N[i], n_total >> 5, t_off,
-                               reinterpret_cast<char*>(workspace), s))
-      return rc;
+    eg.m[i] = ExpandMember{tr ? d.codes_t[i] : d.codes[i], tr ? d.scal_t[i] : d.bscal[i], reinterpret_cast<char*>(workspace), (int)d.K,
+                           (int)d.N[i], (int)t_off};
+    if (!one_launch)
+      if (int rc = launch_expand(tr ? 1 : 3, eg.m[i].codes, eg.m[i].scal, d.K, d.N[i], n_total >> 5, t_off, reinterpret_cast<char*>(workspace), s))
+        return rc;
     t_off += d.N[i] >> 5;
     g.seg[i].X = d.gy[i];
     g.seg[i].Kc = (int)d.N[i];
@@ -905,6 +969,10 @@ int run_gemm_dense_group_dx(const GroupDx& d, const void* gh_cat, void* gx, void
       a.n_end = (int)d.K;
       a.lscale = 1.0f;
     }
+  }
+  if (one_launch) {
+    eg.n = d.n;
+    if (int rc = launch_expand_group(d.codes_t[0] ? 1 : 3, eg, n_total >> 5, s)) return rc;
   }
   g.out[0].C = reinterpret_cast<uint16_t*>(gx);
   g.out[0].n_begin = 0;
