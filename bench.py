@@ -64,7 +64,7 @@ class GemmTimer:
     """HIP-event timing of the fused-GEMM launches while installed in ``ops``.
 
     An event pair costs the stream about 6 us per timed launch (the GPU idles around the markers), 1.6 % of a step if
-    every one of its 445 launches is timed.  So every ``stride``-th launch of each (kind, shape) is timed and the
+    every one of its 255 calls is timed.  So every ``stride``-th launch of each (kind, shape) is timed and the
     others only counted: the averages still come from the timed region itself, the step pays a quarter of the cost."""
 
     def __init__(self, stride: int = 4):
