@@ -77,7 +77,7 @@ class GemmTimer:
         # "fwd" / "bwd": one layer, one call of the library.  "fwd_group" / "bwd_group": the layers of a group with a common
         # input (N and rank are lists), one call; "fwd_gated": the gate / up pair with its gated product in the same call;
         # "bwd_swiglu": the grad-input of the layer after the gated product, carried on to the gradients of gate and up.  Between the events lie all launches of the call: with the weight expanded
-        # once per call (many tokens) one expansion launch per member and one GEMM launch; otherwise one fused launch per
+        # once per call (many tokens) one expansion launch (the weights of a group together) and one GEMM launch; otherwise one fused launch per
         # member (forward) or the single fused grad-input launch over all members' output columns.
         from torchtune_amd import _lib, ops
 
