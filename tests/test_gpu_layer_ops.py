@@ -48,6 +48,29 @@ def test_rms_norm_forward_backward(rows, D):
     assert torch.equal(xd2.grad, xd.grad)
 
 
+def test_rms_norm_backward_when_workgroups_walk_several_rows():
+    """More rows than the scale-gradient form has workgroups (1024): each walks two or three rows, asking for the next one
+    while it works on the current; input and scale gradients against the oracle's autograd, and the input gradient
+    against the form without a scale gradient bit for bit."""
+    rows, D = 2500, 4096
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(rows, D, generator=g).to(BF).requires_grad_()
+    w = (torch.rand(D, generator=g) + 0.5).to(BF).requires_grad_()
+    gy = torch.randn(rows, D, generator=g).to(BF)
+    lo.rms_norm(x, w, 1e-5).backward(gy)
+    m = layer_ops.RMSNorm(D, 1e-5).to(DEV, BF)
+    with torch.no_grad():
+        m.scale.copy_(w)
+    xd = x.detach().to(DEV).requires_grad_()
+    m(xd).backward(gy.to(DEV))
+    _close(xd.grad, x.grad)
+    _close(m.scale.grad, w.grad, rtol=2e-2, atol=2e-2 * float(w.grad.float().abs().max()))
+    m.scale.requires_grad_(False)
+    xd2 = x.detach().to(DEV).requires_grad_()
+    m(xd2).backward(gy.to(DEV))
+    assert torch.equal(xd2.grad, xd.grad)
+
+
 def test_rms_norm_leading_dimensions_and_validation():
     x = torch.randn(2, 3, 256, device=DEV).to(BF)
     w = torch.ones(256, device=DEV, dtype=BF)
