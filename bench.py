@@ -531,6 +531,9 @@ def main() -> int:
                          "instead of a pass of its own (QLoRA workloads)")
     ap.add_argument("--no-qat-tn-group", action="store_true",
                     help="A/B (QAT workloads): one weight-gradient launch per member of a group instead of one for the group")
+    ap.add_argument("--no-fused-add-norm", action="store_true",
+                    help="A/B: the additions of the residual stream as passes of their own instead of inside the RMSNorm that "
+                         "follows each of them")
     ap.add_argument("--no-group", action="store_true",
                     help="one call per projection, as the reference's modules make them, instead of the group kernels for the "
                          "projections that share an input (q/k/v, gate/up): for A/B timing")
@@ -561,6 +564,7 @@ def main() -> int:
     harness.SDPA_BACKEND = args.sdpa
     harness.GROUP_SHARED_INPUT = not args.no_group
     harness.GATED_EPILOGUE = not args.no_gated_epilogue
+    harness.FUSED_ADD_NORM = not args.no_fused_add_norm
     harness.SWIGLU_BWD_EPILOGUE = args.swiglu_bwd_epilogue
     ops.EXPANDED_WEIGHT_PATH = not args.no_expanded_weight
     if args.no_qat_tiled_gemm:

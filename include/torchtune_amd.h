@@ -559,6 +559,21 @@ int ttamd_rms_norm_bwd_bf16(const void* gy, const void* x, const void* scale, co
                             int64_t rows, int64_t D, void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * The residual stream's addition in the same passes (h = attn_out + x and out = h + mlp_out of
+ * torchtune/modules/transformer.py:129-141, each followed by an RMSNorm in the next sub-block):
+ *   ttamd_add_rms_norm_fwd_bf16: h = bf16(x + residual) (written to h) and y = RMSNorm(h); the bits of the addition
+ *     followed by ttamd_rms_norm_fwd_bf16, without reading h back.
+ *   ttamd_rms_norm_bwd_add_bf16: gx = bf16( bf16(gx of ttamd_rms_norm_bwd_bf16) + g_add ), g_add [rows, D] bf16 being the
+ *     gradient that reaches the norm's input on the residual way (NULL: ttamd_rms_norm_bwd_bf16): what autograd's
+ *     accumulation of the two gradients gives, without writing and re-reading the first.
+ * The reference has no counterpart (separate eager kernels).
+ */
+int ttamd_add_rms_norm_fwd_bf16(const void* x, const void* residual, const void* scale, float eps, void* h, void* y, float* rstd,
+                                int64_t rows, int64_t D, void* stream);
+int ttamd_rms_norm_bwd_add_bf16(const void* gy, const void* x, const void* scale, const float* rstd, const void* g_add, void* gx,
+                                void* gscale, int64_t rows, int64_t D, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * Rotary position embedding (torchtune/models/llama3_1/_position_embeddings.py:128-190, positions 0..S-1):
  * x, y [B, S, n_heads, head_dim] bf16; cache [S, head_dim/2, 2] fp32 (cos, sin); consecutive pairs are rotated in
  * fp32.  inverse != 0 rotates by the negative angle, which is the backward pass.  head_dim a multiple of 8.

@@ -44,6 +44,26 @@ def test_activation_checkpointing_gives_the_same_step():
             assert torch.equal(p.grad, q.grad), n
 
 
+@pytest.mark.parametrize("kind", ["qlora", "qat"])
+def test_residual_additions_inside_the_norm_pass_give_the_same_step(monkeypatch, kind):
+    """``harness.FUSED_ADD_NORM``: the additions of the residual stream inside the RMSNorm pass that follows each of them
+    against additions of their own: the same loss and the same gradients, bit for bit (QLoRA: adapter gradients; QAT:
+    every weight and norm scale, so the scale-gradient form of the norm's backward runs as well)."""
+    build = (lambda: harness.build_qlora_decoder("tiny", rank=8, alpha=16.0, device=DEV, seed=0)) if kind == "qlora" else \
+            (lambda: harness.build_qat_decoder("tiny", groupsize=32, device=DEV, seed=0))
+    tokens = torch.randint(0, 1024, (2, 160), device=DEV, generator=torch.Generator(device=DEV).manual_seed(4))
+    out = []
+    for fused in (True, False):
+        monkeypatch.setattr(harness, "FUSED_ADD_NORM", fused)
+        model = build()
+        loss = harness.train_step(model, tokens, tokens)
+        out.append((loss, {n: p.grad.clone() for n, p in model.named_parameters() if p.grad is not None}))
+    assert torch.equal(out[0][0], out[1][0])
+    assert set(out[0][1]) == set(out[1][1]) and out[0][1]
+    for n, gr in out[0][1].items():
+        assert torch.equal(gr, out[1][1][n]), n
+
+
 def test_tiny_qat_decoder_step():
     model = harness.build_qat_decoder("tiny", groupsize=32, device=DEV, seed=0)
     tokens = torch.randint(0, 1024, (2, 64), device=DEV, generator=torch.Generator(device=DEV).manual_seed(3))

@@ -71,6 +71,40 @@ def test_rms_norm_backward_when_workgroups_walk_several_rows():
     assert torch.equal(xd2.grad, xd.grad)
 
 
+@pytest.mark.parametrize("rows,D,train_scale", [(5, 64, True), (70, 4096, True), (2500, 4096, True), (33, 8192, False), (9, 4104, False)])
+def test_add_rms_norm_equals_the_addition_followed_by_the_norm_bitwise(rows, D, train_scale):
+    """``add_rms_norm(x, r, norm)`` against ``h = x + r; norm(h)``: both outputs and the gradients of x, r and the scale
+    bit for bit, with gradients arriving on both outputs (as in a decoder layer) and on the normalised one alone."""
+    g = torch.Generator().manual_seed(rows + D)
+    x = torch.randn(rows, D, generator=g).to(BF).to(DEV)
+    r = torch.randn(rows, D, generator=g).to(BF).to(DEV)
+    gh = torch.randn(rows, D, generator=g).to(BF).to(DEV)
+    gn = torch.randn(rows, D, generator=g).to(BF).to(DEV)
+    m = layer_ops.RMSNorm(D, 1e-5).to(DEV, BF)
+    with torch.no_grad():
+        m.scale.copy_((torch.rand(D, generator=g) + 0.5).to(BF))
+    m.scale.requires_grad_(train_scale)
+
+    def run(fused, both):
+        m.zero_grad()
+        xa, ra = x.clone().requires_grad_(), r.clone().requires_grad_()
+        if fused:
+            h, n = layer_ops.add_rms_norm(xa, ra, m)
+        else:
+            h = xa + ra
+            n = m(h)
+        if both:
+            torch.autograd.backward([h, n], [gh, gn])
+        else:
+            n.backward(gn)
+        out = [h.detach(), n.detach(), xa.grad, ra.grad]
+        return out + ([m.scale.grad.clone()] if train_scale else [])
+
+    for both in (True, False):
+        for a, b in zip(run(True, both), run(False, both)):
+            assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+
+
 def test_rms_norm_leading_dimensions_and_validation():
     x = torch.randn(2, 3, 256, device=DEV).to(BF)
     w = torch.ones(256, device=DEV, dtype=BF)

@@ -143,6 +143,11 @@ SIGNATURES = {
         _int,
         [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _i64, _i64, _c_void_p, _size, _c_void_p],
     ),
+    "ttamd_add_rms_norm_fwd_bf16": (_int, [_c_void_p, _c_void_p, _c_void_p, _f32, _c_void_p, _c_void_p, _c_void_p, _i64, _i64, _c_void_p]),
+    "ttamd_rms_norm_bwd_add_bf16": (
+        _int,
+        [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _i64, _i64, _c_void_p, _size, _c_void_p],
+    ),
     "ttamd_rope_bf16": (_int, [_c_void_p, _c_void_p, _c_void_p, _i64, _i64, _i64, _i64, _int, _c_void_p]),
     "ttamd_repeat_kv_bf16": (_int, [_c_void_p, _c_void_p, _i64, _i64, _i64, _i64, _c_void_p]),
     "ttamd_repeat_kv_bwd_bf16": (_int, [_c_void_p, _c_void_p, _i64, _i64, _i64, _i64, _c_void_p]),

@@ -41,10 +41,13 @@ __device__ __forceinline__ float wave_sum(float v) {
 //   backward: g = bf16(gy * scale) (eager's bf16 product), c = mean(g * x) * rstd^2,
 //             gx = bf16(rstd * (g - x * c));  gscale partial[w][d] = sum over workgroup w's rows of gy * xn
 // ---------------------------------------------------------------------------------------------------
-template <int NV>
-__global__ __launch_bounds__(256) void rms_norm_fwd_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ scale,
-                                                           float eps, uint16_t* __restrict__ y, float* __restrict__ rstd_out,
-                                                           int64_t rows, int D) {
+// ADD: the row normalised is h = bf16(x + res) (the residual stream's addition, torchtune/modules/transformer.py:129-141),
+// which the launch also writes to h_out; same bits as the addition and the norm one after the other.
+template <int NV, bool ADD>
+__global__ __launch_bounds__(256) void rms_norm_fwd_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ res,
+                                                           const uint16_t* __restrict__ scale, float eps,
+                                                           uint16_t* __restrict__ h_out, uint16_t* __restrict__ y,
+                                                           float* __restrict__ rstd_out, int64_t rows, int D) {
   const int lane = threadIdx.x & 63;
   const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= rows) return;
@@ -56,7 +59,15 @@ __global__ __launch_bounds__(256) void rms_norm_fwd_kernel(const uint16_t* __res
   for (int i = 0; i < NV; ++i) {
     const int c = lane + 64 * i;
     v[i] = u32x4_t{0, 0, 0, 0};
-    if (c < chunks) v[i] = *(xr + c);
+    if (c < chunks) {
+      v[i] = *(xr + c);
+      if constexpr (ADD) {
+        const u32x4_t rv = *(reinterpret_cast<const u32x4_t*>(res + row * D) + c);
+#pragma unroll
+        for (int d = 0; d < 4; ++d) v[i][d] = pack2(lo_f(v[i][d]) + lo_f(rv[d]), hi_f(v[i][d]) + hi_f(rv[d]));
+        __builtin_nontemporal_store(v[i], reinterpret_cast<u32x4_t*>(h_out + row * D) + c);
+      }
+    }
 #pragma unroll
     for (int d = 0; d < 4; ++d) {
       const float a = lo_f(v[i][d]), b = hi_f(v[i][d]);
@@ -92,11 +103,13 @@ __global__ __launch_bounds__(256) void rms_norm_fwd_kernel(const uint16_t* __res
 // wave order - the same order in both forms, so the input gradient does not depend on whether the scale is trained; the
 // slot alternates with the row, so one barrier per row is enough.  Workgroup w writes row w of the partial sums (zeros
 // if it saw no row).
+// g_add (or null): a gradient that reaches x on another way (the residual stream); the launch then writes
+// bf16(bf16(gx) + g_add), what autograd's accumulation of the two would give.
 template <int NV, bool GSCALE>
 __global__ __launch_bounds__(256) void rms_norm_bwd_kernel(const uint16_t* __restrict__ gy, const uint16_t* __restrict__ x,
                                                            const uint16_t* __restrict__ scale, const float* __restrict__ rstd_in,
-                                                           uint16_t* __restrict__ gx, float* __restrict__ gscale_part,
-                                                           int64_t rows, int D) {
+                                                           const uint16_t* __restrict__ g_add, uint16_t* __restrict__ gx,
+                                                           float* __restrict__ gscale_part, int64_t rows, int D) {
   __shared__ float dots[2][4];
   const int t = threadIdx.x, wave = t >> 6;
   const int chunks = D >> 3;
@@ -163,6 +176,11 @@ __global__ __launch_bounds__(256) void rms_norm_bwd_kernel(const uint16_t* __res
 #pragma unroll
       for (int d = 0; d < 4; ++d)
         o[d] = pack2(rstd * (lo_f(gv[i][d]) - lo_f(xv[i][d]) * c2), rstd * (hi_f(gv[i][d]) - hi_f(xv[i][d]) * c2));
+      if (g_add) {  // uniform
+        const u32x4_t ga = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(g_add + row * D) + c);
+#pragma unroll
+        for (int d = 0; d < 4; ++d) o[d] = pack2(lo_f(o[d]) + lo_f(ga[d]), hi_f(o[d]) + hi_f(ga[d]));
+      }
       __builtin_nontemporal_store(o, outr + c);
     }
     if constexpr (GSCALE) {
@@ -306,25 +324,46 @@ int nv_for(int64_t D) {
 
 using namespace ttamd;
 
-extern "C" int ttamd_rms_norm_fwd_bf16(const void* x, const void* scale, float eps, void* y, float* rstd, int64_t rows,
-                                       int64_t D, void* stream) {
-  TT_REQUIRE(x && scale && y, "rms_norm_fwd: null pointer argument");
-  TT_REQUIRE(aligned16(x) && aligned16(scale) && aligned16(y), "rms_norm_fwd: pointers must be 16-byte aligned");
+namespace {
+int rms_norm_fwd(const char* who, const void* x, const void* res, const void* scale, float eps, void* h, void* y, float* rstd,
+                 int64_t rows, int64_t D, void* stream) {
+  TT_REQUIRE(x && scale && y && (res == nullptr) == (h == nullptr), "%s: null pointer argument", who);
+  TT_REQUIRE(aligned16(x) && aligned16(scale) && aligned16(y) && aligned16(res) && aligned16(h), "%s: pointers must be 16-byte aligned", who);
   TT_REQUIRE(rows > 0 && D > 0 && D % 8 == 0 && D <= 8192 && rows < (int64_t(1) << 32),
-             "rms_norm_fwd: bad shape rows=%lld D=%lld (D must be a multiple of 8, at most 8192)", (long long)rows, (long long)D);
+             "%s: bad shape rows=%lld D=%lld (D must be a multiple of 8, at most 8192)", who, (long long)rows, (long long)D);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
   const uint16_t* X = reinterpret_cast<const uint16_t*>(x);
+  const uint16_t* R = reinterpret_cast<const uint16_t*>(res);
   const uint16_t* S = reinterpret_cast<const uint16_t*>(scale);
+  uint16_t* H = reinterpret_cast<uint16_t*>(h);
   uint16_t* Y = reinterpret_cast<uint16_t*>(y);
+#define TT_RMS_FWD(NVV)                                                                             \
+  if (res)                                                                                          \
+    rms_norm_fwd_kernel<NVV, true><<<grid, block, 0, s>>>(X, R, S, eps, H, Y, rstd, rows, (int)D);  \
+  else                                                                                              \
+    rms_norm_fwd_kernel<NVV, false><<<grid, block, 0, s>>>(X, nullptr, S, eps, nullptr, Y, rstd, rows, (int)D);
   switch (nv_for(D)) {
-    case 1: rms_norm_fwd_kernel<1><<<grid, block, 0, s>>>(X, S, eps, Y, rstd, rows, (int)D); break;
-    case 2: rms_norm_fwd_kernel<2><<<grid, block, 0, s>>>(X, S, eps, Y, rstd, rows, (int)D); break;
-    case 4: rms_norm_fwd_kernel<4><<<grid, block, 0, s>>>(X, S, eps, Y, rstd, rows, (int)D); break;
-    case 8: rms_norm_fwd_kernel<8><<<grid, block, 0, s>>>(X, S, eps, Y, rstd, rows, (int)D); break;
-    default: rms_norm_fwd_kernel<16><<<grid, block, 0, s>>>(X, S, eps, Y, rstd, rows, (int)D); break;
+    case 1: TT_RMS_FWD(1) break;
+    case 2: TT_RMS_FWD(2) break;
+    case 4: TT_RMS_FWD(4) break;
+    case 8: TT_RMS_FWD(8) break;
+    default: TT_RMS_FWD(16) break;
   }
-  return check_launch("rms_norm_fwd");
+#undef TT_RMS_FWD
+  return check_launch(who);
+}
+}  // namespace
+
+extern "C" int ttamd_rms_norm_fwd_bf16(const void* x, const void* scale, float eps, void* y, float* rstd, int64_t rows,
+                                       int64_t D, void* stream) {
+  return rms_norm_fwd("rms_norm_fwd", x, nullptr, scale, eps, nullptr, y, rstd, rows, D, stream);
+}
+
+extern "C" int ttamd_add_rms_norm_fwd_bf16(const void* x, const void* residual, const void* scale, float eps, void* h, void* y,
+                                           float* rstd, int64_t rows, int64_t D, void* stream) {
+  TT_REQUIRE(residual && h, "add_rms_norm_fwd: null pointer argument");
+  return rms_norm_fwd("add_rms_norm_fwd", x, residual, scale, eps, h, y, rstd, rows, D, stream);
 }
 
 extern "C" size_t ttamd_rms_norm_bwd_workspace_bytes(int64_t D) {
@@ -334,8 +373,15 @@ extern "C" size_t ttamd_rms_norm_bwd_workspace_bytes(int64_t D) {
 extern "C" int ttamd_rms_norm_bwd_bf16(const void* gy, const void* x, const void* scale, const float* rstd, void* gx,
                                        void* gscale, int64_t rows, int64_t D, void* workspace, size_t workspace_bytes,
                                        void* stream) {
+  return ttamd_rms_norm_bwd_add_bf16(gy, x, scale, rstd, nullptr, gx, gscale, rows, D, workspace, workspace_bytes, stream);
+}
+
+extern "C" int ttamd_rms_norm_bwd_add_bf16(const void* gy, const void* x, const void* scale, const float* rstd, const void* g_add,
+                                           void* gx, void* gscale, int64_t rows, int64_t D, void* workspace,
+                                           size_t workspace_bytes, void* stream) {
   TT_REQUIRE(gy && x && scale && rstd && gx, "rms_norm_bwd: null pointer argument");
-  TT_REQUIRE(aligned16(gy) && aligned16(x) && aligned16(scale) && aligned16(gx), "rms_norm_bwd: pointers must be 16-byte aligned");
+  TT_REQUIRE(aligned16(gy) && aligned16(x) && aligned16(scale) && aligned16(gx) && aligned16(g_add),
+             "rms_norm_bwd: pointers must be 16-byte aligned");
   TT_REQUIRE(rows > 0 && D > 0 && D % 8 == 0 && D <= 8192 && rows < (int64_t(1) << 31),
              "rms_norm_bwd: bad shape rows=%lld D=%lld (D must be a multiple of 8, at most 8192)", (long long)rows, (long long)D);
   if (gscale) {
@@ -350,6 +396,7 @@ extern "C" int ttamd_rms_norm_bwd_bf16(const void* gy, const void* x, const void
   const uint16_t* X = reinterpret_cast<const uint16_t*>(x);
   const uint16_t* S = reinterpret_cast<const uint16_t*>(scale);
   uint16_t* GX = reinterpret_cast<uint16_t*>(gx);
+  const uint16_t* GA = reinterpret_cast<const uint16_t*>(g_add);
   // with a scale gradient: a fixed number of workgroups that walk the rows, each of which writes one row of partial
   // sums; without: a workgroup per row
   float* part = reinterpret_cast<float*>(workspace);
@@ -357,9 +404,9 @@ extern "C" int ttamd_rms_norm_bwd_bf16(const void* gy, const void* x, const void
   const int64_t nv = (D / 8 + 255) / 256;  // D <= 8192: at most 4
 #define TT_RMS_BWD(NVV)                                                                                          \
   if (gscale)                                                                                                    \
-    rms_norm_bwd_kernel<NVV, true><<<grid, block, 0, s>>>(G, X, S, rstd, GX, part, rows, (int)D);                \
+    rms_norm_bwd_kernel<NVV, true><<<grid, block, 0, s>>>(G, X, S, rstd, GA, GX, part, rows, (int)D);            \
   else                                                                                                           \
-    rms_norm_bwd_kernel<NVV, false><<<grid, block, 0, s>>>(G, X, S, rstd, GX, nullptr, rows, (int)D);
+    rms_norm_bwd_kernel<NVV, false><<<grid, block, 0, s>>>(G, X, S, rstd, GA, GX, nullptr, rows, (int)D);
   if (nv <= 1) {
     TT_RMS_BWD(1)
   } else if (nv <= 2) {

@@ -79,6 +79,9 @@ SHAPES = {
 }
 
 
+# True: the additions of the residual stream run inside the RMSNorm pass that follows each of them, forward and backward
+# (same bits; one write and one read of the stream less per addition)
+FUSED_ADD_NORM = True
 # True: RMSNorm, RoPE and the SwiGLU gate run as single-pass HIP kernels (bf16 on the GPU); False: the eager op chains
 # of the reference.  The quantized linears are unaffected.
 FUSED_LAYER_OPS = True
@@ -201,6 +204,14 @@ class FeedForward(nn.Module):
         return self.w2(layer_ops.swiglu(g, u) if _fused(g) else F.silu(g) * u)
 
 
+def _add_norm(x: torch.Tensor, delta: torch.Tensor, norm: RMSNorm):
+    """``h = x + delta; return h, norm(h)``: one pass forward and one backward where the fused kernels apply."""
+    if FUSED_ADD_NORM and _fused(x) and norm.scale.dtype == torch.bfloat16 and x.shape[-1] % 8 == 0 and x.shape[-1] <= 8192:
+        return layer_ops.add_rms_norm(x, delta, norm)
+    h = x + delta
+    return h, norm(h)
+
+
 class DecoderLayer(nn.Module):
     def __init__(self, s: LlamaShape, rank: int, alpha: float, quantize_base: bool):
         super().__init__()
@@ -209,9 +220,14 @@ class DecoderLayer(nn.Module):
         self.mlp_norm = RMSNorm(s.dim, s.norm_eps)
         self.mlp = FeedForward(s, rank, alpha, quantize_base)
 
-    def forward(self, x: torch.Tensor, rope: torch.Tensor) -> torch.Tensor:
-        h = x + self.attn(self.sa_norm(x), rope)
-        return h + self.mlp(self.mlp_norm(h))
+    def forward(self, x: torch.Tensor, delta: Optional[torch.Tensor], rope: torch.Tensor):
+        """``x``: the residual stream before the previous layer's feed-forward output ``delta`` is added (``None`` for the
+        first layer).  Returns the stream after the attention sub-block and this layer's feed-forward output, not yet
+        added: every addition of the stream (``torchtune/modules/transformer.py:129-141``) is followed by an RMSNorm and
+        runs in that norm's pass (``_add_norm``)."""
+        h, n = (x, self.sa_norm(x)) if delta is None else _add_norm(x, delta, self.sa_norm)
+        h, n = _add_norm(h, self.attn(n, rope), self.mlp_norm)
+        return h, self.mlp(n)
 
 
 class Decoder(nn.Module):
@@ -240,12 +256,13 @@ class Decoder(nn.Module):
     def forward(self, tokens: torch.Tensor) -> torch.Tensor:
         rope = self._rope_cache(tokens.shape[1], tokens.device)
         h = self.tok_embeddings(tokens)
+        delta = None
         for layer in self.layers:
             if self.ac and torch.is_grad_enabled():
-                h = checkpoint(layer, h, rope, use_reentrant=False)
+                h, delta = checkpoint(layer, h, delta, rope, use_reentrant=False)
             else:
-                h = layer(h, rope)
-        return self.norm(h)
+                h, delta = layer(h, delta, rope)
+        return _add_norm(h, delta, self.norm)[1]
 
     def loss(self, tokens: torch.Tensor, labels: torch.Tensor) -> torch.Tensor:
         """Mean next-token cross entropy; the vocabulary projection is applied chunk by chunk over the sequence."""

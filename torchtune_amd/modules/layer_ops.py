@@ -28,6 +28,33 @@ class _RMSNormFn(torch.autograd.Function):
         return (gx.view(x.shape) if ctx.needs_input_grad[0] else None), gscale, None
 
 
+class _AddRMSNormFn(torch.autograd.Function):
+    """(x, residual, scale) -> (h = x + residual, RMSNorm(h)).  Backward: both inputs receive
+    ``grad h + grad of the norm's input``, summed in the norm's backward pass."""
+
+    @staticmethod
+    def forward(ctx, x, residual, scale, eps: float):
+        h, y, rstd = ops.add_rms_norm_fwd(x, residual, scale, eps)
+        ctx.save_for_backward(h, scale, rstd)
+        ctx.set_materialize_grads(False)  # an output nobody used arrives as None, not as a tensor of zeros
+        return h.view(x.shape), y.view(x.shape)
+
+    @staticmethod
+    def backward(ctx, gh, gy):
+        h, scale, rstd = ctx.saved_tensors
+        if gy is None:  # the normalised output went nowhere
+            return gh, gh, None, None
+        gx, gscale = ops.rms_norm_bwd(gy, h, scale, rstd, want_gscale=ctx.needs_input_grad[2], g_add=gh)
+        gx = gx.view(h.shape)
+        return (gx if ctx.needs_input_grad[0] else None), (gx if ctx.needs_input_grad[1] else None), gscale, None
+
+
+def add_rms_norm(x: torch.Tensor, residual: torch.Tensor, norm: "RMSNorm"):
+    """``h = x + residual; return h, norm(h)``: the residual stream's addition and the norm of the next sub-block
+    (``torchtune/modules/transformer.py:129-141``) as one pass forward and one backward; same bits as the separate ops."""
+    return _AddRMSNormFn.apply(x, residual, norm.scale, norm.eps)
+
+
 class RMSNorm(nn.Module):
     """Root-mean-square normalisation computed in fp32: ``bf16(x * rsqrt(mean(x^2) + eps)) * scale``.
 

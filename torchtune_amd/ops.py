@@ -980,8 +980,31 @@ def rms_norm_fwd(x: torch.Tensor, scale: torch.Tensor, eps: float):
     return y, rstd
 
 
-def rms_norm_bwd(gy: torch.Tensor, x: torch.Tensor, scale: torch.Tensor, rstd: torch.Tensor, want_gscale: bool):
-    """-> (gx like x, gscale [D] bf16 | None)"""
+def add_rms_norm_fwd(x: torch.Tensor, residual: torch.Tensor, scale: torch.Tensor, eps: float):
+    """-> (h = x + residual, y = RMSNorm(h), rstd): the addition of the residual stream and the norm that follows it in
+    one pass; the bits of ``x + residual`` followed by ``rms_norm_fwd``."""
+    xc = _bf16_any(x, "add_rms_norm_fwd: x")
+    rc_ = _bf16_any(residual, "add_rms_norm_fwd: residual")
+    sc = _bf16_any(scale, "add_rms_norm_fwd: scale")
+    if xc.shape != rc_.shape:
+        raise ValueError(f"add_rms_norm_fwd: x {tuple(xc.shape)} and residual {tuple(rc_.shape)} differ in shape")
+    D = xc.shape[-1]
+    rows = xc.numel() // D
+    h = torch.empty_like(xc)
+    y = torch.empty_like(xc)
+    rstd = torch.empty(rows, dtype=torch.float32, device=x.device)
+    lib = _lib.load()
+    with torch.cuda.device(x.device):
+        rc = lib.ttamd_add_rms_norm_fwd_bf16(xc.data_ptr(), rc_.data_ptr(), sc.data_ptr(), float(eps), h.data_ptr(), y.data_ptr(),
+                                             rstd.data_ptr(), rows, D, _stream(x))
+    _lib.check(rc, "add_rms_norm_fwd")
+    return h, y, rstd
+
+
+def rms_norm_bwd(gy: torch.Tensor, x: torch.Tensor, scale: torch.Tensor, rstd: torch.Tensor, want_gscale: bool,
+                 g_add: Optional[torch.Tensor] = None):
+    """-> (gx like x, gscale [D] bf16 | None); ``g_add`` (like x): a gradient that reaches x on another way, added to gx in
+    the same pass (``bf16(bf16(gx) + g_add)``)."""
     gc = _bf16_any(gy, "rms_norm_bwd: gy")
     xc = _bf16_any(x, "rms_norm_bwd: x")
     sc = _bf16_any(scale, "rms_norm_bwd: scale")
@@ -992,9 +1015,14 @@ def rms_norm_bwd(gy: torch.Tensor, x: torch.Tensor, scale: torch.Tensor, rstd: t
     gscale = torch.empty(D, dtype=torch.bfloat16, device=x.device) if want_gscale else None
     nbytes = lib.ttamd_rms_norm_bwd_workspace_bytes(D) if want_gscale else 0
     ws = _workspace(nbytes, x.device) if want_gscale else None
+    ga = None
+    if g_add is not None:
+        ga = _bf16_any(g_add, "rms_norm_bwd: g_add")
+        if ga.shape != xc.shape:
+            raise ValueError(f"rms_norm_bwd: g_add {tuple(ga.shape)} and x {tuple(xc.shape)} differ in shape")
     with torch.cuda.device(x.device):
-        rc = lib.ttamd_rms_norm_bwd_bf16(gc.data_ptr(), xc.data_ptr(), sc.data_ptr(), rstd.data_ptr(), gx.data_ptr(), _ptr(gscale),
-                                         rows, D, _ptr(ws), nbytes, _stream(x))
+        rc = lib.ttamd_rms_norm_bwd_add_bf16(gc.data_ptr(), xc.data_ptr(), sc.data_ptr(), rstd.data_ptr(), _ptr(ga), gx.data_ptr(),
+                                             _ptr(gscale), rows, D, _ptr(ws), nbytes, _stream(x))
     _lib.check(rc, "rms_norm_bwd")
     return gx, gscale
 
