@@ -35,37 +35,41 @@ __device__ __forceinline__ float wave_sum(float v) {
 }
 
 // ---------------------------------------------------------------------------------------------------
-// RMSNorm.  One wave per row, the row held in registers (NV 16-byte chunks per lane, chunk = lane + 64 i); the
-// backward with a scale gradient takes a workgroup per row (see rms_norm_bwd_gscale_kernel).
+// RMSNorm.  One workgroup per row, the row held in registers (NV 16-byte chunks per lane).
 //   forward : xn = bf16(x * rsqrt(mean(x^2) + eps));  y = bf16(xn * scale);  rstd saved for backward
 //   backward: g = bf16(gy * scale) (eager's bf16 product), c = mean(g * x) * rstd^2,
 //             gx = bf16(rstd * (g - x * c));  gscale partial[w][d] = sum over workgroup w's rows of gy * xn
 // ---------------------------------------------------------------------------------------------------
+// Forward: a workgroup per row (four waves, NV chunks of 8 columns per lane, chunk = thread + 256 i); the sums of squares
+// of the four waves meet in LDS in wave order.
 // ADD: the row normalised is h = bf16(x + res) (the residual stream's addition, torchtune/modules/transformer.py:129-141),
 // which the launch also writes to h_out; same bits as the addition and the norm one after the other.
 template <int NV, bool ADD>
 __global__ __launch_bounds__(256) void rms_norm_fwd_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ res,
                                                            const uint16_t* __restrict__ scale, float eps,
                                                            uint16_t* __restrict__ h_out, uint16_t* __restrict__ y,
-                                                           float* __restrict__ rstd_out, int64_t rows, int D) {
-  const int lane = threadIdx.x & 63;
-  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (row >= rows) return;
+                                                           float* __restrict__ rstd_out, int D) {
+  __shared__ float part[4];
+  const int t = threadIdx.x;
+  const int64_t row = blockIdx.x;
   const int chunks = D >> 3;
   const u32x4_t* xr = reinterpret_cast<const u32x4_t*>(x + row * D);
-  u32x4_t v[NV];
+  const u32x4_t* sr = reinterpret_cast<const u32x4_t*>(scale);
+  u32x4_t v[NV], sv[NV];
   float ss = 0.f;
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
-    const int c = lane + 64 * i;
+    const int c = t + 256 * i;
     v[i] = u32x4_t{0, 0, 0, 0};
+    sv[i] = u32x4_t{0, 0, 0, 0};
     if (c < chunks) {
-      v[i] = *(xr + c);
+      v[i] = __builtin_nontemporal_load(xr + c);
+      sv[i] = sr[c];
       if constexpr (ADD) {
-        const u32x4_t rv = *(reinterpret_cast<const u32x4_t*>(res + row * D) + c);
+        const u32x4_t rv = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(res + row * D) + c);
 #pragma unroll
         for (int d = 0; d < 4; ++d) v[i][d] = pack2(lo_f(v[i][d]) + lo_f(rv[d]), hi_f(v[i][d]) + hi_f(rv[d]));
-        __builtin_nontemporal_store(v[i], reinterpret_cast<u32x4_t*>(h_out + row * D) + c);
+        *(reinterpret_cast<u32x4_t*>(h_out + row * D) + c) = v[i];  // read again soon: by the next addition and the backward
       }
     }
 #pragma unroll
@@ -76,20 +80,21 @@ __global__ __launch_bounds__(256) void rms_norm_fwd_kernel(const uint16_t* __res
     }
   }
   ss = wave_sum(ss);
+  if ((t & 63) == 0) part[t >> 6] = ss;
+  __syncthreads();
+  ss = ((part[0] + part[1]) + part[2]) + part[3];
   const float rstd = __builtin_amdgcn_rsqf(ss / (float)D + eps);
-  if (lane == 0 && rstd_out) rstd_out[row] = rstd;
+  if (t == 0 && rstd_out) rstd_out[row] = rstd;
   u32x4_t* yr = reinterpret_cast<u32x4_t*>(y + row * D);
-  const u32x4_t* sr = reinterpret_cast<const u32x4_t*>(scale);
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
-    const int c = lane + 64 * i;
+    const int c = t + 256 * i;
     if (c >= chunks) continue;
-    const u32x4_t s = sr[c];
     u32x4_t o;
 #pragma unroll
     for (int d = 0; d < 4; ++d) {
       const float n0 = round_to_bf16(lo_f(v[i][d]) * rstd), n1 = round_to_bf16(hi_f(v[i][d]) * rstd);
-      o[d] = pack2(n0 * lo_f(s[d]), n1 * hi_f(s[d]));
+      o[d] = pack2(n0 * lo_f(sv[i][d]), n1 * hi_f(sv[i][d]));
     }
     __builtin_nontemporal_store(o, yr + c);
   }
@@ -312,13 +317,6 @@ __global__ __launch_bounds__(256) void swiglu_bwd_kernel(const uint16_t* go, con
   }
 }
 
-int nv_for(int64_t D) {
-  const int64_t chunks = D / 8;
-  int nv = 1;
-  while ((int64_t)nv * 64 < chunks) nv <<= 1;
-  return nv;
-}
-
 }  // namespace
 }  // namespace ttamd
 
@@ -329,26 +327,27 @@ int rms_norm_fwd(const char* who, const void* x, const void* res, const void* sc
                  int64_t rows, int64_t D, void* stream) {
   TT_REQUIRE(x && scale && y && (res == nullptr) == (h == nullptr), "%s: null pointer argument", who);
   TT_REQUIRE(aligned16(x) && aligned16(scale) && aligned16(y) && aligned16(res) && aligned16(h), "%s: pointers must be 16-byte aligned", who);
-  TT_REQUIRE(rows > 0 && D > 0 && D % 8 == 0 && D <= 8192 && rows < (int64_t(1) << 32),
+  TT_REQUIRE(rows > 0 && D > 0 && D % 8 == 0 && D <= 8192 && rows < (int64_t(1) << 31),
              "%s: bad shape rows=%lld D=%lld (D must be a multiple of 8, at most 8192)", who, (long long)rows, (long long)D);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
+  const dim3 grid((unsigned)rows), block(256);
   const uint16_t* X = reinterpret_cast<const uint16_t*>(x);
   const uint16_t* R = reinterpret_cast<const uint16_t*>(res);
   const uint16_t* S = reinterpret_cast<const uint16_t*>(scale);
   uint16_t* H = reinterpret_cast<uint16_t*>(h);
   uint16_t* Y = reinterpret_cast<uint16_t*>(y);
-#define TT_RMS_FWD(NVV)                                                                             \
-  if (res)                                                                                          \
-    rms_norm_fwd_kernel<NVV, true><<<grid, block, 0, s>>>(X, R, S, eps, H, Y, rstd, rows, (int)D);  \
-  else                                                                                              \
-    rms_norm_fwd_kernel<NVV, false><<<grid, block, 0, s>>>(X, nullptr, S, eps, nullptr, Y, rstd, rows, (int)D);
-  switch (nv_for(D)) {
-    case 1: TT_RMS_FWD(1) break;
-    case 2: TT_RMS_FWD(2) break;
-    case 4: TT_RMS_FWD(4) break;
-    case 8: TT_RMS_FWD(8) break;
-    default: TT_RMS_FWD(16) break;
+#define TT_RMS_FWD(NVV)                                                                       \
+  if (res)                                                                                    \
+    rms_norm_fwd_kernel<NVV, true><<<grid, block, 0, s>>>(X, R, S, eps, H, Y, rstd, (int)D);  \
+  else                                                                                        \
+    rms_norm_fwd_kernel<NVV, false><<<grid, block, 0, s>>>(X, nullptr, S, eps, nullptr, Y, rstd, (int)D);
+  const int64_t nv = (D / 8 + 255) / 256;  // D <= 8192: at most 4
+  if (nv <= 1) {
+    TT_RMS_FWD(1)
+  } else if (nv <= 2) {
+    TT_RMS_FWD(2)
+  } else {
+    TT_RMS_FWD(4)
   }
 #undef TT_RMS_FWD
   return check_launch(who);
