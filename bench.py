@@ -531,6 +531,8 @@ def main() -> int:
                          "instead of a pass of its own (QLoRA workloads)")
     ap.add_argument("--no-qat-tn-group", action="store_true",
                     help="A/B (QAT workloads): one weight-gradient launch per member of a group instead of one for the group")
+    ap.add_argument("--no-fused-qkv-post", action="store_true",
+                    help="rotary embedding and key / value head expansion as four launches per layer and direction instead of one")
     ap.add_argument("--no-fused-add-norm", action="store_true",
                     help="A/B: the additions of the residual stream as passes of their own instead of inside the RMSNorm that "
                          "follows each of them")
@@ -565,6 +567,7 @@ def main() -> int:
     harness.GROUP_SHARED_INPUT = not args.no_group
     harness.GATED_EPILOGUE = not args.no_gated_epilogue
     harness.FUSED_ADD_NORM = not args.no_fused_add_norm
+    harness.FUSED_QKV_POST = not args.no_fused_qkv_post
     harness.SWIGLU_BWD_EPILOGUE = args.swiglu_bwd_epilogue
     ops.EXPANDED_WEIGHT_PATH = not args.no_expanded_weight
     if args.no_qat_tiled_gemm:

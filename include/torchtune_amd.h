@@ -592,6 +592,20 @@ int ttamd_repeat_kv_bwd_bf16(const void* gy, void* gx, int64_t tokens, int64_t n
                              void* stream);
 
 /*
+ * Everything between the q / k / v projections and the attention in one launch
+ * (torchtune/modules/attention.py:255-290: the rotary embedding of q and k, then the expansion of the k / v heads):
+ * q_out = rope(q), k_out = repeat(rope(k)), v_out = repeat(v) with q, q_out, k_out, v_out [B, S, n_heads, head_dim] and
+ * k, v [B, S, n_kv, head_dim], rep = n_heads / n_kv (1: k_out = rope(k), v_out = v).  The backward takes the gradients of
+ * the three outputs and writes those of q, k, v.  Both give the bits of ttamd_rope_bf16 and ttamd_repeat_kv(_bwd)_bf16
+ * called one after the other.  n_heads a multiple of n_kv, head_dim a multiple of 8.
+ */
+int ttamd_qkv_rope_repeat_bf16(const void* q, const void* k, const void* v, const float* cache, void* q_out, void* k_out,
+                               void* v_out, int64_t B, int64_t S, int64_t n_heads, int64_t n_kv, int64_t head_dim, void* stream);
+int ttamd_qkv_rope_repeat_bwd_bf16(const void* gq_out, const void* gk_out, const void* gv_out, const float* cache, void* gq,
+                                   void* gk, void* gv, int64_t B, int64_t S, int64_t n_heads, int64_t n_kv, int64_t head_dim,
+                                   void* stream);
+
+/*
  * FeedForward gate (torchtune/modules/feed_forward.py:50-53): out = bf16( bf16(silu(gate)) * up ), and its backward
  * ggate, gup from gout.  All [numel] bf16, numel a multiple of 8.
  */

@@ -64,6 +64,23 @@ def test_residual_additions_inside_the_norm_pass_give_the_same_step(monkeypatch,
         assert torch.equal(gr, out[1][1][n]), n
 
 
+def test_one_launch_for_rope_and_head_expansion_gives_the_same_step(monkeypatch):
+    """``harness.FUSED_QKV_POST``: the rotary embedding of q and k and the expansion of the key / value heads as one launch
+    per direction against the four launches they replace: the same loss and adapter gradients, bit for bit."""
+    tokens = torch.randint(0, 1024, (2, 160), device=DEV, generator=torch.Generator(device=DEV).manual_seed(6))
+    out = []
+    for fused in (True, False):
+        monkeypatch.setattr(harness, "FUSED_QKV_POST", fused)
+        model = harness.build_qlora_decoder("tiny", rank=8, alpha=16.0, device=DEV, seed=0)
+        assert model.layers[0].attn.n_kv != model.layers[0].attn.n_heads
+        loss = harness.train_step(model, tokens, tokens)
+        out.append((loss, {n: p.grad.clone() for n, p in model.named_parameters() if p.grad is not None}))
+    assert torch.equal(out[0][0], out[1][0])
+    assert set(out[0][1]) == set(out[1][1]) and out[0][1]
+    for n, gr in out[0][1].items():
+        assert torch.equal(gr, out[1][1][n]), n
+
+
 def test_tiny_qat_decoder_step():
     model = harness.build_qat_decoder("tiny", groupsize=32, device=DEV, seed=0)
     tokens = torch.randint(0, 1024, (2, 64), device=DEV, generator=torch.Generator(device=DEV).manual_seed(3))

@@ -240,3 +240,38 @@ def test_repeat_kv_forward_backward(b, s, nkv, rep, hd):
         ops.repeat_kv(x.detach()[0], rep)
     with pytest.raises(ValueError):
         ops.repeat_kv_bwd(gy, rep + 1 if (nkv * rep) % (rep + 1) else rep * nkv * 2 + 1)
+
+
+@pytest.mark.parametrize("b,s,nh,nkv,hd", [(2, 33, 8, 2, 128), (1, 7, 6, 2, 64), (3, 5, 8, 1, 8), (1, 4, 4, 4, 16), (2, 256, 32, 8, 128)])
+def test_qkv_rope_repeat_equals_rope_then_repeat_bitwise(b, s, nh, nkv, hd):
+    """``qkv_rope_repeat`` against ``apply_rope`` on q and k followed by ``repeat_kv`` on k and v: the three outputs and the
+    gradients of q, k, v bit for bit (also with one key / value head per query head, where the expansion is a copy)."""
+    g = torch.Generator().manual_seed(11)
+    q0 = torch.randn(b, s, nh, hd, generator=g).to(BF).to(DEV)
+    k0, v0 = (torch.randn(b, s, nkv, hd, generator=g).to(BF).to(DEV) for _ in range(2))
+    gos = [torch.randn(b, s, nh, hd, generator=g).to(BF).to(DEV) for _ in range(3)]
+    pos = torch.arange(s, dtype=torch.float32)
+    theta = 1.0 / (10000.0 ** (torch.arange(0, hd, 2, dtype=torch.float32) / hd))
+    ang = torch.outer(pos, theta)
+    cache = torch.stack([ang.cos(), ang.sin()], dim=-1).to(DEV)
+    rep = nh // nkv
+    res = []
+    for fused in (True, False):
+        q, k, v = (t.clone().requires_grad_() for t in (q0, k0, v0))
+        if fused:
+            outs = layer_ops.qkv_rope_repeat(q, k, v, cache)
+        else:
+            outs = (layer_ops.apply_rope(q, cache), layer_ops.repeat_kv(layer_ops.apply_rope(k, cache), rep),
+                    layer_ops.repeat_kv(v, rep))
+        torch.autograd.backward(outs, gos)
+        res.append([*outs, q.grad, k.grad, v.grad])
+    for i, (x, y) in enumerate(zip(*res)):
+        assert x.shape == y.shape and torch.equal(x, y), i
+
+
+def test_qkv_rope_repeat_refuses_heads_that_do_not_divide():
+    q = torch.zeros(1, 4, 6, 16, dtype=BF, device=DEV)
+    k = torch.zeros(1, 4, 4, 16, dtype=BF, device=DEV)
+    cache = torch.zeros(4, 8, 2, device=DEV)
+    with pytest.raises(ValueError, match="heads"):
+        ops.qkv_rope_repeat(q, k, k, cache)

@@ -151,6 +151,8 @@ SIGNATURES = {
     "ttamd_rope_bf16": (_int, [_c_void_p, _c_void_p, _c_void_p, _i64, _i64, _i64, _i64, _int, _c_void_p]),
     "ttamd_repeat_kv_bf16": (_int, [_c_void_p, _c_void_p, _i64, _i64, _i64, _i64, _c_void_p]),
     "ttamd_repeat_kv_bwd_bf16": (_int, [_c_void_p, _c_void_p, _i64, _i64, _i64, _i64, _c_void_p]),
+    "ttamd_qkv_rope_repeat_bf16": (_int, [_c_void_p] * 7 + [_i64] * 5 + [_c_void_p]),
+    "ttamd_qkv_rope_repeat_bwd_bf16": (_int, [_c_void_p] * 7 + [_i64] * 5 + [_c_void_p]),
     "ttamd_swiglu_fwd_bf16": (_int, [_c_void_p, _c_void_p, _c_void_p, _i64, _c_void_p]),
     "ttamd_cross_entropy_fwd_bwd_bf16": (_int, [_c_void_p, _c_void_p, _i64, _f32, _c_void_p, _c_void_p, _i64, _i64, _c_void_p]),
     "ttamd_swiglu_bwd_bf16": (_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _i64, _c_void_p]),

@@ -243,15 +243,8 @@ static_assert(kRmsBwdGrid <= kRmsBwdWgs * 4, "one partial row per workgroup");
 // Rotary embedding on [b, s, n_h, h_d] with a [s, h_d/2, 2] fp32 (cos, sin) table; `inverse` rotates by -theta,
 // which is the backward pass (the map is orthogonal).  One lane = 8 elements = 4 pairs.
 // ---------------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void rope_kernel(const uint16_t* __restrict__ x, const float* __restrict__ cache,
-                                                   uint16_t* __restrict__ y, int64_t n_chunks, int S, int row_elems, int h_d,
-                                                   int inverse) {
-  const int64_t chunk = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (chunk >= n_chunks) return;
-  const int64_t e = chunk * 8;
-  const int pos = (int)((e / row_elems) % S);
-  const int d = (int)(e % h_d);  // even; h_d % 8 == 0 keeps the 4 pairs inside one head
-  const u32x4_t v = *(reinterpret_cast<const u32x4_t*>(x) + chunk);
+// four pairs of one head at position pos, starting at element d of the head
+__device__ __forceinline__ u32x4_t rope_rotate(u32x4_t v, const float* __restrict__ cache, int pos, int d, int h_d, int inverse) {
   const f32x4_t* cp = reinterpret_cast<const f32x4_t*>(cache + ((int64_t)pos * (h_d >> 1) + (d >> 1)) * 2);
   const f32x4_t c01 = cp[0], c23 = cp[1];
   const float cs[4] = {c01.x, c01.z, c23.x, c23.z};
@@ -263,7 +256,19 @@ __global__ __launch_bounds__(256) void rope_kernel(const uint16_t* __restrict__ 
     const float s = inverse ? -sn[p] : sn[p];
     o[p] = pack2(a * cs[p] - b * s, b * cs[p] + a * s);
   }
-  __builtin_nontemporal_store(o, reinterpret_cast<u32x4_t*>(y) + chunk);
+  return o;
+}
+
+__global__ __launch_bounds__(256) void rope_kernel(const uint16_t* __restrict__ x, const float* __restrict__ cache,
+                                                   uint16_t* __restrict__ y, int64_t n_chunks, int S, int row_elems, int h_d,
+                                                   int inverse) {
+  const int64_t chunk = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (chunk >= n_chunks) return;
+  const int64_t e = chunk * 8;
+  const int pos = (int)((e / row_elems) % S);
+  const int d = (int)(e % h_d);  // even; h_d % 8 == 0 keeps the 4 pairs inside one head
+  const u32x4_t v = *(reinterpret_cast<const u32x4_t*>(x) + chunk);
+  __builtin_nontemporal_store(rope_rotate(v, cache, pos, d, h_d, inverse), reinterpret_cast<u32x4_t*>(y) + chunk);
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -451,13 +456,9 @@ __global__ __launch_bounds__(256) void repeat_kv_kernel(const u32x4_t* __restric
   y[oc] = x[(tok * n_kv + kv) * chunks_per_head + c];
 }
 
-// Its backward: gx[t][kv][:] = bf16(sum_r gy[t][kv * rep + r][:]), fp32 sums in the order r = 0 .. rep - 1.
-__global__ __launch_bounds__(256) void repeat_kv_bwd_kernel(const u32x4_t* __restrict__ gy, u32x4_t* __restrict__ gx, int64_t n_in,
-                                                            int chunks_per_head, int rep) {
-  const int64_t ic = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (ic >= n_in) return;
-  const int64_t in_head = ic / chunks_per_head;
-  const int c = (int)(ic - in_head * chunks_per_head);
+// bf16(sum_r gy[in_head * rep + r][c]), fp32 sums in the order r = 0 .. rep - 1
+__device__ __forceinline__ u32x4_t sum_head_copies(const u32x4_t* __restrict__ gy, int64_t in_head, int c, int chunks_per_head,
+                                                   int rep) {
   float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   for (int r = 0; r < rep; ++r) {
     const u32x4_t v = gy[(in_head * rep + r) * chunks_per_head + c];
@@ -470,7 +471,78 @@ __global__ __launch_bounds__(256) void repeat_kv_bwd_kernel(const u32x4_t* __res
   u32x4_t o;
 #pragma unroll
   for (int d = 0; d < 4; ++d) o[d] = (uint32_t)f32_to_bf16_bits(acc[2 * d]) | ((uint32_t)f32_to_bf16_bits(acc[2 * d + 1]) << 16);
-  gx[ic] = o;
+  return o;
+}
+
+// Its backward: gx[t][kv][:] = bf16(sum_r gy[t][kv * rep + r][:]).
+__global__ __launch_bounds__(256) void repeat_kv_bwd_kernel(const u32x4_t* __restrict__ gy, u32x4_t* __restrict__ gx, int64_t n_in,
+                                                            int chunks_per_head, int rep) {
+  const int64_t ic = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (ic >= n_in) return;
+  const int64_t in_head = ic / chunks_per_head;
+  const int c = (int)(ic - in_head * chunks_per_head);
+  gx[ic] = sum_head_copies(gy, in_head, c, chunks_per_head, rep);
+}
+
+// Everything between the q / k / v projections and the attention in one launch
+// (torchtune/modules/attention.py:255-290: rotary embedding of q and k, expansion of the k / v heads):
+// q_out = rope(q), k_out = repeat(rope(k)), v_out = repeat(v).  One thread per 16-byte chunk of the three outputs
+// (nq chunks each); the same bits as rope_kernel followed by repeat_kv_kernel.
+__global__ __launch_bounds__(256) void qkv_rope_repeat_kernel(const u32x4_t* __restrict__ q, const u32x4_t* __restrict__ k,
+                                                              const u32x4_t* __restrict__ v, const float* __restrict__ cache,
+                                                              u32x4_t* __restrict__ qo, u32x4_t* __restrict__ ko,
+                                                              u32x4_t* __restrict__ vo, int64_t nq, int S, int n_heads, int n_kv,
+                                                              int chunks_per_head) {
+  const int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (g >= 3 * nq) return;
+  const int seg = (int)(g / nq);
+  const int64_t oc = g - seg * nq;
+  const int64_t out_head = oc / chunks_per_head;  // token * n_heads + head
+  const int c = (int)(oc - out_head * chunks_per_head);
+  const int64_t tok = out_head / n_heads;
+  const int pos = (int)(tok % S);
+  const int h_d = chunks_per_head * 8;
+  if (seg == 0) {
+    __builtin_nontemporal_store(rope_rotate(__builtin_nontemporal_load(q + oc), cache, pos, c * 8, h_d, 0), qo + oc);
+    return;
+  }
+  const int rep = n_heads / n_kv;
+  const int kv = (int)(out_head - tok * n_heads) / rep;
+  const int64_t src = (tok * n_kv + kv) * chunks_per_head + c;
+  if (seg == 1)
+    __builtin_nontemporal_store(rope_rotate(k[src], cache, pos, c * 8, h_d, 0), ko + oc);
+  else
+    __builtin_nontemporal_store(v[src], vo + oc);
+}
+
+// Its backward: gq = rope^-1(gq_out), gk = rope^-1(bf16(sum of the copies' gradients)), gv = bf16(sum of the copies'
+// gradients); the same bits as repeat_kv_bwd_kernel followed by rope_kernel with inverse = 1.  The k / v threads (rep
+// reads each) come first.
+__global__ __launch_bounds__(256) void qkv_rope_repeat_bwd_kernel(const u32x4_t* __restrict__ gqo, const u32x4_t* __restrict__ gko,
+                                                                  const u32x4_t* __restrict__ gvo, const float* __restrict__ cache,
+                                                                  u32x4_t* __restrict__ gq, u32x4_t* __restrict__ gk,
+                                                                  u32x4_t* __restrict__ gv, int64_t nq, int64_t nkv, int S,
+                                                                  int n_heads, int n_kv, int chunks_per_head) {
+  const int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (g >= 2 * nkv + nq) return;
+  const int h_d = chunks_per_head * 8;
+  if (g >= 2 * nkv) {
+    const int64_t oc = g - 2 * nkv;
+    const int64_t head = oc / chunks_per_head;
+    const int c = (int)(oc - head * chunks_per_head);
+    const int pos = (int)((head / n_heads) % S);
+    __builtin_nontemporal_store(rope_rotate(__builtin_nontemporal_load(gqo + oc), cache, pos, c * 8, h_d, 1), gq + oc);
+    return;
+  }
+  const bool is_k = g < nkv;
+  const int64_t ic = is_k ? g : g - nkv;
+  const int64_t in_head = ic / chunks_per_head;  // token * n_kv + kv
+  const int c = (int)(ic - in_head * chunks_per_head);
+  const u32x4_t sum = sum_head_copies(is_k ? gko : gvo, in_head, c, chunks_per_head, n_heads / n_kv);
+  if (is_k)
+    __builtin_nontemporal_store(rope_rotate(sum, cache, (int)((in_head / n_kv) % S), c * 8, h_d, 1), gk + ic);
+  else
+    __builtin_nontemporal_store(sum, gv + ic);
 }
 
 int check_repeat_kv(const char* who, const void* a, const void* b, int64_t tokens, int64_t n_kv, int64_t rep, int64_t head_dim) {
@@ -503,6 +575,49 @@ extern "C" int ttamd_repeat_kv_bwd_bf16(const void* gy, void* gx, int64_t tokens
   repeat_kv_bwd_kernel<<<dim3((unsigned)((n_in + 255) / 256)), dim3(256), 0, reinterpret_cast<hipStream_t>(stream)>>>(
       reinterpret_cast<const u32x4_t*>(gy), reinterpret_cast<u32x4_t*>(gx), n_in, (int)(head_dim / 8), (int)rep);
   return check_launch("repeat_kv_bwd");
+}
+
+namespace {
+int check_qkv_rope_repeat(const char* who, const void* const* ptrs, const float* cache, int64_t B, int64_t S, int64_t n_heads,
+                          int64_t n_kv, int64_t head_dim) {
+  for (int i = 0; i < 6; ++i) {
+    TT_REQUIRE(ptrs[i], "%s: null pointer argument", who);
+    TT_REQUIRE(aligned16(ptrs[i]), "%s: pointers must be 16-byte aligned", who);
+  }
+  TT_REQUIRE(cache && aligned16(cache), "%s: the cache must be a 16-byte aligned pointer", who);
+  TT_REQUIRE(B > 0 && S > 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0 && head_dim > 0 && head_dim % 8 == 0 &&
+                 S < (1 << 30) && n_heads < (1 << 20) && head_dim < (1 << 20),
+             "%s: bad shape b=%lld s=%lld n_h=%lld n_kv=%lld h_d=%lld (n_h a multiple of n_kv, h_d a multiple of 8)", who,
+             (long long)B, (long long)S, (long long)n_heads, (long long)n_kv, (long long)head_dim);
+  TT_REQUIRE((3 * B * S * n_heads * (head_dim / 8) + 255) / 256 < (int64_t(1) << 31), "%s: tensors too large for one launch", who);
+  return TTAMD_OK;
+}
+}  // namespace
+
+extern "C" int ttamd_qkv_rope_repeat_bf16(const void* q, const void* k, const void* v, const float* cache, void* q_out,
+                                          void* k_out, void* v_out, int64_t B, int64_t S, int64_t n_heads, int64_t n_kv,
+                                          int64_t head_dim, void* stream) {
+  const void* ptrs[6] = {q, k, v, q_out, k_out, v_out};
+  if (int rc = check_qkv_rope_repeat("qkv_rope_repeat", ptrs, cache, B, S, n_heads, n_kv, head_dim)) return rc;
+  const int64_t nq = B * S * n_heads * (head_dim / 8);
+  qkv_rope_repeat_kernel<<<dim3((unsigned)((3 * nq + 255) / 256)), dim3(256), 0, reinterpret_cast<hipStream_t>(stream)>>>(
+      reinterpret_cast<const u32x4_t*>(q), reinterpret_cast<const u32x4_t*>(k), reinterpret_cast<const u32x4_t*>(v), cache,
+      reinterpret_cast<u32x4_t*>(q_out), reinterpret_cast<u32x4_t*>(k_out), reinterpret_cast<u32x4_t*>(v_out), nq, (int)S,
+      (int)n_heads, (int)n_kv, (int)(head_dim / 8));
+  return check_launch("qkv_rope_repeat");
+}
+
+extern "C" int ttamd_qkv_rope_repeat_bwd_bf16(const void* gq_out, const void* gk_out, const void* gv_out, const float* cache,
+                                              void* gq, void* gk, void* gv, int64_t B, int64_t S, int64_t n_heads, int64_t n_kv,
+                                              int64_t head_dim, void* stream) {
+  const void* ptrs[6] = {gq_out, gk_out, gv_out, gq, gk, gv};
+  if (int rc = check_qkv_rope_repeat("qkv_rope_repeat_bwd", ptrs, cache, B, S, n_heads, n_kv, head_dim)) return rc;
+  const int64_t nq = B * S * n_heads * (head_dim / 8), nkv = B * S * n_kv * (head_dim / 8);
+  qkv_rope_repeat_bwd_kernel<<<dim3((unsigned)((2 * nkv + nq + 255) / 256)), dim3(256), 0, reinterpret_cast<hipStream_t>(stream)>>>(
+      reinterpret_cast<const u32x4_t*>(gq_out), reinterpret_cast<const u32x4_t*>(gk_out),
+      reinterpret_cast<const u32x4_t*>(gv_out), cache, reinterpret_cast<u32x4_t*>(gq), reinterpret_cast<u32x4_t*>(gk),
+      reinterpret_cast<u32x4_t*>(gv), nq, nkv, (int)S, (int)n_heads, (int)n_kv, (int)(head_dim / 8));
+  return check_launch("qkv_rope_repeat_bwd");
 }
 
 extern "C" int ttamd_swiglu_fwd_bf16(const void* gate, const void* up, void* out, int64_t numel, void* stream) {

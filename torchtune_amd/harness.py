@@ -82,6 +82,9 @@ SHAPES = {
 # True: the additions of the residual stream run inside the RMSNorm pass that follows each of them, forward and backward
 # (same bits; one write and one read of the stream less per addition)
 FUSED_ADD_NORM = True
+# True: the rotary embedding of q and k and the grouped-query expansion of k and v run as one launch per direction
+# (same bits; four launches and the intermediate rotated k less per layer and direction)
+FUSED_QKV_POST = True
 # True: RMSNorm, RoPE and the SwiGLU gate run as single-pass HIP kernels (bf16 on the GPU); False: the eager op chains
 # of the reference.  The quantized linears are unaffected.
 FUSED_LAYER_OPS = True
@@ -167,6 +170,11 @@ class Attention(nn.Module):
         q = q.view(b, sl, self.n_heads, self.head_dim)
         k = k.view(b, sl, self.n_kv, self.head_dim)
         v = v.view(b, sl, self.n_kv, self.head_dim)
+        if FUSED_QKV_POST and self.n_kv != self.n_heads and _fused(q) and self.head_dim % 8 == 0:
+            # rotary embedding of q and k and the expansion of the k / v heads: one launch per direction
+            q, k, v = layer_ops.qkv_rope_repeat(q, k, v, rope)
+            o = _sdpa(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2))
+            return self.output_proj(o.transpose(1, 2).reshape(b, sl, -1))
         q = apply_rope(q, rope)
         k = apply_rope(k, rope)
         if self.n_kv != self.n_heads:  # expand kv heads to query heads, as the reference does before SDPA

@@ -90,6 +90,26 @@ def apply_rope(x: torch.Tensor, cache: torch.Tensor) -> torch.Tensor:
     return _RopeFn.apply(x, cache)
 
 
+class _QKVRopeRepeatFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q, k, v, cache):
+        ctx.save_for_backward(cache)
+        ctx.n_kv = k.shape[2]
+        return ops.qkv_rope_repeat(q, k, v, cache)
+
+    @staticmethod
+    def backward(ctx, gq, gk, gv):
+        (cache,) = ctx.saved_tensors
+        return (*ops.qkv_rope_repeat_bwd(gq, gk, gv, cache, ctx.n_kv), None)
+
+
+def qkv_rope_repeat(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cache: torch.Tensor):
+    """What lies between the q / k / v projections and the attention (``torchtune/modules/attention.py:255-290``) as one
+    kernel per direction: ``apply_rope(q)``, ``repeat_kv(apply_rope(k), rep)``, ``repeat_kv(v, rep)`` with
+    ``rep = n_h // n_kv``, bit for bit."""
+    return _QKVRopeRepeatFn.apply(q, k, v, cache)
+
+
 class _RepeatKVFn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, rep: int):

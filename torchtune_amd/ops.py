@@ -1073,6 +1073,55 @@ def repeat_kv_bwd(gy: torch.Tensor, rep: int) -> torch.Tensor:
     return gx
 
 
+def _rope_cache_arg(cache: torch.Tensor, s: int, hd: int, who: str) -> torch.Tensor:
+    _need_gpu(cache, f"{who}: cache")
+    if cache.dtype != torch.float32 or cache.numel() < s * hd or cache.shape[-1] != 2 or cache.shape[-2] != hd // 2:
+        raise ValueError(f"{who}: cache must be fp32 [>= {s}, {hd // 2}, 2], got {tuple(cache.shape)} {cache.dtype}")
+    return cache.contiguous()
+
+
+def _qkv_shapes(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, n_kv: Optional[int], who: str):
+    if q.dim() != 4 or k.dim() != 4 or v.shape != k.shape or q.shape[:2] != k.shape[:2] or q.shape[3] != k.shape[3]:
+        raise ValueError(f"{who}: expected [b, s, n_h, h_d] and two [b, s, n_kv, h_d], got {tuple(q.shape)}, {tuple(k.shape)}, {tuple(v.shape)}")
+    b, s, nh, hd = q.shape
+    nkv = k.shape[2] if n_kv is None else n_kv
+    if nkv < 1 or nh % nkv or (n_kv is not None and k.shape[2] != nh):
+        raise ValueError(f"{who}: {nh} query heads against {nkv} key / value heads (tensors {tuple(q.shape)}, {tuple(k.shape)})")
+    return b, s, nh, nkv, hd
+
+
+def qkv_rope_repeat(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cache: torch.Tensor):
+    """``rope(q)``, ``repeat_kv(rope(k), n_h // n_kv)``, ``repeat_kv(v, n_h // n_kv)`` from one launch; q ``[b, s, n_h, h_d]``,
+    k and v ``[b, s, n_kv, h_d]`` bf16, cache ``[s, h_d/2, 2]`` fp32.  The bits of :func:`rope` and :func:`repeat_kv`."""
+    qc, kc, vc = _bf16_any(q, "qkv_rope_repeat: q"), _bf16_any(k, "qkv_rope_repeat: k"), _bf16_any(v, "qkv_rope_repeat: v")
+    b, s, nh, nkv, hd = _qkv_shapes(qc, kc, vc, None, "qkv_rope_repeat")
+    cc = _rope_cache_arg(cache, s, hd, "qkv_rope_repeat")
+    qo, ko, vo = torch.empty_like(qc), torch.empty_like(qc), torch.empty_like(qc)
+    lib = _lib.load()
+    with torch.cuda.device(q.device):
+        rc = lib.ttamd_qkv_rope_repeat_bf16(qc.data_ptr(), kc.data_ptr(), vc.data_ptr(), cc.data_ptr(), qo.data_ptr(),
+                                            ko.data_ptr(), vo.data_ptr(), b, s, nh, nkv, hd, _stream(q))
+    _lib.check(rc, "qkv_rope_repeat")
+    return qo, ko, vo
+
+
+def qkv_rope_repeat_bwd(gq_out: torch.Tensor, gk_out: torch.Tensor, gv_out: torch.Tensor, cache: torch.Tensor, n_kv: int):
+    """The gradients of q, k, v of :func:`qkv_rope_repeat` from those of its three outputs (each ``[b, s, n_h, h_d]``)."""
+    a, bb, c = (_bf16_any(gq_out, "qkv_rope_repeat_bwd: gq"), _bf16_any(gk_out, "qkv_rope_repeat_bwd: gk"),
+                _bf16_any(gv_out, "qkv_rope_repeat_bwd: gv"))
+    b, s, nh, nkv, hd = _qkv_shapes(a, bb, c, n_kv, "qkv_rope_repeat_bwd")
+    cc = _rope_cache_arg(cache, s, hd, "qkv_rope_repeat_bwd")
+    gq = torch.empty_like(a)
+    gk = torch.empty(b, s, nkv, hd, dtype=torch.bfloat16, device=a.device)
+    gv = torch.empty_like(gk)
+    lib = _lib.load()
+    with torch.cuda.device(a.device):
+        rc = lib.ttamd_qkv_rope_repeat_bwd_bf16(a.data_ptr(), bb.data_ptr(), c.data_ptr(), cc.data_ptr(), gq.data_ptr(),
+                                                gk.data_ptr(), gv.data_ptr(), b, s, nh, nkv, hd, _stream(a))
+    _lib.check(rc, "qkv_rope_repeat_bwd")
+    return gq, gk, gv
+
+
 def swiglu_fwd(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     g = _bf16_any(gate, "swiglu_fwd: gate")
     u = _bf16_any(up, "swiglu_fwd: up")
