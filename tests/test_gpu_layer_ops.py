@@ -242,7 +242,8 @@ def test_repeat_kv_forward_backward(b, s, nkv, rep, hd):
         ops.repeat_kv_bwd(gy, rep + 1 if (nkv * rep) % (rep + 1) else rep * nkv * 2 + 1)
 
 
-@pytest.mark.parametrize("b,s,nh,nkv,hd", [(2, 33, 8, 2, 128), (1, 7, 6, 2, 64), (3, 5, 8, 1, 8), (1, 4, 4, 4, 16), (2, 256, 32, 8, 128)])
+@pytest.mark.parametrize("b,s,nh,nkv,hd", [(2, 33, 8, 2, 128), (1, 7, 6, 2, 64), (3, 5, 8, 1, 8), (1, 4, 4, 4, 16), (2, 256, 32, 8, 128),
+                                            (4, 2048, 32, 8, 128), (1, 4096, 64, 8, 128), (4, 2048, 32, 8, 64)])
 def test_qkv_rope_repeat_equals_rope_then_repeat_bitwise(b, s, nh, nkv, hd):
     """``qkv_rope_repeat`` against ``apply_rope`` on q and k followed by ``repeat_kv`` on k and v: the three outputs and the
     gradients of q, k, v bit for bit (also with one key / value head per query head, where the expansion is a copy)."""
