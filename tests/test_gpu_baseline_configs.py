@@ -115,8 +115,9 @@ def test_projection_at_full_size(name, N, K, M, r, alpha):
     del ref_gx, Df
     ref_ga = gh.T @ xf
     ref_gb = s * (gyf.T @ h)
+    # one bf16 rounding of an fp32-accumulated result, the bound the small cases of test_gpu_lora_linear.py hold
     for got, want in ((layer.lora_a.weight.grad, ref_ga), (layer.lora_b.weight.grad, ref_gb)):
-        torch.testing.assert_close(got.float(), want, rtol=2e-2, atol=2e-2 * float(want.abs().max()))
+        torch.testing.assert_close(got.float(), want, rtol=4e-3, atol=4e-3 * float(want.abs().max()))
 
     # ---- the oracle's own unfused bf16 forward on the last 64 output columns and the first 256 tokens
     r0 = N - 64
