@@ -144,8 +144,13 @@ int ttamd_lora_hidden_bf16(const void* x, const void* lora_a, void* h, int64_t M
  * than the built-in array (the plan of this build never does for rank <= 64).  All calls on one GPU share that
  * array: calls that overlap on the same GPU (different streams or threads) race on it and must be serialised by the
  * caller; calls on different GPUs are independent.  Nothing in the array has to start at zero.
+ * The first use on a device asks the runtime for the array's device address (hipGetSymbolAddress, possibly a lazy
+ * load of the code object): that query must not fall inside a stream capture.  Call ttamd_lora_hidden_static_init()
+ * once per device, with that device current, before capturing (one eager call of the entry point does the same);
+ * later calls only launch kernels.  Returns TTAMD_ELAUNCH if the runtime refuses the query.
  */
 size_t ttamd_lora_hidden_static_max_bytes(void);
+int ttamd_lora_hidden_static_init(void);
 int ttamd_lora_hidden_static_bf16(const void* x, const void* lora_a, void* h, int64_t M, int64_t K, int rank, void* stream);
 
 /*
@@ -284,6 +289,30 @@ size_t ttamd_lora_bwd_workspace_bytes(int64_t M, int64_t N, int64_t K, int rank)
 int ttamd_lora_bwd_bf16(const void* gy, const void* x, const void* h, const void* lora_b, float scale, void* gh, void* ga,
                         void* gb, int64_t M, int64_t N, int64_t K, int rank, void* workspace, size_t workspace_bytes,
                         void* stream);
+
+/*
+ * The whole layer in one call per direction: LoRALinear.forward (torchtune/modules/peft/lora.py:128-147; one Python
+ * call of the module is the reference's unit) and the backward autograd derives for it.
+ *   ttamd_qlora_linear_fwd_bf16 = ttamd_lora_hidden_bf16 -> ttamd_nf4_lora_linear_fwd_ws_bf16:
+ *       h = bf16(x . lora_a^T)   [M,rank], written for the backward (lora.py:144)
+ *       y = x . D(W)^T (+ bias) + scale . h . lora_b^T   [M,N]   (lora.py:137-147)
+ *   ttamd_qlora_linear_bwd_bf16 = ttamd_lora_bwd_bf16 -> ttamd_nf4_linear_bwd_dx_ws_bf16:
+ *       grad_lora_a [rank,K], grad_lora_b [N,rank], and gx = gy . D(W) + gh . lora_a [M,K] unless gx is NULL (the layer's
+ *       input needs no gradient); gh = scale . gy . lora_b lives in the workspace.
+ * The launches, their order and therefore every result bit are those of the two-call sequences, including the dispatch
+ * by size (few tokens, slices of the contraction, the weight expanded once per call).  One workspace per call, sized
+ * by the matching query (the stages of a direction reuse its bytes one after the other).  rank a multiple of 8 in
+ * [8,64]; the other operands as for the entry points above; quantized_data_t / block_scalers_t: both or neither.
+ */
+size_t ttamd_qlora_linear_fwd_workspace_bytes(int64_t M, int64_t N, int64_t K, int rank);
+int ttamd_qlora_linear_fwd_bf16(const void* x, const uint8_t* quantized_data, const void* block_scalers, const void* block_scalers_t,
+                                const void* lora_a, const void* lora_b, int rank, float scale, const void* bias, void* y, void* h,
+                                int64_t M, int64_t N, int64_t K, void* workspace, size_t workspace_bytes, void* stream);
+size_t ttamd_qlora_linear_bwd_workspace_bytes(int64_t M, int64_t N, int64_t K, int rank);
+int ttamd_qlora_linear_bwd_bf16(const void* gy, const void* x, const void* h, const uint8_t* quantized_data, const void* block_scalers,
+                                const uint8_t* quantized_data_t, const void* block_scalers_t, const void* lora_a, const void* lora_b,
+                                int rank, float scale, void* gx, void* grad_lora_a, void* grad_lora_b, int64_t M, int64_t N, int64_t K,
+                                void* workspace, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
  * Groups of LoRA linears with a common input

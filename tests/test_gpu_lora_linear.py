@@ -694,3 +694,83 @@ def test_entry_points_are_reentrant_across_threads_and_streams():
     for i, (w, o) in enumerate(zip(want, got)):
         for name, a, b in zip(("y", "gx", "gA", "gB"), w, o):
             assert torch.equal(a, b), f"case {i}: {name} differs between the concurrent and the serial run"
+
+
+# (M, N, K, rank, bias, transposed copies): the few-token kernel, slices of the contraction, the fused kernel with and
+# without the transposed copies, the weight expanded once per call, a ragged row count
+ONE_CALL_CASES = [
+    (8, 1024, 512, 8, False, False),
+    (96, 512, 1024, 16, True, True),
+    (2048, 2048, 2048, 8, False, True),
+    (2048, 2048, 2048, 8, False, False),
+    (700, 768, 640, 24, True, True),
+    (2304, 4096, 4096, 16, False, False),
+    (4096, 4096, 4096, 64, True, True),
+]
+
+
+@pytest.mark.parametrize("M,N,K,r,bias,copies", ONE_CALL_CASES)
+def test_one_call_per_direction_equals_the_two_call_sequence_bitwise(M, N, K, r, bias, copies):
+    """``ttamd_qlora_linear_fwd_bf16`` / ``ttamd_qlora_linear_bwd_bf16`` (the whole layer, one ABI call per direction, one
+    workspace) against ``lora_hidden`` -> ``nf4_lora_linear_fwd`` and ``lora_bwd`` -> ``nf4_linear_bwd_dx``: every output
+    bit for bit, on two consecutive calls (the second finds the first one's workspace contents)."""
+    W, sbs, A, B, b, x, gy = _make(M, N, K, r, seed=11 + M % 7, bias=bias)
+    t = to_nf4(W.to(DEV), 64, sbs)
+    qd, bs = t.quantized_data, t.block_scalers()
+    tr = ops.nf4_transpose_for_backward(qd, bs, N, K) if copies else None
+    xd, gyd, Ad, Bd = x.to(DEV), gy.to(DEV), A.to(DEV), B.to(DEV)
+    bd = b.to(DEV) if bias else None
+    s = 2.0
+    h2 = ops.lora_hidden(xd, Ad)
+    y2 = ops.nf4_lora_linear_fwd(xd, qd, bs, N, h2, Bd, s, bd, block_scalers_t=tr[1] if tr else None)
+    gh2, ga2, gb2 = ops.lora_bwd(gyd, xd, h2, Bd, s)
+    gx2 = ops.nf4_linear_bwd_dx(gyd, qd, bs, K, gh2, Ad, transposed=tr)
+    for _ in range(2):
+        y1, h1 = ops.qlora_linear_fwd(xd, qd, bs, N, Ad, Bd, s, bd, block_scalers_t=tr[1] if tr else None)
+        gx1, ga1, gb1 = ops.qlora_linear_bwd(gyd, xd, h1, qd, bs, Ad, Bd, s, transposed=tr)
+        for got, want in ((y1, y2), (h1, h2), (gx1, gx2), (ga1, ga2), (gb1, gb2)):
+            assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    # without a grad-input the adapter gradients are the same and nothing is written for gx
+    gx0, ga0, gb0 = ops.qlora_linear_bwd(gyd, xd, h2, qd, bs, Ad, Bd, s, transposed=tr, need_gx=False)
+    assert gx0 is None and torch.equal(ga0, ga2) and torch.equal(gb0, gb2)
+    # and against the oracle (small cases) through the layer, which takes the one-call route
+    if M * N * K <= 2048 ** 3:
+        p, y_o, gx_o, gA_o, gB_o = _oracle(W, sbs, A, B, b, x, gy, s * r, r)
+        _close(y1, y_o, 1e-2, 1e-2)
+        _close(gx1, gx_o, 1e-2, 1e-2)
+
+
+def test_one_call_entry_points_check_their_workspace_and_arguments():
+    lib = _lib.load()
+    M, N, K, r = 256, 512, 256, 8
+    W, sbs, A, B, _, x, gy = _make(M, N, K, r, seed=3)
+    t = to_nf4(W.to(DEV), 64, sbs)
+    qd, bs = t.quantized_data, t.block_scalers()
+    xd, gyd, Ad, Bd = x.to(DEV), gy.to(DEV), A.to(DEV), B.to(DEV)
+    y = torch.empty(M, N, dtype=BF, device=DEV)
+    h = torch.empty(M, r, dtype=BF, device=DEV)
+    need = int(lib.ttamd_qlora_linear_fwd_workspace_bytes(M, N, K, r))
+    assert need > 0 and need % 256 == 0
+    ws = torch.empty(need, dtype=torch.uint8, device=DEV)
+    st = torch.cuda.current_stream().cuda_stream
+    args = (xd.data_ptr(), qd.data_ptr(), bs.data_ptr(), None, Ad.data_ptr(), Bd.data_ptr(), r, 2.0, None, y.data_ptr(), h.data_ptr(), M, N, K)
+    assert lib.ttamd_qlora_linear_fwd_bf16(*args, ws.data_ptr(), need - 1, st) == -3   # TTAMD_EWORKSPACE
+    assert b"qlora_linear_fwd" in lib.ttamd_last_error()
+    assert lib.ttamd_qlora_linear_fwd_bf16(*args, ws.data_ptr(), need, st) == 0
+    bad = list(args)
+    bad[6] = 12                                                                          # rank % 8
+    assert lib.ttamd_qlora_linear_fwd_bf16(*bad, ws.data_ptr(), need, st) == -1
+    nb = int(lib.ttamd_qlora_linear_bwd_workspace_bytes(M, N, K, r))
+    assert nb >= M * r * 2
+    wsb = torch.empty(nb, dtype=torch.uint8, device=DEV)
+    gx = torch.empty(M, K, dtype=BF, device=DEV)
+    ga = torch.empty(r, K, dtype=BF, device=DEV)
+    gb = torch.empty(N, r, dtype=BF, device=DEV)
+    bargs = (gyd.data_ptr(), xd.data_ptr(), h.data_ptr(), qd.data_ptr(), bs.data_ptr(), None, None, Ad.data_ptr(), Bd.data_ptr(), r, 2.0,
+             gx.data_ptr(), ga.data_ptr(), gb.data_ptr(), M, N, K)
+    assert lib.ttamd_qlora_linear_bwd_bf16(*bargs, wsb.data_ptr(), nb - 1, st) == -3
+    assert lib.ttamd_qlora_linear_bwd_bf16(*bargs, wsb.data_ptr(), nb, st) == 0
+    half = list(bargs)
+    half[5] = qd.data_ptr()                                                              # one transposed copy without the other
+    assert lib.ttamd_qlora_linear_bwd_bf16(*half, wsb.data_ptr(), nb, st) == -1
+    torch.cuda.synchronize()

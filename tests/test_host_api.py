@@ -443,6 +443,46 @@ def test_gemm_workspace_query_is_a_host_function():
         assert q(M, N, K) == slices * M * N * 4, (M, N, K)
 
 
+def test_group_grad_input_workspace_query_bounds_the_concatenated_contraction():
+    """``ttamd_nf4_group_bwd_dx_workspace_bytes`` (a host function; the pointers are only checked for alignment) offers
+    the expanded-weight launch for the q / k / v and gate / up groups of the 8B shapes and refuses it (0: the caller
+    stays on the per-member fused kernels) once the members' concatenated columns outgrow the launch's 32-bit offsets,
+    although every member on its own would fit."""
+    from torchtune_amd import _lib
+
+    lib = _lib.load()
+
+    def members(ns):
+        arr = (_lib.LoraGroupMember * len(ns))()
+        for i, n in enumerate(ns):
+            for f in ("quantized_data", "block_scalers", "lora_a", "lora_b", "y"):
+                setattr(arr[i], f, 0x1000)
+            arr[i].N, arr[i].rank, arr[i].scale = n, 16, 2.0
+        return arr
+
+    q = lib.ttamd_nf4_group_bwd_dx_workspace_bytes
+    assert q(members([4096, 1024, 1024]), 3, 8192, 4096) == 2 * 4096 * 6144
+    assert q(members([14336, 14336]), 2, 8192, 4096) == 2 * 4096 * 28672
+    wide = (1 << 20) - 64                       # 2048 rows x this many columns x 2 bytes: just below 2^32 per member
+    assert 2048 * wide * 2 < 1 << 32 <= 2048 * 4 * wide * 2
+    assert q(members([wide]), 1, 2048, 8192) == 2 * 8192 * wide
+    assert q(members([wide] * 4), 4, 2048, 8192) == 0
+    assert q(members([1 << 20]), 1, 2048, 8192) == 0   # one member beyond its own bound
+
+
+def test_built_in_scratch_holds_every_plan_of_the_hidden_product():
+    """The partial sums `ttamd_lora_hidden_static_bf16` keeps in its 2 MiB device array never outgrow it: the workspace
+    query of the same plan (a host function) over every row count up to 8192 and beyond, long contractions, rank 64."""
+    lib = _lib.load()
+    limit = lib.ttamd_lora_hidden_static_max_bytes()
+    assert limit == 2 << 20
+    worst = 0
+    for K in (64, 4096, 14336, 64 * 8 * 256, 1 << 20):
+        for M in list(range(1, 8193)) + [8193, 12288, 16384, 65536, 1 << 20]:
+            worst = max(worst, lib.ttamd_lora_fwd_workspace_bytes(M, K, 64))
+    assert 0 < worst <= limit, worst
+
+
 def test_bench_refuses_more_than_one_gpu():
     """``bench.py --gpus N`` with N > 1 exits with a message before touching any device."""
     import subprocess

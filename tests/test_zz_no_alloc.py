@@ -38,6 +38,29 @@ def test_static_scratch_variant_matches_the_workspace_variant_on_consecutive_cal
         torch.testing.assert_close(got.float(), ref, rtol=1e-2, atol=1e-2 * max(1.0, float(ref.abs().max()) / 8))
 
 
+def test_static_scratch_variant_allocates_nothing():
+    """With inputs and output in place, a call changes neither the device's free memory nor torch's own accounting."""
+    lib = _lib.load()
+    assert lib.ttamd_lora_hidden_static_init() == 0  # the symbol query of a device's first use, outside the measured call
+    g = torch.Generator(device=DEV).manual_seed(1)
+    M, K, r = 512, 14336, 64  # sliced along K: the partial sums use the built-in array
+    assert 0 < lib.ttamd_lora_fwd_workspace_bytes(M, K, r) <= lib.ttamd_lora_hidden_static_max_bytes()
+    x = torch.randn(M, K, device=DEV, generator=g).to(torch.bfloat16)
+    a = (torch.randn(r, K, device=DEV, generator=g) * 0.05).to(torch.bfloat16)
+    h = torch.empty(M, r, dtype=torch.bfloat16, device=DEV)
+    st = torch.cuda.current_stream().cuda_stream
+    assert lib.ttamd_lora_hidden_static_bf16(x.data_ptr(), a.data_ptr(), h.data_ptr(), M, K, r, st) == 0  # warm: code loaded
+    torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info()
+    alloc0, reserved0 = torch.cuda.memory_allocated(), torch.cuda.memory_reserved()
+    for _ in range(3):
+        assert lib.ttamd_lora_hidden_static_bf16(x.data_ptr(), a.data_ptr(), h.data_ptr(), M, K, r, st) == 0
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info()
+    assert free1 == free0
+    assert (torch.cuda.memory_allocated(), torch.cuda.memory_reserved()) == (alloc0, reserved0)
+
+
 def test_static_scratch_variant_rejects_bad_arguments():
     lib = _lib.load()
     x = torch.zeros(64, 128, dtype=torch.bfloat16, device=DEV)

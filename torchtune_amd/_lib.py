@@ -40,6 +40,7 @@ SIGNATURES = {
     "ttamd_lora_fwd_workspace_bytes": (_size, [_i64, _i64, _int]),
     "ttamd_lora_hidden_bf16": (_int, [_c_void_p, _c_void_p, _c_void_p, _i64, _i64, _int, _c_void_p, _size, _c_void_p]),
     "ttamd_lora_hidden_static_max_bytes": (_size, []),
+    "ttamd_lora_hidden_static_init": (_int, []),
     "ttamd_lora_hidden_static_bf16": (_int, [_c_void_p, _c_void_p, _c_void_p, _i64, _i64, _int, _c_void_p]),
     "ttamd_nf4_lora_linear_fwd_bf16": (
         _int,
@@ -90,6 +91,18 @@ SIGNATURES = {
         _int,
         [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _f32, _c_void_p, _c_void_p, _c_void_p, _i64, _i64, _i64, _int,
          _c_void_p, _size, _c_void_p],
+    ),
+    "ttamd_qlora_linear_fwd_workspace_bytes": (_size, [_i64, _i64, _i64, _int]),
+    "ttamd_qlora_linear_fwd_bf16": (
+        _int,
+        [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _int, _f32, _c_void_p, _c_void_p, _c_void_p, _i64, _i64,
+         _i64, _c_void_p, _size, _c_void_p],
+    ),
+    "ttamd_qlora_linear_bwd_workspace_bytes": (_size, [_i64, _i64, _i64, _int]),
+    "ttamd_qlora_linear_bwd_bf16": (
+        _int,
+        [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _int, _f32, _c_void_p,
+         _c_void_p, _c_void_p, _i64, _i64, _i64, _c_void_p, _size, _c_void_p],
     ),
     "ttamd_lora_group_hidden_workspace_bytes": (_size, [_c_void_p, _int, _i64, _i64]),
     "ttamd_lora_group_hidden_bf16": (_int, [_c_void_p, _c_void_p, _int, _c_void_p, _i64, _i64, _c_void_p, _size, _c_void_p]),

@@ -16,7 +16,7 @@ PKG = Path(__file__).resolve().parent
 CSRC = PKG / "csrc"
 LIB_DIR = PKG / "lib"
 LIB_PATH = LIB_DIR / "libtorchtune_amd.so"
-SOURCES = ["capi.hip", "nf4_codec.hip", "fake_quant.hip", "nf4_gemm.hip", "nf4_gemm_rs.hip", "nf4_gemm_dense.hip", "gemm_tn.hip", "nf4_small_m.hip", "lora_skinny.hip", "lora_group.hip", "nf4_merge.hip", "neighbours.hip"]
+SOURCES = ["capi.hip", "nf4_codec.hip", "fake_quant.hip", "nf4_gemm.hip", "nf4_gemm_rs.hip", "nf4_gemm_dense.hip", "gemm_tn.hip", "nf4_small_m.hip", "lora_skinny.hip", "lora_group.hip", "qlora_linear.hip", "nf4_merge.hip", "neighbours.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",

@@ -13,6 +13,7 @@
 // put enough loads in flight and combine the fp32 partial sums in a second, fixed-order pass, so results
 // are deterministic.  For wide layers of rank <= 16 the two products that read gy (gh and gB) come from one pass over
 // it (skinny_tn_gh_kernel).
+#include <atomic>
 #include "common.h"
 #include "group.h"
 #include "nf4_math.h"
@@ -1020,23 +1021,33 @@ static __device__ __align__(256) unsigned char g_hidden_scratch[kStaticScratchBy
 
 namespace {
 // Device address of g_hidden_scratch on the current device.  In host code the array's name is only a handle for the
-// runtime, not a device address: the address is asked for once per device (with that device current) and kept.
+// runtime, not a device address: the address is asked for once per device (with that device current) and kept.  The
+// slots are atomics because threads of different streams may make a device's first call together (both then store the
+// same value).
 int static_scratch(float** out) {
-  static void* ptr[64] = {};
+  static std::atomic<void*> ptr[64] = {};
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return fail(TTAMD_ELAUNCH, "lora_hidden_static: hipGetDevice: %s", hipGetErrorString(e));
-  void* p = (dev >= 0 && dev < 64) ? ptr[dev] : nullptr;
+  void* p = (dev >= 0 && dev < 64) ? ptr[dev].load(std::memory_order_relaxed) : nullptr;
   if (p == nullptr) {
     e = hipGetSymbolAddress(&p, HIP_SYMBOL(g_hidden_scratch));
     if (e != hipSuccess || p == nullptr)
       return fail(TTAMD_ELAUNCH, "lora_hidden_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
-    if (dev >= 0 && dev < 64) ptr[dev] = p;  // a race between threads stores the same value twice
+    if (dev >= 0 && dev < 64) ptr[dev].store(p, std::memory_order_relaxed);
   }
   *out = reinterpret_cast<float*>(p);
   return TTAMD_OK;
 }
 }  // namespace
+
+// Resolves the scratch array's address on the current device.  The query may load the code object, which must not
+// happen while a stream is being captured: callers that capture make this call (or one eager call of the entry point
+// below) once per device beforehand.
+extern "C" int ttamd_lora_hidden_static_init(void) {
+  float* scratch = nullptr;
+  return static_scratch(&scratch);
+}
 
 extern "C" size_t ttamd_lora_hidden_static_max_bytes(void) { return kStaticScratchBytes; }
 

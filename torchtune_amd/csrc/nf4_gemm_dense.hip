@@ -931,7 +931,9 @@ size_t dense_group_dx_workspace_bytes(const GroupDx& d) {
     n_total += d.N[i];
     if (d.M * d.N[i] * 2 >= (int64_t(1) << 32)) return 0;
   }
-  if (d.K % 64 != 0 || !dense_tiles_apply(d.M, ((d.M + 255) / 256) * ((d.K + 255) / 256))) return 0;
+  // the launch contracts over all members' columns: the kernel's 32-bit lane offsets and step counts bound n_total as
+  // they bound the contraction of a single layer
+  if (!dense_path_applies(d.M, d.K, n_total)) return 0;
   return (size_t)d.K * (size_t)n_total * 2;
 }
 

@@ -29,6 +29,10 @@ from ...nf4_tensor import _check_in_features
 from ._adapter_base import LowRankAdapterLinear, _lora_a_init_params, _lora_b_init_params  # noqa: F401
 
 
+# One library call per direction of a QLoRA layer (False: the two stages of a direction are called one by one; same results)
+ONE_CALL_PER_DIRECTION = True
+
+
 class TrainableParams(Enum):
     FULL = "full"
     LORA = "lora"
@@ -36,17 +40,25 @@ class TrainableParams(Enum):
 
 
 class _QLoRALinearFn(torch.autograd.Function):
-    """Fused QLoRA linear.  Inputs: x [..., K] bf16, NF4 weight [N, K], lora_a [r, K], lora_b [N, r], bias or None."""
+    """Fused QLoRA linear.  Inputs: x [..., K] bf16, NF4 weight [N, K], lora_a [r, K], lora_b [N, r], bias or None.
+
+    Each direction is one call into the library (``ttamd_qlora_linear_fwd_bf16`` / ``ttamd_qlora_linear_bwd_bf16``).  While a
+    GEMM timer is installed (``ops.set_gemm_timer``) the two stages of a direction are called one by one instead - the
+    same launches, the same bits - because the timer brackets the GEMM stage alone."""
 
     @staticmethod
     def forward(ctx, x, weight, lora_a, lora_b, bias, scale: float):
         N, K = weight.shape
         _check_in_features(x, weight)
         x2 = x.reshape(-1, K)
-        h = ops.lora_hidden(x2, lora_a)
         tr = weight.backward_copy_for(x2.shape[0], True)
-        y = ops.nf4_lora_linear_fwd(x2, weight.quantized_data, weight.block_scalers(), N, h, lora_b, scale, bias,
-                                    block_scalers_t=tr[1] if tr else None)
+        if ONE_CALL_PER_DIRECTION and not ops.gemm_timer_installed():
+            y, h = ops.qlora_linear_fwd(x2, weight.quantized_data, weight.block_scalers(), N, lora_a, lora_b, scale, bias,
+                                        block_scalers_t=tr[1] if tr else None)
+        else:
+            h = ops.lora_hidden(x2, lora_a)
+            y = ops.nf4_lora_linear_fwd(x2, weight.quantized_data, weight.block_scalers(), N, h, lora_b, scale, bias,
+                                        block_scalers_t=tr[1] if tr else None)
         ctx.save_for_backward(x2, h, weight, lora_a, lora_b)
         ctx.scale = scale
         ctx.x_shape = x.shape
@@ -61,10 +73,15 @@ class _QLoRALinearFn(torch.autograd.Function):
         need_x, _, need_a, need_b, need_bias, _ = ctx.needs_input_grad
         gx = ga = gb = gbias = None
         if need_x or need_a or need_b:
-            gh, ga, gb = ops.lora_bwd(gy2, x2, h, lora_b, ctx.scale)
+            tr = weight.backward_copy_for(gy2.shape[0], False) if need_x else None
+            if ONE_CALL_PER_DIRECTION and not ops.gemm_timer_installed():
+                gx, ga, gb = ops.qlora_linear_bwd(gy2, x2, h, weight.quantized_data, weight.block_scalers(), lora_a, lora_b,
+                                                  ctx.scale, transposed=tr, need_gx=need_x)
+            else:
+                gh, ga, gb = ops.lora_bwd(gy2, x2, h, lora_b, ctx.scale)
+                if need_x:
+                    gx = ops.nf4_linear_bwd_dx(gy2, weight.quantized_data, weight.block_scalers(), K, gh, lora_a, transposed=tr)
             if need_x:
-                gx = ops.nf4_linear_bwd_dx(gy2, weight.quantized_data, weight.block_scalers(), K, gh, lora_a,
-                                           transposed=weight.backward_copy_for(gy2.shape[0], False))
                 gx = gx.view(ctx.x_shape)
             if not need_a:
                 ga = None
@@ -195,8 +212,17 @@ class QATLoRALinear(LoRALinear):
 
     # The base weight of a QAT + LoRA layer is frozen, so its fake-quantised form only changes when the weight is
     # written (load_state_dict, copy_).  With 288 GB of HBM it is kept instead of being rebuilt in every forward; set
-    # to False to recompute it each time, as the reference does.
+    # to False to recompute it each time, as the reference does.  A layer holds ONE form at a time: the row-major copy
+    # (2 B per weight element; few-token calls) or the two tiled copies (forward and transposed, 4 B per element;
+    # many-token calls), whichever its last call used - building one releases the other.  The cache key is the weight's
+    # storage address, shape, dtype and version counter; a write through ``weight.data`` (``weight.data.copy_(...)``)
+    # does not advance that counter, so code that writes this way calls ``invalidate_fake_quant_cache()`` afterwards.
     cache_frozen_weight_fake_quant = True
+
+    def invalidate_fake_quant_cache(self) -> None:
+        """Drop the kept fake-quantised forms of the frozen weight; the next forward rebuilds what it needs."""
+        self._fq_weight_cache = None
+        self._tiled_weight_cache = None
 
     def _fake_quantized_weight(self) -> torch.Tensor:
         w, fq = self.weight, self.weight_fake_quantizer
@@ -212,6 +238,7 @@ class QATLoRALinear(LoRALinear):
             with torch.no_grad():
                 cached = (key, fq(w).detach())
             self._fq_weight_cache = cached
+            self._tiled_weight_cache = None  # one form at a time
         return cached[1]
 
     # From this many tokens (and a full round of 256 x 256 output tiles in both directions) the layer runs on the library's
@@ -233,6 +260,7 @@ class QATLoRALinear(LoRALinear):
             self.weight_fake_quantizer.zero_point = None
             cached = (key, tf, tb)
             self._tiled_weight_cache = cached
+            self._fq_weight_cache = None  # one form at a time
         return cached[1], cached[2]
 
     def _tiled_ok(self, x: torch.Tensor) -> bool:

@@ -152,6 +152,11 @@ def nf4_block_scalers(qscalers: torch.Tensor, qfactor: torch.Tensor, mean: torch
 _gemm_timer = None
 
 
+def gemm_timer_installed() -> bool:
+    """True while ``set_gemm_timer`` has a callback in place."""
+    return _gemm_timer is not None
+
+
 def set_gemm_timer(timer) -> None:
     """Install (or with None remove) a callback ``timer(kind, M, N, K, rank) -> (start_event, end_event)``; the two
     events are recorded on the launch stream immediately before and after every fused-GEMM launch (``kind`` "fwd" /
@@ -363,6 +368,78 @@ def lora_bwd(
         )
     _lib.check(rc, "lora_bwd")
     return gh, ga, gb
+
+
+# ---------------------------------------------------------------------------------------------------
+# The whole layer, one library call per direction
+# ---------------------------------------------------------------------------------------------------
+def qlora_linear_fwd(
+    x: torch.Tensor, qdata: torch.Tensor, block_scalers: torch.Tensor, N: int, lora_a: torch.Tensor, lora_b: torch.Tensor,
+    scale: float, bias: Optional[torch.Tensor] = None, block_scalers_t: Optional[torch.Tensor] = None,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """``(y, h)``: ``h = bf16(x @ lora_a.T)`` and ``y = x @ D(W).T (+ bias) + scale * h @ lora_b.T`` from one call of
+    ``ttamd_qlora_linear_fwd_bf16`` (``lora_hidden`` followed by ``nf4_lora_linear_fwd``, the same launches and bits, out
+    of one workspace)."""
+    x = _bf16_2d(x, "qlora_linear_fwd")
+    lora_a = _bf16_2d(lora_a, "qlora_linear_fwd")
+    lora_b = _bf16_2d(lora_b, "qlora_linear_fwd")
+    M, K = x.shape
+    rank = lora_a.shape[0]
+    _check_nf4_operands("qlora_linear_fwd", N, K, qdata, block_scalers, block_scalers_t)
+    if lora_a.shape[1] != K or tuple(lora_b.shape) != (N, rank):
+        raise ValueError(f"qlora_linear_fwd: lora_a {tuple(lora_a.shape)} / lora_b {tuple(lora_b.shape)} do not fit a "
+                         f"[{N}, {K}] layer")
+    if bias is not None:
+        bias = bias.contiguous()
+        if bias.dtype != torch.bfloat16 or bias.numel() != N:
+            raise ValueError(f"qlora_linear_fwd: bias must be bfloat16 with {N} elements")
+    lib = _lib.load()
+    y = torch.empty(M, N, dtype=torch.bfloat16, device=x.device)
+    h = torch.empty(M, rank, dtype=torch.bfloat16, device=x.device)
+    nbytes = int(lib.ttamd_qlora_linear_fwd_workspace_bytes(M, N, K, rank))
+    ws = _workspace(nbytes, x.device)
+    with torch.cuda.device(x.device):
+        rc = lib.ttamd_qlora_linear_fwd_bf16(
+            x.data_ptr(), qdata.data_ptr(), block_scalers.data_ptr(), _ptr(block_scalers_t), lora_a.data_ptr(), lora_b.data_ptr(),
+            rank, float(scale), _ptr(bias), y.data_ptr(), h.data_ptr(), M, N, K, ws.data_ptr(), ws.numel(), _stream(x))
+    _lib.check(rc, "qlora_linear_fwd")
+    return y, h
+
+
+def qlora_linear_bwd(
+    gy: torch.Tensor, x: torch.Tensor, h: torch.Tensor, qdata: torch.Tensor, block_scalers: torch.Tensor, lora_a: torch.Tensor,
+    lora_b: torch.Tensor, scale: float, transposed=None, need_gx: bool = True,
+) -> Tuple[Optional[torch.Tensor], torch.Tensor, torch.Tensor]:
+    """``(gx or None, gA, gB)`` from one call of ``ttamd_qlora_linear_bwd_bf16`` (``lora_bwd`` followed by
+    ``nf4_linear_bwd_dx``, the same launches and bits, out of one workspace that also holds ``gh``)."""
+    gy = _bf16_2d(gy, "qlora_linear_bwd")
+    x = _bf16_2d(x, "qlora_linear_bwd")
+    h = _bf16_2d(h, "qlora_linear_bwd")
+    lora_a = _bf16_2d(lora_a, "qlora_linear_bwd")
+    lora_b = _bf16_2d(lora_b, "qlora_linear_bwd")
+    M, N = gy.shape
+    K = x.shape[1]
+    rank = h.shape[1]
+    _check_nf4_operands("qlora_linear_bwd", N, K, qdata, block_scalers, transposed[1] if transposed else None)
+    if transposed and (transposed[0].dtype != torch.uint8 or transposed[0].numel() * 2 != N * K):
+        raise ValueError(f"qlora_linear_bwd: the transposed codes do not hold a [{N}, {K}] weight")
+    if x.shape[0] != M or h.shape[0] != M or tuple(lora_b.shape) != (N, rank) or tuple(lora_a.shape) != (rank, K):
+        raise ValueError(f"qlora_linear_bwd: gy {tuple(gy.shape)}, x {tuple(x.shape)}, h {tuple(h.shape)}, lora_a "
+                         f"{tuple(lora_a.shape)} and lora_b {tuple(lora_b.shape)} do not belong to one layer")
+    dev = gy.device
+    lib = _lib.load()
+    gx = torch.empty(M, K, dtype=torch.bfloat16, device=dev) if need_gx else None
+    ga = torch.empty(rank, K, dtype=torch.bfloat16, device=dev)
+    gb = torch.empty(N, rank, dtype=torch.bfloat16, device=dev)
+    ws = _workspace(int(lib.ttamd_qlora_linear_bwd_workspace_bytes(M, N, K, rank)), dev)
+    with torch.cuda.device(dev):
+        rc = lib.ttamd_qlora_linear_bwd_bf16(
+            gy.data_ptr(), x.data_ptr(), h.data_ptr(), qdata.data_ptr(), block_scalers.data_ptr(),
+            _ptr(transposed[0]) if transposed else None, _ptr(transposed[1]) if transposed else None, lora_a.data_ptr(),
+            lora_b.data_ptr(), rank, float(scale), _ptr(gx), ga.data_ptr(), gb.data_ptr(), M, N, K, ws.data_ptr(), ws.numel(),
+            _stream(gy))
+    _lib.check(rc, "qlora_linear_bwd")
+    return gx, ga, gb
 
 
 # ---------------------------------------------------------------------------------------------------

@@ -208,6 +208,11 @@ class FakeQuantizer(nn.Module):
         return out
 
     @staticmethod
+    def forget_shared_input() -> None:
+        """Drop the calling thread's kept per-token result (it holds a fake-quantised copy of one activation)."""
+        FakeQuantizer._last.entry = None
+
+    @staticmethod
     def _drop_entry(_ref) -> None:
         hit = getattr(FakeQuantizer._last, "entry", None)
         if hit is not None and hit[0] is _ref:
@@ -372,10 +377,15 @@ def fake_quantized_linear_group(x: torch.Tensor, layers, swiglu: bool = False) -
             raise ValueError("fake_quantized_linear_group: the gated product needs a pair the group kernels serve")
         return tuple(layer(x) for layer in layers)
     first = layers[0]
-    xq = x if first.activation_fake_quantizer is None else first.activation_fake_quantizer(x)
-    for layer in layers[1:]:  # every member's quantizer records its qparams, as a call of its own would (the result is shared)
-        if layer.activation_fake_quantizer is not None:
-            layer.activation_fake_quantizer(x)
+    a0 = first.activation_fake_quantizer
+    xq = x if a0 is None else a0(x)
+    # every member's quantizer ends up with the qparams a call of its own would have recorded: the members' activation
+    # configurations are equal (_group_tiled_ok), so the first member's are theirs and no kernel runs again
+    if a0 is not None and a0.enabled:
+        for layer in layers[1:]:
+            layer.activation_fake_quantizer.scale = a0.scale
+            layer.activation_fake_quantizer.zero_point = a0.zero_point
+        FakeQuantizer.forget_shared_input()  # the group was the shared result's last user: do not keep fq(x) alive
     flat = []
     for layer in layers:
         flat += [layer.weight, layer.bias]
