@@ -742,7 +742,7 @@ def test_one_call_per_direction_equals_the_two_call_sequence_bitwise(M, N, K, r,
 
 def test_one_call_entry_points_check_their_workspace_and_arguments():
     lib = _lib.load()
-    M, N, K, r = 256, 512, 256, 8
+    M, N, K, r = 96, 512, 1024, 8   # the forward's GEMM slices the contraction: a workspace is needed
     W, sbs, A, B, _, x, gy = _make(M, N, K, r, seed=3)
     t = to_nf4(W.to(DEV), 64, sbs)
     qd, bs = t.quantized_data, t.block_scalers()

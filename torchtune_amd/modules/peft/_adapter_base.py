@@ -79,13 +79,21 @@ class LowRankAdapterLinear(nn.Module):
         )
 
     def _fused_path(self, x: torch.Tensor) -> bool:
-        return (
-            self._quantize_base
-            and not self._dropping()
-            and self._nf4_kernels_apply(x.dtype)
-            and _fused_ok(x, self.weight, self._adapter_rank())
-            and (self.bias is None or self.bias.dtype == torch.bfloat16)
-        )
+        if not self._quantize_base or x.dtype != torch.bfloat16 or self._dropping():
+            return False
+        # what depends on the parameters alone is decided once per set of parameter objects (a swapped or re-created
+        # parameter is another object): attribute reads on an NF4 tensor subclass cost microseconds each
+        w, a, b, bias = self.weight, self.lora_a.weight, self.lora_b.weight, self.bias
+        packed = getattr(w, "quantized_data", None)  # the inner tensor object: another one after a move or a rewrap
+        memo = self.__dict__.get("_fused_memo")
+        if (memo is None or memo[0] is not w or memo[1] is not a or memo[2] is not b or memo[3] is not bias
+                or memo[4] is not packed):
+            ok = (self._nf4_kernels_apply(torch.bfloat16) and _fused_ok(torch.empty(1, dtype=torch.bfloat16, device=w.device), w,
+                                                                        self._adapter_rank())
+                  and (bias is None or bias.dtype == torch.bfloat16))
+            memo = (w, a, b, bias, packed, bool(ok))
+            self.__dict__["_fused_memo"] = memo
+        return memo[5] and x.is_cuda and x.numel() > 0
 
     def _base_out(self, x: torch.Tensor) -> torch.Tensor:
         """The frozen base layer by itself (composed path)."""

@@ -25,7 +25,7 @@ import torch.nn.functional as F
 from torch import nn
 
 from ... import ops
-from ...nf4_tensor import _check_in_features
+from ...nf4_tensor import _check_in_features, shape_and_dtype
 from ._adapter_base import LowRankAdapterLinear, _lora_a_init_params, _lora_b_init_params  # noqa: F401
 
 
@@ -48,7 +48,7 @@ class _QLoRALinearFn(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x, weight, lora_a, lora_b, bias, scale: float):
-        N, K = weight.shape
+        N, K = shape_and_dtype(weight)[0]
         _check_in_features(x, weight)
         x2 = x.reshape(-1, K)
         tr = weight.backward_copy_for(x2.shape[0], True)
@@ -68,7 +68,7 @@ class _QLoRALinearFn(torch.autograd.Function):
     @staticmethod
     def backward(ctx, gy):
         x2, h, weight, lora_a, lora_b = ctx.saved_tensors
-        N, K = weight.shape
+        N, K = shape_and_dtype(weight)[0]
         gy2 = gy.reshape(-1, N)
         need_x, _, need_a, need_b, need_bias, _ = ctx.needs_input_grad
         gx = ga = gb = gbias = None

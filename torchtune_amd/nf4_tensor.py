@@ -14,6 +14,7 @@ implementation); with no GPU present those calls raise.
 from __future__ import annotations
 
 import math
+import weakref
 from typing import Any, Callable, Dict, Iterable, Optional
 
 import torch
@@ -91,6 +92,25 @@ def implements_torch_function(torch_fn):
         return fn
 
     return decorator
+
+
+def shape_and_dtype(weight: "NF4Tensor"):
+    """``(tuple(weight.shape), weight.dtype)`` for the per-call host code.  ``shape`` / ``dtype`` of a tensor subclass are
+    routed through ``__torch_function__`` (microseconds each, a dozen reads per layer call), so the pair is kept on the
+    packed-data tensor object, with a weak reference to the NF4 tensor it describes.  (Not on the NF4 tensor itself: the
+    reference pins the exact key set of its ``__dict__``,
+    tests/torchtune/modules/low_precision/test_nf4_dispatch_registration.py:22-35, and ``torch.utils.swap_tensors``
+    refuses tensors whose slots differ.)"""
+    packed = weight.quantized_data
+    memo = packed.__dict__.get("_ttamd_outer")
+    if memo is not None and memo[0]() is weight:
+        return memo[1], memo[2]
+    shape, dtype = tuple(weight.shape), weight.dtype
+    try:
+        packed._ttamd_outer = (weakref.ref(weight), shape, dtype)
+    except TypeError:
+        pass
+    return shape, dtype
 
 
 def _compute_device(t: torch.Tensor) -> torch.device:
@@ -254,7 +274,7 @@ class NF4Tensor(torch.Tensor):
         """The transposed copy a GEMM call over ``tokens`` rows would use: None when the library serves that call from the
         weight expanded once per call (many tokens; it then reads the weight's own codes, so a purely many-token
         training run never builds the copy), otherwise ``backward_copy()``."""
-        N, K = self.shape
+        N, K = shape_and_dtype(self)[0]
         n_out, k_contract = (N, K) if forward else (K, N)
         if ops.gemm_expands_weight(tokens, n_out, k_contract):
             return None
@@ -520,6 +540,10 @@ class _LinearNF4(torch.autograd.Function):
 def _check_in_features(x: torch.Tensor, weight: torch.Tensor) -> None:
     """The shape error ``F.linear`` raises for a dense weight; the fused kernels take K from the activation, so a wrong
     inner dimension must be stopped on the host."""
+    if isinstance(weight, NF4Tensor):
+        shape = shape_and_dtype(weight)[0]
+        if len(shape) == 2 and x.dim() > 0 and x.shape[-1] == shape[1]:
+            return
     if weight.dim() == 2 and (x.dim() == 0 or x.shape[-1] != weight.shape[1]):
         raise RuntimeError(
             f"mat1 and mat2 shapes cannot be multiplied ({x.numel() // max(x.shape[-1] if x.dim() else 1, 1)}x"
@@ -530,15 +554,16 @@ def _check_in_features(x: torch.Tensor, weight: torch.Tensor) -> None:
 def _fused_ok(x: torch.Tensor, weight: NF4Tensor, rank: int) -> bool:
     """True when the fused dequantise-in-GEMM kernel applies; otherwise the caller dequantises with the
     stand-alone kernel and uses a library GEMM."""
+    shape, dtype = shape_and_dtype(weight)
     return (
         x.is_cuda
         and weight.quantized_data.is_cuda
         and x.dtype == torch.bfloat16
-        and weight.dtype == torch.bfloat16
-        and weight.dim() == 2
+        and dtype == torch.bfloat16
+        and len(shape) == 2
         and weight.block_size == 64
         and x.numel() > 0
-        and ops.fused_shape_ok(weight.shape[0], weight.shape[1], rank)
+        and ops.fused_shape_ok(shape[0], shape[1], rank)
     )
 
 

@@ -38,6 +38,22 @@ def _stream(t: torch.Tensor) -> int:
     return torch.cuda.current_stream(t.device).cuda_stream
 
 
+class _NoGuard:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_GUARD = _NoGuard()
+
+
+def _on_device(device: torch.device):
+    """Context in which ``device`` is the current GPU: nothing to do (and nothing to pay) when it already is."""
+    return _NO_GUARD if torch.cuda.current_device() == device.index else torch.cuda.device(device)
+
+
 def _workspace(nbytes: int, device: torch.device) -> torch.Tensor:
     return torch.empty(max(int(nbytes), 16), dtype=torch.uint8, device=device)
 
@@ -398,7 +414,7 @@ def qlora_linear_fwd(
     h = torch.empty(M, rank, dtype=torch.bfloat16, device=x.device)
     nbytes = int(lib.ttamd_qlora_linear_fwd_workspace_bytes(M, N, K, rank))
     ws = _workspace(nbytes, x.device)
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         rc = lib.ttamd_qlora_linear_fwd_bf16(
             x.data_ptr(), qdata.data_ptr(), block_scalers.data_ptr(), _ptr(block_scalers_t), lora_a.data_ptr(), lora_b.data_ptr(),
             rank, float(scale), _ptr(bias), y.data_ptr(), h.data_ptr(), M, N, K, ws.data_ptr(), ws.numel(), _stream(x))
@@ -432,7 +448,7 @@ def qlora_linear_bwd(
     ga = torch.empty(rank, K, dtype=torch.bfloat16, device=dev)
     gb = torch.empty(N, rank, dtype=torch.bfloat16, device=dev)
     ws = _workspace(int(lib.ttamd_qlora_linear_bwd_workspace_bytes(M, N, K, rank)), dev)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         rc = lib.ttamd_qlora_linear_bwd_bf16(
             gy.data_ptr(), x.data_ptr(), h.data_ptr(), qdata.data_ptr(), block_scalers.data_ptr(),
             _ptr(transposed[0]) if transposed else None, _ptr(transposed[1]) if transposed else None, lora_a.data_ptr(),
