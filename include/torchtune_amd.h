@@ -564,6 +564,19 @@ int ttamd_tiled_linear_group_fwd_bf16(const void* x, const void* tiled_weights, 
 int ttamd_tiled_linear_group_dx_bf16(const void* const* gy, const int64_t* n_out, int n_members, const void* tiled_weights_t, void* gx,
                                      int64_t M, int64_t K, void* stream);
 
+/*
+ * gx[M, K] = gy[M, N] . Wd (+ gh[M, rank] . lora_a[rank, K]) with Wd [N, K] given as the FORWARD tiles
+ * (tiled[N / 16][K / 32][64 lanes][8], what the forward launch of the same layer read): the grad-input of
+ * F.linear(x, Wd) (torchao LinearNF4.backward / autograd of FakeQuantizedLinear, reached from
+ * torchtune/modules/peft/lora.py:138 and recipes/qat_single_device.py:378-386) without a second, transposed copy of the
+ * weight.  The launch transposes the weight operand on its way out of LDS (ds_read_b64_tr_b16); products and their
+ * order of summation are those of ttamd_tiled_lora_linear_bf16 on tiles of Wd^T, so the two results are equal bit for
+ * bit.  rank a multiple of 8 in [0, 64] (0: gh and lora_a NULL); N and K multiples of 64.
+ */
+int ttamd_tiled_linear_dx_bf16(const void* gy, const void* tiled_weight_fwd, const void* gh, const void* lora_a, int rank, void* gx,
+                               int64_t M, int64_t N, int64_t K, void* stream);
+
+
 /* ------------------------------------------------------------------------------------------------
  * Neighbours of the quantized linears inside a decoder layer (one pass over HBM each, bf16 tensors, fp32 math).
  * Floating-point kernels: results agree with the eager sequences to a tolerance (summation order and hardware

@@ -128,6 +128,7 @@ SIGNATURES = {
     "ttamd_tiled_linear_group_fwd_bf16": (_int, [_c_void_p, _c_void_p, _int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _i64, _i64,
                                                  _c_void_p]),
     "ttamd_tiled_linear_group_dx_bf16": (_int, [_c_void_p, _c_void_p, _int, _c_void_p, _c_void_p, _i64, _i64, _c_void_p]),
+    "ttamd_tiled_linear_dx_bf16": (_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _int, _c_void_p, _i64, _i64, _i64, _c_void_p]),
     "ttamd_fq_per_token_int8_asym": (_int, [_c_void_p, _int, _i64, _i64, _int, _c_void_p, _c_void_p, _c_void_p, _c_void_p]),
     "ttamd_fq_per_group_int4_sym": (_int, [_c_void_p, _int, _i64, _i64, _int, _int, _c_void_p, _c_void_p, _c_void_p]),
     "ttamd_quantize_per_group_int4": (

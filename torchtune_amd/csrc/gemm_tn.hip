@@ -10,6 +10,13 @@
 // apart, one in its MFMA part while the other requests loads and reads operands, swapping at workgroup barriers.
 // LDS layout of a stage: row r of the 32 at r * 512, its 16-byte chunk c in slot c ^ (2 (r % 4)) - applied on the
 // global-address side of the loads - so that the four rows a 16-lane group reads together fall on disjoint banks.
+//
+// Last partial round.  256 CUs take 256 tiles at a time; a launch of, say, 3.5 rounds of tiles leaves half the chip idle
+// for the length of one tile (220 us at 8192 tokens).  With a workspace the tiles beyond the last whole round have their
+// contraction cut into 2 - 8 slices, one workgroup per tile and slice, so that the last round fills the chip with
+// shorter pieces of work; each leaves its tile as fp32 in the workspace and gemm_tn_reduce_kernel adds the slices of a
+// tile in slice order (deterministic), rounds once and stores through the same epilogue.  Taken where the time saved
+// pays for the 256 KiB per tile and slice that go to memory and back (long contractions: training token counts).
 #include <type_traits>
 
 #include "common.h"
@@ -44,15 +51,76 @@ struct TnArgs {
   const uint16_t* B;  // [M, K] bf16
   int M, K;
   int tiles_n, tiles_k;  // tiles_n: all members
+  // workgroups [0, full_tiles) run tiles [0, full_tiles) over the whole contraction; workgroup full_tiles + u runs slice
+  // u / tail_tiles of tile full_tiles + u % tail_tiles and leaves it in slabs (slices == 1: no tile is cut, tail_tiles == 0)
+  int full_tiles, tail_tiles, slices;
+  float* slabs;  // [tail_tiles][slices][NT * MT][512 threads][4] fp32
 };
 
 constexpr int kTnStage = 32768;  // 32 rows x 512 bytes of A, then the same of B
 constexpr int kTnLds = 4 * kTnStage;
 constexpr int kLgkmMax = 15;  // the counter field of s_waitcnt holds 4 bits: waiting for fewer outstanding reads is always safe
 
+constexpr int kTnMT = 8, kTnNT = 4;  // 16 x 16 MFMA tiles per wave: MT along the rows of C (columns of A), NT along its columns
+
+// Tile `id` of a launch: the member it belongs to and its first row (within the member) and column.
+__device__ __forceinline__ void tn_locate(const TnArgs& g, int id, int& which, int& n0, int& k0) {
+  int tile_n, tile_k;
+  // tile ids are dealt round-robin to the 8 XCDs: every XCD gets a band of row tiles and walks it column by column
+  if ((g.tiles_n & 7) == 0) {
+    const int xcd = id & 7, slot = id >> 3, band = g.tiles_n >> 3;
+    tile_n = xcd * band + slot % band;
+    tile_k = slot / band;
+  } else {
+    tile_n = id / g.tiles_k;
+    tile_k = id % g.tiles_k;
+  }
+  which = 0;  // uniform over the workgroup
+#pragma unroll
+  for (int q = 0; q < kGroupMax - 1; ++q)
+    if (q < g.n - 1 && tile_n >= g.tile_end[q]) which = q + 1;
+  n0 = (tile_n - (which ? g.tile_end[which - 1] : 0)) * 256;
+  k0 = tile_k * 256;
+}
+
+// acc[j][i][v] = C[n][k], n = n0 + 128 wm + 16 i + l15, k = k0 + 64 wn + 16 j + 4 g4 + v.  Each wave transposes its
+// 128 x 64 band through LDS (128 KiB for the eight waves) and writes whole 128-byte row segments.
+__device__ __forceinline__ void tn_store_tile(const f32x4_t (&acc)[kTnNT][kTnMT], char* smem, uint16_t* C, int K, int n0, int k0) {
+  const int lane = threadIdx.x & 63;
+  const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wm = wv >> 2, wn = wv & 3;
+  const int l15 = lane & 15, g4 = lane >> 4;
+  char* band = smem + wv * 16384;  // 128 rows x 128 bytes
+#pragma unroll
+  for (int j = 0; j < kTnNT; ++j)
+#pragma unroll
+    for (int i = 0; i < kTnMT; ++i) {
+      const int r = 16 * i + l15;
+      u32x2_t o;
+      o.x = pack_bf16x2(acc[j][i][0], acc[j][i][1]);
+      o.y = pack_bf16x2(acc[j][i][2], acc[j][i][3]);
+      *reinterpret_cast<u32x2_t*>(band + r * 128 + (((2 * j + (g4 >> 1)) ^ (r & 7)) << 4) + 8 * (g4 & 1)) = o;
+    }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  const int c = lane & 7;
+  uint16_t* crow = C + k0 + wn * 64 + 8 * c;
+  const int nrow0 = n0 + 128 * wm;
+#pragma unroll 8
+  for (int t = 0; t < 16; ++t) {
+    const int r = 8 * t + (lane >> 3);
+    const u32x4_t v = *reinterpret_cast<const u32x4_t*>(band + r * 128 + ((c ^ (r & 7)) << 4));
+    *reinterpret_cast<u32x4_t*>(crow + (int64_t)(nrow0 + r) * K) = v;
+  }
+}
+
+// Steps [begin, end) of slice `slice` of `slices` over nk steps (every slice non-empty when slices <= nk).
+__device__ __forceinline__ int tn_slice_begin(int slice, int slices, int nk) { return (int)(((int64_t)slice * nk) / slices); }
+
 __global__ __launch_bounds__(512) void gemm_tn_kernel(const TnArgs g) {
 #if defined(__HIP_DEVICE_COMPILE__)
-  constexpr int MT = 8, NT = 4;  // 16 x 16 MFMA tiles per wave: MT along the rows of C (columns of A), NT along its columns
+  constexpr int MT = kTnMT, NT = kTnNT;
   extern __shared__ __attribute__((aligned(16))) char smem[];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -60,28 +128,22 @@ __global__ __launch_bounds__(512) void gemm_tn_kernel(const TnArgs g) {
   const int wm = wv >> 2, wn = wv & 3;
   const int l15 = lane & 15, g4 = lane >> 4;
 
-  int tile_n, tile_k;
-  {
-    // workgroup ids are dealt round-robin to the 8 XCDs: every XCD gets a band of row tiles and walks it column by column
-    const int id = blockIdx.x;
-    if ((g.tiles_n & 7) == 0) {
-      const int xcd = id & 7, slot = id >> 3, band = g.tiles_n >> 3;
-      tile_n = xcd * band + slot % band;
-      tile_k = slot / band;
-    } else {
-      tile_n = id / g.tiles_k;
-      tile_k = id % g.tiles_k;
-    }
+  const int nk_all = g.M >> 5;  // steps of 32 rows
+  int id = blockIdx.x, t_begin = 0, nk = nk_all;  // this workgroup runs steps [t_begin, nk)
+  int slab = -1;
+  if (id >= g.full_tiles) {
+    const int u = id - g.full_tiles;
+    const int slice = u / g.tail_tiles, tl = u - slice * g.tail_tiles;
+    id = g.full_tiles + tl;
+    t_begin = tn_slice_begin(slice, g.slices, nk_all);
+    nk = tn_slice_begin(slice + 1, g.slices, nk_all);
+    slab = tl * g.slices + slice;
   }
-  int which = 0;  // uniform over the workgroup
-#pragma unroll
-  for (int q = 0; q < kGroupMax - 1; ++q)
-    if (q < g.n - 1 && tile_n >= g.tile_end[q]) which = q + 1;
+  int which, n0, k0;
+  tn_locate(g, id, which, n0, k0);
   const uint16_t* const A = g.A[which];
   uint16_t* const C = g.C[which];
   const int N = g.N[which];
-  const int n0 = (tile_n - (which ? g.tile_end[which - 1] : 0)) * 256, k0 = tile_k * 256;  // n0: within the member
-  const int nk = g.M >> 5;  // steps of 32 rows
 
   // ---- loads: per step and wave two instructions for A (rows 4 wv .. + 3 of the 32, two rows of 512 bytes each) and two
   //      for B; lane l of an instruction fetches chunk (l % 32) ^ (2 (row % 4)) of row l / 32 of its pair
@@ -157,15 +219,15 @@ __global__ __launch_bounds__(512) void gemm_tn_kernel(const TnArgs g) {
   //      wave's own loads of step t + 1 must have landed (the other waves read them after the next barrier): they came
   //      from M(t - 2), newer are the 4 + 4 loads of M(t - 1) and M(t).  The transposing reads are written in assembly, so
   //      the wait for them is explicit too and names the registers it releases.
-  issue(0);
-  issue(1);
-  issue(2);
-  asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");  // step 0 landed everywhere
+  issue(t_begin);
+  issue(t_begin + 1);
+  issue(t_begin + 2);
+  asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");  // the first step landed everywhere
   if (wm == 1) asm volatile("s_barrier" ::: "memory");
   // one copy of the loop per wave group: the two differ in one wait, and a branch per step costs 2 - 4 %
   auto main_loop = [&](auto lgkm) {
     constexpr bool kLgkm = decltype(lgkm)::value;
-    for (int t = 0; t < nk; ++t) {
+    for (int t = t_begin; t < nk; ++t) {
       issue(t + 3);
       read_step(t);
       __builtin_amdgcn_sched_barrier(0);
@@ -204,34 +266,48 @@ __global__ __launch_bounds__(512) void gemm_tn_kernel(const TnArgs g) {
   if (wm == 0) asm volatile("s_barrier" ::: "memory");
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the clamped requests of the last steps
 
-  // ---- epilogue: acc[j][i][v] = C[n][k], n = n0 + 128 wm + 16 i + l15, k = k0 + 64 wn + 16 j + 4 g4 + v.  Each wave
-  //      transposes its 128 x 64 band through LDS and writes whole 128-byte row segments.
+  // ---- a slice leaves its partial tile as fp32, in the accumulators' own order: 16 bytes per lane, whole lines per wave
+  if (slab >= 0) {
+    f32x4_t* dst = reinterpret_cast<f32x4_t*>(g.slabs) + (int64_t)slab * (NT * MT * 512) + tid;
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int i = 0; i < MT; ++i) dst[(j * MT + i) * 512] = acc[j][i];
+    return;
+  }
+  // ---- epilogue
   __syncthreads();
-  {
-    char* band = smem + wv * 16384;  // 128 rows x 128 bytes
+  tn_store_tile(acc, smem, C, g.K, n0, k0);
+#endif
+}
+
+// Adds the slices of one tail tile in slice order and stores the tile (one workgroup per tile, the lanes as in gemm_tn_kernel).
+__global__ __launch_bounds__(512) void gemm_tn_reduce_kernel(const TnArgs g) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  constexpr int MT = kTnMT, NT = kTnNT;
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const int tid = threadIdx.x;
+  const int tl = blockIdx.x;
+  int which, n0, k0;
+  tn_locate(g, g.full_tiles + tl, which, n0, k0);
+  f32x4_t acc[NT][MT];
+  const f32x4_t* src = reinterpret_cast<const f32x4_t*>(g.slabs) + (int64_t)tl * g.slices * (NT * MT * 512) + tid;
+#pragma unroll
+  for (int j = 0; j < NT; ++j)
+#pragma unroll
+    for (int i = 0; i < MT; ++i) acc[j][i] = __builtin_nontemporal_load(src + (j * MT + i) * 512);
+  for (int sl = 1; sl < g.slices; ++sl) {
+    src += NT * MT * 512;
 #pragma unroll
     for (int j = 0; j < NT; ++j)
 #pragma unroll
       for (int i = 0; i < MT; ++i) {
-        const int r = 16 * i + l15;
-        u32x2_t o;
-        o.x = pack_bf16x2(acc[j][i][0], acc[j][i][1]);
-        o.y = pack_bf16x2(acc[j][i][2], acc[j][i][3]);
-        *reinterpret_cast<u32x2_t*>(band + r * 128 + (((2 * j + (g4 >> 1)) ^ (r & 7)) << 4) + 8 * (g4 & 1)) = o;
+        const f32x4_t v = __builtin_nontemporal_load(src + (j * MT + i) * 512);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[j][i][e] += v[e];
       }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    const int c = lane & 7;
-    uint16_t* crow = C + k0 + wn * 64 + 8 * c;
-    const int nrow0 = n0 + 128 * wm;
-#pragma unroll 8
-    for (int t = 0; t < 16; ++t) {
-      const int r = 8 * t + (lane >> 3);
-      const u32x4_t v = *reinterpret_cast<const u32x4_t*>(band + r * 128 + ((c ^ (r & 7)) << 4));
-      *reinterpret_cast<u32x4_t*>(crow + (int64_t)(nrow0 + r) * g.K) = v;
-    }
   }
+  tn_store_tile(acc, smem, g.C[which], g.K, n0, k0);
 #endif
 }
 
@@ -250,22 +326,67 @@ using namespace ttamd;
 extern "C" int ttamd_gemm_tn_applies(int64_t M, int64_t N, int64_t K) { return gemm_tn_applies(M, N, K) ? 1 : 0; }
 
 namespace {
-int launch_gemm_tn(TnArgs& g, hipStream_t s) {
+// How the tiles beyond the last whole round of 256 are cut.  A tile of nk steps takes about 0.8 us per step; cutting the
+// tail's contraction into `slices` saves (1 - 1 / slices) of that once per launch and costs a reduce launch plus
+// 256 KiB per tile and slice written and read back (about 0.1 us each at the rate such a burst moves).  Taken when the
+// saving is at least one and a half times the cost; slices of fewer than 32 steps are not made.
+struct TnPlan {
+  int full_tiles, tail_tiles, slices;
+};
+constexpr int kTnChipTiles = 256;
+TnPlan plan_tn(int64_t tiles, int64_t nk) {
+  const int tail = (int)(tiles % kTnChipTiles);
+  TnPlan none = {(int)tiles, 0, 1};
+  if (tail == 0) return none;
+  int slices = kTnChipTiles / tail;
+  slices = slices > 8 ? 8 : slices;
+  while (slices > 1 && nk / slices < 32) --slices;
+  if (slices < 2) return none;
+  const double saved = 0.8 * (double)nk * (1.0 - 1.0 / slices);
+  const double cost = 16.0 + 0.105 * (double)tail * slices;
+  if (saved < 1.5 * cost) return none;
+  return TnPlan{(int)(tiles - tail), tail, slices};
+}
+size_t tn_slab_bytes(const TnPlan& p) { return (size_t)p.tail_tiles * (p.slices > 1 ? p.slices : 0) * 256 * 256 * sizeof(float); }
+
+int launch_gemm_tn(TnArgs& g, void* workspace, size_t workspace_bytes, hipStream_t s) {
+  const int64_t tiles = (int64_t)g.tiles_n * g.tiles_k;
+  TnPlan plan = plan_tn(tiles, g.M >> 5);
+  if (plan.slices > 1 && (workspace == nullptr || workspace_bytes < tn_slab_bytes(plan))) plan = TnPlan{(int)tiles, 0, 1};
+  TT_REQUIRE(plan.slices == 1 || aligned16(workspace), "gemm_tn: workspace must be 16-byte aligned");
+  g.full_tiles = plan.full_tiles;
+  g.tail_tiles = plan.tail_tiles;
+  g.slices = plan.slices;
+  g.slabs = reinterpret_cast<float*>(workspace);
+  const int64_t units = (int64_t)plan.full_tiles + (int64_t)plan.tail_tiles * (plan.slices > 1 ? plan.slices : 0);
   // the LDS limit is a per-device attribute of the function: set it for the current device once (a race only repeats the call)
   static bool attr_set[64] = {};
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = -1;
   if (dev < 0 || !attr_set[dev]) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tn_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kTnLds);
-    if (e != hipSuccess) return fail(TTAMD_ELAUNCH, "gemm_tn: cannot reserve %d bytes of LDS: %s", kTnLds, hipGetErrorString(e));
+    for (const void* fn : {reinterpret_cast<const void*>(&gemm_tn_kernel), reinterpret_cast<const void*>(&gemm_tn_reduce_kernel)}) {
+      hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kTnLds);
+      if (e != hipSuccess) return fail(TTAMD_ELAUNCH, "gemm_tn: cannot reserve %d bytes of LDS: %s", kTnLds, hipGetErrorString(e));
+    }
     if (dev >= 0) attr_set[dev] = true;
   }
-  gemm_tn_kernel<<<dim3((unsigned)(g.tiles_n * g.tiles_k)), dim3(512), kTnLds, s>>>(g);
-  return check_launch("gemm_tn");
+  gemm_tn_kernel<<<dim3((unsigned)units), dim3(512), kTnLds, s>>>(g);
+  if (int rc = check_launch("gemm_tn")) return rc;
+  if (plan.slices > 1) {
+    gemm_tn_reduce_kernel<<<dim3((unsigned)plan.tail_tiles), dim3(512), kTnLds, s>>>(g);
+    return check_launch("gemm_tn_reduce");
+  }
+  return TTAMD_OK;
 }
 }  // namespace
 
-extern "C" int ttamd_gemm_tn_bf16(const void* a, const void* b, void* c, int64_t M, int64_t N, int64_t K, void* stream) {
+extern "C" size_t ttamd_gemm_tn_workspace_bytes(int64_t M, int64_t n_total, int64_t K) {
+  if (M < 32 || n_total <= 0 || K <= 0 || n_total % 256 != 0 || K % 256 != 0) return 0;
+  return tn_slab_bytes(plan_tn((n_total / 256) * (K / 256), M >> 5));
+}
+
+extern "C" int ttamd_gemm_tn_ws_bf16(const void* a, const void* b, void* c, int64_t M, int64_t N, int64_t K, void* workspace,
+                                     size_t workspace_bytes, void* stream) {
   TT_REQUIRE(a && b && c && aligned16(a) && aligned16(b) && aligned16(c), "gemm_tn: pointers must be non-null and 16-byte aligned");
   TT_REQUIRE(M > 0 && N > 0 && K > 0, "gemm_tn: bad shape M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
   if (!gemm_tn_applies(M, N, K))
@@ -280,11 +401,15 @@ extern "C" int ttamd_gemm_tn_bf16(const void* a, const void* b, void* c, int64_t
   g.M = (int)M; g.K = (int)K;
   g.tiles_n = g.tile_end[0] = (int)(N / 256);
   g.tiles_k = (int)(K / 256);
-  return launch_gemm_tn(g, reinterpret_cast<hipStream_t>(stream));
+  return launch_gemm_tn(g, workspace, workspace_bytes, reinterpret_cast<hipStream_t>(stream));
 }
 
-extern "C" int ttamd_gemm_tn_group_bf16(const void* const* a, const void* b, void* const* c, int n_members, int64_t M,
-                                        const int64_t* N, int64_t K, void* stream) {
+extern "C" int ttamd_gemm_tn_bf16(const void* a, const void* b, void* c, int64_t M, int64_t N, int64_t K, void* stream) {
+  return ttamd_gemm_tn_ws_bf16(a, b, c, M, N, K, nullptr, 0, stream);
+}
+
+extern "C" int ttamd_gemm_tn_group_ws_bf16(const void* const* a, const void* b, void* const* c, int n_members, int64_t M,
+                                           const int64_t* N, int64_t K, void* workspace, size_t workspace_bytes, void* stream) {
   TT_REQUIRE(a && b && c && N && aligned16(b), "gemm_tn_group: null or misaligned pointer argument");
   TT_REQUIRE(n_members >= 1 && n_members <= kGroupMax, "gemm_tn_group: %d members (1 .. %d)", n_members, kGroupMax);
   TT_REQUIRE(M > 0 && K > 0, "gemm_tn_group: bad shape M=%lld K=%lld", (long long)M, (long long)K);
@@ -307,5 +432,10 @@ extern "C" int ttamd_gemm_tn_group_bf16(const void* const* a, const void* b, voi
   g.M = (int)M; g.K = (int)K;
   g.tiles_n = (int)tiles;
   g.tiles_k = (int)(K / 256);
-  return launch_gemm_tn(g, reinterpret_cast<hipStream_t>(stream));
+  return launch_gemm_tn(g, workspace, workspace_bytes, reinterpret_cast<hipStream_t>(stream));
+}
+
+extern "C" int ttamd_gemm_tn_group_bf16(const void* const* a, const void* b, void* const* c, int n_members, int64_t M,
+                                        const int64_t* N, int64_t K, void* stream) {
+  return ttamd_gemm_tn_group_ws_bf16(a, b, c, n_members, M, N, K, nullptr, 0, stream);
 }

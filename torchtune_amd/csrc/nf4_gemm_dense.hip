@@ -320,6 +320,11 @@ struct DenseArgs {
   int M, Nout, Kc;  // Nout, Kc: totals
   int lw_row_major, ldlx;
   int tiles_m, tiles_n;
+  // grad-input from the FORWARD tiles: Wt holds tiled[n / 16][k / 32][lane][8] of the weight W [Kc, Nout] (rows n = this
+  // launch's contraction, columns k = its output columns) and the kernel transposes on its way out of LDS.  w_paired:
+  // those tiles are the gated pair's (128 columns of the one member, then 128 of the other): the contraction then visits
+  // the two segments alternately, 128 wide.
+  int w_tr, w_paired;
   uint16_t* act;    // gated launches only: [M, out[0].width] bf16 = silu(out 0) * out 1
   // SwiGLU-backward launches only (one output): the result is the gradient of silu(gate) * up; out[0].C receives the
   // gradient of gate and sw_gup that of up, both [M, out[0].width] like gate and up themselves
@@ -344,7 +349,15 @@ constexpr int kLdsDense = kWBase + 4 * kWStage;
 // is the gradient of silu(gate) * up and is not stored; each 16-byte piece of it meets the same piece of gate and up
 // on its way out and the launch writes the gradients of gate and up instead, the arithmetic of ttamd_swiglu_bwd_bf16 on
 // the rounded result, bit for bit.
-template <bool LW_ROW_MAJOR, int EPI>
+// W_TR (grad-input launches only): the weight operand comes from the tiles the forward launch of the same layer read.
+// A stage then holds, for the 32 rows n of a step, the eight 1 KiB pieces that cover the tile's 256 columns k (row
+// blocks 2 s and 2 s + 1, pieces 8 tile_n .. + 7 of each: 8 KiB contiguous per block), and a lane gathers its operand -
+// 8 consecutive n of one column k - with two ds_read_b64_tr_b16, each of which hands lane i of a 16-lane group element
+// i % 4 of the 8 bytes lane 4 t + i / 4 points at (t = 0..3).  Inside a piece the 16-byte chunk of (row n % 16 = p,
+// k-group kg) sits in slot (p ^ 4 (kg & 1)) + 16 kg (applied on the global-address side of the direct-to-LDS loads), so
+// that the 32 lanes served together touch 64 different banks.  Same products, same order of summation as the launch on
+// tiles of W^T: the results are equal bit for bit.
+template <bool LW_ROW_MAJOR, int EPI, bool W_TR = false>
 __device__ __forceinline__ void gemm_dense_tile(const DenseArgs g) {
 #if defined(__HIP_DEVICE_COMPILE__)
   constexpr bool GATED = EPI == kEpiGated;
@@ -395,12 +408,29 @@ __device__ __forceinline__ void gemm_dense_tile(const DenseArgs g) {
   };
   set_segment();
   const int nblocks = g.Nout >> 4;
-  int T0 = (n0 >> 4) + 2 * wv, T1 = T0 + 1;
-  T0 = T0 < nblocks ? T0 : nblocks - 1;
-  T1 = T1 < nblocks ? T1 : nblocks - 1;
-  const char* wsrc0 = g.Wt + (int64_t)T0 * ((int64_t)nk * 1024);
-  const char* wsrc1 = g.Wt + (int64_t)T1 * ((int64_t)nk * 1024);
-  const uint32_t lane16 = (uint32_t)lane * 16u;
+  const char* wsrc0;
+  const char* wsrc1;
+  int64_t wstep;  // bytes from one k-step's pieces to the next
+  uint32_t lane16;
+  if constexpr (W_TR) {
+    const int npieces = g.Nout >> 5;  // 32-wide pieces along the weight's columns k
+    int p0 = 8 * tile_n + 2 * (wv & 3), p1 = p0 + 1;
+    p0 = p0 < npieces ? p0 : npieces - 1;
+    p1 = p1 < npieces ? p1 : npieces - 1;
+    const int64_t blk = (int64_t)(wv >> 2) * npieces;  // row block 2 s + (wv >> 2) of step s
+    wsrc0 = g.Wt + (blk + p0) * 1024;
+    wsrc1 = g.Wt + (blk + p1) * 1024;
+    wstep = (int64_t)npieces * 2048;
+    lane16 = (uint32_t)(((lane & 15) ^ (((lane >> 4) & 1) << 2)) | (lane & 48)) * 16u;
+  } else {
+    int T0 = (n0 >> 4) + 2 * wv, T1 = T0 + 1;
+    T0 = T0 < nblocks ? T0 : nblocks - 1;
+    T1 = T1 < nblocks ? T1 : nblocks - 1;
+    wsrc0 = g.Wt + (int64_t)T0 * ((int64_t)nk * 1024);
+    wsrc1 = g.Wt + (int64_t)T1 * ((int64_t)nk * 1024);
+    wstep = 1024;
+    lane16 = (uint32_t)lane * 16u;
+  }
 
   auto dma16 = [&](uint32_t voff, const char* base, uint32_t lds, int imm) {
     asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
@@ -410,20 +440,27 @@ __device__ __forceinline__ void gemm_dense_tile(const DenseArgs g) {
   auto issue_w = [&](int t, int stage) {
     const int tk = t < nk ? t : nk - 1;
     const uint32_t sw = lds0 + kWBase + stage * kWStage + wv * 2048;
-    dma16(lane16, wsrc0 + (int64_t)tk * 1024, sw, 0);
-    dma16(lane16, wsrc1 + (int64_t)tk * 1024, sw, 1024);
+    dma16(lane16, wsrc0 + (int64_t)tk * wstep, sw, 0);
+    dma16(lane16, wsrc1 + (int64_t)tk * wstep, sw, 1024);
   };
   // entries are requested in increasing order (past the end: the last one again), so the segment only moves forward
   auto issue_a = [&](int T2, int entry) {
     const int tk = T2 < nk2 ? T2 : nk2 - 1;
-    while (tk >= seg_end) {
-      ++seg;
-      seg_begin = seg_end;
-      seg_end += g.seg[seg].Kc >> 6;
-      a_base = reinterpret_cast<const char*>(g.seg[seg].X);
-      set_segment();
+    const char* xb;
+    if (W_TR && g.w_paired) {
+      // two segments of equal width, visited 128 columns (two entries) at a time: entry tk is entry
+      // 2 (tk / 4) + tk % 2 of segment (tk / 2) % 2; the row pitch is the same for both
+      xb = reinterpret_cast<const char*>(g.seg[(tk >> 1) & 1].X) + ((int64_t)(((tk >> 2) << 1) + (tk & 1)) << 7);
+    } else {
+      while (tk >= seg_end) {
+        ++seg;
+        seg_begin = seg_end;
+        seg_end += g.seg[seg].Kc >> 6;
+        a_base = reinterpret_cast<const char*>(g.seg[seg].X);
+        set_segment();
+      }
+      xb = a_base + ((int64_t)(tk - seg_begin) << 7);  // + 64 elements * 2 bytes per entry
     }
-    const char* xb = a_base + ((int64_t)(tk - seg_begin) << 7);  // + 64 elements * 2 bytes per entry
     const uint32_t sa = lds0 + entry * kAEntry + wv * 4096;
     dma16(a_off[0], xb, sa, 0);
     dma16(a_off[1], xb, sa, 1024);
@@ -445,12 +482,34 @@ __device__ __forceinline__ void gemm_dense_tile(const DenseArgs g) {
 #pragma unroll
       for (int v = 0; v < 4; ++v) acc[j][i][v] = 0.f;
 
+  // W_TR: lane (l15, g4) of a transposing read points at row n = 8 g4 + l15 / 4 (+ 4 for the second half) of the step,
+  // columns 4 (l15 % 4) .. + 3 of the wave's block j: piece 2 wn + j / 2 of row block g4 / 2, k-group 2 (j % 2) + (l15 % 4) / 2
+  int wtr[2] = {0, 0};
+  if constexpr (W_TR) {
+    const int c = l15 & 3, kg1 = c >> 1;
+    const int np = 8 * (g4 & 1) + (l15 >> 2);
+#pragma unroll
+    for (int h2 = 0; h2 < 2; ++h2)
+      wtr[h2] = kWBase + (g4 >> 1) * 8192 + 2 * wn * 1024 + 256 * kg1 + (((np + 4 * h2) ^ (4 * kg1)) << 4) + 8 * (c & 1);
+  }
   bf16x8_t xf[MT], wf[NT];
   auto read_step = [&](int entry, int hf, int wstage) {
     const char* sw = smem + wstage * kWStage;
     const char* sa = smem + entry * kAEntry + xo[hf];
+    if constexpr (W_TR) {
 #pragma unroll
-    for (int j = 0; j < NT; ++j) wf[j] = *reinterpret_cast<const bf16x8_t*>(sw + wo + j * 1024);
+      for (int j = 0; j < NT; ++j) {
+        typedef short s16x4_t __attribute__((ext_vector_type(4)));
+        typedef short s16x8_t __attribute__((ext_vector_type(8)));
+        const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(sw + wtr[0] + j * 512));
+        const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(sw + wtr[1] + j * 512));
+        const s16x8_t both = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        wf[j] = __builtin_bit_cast(bf16x8_t, both);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < NT; ++j) wf[j] = *reinterpret_cast<const bf16x8_t*>(sw + wo + j * 1024);
+    }
 #pragma unroll
     for (int i = 0; i < MT; ++i) xf[i] = *reinterpret_cast<const bf16x8_t*>(sa + i * 2048);
   };
@@ -717,6 +776,8 @@ __global__ __launch_bounds__(512) void nf4_gemm_dense_kernel(const DenseArgs g) 
 }
 // grad-input launch (adapter weights [r, K]) whose result goes on through the backward of silu(gate) * up
 __global__ __launch_bounds__(512) void nf4_gemm_dense_swiglu_bwd_kernel(const DenseArgs g) { gemm_dense_tile<false, kEpiSwigluBwd>(g); }
+// grad-input launch on the forward launch's tiles
+__global__ __launch_bounds__(512) void nf4_gemm_dense_tr_kernel(const DenseArgs g) { gemm_dense_tile<false, kEpiPlain, true>(g); }
 
 // mode 0 / 2 / 1: nf4_expand_tiled_kernel<mode> over the members' stacked blocks of 16 output columns; mode 3: the
 // transposed kernel over the members' 32-row steps (nout = K, kc = N of each member: codes and scalers in the weight's
@@ -771,13 +832,22 @@ int launch_dense(DenseArgs& g, hipStream_t s) {
   if (dev < 0 || !attr_set[dev]) {
     for (const void* fn : {reinterpret_cast<const void*>(&nf4_gemm_dense_kernel<true>), reinterpret_cast<const void*>(&nf4_gemm_dense_kernel<false>),
                            reinterpret_cast<const void*>(&nf4_gemm_dense_kernel<true, true>),
-                           reinterpret_cast<const void*>(&nf4_gemm_dense_swiglu_bwd_kernel)}) {
+                           reinterpret_cast<const void*>(&nf4_gemm_dense_swiglu_bwd_kernel),
+                           reinterpret_cast<const void*>(&nf4_gemm_dense_tr_kernel)}) {
       hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsDense);
       if (e != hipSuccess) return fail(TTAMD_ELAUNCH, "nf4_gemm_dense: cannot reserve %d bytes of LDS: %s", kLdsDense, hipGetErrorString(e));
     }
     if (dev >= 0) attr_set[dev] = true;
   }
   const dim3 grid((unsigned)(g.tiles_m * g.tiles_n)), block(512);
+  if (g.w_tr) {
+    TT_REQUIRE(!g.lw_row_major && !g.act && !g.sw_gup && g.nout == 1 && g.Kc % 64 == 0 && g.Nout % 64 == 0,
+               "nf4_gemm_dense: the launch on forward tiles is a plain grad-input launch");
+    TT_REQUIRE(!g.w_paired || (g.nseg == 2 && g.seg[0].Kc == g.seg[1].Kc && g.seg[0].Kc % 128 == 0),
+               "nf4_gemm_dense: paired forward tiles belong to two members of equal width, a multiple of 128");
+    nf4_gemm_dense_tr_kernel<<<grid, block, kLdsDense, s>>>(g);
+    return check_launch("nf4_gemm_dense_tr");
+  }
   if (g.act) {
     TT_REQUIRE(g.lw_row_major && g.nout == 2 && (g.nad == 2 || g.nad == 0) && g.nseg == 1 && g.out[0].width == g.out[1].width &&
                    g.out[0].width % 128 == 0 && g.Nout == 2 * g.out[0].width,
@@ -1056,6 +1126,40 @@ int tiled_linear(const void* x, const void* tiled_weight, const void* lx, const 
   return launch_dense(g, reinterpret_cast<hipStream_t>(stream));
 }
 }  // namespace
+
+extern "C" int ttamd_tiled_linear_dx_bf16(const void* gy, const void* tiled_weight_fwd, const void* gh, const void* lora_a, int rank,
+                                          void* gx, int64_t M, int64_t N, int64_t K, void* stream) {
+  TT_REQUIRE(gy && tiled_weight_fwd && gx && aligned16(gy) && aligned16(tiled_weight_fwd) && aligned16(gx),
+             "tiled_linear_dx: pointers must be non-null and 16-byte aligned");
+  TT_REQUIRE(M > 0 && N > 0 && K > 0 && N % 64 == 0 && K % 64 == 0, "tiled_linear_dx: N (%lld) and K (%lld) must be positive multiples of 64",
+             (long long)N, (long long)K);
+  if (!(M * N * 2 < (int64_t(1) << 32) && N * 2 * 256 < (int64_t(1) << 32) && M < (1 << 30) && K < (1 << 30)))
+    return fail(TTAMD_EUNSUPPORTED, "tiled_linear_dx: operands too large for 32-bit offsets (M=%lld N=%lld)", (long long)M, (long long)N);
+  TT_REQUIRE(rank >= 0 && rank % 8 == 0 && rank <= 64, "tiled_linear_dx: the adapter rank (%d) must be a multiple of 8, at most 64", rank);
+  TT_REQUIRE(rank == 0 || (gh && lora_a && aligned16(gh) && aligned16(lora_a)), "tiled_linear_dx: adapter operands must be non-null and 16-byte aligned");
+  DenseArgs g = {};
+  g.nseg = g.nout = 1;
+  g.seg[0].X = reinterpret_cast<const uint16_t*>(gy);
+  g.seg[0].Kc = (int)N;
+  g.out[0].C = reinterpret_cast<uint16_t*>(gx);
+  g.out[0].n_begin = 0;
+  g.out[0].width = (int)K;
+  if (rank > 0) {
+    g.nad = 1;
+    g.ad[0].lX = reinterpret_cast<const uint16_t*>(gh);
+    g.ad[0].lW = reinterpret_cast<const uint16_t*>(lora_a);
+    g.ad[0].R = rank;
+    g.ad[0].n_begin = 0;
+    g.ad[0].n_end = (int)K;
+    g.ad[0].lscale = 1.0f;
+  }
+  g.Wt = reinterpret_cast<const char*>(tiled_weight_fwd);
+  g.M = (int)M; g.Nout = (int)K; g.Kc = (int)N;
+  g.lw_row_major = 0;
+  g.ldlx = rank;
+  g.w_tr = 1;
+  return launch_dense(g, reinterpret_cast<hipStream_t>(stream));
+}
 
 extern "C" int ttamd_tiled_linear_bf16(const void* x, const void* tiled_weight, const void* bias, void* y, int64_t M, int64_t n_out,
                                        int64_t k_contract, void* stream) {

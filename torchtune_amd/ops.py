@@ -878,6 +878,36 @@ def tiled_lora_linear(x: torch.Tensor, tiled: torch.Tensor, n_out: int, lx: torc
     return y
 
 
+def tiled_linear_dx(gy: torch.Tensor, tiled_fwd: torch.Tensor, K: int, gh: Optional[torch.Tensor] = None,
+                    lora_a: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``gx = gy @ Wd (+ gh @ lora_a)`` with ``Wd`` [N, K] given as the FORWARD tiles (what ``tiled_linear`` / the expanded
+    NF4 forward read): the grad-input without a transposed copy of the weight, bit-equal to the launch on tiles of
+    ``Wd.T``.  ``tiled_fwd`` may be longer than N * K elements (a workspace whose head holds the tiles)."""
+    gy = _bf16_2d(gy, "tiled_linear_dx")
+    M, N = gy.shape
+    if tiled_fwd.numel() * tiled_fwd.element_size() < 2 * N * K or not tiled_fwd.is_contiguous():
+        raise ValueError(f"tiled_linear_dx: the tiled weight must be contiguous and hold {N} x {K} bfloat16 elements")
+    r = 0
+    if gh is not None:
+        gh = _bf16_2d(gh, "tiled_linear_dx")
+        lora_a = _bf16_2d(lora_a, "tiled_linear_dx")
+        r = gh.shape[1]
+        if gh.shape[0] != M or tuple(lora_a.shape) != (r, K) or r % 8 != 0 or not 0 < r <= 64:
+            raise ValueError(f"tiled_linear_dx: adapter operands {tuple(gh.shape)} / {tuple(lora_a.shape)} do not fit M={M}, K={K}")
+    gx = torch.empty(M, K, dtype=torch.bfloat16, device=gy.device)
+    lib = _lib.load()
+    with _on_device(gy.device):
+        events = _gemm_timer("tiled", M, K, N, 0) if _gemm_timer is not None else None
+        if events:
+            events[0].record()
+        rc = lib.ttamd_tiled_linear_dx_bf16(gy.data_ptr(), tiled_fwd.data_ptr(), _ptr(gh), _ptr(lora_a), r, gx.data_ptr(), M, N, K,
+                                            _stream(gy))
+        if events:
+            events[1].record()
+    _lib.check(rc, "tiled_linear_dx")
+    return gx
+
+
 def gemm_tn_applies(M: int, N: int, K: int) -> bool:
     """Shapes ``gemm_tn`` serves: M a multiple of 32, N and K multiples of 256."""
     return bool(_lib.load().ttamd_gemm_tn_applies(M, N, K))
