@@ -524,6 +524,23 @@ int ttamd_gemm_tn_bf16(const void* a, const void* b, void* c, int64_t M, int64_t
  */
 int ttamd_gemm_tn_group_bf16(const void* const* a, const void* b, void* const* c, int n_members, int64_t M, const int64_t* N,
                              int64_t K, void* stream);
+
+/*
+ * The same two products with a workspace for the last partial round of tiles.  The 256 CUs take 256 output tiles at a
+ * time; when the tile count is not a multiple of 256 (3.5 rounds on a 4096 x 14336 gradient) part of the chip idles for
+ * the length of one tile.  Given ttamd_gemm_tn_workspace_bytes(M, n_total, K) bytes (n_total: N, or the sum of the
+ * members' N[i]), the tiles beyond the last whole round have their contraction cut into 2 - 8 slices (one workgroup per
+ * tile and slice, fp32 partial tiles in the workspace) and a second launch adds a tile's slices in slice order, rounds
+ * once and stores: deterministic; the sliced tiles differ from the unsliced launch in the order of their fp32 sums only.
+ * The query returns 0 where slicing does not pay (short contractions, whole rounds); a smaller workspace, or NULL, runs
+ * the unsliced launch (= the entry points above).  The reference has no counterpart (autograd calls a dense GEMM).
+ */
+size_t ttamd_gemm_tn_workspace_bytes(int64_t M, int64_t n_total, int64_t K);
+int ttamd_gemm_tn_ws_bf16(const void* a, const void* b, void* c, int64_t M, int64_t N, int64_t K, void* workspace,
+                          size_t workspace_bytes, void* stream);
+int ttamd_gemm_tn_group_ws_bf16(const void* const* a, const void* b, void* const* c, int n_members, int64_t M, const int64_t* N,
+                                int64_t K, void* workspace, size_t workspace_bytes, void* stream);
+
 int ttamd_fq_per_group_int4_sym_tiled_bf16(const void* w, int64_t N, int64_t K, int group_size, int qparam_dtype, float eps,
                                            void* tiled_fwd, void* tiled_bwd, float* scale, void* stream);
 int ttamd_tiled_linear_bf16(const void* x, const void* tiled_weight, const void* bias, void* y, int64_t M, int64_t n_out,

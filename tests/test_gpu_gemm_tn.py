@@ -79,9 +79,11 @@ def test_full_size_weight_gradients_of_the_8b_qat_configuration(M, N, K):
     (8192, 4096, (4096, 1024, 1024)),        # q / k / v of the 8B shape at batch 2 x 4096: 384 tiles, one launch
     (8192, 4096, (14336, 14336)),            # gate / up: seven full rounds instead of two launches of three and a half
 ], ids=["small", "four_members", "qkv_8b", "gate_up_8b"])
-def test_group_launch_equals_member_launches_bitwise(M, K, Ns):
+def test_group_launch_equals_member_launches_bitwise(M, K, Ns, monkeypatch):
     """``ttamd_gemm_tn_group_bf16`` against one ``ttamd_gemm_tn_bf16`` per member: the same tiles and the same order of
-    sums, so the same bits; the member launches are themselves compared with fp32 products above."""
+    sums, so the same bits; the member launches are themselves compared with fp32 products above.  (Without slices of
+    the contraction: which tiles of a launch are cut depends on the launch's tile count, see the next test.)"""
+    monkeypatch.setattr(ops, "TN_TAIL_SLICES", False)
     g = torch.Generator().manual_seed(M + K + len(Ns))
     b = torch.randn(M, K, generator=g).to(BF).to(DEV)
     a_list = [torch.randn(M, N, generator=g).to(BF).to(DEV) for N in Ns]
@@ -89,6 +91,64 @@ def test_group_launch_equals_member_launches_bitwise(M, K, Ns):
     assert [tuple(c.shape) for c in cs] == [(N, K) for N in Ns]
     for a, c in zip(a_list, cs):
         assert torch.equal(c.view(torch.int16), ops.gemm_tn(a, b).view(torch.int16))
+
+
+@pytest.mark.parametrize("M,K,Ns", [
+    (8192, 4096, (4096, 1024, 1024)),   # q / k / v at batch 2 x 4096: 384 tiles = one whole round + 128 tiles in two slices
+    (8192, 14336, (4096,)),             # down projection: 896 tiles = three rounds + 128 tiles in two slices
+    (8192, 4096, (1024,)),              # a k / v projection alone: 64 tiles in four slices
+    (4096, 1024, (512, 256)),           # 12 tiles in four slices (a slice keeps at least 32 steps of the 128)
+    (8192, 4096, (14336, 14336)),       # whole rounds: nothing is cut
+], ids=["qkv_8b", "down_8b", "kv_alone", "few_tiles", "whole_rounds"])
+def test_contraction_slices_of_the_last_partial_round(M, K, Ns, monkeypatch):
+    """With the workspace ``ttamd_gemm_tn_workspace_bytes`` asks for, the tiles beyond the last whole round of 256 run as
+    slices of the contraction whose fp32 partial tiles a second launch adds in slice order: against the fp32 product at
+    the tolerance of the unsliced launch, within one bf16 rounding of the unsliced launch (only the order of the fp32
+    sums differs), bit-identical from run to run, exact for one-hot operands, and a workspace that is too small falls
+    back to the unsliced launch's bits."""
+    lib = _lib.load()
+    n_total = sum(Ns)
+    need = int(lib.ttamd_gemm_tn_workspace_bytes(M, n_total, K))
+    tiles = (n_total // 256) * (K // 256)
+    if tiles % 256 == 0:
+        assert need == 0
+    else:
+        assert need > 0 and need % (256 * 256 * 4) == 0 and need // (256 * 256 * 4) <= 256
+    g = torch.Generator().manual_seed(M + K + n_total)
+    b = torch.randn(M, K, generator=g).to(BF).to(DEV)
+    a_list = [torch.randn(M, N, generator=g).to(BF).to(DEV) for N in Ns]
+    run = (lambda: ops.gemm_tn_group(a_list, b)) if len(Ns) > 1 else (lambda: [ops.gemm_tn(a_list[0], b)])
+    sliced = run()
+    again = run()
+    monkeypatch.setattr(ops, "TN_TAIL_SLICES", False)
+    plain = run()
+    for a, c, c2, c0 in zip(a_list, sliced, again, plain):
+        assert torch.equal(c.view(torch.int16), c2.view(torch.int16))
+        want = a.float().t() @ b.float()
+        scale = max(1.0, float(want.abs().max()) / 8)
+        torch.testing.assert_close(c.float(), want, rtol=1e-2, atol=1e-2 * scale)
+        torch.testing.assert_close(c.float(), c0.float(), rtol=2.0 ** -7, atol=2.0 ** -7 * scale)
+        if need == 0:
+            assert torch.equal(c.view(torch.int16), c0.view(torch.int16))
+    if need:
+        # through the C ABI with a workspace one byte short: the unsliced launch
+        a, N = a_list[0], Ns[0]
+        if len(Ns) == 1:
+            ws = torch.empty(need, dtype=torch.uint8, device=DEV)
+            c = torch.empty(N, K, dtype=BF, device=DEV)
+            st = torch.cuda.current_stream().cuda_stream
+            assert lib.ttamd_gemm_tn_ws_bf16(a.data_ptr(), b.data_ptr(), c.data_ptr(), M, N, K, ws.data_ptr(), need - 1, st) == 0
+            assert torch.equal(c.view(torch.int16), plain[0].view(torch.int16))
+            assert lib.ttamd_gemm_tn_ws_bf16(a.data_ptr(), b.data_ptr(), c.data_ptr(), M, N, K, ws.data_ptr(), need, st) == 0
+            assert torch.equal(c.view(torch.int16), sliced[0].view(torch.int16))
+        # one-hot rows of a select rows of b exactly, sliced or not
+        monkeypatch.setattr(ops, "TN_TAIL_SLICES", True)
+        a1 = torch.zeros(M, Ns[0], dtype=BF, device=DEV)
+        R = min(M, Ns[0])
+        cols = torch.randperm(Ns[0], generator=g)[:R].to(DEV)
+        a1[torch.arange(R, device=DEV), cols] = 1.0
+        c1 = ops.gemm_tn_group([a1] + a_list[1:], b)[0] if len(Ns) > 1 else ops.gemm_tn(a1, b)
+        assert torch.equal(c1[cols].view(torch.int16), b[:R].view(torch.int16))
 
 
 def test_group_launch_refuses_bad_members():

@@ -119,6 +119,9 @@ SIGNATURES = {
     "ttamd_gemm_tn_applies": (_int, [_i64, _i64, _i64]),
     "ttamd_gemm_tn_bf16": (_int, [_c_void_p, _c_void_p, _c_void_p, _i64, _i64, _i64, _c_void_p]),
     "ttamd_gemm_tn_group_bf16": (_int, [_c_void_p, _c_void_p, _c_void_p, _int, _i64, _c_void_p, _i64, _c_void_p]),
+    "ttamd_gemm_tn_workspace_bytes": (_size, [_i64, _i64, _i64]),
+    "ttamd_gemm_tn_ws_bf16": (_int, [_c_void_p, _c_void_p, _c_void_p, _i64, _i64, _i64, _c_void_p, _size, _c_void_p]),
+    "ttamd_gemm_tn_group_ws_bf16": (_int, [_c_void_p, _c_void_p, _c_void_p, _int, _i64, _c_void_p, _i64, _c_void_p, _size, _c_void_p]),
     "ttamd_fq_per_group_int4_sym_tiled_bf16": (_int, [_c_void_p, _i64, _i64, _int, _int, _f32, _c_void_p, _c_void_p, _c_void_p, _c_void_p]),
     "ttamd_tiled_linear_bf16": (_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _i64, _i64, _i64, _c_void_p]),
     "ttamd_tiled_lora_linear_bf16": (_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _int, _int, _f32, _c_void_p, _c_void_p, _i64, _i64,

@@ -913,6 +913,18 @@ def gemm_tn_applies(M: int, N: int, K: int) -> bool:
     return bool(_lib.load().ttamd_gemm_tn_applies(M, N, K))
 
 
+# The tiles of a weight-gradient launch beyond its last whole round of 256 get their contraction cut into slices when the
+# library is given room for the partial tiles (False: never, the launch of the plain entry points).
+TN_TAIL_SLICES = True
+
+
+def _tn_workspace(lib, M: int, n_total: int, K: int, device):
+    nbytes = int(lib.ttamd_gemm_tn_workspace_bytes(M, n_total, K)) if TN_TAIL_SLICES else 0
+    if nbytes == 0:
+        return None, 0
+    return torch.empty(nbytes // 4, dtype=torch.float32, device=device), nbytes
+
+
 def gemm_tn(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
     """a [M, N], b [M, K] bf16 -> a.T @ b [N, K] bf16 (fp32 accumulation): the weight gradient of a linear layer."""
     a = _bf16_2d(a, "gemm_tn")
@@ -923,11 +935,12 @@ def gemm_tn(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
     K = b.shape[1]
     c = torch.empty(N, K, dtype=torch.bfloat16, device=a.device)
     lib = _lib.load()
+    ws, ws_bytes = _tn_workspace(lib, M, N, K, a.device)
     with torch.cuda.device(a.device):
         events = _gemm_timer("tn", M, N, K, 0) if _gemm_timer is not None else None
         if events:
             events[0].record()
-        rc = lib.ttamd_gemm_tn_bf16(a.data_ptr(), b.data_ptr(), c.data_ptr(), M, N, K, _stream(a))
+        rc = lib.ttamd_gemm_tn_ws_bf16(a.data_ptr(), b.data_ptr(), c.data_ptr(), M, N, K, _ptr(ws), ws_bytes, _stream(a))
         if events:
             events[1].record()
     _lib.check(rc, "gemm_tn")
@@ -936,7 +949,8 @@ def gemm_tn(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
 
 def gemm_tn_group(a_list: Sequence[torch.Tensor], b: torch.Tensor) -> List[torch.Tensor]:
     """``[a.T @ b for a in a_list]`` (each ``a`` [M, N_i], ``b`` [M, K], bf16) as one launch: the weight gradients of layers
-    with a common input.  Each result carries the bits ``gemm_tn(a, b)`` gives."""
+    with a common input.  Each result carries the bits ``gemm_tn(a, b)`` gives wherever neither launch cuts the tile's
+    contraction into slices (``TN_TAIL_SLICES``: the tiles of a launch's last partial round)."""
     b = _bf16_2d(b, "gemm_tn_group")
     a_list = [_bf16_2d(a, "gemm_tn_group") for a in a_list]
     M, K = b.shape
@@ -951,11 +965,12 @@ def gemm_tn_group(a_list: Sequence[torch.Tensor], b: torch.Tensor) -> List[torch
     c_ptrs = (ctypes.c_void_p * n)(*[c.data_ptr() for c in cs])
     widths = (ctypes.c_int64 * n)(*[a.shape[1] for a in a_list])
     lib = _lib.load()
+    ws, ws_bytes = _tn_workspace(lib, M, sum(a.shape[1] for a in a_list), K, b.device)
     with torch.cuda.device(b.device):
         events = _gemm_timer("tn", M, sum(a.shape[1] for a in a_list), K, 0) if _gemm_timer is not None else None
         if events:
             events[0].record()
-        rc = lib.ttamd_gemm_tn_group_bf16(a_ptrs, b.data_ptr(), c_ptrs, n, M, widths, K, _stream(b))
+        rc = lib.ttamd_gemm_tn_group_ws_bf16(a_ptrs, b.data_ptr(), c_ptrs, n, M, widths, K, _ptr(ws), ws_bytes, _stream(b))
         if events:
             events[1].record()
     _lib.check(rc, "gemm_tn_group")
