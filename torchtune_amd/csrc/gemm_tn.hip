@@ -59,7 +59,6 @@ struct TnArgs {
 
 constexpr int kTnStage = 32768;  // 32 rows x 512 bytes of A, then the same of B
 constexpr int kTnLds = 4 * kTnStage;
-constexpr int kLgkmMax = 15;  // the counter field of s_waitcnt holds 4 bits: waiting for fewer outstanding reads is always safe
 
 constexpr int kTnMT = 8, kTnNT = 4;  // 16 x 16 MFMA tiles per wave: MT along the rows of C (columns of A), NT along its columns
 
@@ -160,11 +159,11 @@ __global__ __launch_bounds__(512) void gemm_tn_kernel(const TnArgs g) {
                  ::"v"(voff), "s"(base), "s"(lds), "n"(imm) : "memory", "m0", "scc");
   };
   const uint32_t lds0 = (uint32_t)(uintptr_t)TT_LDS_PTR(smem);
-  auto issue = [&](int t) {
+  auto issue = [&](int t, int stage) {
     const int tk = t < nk ? t : nk - 1;
     const char* ab = reinterpret_cast<const char*>(A) + (int64_t)tk * 32 * N * 2;
     const char* bb = reinterpret_cast<const char*>(g.B) + (int64_t)tk * 32 * g.K * 2;
-    const uint32_t st = lds0 + (t & 3) * kTnStage + wv * 2048;
+    const uint32_t st = lds0 + stage * kTnStage + wv * 2048;
     dma16(a_off[0], ab, st, 0);
     dma16(a_off[1], ab, st, 1024);
     dma16(b_off[0], bb, st, 16384);
@@ -175,20 +174,24 @@ __global__ __launch_bounds__(512) void gemm_tn_kernel(const TnArgs g) {
   //      operand), columns 4 (l15 % 4) .. + 3 of a 16-column group e, and receives column l15 of that group for rows
   //      8 g4 .. + 3 (+ 4): with both halves the 8 contraction elements of an MFMA operand.  Group e of a row with
   //      row % 4 = q sits at byte 32 (e ^ q) of the row.  A groups of this wave: 8 wm + i; B groups: 4 wn + j.
-  uint32_t ra[4], rb[4];
+  //      The reads go through the compiler's builtin, so that everything of an address that is the same for all lanes
+  //      (stage, half, group of four) rides in the instruction's offset field: eight address additions per two steps.
+  //      With one register operand per read, as hand-written assembly takes it, every read cost a vector-ALU addition
+  //      of its own (24 per step), issued from the memory part of one wave into the MFMA part of the other wave of
+  //      its SIMD.
+  int ra[4], rb[4];  // byte offsets from the start of a stage
   {
     const int q = (l15 >> 2) & 3;
-    const uint32_t rowbase = (uint32_t)(8 * g4 + (l15 >> 2)) * 512u + 8u * (l15 & 3);
+    const int rowbase = (8 * g4 + (l15 >> 2)) * 512 + 8 * (l15 & 3);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      ra[e] = lds0 + rowbase + 32u * (8 * wm) + 32u * (e ^ q);
-      rb[e] = lds0 + 16384u + rowbase + 32u * (4 * wn) + 32u * (e ^ q);
+      ra[e] = rowbase + 32 * (8 * wm) + 32 * (e ^ q);
+      rb[e] = 16384 + rowbase + 32 * (4 * wn) + 32 * (e ^ q);
     }
   }
-  auto tr16 = [&](uint32_t addr) {
-    u32x2_t v;
-    asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(v) : "v"(addr) : "memory");
-    return v;
+  typedef short s16x4_t __attribute__((ext_vector_type(4)));
+  auto tr16 = [&](const char* at) {
+    return __builtin_bit_cast(u32x2_t, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(at)));
   };
 
   f32x4_t acc[NT][MT];
@@ -200,63 +203,92 @@ __global__ __launch_bounds__(512) void gemm_tn_kernel(const TnArgs g) {
       for (int v = 0; v < 4; ++v) acc[j][i][v] = 0.f;
 
   u32x2_t alo[MT], ahi[MT], blo[NT], bhi[NT];
-  auto read_step = [&](int t) {
-    const uint32_t st = (uint32_t)(t & 3) * kTnStage;
+  // pa[e], pb[e]: the lane's addresses in the even stage of the current pair; `odd` adds one stage as a constant
+  auto read_step = [&](const char* const (&pa)[4], const char* const (&pb)[4], int odd) {
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
-      blo[j] = tr16(rb[j] + st);
-      bhi[j] = tr16(rb[j] + st + 2048u);
+      blo[j] = tr16(pb[j] + odd * kTnStage);
+      bhi[j] = tr16(pb[j] + odd * kTnStage + 2048);
     }
 #pragma unroll
     for (int i = 0; i < MT; ++i) {
-      alo[i] = tr16(ra[i & 3] + st + 128u * (i >> 2));
-      ahi[i] = tr16(ra[i & 3] + st + 128u * (i >> 2) + 2048u);
+      alo[i] = tr16(pa[i & 3] + odd * kTnStage + 128 * (i >> 2));
+      ahi[i] = tr16(pa[i & 3] + odd * kTnStage + 128 * (i >> 2) + 2048);
     }
+  };
+  auto compute = [&]() {
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+      const u32x4_t aop = {alo[i].x, alo[i].y, ahi[i].x, ahi[i].y};
+#pragma unroll
+      for (int j = 0; j < NT; ++j) {
+        const u32x4_t bop = {blo[j].x, blo[j].y, bhi[j].x, bhi[j].y};
+        acc[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, bop), __builtin_bit_cast(bf16x8_t, aop),
+                                                           acc[j][i], 0, 0, 0);
+      }
+    }
+    __builtin_amdgcn_s_setprio(0);
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_barrier" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
   };
 
   // ---- pipeline, as in nf4_gemm_dense.hip: memory part M(t) / barrier / compute part C(t) / barrier, the waves with wm = 1
-  //      one barrier behind.  M(t) requests step t + 3 (four loads) and reads the operands of step t.  At the end of M(t) a
-  //      wave's own loads of step t + 1 must have landed (the other waves read them after the next barrier): they came
-  //      from M(t - 2), newer are the 4 + 4 loads of M(t - 1) and M(t).  The transposing reads are written in assembly, so
-  //      the wait for them is explicit too and names the registers it releases.
-  issue(t_begin);
-  issue(t_begin + 1);
-  issue(t_begin + 2);
+  //      one barrier behind.  M(t) requests step t + 3 (four loads) into the stage step t - 1 was read from and reads the
+  //      operands of step t.  At the end of M(t) a wave's own loads of step t + 1 must have landed (the other waves read
+  //      them after the next barrier): they came from M(t - 2), newer are the 4 + 4 loads of M(t - 1) and M(t).  Stages
+  //      are counted from the workgroup's first step (a slice may start anywhere); the loop takes two steps per trip.
+  issue(t_begin, 0);
+  issue(t_begin + 1, 1);
+  issue(t_begin + 2, 2);
   asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");  // the first step landed everywhere
   if (wm == 1) asm volatile("s_barrier" ::: "memory");
   // one copy of the loop per wave group: the two differ in one wait, and a branch per step costs 2 - 4 %
   auto main_loop = [&](auto lgkm) {
     constexpr bool kLgkm = decltype(lgkm)::value;
-    for (int t = t_begin; t < nk; ++t) {
-      issue(t + 3);
-      read_step(t);
+    // what the waves with wm = 1 read in a memory part is overwritten by requests the waves with wm = 0 issue right after
+    // the next barrier: they let their reads complete before they pass it (the others' reads have a whole interval more)
+    auto end_of_memory_part = [&]() {
       __builtin_amdgcn_sched_barrier(0);
-      // what the waves with wm = 1 read here is overwritten by requests the waves with wm = 0 issue right after the next
-      // barrier: they let their reads complete before they pass it (the others' reads have a whole interval more)
       if constexpr (kLgkm)
         asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
       else
         asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");
-      __builtin_amdgcn_sched_barrier(0);
-      __builtin_amdgcn_s_setprio(1);
+    };
+    int ws = 0;  // stage of the even step of the current pair: 0 or 2
+    int t = t_begin;
+    for (; t + 1 < nk; t += 2) {
+      const char* pa[4];
+      const char* pb[4];
 #pragma unroll
-      for (int j = 0; j < NT; ++j)
-        asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(blo[j]), "+v"(bhi[j]) : "n"(kLgkmMax < 2 * MT + 2 * (NT - 1 - j) ? kLgkmMax : 2 * MT + 2 * (NT - 1 - j)));
-#pragma unroll
-      for (int i = 0; i < MT; ++i) {
-        asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(alo[i]), "+v"(ahi[i]) : "n"(kLgkmMax < 2 * (MT - 1 - i) ? kLgkmMax : 2 * (MT - 1 - i)));
-        const u32x4_t aop = {alo[i].x, alo[i].y, ahi[i].x, ahi[i].y};
-#pragma unroll
-        for (int j = 0; j < NT; ++j) {
-          const u32x4_t bop = {blo[j].x, blo[j].y, bhi[j].x, bhi[j].y};
-          acc[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, bop), __builtin_bit_cast(bf16x8_t, aop),
-                                                             acc[j][i], 0, 0, 0);
-        }
+      for (int e = 0; e < 4; ++e) {
+        pa[e] = smem + ws * kTnStage + ra[e];
+        pb[e] = smem + ws * kTnStage + rb[e];
       }
-      __builtin_amdgcn_s_setprio(0);
-      __builtin_amdgcn_sched_barrier(0);
-      asm volatile("s_barrier" ::: "memory");
-      __builtin_amdgcn_sched_barrier(0);
+      issue(t + 3, (ws + 3) & 3);
+      read_step(pa, pb, 0);
+      end_of_memory_part();
+      compute();
+      issue(t + 4, ws);
+      read_step(pa, pb, 1);
+      end_of_memory_part();
+      compute();
+      ws ^= 2;
+    }
+    if (t < nk) {  // an odd number of steps: the last one on its own
+      const char* pa[4];
+      const char* pb[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        pa[e] = smem + ws * kTnStage + ra[e];
+        pb[e] = smem + ws * kTnStage + rb[e];
+      }
+      issue(t + 3, (ws + 3) & 3);
+      read_step(pa, pb, 0);
+      end_of_memory_part();
+      compute();
     }
   };
   if (wm == 1)
