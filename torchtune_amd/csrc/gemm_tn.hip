@@ -8,8 +8,11 @@
 // tiles (32 rows x 512 bytes each) into a ring of four LDS stages by direct-to-LDS loads; wave (wm, wn) owns rows
 // [128 wm, +128) x columns [64 wn, +64) of the tile (128 accumulators per lane); the two waves of a SIMD run half a step
 // apart, one in its MFMA part while the other requests loads and reads operands, swapping at workgroup barriers.
-// LDS layout of a stage: row r of the 32 at r * 512, its 16-byte chunk c in slot c ^ (2 (r % 4)) - applied on the
-// global-address side of the loads - so that the four rows a 16-lane group reads together fall on disjoint banks.
+// LDS layout of a stage: row r of the 32 at r * 512, its 16-byte chunk c in slot c ^ (2 (r % 4)) ^ (8 ((r / 8) % 2)) -
+// applied on the global-address side of the loads.  The first term puts the four rows a 16-lane group reads together on
+// disjoint banks; the second moves the rows of the odd 16-lane groups 128 bytes aside, so that the two groups the LDS
+// serves in one pass (lanes 0 - 31, then 32 - 63; 64 banks of 4 bytes) use different halves of the banks (without it
+// every transposing read takes two passes: SQ_LDS_BANK_CONFLICT = half of SQ_LDS_IDX_ACTIVE).
 //
 // Last partial round.  256 CUs take 256 tiles at a time; a launch of, say, 3.5 rounds of tiles leaves half the chip idle
 // for the length of one tile (220 us at 8192 tokens).  With a workspace the tiles beyond the last whole round have their
@@ -145,12 +148,12 @@ __global__ __launch_bounds__(512) void gemm_tn_kernel(const TnArgs g) {
   const int N = g.N[which];
 
   // ---- loads: per step and wave two instructions for A (rows 4 wv .. + 3 of the 32, two rows of 512 bytes each) and two
-  //      for B; lane l of an instruction fetches chunk (l % 32) ^ (2 (row % 4)) of row l / 32 of its pair
+  //      for B; lane l of an instruction fetches chunk (l % 32) ^ (2 (row % 4)) ^ (8 ((row / 8) % 2)) of row l / 32 of its pair
   uint32_t a_off[2], b_off[2];
 #pragma unroll
   for (int d = 0; d < 2; ++d) {
     const int rl = 4 * wv + 2 * d + (lane >> 5);
-    const int chunk = (lane & 31) ^ ((rl & 3) << 1);
+    const int chunk = (lane & 31) ^ ((rl & 3) << 1) ^ (((rl >> 3) & 1) << 3);
     a_off[d] = (uint32_t)rl * (uint32_t)N * 2u + (uint32_t)n0 * 2u + (uint32_t)chunk * 16u;
     b_off[d] = (uint32_t)rl * (uint32_t)g.K * 2u + (uint32_t)k0 * 2u + (uint32_t)chunk * 16u;
   }
@@ -173,21 +176,24 @@ __global__ __launch_bounds__(512) void gemm_tn_kernel(const TnArgs g) {
   // ---- operand reads.  Lane (l15, g4) of ds_read_b64_tr_b16 points at row 8 g4 + l15 / 4 (+ 4 for the second half of the
   //      operand), columns 4 (l15 % 4) .. + 3 of a 16-column group e, and receives column l15 of that group for rows
   //      8 g4 .. + 3 (+ 4): with both halves the 8 contraction elements of an MFMA operand.  Group e of a row with
-  //      row % 4 = q sits at byte 32 (e ^ q) of the row.  A groups of this wave: 8 wm + i; B groups: 4 wn + j.
+  //      row % 4 = q and (row / 8) % 2 = sb sits at byte 32 ((e ^ q) ^ 4 sb) of the row; sb = g4 % 2 for both halves of an
+  //      operand.  A groups of this wave: 8 wm + i (ra[i % 4] + ah[i / 4]); B groups: 4 wn + j.
   //      The reads go through the compiler's builtin, so that everything of an address that is the same for all lanes
   //      (stage, half, group of four) rides in the instruction's offset field: eight address additions per two steps.
   //      With one register operand per read, as hand-written assembly takes it, every read cost a vector-ALU addition
   //      of its own (24 per step), issued from the memory part of one wave into the MFMA part of the other wave of
   //      its SIMD.
-  int ra[4], rb[4];  // byte offsets from the start of a stage
+  int ra[4], rb[4], ah[2];  // byte offsets from the start of a stage
   {
-    const int q = (l15 >> 2) & 3;
+    const int q = (l15 >> 2) & 3, sb = g4 & 1;
     const int rowbase = (8 * g4 + (l15 >> 2)) * 512 + 8 * (l15 & 3);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       ra[e] = rowbase + 32 * (8 * wm) + 32 * (e ^ q);
-      rb[e] = 16384 + rowbase + 32 * (4 * wn) + 32 * (e ^ q);
+      rb[e] = 16384 + rowbase + 32 * (4 * (wn ^ sb)) + 32 * (e ^ q);
     }
+    ah[0] = 128 * sb;
+    ah[1] = 128 * (1 - sb);
   }
   typedef short s16x4_t __attribute__((ext_vector_type(4)));
   auto tr16 = [&](const char* at) {
@@ -212,8 +218,8 @@ __global__ __launch_bounds__(512) void gemm_tn_kernel(const TnArgs g) {
     }
 #pragma unroll
     for (int i = 0; i < MT; ++i) {
-      alo[i] = tr16(pa[i & 3] + odd * kTnStage + 128 * (i >> 2));
-      ahi[i] = tr16(pa[i & 3] + odd * kTnStage + 128 * (i >> 2) + 2048);
+      alo[i] = tr16(pa[i & 3] + ah[i >> 2] + odd * kTnStage);
+      ahi[i] = tr16(pa[i & 3] + ah[i >> 2] + odd * kTnStage + 2048);
     }
   };
   auto compute = [&]() {
