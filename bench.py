@@ -271,6 +271,91 @@ def cpu_baseline(shape_name: str, rank: int, alpha: float, tokens_sample: int, l
     }
 
 
+def gemm_kernels(dev, tokens=(256, 512, 1024, 1536)) -> dict:
+    """The GEMM kernels of the path in isolation, each against its alternative in the same process (HIP events, best of
+    two rounds of 30 launches, microseconds):
+
+    * ``dispatch_vs_dequantise_plus_vendor_gemm``: what the library's dispatch runs for a forward and a grad-input of the
+      8B projections at evaluation / short-batch token counts against the reference's order of work with the vendor
+      library's GEMM (``ttamd_nf4_dequantize`` into a dense bf16 weight + ``F.linear`` / ``gy @ W``);
+    * ``weight_gradient``: ``gemm_tn`` with and without contraction slices for the last partial round of tiles, and the
+      vendor library's ``a.T @ b``, at the 8B shapes of the 8da4w QAT step (8192 tokens);
+    * ``grad_input_tiles``: the plain GEMM's grad-input on tiles of the transposed weight against the same launch on the
+      forward launch's tiles (transposing LDS reads, no second copy of the weight)."""
+    import torch.nn.functional as F
+
+    from torchtune_amd import ops, to_nf4
+
+    def timed(fn, iters=30):
+        best = None
+        for _ in range(2):
+            for _ in range(5):
+                fn()
+            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record()
+            for _ in range(iters):
+                fn()
+            end.record()
+            torch.cuda.synchronize()
+            us = start.elapsed_time(end) / iters * 1e3
+            best = us if best is None else min(best, us)
+        return round(best, 1)
+
+    BF = torch.bfloat16
+    gen = torch.Generator(device=dev).manual_seed(4)
+    warm = torch.randn(8192, 8192, device=dev, dtype=BF)
+    for _ in range(30):
+        warm @ warm
+    del warm
+    out = {"dispatch_vs_dequantise_plus_vendor_gemm": [], "weight_gradient": [], "grad_input_tiles": []}
+    for N, K in ((4096, 4096), (14336, 4096), (4096, 14336)):
+        t = to_nf4((torch.randn(N, K, device=dev, generator=gen) * 0.02).to(BF))
+        bs = t.block_scalers()
+        A = (torch.randn(16, K, device=dev, generator=gen) * 0.05).to(BF)
+        B = (torch.randn(N, 16, device=dev, generator=gen) * 0.05).to(BF)
+        for M in tokens:
+            x = torch.randn(M, K, device=dev, generator=gen).to(BF)
+            gy = torch.randn(M, N, device=dev, generator=gen).to(BF)
+            h = torch.randn(M, 16, device=dev, generator=gen).to(BF)
+            gh = torch.randn(M, 16, device=dev, generator=gen).to(BF)
+            trf, trb = t.backward_copy_for(M, True), t.backward_copy_for(M, False)
+            out["dispatch_vs_dequantise_plus_vendor_gemm"].append({
+                "weight": f"{N}x{K}", "tokens": M,
+                "fwd_own_us": timed(lambda: ops.nf4_lora_linear_fwd(x, t.quantized_data, bs, N, h, B, 2.0, block_scalers_t=trf[1] if trf else None)),
+                "fwd_dequant_vendor_us": timed(lambda: F.linear(x, t.get_original_weight())),
+                "dx_own_us": timed(lambda: ops.nf4_linear_bwd_dx(gy, t.quantized_data, bs, K, gh, A, transposed=trb)),
+                "dx_dequant_vendor_us": timed(lambda: gy @ t.get_original_weight()),
+            })
+        del t, bs
+    M = 8192
+    for Ns, K in (((4096,), 4096), ((4096, 1024, 1024), 4096), ((14336, 14336), 4096), ((4096,), 14336)):
+        a = [torch.randn(M, N, device=dev, generator=gen).to(BF) for N in Ns]
+        b = torch.randn(M, K, device=dev, generator=gen).to(BF)
+        run = (lambda: ops.gemm_tn_group(a, b)) if len(Ns) > 1 else (lambda: ops.gemm_tn(a[0], b))
+        row = {"a_columns": "+".join(str(n) for n in Ns), "b_columns": K, "tokens": M, "tiles": sum(Ns) // 256 * (K // 256),
+               "flop": 2.0 * M * sum(Ns) * K}
+        ops.TN_TAIL_SLICES = True
+        row["own_us"] = timed(run, 20)
+        ops.TN_TAIL_SLICES = False
+        row["own_unsliced_us"] = timed(run, 20)
+        ops.TN_TAIL_SLICES = True
+        row["vendor_us"] = timed(lambda: [m.t().matmul(b) for m in a], 20)
+        row["own_tflops"] = round(row["flop"] / row["own_us"] / 1e6, 1)
+        out["weight_gradient"].append(row)
+        del a, b
+    for N, K in ((4096, 4096), (14336, 4096), (4096, 14336)):
+        w = (torch.randn(N, K, device=dev, generator=gen) * 0.02).to(BF)
+        tf, tb, _ = ops.fq_per_group_int4_sym_tiled(w, 32)
+        gy = torch.randn(M, N, device=dev, generator=gen).to(BF)
+        row = {"weight": f"{N}x{K}", "tokens": M, "flop": 2.0 * M * N * K,
+               "on_transposed_tiles_us": timed(lambda: ops.tiled_linear(gy, tb, K), 20),
+               "on_forward_tiles_us": timed(lambda: ops.tiled_linear_dx(gy, tf, K), 20)}
+        row["bit_equal"] = bool(torch.equal(ops.tiled_linear(gy, tb, K), ops.tiled_linear_dx(gy, tf, K)))
+        out["grad_input_tiles"].append(row)
+        del w, tf, tb, gy
+    return out
+
+
 def secondary_kernels(dev, offload_leg: bool = True) -> dict:
     """Achieved HBM GB/s of the bandwidth-bound kernels of the path on the largest 8B weight / activation shapes:
     algorithmic bytes (2.515747 B/element for the NF4 codec, 4 B/element for fake quant) / HIP-event time."""
@@ -387,11 +472,13 @@ def config1_leg(dev, runs: int = 15, warmups: int = 3) -> dict:
         layer.lora_b.weight.copy_(B.to(dev))
     xd = x.to(dev).requires_grad_()
 
+    grads = (layer.lora_a.weight, layer.lora_b.weight, xd)
+
     def gpu_run():
         y = layer(xd)
         (y.float() ** 2).sum().backward()
-        layer.zero_grad(set_to_none=True)
-        xd.grad = None
+        for p in grads:  # the three tensors that received a gradient (Module.zero_grad walks the module tree: 20 us)
+            p.grad = None
 
     gpu_ms = []
     for i in range(warmups + runs):
@@ -540,9 +627,12 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
-    ap.add_argument("--workload", default="llama3_1_8b", choices=sorted(WORKLOADS) + ["hbm_kernels", "config1_single_layer"],
+    ap.add_argument("--workload", default="llama3_1_8b", choices=sorted(WORKLOADS) + ["hbm_kernels", "config1_single_layer", "gemm_kernels"],
                     help="a decoder configuration, or 'hbm_kernels': only the bandwidth-bound kernels in isolation (NF4 "
-                         "dequantise / quantise, fake quant, few-token forward), the launches a kernel trace of them should hold")
+                         "dequantise / quantise, fake quant, few-token forward), the launches a kernel trace of them should hold; "
+                         "'gemm_kernels': the GEMM kernels in isolation beside their alternatives (dispatch at a few hundred tokens "
+                         "against dequantise + vendor GEMM, the weight-gradient GEMM with and without slices of its last partial "
+                         "round, the grad-input on forward tiles); 'config1_single_layer': one 2048 x 2048 QLoRA layer")
     ap.add_argument("--no-offload-leg", action="store_true",
                     help="hbm_kernels: skip the dequantise-into-pinned-host-memory leg (PCIe-bound launches of the same kernel)")
     ap.add_argument("--cpu-tokens", type=int, default=512,
@@ -617,6 +707,20 @@ def main() -> int:
         from torchtune_amd import nf4_tensor
         nf4_tensor.BACKWARD_COPY = False
 
+    if args.workload == "gemm_kernels":
+        dev = torch.device("cuda", 0)
+        torch.cuda.set_device(dev)
+        table = gemm_kernels(dev)
+        best = max(table["weight_gradient"], key=lambda r: r["own_tflops"])
+        print(json.dumps({
+            "metric": "weight-gradient GEMM TFLOP/s (gemm_tn, 8192 tokens, 1 GPU)", "value": best["own_tflops"], "unit": "TFLOP/s",
+            "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": None, "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "bf16", "data": "synthetic (random operands)",
+            "config": {"workload": "the GEMM kernels of the path in isolation, each beside its alternative"},
+            "roofline": {"bound": "mfma", "kernel": "gemm_tn_kernel", "achieved": best["own_tflops"], "peak": MFMA_BF16_PEAK_TFLOPS,
+                         "unit": "TFLOP/s", "frac": round(best["own_tflops"] / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None},
+            "gemm_kernels": table}))
+        return 0
     if args.workload == "config1_single_layer":
         dev = torch.device("cuda", 0)
         torch.cuda.set_device(dev)
