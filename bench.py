@@ -672,6 +672,10 @@ def main() -> int:
     ap.add_argument("--no-qat-tiled-gemm", action="store_true",
                     help="QAT workload: row-major fq(W) and the vendor library's GEMM for every matmul, instead of fake-quantising "
                          "the weights straight into the tile order of the library's own GEMM for forward and grad-input")
+    ap.add_argument("--keep-forward-tiles", type=int, default=None, metavar="TOKENS",
+                    help="calls of at most this many tokens hand their expanded weight to the backward of the same layer, whose "
+                         "grad-input GEMM reads it instead of expanding the weight again (0: never; default: the library's rule, "
+                         "torchtune_amd.ops.KEEP_FORWARD_TILES_MAX_TOKENS = 4096)")
     ap.add_argument("--no-backward-copy", action="store_true",
                     help="keep no transposed copy of the NF4 codes (0.5625 B per weight element less): the expanded-weight path then "
                          "builds W^T from the weight's own codes, the fused path falls back to its first-generation grad-input kernel")
@@ -697,6 +701,8 @@ def main() -> int:
     harness.FUSED_QKV_POST = not args.no_fused_qkv_post
     harness.SWIGLU_BWD_EPILOGUE = args.swiglu_bwd_epilogue
     ops.EXPANDED_WEIGHT_PATH = not args.no_expanded_weight
+    if args.keep_forward_tiles is not None:
+        ops.KEEP_FORWARD_TILES_MAX_TOKENS = args.keep_forward_tiles
     if args.no_qat_tiled_gemm:
         from torchtune_amd import qat as qat_module
         qat_module.TILED_GEMM = False

@@ -303,6 +303,13 @@ int ttamd_lora_bwd_bf16(const void* gy, const void* x, const void* h, const void
  * by size (few tokens, slices of the contraction, the weight expanded once per call).  One workspace per call, sized
  * by the matching query (the stages of a direction reuse its bytes one after the other).  rank a multiple of 8 in
  * [8,64]; the other operands as for the entry points above; quantized_data_t / block_scalers_t: both or neither.
+ * One expansion for both directions (optional): when ttamd_nf4_gemm_expands_weight(M, N, K) is 1, the forward call
+ * leaves the weight expanded to bf16, in forward tile order, in the first 2 N K bytes of its workspace.  A caller that
+ * keeps those bytes until the backward passes them as tiles_fwd (else NULL): the grad-input then runs
+ * ttamd_tiled_linear_dx_bf16 on them instead of expanding the weight a second time (same gx up to the order of fp32
+ * sums inside a tile row; pays when the expansion is a large share of the call, i.e. at a few thousand tokens).
+ * With tiles_fwd (or gx == NULL) the backward needs only the bytes of gh and of ttamd_lora_bwd_workspace_bytes, each
+ * rounded up to 256; the query above is the size that serves every case.
  */
 size_t ttamd_qlora_linear_fwd_workspace_bytes(int64_t M, int64_t N, int64_t K, int rank);
 int ttamd_qlora_linear_fwd_bf16(const void* x, const uint8_t* quantized_data, const void* block_scalers, const void* block_scalers_t,
@@ -310,9 +317,9 @@ int ttamd_qlora_linear_fwd_bf16(const void* x, const uint8_t* quantized_data, co
                                 int64_t M, int64_t N, int64_t K, void* workspace, size_t workspace_bytes, void* stream);
 size_t ttamd_qlora_linear_bwd_workspace_bytes(int64_t M, int64_t N, int64_t K, int rank);
 int ttamd_qlora_linear_bwd_bf16(const void* gy, const void* x, const void* h, const uint8_t* quantized_data, const void* block_scalers,
-                                const uint8_t* quantized_data_t, const void* block_scalers_t, const void* lora_a, const void* lora_b,
-                                int rank, float scale, void* gx, void* grad_lora_a, void* grad_lora_b, int64_t M, int64_t N, int64_t K,
-                                void* workspace, size_t workspace_bytes, void* stream);
+                                const uint8_t* quantized_data_t, const void* block_scalers_t, const void* tiles_fwd, const void* lora_a,
+                                const void* lora_b, int rank, float scale, void* gx, void* grad_lora_a, void* grad_lora_b, int64_t M,
+                                int64_t N, int64_t K, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
  * Groups of LoRA linears with a common input
@@ -383,6 +390,20 @@ int ttamd_nf4_group_bwd_dx_bf16(const ttamd_lora_group_member* members, int n_me
 size_t ttamd_nf4_group_bwd_dx_workspace_bytes(const ttamd_lora_group_member* members, int n_members, int64_t M, int64_t K);
 int ttamd_nf4_group_bwd_dx_ws_bf16(const ttamd_lora_group_member* members, int n_members, const void* gh_cat, void* gx, int64_t M,
                                    int64_t K, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * One expansion for both directions of a group.  ttamd_nf4_group_fwd_leaves_tiles says what the group's forward call
+ * (ttamd_nf4_lora_group_fwd_bf16; swiglu != 0: ttamd_nf4_lora_group_swiglu_fwd_bf16) leaves at the start of a workspace
+ * of the size its query asks for: 0 nothing reusable, 1 the members' weights expanded to bf16 and stacked by rows in
+ * forward tile order (2 K sum(N[i]) bytes), 2 the gated pair's layout (128 columns of the gate, then 128 of the up
+ * projection).  ttamd_nf4_group_bwd_dx_tiles_bf16 is ttamd_nf4_group_bwd_dx_ws_bf16 on those bytes (paired = 1 for
+ * layout 2): no expansion launch, the weight operand is transposed on its way out of LDS.  No counterpart in the
+ * reference (autograd re-materialises every dequantised weight for the backward).
+ */
+int ttamd_nf4_group_fwd_leaves_tiles(const ttamd_lora_group_member* members, int n_members, int64_t M, int64_t K, int swiglu);
+int ttamd_nf4_group_bwd_dx_tiles_bf16(const ttamd_lora_group_member* members, int n_members, const void* gh_cat, void* gx, int64_t M,
+                                      int64_t K, const void* tiles_fwd, int paired, void* stream);
+
 
 /* ------------------------------------------------------------------------------------------------
  * QAT fake quantisation (int8 dynamic per-token activations, int4 per-group symmetric weights)

@@ -293,3 +293,96 @@ def test_expanded_path_sweep_vs_fp32_matmul_of_the_dequantised_weight(M, N, K, r
         if r:
             want = want + gh.float() @ A.to(DEV).float()
         torch.testing.assert_close(gx.float(), want, rtol=1e-2, atol=1e-2 * max(1.0, float(want.abs().max()) / 8))
+
+
+def _lora_layers(dims, K, rank, seed):
+    """LoRALinear layers over NF4 with a common input width, non-zero adapters, on the GPU."""
+    from torchtune_amd.modules.peft import LoRALinear
+
+    torch.manual_seed(seed)
+    layers = []
+    prev = torch.get_default_dtype()
+    torch.set_default_dtype(BF)
+    try:
+        for N in dims:
+            with torch.device(DEV):
+                layer = LoRALinear(K, N, rank=rank, alpha=2.0 * rank, quantize_base=True)
+            with torch.no_grad():
+                layer.lora_b.weight.normal_(0, 0.02)
+            layers.append(layer)
+    finally:
+        torch.set_default_dtype(prev)
+    return layers
+
+
+def _grads(fn, x, layers):
+    for layer in layers:
+        layer.zero_grad(set_to_none=True)
+    xg = x.clone().requires_grad_()
+    out = fn(xg)
+    outs = out if isinstance(out, tuple) else (out,)
+    g = torch.Generator(device=DEV).manual_seed(99)
+    torch.autograd.backward(outs, [torch.randn(o.shape, device=DEV, generator=g).to(BF) for o in outs])
+    return [xg.grad] + [p.grad for layer in layers for p in (layer.lora_a.weight, layer.lora_b.weight)], [o.detach() for o in outs]
+
+
+@pytest.mark.parametrize("kind", ["single", "single_two_stage_calls", "qkv_group", "gated_pair", "feed_forward"])
+def test_one_expansion_serves_both_directions(kind, monkeypatch):
+    """With ``ops.KEEP_FORWARD_TILES_MAX_TOKENS`` at or above the token count the forward call's expanded weight stays
+    with the autograd node and the grad-input GEMM reads those forward tiles through transposing LDS reads
+    (``ttamd_tiled_linear_dx_bf16`` / ``ttamd_nf4_group_bwd_dx_tiles_bf16``) instead of expanding the weight again.  Same
+    products in the same order as the launch on tiles of the transposed weight: every gradient bit for bit - except for
+    the gated pair, whose tiles interleave the two members 128 columns at a time, so its grad-input sums the same
+    products in another order (rtol 1e-2, atol 2e-3 of unit-variance gradients)."""
+    from torchtune_amd.modules.peft import group as group_mod
+    from torchtune_amd.modules.peft import lora as lora_mod
+
+    M, K = 2048, 8192   # 8 row tiles: both directions of every layer below give the many-token launch its 256 tiles
+    g = torch.Generator(device=DEV).manual_seed(5)
+    x = torch.randn(M, K, device=DEV, generator=g).to(BF)
+    if kind.startswith("single"):
+        layers = _lora_layers([8192], K, 16, seed=1)
+        fn = lambda t: layers[0](t)
+        if kind == "single_two_stage_calls":
+            monkeypatch.setattr(lora_mod, "ONE_CALL_PER_DIRECTION", False)
+    elif kind == "qkv_group":
+        layers = _lora_layers([4096, 2048, 2048], K, 16, seed=2)
+        fn = lambda t: group_mod.lora_linear_group(t, layers)
+    elif kind == "gated_pair":
+        layers = _lora_layers([4096, 4096], K, 16, seed=3)
+        fn = lambda t: group_mod.lora_swiglu_group(t, layers[0], layers[1])
+    else:
+        layers = _lora_layers([4096, 4096], K, 16, seed=4) + _lora_layers([8192], 4096, 16, seed=5)
+        fn = lambda t: group_mod.lora_feed_forward(t, layers[0], layers[1], layers[2])
+    calls = {"tiles": 0}
+    lib = _lib.load()
+    for name in ("ttamd_tiled_linear_dx_bf16", "ttamd_nf4_group_bwd_dx_tiles_bf16"):
+        real = getattr(lib, name)
+
+        def counted(*a, _real=real):
+            calls["tiles"] += 1
+            return _real(*a)
+
+        monkeypatch.setattr(lib, name, counted)
+    monkeypatch.setattr(ops, "KEEP_FORWARD_TILES_MAX_TOKENS", 0)
+    want, out0 = _grads(fn, x, layers)
+    assert calls["tiles"] == 0
+    monkeypatch.setattr(ops, "KEEP_FORWARD_TILES_MAX_TOKENS", M)
+    got, out1 = _grads(fn, x, layers)
+    # the single layer's one-call backward takes the tiles inside the library; the other routes call the entry points above
+    if kind != "single":
+        assert calls["tiles"] >= 1
+    for a, b in zip(out0, out1):
+        assert torch.equal(a, b)
+    exact = kind in ("single", "single_two_stage_calls", "qkv_group")
+    for i, (a, b) in enumerate(zip(got, want)):
+        if exact or i > 0 and kind == "gated_pair":
+            assert torch.equal(a.view(torch.int16), b.view(torch.int16)), (kind, i)
+        else:
+            torch.testing.assert_close(a.float(), b.float(), rtol=1e-2, atol=2e-3 * max(1.0, float(b.float().abs().max()) / 4))
+    # with activation checkpointing: the recomputation keeps the tiles, the first (no-grad) pass does not
+    from torch.utils.checkpoint import checkpoint
+
+    ck, _ = _grads(lambda t: checkpoint(fn, t, use_reentrant=False), x, layers)
+    for a, b in zip(ck, got):
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16))

@@ -766,8 +766,8 @@ def test_one_call_entry_points_check_their_workspace_and_arguments():
     gx = torch.empty(M, K, dtype=BF, device=DEV)
     ga = torch.empty(r, K, dtype=BF, device=DEV)
     gb = torch.empty(N, r, dtype=BF, device=DEV)
-    bargs = (gyd.data_ptr(), xd.data_ptr(), h.data_ptr(), qd.data_ptr(), bs.data_ptr(), None, None, Ad.data_ptr(), Bd.data_ptr(), r, 2.0,
-             gx.data_ptr(), ga.data_ptr(), gb.data_ptr(), M, N, K)
+    bargs = (gyd.data_ptr(), xd.data_ptr(), h.data_ptr(), qd.data_ptr(), bs.data_ptr(), None, None, None, Ad.data_ptr(), Bd.data_ptr(), r,
+             2.0, gx.data_ptr(), ga.data_ptr(), gb.data_ptr(), M, N, K)   # no transposed copies, no forward tiles
     assert lib.ttamd_qlora_linear_bwd_bf16(*bargs, wsb.data_ptr(), nb - 1, st) == -3
     assert lib.ttamd_qlora_linear_bwd_bf16(*bargs, wsb.data_ptr(), nb, st) == 0
     half = list(bargs)

@@ -76,7 +76,8 @@ size_t dense_group_fwd_workspace_bytes(const GroupGemm& d);
 bool dense_group_gated_applies(const GroupGemm& d);
 int run_gemm_dense_group_fwd(const void* x, const GroupGemm& d, const void* h_cat, void* workspace, hipStream_t s, void* act = nullptr);
 size_t dense_group_dx_workspace_bytes(const GroupDx& d);
-int run_gemm_dense_group_dx(const GroupDx& d, const void* gh_cat, void* gx, void* workspace, hipStream_t s);
+int run_gemm_dense_group_dx(const GroupDx& d, const void* gh_cat, void* gx, void* workspace, hipStream_t s,
+                            const void* tiles_fwd = nullptr, bool paired = false);
 
 // nf4_small_m.hip: y[i] = x . D(W_i)^T (+ bias) + scale . h_i . lora_b[i]^T for a handful of tokens
 int small_m_limit();

@@ -212,3 +212,29 @@ extern "C" int ttamd_nf4_group_bwd_dx_ws_bf16(const ttamd_lora_group_member* mem
   // members without transposed copies are expanded from the weight's own codes
   return run_gemm_dense_group_dx(d.dx, gh_cat, gx, workspace, reinterpret_cast<hipStream_t>(stream));
 }
+
+// Which expanded tiles a forward call of the group leaves at the start of the workspace it was given (when that workspace
+// was large enough): 0 none (few tokens, slices, the fused kernel), 1 the members' weights stacked by rows in forward
+// tile order, 2 the gated pair's layout (swiglu != 0: 128 columns of the gate, then 128 of the up projection).
+extern "C" int ttamd_nf4_group_fwd_leaves_tiles(const ttamd_lora_group_member* members, int n_members, int64_t M, int64_t K, int swiglu) {
+  Decoded d;
+  if (decode("nf4_group_fwd_leaves_tiles", members, n_members, M, K, false, d) != TTAMD_OK) return 0;
+  if (group_small_m(d, true) || dense_group_fwd_workspace_bytes(d.gm) == 0) return 0;
+  return swiglu && dense_group_gated_applies(d.gm) ? 2 : 1;
+}
+
+extern "C" int ttamd_nf4_group_bwd_dx_tiles_bf16(const ttamd_lora_group_member* members, int n_members, const void* gh_cat, void* gx,
+                                                 int64_t M, int64_t K, const void* tiles_fwd, int paired, void* stream) {
+  Decoded d;
+  if (int rc = decode("nf4_group_bwd_dx_tiles", members, n_members, M, K, false, d)) return rc;
+  TT_REQUIRE(gh_cat && gx && tiles_fwd && aligned16(gh_cat) && aligned16(gx) && aligned16(tiles_fwd),
+             "nf4_group_bwd_dx_tiles: gh_cat, gx and tiles_fwd must be non-null and 16-byte aligned");
+  TT_REQUIRE(!paired || (n_members == 2 && members[0].N == members[1].N && members[0].N % 128 == 0),
+             "nf4_group_bwd_dx_tiles: paired tiles belong to two members of equal width, a multiple of 128");
+  for (int i = 0; i < n_members; ++i)
+    TT_REQUIRE(members[i].N % 256 == 0 || paired, "nf4_group_bwd_dx_tiles: member %d: N (%lld) must be a multiple of 256 (as the forward launch required)",
+               i, (long long)members[i].N);
+  if (dense_group_dx_workspace_bytes(d.dx) == 0)
+    return fail(TTAMD_EUNSUPPORTED, "nf4_group_bwd_dx_tiles: shape not served by the many-token launch (M=%lld K=%lld)", (long long)M, (long long)K);
+  return run_gemm_dense_group_dx(d.dx, gh_cat, gx, nullptr, reinterpret_cast<hipStream_t>(stream), tiles_fwd, paired != 0);
+}

@@ -1009,9 +1009,12 @@ size_t dense_group_dx_workspace_bytes(const GroupDx& d) {
   return (size_t)d.K * (size_t)n_total * 2;
 }
 
-int run_gemm_dense_group_dx(const GroupDx& d, const void* gh_cat, void* gx, void* workspace, hipStream_t s) {
+// tiles_fwd != nullptr: no expansion; the launch reads the tiles the forward launch of the same group left in its
+// workspace (the members' weights stacked by rows, or - paired - the gated pair's 128-column alternation).
+int run_gemm_dense_group_dx(const GroupDx& d, const void* gh_cat, void* gx, void* workspace, hipStream_t s, const void* tiles_fwd,
+                            bool paired) {
   TT_REQUIRE(d.n >= 1 && d.n <= kGroupMax && dense_group_dx_workspace_bytes(d) > 0, "nf4_group_dx (expanded): shape not served");
-  TT_REQUIRE(aligned16(workspace), "nf4_group_dx (expanded): workspace must be 16-byte aligned");
+  TT_REQUIRE(tiles_fwd ? aligned16(tiles_fwd) : aligned16(workspace), "nf4_group_dx (expanded): workspace / tiles must be 16-byte aligned");
   int64_t n_total = 0;
   for (int i = 0; i < d.n; ++i) n_total += d.N[i];
   DenseArgs g = {};
@@ -1024,11 +1027,11 @@ int run_gemm_dense_group_dx(const GroupDx& d, const void* gh_cat, void* gx, void
   for (int i = 0; i < d.n; ++i) one_launch = one_launch && (d.codes_t[i] != nullptr) == (d.codes_t[0] != nullptr);
   for (int i = 0; i < d.n; ++i) {
     const bool tr = d.codes_t[i] != nullptr;
-    TT_REQUIRE(aligned16(d.gy[i]) && (tr ? aligned16(d.codes_t[i]) && aligned16(d.scal_t[i]) : aligned16(d.codes[i]) && d.bscal[i] != nullptr),
+    TT_REQUIRE(aligned16(d.gy[i]) && (tiles_fwd || (tr ? aligned16(d.codes_t[i]) && aligned16(d.scal_t[i]) : aligned16(d.codes[i]) && d.bscal[i] != nullptr)),
                "nf4_group_dx (expanded): pointers must be 16-byte aligned");
     eg.m[i] = ExpandMember{tr ? d.codes_t[i] : d.codes[i], tr ? d.scal_t[i] : d.bscal[i], reinterpret_cast<char*>(workspace), (int)d.K,
                            (int)d.N[i], (int)t_off};
-    if (!one_launch)
+    if (!one_launch && !tiles_fwd)
       if (int rc = launch_expand(tr ? 1 : 3, eg.m[i].codes, eg.m[i].scal, d.K, d.N[i], n_total >> 5, t_off, reinterpret_cast<char*>(workspace), s))
         return rc;
     t_off += d.N[i] >> 5;
@@ -1044,17 +1047,19 @@ int run_gemm_dense_group_dx(const GroupDx& d, const void* gh_cat, void* gx, void
       a.lscale = 1.0f;
     }
   }
-  if (one_launch) {
+  if (one_launch && !tiles_fwd) {
     eg.n = d.n;
     if (int rc = launch_expand_group(d.codes_t[0] ? 1 : 3, eg, n_total >> 5, s)) return rc;
   }
   g.out[0].C = reinterpret_cast<uint16_t*>(gx);
   g.out[0].n_begin = 0;
   g.out[0].width = (int)d.K;
-  g.Wt = reinterpret_cast<const char*>(workspace);
+  g.Wt = reinterpret_cast<const char*>(tiles_fwd ? tiles_fwd : workspace);
   g.M = (int)d.M; g.Nout = (int)d.K; g.Kc = (int)n_total;
   g.lw_row_major = 0;
   g.ldlx = d.r_off[d.n];
+  g.w_tr = tiles_fwd ? 1 : 0;
+  g.w_paired = tiles_fwd && paired ? 1 : 0;
   return launch_dense(g, s);
 }
 

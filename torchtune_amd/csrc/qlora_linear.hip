@@ -56,14 +56,16 @@ extern "C" size_t ttamd_qlora_linear_bwd_workspace_bytes(int64_t M, int64_t N, i
 
 extern "C" int ttamd_qlora_linear_bwd_bf16(const void* gy, const void* x, const void* h, const uint8_t* quantized_data,
                                            const void* block_scalers, const uint8_t* quantized_data_t, const void* block_scalers_t,
-                                           const void* lora_a, const void* lora_b, int rank, float scale, void* gx, void* grad_lora_a,
-                                           void* grad_lora_b, int64_t M, int64_t N, int64_t K, void* workspace, size_t workspace_bytes,
-                                           void* stream) {
+                                           const void* tiles_fwd, const void* lora_a, const void* lora_b, int rank, float scale,
+                                           void* gx, void* grad_lora_a, void* grad_lora_b, int64_t M, int64_t N, int64_t K,
+                                           void* workspace, size_t workspace_bytes, void* stream) {
   if (int rc = check_layer("qlora_linear_bwd", M, N, K, rank)) return rc;
   TT_REQUIRE(gy && x && h && quantized_data && block_scalers && lora_a && lora_b && grad_lora_a && grad_lora_b,
              "qlora_linear_bwd: null pointer argument");
   TT_REQUIRE((quantized_data_t == nullptr) == (block_scalers_t == nullptr), "qlora_linear_bwd: pass both transposed copies or neither");
-  const size_t need = ttamd_qlora_linear_bwd_workspace_bytes(M, N, K, rank);
+  // with the forward's tiles at hand (or no grad-input at all) the GEMM stage needs no scratch memory
+  const size_t need = (tiles_fwd || !gx) ? align256((size_t)M * (size_t)rank * 2) + align256(ttamd_lora_bwd_workspace_bytes(M, N, K, rank))
+                                         : ttamd_qlora_linear_bwd_workspace_bytes(M, N, K, rank);
   TT_REQUIRE(workspace && aligned16(workspace), "qlora_linear_bwd: workspace must be non-null and 16-byte aligned");
   if (workspace_bytes < need) return fail(TTAMD_EWORKSPACE, "qlora_linear_bwd: workspace has %zu bytes, needs %zu", workspace_bytes, need);
   char* ws = reinterpret_cast<char*>(workspace);
@@ -73,6 +75,8 @@ extern "C" int ttamd_qlora_linear_bwd_bf16(const void* gy, const void* x, const 
   const size_t skinny = ttamd_lora_bwd_workspace_bytes(M, N, K, rank);
   if (int rc = ttamd_lora_bwd_bf16(gy, x, h, lora_b, scale, gh, grad_lora_a, grad_lora_b, M, N, K, rank, rest, skinny, stream)) return rc;
   if (gx == nullptr) return TTAMD_OK;  // the layer's input needs no gradient
+  // the forward call's expanded weight is still at hand: the grad-input reads it (no expansion, no scratch memory)
+  if (tiles_fwd) return ttamd_tiled_linear_dx_bf16(gy, tiles_fwd, gh, lora_a, rank, gx, M, N, K, stream);
   // stage 2: gx = gy . D(W) + gh . A.  Without the transposed copies only the expanded-weight launch takes a workspace.
   size_t gemm = ttamd_nf4_gemm_workspace_bytes(M, K, N);
   if (!quantized_data_t && !ttamd_nf4_gemm_expands_weight(M, K, N)) gemm = 0;

@@ -41,7 +41,8 @@ class _QLoRAGroupFn(torch.autograd.Function):
         x2 = x.reshape(-1, K)
         members = [ops.GroupMember(w.quantized_data, w.block_scalers(), tr, a, b, bias, s, w.shape[0])
                    for w, tr, a, b, bias, s in zip(weights, _copies(weights, x2.shape[0]), las, lbs, biases, scales)]
-        h_cat, ys = ops.lora_group_fwd(x2, members)
+        h_cat, ys, tiles, paired = ops.lora_group_fwd(x2, members, return_tiles=True)
+        _keep_tiles(ctx, tiles, paired, x2.shape[0], weights)
         ctx.save_for_backward(x2, h_cat, *weights, *las, *lbs)
         ctx.scales = scales
         ctx.x_shape = x.shape
@@ -64,13 +65,25 @@ class _QLoRAGroupFn(torch.autograd.Function):
         return _group_backward(ctx, x2, h_cat, weights, las, lbs, gy2)
 
 
+def _keep_tiles(ctx, tiles, paired: bool, tokens: int, weights) -> None:
+    """The group forward's expanded weights stay with the node when the backward will want a grad-input, the call is
+    short enough for one expansion per layer to pay (``ops.KEEP_FORWARD_TILES_MAX_TOKENS``) and the grouped grad-input is
+    the many-token launch (with few output tiles it stays on the fused kernel)."""
+    keep = (tiles is not None and ctx.needs_input_grad[0] and ops.keeps_forward_tiles(tokens)
+            and ops.group_dx_expands(tokens, weights[0].shape[1], [w.shape[0] for w in weights]))
+    ctx.tiles, ctx.tiles_paired = (tiles, paired) if keep else (None, False)
+
+
 def _group_backward(ctx, x2, h_cat, weights, las, lbs, gy2):
     """Gradients of a group call in the order of its inputs (x, scales, then weight, lora_a, lora_b, bias per member)."""
     n = len(weights)
-    members = [ops.GroupMember(w.quantized_data, w.block_scalers(), tr, a, b, None, s, w.shape[0])
-               for w, tr, a, b, s in zip(weights, _copies(weights, x2.shape[0]), las, lbs, ctx.scales)]
     need_x = ctx.needs_input_grad[0]
-    gx, grads, _ = ops.lora_group_bwd(x2, h_cat, members, gy2, want_gx=need_x)
+    tiles, paired = (ctx.tiles, ctx.tiles_paired) if need_x else (None, False)
+    ctx.tiles = None
+    copies = [None] * n if tiles is not None else _copies(weights, x2.shape[0])
+    members = [ops.GroupMember(w.quantized_data, w.block_scalers(), tr, a, b, None, s, w.shape[0])
+               for w, tr, a, b, s in zip(weights, copies, las, lbs, ctx.scales)]
+    gx, grads, _ = ops.lora_group_bwd(x2, h_cat, members, gy2, want_gx=need_x, tiles=tiles, paired=paired)
     out: List = [gx.view(ctx.x_shape) if need_x else None, None]
     for i in range(n):
         _, need_a, need_b, need_bias = ctx.needs_input_grad[2 + 4 * i:6 + 4 * i]
@@ -93,7 +106,8 @@ class _QLoRAGatedFn(torch.autograd.Function):
         x2 = x.reshape(-1, K)
         members = [ops.GroupMember(w.quantized_data, w.block_scalers(), tr, a, b, bias, s, w.shape[0])
                    for w, tr, a, b, bias, s in zip(weights, _copies(weights, x2.shape[0]), las, lbs, biases, scales)]
-        h_cat, (gate, up, act) = ops.lora_group_fwd(x2, members, swiglu=True)
+        h_cat, (gate, up, act), tiles, paired = ops.lora_group_fwd(x2, members, swiglu=True, return_tiles=True)
+        _keep_tiles(ctx, tiles, paired, x2.shape[0], weights)
         ctx.save_for_backward(x2, h_cat, gate, up, *weights, *las, *lbs)
         ctx.scales = scales
         ctx.x_shape = x.shape
@@ -126,7 +140,8 @@ class _QLoRAFeedForwardFn(torch.autograd.Function):
         x2 = x.reshape(-1, K)
         members = [ops.GroupMember(w.quantized_data, w.block_scalers(), tr, a, b, bias, s, w.shape[0])
                    for w, tr, a, b, bias, s in zip(weights[:2], _copies(weights[:2], x2.shape[0]), las, lbs, biases, scales)]
-        h_cat, (gate, up, act) = ops.lora_group_fwd(x2, members, swiglu=True)
+        h_cat, (gate, up, act), tiles, paired = ops.lora_group_fwd(x2, members, swiglu=True, return_tiles=True)
+        _keep_tiles(ctx, tiles, paired, x2.shape[0], weights[:2])
         w2 = weights[2]
         h2 = ops.lora_hidden(act, las[2])
         tr = w2.backward_copy_for(act.shape[0], True)

@@ -52,13 +52,18 @@ class _QLoRALinearFn(torch.autograd.Function):
         _check_in_features(x, weight)
         x2 = x.reshape(-1, K)
         tr = weight.backward_copy_for(x2.shape[0], True)
+        # the expanded weight of a many-token call stays with the node when the backward will want a grad-input: its
+        # GEMM then reads these tiles instead of expanding the weight again (ops.KEEP_FORWARD_TILES_MAX_TOKENS)
+        # (only where that GEMM is the many-token launch: a grad-input of few output tiles stays on the fused kernel)
+        keep = ctx.needs_input_grad[0] and ops.keeps_forward_tiles(x2.shape[0]) and ops.gemm_expands_weight(x2.shape[0], K, N)
         if ONE_CALL_PER_DIRECTION and not ops.gemm_timer_installed():
-            y, h = ops.qlora_linear_fwd(x2, weight.quantized_data, weight.block_scalers(), N, lora_a, lora_b, scale, bias,
-                                        block_scalers_t=tr[1] if tr else None)
+            y, h, tiles = ops.qlora_linear_fwd(x2, weight.quantized_data, weight.block_scalers(), N, lora_a, lora_b, scale, bias,
+                                               block_scalers_t=tr[1] if tr else None, return_tiles=True)
         else:
             h = ops.lora_hidden(x2, lora_a)
-            y = ops.nf4_lora_linear_fwd(x2, weight.quantized_data, weight.block_scalers(), N, h, lora_b, scale, bias,
-                                        block_scalers_t=tr[1] if tr else None)
+            y, tiles = ops.nf4_lora_linear_fwd(x2, weight.quantized_data, weight.block_scalers(), N, h, lora_b, scale, bias,
+                                               block_scalers_t=tr[1] if tr else None, return_tiles=True)
+        ctx.tiles = tiles if keep else None
         ctx.save_for_backward(x2, h, weight, lora_a, lora_b)
         ctx.scale = scale
         ctx.x_shape = x.shape
@@ -73,13 +78,17 @@ class _QLoRALinearFn(torch.autograd.Function):
         need_x, _, need_a, need_b, need_bias, _ = ctx.needs_input_grad
         gx = ga = gb = gbias = None
         if need_x or need_a or need_b:
-            tr = weight.backward_copy_for(gy2.shape[0], False) if need_x else None
+            tiles = ctx.tiles if need_x else None
+            ctx.tiles = None
+            tr = weight.backward_copy_for(gy2.shape[0], False) if (need_x and tiles is None) else None
             if ONE_CALL_PER_DIRECTION and not ops.gemm_timer_installed():
                 gx, ga, gb = ops.qlora_linear_bwd(gy2, x2, h, weight.quantized_data, weight.block_scalers(), lora_a, lora_b,
-                                                  ctx.scale, transposed=tr, need_gx=need_x)
+                                                  ctx.scale, transposed=tr, need_gx=need_x, tiles=tiles)
             else:
                 gh, ga, gb = ops.lora_bwd(gy2, x2, h, lora_b, ctx.scale)
-                if need_x:
+                if need_x and tiles is not None:
+                    gx = ops.tiled_linear_dx(gy2, tiles, K, gh, lora_a, nf4_backward=True)
+                elif need_x:
                     gx = ops.nf4_linear_bwd_dx(gy2, weight.quantized_data, weight.block_scalers(), K, gh, lora_a, transposed=tr)
             if need_x:
                 gx = gx.view(ctx.x_shape)

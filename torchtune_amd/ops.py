@@ -239,6 +239,19 @@ def lora_hidden(x: torch.Tensor, lora_a: torch.Tensor) -> torch.Tensor:
 EXPANDED_WEIGHT_PATH = True
 
 
+# One expansion for both directions: a forward call that expanded its weight hands the scratch copy to the backward of the
+# same layer, whose grad-input GEMM reads those forward tiles (transposing LDS reads) instead of expanding the weight a
+# second time.  The transposing reads cost the grad-input GEMM 3.5 % whatever the token count, the expansion saved is a
+# fixed cost per weight: at 4096 tokens it is 14 % of a call, at 8192 tokens 7 %, so the tiles are kept for calls of at
+# most this many tokens (0: never; a large number: always).  Kept tiles hold 2 bytes per weight element from a layer's
+# forward to its backward (with activation checkpointing: from the recomputation to the backward of one layer).
+KEEP_FORWARD_TILES_MAX_TOKENS = 4096
+
+
+def keeps_forward_tiles(M: int) -> bool:
+    return bool(EXPANDED_WEIGHT_PATH and 0 < M <= KEEP_FORWARD_TILES_MAX_TOKENS)
+
+
 def gemm_expands_weight(M: int, n_out: int, k_contract: int) -> bool:
     """True when an NF4 GEMM call of this shape runs on the weight expanded once per call (needs no transposed copy)."""
     return bool(EXPANDED_WEIGHT_PATH and _lib.load().ttamd_nf4_gemm_expands_weight(M, n_out, k_contract))
@@ -256,10 +269,13 @@ def _gemm_workspace(lib, M: int, n_out: int, k_contract: int, device):
 def nf4_lora_linear_fwd(
     x: torch.Tensor, qdata: torch.Tensor, block_scalers: torch.Tensor, N: int, h: Optional[torch.Tensor] = None,
     lora_b: Optional[torch.Tensor] = None, scale: float = 0.0, bias: Optional[torch.Tensor] = None,
-    block_scalers_t: Optional[torch.Tensor] = None, col_scale: Optional[torch.Tensor] = None,
-) -> torch.Tensor:
+    block_scalers_t: Optional[torch.Tensor] = None, col_scale: Optional[torch.Tensor] = None, return_tiles: bool = False,
+):
     """y = x @ D(W).T (+bias) + scale * h @ lora_b.T ;  x [M,K] -> [M,N].  ``block_scalers_t``: the scalers transposed
-    ([K/64, N] fp32, second tensor of ``nf4_transpose_for_backward``): same result, cheaper scaler loads."""
+    ([K/64, N] fp32, second tensor of ``nf4_transpose_for_backward``): same result, cheaper scaler loads.
+
+    ``return_tiles=True`` returns ``(y, tiles)``: the call's scratch memory when it holds the weight expanded in forward
+    tile order (many tokens; what ``tiled_linear_dx`` reads), else ``None``."""
     x = _bf16_2d(x, "nf4_lora_linear_fwd")
     M, K = x.shape
     _check_nf4_operands("nf4_lora_linear_fwd", N, K, qdata, block_scalers, block_scalers_t)
@@ -293,6 +309,8 @@ def nf4_lora_linear_fwd(
         if events:
             events[1].record()
     _lib.check(rc, "nf4_lora_linear_fwd")
+    if return_tiles:
+        return y, (ws if ws is not None and lib.ttamd_nf4_gemm_expands_weight(M, N, K) else None)
     return y
 
 
@@ -391,11 +409,12 @@ def lora_bwd(
 # ---------------------------------------------------------------------------------------------------
 def qlora_linear_fwd(
     x: torch.Tensor, qdata: torch.Tensor, block_scalers: torch.Tensor, N: int, lora_a: torch.Tensor, lora_b: torch.Tensor,
-    scale: float, bias: Optional[torch.Tensor] = None, block_scalers_t: Optional[torch.Tensor] = None,
-) -> Tuple[torch.Tensor, torch.Tensor]:
+    scale: float, bias: Optional[torch.Tensor] = None, block_scalers_t: Optional[torch.Tensor] = None, return_tiles: bool = False,
+):
     """``(y, h)``: ``h = bf16(x @ lora_a.T)`` and ``y = x @ D(W).T (+ bias) + scale * h @ lora_b.T`` from one call of
     ``ttamd_qlora_linear_fwd_bf16`` (``lora_hidden`` followed by ``nf4_lora_linear_fwd``, the same launches and bits, out
-    of one workspace)."""
+    of one workspace).  ``return_tiles=True``: ``(y, h, tiles)`` with the call's workspace when its head holds the weight
+    expanded in forward tile order (many tokens), else ``None``."""
     x = _bf16_2d(x, "qlora_linear_fwd")
     lora_a = _bf16_2d(lora_a, "qlora_linear_fwd")
     lora_b = _bf16_2d(lora_b, "qlora_linear_fwd")
@@ -419,15 +438,19 @@ def qlora_linear_fwd(
             x.data_ptr(), qdata.data_ptr(), block_scalers.data_ptr(), _ptr(block_scalers_t), lora_a.data_ptr(), lora_b.data_ptr(),
             rank, float(scale), _ptr(bias), y.data_ptr(), h.data_ptr(), M, N, K, ws.data_ptr(), ws.numel(), _stream(x))
     _lib.check(rc, "qlora_linear_fwd")
+    if return_tiles:
+        return y, h, (ws if EXPANDED_WEIGHT_PATH and lib.ttamd_nf4_gemm_expands_weight(M, N, K) else None)
     return y, h
 
 
 def qlora_linear_bwd(
     gy: torch.Tensor, x: torch.Tensor, h: torch.Tensor, qdata: torch.Tensor, block_scalers: torch.Tensor, lora_a: torch.Tensor,
-    lora_b: torch.Tensor, scale: float, transposed=None, need_gx: bool = True,
+    lora_b: torch.Tensor, scale: float, transposed=None, need_gx: bool = True, tiles: Optional[torch.Tensor] = None,
 ) -> Tuple[Optional[torch.Tensor], torch.Tensor, torch.Tensor]:
     """``(gx or None, gA, gB)`` from one call of ``ttamd_qlora_linear_bwd_bf16`` (``lora_bwd`` followed by
-    ``nf4_linear_bwd_dx``, the same launches and bits, out of one workspace that also holds ``gh``)."""
+    ``nf4_linear_bwd_dx``, the same launches and bits, out of one workspace that also holds ``gh``).  ``tiles``: the
+    forward call's expanded weight (``qlora_linear_fwd(..., return_tiles=True)``); the grad-input then reads it instead
+    of expanding the weight again."""
     gy = _bf16_2d(gy, "qlora_linear_bwd")
     x = _bf16_2d(x, "qlora_linear_bwd")
     h = _bf16_2d(h, "qlora_linear_bwd")
@@ -447,13 +470,19 @@ def qlora_linear_bwd(
     gx = torch.empty(M, K, dtype=torch.bfloat16, device=dev) if need_gx else None
     ga = torch.empty(rank, K, dtype=torch.bfloat16, device=dev)
     gb = torch.empty(N, rank, dtype=torch.bfloat16, device=dev)
-    ws = _workspace(int(lib.ttamd_qlora_linear_bwd_workspace_bytes(M, N, K, rank)), dev)
+    if tiles is not None and (tiles.numel() * tiles.element_size() < 2 * N * K or not tiles.is_contiguous()):
+        raise ValueError(f"qlora_linear_bwd: the forward tiles must be contiguous and hold {N} x {K} bfloat16 elements")
+    if tiles is not None or not need_gx:  # no scratch memory for the GEMM stage
+        nbytes = ((M * rank * 2 + 255) // 256 + (int(lib.ttamd_lora_bwd_workspace_bytes(M, N, K, rank)) + 255) // 256) * 256
+    else:
+        nbytes = int(lib.ttamd_qlora_linear_bwd_workspace_bytes(M, N, K, rank))
+    ws = _workspace(nbytes, dev)
     with _on_device(dev):
         rc = lib.ttamd_qlora_linear_bwd_bf16(
             gy.data_ptr(), x.data_ptr(), h.data_ptr(), qdata.data_ptr(), block_scalers.data_ptr(),
-            _ptr(transposed[0]) if transposed else None, _ptr(transposed[1]) if transposed else None, lora_a.data_ptr(),
-            lora_b.data_ptr(), rank, float(scale), _ptr(gx), ga.data_ptr(), gb.data_ptr(), M, N, K, ws.data_ptr(), ws.numel(),
-            _stream(gy))
+            _ptr(transposed[0]) if transposed else None, _ptr(transposed[1]) if transposed else None,
+            _ptr(tiles) if need_gx else None, lora_a.data_ptr(), lora_b.data_ptr(), rank, float(scale), _ptr(gx), ga.data_ptr(),
+            gb.data_ptr(), M, N, K, ws.data_ptr(), ws.numel(), _stream(gy))
     _lib.check(rc, "qlora_linear_bwd")
     return gx, ga, gb
 
@@ -518,12 +547,16 @@ def _group_array(what: str, members: Sequence[GroupMember], K: int, ys: Sequence
     return arr, keep
 
 
-def lora_group_fwd(x: torch.Tensor, members: Sequence[GroupMember], swiglu: bool = False):
+def lora_group_fwd(x: torch.Tensor, members: Sequence[GroupMember], swiglu: bool = False, return_tiles: bool = False):
     """-> (h_cat [M, sum of ranks], [y_i [M, N_i]]): every member's ``y_i = x @ D(W_i).T (+ bias_i) + scale_i * h_i @ B_i.T``
     with ``h_i = x @ A_i.T`` (columns of ``h_cat``), in one pass over ``x`` for the hidden products.
 
     ``swiglu=True`` (two members of equal width: gate, up) appends ``act = silu(y_0) * y_1`` to the list, formed in the
-    epilogue of the GEMM launch where the many-token path serves the shape (``ttamd_nf4_lora_group_swiglu_fwd_bf16``)."""
+    epilogue of the GEMM launch where the many-token path serves the shape (``ttamd_nf4_lora_group_swiglu_fwd_bf16``).
+
+    ``return_tiles=True`` appends ``(tiles, paired)`` to the result: the call's scratch memory when its head holds the
+    members' weights expanded in forward tile order (``paired``: in the gated pair's layout), else ``(None, False)`` -
+    what ``lora_group_bwd(..., tiles=..., paired=...)`` takes."""
     x = _bf16_2d(x, "lora_group_fwd")
     M, K = x.shape
     dev = x.device
@@ -555,13 +588,20 @@ def lora_group_fwd(x: torch.Tensor, members: Sequence[GroupMember], swiglu: bool
         if events:
             events[1].record()
     _lib.check(rc, "lora_group_fwd")
+    outs = ys + [act] if swiglu else ys
+    if return_tiles:
+        layout = int(lib.ttamd_nf4_group_fwd_leaves_tiles(arr, n, M, K, 1 if swiglu else 0)) if fwd_bytes else 0
+        del keep
+        return h_cat, outs, (ws if layout else None), layout == 2
     del keep
-    return h_cat, (ys + [act] if swiglu else ys)
+    return h_cat, outs
 
 
 def lora_group_bwd(x: torch.Tensor, h_cat: torch.Tensor, members: Sequence[GroupMember], gys: Sequence[torch.Tensor],
-                   want_gx: bool = True):
-    """-> (gx [M, K] or None, [(gA_i, gB_i)], gh_cat): the backward of ``lora_group_fwd`` given the output gradients."""
+                   want_gx: bool = True, tiles: Optional[torch.Tensor] = None, paired: bool = False):
+    """-> (gx [M, K] or None, [(gA_i, gB_i)], gh_cat): the backward of ``lora_group_fwd`` given the output gradients.
+    ``tiles`` / ``paired``: what the forward call returned with ``return_tiles=True``; the grouped grad-input then reads
+    those tiles instead of expanding the members' weights again."""
     x = _bf16_2d(x, "lora_group_bwd")
     h_cat = _bf16_2d(h_cat, "lora_group_bwd")
     M, K = x.shape
@@ -574,7 +614,7 @@ def lora_group_bwd(x: torch.Tensor, h_cat: torch.Tensor, members: Sequence[Group
     r_total = sum(int(e.rank) for e in arr)
     if tuple(h_cat.shape) != (M, r_total):
         raise ValueError(f"lora_group_bwd: h_cat is {tuple(h_cat.shape)}, expected {(M, r_total)}")
-    if want_gx and any(m.transposed is None for m in members) and not (
+    if want_gx and tiles is None and any(m.transposed is None for m in members) and not (
             EXPANDED_WEIGHT_PATH and _lib.load().ttamd_nf4_group_bwd_dx_workspace_bytes(arr, len(members), M, K)):
         raise ValueError("lora_group_bwd: the grouped grad-input needs every member's transposed copy (or a shape the "
                          "expanded-weight path serves)")
@@ -588,12 +628,20 @@ def lora_group_bwd(x: torch.Tensor, h_cat: torch.Tensor, members: Sequence[Group
         _lib.check(rc, "lora_group_bwd")
         if want_gx:
             events = _gemm_timer("bwd_group", M, [m.N for m in members], K, [int(e.rank) for e in arr]) if _gemm_timer is not None else None
-            dx_bytes = int(lib.ttamd_nf4_group_bwd_dx_workspace_bytes(arr, n, M, K)) if EXPANDED_WEIGHT_PATH else 0
-            dx_ws = torch.empty(dx_bytes // 4, dtype=torch.float32, device=dev) if dx_bytes else None
-            if events:
-                events[0].record()
-            rc = lib.ttamd_nf4_group_bwd_dx_ws_bf16(arr, n, gh_cat.data_ptr(), gx.data_ptr(), M, K,
-                                                    dx_ws.data_ptr() if dx_ws is not None else None, dx_bytes, _stream(x))
+            if tiles is not None:
+                if tiles.numel() * tiles.element_size() < 2 * K * sum(m.N for m in members) or not tiles.is_contiguous():
+                    raise ValueError("lora_group_bwd: the forward tiles do not hold the members' weights")
+                if events:
+                    events[0].record()
+                rc = lib.ttamd_nf4_group_bwd_dx_tiles_bf16(arr, n, gh_cat.data_ptr(), gx.data_ptr(), M, K, tiles.data_ptr(),
+                                                           1 if paired else 0, _stream(x))
+            else:
+                dx_bytes = int(lib.ttamd_nf4_group_bwd_dx_workspace_bytes(arr, n, M, K)) if EXPANDED_WEIGHT_PATH else 0
+                dx_ws = torch.empty(dx_bytes // 4, dtype=torch.float32, device=dev) if dx_bytes else None
+                if events:
+                    events[0].record()
+                rc = lib.ttamd_nf4_group_bwd_dx_ws_bf16(arr, n, gh_cat.data_ptr(), gx.data_ptr(), M, K,
+                                                        dx_ws.data_ptr() if dx_ws is not None else None, dx_bytes, _stream(x))
             if events:
                 events[1].record()
             _lib.check(rc, "nf4_group_bwd_dx")
@@ -879,7 +927,7 @@ def tiled_lora_linear(x: torch.Tensor, tiled: torch.Tensor, n_out: int, lx: torc
 
 
 def tiled_linear_dx(gy: torch.Tensor, tiled_fwd: torch.Tensor, K: int, gh: Optional[torch.Tensor] = None,
-                    lora_a: Optional[torch.Tensor] = None) -> torch.Tensor:
+                    lora_a: Optional[torch.Tensor] = None, nf4_backward: bool = False) -> torch.Tensor:
     """``gx = gy @ Wd (+ gh @ lora_a)`` with ``Wd`` [N, K] given as the FORWARD tiles (what ``tiled_linear`` / the expanded
     NF4 forward read): the grad-input without a transposed copy of the weight, bit-equal to the launch on tiles of
     ``Wd.T``.  ``tiled_fwd`` may be longer than N * K elements (a workspace whose head holds the tiles)."""
@@ -897,7 +945,10 @@ def tiled_linear_dx(gy: torch.Tensor, tiled_fwd: torch.Tensor, K: int, gh: Optio
     gx = torch.empty(M, K, dtype=torch.bfloat16, device=gy.device)
     lib = _lib.load()
     with _on_device(gy.device):
-        events = _gemm_timer("tiled", M, K, N, 0) if _gemm_timer is not None else None
+        # an installed timer books the call as what it is: the grad-input of an NF4 layer, or a GEMM on fake-quantised tiles
+        events = None
+        if _gemm_timer is not None:
+            events = _gemm_timer("bwd", M, N, K, r) if nf4_backward else _gemm_timer("tiled", M, K, N, 0)
         if events:
             events[0].record()
         rc = lib.ttamd_tiled_linear_dx_bf16(gy.data_ptr(), tiled_fwd.data_ptr(), _ptr(gh), _ptr(lora_a), r, gx.data_ptr(), M, N, K,
