@@ -564,6 +564,477 @@ __global__ __launch_bounds__(256) void nf4_gemm_rs_kernel(const RsArgs g, const 
 #endif
 }
 
+// The same kernel on v_mfma_f32_16x16x32_bf16.  This part is power-limited under matrix load and the 16 x 16 x 32 shape
+// sustains 13 % more FLOP/s than 32 x 32 x 16 at the same power (2.04 against 1.80 PFLOP/s for MFMA-only loops), so the
+// loop is re-cut for it: a lane (l15, lg) of the weight operand holds row l15 of a 16-column tile and the 8 contraction
+// elements [16 lg + 8 ks, + 8) of substep ks - still exactly one dword of codes - and a 64-wide k-step is two substeps
+// of NT (4) x MT (BM / 16) MFMAs.  Loads, LDS stages and the table are those of the kernel above; what changes is who
+// reads what: the code bytes a direct-to-LDS instruction leaves as 16 bytes per (row, half) are read back as 8 bytes per
+// (row, quarter), the activation operand is chunk 2 lg + ks of its row.
+//   phase p = (substep ks = p / 2, half ih = p % 2): the NT x MT/2 MFMAs of substep ks against activation tiles
+//     [MT/2 ih, + MT/2), the operand reads of the next phase, the finish of the 8 table entries fetched in the previous
+//     phase and the fetch of the next 8 (tiles 0, 1 of a substep in one phase, tiles 2, 3 in the next);
+//   the workgroup barrier of a k-step stands after phase 0: from phase 1 on the entries fetched belong to the next
+//     k-step's codes, which are read back right after it.
+template <int BM, int MODE, bool SPLIT, bool SEG = false>
+__global__ __launch_bounds__(256) void nf4_gemm_rs16_kernel(const RsArgs g, const RsSegs sg) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  static_assert(BM == 256 || BM == 128, "BM");
+  static_assert(!SEG || (MODE == 1 && !SPLIT), "segments: grad-input kernels only");
+  constexpr bool PER_ELEM = MODE == 1;
+  constexpr bool SCAL_T = MODE == 2;
+  using L = RsLayout<BM>;
+  constexpr int MT = BM / 16;       // 16-row activation tiles (MFMA columns) per wave
+  constexpr int MH = MT / 2;        // of which a phase takes half
+  constexpr int NT = 4;             // 16-column weight tiles (MFMA rows) per wave
+  constexpr int ND = 2;             // direct-to-LDS instructions per k-step for the wave's code bytes (32 rows each)
+  constexpr int kALoads = BM / 32;  // and for its share of the activation tile (8 rows each)
+  constexpr int kBatch = kALoads + ND + (MODE == 0 ? ND : 1);
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l31 = lane & 31, h = lane >> 5;    // roles on the load side
+  const int l15 = lane & 15, lg = lane >> 4;   // roles on the MFMA side
+
+  int tile_m, tile_n;
+  {
+    const int id = blockIdx.x;
+    if ((g.tiles_m & 7) == 0) {
+      const int xcd = id & 7, slot = id >> 3, band = g.tiles_m >> 3;
+      tile_m = xcd * band + slot % band;
+      tile_n = slot / band;
+    } else {
+      tile_m = id / g.tiles_n;
+      tile_n = id % g.tiles_n;
+    }
+  }
+  const int m0 = tile_m * BM, n0 = tile_n * kBN;
+  const int Kc = SEG ? sg.Kc[0] : g.Kc;
+  const int nkf = Kc >> 6;
+  int kb = 0, nk = nkf;
+  if constexpr (SEG) {
+    for (int q = 1; q < sg.n; ++q) nk += sg.Kc[q] >> 6;
+  }
+  if constexpr (SPLIT) {
+    kb = blockIdx.y * g.ksteps;
+    nk = nkf - kb < g.ksteps ? nkf - kb : g.ksteps;
+  }
+
+  __shared__ float2 lut_s[256];
+  lut_s[tid] = make_float2(round_to_bf16(kNF4Rs[tid >> 4]), round_to_bf16(kNF4Rs[tid & 15]));
+  const char* lut = reinterpret_cast<const char*>(lut_s);
+
+  // ---- load side: as in nf4_gemm_rs_kernel
+  const int a_r8 = lane >> 3;
+  uint32_t a_off[kALoads];
+  uint32_t w_off[ND], s_off[ND];
+  auto set_offsets = [&](int kc) {
+#pragma unroll
+    for (int i = 0; i < kALoads; ++i) {
+      const int trow = wv * (BM / 4) + 8 * i + a_r8;
+      const int chunk = (lane & 7) ^ ((trow >> 1) & 7);
+      int row = m0 + trow;
+      row = row < g.M ? row : g.M - 1;
+      a_off[i] = ((uint32_t)row * (uint32_t)kc + chunk * 8) * 2u;
+    }
+#pragma unroll
+    for (int j = 0; j < ND; ++j) {
+      int col = n0 + wv * 64 + 32 * j + l31;
+      col = col < g.Nout ? col : g.Nout - 1;
+      w_off[j] = (uint32_t)(((int64_t)col * kc) >> 1) + 16 * h;
+      s_off[j] = (uint32_t)col * (uint32_t)(kc >> 6) * 4u;
+    }
+    if constexpr (SCAL_T) {
+      int col = n0 + wv * 64 + lane;
+      col = col < g.Nout ? col : g.Nout - 1;
+      s_off[0] = (uint32_t)col * 4u;
+    }
+    if constexpr (PER_ELEM) {
+      int ob = (n0 >> 6) + wv;
+      const int nob = g.Nout >> 6;
+      ob = ob < nob ? ob : nob - 1;
+      s_off[0] = ((uint32_t)ob * (uint32_t)kc + lane) * 4u;
+    }
+  };
+  set_offsets(Kc);
+
+  auto dma16 = [&](uint32_t voff, const char* base, uint32_t lds, int imm) {
+    asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 ::"v"(voff), "s"(base), "s"(lds), "n"(imm) : "memory", "m0", "scc");
+  };
+  auto dma4 = [&](uint32_t voff, const char* base, uint32_t lds, int imm) {
+    asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1"
+                 ::"v"(voff), "s"(base), "s"(lds), "n"(imm) : "memory", "m0", "scc");
+  };
+  const uint32_t lds0 = (uint32_t)(uintptr_t)TT_LDS_PTR(smem);
+  struct BatchAddr {
+    const char *xb, *cb, *sb;
+    uint32_t abase, wcodes, wscal;
+  };
+  const int64_t s_stride = PER_ELEM ? 256 : SCAL_T ? (int64_t)g.Nout * 4 : 4;
+  auto batch_addr_at = [&](const char* xb, const char* cb, const char* sb, int sa, int sw) -> BatchAddr {
+    BatchAddr b;
+    b.xb = xb;
+    b.cb = cb;
+    b.sb = sb;
+    b.abase = lds0 + sa * L::kStageA + wv * (BM / 4) * 128;
+    b.wcodes = lds0 + L::kWOff + sw * L::kStageW + wv * ND * 1024;
+    b.wscal = lds0 + L::kWOff + sw * L::kStageW + 8192 + wv * 512;
+    return b;
+  };
+  auto batch_addr = [&](int t, int sa, int sw) -> BatchAddr {
+    const int tk = kb + (t < nk ? t : nk - 1);
+    return batch_addr_at(reinterpret_cast<const char*>(g.X) + ((int64_t)tk << 7),
+                         reinterpret_cast<const char*>(g.codes) + ((int64_t)tk << 5),
+                         reinterpret_cast<const char*>(g.scal) + tk * s_stride, sa, sw);
+  };
+  auto issue_one = [&](const BatchAddr& b, int d) {
+    if (d < kALoads) {
+      dma16(a_off[d], b.xb, b.abase, d * 1024);
+    } else if (d < kALoads + ND) {
+      const int j = d - kALoads;
+      dma16(w_off[j], b.cb, b.wcodes, j * 1024);
+    } else if (d < kBatch) {
+      const int j = d - kALoads - ND;
+      dma4(s_off[j], b.sb, b.wscal, j * 256);
+    }
+  };
+  auto issue = [&](int t, int sa, int sw) {
+    const BatchAddr b = batch_addr(t, sa, sw);
+#pragma unroll
+    for (int d = 0; d < kBatch; ++d) issue_one(b, d);
+  };
+
+  // ---- weights: tile j is rows 16 j + l15 of the wave's 64; substep ks of this lane is code dword 2 lg + ks of the
+  //      row's eight.  A load instruction left row 32 J + r, bytes [16 H, + 16) at lane r + 32 H of piece J.
+  uint32_t codes[NT][2];
+  float sc[NT], sc_next[NT];
+  float2 pend[2][4];  // the eight table entries in flight: [tile of the pair][code byte]
+  u32x4_t wfa[NT], wfb[NT];
+  bf16x8_t xfa[MH], xfb[MH];
+
+  auto fetch_byte = [&](int jj, int j, int ks, int b) {
+    uint32_t off;
+    if (b == 0) {
+      asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_0"
+          : "=v"(off) : "v"(3u), "v"(codes[j][ks]));
+    } else {
+      off = ((codes[j][ks] >> (8 * b)) & 0xffu) << 3;
+    }
+    pend[jj][b] = *reinterpret_cast<const float2*>(lut + off);
+  };
+  auto finish_byte = [&](u32x4_t (&wf)[NT], int jj, int j, int b, const float (&s)[NT], const float (&s8)[8]) {
+    if constexpr (PER_ELEM)
+      wf[j][b] = pack_bf16x2(pend[jj][b].x * s8[2 * b], pend[jj][b].y * s8[2 * b + 1]);
+    else
+      wf[j][b] = pack_bf16x2(pend[jj][b].x * s[j], pend[jj][b].y * s[j]);
+  };
+  auto load_s8 = [&](float (&s8)[8], int sw, int ks) {
+    if constexpr (PER_ELEM) {
+      const f32x4_t* sp = reinterpret_cast<const f32x4_t*>(smem + L::kWOff + sw * L::kStageW + 8192 + wv * 512 + (16 * lg + 8 * ks) * 4);
+      const f32x4_t a = sp[0], b = sp[1];
+      s8[0] = a.x; s8[1] = a.y; s8[2] = a.z; s8[3] = a.w; s8[4] = b.x; s8[5] = b.y; s8[6] = b.z; s8[7] = b.w;
+    }
+  };
+  auto load_codes = [&](int sw, float (&s_out)[NT]) {
+    const char* wbase = smem + L::kWOff + sw * L::kStageW;
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+      const u32x2_t v = *reinterpret_cast<const u32x2_t*>(wbase + (wv * ND + (j >> 1)) * 1024 +
+                                                          (16 * (j & 1) + l15 + 32 * (lg >> 1)) * 16 + 8 * (lg & 1));
+      codes[j][0] = v.x; codes[j][1] = v.y;
+      if constexpr (MODE == 0) s_out[j] = *reinterpret_cast<const float*>(wbase + 8192 + wv * 512 + (j >> 1) * 256 + (16 * (j & 1) + l15) * 4);
+      if constexpr (SCAL_T) s_out[j] = *reinterpret_cast<const float*>(wbase + 8192 + wv * 512 + (16 * j + l15) * 4);
+    }
+  };
+
+  f32x4_t acc[NT][MT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j)
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) acc[j][i][v] = 0.f;
+
+  // operand read offsets inside a stage: row 16 i + l15, chunk 2 lg + ks, slot = chunk ^ ((row >> 1) & 7)
+  int x_off[2];
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks) x_off[ks] = l15 * 128 + (((2 * lg + ks) ^ ((l15 >> 1) & 7)) << 4);
+
+  // One phase, in quarters.  Quarter q:
+  //   MFMAs of weight tile q against the MH activation tiles of the phase's half
+  //   operand reads of the NEXT phase: activation tiles [MH/4 q, + MH/4) of its half
+  //   finish + fetch of code bytes 2 (q % 2), 2 (q % 2) + 1 of tile q / 2 of the pair (finish: what the previous phase
+  //     fetched, into wf_next of the pair jp_fin; fetch: the pair jp_fetch of substep ks_fetch)
+  //   up to two direct-to-LDS loads of batch `b`
+  auto phase = [&](const bf16x8_t (&xf_use)[MH], int ih_use, const u32x4_t (&wf_use)[NT], bf16x8_t (&xf_next)[MH], int st_next,
+                   int ks_next, int ih_next, u32x4_t (&wf_next)[NT], int jp_fin, const float (&s_fin)[NT], int sw_fin, int ks_fin,
+                   int jp_fetch, int ks_fetch, const BatchAddr& b, int d_first, int d_even, int d_odd) {
+    float s8[8];
+    load_s8(s8, sw_fin, ks_fin);
+    const char* sA = smem + st_next * L::kStageA + (MH * ih_next) * 2048;
+    int d = d_first;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int nd = (q & 1) ? d_odd : d_even;
+      const int jj = q >> 1, b0 = 2 * (q & 1);
+      // The MFMAs are written in assembly with the accumulator tied to itself in the AGPR file: left to the register
+      // allocator, the 64 four-register accumulators of this loop get different source and destination registers and are
+      // copied around the loop's back edge (700 v_accvgpr moves per k-step).  The scheduler does not know such a
+      // statement for a matrix instruction, so the interleaving is spelled out: one MFMA, one piece of the quarter's
+      // other work, a scheduling barrier.  A 16 x 16 x 32 MFMA keeps the pipe for 16 cycles and the wave issues in
+      // order: whatever follows it in program order rides in the 12 cycles before the next one can start.
+      auto mfma = [&](int i) {
+        asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[q][MH * ih_use + i]) : "v"(wf_use[q]), "v"(xf_use[i]));
+      };
+      auto other = [&](int slot) {  // the quarter's other work in eight pieces
+        constexpr int kReads = MH / 4;  // operand reads of the next phase per quarter: 2 (BM = 256) or 1
+        switch (slot) {
+          case 0:
+            xf_next[kReads * q] = *reinterpret_cast<const bf16x8_t*>(sA + (kReads * q) * 2048 + x_off[ks_next]);
+            break;
+          case 1: finish_byte(wf_next, jj, 2 * jp_fin + jj, b0, s_fin, s8); break;
+          case 2: fetch_byte(jj, 2 * jp_fetch + jj, ks_fetch, b0); break;
+          case 3:
+            if (kReads > 1) xf_next[kReads * q + 1] = *reinterpret_cast<const bf16x8_t*>(sA + (kReads * q + 1) * 2048 + x_off[ks_next]);
+            break;
+          case 4: finish_byte(wf_next, jj, 2 * jp_fin + jj, b0 + 1, s_fin, s8); break;
+          case 5: fetch_byte(jj, 2 * jp_fetch + jj, ks_fetch, b0 + 1); break;
+          case 6:
+            if (nd > 0) issue_one(b, d);
+            break;
+          default:
+            if (nd > 1) issue_one(b, d + 1);
+            break;
+        }
+      };
+      constexpr int kPer = 8 / MH;  // pieces per MFMA: 1 (BM = 256) or 2
+#pragma unroll
+      for (int i = 0; i < MH; ++i) {
+        mfma(i);
+#pragma unroll
+        for (int u = 0; u < kPer; ++u) other(kPer * i + u);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      d += nd;
+    }
+  };
+
+  // ---- software pipeline: as in nf4_gemm_rs_kernel (activation tile t in A stage t % 4, this wave's codes in W stage
+  //      t % 3, batch t + 2 issued during phases 0 and 1 of step t), with the barrier of step t after phase 0.  There
+  //      this wave's batch t + 1 has landed (it was issued a step ago; the loads phase 0 just issued may be in flight)
+  //      and, past the barrier, everybody's.  A wave that issues batch t + 2 into the A stage of tile t - 2 has passed
+  //      barrier t - 1, which every wave reaches only after its last read of tile t - 2.
+  const char *pxb, *pcb, *psb;
+  auto seg_base = [&](int q, int step) {
+    pxb = reinterpret_cast<const char*>(sg.X[q]) + ((int64_t)step << 7);
+    pcb = reinterpret_cast<const char*>(sg.codes[q]) + ((int64_t)step << 5);
+    psb = reinterpret_cast<const char*>(sg.scal[q]) + (int64_t)step * 256;
+  };
+  if constexpr (SEG) {
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      seg_base(0, t);
+      const BatchAddr bt = batch_addr_at(pxb, pcb, psb, t, t);
+#pragma unroll
+      for (int d = 0; d < kBatch; ++d) issue_one(bt, d);
+    }
+  } else {
+    issue(0, 0, 0);
+    issue(1, 1, 1);
+  }
+  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kBatch) : "memory");  // batch 0 landed everywhere, table written
+  load_codes(0, sc);
+  {
+    // substep 0 in full, and the first pair of substep 1 on its way
+    float s8[8];
+    load_s8(s8, 0, 0);
+#pragma unroll
+    for (int jp = 0; jp < 2; ++jp) {
+#pragma unroll
+      for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+        for (int b = 0; b < 4; ++b) fetch_byte(jj, 2 * jp + jj, 0, b);
+#pragma unroll
+      for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+        for (int b = 0; b < 4; ++b) finish_byte(wfa, jj, 2 * jp + jj, b, sc, s8);
+    }
+#pragma unroll
+    for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+      for (int b = 0; b < 4; ++b) fetch_byte(jj, jj, 1, b);
+  }
+#pragma unroll
+  for (int i = 0; i < MH; ++i) xfa[i] = *reinterpret_cast<const bf16x8_t*>(smem + i * 2048 + x_off[0]);
+
+  constexpr int kDEven = (kBatch + 7) / 8 > 1 ? 2 : 1;
+  constexpr int kDOdd = (kBatch - 4 * kDEven + 3) / 4;
+  static_assert(4 * kDEven + 4 * kDOdd >= kBatch && kDOdd <= 2 && kDOdd >= 0, "batch does not fit the 8 quarter phases");
+  constexpr int kInPhase0 = 2 * (kDEven + kDOdd) < kBatch ? 2 * (kDEven + kDOdd) : kBatch;  // loads phase 0 issues
+  int a0 = 0, w0 = 0;
+  auto k_step = [&](int64_t adv) {
+    const int a1 = (a0 + 1) & 3, a2 = (a0 + 2) & 3;
+    const int w1 = w0 == 2 ? 0 : w0 + 1, w2 = w1 == 2 ? 0 : w1 + 1;
+    const BatchAddr b = batch_addr_at(pxb, pcb, psb, a2, w2);
+    pxb += adv << 7;
+    pcb += adv << 5;
+    psb += adv * s_stride;
+    //    use        use   next operands          builds  finish: pair, scalers, stage, substep   fetch: pair, substep
+    phase(xfa, 0, wfa, xfb, a0, 0, 1, wfb, 0, sc, w0, 1, 1, 1, b, 0, kDEven, kDOdd);
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kInPhase0) : "memory");
+    load_codes(w1, sc_next);
+    phase(xfb, 1, wfa, xfa, a0, 1, 0, wfb, 1, sc, w0, 1, 0, 0, b, kInPhase0, kDEven, kDOdd);
+    phase(xfa, 0, wfb, xfb, a0, 1, 1, wfa, 0, sc_next, w1, 0, 1, 0, b, kBatch, 0, 0);
+    phase(xfb, 1, wfb, xfa, a1, 0, 0, wfa, 1, sc_next, w1, 0, 0, 1, b, kBatch, 0, 0);
+#pragma unroll
+    for (int j = 0; j < NT; ++j) sc[j] = sc_next[j];
+    a0 = a1;
+    w0 = w1;
+  };
+  if constexpr (!SEG) {
+    const BatchAddr b2 = batch_addr(2, 0, 0);
+    pxb = b2.xb; pcb = b2.cb; psb = b2.sb;
+    for (int kt = 0; kt < nk; ++kt) k_step(kt + 3 < nk ? 1 : 0);
+  } else {
+    int issued = 2;
+    for (int q = 0; q < sg.n; ++q) {
+      int steps = sg.Kc[q] >> 6;
+      if (q == 0) {
+        steps -= 2;
+        seg_base(0, nk > 2 ? 2 : 1);
+      } else {
+        set_offsets(sg.Kc[q]);
+        seg_base(q, 0);
+      }
+      if (q == sg.n - 1) steps += 2;
+      for (int it = 0; it < steps; ++it) {
+        k_step(issued + 1 < nk ? 1 : 0);
+        ++issued;
+      }
+    }
+  }
+
+  // the clamped batches issued by the last two steps; and the last MFMAs of the loop (assembly: the compiler does not
+  // know they are matrix instructions) have left the pipeline before anything reads their accumulators
+  asm volatile("s_waitcnt vmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+  // ---- adapter: one MFMA step per 32 ranks, operands straight from global memory; lane (l15, lg) holds ranks
+  //      rc + 8 lg .. + 7 of weight column / activation row l15 of its tile
+  const int n_adapters = SEG ? sg.n : 1;
+  for (int ad = 0; ad < n_adapters; ++ad) {
+    const uint16_t* __restrict__ lX = SEG ? sg.lX[ad] : g.lX;
+    const uint16_t* __restrict__ lW = SEG ? sg.lW[ad] : g.lW;
+    const int R = SEG ? sg.R[ad] : g.R;
+    if (!(R > 0 && lX != nullptr && (!SPLIT || blockIdx.y == 0))) continue;
+    for (int rc = 0; rc < R; rc += 32) {
+      const int r0 = rc + 8 * lg;
+      const bool in = r0 < R;  // R % 8 == 0: a lane's 8 indices are all in or all out
+      bf16x8_t wfr[NT];
+#pragma unroll
+      for (int j = 0; j < NT; ++j) {
+        int col = n0 + wv * 64 + 16 * j + l15;
+        col = col < g.Nout ? col : g.Nout - 1;
+        u32x4_t raw = {0, 0, 0, 0};
+        if (in) {
+          if (g.lw_row_major) {
+            raw = *reinterpret_cast<const u32x4_t*>(lW + (int64_t)col * R + r0);
+          } else {
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+              const uint32_t lo = lW[(int64_t)(r0 + 2 * d) * g.Nout + col];
+              const uint32_t hi = lW[(int64_t)(r0 + 2 * d + 1) * g.Nout + col];
+              raw[d] = lo | (hi << 16);
+            }
+          }
+        }
+        wfr[j] = __builtin_bit_cast(bf16x8_t, raw);
+      }
+#pragma unroll
+      for (int ih = 0; ih < 2; ++ih) {
+        bf16x8_t xfr[MH];
+#pragma unroll
+        for (int i = 0; i < MH; ++i) {
+          int row = m0 + 16 * (MH * ih + i) + l15;
+          row = row < g.M ? row : g.M - 1;
+          u32x4_t raw = {0, 0, 0, 0};
+          if (in) raw = *reinterpret_cast<const u32x4_t*>(lX + (int64_t)row * g.ldlx + r0);
+          if (g.lscale != 1.0f) {
+#pragma unroll
+            for (int d = 0; d < 4; ++d)
+              raw[d] = pack_bf16x2(bits_f32(raw[d] << 16) * g.lscale, bits_f32(raw[d] & 0xffff0000u) * g.lscale);
+          }
+          xfr[i] = __builtin_bit_cast(bf16x8_t, raw);
+        }
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+#pragma unroll
+          for (int i = 0; i < MH; ++i)
+            acc[j][MH * ih + i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wfr[j], xfr[i], acc[j][MH * ih + i], 0, 0, 0);
+      }
+    }
+  }
+
+  // ---- epilogue.  acc[j][i][v] = C[m][n] with m = m0 + 16 i + l15 and n = n0 + 64 wv + 16 j + 4 lg + v.
+  if constexpr (SPLIT) {
+    // fp32 partial tile straight from the registers: a lane holds four consecutive columns of a row (16 bytes), the
+    // four lane groups make the 64 bytes of a weight tile's columns
+    if (n0 + wv * 64 >= g.Nout) return;
+    float* P = g.part + (int64_t)blockIdx.y * g.M * g.Nout + n0 + wv * 64 + 4 * lg;
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+      const int row = m0 + 16 * i + l15;
+      if (row >= g.M) continue;
+#pragma unroll
+      for (int j = 0; j < NT; ++j) *reinterpret_cast<f32x4_t*>(P + (int64_t)row * g.Nout + 16 * j) = acc[j][i];
+    }
+    return;
+  }
+  __syncthreads();                      // every wave is done reading the activation ring
+  if (n0 + wv * 64 >= g.Nout) return;  // the whole 64-column band of this wave lies outside (no barrier follows)
+  {
+    // each wave transposes its BM x 64 band through LDS (BM x 128 bytes per wave) and writes whole 128-byte row
+    // segments; 16-byte chunk c of row r sits in slot c ^ (r & 7)
+    char* band = smem + wv * (BM * 128);
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+      float b4[4] = {0.f, 0.f, 0.f, 0.f};
+      if (g.bias) {
+        const u32x2_t bb = *reinterpret_cast<const u32x2_t*>(g.bias + n0 + wv * 64 + 16 * j + 4 * lg);
+        b4[0] = bits_f32(bb.x << 16); b4[1] = bits_f32(bb.x & 0xffff0000u);
+        b4[2] = bits_f32(bb.y << 16); b4[3] = bits_f32(bb.y & 0xffff0000u);
+      }
+      float c4[4] = {1.f, 1.f, 1.f, 1.f};
+      if (g.cscale) {
+        const u32x2_t cc = *reinterpret_cast<const u32x2_t*>(g.cscale + n0 + wv * 64 + 16 * j + 4 * lg);
+        c4[0] = bits_f32(cc.x << 16); c4[1] = bits_f32(cc.x & 0xffff0000u);
+        c4[2] = bits_f32(cc.y << 16); c4[3] = bits_f32(cc.y & 0xffff0000u);
+      }
+#pragma unroll
+      for (int i = 0; i < MT; ++i) {
+        const int r = 16 * i + l15;
+        u32x2_t o;
+        o.x = pack_bf16x2((acc[j][i][0] + b4[0]) * c4[0], (acc[j][i][1] + b4[1]) * c4[1]);
+        o.y = pack_bf16x2((acc[j][i][2] + b4[2]) * c4[2], (acc[j][i][3] + b4[3]) * c4[3]);
+        *reinterpret_cast<u32x2_t*>(band + r * 128 + (((2 * j + (lg >> 1)) ^ (r & 7)) << 4) + 8 * (lg & 1)) = o;
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const int c = lane & 7;
+    uint16_t* crow = g.C + n0 + wv * 64 + 8 * c;
+#pragma unroll 8
+    for (int t = 0; t < BM / 8; ++t) {
+      const int r = 8 * t + (lane >> 3);
+      const u32x4_t v = *reinterpret_cast<const u32x4_t*>(band + r * 128 + ((c ^ (r & 7)) << 4));
+      if (m0 + r < g.M) *reinterpret_cast<u32x4_t*>(crow + (int64_t)(m0 + r) * g.Nout) = v;
+    }
+  }
+#endif
+}
+
 // C[m][n] = bf16((sum over slices of part[s][m][n] + bias[n]) * cscale[n]); a thread takes 8 consecutive columns.
 __global__ __launch_bounds__(256) void nf4_gemm_rs_reduce_kernel(const float* __restrict__ part, int splits, int64_t mn,
                                                                  int Nout, const uint16_t* __restrict__ bias,
@@ -608,20 +1079,31 @@ int launch_rs(RsArgs& g, int splits, hipStream_t s, const RsSegs* segs = nullptr
   using L = RsLayout<BM>;
   g.tiles_m = (g.M + BM - 1) / BM;
   g.tiles_n = (g.Nout + kBN - 1) / kBN;
-  // the limit is a per-device attribute of the function: set it for the current device once (a race only repeats the call)
+  // Full tiles of a single layer run the 16 x 16 x 32 form of the loop: 1 - 5 % faster there (the part clocks 15 % higher
+  // on that MFMA shape, and the loop needs 15 % more cycles for the 64 extra MFMA issues of a k-step); with 128-row tiles
+  // it is 1 - 5 % slower and with segments it spills, so those keep the 32 x 32 x 16 form.
+  constexpr bool kMfma16 = BM == 256 && !SPLIT && !SEG;
+  const void* fn;
+  if constexpr (kMfma16)
+    fn = reinterpret_cast<const void*>(&nf4_gemm_rs16_kernel<BM, MODE, SPLIT, SEG>);
+  else
+    fn = reinterpret_cast<const void*>(&nf4_gemm_rs_kernel<BM, MODE, SPLIT, SEG>);
+  // the LDS limit is a per-device attribute of the function: set it for the current device once (a race only repeats the call)
   static bool attr_set[64] = {};
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = -1;
   if (dev < 0 || !attr_set[dev]) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&nf4_gemm_rs_kernel<BM, MODE, SPLIT, SEG>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, L::kTotal);
+    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, L::kTotal);
     if (e != hipSuccess)
       return fail(TTAMD_ELAUNCH, "nf4_gemm_rs: cannot reserve %d bytes of LDS: %s", L::kTotal, hipGetErrorString(e));
     if (dev >= 0) attr_set[dev] = true;
   }
   static const RsSegs no_segs = {};
-  nf4_gemm_rs_kernel<BM, MODE, SPLIT, SEG><<<dim3((unsigned)(g.tiles_m * g.tiles_n), (unsigned)splits), dim3(256), L::kTotal, s>>>(
-      g, segs ? *segs : no_segs);
+  const dim3 grid((unsigned)(g.tiles_m * g.tiles_n), (unsigned)splits), block(256);
+  if constexpr (kMfma16)
+    nf4_gemm_rs16_kernel<BM, MODE, SPLIT, SEG><<<grid, block, L::kTotal, s>>>(g, segs ? *segs : no_segs);
+  else
+    nf4_gemm_rs_kernel<BM, MODE, SPLIT, SEG><<<grid, block, L::kTotal, s>>>(g, segs ? *segs : no_segs);
   return check_launch("nf4_gemm_rs");
 }
 
