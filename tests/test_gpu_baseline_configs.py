@@ -11,7 +11,7 @@ These tensors are too large for an eager CPU pass, so parity is shown in two lin
   codes, scaler bytes, factors and dequantised values bit for bit, with the one quantity that couples the whole tensor,
   the scaler mean, checked separately against an exact fp64 mean;
 * the fused layer (forward, grad-input, both adapter gradients) against fp32 matmuls of that bit-exactly dequantised
-  weight on the GPU, at rtol 1e-2 / atol 1e-2 (bf16 inputs, fp32 accumulation on both sides; adapter gradients at 2e-2 of
+  weight on the GPU, at rtol 1e-2 / atol 1e-2 (bf16 inputs, fp32 accumulation on both sides; adapter gradients at 4e-3 of
   their largest entry), plus the CPU oracle's own unfused bf16 forward on the slice.
 
 The 8da4w configuration gets the same treatment: fake quantisation and ``convert()`` at the full weight and activation
@@ -165,7 +165,7 @@ def test_two_layer_70b_width_stack_with_activation_checkpointing():
     assert l_ac == l_plain
     for n in g_ac:
         want = g_plain[n].float()
-        torch.testing.assert_close(g_ac[n].float(), want, rtol=2e-2, atol=2e-2 * float(want.abs().max()), msg=n)
+        torch.testing.assert_close(g_ac[n].float(), want, rtol=4e-3, atol=4e-3 * float(want.abs().max()), msg=n)
 
 
 # ---------------------------------------------------------------------------------------------------------------------
@@ -245,7 +245,7 @@ def test_qat_linear_at_full_size_against_the_oracle_on_slices():
     ref_gx = gy.float() @ wq.float()
     torch.testing.assert_close(x.grad.float(), ref_gx, rtol=1e-2, atol=1e-2 * max(1.0, float(ref_gx.abs().max()) / 8))
     ref_gw = gy.float().T @ xq.float()
-    torch.testing.assert_close(model[0].weight.grad.float(), ref_gw, rtol=2e-2, atol=2e-2 * float(ref_gw.abs().max()))
+    torch.testing.assert_close(model[0].weight.grad.float(), ref_gw, rtol=4e-3, atol=4e-3 * float(ref_gw.abs().max()))
     del ref_gx, ref_gw
     model = qz.convert(model)
     assert isinstance(model[0], Int8DynActInt4WeightLinear)
