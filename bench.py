@@ -676,6 +676,11 @@ def main() -> int:
                     help="calls of at most this many tokens hand their expanded weight to the backward of the same layer, whose "
                          "grad-input GEMM reads it instead of expanding the weight again (0: never; default: the library's rule, "
                          "torchtune_amd.ops.KEEP_FORWARD_TILES_MAX_TOKENS = 4096)")
+    ap.add_argument("--resident-tiles-gib", type=float, default=0.0, metavar="GIB",
+                    help="keep up to this many GiB of expanded NF4 weights across calls (2 B per weight element; the frozen base "
+                         "weight never changes, so later steps run their GEMMs on the kept tiles and launch no expansion; "
+                         "torchtune_amd.ops.RESIDENT_TILES_MAX_BYTES). Default 0: every call expands its weight, as the "
+                         "reference dequantises it in every call")
     ap.add_argument("--no-backward-copy", action="store_true",
                     help="keep no transposed copy of the NF4 codes (0.5625 B per weight element less): the expanded-weight path then "
                          "builds W^T from the weight's own codes, the fused path falls back to its first-generation grad-input kernel")
@@ -703,6 +708,7 @@ def main() -> int:
     ops.EXPANDED_WEIGHT_PATH = not args.no_expanded_weight
     if args.keep_forward_tiles is not None:
         ops.KEEP_FORWARD_TILES_MAX_TOKENS = args.keep_forward_tiles
+    ops.RESIDENT_TILES_MAX_BYTES = int(args.resident_tiles_gib * 2**30)
     if args.no_qat_tiled_gemm:
         from torchtune_amd import qat as qat_module
         qat_module.TILED_GEMM = False
@@ -927,6 +933,10 @@ def main() -> int:
     }
     result["with_adamw"] = with_adamw
     result["peak_memory_gib_timed_steps"] = round(peak_timed / 2**30, 3)
+    if ops.resident_tiles_enabled():
+        result["resident_tiles"] = {
+            "budget_gib": args.resident_tiles_gib, "held_gib": round(ops.resident_tiles_bytes() / 2**30, 3),
+            "note": "expanded NF4 weights kept across steps (opt-in): the timed steps launch no expansion for the layers held"}
     del model
     torch.cuda.empty_cache()
     if not args.no_memory_leg:

@@ -403,6 +403,12 @@ int ttamd_nf4_group_bwd_dx_ws_bf16(const ttamd_lora_group_member* members, int n
 int ttamd_nf4_group_fwd_leaves_tiles(const ttamd_lora_group_member* members, int n_members, int64_t M, int64_t K, int swiglu);
 int ttamd_nf4_group_bwd_dx_tiles_bf16(const ttamd_lora_group_member* members, int n_members, const void* gh_cat, void* gx, int64_t M,
                                       int64_t K, const void* tiles_fwd, int paired, void* stream);
+/* The group's forward on tiles that an earlier forward call of the same members left behind (a caller that keeps them
+ * across calls: the base weight of a QLoRA run never changes): ttamd_nf4_lora_group_fwd_bf16 (act NULL, paired 0) or
+ * ttamd_nf4_lora_group_swiglu_fwd_bf16 (act non-NULL, paired 1) without the expansion launches, same bits.  Shapes for
+ * which ttamd_nf4_group_fwd_leaves_tiles gives 0 return TTAMD_EUNSUPPORTED. */
+int ttamd_nf4_lora_group_fwd_tiles_bf16(const void* x, const ttamd_lora_group_member* members, int n_members, const void* h_cat,
+                                        void* act, int64_t M, int64_t K, const void* tiles_fwd, int paired, void* stream);
 
 
 /* ------------------------------------------------------------------------------------------------

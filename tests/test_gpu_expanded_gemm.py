@@ -386,3 +386,85 @@ def test_one_expansion_serves_both_directions(kind, monkeypatch):
     ck, _ = _grads(lambda t: checkpoint(fn, t, use_reentrant=False), x, layers)
     for a, b in zip(ck, got):
         assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+
+
+@pytest.mark.parametrize("kind", ["single", "qkv_group", "gated_pair"])
+def test_expanded_weights_kept_across_calls(kind, monkeypatch):
+    """With a budget in ``ops.RESIDENT_TILES_MAX_BYTES`` the first many-token forward of a layer (or group) leaves its
+    expanded weights with the weight; later calls run forward and grad-input on them and launch no expansion.  Outputs and
+    gradients: the bits of the calls that expand per call with the forward's tiles handed to the backward
+    (``KEEP_FORWARD_TILES_MAX_TOKENS``); a write into the weight drops the tiles; no budget, nothing kept."""
+    from torchtune_amd.modules.peft import group as group_mod
+
+    M, K = 2048, 8192
+    g = torch.Generator(device=DEV).manual_seed(6)
+    x = torch.randn(M, K, device=DEV, generator=g).to(BF)
+    if kind == "single":
+        layers = _lora_layers([8192], K, 16, seed=11)
+        fn = lambda t: layers[0](t)
+        tiles_bytes = 2 * 8192 * K
+    elif kind == "qkv_group":
+        layers = _lora_layers([4096, 2048, 2048], K, 16, seed=12)
+        fn = lambda t: group_mod.lora_linear_group(t, layers)
+        tiles_bytes = 2 * 8192 * K
+    else:
+        layers = _lora_layers([4096, 4096], K, 16, seed=13)
+        fn = lambda t: group_mod.lora_swiglu_group(t, layers[0], layers[1])
+        tiles_bytes = 2 * 8192 * K
+    monkeypatch.setattr(ops, "KEEP_FORWARD_TILES_MAX_TOKENS", M)
+    monkeypatch.setattr(ops, "RESIDENT_TILES_MAX_BYTES", 0)
+    want, out0 = _grads(fn, x, layers)
+    assert ops.resident_tiles_bytes() == 0
+    # a budget too small for this layer: nothing is kept, nothing changes
+    monkeypatch.setattr(ops, "RESIDENT_TILES_MAX_BYTES", tiles_bytes // 2)
+    small, out_small = _grads(fn, x, layers)
+    assert ops.resident_tiles_bytes() == 0
+    for a, b in zip(small + out_small, want + out0):
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+    monkeypatch.setattr(ops, "RESIDENT_TILES_MAX_BYTES", 1 << 32)
+    first, out1 = _grads(fn, x, layers)    # expands, leaves the tiles
+    held = ops.resident_tiles_bytes()
+    assert tiles_bytes <= held <= tiles_bytes + (8 << 20)
+    expansions = {"n": 0}
+    lib = _lib.load()
+    for name in ("ttamd_qlora_linear_fwd_bf16", "ttamd_nf4_lora_linear_fwd_ws_bf16", "ttamd_nf4_lora_group_fwd_bf16",
+                 "ttamd_nf4_lora_group_swiglu_fwd_bf16", "ttamd_nf4_group_bwd_dx_ws_bf16", "ttamd_nf4_linear_bwd_dx_ws_bf16"):
+        real = getattr(lib, name)
+
+        def counted(*a, _real=real):
+            expansions["n"] += 1
+            return _real(*a)
+
+        monkeypatch.setattr(lib, name, counted)
+    second, out2 = _grads(fn, x, layers)   # runs on them: none of the entry points that expand is called
+    assert expansions["n"] == 0
+    assert ops.resident_tiles_bytes() == held
+    for a, b, c in zip(first + out1, second + out2, want + out0):
+        assert torch.equal(a.view(torch.int16), c.view(torch.int16))
+        assert torch.equal(b.view(torch.int16), c.view(torch.int16))
+    # with activation checkpointing both passes of the forward run on the kept tiles
+    from torch.utils.checkpoint import checkpoint
+
+    ck, _ = _grads(lambda t: checkpoint(fn, t, use_reentrant=False), x, layers)
+    assert expansions["n"] == 0
+    for a, b in zip(ck, want):
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+    # a write into a weight drops the tiles: the next call follows the new weight and leaves new tiles
+    from torchtune_amd import to_nf4
+
+    last = layers[-1]
+    new_w = to_nf4((torch.randn(last.weight.shape, device=DEV, generator=g) * 0.02).to(BF))
+    with torch.no_grad():
+        last.weight.copy_(new_w)
+    third, out3 = _grads(fn, x, layers)
+    assert expansions["n"] >= 1
+    monkeypatch.setattr(ops, "RESIDENT_TILES_MAX_BYTES", 0)
+    fresh, out_fresh = _grads(fn, x, layers)
+    for a, b in zip(third + out3, fresh + out_fresh):
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+    assert not torch.equal(out3[-1], out2[-1])
+    del layers, fn, last, new_w
+    import gc
+
+    gc.collect()
+    assert ops.resident_tiles_bytes() == 0

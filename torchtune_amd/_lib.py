@@ -117,6 +117,7 @@ SIGNATURES = {
     "ttamd_nf4_group_bwd_dx_ws_bf16": (_int, [_c_void_p, _int, _c_void_p, _c_void_p, _i64, _i64, _c_void_p, _size, _c_void_p]),
     "ttamd_nf4_group_fwd_leaves_tiles": (_int, [_c_void_p, _int, _i64, _i64, _int]),
     "ttamd_nf4_group_bwd_dx_tiles_bf16": (_int, [_c_void_p, _int, _c_void_p, _c_void_p, _i64, _i64, _c_void_p, _int, _c_void_p]),
+    "ttamd_nf4_lora_group_fwd_tiles_bf16": (_int, [_c_void_p, _c_void_p, _int, _c_void_p, _c_void_p, _i64, _i64, _c_void_p, _int, _c_void_p]),
     "ttamd_tiled_weight_bytes": (_size, [_i64, _i64]),
     "ttamd_gemm_tn_applies": (_int, [_i64, _i64, _i64]),
     "ttamd_gemm_tn_bf16": (_int, [_c_void_p, _c_void_p, _c_void_p, _i64, _i64, _i64, _c_void_p]),

@@ -74,7 +74,8 @@ int run_gemm_dense(const void* X, const uint8_t* codes, const void* scal, int mo
 size_t dense_group_fwd_workspace_bytes(const GroupGemm& d);
 // act != nullptr: two members of equal width (gate, up); the launch also writes act = silu(y[0]) * y[1]
 bool dense_group_gated_applies(const GroupGemm& d);
-int run_gemm_dense_group_fwd(const void* x, const GroupGemm& d, const void* h_cat, void* workspace, hipStream_t s, void* act = nullptr);
+int run_gemm_dense_group_fwd(const void* x, const GroupGemm& d, const void* h_cat, void* workspace, hipStream_t s, void* act = nullptr,
+                             const void* tiles = nullptr);
 size_t dense_group_dx_workspace_bytes(const GroupDx& d);
 int run_gemm_dense_group_dx(const GroupDx& d, const void* gh_cat, void* gx, void* workspace, hipStream_t s,
                             const void* tiles_fwd = nullptr, bool paired = false);

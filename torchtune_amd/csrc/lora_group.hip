@@ -238,3 +238,20 @@ extern "C" int ttamd_nf4_group_bwd_dx_tiles_bf16(const ttamd_lora_group_member* 
     return fail(TTAMD_EUNSUPPORTED, "nf4_group_bwd_dx_tiles: shape not served by the many-token launch (M=%lld K=%lld)", (long long)M, (long long)K);
   return run_gemm_dense_group_dx(d.dx, gh_cat, gx, nullptr, reinterpret_cast<hipStream_t>(stream), tiles_fwd, paired != 0);
 }
+
+// The group's forward on tiles an earlier forward call of the same members left behind (layout 1 or 2 of
+// ttamd_nf4_group_fwd_leaves_tiles): the many-token launch without its expansion launches.
+extern "C" int ttamd_nf4_lora_group_fwd_tiles_bf16(const void* x, const ttamd_lora_group_member* members, int n_members,
+                                                   const void* h_cat, void* act, int64_t M, int64_t K, const void* tiles_fwd,
+                                                   int paired, void* stream) {
+  Decoded d;
+  if (int rc = decode("nf4_lora_group_fwd_tiles", members, n_members, M, K, false, d)) return rc;
+  TT_REQUIRE(x && h_cat && tiles_fwd && aligned16(x) && aligned16(h_cat) && aligned16(tiles_fwd),
+             "nf4_lora_group_fwd_tiles: x, h_cat and tiles_fwd must be non-null and 16-byte aligned");
+  TT_REQUIRE((paired != 0) == (act != nullptr), "nf4_lora_group_fwd_tiles: paired tiles are those of the call that writes act, and only those");
+  TT_REQUIRE(!act || aligned16(act), "nf4_lora_group_fwd_tiles: act must be 16-byte aligned");
+  if (group_small_m(d, true) || dense_group_fwd_workspace_bytes(d.gm) == 0 || (paired && !dense_group_gated_applies(d.gm)))
+    return fail(TTAMD_EUNSUPPORTED, "nf4_lora_group_fwd_tiles: shape not served by the many-token launch (M=%lld K=%lld)", (long long)M,
+                (long long)K);
+  return run_gemm_dense_group_fwd(x, d.gm, h_cat, nullptr, reinterpret_cast<hipStream_t>(stream), act, tiles_fwd);
+}

@@ -948,9 +948,12 @@ bool dense_group_gated_applies(const GroupGemm& d) {
 }
 
 // act != nullptr: the pair (gate, up) with act = silu(y_0) * y_1 written by the same launch (dense_group_gated_applies)
-int run_gemm_dense_group_fwd(const void* x, const GroupGemm& d, const void* h_cat, void* workspace, hipStream_t s, void* act) {
+// tiles != nullptr: the members' weights as an earlier call of this function left them in its workspace (the same
+// members, the same act-or-not): no expansion launch, workspace is not touched
+int run_gemm_dense_group_fwd(const void* x, const GroupGemm& d, const void* h_cat, void* workspace, hipStream_t s, void* act,
+                             const void* tiles) {
   TT_REQUIRE(d.n >= 2 && d.n <= kGroupMax && dense_group_fwd_workspace_bytes(d) > 0, "nf4_lora_group_fwd (expanded): shape not served");
-  TT_REQUIRE(aligned16(workspace) && aligned16(x), "nf4_lora_group_fwd (expanded): pointers must be 16-byte aligned");
+  TT_REQUIRE(aligned16(tiles ? tiles : workspace) && aligned16(x), "nf4_lora_group_fwd (expanded): pointers must be 16-byte aligned");
   const bool gated = act != nullptr;
   TT_REQUIRE(!gated || (dense_group_gated_applies(d) && aligned16(act)), "nf4_lora_group_swiglu_fwd (expanded): shape not served");
   DenseArgs g = {};
@@ -969,7 +972,7 @@ int run_gemm_dense_group_fwd(const void* x, const GroupGemm& d, const void* h_ca
     // gated: the members' column blocks alternate 8 by 8, the second member starting 8 blocks (128 columns) in
     char* dst = reinterpret_cast<char*>(workspace) + (gated ? (int64_t)i * 128 : n_off) * d.K * 2;
     eg.m[i] = ExpandMember{d.codes[i], tr ? d.bscal_t[i] : d.bscal[i], dst, (int)d.N[i], (int)d.K, 0};
-    if (!one_launch)
+    if (!one_launch && !tiles)
       if (int rc = launch_expand(tr ? 2 : 0, eg.m[i].codes, eg.m[i].scal, d.N[i], d.K, d.K >> 5, 0, dst, s, gated)) return rc;
     g.ad[i].lX = reinterpret_cast<const uint16_t*>(h_cat) + d.r_off[i];
     g.ad[i].lW = d.lora_b[i];
@@ -984,11 +987,11 @@ int run_gemm_dense_group_fwd(const void* x, const GroupGemm& d, const void* h_ca
     g.out[i].width = (int)d.N[i];
     n_off += d.N[i];
   }
-  if (one_launch) {
+  if (one_launch && !tiles) {
     eg.n = d.n;
     if (int rc = launch_expand_group(d.bscal_t[0] ? 2 : 0, eg, d.K >> 5, s, gated)) return rc;
   }
-  g.Wt = reinterpret_cast<const char*>(workspace);
+  g.Wt = reinterpret_cast<const char*>(tiles ? tiles : workspace);
   g.M = (int)d.M; g.Nout = (int)n_off; g.Kc = (int)d.K;
   g.lw_row_major = 1;
   g.ldlx = d.r_off[d.n];

@@ -41,8 +41,7 @@ class _QLoRAGroupFn(torch.autograd.Function):
         x2 = x.reshape(-1, K)
         members = [ops.GroupMember(w.quantized_data, w.block_scalers(), tr, a, b, bias, s, w.shape[0])
                    for w, tr, a, b, bias, s in zip(weights, _copies(weights, x2.shape[0]), las, lbs, biases, scales)]
-        h_cat, ys, tiles, paired = ops.lora_group_fwd(x2, members, return_tiles=True)
-        _keep_tiles(ctx, tiles, paired, x2.shape[0], weights)
+        h_cat, ys = _group_forward(ctx, x2, members, weights, False)
         ctx.save_for_backward(x2, h_cat, *weights, *las, *lbs)
         ctx.scales = scales
         ctx.x_shape = x.shape
@@ -65,11 +64,29 @@ class _QLoRAGroupFn(torch.autograd.Function):
         return _group_backward(ctx, x2, h_cat, weights, las, lbs, gy2)
 
 
-def _keep_tiles(ctx, tiles, paired: bool, tokens: int, weights) -> None:
+def _group_forward(ctx, x2, members, weights, swiglu: bool):
+    """``ops.lora_group_fwd`` on the expanded weights an earlier call left with the group where such tiles are kept across
+    calls (``ops.RESIDENT_TILES_MAX_BYTES``), leaving this call's there when there are none yet; decides which tiles the
+    node hands to its backward.  -> (h_cat, outputs)"""
+    tokens = x2.shape[0]
+    found = nf4_tensor.resident_group_tiles(weights, swiglu) if ops.resident_tiles_enabled() else None
+    if found is not None:
+        h_cat, outs, tiles, paired = ops.lora_group_fwd(x2, members, swiglu=swiglu, return_tiles=True, tiles=found[0], paired=found[1])
+        resident = tiles is found[0]
+    else:
+        h_cat, outs, tiles, paired = ops.lora_group_fwd(x2, members, swiglu=swiglu, return_tiles=True)
+        resident = (tiles is not None and ops.resident_tiles_enabled()
+                    and nf4_tensor.keep_resident_group_tiles(weights, swiglu, tiles, paired))
+    _keep_tiles(ctx, tiles, paired, tokens, weights, resident)
+    return h_cat, outs
+
+
+def _keep_tiles(ctx, tiles, paired: bool, tokens: int, weights, resident: bool = False) -> None:
     """The group forward's expanded weights stay with the node when the backward will want a grad-input, the call is
-    short enough for one expansion per layer to pay (``ops.KEEP_FORWARD_TILES_MAX_TOKENS``) and the grouped grad-input is
-    the many-token launch (with few output tiles it stays on the fused kernel)."""
-    keep = (tiles is not None and ctx.needs_input_grad[0] and ops.keeps_forward_tiles(tokens)
+    short enough for one expansion per layer to pay (``ops.KEEP_FORWARD_TILES_MAX_TOKENS``; any length when the tiles are
+    kept across calls anyway) and the grouped grad-input is the many-token launch (with few output tiles it stays on the
+    fused kernel)."""
+    keep = (tiles is not None and ctx.needs_input_grad[0] and (resident or ops.keeps_forward_tiles(tokens))
             and ops.group_dx_expands(tokens, weights[0].shape[1], [w.shape[0] for w in weights]))
     ctx.tiles, ctx.tiles_paired = (tiles, paired) if keep else (None, False)
 
@@ -106,8 +123,7 @@ class _QLoRAGatedFn(torch.autograd.Function):
         x2 = x.reshape(-1, K)
         members = [ops.GroupMember(w.quantized_data, w.block_scalers(), tr, a, b, bias, s, w.shape[0])
                    for w, tr, a, b, bias, s in zip(weights, _copies(weights, x2.shape[0]), las, lbs, biases, scales)]
-        h_cat, (gate, up, act), tiles, paired = ops.lora_group_fwd(x2, members, swiglu=True, return_tiles=True)
-        _keep_tiles(ctx, tiles, paired, x2.shape[0], weights)
+        h_cat, (gate, up, act) = _group_forward(ctx, x2, members, weights, True)
         ctx.save_for_backward(x2, h_cat, gate, up, *weights, *las, *lbs)
         ctx.scales = scales
         ctx.x_shape = x.shape
@@ -140,8 +156,7 @@ class _QLoRAFeedForwardFn(torch.autograd.Function):
         x2 = x.reshape(-1, K)
         members = [ops.GroupMember(w.quantized_data, w.block_scalers(), tr, a, b, bias, s, w.shape[0])
                    for w, tr, a, b, bias, s in zip(weights[:2], _copies(weights[:2], x2.shape[0]), las, lbs, biases, scales)]
-        h_cat, (gate, up, act), tiles, paired = ops.lora_group_fwd(x2, members, swiglu=True, return_tiles=True)
-        _keep_tiles(ctx, tiles, paired, x2.shape[0], weights[:2])
+        h_cat, (gate, up, act) = _group_forward(ctx, x2, members, weights[:2], True)
         w2 = weights[2]
         h2 = ops.lora_hidden(act, las[2])
         tr = w2.backward_copy_for(act.shape[0], True)

@@ -56,13 +56,24 @@ class _QLoRALinearFn(torch.autograd.Function):
         # GEMM then reads these tiles instead of expanding the weight again (ops.KEEP_FORWARD_TILES_MAX_TOKENS)
         # (only where that GEMM is the many-token launch: a grad-input of few output tiles stays on the fused kernel)
         keep = ctx.needs_input_grad[0] and ops.keeps_forward_tiles(x2.shape[0]) and ops.gemm_expands_weight(x2.shape[0], K, N)
-        if ONE_CALL_PER_DIRECTION and not ops.gemm_timer_installed():
+        # expanded weights kept across calls (ops.RESIDENT_TILES_MAX_BYTES): a many-token forward runs on the tiles an
+        # earlier one left with the weight, and leaves its own there when there are none yet
+        resident = ops.resident_tiles_enabled() and ops.gemm_expands_weight(x2.shape[0], N, K)
+        tiles = weight.resident_tiles() if resident else None
+        if tiles is not None:
+            h = ops.lora_hidden(x2, lora_a)
+            y = ops.tiled_lora_linear(x2, tiles, N, h, lora_b, scale, True, bias, nf4_forward=True)
+        elif ONE_CALL_PER_DIRECTION and not ops.gemm_timer_installed():
             y, h, tiles = ops.qlora_linear_fwd(x2, weight.quantized_data, weight.block_scalers(), N, lora_a, lora_b, scale, bias,
                                                block_scalers_t=tr[1] if tr else None, return_tiles=True)
+            resident = resident and tiles is not None and weight.keep_resident_tiles(tiles)
         else:
             h = ops.lora_hidden(x2, lora_a)
             y, tiles = ops.nf4_lora_linear_fwd(x2, weight.quantized_data, weight.block_scalers(), N, h, lora_b, scale, bias,
                                                block_scalers_t=tr[1] if tr else None, return_tiles=True)
+            resident = resident and tiles is not None and weight.keep_resident_tiles(tiles)
+        if resident:  # the tiles exist anyway: the grad-input reads them wherever it is a many-token launch
+            keep = ctx.needs_input_grad[0] and ops.gemm_expands_weight(x2.shape[0], K, N)
         ctx.tiles = tiles if keep else None
         ctx.save_for_backward(x2, h, weight, lora_a, lora_b)
         ctx.scale = scale

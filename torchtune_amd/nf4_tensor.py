@@ -270,6 +270,19 @@ class NF4Tensor(torch.Tensor):
         qs._ttamd_backward_copy = (key, val)
         return val
 
+    def resident_tiles(self):
+        """The expanded weight a many-token forward left behind and ``keep_resident_tiles`` stored, while the weight is
+        unchanged (``ops.RESIDENT_TILES_MAX_BYTES``); else None."""
+        cached = getattr(self.quantized_scalers, "_ttamd_tiles", None)
+        return cached[1] if cached is not None and cached[0] == _tiles_key(self) else None
+
+    def keep_resident_tiles(self, tiles: torch.Tensor) -> bool:
+        """Stores a forward call's tiles with the weight if the budget admits them; True when stored."""
+        if not ops.resident_tiles_admit(tiles):
+            return False
+        self.quantized_scalers._ttamd_tiles = (_tiles_key(self), tiles)
+        return True
+
     def backward_copy_for(self, tokens: int, forward: bool):
         """The transposed copy a GEMM call over ``tokens`` rows would use: None when the library serves that call from the
         weight expanded once per call (many tokens; it then reads the weight's own codes, so a purely many-token
@@ -332,6 +345,29 @@ class NF4Tensor(torch.Tensor):
             return func(*args, **kwargs)
 
 
+def _tiles_key(w: "NF4Tensor"):
+    qs = w.quantized_scalers
+    return (qs._version, w.quantization_factor._version, w.scaler_mean._version, w.quantized_data._version, qs.data_ptr(),
+            w.quantized_data.data_ptr(), _generation(qs))
+
+
+def resident_group_tiles(weights, swiglu: bool):
+    """``(tiles, paired)`` that ``keep_resident_group_tiles`` stored for exactly these weights (unchanged since) and this
+    kind of group call, or None."""
+    cached = getattr(weights[0].quantized_scalers, "_ttamd_group_tiles", None)
+    if cached is not None and cached[0] == (bool(swiglu),) + tuple(_tiles_key(w) for w in weights):
+        return cached[1], cached[2]
+    return None
+
+
+def keep_resident_group_tiles(weights, swiglu: bool, tiles: torch.Tensor, paired: bool) -> bool:
+    """Stores a group forward's tiles with the group's first weight if the budget admits them; True when stored."""
+    if not ops.resident_tiles_admit(tiles):
+        return False
+    weights[0].quantized_scalers._ttamd_group_tiles = ((bool(swiglu),) + tuple(_tiles_key(w) for w in weights), tiles, paired)
+    return True
+
+
 # ---- aten-level behaviour -----------------------------------------------------------------------------
 def _carry_cache(src: NF4Tensor, dst: NF4Tensor) -> None:
     cached = getattr(src.quantized_scalers, "_ttamd_block_scalers", None)
@@ -367,6 +403,8 @@ def _nf4_copy_(func, args, kwargs):
     # this tensor object are dropped and the storage's write generation is bumped for those of its aliases
     dst.quantized_scalers._ttamd_block_scalers = None
     dst.quantized_scalers._ttamd_backward_copy = None
+    dst.quantized_scalers._ttamd_tiles = None
+    dst.quantized_scalers._ttamd_group_tiles = None
     _bump_generation(dst.quantized_scalers)
     if isinstance(src, NF4Tensor):
         same_meta = (

@@ -6,6 +6,7 @@ Every function requires HIP (``cuda``) tensors.  There is no CPU implementation 
 from __future__ import annotations
 
 import ctypes
+import weakref
 from typing import List, Optional, Sequence, Tuple
 
 import torch
@@ -250,6 +251,43 @@ KEEP_FORWARD_TILES_MAX_TOKENS = 4096
 
 def keeps_forward_tiles(M: int) -> bool:
     return bool(EXPANDED_WEIGHT_PATH and 0 < M <= KEEP_FORWARD_TILES_MAX_TOKENS)
+
+
+# Expanded weights kept ACROSS calls.  The base weight of a QLoRA run never changes, so the tiles a many-token forward
+# expands it into can stay: every later forward and grad-input of the layer (or group of layers) then runs its GEMM on
+# them and no expansion launch is left in the step.  The price is 2 bytes per weight element of device memory for as long
+# as the weight lives (14 GB for an 8B model, 137 GB for a 70B one), which is why it is off unless a budget is given:
+# tiles are admitted first come, first served while their sum stays within RESIDENT_TILES_MAX_BYTES, layers beyond
+# the budget keep expanding per call.  The cache entries ride on the weight and are keyed like its block scalers (a write
+# into the weight drops them).  Results are the same bits either way: the same tiles feed the same GEMM launch.
+RESIDENT_TILES_MAX_BYTES = 0
+_resident_tiles_bytes = 0
+
+
+def resident_tiles_enabled() -> bool:
+    return bool(EXPANDED_WEIGHT_PATH and RESIDENT_TILES_MAX_BYTES > 0)
+
+
+def resident_tiles_bytes() -> int:
+    """Bytes of expanded weights currently held across calls."""
+    return _resident_tiles_bytes
+
+
+def _resident_release(nbytes: int) -> None:
+    global _resident_tiles_bytes
+    _resident_tiles_bytes -= nbytes
+
+
+def resident_tiles_admit(tiles: torch.Tensor) -> bool:
+    """Counts ``tiles`` (a forward call's scratch memory whose head holds expanded weights) against the budget; True when
+    the caller may keep it.  The bytes are given back when the tensor is freed."""
+    global _resident_tiles_bytes
+    nbytes = tiles.numel() * tiles.element_size()
+    if not resident_tiles_enabled() or _resident_tiles_bytes + nbytes > RESIDENT_TILES_MAX_BYTES:
+        return False
+    _resident_tiles_bytes += nbytes
+    weakref.finalize(tiles, _resident_release, nbytes)
+    return True
 
 
 def gemm_expands_weight(M: int, n_out: int, k_contract: int) -> bool:
@@ -547,7 +585,8 @@ def _group_array(what: str, members: Sequence[GroupMember], K: int, ys: Sequence
     return arr, keep
 
 
-def lora_group_fwd(x: torch.Tensor, members: Sequence[GroupMember], swiglu: bool = False, return_tiles: bool = False):
+def lora_group_fwd(x: torch.Tensor, members: Sequence[GroupMember], swiglu: bool = False, return_tiles: bool = False,
+                   tiles: Optional[torch.Tensor] = None, paired: bool = False):
     """-> (h_cat [M, sum of ranks], [y_i [M, N_i]]): every member's ``y_i = x @ D(W_i).T (+ bias_i) + scale_i * h_i @ B_i.T``
     with ``h_i = x @ A_i.T`` (columns of ``h_cat``), in one pass over ``x`` for the hidden products.
 
@@ -556,7 +595,11 @@ def lora_group_fwd(x: torch.Tensor, members: Sequence[GroupMember], swiglu: bool
 
     ``return_tiles=True`` appends ``(tiles, paired)`` to the result: the call's scratch memory when its head holds the
     members' weights expanded in forward tile order (``paired``: in the gated pair's layout), else ``(None, False)`` -
-    what ``lora_group_bwd(..., tiles=..., paired=...)`` takes."""
+    what ``lora_group_bwd(..., tiles=..., paired=...)`` takes.
+
+    ``tiles`` / ``paired``: such a pair from an earlier call with the same members (weights unchanged since) and the same
+    ``swiglu``; where this call would expand the weights into the same layout it runs its GEMM on them instead
+    (``ttamd_nf4_lora_group_fwd_tiles_bf16``), otherwise they are ignored."""
     x = _bf16_2d(x, "lora_group_fwd")
     M, K = x.shape
     dev = x.device
@@ -571,7 +614,11 @@ def lora_group_fwd(x: torch.Tensor, members: Sequence[GroupMember], swiglu: bool
     fwd_bytes = lib.ttamd_lora_group_fwd_workspace_bytes(arr, n, M, K)
     if not EXPANDED_WEIGHT_PATH and any(lib.ttamd_nf4_gemm_expands_weight(M, m.N, K) for m in members):
         fwd_bytes = 0  # less than the library asks for: it keeps the fused kernel
-    ws = _workspace(max(lib.ttamd_lora_group_hidden_workspace_bytes(arr, n, M, K), fwd_bytes), dev)
+    on_tiles = (tiles is not None and fwd_bytes > 0
+                and int(lib.ttamd_nf4_group_fwd_leaves_tiles(arr, n, M, K, 1 if swiglu else 0)) == (2 if paired else 1))
+    if on_tiles and (tiles.numel() * tiles.element_size() < 2 * K * sum(m.N for m in members) or not tiles.is_contiguous()):
+        raise ValueError("lora_group_fwd: the given tiles do not hold the members' weights")
+    ws = _workspace(max(lib.ttamd_lora_group_hidden_workspace_bytes(arr, n, M, K), 0 if on_tiles else fwd_bytes), dev)
     with torch.cuda.device(dev):
         rc = lib.ttamd_lora_group_hidden_bf16(x.data_ptr(), arr, n, h_cat.data_ptr(), M, K, ws.data_ptr(), ws.numel(), _stream(x))
         _lib.check(rc, "lora_group_hidden")
@@ -579,8 +626,11 @@ def lora_group_fwd(x: torch.Tensor, members: Sequence[GroupMember], swiglu: bool
                   if _gemm_timer is not None else None)
         if events:
             events[0].record()
-        if swiglu:
-            act = torch.empty(M, members[0].N, dtype=torch.bfloat16, device=dev)
+        act = torch.empty(M, members[0].N, dtype=torch.bfloat16, device=dev) if swiglu else None
+        if on_tiles:
+            rc = lib.ttamd_nf4_lora_group_fwd_tiles_bf16(x.data_ptr(), arr, n, h_cat.data_ptr(), _ptr(act), M, K, tiles.data_ptr(),
+                                                         1 if paired else 0, _stream(x))
+        elif swiglu:
             rc = lib.ttamd_nf4_lora_group_swiglu_fwd_bf16(x.data_ptr(), arr, n, h_cat.data_ptr(), act.data_ptr(), M, K, ws.data_ptr(),
                                                           ws.numel(), _stream(x))
         else:
@@ -590,8 +640,10 @@ def lora_group_fwd(x: torch.Tensor, members: Sequence[GroupMember], swiglu: bool
     _lib.check(rc, "lora_group_fwd")
     outs = ys + [act] if swiglu else ys
     if return_tiles:
-        layout = int(lib.ttamd_nf4_group_fwd_leaves_tiles(arr, n, M, K, 1 if swiglu else 0)) if fwd_bytes else 0
         del keep
+        if on_tiles:
+            return h_cat, outs, tiles, paired
+        layout = int(lib.ttamd_nf4_group_fwd_leaves_tiles(arr, n, M, K, 1 if swiglu else 0)) if fwd_bytes else 0
         return h_cat, outs, (ws if layout else None), layout == 2
     del keep
     return h_cat, outs
@@ -894,17 +946,18 @@ def tiled_linear(x: torch.Tensor, tiled: torch.Tensor, n_out: int, bias: Optiona
 
 
 def tiled_lora_linear(x: torch.Tensor, tiled: torch.Tensor, n_out: int, lx: torch.Tensor, lw: torch.Tensor, lscale: float,
-                      lw_row_major: bool, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+                      lw_row_major: bool, bias: Optional[torch.Tensor] = None, nf4_forward: bool = False) -> torch.Tensor:
     """``tiled_linear`` with a low-rank adapter in the GEMM's epilogue: ``y = x @ Wd.T (+ bias) + lscale * lx @ lw.T``
     with ``lw`` [n_out, r] (``lw_row_major``, the forward: ``lora_b``) or ``lw.T`` given as [r, n_out] (the grad-input:
-    ``lora_a``)."""
+    ``lora_a``).  ``tiled`` may be longer than n_out * K elements (a workspace whose head holds the tiles);
+    ``nf4_forward``: the tiles are an NF4 weight's expansion kept from an earlier call (what a GEMM timer is told)."""
     x = _bf16_2d(x, "tiled_lora_linear")
     lx = _bf16_2d(lx, "tiled_lora_linear")
     lw = _bf16_2d(lw, "tiled_lora_linear")
     M, K = x.shape
     r = lx.shape[1]
-    if tiled.dtype != torch.bfloat16 or tiled.numel() != n_out * K or not tiled.is_contiguous():
-        raise ValueError(f"tiled_lora_linear: the tiled weight must be a contiguous bfloat16 tensor of {n_out} x {K} elements")
+    if tiled.numel() * tiled.element_size() < 2 * n_out * K or not tiled.is_contiguous():
+        raise ValueError(f"tiled_lora_linear: the tiled weight must be contiguous and hold {n_out} x {K} bfloat16 elements")
     if lx.shape[0] != M or tuple(lw.shape) != ((n_out, r) if lw_row_major else (r, n_out)) or r % 8 != 0 or not 0 < r <= 64:
         raise ValueError(f"tiled_lora_linear: adapter operands {tuple(lx.shape)} / {tuple(lw.shape)} do not fit M={M}, n_out={n_out} "
                          "(rank: a multiple of 8, at most 64)")
@@ -915,7 +968,9 @@ def tiled_lora_linear(x: torch.Tensor, tiled: torch.Tensor, n_out: int, lx: torc
     y = torch.empty(M, n_out, dtype=torch.bfloat16, device=x.device)
     lib = _lib.load()
     with torch.cuda.device(x.device):
-        events = _gemm_timer("tiled", M, n_out, K, 0) if _gemm_timer is not None else None
+        events = None
+        if _gemm_timer is not None:
+            events = _gemm_timer("fwd", M, n_out, K, r) if nf4_forward else _gemm_timer("tiled", M, n_out, K, 0)
         if events:
             events[0].record()
         rc = lib.ttamd_tiled_lora_linear_bf16(x.data_ptr(), tiled.data_ptr(), lx.data_ptr(), lw.data_ptr(), 1 if lw_row_major else 0, r,
