@@ -598,6 +598,20 @@ __device__ __forceinline__ void gemm_dense_tile(const DenseArgs g) {
     const float lscale = g.ad[aidx].lscale;
     // first column of the tile among the adapter's columns (GATED: such that + 64 wn lands on the wave's own columns)
     const int nl0 = GATED ? 128 * tile_n - 128 * (wn >> 1) : n0 - nb;
+    // Every request of a 32-rank step is issued before the first use of any of them: one trip to memory per step instead
+    // of one per operand (with the scaling between two loads the compiler waited for each load in turn, ~5 us a tile).
+    u32x4_t xraw[MT], wraw[NT];
+    auto load_x = [&](int rc) {
+      const int r0 = rc + 8 * g4;
+#pragma unroll
+      for (int i = 0; i < MT; ++i) {
+        int row = m0 + 128 * wm + 16 * i + l15;
+        row = row < g.M ? row : g.M - 1;
+        xraw[i] = u32x4_t{0, 0, 0, 0};
+        if (r0 < R) xraw[i] = *reinterpret_cast<const u32x4_t*>(lX + (int64_t)row * g.ldlx + r0);  // R % 8 == 0: 8 ranks all in or all out
+      }
+    };
+    load_x(0);
     int pitch = 0;  // bytes per column of the staged adapter weights
     if constexpr (!LW_ROW_MAJOR) {
       // lW is [R, Nout]: a lane needs 8 ranks of one column, 8 elements Nout apart.  The workgroup copies the 256
@@ -617,36 +631,36 @@ __device__ __forceinline__ void gemm_dense_tile(const DenseArgs g) {
     }
     for (int rc = 0; rc < R; rc += 32) {
       const int r0 = rc + 8 * g4;
-      const bool in = r0 < R;  // R % 8 == 0: a lane's 8 ranks are all in or all out
-      bf16x8_t wfr[NT], xfr[MT];
+      const bool in = r0 < R;
+      if (rc > 0) load_x(rc);
 #pragma unroll
       for (int j = 0; j < NT; ++j) {
-        u32x4_t raw = {0, 0, 0, 0};
+        wraw[j] = u32x4_t{0, 0, 0, 0};
         if (in) {
           if constexpr (LW_ROW_MAJOR) {
             int col = nl0 + wn * 64 + 16 * j + l15;
             col = col < ncols ? col : ncols - 1;
-            raw = *reinterpret_cast<const u32x4_t*>(lW + (int64_t)col * R + r0);
+            wraw[j] = *reinterpret_cast<const u32x4_t*>(lW + (int64_t)col * R + r0);
           } else {
-            raw = *reinterpret_cast<const u32x4_t*>(smem + (wn * 64 + 16 * j + l15) * pitch + 2 * r0);
+            wraw[j] = *reinterpret_cast<const u32x4_t*>(smem + (wn * 64 + 16 * j + l15) * pitch + 2 * r0);
           }
         }
-        wfr[j] = __builtin_bit_cast(bf16x8_t, raw);
       }
       __builtin_amdgcn_sched_barrier(0);
+      bf16x8_t wfr[NT], xfr[MT];
+      // the adapter's scale goes onto the activation side, bf16(lscale * lX), as in the fused kernel; a power of two is
+      // exact on either operand, and the weight side has half as many registers to scale
+      const bool on_w = (f32_bits(lscale) & 0x007fffffu) == 0;
+      auto scaled = [&](u32x4_t raw) {
 #pragma unroll
-      for (int i = 0; i < MT; ++i) {
-        int row = m0 + 128 * wm + 16 * i + l15;
-        row = row < g.M ? row : g.M - 1;
-        u32x4_t raw = {0, 0, 0, 0};
-        if (in) raw = *reinterpret_cast<const u32x4_t*>(lX + (int64_t)row * g.ldlx + r0);
-        if (lscale != 1.0f) {
+        for (int d = 0; d < 4; ++d)
+          raw[d] = pack_bf16x2(bits_f32(raw[d] << 16) * lscale, bits_f32(raw[d] & 0xffff0000u) * lscale);
+        return raw;
+      };
 #pragma unroll
-          for (int d = 0; d < 4; ++d)
-            raw[d] = pack_bf16x2(bits_f32(raw[d] << 16) * lscale, bits_f32(raw[d] & 0xffff0000u) * lscale);
-        }
-        xfr[i] = __builtin_bit_cast(bf16x8_t, raw);
-      }
+      for (int j = 0; j < NT; ++j) wfr[j] = __builtin_bit_cast(bf16x8_t, lscale != 1.0f && on_w ? scaled(wraw[j]) : wraw[j]);
+#pragma unroll
+      for (int i = 0; i < MT; ++i) xfr[i] = __builtin_bit_cast(bf16x8_t, lscale != 1.0f && !on_w ? scaled(xraw[i]) : xraw[i]);
 #pragma unroll
       for (int j = 0; j < NT; ++j)
 #pragma unroll
@@ -688,6 +702,19 @@ __device__ __forceinline__ void gemm_dense_tile(const DenseArgs g) {
       }
     };
     if constexpr (EPI == kEpiSwigluBwd) sw_fetch(0);
+    if (!bias && !cscale) {
+      // nothing to add or scale: two conversions per four values instead of ten operations
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+          const int r = 16 * i + l15;
+          u32x2_t o;
+          o.x = pack_bf16x2(acc[j][i][0], acc[j][i][1]);
+          o.y = pack_bf16x2(acc[j][i][2], acc[j][i][3]);
+          *reinterpret_cast<u32x2_t*>(band + r * 128 + (((2 * j + (g4 >> 1)) ^ (r & 7)) << 4) + 8 * (g4 & 1)) = o;
+        }
+    } else
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
       float b4[4] = {0.f, 0.f, 0.f, 0.f};
