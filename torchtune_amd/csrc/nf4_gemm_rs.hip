@@ -457,6 +457,16 @@ __global__ __launch_bounds__(256) void nf4_gemm_rs_kernel(const RsArgs g, const 
       const int r0 = rc + 8 * h;
       const bool in = r0 < R;  // R % 8 == 0: a lane's 8 indices are all in or all out
       bf16x8_t wfr[NT], xfr[MT];
+      // every request of the step first, then their uses: one trip to memory per step (with the scaling between two
+      // loads the compiler waited for each of them in turn)
+      u32x4_t xraw[MT];
+#pragma unroll
+      for (int i = 0; i < MT; ++i) {
+        int row = m0 + 32 * i + l31;
+        row = row < g.M ? row : g.M - 1;
+        xraw[i] = u32x4_t{0, 0, 0, 0};
+        if (in) xraw[i] = *reinterpret_cast<const u32x4_t*>(lX + (int64_t)row * g.ldlx + r0);
+      }
 #pragma unroll
       for (int j = 0; j < NT; ++j) {
         int col = n0 + wv * 64 + 32 * j + l31;
@@ -466,22 +476,19 @@ __global__ __launch_bounds__(256) void nf4_gemm_rs_kernel(const RsArgs g, const 
           if (g.lw_row_major) {
             raw = *reinterpret_cast<const u32x4_t*>(lW + (int64_t)col * R + r0);
           } else {
+            uint32_t e[8];
 #pragma unroll
-            for (int d = 0; d < 4; ++d) {
-              const uint32_t lo = lW[(int64_t)(r0 + 2 * d) * g.Nout + col];
-              const uint32_t hi = lW[(int64_t)(r0 + 2 * d + 1) * g.Nout + col];
-              raw[d] = lo | (hi << 16);
-            }
+            for (int d = 0; d < 8; ++d) e[d] = lW[(int64_t)(r0 + d) * g.Nout + col];
+#pragma unroll
+            for (int d = 0; d < 4; ++d) raw[d] = e[2 * d] | (e[2 * d + 1] << 16);
           }
         }
         wfr[j] = __builtin_bit_cast(bf16x8_t, raw);
       }
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int i = 0; i < MT; ++i) {
-        int row = m0 + 32 * i + l31;
-        row = row < g.M ? row : g.M - 1;
-        u32x4_t raw = {0, 0, 0, 0};
-        if (in) raw = *reinterpret_cast<const u32x4_t*>(lX + (int64_t)row * g.ldlx + r0);
+        u32x4_t raw = xraw[i];
         if (g.lscale != 1.0f) {
 #pragma unroll
           for (int d = 0; d < 4; ++d)
@@ -932,6 +939,19 @@ __global__ __launch_bounds__(256) void nf4_gemm_rs16_kernel(const RsArgs g, cons
       const int r0 = rc + 8 * lg;
       const bool in = r0 < R;  // R % 8 == 0: a lane's 8 indices are all in or all out
       bf16x8_t wfr[NT];
+      // the requests of half a step first, then their uses: two trips to memory per step (with the scaling between two
+      // loads the compiler waited for each of them in turn)
+      u32x4_t xraw[MH];
+      auto load_x = [&](int ih) {
+#pragma unroll
+        for (int i = 0; i < MH; ++i) {
+          int row = m0 + 16 * (MH * ih + i) + l15;
+          row = row < g.M ? row : g.M - 1;
+          xraw[i] = u32x4_t{0, 0, 0, 0};
+          if (in) xraw[i] = *reinterpret_cast<const u32x4_t*>(lX + (int64_t)row * g.ldlx + r0);
+        }
+      };
+      load_x(0);
 #pragma unroll
       for (int j = 0; j < NT; ++j) {
         int col = n0 + wv * 64 + 16 * j + l15;
@@ -941,12 +961,11 @@ __global__ __launch_bounds__(256) void nf4_gemm_rs16_kernel(const RsArgs g, cons
           if (g.lw_row_major) {
             raw = *reinterpret_cast<const u32x4_t*>(lW + (int64_t)col * R + r0);
           } else {
+            uint32_t e[8];
 #pragma unroll
-            for (int d = 0; d < 4; ++d) {
-              const uint32_t lo = lW[(int64_t)(r0 + 2 * d) * g.Nout + col];
-              const uint32_t hi = lW[(int64_t)(r0 + 2 * d + 1) * g.Nout + col];
-              raw[d] = lo | (hi << 16);
-            }
+            for (int d = 0; d < 8; ++d) e[d] = lW[(int64_t)(r0 + d) * g.Nout + col];
+#pragma unroll
+            for (int d = 0; d < 4; ++d) raw[d] = e[2 * d] | (e[2 * d + 1] << 16);
           }
         }
         wfr[j] = __builtin_bit_cast(bf16x8_t, raw);
@@ -954,12 +973,11 @@ __global__ __launch_bounds__(256) void nf4_gemm_rs16_kernel(const RsArgs g, cons
 #pragma unroll
       for (int ih = 0; ih < 2; ++ih) {
         bf16x8_t xfr[MH];
+        if (ih == 1) load_x(1);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int i = 0; i < MH; ++i) {
-          int row = m0 + 16 * (MH * ih + i) + l15;
-          row = row < g.M ? row : g.M - 1;
-          u32x4_t raw = {0, 0, 0, 0};
-          if (in) raw = *reinterpret_cast<const u32x4_t*>(lX + (int64_t)row * g.ldlx + r0);
+          u32x4_t raw = xraw[i];
           if (g.lscale != 1.0f) {
 #pragma unroll
             for (int d = 0; d < 4; ++d)
