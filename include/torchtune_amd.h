@@ -306,8 +306,9 @@ int ttamd_lora_bwd_bf16(const void* gy, const void* x, const void* h, const void
  * One expansion for both directions (optional): when ttamd_nf4_gemm_expands_weight(M, N, K) is 1, the forward call
  * leaves the weight expanded to bf16, in forward tile order, in the first 2 N K bytes of its workspace.  A caller that
  * keeps those bytes until the backward passes them as tiles_fwd (else NULL): the grad-input then runs
- * ttamd_tiled_linear_dx_bf16 on them instead of expanding the weight a second time (same gx up to the order of fp32
- * sums inside a tile row; pays when the expansion is a large share of the call, i.e. at a few thousand tokens).
+ * ttamd_tiled_linear_dx_bf16 on them instead of expanding the weight a second time (the same products summed in the
+ * same order: the same gx bit for bit; pays when the expansion is a large share of the call, i.e. at a few thousand
+ * tokens).
  * With tiles_fwd (or gx == NULL) the backward needs only the bytes of gh and of ttamd_lora_bwd_workspace_bytes, each
  * rounded up to 256; the query above is the size that serves every case.
  */
