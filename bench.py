@@ -660,6 +660,9 @@ def main() -> int:
                     help="A/B (QAT workloads): one weight-gradient launch per member of a group instead of one for the group")
     ap.add_argument("--no-fused-qkv-post", action="store_true",
                     help="rotary embedding and key / value head expansion as four launches per layer and direction instead of one")
+    ap.add_argument("--no-fused-output-loss", action="store_true",
+                    help="QAT workload: the fake-quantised output projection and the loss as two autograd nodes (the gradient of the "
+                         "logits is then rescaled by the incoming gradient in a pass of its own) instead of one")
     ap.add_argument("--no-fused-add-norm", action="store_true",
                     help="A/B: the additions of the residual stream as passes of their own instead of inside the RMSNorm that "
                          "follows each of them")
@@ -704,6 +707,7 @@ def main() -> int:
     harness.GATED_EPILOGUE = not args.no_gated_epilogue
     harness.FUSED_ADD_NORM = not args.no_fused_add_norm
     harness.FUSED_QKV_POST = not args.no_fused_qkv_post
+    harness.FUSED_QAT_OUTPUT_LOSS = not args.no_fused_output_loss
     harness.SWIGLU_BWD_EPILOGUE = args.swiglu_bwd_epilogue
     ops.EXPANDED_WEIGHT_PATH = not args.no_expanded_weight
     if args.keep_forward_tiles is not None:

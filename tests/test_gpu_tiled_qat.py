@@ -225,3 +225,43 @@ def test_fake_quantized_gated_pair_matches_group_then_swiglu(N, K, M, monkeypatc
     layers[1].weight_fake_quantizer.enabled = False
     assert qat.fake_quantized_swiglu_group(x, layers[0], layers[1]) is None
 
+
+
+def test_output_projection_and_loss_as_one_node_equals_the_two_nodes():
+    """``FakeQuantizedLinear.cross_entropy_sum``: the fake-quantised vocabulary projection and the loss of a chunk of rows
+    as one autograd node against the layer followed by ``layer_ops.cross_entropy_sum``.  With the loss's own gradient (1)
+    coming in: the same loss, input gradient and weight gradient bit for bit (the factor multiplies other operands, and
+    multiplying by one is exact); with another factor: within a rounding of bf16."""
+    from torchtune_amd.modules import layer_ops
+
+    M, K, N = 2048, 8192, 8192
+    gen = torch.Generator(device=DEV).manual_seed(21)
+    layer = Int8DynActInt4WeightQATLinear(K, N, bias=False, groupsize=32, device=DEV, precision=BF)
+    with torch.no_grad():
+        layer.weight.copy_((torch.randn(N, K, device=DEV, generator=gen) * 0.02).to(BF))
+    x = torch.randn(M, K, device=DEV, generator=gen).to(BF)
+    target = torch.randint(0, N, (M,), device=DEV, generator=gen)
+    target[::7] = -100
+
+    def run(fused: bool, factor: float):
+        layer.zero_grad(set_to_none=True)
+        xg = x.clone().requires_grad_()
+        if fused:
+            loss = layer.cross_entropy_sum(xg, target, scale=1.0 / M)
+            assert loss is not None
+        else:
+            loss = layer_ops.cross_entropy_sum(layer(xg), target, scale=1.0 / M)
+        (loss * factor).backward()
+        return loss.detach(), xg.grad, layer.weight.grad
+
+    a, b = run(True, 1.0), run(False, 1.0)
+    assert torch.equal(a[0], b[0])
+    assert torch.equal(a[1].view(torch.int16), b[1].view(torch.int16))
+    assert torch.equal(a[2].view(torch.int16), b[2].view(torch.int16))
+    assert float(a[2].float().abs().max()) > 0
+    a, b = run(True, 3.0), run(False, 3.0)
+    for u, v in zip(a[1:], b[1:]):
+        torch.testing.assert_close(u.float(), v.float(), rtol=2.0 ** -6, atol=2.0 ** -7 * float(v.float().abs().max()))
+    # a layer with a bias, or too small for the library's own GEMM, is left to the caller
+    small = Int8DynActInt4WeightQATLinear(256, 512, bias=False, groupsize=32, device=DEV, precision=BF)
+    assert small.cross_entropy_sum(torch.randn(64, 256, device=DEV).to(BF), torch.zeros(64, dtype=torch.long, device=DEV)) is None

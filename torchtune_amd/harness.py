@@ -85,6 +85,10 @@ FUSED_ADD_NORM = True
 # True: the rotary embedding of q and k and the grouped-query expansion of k and v run as one launch per direction
 # (same bits; four launches and the intermediate rotated k less per layer and direction)
 FUSED_QKV_POST = True
+# A fake-quantised output projection and the loss of a chunk of rows as one autograd node
+# (``FakeQuantizedLinear.cross_entropy_sum``): backward then scales the [rows, dim] operands by the incoming gradient instead
+# of the [rows, vocabulary] gradient of the logits (False: the layer's output followed by ``layer_ops.cross_entropy_sum``).
+FUSED_QAT_OUTPUT_LOSS = True
 # True: RMSNorm, RoPE and the SwiGLU gate run as single-pass HIP kernels (bf16 on the GPU); False: the eager op chains
 # of the reference.  The quantized linears are unaffected.
 FUSED_LAYER_OPS = True
@@ -285,6 +289,11 @@ class Decoder(nn.Module):
             if plain and _fused(hc) and out.weight.dtype == hc.dtype:
                 total = total + layer_ops.linear_cross_entropy_sum(hc, out.weight, tc, scale=1.0 / n)
                 continue
+            if FUSED_QAT_OUTPUT_LOSS and hasattr(out, "cross_entropy_sum") and _fused(hc):
+                part = out.cross_entropy_sum(hc, tc, scale=1.0 / n)
+                if part is not None:
+                    total = total + part
+                    continue
             logits = self.output(hc)
             if _fused(logits) and logits.shape[-1] % 8 == 0 and logits.shape[-1] <= 131072:
                 total = total + layer_ops.cross_entropy_sum(logits, tc, scale=1.0 / n)

@@ -296,6 +296,45 @@ class _TiledFakeQuantLinearFn(torch.autograd.Function):
         return gx, gw, gb, None
 
 
+class _TiledFakeQuantLinearCrossEntropySumFn(torch.autograd.Function):
+    """``scale * cross_entropy(x @ fq(W).T, target, reduction="sum")`` as one node: the vocabulary projection of a
+    fake-quantised output layer and the loss of one chunk of rows (the reference: ``LinearCrossEntropyLoss.compute_cross_entropy``,
+    ``torchtune/modules/loss/cross_entropy_loss.py:86-112``, on a ``FakeQuantizedLinear``).  The loss kernel leaves the
+    gradient of the logits; in backward the incoming scalar multiplies the ``[rows, dim]`` operands of the two products
+    instead of that ``[rows, vocabulary]`` gradient (1 GB per chunk at 4096 x 128256)."""
+
+    @staticmethod
+    def forward(ctx, x, weight, quantizer, target, ignore_index: int, scale: float):
+        c = quantizer.config
+        N, K = weight.shape
+        x2 = x.reshape(-1, K)
+        need_gx = ctx.needs_input_grad[0]
+        tf, tb, qscale = ops.fq_per_group_int4_sym_tiled(weight.detach(), c.group_size, forward=True, backward=need_gx,
+                                                         qparam_dtype=c.scale_precision, eps=c.eps)
+        quantizer.scale = qscale.to(c.scale_precision)
+        quantizer.zero_point = None
+        logits = ops.tiled_linear(x2, tf, N)
+        loss, grad = ops.cross_entropy_fwd_bwd(logits, target.reshape(-1), ignore_index, scale)
+        ctx.save_for_backward(grad, x2, tb)
+        ctx.x_shape = x.shape
+        ctx.shape = (N, K)
+        return loss.sum() * scale
+
+    @staticmethod
+    def backward(ctx, g):
+        grad, x2, tb = ctx.saved_tensors
+        N, K = ctx.shape
+        need_x, need_w = ctx.needs_input_grad[:2]
+        g1 = g.float().reshape(1)  # a 1-D fp32 factor: products in fp32, rounded to bf16 once
+        gx = ops.tiled_linear(grad, tb, K).mul_(g1).view(ctx.x_shape) if need_x else None
+        gw = None
+        if need_w:
+            xs = x2.clone().mul_(g1)
+            own = ops.gemm_tn_applies(grad.shape[0], N, K) and (N // 256) * (K // 256) >= TN_GEMM_MIN_TILES
+            gw = ops.gemm_tn(grad, xs) if own else grad.t().matmul(xs)
+        return gx, gw, None, None, None, None
+
+
 class _TiledFakeQuantGroupFn(torch.autograd.Function):
     """Fake-quantised linears that read the same (already fake-quantised) input, as one node: every weight's fake
     quantisation goes into one stack of tiles per direction, the forward is one GEMM launch over the members' output
@@ -465,6 +504,21 @@ class FakeQuantizedLinear(nn.Linear):
             return _TiledFakeQuantLinearFn.apply(x, self.weight, self.bias, self.weight_fake_quantizer)
         w = self.weight if self.weight_fake_quantizer is None else self.weight_fake_quantizer(self.weight)
         return F.linear(x, w, self.bias)
+
+    def cross_entropy_sum(self, x: torch.Tensor, target: torch.Tensor, ignore_index: int = -100, scale: float = 1.0):
+        """``scale * F.cross_entropy(self(x).float(), target, reduction="sum", ignore_index=ignore_index)`` for one chunk of
+        rows, or None where this layer does not run on the library's own GEMM (the caller then composes it from
+        ``self(x)``).  Same loss and gradients as the composition, without the pass that rescales the logits' gradient."""
+        if self.bias is not None or self.weight_fake_quantizer is None:
+            return None
+        N = self.weight.shape[0]
+        if N % 8 != 0 or N > 131072:
+            return None
+        if self.activation_fake_quantizer is not None:
+            x = self.activation_fake_quantizer(x)
+        if not self._tiled_ok(x):
+            return None
+        return _TiledFakeQuantLinearCrossEntropySumFn.apply(x, self.weight, self.weight_fake_quantizer, target, ignore_index, scale)
 
     def to_linear(self) -> nn.Linear:
         new = nn.Linear(self.in_features, self.out_features, self.bias is not None, device=self.weight.device,
