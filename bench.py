@@ -663,6 +663,9 @@ def main() -> int:
     ap.add_argument("--no-fused-output-loss", action="store_true",
                     help="QAT workload: the fake-quantised output projection and the loss as two autograd nodes (the gradient of the "
                          "logits is then rescaled by the incoming gradient in a pass of its own) instead of one")
+    ap.add_argument("--no-fused-swiglu-bwd", action="store_true",
+                    help="the backward of silu(gate) * up as a pass of its own ahead of the gate / up pair's adapter backward, instead "
+                         "of inside the pass that multiplies its results with the adapters")
     ap.add_argument("--no-fused-add-norm", action="store_true",
                     help="A/B: the additions of the residual stream as passes of their own instead of inside the RMSNorm that "
                          "follows each of them")
@@ -708,6 +711,8 @@ def main() -> int:
     harness.FUSED_ADD_NORM = not args.no_fused_add_norm
     harness.FUSED_QKV_POST = not args.no_fused_qkv_post
     harness.FUSED_QAT_OUTPUT_LOSS = not args.no_fused_output_loss
+    from torchtune_amd.modules.peft import group as _peft_group
+    _peft_group.FUSED_SWIGLU_BWD = not args.no_fused_swiglu_bwd
     harness.SWIGLU_BWD_EPILOGUE = args.swiglu_bwd_epilogue
     ops.EXPANDED_WEIGHT_PATH = not args.no_expanded_weight
     if args.keep_forward_tiles is not None:

@@ -383,6 +383,16 @@ int ttamd_nf4_lora_group_swiglu_fwd_bf16(const void* x, const ttamd_lora_group_m
 size_t ttamd_lora_group_bwd_workspace_bytes(const ttamd_lora_group_member* members, int n_members, int64_t M, int64_t K);
 int ttamd_lora_group_bwd_bf16(const void* x, const void* h_cat, const ttamd_lora_group_member* members, int n_members,
                               void* gh_cat, int64_t M, int64_t K, void* workspace, size_t workspace_bytes, void* stream);
+/* The same for the gate / up pair of a SwiGLU feed-forward (torchtune/modules/feed_forward.py:50-53), starting one step
+ * earlier: from gact, the gradient of silu(w1 x) * w3 x, and the two projections gate = w1 x, up = w3 x (bf16 [M, N]).
+ * members[0] = w1 (gate), members[1] = w3 (up), equal N; members[i].y = OUT, the gradients of the two projections (the
+ * bits of ttamd_swiglu_bwd_bf16), then everything ttamd_lora_group_bwd_bf16 writes (the same bits).  Wide members
+ * (N >= 8192, rank <= 16, M >= 1024) get both from one pass: the gradients are formed and stored by the kernel that
+ * multiplies them with lora_b and h, and are not read back; otherwise the two steps run one after the other.
+ * Workspace: ttamd_lora_group_bwd_workspace_bytes.  No counterpart in the reference (autograd runs the two steps). */
+int ttamd_lora_group_swiglu_bwd_bf16(const void* x, const void* h_cat, const ttamd_lora_group_member* members, int n_members,
+                                     const void* gact, const void* gate, const void* up, void* gh_cat, int64_t M, int64_t K,
+                                     void* workspace, size_t workspace_bytes, void* stream);
 /* gx out, bf16 [M, K], from gh_cat and members[i].y = gy_i, quantized_data_t, block_scalers_t, lora_a */
 int ttamd_nf4_group_bwd_dx_bf16(const ttamd_lora_group_member* members, int n_members, const void* gh_cat, void* gx, int64_t M,
                                 int64_t K, void* stream);

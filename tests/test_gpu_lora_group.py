@@ -426,3 +426,33 @@ def test_group_rejects_mismatched_operands():
                                                                     torch.zeros(8, 64, device=DEV, dtype=BF)])
     with pytest.raises(ValueError):
         ops.lora_group_fwd(x, members * 3)  # six members
+
+
+@pytest.mark.parametrize("M,K,N,ranks", [
+    (8192, 4096, 14336, (16, 16)),   # the 8B gate / up pair: the pass that forms the gradients also multiplies them
+    (1100, 512, 8192, (16, 8)),      # ragged rows, different ranks, still wide
+    (2048, 512, 8256, (8, 8)),       # a width that is no multiple of the 256-column groups
+    (300, 512, 1024, (16, 16)),      # narrow: the two steps one after the other inside the call
+])
+def test_swiglu_backward_inside_the_adapter_backward_equals_the_two_steps_bitwise(M, K, N, ranks):
+    """``ops.lora_group_bwd(..., swiglu=(gact, gate, up))`` (``ttamd_lora_group_swiglu_bwd_bf16``) against
+    ``ops.swiglu_bwd`` followed by ``ops.lora_group_bwd`` on its results: gh, grad A and (through the grouped grad-input,
+    which reads the gradients the call left in memory) gx bit for bit; grad B up to the order of its fp32 sums over the
+    row ranges (the pair kernel cuts the rows into twice as many ranges: rtol 2^-7, atol 2^-7 of the largest entry)."""
+    mem = _members(K, (N, N), ranks, seed=M + N)
+    members = [m[0] for m in mem]
+    g = torch.Generator().manual_seed(9)
+    x = torch.randn(M, K, generator=g).to(BF).to(DEV)
+    h_cat = (torch.randn(M, sum(ranks), generator=g) * 0.5).to(BF).to(DEV)
+    gact = torch.randn(M, N, generator=g).to(BF).to(DEV)
+    gate = (torch.randn(M, N, generator=g) * 2).to(BF).to(DEV)
+    up = torch.randn(M, N, generator=g).to(BF).to(DEV)
+    ggate, gup = ops.swiglu_bwd(gact, gate, up)
+    gx0, grads0, gh0 = ops.lora_group_bwd(x, h_cat, members, [ggate, gup], want_gx=True)
+    gx1, grads1, gh1 = ops.lora_group_bwd(x, h_cat, members, None, want_gx=True, swiglu=(gact, gate, up))
+    assert torch.equal(gh0.view(torch.int16), gh1.view(torch.int16))
+    assert torch.equal(gx0.view(torch.int16), gx1.view(torch.int16))
+    for (a0, b0), (a1, b1) in zip(grads0, grads1):
+        assert torch.equal(a0.view(torch.int16), a1.view(torch.int16))
+        torch.testing.assert_close(b1.float(), b0.float(), rtol=2.0 ** -7, atol=2.0 ** -7 * float(b0.float().abs().max()))
+    assert float(gh1.float().abs().max()) > 0 and float(gx1.float().abs().max()) > 0

@@ -112,6 +112,7 @@ SIGNATURES = {
                                                     _c_void_p]),
     "ttamd_lora_group_bwd_workspace_bytes": (_size, [_c_void_p, _int, _i64, _i64]),
     "ttamd_lora_group_bwd_bf16": (_int, [_c_void_p, _c_void_p, _c_void_p, _int, _c_void_p, _i64, _i64, _c_void_p, _size, _c_void_p]),
+    "ttamd_lora_group_swiglu_bwd_bf16": (_int, [_c_void_p, _c_void_p, _c_void_p, _int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _i64, _i64, _c_void_p, _size, _c_void_p]),
     "ttamd_nf4_group_bwd_dx_bf16": (_int, [_c_void_p, _int, _c_void_p, _c_void_p, _i64, _i64, _c_void_p]),
     "ttamd_nf4_group_bwd_dx_workspace_bytes": (_size, [_c_void_p, _int, _i64, _i64]),
     "ttamd_nf4_group_bwd_dx_ws_bf16": (_int, [_c_void_p, _int, _c_void_p, _c_void_p, _i64, _i64, _c_void_p, _size, _c_void_p]),

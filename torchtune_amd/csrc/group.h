@@ -93,6 +93,15 @@ int run_group_hidden(const uint16_t* x, const GroupSkinny& g, uint16_t* h_cat, f
 size_t group_lora_bwd_ws_bytes(const GroupSkinny& g);
 // gh_cat[:, member i] = scale[i] . gy[i] . lora_b[i];  ga[i] = gh_i^T . x (one pass over x for all members);
 // gb[i] = scale[i] . gy[i]^T . h_i
-int run_group_lora_bwd(const uint16_t* x, const uint16_t* h_cat, const GroupSkinny& g, uint16_t* gh_cat, float* ws, hipStream_t s);
+// sw (optional; the gate / up pair of a SwiGLU feed-forward): g.gy[0] and g.gy[1] are then OUTPUTS, the gradients of gate
+// and up, which this call derives from the gradient of silu(gate) * up first - in the same pass that forms the products
+// reading them where that pass exists (two wide members of equal width), otherwise by the stand-alone kernel.
+struct SwigluBwdInputs {
+  const uint16_t* gact;  // [M, N]
+  const uint16_t* gate;  // [M, N]
+  const uint16_t* up;    // [M, N]
+};
+int run_group_lora_bwd(const uint16_t* x, const uint16_t* h_cat, const GroupSkinny& g, uint16_t* gh_cat, float* ws, hipStream_t s,
+                       const SwigluBwdInputs* sw = nullptr);
 
 }  // namespace ttamd

@@ -184,6 +184,25 @@ extern "C" int ttamd_lora_group_bwd_bf16(const void* x, const void* h_cat, const
                             reinterpret_cast<uint16_t*>(gh_cat), reinterpret_cast<float*>(workspace), reinterpret_cast<hipStream_t>(stream));
 }
 
+// The pair's adapter backward from the gradient of silu(gate) * up: members[0] = gate, members[1] = up, members[i].y = OUT
+// (the gradients of the two projections, which the grouped grad-input then reads).
+extern "C" int ttamd_lora_group_swiglu_bwd_bf16(const void* x, const void* h_cat, const ttamd_lora_group_member* members, int n_members,
+                                                const void* gact, const void* gate, const void* up, void* gh_cat, int64_t M, int64_t K,
+                                                void* workspace, size_t workspace_bytes, void* stream) {
+  TT_REQUIRE(n_members == 2 && members && members[0].N == members[1].N,
+             "lora_group_swiglu_bwd: takes the gate and the up projection, two members of equal width");
+  Decoded d;
+  if (int rc = decode("lora_group_swiglu_bwd", members, n_members, M, K, true, d)) return rc;
+  TT_REQUIRE(x && h_cat && gh_cat && workspace && gact && gate && up, "lora_group_swiglu_bwd: null pointer argument");
+  TT_REQUIRE(aligned16(x) && aligned16(h_cat) && aligned16(gh_cat) && aligned16(workspace), "lora_group_swiglu_bwd: pointers must be 16-byte aligned");
+  const size_t need = group_lora_bwd_ws_bytes(d.sk);
+  if (workspace_bytes < need) return fail(TTAMD_EWORKSPACE, "lora_group_swiglu_bwd: workspace has %zu bytes, needs %zu", workspace_bytes, need);
+  const SwigluBwdInputs sw = {reinterpret_cast<const uint16_t*>(gact), reinterpret_cast<const uint16_t*>(gate),
+                              reinterpret_cast<const uint16_t*>(up)};
+  return run_group_lora_bwd(reinterpret_cast<const uint16_t*>(x), reinterpret_cast<const uint16_t*>(h_cat), d.sk,
+                            reinterpret_cast<uint16_t*>(gh_cat), reinterpret_cast<float*>(workspace), reinterpret_cast<hipStream_t>(stream), &sw);
+}
+
 extern "C" int ttamd_nf4_group_bwd_dx_bf16(const ttamd_lora_group_member* members, int n_members, const void* gh_cat, void* gx,
                                            int64_t M, int64_t K, void* stream) {
   Decoded d;

@@ -17,6 +17,7 @@
 #include "common.h"
 #include "group.h"
 #include "nf4_math.h"
+#include "swiglu_math.h"
 
 namespace ttamd {
 namespace {
@@ -661,6 +662,262 @@ __global__ __launch_bounds__(256) void skinny_tn_gh_kernel(const TnGhBatch a) {
 #endif
 }
 
+// ---------------------------------------------------------------------------------------------------
+// swiglu_bwd_tn_gh: the backward of act = silu(gate) * up (torchtune/modules/feed_forward.py:50-53) and, from the same
+// pass, both products of the gate / up pair's adapters that read the gradients it produces.  The stand-alone sequence is
+// ttamd_swiglu_bwd_bf16 (reads gact, gate, up; writes ggate, gup) followed by skinny_tn_gh on (ggate, gup), which reads
+// the two gradients back; here a wave computes a 32 x 128 piece of ggate and of gup from the matching pieces of gact,
+// gate and up (swiglu_math.h: the bits of the stand-alone kernel), stores both, and feeds them from its registers to
+// the LDS copy-in of skinny_tn_gh's two products, member 0 (gate) and then member 1 (up).  Sums, their order and the
+// partial-sum layouts are those of skinny_tn_gh_kernel on a batch of the two members, so every result is the same bits.
+// The inputs of the next piece are requested while the current one is multiplied.
+// ---------------------------------------------------------------------------------------------------
+struct SwigluGhArgs {
+  const uint16_t* gact;  // [M, Kc]
+  const uint16_t* gate;  // [M, Kc]
+  const uint16_t* up;    // [M, Kc]
+  uint16_t* gx[2];       // out: ggate, gup [M, Kc]
+  const uint16_t* G[2];  // h of the member: rows ldg elements apart
+  const uint16_t* Bm[2]; // lora_b [Kc, R]
+  float* part[2];        // [splits, R, Kc]
+  float* part_h[2];      // [column groups, M, R]
+  int R[2];
+  int Kc, ldg, M, rows_per_split;
+};
+
+__global__ __launch_bounds__(256) void swiglu_bwd_tn_gh_kernel(const SwigluGhArgs a) {
+  constexpr int kTrWaveLds = tn_wave_lds(1);
+#if defined(__HIP_DEVICE_COMPILE__)
+  const int Kc = a.Kc, M = a.M, ldg = a.ldg, rows_per_split = a.rows_per_split;
+  const int col_group = (int)blockIdx.x;
+  __shared__ __attribute__((aligned(16))) char stage[4 * kTrWaveLds];
+  static_assert(sizeof(stage) >= 3 * 32 * 64 * sizeof(float), "the reduction reuses the staging memory");
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int g = lane >> 4, i = lane & 15;
+  const int c0 = col_group * kTnGhCols;
+  const int split = blockIdx.y;
+  const int m_begin = split * rows_per_split;
+  int m_end = m_begin + rows_per_split;
+  m_end = m_end < M ? m_end : M;
+
+  char* my = stage + wave * kTrWaveLds;
+  bool xcol_ok[2];
+  int64_t xcol[2];
+#pragma unroll
+  for (int p = 0; p < 2; ++p) {
+    const int c = c0 + 128 * p + 8 * i;
+    xcol_ok[p] = c < Kc;  // Kc % 8 == 0
+    xcol[p] = xcol_ok[p] ? c : 0;
+  }
+  char* xdst = my + g * kTrPitchX + 16 * i;
+  const int gcol = 8 * (lane & 1);
+  char* gdst = my + 32 * kTrPitchX + (lane >> 1) * 32 + 16 * (lane & 1);
+  const uint32_t my_lds = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)my);
+  const uint32_t xrd = my_lds + (8 * g + (i >> 2)) * kTrPitchX + 8 * (i & 3);
+  const uint32_t grd = my_lds + 32 * kTrPitchX + (8 * g + (i >> 2)) * 32 + 8 * (i & 3);
+  const char* prd = my + i * kTrPitchX + 32 * g;
+
+  // Bm operands of both members, staged and read back as in skinny_tn_gh_kernel
+  u32x4_t bfrag[2][2][2][2];
+#pragma unroll
+  for (int mem = 0; mem < 2; ++mem) {
+    const uint16_t* __restrict__ Bm = a.Bm[mem];
+    const int R = a.R[mem];
+    const int ppr = R >> 3;
+    const uint32_t brd = my_lds + (16 * g + (i >> 2)) * 32 + 8 * (i & 3);
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int pc = lane + 64 * q;
+        if (pc < 16 * R) {
+          const int n = c0 + 128 * p + pc / ppr;
+          u32x4_t v = u32x4_t{0, 0, 0, 0};
+          if (n < Kc) v = *reinterpret_cast<const u32x4_t*>(Bm + (int64_t)n * R + 8 * (pc % ppr));
+          *reinterpret_cast<u32x4_t*>(my + (pc / ppr) * 32 + 16 * (pc % ppr)) = v;
+        }
+      }
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // LDS operations of a wave complete in order
+      u32x2_t lo[2][2], hi[2][2];
+#pragma unroll
+      for (int H = 0; H < 2; ++H)
+#pragma unroll
+        for (int hh = 0; hh < 2; ++hh) {
+          lo[H][hh] = lds_read_tr16(brd, (64 * H + 8 * hh) * 32);
+          hi[H][hh] = lds_read_tr16(brd, (64 * H + 8 * hh + 4) * 32);
+        }
+#pragma unroll
+      for (int H = 0; H < 2; ++H)
+#pragma unroll
+        for (int hh = 0; hh < 2; ++hh) {
+          asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(lo[H][hh]), "+v"(hi[H][hh]));
+          bfrag[mem][p][H][hh] = u32x4_t{lo[H][hh].x, lo[H][hh].y, hi[H][hh].x, hi[H][hh].y};
+        }
+    }
+  }
+
+  f32x4_t acc[2][2][8];
+#pragma unroll
+  for (int mem = 0; mem < 2; ++mem)
+#pragma unroll
+    for (int p = 0; p < 2; ++p)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[mem][p][e] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+  // the inputs of one piece: rows m + 4 u + g, the 8 columns at xcol[p]
+  u32x4_t in_o[8], in_g[8], in_u[8], gv[2];
+  auto fetch_u = [&](int m, int p, int u) {
+    const int row = m + 4 * u + g;
+    in_o[u] = in_g[u] = in_u[u] = u32x4_t{0, 0, 0, 0};
+    if (row < m_end && xcol_ok[p]) {
+      const int64_t at = (int64_t)row * Kc + xcol[p];
+      in_o[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(a.gact + at));
+      in_g[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(a.gate + at));
+      in_u[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(a.up + at));
+    }
+  };
+  auto fetch = [&](int m, int p) {
+#pragma unroll
+    for (int u = 0; u < 8; ++u) fetch_u(m, p, u);
+  };
+  auto fetch_h = [&](int m) {
+    const int grow = m + (lane >> 1);
+#pragma unroll
+    for (int mem = 0; mem < 2; ++mem) {
+      gv[mem] = u32x4_t{0, 0, 0, 0};
+      if (grow < m_end && gcol < a.R[mem]) gv[mem] = *reinterpret_cast<const u32x4_t*>(a.G[mem] + (int64_t)grow * ldg + gcol);
+    }
+  };
+  int m = m_begin + 32 * wave;
+  if (m < m_end) {
+    fetch(m, 0);
+    fetch_h(m);
+  }
+  for (; m < m_end; m += 128) {
+    f32x4_t acc_h[2][2];
+#pragma unroll
+    for (int mem = 0; mem < 2; ++mem) acc_h[mem][0] = acc_h[mem][1] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    u32x4_t gop[2];
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {
+      // the piece of both gradients, stored and kept in registers for the two copy-ins below; as soon as a row group's
+      // inputs are used up, the same registers are asked for the next piece's, so that those requests are in flight
+      // through the arithmetic of the remaining row groups and the products below
+      u32x4_t xg[2][8];
+      const bool more = p == 0 || m + 128 < m_end;  // uniform over the wave
+      const int next_m = p == 0 ? m : m + 128, next_p = p ^ 1;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+          uint32_t dg, du;
+          swiglu_bwd_pair(in_o[u][d], in_g[u][d], in_u[u][d], dg, du);
+          xg[0][u][d] = dg;
+          xg[1][u][d] = du;
+        }
+        if (more) fetch_u(next_m, next_p, u);
+        const int row = m + 4 * u + g;
+        if (row < m_end && xcol_ok[p]) {
+          const int64_t at = (int64_t)row * Kc + xcol[p];
+          __builtin_nontemporal_store(xg[0][u], reinterpret_cast<u32x4_t*>(a.gx[0] + at));
+          __builtin_nontemporal_store(xg[1][u], reinterpret_cast<u32x4_t*>(a.gx[1] + at));
+        }
+      }
+      u32x4_t gvn[2] = {gv[0], gv[1]};
+      if (p == 1 && more) fetch_h(m + 128);
+#pragma unroll
+      for (int mem = 0; mem < 2; ++mem) {
+        // every read of this region has been waited for before the MFMA that used it
+#pragma unroll
+        for (int u = 0; u < 8; ++u) *reinterpret_cast<u32x4_t*>(xdst + 4 * u * kTrPitchX) = xg[mem][u];
+        if (p == 0) *reinterpret_cast<u32x4_t*>(gdst) = gvn[mem];  // zeros beyond R
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");       // the copy-in has landed
+        if (p == 0) {
+          u32x2_t ga = lds_read_tr16(grd, 0), gb = lds_read_tr16(grd, 4 * 32);
+          asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(ga), "+v"(gb));
+          gop[mem] = u32x4_t{ga.x, ga.y, gb.x, gb.y};
+        }
+        u32x2_t xa[8], xb[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          xa[e] = lds_read_tr16(xrd, 32 * e);
+          xb[e] = lds_read_tr16(xrd, 32 * e + 4 * kTrPitchX);
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(xa[e]), "+v"(xb[e]) : "n"(14 - 2 * e));
+          const u32x4_t xop = {xa[e].x, xa[e].y, xb[e].x, xb[e].y};
+          acc[mem][p][e] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, gop[mem]), __builtin_bit_cast(bf16x8_t, xop),
+                                                                  acc[mem][p][e], 0, 0, 0);
+        }
+        u32x4_t pr[2][2][2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int H = 0; H < 2; ++H)
+#pragma unroll
+            for (int hh = 0; hh < 2; ++hh)
+              pr[t][H][hh] = *reinterpret_cast<const u32x4_t*>(prd + 16 * t * kTrPitchX + 128 * H + 16 * hh);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // before the region is written again
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int H = 0; H < 2; ++H)
+#pragma unroll
+            for (int hh = 0; hh < 2; ++hh)
+              acc_h[mem][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, pr[t][H][hh]),
+                                                                     __builtin_bit_cast(bf16x8_t, bfrag[mem][p][H][hh]), acc_h[mem][t], 0, 0, 0);
+      }
+    }
+#pragma unroll
+    for (int mem = 0; mem < 2; ++mem) {
+      const int R = a.R[mem];
+      if (i < R) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int v = 0; v < 4; ++v) {
+            const int row = m + 16 * t + 4 * g + v;
+            if (row < m_end) a.part_h[mem][((int64_t)col_group * M + row) * R + i] = acc_h[mem][t][v];
+          }
+      }
+    }
+  }
+  float (*red)[32][64] = reinterpret_cast<float (*)[32][64]>(stage);
+#pragma unroll
+  for (int mem = 0; mem < 2; ++mem) {
+    const int R = a.R[mem];
+    float* __restrict__ part = a.part[mem];
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {
+      __syncthreads();  // the staging regions (or the previous piece's sums) are free
+      if (wave > 0) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+#pragma unroll
+          for (int v = 0; v < 4; ++v) red[wave - 1][v * 8 + e][lane] = acc[mem][p][e][v];
+      }
+      __syncthreads();
+      if (wave == 0) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          const int r = 4 * g + v;
+          if (r >= R) continue;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const int col = c0 + 128 * p + 16 * e + i;
+            if (col >= Kc) continue;
+            part[((int64_t)split * R + r) * Kc + col] =
+                ((acc[mem][p][e][v] + red[0][v * 8 + e][lane]) + red[1][v * 8 + e][lane]) + red[2][v * 8 + e][lane];
+          }
+        }
+      }
+    }
+  }
+#endif
+}
+
 // out[r * stride_r + k * stride_k] = bf16(scale * sum_s part[s * split_stride + r * Kc + k]) for r < R, k < Kc
 struct TnSum {
   const float* part;
@@ -836,9 +1093,15 @@ TnPlan plan_tn_gh(const GroupSkinny& g) {
   for (int i = 0; i < g.n; ++i) groups += tn_gh_col_groups(g.N[i]);
   return plan_tn(g.M, groups);
 }
-// fp32 partial sums of the fused pass: per member the column groups' [M, R] and the row splits' [R, N]
+// The pair kernel (swiglu_bwd_tn_gh_kernel) serves both members from one workgroup per column group: half as many
+// column groups in the grid, so twice the row splits fill the chip.
+bool tn_gh_pair(const GroupSkinny& g) { return g.n == 2 && g.N[0] == g.N[1]; }
+TnPlan plan_tn_gh_pair(const GroupSkinny& g) { return plan_tn(g.M, tn_gh_col_groups(g.N[0])); }
+// fp32 partial sums of the fused pass: per member the column groups' [M, R] and the row splits' [R, N] (room for the
+// plan with more splits where both kernels can serve the group)
 size_t tn_gh_part_bytes(const GroupSkinny& g) {
-  const TnPlan pl = plan_tn_gh(g);
+  TnPlan pl = plan_tn_gh(g);
+  if (tn_gh_pair(g) && plan_tn_gh_pair(g).splits > pl.splits) pl = plan_tn_gh_pair(g);
   size_t total = 0;
   for (int i = 0; i < g.n; ++i)
     total += align256(((size_t)tn_gh_col_groups(g.N[i]) * g.M + (size_t)pl.splits * g.N[i]) * g.rank[i] * sizeof(float));
@@ -910,12 +1173,24 @@ size_t group_lora_bwd_ws_bytes(const GroupSkinny& g) {
   return align256(nt > tn ? nt : tn);
 }
 
-int run_group_lora_bwd(const uint16_t* x, const uint16_t* h_cat, const GroupSkinny& g, uint16_t* gh_cat, float* ws, hipStream_t s) {
+int run_group_lora_bwd(const uint16_t* x, const uint16_t* h_cat, const GroupSkinny& g, uint16_t* gh_cat, float* ws, hipStream_t s,
+                       const SwigluBwdInputs* sw) {
   const int rt = g.r_off[g.n];
+  // the pair's gradients from the pass that reads them (swiglu_bwd_tn_gh_kernel) where that pass exists
+  const bool sw_fused = sw && tn_gh_pair(g) && tn_gh_applies(g);
+  if (sw) {
+    TT_REQUIRE(g.n == 2 && g.N[0] == g.N[1] && sw->gact && sw->gate && sw->up && aligned16(sw->gact) && aligned16(sw->gate) &&
+                   aligned16(sw->up) && aligned16(g.gy[0]) && aligned16(g.gy[1]),
+               "lora_group_swiglu_bwd: takes the gate and the up projection (equal widths) and 16-byte aligned gact, gate, up, ggate, gup");
+    if (!sw_fused)
+      if (int rc = ttamd_swiglu_bwd_bf16(sw->gact, sw->gate, sw->up, const_cast<uint16_t*>(g.gy[0]), const_cast<uint16_t*>(g.gy[1]),
+                                         g.M * g.N[0], s))
+        return rc;
+  }
   if (tn_gh_applies(g)) {
     // one pass over every gy for gB and gh, the column groups of gh summed, then gA over x; the reductions of gA and gB
     // share the last launch
-    const TnPlan pl = plan_tn_gh(g);
+    const TnPlan pl = sw_fused ? plan_tn_gh_pair(g) : plan_tn_gh(g);
     TnGhBatch b = {};
     NtBatch sums = {};
     TnSumBatch f = {};
@@ -943,7 +1218,18 @@ int run_group_lora_bwd(const uint16_t* x, const uint16_t* h_cat, const GroupSkin
       S.scale = g.scale[i];
       f.p[g.n + i] = TnSum{P.part, g.gb[i], (int)g.N[i], g.rank[i], g.scale[i], (int64_t)g.rank[i] * g.N[i], 1, g.rank[i], pl.splits};
     }
-    skinny_tn_gh_kernel<<<dim3((unsigned)groups, (unsigned)pl.splits), dim3(256), 0, s>>>(b);
+    if (sw_fused) {
+      SwigluGhArgs f2 = {};
+      f2.gact = sw->gact; f2.gate = sw->gate; f2.up = sw->up;
+      for (int i = 0; i < 2; ++i) {
+        f2.gx[i] = const_cast<uint16_t*>(g.gy[i]);
+        f2.G[i] = b.p[i].G; f2.Bm[i] = b.p[i].Bm; f2.part[i] = b.p[i].part; f2.part_h[i] = b.p[i].part_h; f2.R[i] = b.p[i].R;
+      }
+      f2.Kc = (int)g.N[0]; f2.ldg = rt; f2.M = (int)g.M; f2.rows_per_split = pl.rows_per_split;
+      swiglu_bwd_tn_gh_kernel<<<dim3((unsigned)tn_gh_col_groups(g.N[0]), (unsigned)pl.splits), dim3(256), 0, s>>>(f2);
+    } else {
+      skinny_tn_gh_kernel<<<dim3((unsigned)groups, (unsigned)pl.splits), dim3(256), 0, s>>>(b);
+    }
     sum_partials_kernel<<<dim3((unsigned)((g.M * 16 + 255) / 256), (unsigned)g.n), dim3(256), 0, s>>>(sums);
     if (int rc = check_launch("skinny_tn_gh")) return rc;
     TnBatch t = {};

@@ -20,6 +20,11 @@ from ...nf4_tensor import _check_in_features
 from .lora import LoRALinear
 
 
+# The backward of ``silu(gate) * up`` inside the library call that multiplies its results with the pair's adapters (one pass
+# over the two gradients less per layer at training sizes); False: ``ops.swiglu_bwd`` first.  Same results.
+FUSED_SWIGLU_BWD = True
+
+
 def _copies(weights, tokens: int):
     """The members' transposed copies for a call over ``tokens`` rows: none when the grouped grad-input runs on the
     expanded-weight path (it reads the weights' own codes), else every member's ``backward_copy()``."""
@@ -91,8 +96,10 @@ def _keep_tiles(ctx, tiles, paired: bool, tokens: int, weights, resident: bool =
     ctx.tiles, ctx.tiles_paired = (tiles, paired) if keep else (None, False)
 
 
-def _group_backward(ctx, x2, h_cat, weights, las, lbs, gy2):
-    """Gradients of a group call in the order of its inputs (x, scales, then weight, lora_a, lora_b, bias per member)."""
+def _group_backward(ctx, x2, h_cat, weights, las, lbs, gy2, swiglu=None):
+    """Gradients of a group call in the order of its inputs (x, scales, then weight, lora_a, lora_b, bias per member).
+    ``swiglu=(gact, gate, up)`` with ``gy2`` None: the output gradients are those of ``silu(gate) * up``, formed inside the
+    library call (``ops.lora_group_bwd``); biases then get no gradient here (the gated pair has none)."""
     n = len(weights)
     need_x = ctx.needs_input_grad[0]
     tiles, paired = (ctx.tiles, ctx.tiles_paired) if need_x else (None, False)
@@ -100,12 +107,12 @@ def _group_backward(ctx, x2, h_cat, weights, las, lbs, gy2):
     copies = [None] * n if tiles is not None else _copies(weights, x2.shape[0])
     members = [ops.GroupMember(w.quantized_data, w.block_scalers(), tr, a, b, None, s, w.shape[0])
                for w, tr, a, b, s in zip(weights, copies, las, lbs, ctx.scales)]
-    gx, grads, _ = ops.lora_group_bwd(x2, h_cat, members, gy2, want_gx=need_x, tiles=tiles, paired=paired)
+    gx, grads, _ = ops.lora_group_bwd(x2, h_cat, members, gy2, want_gx=need_x, tiles=tiles, paired=paired, swiglu=swiglu)
     out: List = [gx.view(ctx.x_shape) if need_x else None, None]
     for i in range(n):
         _, need_a, need_b, need_bias = ctx.needs_input_grad[2 + 4 * i:6 + 4 * i]
         out += [None, grads[i][0] if need_a else None, grads[i][1] if need_b else None,
-                gy2[i].sum(dim=0) if (ctx.has_bias[i] and need_bias) else None]
+                gy2[i].sum(dim=0) if (gy2 is not None and ctx.has_bias[i] and need_bias) else None]
     return tuple(out)
 
 
@@ -136,6 +143,8 @@ class _QLoRAGatedFn(torch.autograd.Function):
         x2, h_cat, gate, up = saved[:4]
         rest = saved[4:]
         weights, las, lbs = rest[:2], rest[2:4], rest[4:6]
+        if FUSED_SWIGLU_BWD and not any(ctx.has_bias):
+            return _group_backward(ctx, x2, h_cat, weights, las, lbs, None, swiglu=(gact.reshape(gate.shape), gate, up))
         ggate, gup = ops.swiglu_bwd(gact.reshape(gate.shape), gate, up)
         return _group_backward(ctx, x2, h_cat, weights, las, lbs, [ggate, gup])
 

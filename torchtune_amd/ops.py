@@ -649,15 +649,27 @@ def lora_group_fwd(x: torch.Tensor, members: Sequence[GroupMember], swiglu: bool
     return h_cat, outs
 
 
-def lora_group_bwd(x: torch.Tensor, h_cat: torch.Tensor, members: Sequence[GroupMember], gys: Sequence[torch.Tensor],
-                   want_gx: bool = True, tiles: Optional[torch.Tensor] = None, paired: bool = False):
+def lora_group_bwd(x: torch.Tensor, h_cat: torch.Tensor, members: Sequence[GroupMember], gys: Optional[Sequence[torch.Tensor]],
+                   want_gx: bool = True, tiles: Optional[torch.Tensor] = None, paired: bool = False, swiglu=None):
     """-> (gx [M, K] or None, [(gA_i, gB_i)], gh_cat): the backward of ``lora_group_fwd`` given the output gradients.
     ``tiles`` / ``paired``: what the forward call returned with ``return_tiles=True``; the grouped grad-input then reads
-    those tiles instead of expanding the members' weights again."""
+    those tiles instead of expanding the members' weights again.
+
+    ``swiglu=(gact, gate, up)`` (two members of equal width, the gate and the up projection; ``gys`` None): the output
+    gradients are those of ``act = silu(gate) * up`` given the gradient of ``act`` - ``swiglu_bwd(gact, gate, up)``, formed
+    by the library in the pass that multiplies them with the adapters where such a pass exists
+    (``ttamd_lora_group_swiglu_bwd_bf16``); same results as the two steps."""
     x = _bf16_2d(x, "lora_group_bwd")
     h_cat = _bf16_2d(h_cat, "lora_group_bwd")
     M, K = x.shape
     dev = x.device
+    if swiglu is not None:
+        if gys is not None or len(members) != 2 or members[0].N != members[1].N:
+            raise ValueError("lora_group_bwd: swiglu takes the gate and the up projection (equal widths) and no output gradients")
+        sw = [_bf16_2d(t, "lora_group_bwd") for t in swiglu]
+        if any(tuple(t.shape) != (M, members[0].N) for t in sw):
+            raise ValueError(f"lora_group_bwd: gact, gate and up must be [{M}, {members[0].N}]")
+        gys = [torch.empty(M, members[0].N, dtype=torch.bfloat16, device=dev) for _ in range(2)]
     gys = [_bf16_2d(g, "lora_group_bwd") for g in gys]
     grads = [(torch.empty(m.lora_a.shape, dtype=torch.bfloat16, device=dev), torch.empty(m.lora_b.shape, dtype=torch.bfloat16, device=dev))
              for m in members]
@@ -675,8 +687,12 @@ def lora_group_bwd(x: torch.Tensor, h_cat: torch.Tensor, members: Sequence[Group
     lib = _lib.load()
     ws = _workspace(lib.ttamd_lora_group_bwd_workspace_bytes(arr, n, M, K), dev)
     with torch.cuda.device(dev):
-        rc = lib.ttamd_lora_group_bwd_bf16(x.data_ptr(), h_cat.data_ptr(), arr, n, gh_cat.data_ptr(), M, K, ws.data_ptr(), ws.numel(),
-                                           _stream(x))
+        if swiglu is not None:
+            rc = lib.ttamd_lora_group_swiglu_bwd_bf16(x.data_ptr(), h_cat.data_ptr(), arr, n, sw[0].data_ptr(), sw[1].data_ptr(),
+                                                      sw[2].data_ptr(), gh_cat.data_ptr(), M, K, ws.data_ptr(), ws.numel(), _stream(x))
+        else:
+            rc = lib.ttamd_lora_group_bwd_bf16(x.data_ptr(), h_cat.data_ptr(), arr, n, gh_cat.data_ptr(), M, K, ws.data_ptr(), ws.numel(),
+                                               _stream(x))
         _lib.check(rc, "lora_group_bwd")
         if want_gx:
             events = _gemm_timer("bwd_group", M, [m.N for m in members], K, [int(e.rank) for e in arr]) if _gemm_timer is not None else None
