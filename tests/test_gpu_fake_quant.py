@@ -275,7 +275,7 @@ def test_post_training_quantizers_use_the_convert_arithmetic():
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 def test_bf16_scale_precision_bit_exact(dtype):
-    """scale_precision = bfloat16 (BASELINE config 4 asks for bf16 scales; the reference's default is float32): the scale
+    """scale_precision = bfloat16 (the QAT benchmark configuration asks for bf16 scales; the reference's default is float32): the scale
     is rounded to bf16 once chosen and the rounded scale quantises and dequantises, in the per-token, the per-group and
     the convert kernels, and the converted layer reproduces the fake-quantised one."""
     gen = torch.Generator().manual_seed(41)
