@@ -388,6 +388,49 @@ def test_one_expansion_serves_both_directions(kind, monkeypatch):
         assert torch.equal(a.view(torch.int16), b.view(torch.int16))
 
 
+@pytest.mark.parametrize("kind", ["single", "qkv_group", "gated_pair", "feed_forward"])
+def test_kept_tiles_do_not_outlive_the_first_pass_of_a_checkpointed_forward(kind, monkeypatch):
+    """The kept tiles are one of the node's saved tensors, so a checkpointed forward (``use_reentrant=False``) lets go of
+    them with everything else it saved: between the forward and the backward of a checkpointed layer no more memory is
+    allocated than with the tiles not kept at all (2 B per weight element otherwise - every layer's, in a stack of
+    checkpointed layers); without checkpointing they are held, which is what keeping them means."""
+    from torch.utils.checkpoint import checkpoint
+    from torchtune_amd.modules.peft import group as group_mod
+
+    M, K = 2048, 8192
+    g = torch.Generator(device=DEV).manual_seed(6)
+    x = torch.randn(M, K, device=DEV, generator=g).to(BF)
+    if kind == "single":
+        layers = _lora_layers([8192], K, 16, seed=1)
+        fn = lambda t: layers[0](t)
+    elif kind == "qkv_group":
+        layers = _lora_layers([4096, 2048, 2048], K, 16, seed=2)
+        fn = lambda t: group_mod.lora_linear_group(t, layers)
+    elif kind == "gated_pair":
+        layers = _lora_layers([4096, 4096], K, 16, seed=3)
+        fn = lambda t: group_mod.lora_swiglu_group(t, layers[0], layers[1])
+    else:
+        layers = _lora_layers([4096, 4096], K, 16, seed=4) + _lora_layers([8192], 4096, 16, seed=5)
+        fn = lambda t: group_mod.lora_feed_forward(t, layers[0], layers[1], layers[2])
+    weight_elements = sum(layer.weight.shape[0] * layer.weight.shape[1] for layer in layers if layer.weight.shape[1] == K)
+
+    def held_after_forward(keep_tokens, checkpointed):
+        monkeypatch.setattr(ops, "KEEP_FORWARD_TILES_MAX_TOKENS", keep_tokens)
+        xg = x.clone().requires_grad_()
+        torch.cuda.synchronize()
+        before = torch.cuda.memory_allocated()
+        out = checkpoint(fn, xg, use_reentrant=False) if checkpointed else fn(xg)
+        torch.cuda.synchronize()
+        held = torch.cuda.memory_allocated() - before
+        outs = out if isinstance(out, tuple) else (out,)
+        torch.autograd.backward(outs, [torch.ones_like(o) for o in outs])
+        return held
+
+    held_after_forward(M, True)   # first calls build the weights' derived caches: not part of what is compared
+    assert held_after_forward(M, True) == held_after_forward(0, True)
+    assert held_after_forward(M, False) - held_after_forward(0, False) >= 2 * weight_elements
+
+
 @pytest.mark.parametrize("kind", ["single", "qkv_group", "gated_pair"])
 def test_expanded_weights_kept_across_calls(kind, monkeypatch):
     """With a budget in ``ops.RESIDENT_TILES_MAX_BYTES`` the first many-token forward of a layer (or group) leaves its

@@ -46,8 +46,8 @@ class _QLoRAGroupFn(torch.autograd.Function):
         x2 = x.reshape(-1, K)
         members = [ops.GroupMember(w.quantized_data, w.block_scalers(), tr, a, b, bias, s, w.shape[0])
                    for w, tr, a, b, bias, s in zip(weights, _copies(weights, x2.shape[0]), las, lbs, biases, scales)]
-        h_cat, ys = _group_forward(ctx, x2, members, weights, False)
-        ctx.save_for_backward(x2, h_cat, *weights, *las, *lbs)
+        h_cat, ys, kept = _group_forward(ctx, x2, members, weights, False)
+        ctx.save_for_backward(x2, h_cat, *weights, *las, *lbs, kept)
         ctx.scales = scales
         ctx.x_shape = x.shape
         ctx.has_bias = tuple(b is not None for b in biases)
@@ -59,7 +59,7 @@ class _QLoRAGroupFn(torch.autograd.Function):
         n = len(ctx.scales)
         saved = ctx.saved_tensors  # read once: activation checkpointing unpacks on every access
         x2, h_cat = saved[:2]
-        rest = saved[2:]
+        rest, ctx.kept_tiles = saved[2:-1], saved[-1]
         weights, las, lbs = rest[:n], rest[n:2 * n], rest[2 * n:3 * n]
         gy2 = []
         for g, w in zip(gys, weights):
@@ -72,7 +72,7 @@ class _QLoRAGroupFn(torch.autograd.Function):
 def _group_forward(ctx, x2, members, weights, swiglu: bool):
     """``ops.lora_group_fwd`` on the expanded weights an earlier call left with the group where such tiles are kept across
     calls (``ops.RESIDENT_TILES_MAX_BYTES``), leaving this call's there when there are none yet; decides which tiles the
-    node hands to its backward.  -> (h_cat, outputs)"""
+    node hands to its backward.  -> (h_cat, outputs, the tiles to save for backward or None)"""
     tokens = x2.shape[0]
     found = nf4_tensor.resident_group_tiles(weights, swiglu) if ops.resident_tiles_enabled() else None
     if found is not None:
@@ -82,18 +82,20 @@ def _group_forward(ctx, x2, members, weights, swiglu: bool):
         h_cat, outs, tiles, paired = ops.lora_group_fwd(x2, members, swiglu=swiglu, return_tiles=True)
         resident = (tiles is not None and ops.resident_tiles_enabled()
                     and nf4_tensor.keep_resident_group_tiles(weights, swiglu, tiles, paired))
-    _keep_tiles(ctx, tiles, paired, tokens, weights, resident)
-    return h_cat, outs
+    return h_cat, outs, _keep_tiles(ctx, tiles, paired, tokens, weights, resident)
 
 
-def _keep_tiles(ctx, tiles, paired: bool, tokens: int, weights, resident: bool = False) -> None:
+def _keep_tiles(ctx, tiles, paired: bool, tokens: int, weights, resident: bool = False):
     """The group forward's expanded weights stay with the node when the backward will want a grad-input, the call is
     short enough for one expansion per layer to pay (``ops.KEEP_FORWARD_TILES_MAX_TOKENS``; any length when the tiles are
     kept across calls anyway) and the grouped grad-input is the many-token launch (with few output tiles it stays on the
-    fused kernel)."""
+    fused kernel).  Returns what the node saves for backward (the LAST of its saved tensors: a saved tensor, not an
+    attribute of the node, so that activation checkpointing drops it with the first pass and the recomputation brings it
+    back - one layer's tiles alive at a time), or None."""
     keep = (tiles is not None and ctx.needs_input_grad[0] and (resident or ops.keeps_forward_tiles(tokens))
             and ops.group_dx_expands(tokens, weights[0].shape[1], [w.shape[0] for w in weights]))
-    ctx.tiles, ctx.tiles_paired = (tiles, paired) if keep else (None, False)
+    ctx.tiles_paired = bool(keep and paired)
+    return tiles if keep else None
 
 
 def _group_backward(ctx, x2, h_cat, weights, las, lbs, gy2, swiglu=None):
@@ -102,8 +104,8 @@ def _group_backward(ctx, x2, h_cat, weights, las, lbs, gy2, swiglu=None):
     library call (``ops.lora_group_bwd``); biases then get no gradient here (the gated pair has none)."""
     n = len(weights)
     need_x = ctx.needs_input_grad[0]
-    tiles, paired = (ctx.tiles, ctx.tiles_paired) if need_x else (None, False)
-    ctx.tiles = None
+    tiles, paired = (ctx.kept_tiles, ctx.tiles_paired) if need_x else (None, False)
+    ctx.kept_tiles = None
     copies = [None] * n if tiles is not None else _copies(weights, x2.shape[0])
     members = [ops.GroupMember(w.quantized_data, w.block_scalers(), tr, a, b, None, s, w.shape[0])
                for w, tr, a, b, s in zip(weights, copies, las, lbs, ctx.scales)]
@@ -130,8 +132,8 @@ class _QLoRAGatedFn(torch.autograd.Function):
         x2 = x.reshape(-1, K)
         members = [ops.GroupMember(w.quantized_data, w.block_scalers(), tr, a, b, bias, s, w.shape[0])
                    for w, tr, a, b, bias, s in zip(weights, _copies(weights, x2.shape[0]), las, lbs, biases, scales)]
-        h_cat, (gate, up, act) = _group_forward(ctx, x2, members, weights, True)
-        ctx.save_for_backward(x2, h_cat, gate, up, *weights, *las, *lbs)
+        h_cat, (gate, up, act), kept = _group_forward(ctx, x2, members, weights, True)
+        ctx.save_for_backward(x2, h_cat, gate, up, *weights, *las, *lbs, kept)
         ctx.scales = scales
         ctx.x_shape = x.shape
         ctx.has_bias = tuple(b is not None for b in biases)
@@ -141,7 +143,7 @@ class _QLoRAGatedFn(torch.autograd.Function):
     def backward(ctx, gact):
         saved = ctx.saved_tensors
         x2, h_cat, gate, up = saved[:4]
-        rest = saved[4:]
+        rest, ctx.kept_tiles = saved[4:-1], saved[-1]
         weights, las, lbs = rest[:2], rest[2:4], rest[4:6]
         if FUSED_SWIGLU_BWD and not any(ctx.has_bias):
             return _group_backward(ctx, x2, h_cat, weights, las, lbs, None, swiglu=(gact.reshape(gate.shape), gate, up))
@@ -165,13 +167,13 @@ class _QLoRAFeedForwardFn(torch.autograd.Function):
         x2 = x.reshape(-1, K)
         members = [ops.GroupMember(w.quantized_data, w.block_scalers(), tr, a, b, bias, s, w.shape[0])
                    for w, tr, a, b, bias, s in zip(weights[:2], _copies(weights[:2], x2.shape[0]), las, lbs, biases, scales)]
-        h_cat, (gate, up, act) = _group_forward(ctx, x2, members, weights[:2], True)
+        h_cat, (gate, up, act), kept = _group_forward(ctx, x2, members, weights[:2], True)
         w2 = weights[2]
         h2 = ops.lora_hidden(act, las[2])
         tr = w2.backward_copy_for(act.shape[0], True)
         y = ops.nf4_lora_linear_fwd(act, w2.quantized_data, w2.block_scalers(), w2.shape[0], h2, lbs[2], scales[2], biases[2],
                                     block_scalers_t=tr[1] if tr else None)
-        ctx.save_for_backward(x2, h_cat, gate, up, act, h2, *weights, *las, *lbs)
+        ctx.save_for_backward(x2, h_cat, gate, up, act, h2, *weights, *las, *lbs, kept)
         ctx.scales = scales
         ctx.x_shape = x.shape
         ctx.has_bias = tuple(b is not None for b in biases)
@@ -181,7 +183,7 @@ class _QLoRAFeedForwardFn(torch.autograd.Function):
     def backward(ctx, gy):
         saved = ctx.saved_tensors
         x2, h_cat, gate, up, act, h2 = saved[:6]
-        rest = saved[6:]
+        rest, ctx.kept_tiles = saved[6:-1], saved[-1]
         weights, las, lbs = rest[:3], rest[3:6], rest[6:9]
         w2 = weights[2]
         gy2 = gy.reshape(-1, w2.shape[0])

@@ -74,8 +74,9 @@ class _QLoRALinearFn(torch.autograd.Function):
             resident = resident and tiles is not None and weight.keep_resident_tiles(tiles)
         if resident:  # the tiles exist anyway: the grad-input reads them wherever it is a many-token launch
             keep = ctx.needs_input_grad[0] and ops.gemm_expands_weight(x2.shape[0], K, N)
-        ctx.tiles = tiles if keep else None
-        ctx.save_for_backward(x2, h, weight, lora_a, lora_b)
+        # kept as a saved tensor, not as an attribute of the node: activation checkpointing then drops it with the other
+        # saved tensors of the first pass and the recomputation brings it back, so that one layer's tiles are alive at a time
+        ctx.save_for_backward(x2, h, weight, lora_a, lora_b, tiles if keep else None)
         ctx.scale = scale
         ctx.x_shape = x.shape
         ctx.has_bias = bias is not None
@@ -83,14 +84,13 @@ class _QLoRALinearFn(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, gy):
-        x2, h, weight, lora_a, lora_b = ctx.saved_tensors
+        x2, h, weight, lora_a, lora_b, kept = ctx.saved_tensors
         N, K = shape_and_dtype(weight)[0]
         gy2 = gy.reshape(-1, N)
         need_x, _, need_a, need_b, need_bias, _ = ctx.needs_input_grad
         gx = ga = gb = gbias = None
         if need_x or need_a or need_b:
-            tiles = ctx.tiles if need_x else None
-            ctx.tiles = None
+            tiles = kept if need_x else None
             tr = weight.backward_copy_for(gy2.shape[0], False) if (need_x and tiles is None) else None
             if ONE_CALL_PER_DIRECTION and not ops.gemm_timer_installed():
                 gx, ga, gb = ops.qlora_linear_bwd(gy2, x2, h, weight.quantized_data, weight.block_scalers(), lora_a, lora_b,
