@@ -269,6 +269,8 @@ SWEEP = [
     # M, N, K, rank: shortest contractions (one and two 64-wide entries), ragged rows, widths off the 256 grid
     (2048, 8192, 64, 8), (2048, 8192, 128, 16), (2049, 8192 + 192, 192, 8), (2304, 7424, 320, 32), (3000, 5568, 448, 16),
     (8192, 2048, 256, 8), (4096, 4096, 1024, 16), (2048, 16384, 64, 0),
+    # ranks beyond 32 (two steps of adapter operands), also over the shortest contractions
+    (2048, 8192, 64, 64), (2048, 8192, 128, 40), (2304, 7424, 320, 64),
 ]
 
 

@@ -53,6 +53,8 @@ SHAPES = [
     (1000, 1024, (512, 256, 256, 64), (32, 16, 8, 8)),
     (4096, 1024, (1024, 256, 256), (16, 16, 16)),   # 256-row tiles, unsliced rank-r products
     (2048, 256, (4096, 4096), (32, 32)),
+    (2048, 256, (4096, 4096), (40, 24)),            # many-token launch, a rank beyond 32: two steps of adapter operands
+    (2048, 64, (4096, 2048, 2048), (8, 16, 8)),     # many-token launch over the shortest contraction
 ]
 
 
@@ -258,6 +260,9 @@ GATED_SHAPES = [
     (16, 512, 1024, (8, 8), False),             # few tokens: group launch + a pass of its own
     (300, 512, 512, (16, 16), True),            # tiled kernels + a pass of its own
     (2048, 256, 1152, (16, 16), False),         # many tokens, too few tiles for the expanded path
+    (2048, 256, 4096, (40, 24), False),         # a rank beyond 32: the members' adapter operands in entries of their own
+    (2048, 64, 4096, (16, 8), True),            # the shortest contraction: the adapter's operands are requested up front
+    (2048, 128, 4096, (8, 32), False),          # two trips of the loop, both past the weight
 ]
 
 

@@ -335,6 +335,9 @@ struct DenseArgs {
 
 constexpr int kEpiPlain = 0, kEpiGated = 1, kEpiSwigluBwd = 2;
 
+// what the direct-to-LDS requests of the adapter's operands read for ranks beyond R
+static __device__ __attribute__((aligned(16))) const uint32_t kZero16[4] = {0u, 0u, 0u, 0u};
+
 constexpr int kAEntry = 32768;  // activation ring: 3 entries of 256 rows x 64 k
 constexpr int kWBase = 3 * kAEntry;
 constexpr int kWStage = 16384;  // weight ring: 4 stages of 256 columns x 32 k
@@ -452,12 +455,14 @@ __device__ __forceinline__ void gemm_dense_tile(const DenseArgs g) {
       // 2 (tk / 4) + tk % 2 of segment (tk / 2) % 2; the row pitch is the same for both
       xb = reinterpret_cast<const char*>(g.seg[(tk >> 1) & 1].X) + ((int64_t)(((tk >> 2) << 1) + (tk & 1)) << 7);
     } else {
-      while (tk >= seg_end) {
-        ++seg;
-        seg_begin = seg_end;
-        seg_end += g.seg[seg].Kc >> 6;
-        a_base = reinterpret_cast<const char*>(g.seg[seg].X);
-        set_segment();
+      if constexpr (!LW_ROW_MAJOR) {  // a forward launch has one segment (checked on the host): no walk in its loop
+        while (tk >= seg_end) {
+          ++seg;
+          seg_begin = seg_end;
+          seg_end += g.seg[seg].Kc >> 6;
+          a_base = reinterpret_cast<const char*>(g.seg[seg].X);
+          set_segment();
+        }
       }
       xb = a_base + ((int64_t)(tk - seg_begin) << 7);  // + 64 elements * 2 bytes per entry
     }
@@ -466,6 +471,99 @@ __device__ __forceinline__ void gemm_dense_tile(const DenseArgs g) {
     dma16(a_off[1], xb, sa, 1024);
     dma16(a_off[2], xb, sa, 2048);
     dma16(a_off[3], xb, sa, 3072);
+  };
+
+  // ---- forward launches: the adapter's operands travel through the same rings as further k-steps of the contraction.
+  //      Past the end of the weight the loop's requests used to fetch the last step again; they now fetch the adapter:
+  //      16 bytes (8 ranks of one row of lX / one row of lW) per lane, zeros beyond R, so that by the end of the loop the
+  //      operands sit in LDS in the loop's own layout and the adapter costs one more k-step per 32 ranks instead of a trip
+  //      to memory.  Ranks of at most 32 (ad_compact) need activation entry nk2 and weight step nk only: the entry's first
+  //      half holds the 32 ranks of lX (GATED: of the gate's lX, and the second half those of the up projection's), the
+  //      step the ranks of lW for the tile's 256 columns; nothing is requested in the loop's last trip then, and nothing
+  //      is in flight when the loop ends.  Otherwise entry nk2 holds 64 ranks (GATED: the gate's, and entry nk2 + 1 the up
+  //      projection's) and steps nk, nk + 1 ranks [0, 32) and [32, 64).
+  bool ad_rings = false;  // uniform over the workgroup
+  bool ad_compact = false;
+  // the tile's adapter ([0]; GATED: the two members'), read once and held in scalar registers: R = 0 where there is none
+  int ad_R[2] = {0, 0}, ad_ncols[2] = {0, 0};
+  const uint16_t* ad_lX[2] = {nullptr, nullptr};
+  const uint16_t* ad_lW[2] = {nullptr, nullptr};
+  float ad_lscale[2] = {1.0f, 1.0f};
+  int ad_col0 = 0;  // first column of the tile among the adapter's columns
+  const char* const zero_src = reinterpret_cast<const char*>(kZero16);
+  auto ad_src_a = [&](int q, int i) -> const char* {  // what request i of entry nk2 + q reads
+    const int c = a_chunk[i] >> 4;                    // 16-byte chunk of the entry's row: 8 ranks
+    int a, r0;                                        // member and first rank this chunk holds
+    if (GATED) {
+      a = ad_compact ? c >> 2 : q;
+      r0 = ad_compact ? 8 * (c & 3) : 8 * c;
+    } else {
+      a = 0;
+      r0 = q == 0 ? 8 * c : 64;
+    }
+    const uint16_t* lX = a ? ad_lX[1] : ad_lX[0];
+    return r0 < (a ? ad_R[1] : ad_R[0]) ? reinterpret_cast<const char*>(lX + (int64_t)a_row[i] * g.ldlx + r0) : zero_src;
+  };
+  auto ad_src_w = [&](int step, int b) -> const char* {  // what request b of step nk + step reads
+    const int a = GATED ? wm : 0;                        // GATED: column blocks 2 wv, 2 wv + 1 are the gate's for wv < 4
+    const int R = a ? ad_R[1] : ad_R[0], ncols = a ? ad_ncols[1] : ad_ncols[0];
+    const uint16_t* lW = a ? ad_lW[1] : ad_lW[0];
+    const int r0 = 32 * step + 8 * g4;
+    int col = ad_col0 + 16 * (GATED ? (2 * wv + b) & 7 : 2 * wv + b) + l15;
+    col = col < ncols ? col : ncols - 1;
+    return r0 < R ? reinterpret_cast<const char*>(lW + (int64_t)col * R + r0) : zero_src;
+  };
+  // per-lane sources of entry nk2 and step nk, worked out while the prologue's requests are on their way
+  const char* ad_a0[4] = {zero_src, zero_src, zero_src, zero_src};
+  const char* ad_w0[2] = {zero_src, zero_src};
+  auto ad_setup = [&]() {
+    if constexpr (LW_ROW_MAJOR) {
+      auto take = [&](int slot, int aidx) {
+        ad_R[slot] = g.ad[aidx].R;
+        ad_ncols[slot] = g.ad[aidx].n_end - g.ad[aidx].n_begin;
+        ad_lX[slot] = g.ad[aidx].lX;
+        ad_lW[slot] = g.ad[aidx].lW;
+        ad_lscale[slot] = g.ad[aidx].lscale;
+      };
+      if constexpr (GATED) {
+        if (g.nad > 0 && g.ad[0].R > 0) take(0, 0);
+        if (g.nad > 1 && g.ad[1].R > 0) take(1, 1);
+        ad_col0 = 128 * tile_n;
+      } else {
+        int ad_idx = -1;
+        for (int aidx = 0; aidx < g.nad; ++aidx)
+          if (g.ad[aidx].R > 0 && n0 >= g.ad[aidx].n_begin && n0 < g.ad[aidx].n_end) ad_idx = aidx;
+        ad_idx = __builtin_amdgcn_readfirstlane(ad_idx);  // the same in every lane: the fields come through scalar loads
+        if (ad_idx >= 0) {
+          take(0, ad_idx);
+          ad_col0 = n0 - g.ad[ad_idx].n_begin;
+        }
+      }
+      ad_rings = ad_R[0] > 0 || ad_R[1] > 0;
+      ad_compact = ad_R[0] <= 32 && ad_R[1] <= 32;
+      if (ad_rings) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) ad_a0[i] = ad_src_a(0, i);
+#pragma unroll
+        for (int b = 0; b < 2; ++b) ad_w0[b] = ad_src_w(0, b);
+      }
+    }
+  };
+  auto dma16v = [&](const char* src, uint32_t lds, int imm) {
+    asm volatile("s_add_u32 m0, %1, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                 ::"v"(src), "s"(lds), "n"(imm) : "memory", "m0", "scc");
+  };
+  auto issue_a_ad = [&](int q, int entry) {  // q = 0: entry nk2, 1: entry nk2 + 1
+    const uint32_t sa = lds0 + entry * kAEntry + wv * 4096;
+    dma16v(q == 0 ? ad_a0[0] : ad_src_a(1, 0), sa, 0);
+    dma16v(q == 0 ? ad_a0[1] : ad_src_a(1, 1), sa, 1024);
+    dma16v(q == 0 ? ad_a0[2] : ad_src_a(1, 2), sa, 2048);
+    dma16v(q == 0 ? ad_a0[3] : ad_src_a(1, 3), sa, 3072);
+  };
+  auto issue_w_ad = [&](int step, int stage) {  // step = 0: ranks [0, 32), 1: ranks [32, 64)
+    const uint32_t sw = lds0 + kWBase + stage * kWStage + wv * 2048;
+    dma16v(step == 0 ? ad_w0[0] : ad_src_w(1, 0), sw, 0);
+    dma16v(step == 0 ? ad_w0[1] : ad_src_w(1, 1), sw, 1024);
   };
 
   // operand read offsets: activation tile 0 of this wave, half hf of the entry: row 128 wm + l15, chunk 4 hf + g4
@@ -543,37 +641,94 @@ __device__ __forceinline__ void gemm_dense_tile(const DenseArgs g) {
   issue_a(0, 0);
   issue_w(0, 0);
   issue_w(1, 1);
-  issue_a(1, 1);
-  issue_w(2, 2);
+  if (LW_ROW_MAJOR && nk == 2) {  // a contraction of 64: the prologue already reaches past the weight
+    ad_setup();
+    if (ad_rings) {
+      issue_a_ad(0, 1);
+      issue_w_ad(0, 2);
+    } else {
+      issue_a(1, 1);
+      issue_w(2, 2);
+    }
+  } else {
+    issue_a(1, 1);
+    issue_w(2, 2);
+    ad_setup();
+  }
   asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");  // A(0), W(0) landed everywhere
   if (wm == 1) asm volatile("s_barrier" ::: "memory");
   // one copy of the loop per wave group: the two differ in one wait, and a branch per step costs 2 - 4 %
   auto main_loop = [&](auto lgkm) {
     constexpr bool kLgkm = decltype(lgkm)::value;
     int e0 = 0, ws = 0;  // activation entry of the current pair of steps, weight stage of the current step
-    for (int t = 0; t < nk; t += 2) {
+    // The last two trips, whose requests reach past the weight, are copies of the loop that ask for the adapter's
+    // operands instead (ad_rings; no trip of the first copy pays for the choice).  kTrip 1 (t = nk - 4) requests entry
+    // nk2 and step nk where the others request the activations and the weight; kTrip 2 (t = nk - 2) requests step nk + 1,
+    // entry nk2 + 1 and step nk + 1 again (the count of requests in flight stays what the waits assume) - or nothing
+    // (ad_compact), and then waits by the counts of that case: newer than W(nk - 1) are A x4 and W(nk) x2, and by the end
+    // of the last step everything has landed.
+    auto pair = [&](int t, auto trip) {
+      constexpr int kTrip = decltype(trip)::value;
+      const bool nothing = kTrip == 2 && ad_compact;
       const int e1 = e0 == 2 ? 0 : e0 + 1, e2 = e1 == 2 ? 0 : e1 + 1;
       // ---- even step t
-      issue_w(t + 3, (ws + 3) & 3);
-      issue_a((t >> 1) + 2, e2);
+      if constexpr (kTrip == 2) {
+        if (!nothing) {
+          issue_w_ad(1, (ws + 3) & 3);
+          issue_a_ad(1, e2);
+        }
+      } else {
+        issue_w(t + 3, (ws + 3) & 3);
+        if constexpr (kTrip == 1)
+          issue_a_ad(0, e2);
+        else
+          issue_a((t >> 1) + 2, e2);
+      }
       read_step(e0, 0, ws);
       __builtin_amdgcn_sched_barrier(0);
-      if constexpr (kLgkm)
-        asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-      else
-        asm volatile("s_waitcnt vmcnt(12)\n\ts_barrier" ::: "memory");
+      if (nothing) {
+        if constexpr (kLgkm)
+          asm volatile("s_waitcnt vmcnt(6) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        else
+          asm volatile("s_waitcnt vmcnt(6)\n\ts_barrier" ::: "memory");
+      } else {
+        if constexpr (kLgkm)
+          asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        else
+          asm volatile("s_waitcnt vmcnt(12)\n\ts_barrier" ::: "memory");
+      }
       compute();
       // ---- odd step t + 1
-      issue_w(t + 4, ws);
+      if constexpr (kTrip == 0)
+        issue_w(t + 4, ws);
+      else if constexpr (kTrip == 1)
+        issue_w_ad(0, ws);
+      else if (!nothing)
+        issue_w_ad(1, ws);
       read_step(e0, 1, (ws + 1) & 3);
       __builtin_amdgcn_sched_barrier(0);
-      if constexpr (kLgkm)
-        asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-      else
-        asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");
+      if (nothing) {
+        if constexpr (kLgkm)
+          asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        else
+          asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+      } else {
+        if constexpr (kLgkm)
+          asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        else
+          asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");
+      }
       compute();
       e0 = e1;
       ws = (ws + 2) & 3;
+    };
+    const int t_tail = ad_rings ? nk - 4 : nk;
+    for (int t = 0; t < t_tail; t += 2) pair(t, std::integral_constant<int, 0>{});
+    if constexpr (LW_ROW_MAJOR) {
+      if (ad_rings) {
+        if (nk >= 4) pair(nk - 4, std::integral_constant<int, 1>{});
+        pair(nk - 2, std::integral_constant<int, 2>{});
+      }
     }
   };
   if (wm == 1)
@@ -583,9 +738,42 @@ __device__ __forceinline__ void gemm_dense_tile(const DenseArgs g) {
   if (wm == 0) asm volatile("s_barrier" ::: "memory");
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the clamped requests of the last steps
 
-  // ---- adapters: one MFMA step per 32 ranks and segment, operands straight from global memory.  Lane (l15, g4) holds
+  // the adapter's scale goes onto the activation side, bf16(lscale * lX), as in the fused kernel; a power of two is
+  // exact on either operand, and the weight side has half as many registers to scale
+  auto scaled = [&](u32x4_t raw, float lscale) {
+#pragma unroll
+    for (int d = 0; d < 4; ++d)
+      raw[d] = pack_bf16x2(bits_f32(raw[d] << 16) * lscale, bits_f32(raw[d] & 0xffff0000u) * lscale);
+    return raw;
+  };
+  // ---- adapters from the rings (see issue_a_ad): steps nk, nk + 1 of the loop with the scale on one operand
+  if (ad_rings) {
+    __syncthreads();  // every wave's requests have landed
+    const int a = GATED ? (wn >> 1) : 0;
+    const int R = a ? ad_R[1] : ad_R[0];
+    const float lscale = a ? ad_lscale[1] : ad_lscale[0];
+    const bool on_w = (f32_bits(lscale) & 0x007fffffu) == 0;
+    const int entry = (nk2 + (GATED && !ad_compact ? a : 0)) % 3;
+    for (int step = 0; 32 * step < R; ++step) {
+      read_step(entry, GATED && ad_compact ? a : step, (nk + step) & 3);
+      bf16x8_t wfr[NT], xfr[MT];
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+        wfr[j] = lscale != 1.0f && on_w ? __builtin_bit_cast(bf16x8_t, scaled(__builtin_bit_cast(u32x4_t, wf[j]), lscale)) : wf[j];
+#pragma unroll
+      for (int i = 0; i < MT; ++i)
+        xfr[i] = lscale != 1.0f && !on_w ? __builtin_bit_cast(bf16x8_t, scaled(__builtin_bit_cast(u32x4_t, xf[i]), lscale)) : xf[i];
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int i = 0; i < MT; ++i) acc[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wfr[j], xfr[i], acc[j][i], 0, 0, 0);
+    }
+  }
+
+  // ---- adapters of the grad-input launches, whose lW lies the other way: one MFMA
+  //      step per 32 ranks and segment, operands straight from global memory.  Lane (l15, g4) holds
   //      ranks rc + 8 g4 .. + 7 of weight column / activation row l15 of its tile; ranks beyond R are zero.
-  for (int aidx = 0; aidx < g.nad; ++aidx) {
+  for (int aidx = 0; aidx < (LW_ROW_MAJOR ? 0 : g.nad); ++aidx) {
     const int R = g.ad[aidx].R;
     const int nb = g.ad[aidx].n_begin, ncols = g.ad[aidx].n_end - nb;
     if constexpr (GATED) {
@@ -648,19 +836,11 @@ __device__ __forceinline__ void gemm_dense_tile(const DenseArgs g) {
       }
       __builtin_amdgcn_sched_barrier(0);
       bf16x8_t wfr[NT], xfr[MT];
-      // the adapter's scale goes onto the activation side, bf16(lscale * lX), as in the fused kernel; a power of two is
-      // exact on either operand, and the weight side has half as many registers to scale
       const bool on_w = (f32_bits(lscale) & 0x007fffffu) == 0;
-      auto scaled = [&](u32x4_t raw) {
 #pragma unroll
-        for (int d = 0; d < 4; ++d)
-          raw[d] = pack_bf16x2(bits_f32(raw[d] << 16) * lscale, bits_f32(raw[d] & 0xffff0000u) * lscale);
-        return raw;
-      };
+      for (int j = 0; j < NT; ++j) wfr[j] = __builtin_bit_cast(bf16x8_t, lscale != 1.0f && on_w ? scaled(wraw[j], lscale) : wraw[j]);
 #pragma unroll
-      for (int j = 0; j < NT; ++j) wfr[j] = __builtin_bit_cast(bf16x8_t, lscale != 1.0f && on_w ? scaled(wraw[j]) : wraw[j]);
-#pragma unroll
-      for (int i = 0; i < MT; ++i) xfr[i] = __builtin_bit_cast(bf16x8_t, lscale != 1.0f && !on_w ? scaled(xraw[i]) : xraw[i]);
+      for (int i = 0; i < MT; ++i) xfr[i] = __builtin_bit_cast(bf16x8_t, lscale != 1.0f && !on_w ? scaled(xraw[i], lscale) : xraw[i]);
 #pragma unroll
       for (int j = 0; j < NT; ++j)
 #pragma unroll
@@ -869,6 +1049,11 @@ int launch_dense(DenseArgs& g, hipStream_t s) {
     if (dev >= 0) attr_set[dev] = true;
   }
   const dim3 grid((unsigned)(g.tiles_m * g.tiles_n)), block(512);
+  TT_REQUIRE(!g.lw_row_major || g.nseg == 1, "nf4_gemm_dense: a forward launch contracts over one activation tensor (%d given)", g.nseg);
+  if (g.lw_row_major)  // forward: the adapter's operands ride the rings behind the weight's last steps
+    for (int i = 0; i < g.nad; ++i)
+      TT_REQUIRE(g.ad[i].R <= 0 || (g.ad[i].R <= 64 && g.ad[i].R % 8 == 0 && g.ldlx % 8 == 0),
+                 "nf4_gemm_dense: the adapter of a forward launch needs a rank that is a multiple of 8, at most 64 (%d)", g.ad[i].R);
   if (g.w_tr) {
     TT_REQUIRE(!g.lw_row_major && !g.act && !g.sw_gup && g.nout == 1 && g.Kc % 64 == 0 && g.Nout % 64 == 0,
                "nf4_gemm_dense: the launch on forward tiles is a plain grad-input launch");
