@@ -1093,10 +1093,25 @@ TnPlan plan_tn_gh(const GroupSkinny& g) {
   for (int i = 0; i < g.n; ++i) groups += tn_gh_col_groups(g.N[i]);
   return plan_tn(g.M, groups);
 }
-// The pair kernel (swiglu_bwd_tn_gh_kernel) serves both members from one workgroup per column group: half as many
-// column groups in the grid, so twice the row splits fill the chip.
+// The pair kernel (swiglu_bwd_tn_gh_kernel) serves both members from one workgroup per column group.
 bool tn_gh_pair(const GroupSkinny& g) { return g.n == 2 && g.N[0] == g.N[1]; }
-TnPlan plan_tn_gh_pair(const GroupSkinny& g) { return plan_tn(g.M, tn_gh_col_groups(g.N[0])); }
+TnPlan plan_tn_gh_pair(const GroupSkinny& g) {
+  // The pair kernel holds a compute unit by itself (one workgroup of four waves at its register count), and what a
+  // workgroup does once - staging lora_b, the reduction of its sums - is a tenth of a 1024-row range's time: one round of
+  // long ranges beats two of short ones (8192 x 14336: 288 us with 4 splits = 224 workgroups against 302 with 8 and 388
+  // with 5, which start a second round; 4096 x 28672: 284 with 2, 303 with 4; 8192 x 8192: 170 with 8, 186 with 16).
+  // Hence: as many row splits as still fit one round of the chip.
+  const int64_t col_groups = tn_gh_col_groups(g.N[0]);
+  constexpr int64_t kCUs = 256;  // MI355X
+  int s = (int)(kCUs / col_groups);
+  s = s < 1 ? 1 : s;
+  const int max_s = (int)((g.M + 127) / 128);
+  s = s > max_s ? max_s : s;
+  TnPlan p;
+  p.rows_per_split = (int)(((g.M + s - 1) / s + 127) / 128 * 128);
+  p.splits = (int)((g.M + p.rows_per_split - 1) / p.rows_per_split);
+  return p;
+}
 // fp32 partial sums of the fused pass: per member the column groups' [M, R] and the row splits' [R, N] (room for the
 // plan with more splits where both kernels can serve the group)
 size_t tn_gh_part_bytes(const GroupSkinny& g) {
