@@ -326,6 +326,7 @@ struct DenseArgs {
   // the two segments alternately, 128 wide.
   int w_tr, w_paired;
   uint16_t* act;    // gated launches only: [M, out[0].width] bf16 = silu(out 0) * out 1
+  int stream_members;  // gated launches only: out 0 and out 1 go out as streaming (non-temporal) stores
   // SwiGLU-backward launches only (one output): the result is the gradient of silu(gate) * up; out[0].C receives the
   // gradient of gate and sw_gup that of up, both [M, out[0].width] like gate and up themselves
   const uint16_t* sw_gate;
@@ -950,12 +951,27 @@ __device__ __forceinline__ void gemm_dense_tile(const DenseArgs g) {
       }
       return;
     }
+    auto store_band = [&](auto streaming) {
 #pragma unroll 8
-    for (int t = 0; t < 16; ++t) {
-      const int r = 8 * t + (lane >> 3);
-      const u32x4_t v = *reinterpret_cast<const u32x4_t*>(band + r * 128 + ((c ^ (r & 7)) << 4));
-      if (mrow0 + r < g.M) *reinterpret_cast<u32x4_t*>(crow + (int64_t)(mrow0 + r) * width) = v;
-    }
+      for (int t = 0; t < 16; ++t) {
+        const int r = 8 * t + (lane >> 3);
+        const u32x4_t v = *reinterpret_cast<const u32x4_t*>(band + r * 128 + ((c ^ (r & 7)) << 4));
+        if (mrow0 + r < g.M) {
+          u32x4_t* dst = reinterpret_cast<u32x4_t*>(crow + (int64_t)(mrow0 + r) * width);
+          if constexpr (decltype(streaming)::value)
+            __builtin_nontemporal_store(v, dst);
+          else
+            *dst = v;
+        }
+      }
+    };
+    // stream_members (gated launches): gate and up are not read again before the backward, act is read twice right away
+    // (by the next layer's rank-r product and by its GEMM); written as streaming stores the two do not push act out of
+    // the memory-side cache where act fits it
+    if (GATED && g.stream_members)
+      store_band(std::true_type{});
+    else
+      store_band(std::false_type{});
     if constexpr (GATED) {
       // act: the 128 x 64 piece (wm, wn & 1) is shared by the two waves that hold its gate and up bands, 64 rows each
       const char* gband = smem + (4 * wm + (wn & 1)) * 16384;
@@ -1066,6 +1082,9 @@ int launch_dense(DenseArgs& g, hipStream_t s) {
     TT_REQUIRE(g.lw_row_major && g.nout == 2 && (g.nad == 2 || g.nad == 0) && g.nseg == 1 && g.out[0].width == g.out[1].width &&
                    g.out[0].width % 128 == 0 && g.Nout == 2 * g.out[0].width,
                "nf4_gemm_dense: the gated launch takes two members of equal width, a multiple of 128");
+    // act alone must fit the 256 MB memory-side cache with room to spare (measured: 8192 x 8192 bf16, 134 MB: the gated
+    // launch 449 -> 437 us and the step -1 %; 8192 x 14336, 235 MB: the launch 1366 -> 1382 us, the step unchanged)
+    g.stream_members = (int64_t)g.M * g.out[0].width * 2 <= (int64_t(160) << 20) ? 1 : 0;
     nf4_gemm_dense_kernel<true, true><<<grid, block, kLdsDense, s>>>(g);
   } else if (g.sw_gup) {
     TT_REQUIRE(!g.lw_row_major && g.nout == 1 && g.out[0].n_begin == 0 && g.out[0].width == g.Nout && !g.out[0].bias &&
