@@ -475,7 +475,8 @@ __device__ __forceinline__ void gemm_dense_tile(const DenseArgs g) {
   };
 
   // ---- forward launches: the adapter's operands travel through the same rings as further k-steps of the contraction.
-  //      Past the end of the weight the loop's requests used to fetch the last step again; they now fetch the adapter:
+  //      The loop's last trips request past the end of the weight (the waits count a fixed number of requests in flight,
+  //      so the requests keep coming); in a forward launch with an adapter those requests fetch the adapter instead:
   //      16 bytes (8 ranks of one row of lX / one row of lW) per lane, zeros beyond R, so that by the end of the loop the
   //      operands sit in LDS in the loop's own layout and the adapter costs one more k-step per 32 ranks instead of a trip
   //      to memory.  Ranks of at most 32 (ad_compact) need activation entry nk2 and weight step nk only: the entry's first
