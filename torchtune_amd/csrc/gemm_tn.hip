@@ -68,8 +68,27 @@ constexpr int kTnMT = 8, kTnNT = 4;  // 16 x 16 MFMA tiles per wave: MT along th
 // Tile `id` of a launch: the member it belongs to and its first row (within the member) and column.
 __device__ __forceinline__ void tn_locate(const TnArgs& g, int id, int& which, int& n0, int& k0) {
   int tile_n, tile_k;
-  // tile ids are dealt round-robin to the 8 XCDs: every XCD gets a band of row tiles and walks it column by column
-  if ((g.tiles_n & 7) == 0) {
+  // Tile ids are dealt round-robin to the 8 XCDs (one L2 each), 32 at a time.  Where the grid divides into blocks of
+  // 4 x 8 tiles, eight at a time, an XCD works on one block at a time: 4 + 8 operand panels of 256 columns through its L2
+  // per round (bands of two row tiles walked column by column would be 2 + 16); the XCDs of a round take different rows of
+  // the same eight columns.
+  // The blocks beyond the last whole eight (the tiles of a last partial round, ids from 256 * rounds on) follow in order.
+  const int super_rows = g.tiles_n >> 2, runs = g.tiles_k >> 3;
+  if ((g.tiles_n & 3) == 0 && (g.tiles_k & 7) == 0) {
+    const int whole = (super_rows * runs) & ~7;  // blocks in whole rounds
+    int block, t;
+    if (id < 32 * whole) {
+      const int xcd = id & 7, slot = id >> 3;
+      block = (slot >> 5) * 8 + xcd;
+      t = slot & 31;
+    } else {
+      block = whole + ((id - 32 * whole) >> 5);
+      t = id & 31;
+    }
+    tile_n = 4 * (block % super_rows) + (t & 3);
+    tile_k = 8 * (block / super_rows) + (t >> 2);
+  } else if ((g.tiles_n & 7) == 0) {
+    // otherwise every XCD gets a band of row tiles and walks it column by column
     const int xcd = id & 7, slot = id >> 3, band = g.tiles_n >> 3;
     tile_n = xcd * band + slot % band;
     tile_k = slot / band;
