@@ -335,6 +335,7 @@ struct DenseArgs {
 };
 
 constexpr int kEpiPlain = 0, kEpiGated = 1, kEpiSwigluBwd = 2;
+constexpr int kSegWalk = 0, kSegOne = 1, kSegPaired = 2;
 
 // what the direct-to-LDS requests of the adapter's operands read for ranks beyond R
 static __device__ __attribute__((aligned(16))) const uint32_t kZero16[4] = {0u, 0u, 0u, 0u};
@@ -361,7 +362,15 @@ constexpr int kLdsDense = kWBase + 4 * kWStage;
 // k-group kg) sits in slot (p ^ 4 (kg & 1)) + 16 kg (applied on the global-address side of the direct-to-LDS loads), so
 // that the 32 lanes served together touch 64 different banks.  Same products, same order of summation as the launch on
 // tiles of W^T: the results are equal bit for bit.
-template <bool LW_ROW_MAJOR, int EPI, bool W_TR = false>
+// SEGS: how the contraction's activation segments are found - kSegOne: there is one (every forward launch; checked on the
+// host); kSegPaired (W_TR only): two of equal width, visited 128 columns at a time, chosen by mask arithmetic on two base
+// addresses held in scalar registers; kSegWalk: up to kGroupMax, walked as the requests move forward.  With kSegOne and
+// kSegPaired the main loop is one block with one backward branch; the walk costs two more taken branches per trip,
+// which the single-segment launches on forward tiles paid with 5 % of their time while they shared its code.  (A
+// branch-free table for the general case - every segment's first entry, base and pitch in scalar registers, selected
+// per request - was 2 - 3 % slower than the walk: 30 more scalar instructions per trip in a loop that is bound by
+// what a wave can issue.)
+template <bool LW_ROW_MAJOR, int EPI, bool W_TR = false, int SEGS = LW_ROW_MAJOR ? kSegOne : kSegWalk>
 __device__ __forceinline__ void gemm_dense_tile(const DenseArgs g) {
 #if defined(__HIP_DEVICE_COMPILE__)
   constexpr bool GATED = EPI == kEpiGated;
@@ -414,8 +423,10 @@ __device__ __forceinline__ void gemm_dense_tile(const DenseArgs g) {
     const int row = m0 + trow;
     a_row[i] = row < g.M ? row : g.M - 1;
   }
+  // segment q: entries [seg_first[q], seg_first[q + 1]) of the contraction, rows seg_pitch[q] bytes apart (absent ones
+  // begin beyond every entry)
   uint32_t a_off[4];
-  int seg = 0, seg_begin = 0, seg_end = g.seg[0].Kc >> 6;  // entries [seg_begin, seg_end) belong to segment seg
+  int seg = 0, seg_begin = 0, seg_end = g.seg[0].Kc >> 6;  // kSegWalk: entries [seg_begin, seg_end) belong to segment seg
   const char* a_base = reinterpret_cast<const char*>(g.seg[0].X);
   auto set_segment = [&]() {
     const uint32_t pitch = (uint32_t)g.seg[seg].Kc * 2u;
@@ -423,6 +434,9 @@ __device__ __forceinline__ void gemm_dense_tile(const DenseArgs g) {
     for (int i = 0; i < 4; ++i) a_off[i] = (uint32_t)a_row[i] * pitch + (uint32_t)a_chunk[i];
   };
   set_segment();
+  // kSegPaired: the two bases as integers (a select among pointers read from the argument struct becomes an indexed load
+  // inside the loop, and the wait for it drains the ring's requests)
+  const int64_t pair_base0 = (int64_t)(uintptr_t)g.seg[0].X, pair_base1 = (int64_t)(uintptr_t)g.seg[SEGS == kSegPaired ? 1 : 0].X;
   const int nblocks = g.Nout >> 4;
   const char* wsrc0;
   const char* wsrc1;
@@ -459,25 +473,27 @@ __device__ __forceinline__ void gemm_dense_tile(const DenseArgs g) {
     dma16(lane16, wsrc0 + (int64_t)tk * wstep, sw, 0);
     dma16(lane16, wsrc1 + (int64_t)tk * wstep, sw, 1024);
   };
-  // entries are requested in increasing order (past the end: the last one again), so the segment only moves forward
   auto issue_a = [&](int T2, int entry) {
     const int tk = T2 < nk2 ? T2 : nk2 - 1;
     const char* xb;
-    if (W_TR && g.w_paired) {
+    if constexpr (SEGS == kSegOne) {
+      xb = a_base + ((int64_t)tk << 7);  // + 64 elements * 2 bytes per entry
+    } else if constexpr (SEGS == kSegPaired) {
       // two segments of equal width, visited 128 columns (two entries) at a time: entry tk is entry
       // 2 (tk / 4) + tk % 2 of segment (tk / 2) % 2; the row pitch is the same for both
-      xb = reinterpret_cast<const char*>(g.seg[(tk >> 1) & 1].X) + ((int64_t)(((tk >> 2) << 1) + (tk & 1)) << 7);
+      const int64_t second = -(int64_t)((tk >> 1) & 1);
+      xb = reinterpret_cast<const char*>((uintptr_t)((pair_base0 ^ ((pair_base0 ^ pair_base1) & second)) +
+                                                     ((int64_t)(((tk >> 2) << 1) + (tk & 1)) << 7)));
     } else {
-      if constexpr (!LW_ROW_MAJOR) {  // a forward launch has one segment (checked on the host): no walk in its loop
-        while (tk >= seg_end) {
-          ++seg;
-          seg_begin = seg_end;
-          seg_end += g.seg[seg].Kc >> 6;
-          a_base = reinterpret_cast<const char*>(g.seg[seg].X);
-          set_segment();
-        }
+      // entries are requested in increasing order (past the end: the last one again), so the segment only moves forward
+      while (tk >= seg_end) {
+        ++seg;
+        seg_begin = seg_end;
+        seg_end += g.seg[seg].Kc >> 6;
+        a_base = reinterpret_cast<const char*>(g.seg[seg].X);
+        set_segment();
       }
-      xb = a_base + ((int64_t)(tk - seg_begin) << 7);  // + 64 elements * 2 bytes per entry
+      xb = a_base + ((int64_t)(tk - seg_begin) << 7);
     }
     const uint32_t sa = lds0 + entry * kAEntry + wv * 4096;
     dma16(a_off[0], xb, sa, 0);
@@ -1010,8 +1026,12 @@ template <bool LW_ROW_MAJOR, bool GATED = false>
 __global__ __launch_bounds__(512) void nf4_gemm_dense_kernel(const DenseArgs g) {
   gemm_dense_tile<LW_ROW_MAJOR, GATED ? kEpiGated : kEpiPlain>(g);
 }
+// grad-input launches of a single layer (one segment) and, on forward tiles, of the gated pair (paired segments)
+__global__ __launch_bounds__(512) void nf4_gemm_dense_dx1_kernel(const DenseArgs g) { gemm_dense_tile<false, kEpiPlain, false, kSegOne>(g); }
+__global__ __launch_bounds__(512) void nf4_gemm_dense_tr1_kernel(const DenseArgs g) { gemm_dense_tile<false, kEpiPlain, true, kSegOne>(g); }
+__global__ __launch_bounds__(512) void nf4_gemm_dense_trp_kernel(const DenseArgs g) { gemm_dense_tile<false, kEpiPlain, true, kSegPaired>(g); }
 // grad-input launch (adapter weights [r, K]) whose result goes on through the backward of silu(gate) * up
-__global__ __launch_bounds__(512) void nf4_gemm_dense_swiglu_bwd_kernel(const DenseArgs g) { gemm_dense_tile<false, kEpiSwigluBwd>(g); }
+__global__ __launch_bounds__(512) void nf4_gemm_dense_swiglu_bwd_kernel(const DenseArgs g) { gemm_dense_tile<false, kEpiSwigluBwd, false, kSegOne>(g); }
 // grad-input launch on the forward launch's tiles
 __global__ __launch_bounds__(512) void nf4_gemm_dense_tr_kernel(const DenseArgs g) { gemm_dense_tile<false, kEpiPlain, true>(g); }
 
@@ -1071,7 +1091,10 @@ int launch_dense(DenseArgs& g, hipStream_t s) {
     for (const void* fn : {reinterpret_cast<const void*>(&nf4_gemm_dense_kernel<true>), reinterpret_cast<const void*>(&nf4_gemm_dense_kernel<false>),
                            reinterpret_cast<const void*>(&nf4_gemm_dense_kernel<true, true>),
                            reinterpret_cast<const void*>(&nf4_gemm_dense_swiglu_bwd_kernel),
-                           reinterpret_cast<const void*>(&nf4_gemm_dense_tr_kernel)}) {
+                           reinterpret_cast<const void*>(&nf4_gemm_dense_tr_kernel),
+                           reinterpret_cast<const void*>(&nf4_gemm_dense_dx1_kernel),
+                           reinterpret_cast<const void*>(&nf4_gemm_dense_tr1_kernel),
+                           reinterpret_cast<const void*>(&nf4_gemm_dense_trp_kernel)}) {
       hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsDense);
       if (e != hipSuccess) return fail(TTAMD_ELAUNCH, "nf4_gemm_dense: cannot reserve %d bytes of LDS: %s", kLdsDense, hipGetErrorString(e));
     }
@@ -1088,7 +1111,12 @@ int launch_dense(DenseArgs& g, hipStream_t s) {
                "nf4_gemm_dense: the launch on forward tiles is a plain grad-input launch");
     TT_REQUIRE(!g.w_paired || (g.nseg == 2 && g.seg[0].Kc == g.seg[1].Kc && g.seg[0].Kc % 128 == 0),
                "nf4_gemm_dense: paired forward tiles belong to two members of equal width, a multiple of 128");
-    nf4_gemm_dense_tr_kernel<<<grid, block, kLdsDense, s>>>(g);
+    if (g.w_paired)
+      nf4_gemm_dense_trp_kernel<<<grid, block, kLdsDense, s>>>(g);
+    else if (g.nseg == 1)
+      nf4_gemm_dense_tr1_kernel<<<grid, block, kLdsDense, s>>>(g);
+    else
+      nf4_gemm_dense_tr_kernel<<<grid, block, kLdsDense, s>>>(g);
     return check_launch("nf4_gemm_dense_tr");
   }
   if (g.act) {
@@ -1106,6 +1134,8 @@ int launch_dense(DenseArgs& g, hipStream_t s) {
     nf4_gemm_dense_swiglu_bwd_kernel<<<grid, block, kLdsDense, s>>>(g);
   } else if (g.lw_row_major)
     nf4_gemm_dense_kernel<true><<<grid, block, kLdsDense, s>>>(g);
+  else if (g.nseg == 1)
+    nf4_gemm_dense_dx1_kernel<<<grid, block, kLdsDense, s>>>(g);
   else
     nf4_gemm_dense_kernel<false><<<grid, block, kLdsDense, s>>>(g);
   return check_launch("nf4_gemm_dense");
