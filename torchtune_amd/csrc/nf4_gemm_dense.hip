@@ -425,18 +425,23 @@ __device__ __forceinline__ void gemm_dense_tile(const DenseArgs g) {
   }
   // segment q: entries [seg_first[q], seg_first[q + 1]) of the contraction, rows seg_pitch[q] bytes apart (absent ones
   // begin beyond every entry)
+  // The four requests of an entry (and the two of a weight step) name their LDS destinations through the instruction's
+  // offset field, which moves the global address along with the LDS address: one M0 write per entry / step instead of
+  // one per request.  Request i therefore carries offset 1024 i and a lane offset that is 1024 i short, all of them
+  // lifted by kAShift so that none is negative, against a base lowered by as much.
+  constexpr int kAShift = 3072;
   uint32_t a_off[4];
   int seg = 0, seg_begin = 0, seg_end = g.seg[0].Kc >> 6;  // kSegWalk: entries [seg_begin, seg_end) belong to segment seg
-  const char* a_base = reinterpret_cast<const char*>(g.seg[0].X);
+  const char* a_base = reinterpret_cast<const char*>(g.seg[0].X) - kAShift;
   auto set_segment = [&]() {
     const uint32_t pitch = (uint32_t)g.seg[seg].Kc * 2u;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) a_off[i] = (uint32_t)a_row[i] * pitch + (uint32_t)a_chunk[i];
+    for (int i = 0; i < 4; ++i) a_off[i] = (uint32_t)a_row[i] * pitch + (uint32_t)a_chunk[i] + (uint32_t)(kAShift - 1024 * i);
   };
   set_segment();
   // kSegPaired: the two bases as integers (a select among pointers read from the argument struct becomes an indexed load
   // inside the loop, and the wait for it drains the ring's requests)
-  const int64_t pair_base0 = (int64_t)(uintptr_t)g.seg[0].X, pair_base1 = (int64_t)(uintptr_t)g.seg[SEGS == kSegPaired ? 1 : 0].X;
+  const int64_t pair_base0 = (int64_t)(uintptr_t)g.seg[0].X - kAShift, pair_base1 = (int64_t)(uintptr_t)g.seg[SEGS == kSegPaired ? 1 : 0].X - kAShift;
   const int nblocks = g.Nout >> 4;
   const char* wsrc0;
   const char* wsrc1;
@@ -462,16 +467,18 @@ __device__ __forceinline__ void gemm_dense_tile(const DenseArgs g) {
     lane16 = (uint32_t)lane * 16u;
   }
 
-  auto dma16 = [&](uint32_t voff, const char* base, uint32_t lds, int imm) {
-    asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                 ::"v"(voff), "s"(base), "s"(lds), "n"(imm) : "memory", "m0", "scc");
-  };
+  // the two requests of a weight step: one base (the first piece's, lowered by 1024) and the second piece's distance in
+  // the lane offset
+  const char* const wbase = wsrc0 - 1024;
+  const uint32_t w_voff0 = lane16 + 1024u, w_voff1 = lane16 + (uint32_t)(wsrc1 - wsrc0);
   const uint32_t lds0 = (uint32_t)(uintptr_t)TT_LDS_PTR(smem);
   auto issue_w = [&](int t, int stage) {
     const int tk = t < nk ? t : nk - 1;
     const uint32_t sw = lds0 + kWBase + stage * kWStage + wv * 2048;
-    dma16(lane16, wsrc0 + (int64_t)tk * wstep, sw, 0);
-    dma16(lane16, wsrc1 + (int64_t)tk * wstep, sw, 1024);
+    asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\t"
+                 "global_load_lds_dwordx4 %0, %2\n\t"
+                 "global_load_lds_dwordx4 %1, %2 offset:1024"
+                 ::"v"(w_voff0), "v"(w_voff1), "s"(wbase + (int64_t)tk * wstep), "s"(sw) : "memory", "m0");
   };
   auto issue_a = [&](int T2, int entry) {
     const int tk = T2 < nk2 ? T2 : nk2 - 1;
@@ -490,16 +497,18 @@ __device__ __forceinline__ void gemm_dense_tile(const DenseArgs g) {
         ++seg;
         seg_begin = seg_end;
         seg_end += g.seg[seg].Kc >> 6;
-        a_base = reinterpret_cast<const char*>(g.seg[seg].X);
+        a_base = reinterpret_cast<const char*>(g.seg[seg].X) - kAShift;
         set_segment();
       }
       xb = a_base + ((int64_t)(tk - seg_begin) << 7);
     }
     const uint32_t sa = lds0 + entry * kAEntry + wv * 4096;
-    dma16(a_off[0], xb, sa, 0);
-    dma16(a_off[1], xb, sa, 1024);
-    dma16(a_off[2], xb, sa, 2048);
-    dma16(a_off[3], xb, sa, 3072);
+    asm volatile("s_mov_b32 m0, %5\n\ts_nop 0\n\t"
+                 "global_load_lds_dwordx4 %0, %4\n\t"
+                 "global_load_lds_dwordx4 %1, %4 offset:1024\n\t"
+                 "global_load_lds_dwordx4 %2, %4 offset:2048\n\t"
+                 "global_load_lds_dwordx4 %3, %4 offset:3072"
+                 ::"v"(a_off[0]), "v"(a_off[1]), "v"(a_off[2]), "v"(a_off[3]), "s"(xb), "s"(sa) : "memory", "m0");
   };
 
   // ---- forward launches: the adapter's operands travel through the same rings as further k-steps of the contraction.
