@@ -472,16 +472,18 @@ __device__ __forceinline__ void gemm_dense_tile(const DenseArgs g) {
   const char* const wbase = wsrc0 - 1024;
   const uint32_t w_voff0 = lane16 + 1024u, w_voff1 = lane16 + (uint32_t)(wsrc1 - wsrc0);
   const uint32_t lds0 = (uint32_t)(uintptr_t)TT_LDS_PTR(smem);
-  auto issue_w = [&](int t, int stage) {
-    const int tk = t < nk ? t : nk - 1;
+  // inside: the caller knows that the step / entry exists (no clamp: the address is then a constant distance from the
+  // loop's counter, which the compiler carries as a running pointer)
+  auto issue_w = [&](int t, int stage, bool inside = false) {
+    const int tk = inside || t < nk ? t : nk - 1;
     const uint32_t sw = lds0 + kWBase + stage * kWStage + wv * 2048;
     asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\t"
                  "global_load_lds_dwordx4 %0, %2\n\t"
                  "global_load_lds_dwordx4 %1, %2 offset:1024"
                  ::"v"(w_voff0), "v"(w_voff1), "s"(wbase + (int64_t)tk * wstep), "s"(sw) : "memory", "m0");
   };
-  auto issue_a = [&](int T2, int entry) {
-    const int tk = T2 < nk2 ? T2 : nk2 - 1;
+  auto issue_a = [&](int T2, int entry, bool inside = false) {
+    const int tk = inside || T2 < nk2 ? T2 : nk2 - 1;
     const char* xb;
     if constexpr (SEGS == kSegOne) {
       xb = a_base + ((int64_t)tk << 7);  // + 64 elements * 2 bytes per entry
@@ -699,16 +701,25 @@ __device__ __forceinline__ void gemm_dense_tile(const DenseArgs g) {
   // one copy of the loop per wave group: the two differ in one wait, and a branch per step costs 2 - 4 %
   auto main_loop = [&](auto lgkm) {
     constexpr bool kLgkm = decltype(lgkm)::value;
-    int e0 = 0, ws = 0;  // activation entry of the current pair of steps, weight stage of the current step
+    int e0_running = 0;  // activation entry of the current pair of steps; the weight stage of step t is t % 4
     // The last two trips, whose requests reach past the weight, are copies of the loop that ask for the adapter's
     // operands instead (ad_rings; no trip of the first copy pays for the choice).  kTrip 1 (t = nk - 4) requests entry
     // nk2 and step nk where the others request the activations and the weight; kTrip 2 (t = nk - 2) requests step nk + 1,
     // entry nk2 + 1 and step nk + 1 again (the count of requests in flight stays what the waits assume) - or nothing
     // (ad_compact), and then waits by the counts of that case: newer than W(nk - 1) are A x4 and W(nk) x2, and by the end
     // of the last step everything has landed.
-    auto pair = [&](int t, auto trip) {
+    // kWs: the weight stage of the trip's even step where the caller knows it (the loop below takes two trips at a time,
+    // so that stage offsets are constants of the instructions: no arithmetic on them in the loop), -1: t % 4
+    // kE0: the activation entry of the trip where the caller knows it, -1: the running one.  Both known: every LDS offset
+    // of the trip is a constant of its instructions, and none of its requests reaches past the weight.
+    auto pair = [&](int t, auto trip, auto stage, auto entry) {
       constexpr int kTrip = decltype(trip)::value;
+      constexpr int kWs = decltype(stage)::value;
+      constexpr int kE0 = decltype(entry)::value;
+      constexpr bool kInside = kE0 >= 0;
+      const int ws = kWs >= 0 ? kWs : (t & 3);
       const bool nothing = kTrip == 2 && ad_compact;
+      const int e0 = kE0 >= 0 ? kE0 : e0_running;
       const int e1 = e0 == 2 ? 0 : e0 + 1, e2 = e1 == 2 ? 0 : e1 + 1;
       // ---- even step t
       if constexpr (kTrip == 2) {
@@ -717,11 +728,11 @@ __device__ __forceinline__ void gemm_dense_tile(const DenseArgs g) {
           issue_a_ad(1, e2);
         }
       } else {
-        issue_w(t + 3, (ws + 3) & 3);
+        issue_w(t + 3, (ws + 3) & 3, kInside);
         if constexpr (kTrip == 1)
           issue_a_ad(0, e2);
         else
-          issue_a((t >> 1) + 2, e2);
+          issue_a((t >> 1) + 2, e2, kInside);
       }
       read_step(e0, 0, ws);
       __builtin_amdgcn_sched_barrier(0);
@@ -739,7 +750,7 @@ __device__ __forceinline__ void gemm_dense_tile(const DenseArgs g) {
       compute();
       // ---- odd step t + 1
       if constexpr (kTrip == 0)
-        issue_w(t + 4, ws);
+        issue_w(t + 4, ws, kInside);
       else if constexpr (kTrip == 1)
         issue_w_ad(0, ws);
       else if (!nothing)
@@ -758,15 +769,33 @@ __device__ __forceinline__ void gemm_dense_tile(const DenseArgs g) {
           asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");
       }
       compute();
-      e0 = e1;
-      ws = (ws + 2) & 3;
+      e0_running = e1;
     };
+    using C0 = std::integral_constant<int, 0>;
+    using C1 = std::integral_constant<int, 1>;
+    using C2 = std::integral_constant<int, 2>;
+    using Cr = std::integral_constant<int, -1>;
     const int t_tail = ad_rings ? nk - 4 : nk;
-    for (int t = 0; t < t_tail; t += 2) pair(t, std::integral_constant<int, 0>{});
+    if constexpr (SEGS == kSegWalk) {  // the walk's state on top of several trips' worth of code does not fit the registers
+      for (int t = 0; t < t_tail; t += 2) pair(t, C0{}, Cr{}, Cr{});
+    } else {
+      // six trips at a time (the weight ring repeats every two, the activation ring every three), as long as all of
+      // their requests stay inside the weight; the rest one by one with running indices and clamped requests
+      int t = 0;
+      for (; t + 12 <= t_tail && t + 16 <= nk; t += 12) {
+        pair(t, C0{}, C0{}, C0{});
+        pair(t + 2, C0{}, C2{}, C1{});
+        pair(t + 4, C0{}, C0{}, C2{});
+        pair(t + 6, C0{}, C2{}, C0{});
+        pair(t + 8, C0{}, C0{}, C1{});
+        pair(t + 10, C0{}, C2{}, C2{});
+      }
+      for (; t < t_tail; t += 2) pair(t, C0{}, Cr{}, Cr{});
+    }
     if constexpr (LW_ROW_MAJOR) {
       if (ad_rings) {
-        if (nk >= 4) pair(nk - 4, std::integral_constant<int, 1>{});
-        pair(nk - 2, std::integral_constant<int, 2>{});
+        if (nk >= 4) pair(nk - 4, C1{}, Cr{}, Cr{});
+        pair(nk - 2, C2{}, Cr{}, Cr{});
       }
     }
   };
