@@ -335,7 +335,7 @@ struct DenseArgs {
 };
 
 constexpr int kEpiPlain = 0, kEpiGated = 1, kEpiSwigluBwd = 2;
-constexpr int kSegWalk = 0, kSegOne = 1, kSegPaired = 2;
+constexpr int kSegWalk = 0, kSegOne = 1, kSegPaired = 2, kSegHalves = 3;
 
 // what the direct-to-LDS requests of the adapter's operands read for ranks beyond R
 static __device__ __attribute__((aligned(16))) const uint32_t kZero16[4] = {0u, 0u, 0u, 0u};
@@ -364,8 +364,9 @@ constexpr int kLdsDense = kWBase + 4 * kWStage;
 // tiles of W^T: the results are equal bit for bit.
 // SEGS: how the contraction's activation segments are found - kSegOne: there is one (every forward launch; checked on the
 // host); kSegPaired (W_TR only): two of equal width, visited 128 columns at a time, chosen by mask arithmetic on two base
-// addresses held in scalar registers; kSegWalk: up to kGroupMax, walked as the requests move forward.  With kSegOne and
-// kSegPaired the main loop is one block with one backward branch; the walk costs two more taken branches per trip,
+// addresses held in scalar registers; kSegHalves: two of equal width one after the other (the gate / up pair's output
+// gradients), the second base taken from the entry on where the first ends; kSegWalk: up to kGroupMax, walked as the
+// requests move forward.  With all but the walk the main loop is one block with one backward branch; the walk costs two more taken branches per trip,
 // which the single-segment launches on forward tiles paid with 5 % of their time while they shared its code.  (A
 // branch-free table for the general case - every segment's first entry, base and pitch in scalar registers, selected
 // per request - was 2 - 3 % slower than the walk: 30 more scalar instructions per trip in a loop that is bound by
@@ -441,7 +442,10 @@ __device__ __forceinline__ void gemm_dense_tile(const DenseArgs g) {
   set_segment();
   // kSegPaired: the two bases as integers (a select among pointers read from the argument struct becomes an indexed load
   // inside the loop, and the wait for it drains the ring's requests)
-  const int64_t pair_base0 = (int64_t)(uintptr_t)g.seg[0].X - kAShift, pair_base1 = (int64_t)(uintptr_t)g.seg[SEGS == kSegPaired ? 1 : 0].X - kAShift;
+  const int64_t pair_base0 = (int64_t)(uintptr_t)g.seg[0].X - kAShift, pair_base1 = (int64_t)(uintptr_t)g.seg[SEGS == kSegPaired || SEGS == kSegHalves ? 1 : 0].X - kAShift;
+  // kSegHalves: what the second segment's entries add to an address counted from the first segment's base
+  const int half_entries = g.seg[0].Kc >> 6;
+  const int64_t half_jump = pair_base1 - pair_base0 - ((int64_t)half_entries << 7);
   const int nblocks = g.Nout >> 4;
   const char* wsrc0;
   const char* wsrc1;
@@ -493,6 +497,8 @@ __device__ __forceinline__ void gemm_dense_tile(const DenseArgs g) {
       const int64_t second = -(int64_t)((tk >> 1) & 1);
       xb = reinterpret_cast<const char*>((uintptr_t)((pair_base0 ^ ((pair_base0 ^ pair_base1) & second)) +
                                                      ((int64_t)(((tk >> 2) << 1) + (tk & 1)) << 7)));
+    } else if constexpr (SEGS == kSegHalves) {
+      xb = reinterpret_cast<const char*>((uintptr_t)(pair_base0 + ((int64_t)tk << 7) + (half_jump & -(int64_t)(tk >= half_entries))));
     } else {
       // entries are requested in increasing order (past the end: the last one again), so the segment only moves forward
       while (tk >= seg_end) {
@@ -1068,6 +1074,8 @@ __global__ __launch_bounds__(512) void nf4_gemm_dense_kernel(const DenseArgs g) 
 __global__ __launch_bounds__(512) void nf4_gemm_dense_dx1_kernel(const DenseArgs g) { gemm_dense_tile<false, kEpiPlain, false, kSegOne>(g); }
 __global__ __launch_bounds__(512) void nf4_gemm_dense_tr1_kernel(const DenseArgs g) { gemm_dense_tile<false, kEpiPlain, true, kSegOne>(g); }
 __global__ __launch_bounds__(512) void nf4_gemm_dense_trp_kernel(const DenseArgs g) { gemm_dense_tile<false, kEpiPlain, true, kSegPaired>(g); }
+// grad-input launch of two members of equal width on transposed tiles (the gate / up pair)
+__global__ __launch_bounds__(512) void nf4_gemm_dense_dx2_kernel(const DenseArgs g) { gemm_dense_tile<false, kEpiPlain, false, kSegHalves>(g); }
 // grad-input launch (adapter weights [r, K]) whose result goes on through the backward of silu(gate) * up
 __global__ __launch_bounds__(512) void nf4_gemm_dense_swiglu_bwd_kernel(const DenseArgs g) { gemm_dense_tile<false, kEpiSwigluBwd, false, kSegOne>(g); }
 // grad-input launch on the forward launch's tiles
@@ -1132,7 +1140,8 @@ int launch_dense(DenseArgs& g, hipStream_t s) {
                            reinterpret_cast<const void*>(&nf4_gemm_dense_tr_kernel),
                            reinterpret_cast<const void*>(&nf4_gemm_dense_dx1_kernel),
                            reinterpret_cast<const void*>(&nf4_gemm_dense_tr1_kernel),
-                           reinterpret_cast<const void*>(&nf4_gemm_dense_trp_kernel)}) {
+                           reinterpret_cast<const void*>(&nf4_gemm_dense_trp_kernel),
+                           reinterpret_cast<const void*>(&nf4_gemm_dense_dx2_kernel)}) {
       hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsDense);
       if (e != hipSuccess) return fail(TTAMD_ELAUNCH, "nf4_gemm_dense: cannot reserve %d bytes of LDS: %s", kLdsDense, hipGetErrorString(e));
     }
@@ -1174,6 +1183,8 @@ int launch_dense(DenseArgs& g, hipStream_t s) {
     nf4_gemm_dense_kernel<true><<<grid, block, kLdsDense, s>>>(g);
   else if (g.nseg == 1)
     nf4_gemm_dense_dx1_kernel<<<grid, block, kLdsDense, s>>>(g);
+  else if (g.nseg == 2 && g.seg[0].Kc == g.seg[1].Kc)
+    nf4_gemm_dense_dx2_kernel<<<grid, block, kLdsDense, s>>>(g);
   else
     nf4_gemm_dense_kernel<false><<<grid, block, kLdsDense, s>>>(g);
   return check_launch("nf4_gemm_dense");
