@@ -176,20 +176,29 @@ __global__ __launch_bounds__(512) void gemm_tn_kernel(const TnArgs g) {
     a_off[d] = (uint32_t)rl * (uint32_t)N * 2u + (uint32_t)n0 * 2u + (uint32_t)chunk * 16u;
     b_off[d] = (uint32_t)rl * (uint32_t)g.K * 2u + (uint32_t)k0 * 2u + (uint32_t)chunk * 16u;
   }
-  auto dma16 = [&](uint32_t voff, const char* base, uint32_t lds, int imm) {
-    asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                 ::"v"(voff), "s"(base), "s"(lds), "n"(imm) : "memory", "m0", "scc");
-  };
+  // The two requests of an operand name their LDS destinations through the instruction's offset field, which moves the
+  // global address along with the LDS address: one M0 write per operand and step.  The second request therefore carries
+  // offset 1024 and a lane offset that is 1024 short; both are lifted by 1024 against a base lowered by as much, so that
+  // neither is negative.
+  const uint32_t a_v0 = a_off[0] + 1024u, a_v1 = a_off[1], b_v0 = b_off[0] + 1024u, b_v1 = b_off[1];
+  const char* const a_base = reinterpret_cast<const char*>(A) - 1024;
+  const char* const b_base = reinterpret_cast<const char*>(g.B) - 1024;
+  const int64_t a_step = (int64_t)N * 64, b_step = (int64_t)g.K * 64;  // 32 rows of the operand
   const uint32_t lds0 = (uint32_t)(uintptr_t)TT_LDS_PTR(smem);
-  auto issue = [&](int t, int stage) {
-    const int tk = t < nk ? t : nk - 1;
-    const char* ab = reinterpret_cast<const char*>(A) + (int64_t)tk * 32 * N * 2;
-    const char* bb = reinterpret_cast<const char*>(g.B) + (int64_t)tk * 32 * g.K * 2;
+  auto request = [&](const char* ab, const char* bb, int stage) {
     const uint32_t st = lds0 + stage * kTnStage + wv * 2048;
-    dma16(a_off[0], ab, st, 0);
-    dma16(a_off[1], ab, st, 1024);
-    dma16(b_off[0], bb, st, 16384);
-    dma16(b_off[1], bb, st, 16384 + 1024);
+    asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\t"
+                 "global_load_lds_dwordx4 %0, %2\n\t"
+                 "global_load_lds_dwordx4 %1, %2 offset:1024"
+                 ::"v"(a_v0), "v"(a_v1), "s"(ab), "s"(st) : "memory", "m0");
+    asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\t"
+                 "global_load_lds_dwordx4 %0, %2\n\t"
+                 "global_load_lds_dwordx4 %1, %2 offset:1024"
+                 ::"v"(b_v0), "v"(b_v1), "s"(bb), "s"(st + 16384u) : "memory", "m0");
+  };
+  auto issue = [&](int t, int stage) {  // past the end: the last step again (the waits count a fixed number in flight)
+    const int tk = t < nk ? t : nk - 1;
+    request(a_base + (int64_t)tk * a_step, b_base + (int64_t)tk * b_step, stage);
   };
 
   // ---- operand reads.  Lane (l15, g4) of ds_read_b64_tr_b16 points at row 8 g4 + l15 / 4 (+ 4 for the second half of the
@@ -282,8 +291,49 @@ __global__ __launch_bounds__(512) void gemm_tn_kernel(const TnArgs g) {
       else
         asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");
     };
-    int ws = 0;  // stage of the even step of the current pair: 0 or 2
     int t = t_begin;
+    // four steps at a time (the ring has four stages: every stage is then a constant of the instructions), as long as
+    // all of their requests stay inside the operands; the rest two by two with a running stage and clamped requests
+    {
+      const char* pa0[4];
+      const char* pb0[4];
+      const char* pa2[4];
+      const char* pb2[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        pa0[e] = smem + ra[e];
+        pb0[e] = smem + rb[e];
+        pa2[e] = smem + 2 * kTnStage + ra[e];
+        pb2[e] = smem + 2 * kTnStage + rb[e];
+      }
+      // the requests of the block run three steps ahead of t, on pointers of their own
+      const char* ap = a_base + (int64_t)(t + 3) * a_step;
+      const char* bp = b_base + (int64_t)(t + 3) * b_step;
+      auto next = [&](int stage) {
+        request(ap, bp, stage);
+        ap += a_step;
+        bp += b_step;
+      };
+      for (; t + 8 <= nk; t += 4) {
+        next(3);
+        read_step(pa0, pb0, 0);
+        end_of_memory_part();
+        compute();
+        next(0);
+        read_step(pa0, pb0, 1);
+        end_of_memory_part();
+        compute();
+        next(1);
+        read_step(pa2, pb2, 0);
+        end_of_memory_part();
+        compute();
+        next(2);
+        read_step(pa2, pb2, 1);
+        end_of_memory_part();
+        compute();
+      }
+    }
+    int ws = 0;  // stage of the even step of the current pair: 0 or 2 (whole rounds of the ring lie behind)
     for (; t + 1 < nk; t += 2) {
       const char* pa[4];
       const char* pb[4];
