@@ -73,7 +73,9 @@ class GemmTimer:
         self.counts = {}
         self.expanded_calls = 0
 
-    def __call__(self, kind, M, N, K, rank):
+    def __call__(self, kind, M, N, K, rank, on_tiles=False):
+        # on_tiles (grad-input calls): the GEMM reads the expanded weight its layer's forward call left behind - no expansion
+        # launch, and 2 B per weight element instead of the packed weight plus a copy written and read back
         # "fwd" / "bwd": one layer, one call of the library.  "fwd_group" / "bwd_group": the layers of a group with a common
         # input (N and rank are lists), one call; "fwd_gated": the gate / up pair with its gated product in the same call;
         # "bwd_swiglu": the grad-input of the layer after the gated product, carried on to the gradients of gate and up.  Between the events lie all launches of the call: with the weight expanded
@@ -101,7 +103,7 @@ class GemmTimer:
         # algorithmic bytes of a call: both activation tensors once, the packed weight with its fp32 block scalers
         # (0.5 + 4/64 B per element), the adapter operands; with the weight expanded once also the bf16 copy written and
         # read back (4 B per element)
-        per_w = 0.5625 + (4.0 if expanded else 0.0)
+        per_w = 2.0 if on_tiles else 0.5625 + (4.0 if expanded else 0.0)
         if fwd:
             launches = 1 if expanded else len(Ns)
             nbytes = (2.0 * M * K if expanded else 2.0 * M * K * len(Ns)) + sum(2.0 * M * n + per_w * n * K + 2.0 * r * (M + n) for n, r in zip(Ns, ranks))
@@ -681,7 +683,7 @@ def main() -> int:
     ap.add_argument("--keep-forward-tiles", type=int, default=None, metavar="TOKENS",
                     help="calls of at most this many tokens hand their expanded weight to the backward of the same layer, whose "
                          "grad-input GEMM reads it instead of expanding the weight again (0: never; default: the library's rule, "
-                         "torchtune_amd.ops.KEEP_FORWARD_TILES_MAX_TOKENS = 4096)")
+                         "torchtune_amd.ops.KEEP_FORWARD_TILES_MAX_TOKENS = 8192)")
     ap.add_argument("--resident-tiles-gib", type=float, default=0.0, metavar="GIB",
                     help="keep up to this many GiB of expanded NF4 weights across calls (2 B per weight element; the frozen base "
                          "weight never changes, so later steps run their GEMMs on the kept tiles and launch no expansion; "

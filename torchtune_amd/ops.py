@@ -175,10 +175,11 @@ def gemm_timer_installed() -> bool:
 
 
 def set_gemm_timer(timer) -> None:
-    """Install (or with None remove) a callback ``timer(kind, M, N, K, rank) -> (start_event, end_event)``; the two
-    events are recorded on the launch stream immediately before and after every fused-GEMM launch (``kind`` "fwd" /
-    "bwd"; for the group calls "fwd_group" / "bwd_group" with ``N`` and ``rank`` lists over the members).  Used by the
-    benchmark to time the dominant kernel in place."""
+    """Install (or with None remove) a callback ``timer(kind, M, N, K, rank, on_tiles=False) -> (start_event, end_event)``;
+    the two events are recorded on the launch stream immediately before and after every fused-GEMM launch (``kind`` "fwd" /
+    "bwd"; for the group calls "fwd_group" / "bwd_group" with ``N`` and ``rank`` lists over the members; ``on_tiles``: a
+    grad-input that reads the expanded weight its layer's forward call kept).  Used by the benchmark to time the
+    dominant kernel in place."""
     global _gemm_timer
     _gemm_timer = timer
 
@@ -242,11 +243,12 @@ EXPANDED_WEIGHT_PATH = True
 
 # One expansion for both directions: a forward call that expanded its weight hands the scratch copy to the backward of the
 # same layer, whose grad-input GEMM reads those forward tiles (transposing LDS reads) instead of expanding the weight a
-# second time.  The transposing reads cost the grad-input GEMM 3.5 % whatever the token count, the expansion saved is a
-# fixed cost per weight: at 4096 tokens it is 14 % of a call, at 8192 tokens 7 %, so the tiles are kept for calls of at
-# most this many tokens (0: never; a large number: always).  Kept tiles hold 2 bytes per weight element from a layer's
-# forward to its backward (with activation checkpointing: from the recomputation to the backward of one layer).
-KEEP_FORWARD_TILES_MAX_TOKENS = 4096
+# second time.  The launch on forward tiles takes as long as the one on transposed tiles (within 2 % either way at 8192
+# tokens), so what decides is memory: kept tiles hold 2 bytes per weight element from a layer's forward to its backward -
+# every layer's at once without activation checkpointing (13 GiB for an 8B model), one layer's at a time with it (from
+# the recomputation to the backward).  Measured up to 8192 tokens per call (8B step -0.8 %, 1B -1.2 % against a limit of
+# 4096); 0: never keep, a large number: always.
+KEEP_FORWARD_TILES_MAX_TOKENS = 8192
 
 
 def keeps_forward_tiles(M: int) -> bool:
@@ -695,7 +697,8 @@ def lora_group_bwd(x: torch.Tensor, h_cat: torch.Tensor, members: Sequence[Group
                                                _stream(x))
         _lib.check(rc, "lora_group_bwd")
         if want_gx:
-            events = _gemm_timer("bwd_group", M, [m.N for m in members], K, [int(e.rank) for e in arr]) if _gemm_timer is not None else None
+            events = (_gemm_timer("bwd_group", M, [m.N for m in members], K, [int(e.rank) for e in arr], on_tiles=tiles is not None)
+                      if _gemm_timer is not None else None)
             if tiles is not None:
                 if tiles.numel() * tiles.element_size() < 2 * K * sum(m.N for m in members) or not tiles.is_contiguous():
                     raise ValueError("lora_group_bwd: the forward tiles do not hold the members' weights")
@@ -1019,7 +1022,7 @@ def tiled_linear_dx(gy: torch.Tensor, tiled_fwd: torch.Tensor, K: int, gh: Optio
         # an installed timer books the call as what it is: the grad-input of an NF4 layer, or a GEMM on fake-quantised tiles
         events = None
         if _gemm_timer is not None:
-            events = _gemm_timer("bwd", M, N, K, r) if nf4_backward else _gemm_timer("tiled", M, K, N, 0)
+            events = _gemm_timer("bwd", M, N, K, r, on_tiles=True) if nf4_backward else _gemm_timer("tiled", M, K, N, 0)
         if events:
             events[0].record()
         rc = lib.ttamd_tiled_linear_dx_bf16(gy.data_ptr(), tiled_fwd.data_ptr(), _ptr(gh), _ptr(lora_a), r, gx.data_ptr(), M, N, K,
